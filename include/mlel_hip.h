@@ -1,0 +1,338 @@
+/*
+ * mlel_hip.h -- C ABI of the MI355X (gfx950) execution backend for TOSA 1.0 data-graph operators.
+ *
+ * This is the boundary the host-side operator surface (GraphPipeline::make<Op>, the mirror of the
+ * reference's graph/compute_graph_op.hpp:1204-1549) calls instead of building a VkPipeline and recording
+ * vkCmdDispatch (reference: graph/compute_graph_op.cpp:526-590).  One entry point per TOSA operator class
+ * of the reference; each takes tensor views (device pointer, dims, byte strides) and an attribute struct that
+ * is field-for-field the reference's push-constant + specialisation-constant set for that operator.
+ *
+ * Conventions
+ *   - plain C, no exceptions; every function returns 0 on success or a negative mlel_status and leaves a
+ *     human readable message retrievable with mlel_hip_last_error() (thread local);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); launches are asynchronous;
+ *   - tensor pointers are device pointers; strides are in BYTES (reference: tensor/tensor_arm.cpp:67-93),
+ *     rank <= 6 (reference: graph/shaders/graph_op/common.comp:11);
+ *   - reads outside a tensor's dims yield 0 and writes outside are dropped
+ *     (reference: tensor/shaders/tensor.glsl:26-81);
+ *   - nothing here falls back to a CPU implementation: without a GPU every launch returns MLEL_ERR_DEVICE.
+ */
+#ifndef MLEL_HIP_H
+#define MLEL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLEL_MAX_RANK 6
+
+/* Status codes. */
+typedef enum mlel_status {
+    MLEL_OK = 0,
+    MLEL_ERR_INVALID = -1,     /* bad argument: shape / dtype / attribute combination not accepted */
+    MLEL_ERR_UNSUPPORTED = -2, /* valid TOSA, but no kernel for this dtype combination              */
+    MLEL_ERR_DEVICE = -3,      /* HIP runtime error (no device, launch failure, out of memory)       */
+    MLEL_ERR_LIMIT = -4        /* size beyond a documented limit                                     */
+} mlel_status;
+
+/* Element types.  Mirrors the VkFormat -> shader type table of the reference (common/utils.cpp:119-228). */
+typedef enum mlel_dtype {
+    MLEL_BOOL = 0, /* VK_FORMAT_R8_BOOL_ARM, one byte, 0/1 */
+    MLEL_I8 = 1,
+    MLEL_U8 = 2,
+    MLEL_I16 = 3,
+    MLEL_U16 = 4,
+    MLEL_I32 = 5,
+    MLEL_U32 = 6,
+    MLEL_I64 = 7,
+    MLEL_U64 = 8,
+    MLEL_F16 = 9,
+    MLEL_BF16 = 10,
+    MLEL_F32 = 11,
+    MLEL_F64 = 12,
+    MLEL_F8E4M3 = 13,
+    MLEL_F8E5M2 = 14,
+    MLEL_DTYPE_COUNT = 15
+} mlel_dtype;
+
+/* Accumulator type codes as decoded from the SPIR-V operand (reference: graph/compute_graph_op.cpp:39-67). */
+enum { MLEL_ACC_I32 = 1, MLEL_ACC_F16 = 2, MLEL_ACC_F32 = 3, MLEL_ACC_I64 = 4 };
+/* NaN propagation modes (reference: graph/compute_graph_op.hpp:32-35). */
+enum { MLEL_NAN_PROPAGATE = 1, MLEL_NAN_IGNORE = 2 };
+/* RESCALE rounding modes (reference: graph/graph_tosa_1_0_ext_inst.cpp:29-33). */
+enum { MLEL_ROUND_SINGLE = 1, MLEL_ROUND_INEXACT = 2, MLEL_ROUND_DOUBLE = 3 };
+
+/* Tensor view.  Replaces the reference's tensor descriptor {address, dims[6], strides[6]}
+ * (reference: tensor/tensor_descriptor.cpp:56-80). */
+typedef struct mlel_tensor {
+    void *ptr;
+    int32_t dtype; /* mlel_dtype */
+    int32_t rank;  /* 1..6 */
+    int64_t dims[MLEL_MAX_RANK];
+    int64_t strides[MLEL_MAX_RANK]; /* bytes */
+} mlel_tensor;
+
+/* ---- attribute structs (same fields as the reference push constants) ---- */
+
+/* CONV2D / DEPTHWISE_CONV2D (reference: graph/compute_graph_op.hpp:418-425, 509-515).
+ * pad = {top, bottom, left, right}; stride = {y, x}; dilation = {y, x}. */
+typedef struct mlel_conv2d_attr {
+    int32_t input_zp;
+    int32_t weight_zp;
+    int32_t pad[4];
+    int32_t stride[2];
+    int32_t dilation[2];
+    uint32_t acc_type; /* MLEL_ACC_* */
+} mlel_conv2d_attr;
+
+/* MATMUL (reference: graph/compute_graph_op.hpp:655-658). */
+typedef struct mlel_matmul_attr {
+    int32_t a_zp;
+    int32_t b_zp;
+} mlel_matmul_attr;
+
+/* RESCALE (reference: push constants graph/compute_graph_op.hpp:846-849, specialisation constants
+ * {rank, scale32, doubleRound, perChannel} graph/compute_graph_op.cpp:1729, unsigned twins :1761-1762). */
+typedef struct mlel_rescale_attr {
+    int32_t input_zp;
+    int32_t output_zp;
+    uint32_t scale32;
+    uint32_t double_round;
+    uint32_t per_channel;
+    uint32_t input_unsigned;
+    uint32_t output_unsigned;
+} mlel_rescale_attr;
+
+/* CLAMP (reference: graph/compute_graph_op.hpp:352-356); min/max travel as double. */
+typedef struct mlel_clamp_attr {
+    double min_val;
+    double max_val;
+    uint32_t nan_mode;
+} mlel_clamp_attr;
+
+/* AVG_POOL2D / MAX_POOL2D (reference: graph/compute_graph_op.hpp:296-302, 688-693).
+ * kernel = {y, x}; stride = {y, x}; pad = {top, bottom, left, right}. */
+typedef struct mlel_pool2d_attr {
+    int32_t kernel[2];
+    int32_t stride[2];
+    int32_t pad[4];
+    int32_t input_zp;  /* AVG only */
+    int32_t output_zp; /* AVG only */
+    uint32_t acc_type; /* AVG only */
+    uint32_t nan_mode; /* MAX only */
+} mlel_pool2d_attr;
+
+/* Elementwise binary operator selector.  One value per `%operation%` string the reference substitutes into
+ * elementwise_binary.comp (reference: graph/compute_graph_op.cpp:2527-2946). */
+typedef enum mlel_binary_op {
+    MLEL_BIN_ADD = 0,
+    MLEL_BIN_SUB,
+    MLEL_BIN_BITWISE_AND,
+    MLEL_BIN_BITWISE_OR,
+    MLEL_BIN_BITWISE_XOR,
+    MLEL_BIN_INTDIV,
+    MLEL_BIN_LOGICAL_AND,
+    MLEL_BIN_LOGICAL_OR,
+    MLEL_BIN_LOGICAL_XOR,
+    MLEL_BIN_LOGICAL_LEFT_SHIFT,
+    MLEL_BIN_LOGICAL_RIGHT_SHIFT,
+    MLEL_BIN_MAXIMUM,
+    MLEL_BIN_MINIMUM,
+    MLEL_BIN_POW,
+    MLEL_BIN_EQUAL,
+    MLEL_BIN_GREATER,
+    MLEL_BIN_GREATER_EQUAL,
+    MLEL_BIN_COUNT
+} mlel_binary_op;
+
+/* Elementwise unary operator selector (reference: elementwise_unary.comp `%operation%` strings,
+ * graph/compute_graph_op.cpp:2527-2946). */
+typedef enum mlel_unary_op {
+    MLEL_UN_ABS = 0,
+    MLEL_UN_BITWISE_NOT,
+    MLEL_UN_CEIL,
+    MLEL_UN_CLZ,
+    MLEL_UN_COS,
+    MLEL_UN_ERF,
+    MLEL_UN_EXP,
+    MLEL_UN_FLOOR,
+    MLEL_UN_LOG,
+    MLEL_UN_LOGICAL_NOT,
+    MLEL_UN_RECIPROCAL,
+    MLEL_UN_RSQRT,
+    MLEL_UN_SIGMOID,
+    MLEL_UN_SIN,
+    MLEL_UN_TANH,
+    MLEL_UN_COUNT
+} mlel_unary_op;
+
+/* Reduction selector (reference: reduce.comp init/operation strings, graph/compute_graph_op.cpp:2819-2859). */
+typedef enum mlel_reduce_op {
+    MLEL_RED_ALL = 0,
+    MLEL_RED_ANY,
+    MLEL_RED_MAX,
+    MLEL_RED_MIN,
+    MLEL_RED_PRODUCT,
+    MLEL_RED_SUM,
+    MLEL_RED_COUNT
+} mlel_reduce_op;
+
+/* Fused epilogue of a contraction: RESCALE (always) then optional CLAMP, applied to the int32 accumulator
+ * before it is narrowed and stored.  Bit-identical to running the three operators one after another. */
+typedef struct mlel_epilogue {
+    const mlel_tensor *multiplier; /* i32[C] (scale32) or i16[C]; C == 1 unless per_channel */
+    const mlel_tensor *shift;      /* i8[C] */
+    mlel_rescale_attr rescale;
+    int32_t has_clamp;
+    mlel_clamp_attr clamp;
+} mlel_epilogue;
+
+/* ---- context, memory, streams, events ---- */
+
+typedef struct mlel_ctx mlel_ctx;
+
+/* Thread-local description of the last failure on the calling thread. */
+const char *mlel_hip_last_error(void);
+
+/* Library / device queries.  mlel_hip_device_count() never fails: it returns 0 when no GPU is visible. */
+int mlel_hip_device_count(void);
+int mlel_hip_init(int device, mlel_ctx **out_ctx);
+void mlel_hip_destroy(mlel_ctx *ctx);
+/* Fills compute units, engine clock (kHz), memory clock (kHz), bus width (bits), name (<=255 chars). */
+int mlel_hip_device_info(mlel_ctx *ctx, int32_t *cu_count, int32_t *clock_khz, int32_t *mem_clock_khz,
+                         int32_t *bus_width_bits, char *name, size_t name_len);
+
+/* Device arena (hipMalloc'd HBM).  Replaces VkDeviceMemory allocation of the reference
+ * (graph/tensor.cpp:95-114 for constants, utilities/tensor.cpp:100-108 for test tensors, zero-filled). */
+int mlel_hip_arena_alloc(mlel_ctx *ctx, size_t bytes, void **dptr);
+int mlel_hip_arena_free(mlel_ctx *ctx, void *dptr);
+/* Import of a Vulkan allocation exported as an opaque fd (VK_KHR_external_memory_fd) into the HIP address
+ * space; the returned pointer aliases the VkDeviceMemory. */
+int mlel_hip_arena_import_fd(mlel_ctx *ctx, int fd, size_t bytes, void **dptr, void **out_handle);
+int mlel_hip_arena_release_import(mlel_ctx *ctx, void *handle);
+int mlel_hip_memcpy_h2d(mlel_ctx *ctx, void *dst, const void *src, size_t bytes, void *stream);
+int mlel_hip_memcpy_d2h(mlel_ctx *ctx, void *dst, const void *src, size_t bytes, void *stream);
+int mlel_hip_memcpy_d2d(mlel_ctx *ctx, void *dst, const void *src, size_t bytes, void *stream);
+int mlel_hip_memset(mlel_ctx *ctx, void *dst, int value, size_t bytes, void *stream);
+
+int mlel_hip_stream_create(mlel_ctx *ctx, void **out_stream);
+int mlel_hip_stream_destroy(mlel_ctx *ctx, void *stream);
+int mlel_hip_sync(mlel_ctx *ctx, void *stream); /* NULL = whole device */
+
+/* Per-operator timing.  Replaces the reference's timestamp queries around each dispatch
+ * (graph/graph_profiler.cpp:157-191). */
+int mlel_hip_event_create(mlel_ctx *ctx, void **out_event);
+int mlel_hip_event_destroy(mlel_ctx *ctx, void *event);
+int mlel_hip_event_record(mlel_ctx *ctx, void *event, void *stream);
+int mlel_hip_event_elapsed_ms(mlel_ctx *ctx, void *start, void *stop, float *ms); /* synchronises on stop */
+
+/* HIP-graph capture of a sequence of launches on `stream`, used to replay a whole TOSA graph with one
+ * submission.  Replaces command-buffer recording + vkQueueSubmit (reference: graph/graph_layer.cpp:1844-1980). */
+int mlel_hip_capture_begin(mlel_ctx *ctx, void *stream);
+int mlel_hip_capture_end(mlel_ctx *ctx, void *stream, void **out_graph_exec);
+int mlel_hip_graph_launch(mlel_ctx *ctx, void *graph_exec, void *stream);
+int mlel_hip_graph_destroy(mlel_ctx *ctx, void *graph_exec);
+
+/* ---- operators ---- */
+
+/* CONV2D.  in [N,H,W,IC], w [OC,KH,KW,IC], bias [OC] or [1] typed as the output, out [N,OH,OW,OC].
+ * Replaces class Conv2D (reference: graph/compute_graph_op.cpp:914-1023) running conv2d.comp:40-116. */
+int mlel_hip_conv2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                    const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv2d_attr *attr);
+
+/* DEPTHWISE_CONV2D.  w [KH,KW,C,M], out channel = c*M+m.
+ * Replaces class DepthwiseConv2D (reference: graph/compute_graph_op.cpp:1116-1199), depthwise_conv2d.comp:31-78. */
+int mlel_hip_depthwise_conv2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                              const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv2d_attr *attr);
+
+/* MATMUL.  a [N,H,C], b [N,C,W], out [N,H,W].
+ * Replaces class Matmul (reference: graph/compute_graph_op.cpp:1387-1436), matmul.comp:30-73. */
+int mlel_hip_matmul(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
+                    const mlel_tensor *b, const mlel_matmul_attr *attr);
+
+/* RESCALE.  Replaces class Rescale (reference: graph/compute_graph_op.cpp:1719-1779), rescale.comp:27-72. */
+int mlel_hip_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                     const mlel_tensor *multiplier, const mlel_tensor *shift, const mlel_rescale_attr *attr);
+
+/* CLAMP.  Replaces class Clamp (reference: graph/compute_graph_op.cpp:811-853), clamp.comp:24-53. */
+int mlel_hip_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                   const mlel_clamp_attr *attr);
+
+/* ADD, SUB, MAXIMUM, ... with size-1 broadcast.  Replaces class ElementwiseBinary
+ * (reference: graph/compute_graph_op.cpp:1205-1255), elementwise_binary.comp:146-173. */
+int mlel_hip_elementwise_binary(mlel_ctx *ctx, void *stream, int32_t op, const mlel_tensor *out,
+                                const mlel_tensor *in1, const mlel_tensor *in2, uint32_t nan_mode);
+
+/* MUL.  Replaces class Mul (reference: graph/compute_graph_op.cpp:1508-1557), mul.comp:24-59. */
+int mlel_hip_mul(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1,
+                 const mlel_tensor *in2, uint32_t shift);
+
+/* ABS ... TANH.  Replaces class ElementwiseUnary (reference: graph/compute_graph_op.cpp:1261-1297),
+ * elementwise_unary.comp:188-205. */
+int mlel_hip_elementwise_unary(mlel_ctx *ctx, void *stream, int32_t op, const mlel_tensor *out,
+                               const mlel_tensor *in);
+
+/* REDUCE_*.  Output keeps the reduced axis with extent 1.  Replaces class Reduce
+ * (reference: graph/compute_graph_op.cpp:1665-1713), reduce.comp:24-70. */
+int mlel_hip_reduce(mlel_ctx *ctx, void *stream, int32_t op, const mlel_tensor *out, const mlel_tensor *in,
+                    uint32_t axis, uint32_t nan_mode);
+
+/* AVG_POOL2D / MAX_POOL2D.  Replace classes AvgPool2D / MaxPool2D
+ * (reference: graph/compute_graph_op.cpp:694-760, 1442-1502), avgpool2d.comp:27-75, maxpool2d.comp:23-72. */
+int mlel_hip_avg_pool2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                        const mlel_pool2d_attr *attr);
+int mlel_hip_max_pool2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                        const mlel_pool2d_attr *attr);
+
+/* TABLE.  Replaces class Table (reference: graph/compute_graph_op.cpp:2090-2126), table.comp:17-52. */
+int mlel_hip_table(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                   const mlel_tensor *table);
+
+/* CAST.  Replaces class Cast (reference: graph/compute_graph_op.cpp:766-805), cast.comp:22-103. */
+int mlel_hip_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in);
+
+/* NEGATE.  Replaces class Negate (reference: negate.comp:29-47). */
+int mlel_hip_negate(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                    int32_t input_zp, int32_t output_zp);
+
+/* Data movement.  Replace classes Reshape, Transpose, Concat (one call per input, running `offset` along
+ * `axis`, reference: graph/compute_graph_op.cpp:2607-2615), Slice, Pad and the shaders of the same names. */
+int mlel_hip_reshape(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in);
+int mlel_hip_transpose(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                       const uint32_t *perms);
+int mlel_hip_concat(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis,
+                    uint32_t offset);
+int mlel_hip_slice(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                   const uint32_t *start);
+int mlel_hip_pad(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                 const mlel_tensor *padding, double pad_const, int32_t pad_const_int);
+
+/* ---- fused entry points (chosen only by the host-side fusion pass; no counterpart in the reference, which
+ * runs one dispatch per TOSA instruction: graph/compute_graph_op.cpp:2500-2509).  Each equals, bit for bit,
+ * the unfused sequence <contraction> -> RESCALE -> [CLAMP] with an int32 intermediate. ---- */
+int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                  const mlel_tensor *weights, const mlel_tensor *bias,
+                                  const mlel_conv2d_attr *attr, const mlel_epilogue *epi);
+int mlel_hip_matmul_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
+                            const mlel_tensor *b, const mlel_matmul_attr *attr, const mlel_epilogue *epi);
+int mlel_hip_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                  const mlel_tensor *weights, const mlel_tensor *bias,
+                                  const mlel_conv2d_attr *attr, const mlel_epilogue *epi);
+/* out = RESCALE_o( RESCALE_a(in1) + RESCALE_b(in2) ): the residual-add pattern with both operands brought to
+ * a common int32 scale, added with wraparound, and requantised. */
+int mlel_hip_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1,
+                                 const mlel_epilogue *scale1, const mlel_tensor *in2, const mlel_epilogue *scale2,
+                                 const mlel_epilogue *scale_out);
+
+/* Plain device-to-device copy kernel of `bytes` bytes with 128-bit accesses; the calibration kernel for
+ * memory-traffic counters and the measured HBM ceiling. */
+int mlel_hip_copy_kernel(mlel_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MLEL_HIP_H */
