@@ -1,0 +1,402 @@
+// extern "C" operator entry points of include/mlel_hip.h: argument validation (the host-side checks that keep
+// every kernel's indexing assumptions true), then dispatch to a specialised gfx950 kernel or the generic path.
+#include "common.hpp"
+#include "dispatch.hpp"
+
+using namespace mlel;
+
+namespace {
+
+int require_ctx(mlel_ctx *ctx, const char *what) {
+    MLEL_REQUIRE(ctx != nullptr, MLEL_ERR_INVALID, "%s: null context", what);
+    hipError_t e = hipSetDevice(ctx->device);
+    if (e != hipSuccess) return set_error(MLEL_ERR_DEVICE, "%s: hipSetDevice: %s", what, hipGetErrorString(e));
+    return 0;
+}
+
+bool is_arith_dtype(int dt) { return dt_is_int(dt) || dt_is_float(dt); }
+
+int check_supported(const mlel_tensor *t, const char *what) {
+    MLEL_TRY(check_tensor(t, what));
+    MLEL_REQUIRE(is_arith_dtype(t->dtype), MLEL_ERR_UNSUPPORTED,
+                 "%s: element type %d (bf16/fp8 storage) has no kernel yet", what, t->dtype);
+    return 0;
+}
+
+int check_conv(const char *name, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
+               const mlel_tensor *bias, const mlel_conv2d_attr *a) {
+    MLEL_REQUIRE(a != nullptr, MLEL_ERR_INVALID, "%s: null attributes", name);
+    MLEL_TRY(check_supported(out, name));
+    MLEL_TRY(check_supported(in, name));
+    MLEL_TRY(check_supported(w, name));
+    MLEL_TRY(check_supported(bias, name));
+    MLEL_REQUIRE(out->rank == 4 && in->rank == 4 && w->rank == 4 && bias->rank == 1, MLEL_ERR_INVALID,
+                 "%s: ranks must be 4,4,4,1", name);
+    MLEL_REQUIRE(a->acc_type >= 1 && a->acc_type <= 4, MLEL_ERR_INVALID, "Unsupported acc type %u", a->acc_type);
+    const bool facc = a->acc_type == MLEL_ACC_F16 || a->acc_type == MLEL_ACC_F32;
+    MLEL_REQUIRE(facc == dt_is_float(in->dtype) && facc == dt_is_float(out->dtype), MLEL_ERR_INVALID,
+                 "%s: accumulator type %u does not match the tensor types", name, a->acc_type);
+    MLEL_REQUIRE(bias->dtype == out->dtype, MLEL_ERR_INVALID, "%s: bias must have the output type", name);
+    return 0;
+}
+
+int make_epilogue(const mlel_epilogue *epi, int in_dtype, const mlel_tensor *out, int64_t channels,
+                  FusedEpilogue *fe) {
+    MLEL_REQUIRE(epi != nullptr && epi->multiplier != nullptr && epi->shift != nullptr, MLEL_ERR_INVALID,
+                 "fused epilogue: null argument");
+    MLEL_TRY(check_scale_tensors(epi->multiplier, epi->shift, &epi->rescale, channels));
+    MLEL_REQUIRE(is_packed(epi->multiplier) && is_packed(epi->shift), MLEL_ERR_INVALID,
+                 "fused epilogue: multiplier/shift must be contiguous");
+    MLEL_REQUIRE(dt_is_int(out->dtype) && dt_size(out->dtype) <= 4 && out->dtype != MLEL_BOOL, MLEL_ERR_INVALID,
+                 "fused epilogue: output must be an 8/16/32-bit integer tensor");
+    MLEL_TRY(make_rescale_params(&epi->rescale, in_dtype, out->dtype, epi->has_clamp ? &epi->clamp : nullptr, &fe->p));
+    fe->mult = epi->multiplier;
+    fe->shift = epi->shift;
+    fe->scale32 = epi->rescale.scale32 != 0;
+    fe->in_dt = dt_unsigned_twin(in_dtype, epi->rescale.input_unsigned != 0);
+    return 0;
+}
+
+// scratch int32 tensor for a fused request that no specialised kernel takes: the unfused sequence is run instead
+struct Scratch {
+    void *ptr = nullptr;
+    ~Scratch() {
+        if (ptr) (void)hipFree(ptr);
+    }
+};
+
+int run_unfused_tail(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *acc,
+                     const mlel_epilogue *epi) {
+    // RESCALE into `out`, then CLAMP in place: exactly the operator sequence the fused kernels replace
+    MLEL_TRY(mlel_hip_rescale(ctx, s, out, acc, epi->multiplier, epi->shift, &epi->rescale));
+    if (epi->has_clamp) MLEL_TRY(mlel_hip_clamp(ctx, s, out, out, &epi->clamp));
+    return 0;
+}
+
+mlel_tensor packed_like(const mlel_tensor *t, int dtype, void *ptr) {
+    mlel_tensor r = *t;
+    r.dtype = dtype;
+    r.ptr = ptr;
+    int64_t s = dt_size(dtype);
+    for (int i = r.rank - 1; i >= 0; i--) {
+        r.strides[i] = s;
+        s *= r.dims[i];
+    }
+    return r;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mlel_hip_conv2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                    const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv2d_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "conv2d"));
+    MLEL_TRY(check_conv("conv2d", out, in, weights, bias, attr));
+    const int rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, out, in, weights, bias, attr, nullptr);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    return conv2d_generic_launch((hipStream_t)stream, out, in, weights, bias, attr);
+}
+
+int mlel_hip_depthwise_conv2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                              const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv2d_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "depthwise_conv2d"));
+    MLEL_TRY(check_conv("depthwise_conv2d", out, in, weights, bias, attr));
+    MLEL_REQUIRE(weights->dims[3] > 0, MLEL_ERR_INVALID, "depthwise_conv2d: channel multiplier must be > 0");
+    const int rc = try_dwconv_i8_fast(ctx, (hipStream_t)stream, out, in, weights, bias, attr, nullptr);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    return dwconv_generic_launch((hipStream_t)stream, out, in, weights, bias, attr);
+}
+
+int mlel_hip_matmul(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a, const mlel_tensor *b,
+                    const mlel_matmul_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "matmul"));
+    MLEL_REQUIRE(attr != nullptr, MLEL_ERR_INVALID, "matmul: null attributes");
+    MLEL_TRY(check_supported(out, "matmul out"));
+    MLEL_TRY(check_supported(a, "matmul a"));
+    MLEL_TRY(check_supported(b, "matmul b"));
+    MLEL_REQUIRE(out->rank == 3 && a->rank == 3 && b->rank == 3, MLEL_ERR_INVALID, "matmul: rank must be 3");
+    MLEL_REQUIRE(a->dtype == b->dtype, MLEL_ERR_INVALID, "matmul: operand types differ");
+    MLEL_REQUIRE(dt_is_float(a->dtype) == dt_is_float(out->dtype), MLEL_ERR_INVALID,
+                 "matmul: integer/float mismatch between operands and output");
+    const int rc = try_matmul_i8_mfma(ctx, (hipStream_t)stream, out, a, b, attr, nullptr);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    return matmul_generic_launch((hipStream_t)stream, out, a, b, attr);
+}
+
+int mlel_hip_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                     const mlel_tensor *multiplier, const mlel_tensor *shift, const mlel_rescale_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "rescale"));
+    MLEL_REQUIRE(attr != nullptr, MLEL_ERR_INVALID, "rescale: null attributes");
+    MLEL_TRY(check_tensor(out, "rescale out"));
+    MLEL_TRY(check_tensor(in, "rescale in"));
+    MLEL_REQUIRE(in->rank == out->rank, MLEL_ERR_INVALID, "rescale: ranks differ");
+    MLEL_TRY(check_scale_tensors(multiplier, shift, attr, out->dims[out->rank - 1]));
+    RescaleParams p;
+    MLEL_TRY(make_rescale_params(attr, in->dtype, out->dtype, nullptr, &p));
+    const int rc = try_rescale_fast(ctx, (hipStream_t)stream, out, in, multiplier, shift, attr, p);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    return rescale_generic_launch((hipStream_t)stream, out, in, multiplier, shift, attr, p);
+}
+
+int mlel_hip_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                   const mlel_clamp_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "clamp"));
+    MLEL_REQUIRE(attr != nullptr, MLEL_ERR_INVALID, "clamp: null attributes");
+    MLEL_TRY(check_supported(out, "clamp out"));
+    MLEL_TRY(check_supported(in, "clamp in"));
+    MLEL_REQUIRE(in->dtype == out->dtype && in->rank == out->rank, MLEL_ERR_INVALID, "clamp: type/rank mismatch");
+    const int rc = try_clamp_fast(ctx, (hipStream_t)stream, out, in, attr);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    return clamp_generic_launch((hipStream_t)stream, out, in, attr);
+}
+
+int mlel_hip_elementwise_binary(mlel_ctx *ctx, void *stream, int32_t op, const mlel_tensor *out,
+                                const mlel_tensor *in1, const mlel_tensor *in2, uint32_t nan_mode) {
+    MLEL_TRY(require_ctx(ctx, "elementwise_binary"));
+    MLEL_REQUIRE(op >= 0 && op < MLEL_BIN_COUNT, MLEL_ERR_INVALID, "elementwise_binary: unknown op %d", op);
+    MLEL_TRY(check_supported(out, "binary out"));
+    MLEL_TRY(check_supported(in1, "binary in1"));
+    MLEL_TRY(check_supported(in2, "binary in2"));
+    MLEL_REQUIRE(in1->dtype == in2->dtype, MLEL_ERR_INVALID, "elementwise_binary: input types differ");
+    MLEL_REQUIRE(in1->rank == out->rank && in2->rank == out->rank, MLEL_ERR_INVALID,
+                 "elementwise_binary: ranks differ");
+    const int rc = try_binary_fast(ctx, (hipStream_t)stream, op, out, in1, in2);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    return binary_generic_launch((hipStream_t)stream, op, out, in1, in2, nan_mode);
+}
+
+int mlel_hip_mul(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1, const mlel_tensor *in2,
+                 uint32_t shift) {
+    MLEL_TRY(require_ctx(ctx, "mul"));
+    MLEL_TRY(check_supported(out, "mul out"));
+    MLEL_TRY(check_supported(in1, "mul in1"));
+    MLEL_TRY(check_supported(in2, "mul in2"));
+    MLEL_REQUIRE(in1->dtype == in2->dtype, MLEL_ERR_INVALID, "mul: input types differ");
+    MLEL_REQUIRE(in1->rank == out->rank && in2->rank == out->rank, MLEL_ERR_INVALID, "mul: ranks differ");
+    MLEL_REQUIRE(shift <= 63, MLEL_ERR_INVALID, "mul: shift %u", shift);
+    return mul_generic_launch((hipStream_t)stream, out, in1, in2, shift);
+}
+
+int mlel_hip_elementwise_unary(mlel_ctx *ctx, void *stream, int32_t op, const mlel_tensor *out,
+                               const mlel_tensor *in) {
+    MLEL_TRY(require_ctx(ctx, "elementwise_unary"));
+    MLEL_REQUIRE(op >= 0 && op < MLEL_UN_COUNT, MLEL_ERR_INVALID, "elementwise_unary: unknown op %d", op);
+    MLEL_TRY(check_supported(out, "unary out"));
+    MLEL_TRY(check_supported(in, "unary in"));
+    MLEL_REQUIRE(in->dtype == out->dtype && in->rank == out->rank, MLEL_ERR_INVALID, "unary: type/rank mismatch");
+    return unary_generic_launch((hipStream_t)stream, op, out, in);
+}
+
+int mlel_hip_reduce(mlel_ctx *ctx, void *stream, int32_t op, const mlel_tensor *out, const mlel_tensor *in,
+                    uint32_t axis, uint32_t nan_mode) {
+    MLEL_TRY(require_ctx(ctx, "reduce"));
+    MLEL_REQUIRE(op >= 0 && op < MLEL_RED_COUNT, MLEL_ERR_INVALID, "reduce: unknown op %d", op);
+    MLEL_TRY(check_supported(out, "reduce out"));
+    MLEL_TRY(check_supported(in, "reduce in"));
+    MLEL_REQUIRE(in->dtype == out->dtype && in->rank == out->rank, MLEL_ERR_INVALID, "reduce: type/rank mismatch");
+    MLEL_REQUIRE((int)axis < in->rank, MLEL_ERR_INVALID, "reduce: axis %u outside rank %d", axis, in->rank);
+    if (!dt_is_float(in->dtype)) nan_mode = MLEL_NAN_PROPAGATE;  // reference: compute_graph_op.cpp:1674-1680
+    return reduce_generic_launch((hipStream_t)stream, op, out, in, axis, nan_mode);
+}
+
+int mlel_hip_avg_pool2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                        const mlel_pool2d_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "avg_pool2d"));
+    MLEL_REQUIRE(attr != nullptr, MLEL_ERR_INVALID, "avg_pool2d: null attributes");
+    MLEL_TRY(check_supported(out, "avg_pool2d out"));
+    MLEL_TRY(check_supported(in, "avg_pool2d in"));
+    MLEL_REQUIRE(out->rank == 4 && in->rank == 4 && in->dtype == out->dtype, MLEL_ERR_INVALID,
+                 "avg_pool2d: rank 4 tensors of one type");
+    MLEL_REQUIRE(attr->acc_type >= 1 && attr->acc_type <= 4, MLEL_ERR_INVALID, "Unsupported AVG_POOL2D acc type %u",
+                 attr->acc_type);
+    const int rc = try_avgpool_fast(ctx, (hipStream_t)stream, out, in, attr);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    return pool_generic_launch((hipStream_t)stream, true, out, in, attr);
+}
+
+int mlel_hip_max_pool2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                        const mlel_pool2d_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "max_pool2d"));
+    MLEL_REQUIRE(attr != nullptr, MLEL_ERR_INVALID, "max_pool2d: null attributes");
+    MLEL_TRY(check_supported(out, "max_pool2d out"));
+    MLEL_TRY(check_supported(in, "max_pool2d in"));
+    MLEL_REQUIRE(out->rank == 4 && in->rank == 4 && in->dtype == out->dtype, MLEL_ERR_INVALID,
+                 "max_pool2d: rank 4 tensors of one type");
+    return pool_generic_launch((hipStream_t)stream, false, out, in, attr);
+}
+
+int mlel_hip_table(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                   const mlel_tensor *table) {
+    MLEL_TRY(require_ctx(ctx, "table"));
+    MLEL_TRY(check_tensor(out, "table out"));
+    MLEL_TRY(check_tensor(in, "table in"));
+    MLEL_TRY(check_tensor(table, "table table"));
+    MLEL_REQUIRE(in->dtype == MLEL_I8 || in->dtype == MLEL_I16, MLEL_ERR_UNSUPPORTED, "table: input must be i8 or i16");
+    MLEL_REQUIRE(table->dtype == in->dtype && table->rank == 1, MLEL_ERR_INVALID,
+                 "table: the table is a rank-1 tensor of the input type");
+    MLEL_REQUIRE(out->dtype == (in->dtype == MLEL_I8 ? MLEL_I8 : MLEL_I32) && out->rank == in->rank, MLEL_ERR_INVALID,
+                 "table: i8 -> i8 or i16 -> i32");
+    return table_generic_launch((hipStream_t)stream, out, in, table);
+}
+
+int mlel_hip_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in) {
+    MLEL_TRY(require_ctx(ctx, "cast"));
+    MLEL_TRY(check_supported(out, "cast out"));
+    MLEL_TRY(check_supported(in, "cast in"));
+    MLEL_REQUIRE(in->rank == out->rank, MLEL_ERR_INVALID, "cast: ranks differ");
+    return cast_generic_launch((hipStream_t)stream, out, in);
+}
+
+int mlel_hip_negate(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in, int32_t input_zp,
+                    int32_t output_zp) {
+    MLEL_TRY(require_ctx(ctx, "negate"));
+    MLEL_TRY(check_supported(out, "negate out"));
+    MLEL_TRY(check_supported(in, "negate in"));
+    MLEL_REQUIRE(in->dtype == out->dtype && in->rank == out->rank, MLEL_ERR_INVALID, "negate: type/rank mismatch");
+    return negate_generic_launch((hipStream_t)stream, out, in, input_zp, output_zp);
+}
+
+int mlel_hip_reshape(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in) {
+    MLEL_TRY(require_ctx(ctx, "reshape"));
+    MLEL_TRY(check_tensor(out, "reshape out"));
+    MLEL_TRY(check_tensor(in, "reshape in"));
+    MLEL_REQUIRE(dt_size(in->dtype) == dt_size(out->dtype), MLEL_ERR_INVALID, "reshape: element size differs");
+    return move_generic_launch((hipStream_t)stream, kReshape, out, in, nullptr, 0, 0);
+}
+
+int mlel_hip_transpose(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                       const uint32_t *perms) {
+    MLEL_TRY(require_ctx(ctx, "transpose"));
+    MLEL_TRY(check_tensor(out, "transpose out"));
+    MLEL_TRY(check_tensor(in, "transpose in"));
+    MLEL_REQUIRE(perms != nullptr && in->rank == out->rank && dt_size(in->dtype) == dt_size(out->dtype),
+                 MLEL_ERR_INVALID, "transpose: bad arguments");
+    for (int i = 0; i < out->rank; i++)
+        MLEL_REQUIRE((int)perms[i] < out->rank, MLEL_ERR_INVALID, "transpose: perms[%d] = %u", i, perms[i]);
+    return move_generic_launch((hipStream_t)stream, kTranspose, out, in, perms, 0, 0);
+}
+
+int mlel_hip_concat(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis,
+                    uint32_t offset) {
+    MLEL_TRY(require_ctx(ctx, "concat"));
+    MLEL_TRY(check_tensor(out, "concat out"));
+    MLEL_TRY(check_tensor(in, "concat in"));
+    MLEL_REQUIRE(in->rank == out->rank && (int)axis < in->rank && dt_size(in->dtype) == dt_size(out->dtype),
+                 MLEL_ERR_INVALID, "concat: bad arguments");
+    return move_generic_launch((hipStream_t)stream, kConcat, out, in, nullptr, axis, offset);
+}
+
+int mlel_hip_slice(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                   const uint32_t *start) {
+    MLEL_TRY(require_ctx(ctx, "slice"));
+    MLEL_TRY(check_tensor(out, "slice out"));
+    MLEL_TRY(check_tensor(in, "slice in"));
+    MLEL_REQUIRE(start != nullptr && in->rank == out->rank && dt_size(in->dtype) == dt_size(out->dtype),
+                 MLEL_ERR_INVALID, "slice: bad arguments");
+    return move_generic_launch((hipStream_t)stream, kSlice, out, in, start, 0, 0);
+}
+
+int mlel_hip_pad(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                 const mlel_tensor *padding, double pad_const, int32_t pad_const_int) {
+    MLEL_TRY(require_ctx(ctx, "pad"));
+    MLEL_TRY(check_supported(out, "pad out"));
+    MLEL_TRY(check_supported(in, "pad in"));
+    MLEL_TRY(check_tensor(padding, "pad padding"));
+    MLEL_REQUIRE(in->rank == out->rank && in->dtype == out->dtype, MLEL_ERR_INVALID, "pad: type/rank mismatch");
+    MLEL_REQUIRE(padding->rank == 1 && padding->dtype == MLEL_I32 && padding->dims[0] >= 2 * in->rank,
+                 MLEL_ERR_INVALID, "pad: padding must be int32[2*rank]");
+    return pad_generic_launch((hipStream_t)stream, out, in, padding, pad_const, pad_const_int);
+}
+
+// ---- fused entry points ----
+
+int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                  const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv2d_attr *attr,
+                                  const mlel_epilogue *epi) {
+    MLEL_TRY(require_ctx(ctx, "conv2d_rescale_clamp"));
+    MLEL_REQUIRE(out != nullptr && attr != nullptr, MLEL_ERR_INVALID, "conv2d_rescale_clamp: null argument");
+    MLEL_TRY(check_tensor(out, "conv2d_rescale_clamp out"));
+    mlel_tensor acc_view = packed_like(out, MLEL_I32, out->ptr);  // shape carrier for validation
+    MLEL_TRY(check_conv("conv2d_rescale_clamp", &acc_view, in, weights, bias, attr));
+    FusedEpilogue fe;
+    MLEL_TRY(make_epilogue(epi, MLEL_I32, out, out->dims[3], &fe));
+    const int rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    // no specialised kernel for this layout: run the unfused operator sequence through an int32 scratch tensor
+    Scratch scratch;
+    MLEL_HIP_CHECK(hipMalloc(&scratch.ptr, (size_t)numel(out) * 4 + 16));
+    mlel_tensor acc = packed_like(out, MLEL_I32, scratch.ptr);
+    MLEL_TRY(mlel_hip_conv2d(ctx, stream, &acc, in, weights, bias, attr));
+    MLEL_TRY(run_unfused_tail(ctx, (hipStream_t)stream, out, &acc, epi));
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+int mlel_hip_matmul_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
+                            const mlel_tensor *b, const mlel_matmul_attr *attr, const mlel_epilogue *epi) {
+    MLEL_TRY(require_ctx(ctx, "matmul_rescale"));
+    MLEL_REQUIRE(attr != nullptr, MLEL_ERR_INVALID, "matmul_rescale: null attributes");
+    MLEL_TRY(check_tensor(out, "matmul_rescale out"));
+    MLEL_TRY(check_supported(a, "matmul_rescale a"));
+    MLEL_TRY(check_supported(b, "matmul_rescale b"));
+    MLEL_REQUIRE(out->rank == 3 && a->rank == 3 && b->rank == 3, MLEL_ERR_INVALID, "matmul_rescale: rank must be 3");
+    MLEL_REQUIRE(a->dtype == b->dtype && dt_is_int(a->dtype), MLEL_ERR_INVALID, "matmul_rescale: integer operands");
+    FusedEpilogue fe;
+    MLEL_TRY(make_epilogue(epi, MLEL_I32, out, out->dims[2], &fe));
+    const int rc = try_matmul_i8_mfma(ctx, (hipStream_t)stream, out, a, b, attr, &fe);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    Scratch scratch;
+    MLEL_HIP_CHECK(hipMalloc(&scratch.ptr, (size_t)numel(out) * 4 + 16));
+    mlel_tensor acc = packed_like(out, MLEL_I32, scratch.ptr);
+    MLEL_TRY(mlel_hip_matmul(ctx, stream, &acc, a, b, attr));
+    MLEL_TRY(run_unfused_tail(ctx, (hipStream_t)stream, out, &acc, epi));
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+int mlel_hip_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                  const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv2d_attr *attr,
+                                  const mlel_epilogue *epi) {
+    MLEL_TRY(require_ctx(ctx, "dwconv_rescale_clamp"));
+    MLEL_REQUIRE(out != nullptr && attr != nullptr, MLEL_ERR_INVALID, "dwconv_rescale_clamp: null argument");
+    MLEL_TRY(check_tensor(out, "dwconv_rescale_clamp out"));
+    mlel_tensor acc_view = packed_like(out, MLEL_I32, out->ptr);
+    MLEL_TRY(check_conv("dwconv_rescale_clamp", &acc_view, in, weights, bias, attr));
+    MLEL_REQUIRE(weights->dims[3] > 0, MLEL_ERR_INVALID, "dwconv_rescale_clamp: channel multiplier must be > 0");
+    FusedEpilogue fe;
+    MLEL_TRY(make_epilogue(epi, MLEL_I32, out, out->dims[3], &fe));
+    const int rc = try_dwconv_i8_fast(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    Scratch scratch;
+    MLEL_HIP_CHECK(hipMalloc(&scratch.ptr, (size_t)numel(out) * 4 + 16));
+    mlel_tensor acc = packed_like(out, MLEL_I32, scratch.ptr);
+    MLEL_TRY(mlel_hip_depthwise_conv2d(ctx, stream, &acc, in, weights, bias, attr));
+    MLEL_TRY(run_unfused_tail(ctx, (hipStream_t)stream, out, &acc, epi));
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+int mlel_hip_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1,
+                                 const mlel_epilogue *scale1, const mlel_tensor *in2, const mlel_epilogue *scale2,
+                                 const mlel_epilogue *scale_out) {
+    MLEL_TRY(require_ctx(ctx, "rescale_add_rescale"));
+    MLEL_TRY(check_tensor(out, "rescale_add_rescale out"));
+    MLEL_TRY(check_tensor(in1, "rescale_add_rescale in1"));
+    MLEL_TRY(check_tensor(in2, "rescale_add_rescale in2"));
+    MLEL_REQUIRE(same_shape(out, in1) && same_shape(out, in2), MLEL_ERR_INVALID,
+                 "rescale_add_rescale: shapes differ (no broadcast in the fused form)");
+    MLEL_REQUIRE(scale1 && scale2 && scale_out, MLEL_ERR_INVALID, "rescale_add_rescale: null scale");
+    MLEL_REQUIRE(!scale1->has_clamp && !scale2->has_clamp, MLEL_ERR_INVALID,
+                 "rescale_add_rescale: only the output stage may carry a clamp");
+    const int64_t ch = out->dims[out->rank - 1];
+    // the two input stages produce int32; build their parameters against a virtual int32 tensor
+    mlel_tensor mid = packed_like(out, MLEL_I32, out->ptr);
+    FusedEpilogue f1, f2, fo;
+    MLEL_TRY(make_epilogue(scale1, in1->dtype, &mid, ch, &f1));
+    MLEL_TRY(make_epilogue(scale2, in2->dtype, &mid, ch, &f2));
+    MLEL_TRY(make_epilogue(scale_out, MLEL_I32, out, ch, &fo));
+    return rescale_add_rescale_launch(ctx, (hipStream_t)stream, out, in1, f1, in2, f2, fo);
+}
+
+}  // extern "C"

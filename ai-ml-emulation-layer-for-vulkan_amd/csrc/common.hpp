@@ -1,0 +1,267 @@
+// Shared host/device helpers of the gfx950 TOSA backend: error reporting, tensor views passed by value to
+// kernels, the dtype table and generic element accessors with the reference's out-of-bounds semantics.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/mlel_hip.h"
+
+namespace mlel {
+
+// ---------------------------------------------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------------------------------------------
+int set_error(int code, const char *fmt, ...);
+
+#define MLEL_HIP_CHECK(expr)                                                                                           \
+    do {                                                                                                               \
+        hipError_t e_ = (expr);                                                                                        \
+        if (e_ != hipSuccess)                                                                                          \
+            return ::mlel::set_error(MLEL_ERR_DEVICE, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, \
+                                     __LINE__);                                                                        \
+    } while (0)
+
+#define MLEL_REQUIRE(cond, code, ...)                                                                                  \
+    do {                                                                                                               \
+        if (!(cond)) return ::mlel::set_error((code), __VA_ARGS__);                                                    \
+    } while (0)
+
+#define MLEL_TRY(expr)                                                                                                 \
+    do {                                                                                                               \
+        int rc_ = (expr);                                                                                              \
+        if (rc_ != 0) return rc_;                                                                                      \
+    } while (0)
+
+int check_launch(const char *what);
+
+// ---------------------------------------------------------------------------------------------------------------
+// dtype table (mirrors the format table of the reference: common/utils.cpp:119-228)
+// ---------------------------------------------------------------------------------------------------------------
+__host__ __device__ inline int dt_size(int dt) {
+    switch (dt) {
+    case MLEL_BOOL: case MLEL_I8: case MLEL_U8: case MLEL_F8E4M3: case MLEL_F8E5M2: return 1;
+    case MLEL_I16: case MLEL_U16: case MLEL_F16: case MLEL_BF16: return 2;
+    case MLEL_I32: case MLEL_U32: case MLEL_F32: return 4;
+    case MLEL_I64: case MLEL_U64: case MLEL_F64: return 8;
+    default: return 0;
+    }
+}
+__host__ __device__ inline bool dt_is_int(int dt) { return dt >= MLEL_BOOL && dt <= MLEL_U64; }
+__host__ __device__ inline bool dt_is_float(int dt) { return dt == MLEL_F16 || dt == MLEL_F32 || dt == MLEL_F64; }
+__host__ __device__ inline int64_t dt_lowest(int dt) {
+    switch (dt) {
+    case MLEL_I8: return -128;
+    case MLEL_I16: return -32768;
+    case MLEL_I32: return INT32_MIN;
+    case MLEL_I64: return INT64_MIN;
+    default: return 0;
+    }
+}
+__host__ __device__ inline int64_t dt_max(int dt) {
+    switch (dt) {
+    case MLEL_BOOL: return 1;
+    case MLEL_I8: return 127;
+    case MLEL_U8: return 255;
+    case MLEL_I16: return 32767;
+    case MLEL_U16: return 65535;
+    case MLEL_I32: return INT32_MAX;
+    case MLEL_U32: return UINT32_MAX;
+    default: return INT64_MAX;
+    }
+}
+inline int dt_unsigned_twin(int dt, bool is_unsigned) {
+    if (is_unsigned) {
+        switch (dt) {
+        case MLEL_I8: return MLEL_U8;
+        case MLEL_I16: return MLEL_U16;
+        case MLEL_I32: return MLEL_U32;
+        case MLEL_I64: return MLEL_U64;
+        default: return dt;
+        }
+    }
+    switch (dt) {
+    case MLEL_U8: return MLEL_I8;
+    case MLEL_U16: return MLEL_I16;
+    case MLEL_U32: return MLEL_I32;
+    case MLEL_U64: return MLEL_I64;
+    default: return dt;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// tensor view handed to kernels by value
+// ---------------------------------------------------------------------------------------------------------------
+struct TV {
+    char *ptr;
+    int32_t dtype;
+    int32_t rank;
+    int64_t dims[MLEL_MAX_RANK];
+    int64_t strides[MLEL_MAX_RANK];
+};
+
+inline TV make_tv(const mlel_tensor *t) {
+    TV v{};
+    v.ptr = static_cast<char *>(t->ptr);
+    v.dtype = t->dtype;
+    v.rank = t->rank;
+    for (int i = 0; i < MLEL_MAX_RANK; i++) {
+        v.dims[i] = i < t->rank ? t->dims[i] : 1;
+        v.strides[i] = i < t->rank ? t->strides[i] : 0;
+    }
+    return v;
+}
+
+int check_tensor(const mlel_tensor *t, const char *what);
+int64_t numel(const mlel_tensor *t);
+bool is_packed(const mlel_tensor *t);
+bool same_shape(const mlel_tensor *a, const mlel_tensor *b);
+
+// flat invocation index -> multi-index over `t`'s dims, row-major
+__device__ inline void unflatten(const TV &t, int64_t flat, int64_t *idx) {
+    for (int i = t.rank - 1; i >= 0; i--) {
+        const int64_t d = t.dims[i];
+        if (flat < (int64_t(1) << 31) && d < (int64_t(1) << 31)) {
+            const uint32_t f = (uint32_t)flat, dd = (uint32_t)d;
+            idx[i] = f % dd;
+            flat = f / dd;
+        } else {
+            idx[i] = flat % d;
+            flat /= d;
+        }
+    }
+}
+
+__device__ inline bool elem_off(const TV &t, const int64_t *idx, int64_t *off) {
+    int64_t o = 0;
+    for (int i = 0; i < t.rank; i++) {
+        if (idx[i] < 0 || idx[i] >= t.dims[i]) return false;
+        o += idx[i] * t.strides[i];
+    }
+    *off = o;
+    return true;
+}
+
+__device__ inline int64_t raw_ld_i(const char *p, int dt) {
+    switch (dt) {
+    case MLEL_BOOL: return *(const uint8_t *)p != 0;
+    case MLEL_I8: return *(const int8_t *)p;
+    case MLEL_U8: case MLEL_F8E4M3: case MLEL_F8E5M2: return *(const uint8_t *)p;
+    case MLEL_I16: return *(const int16_t *)p;
+    case MLEL_U16: case MLEL_F16: case MLEL_BF16: return *(const uint16_t *)p;
+    case MLEL_I32: return *(const int32_t *)p;
+    case MLEL_U32: return *(const uint32_t *)p;
+    case MLEL_I64: case MLEL_U64: return *(const int64_t *)p;
+    default: return 0;
+    }
+}
+__device__ inline void raw_st_i(char *p, int dt, int64_t v) {
+    switch (dt) {
+    case MLEL_BOOL: *(uint8_t *)p = (uint8_t)(v != 0); break;
+    case MLEL_I8: case MLEL_U8: case MLEL_F8E4M3: case MLEL_F8E5M2: *(uint8_t *)p = (uint8_t)v; break;
+    case MLEL_I16: case MLEL_U16: case MLEL_F16: case MLEL_BF16: *(uint16_t *)p = (uint16_t)v; break;
+    case MLEL_I32: case MLEL_U32: *(uint32_t *)p = (uint32_t)v; break;
+    case MLEL_I64: case MLEL_U64: *(int64_t *)p = v; break;
+    default: break;
+    }
+}
+__device__ inline float raw_ld_f(const char *p, int dt) {
+    switch (dt) {
+    case MLEL_F16: return __half2float(*(const __half *)p);
+    case MLEL_F32: return *(const float *)p;
+    case MLEL_F64: return (float)*(const double *)p;
+    default: return (float)raw_ld_i(p, dt);
+    }
+}
+__device__ inline void raw_st_f(char *p, int dt, float v) {
+    switch (dt) {
+    case MLEL_F16: *(__half *)p = __float2half_rn(v); break;
+    case MLEL_F32: *(float *)p = v; break;
+    case MLEL_F64: *(double *)p = (double)v; break;
+    default: break;
+    }
+}
+__device__ inline int64_t ld_i(const TV &t, const int64_t *idx) {
+    int64_t off;
+    if (!elem_off(t, idx, &off)) return 0;
+    return raw_ld_i(t.ptr + off, t.dtype);
+}
+__device__ inline float ld_f(const TV &t, const int64_t *idx) {
+    int64_t off;
+    if (!elem_off(t, idx, &off)) return 0.f;
+    return raw_ld_f(t.ptr + off, t.dtype);
+}
+__device__ inline void st_i(const TV &t, const int64_t *idx, int64_t v) {
+    int64_t off;
+    if (!elem_off(t, idx, &off)) return;
+    raw_st_i(t.ptr + off, t.dtype, v);
+}
+__device__ inline void st_f(const TV &t, const int64_t *idx, float v) {
+    int64_t off;
+    if (!elem_off(t, idx, &off)) return;
+    raw_st_f(t.ptr + off, t.dtype, v);
+}
+__device__ inline float rnd_f16(float v) { return __half2float(__float2half_rn(v)); }
+__device__ inline float round_to(int dt, float v) { return dt == MLEL_F16 ? rnd_f16(v) : v; }
+
+__host__ __device__ inline int64_t narrow_to(int dt, int64_t v) {
+    switch (dt) {
+    case MLEL_BOOL: return v != 0;
+    case MLEL_I8: return (int8_t)v;
+    case MLEL_U8: return (uint8_t)v;
+    case MLEL_I16: return (int16_t)v;
+    case MLEL_U16: return (uint16_t)v;
+    case MLEL_I32: return (int32_t)v;
+    case MLEL_U32: return (uint32_t)v;
+    default: return v;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// RESCALE arithmetic shared by the stand-alone kernel and the fused epilogues
+// (follows the reference shader graph/shaders/graph_op/tosa/rescale.comp:27-46)
+// ---------------------------------------------------------------------------------------------------------------
+struct RescaleParams {
+    int32_t in_zp;   // already narrowed to the (un)signed input type
+    int32_t out_zp;  // already narrowed to the (un)signed output type
+    int32_t out_lo;  // clamp range: output type range intersected with a fused CLAMP
+    int32_t out_hi;
+    int32_t double_round;  // scale32 && double_round
+    int32_t per_channel;
+    int32_t clamp_out;  // 0 for 32-bit outputs (the clamp is the identity there)
+};
+
+__device__ __forceinline__ int32_t apply_scale(int64_t value, int32_t mult, int32_t shift, bool double_round) {
+    int64_t round = shift > 0 ? (int64_t(1) << (shift - 1)) : 0;
+    if (double_round && shift > 31) round += value >= 0 ? (int64_t(1) << 30) : -(int64_t(1) << 30);
+    const uint64_t prod = (uint64_t)value * (uint64_t)(int64_t)mult + (uint64_t)round;
+    const int s = shift < 0 ? 0 : (shift > 63 ? 63 : shift);
+    return (int32_t)((int64_t)prod >> s);
+}
+
+// int32 accumulator -> requantised value, the hot form used by fused epilogues (value fits in int32)
+__device__ __forceinline__ int32_t requant_i32(int32_t acc, int32_t mult, int32_t shift, const RescaleParams &p) {
+    const int64_t value = (int64_t)acc - (int64_t)p.in_zp;
+    int32_t r = apply_scale(value, mult, shift, p.double_round != 0);
+    r = (int32_t)((uint32_t)r + (uint32_t)p.out_zp);
+    if (p.clamp_out) r = r < p.out_lo ? p.out_lo : (r > p.out_hi ? p.out_hi : r);
+    return r;
+}
+
+int make_rescale_params(const mlel_rescale_attr *attr, int in_dtype, int out_dtype, const mlel_clamp_attr *clamp,
+                        RescaleParams *out);
+int check_scale_tensors(const mlel_tensor *mult, const mlel_tensor *shift, const mlel_rescale_attr *attr,
+                        int64_t channels);
+
+inline dim3 grid_1d(int64_t work_items, int block) { return dim3((unsigned)((work_items + block - 1) / block)); }
+
+}  // namespace mlel
+
+struct mlel_ctx {
+    int device;
+    hipDeviceProp_t props;
+};

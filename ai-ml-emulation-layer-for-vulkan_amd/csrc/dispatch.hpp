@@ -1,0 +1,72 @@
+// Internal launch functions behind the C ABI: the generic one-thread-per-element path and the specialised
+// gfx950 kernels.  The `try_*` functions return 1 when they took the case, 0 when the caller must fall through to
+// the generic path, and a negative mlel_status on error.
+#pragma once
+
+#include "common.hpp"
+
+namespace mlel {
+
+enum MoveKind { kReshape = 0, kTranspose = 1, kConcat = 2, kSlice = 3 };
+
+// ---- generic path (ops_generic.hip) ----
+int conv2d_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
+                          const mlel_tensor *bias, const mlel_conv2d_attr *a);
+int dwconv_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
+                          const mlel_tensor *bias, const mlel_conv2d_attr *a);
+int matmul_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *a, const mlel_tensor *b,
+                          const mlel_matmul_attr *attr);
+int rescale_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *mult,
+                           const mlel_tensor *shift, const mlel_rescale_attr *attr, const RescaleParams &p);
+int clamp_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_clamp_attr *a);
+int binary_generic_launch(hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in1,
+                          const mlel_tensor *in2, uint32_t nan_mode);
+int mul_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in1, const mlel_tensor *in2,
+                       uint32_t shift);
+int unary_generic_launch(hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in);
+int reduce_generic_launch(hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis,
+                          uint32_t nan_mode);
+int pool_generic_launch(hipStream_t s, bool avg, const mlel_tensor *out, const mlel_tensor *in,
+                        const mlel_pool2d_attr *a);
+int table_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *table);
+int cast_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in);
+int negate_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, int32_t zi, int32_t zo);
+int move_generic_launch(hipStream_t s, int kind, const mlel_tensor *out, const mlel_tensor *in, const uint32_t *v,
+                        uint32_t axis, uint32_t offset);
+int pad_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *padding,
+                       double pad_const, int32_t pad_const_int);
+
+// ---- int8 MFMA contractions (gemm_i8.hip) ----
+// Optional fused epilogue: when `epi` is non-null the int32 accumulator is requantised (RESCALE [+CLAMP]) and
+// stored as int8/int16/int32 `out`; otherwise the int32 accumulator (plus bias) is stored.
+struct FusedEpilogue {
+    const mlel_tensor *mult;
+    const mlel_tensor *shift;
+    RescaleParams p;
+    bool scale32;
+    int in_dt;  // input storage type viewed through input_unsigned
+};
+int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                       const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
+                       const FusedEpilogue *epi);
+int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
+                       const mlel_tensor *b, const mlel_matmul_attr *attr, const FusedEpilogue *epi);
+
+// ---- bandwidth-bound specialisations (ops_fast.hip) ----
+int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                       const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
+                       const FusedEpilogue *epi);
+int try_rescale_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                     const mlel_tensor *mult, const mlel_tensor *shift, const mlel_rescale_attr *attr,
+                     const RescaleParams &p);
+int try_clamp_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                   const mlel_clamp_attr *a);
+int try_binary_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in1,
+                    const mlel_tensor *in2);
+int try_avgpool_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                     const mlel_pool2d_attr *a);
+int rescale_add_rescale_launch(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in1,
+                               const FusedEpilogue &s1, const mlel_tensor *in2, const FusedEpilogue &s2,
+                               const FusedEpilogue &so);
+
+}  // namespace mlel

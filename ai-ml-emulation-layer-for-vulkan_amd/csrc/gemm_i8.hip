@@ -1,0 +1,609 @@
+// int8 x int8 -> int32 contractions on the gfx950 matrix cores: CONV2D (implicit GEMM over NHWC input and OHWI
+// weights) and MATMUL, with the zero-point handling of the reference shaders and an optional fused
+// RESCALE(+CLAMP) epilogue.
+//
+// What is computed.  out[m][n] = sum_k (X[m][k] - zx) * (Wt[n][k] - zw) + bias[n], where
+//   CONV2D : m = (image, oy, ox), n = oc, k = (ky, kx, ic); X[m][k] is the input element under tap (ky,kx) or, for
+//            a tap that falls into the padding, the value zx itself so that the tap contributes nothing
+//            (the reference skips such taps: conv2d.comp:64);
+//   MATMUL : per batch, X = A[m][k], Wt[n][k] = B[k][n] (B is stored K-major and transposed while it is staged
+//            into LDS) (reference: matmul.comp:30-73).
+// The sum is expanded as  sum X*Wt - zw*sum_k X - zx*sum_k Wt + K*zx*zw  so that the matrix cores multiply the raw
+// int8 operands (X - zx does not fit in int8).  All arithmetic is int32 with wraparound, as in the shaders, so the
+// regrouping is exact.
+//
+// Kernel shape.  256 threads = 4 wavefronts of 64.  A block owns a BM x BN output tile; K is walked in steps of
+// 64 bytes through two LDS buffers (global loads of step i+1 are in flight while step i is multiplied).  Each
+// wavefront owns a (32*TM) x (32*TN) sub-tile and issues v_mfma_i32_32x32x32_i8 with the weights as the row
+// operand and the activations as the column operand: a lane then holds, for ONE output position m, groups of four
+// consecutive output channels n, which is the byte order of the NHWC / [M][N] output, so requantised results are
+// packed four to a dword and stored without a transpose.  Per-channel epilogue constants live in LDS.
+#include "common.hpp"
+#include "dispatch.hpp"
+
+namespace mlel {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 64;            // bytes of K per step
+constexpr int PITCH = BK + 16;    // LDS row pitch: 80 B keeps 16-lane groups of 128-bit reads on distinct banks
+constexpr int NTHREADS = 256;
+
+struct GemmArgs {
+    // problem
+    int32_t M, N, K, batches;
+    // X operand (rows m): conv gather over NHWC; the plain [M][K] case is the 1x1 conv with H = W = 1
+    const int8_t *x;
+    int64_t x_batch, x_sn, x_sy, x_sx;  // byte strides
+    int32_t H, W, IC, OHW, OW, KH, KW, sy, sx, dy, dx, pad_t, pad_l;
+    int32_t plain;  // 1: m indexes rows of pitch x_sx directly
+    int32_t xch;    // bytes per aligned global load of X: 16, 4 or 1
+    // W operand (rows n)
+    const int8_t *w;
+    int64_t w_batch, ldw;
+    int32_t w_kmajor;  // 0: [N][K] rows of pitch ldw; 1: [K][N] rows of pitch ldw
+    int32_t wch;       // bytes per aligned global load of W: 16, 4 or 1
+    int32_t zx, zw;
+    // bias (int32, length 1 or N) and output
+    const int32_t *bias;
+    int32_t bias_len;
+    char *out;
+    int64_t out_batch, ldo;  // ldo in elements
+    int32_t out_size;        // bytes per output element: 1, 2 or 4
+    int32_t out_vec_ok;      // four consecutive channels may be stored as one aligned unit
+    // fused epilogue
+    int32_t fused;
+    const char *mult;  // int32 or int16 per channel (or one)
+    const int8_t *shift;
+    int32_t mult16;
+    RescaleParams rp;
+    // launch geometry
+    int32_t tiles_m, tiles_n, total_tiles, chunk;
+};
+
+struct ChanParams {  // per output channel, in LDS
+    int32_t bias_adj;
+    int32_t mult;
+    int32_t shift;
+    int32_t pad;
+};
+
+struct RowState {
+    const int8_t *base;
+    int32_t iy0, ix0;
+    int32_t valid;
+};
+
+struct KState {
+    int32_t ky, kx, ic;
+};
+
+__device__ __forceinline__ void kstate_advance(KState &s, int step, int IC, int KW) {
+    s.ic += step;
+    while (s.ic >= IC) {
+        s.ic -= IC;
+        if (++s.kx == KW) {
+            s.kx = 0;
+            ++s.ky;
+        }
+    }
+}
+
+__device__ __forceinline__ uint32_t splat8(int v) { return (uint32_t)(uint8_t)v * 0x01010101u; }
+
+// One 16-byte piece of row `r` of the X operand starting at k-position `s`.
+__device__ __forceinline__ uint4 load_x_chunk(const GemmArgs &g, const RowState &r, KState s) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (!r.valid) return v;
+    if (g.xch == 16) {
+        if (s.ky >= g.KH) return v;
+        const int y = r.iy0 + s.ky * g.dy, x = r.ix0 + s.kx * g.dx;
+        if ((unsigned)y >= (unsigned)g.H || (unsigned)x >= (unsigned)g.W) {
+            const uint32_t z = splat8(g.zx);
+            return make_uint4(z, z, z, z);
+        }
+        return *reinterpret_cast<const uint4 *>(r.base + (int64_t)y * g.x_sy + (int64_t)x * g.x_sx + s.ic);
+    }
+    uint32_t d[4];
+    if (g.xch == 4) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t val = 0;
+            if (s.ky < g.KH) {
+                const int y = r.iy0 + s.ky * g.dy, x = r.ix0 + s.kx * g.dx;
+                if ((unsigned)y >= (unsigned)g.H || (unsigned)x >= (unsigned)g.W)
+                    val = splat8(g.zx);
+                else
+                    val = *reinterpret_cast<const uint32_t *>(r.base + (int64_t)y * g.x_sy + (int64_t)x * g.x_sx +
+                                                              s.ic);
+            }
+            d[j] = val;
+            kstate_advance(s, 4, g.IC, g.KW);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t val = 0;
+            for (int b = 0; b < 4; b++) {
+                uint32_t byte = 0;
+                if (s.ky < g.KH) {
+                    const int y = r.iy0 + s.ky * g.dy, x = r.ix0 + s.kx * g.dx;
+                    if ((unsigned)y >= (unsigned)g.H || (unsigned)x >= (unsigned)g.W)
+                        byte = (uint8_t)g.zx;
+                    else
+                        byte = (uint8_t)r.base[(int64_t)y * g.x_sy + (int64_t)x * g.x_sx + s.ic];
+                }
+                val |= byte << (8 * b);
+                kstate_advance(s, 1, g.IC, g.KW);
+            }
+            d[j] = val;
+        }
+    }
+    return make_uint4(d[0], d[1], d[2], d[3]);
+}
+
+// One 16-byte piece of row n of the W operand stored as [N][K].
+__device__ __forceinline__ uint4 load_w_chunk(const GemmArgs &g, const int8_t *wb, int n, int k) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (n >= g.N || k >= g.K) return v;
+    const int8_t *p = wb + (int64_t)n * g.ldw + k;
+    if (g.wch == 16) return *reinterpret_cast<const uint4 *>(p);
+    uint32_t d[4];
+    if (g.wch == 4) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) d[j] = (k + 4 * j < g.K) ? *reinterpret_cast<const uint32_t *>(p + 4 * j) : 0u;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t val = 0;
+            for (int b = 0; b < 4; b++)
+                if (k + 4 * j + b < g.K) val |= (uint32_t)(uint8_t)p[4 * j + b] << (8 * b);
+            d[j] = val;
+        }
+    }
+    return make_uint4(d[0], d[1], d[2], d[3]);
+}
+
+// A 4(k) x 4(n) byte block of the K-major W operand, returned transposed: d[j] = the four k-bytes of column n+j.
+__device__ __forceinline__ uint4 load_w_block_kmajor(const GemmArgs &g, const int8_t *wb, int n, int k) {
+    uint32_t r[4] = {0, 0, 0, 0};
+    if (n < g.N) {
+        if (g.wch >= 4) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (k + i < g.K) r[i] = *reinterpret_cast<const uint32_t *>(wb + (int64_t)(k + i) * g.ldw + n);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (k + i < g.K)
+                    for (int b = 0; b < 4; b++)
+                        if (n + b < g.N) r[i] |= (uint32_t)(uint8_t)wb[(int64_t)(k + i) * g.ldw + n + b] << (8 * b);
+        }
+    }
+    // 4x4 byte transpose with v_perm_b32 (selector bytes 0-3 pick from the second source, 4-7 from the first)
+    const uint32_t t0 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u);
+    const uint32_t t1 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);
+    const uint32_t t2 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+    return make_uint4(__builtin_amdgcn_perm(t2, t0, 0x05040100u), __builtin_amdgcn_perm(t2, t0, 0x07060302u),
+                      __builtin_amdgcn_perm(t3, t1, 0x05040100u), __builtin_amdgcn_perm(t3, t1, 0x07060302u));
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wavefront sub-tile
+    constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 MFMA tiles per wavefront
+    constexpr int XROWS = BM / 64;                       // X rows per thread (4 chunks of 16 B per row)
+    constexpr int WCHUNKS = (BN * 4 + NTHREADS - 1) / NTHREADS;
+    static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per block");
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wavefront tile is a multiple of the 32x32 MFMA tile");
+
+    extern __shared__ __align__(16) char smem[];
+    char *xs = smem;                             // [2][BM][PITCH]
+    char *ws = smem + 2 * BM * PITCH;            // [2][BN][PITCH]
+    ChanParams *cp = reinterpret_cast<ChanParams *>(smem + 2 * (BM + BN) * PITCH);  // [BN]
+
+    // ---- XCD-aware tile assignment: consecutive block ids land on different XCDs (8 of them, each with its own
+    // L2), so block b is given tile (b % 8) * chunk + b / 8: tiles that share operands stay on one XCD.
+    const int lin = (int)(blockIdx.x % 8) * g.chunk + (int)(blockIdx.x / 8);
+    if (lin >= g.total_tiles) return;
+    const int tiles_per_batch = g.tiles_m * g.tiles_n;
+    const int batch = lin / tiles_per_batch;
+    const int t_in = lin - batch * tiles_per_batch;
+    const int tile_m = t_in / g.tiles_n, tile_n = t_in - tile_m * g.tiles_n;
+    const int m_base = tile_m * BM, n_base = tile_n * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+
+    const int8_t *xb = g.x + (int64_t)batch * g.x_batch;
+    const int8_t *wb = g.w + (int64_t)batch * g.w_batch;
+
+    // ---- per-channel epilogue constants
+    for (int n = tid; n < BN; n += NTHREADS) {
+        ChanParams c{0, 0, 0, 0};
+        const int gn = n_base + n;
+        if (gn < g.N) {
+            c.bias_adj = g.bias ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
+            if (g.fused) {
+                const int ci = g.rp.per_channel ? gn : 0;
+                c.mult = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
+                                  : reinterpret_cast<const int32_t *>(g.mult)[ci];
+                c.shift = (int32_t)g.shift[ci];
+            }
+        }
+        cp[n] = c;
+    }
+
+    // ---- loader state
+    RowState rows[XROWS];
+    const int x_kc = tid & 3;  // which 16-byte piece of the 64-byte K step this thread stages
+#pragma unroll
+    for (int i = 0; i < XROWS; i++) {
+        const int m = m_base + (tid >> 2) + 64 * i;
+        RowState r{xb, 0, 0, m < g.M};
+        if (r.valid) {
+            if (g.plain) {
+                r.base = xb + (int64_t)m * g.x_sx;
+            } else {
+                const int img = m / g.OHW, rem = m - img * g.OHW;
+                const int oy = rem / g.OW, ox = rem - oy * g.OW;
+                r.base = xb + (int64_t)img * g.x_sn;
+                r.iy0 = oy * g.sy - g.pad_t;
+                r.ix0 = ox * g.sx - g.pad_l;
+            }
+        }
+        rows[i] = r;
+    }
+    KState ks{0, 0, 0};
+    kstate_advance(ks, x_kc * 16, g.IC, g.KW);
+
+    uint4 xr[XROWS], wr[WCHUNKS];
+    auto prefetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < XROWS; i++) xr[i] = load_x_chunk(g, rows[i], ks);
+        kstate_advance(ks, BK, g.IC, g.KW);
+        if (!g.w_kmajor) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                if (c < BN * 4) wr[i] = load_w_chunk(g, wb, n_base + (c >> 2), k0 + (c & 3) * 16);
+            }
+        } else {
+            // (BK/4) x (BN/4) blocks of 4x4 bytes; consecutive lanes take consecutive column groups
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                if (c < BN * 4) wr[i] = load_w_block_kmajor(g, wb, n_base + (c % (BN / 4)) * 4, k0 + (c / (BN / 4)) * 4);
+            }
+        }
+    };
+    auto stage = [&](int buf) {
+        char *xd = xs + buf * BM * PITCH;
+        char *wd = ws + buf * BN * PITCH;
+#pragma unroll
+        for (int i = 0; i < XROWS; i++)
+            *reinterpret_cast<uint4 *>(xd + ((tid >> 2) + 64 * i) * PITCH + x_kc * 16) = xr[i];
+        if (!g.w_kmajor) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                if (c < BN * 4) *reinterpret_cast<uint4 *>(wd + (c >> 2) * PITCH + (c & 3) * 16) = wr[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                if (c < BN * 4) {
+                    const int nl = (c % (BN / 4)) * 4, kl = (c / (BN / 4)) * 4;
+                    *reinterpret_cast<uint32_t *>(wd + (nl + 0) * PITCH + kl) = wr[i].x;
+                    *reinterpret_cast<uint32_t *>(wd + (nl + 1) * PITCH + kl) = wr[i].y;
+                    *reinterpret_cast<uint32_t *>(wd + (nl + 2) * PITCH + kl) = wr[i].z;
+                    *reinterpret_cast<uint32_t *>(wd + (nl + 3) * PITCH + kl) = wr[i].w;
+                }
+            }
+        }
+    };
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+    int32_t xsum[TM], wsum[TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++) xsum[i] = 0;
+#pragma unroll
+    for (int j = 0; j < TN; j++) wsum[j] = 0;
+    const bool need_xsum = g.zw != 0, need_wsum = g.zx != 0;
+
+    const int nk = (g.K + BK - 1) / BK;
+    prefetch(0);
+    stage(0);
+    __syncthreads();
+    for (int step = 0; step < nk; step++) {
+        const int cur = step & 1;
+        if (step + 1 < nk) prefetch((step + 1) * BK);
+        const char *xd = xs + cur * BM * PITCH + (wave_m * WM + (lane & 31)) * PITCH + (lane >> 5) * 16;
+        const char *wd = ws + cur * BN * PITCH + (wave_n * WN + (lane & 31)) * PITCH + (lane >> 5) * 16;
+#pragma unroll
+        for (int kk = 0; kk < BK / 32; kk++) {
+            v4i xf[TM], wf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) xf[i] = *reinterpret_cast<const v4i *>(xd + i * 32 * PITCH + kk * 32);
+#pragma unroll
+            for (int j = 0; j < TN; j++) wf[j] = *reinterpret_cast<const v4i *>(wd + j * 32 * PITCH + kk * 32);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
+            if (need_xsum) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) xsum[i] = __builtin_amdgcn_sdot4(xf[i][q], 0x01010101, xsum[i], false);
+            }
+            if (need_wsum) {
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) wsum[j] = __builtin_amdgcn_sdot4(wf[j][q], 0x01010101, wsum[j], false);
+            }
+        }
+        if (step + 1 < nk) stage(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- fold the zero-point terms that depend on the channel only into the per-channel bias
+    if (need_wsum && wave_m == 0) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int32_t s = wsum[j] + __shfl_xor(wsum[j], 32);
+            if (lane < 32) {
+                const int n = wave_n * WN + j * 32 + lane;
+                cp[n].bias_adj += -g.zx * s + g.K * g.zx * g.zw;
+            }
+        }
+    }
+    if (need_xsum) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) xsum[i] = (xsum[i] + __shfl_xor(xsum[i], 32)) * g.zw;
+    }
+    __syncthreads();
+
+    // ---- epilogue: lane holds output position m = lane % 32 of each tile row and, per register group q, the four
+    // channels n0 .. n0+3 with n0 = 8q + 4 * (lane / 32)
+    char *ob = g.out + (int64_t)batch * g.out_batch;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
+        if (m >= g.M) continue;
+        const int32_t xcorr = need_xsum ? xsum[i] : 0;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int nl = wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+                const int n0 = n_base + nl;
+                if (n0 >= g.N) continue;
+                int32_t v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const ChanParams c = cp[nl + e];
+                    int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)c.bias_adj - (uint32_t)xcorr);
+                    if (g.fused) a = requant_i32(a, c.mult, c.shift, g.rp);
+                    v[e] = a;
+                }
+                const int64_t off = (int64_t)m * g.ldo + n0;
+                if (g.out_vec_ok && n0 + 3 < g.N) {
+                    if (g.out_size == 1) {
+                        const uint32_t packed = (uint32_t)(uint8_t)v[0] | ((uint32_t)(uint8_t)v[1] << 8) |
+                                                ((uint32_t)(uint8_t)v[2] << 16) | ((uint32_t)(uint8_t)v[3] << 24);
+                        *reinterpret_cast<uint32_t *>(ob + off) = packed;
+                    } else if (g.out_size == 2) {
+                        const uint32_t lo = (uint32_t)(uint16_t)v[0] | ((uint32_t)(uint16_t)v[1] << 16);
+                        const uint32_t hi = (uint32_t)(uint16_t)v[2] | ((uint32_t)(uint16_t)v[3] << 16);
+                        *reinterpret_cast<uint2 *>(ob + off * 2) = make_uint2(lo, hi);
+                    } else {
+                        *reinterpret_cast<int4 *>(ob + off * 4) = make_int4(v[0], v[1], v[2], v[3]);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (n0 + e >= g.N) break;
+                        if (g.out_size == 1)
+                            *reinterpret_cast<int8_t *>(ob + off + e) = (int8_t)v[e];
+                        else if (g.out_size == 2)
+                            *reinterpret_cast<int16_t *>(ob + (off + e) * 2) = (int16_t)v[e];
+                        else
+                            *reinterpret_cast<int32_t *>(ob + (off + e) * 4) = v[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN>
+constexpr size_t smem_bytes() {
+    return (size_t)2 * (BM + BN) * PITCH + (size_t)BN * sizeof(ChanParams);
+}
+
+int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
+    (void)ctx;
+    // tile choice: least padded channel extent, larger tile on ties
+    const int bn_opts[3] = {128, 64, 32};
+    int best = 0;
+    int64_t best_pad = INT64_MAX;
+    for (int i = 0; i < 3; i++) {
+        const int64_t padded = (int64_t)((g.N + bn_opts[i] - 1) / bn_opts[i]) * bn_opts[i];
+        if (padded < best_pad) {
+            best_pad = padded;
+            best = i;
+        }
+    }
+    const int BN = bn_opts[best];
+    const int BM = BN == 128 ? 128 : 256;
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    const int64_t total = (int64_t)g.tiles_m * g.tiles_n * g.batches;
+    MLEL_REQUIRE(total > 0 && total < (int64_t(1) << 30), MLEL_ERR_LIMIT, "contraction: %lld tiles", (long long)total);
+    g.total_tiles = (int)total;
+    g.chunk = (int)((total + 7) / 8);
+    const dim3 grid((unsigned)(g.chunk * 8));
+    if (BN == 128) {
+        const size_t sm = smem_bytes<128, 128>();
+        gemm_i8_kernel<128, 128, 2, 2><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    } else if (BN == 64) {
+        const size_t sm = smem_bytes<256, 64>();
+        gemm_i8_kernel<256, 64, 4, 1><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    } else {
+        const size_t sm = smem_bytes<256, 32>();
+        gemm_i8_kernel<256, 32, 4, 1><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    }
+    return check_launch("int8 contraction");
+}
+
+int align_of(const void *p, int64_t a, int64_t b = 16, int64_t c = 16, int64_t d = 16) {
+    auto ok = [&](int64_t n) { return ((uintptr_t)p % n) == 0 && a % n == 0 && b % n == 0 && c % n == 0 && d % n == 0; };
+    return ok(16) ? 16 : (ok(4) ? 4 : 1);
+}
+
+int fill_epilogue(GemmArgs &g, const mlel_tensor *out, const FusedEpilogue *epi) {
+    g.out = static_cast<char *>(out->ptr);
+    g.out_size = dt_size(out->dtype);
+    g.fused = epi != nullptr;
+    if (epi) {
+        g.mult = static_cast<const char *>(epi->mult->ptr);
+        g.shift = static_cast<const int8_t *>(epi->shift->ptr);
+        g.mult16 = epi->scale32 ? 0 : 1;
+        g.rp = epi->p;
+    }
+    const int64_t unit = 4 * g.out_size;
+    g.out_vec_ok = (g.N % 4 == 0) && ((g.ldo * g.out_size) % unit == 0) && ((uintptr_t)out->ptr % unit == 0) &&
+                   ((g.out_batch) % unit == 0);
+    return 0;
+}
+
+bool packed_tail(const mlel_tensor *t, int from) {
+    // dims[from..] are laid out contiguously (row-major, no gaps)
+    int64_t s = dt_size(t->dtype);
+    for (int i = t->rank - 1; i >= from; i--) {
+        if (t->strides[i] != s) return false;
+        s *= t->dims[i];
+    }
+    return true;
+}
+
+}  // namespace
+
+int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                       const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
+                       const FusedEpilogue *epi) {
+    if (in->dtype != MLEL_I8 || w->dtype != MLEL_I8 || bias->dtype != MLEL_I32 || a->acc_type != MLEL_ACC_I32) return 0;
+    if (epi == nullptr && out->dtype != MLEL_I32) return 0;
+    if (epi != nullptr && dt_size(out->dtype) > 4) return 0;
+    const int64_t N = out->dims[0], OH = out->dims[1], OW = out->dims[2], OC = out->dims[3];
+    const int64_t H = in->dims[1], W = in->dims[2], IC = in->dims[3];
+    const int64_t KH = w->dims[1], KW = w->dims[2];
+    // shapes the kernel's indexing assumes; anything else goes to the generic path
+    if (in->dims[0] < N || w->dims[0] < OC || w->dims[3] != IC || IC <= 0 || KH <= 0 || KW <= 0) return 0;
+    if (!(bias->dims[0] == 1 || bias->dims[0] >= OC) || bias->strides[0] != 4) return 0;
+    if (in->strides[3] != 1 || !packed_tail(w, 1) || !is_packed(out)) return 0;
+    if (a->stride[0] <= 0 || a->stride[1] <= 0 || a->dilation[0] <= 0 || a->dilation[1] <= 0) return 0;
+    const int64_t M = N * OH * OW, K = KH * KW * IC;
+    if (M <= 0 || OC <= 0) return 1;  // nothing to do
+    if (M >= (int64_t(1) << 31) || K >= (int64_t(1) << 30) || OC >= (int64_t(1) << 30)) return 0;
+    if (H >= (1 << 30) || W >= (1 << 30)) return 0;
+
+    GemmArgs g{};
+    g.M = (int)M;
+    g.N = (int)OC;
+    g.K = (int)K;
+    g.batches = 1;
+    g.x = static_cast<const int8_t *>(in->ptr);
+    g.x_sn = in->strides[0];
+    g.x_sy = in->strides[1];
+    g.x_sx = in->strides[2];
+    g.H = (int)H;
+    g.W = (int)W;
+    g.IC = (int)IC;
+    g.OHW = (int)(OH * OW);
+    g.OW = (int)OW;
+    g.KH = (int)KH;
+    g.KW = (int)KW;
+    g.sy = a->stride[0];
+    g.sx = a->stride[1];
+    g.dy = a->dilation[0];
+    g.dx = a->dilation[1];
+    g.pad_t = a->pad[0];
+    g.pad_l = a->pad[2];
+    g.plain = 0;
+    g.xch = align_of(in->ptr, IC, in->strides[0], in->strides[1], in->strides[2]);
+    g.w = static_cast<const int8_t *>(w->ptr);
+    g.ldw = w->strides[0];
+    g.w_kmajor = 0;
+    g.wch = align_of(w->ptr, K, w->strides[0]);
+    g.zx = a->input_zp;
+    g.zw = a->weight_zp;
+    g.bias = static_cast<const int32_t *>(bias->ptr);
+    g.bias_len = (int)bias->dims[0];
+    g.ldo = OC;
+    g.out_batch = 0;
+    MLEL_TRY(fill_epilogue(g, out, epi));
+    MLEL_TRY(launch_gemm(ctx, s, g));
+    return 1;
+}
+
+int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *A,
+                       const mlel_tensor *B, const mlel_matmul_attr *attr, const FusedEpilogue *epi) {
+    if (A->dtype != MLEL_I8 || B->dtype != MLEL_I8) return 0;
+    if (epi == nullptr && out->dtype != MLEL_I32) return 0;
+    if (epi != nullptr && dt_size(out->dtype) > 4) return 0;
+    const int64_t NB = out->dims[0], M = out->dims[1], N = out->dims[2], K = A->dims[2];
+    if (A->dims[0] < NB || B->dims[0] < NB || A->dims[1] < M || B->dims[1] != K || B->dims[2] < N) return 0;
+    if (A->strides[2] != 1 || B->strides[2] != 1 || !is_packed(out)) return 0;
+    if (M <= 0 || N <= 0 || NB <= 0) return 1;
+    if (K <= 0) return 0;
+    if (M >= (int64_t(1) << 30) || N >= (int64_t(1) << 30) || K >= (int64_t(1) << 30) || NB >= (1 << 20)) return 0;
+
+    GemmArgs g{};
+    g.M = (int)M;
+    g.N = (int)N;
+    g.K = (int)K;
+    g.batches = (int)NB;
+    g.x = static_cast<const int8_t *>(A->ptr);
+    g.x_batch = A->strides[0];
+    g.x_sx = A->strides[1];
+    g.H = 1;
+    g.W = 1;
+    g.IC = (int)K;
+    g.OHW = 1;
+    g.OW = 1;
+    g.KH = 1;
+    g.KW = 1;
+    g.sy = g.sx = g.dy = g.dx = 1;
+    g.plain = 1;
+    g.xch = align_of(A->ptr, K, A->strides[0], A->strides[1]);
+    g.w = static_cast<const int8_t *>(B->ptr);
+    g.w_batch = B->strides[0];
+    g.ldw = B->strides[1];
+    g.w_kmajor = 1;
+    g.wch = align_of(B->ptr, N, B->strides[0], B->strides[1]) >= 4 ? 4 : 1;
+    g.zx = attr->a_zp;
+    g.zw = attr->b_zp;
+    g.bias = nullptr;
+    g.bias_len = 0;
+    g.ldo = N;
+    g.out_batch = out->strides[0];
+    MLEL_TRY(fill_epilogue(g, out, epi));
+    MLEL_TRY(launch_gemm(ctx, s, g));
+    return 1;
+}
+
+}  // namespace mlel

@@ -1,0 +1,208 @@
+"""Helpers for the GPU parity tests: run one operator through the C ABI on numpy inputs."""
+import ctypes as C
+import importlib
+
+import numpy as np
+
+abi = importlib.import_module("ai-ml-emulation-layer-for-vulkan_amd.abi")
+hb = importlib.import_module("ai-ml-emulation-layer-for-vulkan_amd.hip_backend")
+
+
+def gpu_available():
+    try:
+        return hb.device_count() > 0
+    except Exception:
+        return False
+
+
+class Runner:
+    """Uploads numpy inputs, runs one C-ABI entry point, downloads the output; frees everything after."""
+
+    def __init__(self, dev):
+        self.dev = dev
+        self.live = []
+
+    def put(self, arr, dtype=None, strides=None):
+        t = self.dev.from_numpy(np.asarray(arr), dtype, strides)
+        self.live.append(t)
+        return t
+
+    def new(self, dtype, shape, strides=None):
+        t = self.dev.tensor(dtype, shape, strides)
+        self.live.append(t)
+        return t
+
+    def done(self):
+        for t in self.live:
+            t.free()
+        self.live = []
+
+    # ---- operators -------------------------------------------------------------------------------------------
+    def conv2d(self, x, w, b, out_shape, out_dtype, attr, depthwise=False, epilogue=None, x_strides=None):
+        tx, tw, tb = self.put(x, strides=x_strides), self.put(w), self.put(b)
+        to = self.new(out_dtype, out_shape)
+        name = "depthwise_conv2d" if depthwise else "conv2d"
+        if epilogue is None:
+            self.dev.op(name, to.ref, tx.ref, tw.ref, tb.ref, C.byref(attr))
+        else:
+            e = self._epi(*epilogue)
+            self.dev.op("dwconv_rescale_clamp" if depthwise else "conv2d_rescale_clamp", to.ref, tx.ref, tw.ref,
+                        tb.ref, C.byref(attr), C.byref(e))
+        r = to.download()
+        self.done()
+        return r
+
+    def _epi(self, mult, shift, rattr, clamp):
+        return self.dev.epilogue(self.put(mult), self.put(shift), rattr, clamp)
+
+    def matmul(self, a, b, out_dtype, a_zp=0, b_zp=0, epilogue=None):
+        ta, tb = self.put(a), self.put(b)
+        to = self.new(out_dtype, (a.shape[0], a.shape[1], b.shape[2]))
+        attr = abi.MatmulAttr(int(a_zp), int(b_zp))
+        if epilogue is None:
+            self.dev.op("matmul", to.ref, ta.ref, tb.ref, C.byref(attr))
+        else:
+            e = self._epi(*epilogue)
+            self.dev.op("matmul_rescale", to.ref, ta.ref, tb.ref, C.byref(attr), C.byref(e))
+        r = to.download()
+        self.done()
+        return r
+
+    def rescale(self, x, mult, shift, out_dtype, attr, in_dtype=None):
+        tx, tm, ts = self.put(x, in_dtype), self.put(mult), self.put(shift)
+        to = self.new(out_dtype, x.shape)
+        self.dev.op("rescale", to.ref, tx.ref, tm.ref, ts.ref, C.byref(attr))
+        r = to.download()
+        self.done()
+        return r
+
+    def clamp(self, x, mn, mx, nan_mode=abi.NAN_PROPAGATE):
+        tx = self.put(x)
+        to = self.new(tx.dtype, x.shape)
+        self.dev.op("clamp", to.ref, tx.ref, C.byref(abi.ClampAttr(float(mn), float(mx), int(nan_mode))))
+        r = to.download()
+        self.done()
+        return r
+
+    def binary(self, op, a, b, out_shape, out_dtype, nan_mode=abi.NAN_PROPAGATE):
+        ta, tb = self.put(a), self.put(b)
+        to = self.new(out_dtype, out_shape)
+        self.dev.op("elementwise_binary", abi.BIN[op], to.ref, ta.ref, tb.ref, int(nan_mode))
+        r = to.download()
+        self.done()
+        return r
+
+    def mul(self, a, b, out_shape, out_dtype, shift=0):
+        ta, tb = self.put(a), self.put(b)
+        to = self.new(out_dtype, out_shape)
+        self.dev.op("mul", to.ref, ta.ref, tb.ref, int(shift))
+        r = to.download()
+        self.done()
+        return r
+
+    def unary(self, op, x):
+        tx = self.put(x)
+        to = self.new(tx.dtype, x.shape)
+        self.dev.op("elementwise_unary", abi.UN[op], to.ref, tx.ref)
+        r = to.download()
+        self.done()
+        return r
+
+    def reduce(self, op, x, axis, nan_mode=abi.NAN_PROPAGATE):
+        tx = self.put(x)
+        shape = list(x.shape)
+        shape[axis] = 1
+        to = self.new(tx.dtype, shape)
+        self.dev.op("reduce", abi.RED[op], to.ref, tx.ref, int(axis), int(nan_mode))
+        r = to.download()
+        self.done()
+        return r
+
+    def pool(self, kind, x, out_shape, attr):
+        tx = self.put(x)
+        to = self.new(tx.dtype, out_shape)
+        self.dev.op(kind, to.ref, tx.ref, C.byref(attr))
+        r = to.download()
+        self.done()
+        return r
+
+    def table(self, x, tab, out_dtype):
+        tx, tt = self.put(x), self.put(tab)
+        to = self.new(out_dtype, x.shape)
+        self.dev.op("table", to.ref, tx.ref, tt.ref)
+        r = to.download()
+        self.done()
+        return r
+
+    def cast(self, x, out_dtype):
+        tx = self.put(x)
+        to = self.new(out_dtype, x.shape)
+        self.dev.op("cast", to.ref, tx.ref)
+        r = to.download()
+        self.done()
+        return r
+
+    def negate(self, x, zi=0, zo=0):
+        tx = self.put(x)
+        to = self.new(tx.dtype, x.shape)
+        self.dev.op("negate", to.ref, tx.ref, int(zi), int(zo))
+        r = to.download()
+        self.done()
+        return r
+
+    def reshape(self, x, out_shape):
+        tx = self.put(x)
+        to = self.new(tx.dtype, out_shape)
+        self.dev.op("reshape", to.ref, tx.ref)
+        r = to.download()
+        self.done()
+        return r
+
+    def transpose(self, x, perms):
+        tx = self.put(x)
+        to = self.new(tx.dtype, [x.shape[p] for p in perms])
+        arr = (C.c_uint32 * abi.MAX_RANK)(*[int(p) for p in perms])
+        self.dev.op("transpose", to.ref, tx.ref, arr)
+        r = to.download()
+        self.done()
+        return r
+
+    def concat(self, inputs, axis):
+        shape = list(inputs[0].shape)
+        shape[axis] = sum(i.shape[axis] for i in inputs)
+        to = self.new(abi.dtype_of_numpy(inputs[0].dtype), shape)
+        off = 0
+        for i in inputs:
+            ti = self.put(i)
+            self.dev.op("concat", to.ref, ti.ref, int(axis), int(off))
+            off += i.shape[axis]
+        r = to.download()
+        self.done()
+        return r
+
+    def slice_(self, x, start, size):
+        tx = self.put(x)
+        to = self.new(tx.dtype, size)
+        arr = (C.c_uint32 * abi.MAX_RANK)(*[int(p) for p in start])
+        self.dev.op("slice", to.ref, tx.ref, arr)
+        r = to.download()
+        self.done()
+        return r
+
+    def pad(self, x, padding, out_shape, pad_const=0.0, pad_const_int=0):
+        tx = self.put(x)
+        tp = self.put(np.ascontiguousarray(padding, dtype=np.int32).reshape(-1))
+        to = self.new(tx.dtype, out_shape)
+        self.dev.op("pad", to.ref, tx.ref, tp.ref, float(pad_const), int(pad_const_int))
+        r = to.download()
+        self.done()
+        return r
+
+    def rescale_add_rescale(self, a, ea, b, eb, eo, out_dtype):
+        ta, tb = self.put(a), self.put(b)
+        to = self.new(out_dtype, a.shape)
+        e1, e2, e3 = self._epi(*ea), self._epi(*eb), self._epi(*eo)
+        self.dev.op("rescale_add_rescale", to.ref, ta.ref, C.byref(e1), tb.ref, C.byref(e2), C.byref(e3))
+        r = to.download()
+        self.done()
+        return r

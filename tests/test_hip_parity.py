@@ -1,0 +1,451 @@
+"""GPU parity: every operator of the C ABI against the CPU oracle on the same seeded inputs (bit-exact for
+integers, stated tolerance for floats), the reference's known-answer vectors run on the GPU, and the
+BASELINE configs 0 and 1 at full size."""
+import zlib
+
+import numpy as np
+import pytest
+
+from conftest import fixture_array as arr
+from hip_util import Runner, abi, gpu_available, hb
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def run():
+    if not gpu_available():
+        pytest.skip("no GPU visible")
+    dev = hb.Device(0)
+    yield Runner(dev)
+    dev.close()
+
+
+def ri(rng, lo, hi, shape, dt):
+    return rng.integers(lo, hi, size=shape, endpoint=True).astype(dt)
+
+
+def rescale_params(rng, channels, per_channel=True):
+    n = channels if per_channel else 1
+    mult = ri(rng, 2 ** 30, 2 ** 31 - 1, (n,), np.int32)
+    shift = ri(rng, 30, 38, (n,), np.int8)
+    return mult, shift
+
+
+# ------------------------------------------------------------------------------------------------ reference KATs
+def test_kat_conv2d(run, kats):
+    k = kats["conv2d"]
+    a = k["attr"]
+    exp = arr(k["expected"])
+    attr = abi.conv2d_attr(a["pad"], a["stride"], a["dilation"], a["input_zp"], a["weight_zp"], a["acc_type"])
+    out = run.conv2d(arr(k["input"]), arr(k["weights"]), arr(k["bias"]), exp.shape, abi.I32, attr)
+    np.testing.assert_array_equal(out, exp)
+
+
+def test_kat_higher_rank_constant(run, kats):
+    k = kats["higher_rank_constant"]
+    a = k["attr"]
+    attr = abi.conv2d_attr(a["pad"], a["stride"], a["dilation"], a["input_zp"], a["weight_zp"], a["acc_type"])
+    acc = run.conv2d(arr(k["input"]), arr(k["weights"]), arr(k["bias"]), k["expected"]["shape"], abi.I32, attr)
+    np.testing.assert_array_equal(run.cast(acc, abi.I8), arr(k["expected"]))
+
+
+def test_kat_conv2d_acc_int64(run, kats):
+    k = kats["conv2d_acc_int64"]
+    a = k["attr"]
+    exp = arr(k["expected"])
+    attr = abi.conv2d_attr(a["pad"], a["stride"], a["dilation"], a["input_zp"], a["weight_zp"], a["acc_type"])
+    out = run.conv2d(arr(k["input"]), arr(k["weights"]), arr(k["bias"]), exp.shape, abi.I64, attr)
+    np.testing.assert_array_equal(out, exp)
+
+
+@pytest.mark.parametrize("which", ["oc", "w", "h"])
+def test_kat_conv2d_large_dims(run, kats, which):
+    """Reference sizes: OC = 262144, W or H = 524281 (beyond a Vulkan work-group-count limit there)."""
+    k = kats["conv2d_all_ones"]
+    c = k["channels"]
+    if which == "oc":
+        oc, h, w = k["large_oc"], 1, 1
+    elif which == "w":
+        oc, h, w = c, 1, k["large_spatial"]
+    else:
+        oc, h, w = c, k["large_spatial"], 1
+    x = np.ones((1, h, w, c), np.int8)
+    wt = np.ones((oc, 1, 1, c), np.int8)
+    out = run.conv2d(x, wt, np.zeros(oc, np.int32), (1, h, w, oc), abi.I32, abi.conv2d_attr())
+    assert out.shape == (1, h, w, oc) and (out == c).all()
+
+
+def test_kat_max_pool2d_and_two_layers(run, kats):
+    k = kats["max_pool2d"]
+    a = k["attr"]
+    attr = abi.pool2d_attr(a["kernel"], a["stride"], a["pad"], nan_mode=a["nan_mode"])
+    out = run.pool("max_pool2d", arr(k["input"]), k["expected"]["shape"], attr)
+    np.testing.assert_array_equal(out, arr(k["expected"]))
+    k2 = kats["two_layer_max_pool2d"]
+    out2 = run.pool("max_pool2d", out, k2["expected"]["shape"], attr)
+    np.testing.assert_array_equal(out2, arr(k2["expected"]))
+
+
+def test_kat_graph_constant_arm(run, kats):
+    k = kats["graph_constant_arm"]
+    r = k["rescale"]
+    attr = abi.rescale_attr(r["input_zp"], r["output_zp"], r["scale32"], r["double_round"], r["per_channel"])
+    m = [np.array([v], np.int32) for v in k["multipliers"]]
+    s = [np.array([v], np.int8) for v in k["shifts"]]
+    a = run.rescale(arr(k["input0"]), m[0], s[0], abi.I32, attr)
+    b = run.rescale(arr(k["input1"]), m[1], s[1], abi.I32, attr)
+    c = run.binary("ADD", a, b, a.shape, abi.I32)
+    np.testing.assert_array_equal(run.rescale(c, m[2], s[2], abi.I8, attr), arr(k["expected"]))
+    fused = run.rescale_add_rescale(arr(k["input0"]), (m[0], s[0], attr, None), arr(k["input1"]),
+                                    (m[1], s[1], attr, None), (m[2], s[2], attr, None), abi.I8)
+    np.testing.assert_array_equal(fused, arr(k["expected"]))
+
+
+def test_kat_data_movement_and_maximum(run, kats):
+    k = kats["concat"]
+    np.testing.assert_array_equal(run.concat([arr(k["input0"]), arr(k["input1"])], k["axis"]), arr(k["expected"]))
+    k = kats["slice"]
+    np.testing.assert_array_equal(run.slice_(arr(k["input"]), k["start"], k["size"]), arr(k["expected"]))
+    k = kats["concat_interval"]
+    s = run.binary("ADD", arr(k["input"]), arr(k["one"]), (3, 3), abi.F32)
+    np.testing.assert_array_equal(run.reshape(run.concat([s, arr(k["zero"])], 1), (12,)), arr(k["expected"]))
+    k = kats["maximum"]
+    out = run.binary("MAXIMUM", arr(k["input0"]), arr(k["input1"]), k["expected"]["shape"], abi.I32, k["nan_mode"])
+    np.testing.assert_array_equal(out, arr(k["expected"]))
+    k = kats["nop_outputs"]
+    np.testing.assert_array_equal(run.cast(arr(k["input"]), abi.I8), arr(k["input"]))
+    k = kats["sin"]
+    out = run.unary("SIN", np.array([k["input"]], np.float32))
+    assert abs(float(out[0]) - k["reference"]) <= k["error_bound"]
+
+
+# ------------------------------------------------------------------------------------------------ CONV2D int8
+CONV_CASES = [
+    # name, x shape, OC, (KH,KW), pad, stride, dil, zi, zw
+    ("c0_like_small", (1, 12, 12, 64), 64, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -5, 0),
+    ("stem_ic3_s2", (2, 17, 17, 3), 32, (3, 3), (0, 1, 0, 1), (2, 2), (1, 1), 7, 0),
+    ("pw_24_144", (2, 9, 9, 24), 144, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -3, 0),
+    ("pw_144_24", (2, 9, 9, 144), 24, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 4, 0),
+    ("pw_16_96_big_m", (3, 20, 21, 16), 96, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -128, 0),
+    ("both_zp", (1, 10, 7, 32), 40, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), 11, -7),
+    ("dilated_rect", (1, 13, 11, 8), 10, (2, 3), (2, 0, 1, 2), (1, 2), (2, 1), -128, 127),
+    ("odd_everything", (2, 7, 5, 5), 7, (3, 2), (1, 0, 0, 1), (2, 1), (1, 1), 3, 2),
+    ("ic20_oc130", (1, 6, 6, 20), 130, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 1, 0),
+    ("k_tail_ic48", (1, 5, 5, 48), 64, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 0, 0),
+    ("pw_960_320", (1, 7, 7, 960), 320, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -1, 0),
+]
+
+
+def out_hw(h, w, k, pad, stride, dil):
+    oh = (h + pad[0] + pad[1] - (k[0] - 1) * dil[0] - 1) // stride[0] + 1
+    ow = (w + pad[2] + pad[3] - (k[1] - 1) * dil[1] - 1) // stride[1] + 1
+    return oh, ow
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=[c[0] for c in CONV_CASES])
+def test_conv2d_i8_vs_oracle(run, oracle, case):
+    name, xs, oc, k, pad, stride, dil, zi, zw = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    x = ri(rng, -128, 127, xs, np.int8)
+    w = ri(rng, -128, 127, (oc,) + k + (xs[3],), np.int8)
+    b = ri(rng, -2 ** 15, 2 ** 15, (oc,), np.int32)
+    oh, ow = out_hw(xs[1], xs[2], k, pad, stride, dil)
+    attr = abi.conv2d_attr(pad, stride, dil, zi, zw)
+    shape = (xs[0], oh, ow, oc)
+    exp = oracle.conv2d(x, w, b, shape, abi.I32, attr)
+    out = run.conv2d(x, w, b, shape, abi.I32, attr)
+    np.testing.assert_array_equal(out, exp)
+    # fused RESCALE + CLAMP epilogue == the three operators one after another
+    mult, shift = rescale_params(rng, oc)
+    rattr = abi.rescale_attr(0, 3, True, True, True)
+    exp8 = oracle.clamp(oracle.rescale(exp, mult, shift, abi.I8, rattr), -20, 90)
+    out8 = run.conv2d(x, w, b, shape, abi.I8, attr, epilogue=(mult, shift, rattr, (-20, 90)))
+    np.testing.assert_array_equal(out8, exp8)
+
+
+def test_conv2d_bias_broadcast_and_strided_input(run, oracle):
+    rng = np.random.default_rng(5)
+    x = ri(rng, -128, 127, (1, 6, 6, 16), np.int8)
+    w = ri(rng, -128, 127, (8, 3, 3, 16), np.int8)
+    b = np.array([1234], np.int32)
+    attr = abi.conv2d_attr((1, 1, 1, 1), input_zp=9)
+    exp = oracle.conv2d(x, w, b, (1, 6, 6, 8), abi.I32, attr)
+    np.testing.assert_array_equal(run.conv2d(x, w, b, (1, 6, 6, 8), abi.I32, attr), exp)
+    # input rows padded to 32 bytes per pixel (explicit strides are honoured)
+    strides = (6 * 6 * 32, 6 * 32, 32, 1)
+    np.testing.assert_array_equal(run.conv2d(x, w, b, (1, 6, 6, 8), abi.I32, attr, x_strides=strides), exp)
+
+
+def test_conv2d_i16_and_f32_generic(run, oracle):
+    rng = np.random.default_rng(6)
+    x = ri(rng, -3000, 3000, (1, 5, 5, 3), np.int16)
+    w = ri(rng, -128, 127, (4, 3, 3, 3), np.int8)
+    b = ri(rng, -10 ** 9, 10 ** 9, (4,), np.int64)
+    attr = abi.conv2d_attr((1, 1, 1, 1), acc_type=abi.ACC_I64)
+    np.testing.assert_array_equal(run.conv2d(x, w, b, (1, 5, 5, 4), abi.I64, attr),
+                                  oracle.conv2d(x, w, b, (1, 5, 5, 4), abi.I64, attr))
+    xf = rng.standard_normal((1, 5, 5, 3)).astype(np.float32)
+    wf = rng.standard_normal((4, 3, 3, 3)).astype(np.float32)
+    bf = rng.standard_normal(4).astype(np.float32)
+    attrf = abi.conv2d_attr((1, 1, 1, 1), acc_type=abi.ACC_F32)
+    np.testing.assert_allclose(run.conv2d(xf, wf, bf, (1, 5, 5, 4), abi.F32, attrf),
+                               oracle.conv2d(xf, wf, bf, (1, 5, 5, 4), abi.F32, attrf), rtol=1e-5, atol=1e-5)
+
+
+# ------------------------------------------------------------------------------------------------ MATMUL int8
+MM_CASES = [
+    ("aligned", 2, 128, 128, 128, 2, -1),
+    ("c1_like_small", 3, 96, 256, 192, 2, -1),
+    ("ragged", 2, 37, 53, 29, -4, 6),
+    ("n_mod4", 1, 64, 70, 36, 0, 0),
+    ("fc_like", 1, 32, 1280, 1000, 0, 0),
+    ("zp_a_only", 2, 33, 64, 64, 9, 0),
+    ("zp_b_only", 2, 33, 64, 64, 0, -9),
+    ("k_small", 4, 300, 8, 16, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", MM_CASES, ids=[c[0] for c in MM_CASES])
+def test_matmul_i8_vs_oracle(run, oracle, case):
+    name, nb, m, k, n, za, zb = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    a = ri(rng, -128, 127, (nb, m, k), np.int8)
+    b = ri(rng, -128, 127, (nb, k, n), np.int8)
+    exp = oracle.matmul(a, b, abi.I32, za, zb)
+    np.testing.assert_array_equal(run.matmul(a, b, abi.I32, za, zb), exp)
+    mult, shift = np.array([1518500250], np.int32), np.array([39], np.int8)
+    rattr = abi.rescale_attr(0, 0, True, True, False)
+    exp8 = oracle.rescale(exp, mult, shift, abi.I8, rattr)
+    np.testing.assert_array_equal(run.matmul(a, b, abi.I8, za, zb, epilogue=(mult, shift, rattr, None)), exp8)
+
+
+def test_matmul_float_generic(run, oracle):
+    rng = np.random.default_rng(8)
+    a = rng.standard_normal((2, 9, 33)).astype(np.float32)
+    b = rng.standard_normal((2, 33, 12)).astype(np.float32)
+    np.testing.assert_allclose(run.matmul(a, b, abi.F32), oracle.matmul(a, b, abi.F32), rtol=1e-5, atol=1e-5)
+    a16, b16 = a.astype(np.float16), b.astype(np.float16)
+    # fp16 inputs with fp32 accumulate: max abs error <= 1e-2
+    out = run.matmul(a16, b16, abi.F32)
+    assert np.max(np.abs(out - oracle.matmul(a16, b16, abi.F32))) <= 1e-2
+
+
+# ------------------------------------------------------------------------------------------------ DEPTHWISE
+DW_CASES = [
+    ("c2_like_small", (2, 14, 14, 144), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -4, 0),
+    ("stride2", (1, 16, 16, 96), 1, (3, 3), (0, 1, 0, 1), (2, 2), (1, 1), 6, 0),
+    ("c32", (1, 9, 9, 32), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -128, 0),
+    ("mult2_zw", (1, 7, 8, 5), 2, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), 3, -2),
+    ("k5_dil", (1, 11, 11, 8), 1, (5, 5), (2, 2, 2, 2), (1, 1), (1, 1), 0, 0),
+    ("c960", (1, 7, 7, 960), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -1, 0),
+]
+
+
+@pytest.mark.parametrize("case", DW_CASES, ids=[c[0] for c in DW_CASES])
+def test_depthwise_vs_oracle(run, oracle, case):
+    name, xs, mch, k, pad, stride, dil, zi, zw = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    c = xs[3]
+    x = ri(rng, -128, 127, xs, np.int8)
+    w = ri(rng, -128, 127, k + (c, mch), np.int8)
+    b = ri(rng, -2 ** 15, 2 ** 15, (c * mch,), np.int32)
+    oh, ow = out_hw(xs[1], xs[2], k, pad, stride, dil)
+    shape = (xs[0], oh, ow, c * mch)
+    attr = abi.conv2d_attr(pad, stride, dil, zi, zw)
+    exp = oracle.depthwise_conv2d(x, w, b, shape, abi.I32, attr)
+    np.testing.assert_array_equal(run.conv2d(x, w, b, shape, abi.I32, attr, depthwise=True), exp)
+    mult, shift = rescale_params(rng, c * mch)
+    rattr = abi.rescale_attr(0, -7, True, True, True)
+    exp8 = oracle.clamp(oracle.rescale(exp, mult, shift, abi.I8, rattr), -7, 100)
+    out8 = run.conv2d(x, w, b, shape, abi.I8, attr, depthwise=True, epilogue=(mult, shift, rattr, (-7, 100)))
+    np.testing.assert_array_equal(out8, exp8)
+
+
+# ------------------------------------------------------------------------------------------------ RESCALE & co
+@pytest.mark.parametrize("double_round", [False, True])
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_rescale_vs_oracle(run, oracle, double_round, per_channel):
+    rng = np.random.default_rng(11)
+    c = 24
+    x = ri(rng, -2 ** 26, 2 ** 26, (3, 7, 5, c), np.int32)
+    mult, shift = rescale_params(rng, c, per_channel)
+    if per_channel:
+        shift[:4] = [2, 31, 32, 62]
+    attr = abi.rescale_attr(0, -3, True, double_round, per_channel)
+    for odt in (abi.I8, abi.I16, abi.I32):
+        np.testing.assert_array_equal(run.rescale(x, mult, shift, odt, attr), oracle.rescale(x, mult, shift, odt, attr))
+    x8 = ri(rng, -128, 127, (3, 7, 5, c), np.int8)
+    attr8 = abi.rescale_attr(-5, 0, True, double_round, per_channel)
+    np.testing.assert_array_equal(run.rescale(x8, mult, shift, abi.I32, attr8),
+                                  oracle.rescale(x8, mult, shift, abi.I32, attr8))
+    attru = abi.rescale_attr(128, 0, True, double_round, per_channel, input_unsigned=True, output_unsigned=True)
+    np.testing.assert_array_equal(run.rescale(x8, mult, shift, abi.I8, attru),
+                                  oracle.rescale(x8, mult, shift, abi.I8, attru))
+    m16 = ri(rng, 1, 32767, mult.shape, np.int16)
+    s16 = ri(rng, 8, 20, shift.shape, np.int8)
+    attr16 = abi.rescale_attr(0, 1, False, True, per_channel)
+    np.testing.assert_array_equal(run.rescale(x, m16, s16, abi.I16, attr16),
+                                  oracle.rescale(x, m16, s16, abi.I16, attr16))
+
+
+def test_rescale_add_rescale_vs_oracle(run, oracle):
+    rng = np.random.default_rng(12)
+    c = 24
+    a = ri(rng, -128, 127, (2, 9, 9, c), np.int8)
+    b = ri(rng, -128, 127, (2, 9, 9, c), np.int8)
+    m1, s1 = np.array([1 << 30], np.int32), np.array([11], np.int8)
+    m2, s2 = np.array([1431655765], np.int32), np.array([12], np.int8)
+    mo, so = np.array([1717986918], np.int32), np.array([50], np.int8)
+    a1 = abi.rescale_attr(-3, 0, True, True, False)
+    a2 = abi.rescale_attr(5, 0, True, True, False)
+    ao = abi.rescale_attr(0, -1, True, True, False)
+    ra = oracle.rescale(a, m1, s1, abi.I32, a1)
+    rb = oracle.rescale(b, m2, s2, abi.I32, a2)
+    exp = oracle.rescale(oracle.elementwise_binary("ADD", ra, rb, ra.shape, abi.I32), mo, so, abi.I8, ao)
+    out = run.rescale_add_rescale(a, (m1, s1, a1, None), b, (m2, s2, a2, None), (mo, so, ao, None), abi.I8)
+    np.testing.assert_array_equal(out, exp)
+
+
+def test_clamp_binary_mul_table_vs_oracle(run, oracle):
+    rng = np.random.default_rng(13)
+    x8 = ri(rng, -128, 127, (4, 33, 7), np.int8)
+    np.testing.assert_array_equal(run.clamp(x8, -3, 100), oracle.clamp(x8, -3, 100))
+    f = rng.standard_normal((5, 40)).astype(np.float32)
+    f[1, 3] = np.nan
+    for mode in (abi.NAN_PROPAGATE, abi.NAN_IGNORE):
+        np.testing.assert_array_equal(run.clamp(f, -0.5, 0.25, mode), oracle.clamp(f, -0.5, 0.25, mode))
+    a = ri(rng, -2 ** 31, 2 ** 31 - 1, (2, 3, 40), np.int32)
+    b = ri(rng, -2 ** 31, 2 ** 31 - 1, (2, 1, 40), np.int32)
+    for op in ("ADD", "SUB", "MAXIMUM", "MINIMUM", "BITWISE_AND", "BITWISE_OR", "BITWISE_XOR"):
+        np.testing.assert_array_equal(run.binary(op, a, b, a.shape, abi.I32),
+                                      oracle.elementwise_binary(op, a, b, a.shape, abi.I32), err_msg=op)
+    for op in ("EQUAL", "GREATER", "GREATER_EQUAL"):
+        np.testing.assert_array_equal(run.binary(op, a, b, a.shape, abi.BOOL),
+                                      oracle.elementwise_binary(op, a, b, a.shape, abi.BOOL), err_msg=op)
+    sh = ri(rng, 0, 31, (2, 3, 40), np.int32)
+    for op in ("LOGICAL_LEFT_SHIFT", "LOGICAL_RIGHT_SHIFT"):
+        np.testing.assert_array_equal(run.binary(op, a, sh, a.shape, abi.I32),
+                                      oracle.elementwise_binary(op, a, sh, a.shape, abi.I32), err_msg=op)
+    for shift in (0, 7, 31):
+        np.testing.assert_array_equal(run.mul(a, b, a.shape, abi.I32, shift), oracle.mul(a, b, a.shape, abi.I32, shift))
+    tab = ri(rng, -128, 127, (256,), np.int8)
+    np.testing.assert_array_equal(run.table(x8, tab, abi.I8), oracle.table(x8, tab, abi.I8))
+    x16 = ri(rng, -32768, 32767, (500,), np.int16)
+    t16 = ri(rng, -32768, 32767, (513,), np.int16)
+    np.testing.assert_array_equal(run.table(x16, t16, abi.I32), oracle.table(x16, t16, abi.I32))
+
+
+def test_pool_reduce_cast_negate_vs_oracle(run, oracle):
+    rng = np.random.default_rng(14)
+    x = ri(rng, -128, 127, (2, 7, 7, 40), np.int8)
+    a = abi.pool2d_attr((7, 7), (1, 1), (0, 0, 0, 0), input_zp=-3, output_zp=2)
+    np.testing.assert_array_equal(run.pool("avg_pool2d", x, (2, 1, 1, 40), a), oracle.avg_pool2d(x, (2, 1, 1, 40), a))
+    a2 = abi.pool2d_attr((3, 3), (2, 2), (1, 1, 1, 1), input_zp=4, output_zp=-1)
+    np.testing.assert_array_equal(run.pool("avg_pool2d", x, (2, 4, 4, 40), a2), oracle.avg_pool2d(x, (2, 4, 4, 40), a2))
+    np.testing.assert_array_equal(run.pool("max_pool2d", x, (2, 4, 4, 40), a2), oracle.max_pool2d(x, (2, 4, 4, 40), a2))
+    r = ri(rng, -1000, 1000, (3, 4, 50), np.int32)
+    for op in ("SUM", "MAX", "MIN", "PRODUCT"):
+        for axis in range(3):
+            np.testing.assert_array_equal(run.reduce(op, r, axis), oracle.reduce(op, r, axis), err_msg=f"{op}{axis}")
+    big = ri(rng, -2 ** 31, 2 ** 31 - 1, (1000,), np.int32)
+    for odt in (abi.I8, abi.I16, abi.BOOL):
+        np.testing.assert_array_equal(run.cast(big, odt), oracle.cast(big, odt))
+    f = (rng.standard_normal(1000) * 100).astype(np.float32)
+    f[:6] = [0.5, 1.5, 2.5, -0.5, 1e9, -1e9]
+    np.testing.assert_array_equal(run.cast(f, abi.I8), oracle.cast(f, abi.I8))
+    np.testing.assert_array_equal(run.cast(big, abi.F16).view(np.uint16), oracle.cast(big, abi.F16).view(np.uint16))
+    x1 = ri(rng, -128, 127, (300,), np.int8)
+    np.testing.assert_array_equal(run.negate(x1, 3, -2), oracle.negate(x1, 3, -2))
+
+
+def test_data_movement_vs_oracle(run, oracle):
+    rng = np.random.default_rng(15)
+    x = ri(rng, -128, 127, (2, 3, 4, 5), np.int8)
+    np.testing.assert_array_equal(run.reshape(x, (6, 20)), x.reshape(6, 20))
+    for perms in [(0, 2, 1, 3), (3, 2, 1, 0), (1, 0, 3, 2)]:
+        np.testing.assert_array_equal(run.transpose(x, perms), x.transpose(perms))
+    np.testing.assert_array_equal(run.slice_(x, (1, 0, 2, 1), (1, 3, 2, 3)), x[1:2, 0:3, 2:4, 1:4])
+    pads = [(0, 0), (1, 2), (0, 1), (2, 0)]
+    shape = tuple(d + a + b for d, (a, b) in zip(x.shape, pads))
+    x32 = x.astype(np.int32)
+    np.testing.assert_array_equal(run.pad(x32, np.array(pads).reshape(-1), shape, pad_const_int=-7),
+                                  np.pad(x32, pads, constant_values=-7))
+    h = rng.standard_normal((8, 16, 4, 6)).astype(np.float16)
+    np.testing.assert_array_equal(run.transpose(h, (0, 2, 1, 3)).view(np.uint16),
+                                  h.transpose(0, 2, 1, 3).view(np.uint16))
+
+
+def test_float_unary_and_reduce_tolerance(run, oracle):
+    """fp16/fp32 elementwise: the reference's results depend on its driver's builtins (parity unpinned); the
+    bar is max abs error <= 1e-2 against the oracle's fp32 evaluation rounded once to the storage type."""
+    rng = np.random.default_rng(16)
+    x = rng.standard_normal((4, 300)).astype(np.float16)
+    for op in ("EXP", "TANH", "SIGMOID", "ABS", "FLOOR", "CEIL", "ERF", "SIN", "COS"):
+        d = np.abs(run.unary(op, x).astype(np.float32) - oracle.elementwise_unary(op, x).astype(np.float32))
+        assert np.nanmax(d) <= 1e-2, op
+    xp = np.abs(x) + np.float16(0.5)
+    for op in ("RECIPROCAL", "RSQRT", "LOG"):
+        d = np.abs(run.unary(op, xp).astype(np.float32) - oracle.elementwise_unary(op, xp).astype(np.float32))
+        assert np.nanmax(d) <= 1e-2, op
+    f = rng.standard_normal((6, 512)).astype(np.float32)
+    np.testing.assert_allclose(run.reduce("SUM", f, 1), oracle.reduce("SUM", f, 1), rtol=1e-5, atol=1e-4)
+    np.testing.assert_array_equal(run.reduce("MAX", f, 1), oracle.reduce("MAX", f, 1))
+    a = rng.standard_normal((4, 1, 64)).astype(np.float16)
+    b = rng.standard_normal((4, 8, 64)).astype(np.float16)
+    for op in ("ADD", "SUB"):
+        np.testing.assert_array_equal(run.binary(op, a, b, b.shape, abi.F16).view(np.uint16),
+                                      oracle.elementwise_binary(op, a, b, b.shape, abi.F16).view(np.uint16))
+    np.testing.assert_array_equal(run.mul(a, b, b.shape, abi.F16).view(np.uint16),
+                                  oracle.mul(a, b, b.shape, abi.F16).view(np.uint16))
+
+
+# ------------------------------------------------------------------------------------------------ error paths
+def test_error_conventions(run):
+    x = np.zeros((1, 4, 4, 4), np.int8)
+    w = np.zeros((4, 1, 1, 4), np.int8)
+    b = np.zeros(4, np.int32)
+    with pytest.raises(hb.MlelError) as e:
+        run.conv2d(x, w, b, (1, 4, 4, 4), abi.I32, abi.conv2d_attr(acc_type=9))
+    run.done()
+    assert e.value.code == abi.ERR_INVALID and "Unsupported acc type 9" in str(e.value)
+    with pytest.raises(hb.MlelError):
+        run.rescale(np.zeros(4, np.int32), np.zeros(1, np.int16), np.zeros(1, np.int8), abi.I8,
+                    abi.rescale_attr(scale32=True))
+    run.done()
+
+
+# ------------------------------------------------------------------------------------------------ BASELINE configs
+def test_config0_conv_rescale_full_size(run, oracle):
+    """BASELINE config 0: CONV2D 1x56x56x64 -> 64, 3x3 s1 p1, zi=-5, then per-channel RESCALE (double round) to
+    int8 with output zero point 3; unfused and fused must both equal the oracle."""
+    rng = np.random.default_rng(1000)
+    x = ri(rng, -128, 127, (1, 56, 56, 64), np.int8)
+    w = ri(rng, -127, 127, (64, 3, 3, 64), np.int8)
+    b = ri(rng, -2 ** 15, 2 ** 15, (64,), np.int32)
+    mult = ri(rng, 2 ** 30, 2 ** 31 - 1, (64,), np.int32)
+    shift = ri(rng, 30, 38, (64,), np.int8)
+    attr = abi.conv2d_attr((1, 1, 1, 1), (1, 1), (1, 1), -5, 0)
+    rattr = abi.rescale_attr(0, 3, True, True, True)
+    acc = oracle.conv2d(x, w, b, (1, 56, 56, 64), abi.I32, attr)
+    exp = oracle.rescale(acc, mult, shift, abi.I8, rattr)
+    np.testing.assert_array_equal(run.conv2d(x, w, b, (1, 56, 56, 64), abi.I32, attr), acc)
+    np.testing.assert_array_equal(run.rescale(acc, mult, shift, abi.I8, rattr), exp)
+    np.testing.assert_array_equal(run.conv2d(x, w, b, (1, 56, 56, 64), abi.I8, attr,
+                                             epilogue=(mult, shift, rattr, None)), exp)
+
+
+def test_config1_matmul_rescale_full_size(run, oracle):
+    """BASELINE config 1: MATMUL 8x512x1024 . 8x1024x1024 int8, a_zp=2, b_zp=-1, then per-tensor RESCALE
+    (multiplier 1518500250, shift 39, double round) to int8."""
+    rng = np.random.default_rng(1001)
+    a = ri(rng, -128, 127, (8, 512, 1024), np.int8)
+    b = ri(rng, -128, 127, (8, 1024, 1024), np.int8)
+    mult, shift = np.array([1518500250], np.int32), np.array([39], np.int8)
+    rattr = abi.rescale_attr(0, 0, True, True, False)
+    acc = oracle.matmul(a, b, abi.I32, 2, -1)
+    exp = oracle.rescale(acc, mult, shift, abi.I8, rattr)
+    np.testing.assert_array_equal(run.matmul(a, b, abi.I32, 2, -1), acc)
+    np.testing.assert_array_equal(run.matmul(a, b, abi.I8, 2, -1, epilogue=(mult, shift, rattr, None)), exp)
+    # the requantised result uses the whole int8 range (a degenerate all-zero output would prove nothing)
+    assert exp.min() < -20 and exp.max() > 20
