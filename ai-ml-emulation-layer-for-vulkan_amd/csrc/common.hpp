@@ -243,12 +243,47 @@ __device__ __forceinline__ int32_t apply_scale(int64_t value, int32_t mult, int3
     return (int32_t)((int64_t)prod >> s);
 }
 
-// int32 accumulator -> requantised value, the hot form used by fused epilogues (value fits in int32)
+// int32 accumulator -> requantised value (any shift, general form)
 __device__ __forceinline__ int32_t requant_i32(int32_t acc, int32_t mult, int32_t shift, const RescaleParams &p) {
     const int64_t value = (int64_t)acc - (int64_t)p.in_zp;
     int32_t r = apply_scale(value, mult, shift, p.double_round != 0);
     r = (int32_t)((uint32_t)r + (uint32_t)p.out_zp);
     if (p.clamp_out) r = r < p.out_lo ? p.out_lo : (r > p.out_hi ? p.out_hi : r);
+    return r;
+}
+
+// The same arithmetic with everything that depends only on the channel hoisted out of the per-element path:
+//   (value * mult + round) >> shift,  value = acc - in_zp,  round = 2^(shift-1) [+/- 2^30 by the sign of value]
+// becomes  acc * mult + (round - in_zp * mult)  as one 64-bit multiply-add, plus the sign-dependent nudge.
+struct ChanScale {
+    int32_t mult;
+    int32_t shift;     // clamped to 0..63
+    int32_t nudge;     // 2^30 when double rounding applies to this channel (shift > 31), else 0
+    int32_t pad;
+    int64_t round;     // 2^(shift-1) - in_zp * mult (wraparound), 0 when shift == 0
+};
+
+__host__ __device__ inline ChanScale make_chan_scale(int32_t mult, int32_t shift, const RescaleParams &p) {
+    ChanScale c;
+    c.mult = mult;
+    c.shift = shift < 0 ? 0 : (shift > 63 ? 63 : shift);
+    c.nudge = (p.double_round && shift > 31) ? (1 << 30) : 0;
+    c.pad = 0;
+    const uint64_t base = shift > 0 ? (uint64_t(1) << (c.shift - 1)) : 0;
+    c.round = (int64_t)(base - (uint64_t)(int64_t)p.in_zp * (uint64_t)(int64_t)mult);
+    return c;
+}
+
+template <bool ZERO_IN_ZP>
+__device__ __forceinline__ int32_t requant_chan(int32_t acc, const ChanScale &c, const RescaleParams &p) {
+    // sign of value = acc - in_zp as an all-ones / all-zeros mask
+    const int32_t neg = ZERO_IN_ZP ? (acc >> 31) : (acc < p.in_zp ? -1 : 0);
+    const int32_t nudge = (c.nudge ^ neg) - neg;  // +2^30, -2^30 or 0
+    uint64_t t = (uint64_t)((int64_t)acc * (int64_t)c.mult) + (uint64_t)c.round;
+    t += (uint64_t)(int64_t)nudge;
+    int32_t r = (int32_t)((int64_t)t >> c.shift);
+    r = (int32_t)((uint32_t)r + (uint32_t)p.out_zp);
+    if (p.clamp_out) r = min(max(r, p.out_lo), p.out_hi);
     return r;
 }
 

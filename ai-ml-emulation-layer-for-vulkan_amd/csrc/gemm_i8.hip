@@ -26,6 +26,8 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) v2i lds_v2i;
 
 constexpr int BK = 64;            // bytes of K per step
 constexpr int PITCH = BK + 16;    // LDS row pitch: 80 B keeps 16-lane groups of 128-bit reads on distinct banks
@@ -40,6 +42,7 @@ struct GemmArgs {
     int32_t H, W, IC, OHW, OW, KH, KW, sy, sx, dy, dx, pad_t, pad_l;
     int32_t plain;  // 1: m indexes rows of pitch x_sx directly
     int32_t xch;    // bytes per aligned global load of X: 16, 4 or 1
+    uint32_t x_bytes, w_bytes;  // per-batch extent of each operand (buffer-load bounds of the fast fetch modes)
     // W operand (rows n)
     const int8_t *w;
     int64_t w_batch, ldw;
@@ -63,12 +66,12 @@ struct GemmArgs {
     int32_t tiles_m, tiles_n, total_tiles, chunk;
 };
 
-struct ChanParams {  // per output channel, in LDS
+struct ChanParams {  // per output channel, in LDS: 32 bytes = two 128-bit reads
+    ChanScale q;
     int32_t bias_adj;
-    int32_t mult;
-    int32_t shift;
-    int32_t pad;
+    int32_t pad[1];
 };
+static_assert(sizeof(ChanParams) == 32, "ChanParams layout");
 
 struct RowState {
     const int8_t *base;
@@ -191,28 +194,66 @@ __device__ __forceinline__ uint4 load_w_block_kmajor(const GemmArgs &g, const in
                       __builtin_amdgcn_perm(t3, t1, 0x05040100u), __builtin_amdgcn_perm(t3, t1, 0x07060302u));
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+// Buffer-addressed loads: 32-bit offsets, and an offset at or beyond the extent of the resource returns 0
+// without touching memory, which removes every bounds branch from the fast fetch modes.
+constexpr uint32_t kOobOffset = 0x80000000u;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+    const v4i v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+    return make_uint4((uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w);
+}
+__device__ __forceinline__ uint32_t buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+    return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0);
+}
+
+template <int BN>
+constexpr int w_buf_bytes() {
+    return BN * PITCH > BK * (BN + 16) ? BN * PITCH : BK * (BN + 16);
+}
+
+// How the two operands are fetched; fixed at compile time so that the hot loops carry no per-byte logic.
+enum XMode {
+    X_PLAIN = 0,    // X[m][k] = base + m * pitch + k, 16-byte pieces (MATMUL A; 1x1 stride-1 CONV2D on a dense input)
+    X_TAP = 1,      // 16-byte pieces, IC % 64 == 0: one K step lies inside one filter tap (uniform tap state)
+    X_GENERIC = 2,  // anything else: per-piece tap tracking, 16 / 4 / 1-byte loads
+};
+enum WMode {
+    W_ROWS = 0,     // [N][K], 16-byte pieces
+    W_KMAJOR = 1,   // [K][N] kept K-major in LDS; MFMA operands are gathered with ds_read_b64_tr_b8
+    W_GENERIC = 2,  // either layout, any alignment
+};
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int XMODE, int WMODE, bool SUMS>
 __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wavefront sub-tile
     constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 MFMA tiles per wavefront
-    constexpr int XROWS = BM / 64;                       // X rows per thread (4 chunks of 16 B per row)
+    constexpr int XROWS = BM / 64;                       // X rows per thread (4 pieces of 16 B per row)
     constexpr int WCHUNKS = (BN * 4 + NTHREADS - 1) / NTHREADS;
     static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per block");
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wavefront tile is a multiple of the 32x32 MFMA tile");
 
+    constexpr int PW = BN + 16;           // W_KMAJOR: LDS pitch of one K row of BN channels (bytes)
+    constexpr int WBUF = w_buf_bytes<BN>();  // one W buffer: [BN][PITCH] or [BK][PW], whichever is larger
+    constexpr int N16 = BN / 16;          // 16-byte pieces per K row of the K-major tile
+
     extern __shared__ __align__(16) char smem[];
-    char *xs = smem;                             // [2][BM][PITCH]
-    char *ws = smem + 2 * BM * PITCH;            // [2][BN][PITCH]
-    ChanParams *cp = reinterpret_cast<ChanParams *>(smem + 2 * (BM + BN) * PITCH);  // [BN]
+    char *xs = smem;                     // [2][BM][PITCH]
+    char *ws = smem + 2 * BM * PITCH;    // [2][WBUF]
+    ChanParams *cp = reinterpret_cast<ChanParams *>(smem + 2 * BM * PITCH + 2 * WBUF);  // [BN]
 
     // ---- XCD-aware tile assignment: consecutive block ids land on different XCDs (8 of them, each with its own
     // L2), so block b is given tile (b % 8) * chunk + b / 8: tiles that share operands stay on one XCD.
     const int lin = (int)(blockIdx.x % 8) * g.chunk + (int)(blockIdx.x / 8);
     if (lin >= g.total_tiles) return;
     const int tiles_per_batch = g.tiles_m * g.tiles_n;
-    const int batch = lin / tiles_per_batch;
+    // the divisions run on the vector ALU; readfirstlane returns the (wave-uniform) results to scalar registers so
+    // that everything derived from them (base pointers, buffer resources) is scalar as well
+    const int batch = __builtin_amdgcn_readfirstlane(lin / tiles_per_batch);
     const int t_in = lin - batch * tiles_per_batch;
-    const int tile_m = t_in / g.tiles_n, tile_n = t_in - tile_m * g.tiles_n;
+    const int tile_m = __builtin_amdgcn_readfirstlane(t_in / g.tiles_n);
+    const int tile_n = t_in - tile_m * g.tiles_n;
     const int m_base = tile_m * BM, n_base = tile_n * BN;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -223,56 +264,127 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
 
     // ---- per-channel epilogue constants
     for (int n = tid; n < BN; n += NTHREADS) {
-        ChanParams c{0, 0, 0, 0};
+        ChanParams c{};
         const int gn = n_base + n;
         if (gn < g.N) {
             c.bias_adj = g.bias ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
             if (g.fused) {
                 const int ci = g.rp.per_channel ? gn : 0;
-                c.mult = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
-                                  : reinterpret_cast<const int32_t *>(g.mult)[ci];
-                c.shift = (int32_t)g.shift[ci];
+                const int32_t m = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
+                                           : reinterpret_cast<const int32_t *>(g.mult)[ci];
+                c.q = make_chan_scale(m, (int32_t)g.shift[ci], g.rp);
             }
         }
         cp[n] = c;
     }
 
     // ---- loader state
-    RowState rows[XROWS];
     const int x_kc = tid & 3;  // which 16-byte piece of the 64-byte K step this thread stages
+    RowState rows[XROWS];      // X_GENERIC: pointers; X_TAP: tap origin
+    uint32_t xoff[XROWS];      // fast modes: byte offset of the row (X_PLAIN) / image (X_TAP), or kOobOffset
 #pragma unroll
     for (int i = 0; i < XROWS; i++) {
         const int m = m_base + (tid >> 2) + 64 * i;
         RowState r{xb, 0, 0, m < g.M};
+        xoff[i] = kOobOffset;
         if (r.valid) {
             if (g.plain) {
                 r.base = xb + (int64_t)m * g.x_sx;
+                xoff[i] = (uint32_t)m * (uint32_t)g.x_sx + x_kc * 16;
             } else {
                 const int img = m / g.OHW, rem = m - img * g.OHW;
                 const int oy = rem / g.OW, ox = rem - oy * g.OW;
                 r.base = xb + (int64_t)img * g.x_sn;
                 r.iy0 = oy * g.sy - g.pad_t;
                 r.ix0 = ox * g.sx - g.pad_l;
+                xoff[i] = (uint32_t)img * (uint32_t)g.x_sn + x_kc * 16;
             }
         }
         rows[i] = r;
     }
-    KState ks{0, 0, 0};
-    kstate_advance(ks, x_kc * 16, g.IC, g.KW);
+    KState ks{0, 0, 0};                      // X_GENERIC: k position of this thread's piece
+    if (XMODE == X_GENERIC) kstate_advance(ks, x_kc * 16, g.IC, g.KW);
+    int tap_ky = 0, tap_kx = 0, tap_ic = 0;  // X_TAP: uniform position of the K step
+    const __amdgpu_buffer_rsrc_t xres = make_rsrc(xb, g.x_bytes), wres = make_rsrc(wb, g.w_bytes);
 
-    uint4 xr[XROWS], wr[WCHUNKS];
-    auto prefetch = [&](int k0) {
+    uint32_t woff[WCHUNKS];  // fast modes: byte offset of the piece at k = 0, or kOobOffset
 #pragma unroll
-        for (int i = 0; i < XROWS; i++) xr[i] = load_x_chunk(g, rows[i], ks);
-        kstate_advance(ks, BK, g.IC, g.KW);
-        if (!g.w_kmajor) {
+    for (int i = 0; i < WCHUNKS; i++) {
+        const int c = tid + NTHREADS * i;
+        woff[i] = kOobOffset;
+        if (c < BN * 4) {
+            if (WMODE == W_ROWS) {
+                const int n = n_base + (c >> 2);
+                if (n < g.N) woff[i] = (uint32_t)n * (uint32_t)g.ldw + (c & 3) * 16;
+            } else if (WMODE == W_KMAJOR) {
+                // piece c = 16 channels of K row c / N16; rows at or beyond K lie past the end of the buffer
+                // resource and read as 0 without a test
+                const int n = n_base + (c % N16) * 16;
+                if (n < g.N) woff[i] = (uint32_t)(c / N16) * (uint32_t)g.ldw + n;
+            }
+        }
+    }
+
+    // global -> registers for the K step starting at k0 (the steps are requested in increasing order)
+    auto prefetch = [&](int k0, uint4 (&xr)[XROWS], uint4 (&wr)[WCHUNKS], uint32_t &xpad) {
+        xpad = 0;
+        if (XMODE == X_PLAIN) {
+            const bool kin = k0 + x_kc * 16 < g.K;
+#pragma unroll
+            for (int i = 0; i < XROWS; i++) xr[i] = buf_load16(xres, kin ? xoff[i] + (uint32_t)k0 : kOobOffset);
+        } else if (XMODE == X_TAP) {
+            const bool kin = tap_ky < g.KH;
+            const int oy = tap_ky * g.dy, ox = tap_kx * g.dx;
+#pragma unroll
+            for (int i = 0; i < XROWS; i++) {
+                const int y = rows[i].iy0 + oy, x = rows[i].ix0 + ox;
+                const bool inb = (unsigned)y < (unsigned)g.H && (unsigned)x < (unsigned)g.W;
+                const uint32_t off = xoff[i] + (uint32_t)y * (uint32_t)g.x_sy + (uint32_t)x * (uint32_t)g.x_sx +
+                                     (uint32_t)tap_ic;
+                xr[i] = buf_load16(xres, (kin && inb && rows[i].valid) ? off : kOobOffset);
+                if (kin && !inb && rows[i].valid) xpad |= 1u << i;  // a padded tap: filled with zx when staged
+            }
+            tap_ic += BK;
+            if (tap_ic >= g.IC) {
+                tap_ic = 0;
+                if (++tap_kx == g.KW) {
+                    tap_kx = 0;
+                    ++tap_ky;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < XROWS; i++) xr[i] = load_x_chunk(g, rows[i], ks);
+            kstate_advance(ks, BK, g.IC, g.KW);
+        }
+        if (WMODE == W_ROWS) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                const bool kin = k0 + (c & 3) * 16 < g.K;
+                wr[i] = buf_load16(wres, kin ? woff[i] + (uint32_t)k0 : kOobOffset);
+            }
+        } else if (WMODE == W_KMAJOR) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const uint32_t off = woff[i] + (uint32_t)k0 * (uint32_t)g.ldw;
+                if (g.wch == 16) {
+                    wr[i] = buf_load16(wres, off);
+                } else {  // rows are only dword aligned: four loads, channels at or beyond N masked
+                    const int n = n_base + ((tid + NTHREADS * i) % N16) * 16;
+                    wr[i].x = buf_load4(wres, n + 0 < g.N ? off + 0 : kOobOffset);
+                    wr[i].y = buf_load4(wres, n + 4 < g.N ? off + 4 : kOobOffset);
+                    wr[i].z = buf_load4(wres, n + 8 < g.N ? off + 8 : kOobOffset);
+                    wr[i].w = buf_load4(wres, n + 12 < g.N ? off + 12 : kOobOffset);
+                }
+            }
+        } else if (!g.w_kmajor) {
 #pragma unroll
             for (int i = 0; i < WCHUNKS; i++) {
                 const int c = tid + NTHREADS * i;
                 if (c < BN * 4) wr[i] = load_w_chunk(g, wb, n_base + (c >> 2), k0 + (c & 3) * 16);
             }
         } else {
-            // (BK/4) x (BN/4) blocks of 4x4 bytes; consecutive lanes take consecutive column groups
 #pragma unroll
             for (int i = 0; i < WCHUNKS; i++) {
                 const int c = tid + NTHREADS * i;
@@ -280,13 +392,24 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
             }
         }
     };
-    auto stage = [&](int buf) {
+    // registers -> LDS buffer `buf`
+    auto stage = [&](int buf, const uint4 (&xr)[XROWS], const uint4 (&wr)[WCHUNKS], uint32_t xpad) {
         char *xd = xs + buf * BM * PITCH;
-        char *wd = ws + buf * BN * PITCH;
+        char *wd = ws + buf * WBUF;
+        const uint32_t z = splat8(g.zx);
 #pragma unroll
-        for (int i = 0; i < XROWS; i++)
-            *reinterpret_cast<uint4 *>(xd + ((tid >> 2) + 64 * i) * PITCH + x_kc * 16) = xr[i];
-        if (!g.w_kmajor) {
+        for (int i = 0; i < XROWS; i++) {
+            uint4 v = xr[i];
+            if (XMODE == X_TAP && ((xpad >> i) & 1u)) v = make_uint4(z, z, z, z);
+            *reinterpret_cast<uint4 *>(xd + ((tid >> 2) + 64 * i) * PITCH + x_kc * 16) = v;
+        }
+        if (WMODE == W_KMAJOR) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                if (c < BN * 4) *reinterpret_cast<uint4 *>(wd + (c / N16) * PW + (c % N16) * 16) = wr[i];
+            }
+        } else if (WMODE == W_ROWS || !g.w_kmajor) {
 #pragma unroll
             for (int i = 0; i < WCHUNKS; i++) {
                 const int c = tid + NTHREADS * i;
@@ -319,45 +442,74 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
     for (int i = 0; i < TM; i++) xsum[i] = 0;
 #pragma unroll
     for (int j = 0; j < TN; j++) wsum[j] = 0;
-    const bool need_xsum = g.zw != 0, need_wsum = g.zx != 0;
+    const bool need_xsum = SUMS && g.zw != 0, need_wsum = SUMS && g.zx != 0;
 
-    const int nk = (g.K + BK - 1) / BK;
-    prefetch(0);
-    stage(0);
-    __syncthreads();
-    for (int step = 0; step < nk; step++) {
-        const int cur = step & 1;
-        if (step + 1 < nk) prefetch((step + 1) * BK);
-        const char *xd = xs + cur * BM * PITCH + (wave_m * WM + (lane & 31)) * PITCH + (lane >> 5) * 16;
-        const char *wd = ws + cur * BN * PITCH + (wave_n * WN + (lane & 31)) * PITCH + (lane >> 5) * 16;
+    auto compute = [&](int buf) {
+        const char *xd = xs + buf * BM * PITCH + (wave_m * WM + (lane & 31)) * PITCH + (lane >> 5) * 16;
+        const char *wd = ws + buf * WBUF + (wave_n * WN + (lane & 31)) * PITCH + (lane >> 5) * 16;
+        // K-major tile: a 16-lane group transposes an 8(k) x 16(n) byte block; lane L of the group supplies the
+        // address of K row L / 2, channel half L % 2, and receives the 8 k-bytes of channel L.  Groups 0/1 cover
+        // channels 0-15 / 16-31 of the tile for k 0-15, groups 2/3 the same channels for k 16-31.
+        const char *wt = ws + buf * WBUF + ((lane >> 5) * 16 + ((lane & 15) >> 1)) * PW + wave_n * WN +
+                         ((lane >> 4) & 1) * 16 + (lane & 1) * 8;
 #pragma unroll
         for (int kk = 0; kk < BK / 32; kk++) {
             v4i xf[TM], wf[TN];
 #pragma unroll
             for (int i = 0; i < TM; i++) xf[i] = *reinterpret_cast<const v4i *>(xd + i * 32 * PITCH + kk * 32);
 #pragma unroll
-            for (int j = 0; j < TN; j++) wf[j] = *reinterpret_cast<const v4i *>(wd + j * 32 * PITCH + kk * 32);
+            for (int j = 0; j < TN; j++) {
+                if (WMODE == W_KMAJOR) {
+                    const char *p = wt + kk * 32 * PW + j * 32;
+                    const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(p));
+                    const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(p + 8 * PW));
+                    wf[j] = v4i{lo.x, lo.y, hi.x, hi.y};
+                } else {
+                    wf[j] = *reinterpret_cast<const v4i *>(wd + j * 32 * PITCH + kk * 32);
+                }
+            }
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
-            if (need_xsum) {
+            if (SUMS) {  // both sums are kept whenever a zero point is non-zero: 16 dot4 beside 8 MFMAs
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
                     for (int q = 0; q < 4; q++) xsum[i] = __builtin_amdgcn_sdot4(xf[i][q], 0x01010101, xsum[i], false);
-            }
-            if (need_wsum) {
 #pragma unroll
                 for (int j = 0; j < TN; j++)
 #pragma unroll
                     for (int q = 0; q < 4; q++) wsum[j] = __builtin_amdgcn_sdot4(wf[j][q], 0x01010101, wsum[j], false);
             }
         }
-        if (step + 1 < nk) stage(cur ^ 1);
+    };
+
+    // ---- main loop: two K steps of global loads in flight (register sets A and B), two LDS buffers.
+    // Invariant at the top of iteration `step` (even): LDS[0] holds step, set B holds step+1 (loads issued).
+    const int nk = (g.K + BK - 1) / BK;
+    uint4 xa[XROWS], wa[WCHUNKS], xb2[XROWS], wb2[WCHUNKS];
+    uint32_t pa = 0, pb = 0;
+    // Every prefetch and stage below is unconditional: a K step at or beyond K loads nothing (the buffer bounds /
+    // tap state return zeros) and is never multiplied, and straight-line code lets the compiler count exactly how
+    // many loads may stay in flight at each wait instead of draining them all.
+    prefetch(0, xa, wa, pa);
+    prefetch(BK, xb2, wb2, pb);
+    stage(0, xa, wa, pa);
+    __syncthreads();
+    int step = 0;
+    for (; step + 1 < nk; step += 2) {  // LDS[0] holds `step`, registers B hold `step + 1`
+        prefetch((step + 2) * BK, xa, wa, pa);
+        compute(0);
+        stage(1, xb2, wb2, pb);
+        __syncthreads();
+        prefetch((step + 3) * BK, xb2, wb2, pb);
+        compute(1);
+        stage(0, xa, wa, pa);
         __syncthreads();
     }
+    if (step < nk) compute(0);  // odd number of K steps: the last one sits in LDS[0]
 
     // ---- fold the zero-point terms that depend on the channel only into the per-channel bias
     if (need_wsum && wave_m == 0) {
@@ -366,13 +518,15 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
             const int32_t s = wsum[j] + __shfl_xor(wsum[j], 32);
             if (lane < 32) {
                 const int n = wave_n * WN + j * 32 + lane;
-                cp[n].bias_adj += -g.zx * s + g.K * g.zx * g.zw;
+                cp[n].bias_adj = (int32_t)((uint32_t)cp[n].bias_adj - (uint32_t)g.zx * (uint32_t)s +
+                                           (uint32_t)g.K * (uint32_t)g.zx * (uint32_t)g.zw);
             }
         }
     }
     if (need_xsum) {
 #pragma unroll
-        for (int i = 0; i < TM; i++) xsum[i] = (xsum[i] + __shfl_xor(xsum[i], 32)) * g.zw;
+        for (int i = 0; i < TM; i++)
+            xsum[i] = (int32_t)((uint32_t)(xsum[i] + __shfl_xor(xsum[i], 32)) * (uint32_t)g.zw);
     }
     __syncthreads();
 
@@ -394,10 +548,14 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
                 int32_t v[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const ChanParams c = cp[nl + e];
-                    int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)c.bias_adj - (uint32_t)xcorr);
-                    if (g.fused) a = requant_i32(a, c.mult, c.shift, g.rp);
-                    v[e] = a;
+                    const int32_t a =
+                        (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)cp[nl + e].bias_adj - (uint32_t)xcorr);
+                    if (!g.fused)
+                        v[e] = a;
+                    else if (g.rp.in_zp == 0)
+                        v[e] = requant_chan<true>(a, cp[nl + e].q, g.rp);
+                    else
+                        v[e] = requant_chan<false>(a, cp[nl + e].q, g.rp);
                 }
                 const int64_t off = (int64_t)m * g.ldo + n0;
                 if (g.out_vec_ok && n0 + 3 < g.N) {
@@ -431,11 +589,49 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
 
 template <int BM, int BN>
 constexpr size_t smem_bytes() {
-    return (size_t)2 * (BM + BN) * PITCH + (size_t)BN * sizeof(ChanParams);
+    return (size_t)2 * BM * PITCH + (size_t)2 * w_buf_bytes<BN>() + (size_t)BN * sizeof(ChanParams);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool SUMS>
+void launch_tile(const GemmArgs &g, int xmode, int wmode, dim3 grid, hipStream_t s) {
+    const size_t sm = smem_bytes<BM, BN>();
+    if (xmode == X_PLAIN && wmode == W_ROWS)
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_ROWS, SUMS><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    else if (xmode == X_TAP && wmode == W_ROWS)
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_TAP, W_ROWS, SUMS><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    else if (xmode == X_PLAIN && wmode == W_KMAJOR)
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR, SUMS><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    else
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_GENERIC, W_GENERIC, SUMS><<<grid, dim3(NTHREADS), sm, s>>>(g);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+void launch_tile_zp(const GemmArgs &g, int xmode, int wmode, dim3 grid, hipStream_t s) {
+    if (g.zx != 0 || g.zw != 0)
+        launch_tile<BM, BN, WAVES_M, WAVES_N, true>(g, xmode, wmode, grid, s);
+    else
+        launch_tile<BM, BN, WAVES_M, WAVES_N, false>(g, xmode, wmode, grid, s);
 }
 
 int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
     (void)ctx;
+    // operand fetch modes
+    int xmode = X_GENERIC, wmode = W_GENERIC;
+    const bool small = g.x_bytes != 0 && g.w_bytes != 0;  // both operand extents fit 31-bit buffer offsets
+    if (g.xch == 16 && small) {
+        if (g.plain)
+            xmode = X_PLAIN;
+        else if (g.IC % BK == 0)
+            xmode = X_TAP;
+    }
+    if (!g.w_kmajor && g.wch == 16 && small) wmode = W_ROWS;
+    if (g.w_kmajor && g.wch >= 4 && small) wmode = W_KMAJOR;
+    const bool fast = (xmode == X_PLAIN && wmode == W_ROWS) || (xmode == X_TAP && wmode == W_ROWS) ||
+                      (xmode == X_PLAIN && wmode == W_KMAJOR);
+    if (!fast) {
+        xmode = X_GENERIC;
+        wmode = W_GENERIC;
+    }
     // tile choice: least padded channel extent, larger tile on ties
     const int bn_opts[3] = {128, 64, 32};
     int best = 0;
@@ -456,16 +652,12 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
     g.total_tiles = (int)total;
     g.chunk = (int)((total + 7) / 8);
     const dim3 grid((unsigned)(g.chunk * 8));
-    if (BN == 128) {
-        const size_t sm = smem_bytes<128, 128>();
-        gemm_i8_kernel<128, 128, 2, 2><<<grid, dim3(NTHREADS), sm, s>>>(g);
-    } else if (BN == 64) {
-        const size_t sm = smem_bytes<256, 64>();
-        gemm_i8_kernel<256, 64, 4, 1><<<grid, dim3(NTHREADS), sm, s>>>(g);
-    } else {
-        const size_t sm = smem_bytes<256, 32>();
-        gemm_i8_kernel<256, 32, 4, 1><<<grid, dim3(NTHREADS), sm, s>>>(g);
-    }
+    if (BN == 128)
+        launch_tile_zp<128, 128, 2, 2>(g, xmode, wmode, grid, s);
+    else if (BN == 64)
+        launch_tile_zp<256, 64, 4, 1>(g, xmode, wmode, grid, s);
+    else
+        launch_tile_zp<256, 32, 4, 1>(g, xmode, wmode, grid, s);
     return check_launch("int8 contraction");
 }
 
@@ -545,6 +737,18 @@ int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     g.pad_l = a->pad[2];
     g.plain = 0;
     g.xch = align_of(in->ptr, IC, in->strides[0], in->strides[1], in->strides[2]);
+    // a 1x1, stride-1, unpadded convolution over a dense image is a plain [M][K] operand with the pixel pitch
+    if (KH == 1 && KW == 1 && a->stride[0] == 1 && a->stride[1] == 1 && a->pad[0] == 0 && a->pad[2] == 0 && OH == H &&
+        OW == W && in->strides[1] == W * in->strides[2] && in->strides[0] == H * in->strides[1]) {
+        g.plain = 1;
+        g.H = g.W = 1;
+        g.OHW = g.OW = 1;
+    }
+    {
+        const int64_t xb = in->dims[0] * in->strides[0], wbytes = (OC - 1) * w->strides[0] + K;
+        g.x_bytes = xb < (int64_t(1) << 31) ? (uint32_t)xb : 0;
+        g.w_bytes = wbytes < (int64_t(1) << 31) ? (uint32_t)wbytes : 0;
+    }
     g.w = static_cast<const int8_t *>(w->ptr);
     g.ldw = w->strides[0];
     g.w_kmajor = 0;
@@ -590,11 +794,16 @@ int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     g.sy = g.sx = g.dy = g.dx = 1;
     g.plain = 1;
     g.xch = align_of(A->ptr, K, A->strides[0], A->strides[1]);
+    {
+        const int64_t xb = (M - 1) * A->strides[1] + K, wbytes = (K - 1) * B->strides[1] + N;
+        g.x_bytes = xb < (int64_t(1) << 31) ? (uint32_t)xb : 0;
+        g.w_bytes = wbytes < (int64_t(1) << 31) ? (uint32_t)wbytes : 0;
+    }
     g.w = static_cast<const int8_t *>(B->ptr);
     g.w_batch = B->strides[0];
     g.ldw = B->strides[1];
     g.w_kmajor = 1;
-    g.wch = align_of(B->ptr, N, B->strides[0], B->strides[1]) >= 4 ? 4 : 1;
+    g.wch = align_of(B->ptr, N, B->strides[0], B->strides[1]);
     g.zx = attr->a_zp;
     g.zw = attr->b_zp;
     g.bias = nullptr;
