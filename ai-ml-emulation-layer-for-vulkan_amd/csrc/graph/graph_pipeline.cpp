@@ -1,0 +1,804 @@
+#include "graph_pipeline.hpp"
+
+#include <algorithm>
+#include <cstring>
+
+#include "session_planner.hpp"
+
+namespace mlel::graph {
+
+namespace {
+
+[[noreturn]] void fail(const std::string &what) { throw std::runtime_error(what); }
+
+void check(int rc, const char *what) {
+    if (rc != 0) fail(std::string(what) + ": " + mlel_hip_last_error());
+}
+
+std::vector<int64_t> packedStrides(int32_t dtype, const std::vector<int64_t> &dims) {
+    // reference: tensor/tensor_arm.cpp:82-92
+    std::vector<int64_t> s(dims.size());
+    int64_t v = static_cast<int64_t>(dtypeSize(dtype));
+    for (size_t i = dims.size(); i-- > 0;) {
+        s[i] = v;
+        v *= dims[i];
+    }
+    return s;
+}
+
+}  // namespace
+
+mlel_dtype dtypeFromVkFormat(const int32_t f) {
+    switch (f) {
+    case VK_FORMAT_R8_SINT: return MLEL_I8;
+    case VK_FORMAT_R8_UINT:
+    case VK_FORMAT_S8_UINT: return MLEL_U8;
+    case VK_FORMAT_R8_BOOL_ARM: return MLEL_BOOL;
+    case VK_FORMAT_R16_SINT: return MLEL_I16;
+    case VK_FORMAT_R16_UINT: return MLEL_U16;
+    case VK_FORMAT_R16_SFLOAT: return MLEL_F16;
+    case VK_FORMAT_R32_SINT: return MLEL_I32;
+    case VK_FORMAT_R32_UINT: return MLEL_U32;
+    case VK_FORMAT_R32_SFLOAT: return MLEL_F32;
+    case VK_FORMAT_R64_SINT: return MLEL_I64;
+    case VK_FORMAT_R64_UINT: return MLEL_U64;
+    case VK_FORMAT_R64_SFLOAT: return MLEL_F64;
+    default: fail("Unsupported tensor buffer format: " + std::to_string(f));
+    }
+}
+
+size_t dtypeSize(const int32_t dtype) {
+    switch (dtype) {
+    case MLEL_BOOL: case MLEL_I8: case MLEL_U8: case MLEL_F8E4M3: case MLEL_F8E5M2: return 1;
+    case MLEL_I16: case MLEL_U16: case MLEL_F16: case MLEL_BF16: return 2;
+    case MLEL_I32: case MLEL_U32: case MLEL_F32: return 4;
+    case MLEL_I64: case MLEL_U64: case MLEL_F64: return 8;
+    default: fail("Unsupported tensor element type: " + std::to_string(dtype));
+    }
+}
+
+/*******************************************************************************
+ * TensorDescriptor
+ *******************************************************************************/
+
+TensorDescriptor::TensorDescriptor(const int32_t _dtype, std::vector<int64_t> _dimensions,
+                                   std::vector<int64_t> _strides, const TensorKind _kind)
+    : dtype{_dtype}, dimensions{std::move(_dimensions)}, strides{std::move(_strides)}, kind{_kind} {
+    (void)dtypeSize(dtype);
+    if (dimensions.empty() || dimensions.size() > MLEL_MAX_RANK)
+        fail("Tensor rank must be between 1 and " + std::to_string(MLEL_MAX_RANK));
+    if (strides.empty()) strides = packedStrides(dtype, dimensions);
+    if (strides.size() != dimensions.size()) fail("Tensor strides and dimensions differ in length");
+    if (strides[0] < 0) fail("Strides must be greater than zero.");
+}
+
+size_t TensorDescriptor::getShapeSize() const {
+    size_t n = 1;
+    for (const auto d : dimensions) n *= static_cast<size_t>(d);
+    return n;
+}
+
+size_t TensorDescriptor::getSize() const { return static_cast<size_t>(dimensions[0] * strides[0]); }
+
+bool TensorDescriptor::isPacked() const { return strides == packedStrides(dtype, dimensions); }
+
+mlel_tensor TensorDescriptor::view() const {
+    mlel_tensor t{};
+    t.ptr = ptr;
+    t.dtype = dtype;
+    t.rank = static_cast<int32_t>(dimensions.size());
+    for (size_t i = 0; i < dimensions.size(); i++) {
+        t.dims[i] = dimensions[i];
+        t.strides[i] = strides[i];
+    }
+    return t;
+}
+
+/*******************************************************************************
+ * GraphPipeline: tensors
+ *******************************************************************************/
+
+// A null context is accepted for building and planning a graph (host-side logic needs no device); constants are
+// then not uploaded and dispatch() refuses to run.
+GraphPipeline::GraphPipeline(mlel_ctx *_ctx) : ctx{_ctx} {}
+
+GraphPipeline::~GraphPipeline() {
+    if (ctx != nullptr)
+        for (void *p : constantsDeviceMemory) (void)mlel_hip_arena_free(ctx, p);
+}
+
+TensorPtr GraphPipeline::registerTensor(TensorPtr t) {
+    t->id = static_cast<int>(allTensors.size());
+    allTensors.push_back(t);
+    return t;
+}
+
+void *GraphPipeline::uploadConstant(const TensorDescriptor &t, const void *data) {
+    if (data == nullptr || ctx == nullptr) return nullptr;  // reference: null data -> VK_NULL_HANDLE
+    void *dptr = nullptr;
+    check(mlel_hip_arena_alloc(ctx, t.getSize(), &dptr), "allocating constant tensor");
+    constantsDeviceMemory.push_back(dptr);
+    check(mlel_hip_memcpy_h2d(ctx, dptr, data, t.getSize(), nullptr), "uploading constant tensor");
+    return dptr;
+}
+
+void GraphPipeline::makeConstTensor(const uint32_t id, const int32_t dtype, const std::vector<int64_t> &dimensions,
+                                    const std::vector<int64_t> &strides, const void *data) {
+    auto t = std::make_shared<TensorDescriptor>(dtype, dimensions, strides, TensorKind::Constant);
+    t->bind(uploadConstant(*t, data));
+    constTensorMap[id] = registerTensor(std::move(t));
+}
+
+TensorPtr GraphPipeline::getConstTensor(const uint32_t id) const { return constTensorMap.at(id); }
+
+TensorPtr GraphPipeline::makeConstCompositeTensor(const int32_t dtype, std::vector<int64_t> dimensions,
+                                                  const void *data) {
+    auto t = std::make_shared<TensorDescriptor>(dtype, std::move(dimensions), std::vector<int64_t>{},
+                                                TensorKind::Constant);
+    t->bind(uploadConstant(*t, data));
+    compositeTensors.push_back(registerTensor(t));
+    return t;
+}
+
+void GraphPipeline::makeDescriptorSetBinding(const uint32_t set, const uint32_t binding, const uint32_t arrayIndex,
+                                             const int32_t dtype, const std::vector<int64_t> &dimensions,
+                                             const std::vector<int64_t> &strides) {
+    auto t = std::make_shared<TensorDescriptor>(dtype, dimensions, strides, TensorKind::External);
+    auto &vec = tensorMap[set][binding];
+    vec.resize(std::max(vec.size(), static_cast<size_t>(arrayIndex) + 1));
+    vec[arrayIndex] = registerTensor(std::move(t));
+}
+
+TensorPtr GraphPipeline::getTensor(const uint32_t set, const uint32_t binding, const uint32_t arrayIndex) const {
+    return tensorMap.at(set).at(binding).at(arrayIndex);
+}
+
+TensorPtr GraphPipeline::makeTensor(const int32_t dtype, std::vector<int64_t> dimensions,
+                                    std::vector<int64_t> strides) {
+    auto t = std::make_shared<TensorDescriptor>(dtype, std::move(dimensions), std::move(strides), TensorKind::Session);
+    if (tensorSet.insert(t).second) tensors.push_back(t);
+    return registerTensor(t);
+}
+
+void GraphPipeline::makeInput(const TensorPtr &tensor) {
+    tensor->isGraphInput = true;
+    inputs.push_back(tensor);
+}
+
+void GraphPipeline::makeOutput(const TensorPtr &tensor) {
+    tensor->isGraphOutput = true;
+    outputs.push_back(tensor);
+}
+
+/*******************************************************************************
+ * GraphPipeline: operators
+ *******************************************************************************/
+
+std::shared_ptr<OpNode> GraphPipeline::addOp(const OpKind kind, const char *tosaName, const std::string &debugName,
+                                             std::vector<TensorPtr> ins, std::vector<TensorPtr> outs) {
+    if (finalized) fail("GraphPipeline is finalized; no more operators can be added");
+    for (const auto &t : ins)
+        if (!t) fail(std::string(tosaName) + ": null input tensor");
+    for (const auto &t : outs)
+        if (!t) fail(std::string(tosaName) + ": null output tensor");
+    auto op = std::make_shared<OpNode>();
+    op->kind = kind;
+    op->tosaName = tosaName;
+    op->debugName = debugName;
+    op->inputs = std::move(ins);
+    op->outputs = std::move(outs);
+    for (const auto &t : op->outputs) t->setProducer(op.get());
+    for (const auto &t : op->inputs) op->originalTensors.push_back(t.get());
+    for (const auto &t : op->outputs) op->originalTensors.push_back(t.get());
+    ops.push_back(op);
+    return op;
+}
+
+void GraphPipeline::unsupported(const char *tosaName) const {
+    fail(std::string("TOSA operator ") + tosaName + " has no kernel on the HIP backend yet");
+}
+
+namespace {
+
+mlel_conv2d_attr convAttr(const std::vector<int32_t> &pad, const std::vector<int32_t> &stride,
+                          const std::vector<int32_t> &dilation, const int8_t zi, const int8_t zw,
+                          const uint32_t accType) {
+    if (pad.size() < 4 || stride.size() < 2 || dilation.size() < 2)
+        fail("convolution: pad/stride/dilation need 4/2/2 values");
+    if (accType < 1 || accType > 4) fail("Unsupported acc type " + std::to_string(accType));
+    mlel_conv2d_attr a{};
+    a.input_zp = zi;
+    a.weight_zp = zw;
+    for (int i = 0; i < 4; i++) a.pad[i] = pad[static_cast<size_t>(i)];
+    for (int i = 0; i < 2; i++) {
+        a.stride[i] = stride[static_cast<size_t>(i)];
+        a.dilation[i] = dilation[static_cast<size_t>(i)];
+    }
+    a.acc_type = accType;
+    return a;
+}
+
+mlel_pool2d_attr poolAttr(const std::vector<int32_t> &kernel, const std::vector<int32_t> &stride,
+                          const std::vector<int32_t> &pad) {
+    if (kernel.size() < 2 || stride.size() < 2 || pad.size() < 4) fail("pooling: kernel/stride/pad need 2/2/4 values");
+    mlel_pool2d_attr a{};
+    for (int i = 0; i < 2; i++) {
+        a.kernel[i] = kernel[static_cast<size_t>(i)];
+        a.stride[i] = stride[static_cast<size_t>(i)];
+    }
+    for (int i = 0; i < 4; i++) a.pad[i] = pad[static_cast<size_t>(i)];
+    a.acc_type = MLEL_ACC_I32;
+    a.nan_mode = MLEL_NAN_PROPAGATE;
+    return a;
+}
+
+}  // namespace
+
+void GraphPipeline::makeBinary(const int32_t op, const char *name, const TensorPtr &a, const TensorPtr &b,
+                               const TensorPtr &out, const uint32_t nanMode, const std::string &debugName) {
+    auto n = addOp(OpKind::Binary, name, debugName, {a, b}, {out});
+    n->selector = op;
+    n->nanMode = nanMode;
+}
+
+void GraphPipeline::makeUnary(const int32_t op, const char *name, const TensorPtr &in, const TensorPtr &out,
+                              const std::string &debugName) {
+    addOp(OpKind::Unary, name, debugName, {in}, {out})->selector = op;
+}
+
+void GraphPipeline::makeReduce(const int32_t op, const char *name, const TensorPtr &in, const TensorPtr &out,
+                               const uint32_t axis, const uint32_t nanMode, const std::string &debugName) {
+    auto n = addOp(OpKind::Reduce, name, debugName, {in}, {out});
+    n->selector = op;
+    n->axis = axis;
+    n->nanMode = nanMode;
+}
+
+#define MLEL_UNARY(Method, Enum, Name)                                                                                 \
+    void GraphPipeline::Method(const TensorPtr &i, const TensorPtr &o, const std::string &d) {                        \
+        makeUnary(Enum, Name, i, o, d);                                                                                \
+    }
+MLEL_UNARY(makeAbs, MLEL_UN_ABS, "ABS")
+MLEL_UNARY(makeBitwiseNot, MLEL_UN_BITWISE_NOT, "BITWISE_NOT")
+MLEL_UNARY(makeCeil, MLEL_UN_CEIL, "CEIL")
+MLEL_UNARY(makeClz, MLEL_UN_CLZ, "CLZ")
+MLEL_UNARY(makeCos, MLEL_UN_COS, "COS")
+MLEL_UNARY(makeErf, MLEL_UN_ERF, "ERF")
+MLEL_UNARY(makeExp, MLEL_UN_EXP, "EXP")
+MLEL_UNARY(makeFloor, MLEL_UN_FLOOR, "FLOOR")
+MLEL_UNARY(makeLog, MLEL_UN_LOG, "LOG")
+MLEL_UNARY(makeLogicalNot, MLEL_UN_LOGICAL_NOT, "LOGICAL_NOT")
+MLEL_UNARY(makeReciprocal, MLEL_UN_RECIPROCAL, "RECIPROCAL")
+MLEL_UNARY(makeRsqrt, MLEL_UN_RSQRT, "RSQRT")
+MLEL_UNARY(makeSigmoid, MLEL_UN_SIGMOID, "SIGMOID")
+MLEL_UNARY(makeSin, MLEL_UN_SIN, "SIN")
+MLEL_UNARY(makeTanh, MLEL_UN_TANH, "TANH")
+#undef MLEL_UNARY
+
+#define MLEL_BINARY(Method, Enum, Name)                                                                                \
+    void GraphPipeline::Method(const TensorPtr &a, const TensorPtr &b, const TensorPtr &o, const std::string &d) {    \
+        makeBinary(Enum, Name, a, b, o, MLEL_NAN_PROPAGATE, d);                                                        \
+    }
+MLEL_BINARY(makeAdd, MLEL_BIN_ADD, "ADD")
+MLEL_BINARY(makeSub, MLEL_BIN_SUB, "SUB")
+MLEL_BINARY(makeBitwiseAnd, MLEL_BIN_BITWISE_AND, "BITWISE_AND")
+MLEL_BINARY(makeBitwiseOr, MLEL_BIN_BITWISE_OR, "BITWISE_OR")
+MLEL_BINARY(makeBitwiseXor, MLEL_BIN_BITWISE_XOR, "BITWISE_XOR")
+MLEL_BINARY(makeIntdiv, MLEL_BIN_INTDIV, "INTDIV")
+MLEL_BINARY(makeLogicalAnd, MLEL_BIN_LOGICAL_AND, "LOGICAL_AND")
+MLEL_BINARY(makeLogicalOr, MLEL_BIN_LOGICAL_OR, "LOGICAL_OR")
+MLEL_BINARY(makeLogicalXor, MLEL_BIN_LOGICAL_XOR, "LOGICAL_XOR")
+MLEL_BINARY(makeLogicalLeftShift, MLEL_BIN_LOGICAL_LEFT_SHIFT, "LOGICAL_LEFT_SHIFT")
+MLEL_BINARY(makeLogicalRightShift, MLEL_BIN_LOGICAL_RIGHT_SHIFT, "LOGICAL_RIGHT_SHIFT")
+MLEL_BINARY(makePow, MLEL_BIN_POW, "POW")
+MLEL_BINARY(makeEqual, MLEL_BIN_EQUAL, "EQUAL")
+MLEL_BINARY(makeGreater, MLEL_BIN_GREATER, "GREATER")
+MLEL_BINARY(makeGreaterEqual, MLEL_BIN_GREATER_EQUAL, "GREATER_EQUAL")
+#undef MLEL_BINARY
+
+void GraphPipeline::makeMaximum(const TensorPtr &a, const TensorPtr &b, const TensorPtr &o, const uint32_t nanMode,
+                                const std::string &d) {
+    makeBinary(MLEL_BIN_MAXIMUM, "MAXIMUM", a, b, o, nanMode, d);
+}
+void GraphPipeline::makeMinimum(const TensorPtr &a, const TensorPtr &b, const TensorPtr &o, const uint32_t nanMode,
+                                const std::string &d) {
+    makeBinary(MLEL_BIN_MINIMUM, "MINIMUM", a, b, o, nanMode, d);
+}
+
+void GraphPipeline::makeReduceAll(const TensorPtr &i, const TensorPtr &o, const uint32_t axis, const std::string &d) {
+    makeReduce(MLEL_RED_ALL, "REDUCE_ALL", i, o, axis, MLEL_NAN_PROPAGATE, d);
+}
+void GraphPipeline::makeReduceAny(const TensorPtr &i, const TensorPtr &o, const uint32_t axis, const std::string &d) {
+    makeReduce(MLEL_RED_ANY, "REDUCE_ANY", i, o, axis, MLEL_NAN_PROPAGATE, d);
+}
+void GraphPipeline::makeReduceMax(const TensorPtr &i, const TensorPtr &o, const uint32_t axis, const uint32_t nanMode,
+                                  const std::string &d) {
+    makeReduce(MLEL_RED_MAX, "REDUCE_MAX", i, o, axis, nanMode, d);
+}
+void GraphPipeline::makeReduceMin(const TensorPtr &i, const TensorPtr &o, const uint32_t axis, const uint32_t nanMode,
+                                  const std::string &d) {
+    makeReduce(MLEL_RED_MIN, "REDUCE_MIN", i, o, axis, nanMode, d);
+}
+void GraphPipeline::makeReduceProduct(const TensorPtr &i, const TensorPtr &o, const uint32_t axis,
+                                      const std::string &d) {
+    makeReduce(MLEL_RED_PRODUCT, "REDUCE_PRODUCT", i, o, axis, MLEL_NAN_PROPAGATE, d);
+}
+void GraphPipeline::makeReduceSum(const TensorPtr &i, const TensorPtr &o, const uint32_t axis, const std::string &d) {
+    makeReduce(MLEL_RED_SUM, "REDUCE_SUM", i, o, axis, MLEL_NAN_PROPAGATE, d);
+}
+
+void GraphPipeline::makeAvgPool2D(const TensorPtr &input, const TensorPtr &output, const std::vector<int32_t> &kernel,
+                                  const std::vector<int32_t> &stride, const std::vector<int32_t> &pad,
+                                  const uint32_t accType, const int8_t inputZeroPoint, const int8_t outputZeroPoint,
+                                  const std::string &debugName) {
+    if (accType < 1 || accType > 4) fail("Unsupported AVG_POOL2D acc type " + std::to_string(accType));
+    auto n = addOp(OpKind::AvgPool2D, "AVG_POOL2D", debugName, {input}, {output});
+    n->pool = poolAttr(kernel, stride, pad);
+    n->pool.acc_type = accType;
+    n->pool.input_zp = inputZeroPoint;
+    n->pool.output_zp = outputZeroPoint;
+}
+
+void GraphPipeline::makeMaxPool2D(const TensorPtr &input, const TensorPtr &output, const std::vector<int32_t> &kernel,
+                                  const std::vector<int32_t> &stride, const std::vector<int32_t> &pad,
+                                  const uint32_t nanMode, const std::string &debugName) {
+    auto n = addOp(OpKind::MaxPool2D, "MAX_POOL2D", debugName, {input}, {output});
+    n->pool = poolAttr(kernel, stride, pad);
+    n->pool.nan_mode = nanMode;
+}
+
+void GraphPipeline::makeCast(const TensorPtr &input, const TensorPtr &output, const std::string &debugName) {
+    addOp(OpKind::Cast, "CAST", debugName, {input}, {output});
+}
+
+void GraphPipeline::makeClamp(const TensorPtr &input, const TensorPtr &output, const real_t min, const real_t max,
+                              const uint32_t nanMode, const std::string &debugName) {
+    auto n = addOp(OpKind::Clamp, "CLAMP", debugName, {input}, {output});
+    n->clamp = mlel_clamp_attr{min, max, nanMode};
+}
+
+void GraphPipeline::makeConcat(const std::vector<TensorPtr> &_inputs, const TensorPtr &output, const uint32_t axis,
+                               const std::string &debugName) {
+    // one operator per input with a running offset along `axis` (reference: compute_graph_op.cpp:2607-2615)
+    uint32_t offset = 0;
+    for (const auto &input : _inputs) {
+        auto n = addOp(OpKind::Concat, "CONCAT", debugName, {input}, {output});
+        n->axis = axis;
+        n->offset = offset;
+        if (axis >= input->getRank()) fail("CONCAT: axis outside the input rank");
+        offset += static_cast<uint32_t>(input->getDimensions()[axis]);
+    }
+}
+
+void GraphPipeline::makeConv2D(const TensorPtr &input, const TensorPtr &output, const TensorPtr &weights,
+                               const TensorPtr &biases, const std::vector<int32_t> &pad,
+                               const std::vector<int32_t> &stride, const std::vector<int32_t> &dilation,
+                               const int8_t inputZeroPoint, const int8_t weightZeroPoint, const uint32_t accType,
+                               const std::string &debugName) {
+    const auto attr = convAttr(pad, stride, dilation, inputZeroPoint, weightZeroPoint, accType);
+    addOp(OpKind::Conv2D, "CONV2D", debugName, {input, weights, biases}, {output})->conv = attr;
+}
+
+void GraphPipeline::makeDepthwiseConv2D(const TensorPtr &input, const TensorPtr &output, const TensorPtr &weights,
+                                        const TensorPtr &biases, const std::vector<int32_t> &pad,
+                                        const std::vector<int32_t> &stride, const std::vector<int32_t> &dilation,
+                                        const int8_t inputZeroPoint, const int8_t weightZeroPoint,
+                                        const uint32_t accType, const std::string &debugName) {
+    const auto attr = convAttr(pad, stride, dilation, inputZeroPoint, weightZeroPoint, accType);
+    addOp(OpKind::DepthwiseConv2D, "DEPTHWISE_CONV2D", debugName, {input, weights, biases}, {output})->conv = attr;
+}
+
+void GraphPipeline::makeMatmul(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                               const int32_t inputZeroPoint1, const int32_t inputZeroPoint2,
+                               const std::string &debugName) {
+    addOp(OpKind::Matmul, "MATMUL", debugName, {input1, input2}, {output})->matmul =
+        mlel_matmul_attr{inputZeroPoint1, inputZeroPoint2};
+}
+
+void GraphPipeline::makeMul(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                            const uint32_t shift, const std::string &debugName) {
+    addOp(OpKind::Mul, "MUL", debugName, {input1, input2}, {output})->shift = shift;
+}
+
+void GraphPipeline::makeNegate(const TensorPtr &input, const TensorPtr &output, const int32_t inputZeroPoint,
+                               const int32_t outputZeroPoint, const std::string &debugName) {
+    auto n = addOp(OpKind::Negate, "NEGATE", debugName, {input}, {output});
+    n->inputZeroPoint = inputZeroPoint;
+    n->outputZeroPoint = outputZeroPoint;
+}
+
+void GraphPipeline::makePad(const TensorPtr &input, const TensorPtr &output, const TensorPtr &padding,
+                            const real_t padConst, const int32_t padConstInt, const std::string &debugName) {
+    auto n = addOp(OpKind::Pad, "PAD", debugName, {input, padding}, {output});
+    n->padConst = padConst;
+    n->padConstInt = padConstInt;
+}
+
+void GraphPipeline::makeRescale(const TensorPtr &input, const TensorPtr &output, const int32_t inputZeroPoint,
+                                const int32_t outputZeroPoint, const TensorPtr &multiplier, const TensorPtr &shift,
+                                const bool scale32, const bool doubleRound, const bool perChannel,
+                                const bool inputUnsigned, const bool outputUnsigned, const std::string &debugName) {
+    auto n = addOp(OpKind::Rescale, "RESCALE", debugName, {input, multiplier, shift}, {output});
+    n->rescale = mlel_rescale_attr{inputZeroPoint, outputZeroPoint, scale32, doubleRound, perChannel,
+                                   inputUnsigned,  outputUnsigned};
+}
+
+void GraphPipeline::makeReshape(const TensorPtr &input, const TensorPtr &output, const std::string &debugName) {
+    addOp(OpKind::Reshape, "RESHAPE", debugName, {input}, {output});
+}
+
+void GraphPipeline::makeSlice(const TensorPtr &input, const TensorPtr &output, const std::vector<uint32_t> &start,
+                              const std::string &debugName) {
+    auto n = addOp(OpKind::Slice, "SLICE", debugName, {input}, {output});
+    if (start.size() < input->getRank()) fail("SLICE: start has fewer values than the tensor rank");
+    for (uint32_t i = 0; i < input->getRank(); i++) n->vec[i] = start[i];
+}
+
+void GraphPipeline::makeTable(const TensorPtr &input, const TensorPtr &output, const TensorPtr &table,
+                              const std::string &debugName) {
+    addOp(OpKind::Table, "TABLE", debugName, {input, table}, {output});
+}
+
+void GraphPipeline::makeTranspose(const TensorPtr &input, const TensorPtr &output, const std::vector<uint32_t> &perms,
+                                  const std::string &debugName) {
+    auto n = addOp(OpKind::Transpose, "TRANSPOSE", debugName, {input}, {output});
+    if (perms.size() < input->getRank()) fail("TRANSPOSE: perms has fewer values than the tensor rank");
+    for (uint32_t i = 0; i < input->getRank(); i++) n->vec[i] = perms[i];
+}
+
+// operators of the reference's surface that have no HIP kernel yet: the call fails like an unknown operator does in
+// the reference's decoder (graph_tosa_1_0_ext_inst.cpp:311)
+void GraphPipeline::makeArgmax(const TensorPtr &, const TensorPtr &, uint32_t, uint32_t, const std::string &) {
+    unsupported("ARGMAX");
+}
+void GraphPipeline::makeArithmeticRightShift(const TensorPtr &, const TensorPtr &, const TensorPtr &, bool,
+                                             const std::string &) {
+    unsupported("ARITHMETIC_RIGHT_SHIFT");
+}
+void GraphPipeline::makeConv3D(const TensorPtr &, const TensorPtr &, const TensorPtr &, const TensorPtr &,
+                               const std::vector<int32_t> &, const std::vector<int32_t> &, const std::vector<int32_t> &,
+                               int8_t, int8_t, uint32_t, const std::string &) {
+    unsupported("CONV3D");
+}
+void GraphPipeline::makeFft2D(const TensorPtr &, const TensorPtr &, const TensorPtr &, const TensorPtr &, bool,
+                              const std::string &) {
+    unsupported("FFT2D");
+}
+void GraphPipeline::makeGather(const TensorPtr &, const TensorPtr &, const TensorPtr &, const std::string &) {
+    unsupported("GATHER");
+}
+void GraphPipeline::makeResize(const TensorPtr &, const TensorPtr &, const std::vector<int32_t> &,
+                               const std::vector<int32_t> &, const std::vector<int32_t> &, uint32_t,
+                               const std::string &) {
+    unsupported("RESIZE");
+}
+void GraphPipeline::makeReverse(const TensorPtr &, const TensorPtr &, uint32_t, const std::string &) {
+    unsupported("REVERSE");
+}
+void GraphPipeline::makeRfft2D(const TensorPtr &, const TensorPtr &, const TensorPtr &, const std::string &) {
+    unsupported("RFFT2D");
+}
+void GraphPipeline::makeScatter(const TensorPtr &, const TensorPtr &, const TensorPtr &, const TensorPtr &,
+                                const std::string &) {
+    unsupported("SCATTER");
+}
+void GraphPipeline::makeSelect(const TensorPtr &, const TensorPtr &, const TensorPtr &, const TensorPtr &,
+                               const std::string &) {
+    unsupported("SELECT");
+}
+void GraphPipeline::makeTile(const TensorPtr &, const TensorPtr &, const std::string &) { unsupported("TILE"); }
+void GraphPipeline::makeTransposeConv2D(const TensorPtr &, const TensorPtr &, const TensorPtr &, const TensorPtr &,
+                                        const std::vector<int32_t> &, const std::vector<int32_t> &, int8_t, int8_t,
+                                        uint32_t, const std::string &) {
+    unsupported("TRANSPOSE_CONV2D");
+}
+
+/*******************************************************************************
+ * GraphPipeline: fusion
+ *******************************************************************************/
+
+namespace {
+
+// operators (not folded away) that read `t`
+std::vector<OpNode *> consumersOf(const std::vector<std::shared_ptr<OpNode>> &ops, const TensorDescriptor *t) {
+    std::vector<OpNode *> r;
+    for (const auto &op : ops) {
+        if (op->fusedAway) continue;
+        for (const auto &in : op->inputs)
+            if (in.get() == t) {
+                r.push_back(op.get());
+                break;
+            }
+    }
+    return r;
+}
+
+bool sameShape(const TensorDescriptor &a, const TensorDescriptor &b) { return a.getDimensions() == b.getDimensions(); }
+
+// an intermediate may disappear only if nothing outside the fused group can observe it
+bool isPrivateIntermediate(const TensorDescriptor &t) {
+    return t.getKind() == TensorKind::Session && !t.isGraphOutput && !t.isGraphInput && t.isPacked();
+}
+
+bool scaleTensorsOk(const OpNode &rescale) {
+    const auto &m = rescale.inputs[1], &s = rescale.inputs[2];
+    // read at the fused node's (earlier) position: they must not be produced inside the graph
+    if (m->getKind() == TensorKind::Session || s->getKind() == TensorKind::Session) return false;
+    return m->getRank() == 1 && s->getRank() == 1 && m->isPacked() && s->isPacked() &&
+           m->getFormat() == (rescale.rescale.scale32 ? MLEL_I32 : MLEL_I16) && s->getFormat() == MLEL_I8;
+}
+
+bool isSmallInt(int32_t dt) { return dt == MLEL_I8 || dt == MLEL_I16 || dt == MLEL_I32; }
+
+}  // namespace
+
+void GraphPipeline::fuse() {
+    // Pattern 1: CONV2D | DEPTHWISE_CONV2D | MATMUL (int8 x int8 -> int32)  ->  RESCALE  [-> CLAMP]
+    // Legal when the int32 accumulator tensor (and, for the CLAMP, the RESCALE result) is a private intermediate
+    // with exactly one consumer.  The fused kernels compute exactly RESCALE(CLAMP) of the int32 accumulator, so the
+    // result is bit-identical to the three operators run one after another.
+    for (const auto &opPtr : ops) {
+        OpNode &op = *opPtr;
+        if (op.fusedAway) continue;
+        const bool isConv = op.kind == OpKind::Conv2D, isDw = op.kind == OpKind::DepthwiseConv2D,
+                   isMm = op.kind == OpKind::Matmul;
+        if (!isConv && !isDw && !isMm) continue;
+        const auto &acc = op.outputs[0];
+        if (acc->getFormat() != MLEL_I32 || op.inputs[0]->getFormat() != MLEL_I8 ||
+            op.inputs[1]->getFormat() != MLEL_I8 || !isPrivateIntermediate(*acc))
+            continue;
+        if (!isMm && op.conv.acc_type != MLEL_ACC_I32) continue;
+        const auto users = consumersOf(ops, acc.get());
+        if (users.size() != 1 || users[0]->kind != OpKind::Rescale || users[0]->inputs[0].get() != acc.get()) continue;
+        OpNode &rs = *users[0];
+        const auto &rsOut = rs.outputs[0];
+        if (!isSmallInt(rsOut->getFormat()) || !sameShape(*acc, *rsOut) || !rsOut->isPacked() || !scaleTensorsOk(rs) ||
+            rs.rescale.input_unsigned)
+            continue;
+        // optional CLAMP
+        OpNode *clamp = nullptr;
+        if (isPrivateIntermediate(*rsOut) && !rs.rescale.output_unsigned) {
+            const auto rsUsers = consumersOf(ops, rsOut.get());
+            if (rsUsers.size() == 1 && rsUsers[0]->kind == OpKind::Clamp &&
+                rsUsers[0]->outputs[0]->getFormat() == rsOut->getFormat() && sameShape(*rsOut, *rsUsers[0]->outputs[0]) &&
+                rsUsers[0]->outputs[0]->isPacked() && rsUsers[0]->clamp.min_val <= rsUsers[0]->clamp.max_val)
+                clamp = rsUsers[0];
+        }
+        op.kind = isConv ? OpKind::FusedConv2D : (isDw ? OpKind::FusedDepthwiseConv2D : OpKind::FusedMatmul);
+        op.epilogue = RescaleSpec{rs.inputs[1], rs.inputs[2], rs.rescale};
+        rs.fusedAway = true;
+        TensorPtr finalOut = rsOut;
+        if (clamp) {
+            op.hasClamp = true;
+            op.clamp = clamp->clamp;
+            clamp->fusedAway = true;
+            finalOut = clamp->outputs[0];
+        }
+        op.outputs[0] = finalOut;
+        finalOut->setProducer(&op);
+    }
+
+    // Pattern 2 (residual add): RESCALE(a -> i32), RESCALE(b -> i32), ADD(i32), RESCALE(-> i8/i16/i32)
+    for (const auto &opPtr : ops) {
+        OpNode &add = *opPtr;
+        if (add.fusedAway || add.kind != OpKind::Binary || add.selector != MLEL_BIN_ADD) continue;
+        const auto &sum = add.outputs[0];
+        if (sum->getFormat() != MLEL_I32 || !isPrivateIntermediate(*sum)) continue;
+        OpNode *ra = add.inputs[0]->getProducer(), *rb = add.inputs[1]->getProducer();
+        if (!ra || !rb || ra == rb || ra->fusedAway || rb->fusedAway || ra->kind != OpKind::Rescale ||
+            rb->kind != OpKind::Rescale)
+            continue;
+        const auto &ta = add.inputs[0], &tb = add.inputs[1];
+        if (!isPrivateIntermediate(*ta) || !isPrivateIntermediate(*tb) || ta->getFormat() != MLEL_I32 ||
+            tb->getFormat() != MLEL_I32 || !sameShape(*ta, *sum) || !sameShape(*tb, *sum))
+            continue;
+        if (consumersOf(ops, ta.get()).size() != 1 || consumersOf(ops, tb.get()).size() != 1) continue;
+        const auto users = consumersOf(ops, sum.get());
+        if (users.size() != 1 || users[0]->kind != OpKind::Rescale || users[0]->inputs[0].get() != sum.get()) continue;
+        OpNode &ro = *users[0];
+        if (!isSmallInt(ro.outputs[0]->getFormat()) || !sameShape(*sum, *ro.outputs[0]) || !scaleTensorsOk(*ra) ||
+            !scaleTensorsOk(*rb) || !scaleTensorsOk(ro) || ro.rescale.input_unsigned ||
+            !sameShape(*ra->inputs[0], *sum) || !sameShape(*rb->inputs[0], *sum) ||
+            !isSmallInt(ra->inputs[0]->getFormat()) || !isSmallInt(rb->inputs[0]->getFormat()))
+            continue;
+        // the fused node takes the place of the ADD (all three producers precede it in creation order)
+        add.kind = OpKind::FusedRescaleAddRescale;
+        add.scaleA = RescaleSpec{ra->inputs[1], ra->inputs[2], ra->rescale};
+        add.scaleB = RescaleSpec{rb->inputs[1], rb->inputs[2], rb->rescale};
+        add.epilogue = RescaleSpec{ro.inputs[1], ro.inputs[2], ro.rescale};
+        add.inputs = {ra->inputs[0], rb->inputs[0]};
+        add.outputs[0] = ro.outputs[0];
+        ro.outputs[0]->setProducer(&add);
+        ra->fusedAway = rb->fusedAway = ro.fusedAway = true;
+    }
+}
+
+/*******************************************************************************
+ * GraphPipeline: planning, binding, dispatch
+ *******************************************************************************/
+
+std::vector<const OpNode *> GraphPipeline::executionList() const {
+    std::vector<const OpNode *> r;
+    for (const auto &op : ops)
+        if (!op->fusedAway) r.push_back(op.get());
+    return r;
+}
+
+void GraphPipeline::plan() {
+    // Live ranges as the reference builds them (interval_memory_planner.cpp:53-115): execution index 0 belongs to the
+    // graph inputs, operator i (in execution order) to index i + 1, the graph outputs to the index after the last
+    // operator; every session tensor an operator reads or writes has its range stretched over that index.
+    std::map<const TensorDescriptor *, size_t> order;
+    for (size_t i = 0; i < tensors.size(); i++) order[tensors[i].get()] = i;
+    ranges.clear();
+    const auto touch = [&](const TensorPtr &t, uint32_t idx) {
+        if (!t || order.find(t.get()) == order.end()) return;
+        auto [it, inserted] = ranges.emplace(t.get(), std::array<uint32_t, 2>{idx, idx});
+        if (!inserted) {
+            it->second[0] = std::min(it->second[0], idx);
+            it->second[1] = std::max(it->second[1], idx);
+        }
+    };
+    uint32_t idx = 0;
+    for (const auto &t : inputs) touch(t, idx);
+    idx++;
+    for (const auto &op : ops) {
+        if (op->fusedAway) continue;
+        for (const auto &t : op->inputs) touch(t, idx);
+        for (const auto &t : op->outputs) touch(t, idx);
+        for (const auto *spec : {&op->epilogue, &op->scaleA, &op->scaleB}) {
+            touch(spec->multiplier, idx);
+            touch(spec->shift, idx);
+        }
+        idx++;
+    }
+    for (const auto &t : outputs) touch(t, idx);
+
+    const auto aligned = [](size_t v) { return (v + kSessionAlignment - 1) / kSessionAlignment * kSessionAlignment; };
+    std::vector<details::LiveInterval> intervals;
+    std::vector<details::UnseenAllocation> unseen;
+    // a tensor some operator of the graph used, but no executed operator uses any more, was folded into a fused
+    // kernel: it no longer exists at run time and gets no storage (a tensor no operator ever used keeps storage of
+    // its own, as in the reference)
+    std::set<const TensorDescriptor *> eliminated;
+    for (const auto &op : ops) {
+        for (const auto &t : op->originalTensors)
+            if (ranges.find(t) == ranges.end()) eliminated.insert(t);
+    }
+    for (size_t i = 0; i < tensors.size(); i++) {
+        const auto *t = tensors[i].get();
+        const auto it = ranges.find(t);
+        if (it != ranges.end())
+            intervals.push_back({i, it->second[0], it->second[1], aligned(t->getSize()), i});
+        else if (eliminated.find(t) == eliminated.end() || t->isGraphOutput)
+            unseen.push_back({i, aligned(t->getSize())});
+    }
+    const auto planResult = details::allocateIntervals(std::move(intervals), unseen, kSessionAlignment);
+    offsets.clear();
+    for (const auto &[id, off] : planResult.offsets) offsets[tensors[id].get()] = static_cast<size_t>(off);
+    sessionSize = static_cast<size_t>(planResult.memorySize);
+}
+
+std::vector<std::array<uint32_t, 2>> GraphPipeline::liveRanges() const {
+    std::vector<std::array<uint32_t, 2>> r;
+    for (const auto &t : tensors) {
+        const auto it = ranges.find(t.get());
+        r.push_back(it == ranges.end() ? std::array<uint32_t, 2>{~0u, ~0u} : it->second);
+    }
+    return r;
+}
+
+void GraphPipeline::finalize(const bool enableFusion) {
+    if (finalized) return;
+    if (enableFusion) fuse();
+    plan();
+    finalized = true;
+}
+
+void GraphPipeline::bindSessionMemory(void *deviceBase) {
+    if (!finalized) fail("bindSessionMemory: finalize() has not run");
+    if (sessionSize != 0 && deviceBase == nullptr) fail("bindSessionMemory: null session memory");
+    if (reinterpret_cast<uintptr_t>(deviceBase) % kSessionAlignment != 0)
+        fail("bindSessionMemory: session memory must be aligned to " + std::to_string(kSessionAlignment) + " bytes");
+    for (const auto &[t, off] : offsets) const_cast<TensorDescriptor *>(t)->bind(static_cast<char *>(deviceBase) + off);
+}
+
+void GraphPipeline::bindExternal(const uint32_t set, const uint32_t binding, const uint32_t arrayIndex,
+                                 void *devicePtr) {
+    getTensor(set, binding, arrayIndex)->bind(devicePtr);
+}
+
+namespace {
+
+mlel_epilogue makeEpilogue(const RescaleSpec &spec, const mlel_tensor *mult, const mlel_tensor *shift, bool hasClamp,
+                           const mlel_clamp_attr &clamp) {
+    mlel_epilogue e{};
+    e.multiplier = mult;
+    e.shift = shift;
+    e.rescale = spec.attr;
+    e.has_clamp = hasClamp ? 1 : 0;
+    e.clamp = clamp;
+    return e;
+}
+
+}  // namespace
+
+void GraphPipeline::run(const OpNode &op, void *stream) {
+    std::array<mlel_tensor, 4> in{};
+    for (size_t i = 0; i < op.inputs.size() && i < in.size(); i++) {
+        in[i] = op.inputs[i]->view();
+        if (in[i].ptr == nullptr && op.inputs[i]->getShapeSize() != 0)
+            fail(op.tosaName + " (" + op.debugName + "): input tensor " + std::to_string(i) + " has no memory bound");
+    }
+    mlel_tensor out = op.outputs[0]->view();
+    if (out.ptr == nullptr && op.outputs[0]->getShapeSize() != 0)
+        fail(op.tosaName + " (" + op.debugName + "): output tensor has no memory bound");
+    int rc = 0;
+    switch (op.kind) {
+    case OpKind::Conv2D: rc = mlel_hip_conv2d(ctx, stream, &out, &in[0], &in[1], &in[2], &op.conv); break;
+    case OpKind::DepthwiseConv2D:
+        rc = mlel_hip_depthwise_conv2d(ctx, stream, &out, &in[0], &in[1], &in[2], &op.conv);
+        break;
+    case OpKind::Matmul: rc = mlel_hip_matmul(ctx, stream, &out, &in[0], &in[1], &op.matmul); break;
+    case OpKind::Rescale: rc = mlel_hip_rescale(ctx, stream, &out, &in[0], &in[1], &in[2], &op.rescale); break;
+    case OpKind::Clamp: rc = mlel_hip_clamp(ctx, stream, &out, &in[0], &op.clamp); break;
+    case OpKind::Binary:
+        rc = mlel_hip_elementwise_binary(ctx, stream, op.selector, &out, &in[0], &in[1], op.nanMode);
+        break;
+    case OpKind::Mul: rc = mlel_hip_mul(ctx, stream, &out, &in[0], &in[1], op.shift); break;
+    case OpKind::Unary: rc = mlel_hip_elementwise_unary(ctx, stream, op.selector, &out, &in[0]); break;
+    case OpKind::Reduce: rc = mlel_hip_reduce(ctx, stream, op.selector, &out, &in[0], op.axis, op.nanMode); break;
+    case OpKind::AvgPool2D: rc = mlel_hip_avg_pool2d(ctx, stream, &out, &in[0], &op.pool); break;
+    case OpKind::MaxPool2D: rc = mlel_hip_max_pool2d(ctx, stream, &out, &in[0], &op.pool); break;
+    case OpKind::Table: rc = mlel_hip_table(ctx, stream, &out, &in[0], &in[1]); break;
+    case OpKind::Cast: rc = mlel_hip_cast(ctx, stream, &out, &in[0]); break;
+    case OpKind::Negate:
+        rc = mlel_hip_negate(ctx, stream, &out, &in[0], op.inputZeroPoint, op.outputZeroPoint);
+        break;
+    case OpKind::Reshape: rc = mlel_hip_reshape(ctx, stream, &out, &in[0]); break;
+    case OpKind::Transpose: rc = mlel_hip_transpose(ctx, stream, &out, &in[0], op.vec.data()); break;
+    case OpKind::Concat: rc = mlel_hip_concat(ctx, stream, &out, &in[0], op.axis, op.offset); break;
+    case OpKind::Slice: rc = mlel_hip_slice(ctx, stream, &out, &in[0], op.vec.data()); break;
+    case OpKind::Pad: rc = mlel_hip_pad(ctx, stream, &out, &in[0], &in[1], op.padConst, op.padConstInt); break;
+    case OpKind::FusedConv2D:
+    case OpKind::FusedDepthwiseConv2D:
+    case OpKind::FusedMatmul: {
+        const mlel_tensor mult = op.epilogue.multiplier->view(), shift = op.epilogue.shift->view();
+        const mlel_epilogue e = makeEpilogue(op.epilogue, &mult, &shift, op.hasClamp, op.clamp);
+        if (op.kind == OpKind::FusedConv2D)
+            rc = mlel_hip_conv2d_rescale_clamp(ctx, stream, &out, &in[0], &in[1], &in[2], &op.conv, &e);
+        else if (op.kind == OpKind::FusedDepthwiseConv2D)
+            rc = mlel_hip_dwconv_rescale_clamp(ctx, stream, &out, &in[0], &in[1], &in[2], &op.conv, &e);
+        else
+            rc = mlel_hip_matmul_rescale(ctx, stream, &out, &in[0], &in[1], &op.matmul, &e);
+        break;
+    }
+    case OpKind::FusedRescaleAddRescale: {
+        const mlel_tensor ma = op.scaleA.multiplier->view(), sa = op.scaleA.shift->view();
+        const mlel_tensor mb = op.scaleB.multiplier->view(), sb = op.scaleB.shift->view();
+        const mlel_tensor mo = op.epilogue.multiplier->view(), so = op.epilogue.shift->view();
+        const mlel_clamp_attr none{};
+        const mlel_epilogue ea = makeEpilogue(op.scaleA, &ma, &sa, false, none);
+        const mlel_epilogue eb = makeEpilogue(op.scaleB, &mb, &sb, false, none);
+        const mlel_epilogue eo = makeEpilogue(op.epilogue, &mo, &so, false, none);
+        rc = mlel_hip_rescale_add_rescale(ctx, stream, &out, &in[0], &ea, &in[1], &eb, &eo);
+        break;
+    }
+    }
+    if (rc != 0) fail(op.tosaName + " (" + op.debugName + "): " + mlel_hip_last_error());
+}
+
+void GraphPipeline::dispatch(void *stream, const DispatchDecorator &decorator) {
+    if (!finalized) fail("dispatch: finalize() has not run");
+    if (ctx == nullptr) fail("dispatch: this GraphPipeline was built without a device context; there is no CPU path");
+    uint32_t index = 0;
+    for (const auto &op : ops) {
+        if (op->fusedAway) continue;
+        if (decorator) decorator(*op, index, true);
+        run(*op, stream);
+        if (decorator) decorator(*op, index, false);
+        index++;
+    }
+}
+
+}  // namespace mlel::graph

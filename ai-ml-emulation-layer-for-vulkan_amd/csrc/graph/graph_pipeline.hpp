@@ -1,0 +1,346 @@
+// Host-side operator surface of the TOSA data-graph backend.
+//
+// class GraphPipeline mirrors the reference's class of the same name (graph/compute_graph_op.hpp:1204-1549): the
+// SPIR-V graph decoder (graph/graph_tosa_1_0_ext_inst.cpp) calls make<Op>() once per TOSA instruction, the layer
+// registers constants / external tensors / session tensors through makeConstTensor, makeDescriptorSetBinding and
+// makeTensor, and finally dispatches.  Where the reference builds one VkPipeline per operator and records
+// vkCmdDispatch (compute_graph_op.cpp:526-590, 2500-2509), this class records an operator node and, at dispatch,
+// calls the C ABI of include/mlel_hip.h, which launches hand-written gfx950 kernels.
+//
+// Differences that follow from running on HIP instead of Vulkan:
+//   * tensors are (device pointer, dims, byte strides); the element type is mlel_dtype (the VkFormat -> type table
+//     of common/utils.cpp:119-228 is provided by dtypeFromVkFormat());
+//   * finalize() runs a fusion pass (CONV2D/DEPTHWISE_CONV2D/MATMUL + RESCALE [+ CLAMP] into one launch,
+//     RESCALE + RESCALE + ADD + RESCALE into one launch; the fused kernels are bit-identical to the sequence) and
+//     the interval memory planner over the fused operator list;
+//   * dispatch(stream) replaces cmdBindAndDispatch(commandBuffer, ...): operators run in creation order on one HIP
+//     stream, which gives the same ordering the reference enforces with a barrier on every input tensor.
+#pragma once
+
+#include <array>
+#include <cstdint>
+#include <functional>
+#include <map>
+#include <memory>
+#include <set>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../../include/mlel_hip.h"
+
+namespace mlel::graph {
+
+using real_t = double;  // reference: common/include/mlel/float.hpp (double unless VMEL_USE_FLOAT_AS_DOUBLE)
+
+// VkFormat values of the tensor formats the reference accepts (Vulkan-Headers; only the numbers are used here).
+enum VkFormatValue : int32_t {
+    VK_FORMAT_R8_UINT = 13,
+    VK_FORMAT_R8_SINT = 14,
+    VK_FORMAT_R16_UINT = 74,
+    VK_FORMAT_R16_SINT = 75,
+    VK_FORMAT_R16_SFLOAT = 76,
+    VK_FORMAT_R32_UINT = 98,
+    VK_FORMAT_R32_SINT = 99,
+    VK_FORMAT_R32_SFLOAT = 100,
+    VK_FORMAT_R64_UINT = 110,
+    VK_FORMAT_R64_SINT = 111,
+    VK_FORMAT_R64_SFLOAT = 112,
+    VK_FORMAT_S8_UINT = 127,
+    VK_FORMAT_R8_BOOL_ARM = 1000460000,
+};
+// Throws std::runtime_error("Unsupported tensor buffer format: <n>") like getFormatInfo (common/utils.cpp:185).
+mlel_dtype dtypeFromVkFormat(int32_t vkFormat);
+size_t dtypeSize(int32_t dtype);
+
+enum class TensorKind { Session, Constant, External };
+
+class OpNode;
+
+// Reference counterpart: class TensorDescriptor (graph/tensor.hpp, graph/tensor.cpp:70-114,185-255).
+class TensorDescriptor {
+  public:
+    TensorDescriptor(int32_t dtype, std::vector<int64_t> dimensions, std::vector<int64_t> strides, TensorKind kind);
+
+    int32_t getFormat() const { return dtype; }
+    const std::vector<int64_t> &getDimensions() const { return dimensions; }
+    const std::vector<int64_t> &getStrides() const { return strides; }
+    uint32_t getRank() const { return static_cast<uint32_t>(dimensions.size()); }
+    size_t getShapeSize() const;
+    size_t getSize() const;  // dims[0] * strides[0]: the extent in bytes (reference: tensor.cpp:197-203)
+    TensorKind getKind() const { return kind; }
+    bool isPacked() const;
+
+    OpNode *getProducer() const { return producer; }
+    void setProducer(OpNode *op) { producer = op; }
+
+    void *devicePointer() const { return ptr; }
+    void bind(void *devicePtr) { ptr = devicePtr; }
+    mlel_tensor view() const;
+
+    int id = -1;  // handle used by the C API
+    bool isGraphInput = false, isGraphOutput = false;
+
+  private:
+    int32_t dtype;
+    std::vector<int64_t> dimensions;
+    std::vector<int64_t> strides;
+    TensorKind kind;
+    OpNode *producer = nullptr;
+    void *ptr = nullptr;
+};
+using TensorPtr = std::shared_ptr<TensorDescriptor>;
+
+enum class OpKind {
+    Conv2D, DepthwiseConv2D, Matmul, Rescale, Clamp, Binary, Mul, Unary, Reduce, AvgPool2D, MaxPool2D, Table, Cast,
+    Negate, Reshape, Transpose, Concat, Slice, Pad,
+    // produced by the fusion pass only
+    FusedConv2D, FusedDepthwiseConv2D, FusedMatmul, FusedRescaleAddRescale,
+};
+
+struct RescaleSpec {
+    TensorPtr multiplier, shift;
+    mlel_rescale_attr attr{};
+};
+
+// One recorded operator.  Reference counterpart: the ComputePipeline subclasses (compute_graph_op.hpp:226-1198).
+class OpNode {
+  public:
+    OpKind kind{};
+    std::string tosaName;   // "CONV2D", "RESCALE", ... as in graph_tosa_1_0_ext_inst.cpp:41-108
+    std::string debugName;
+    std::vector<TensorPtr> inputs;   // data inputs first, then parameter tensors (weights, bias, multiplier ...)
+    std::vector<TensorPtr> outputs;
+    std::vector<const TensorDescriptor *> originalTensors;  // operands as recorded, before any fusion
+    // attributes (a plain union-of-fields record; only the fields of `kind` are meaningful)
+    mlel_conv2d_attr conv{};
+    mlel_matmul_attr matmul{};
+    mlel_rescale_attr rescale{};
+    mlel_clamp_attr clamp{};
+    mlel_pool2d_attr pool{};
+    int32_t selector = 0;  // mlel_binary_op / mlel_unary_op / mlel_reduce_op
+    uint32_t nanMode = MLEL_NAN_PROPAGATE, axis = 0, shift = 0, offset = 0;
+    int32_t inputZeroPoint = 0, outputZeroPoint = 0, padConstInt = 0;
+    real_t padConst = 0;
+    std::array<uint32_t, MLEL_MAX_RANK> vec{};  // perms / start
+    // fusion results
+    bool fusedAway = false;          // folded into another node; not executed
+    RescaleSpec epilogue;            // Fused*: RESCALE applied to the accumulator
+    bool hasClamp = false;           // Fused*: CLAMP after the RESCALE
+    RescaleSpec scaleA, scaleB;      // FusedRescaleAddRescale: the two input stages (epilogue = output stage)
+};
+
+class GraphPipeline {
+  public:
+    explicit GraphPipeline(mlel_ctx *ctx);
+    ~GraphPipeline();
+    GraphPipeline(const GraphPipeline &) = delete;
+    GraphPipeline &operator=(const GraphPipeline &) = delete;
+
+    // ---- constant tensors owned by the pipeline; the data is copied (reference: compute_graph_op.cpp:2398-2420)
+    void makeConstTensor(uint32_t id, int32_t dtype, const std::vector<int64_t> &dimensions,
+                         const std::vector<int64_t> &strides, const void *data);
+    TensorPtr getConstTensor(uint32_t id) const;  // throws std::out_of_range like the reference's map::at
+    TensorPtr makeConstCompositeTensor(int32_t dtype, std::vector<int64_t> dimensions, const void *data);
+
+    // ---- external tensors owned by the application (reference: compute_graph_op.cpp:2441-2455)
+    void makeDescriptorSetBinding(uint32_t set, uint32_t binding, uint32_t arrayIndex, int32_t dtype,
+                                  const std::vector<int64_t> &dimensions, const std::vector<int64_t> &strides);
+    TensorPtr getTensor(uint32_t set, uint32_t binding, uint32_t arrayIndex = 0) const;
+
+    // ---- tensors allocated in session RAM (reference: compute_graph_op.cpp:2457-2471)
+    TensorPtr makeTensor(int32_t dtype, std::vector<int64_t> dimensions = {}, std::vector<int64_t> strides = {});
+    const std::vector<TensorPtr> &getTensors() const { return tensors; }
+
+    void makeInput(const TensorPtr &tensor);
+    void makeOutput(const TensorPtr &tensor);
+    const std::vector<TensorPtr> &getInputs() const { return inputs; }
+    const std::vector<TensorPtr> &getOutputs() const { return outputs; }
+    const std::vector<std::shared_ptr<OpNode>> &getPipelines() const { return ops; }
+
+    // ---- TOSA operators: names, argument order and meaning as in compute_graph_op.hpp:1249-1483
+    void makeAbs(const TensorPtr &input, const TensorPtr &output, const std::string &debugName);
+    void makeAdd(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output, const std::string &debugName);
+    void makeArgmax(const TensorPtr &input, const TensorPtr &output, uint32_t axis, uint32_t nanMode,
+                    const std::string &debugName);
+    void makeArithmeticRightShift(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output, bool round,
+                                  const std::string &debugName);
+    void makeAvgPool2D(const TensorPtr &input, const TensorPtr &output, const std::vector<int32_t> &kernel,
+                       const std::vector<int32_t> &stride, const std::vector<int32_t> &pad, uint32_t accType,
+                       int8_t inputZeroPoint, int8_t outputZeroPoint, const std::string &debugName);
+    void makeBitwiseAnd(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                        const std::string &debugName);
+    void makeBitwiseNot(const TensorPtr &input, const TensorPtr &output, const std::string &debugName);
+    void makeBitwiseOr(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                       const std::string &debugName);
+    void makeBitwiseXor(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                        const std::string &debugName);
+    void makeCast(const TensorPtr &input1, const TensorPtr &output, const std::string &debugName);
+    void makeCeil(const TensorPtr &input1, const TensorPtr &output, const std::string &debugName);
+    void makeClamp(const TensorPtr &input, const TensorPtr &output, real_t min, real_t max, uint32_t nanMode,
+                   const std::string &debugName);
+    void makeClz(const TensorPtr &input1, const TensorPtr &output, const std::string &debugName);
+    void makeConcat(const std::vector<TensorPtr> &inputs, const TensorPtr &output, uint32_t axis,
+                    const std::string &debugName);
+    void makeConv2D(const TensorPtr &input, const TensorPtr &output, const TensorPtr &weights, const TensorPtr &biases,
+                    const std::vector<int32_t> &pad, const std::vector<int32_t> &stride,
+                    const std::vector<int32_t> &dilation, int8_t inputZeroPoint, int8_t weightZeroPoint,
+                    uint32_t accType, const std::string &debugName);
+    void makeConv3D(const TensorPtr &input, const TensorPtr &output, const TensorPtr &weights, const TensorPtr &biases,
+                    const std::vector<int32_t> &pad, const std::vector<int32_t> &stride,
+                    const std::vector<int32_t> &dilation, int8_t inputZeroPoint, int8_t weightZeroPoint,
+                    uint32_t accType, const std::string &debugName);
+    void makeCos(const TensorPtr &input1, const TensorPtr &output, const std::string &debugName);
+    void makeDepthwiseConv2D(const TensorPtr &input, const TensorPtr &output, const TensorPtr &weights,
+                             const TensorPtr &biases, const std::vector<int32_t> &pad,
+                             const std::vector<int32_t> &stride, const std::vector<int32_t> &dilation,
+                             int8_t inputZeroPoint, int8_t weightZeroPoint, uint32_t accType,
+                             const std::string &debugName);
+    void makeEqual(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                   const std::string &debugName);
+    void makeErf(const TensorPtr &input, const TensorPtr &output, const std::string &debugName);
+    void makeExp(const TensorPtr &input, const TensorPtr &output, const std::string &debugName);
+    void makeFft2D(const TensorPtr &inputReal, const TensorPtr &inputImag, const TensorPtr &outputReal,
+                   const TensorPtr &outputImag, bool inverse, const std::string &debugName);
+    void makeFloor(const TensorPtr &input1, const TensorPtr &output, const std::string &debugName);
+    void makeGather(const TensorPtr &values, const TensorPtr &indices, const TensorPtr &output,
+                    const std::string &debugName);
+    void makeGreater(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                     const std::string &debugName);
+    void makeGreaterEqual(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                          const std::string &debugName);
+    void makeIntdiv(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                    const std::string &debugName);
+    void makeLog(const TensorPtr &input1, const TensorPtr &output, const std::string &debugName);
+    void makeLogicalAnd(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                        const std::string &debugName);
+    void makeLogicalLeftShift(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                              const std::string &debugName);
+    void makeLogicalNot(const TensorPtr &input, const TensorPtr &output, const std::string &debugName);
+    void makeLogicalRightShift(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                               const std::string &debugName);
+    void makeLogicalOr(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                       const std::string &debugName);
+    void makeLogicalXor(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                        const std::string &debugName);
+    void makeMaximum(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output, uint32_t nanMode,
+                     const std::string &debugName);
+    void makeMinimum(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output, uint32_t nanMode,
+                     const std::string &debugName);
+    void makeMatmul(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output, int32_t inputZeroPoint1,
+                    int32_t inputZeroPoint2, const std::string &debugName);
+    void makeMaxPool2D(const TensorPtr &input, const TensorPtr &output, const std::vector<int32_t> &kernel,
+                       const std::vector<int32_t> &stride, const std::vector<int32_t> &pad, uint32_t nanMode,
+                       const std::string &debugName);
+    void makeMul(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output, uint32_t shift,
+                 const std::string &debugName);
+    void makeNegate(const TensorPtr &input, const TensorPtr &output, int32_t inputZeroPoint, int32_t outputZeroPoint,
+                    const std::string &debugName);
+    void makePad(const TensorPtr &input, const TensorPtr &output, const TensorPtr &padding, real_t padConst,
+                 int32_t padConstInt, const std::string &debugName);
+    void makePow(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                 const std::string &debugName);
+    void makeReciprocal(const TensorPtr &input, const TensorPtr &output, const std::string &debugName);
+    void makeReduceAll(const TensorPtr &input, const TensorPtr &output, uint32_t axis, const std::string &debugName);
+    void makeReduceAny(const TensorPtr &input, const TensorPtr &output, uint32_t axis, const std::string &debugName);
+    void makeReduceMax(const TensorPtr &input, const TensorPtr &output, uint32_t axis, uint32_t nanMode,
+                       const std::string &debugName);
+    void makeReduceMin(const TensorPtr &input, const TensorPtr &output, uint32_t axis, uint32_t nanMode,
+                       const std::string &debugName);
+    void makeReduceProduct(const TensorPtr &input, const TensorPtr &output, uint32_t axis,
+                           const std::string &debugName);
+    void makeReduceSum(const TensorPtr &input, const TensorPtr &output, uint32_t axis, const std::string &debugName);
+    void makeRescale(const TensorPtr &input, const TensorPtr &output, int32_t inputZeroPoint, int32_t outputZeroPoint,
+                     const TensorPtr &multiplier, const TensorPtr &shift, bool scale32, bool doubleRound,
+                     bool perChannel, bool inputUnsigned, bool outputUnsigned, const std::string &debugName);
+    void makeReshape(const TensorPtr &input, const TensorPtr &output, const std::string &debugName);
+    void makeResize(const TensorPtr &input, const TensorPtr &output, const std::vector<int32_t> &scale,
+                    const std::vector<int32_t> &offset, const std::vector<int32_t> &border, uint32_t mode,
+                    const std::string &debugName);
+    void makeReverse(const TensorPtr &input, const TensorPtr &output, uint32_t axis, const std::string &debugName);
+    void makeRfft2D(const TensorPtr &input, const TensorPtr &outputReal, const TensorPtr &outputImag,
+                    const std::string &debugName);
+    void makeRsqrt(const TensorPtr &input1, const TensorPtr &output, const std::string &debugName);
+    void makeScatter(const TensorPtr &input, const TensorPtr &values, const TensorPtr &indices,
+                     const TensorPtr &output, const std::string &debugName);
+    void makeSelect(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &input3, const TensorPtr &output,
+                    const std::string &debugName);
+    void makeSigmoid(const TensorPtr &input, const TensorPtr &output, const std::string &debugName);
+    void makeSin(const TensorPtr &input1, const TensorPtr &output, const std::string &debugName);
+    void makeSlice(const TensorPtr &input, const TensorPtr &output, const std::vector<uint32_t> &start,
+                   const std::string &debugName);
+    void makeSub(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                 const std::string &debugName);
+    void makeTable(const TensorPtr &input, const TensorPtr &output, const TensorPtr &table,
+                   const std::string &debugName);
+    void makeTanh(const TensorPtr &input1, const TensorPtr &output, const std::string &debugName);
+    void makeTile(const TensorPtr &input, const TensorPtr &output, const std::string &debugName);
+    void makeTranspose(const TensorPtr &input, const TensorPtr &output, const std::vector<uint32_t> &perms,
+                       const std::string &debugName);
+    void makeTransposeConv2D(const TensorPtr &input, const TensorPtr &output, const TensorPtr &weights,
+                             const TensorPtr &biases, const std::vector<int32_t> &pad,
+                             const std::vector<int32_t> &stride, int8_t inputZeroPoint, int8_t weightZeroPoint,
+                             uint32_t accType, const std::string &debugName);
+
+    // ---- HIP side ------------------------------------------------------------------------------------------
+    // Runs the fusion pass (unless disabled) and plans session memory.  Called once, after the last make<Op>().
+    void finalize(bool enableFusion = true);
+    bool isFinalized() const { return finalized; }
+    // Session memory requirements (reference: vkGetDataGraphPipelineSessionMemoryRequirementsARM,
+    // graph_layer.cpp:1382-1389): size and alignment of the one allocation all intermediates live in.
+    size_t sessionMemorySize() const { return sessionSize; }
+    size_t sessionMemoryAlignment() const { return kSessionAlignment; }
+    // Reference: vkBindDataGraphPipelineSessionMemoryARM -> bindGraphPipelineSessionMemory
+    // (interval_memory_planner.cpp:251-272): every planned tensor is bound at base + its offset.
+    void bindSessionMemory(void *deviceBase);
+    // External tensors may be re-bound between dispatches (update-after-bind in the reference).
+    void bindExternal(uint32_t set, uint32_t binding, uint32_t arrayIndex, void *devicePtr);
+    // Reference: cmdBindAndDispatch (compute_graph_op.cpp:2500-2509).  The decorator, when set, brackets every
+    // executed operator (the reference's ComputePipelineDispatchDecorator, used by its profiler).
+    using DispatchDecorator = std::function<void(const OpNode &, uint32_t index, bool before)>;
+    void dispatch(void *stream, const DispatchDecorator &decorator = {});
+
+    // introspection used by tests and the profiler
+    std::vector<const OpNode *> executionList() const;
+    const std::map<const TensorDescriptor *, size_t> &sessionOffsets() const { return offsets; }
+    std::vector<std::array<uint32_t, 2>> liveRanges() const;  // per getTensors() entry: {first, last} or {~0,~0}
+
+    static constexpr size_t kSessionAlignment = 256;
+
+  private:
+    std::shared_ptr<OpNode> addOp(OpKind kind, const char *tosaName, const std::string &debugName,
+                                  std::vector<TensorPtr> ins, std::vector<TensorPtr> outs);
+    void makeBinary(int32_t op, const char *name, const TensorPtr &a, const TensorPtr &b, const TensorPtr &out,
+                    uint32_t nanMode, const std::string &debugName);
+    void makeUnary(int32_t op, const char *name, const TensorPtr &in, const TensorPtr &out,
+                   const std::string &debugName);
+    void makeReduce(int32_t op, const char *name, const TensorPtr &in, const TensorPtr &out, uint32_t axis,
+                    uint32_t nanMode, const std::string &debugName);
+    TensorPtr registerTensor(TensorPtr t);
+    void *uploadConstant(const TensorDescriptor &t, const void *data);
+    void fuse();
+    void plan();
+    void run(const OpNode &op, void *stream);
+    [[noreturn]] void unsupported(const char *tosaName) const;
+
+    mlel_ctx *ctx;
+    std::vector<std::shared_ptr<OpNode>> ops;
+    std::vector<TensorPtr> tensors;             // session tensors in creation order
+    std::set<TensorPtr> tensorSet;
+    std::vector<TensorPtr> allTensors;          // every tensor this pipeline knows (handles)
+    std::map<uint32_t, TensorPtr> constTensorMap;
+    std::vector<TensorPtr> compositeTensors;
+    std::map<uint32_t, std::map<uint32_t, std::vector<TensorPtr>>> tensorMap;  // set -> binding -> array
+    std::vector<void *> constantsDeviceMemory;
+    std::vector<TensorPtr> inputs, outputs;
+    std::map<const TensorDescriptor *, size_t> offsets;
+    std::map<const TensorDescriptor *, std::array<uint32_t, 2>> ranges;
+    size_t sessionSize = 0;
+    bool finalized = false;
+
+    friend class CApi;
+  public:
+    const std::vector<TensorPtr> &handles() const { return allTensors; }
+};
+
+}  // namespace mlel::graph

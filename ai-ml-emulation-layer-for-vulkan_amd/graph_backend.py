@@ -1,0 +1,206 @@
+"""ctypes harness over libmlel_graph.so, the C view (include/mlel_graph.h) of the host-side GraphPipeline.
+
+Builds a data graph from a neutral description (see graphs.py), binds device memory and dispatches it.  As in the
+reference's test client (utilities/pipeline.cpp:297-330) external tensors are allocated by the caller, session
+memory is queried, allocated and bound once, and a dispatch is followed by a wait.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import abi
+from .hip_backend import MlelError, load_library
+
+_glib = None
+
+_I64P = C.POINTER(C.c_int64)
+_V = C.c_void_p
+
+
+def load_graph_library():
+    global _glib
+    if _glib is None:
+        load_library()  # libmlel_hip.so first: the graph library is linked against it
+        if not os.path.exists(abi.GRAPH_LIB_PATH):
+            raise MlelError(abi.ERR_DEVICE, f"{abi.GRAPH_LIB_PATH} is not built; run __graft_entry__.build()")
+        lib = C.CDLL(abi.GRAPH_LIB_PATH)
+        lib.mlel_graph_last_error.restype = C.c_char_p
+        lib.mlel_graph_create.argtypes = [_V, C.POINTER(_V)]
+        lib.mlel_graph_destroy.argtypes = [_V]
+        lib.mlel_graph_destroy.restype = None
+        lib.mlel_graph_make_const_tensor.argtypes = [_V, C.c_uint32, C.c_int32, C.c_int32, _I64P, _I64P, _V]
+        lib.mlel_graph_get_const_tensor.argtypes = [_V, C.c_uint32]
+        lib.mlel_graph_make_const_composite_tensor.argtypes = [_V, C.c_int32, C.c_int32, _I64P, _V]
+        lib.mlel_graph_make_descriptor_set_binding.argtypes = [_V, C.c_uint32, C.c_uint32, C.c_uint32, C.c_int32,
+                                                               C.c_int32, _I64P, _I64P]
+        lib.mlel_graph_get_tensor.argtypes = [_V, C.c_uint32, C.c_uint32, C.c_uint32]
+        lib.mlel_graph_make_tensor.argtypes = [_V, C.c_int32, C.c_int32, _I64P, _I64P]
+        lib.mlel_graph_make_input.argtypes = [_V, C.c_int]
+        lib.mlel_graph_make_output.argtypes = [_V, C.c_int]
+        lib.mlel_graph_make_op.argtypes = [_V, C.c_char_p, C.POINTER(C.c_int), C.c_int, C.POINTER(C.c_int), C.c_int,
+                                           _I64P, C.c_int, C.POINTER(C.c_double), C.c_int, C.c_char_p]
+        lib.mlel_graph_finalize.argtypes = [_V, C.c_int]
+        lib.mlel_graph_session_memory_requirements.argtypes = [_V, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
+        lib.mlel_graph_bind_session_memory.argtypes = [_V, _V]
+        lib.mlel_graph_bind_external.argtypes = [_V, C.c_uint32, C.c_uint32, C.c_uint32, _V]
+        lib.mlel_graph_dispatch.argtypes = [_V, _V]
+        lib.mlel_graph_dispatch_profiled.argtypes = [_V, _V, C.POINTER(C.c_float), C.c_int]
+        lib.mlel_graph_op_count.argtypes = [_V]
+        lib.mlel_graph_op_name.argtypes = [_V, C.c_int, C.c_char_p, C.c_size_t]
+        lib.mlel_graph_session_tensor_count.argtypes = [_V]
+        lib.mlel_graph_session_tensor_info.argtypes = [_V, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_uint64),
+                                                       C.POINTER(C.c_uint64), C.POINTER(C.c_uint32),
+                                                       C.POINTER(C.c_uint32)]
+        lib.mlel_graph_allocate_intervals.argtypes = [C.POINTER(C.c_uint64), C.c_int, C.POINTER(C.c_uint64), C.c_int,
+                                                      C.c_uint64, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
+        lib.mlel_graph_dtype_from_vk_format.argtypes = [C.c_int32]
+        _glib = lib
+    return _glib
+
+
+def _i64(values):
+    values = [int(v) for v in values]
+    return (C.c_int64 * max(1, len(values)))(*values)
+
+
+def allocate_intervals(intervals, unseen, alignment):
+    """details::allocateIntervals on its own: ({id: offset}, memory_size)."""
+    lib = load_graph_library()
+    flat_i = [v for iv in intervals for v in iv]
+    flat_u = [v for u in unseen for v in u]
+    n, m = len(intervals), len(unseen)
+    ai = (C.c_uint64 * max(1, len(flat_i)))(*flat_i)
+    au = (C.c_uint64 * max(1, len(flat_u)))(*flat_u)
+    out = (C.c_uint64 * max(2, 2 * (n + m)))()
+    size = C.c_uint64()
+    k = lib.mlel_graph_allocate_intervals(ai, n, au, m, alignment, out, C.byref(size))
+    if k < 0:
+        raise MlelError(k, lib.mlel_graph_last_error().decode())
+    return {int(out[2 * i]): int(out[2 * i + 1]) for i in range(k)}, int(size.value)
+
+
+class Graph:
+    """One GraphPipeline.  Tensors are named; names map to the integer handles of the C API."""
+
+    def __init__(self, dev):
+        self.dev = dev
+        self.lib = load_graph_library()
+        g = _V()
+        self._check(self.lib.mlel_graph_create(dev.ctx, C.byref(g)))
+        self.g = g
+        self.handles = {}
+        self.externals = {}      # name -> (set, binding, array index, dtype, shape)
+        self.session_mem = None
+        self.ext_tensors = {}    # name -> DeviceTensor
+        self.next_binding = 0
+        self.next_const = 0
+
+    def _check(self, rc):
+        if rc < 0:
+            raise MlelError(rc, self.lib.mlel_graph_last_error().decode(errors="replace"))
+        return rc
+
+    def close(self):
+        if self.g:
+            self.lib.mlel_graph_destroy(self.g)
+            self.g = None
+        if self.session_mem:
+            self.dev.free(self.session_mem)
+            self.session_mem = None
+        for t in self.ext_tensors.values():
+            t.free()
+        self.ext_tensors = {}
+
+    # ---- tensors
+    def const(self, name, array, dtype=None):
+        array = np.ascontiguousarray(array)
+        if dtype is None:
+            dtype = abi.dtype_of_numpy(array.dtype)
+        dims = array.shape if array.ndim else (1,)
+        h = self._check(self.lib.mlel_graph_make_const_tensor(self.g, self.next_const, int(dtype), len(dims),
+                                                              _i64(dims), None, array.ctypes.data))
+        self.next_const += 1
+        self.handles[name] = h
+        return h
+
+    def external(self, name, dtype, shape, set_=0, binding=None, array_index=0, strides=None):
+        if binding is None:
+            binding = self.next_binding
+            self.next_binding += 1
+        h = self._check(self.lib.mlel_graph_make_descriptor_set_binding(
+            self.g, set_, binding, array_index, int(dtype), len(shape), _i64(shape),
+            _i64(strides) if strides is not None else None))
+        self.handles[name] = h
+        self.externals[name] = (set_, binding, array_index, int(dtype), tuple(shape), strides)
+        return h
+
+    def tensor(self, name, dtype, shape):
+        h = self._check(self.lib.mlel_graph_make_tensor(self.g, int(dtype), len(shape), _i64(shape), None))
+        self.handles[name] = h
+        return h
+
+    def mark_input(self, name):
+        self._check(self.lib.mlel_graph_make_input(self.g, self.handles[name]))
+
+    def mark_output(self, name):
+        self._check(self.lib.mlel_graph_make_output(self.g, self.handles[name]))
+
+    # ---- operators
+    def op(self, tosa_name, inputs, outputs, iattr=(), fattr=(), debug_name=""):
+        ins = (C.c_int * max(1, len(inputs)))(*[self.handles[n] for n in inputs])
+        outs = (C.c_int * max(1, len(outputs)))(*[self.handles[n] for n in outputs])
+        fa = (C.c_double * max(1, len(fattr)))(*[float(v) for v in fattr])
+        self._check(self.lib.mlel_graph_make_op(self.g, tosa_name.encode(), ins, len(inputs), outs, len(outputs),
+                                                _i64(iattr), len(iattr), fa, len(fattr), debug_name.encode()))
+
+    # ---- finalize / memory / run
+    def finalize(self, fuse=True):
+        self._check(self.lib.mlel_graph_finalize(self.g, 1 if fuse else 0))
+        size, align = C.c_uint64(), C.c_uint64()
+        self._check(self.lib.mlel_graph_session_memory_requirements(self.g, C.byref(size), C.byref(align)))
+        self.session_size = int(size.value)
+        self.session_mem = self.dev.alloc(max(self.session_size, 256))
+        self._check(self.lib.mlel_graph_bind_session_memory(self.g, C.c_void_p(self.session_mem)))
+        for name, (s, b, a, dtype, shape, strides) in self.externals.items():
+            t = self.dev.tensor(dtype, shape, strides)
+            self.ext_tensors[name] = t
+            self._check(self.lib.mlel_graph_bind_external(self.g, s, b, a, C.c_void_p(t.ptr)))
+        return self.session_size
+
+    def set_input(self, name, array):
+        self.ext_tensors[name].upload(array)
+
+    def get_output(self, name):
+        return self.ext_tensors[name].download()
+
+    def dispatch(self):
+        self._check(self.lib.mlel_graph_dispatch(self.g, self.dev.stream))
+
+    def dispatch_profiled(self):
+        n = self.op_count()
+        ms = (C.c_float * max(1, n))()
+        self._check(self.lib.mlel_graph_dispatch_profiled(self.g, self.dev.stream, ms, n))
+        return [(self.op_name(i), float(ms[i])) for i in range(n)]
+
+    def op_count(self):
+        return self._check(self.lib.mlel_graph_op_count(self.g))
+
+    def op_name(self, i):
+        buf = C.create_string_buffer(128)
+        self._check(self.lib.mlel_graph_op_name(self.g, i, buf, 128))
+        return buf.value.decode()
+
+    def op_names(self):
+        return [self.op_name(i) for i in range(self.op_count())]
+
+    def session_tensors(self):
+        n = self._check(self.lib.mlel_graph_session_tensor_count(self.g))
+        out = []
+        for i in range(n):
+            h, off, size, first, last = C.c_int(), C.c_uint64(), C.c_uint64(), C.c_uint32(), C.c_uint32()
+            self._check(self.lib.mlel_graph_session_tensor_info(self.g, i, C.byref(h), C.byref(off), C.byref(size),
+                                                                C.byref(first), C.byref(last)))
+            out.append({"handle": h.value, "offset": None if off.value == 2 ** 64 - 1 else off.value,
+                        "size": size.value, "first": first.value, "last": last.value})
+        return out

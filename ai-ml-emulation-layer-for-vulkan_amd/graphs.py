@@ -1,0 +1,257 @@
+"""Neutral descriptions of the benchmark data graphs (BASELINE configs 2 and 3) and their construction on the
+GraphPipeline.  A description is plain data: named tensors, numpy constants and a list of TOSA operators with the
+operand order of the TOSA.001000.1 instruction set as the reference decodes it
+(graph/graph_tosa_1_0_ext_inst.cpp:37-1032), so the same description can be executed operator by operator by
+any backend (the tests run it through the CPU oracle, unfused, the way the reference executes it).
+"""
+import time
+
+import numpy as np
+
+from . import abi
+from .graph_backend import Graph
+
+# MobileNetV2 1.0: (expansion t, output channels c, repeats n, stride s)
+MOBILENETV2_BLOCKS = [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2),
+                      (6, 320, 1, 1)]
+
+
+class Spec:
+    def __init__(self):
+        self.tensors = {}   # name -> (dtype, shape): intermediates in session memory
+        self.consts = {}    # name -> ndarray
+        self.inputs = []    # (name, dtype, shape)
+        self.outputs = []   # (name, dtype, shape)
+        self.ops = []       # dicts: op, in, out, iattr, fattr, name
+        self.macs = {"dense": 0, "depthwise": 0}
+        self._n = 0
+
+    def fresh(self, prefix):
+        self._n += 1
+        return f"{prefix}{self._n}"
+
+    def const(self, prefix, array):
+        name = self.fresh(prefix)
+        self.consts[name] = np.ascontiguousarray(array)
+        return name
+
+    def tensor(self, prefix, dtype, shape):
+        name = self.fresh(prefix)
+        self.tensors[name] = (dtype, tuple(int(d) for d in shape))
+        return name
+
+    def op(self, op, ins, outs, iattr=(), fattr=(), name=""):
+        self.ops.append({"op": op, "in": list(ins), "out": list(outs), "iattr": [int(v) for v in iattr],
+                         "fattr": [float(v) for v in fattr], "name": name or f"{op.lower()}_{len(self.ops)}"})
+
+    def shape_of(self, name):
+        if name in self.tensors:
+            return self.tensors[name][1]
+        if name in self.consts:
+            return self.consts[name].shape
+        for n, _, s in self.inputs + self.outputs:
+            if n == name:
+                return s
+        raise KeyError(name)
+
+
+class _Quant:
+    """Draws RESCALE parameters: multiplier U[2^30, 2^31), shift U[30, 38] (BASELINE config 0).  With
+    `spread=True` the shift grows with log2 of the contraction length so activations keep using the int8 range
+    instead of saturating (used by the parity tests next to the literal draw)."""
+
+    def __init__(self, rng, spread):
+        self.rng = rng
+        self.spread = spread
+
+    def scale(self, channels, k):
+        mult = self.rng.integers(2 ** 30, 2 ** 31 - 1, (channels,), endpoint=True).astype(np.int32)
+        shift = self.rng.integers(30, 38, (channels,), endpoint=True).astype(np.int8)
+        if self.spread:
+            shift = (shift + int(np.ceil(np.log2(max(k, 1)))) // 2 + 2).astype(np.int8)
+        return mult, shift
+
+
+RELU6_ZP, RELU6_LO, RELU6_HI = -100, -100, 110   # output zero point and CLAMP bounds of the ReLU6 layers
+LINEAR_ZP = 3                                    # output zero point of the linear (project) layers
+
+
+def _conv_block(spec, q, rng, x, x_zp, cin, cout, k, stride, depthwise, relu6, out_name=None, out_kind="tensor"):
+    """CONV2D | DEPTHWISE_CONV2D (int32) -> RESCALE (int8, per channel, double round) [-> CLAMP]."""
+    n, h, w, _ = spec.shape_of(x)
+    if k == 1:
+        pad = (0, 0, 0, 0)
+    elif stride == 1:
+        pad = (1, 1, 1, 1)
+    else:
+        pad = (0, 1, 0, 1)  # even extents at stride 2: the only padding for which the TOSA output size divides
+    oh = (h + pad[0] + pad[1] - k) // stride + 1
+    ow = (w + pad[2] + pad[3] - k) // stride + 1
+    if depthwise:
+        wt = spec.const("dw_w", rng.integers(-127, 127, (k, k, cin, 1), endpoint=True).astype(np.int8))
+        contraction = k * k
+        spec.macs["depthwise"] += n * oh * ow * cout * k * k
+    else:
+        wt = spec.const("w", rng.integers(-127, 127, (cout, k, k, cin), endpoint=True).astype(np.int8))
+        contraction = k * k * cin
+        spec.macs["dense"] += n * oh * ow * cout * k * k * cin
+    bias = spec.const("b", rng.integers(-2 ** 15, 2 ** 15, (cout,), endpoint=True).astype(np.int32))
+    acc = spec.tensor("acc", abi.I32, (n, oh, ow, cout))
+    spec.op("DEPTHWISE_CONV2D" if depthwise else "CONV2D", [x, wt, bias], [acc],
+            list(pad) + [stride, stride, 1, 1, x_zp, 0, abi.ACC_I32])
+    mult, shift = q.scale(cout, contraction)
+    m, s = spec.const("m", mult), spec.const("s", shift)
+    out_zp = RELU6_ZP if relu6 else LINEAR_ZP
+    final_shape = (n, oh, ow, cout)
+
+    def make_out(prefix):
+        if out_name is not None:
+            return out_name
+        return spec.tensor(prefix, abi.I8, final_shape)
+
+    if relu6:
+        r = spec.tensor("r", abi.I8, final_shape)
+        spec.op("RESCALE", [acc, m, s], [r], [0, out_zp, 1, 1, 1, 0, 0])
+        y = make_out("y")
+        spec.op("CLAMP", [r], [y], [abi.NAN_PROPAGATE], [RELU6_LO, RELU6_HI])
+    else:
+        y = make_out("y")
+        spec.op("RESCALE", [acc, m, s], [y], [0, out_zp, 1, 1, 1, 0, 0])
+    return y, out_zp
+
+
+def _residual(spec, q, rng, x, x_zp, y, y_zp):
+    """RESCALE(x -> i32) + RESCALE(y -> i32) -> ADD -> RESCALE(-> i8): the reference's residual-add pattern
+    (tests/shader/graph-constant-arm.spvasm)."""
+    shape = spec.shape_of(x)
+    one = lambda v, dt: np.array([v], dt)
+    ma = spec.const("m", one(rng.integers(2 ** 30, 2 ** 31 - 1), np.int32))
+    mb = spec.const("m", one(rng.integers(2 ** 30, 2 ** 31 - 1), np.int32))
+    mo = spec.const("m", one(rng.integers(2 ** 30, 2 ** 31 - 1), np.int32))
+    sa, sb, so = spec.const("s", one(20, np.int8)), spec.const("s", one(20, np.int8)), spec.const("s", one(42, np.int8))
+    xa, yb = spec.tensor("ra", abi.I32, shape), spec.tensor("rb", abi.I32, shape)
+    spec.op("RESCALE", [x, ma, sa], [xa], [x_zp, 0, 1, 1, 0, 0, 0])
+    spec.op("RESCALE", [y, mb, sb], [yb], [y_zp, 0, 1, 1, 0, 0, 0])
+    total = spec.tensor("sum", abi.I32, shape)
+    spec.op("ADD", [xa, yb], [total])
+    out = spec.tensor("res", abi.I8, shape)
+    spec.op("RESCALE", [total, mo, so], [out], [0, LINEAR_ZP, 1, 1, 0, 0, 0])
+    return out, LINEAR_ZP
+
+
+def _inverted_residual(spec, q, rng, x, x_zp, cin, cout, t, stride):
+    h = x
+    h_zp = x_zp
+    hidden = cin * t
+    if t != 1:
+        h, h_zp = _conv_block(spec, q, rng, h, h_zp, cin, hidden, 1, 1, False, True)
+    h, h_zp = _conv_block(spec, q, rng, h, h_zp, hidden, hidden, 3, stride, True, True)
+    h, h_zp = _conv_block(spec, q, rng, h, h_zp, hidden, cout, 1, 1, False, False)
+    if stride == 1 and cin == cout:
+        h, h_zp = _residual(spec, q, rng, x, x_zp, h, h_zp)
+    return h, h_zp
+
+
+def inverted_residual_spec(batch=16, hw=56, channels=24, expansion=6, seed=1002, spread=False):
+    """BASELINE config 2: one MobileNetV2 inverted-residual block with the residual add."""
+    rng = np.random.default_rng(seed)
+    spec, q = Spec(), None
+    q = _Quant(rng, spread)
+    spec.inputs.append(("input", abi.I8, (batch, hw, hw, channels)))
+    y, _ = _inverted_residual(spec, q, rng, "input", -5, channels, channels, expansion, 1)
+    # the last operator writes the graph output tensor
+    _retarget_output(spec, y, "output")
+    return spec
+
+
+def mobilenetv2_spec(batch=32, image=224, seed=1003, spread=False, classes=1000):
+    """BASELINE config 3: MobileNetV2-shaped int8 graph; 35 CONV2D, 17 DEPTHWISE_CONV2D, AVG_POOL2D and one
+    MATMUL (the fully connected layer), RESCALE after every contraction, CLAMP for ReLU6."""
+    rng = np.random.default_rng(seed)
+    spec = Spec()
+    q = _Quant(rng, spread)
+    spec.inputs.append(("input", abi.I8, (batch, image, image, 3)))
+    x, zp = _conv_block(spec, q, rng, "input", -5, 3, 32, 3, 2, False, True)
+    cin = 32
+    for t, c, n, s in MOBILENETV2_BLOCKS:
+        for i in range(n):
+            x, zp = _inverted_residual(spec, q, rng, x, zp, cin, c, t, s if i == 0 else 1)
+            cin = c
+    x, zp = _conv_block(spec, q, rng, x, zp, cin, 1280, 1, 1, False, True)
+    n, h, w, c = spec.shape_of(x)
+    pooled = spec.tensor("pool", abi.I8, (n, 1, 1, c))
+    spec.op("AVG_POOL2D", [x], [pooled], [h, w, 1, 1, 0, 0, 0, 0, abi.ACC_I32, zp, zp])
+    flat = spec.tensor("flat", abi.I8, (1, n, c))
+    spec.op("RESHAPE", [pooled], [flat])
+    fc_w = spec.const("fc_w", rng.integers(-127, 127, (1, c, classes), endpoint=True).astype(np.int8))
+    logits = spec.tensor("fc_acc", abi.I32, (1, n, classes))
+    spec.op("MATMUL", [flat, fc_w], [logits], [zp, 0])
+    spec.macs["dense"] += n * c * classes
+    mult, shift = q.scale(1, c)
+    m, s = spec.const("m", mult), spec.const("s", shift)
+    spec.op("RESCALE", [logits, m, s], ["output"], [0, 0, 1, 1, 0, 0, 0])
+    spec.outputs.append(("output", abi.I8, (1, n, classes)))
+    return spec
+
+
+def _retarget_output(spec, produced, name):
+    """Makes the operator that produces `produced` write the external output tensor `name` instead."""
+    dtype, shape = spec.tensors.pop(produced)
+    for op in spec.ops:
+        op["out"] = [name if o == produced else o for o in op["out"]]
+        op["in"] = [name if i == produced else i for i in op["in"]]
+    spec.outputs.append((name, dtype, shape))
+
+
+def build(dev, spec, fuse=True):
+    """Creates the GraphPipeline for `spec` on `dev`: constants are uploaded, inputs/outputs become external
+    tensors, everything else lives in planned session memory."""
+    g = Graph(dev)
+    for name, dtype, shape in spec.inputs + spec.outputs:
+        g.external(name, dtype, shape)
+    for name, array in spec.consts.items():
+        g.const(name, array)
+    for name, (dtype, shape) in spec.tensors.items():
+        g.tensor(name, dtype, shape)
+    for name, _, _ in spec.inputs:
+        g.mark_input(name)
+    for op in spec.ops:
+        g.op(op["op"], op["in"], op["out"], op["iattr"], op["fattr"], op["name"])
+    for name, _, _ in spec.outputs:
+        g.mark_output(name)
+    g.finalize(fuse)
+    return g
+
+
+def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32):
+    """Times whole-graph dispatches of BASELINE config 3 (inputs resident in HBM) and returns the extra fields
+    bench.py adds to its JSON line."""
+    spec = mobilenetv2_spec(batch=batch)
+    g = build(dev, spec, fuse=True)
+    rng = np.random.default_rng(1003)
+    g.set_input("input", rng.integers(-128, 127, spec.inputs[0][2], endpoint=True).astype(np.int8))
+    for _ in range(warmup):
+        g.dispatch()
+    dev.sync()
+    ev0, ev1 = dev.event(), dev.event()
+    t0 = time.perf_counter()
+    dev.record(ev0)
+    for _ in range(steps):
+        g.dispatch()
+    dev.record(ev1)
+    dev.sync()
+    wall = (time.perf_counter() - t0) / steps
+    gpu_ms = dev.elapsed_ms(ev0, ev1) / steps
+    per_op = g.dispatch_profiled()
+    dev.sync()
+    by_kind = {}
+    for name, ms in per_op:
+        by_kind[name] = by_kind.get(name, 0.0) + ms
+    macs = spec.macs["dense"] + spec.macs["depthwise"]
+    res = {"mobilenetv2_b32": {
+        "img_per_s": batch / wall, "ms_per_graph": wall * 1e3, "gpu_ms_per_graph": gpu_ms,
+        "tops": 2.0 * macs / wall / 1e12, "gmac": macs / 1e9, "operators_executed": g.op_count(),
+        "operators_in_graph": len(spec.ops), "session_memory_bytes": g.session_size,
+        "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}}
+    g.close()
+    return res

@@ -1,0 +1,83 @@
+/*
+ * mlel_graph.h -- C view of the host-side operator surface (class mlel::graph::GraphPipeline).
+ *
+ * The C++ class is the drop-in for the reference's GraphPipeline (graph/compute_graph_op.hpp:1204-1549); this C
+ * wrapper exists so that harnesses without a C++ toolchain (ctypes, cgo, JNI ...) can build and run a data graph.
+ * Tensors are referred to by non-negative integer handles; every function returns 0 / a handle on success or a
+ * negative mlel_status, with the message in mlel_graph_last_error().  C++ exceptions (the reference's inner layer
+ * throws std::runtime_error: graph/compute_graph_op.cpp:50,363,477) are caught at this boundary.
+ */
+#ifndef MLEL_GRAPH_H
+#define MLEL_GRAPH_H
+
+#include "mlel_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mlel_graph mlel_graph;
+
+const char *mlel_graph_last_error(void);
+
+/* Reference: GraphPipeline constructor (compute_graph_op.cpp:2379-2390). */
+int mlel_graph_create(mlel_ctx *ctx, mlel_graph **out);
+void mlel_graph_destroy(mlel_graph *g);
+
+/* Reference: makeConstTensor / getConstTensor / makeConstCompositeTensor (compute_graph_op.cpp:2398-2420).
+ * strides may be NULL (packed).  The data is copied. */
+int mlel_graph_make_const_tensor(mlel_graph *g, uint32_t id, int32_t dtype, int32_t rank, const int64_t *dims,
+                                 const int64_t *strides, const void *data);
+int mlel_graph_get_const_tensor(mlel_graph *g, uint32_t id);
+int mlel_graph_make_const_composite_tensor(mlel_graph *g, int32_t dtype, int32_t rank, const int64_t *dims,
+                                           const void *data);
+/* Reference: makeDescriptorSetBinding / getTensor (compute_graph_op.cpp:2441-2455). */
+int mlel_graph_make_descriptor_set_binding(mlel_graph *g, uint32_t set, uint32_t binding, uint32_t array_index,
+                                           int32_t dtype, int32_t rank, const int64_t *dims, const int64_t *strides);
+int mlel_graph_get_tensor(mlel_graph *g, uint32_t set, uint32_t binding, uint32_t array_index);
+/* Reference: makeTensor (compute_graph_op.cpp:2457-2469). */
+int mlel_graph_make_tensor(mlel_graph *g, int32_t dtype, int32_t rank, const int64_t *dims, const int64_t *strides);
+int mlel_graph_make_input(mlel_graph *g, int tensor);
+int mlel_graph_make_output(mlel_graph *g, int tensor);
+
+/* One TOSA operator, named as in the TOSA.001000.1 extended instruction set ("CONV2D", "RESCALE", "ADD", ...).
+ * `inputs` / `outputs` are tensor handles in the order of the corresponding GraphPipeline::make<Op> signature
+ * (tensor arguments only); `iattr` carries the integer attributes and `fattr` the real-valued ones in signature
+ * order (vectors flattened).  See the table in the implementation (graph/c_api.cpp) for each operator. */
+int mlel_graph_make_op(mlel_graph *g, const char *tosa_name, const int *inputs, int n_inputs, const int *outputs,
+                       int n_outputs, const int64_t *iattr, int n_iattr, const double *fattr, int n_fattr,
+                       const char *debug_name);
+
+/* Fusion + session memory planning; then the session requirements
+ * (reference: vkGetDataGraphPipelineSessionMemoryRequirementsARM, graph_layer.cpp:1382-1389). */
+int mlel_graph_finalize(mlel_graph *g, int enable_fusion);
+int mlel_graph_session_memory_requirements(mlel_graph *g, uint64_t *size, uint64_t *alignment);
+/* Reference: vkBindDataGraphPipelineSessionMemoryARM (graph_layer.cpp:1391-1420). */
+int mlel_graph_bind_session_memory(mlel_graph *g, void *device_base);
+int mlel_graph_bind_external(mlel_graph *g, uint32_t set, uint32_t binding, uint32_t array_index, void *device_ptr);
+/* Reference: vkCmdDispatchDataGraphARM -> cmdBindAndDispatch (graph_layer.cpp:1844-1980). */
+int mlel_graph_dispatch(mlel_graph *g, void *stream);
+/* Dispatch with a pair of events around every operator; per-operator milliseconds are written to `ms`
+ * (reference: the profiler's timestamp pairs, graph/graph_profiler.cpp:157-191).  Returns the operator count. */
+int mlel_graph_dispatch_profiled(mlel_graph *g, void *stream, float *ms, int capacity);
+
+/* Introspection (tests, profiler). */
+int mlel_graph_op_count(mlel_graph *g);        /* operators executed after fusion */
+int mlel_graph_op_name(mlel_graph *g, int index, char *buf, size_t len); /* "CONV2D+RESCALE+CLAMP", ... */
+int mlel_graph_session_tensor_count(mlel_graph *g);
+/* offset == UINT64_MAX: the tensor was folded into a fused kernel and has no storage */
+int mlel_graph_session_tensor_info(mlel_graph *g, int index, int *tensor, uint64_t *offset, uint64_t *size,
+                                   uint32_t *first_use, uint32_t *last_use);
+
+/* The interval allocator on its own (reference: details::allocateIntervals, interval_memory_planner.cpp:170-215).
+ * intervals: n x {id, first, last, size, order}; unseen: m x {id, size}; out_offsets: (n + m) x {id, offset}. */
+int mlel_graph_allocate_intervals(const uint64_t *intervals, int n, const uint64_t *unseen, int m,
+                                  uint64_t alignment, uint64_t *out_offsets, uint64_t *out_memory_size);
+
+/* VkFormat number -> mlel_dtype (reference: getFormatInfo, common/utils.cpp:119-228); negative when unsupported. */
+int mlel_graph_dtype_from_vk_format(int32_t vk_format);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLEL_GRAPH_H */

@@ -1,0 +1,87 @@
+"""GPU parity of whole data graphs executed through the host-side GraphPipeline (fusion + planned session memory)
+against the CPU oracle executing the same description operator by operator, unfused."""
+import importlib
+
+import numpy as np
+import pytest
+
+from hip_util import gpu_available, hb
+from oracle_graph import run_spec
+
+graphs = importlib.import_module("ai-ml-emulation-layer-for-vulkan_amd.graphs")
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not gpu_available():
+        pytest.skip("no GPU visible")
+    d = hb.Device(0)
+    yield d
+    d.close()
+
+
+def run_graph(dev, spec, x, fuse):
+    g = graphs.build(dev, spec, fuse=fuse)
+    g.set_input("input", x)
+    g.dispatch()
+    out = g.get_output("output")
+    # a second dispatch of the same pipeline (session memory is reused) must give the same answer
+    g.dispatch()
+    again = g.get_output("output")
+    names = g.op_names()
+    g.close()
+    np.testing.assert_array_equal(out, again)
+    return out, names
+
+
+def random_input(spec, seed):
+    rng = np.random.default_rng(seed)
+    return rng.integers(-128, 127, spec.inputs[0][2], endpoint=True).astype(np.int8)
+
+
+@pytest.mark.parametrize("spread", [False, True], ids=["literal_scales", "spread_scales"])
+@pytest.mark.parametrize("fuse", [False, True], ids=["unfused", "fused"])
+def test_inverted_residual_block_small(dev, oracle, fuse, spread):
+    spec = graphs.inverted_residual_spec(batch=2, hw=14, spread=spread)
+    x = random_input(spec, 21)
+    exp, _ = run_spec(oracle, spec, {"input": x})
+    out, names = run_graph(dev, spec, x, fuse)
+    assert len(names) == (4 if fuse else len(spec.ops))
+    np.testing.assert_array_equal(out, exp["output"])
+    if spread:
+        assert len(np.unique(out)) > 50  # the result really uses the int8 range
+
+
+def test_config2_inverted_residual_full_size(dev, oracle):
+    """BASELINE config 2: 16x56x56x24, t=6, residual add."""
+    spec = graphs.inverted_residual_spec(batch=16, hw=56, spread=True)
+    x = random_input(spec, 1002)
+    exp, _ = run_spec(oracle, spec, {"input": x})
+    out, _ = run_graph(dev, spec, x, True)
+    np.testing.assert_array_equal(out, exp["output"])
+
+
+@pytest.mark.parametrize("fuse", [False, True], ids=["unfused", "fused"])
+def test_mobilenetv2_small(dev, oracle, fuse):
+    spec = graphs.mobilenetv2_spec(batch=2, image=64, spread=True, classes=40)
+    x = random_input(spec, 33)
+    exp, _ = run_spec(oracle, spec, {"input": x})
+    out, names = run_graph(dev, spec, x, fuse)
+    np.testing.assert_array_equal(out, exp["output"])
+    assert len(np.unique(out)) > 20
+
+
+def test_config3_mobilenetv2_b32_full_size(dev, oracle):
+    """BASELINE config 3 at full size (32x224x224x3): fused GPU graph == unfused oracle graph, bit for bit, and the
+    first image alone gives the same logits as inside the batch (operators are independent across the batch)."""
+    spec = graphs.mobilenetv2_spec(batch=32, spread=True)
+    x = random_input(spec, 1003)
+    out, names = run_graph(dev, spec, x, True)
+    assert len(names) == 65
+    exp, _ = run_spec(oracle, spec, {"input": x})
+    np.testing.assert_array_equal(out, exp["output"])
+    one = graphs.mobilenetv2_spec(batch=1, spread=True)
+    out1, _ = run_graph(dev, one, x[:1], True)
+    np.testing.assert_array_equal(out1[0, 0], out[0, 0])
