@@ -252,39 +252,36 @@ __device__ __forceinline__ int32_t requant_i32(int32_t acc, int32_t mult, int32_
     return r;
 }
 
-// The same arithmetic with everything that depends only on the channel hoisted out of the per-element path:
-//   (value * mult + round) >> shift,  value = acc - in_zp,  round = 2^(shift-1) [+/- 2^30 by the sign of value]
-// becomes  acc * mult + (round - in_zp * mult)  as one 64-bit multiply-add, plus the sign-dependent nudge.
+// Per-channel RESCALE constants with everything that does not depend on the accumulator folded in:
+//   result = clamp(int32((int64(acc) * mult + R) >> shift) + out_zp),
+//   R = 2^(shift-1) - in_zp * mult  (+ 2^30 when acc >= in_zp, - 2^30 otherwise, if double rounding applies).
+// Both signed variants of R are stored so that the choice is one compare and two selects.
 struct ChanScale {
+    int64_t round_pos;
+    int64_t round_neg;
     int32_t mult;
-    int32_t shift;     // clamped to 0..63
-    int32_t nudge;     // 2^30 when double rounding applies to this channel (shift > 31), else 0
-    int32_t pad;
-    int64_t round;     // 2^(shift-1) - in_zp * mult (wraparound), 0 when shift == 0
+    int32_t shift;
 };
 
 __host__ __device__ inline ChanScale make_chan_scale(int32_t mult, int32_t shift, const RescaleParams &p) {
     ChanScale c;
     c.mult = mult;
     c.shift = shift < 0 ? 0 : (shift > 63 ? 63 : shift);
-    c.nudge = (p.double_round && shift > 31) ? (1 << 30) : 0;
-    c.pad = 0;
+    const uint64_t nudge = (p.double_round && shift > 31) ? (uint64_t(1) << 30) : 0;
     const uint64_t base = shift > 0 ? (uint64_t(1) << (c.shift - 1)) : 0;
-    c.round = (int64_t)(base - (uint64_t)(int64_t)p.in_zp * (uint64_t)(int64_t)mult);
+    const uint64_t round = base - (uint64_t)(int64_t)p.in_zp * (uint64_t)(int64_t)mult;
+    c.round_pos = (int64_t)(round + nudge);
+    c.round_neg = (int64_t)(round - nudge);
     return c;
 }
 
-template <bool ZERO_IN_ZP>
+// out_lo / out_hi span the whole int32 range for 32-bit outputs, so the clamp is always applied.
 __device__ __forceinline__ int32_t requant_chan(int32_t acc, const ChanScale &c, const RescaleParams &p) {
-    // sign of value = acc - in_zp as an all-ones / all-zeros mask
-    const int32_t neg = ZERO_IN_ZP ? (acc >> 31) : (acc < p.in_zp ? -1 : 0);
-    const int32_t nudge = (c.nudge ^ neg) - neg;  // +2^30, -2^30 or 0
-    uint64_t t = (uint64_t)((int64_t)acc * (int64_t)c.mult) + (uint64_t)c.round;
-    t += (uint64_t)(int64_t)nudge;
-    int32_t r = (int32_t)((int64_t)t >> c.shift);
-    r = (int32_t)((uint32_t)r + (uint32_t)p.out_zp);
-    if (p.clamp_out) r = min(max(r, p.out_lo), p.out_hi);
-    return r;
+    const int64_t r = acc < p.in_zp ? c.round_neg : c.round_pos;
+    const uint64_t t = (uint64_t)((int64_t)acc * (int64_t)c.mult) + (uint64_t)r;
+    int32_t v = (int32_t)((int64_t)t >> c.shift);
+    v = (int32_t)((uint32_t)v + (uint32_t)p.out_zp);
+    return min(max(v, p.out_lo), p.out_hi);
 }
 
 int make_rescale_params(const mlel_rescale_attr *attr, int in_dtype, int out_dtype, const mlel_clamp_attr *clamp,

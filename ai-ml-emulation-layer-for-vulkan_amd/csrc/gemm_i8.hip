@@ -56,6 +56,7 @@ struct GemmArgs {
     int64_t out_batch, ldo;  // ldo in elements
     int32_t out_size;        // bytes per output element: 1, 2 or 4
     int32_t out_vec_ok;      // four consecutive channels may be stored as one aligned unit
+    uint32_t o_bytes;        // per-batch extent of the output when it fits 31-bit buffer offsets, else 0
     // fused epilogue
     int32_t fused;
     const char *mult;  // int32 or int16 per channel (or one)
@@ -221,11 +222,12 @@ enum XMode {
 };
 enum WMode {
     W_ROWS = 0,     // [N][K], 16-byte pieces
-    W_KMAJOR = 1,   // [K][N] kept K-major in LDS; MFMA operands are gathered with ds_read_b64_tr_b8
+    W_KMAJOR = 1,   // [K][N] kept K-major in LDS; MFMA operands are gathered with ds_read_b64_tr_b8; 16-byte loads
     W_GENERIC = 2,  // either layout, any alignment
+    W_KMAJOR4 = 3,  // as W_KMAJOR for rows that are only dword aligned (N % 4 == 0): four dword loads per piece
 };
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int XMODE, int WMODE, bool SUMS>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int XMODE, int WMODE, bool SUMS, bool Q8>
 __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wavefront sub-tile
     constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 MFMA tiles per wavefront
@@ -316,7 +318,7 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
             if (WMODE == W_ROWS) {
                 const int n = n_base + (c >> 2);
                 if (n < g.N) woff[i] = (uint32_t)n * (uint32_t)g.ldw + (c & 3) * 16;
-            } else if (WMODE == W_KMAJOR) {
+            } else if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
                 // piece c = 16 channels of K row c / N16; rows at or beyond K lie past the end of the buffer
                 // resource and read as 0 without a test
                 const int n = n_base + (c % N16) * 16;
@@ -364,11 +366,11 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
                 const bool kin = k0 + (c & 3) * 16 < g.K;
                 wr[i] = buf_load16(wres, kin ? woff[i] + (uint32_t)k0 : kOobOffset);
             }
-        } else if (WMODE == W_KMAJOR) {
+        } else if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
 #pragma unroll
             for (int i = 0; i < WCHUNKS; i++) {
                 const uint32_t off = woff[i] + (uint32_t)k0 * (uint32_t)g.ldw;
-                if (g.wch == 16) {
+                if (WMODE == W_KMAJOR) {
                     wr[i] = buf_load16(wres, off);
                 } else {  // rows are only dword aligned: four loads, channels at or beyond N masked
                     const int n = n_base + ((tid + NTHREADS * i) % N16) * 16;
@@ -403,7 +405,7 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
             if (XMODE == X_TAP && ((xpad >> i) & 1u)) v = make_uint4(z, z, z, z);
             *reinterpret_cast<uint4 *>(xd + ((tid >> 2) + 64 * i) * PITCH + x_kc * 16) = v;
         }
-        if (WMODE == W_KMAJOR) {
+        if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
 #pragma unroll
             for (int i = 0; i < WCHUNKS; i++) {
                 const int c = tid + NTHREADS * i;
@@ -459,7 +461,7 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
             for (int i = 0; i < TM; i++) xf[i] = *reinterpret_cast<const v4i *>(xd + i * 32 * PITCH + kk * 32);
 #pragma unroll
             for (int j = 0; j < TN; j++) {
-                if (WMODE == W_KMAJOR) {
+                if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
                     const char *p = wt + kk * 32 * PW + j * 32;
                     const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(p));
                     const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(p + 8 * PW));
@@ -486,30 +488,31 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
         }
     };
 
-    // ---- main loop: two K steps of global loads in flight (register sets A and B), two LDS buffers.
-    // Invariant at the top of iteration `step` (even): LDS[0] holds step, set B holds step+1 (loads issued).
+    // ---- main loop: a ring of DEPTH register sets keeps DEPTH - 1 K steps of global loads in flight while one
+    // step is multiplied out of LDS (two LDS buffers).  At the top of sub-iteration s: LDS[s & 1] holds step s and
+    // register set (s + j) % DEPTH holds step s + j for j = 1 .. DEPTH - 1; the set of step s is free again.
+    // Every prefetch and stage is unconditional: a K step at or beyond K loads nothing (buffer bounds / tap state
+    // return zeros) and is never multiplied, and the straight-line body lets the compiler count exactly how many
+    // loads may remain in flight at each wait instead of draining them all.
+    constexpr int DEPTH = 4;
     const int nk = (g.K + BK - 1) / BK;
-    uint4 xa[XROWS], wa[WCHUNKS], xb2[XROWS], wb2[WCHUNKS];
-    uint32_t pa = 0, pb = 0;
-    // Every prefetch and stage below is unconditional: a K step at or beyond K loads nothing (the buffer bounds /
-    // tap state return zeros) and is never multiplied, and straight-line code lets the compiler count exactly how
-    // many loads may stay in flight at each wait instead of draining them all.
-    prefetch(0, xa, wa, pa);
-    prefetch(BK, xb2, wb2, pb);
-    stage(0, xa, wa, pa);
+    uint4 xr[DEPTH][XROWS], wr[DEPTH][WCHUNKS];
+    uint32_t xp[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) prefetch(d * BK, xr[d], wr[d], xp[d]);
+    stage(0, xr[0], wr[0], xp[0]);
     __syncthreads();
-    int step = 0;
-    for (; step + 1 < nk; step += 2) {  // LDS[0] holds `step`, registers B hold `step + 1`
-        prefetch((step + 2) * BK, xa, wa, pa);
-        compute(0);
-        stage(1, xb2, wb2, pb);
-        __syncthreads();
-        prefetch((step + 3) * BK, xb2, wb2, pb);
-        compute(1);
-        stage(0, xa, wa, pa);
-        __syncthreads();
+    for (int step = 0; step < nk; step += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            if (step + d < nk) {  // uniform
+                prefetch((step + d + DEPTH) * BK, xr[d], wr[d], xp[d]);
+                compute(d & 1);
+                stage((d + 1) & 1, xr[(d + 1) % DEPTH], wr[(d + 1) % DEPTH], xp[(d + 1) % DEPTH]);
+                __syncthreads();
+            }
+        }
     }
-    if (step < nk) compute(0);  // odd number of K steps: the last one sits in LDS[0]
 
     // ---- fold the zero-point terms that depend on the channel only into the per-channel bias
     if (need_wsum && wave_m == 0) {
@@ -533,6 +536,43 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
     // ---- epilogue: lane holds output position m = lane % 32 of each tile row and, per register group q, the four
     // channels n0 .. n0+3 with n0 = 8q + 4 * (lane / 32)
     char *ob = g.out + (int64_t)batch * g.out_batch;
+    if (Q8) {
+        // Fused RESCALE(+CLAMP) to 8-bit outputs, N % 4 == 0, output extent below 2^31: straight-line code.  Rows and
+        // channels outside the problem get an offset beyond the buffer bounds, which drops the store.
+        const __amdgpu_buffer_rsrc_t ores = make_rsrc(ob, g.o_bytes);
+        uint32_t row_off[TM];
+        int32_t xcorr[TM];
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
+            row_off[i] = m < g.M ? (uint32_t)m * (uint32_t)g.ldo : kOobOffset;
+            xcorr[i] = need_xsum ? xsum[i] : 0;
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int nl = wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+                const int n0 = n_base + nl;
+                ChanParams c[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) c[e] = cp[nl + e];
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    uint32_t packed = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)c[e].bias_adj -
+                                                    (uint32_t)xcorr[i]);
+                        packed |= ((uint32_t)requant_chan(a, c[e].q, g.rp) & 0xffu) << (8 * e);
+                    }
+                    const uint32_t off = (n0 < g.N && row_off[i] != kOobOffset) ? row_off[i] + (uint32_t)n0 : kOobOffset;
+                    __builtin_amdgcn_raw_buffer_store_b32(packed, ores, (int)off, 0, 0);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
@@ -552,10 +592,8 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
                         (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)cp[nl + e].bias_adj - (uint32_t)xcorr);
                     if (!g.fused)
                         v[e] = a;
-                    else if (g.rp.in_zp == 0)
-                        v[e] = requant_chan<true>(a, cp[nl + e].q, g.rp);
                     else
-                        v[e] = requant_chan<false>(a, cp[nl + e].q, g.rp);
+                        v[e] = requant_chan(a, cp[nl + e].q, g.rp);
                 }
                 const int64_t off = (int64_t)m * g.ldo + n0;
                 if (g.out_vec_ok && n0 + 3 < g.N) {
@@ -592,25 +630,33 @@ constexpr size_t smem_bytes() {
     return (size_t)2 * BM * PITCH + (size_t)2 * w_buf_bytes<BN>() + (size_t)BN * sizeof(ChanParams);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool SUMS>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool SUMS, bool Q8>
 void launch_tile(const GemmArgs &g, int xmode, int wmode, dim3 grid, hipStream_t s) {
     const size_t sm = smem_bytes<BM, BN>();
     if (xmode == X_PLAIN && wmode == W_ROWS)
-        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_ROWS, SUMS><<<grid, dim3(NTHREADS), sm, s>>>(g);
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_ROWS, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
     else if (xmode == X_TAP && wmode == W_ROWS)
-        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_TAP, W_ROWS, SUMS><<<grid, dim3(NTHREADS), sm, s>>>(g);
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_TAP, W_ROWS, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
     else if (xmode == X_PLAIN && wmode == W_KMAJOR)
-        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR, SUMS><<<grid, dim3(NTHREADS), sm, s>>>(g);
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    else if (xmode == X_PLAIN && wmode == W_KMAJOR4)
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR4, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
     else
-        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_GENERIC, W_GENERIC, SUMS><<<grid, dim3(NTHREADS), sm, s>>>(g);
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_GENERIC, W_GENERIC, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 void launch_tile_zp(const GemmArgs &g, int xmode, int wmode, dim3 grid, hipStream_t s) {
-    if (g.zx != 0 || g.zw != 0)
-        launch_tile<BM, BN, WAVES_M, WAVES_N, true>(g, xmode, wmode, grid, s);
+    const bool sums = g.zx != 0 || g.zw != 0;
+    const bool q8 = g.fused && g.out_size == 1 && g.out_vec_ok && g.o_bytes != 0;
+    if (sums && q8)
+        launch_tile<BM, BN, WAVES_M, WAVES_N, true, true>(g, xmode, wmode, grid, s);
+    else if (sums)
+        launch_tile<BM, BN, WAVES_M, WAVES_N, true, false>(g, xmode, wmode, grid, s);
+    else if (q8)
+        launch_tile<BM, BN, WAVES_M, WAVES_N, false, true>(g, xmode, wmode, grid, s);
     else
-        launch_tile<BM, BN, WAVES_M, WAVES_N, false>(g, xmode, wmode, grid, s);
+        launch_tile<BM, BN, WAVES_M, WAVES_N, false, false>(g, xmode, wmode, grid, s);
 }
 
 int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
@@ -625,9 +671,9 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
             xmode = X_TAP;
     }
     if (!g.w_kmajor && g.wch == 16 && small) wmode = W_ROWS;
-    if (g.w_kmajor && g.wch >= 4 && small) wmode = W_KMAJOR;
+    if (g.w_kmajor && g.wch >= 4 && small) wmode = g.wch == 16 ? W_KMAJOR : W_KMAJOR4;
     const bool fast = (xmode == X_PLAIN && wmode == W_ROWS) || (xmode == X_TAP && wmode == W_ROWS) ||
-                      (xmode == X_PLAIN && wmode == W_KMAJOR);
+                      (xmode == X_PLAIN && (wmode == W_KMAJOR || wmode == W_KMAJOR4));
     if (!fast) {
         xmode = X_GENERIC;
         wmode = W_GENERIC;
@@ -679,6 +725,8 @@ int fill_epilogue(GemmArgs &g, const mlel_tensor *out, const FusedEpilogue *epi)
     const int64_t unit = 4 * g.out_size;
     g.out_vec_ok = (g.N % 4 == 0) && ((g.ldo * g.out_size) % unit == 0) && ((uintptr_t)out->ptr % unit == 0) &&
                    ((g.out_batch) % unit == 0);
+    const int64_t ob = ((int64_t)(g.M - 1) * g.ldo + g.N) * g.out_size;
+    g.o_bytes = ob < (int64_t(1) << 31) ? (uint32_t)ob : 0;
     return 0;
 }
 

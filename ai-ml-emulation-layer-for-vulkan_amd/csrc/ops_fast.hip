@@ -71,9 +71,9 @@ __global__ void __launch_bounds__(kBlock) rescale_add_rescale_i8x16_kernel(uint4
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             const int32_t x1 = (int8_t)(av[d] >> (8 * e)), x2 = (int8_t)(bv[d] >> (8 * e));
-            const int32_t r1 = requant_chan<false>(x1, q1, s1.p), r2 = requant_chan<false>(x2, q2, s2.p);
+            const int32_t r1 = requant_chan(x1, q1, s1.p), r2 = requant_chan(x2, q2, s2.p);
             const int32_t sum = (int32_t)((uint32_t)r1 + (uint32_t)r2);
-            const int32_t r = so.p.in_zp == 0 ? requant_chan<true>(sum, qo, so.p) : requant_chan<false>(sum, qo, so.p);
+            const int32_t r = requant_chan(sum, qo, so.p);
             packed |= (uint32_t)(uint8_t)r << (8 * e);
         }
         ov[d] = packed;
@@ -249,8 +249,7 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
         for (int e = 0; e < 4; e++) {
             int32_t s = (int32_t)((uint32_t)acc[t][e] + (uint32_t)ch[e].bias_adj);
             if (ZW) s = (int32_t)((uint32_t)s - (uint32_t)a.zw * (uint32_t)xs[t][e]);
-            if (a.fused) s = a.scale.p.in_zp == 0 ? requant_chan<true>(s, ch[e].q, a.scale.p)
-                                                  : requant_chan<false>(s, ch[e].q, a.scale.p);
+            if (a.fused) s = requant_chan(s, ch[e].q, a.scale.p);
             v[e] = s;
         }
         const int64_t off = (orow + ox) * a.C + c;
