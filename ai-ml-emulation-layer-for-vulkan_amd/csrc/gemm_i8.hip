@@ -494,7 +494,7 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
     // Every prefetch and stage is unconditional: a K step at or beyond K loads nothing (buffer bounds / tap state
     // return zeros) and is never multiplied, and the straight-line body lets the compiler count exactly how many
     // loads may remain in flight at each wait instead of draining them all.
-    constexpr int DEPTH = 4;
+    constexpr int DEPTH = (XMODE == X_GENERIC || WMODE == W_GENERIC) ? 2 : 4;  // the generic fetch state is large
     const int nk = (g.K + BK - 1) / BK;
     uint4 xr[DEPTH][XROWS], wr[DEPTH][WCHUNKS];
     uint32_t xp[DEPTH];
