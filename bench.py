@@ -27,6 +27,11 @@ PKG = "ai-ml-emulation-layer-for-vulkan_amd"
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X published dense int8 peak, TOP/s
 HBM_PEAK_GBS = 8000.0         # MI355X published HBM3E bandwidth, GB/s
 
+# HBM bytes per launch of the config 1 kernel from two rocprofv3 --pmc runs of this script (profiles/):
+# FETCH_SIZE 6252 KiB scaled by 2.0 plus WRITE_SIZE 4096 KiB scaled by 1.0, the factors being what the same
+# counters read for the 256 MiB copy kernel below (131083 KiB and 262144 KiB).
+CONFIG1_TRAFFIC_BYTES = int((6252 * 2.0 + 4096 * 1.0) * 1024)
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -74,6 +79,14 @@ def bench_config1(dev, abi, steps, warmup):
     }
     out = to.download()
     dev.stream = None
+    # the same step when the caller hands over host buffers: upload A and B, launch, download the result
+    t0 = time.perf_counter()
+    for _ in range(3):
+        ta.upload(a)
+        tb.upload(b)
+        step()
+        to.download()
+    res["host_buffers_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / 3
     return res, (a, b, mult, shift, out)
 
 
@@ -173,7 +186,8 @@ def main():
                                "+ per-tensor RESCALE (1518500250, 39, double_round) -> int8, one fused launch",
                    "device": info["name"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "mfma", "achieved": c1["kernel_tops"], "peak": INT8_MFMA_PEAK_TOPS / 1.0,
-                     "unit": "TFLOP/s", "ops_are": "int8 multiply and add counted as 2 ops", "frac": c1["kernel_tops"] / INT8_MFMA_PEAK_TOPS, "traffic": None,
+                     "unit": "TFLOP/s", "ops_are": "int8 multiply and add counted as 2 ops", "frac": c1["kernel_tops"] / INT8_MFMA_PEAK_TOPS,
+                     "traffic": CONFIG1_TRAFFIC_BYTES,
                      "kernel": "gemm_i8_kernel<128,128,2,2>", "kernel_ms": c1["kernel_ms"],
                      "algorithmic_bytes": c1["algorithmic_bytes"],
                      "hbm_frac_if_bandwidth_bound": c1["algorithmic_bytes"] / (c1["kernel_ms"] * 1e-3) / 1e9 /
@@ -181,6 +195,7 @@ def main():
         "cpu_baseline": cpu,
         "bit_exact_vs_oracle": parity_ok,
         "copy_kernel_gbs": copy_gbs,
+        "host_buffers_ms_per_step": c1["host_buffers_ms_per_step"],
     }
     line.update(extra)
     print(json.dumps(line), flush=True)
