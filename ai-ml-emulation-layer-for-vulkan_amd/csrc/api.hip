@@ -262,6 +262,10 @@ int mlel_hip_reshape(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const 
     MLEL_TRY(check_tensor(out, "reshape out"));
     MLEL_TRY(check_tensor(in, "reshape in"));
     MLEL_REQUIRE(dt_size(in->dtype) == dt_size(out->dtype), MLEL_ERR_INVALID, "reshape: element size differs");
+    // two packed tensors of the same element count: RESHAPE (reshape.comp:16-27, a flat-index copy) is a plain copy
+    if (is_packed(in) && is_packed(out) && numel(in) == numel(out) && ((uintptr_t)in->ptr % 16) == 0 &&
+        ((uintptr_t)out->ptr % 16) == 0)
+        return mlel_hip_copy_kernel(ctx, stream, out->ptr, in->ptr, (size_t)numel(out) * dt_size(out->dtype));
     return move_generic_launch((hipStream_t)stream, kReshape, out, in, nullptr, 0, 0);
 }
 

@@ -219,12 +219,14 @@ enum XMode {
     X_PLAIN = 0,    // X[m][k] = base + m * pitch + k, 16-byte pieces (MATMUL A; 1x1 stride-1 CONV2D on a dense input)
     X_TAP = 1,      // 16-byte pieces, IC % 64 == 0: one K step lies inside one filter tap (uniform tap state)
     X_GENERIC = 2,  // anything else: per-piece tap tracking, 16 / 4 / 1-byte loads
+    X_PLAIN4 = 3,   // as X_PLAIN for rows that are only dword aligned (K % 4 == 0): four dword loads per piece
 };
 enum WMode {
     W_ROWS = 0,     // [N][K], 16-byte pieces
     W_KMAJOR = 1,   // [K][N] kept K-major in LDS; MFMA operands are gathered with ds_read_b64_tr_b8; 16-byte loads
     W_GENERIC = 2,  // either layout, any alignment
     W_KMAJOR4 = 3,  // as W_KMAJOR for rows that are only dword aligned (N % 4 == 0): four dword loads per piece
+    W_ROWS4 = 4,    // as W_ROWS for rows that are only dword aligned (K % 4 == 0)
 };
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int XMODE, int WMODE, bool SUMS, bool Q8>
@@ -315,7 +317,7 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
         const int c = tid + NTHREADS * i;
         woff[i] = kOobOffset;
         if (c < BN * 4) {
-            if (WMODE == W_ROWS) {
+            if (WMODE == W_ROWS || WMODE == W_ROWS4) {
                 const int n = n_base + (c >> 2);
                 if (n < g.N) woff[i] = (uint32_t)n * (uint32_t)g.ldw + (c & 3) * 16;
             } else if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
@@ -334,6 +336,17 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
             const bool kin = k0 + x_kc * 16 < g.K;
 #pragma unroll
             for (int i = 0; i < XROWS; i++) xr[i] = buf_load16(xres, kin ? xoff[i] + (uint32_t)k0 : kOobOffset);
+        } else if (XMODE == X_PLAIN4) {
+            const int kp = k0 + x_kc * 16;  // K % 4 == 0: a dword lies wholly inside or outside the row
+#pragma unroll
+            for (int i = 0; i < XROWS; i++) {
+                const uint32_t off = xoff[i] + (uint32_t)k0;
+                const bool v = xoff[i] != kOobOffset;
+                xr[i].x = buf_load4(xres, (v && kp + 0 < g.K) ? off + 0 : kOobOffset);
+                xr[i].y = buf_load4(xres, (v && kp + 4 < g.K) ? off + 4 : kOobOffset);
+                xr[i].z = buf_load4(xres, (v && kp + 8 < g.K) ? off + 8 : kOobOffset);
+                xr[i].w = buf_load4(xres, (v && kp + 12 < g.K) ? off + 12 : kOobOffset);
+            }
         } else if (XMODE == X_TAP) {
             const bool kin = tap_ky < g.KH;
             const int oy = tap_ky * g.dy, ox = tap_kx * g.dx;
@@ -365,6 +378,17 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
                 const int c = tid + NTHREADS * i;
                 const bool kin = k0 + (c & 3) * 16 < g.K;
                 wr[i] = buf_load16(wres, kin ? woff[i] + (uint32_t)k0 : kOobOffset);
+            }
+        } else if (WMODE == W_ROWS4) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int kp = k0 + ((tid + NTHREADS * i) & 3) * 16;
+                const uint32_t off = woff[i] + (uint32_t)k0;
+                const bool v = woff[i] != kOobOffset;
+                wr[i].x = buf_load4(wres, (v && kp + 0 < g.K) ? off + 0 : kOobOffset);
+                wr[i].y = buf_load4(wres, (v && kp + 4 < g.K) ? off + 4 : kOobOffset);
+                wr[i].z = buf_load4(wres, (v && kp + 8 < g.K) ? off + 8 : kOobOffset);
+                wr[i].w = buf_load4(wres, (v && kp + 12 < g.K) ? off + 12 : kOobOffset);
             }
         } else if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
 #pragma unroll
@@ -411,7 +435,7 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
                 const int c = tid + NTHREADS * i;
                 if (c < BN * 4) *reinterpret_cast<uint4 *>(wd + (c / N16) * PW + (c % N16) * 16) = wr[i];
             }
-        } else if (WMODE == W_ROWS || !g.w_kmajor) {
+        } else if (WMODE == W_ROWS || WMODE == W_ROWS4 || !g.w_kmajor) {
 #pragma unroll
             for (int i = 0; i < WCHUNKS; i++) {
                 const int c = tid + NTHREADS * i;
@@ -641,6 +665,8 @@ void launch_tile(const GemmArgs &g, int xmode, int wmode, dim3 grid, hipStream_t
         gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
     else if (xmode == X_PLAIN && wmode == W_KMAJOR4)
         gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR4, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    else if (xmode == X_PLAIN4 && wmode == W_ROWS4)
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN4, W_ROWS4, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
     else
         gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_GENERIC, W_GENERIC, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
 }
@@ -670,10 +696,15 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
         else if (g.IC % BK == 0)
             xmode = X_TAP;
     }
+    if (g.xch == 4 && small && g.plain && g.K % 4 == 0) xmode = X_PLAIN4;
     if (!g.w_kmajor && g.wch == 16 && small) wmode = W_ROWS;
+    if (!g.w_kmajor && g.wch == 4 && small && g.K % 4 == 0) wmode = W_ROWS4;
+    if (xmode == X_PLAIN4 && wmode == W_ROWS) wmode = W_ROWS4;  // the dword forms also serve 16-byte aligned rows
+    if (xmode == X_PLAIN && wmode == W_ROWS4) xmode = X_PLAIN4;
     if (g.w_kmajor && g.wch >= 4 && small) wmode = g.wch == 16 ? W_KMAJOR : W_KMAJOR4;
     const bool fast = (xmode == X_PLAIN && wmode == W_ROWS) || (xmode == X_TAP && wmode == W_ROWS) ||
-                      (xmode == X_PLAIN && (wmode == W_KMAJOR || wmode == W_KMAJOR4));
+                      (xmode == X_PLAIN && (wmode == W_KMAJOR || wmode == W_KMAJOR4)) ||
+                      (xmode == X_PLAIN4 && wmode == W_ROWS4);
     if (!fast) {
         xmode = X_GENERIC;
         wmode = W_GENERIC;

@@ -113,14 +113,16 @@ namespace {
 // ---------------------------------------------------------------------------------------------------------------
 // DEPTHWISE_CONV2D 3x3, int8 NHWC, channel multiplier 1, fused RESCALE (+CLAMP) or int32 output.
 //
-// Work item = 4 consecutive channels x TX consecutive output positions of one output row.  Lanes run over the
-// channel quads first, so every load and store instruction of a wavefront covers consecutive dwords of a pixel.
-// For each input column the three rows are transposed (v_perm_b32) into one dword per channel holding the three
-// vertical taps; a v_dot4_i32_i8 against the matching weight column then adds three taps at once, and a column is
-// shared by up to three neighbouring outputs.  Padded taps are filled with the input zero point, so the expansion
+// Work item = 4 consecutive channels x TX consecutive output columns x TY consecutive output rows.  Lanes run over
+// the channel quads first, so every load and store instruction of a wavefront covers consecutive dwords of a pixel.
+// For each input column the rows are transposed (v_perm_b32) into one dword per channel holding three vertical
+// taps; a v_dot4_i32_i8 against the matching weight column then adds three taps at once, and a column is shared by
+// up to three neighbouring outputs.  Padded taps are filled with the input zero point, so the expansion
 //   sum (x - zi)(w - zw) = sum x*w - zw * sum x - zi * sum w + 9 * zi * zw
-// gives exactly the reference's result (padded taps contribute nothing).  Weight columns and per-channel
-// requantisation constants are prepared once per block in LDS.
+// gives exactly the reference's result (padded taps contribute nothing).  Every thread prepares the weight columns
+// and requantisation constants of its own four channels in registers (dword loads that hit in cache), so there is
+// no shared-memory stage and no barrier.  Consecutive blocks are dealt to the XCDs in contiguous runs, so rows
+// shared by vertically adjacent items are fetched into one L2 only.
 // ---------------------------------------------------------------------------------------------------------------
 struct DwArgs {
     const int8_t *x, *w;
@@ -131,61 +133,82 @@ struct DwArgs {
     int32_t sy, sx, pad_t, pad_l, zi, zw, bias_len;
     int32_t fused, out_size;
     ScaleRef scale;
-    int64_t items;  // N * OH * strips * C/4
-    int32_t strips;
+    int64_t items;  // N * row groups * strips * C/4
+    int32_t strips, row_groups;
+    int32_t blocks, chunk;  // launch geometry: `chunk` consecutive blocks of items per XCD
 };
 
-struct DwChan {  // per channel, in LDS (32 bytes)
-    ChanScale q;
-    int32_t bias_adj;
-    int32_t pad;
-};
+// 3 rows x 4 channels (bytes) -> 4 channels x (3 taps, 0)
+__device__ __forceinline__ void transpose_3x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t (&col)[4]) {
+    // selector bytes 0-3 pick from the second operand, 4-7 from the first, 0x0c gives zero
+    const uint32_t t0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);  // [r0.b0 r1.b0 r0.b1 r1.b1]
+    const uint32_t t1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);  // [r0.b2 r1.b2 r0.b3 r1.b3]
+    col[0] = __builtin_amdgcn_perm(r2, t0, 0x0c040100u);             // [t0.b0 t0.b1 r2.b0 0]
+    col[1] = __builtin_amdgcn_perm(r2, t0, 0x0c050302u);             // [t0.b2 t0.b3 r2.b1 0]
+    col[2] = __builtin_amdgcn_perm(r2, t1, 0x0c060100u);             // [t1.b0 t1.b1 r2.b2 0]
+    col[3] = __builtin_amdgcn_perm(r2, t1, 0x0c070302u);             // [t1.b2 t1.b3 r2.b3 0]
+}
 
-template <int TX, int SX, bool ZW>
+template <int TX, int TY, int SX, bool ZW>
 __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
-    extern __shared__ __align__(16) char smem[];
-    uint32_t *wcol = reinterpret_cast<uint32_t *>(smem);                // [3][C]: bytes (w[0][kx][c], w[1].., w[2].., 0)
-    DwChan *chan = reinterpret_cast<DwChan *>(smem + (size_t)3 * a.C * 4);  // [C]
-    for (int i = threadIdx.x; i < 3 * a.C; i += kBlock) {
-        const int kx = i / a.C, c = i - kx * a.C;
-        const uint32_t b0 = (uint8_t)a.w[(0 * 3 + kx) * a.C + c], b1 = (uint8_t)a.w[(1 * 3 + kx) * a.C + c],
-                       b2 = (uint8_t)a.w[(2 * 3 + kx) * a.C + c];
-        wcol[i] = b0 | (b1 << 8) | (b2 << 16);
-    }
-    for (int c = threadIdx.x; c < a.C; c += kBlock) {
-        int32_t wsum = 0;
-        for (int t = 0; t < 9; t++) wsum += a.w[t * a.C + c];
-        DwChan d{};
-        const int32_t bias = a.bias[a.bias_len == 1 ? 0 : c];
-        d.bias_adj = (int32_t)((uint32_t)bias - (uint32_t)a.zi * (uint32_t)wsum + 9u * (uint32_t)a.zi * (uint32_t)a.zw);
-        if (a.fused) {
-            const int ci = a.scale.p.per_channel ? c : 0;
-            d.q = make_chan_scale(load_mult(a.scale, ci), (int32_t)a.scale.shift[ci], a.scale.p);
-        }
-        chan[c] = d;
-    }
-    __syncthreads();
-
-    const int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    // blocks are dealt round-robin to the XCDs: give XCD k the k-th contiguous run of blocks
+    const int bid = (int)(blockIdx.x % 8u) * a.chunk + (int)(blockIdx.x / 8u);
+    if (bid >= a.blocks) return;
+    const int64_t item = (int64_t)bid * kBlock + threadIdx.x;
     if (item >= a.items) return;
     const int c4n = a.C >> 2;
     const int c4 = (int)(item % c4n);
     int64_t rest = item / c4n;
     const int strip = (int)(rest % a.strips);
     rest /= a.strips;
-    const int oy = (int)(rest % a.OH);
-    const int n = (int)(rest / a.OH);
+    const int rg = (int)(rest % a.row_groups);
+    const int n = (int)(rest / a.row_groups);
     const int c = c4 * 4;
-    const int ox0 = strip * TX;
+    const int ox0 = strip * TX, oy0 = rg * TY;
 
-    // ---- input columns ix0 .. ix0 + NCOL - 1, three rows each, transposed to one dword per channel
+    // ---- this thread's constants: weight columns, bias with the zero-point terms folded in, scales
+    uint32_t wc[3][4];
+    int32_t wsum[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int kx = 0; kx < 3; kx++) {
+        const uint32_t w0 = *reinterpret_cast<const uint32_t *>(a.w + (0 * 3 + kx) * a.C + c);
+        const uint32_t w1 = *reinterpret_cast<const uint32_t *>(a.w + (1 * 3 + kx) * a.C + c);
+        const uint32_t w2 = *reinterpret_cast<const uint32_t *>(a.w + (2 * 3 + kx) * a.C + c);
+        transpose_3x4(w0, w1, w2, wc[kx]);
+#pragma unroll
+        for (int e = 0; e < 4; e++) wsum[e] = __builtin_amdgcn_sdot4((int)wc[kx][e], 0x00010101, wsum[e], false);
+    }
+    int32_t bias_adj[4];
+    ChanScale q[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int32_t bias = a.bias[a.bias_len == 1 ? 0 : c + e];
+        bias_adj[e] = (int32_t)((uint32_t)bias - (uint32_t)a.zi * (uint32_t)wsum[e] +
+                                9u * (uint32_t)a.zi * (uint32_t)a.zw);
+        if (a.fused) {
+            const int ci = a.scale.p.per_channel ? c + e : 0;
+            q[e] = make_chan_scale(load_mult(a.scale, ci), (int32_t)a.scale.shift[ci], a.scale.p);
+        }
+    }
+
+    // ---- input columns ix0 .. ix0 + NCOL - 1 of rows iy0 .. iy0 + NROW - 1
     constexpr int NCOL = SX * (TX - 1) + 3;
-    const int iy0 = oy * a.sy - a.pad_t, ix0 = ox0 * SX - a.pad_l;
+    constexpr int sy = SX;  // the host only sends equal strides here
+    const int iy0 = oy0 * sy - a.pad_t, ix0 = ox0 * SX - a.pad_l;
     const uint32_t zsplat = (uint32_t)(uint8_t)a.zi * 0x01010101u;
     const int8_t *xb = a.x + (int64_t)n * a.x_sn + c;
-    uint32_t raw[3][NCOL];
+    int32_t acc[TY][TX][4], xs[TY][TX][4];
 #pragma unroll
-    for (int r = 0; r < 3; r++) {
+    for (int ty = 0; ty < TY; ty++)
+#pragma unroll
+        for (int t = 0; t < TX; t++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[ty][t][e] = xs[ty][t][e] = 0;
+
+    constexpr int NROW_MAX = SX * (TY - 1) + 3;
+    uint32_t raw[NROW_MAX][NCOL];
+#pragma unroll
+    for (int r = 0; r < NROW_MAX; r++) {
         const int y = iy0 + r;
         const bool yin = (unsigned)y < (unsigned)a.H;
 #pragma unroll
@@ -197,71 +220,54 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
             raw[r][j] = v;
         }
     }
-    uint32_t wc[3][4];
 #pragma unroll
-    for (int kx = 0; kx < 3; kx++) {
-        const uint4 t = *reinterpret_cast<const uint4 *>(wcol + kx * a.C + c);
-        wc[kx][0] = t.x;
-        wc[kx][1] = t.y;
-        wc[kx][2] = t.z;
-        wc[kx][3] = t.w;
-    }
-    int32_t acc[TX][4], xs[TX][4];
+    for (int ty = 0; ty < TY; ty++) {
 #pragma unroll
-    for (int t = 0; t < TX; t++)
+        for (int j = 0; j < NCOL; j++) {
+            uint32_t col[4];
+            transpose_3x4(raw[ty * SX][j], raw[ty * SX + 1][j], raw[ty * SX + 2][j], col);
 #pragma unroll
-        for (int e = 0; e < 4; e++) acc[t][e] = xs[t][e] = 0;
+            for (int t = 0; t < TX; t++) {
+                const int kx = j - t * SX;  // this column is tap kx of output t (compile-time after unrolling)
+                if (kx < 0 || kx > 2) continue;
 #pragma unroll
-    for (int j = 0; j < NCOL; j++) {
-        // 3 rows x 4 channels (bytes) -> 4 channels x (3 taps, 0): selector bytes 0-3 pick from the 2nd operand
-        const uint32_t r0 = raw[0][j], r1 = raw[1][j], r2 = raw[2][j];
-        const uint32_t t0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);  // [r0.b0 r1.b0 r0.b1 r1.b1]
-        const uint32_t t1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);  // [r0.b2 r1.b2 r0.b3 r1.b3]
-        uint32_t col[4];
-        col[0] = __builtin_amdgcn_perm(r2, t0, 0x0c040100u);  // [t0.b0 t0.b1 r2.b0 0]
-        col[1] = __builtin_amdgcn_perm(r2, t0, 0x0c050302u);  // [t0.b2 t0.b3 r2.b1 0]
-        col[2] = __builtin_amdgcn_perm(r2, t1, 0x0c060100u);  // [t1.b0 t1.b1 r2.b2 0]
-        col[3] = __builtin_amdgcn_perm(r2, t1, 0x0c070302u);  // [t1.b2 t1.b3 r2.b3 0]
-#pragma unroll
-        for (int t = 0; t < TX; t++) {
-            const int kx = j - t * SX;  // this column is tap kx of output t (compile-time after unrolling)
-            if (kx < 0 || kx > 2) continue;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const uint32_t w = wc[kx][e];
-                acc[t][e] = __builtin_amdgcn_sdot4((int)col[e], (int)w, acc[t][e], false);
-                if (ZW) xs[t][e] = __builtin_amdgcn_sdot4((int)col[e], 0x00010101, xs[t][e], false);
+                for (int e = 0; e < 4; e++) {
+                    acc[ty][t][e] = __builtin_amdgcn_sdot4((int)col[e], (int)wc[kx][e], acc[ty][t][e], false);
+                    if (ZW) xs[ty][t][e] = __builtin_amdgcn_sdot4((int)col[e], 0x00010101, xs[ty][t][e], false);
+                }
             }
         }
     }
 
     // ---- epilogue
-    DwChan ch[4];
 #pragma unroll
-    for (int e = 0; e < 4; e++) ch[e] = chan[c + e];
-    const int64_t orow = ((int64_t)n * a.OH + oy) * a.OW;
+    for (int ty = 0; ty < TY; ty++) {
+        const int oy = oy0 + ty;
+        if (oy >= a.OH) break;
+        const int64_t orow = ((int64_t)n * a.OH + oy) * a.OW;
 #pragma unroll
-    for (int t = 0; t < TX; t++) {
-        const int ox = ox0 + t;
-        if (ox >= a.OW) break;
-        int32_t v[4];
+        for (int t = 0; t < TX; t++) {
+            const int ox = ox0 + t;
+            if (ox >= a.OW) break;
+            int32_t v[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            int32_t s = (int32_t)((uint32_t)acc[t][e] + (uint32_t)ch[e].bias_adj);
-            if (ZW) s = (int32_t)((uint32_t)s - (uint32_t)a.zw * (uint32_t)xs[t][e]);
-            if (a.fused) s = requant_chan(s, ch[e].q, a.scale.p);
-            v[e] = s;
-        }
-        const int64_t off = (orow + ox) * a.C + c;
-        if (a.out_size == 1) {
-            *reinterpret_cast<uint32_t *>(a.out + off) = (uint32_t)(uint8_t)v[0] | ((uint32_t)(uint8_t)v[1] << 8) |
-                                                         ((uint32_t)(uint8_t)v[2] << 16) | ((uint32_t)(uint8_t)v[3] << 24);
-        } else if (a.out_size == 2) {
-            *reinterpret_cast<uint2 *>(a.out + off * 2) =
-                make_uint2((uint32_t)(uint16_t)v[0] | ((uint32_t)(uint16_t)v[1] << 16),
-                           (uint32_t)(uint16_t)v[2] | ((uint32_t)(uint16_t)v[3] << 16));
-        } else {
-            *reinterpret_cast<int4 *>(a.out + off * 4) = make_int4(v[0], v[1], v[2], v[3]);
+            for (int e = 0; e < 4; e++) {
+                int32_t s = (int32_t)((uint32_t)acc[ty][t][e] + (uint32_t)bias_adj[e]);
+                if (ZW) s = (int32_t)((uint32_t)s - (uint32_t)a.zw * (uint32_t)xs[ty][t][e]);
+                if (a.fused) s = requant_chan(s, q[e], a.scale.p);
+                v[e] = s;
+            }
+            const int64_t off = (orow + ox) * a.C + c;
+            if (a.out_size == 1) {
+                *reinterpret_cast<uint32_t *>(a.out + off) = ((uint32_t)v[0] & 0xffu) | (((uint32_t)v[1] & 0xffu) << 8) |
+                                                             (((uint32_t)v[2] & 0xffu) << 16) | ((uint32_t)v[3] << 24);
+            } else if (a.out_size == 2) {
+                *reinterpret_cast<uint2 *>(a.out + off * 2) =
+                    make_uint2((uint32_t)(uint16_t)v[0] | ((uint32_t)(uint16_t)v[1] << 16),
+                               (uint32_t)(uint16_t)v[2] | ((uint32_t)(uint16_t)v[3] << 16));
+            } else {
+                *reinterpret_cast<int4 *>(a.out + off * 4) = make_int4(v[0], v[1], v[2], v[3]);
+            }
         }
     }
 }
@@ -281,7 +287,9 @@ int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     if (w->dims[0] != 3 || w->dims[1] != 3 || w->dims[3] != 1 || w->dims[2] != C || in->dims[3] != C) return 0;
     if (a->dilation[0] != 1 || a->dilation[1] != 1) return 0;
     if (a->stride[0] < 1 || a->stride[0] > 2 || a->stride[1] < 1 || a->stride[1] > 2) return 0;
-    if (C % 4 != 0 || C <= 0 || C > 2048 || in->dims[0] < N) return 0;
+    if (C % 4 != 0 || C <= 0 || C >= (1 << 24) || in->dims[0] < N) return 0;
+    if (a->stride[0] != a->stride[1]) return 0;
+    if (((uintptr_t)w->ptr % 4) != 0 || ((uintptr_t)bias->ptr % 4) != 0) return 0;
     if (!is_packed(w) || !is_packed(out) || in->strides[3] != 1) return 0;
     if (!(bias->dims[0] == 1 || bias->dims[0] >= C) || bias->strides[0] != 4) return 0;
     if (((uintptr_t)in->ptr % 4) || in->strides[0] % 4 || in->strides[1] % 4 || in->strides[2] % 4) return 0;
@@ -290,6 +298,7 @@ int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     if (in->dims[1] >= (1 << 30) || in->dims[2] >= (1 << 30) || OH >= (1 << 30) || OW >= (1 << 30)) return 0;
 
     constexpr int TX = 4;
+    const int TY = OH >= 2 ? 2 : 1;
     DwArgs g{};
     g.x = static_cast<const int8_t *>(in->ptr);
     g.w = static_cast<const int8_t *>(w->ptr);
@@ -315,19 +324,24 @@ int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     g.out_size = dt_size(out->dtype);
     if (epi) g.scale = make_ref(*epi);
     g.strips = (int)((OW + TX - 1) / TX);
-    g.items = N * OH * g.strips * (C / 4);
-    const size_t smem = (size_t)3 * C * 4 + (size_t)C * sizeof(DwChan);
+    g.row_groups = (int)((OH + TY - 1) / TY);
+    g.items = N * g.row_groups * g.strips * (C / 4);
     const int64_t blocks = (g.items + kBlock - 1) / kBlock;
-    MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "depthwise_conv2d: too many work items");
-    const dim3 grid((unsigned)blocks), block(kBlock);
-    if (g.sx == 1 && g.zw == 0)
-        dwconv3x3_i8_kernel<TX, 1, false><<<grid, block, smem, s>>>(g);
-    else if (g.sx == 1)
-        dwconv3x3_i8_kernel<TX, 1, true><<<grid, block, smem, s>>>(g);
-    else if (g.zw == 0)
-        dwconv3x3_i8_kernel<TX, 2, false><<<grid, block, smem, s>>>(g);
-    else
-        dwconv3x3_i8_kernel<TX, 2, true><<<grid, block, smem, s>>>(g);
+    MLEL_REQUIRE(blocks < (int64_t(1) << 30), MLEL_ERR_LIMIT, "depthwise_conv2d: too many work items");
+    g.blocks = (int)blocks;
+    g.chunk = (int)((blocks + 7) / 8);
+    const dim3 grid((unsigned)(g.chunk * 8)), block(kBlock);
+    const int variant = (TY == 2 ? 4 : 0) + (g.sx == 2 ? 2 : 0) + (g.zw != 0 ? 1 : 0);
+    switch (variant) {
+    case 0: dwconv3x3_i8_kernel<TX, 1, 1, false><<<grid, block, 0, s>>>(g); break;
+    case 1: dwconv3x3_i8_kernel<TX, 1, 1, true><<<grid, block, 0, s>>>(g); break;
+    case 2: dwconv3x3_i8_kernel<TX, 1, 2, false><<<grid, block, 0, s>>>(g); break;
+    case 3: dwconv3x3_i8_kernel<TX, 1, 2, true><<<grid, block, 0, s>>>(g); break;
+    case 4: dwconv3x3_i8_kernel<TX, 2, 1, false><<<grid, block, 0, s>>>(g); break;
+    case 5: dwconv3x3_i8_kernel<TX, 2, 1, true><<<grid, block, 0, s>>>(g); break;
+    case 6: dwconv3x3_i8_kernel<TX, 2, 2, false><<<grid, block, 0, s>>>(g); break;
+    default: dwconv3x3_i8_kernel<TX, 2, 2, true><<<grid, block, 0, s>>>(g); break;
+    }
     MLEL_TRY(check_launch("depthwise_conv2d 3x3 int8"));
     return 1;
 }
@@ -342,8 +356,150 @@ int try_clamp_fast(mlel_ctx *, hipStream_t, const mlel_tensor *, const mlel_tens
 int try_binary_fast(mlel_ctx *, hipStream_t, int, const mlel_tensor *, const mlel_tensor *, const mlel_tensor *) {
     return 0;
 }
-int try_avgpool_fast(mlel_ctx *, hipStream_t, const mlel_tensor *, const mlel_tensor *, const mlel_pool2d_attr *) {
-    return 0;
+namespace {
+
+// ---------------------------------------------------------------------------------------------------------------
+// AVG_POOL2D, int8 NHWC, int32 accumulator.  Work item = 4 consecutive channels of one output position; lanes run
+// over the channel quads, so a wavefront reads consecutive dwords of each input pixel.  The bytes of a dword are
+// widened and accumulated with v_dot4_i32_i8 against a one-hot byte vector.  Arithmetic as avgpool2d.comp:27-75:
+// sum of (x - input_zp) over the in-bounds taps, divided by their count with rounding half away from zero,
+// output zero point added, clamped to the output type.
+// ---------------------------------------------------------------------------------------------------------------
+struct AvgArgs {
+    const int8_t *x;
+    int8_t *out;
+    int32_t H, W, C, OH, OW;
+    int64_t x_sn, x_sy, x_sx, o_sn, o_sy, o_sx;
+    int32_t kh, kw, sy, sx, pad_t, pad_l, zi, zo;
+    int64_t items;  // N * OH * OW * C/4
+};
+
+// SPLIT threads share the window of one work item (taps dealt round-robin) and combine through shared memory:
+// used when there are too few outputs to fill the machine and the window is large (global average pooling).
+template <int SPLIT>
+__global__ void __launch_bounds__(kBlock) avgpool_i8x4_kernel(const AvgArgs a) {
+    constexpr int ITEMS = kBlock / SPLIT;
+    __shared__ int32_t partial[SPLIT > 1 ? SPLIT : 1][ITEMS][4];
+    const int slot = threadIdx.x % ITEMS, part = threadIdx.x / ITEMS;
+    const int64_t item = (int64_t)blockIdx.x * ITEMS + slot;
+    const bool live = item < a.items;
+    const int c4n = a.C >> 2;
+    const int c = live ? (int)(item % c4n) * 4 : 0;
+    int64_t rest = live ? item / c4n : 0;
+    const int ox = (int)(rest % a.OW);
+    rest /= a.OW;
+    const int oy = (int)(rest % a.OH);
+    const int n = (int)(rest / a.OH);
+    const int y0 = max(0, oy * a.sy - a.pad_t), y1 = min(a.H, oy * a.sy - a.pad_t + a.kh);
+    const int x0 = max(0, ox * a.sx - a.pad_l), x1 = min(a.W, ox * a.sx - a.pad_l + a.kw);
+    const int nx = x1 - x0;
+    const int count = (live && y1 > y0 && nx > 0) ? (y1 - y0) * nx : 0;
+    int32_t acc[4] = {0, 0, 0, 0};
+    const int8_t *xb = a.x + (int64_t)n * a.x_sn + c;
+    // taps part, part + SPLIT, ... in batches of four independent loads
+    int ty = y0, tx = x0 + part;
+    for (int t = part; t < count; t += 4 * SPLIT) {
+        int v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            while (tx >= x1) {
+                tx -= nx;
+                ty++;
+            }
+            v[k] = (t + k * SPLIT < count)
+                       ? *reinterpret_cast<const int32_t *>(xb + (int64_t)ty * a.x_sy + (int64_t)tx * a.x_sx)
+                       : 0;
+            tx += SPLIT;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            acc[0] = __builtin_amdgcn_sdot4(v[k], 0x00000001, acc[0], false);
+            acc[1] = __builtin_amdgcn_sdot4(v[k], 0x00000100, acc[1], false);
+            acc[2] = __builtin_amdgcn_sdot4(v[k], 0x00010000, acc[2], false);
+            acc[3] = __builtin_amdgcn_sdot4(v[k], 0x01000000, acc[3], false);
+        }
+    }
+    if (SPLIT > 1) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) partial[part][slot][e] = acc[e];
+        __syncthreads();
+        if (part != 0) return;
+#pragma unroll
+        for (int p = 1; p < SPLIT; p++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[e] += partial[p][slot][e];
+    }
+    if (!live) return;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        int32_t r = 0;
+        if (count > 0) {
+            const int32_t s = (int32_t)((uint32_t)acc[e] - (uint32_t)a.zi * (uint32_t)count);
+            r = (s + (s < 0 ? -(count >> 1) : (count >> 1))) / count;
+        }
+        r = min(max(r + a.zo, -128), 127);
+        packed |= ((uint32_t)r & 0xffu) << (8 * e);
+    }
+    *reinterpret_cast<uint32_t *>(a.out + (int64_t)n * a.o_sn + (int64_t)oy * a.o_sy + (int64_t)ox * a.o_sx + c) = packed;
+}
+
+}  // namespace
+
+int try_avgpool_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                     const mlel_pool2d_attr *attr) {
+    (void)ctx;
+    if (in->dtype != MLEL_I8 || out->dtype != MLEL_I8 || attr->acc_type != MLEL_ACC_I32) return 0;
+    const int64_t N = out->dims[0], OH = out->dims[1], OW = out->dims[2], C = out->dims[3];
+    // the kernel's indexing assumes: channel quads contiguous and dword aligned on both sides, 32-bit coordinates,
+    // a window small enough that the rounded sum stays inside int32
+    if (C % 4 != 0 || in->dims[3] != C || in->dims[0] < N) return 0;
+    if (in->strides[3] != 1 || out->strides[3] != 1) return 0;
+    for (int i = 0; i < 3; i++)
+        if (in->strides[i] % 4 != 0 || out->strides[i] % 4 != 0) return 0;
+    if (((uintptr_t)in->ptr % 4) != 0 || ((uintptr_t)out->ptr % 4) != 0) return 0;
+    if (attr->kernel[0] < 1 || attr->kernel[1] < 1 || (int64_t)attr->kernel[0] * attr->kernel[1] > 65536) return 0;
+    if (attr->stride[0] < 1 || attr->stride[1] < 1) return 0;
+    if (attr->input_zp < -128 || attr->input_zp > 127 || attr->output_zp < -128 || attr->output_zp > 127) return 0;
+    const int64_t lim = int64_t(1) << 24;
+    if (in->dims[1] >= lim || in->dims[2] >= lim || OH >= lim || OW >= lim || C >= lim) return 0;
+    if ((int64_t)attr->stride[0] >= lim || (int64_t)attr->stride[1] >= lim || (int64_t)attr->pad[0] >= lim ||
+        (int64_t)attr->pad[2] >= lim || attr->pad[0] < 0 || attr->pad[2] < 0)
+        return 0;
+    if (N <= 0 || OH <= 0 || OW <= 0 || C <= 0) return 1;
+    AvgArgs g{};
+    g.x = static_cast<const int8_t *>(in->ptr);
+    g.out = static_cast<int8_t *>(out->ptr);
+    g.H = (int)in->dims[1];
+    g.W = (int)in->dims[2];
+    g.C = (int)C;
+    g.OH = (int)OH;
+    g.OW = (int)OW;
+    g.x_sn = in->strides[0];
+    g.x_sy = in->strides[1];
+    g.x_sx = in->strides[2];
+    g.o_sn = out->strides[0];
+    g.o_sy = out->strides[1];
+    g.o_sx = out->strides[2];
+    g.kh = attr->kernel[0];
+    g.kw = attr->kernel[1];
+    g.sy = attr->stride[0];
+    g.sx = attr->stride[1];
+    g.pad_t = attr->pad[0];
+    g.pad_l = attr->pad[2];
+    g.zi = attr->input_zp;
+    g.zo = attr->output_zp;
+    g.items = N * OH * OW * (C / 4);
+    const bool split = g.items < 256 * 1024 && (int64_t)g.kh * g.kw >= 16;
+    const int per_block = split ? kBlock / 8 : kBlock;
+    const int64_t blocks = (g.items + per_block - 1) / per_block;
+    MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "avg_pool2d: too many work items");
+    if (split)
+        avgpool_i8x4_kernel<8><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(g);
+    else
+        avgpool_i8x4_kernel<1><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(g);
+    MLEL_TRY(check_launch("avg_pool2d int8"));
+    return 1;
 }
 
 }  // namespace mlel

@@ -134,6 +134,9 @@ CONV_CASES = [
     ("ic20_oc130", (1, 6, 6, 20), 130, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 1, 0),
     ("k_tail_ic48", (1, 5, 5, 48), 64, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 0, 0),
     ("pw_960_320", (1, 7, 7, 960), 320, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -1, 0),
+    ("pw_24_both_zp", (2, 9, 9, 24), 40, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 5, -3),
+    ("pw_36_k_tail_dwords", (1, 5, 7, 36), 20, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -2, 0),
+    ("pw_72_two_k_steps", (3, 8, 8, 72), 24, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 9, 1),
 ]
 
 
@@ -239,6 +242,11 @@ DW_CASES = [
     ("mult2_zw", (1, 7, 8, 5), 2, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), 3, -2),
     ("k5_dil", (1, 11, 11, 8), 1, (5, 5), (2, 2, 2, 2), (1, 1), (1, 1), 0, 0),
     ("c960", (1, 7, 7, 960), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -1, 0),
+    ("odd_rows_zw", (2, 9, 10, 12), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), 8, 3),
+    ("single_row_out", (1, 3, 13, 8), 1, (3, 3), (0, 0, 1, 1), (1, 1), (1, 1), -9, 0),
+    ("stride2_odd", (2, 15, 13, 20), 1, (3, 3), (1, 1, 1, 1), (2, 2), (1, 1), 2, -1),
+    ("stride_2x1", (1, 9, 9, 8), 1, (3, 3), (1, 1, 1, 1), (2, 1), (1, 1), 1, 0),
+    ("c2052", (1, 4, 5, 2052), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -3, 0),
 ]
 
 
@@ -344,6 +352,17 @@ def test_pool_reduce_cast_negate_vs_oracle(run, oracle):
     a2 = abi.pool2d_attr((3, 3), (2, 2), (1, 1, 1, 1), input_zp=4, output_zp=-1)
     np.testing.assert_array_equal(run.pool("avg_pool2d", x, (2, 4, 4, 40), a2), oracle.avg_pool2d(x, (2, 4, 4, 40), a2))
     np.testing.assert_array_equal(run.pool("max_pool2d", x, (2, 4, 4, 40), a2), oracle.max_pool2d(x, (2, 4, 4, 40), a2))
+    # channel counts off the dword fast path, rectangular windows, extreme values against the zero point
+    x5 = ri(rng, -128, 127, (1, 6, 5, 5), np.int8)
+    a3 = abi.pool2d_attr((2, 3), (1, 2), (1, 0, 0, 2), input_zp=100, output_zp=-100)
+    np.testing.assert_array_equal(run.pool("avg_pool2d", x5, (1, 6, 3, 5), a3), oracle.avg_pool2d(x5, (1, 6, 3, 5), a3))
+    lo = np.full((3, 9, 11, 64), -128, np.int8)
+    lo[:, ::2] = 127
+    a4 = abi.pool2d_attr((3, 2), (2, 1), (1, 0, 1, 0), input_zp=127, output_zp=127)
+    np.testing.assert_array_equal(run.pool("avg_pool2d", lo, (3, 4, 11, 64), a4), oracle.avg_pool2d(lo, (3, 4, 11, 64), a4))
+    g = ri(rng, -128, 127, (4, 7, 7, 1280), np.int8)
+    a5 = abi.pool2d_attr((7, 7), (1, 1), (0, 0, 0, 0), input_zp=-100, output_zp=-100)
+    np.testing.assert_array_equal(run.pool("avg_pool2d", g, (4, 1, 1, 1280), a5), oracle.avg_pool2d(g, (4, 1, 1, 1280), a5))
     r = ri(rng, -1000, 1000, (3, 4, 50), np.int32)
     for op in ("SUM", "MAX", "MIN", "PRODUCT"):
         for axis in range(3):
