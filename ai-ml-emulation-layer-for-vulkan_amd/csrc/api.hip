@@ -93,7 +93,8 @@ int mlel_hip_conv2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const m
                     const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv2d_attr *attr) {
     MLEL_TRY(require_ctx(ctx, "conv2d"));
     MLEL_TRY(check_conv("conv2d", out, in, weights, bias, attr));
-    const int rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, out, in, weights, bias, attr, nullptr);
+    int rc = try_conv2d_i8_direct(ctx, (hipStream_t)stream, out, in, weights, bias, attr, nullptr);
+    if (rc == 0) rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, out, in, weights, bias, attr, nullptr);
     if (rc != 0) return rc < 0 ? rc : 0;
     return conv2d_generic_launch((hipStream_t)stream, out, in, weights, bias, attr);
 }
@@ -325,7 +326,8 @@ int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor
     MLEL_TRY(check_conv("conv2d_rescale_clamp", &acc_view, in, weights, bias, attr));
     FusedEpilogue fe;
     MLEL_TRY(make_epilogue(epi, MLEL_I32, out, out->dims[3], &fe));
-    const int rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe);
+    int rc = try_conv2d_i8_direct(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe);
+    if (rc == 0) rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe);
     if (rc != 0) return rc < 0 ? rc : 0;
     // no specialised kernel for this layout: run the unfused operator sequence through an int32 scratch tensor
     Scratch scratch;

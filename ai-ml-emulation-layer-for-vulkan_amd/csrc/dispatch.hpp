@@ -46,9 +46,33 @@ struct FusedEpilogue {
     bool scale32;
     int in_dt;  // input storage type viewed through input_unsigned
 };
+// The same, as a kernel argument: raw pointers to the multiplier (int32 or int16) and shift (int8) arrays.
+struct ScaleRef {
+    const char *mult;
+    const int8_t *shift;
+    int32_t mult16;
+    RescaleParams p;
+};
+inline ScaleRef make_ref(const FusedEpilogue &f) {
+    ScaleRef r;
+    r.mult = static_cast<const char *>(f.mult->ptr);
+    r.shift = static_cast<const int8_t *>(f.shift->ptr);
+    r.mult16 = f.scale32 ? 0 : 1;
+    r.p = f.p;
+    return r;
+}
+__device__ __forceinline__ int32_t load_mult(const ScaleRef &s, int64_t c) {
+    return s.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(s.mult)[c]
+                    : reinterpret_cast<const int32_t *>(s.mult)[c];
+}
+
 int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                        const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
                        const FusedEpilogue *epi);
+// ---- direct (dot4) convolution for very small input channel counts (conv_direct.hip) ----
+int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                         const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
+                         const FusedEpilogue *epi);
 int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
                        const mlel_tensor *b, const mlel_matmul_attr *attr, const FusedEpilogue *epi);
 

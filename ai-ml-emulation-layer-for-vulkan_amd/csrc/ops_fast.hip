@@ -9,27 +9,6 @@ namespace {
 
 constexpr int kBlock = 256;
 
-struct ScaleRef {
-    const char *mult;
-    const int8_t *shift;
-    int32_t mult16;
-    RescaleParams p;
-};
-
-ScaleRef make_ref(const FusedEpilogue &f) {
-    ScaleRef r;
-    r.mult = static_cast<const char *>(f.mult->ptr);
-    r.shift = static_cast<const int8_t *>(f.shift->ptr);
-    r.mult16 = f.scale32 ? 0 : 1;
-    r.p = f.p;
-    return r;
-}
-
-__device__ __forceinline__ int32_t load_mult(const ScaleRef &s, int64_t c) {
-    return s.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(s.mult)[c]
-                    : reinterpret_cast<const int32_t *>(s.mult)[c];
-}
-
 // out = RESCALE_o(RESCALE_1(in1) + RESCALE_2(in2)), any integer storage types, any strides
 __global__ void __launch_bounds__(kBlock) rescale_add_rescale_kernel(TV out, TV in1, TV in2, ScaleRef s1, ScaleRef s2,
                                                                      ScaleRef so, int in1_dt, int in2_dt,
