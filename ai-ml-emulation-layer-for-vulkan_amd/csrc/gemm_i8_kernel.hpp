@@ -1,0 +1,707 @@
+// int8 x int8 -> int32 contractions on the gfx950 matrix cores: CONV2D (implicit GEMM over NHWC input and OHWI
+// weights) and MATMUL, with the zero-point handling of the reference shaders and an optional fused
+// RESCALE(+CLAMP) epilogue.
+//
+// What is computed.  out[m][n] = sum_k (X[m][k] - zx) * (Wt[n][k] - zw) + bias[n], where
+//   CONV2D : m = (image, oy, ox), n = oc, k = (ky, kx, ic); X[m][k] is the input element under tap (ky,kx) or, for
+//            a tap that falls into the padding, the value zx itself so that the tap contributes nothing
+//            (the reference skips such taps: conv2d.comp:64);
+//   MATMUL : per batch, X = A[m][k], Wt[n][k] = B[k][n] (B is stored K-major and transposed while it is staged
+//            into LDS) (reference: matmul.comp:30-73).
+// The sum is expanded as  sum X*Wt - zw*sum_k X - zx*sum_k Wt + K*zx*zw  so that the matrix cores multiply the raw
+// int8 operands (X - zx does not fit in int8).  All arithmetic is int32 with wraparound, as in the shaders, so the
+// regrouping is exact.
+//
+// Kernel shape.  256 threads = 4 wavefronts of 64.  A block owns a BM x BN output tile; K is walked in steps of
+// 64 bytes through two LDS buffers (global loads of step i+1 are in flight while step i is multiplied).  Each
+// wavefront owns a (32*TM) x (32*TN) sub-tile and issues v_mfma_i32_32x32x32_i8 with the weights as the row
+// operand and the activations as the column operand: a lane then holds, for ONE output position m, groups of four
+// consecutive output channels n, which is the byte order of the NHWC / [M][N] output, so requantised results are
+// packed four to a dword and stored without a transpose.  Per-channel epilogue constants live in LDS.
+#pragma once
+
+#include "common.hpp"
+#include "dispatch.hpp"
+
+namespace mlel {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) v2i lds_v2i;
+
+constexpr int BK = 64;            // bytes of K per step
+constexpr int PITCH = BK + 16;    // LDS row pitch: 80 B keeps 16-lane groups of 128-bit reads on distinct banks
+constexpr int NTHREADS = 256;
+
+struct GemmArgs {
+    // problem
+    int32_t M, N, K, batches;
+    // X operand (rows m): conv gather over NHWC; the plain [M][K] case is the 1x1 conv with H = W = 1
+    const int8_t *x;
+    int64_t x_batch, x_sn, x_sy, x_sx;  // byte strides
+    int32_t H, W, IC, OHW, OW, KH, KW, sy, sx, dy, dx, pad_t, pad_l;
+    int32_t plain;  // 1: m indexes rows of pitch x_sx directly
+    int32_t xch;    // bytes per aligned global load of X: 16, 4 or 1
+    uint32_t x_bytes, w_bytes;  // per-batch extent of each operand (buffer-load bounds of the fast fetch modes)
+    // W operand (rows n)
+    const int8_t *w;
+    int64_t w_batch, ldw;
+    int32_t w_kmajor;  // 0: [N][K] rows of pitch ldw; 1: [K][N] rows of pitch ldw
+    int32_t wch;       // bytes per aligned global load of W: 16, 4 or 1
+    int32_t zx, zw;
+    // bias (int32, length 1 or N) and output
+    const int32_t *bias;
+    int32_t bias_len;
+    char *out;
+    int64_t out_batch, ldo;  // ldo in elements
+    int32_t out_size;        // bytes per output element: 1, 2 or 4
+    int32_t out_vec_ok;      // four consecutive channels may be stored as one aligned unit
+    uint32_t o_bytes;        // per-batch extent of the output when it fits 31-bit buffer offsets, else 0
+    // fused epilogue
+    int32_t fused;
+    const char *mult;  // int32 or int16 per channel (or one)
+    const int8_t *shift;
+    int32_t mult16;
+    RescaleParams rp;
+    // launch geometry
+    int32_t tiles_m, tiles_n, total_tiles, chunk;
+};
+
+struct ChanParams {  // per output channel, in LDS: 32 bytes = two 128-bit reads
+    ChanScale q;
+    int32_t bias_adj;
+    int32_t pad[1];
+};
+static_assert(sizeof(ChanParams) == 32, "ChanParams layout");
+
+struct RowState {
+    const int8_t *base;
+    int32_t iy0, ix0;
+    int32_t valid;
+};
+
+struct KState {
+    int32_t ky, kx, ic;
+};
+
+__device__ __forceinline__ void kstate_advance(KState &s, int step, int IC, int KW) {
+    s.ic += step;
+    while (s.ic >= IC) {
+        s.ic -= IC;
+        if (++s.kx == KW) {
+            s.kx = 0;
+            ++s.ky;
+        }
+    }
+}
+
+__device__ __forceinline__ uint32_t splat8(int v) { return (uint32_t)(uint8_t)v * 0x01010101u; }
+
+// One 16-byte piece of row `r` of the X operand starting at k-position `s`.
+__device__ __forceinline__ uint4 load_x_chunk(const GemmArgs &g, const RowState &r, KState s) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (!r.valid) return v;
+    if (g.xch == 16) {
+        if (s.ky >= g.KH) return v;
+        const int y = r.iy0 + s.ky * g.dy, x = r.ix0 + s.kx * g.dx;
+        if ((unsigned)y >= (unsigned)g.H || (unsigned)x >= (unsigned)g.W) {
+            const uint32_t z = splat8(g.zx);
+            return make_uint4(z, z, z, z);
+        }
+        return *reinterpret_cast<const uint4 *>(r.base + (int64_t)y * g.x_sy + (int64_t)x * g.x_sx + s.ic);
+    }
+    uint32_t d[4];
+    if (g.xch == 4) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t val = 0;
+            if (s.ky < g.KH) {
+                const int y = r.iy0 + s.ky * g.dy, x = r.ix0 + s.kx * g.dx;
+                if ((unsigned)y >= (unsigned)g.H || (unsigned)x >= (unsigned)g.W)
+                    val = splat8(g.zx);
+                else
+                    val = *reinterpret_cast<const uint32_t *>(r.base + (int64_t)y * g.x_sy + (int64_t)x * g.x_sx +
+                                                              s.ic);
+            }
+            d[j] = val;
+            kstate_advance(s, 4, g.IC, g.KW);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t val = 0;
+            for (int b = 0; b < 4; b++) {
+                uint32_t byte = 0;
+                if (s.ky < g.KH) {
+                    const int y = r.iy0 + s.ky * g.dy, x = r.ix0 + s.kx * g.dx;
+                    if ((unsigned)y >= (unsigned)g.H || (unsigned)x >= (unsigned)g.W)
+                        byte = (uint8_t)g.zx;
+                    else
+                        byte = (uint8_t)r.base[(int64_t)y * g.x_sy + (int64_t)x * g.x_sx + s.ic];
+                }
+                val |= byte << (8 * b);
+                kstate_advance(s, 1, g.IC, g.KW);
+            }
+            d[j] = val;
+        }
+    }
+    return make_uint4(d[0], d[1], d[2], d[3]);
+}
+
+// One 16-byte piece of row n of the W operand stored as [N][K].
+__device__ __forceinline__ uint4 load_w_chunk(const GemmArgs &g, const int8_t *wb, int n, int k) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (n >= g.N || k >= g.K) return v;
+    const int8_t *p = wb + (int64_t)n * g.ldw + k;
+    if (g.wch == 16) return *reinterpret_cast<const uint4 *>(p);
+    uint32_t d[4];
+    if (g.wch == 4) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) d[j] = (k + 4 * j < g.K) ? *reinterpret_cast<const uint32_t *>(p + 4 * j) : 0u;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t val = 0;
+            for (int b = 0; b < 4; b++)
+                if (k + 4 * j + b < g.K) val |= (uint32_t)(uint8_t)p[4 * j + b] << (8 * b);
+            d[j] = val;
+        }
+    }
+    return make_uint4(d[0], d[1], d[2], d[3]);
+}
+
+// A 4(k) x 4(n) byte block of the K-major W operand, returned transposed: d[j] = the four k-bytes of column n+j.
+__device__ __forceinline__ uint4 load_w_block_kmajor(const GemmArgs &g, const int8_t *wb, int n, int k) {
+    uint32_t r[4] = {0, 0, 0, 0};
+    if (n < g.N) {
+        if (g.wch >= 4) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (k + i < g.K) r[i] = *reinterpret_cast<const uint32_t *>(wb + (int64_t)(k + i) * g.ldw + n);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (k + i < g.K)
+                    for (int b = 0; b < 4; b++)
+                        if (n + b < g.N) r[i] |= (uint32_t)(uint8_t)wb[(int64_t)(k + i) * g.ldw + n + b] << (8 * b);
+        }
+    }
+    // 4x4 byte transpose with v_perm_b32 (selector bytes 0-3 pick from the second source, 4-7 from the first)
+    const uint32_t t0 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u);
+    const uint32_t t1 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);
+    const uint32_t t2 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+    return make_uint4(__builtin_amdgcn_perm(t2, t0, 0x05040100u), __builtin_amdgcn_perm(t2, t0, 0x07060302u),
+                      __builtin_amdgcn_perm(t3, t1, 0x05040100u), __builtin_amdgcn_perm(t3, t1, 0x07060302u));
+}
+
+// Buffer-addressed loads: 32-bit offsets, and an offset at or beyond the extent of the resource returns 0
+// without touching memory, which removes every bounds branch from the fast fetch modes.
+constexpr uint32_t kOobOffset = 0x80000000u;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+    const v4i v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+    return make_uint4((uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w);
+}
+__device__ __forceinline__ uint32_t buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+    return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0);
+}
+
+template <int BN>
+constexpr int w_buf_bytes() {
+    return BN * PITCH > BK * (BN + 16) ? BN * PITCH : BK * (BN + 16);
+}
+
+// How the two operands are fetched; fixed at compile time so that the hot loops carry no per-byte logic.
+enum XMode {
+    X_PLAIN = 0,    // X[m][k] = base + m * pitch + k, 16-byte pieces (MATMUL A; 1x1 stride-1 CONV2D on a dense input)
+    X_TAP = 1,      // 16-byte pieces, IC % 64 == 0: one K step lies inside one filter tap (uniform tap state)
+    X_GENERIC = 2,  // anything else: per-piece tap tracking, 16 / 4 / 1-byte loads
+    X_PLAIN4 = 3,   // as X_PLAIN for rows that are only dword aligned (K % 4 == 0): four dword loads per piece
+};
+enum WMode {
+    W_ROWS = 0,     // [N][K], 16-byte pieces
+    W_KMAJOR = 1,   // [K][N] kept K-major in LDS; MFMA operands are gathered with ds_read_b64_tr_b8; 16-byte loads
+    W_GENERIC = 2,  // either layout, any alignment
+    W_KMAJOR4 = 3,  // as W_KMAJOR for rows that are only dword aligned (N % 4 == 0): four dword loads per piece
+    W_ROWS4 = 4,    // as W_ROWS for rows that are only dword aligned (K % 4 == 0)
+};
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int XMODE, int WMODE, bool SUMS, bool Q8>
+__global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wavefront sub-tile
+    constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 MFMA tiles per wavefront
+    constexpr int XROWS = BM / 64;                       // X rows per thread (4 pieces of 16 B per row)
+    constexpr int WCHUNKS = (BN * 4 + NTHREADS - 1) / NTHREADS;
+    static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per block");
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wavefront tile is a multiple of the 32x32 MFMA tile");
+
+    constexpr int PW = BN + 16;           // W_KMAJOR: LDS pitch of one K row of BN channels (bytes)
+    constexpr int WBUF = w_buf_bytes<BN>();  // one W buffer: [BN][PITCH] or [BK][PW], whichever is larger
+    constexpr int N16 = BN / 16;          // 16-byte pieces per K row of the K-major tile
+
+    extern __shared__ __align__(16) char smem[];
+    char *xs = smem;                     // [2][BM][PITCH]
+    char *ws = smem + 2 * BM * PITCH;    // [2][WBUF]
+    ChanParams *cp = reinterpret_cast<ChanParams *>(smem + 2 * BM * PITCH + 2 * WBUF);  // [BN]
+
+    // ---- XCD-aware tile assignment: consecutive block ids land on different XCDs (8 of them, each with its own
+    // L2), so block b is given tile (b % 8) * chunk + b / 8: tiles that share operands stay on one XCD.
+    const int lin = (int)(blockIdx.x % 8) * g.chunk + (int)(blockIdx.x / 8);
+    if (lin >= g.total_tiles) return;
+    const int tiles_per_batch = g.tiles_m * g.tiles_n;
+    // the divisions run on the vector ALU; readfirstlane returns the (wave-uniform) results to scalar registers so
+    // that everything derived from them (base pointers, buffer resources) is scalar as well
+    const int batch = __builtin_amdgcn_readfirstlane(lin / tiles_per_batch);
+    const int t_in = lin - batch * tiles_per_batch;
+    const int tile_m = __builtin_amdgcn_readfirstlane(t_in / g.tiles_n);
+    const int tile_n = t_in - tile_m * g.tiles_n;
+    const int m_base = tile_m * BM, n_base = tile_n * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+
+    const int8_t *xb = g.x + (int64_t)batch * g.x_batch;
+    const int8_t *wb = g.w + (int64_t)batch * g.w_batch;
+
+    // ---- per-channel epilogue constants
+    for (int n = tid; n < BN; n += NTHREADS) {
+        ChanParams c{};
+        const int gn = n_base + n;
+        if (gn < g.N) {
+            c.bias_adj = g.bias ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
+            if (g.fused) {
+                const int ci = g.rp.per_channel ? gn : 0;
+                const int32_t m = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
+                                           : reinterpret_cast<const int32_t *>(g.mult)[ci];
+                c.q = make_chan_scale(m, (int32_t)g.shift[ci], g.rp);
+            }
+        }
+        cp[n] = c;
+    }
+
+    // ---- loader state
+    const int x_kc = tid & 3;  // which 16-byte piece of the 64-byte K step this thread stages
+    RowState rows[XROWS];      // X_GENERIC: pointers; X_TAP: tap origin
+    uint32_t xoff[XROWS];      // fast modes: byte offset of the row (X_PLAIN) / image (X_TAP), or kOobOffset
+#pragma unroll
+    for (int i = 0; i < XROWS; i++) {
+        const int m = m_base + (tid >> 2) + 64 * i;
+        RowState r{xb, 0, 0, m < g.M};
+        xoff[i] = kOobOffset;
+        if (r.valid) {
+            if (g.plain) {
+                r.base = xb + (int64_t)m * g.x_sx;
+                xoff[i] = (uint32_t)m * (uint32_t)g.x_sx + x_kc * 16;
+            } else {
+                const int img = m / g.OHW, rem = m - img * g.OHW;
+                const int oy = rem / g.OW, ox = rem - oy * g.OW;
+                r.base = xb + (int64_t)img * g.x_sn;
+                r.iy0 = oy * g.sy - g.pad_t;
+                r.ix0 = ox * g.sx - g.pad_l;
+                xoff[i] = (uint32_t)img * (uint32_t)g.x_sn + x_kc * 16;
+            }
+        }
+        rows[i] = r;
+    }
+    KState ks{0, 0, 0};                      // X_GENERIC: k position of this thread's piece
+    if (XMODE == X_GENERIC) kstate_advance(ks, x_kc * 16, g.IC, g.KW);
+    int tap_ky = 0, tap_kx = 0, tap_ic = 0;  // X_TAP: uniform position of the K step
+    const __amdgpu_buffer_rsrc_t xres = make_rsrc(xb, g.x_bytes), wres = make_rsrc(wb, g.w_bytes);
+
+    uint32_t woff[WCHUNKS];  // fast modes: byte offset of the piece at k = 0, or kOobOffset
+#pragma unroll
+    for (int i = 0; i < WCHUNKS; i++) {
+        const int c = tid + NTHREADS * i;
+        woff[i] = kOobOffset;
+        if (c < BN * 4) {
+            if (WMODE == W_ROWS || WMODE == W_ROWS4) {
+                const int n = n_base + (c >> 2);
+                if (n < g.N) woff[i] = (uint32_t)n * (uint32_t)g.ldw + (c & 3) * 16;
+            } else if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
+                // piece c = 16 channels of K row c / N16; rows at or beyond K lie past the end of the buffer
+                // resource and read as 0 without a test
+                const int n = n_base + (c % N16) * 16;
+                if (n < g.N) woff[i] = (uint32_t)(c / N16) * (uint32_t)g.ldw + n;
+            }
+        }
+    }
+
+    // global -> registers for the K step starting at k0 (the steps are requested in increasing order)
+    auto prefetch = [&](int k0, uint4 (&xr)[XROWS], uint4 (&wr)[WCHUNKS], uint32_t &xpad) {
+        xpad = 0;
+        if (XMODE == X_PLAIN) {
+            const bool kin = k0 + x_kc * 16 < g.K;
+#pragma unroll
+            for (int i = 0; i < XROWS; i++) xr[i] = buf_load16(xres, kin ? xoff[i] + (uint32_t)k0 : kOobOffset);
+        } else if (XMODE == X_PLAIN4) {
+            const int kp = k0 + x_kc * 16;  // K % 4 == 0: a dword lies wholly inside or outside the row
+#pragma unroll
+            for (int i = 0; i < XROWS; i++) {
+                const uint32_t off = xoff[i] + (uint32_t)k0;
+                const bool v = xoff[i] != kOobOffset;
+                xr[i].x = buf_load4(xres, (v && kp + 0 < g.K) ? off + 0 : kOobOffset);
+                xr[i].y = buf_load4(xres, (v && kp + 4 < g.K) ? off + 4 : kOobOffset);
+                xr[i].z = buf_load4(xres, (v && kp + 8 < g.K) ? off + 8 : kOobOffset);
+                xr[i].w = buf_load4(xres, (v && kp + 12 < g.K) ? off + 12 : kOobOffset);
+            }
+        } else if (XMODE == X_TAP) {
+            const bool kin = tap_ky < g.KH;
+            const int oy = tap_ky * g.dy, ox = tap_kx * g.dx;
+#pragma unroll
+            for (int i = 0; i < XROWS; i++) {
+                const int y = rows[i].iy0 + oy, x = rows[i].ix0 + ox;
+                const bool inb = (unsigned)y < (unsigned)g.H && (unsigned)x < (unsigned)g.W;
+                const uint32_t off = xoff[i] + (uint32_t)y * (uint32_t)g.x_sy + (uint32_t)x * (uint32_t)g.x_sx +
+                                     (uint32_t)tap_ic;
+                xr[i] = buf_load16(xres, (kin && inb && rows[i].valid) ? off : kOobOffset);
+                if (kin && !inb && rows[i].valid) xpad |= 1u << i;  // a padded tap: filled with zx when staged
+            }
+            tap_ic += BK;
+            if (tap_ic >= g.IC) {
+                tap_ic = 0;
+                if (++tap_kx == g.KW) {
+                    tap_kx = 0;
+                    ++tap_ky;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < XROWS; i++) xr[i] = load_x_chunk(g, rows[i], ks);
+            kstate_advance(ks, BK, g.IC, g.KW);
+        }
+        if (WMODE == W_ROWS) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                const bool kin = k0 + (c & 3) * 16 < g.K;
+                wr[i] = buf_load16(wres, kin ? woff[i] + (uint32_t)k0 : kOobOffset);
+            }
+        } else if (WMODE == W_ROWS4) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int kp = k0 + ((tid + NTHREADS * i) & 3) * 16;
+                const uint32_t off = woff[i] + (uint32_t)k0;
+                const bool v = woff[i] != kOobOffset;
+                wr[i].x = buf_load4(wres, (v && kp + 0 < g.K) ? off + 0 : kOobOffset);
+                wr[i].y = buf_load4(wres, (v && kp + 4 < g.K) ? off + 4 : kOobOffset);
+                wr[i].z = buf_load4(wres, (v && kp + 8 < g.K) ? off + 8 : kOobOffset);
+                wr[i].w = buf_load4(wres, (v && kp + 12 < g.K) ? off + 12 : kOobOffset);
+            }
+        } else if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const uint32_t off = woff[i] + (uint32_t)k0 * (uint32_t)g.ldw;
+                if (WMODE == W_KMAJOR) {
+                    wr[i] = buf_load16(wres, off);
+                } else {  // rows are only dword aligned: four loads, channels at or beyond N masked
+                    const int n = n_base + ((tid + NTHREADS * i) % N16) * 16;
+                    wr[i].x = buf_load4(wres, n + 0 < g.N ? off + 0 : kOobOffset);
+                    wr[i].y = buf_load4(wres, n + 4 < g.N ? off + 4 : kOobOffset);
+                    wr[i].z = buf_load4(wres, n + 8 < g.N ? off + 8 : kOobOffset);
+                    wr[i].w = buf_load4(wres, n + 12 < g.N ? off + 12 : kOobOffset);
+                }
+            }
+        } else if (!g.w_kmajor) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                if (c < BN * 4) wr[i] = load_w_chunk(g, wb, n_base + (c >> 2), k0 + (c & 3) * 16);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                if (c < BN * 4) wr[i] = load_w_block_kmajor(g, wb, n_base + (c % (BN / 4)) * 4, k0 + (c / (BN / 4)) * 4);
+            }
+        }
+    };
+    // registers -> LDS buffer `buf`
+    auto stage = [&](int buf, const uint4 (&xr)[XROWS], const uint4 (&wr)[WCHUNKS], uint32_t xpad) {
+        char *xd = xs + buf * BM * PITCH;
+        char *wd = ws + buf * WBUF;
+        const uint32_t z = splat8(g.zx);
+#pragma unroll
+        for (int i = 0; i < XROWS; i++) {
+            uint4 v = xr[i];
+            if (XMODE == X_TAP && ((xpad >> i) & 1u)) v = make_uint4(z, z, z, z);
+            *reinterpret_cast<uint4 *>(xd + ((tid >> 2) + 64 * i) * PITCH + x_kc * 16) = v;
+        }
+        if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                if (c < BN * 4) *reinterpret_cast<uint4 *>(wd + (c / N16) * PW + (c % N16) * 16) = wr[i];
+            }
+        } else if (WMODE == W_ROWS || WMODE == W_ROWS4 || !g.w_kmajor) {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                if (c < BN * 4) *reinterpret_cast<uint4 *>(wd + (c >> 2) * PITCH + (c & 3) * 16) = wr[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < WCHUNKS; i++) {
+                const int c = tid + NTHREADS * i;
+                if (c < BN * 4) {
+                    const int nl = (c % (BN / 4)) * 4, kl = (c / (BN / 4)) * 4;
+                    *reinterpret_cast<uint32_t *>(wd + (nl + 0) * PITCH + kl) = wr[i].x;
+                    *reinterpret_cast<uint32_t *>(wd + (nl + 1) * PITCH + kl) = wr[i].y;
+                    *reinterpret_cast<uint32_t *>(wd + (nl + 2) * PITCH + kl) = wr[i].z;
+                    *reinterpret_cast<uint32_t *>(wd + (nl + 3) * PITCH + kl) = wr[i].w;
+                }
+            }
+        }
+    };
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+    int32_t xsum[TM], wsum[TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++) xsum[i] = 0;
+#pragma unroll
+    for (int j = 0; j < TN; j++) wsum[j] = 0;
+    const bool need_xsum = SUMS && g.zw != 0, need_wsum = SUMS && g.zx != 0;
+
+    auto compute = [&](int buf) {
+        const char *xd = xs + buf * BM * PITCH + (wave_m * WM + (lane & 31)) * PITCH + (lane >> 5) * 16;
+        const char *wd = ws + buf * WBUF + (wave_n * WN + (lane & 31)) * PITCH + (lane >> 5) * 16;
+        // K-major tile: a 16-lane group transposes an 8(k) x 16(n) byte block; lane L of the group supplies the
+        // address of K row L / 2, channel half L % 2, and receives the 8 k-bytes of channel L.  Groups 0/1 cover
+        // channels 0-15 / 16-31 of the tile for k 0-15, groups 2/3 the same channels for k 16-31.
+        const char *wt = ws + buf * WBUF + ((lane >> 5) * 16 + ((lane & 15) >> 1)) * PW + wave_n * WN +
+                         ((lane >> 4) & 1) * 16 + (lane & 1) * 8;
+#pragma unroll
+        for (int kk = 0; kk < BK / 32; kk++) {
+            v4i xf[TM], wf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) xf[i] = *reinterpret_cast<const v4i *>(xd + i * 32 * PITCH + kk * 32);
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
+                    const char *p = wt + kk * 32 * PW + j * 32;
+                    const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(p));
+                    const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(p + 8 * PW));
+                    wf[j] = v4i{lo.x, lo.y, hi.x, hi.y};
+                } else {
+                    wf[j] = *reinterpret_cast<const v4i *>(wd + j * 32 * PITCH + kk * 32);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
+            if (SUMS) {  // both sums are kept whenever a zero point is non-zero: 16 dot4 beside 8 MFMAs
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) xsum[i] = __builtin_amdgcn_sdot4(xf[i][q], 0x01010101, xsum[i], false);
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) wsum[j] = __builtin_amdgcn_sdot4(wf[j][q], 0x01010101, wsum[j], false);
+            }
+        }
+    };
+
+    // ---- main loop: a ring of DEPTH register sets keeps DEPTH - 1 K steps of global loads in flight while one
+    // step is multiplied out of LDS (two LDS buffers).  At the top of sub-iteration s: LDS[s & 1] holds step s and
+    // register set (s + j) % DEPTH holds step s + j for j = 1 .. DEPTH - 1; the set of step s is free again.
+    // Every prefetch and stage is unconditional: a K step at or beyond K loads nothing (buffer bounds / tap state
+    // return zeros) and is never multiplied, and the straight-line body lets the compiler count exactly how many
+    // loads may remain in flight at each wait instead of draining them all.
+    constexpr int DEPTH = (XMODE == X_GENERIC || WMODE == W_GENERIC) ? 2 : 4;  // the generic fetch state is large
+    const int nk = (g.K + BK - 1) / BK;
+    uint4 xr[DEPTH][XROWS], wr[DEPTH][WCHUNKS];
+    uint32_t xp[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) prefetch(d * BK, xr[d], wr[d], xp[d]);
+    stage(0, xr[0], wr[0], xp[0]);
+    __syncthreads();
+    for (int step = 0; step < nk; step += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            if (step + d < nk) {  // uniform
+                prefetch((step + d + DEPTH) * BK, xr[d], wr[d], xp[d]);
+                compute(d & 1);
+                stage((d + 1) & 1, xr[(d + 1) % DEPTH], wr[(d + 1) % DEPTH], xp[(d + 1) % DEPTH]);
+                __syncthreads();
+            }
+        }
+    }
+
+    // ---- fold the zero-point terms that depend on the channel only into the per-channel bias
+    if (need_wsum && wave_m == 0) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int32_t s = wsum[j] + __shfl_xor(wsum[j], 32);
+            if (lane < 32) {
+                const int n = wave_n * WN + j * 32 + lane;
+                cp[n].bias_adj = (int32_t)((uint32_t)cp[n].bias_adj - (uint32_t)g.zx * (uint32_t)s +
+                                           (uint32_t)g.K * (uint32_t)g.zx * (uint32_t)g.zw);
+            }
+        }
+    }
+    if (need_xsum) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            xsum[i] = (int32_t)((uint32_t)(xsum[i] + __shfl_xor(xsum[i], 32)) * (uint32_t)g.zw);
+    }
+    __syncthreads();
+
+    // ---- epilogue: lane holds output position m = lane % 32 of each tile row and, per register group q, the four
+    // channels n0 .. n0+3 with n0 = 8q + 4 * (lane / 32)
+    char *ob = g.out + (int64_t)batch * g.out_batch;
+    if (Q8) {
+        // Fused RESCALE(+CLAMP) to 8-bit outputs, N % 4 == 0, output extent below 2^31: straight-line code.  Rows and
+        // channels outside the problem get an offset beyond the buffer bounds, which drops the store.
+        const __amdgpu_buffer_rsrc_t ores = make_rsrc(ob, g.o_bytes);
+        uint32_t row_off[TM];
+        int32_t xcorr[TM];
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
+            row_off[i] = m < g.M ? (uint32_t)m * (uint32_t)g.ldo : kOobOffset;
+            xcorr[i] = need_xsum ? xsum[i] : 0;
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int nl = wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+                const int n0 = n_base + nl;
+                ChanParams c[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) c[e] = cp[nl + e];
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    uint32_t packed = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)c[e].bias_adj -
+                                                    (uint32_t)xcorr[i]);
+                        packed |= ((uint32_t)requant_chan(a, c[e].q, g.rp) & 0xffu) << (8 * e);
+                    }
+                    const uint32_t off = (n0 < g.N && row_off[i] != kOobOffset) ? row_off[i] + (uint32_t)n0 : kOobOffset;
+                    __builtin_amdgcn_raw_buffer_store_b32(packed, ores, (int)off, 0, 0);
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
+        if (m >= g.M) continue;
+        const int32_t xcorr = need_xsum ? xsum[i] : 0;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int nl = wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+                const int n0 = n_base + nl;
+                if (n0 >= g.N) continue;
+                int32_t v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int32_t a =
+                        (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)cp[nl + e].bias_adj - (uint32_t)xcorr);
+                    if (!g.fused)
+                        v[e] = a;
+                    else
+                        v[e] = requant_chan(a, cp[nl + e].q, g.rp);
+                }
+                const int64_t off = (int64_t)m * g.ldo + n0;
+                if (g.out_vec_ok && n0 + 3 < g.N) {
+                    if (g.out_size == 1) {
+                        const uint32_t packed = (uint32_t)(uint8_t)v[0] | ((uint32_t)(uint8_t)v[1] << 8) |
+                                                ((uint32_t)(uint8_t)v[2] << 16) | ((uint32_t)(uint8_t)v[3] << 24);
+                        *reinterpret_cast<uint32_t *>(ob + off) = packed;
+                    } else if (g.out_size == 2) {
+                        const uint32_t lo = (uint32_t)(uint16_t)v[0] | ((uint32_t)(uint16_t)v[1] << 16);
+                        const uint32_t hi = (uint32_t)(uint16_t)v[2] | ((uint32_t)(uint16_t)v[3] << 16);
+                        *reinterpret_cast<uint2 *>(ob + off * 2) = make_uint2(lo, hi);
+                    } else {
+                        *reinterpret_cast<int4 *>(ob + off * 4) = make_int4(v[0], v[1], v[2], v[3]);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (n0 + e >= g.N) break;
+                        if (g.out_size == 1)
+                            *reinterpret_cast<int8_t *>(ob + off + e) = (int8_t)v[e];
+                        else if (g.out_size == 2)
+                            *reinterpret_cast<int16_t *>(ob + (off + e) * 2) = (int16_t)v[e];
+                        else
+                            *reinterpret_cast<int32_t *>(ob + (off + e) * 4) = v[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN>
+constexpr size_t smem_bytes() {
+    return (size_t)2 * BM * PITCH + (size_t)2 * w_buf_bytes<BN>() + (size_t)BN * sizeof(ChanParams);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool SUMS, bool Q8>
+void launch_tile(const GemmArgs &g, int xmode, int wmode, dim3 grid, hipStream_t s) {
+    const size_t sm = smem_bytes<BM, BN>();
+    if (xmode == X_PLAIN && wmode == W_ROWS)
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_ROWS, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    else if (xmode == X_TAP && wmode == W_ROWS)
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_TAP, W_ROWS, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    else if (xmode == X_PLAIN && wmode == W_KMAJOR)
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    else if (xmode == X_PLAIN && wmode == W_KMAJOR4)
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR4, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    else if (xmode == X_PLAIN4 && wmode == W_ROWS4)
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN4, W_ROWS4, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+    else
+        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_GENERIC, W_GENERIC, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+void launch_tile_zp(const GemmArgs &g, int xmode, int wmode, dim3 grid, hipStream_t s) {
+    const bool sums = g.zx != 0 || g.zw != 0;
+    const bool q8 = g.fused && g.out_size == 1 && g.out_vec_ok && g.o_bytes != 0;
+    if (sums && q8)
+        launch_tile<BM, BN, WAVES_M, WAVES_N, true, true>(g, xmode, wmode, grid, s);
+    else if (sums)
+        launch_tile<BM, BN, WAVES_M, WAVES_N, true, false>(g, xmode, wmode, grid, s);
+    else if (q8)
+        launch_tile<BM, BN, WAVES_M, WAVES_N, false, true>(g, xmode, wmode, grid, s);
+    else
+        launch_tile<BM, BN, WAVES_M, WAVES_N, false, false>(g, xmode, wmode, grid, s);
+}
+
+}  // namespace
+
+// One function per tile shape, each compiled in its own translation unit (gemm_i8_tile*.hip) so that the tile
+// shapes build in parallel.  Tile ids: see kGemmTiles in gemm_i8.hip.
+#define MLEL_DECLARE_GEMM_TILE(ID) \
+    void launch_gemm_tile##ID(const void *args, int xmode, int wmode, dim3 grid, hipStream_t s)
+MLEL_DECLARE_GEMM_TILE(0);
+MLEL_DECLARE_GEMM_TILE(1);
+MLEL_DECLARE_GEMM_TILE(2);
+MLEL_DECLARE_GEMM_TILE(3);
+MLEL_DECLARE_GEMM_TILE(4);
+MLEL_DECLARE_GEMM_TILE(5);
+#define MLEL_DEFINE_GEMM_TILE(ID, BM, BN, WAVES_M, WAVES_N)                                          \
+    void launch_gemm_tile##ID(const void *args, int xmode, int wmode, dim3 grid, hipStream_t s) {    \
+        launch_tile_zp<BM, BN, WAVES_M, WAVES_N>(*static_cast<const GemmArgs *>(args), xmode, wmode, grid, s); \
+    }
+
+}  // namespace mlel

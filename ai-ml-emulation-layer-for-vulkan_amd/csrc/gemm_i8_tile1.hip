@@ -1,0 +1,6 @@
+// int8 contraction kernel, tile shape 256 x 64 (wavefronts 4 x 1): see gemm_i8_kernel.hpp
+#include "gemm_i8_kernel.hpp"
+
+namespace mlel {
+MLEL_DEFINE_GEMM_TILE(1, 256, 64, 4, 1)
+}  // namespace mlel
