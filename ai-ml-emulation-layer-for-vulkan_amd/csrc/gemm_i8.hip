@@ -51,8 +51,7 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
     const int64_t tiles_n = (g.N + BN - 1) / BN;
     const int64_t tall_total = (int64_t)((g.M + tall.bm - 1) / tall.bm) * tiles_n * g.batches;
     const int cus = ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
-    Tile tile = tall_total >= 2 * (int64_t)cus ? tall : low;
-    if (const char *force = getenv("MLEL_GEMM_TILE_HEIGHT")) tile = force[0] == 't' ? tall : low;
+    const Tile tile = tall_total >= 2 * (int64_t)cus ? tall : low;
     g.tiles_m = (g.M + tile.bm - 1) / tile.bm;
     g.tiles_n = (int)tiles_n;
     const int64_t total = (int64_t)g.tiles_m * g.tiles_n * g.batches;

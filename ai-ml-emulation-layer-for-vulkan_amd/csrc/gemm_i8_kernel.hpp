@@ -33,7 +33,6 @@ typedef __attribute__((address_space(3))) v2i lds_v2i;
 
 constexpr int BK = 64;            // bytes of K per step
 constexpr int PITCH = BK + 16;    // LDS row pitch: 80 B keeps 16-lane groups of 128-bit reads on distinct banks
-constexpr int NTHREADS = 256;
 
 struct GemmArgs {
     // problem
@@ -232,12 +231,14 @@ enum WMode {
 };
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int XMODE, int WMODE, bool SUMS, bool Q8>
-__global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
+__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const GemmArgs g) {
+    constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wavefront sub-tile
     constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 MFMA tiles per wavefront
-    constexpr int XROWS = BM / 64;                       // X rows per thread (4 pieces of 16 B per row)
+    constexpr int XROWS = BM * 4 / NTHREADS;             // X rows per thread (4 pieces of 16 B per row)
     constexpr int WCHUNKS = (BN * 4 + NTHREADS - 1) / NTHREADS;
-    static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per block");
+    static_assert(WAVES_M * WAVES_N == 4 || WAVES_M * WAVES_N == 8, "four or eight wavefronts per block");
+    static_assert((BM * 4) % NTHREADS == 0, "whole X rows per thread");
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wavefront tile is a multiple of the 32x32 MFMA tile");
 
     constexpr int PW = BN + 16;           // W_KMAJOR: LDS pitch of one K row of BN channels (bytes)
@@ -268,20 +269,20 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
     const int8_t *xb = g.x + (int64_t)batch * g.x_batch;
     const int8_t *wb = g.w + (int64_t)batch * g.w_batch;
 
-    // ---- per-channel epilogue constants
-    for (int n = tid; n < BN; n += NTHREADS) {
-        ChanParams c{};
-        const int gn = n_base + n;
-        if (gn < g.N) {
-            c.bias_adj = g.bias ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
-            if (g.fused) {
-                const int ci = g.rp.per_channel ? gn : 0;
-                const int32_t m = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
-                                           : reinterpret_cast<const int32_t *>(g.mult)[ci];
-                c.q = make_chan_scale(m, (int32_t)g.shift[ci], g.rp);
-            }
+    // ---- per-channel epilogue constants: thread n < BN owns channel n.  The loads are issued here, ahead of the
+    // operand prefetch, but only consumed after the main loop, so their latency is never waited for.
+    static_assert(BN <= NTHREADS, "one thread per channel of the tile");
+    int32_t chan_bias = 0, chan_mult = 0, chan_shift = 0;
+    const bool chan_live = tid < BN && n_base + tid < g.N;
+    if (chan_live) {
+        const int gn = n_base + tid;
+        chan_bias = g.bias ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
+        if (g.fused) {
+            const int ci = g.rp.per_channel ? gn : 0;
+            chan_mult = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
+                                 : reinterpret_cast<const int32_t *>(g.mult)[ci];
+            chan_shift = (int32_t)g.shift[ci];
         }
-        cp[n] = c;
     }
 
     // ---- loader state
@@ -290,7 +291,7 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
     uint32_t xoff[XROWS];      // fast modes: byte offset of the row (X_PLAIN) / image (X_TAP), or kOobOffset
 #pragma unroll
     for (int i = 0; i < XROWS; i++) {
-        const int m = m_base + (tid >> 2) + 64 * i;
+        const int m = m_base + (tid >> 2) + (NTHREADS / 4) * i;
         RowState r{xb, 0, 0, m < g.M};
         xoff[i] = kOobOffset;
         if (r.valid) {
@@ -429,7 +430,7 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
         for (int i = 0; i < XROWS; i++) {
             uint4 v = xr[i];
             if (XMODE == X_TAP && ((xpad >> i) & 1u)) v = make_uint4(z, z, z, z);
-            *reinterpret_cast<uint4 *>(xd + ((tid >> 2) + 64 * i) * PITCH + x_kc * 16) = v;
+            *reinterpret_cast<uint4 *>(xd + ((tid >> 2) + (NTHREADS / 4) * i) * PITCH + x_kc * 16) = v;
         }
         if (WMODE == W_KMAJOR || WMODE == W_KMAJOR4) {
 #pragma unroll
@@ -520,7 +521,8 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
     // Every prefetch and stage is unconditional: a K step at or beyond K loads nothing (buffer bounds / tap state
     // return zeros) and is never multiplied, and the straight-line body lets the compiler count exactly how many
     // loads may remain in flight at each wait instead of draining them all.
-    constexpr int DEPTH = (XMODE == X_GENERIC || WMODE == W_GENERIC) ? 2 : 4;  // the generic fetch state is large
+    // the generic fetch state is large, and so are the register sets of the widest tiles
+    constexpr int DEPTH = (XMODE == X_GENERIC || WMODE == W_GENERIC || XROWS + WCHUNKS > 4) ? 2 : 4;
     const int nk = (g.K + BK - 1) / BK;
     uint4 xr[DEPTH][XROWS], wr[DEPTH][WCHUNKS];
     uint32_t xp[DEPTH];
@@ -540,6 +542,15 @@ __global__ void __launch_bounds__(NTHREADS) gemm_i8_kernel(const GemmArgs g) {
         }
     }
 
+    if (tid < BN) {
+        ChanParams c{};
+        if (chan_live) {
+            c.bias_adj = chan_bias;
+            if (g.fused) c.q = make_chan_scale(chan_mult, chan_shift, g.rp);
+        }
+        cp[tid] = c;
+    }
+    __syncthreads();
     // ---- fold the zero-point terms that depend on the channel only into the per-channel bias
     if (need_wsum && wave_m == 0) {
 #pragma unroll
@@ -656,21 +667,34 @@ constexpr size_t smem_bytes() {
     return (size_t)2 * BM * PITCH + (size_t)2 * w_buf_bytes<BN>() + (size_t)BN * sizeof(ChanParams);
 }
 
+template <typename Kernel>
+void launch_kernel(Kernel kernel, const GemmArgs &g, int threads, size_t sm, dim3 grid, hipStream_t s) {
+    if (sm > 48 * 1024) {  // above the default dynamic LDS limit: raise it once per kernel
+        static bool raised = false;
+        if (!raised) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)sm);
+            raised = true;
+        }
+    }
+    kernel<<<grid, dim3(threads), sm, s>>>(g);
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool SUMS, bool Q8>
 void launch_tile(const GemmArgs &g, int xmode, int wmode, dim3 grid, hipStream_t s) {
     const size_t sm = smem_bytes<BM, BN>();
     if (xmode == X_PLAIN && wmode == W_ROWS)
-        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_ROWS, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+        launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_ROWS, SUMS, Q8>, g, WAVES_M * WAVES_N * 64, sm, grid, s);
     else if (xmode == X_TAP && wmode == W_ROWS)
-        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_TAP, W_ROWS, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+        launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_TAP, W_ROWS, SUMS, Q8>, g, WAVES_M * WAVES_N * 64, sm, grid, s);
     else if (xmode == X_PLAIN && wmode == W_KMAJOR)
-        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+        launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR, SUMS, Q8>, g, WAVES_M * WAVES_N * 64, sm, grid, s);
     else if (xmode == X_PLAIN && wmode == W_KMAJOR4)
-        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR4, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+        launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_KMAJOR4, SUMS, Q8>, g, WAVES_M * WAVES_N * 64, sm, grid, s);
     else if (xmode == X_PLAIN4 && wmode == W_ROWS4)
-        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN4, W_ROWS4, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+        launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN4, W_ROWS4, SUMS, Q8>, g, WAVES_M * WAVES_N * 64, sm, grid, s);
     else
-        gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_GENERIC, W_GENERIC, SUMS, Q8><<<grid, dim3(NTHREADS), sm, s>>>(g);
+        launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_GENERIC, W_GENERIC, SUMS, Q8>, g, WAVES_M * WAVES_N * 64, sm, grid, s);
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N>

@@ -194,6 +194,100 @@ def mobilenetv2_spec(batch=32, image=224, seed=1003, spread=False, classes=1000)
     return spec
 
 
+def transformer_block_spec(batch=8, seq=512, d_model=768, heads=12, ffn=3072, seed=1004):
+    """BASELINE config 4: one fp16 transformer encoder block (pre-LayerNorm).  Projections are MATMUL with fp16
+    operands and an fp32 result (bias added in fp32, then CAST to fp16); attention is MATMUL for QK^T, softmax as
+    REDUCE_MAX / SUB / EXP / REDUCE_SUM / RECIPROCAL / MUL, then MATMUL with V; LayerNorm uses REDUCE_SUM and RSQRT;
+    GELU uses TANH.  Activations ~N(0,1), weights ~N(0,0.02)."""
+    rng = np.random.default_rng(seed)
+    spec = Spec()
+    spec.flops = 0
+    B, S, D, H, F = batch, seq, d_model, heads, ffn
+    dh = D // H
+    f16, f32 = abi.F16, abi.F32
+    spec.inputs.append(("input", f16, (B, S, D)))
+
+    def c16(v):
+        return spec.const("c", np.array(v, np.float16).reshape(1, 1, 1))
+
+    def un(op, x, shape, dt=f16):
+        y = spec.tensor("t", dt, shape)
+        spec.op(op, [x], [y])
+        return y
+
+    def bi(op, a, b, shape, dt=f16):
+        y = spec.tensor("t", dt, shape)
+        spec.op(op, [a, b], [y], [0] if op == "MUL" else [])
+        return y
+
+    def red(op, x, shape):
+        out = tuple(shape[:2]) + (1,)
+        y = spec.tensor("t", f16, out)
+        spec.op(op, [x], [y], [2, abi.NAN_PROPAGATE] if op in ("REDUCE_MAX", "REDUCE_MIN") else [2])
+        return y
+
+    def layer_norm(x, shape):
+        inv = c16(1.0 / shape[2])
+        mean = bi("MUL", red("REDUCE_SUM", x, shape), inv, shape[:2] + (1,))
+        xc = bi("SUB", x, mean, shape)
+        var = bi("MUL", red("REDUCE_SUM", bi("MUL", xc, xc, shape), shape), inv, shape[:2] + (1,))
+        rstd = un("RSQRT", bi("ADD", var, c16(1e-3), shape[:2] + (1,)), shape[:2] + (1,))
+        xn = bi("MUL", xc, rstd, shape)
+        gamma = spec.const("gamma", (1.0 + 0.02 * rng.standard_normal((1, 1, shape[2]))).astype(np.float16))
+        beta = spec.const("beta", (0.02 * rng.standard_normal((1, 1, shape[2]))).astype(np.float16))
+        return bi("ADD", bi("MUL", xn, gamma, shape), beta, shape)
+
+    def reshape(x, shape, dt=f16):
+        y = spec.tensor("t", dt, shape)
+        spec.op("RESHAPE", [x], [y])
+        return y
+
+    def transpose(x, perms):
+        src = spec.shape_of(x)
+        shape = tuple(src[p] for p in perms)
+        y = spec.tensor("t", f16, shape)
+        spec.op("TRANSPOSE", [x], [y], list(perms))
+        return y
+
+    def linear(x2, k, n, rows):
+        """x2 [1, rows, k] fp16 -> [1, rows, n] fp16: MATMUL (fp32 result) + bias (fp32) -> CAST."""
+        w = spec.const("w", (0.02 * rng.standard_normal((1, k, n))).astype(np.float16))
+        b = spec.const("b", (0.02 * rng.standard_normal((1, 1, n))).astype(np.float32))
+        acc = spec.tensor("acc", f32, (1, rows, n))
+        spec.op("MATMUL", [x2, w], [acc], [0, 0])
+        spec.flops += 2 * rows * k * n
+        return un("CAST", bi("ADD", acc, b, (1, rows, n), f32), (1, rows, n))
+
+    rows = B * S
+    x = "input"
+    y = reshape(layer_norm(x, (B, S, D)), (1, rows, D))
+    q = reshape(transpose(reshape(linear(y, D, D, rows), (B, S, H, dh)), (0, 2, 1, 3)), (B * H, S, dh))
+    kt = reshape(transpose(reshape(linear(y, D, D, rows), (B, S, H, dh)), (0, 2, 3, 1)), (B * H, dh, S))
+    v = reshape(transpose(reshape(linear(y, D, D, rows), (B, S, H, dh)), (0, 2, 1, 3)), (B * H, S, dh))
+    sc32 = spec.tensor("acc", f32, (B * H, S, S))
+    spec.op("MATMUL", [q, kt], [sc32], [0, 0])
+    spec.flops += 2 * B * H * S * S * dh
+    pshape = (B * H, S, S)
+    sc = bi("MUL", un("CAST", sc32, pshape), c16(1.0 / np.sqrt(dh)), pshape)
+    e = un("EXP", bi("SUB", sc, red("REDUCE_MAX", sc, pshape), pshape), pshape)
+    prob = bi("MUL", e, un("RECIPROCAL", red("REDUCE_SUM", e, pshape), (B * H, S, 1)), pshape)
+    ctx32 = spec.tensor("acc", f32, (B * H, S, dh))
+    spec.op("MATMUL", [prob, v], [ctx32], [0, 0])
+    spec.flops += 2 * B * H * S * S * dh
+    ctx = reshape(transpose(reshape(un("CAST", ctx32, (B * H, S, dh)), (B, H, S, dh)), (0, 2, 1, 3)), (1, rows, D))
+    x1 = bi("ADD", x, reshape(linear(ctx, D, D, rows), (B, S, D)), (B, S, D))
+    y2 = reshape(layer_norm(x1, (B, S, D)), (1, rows, D))
+    h = linear(y2, D, F, rows)
+    hs = (1, rows, F)
+    inner = bi("MUL", bi("ADD", h, bi("MUL", bi("MUL", bi("MUL", h, h, hs), h, hs), c16(0.044715), hs), hs),
+               c16(np.sqrt(2.0 / np.pi)), hs)
+    gelu = bi("MUL", bi("MUL", h, c16(0.5), hs), bi("ADD", un("TANH", inner, hs), c16(1.0), hs), hs)
+    f = reshape(linear(gelu, F, D, rows), (B, S, D))
+    spec.op("ADD", [x1, f], ["output"])
+    spec.outputs.append(("output", f16, (B, S, D)))
+    return spec
+
+
 def _retarget_output(spec, produced, name):
     """Makes the operator that produces `produced` write the external output tensor `name` instead."""
     dtype, shape = spec.tensors.pop(produced)

@@ -29,8 +29,18 @@ def run_spec(oracle, spec, inputs):
             r = oracle.rescale(ins[0], ins[1], ins[2], odt, attr)
         elif kind == "CLAMP":
             r = oracle.clamp(ins[0], fa[0], fa[1], ia[0])
-        elif kind == "ADD":
-            r = oracle.elementwise_binary("ADD", ins[0], ins[1], oshape, odt)
+        elif kind in ("ADD", "SUB"):
+            r = oracle.elementwise_binary(kind, ins[0], ins[1], oshape, odt)
+        elif kind == "MUL":
+            r = oracle.mul(ins[0], ins[1], oshape, odt, ia[0])
+        elif kind in ("EXP", "RECIPROCAL", "RSQRT", "TANH"):
+            r = oracle.elementwise_unary(kind, ins[0])
+        elif kind in ("REDUCE_SUM", "REDUCE_MAX"):
+            r = oracle.reduce(kind[len("REDUCE_"):], ins[0], ia[0], ia[1] if len(ia) > 1 else abi.NAN_PROPAGATE)
+        elif kind == "CAST":
+            r = oracle.cast(ins[0], odt)
+        elif kind == "TRANSPOSE":
+            r = oracle.transpose(ins[0], ia)
         elif kind == "AVG_POOL2D":
             r = oracle.avg_pool2d(ins[0], oshape, abi.pool2d_attr(ia[0:2], ia[2:4], ia[4:8], ia[9], ia[10], ia[8]))
         elif kind == "RESHAPE":

@@ -85,3 +85,44 @@ def test_config3_mobilenetv2_b32_full_size(dev, oracle):
     one = graphs.mobilenetv2_spec(batch=1, spread=True)
     out1, _ = run_graph(dev, one, x[:1], True)
     np.testing.assert_array_equal(out1[0, 0], out[0, 0])
+
+
+# ------------------------------------------------------------------------------------------------ config 4 (fp16)
+def run_float_graph(dev, spec, x):
+    g = graphs.build(dev, spec, fuse=True)
+    g.set_input("input", x)
+    g.dispatch()
+    out = g.get_output("output")
+    g.close()
+    return out
+
+
+@pytest.mark.parametrize("cfg", [dict(batch=2, seq=32, d_model=64, heads=4, ffn=128),
+                                 dict(batch=2, seq=128, d_model=768, heads=12, ffn=3072)],
+                         ids=["tiny", "d768"])
+def test_transformer_block_vs_oracle(dev, oracle, cfg):
+    """fp16 encoder block (BASELINE config 4 operators and widths): max abs error <= 1e-2 against the oracle running
+    the same operator list (fp16 storage, fp32 accumulation in MATMUL)."""
+    spec = graphs.transformer_block_spec(**cfg)
+    x = np.random.default_rng(44).standard_normal(spec.inputs[0][2]).astype(np.float16)
+    exp, _ = run_spec(oracle, spec, {"input": x})
+    out = run_float_graph(dev, spec, x)
+    err = np.abs(out.astype(np.float32) - exp["output"].astype(np.float32)).max()
+    assert np.isfinite(out.astype(np.float32)).all()
+    assert err <= 1e-2, err
+
+
+def test_config4_transformer_block_full_size(dev):
+    """BASELINE config 4 at full size (batch 8, seq 512, d_model 768, 12 heads, FFN 3072) against an independent fp32
+    numpy computation of the block; the oracle would need minutes here.  The bound is looser than 1e-2 because the
+    comparison is against exact fp32 mathematics, not against the fp16 operator sequence: the sequential fp16
+    REDUCE_SUM over 768 and 512 elements alone moves results by about 1e-2 (measured oracle-vs-fp32 at d_model 768:
+    1.3e-2)."""
+    from transformer_ref import encoder_block_fp32
+    spec = graphs.transformer_block_spec()
+    x = np.random.default_rng(1004).standard_normal(spec.inputs[0][2]).astype(np.float16)
+    out = run_float_graph(dev, spec, x).astype(np.float32)
+    ref = encoder_block_fp32(spec, x, 12)
+    assert np.isfinite(out).all()
+    assert np.abs(out - ref).max() <= 4e-2, np.abs(out - ref).max()
+    assert np.abs(out - ref).mean() <= 2e-3

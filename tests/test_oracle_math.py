@@ -341,3 +341,22 @@ def test_f16_codec_matches_numpy_for_all_bit_patterns(oracle):
                            6e-8, 5.96e-8, 2.98e-8, 2.9802322e-8, 0.0, -0.0]]).astype(np.float32)
     for v in vals:
         assert lib.mlel_cpu_f32_to_f16(float(v)) == int(np.float32(v).astype(np.float16).view(np.uint16))
+
+
+def test_transformer_block_oracle_vs_fp32_numpy(oracle):
+    """The fp16 encoder-block description executed by the oracle agrees with an independent fp32 numpy
+    computation of the same mathematics (tests/transformer_ref.py) to fp16 rounding of the intermediates."""
+    import importlib
+    from oracle_graph import run_spec
+    from transformer_ref import encoder_block_fp32
+    graphs = importlib.import_module("ai-ml-emulation-layer-for-vulkan_amd.graphs")
+    spec = graphs.transformer_block_spec(batch=2, seq=48, d_model=128, heads=4, ffn=256)
+    assert len(spec.ops) == 78
+    x = np.random.default_rng(7).standard_normal((2, 48, 128)).astype(np.float16)
+    out, env = run_spec(oracle, spec, {"input": x})
+    ref = encoder_block_fp32(spec, x, 4)
+    assert np.abs(out["output"].astype(np.float32) - ref).max() <= 5e-3
+    # softmax rows (the MUL that follows RECIPROCAL) sum to 1 within fp16 rounding
+    probs = [v for k, v in env.items() if isinstance(v, np.ndarray) and v.shape == (8, 48, 48) and v.dtype == np.float16
+             and v.min() >= 0 and abs(float(v[0, 0].astype(np.float32).sum()) - 1.0) < 2e-2]
+    assert probs, "no tensor with unit row sums found"
