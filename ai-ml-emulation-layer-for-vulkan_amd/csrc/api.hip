@@ -120,7 +120,8 @@ int mlel_hip_matmul(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const m
     MLEL_REQUIRE(a->dtype == b->dtype, MLEL_ERR_INVALID, "matmul: operand types differ");
     MLEL_REQUIRE(dt_is_float(a->dtype) == dt_is_float(out->dtype), MLEL_ERR_INVALID,
                  "matmul: integer/float mismatch between operands and output");
-    const int rc = try_matmul_i8_mfma(ctx, (hipStream_t)stream, out, a, b, attr, nullptr);
+    int rc = try_matmul_i8_mfma(ctx, (hipStream_t)stream, out, a, b, attr, nullptr);
+    if (rc == 0) rc = try_matmul_f16_mfma(ctx, (hipStream_t)stream, out, a, b, attr);
     if (rc != 0) return rc < 0 ? rc : 0;
     return matmul_generic_launch((hipStream_t)stream, out, a, b, attr);
 }

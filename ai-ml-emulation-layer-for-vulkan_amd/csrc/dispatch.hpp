@@ -76,6 +76,10 @@ int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, c
 int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
                        const mlel_tensor *b, const mlel_matmul_attr *attr, const FusedEpilogue *epi);
 
+// ---- fp16 MFMA MATMUL with fp32 result (gemm_f16.hip) ----
+int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
+                        const mlel_tensor *b, const mlel_matmul_attr *attr);
+
 // ---- bandwidth-bound specialisations (ops_fast.hip) ----
 int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                        const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,

@@ -1,0 +1,272 @@
+// fp16 x fp16 -> fp32 MATMUL on the gfx950 matrix cores (reference arithmetic: matmul.comp:30-73 with an fp32
+// accumulator: out[b][m][n] = sum_k A[b][m][k] * B[b][k][n]; the order of the fp32 additions differs from the
+// shader's sequential loop, which is why floating-point graphs are compared within a tolerance).
+//
+// Kernel shape.  256 threads = 4 wavefronts; a block owns a BM x BN tile of one batch and walks K in steps of 32
+// halfs through two LDS buffers, with the global loads of the next step in flight while the current one is
+// multiplied (v_mfma_f32_32x32x16_f16).  As in the int8 kernel the B matrix supplies the MFMA row operand and A the
+// column operand, so a lane ends up with four consecutive output columns of one output row per register quad and
+// stores them as one 128-bit word.
+//   A tile: [BM][32 halfs], 80-byte pitch, operands read with ds_read_b128 (8 consecutive k of one row);
+//   B tile: kept K-major as in memory, [32][BN halfs]; operands are gathered with ds_read_b64_tr_b16, which hands
+//           lane L of a 16-lane group the four k values of column L out of a 4(k) x 16(n) block whose rows are
+//           addressed by the group's lanes (lane s points at row s / 4, columns 4 * (s % 4) ..).
+// All global loads are buffer loads: an offset at or beyond the extent returns 0, which pads M, N and K tails.
+#include "common.hpp"
+#include "dispatch.hpp"
+
+namespace mlel {
+namespace {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4s lds_v4s;
+
+constexpr int NT = 256;
+constexpr int BKH = 32;          // halfs of K per step
+constexpr int XPITCH = 64 + 16;  // bytes per A row in LDS
+constexpr uint32_t kOob = 0x80000000u;
+
+struct HGemmArgs {
+    const char *a, *b;
+    char *out;
+    int32_t M, N, K, batches;
+    int64_t a_batch, b_batch, o_batch;  // bytes
+    uint32_t lda, ldb, ldo;             // bytes per row
+    uint32_t a_bytes, b_bytes, o_bytes; // per-batch extents (all below 2^31)
+    int32_t tiles_m, tiles_n, total_tiles, chunk;
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+    const v4i v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+    return make_uint4((uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int XROWS = BM / 64;            // 16-byte pieces of A per thread and step
+    constexpr int WPITCH = 2 * BN + 32;       // bytes per K row of the B tile: 4 rows x 32 B land on distinct banks
+    constexpr int WROW16 = BN / 8;            // 16-byte pieces per K row
+    constexpr int WCHUNKS = (BKH * WROW16) / NT;
+    static_assert(WAVES_M * WAVES_N == 4 && WM % 32 == 0 && WN % 32 == 0 && (BKH * WROW16) % NT == 0, "tile shape");
+    constexpr int XBUF = BM * XPITCH, WBUF = BKH * WPITCH;
+    extern __shared__ __align__(16) char smem[];
+    char *xs = smem;             // [2][BM][XPITCH]
+    char *ws = smem + 2 * XBUF;  // [2][BKH][WPITCH]
+
+    // consecutive tiles (sharing operand panels) go to the same XCD; blocks are dealt to XCDs round-robin
+    const int lin = __builtin_amdgcn_readfirstlane((int)(blockIdx.x % 8u) * g.chunk + (int)(blockIdx.x / 8u));
+    if (lin >= g.total_tiles) return;
+    const int per_batch = g.tiles_m * g.tiles_n;
+    const int batch = lin / per_batch;
+    const int t_in = lin - batch * per_batch;
+    const int tile_m = t_in / g.tiles_n, tile_n = t_in - tile_m * g.tiles_n;
+    const int m_base = tile_m * BM, n_base = tile_n * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+
+    const __amdgpu_buffer_rsrc_t ares = rsrc(g.a + (int64_t)batch * g.a_batch, g.a_bytes);
+    const __amdgpu_buffer_rsrc_t bres = rsrc(g.b + (int64_t)batch * g.b_batch, g.b_bytes);
+
+    uint32_t xoff[XROWS], woff[WCHUNKS];
+#pragma unroll
+    for (int i = 0; i < XROWS; i++) {
+        const int m = m_base + (tid >> 2) + 64 * i;
+        xoff[i] = m < g.M ? (uint32_t)m * g.lda + (tid & 3) * 16 : kOob;
+    }
+#pragma unroll
+    for (int i = 0; i < WCHUNKS; i++) {
+        const int c = tid + NT * i;
+        const int n = n_base + (c % WROW16) * 8;
+        woff[i] = n < g.N ? (uint32_t)(c / WROW16) * g.ldb + (uint32_t)n * 2 : kOob;
+    }
+    auto prefetch = [&](int k0, uint4 (&xr)[XROWS], uint4 (&wr)[WCHUNKS]) {
+        const bool kin = k0 + (tid & 3) * 8 < g.K;  // K % 8 == 0: a piece lies wholly inside or outside
+#pragma unroll
+        for (int i = 0; i < XROWS; i++) xr[i] = load16(ares, (kin && xoff[i] != kOob) ? xoff[i] + (uint32_t)k0 * 2 : kOob);
+#pragma unroll
+        for (int i = 0; i < WCHUNKS; i++) {
+            const int row = (tid + NT * i) / WROW16;
+            wr[i] = load16(bres, (k0 + row < g.K && woff[i] != kOob) ? woff[i] + (uint32_t)k0 * g.ldb : kOob);
+        }
+    };
+    auto stage = [&](int buf, const uint4 (&xr)[XROWS], const uint4 (&wr)[WCHUNKS]) {
+#pragma unroll
+        for (int i = 0; i < XROWS; i++)
+            *reinterpret_cast<uint4 *>(xs + buf * XBUF + ((tid >> 2) + 64 * i) * XPITCH + (tid & 3) * 16) = xr[i];
+#pragma unroll
+        for (int i = 0; i < WCHUNKS; i++) {
+            const int c = tid + NT * i;
+            *reinterpret_cast<uint4 *>(ws + buf * WBUF + (c / WROW16) * WPITCH + (c % WROW16) * 16) = wr[i];
+        }
+    };
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    // operand addresses inside a tile: A row = lane % 32, k group = lane / 32 (8 halfs each);
+    // B: 16-lane group q = lane / 16 covers columns 16 * (q & 1) .., k group q / 2; lane s = lane % 16 points at
+    // row s / 4, columns 4 * (s % 4) of the 4 x 16 block
+    const int a_row = lane & 31, a_kg = lane >> 5;
+    const int s16 = lane & 15, q16 = lane >> 4;
+    const int b_row = 8 * (q16 >> 1) + (s16 >> 2), b_col = 16 * (q16 & 1) + 4 * (s16 & 3);
+    auto compute = [&](int buf) {
+        const char *xt = xs + buf * XBUF;
+        const char *wt = ws + buf * WBUF;
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            v8h af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                af[i] = *reinterpret_cast<const v8h *>(xt + (wave_m * WM + i * 32 + a_row) * XPITCH + kk * 32 + a_kg * 16);
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const char *p = wt + (kk * 16 + b_row) * WPITCH + (wave_n * WN + j * 32 + b_col) * 2;
+                const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)p);
+                const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)(p + 4 * WPITCH));
+                union {
+                    v4s s[2];
+                    v8h h;
+                } u;
+                u.s[0] = lo;
+                u.s[1] = hi;
+                bf[j] = u.h;
+            }
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    // ring of DEPTH register sets: DEPTH - 1 steps of global loads in flight while one step is multiplied
+    constexpr int DEPTH = 4;
+    const int nk = (g.K + BKH - 1) / BKH;
+    uint4 xr[DEPTH][XROWS], wr[DEPTH][WCHUNKS];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) prefetch(d * BKH, xr[d], wr[d]);
+    stage(0, xr[0], wr[0]);
+    __syncthreads();
+    for (int step = 0; step < nk; step += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            if (step + d < nk) {  // uniform
+                prefetch((step + d + DEPTH) * BKH, xr[d], wr[d]);
+                compute(d & 1);
+                stage((d + 1) & 1, xr[(d + 1) % DEPTH], wr[(d + 1) % DEPTH]);
+                __syncthreads();
+            }
+        }
+    }
+
+    // ---- store: lane holds row m = lane % 32 of each sub-tile and, per register quad q, columns 8q + 4 * (lane / 32)
+    const __amdgpu_buffer_rsrc_t ores = rsrc(g.out + (int64_t)batch * g.o_batch, g.o_bytes);
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
+        const uint32_t row_off = m < g.M ? (uint32_t)m * g.ldo : kOob;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int n0 = n_base + wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+                const uint32_t off = (row_off != kOob && n0 < g.N) ? row_off + (uint32_t)n0 * 4 : kOob;
+                v4i v;
+                v.x = __float_as_int(acc[i][j][4 * q + 0]);
+                v.y = __float_as_int(acc[i][j][4 * q + 1]);
+                v.z = __float_as_int(acc[i][j][4 * q + 2]);
+                v.w = __float_as_int(acc[i][j][4 * q + 3]);
+                __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+void launch(const HGemmArgs &g, dim3 grid, hipStream_t s) {
+    constexpr size_t sm = (size_t)2 * BM * XPITCH + (size_t)2 * BKH * (2 * BN + 32);
+    gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N><<<grid, dim3(NT), sm, s>>>(g);
+}
+
+bool dense_rows(const mlel_tensor *t) { return t->strides[2] == 2 && t->strides[1] >= t->dims[2] * 2; }
+
+}  // namespace
+
+int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
+                        const mlel_tensor *b, const mlel_matmul_attr *attr) {
+    if (a->dtype != MLEL_F16 || b->dtype != MLEL_F16 || out->dtype != MLEL_F32) return 0;
+    if (attr->a_zp != 0 || attr->b_zp != 0) return 0;
+    const int64_t NB = out->dims[0], M = out->dims[1], N = out->dims[2], K = a->dims[2];
+    // what the kernel's indexing assumes: element-contiguous rows, 16-byte aligned rows and bases, K and N in
+    // multiples of 8, per-batch extents below 2^31, operands at least as large as the output implies
+    if (a->dims[0] < NB || b->dims[0] < NB || a->dims[1] < M || b->dims[1] < K || b->dims[2] < N) return 0;
+    if (!dense_rows(a) || !dense_rows(b) || out->strides[2] != 4) return 0;
+    if (K % 8 != 0 || N % 8 != 0 || K <= 0) return 0;
+    auto aligned = [](const mlel_tensor *t) {
+        return ((uintptr_t)t->ptr % 16) == 0 && t->strides[0] % 16 == 0 && t->strides[1] % 16 == 0;
+    };
+    if (!aligned(a) || !aligned(b) || !aligned(out)) return 0;
+    const int64_t lim = (int64_t(1) << 31) - 64;
+    const int64_t ab = a->dims[1] * a->strides[1], bb = b->dims[1] * b->strides[1], ob = M * out->strides[1];
+    if (ab >= lim || bb >= lim || ob >= lim || a->strides[1] >= lim || b->strides[1] >= lim) return 0;
+    if (M >= (1 << 24) || N >= (1 << 24) || K >= (1 << 24)) return 0;
+    if (NB <= 0 || M <= 0 || N <= 0) return 1;
+
+    HGemmArgs g{};
+    g.a = static_cast<const char *>(a->ptr);
+    g.b = static_cast<const char *>(b->ptr);
+    g.out = static_cast<char *>(out->ptr);
+    g.M = (int)M;
+    g.N = (int)N;
+    g.K = (int)K;
+    g.batches = (int)NB;
+    g.a_batch = a->strides[0];
+    g.b_batch = b->strides[0];
+    g.o_batch = out->strides[0];
+    g.lda = (uint32_t)a->strides[1];
+    g.ldb = (uint32_t)b->strides[1];
+    g.ldo = (uint32_t)out->strides[1];
+    g.a_bytes = (uint32_t)ab;
+    g.b_bytes = (uint32_t)bb;
+    g.o_bytes = (uint32_t)ob;
+    // tile choice: the width with the least padding of N; the tall tile when it still gives every compute unit two
+    // blocks, otherwise the short one
+    const int BN = ((N + 127) / 128) * 128 <= ((N + 63) / 64) * 64 ? 128 : 64;
+    const int cus = ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
+    const int64_t tiles_n = (N + BN - 1) / BN;
+    const bool tall = ((M + 127) / 128) * tiles_n * NB >= 2 * (int64_t)cus;
+    const int BM = tall ? 128 : 64;
+    g.tiles_m = (int)((M + BM - 1) / BM);
+    g.tiles_n = (int)tiles_n;
+    const int64_t total = (int64_t)g.tiles_m * g.tiles_n * NB;
+    MLEL_REQUIRE(total < (int64_t(1) << 30), MLEL_ERR_LIMIT, "matmul: %lld tiles", (long long)total);
+    g.total_tiles = (int)total;
+    g.chunk = (int)((total + 7) / 8);
+    const dim3 grid((unsigned)(g.chunk * 8));
+    if (BN == 128 && tall)
+        launch<128, 128, 2, 2>(g, grid, s);
+    else if (BN == 128)
+        launch<64, 128, 1, 4>(g, grid, s);
+    else if (tall)
+        launch<128, 64, 2, 2>(g, grid, s);
+    else
+        launch<64, 64, 2, 2>(g, grid, s);
+    MLEL_TRY(check_launch("matmul fp16"));
+    return 1;
+}
+
+}  // namespace mlel

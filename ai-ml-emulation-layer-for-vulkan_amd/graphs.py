@@ -349,3 +349,36 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32):
         "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}}
     g.close()
     return res
+
+
+def bench_transformer(dev, steps=5, warmup=2):
+    """Times whole-graph dispatches of BASELINE config 4 (fp16 encoder block, batch 8, seq 512, d_model 768) and
+    returns the extra fields bench.py adds to its JSON line."""
+    spec = transformer_block_spec()
+    g = build(dev, spec, fuse=True)
+    rng = np.random.default_rng(1004)
+    g.set_input("input", rng.standard_normal(spec.inputs[0][2]).astype(np.float16))
+    for _ in range(warmup):
+        g.dispatch()
+    dev.sync()
+    ev0, ev1 = dev.event(), dev.event()
+    t0 = time.perf_counter()
+    dev.record(ev0)
+    for _ in range(steps):
+        g.dispatch()
+    dev.record(ev1)
+    dev.sync()
+    wall = (time.perf_counter() - t0) / steps
+    gpu_ms = dev.elapsed_ms(ev0, ev1) / steps
+    per_op = g.dispatch_profiled()
+    dev.sync()
+    by_kind = {}
+    for name, ms in per_op:
+        by_kind[name] = by_kind.get(name, 0.0) + ms
+    res = {"transformer_b8_s512_d768": {
+        "ms_per_graph": wall * 1e3, "gpu_ms_per_graph": gpu_ms, "tflops": spec.flops / wall / 1e12,
+        "gflop": spec.flops / 1e9, "operators_executed": g.op_count(), "operators_in_graph": len(spec.ops),
+        "session_memory_bytes": g.session_size,
+        "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}}
+    g.close()
+    return res

@@ -159,6 +159,9 @@ def main():
             graphs = importlib.import_module(PKG + ".graphs")
             extra = graphs.bench_mobilenetv2(dev, steps=max(5, args.steps // 10), warmup=max(2, args.warmup // 10))
             log("config 3:", extra)
+            c4 = graphs.bench_transformer(dev)
+            log("config 4:", c4)
+            extra.update(c4)
         except Exception as e:  # the line below still reports config 1; the failure is visible
             log("config 3 leg failed:", repr(e))
             extra = {"mobilenetv2_b32": {"error": repr(e)}}

@@ -240,6 +240,38 @@ def test_matmul_float_generic(run, oracle):
     assert np.max(np.abs(out - oracle.matmul(a16, b16, abi.F32))) <= 1e-2
 
 
+HMM_CASES = [
+    # name, batches, M, K, N
+    ("proj_like", 1, 200, 768, 256),
+    ("scores_like", 6, 128, 64, 128),
+    ("av_like", 6, 128, 128, 64),
+    ("ragged_m_n", 2, 77, 40, 72),
+    ("k_tail", 1, 130, 104, 136),
+    ("tiny", 1, 3, 8, 8),
+    ("wide", 1, 64, 256, 1000),
+]
+
+
+@pytest.mark.parametrize("case", HMM_CASES, ids=[c[0] for c in HMM_CASES])
+def test_matmul_f16_mfma_vs_oracle(run, oracle, case):
+    """fp16 operands, fp32 result (the matrix-core kernel): max abs error <= 1e-2 against the oracle's sequential
+    fp32 accumulation, on activations ~N(0,1) and weights ~N(0,0.02) as in config 4, and on unit-normal operands."""
+    name, nb, m, k, n = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    a = rng.standard_normal((nb, m, k)).astype(np.float16)
+    for scale in (0.02, 1.0):
+        b = (scale * rng.standard_normal((nb, k, n))).astype(np.float16)
+        exp = oracle.matmul(a, b, abi.F32)
+        out = run.matmul(a, b, abi.F32)
+        assert out.shape == exp.shape
+        err = np.abs(out - exp).max()
+        assert err <= 1e-2 and err <= 1e-5 * max(1.0, np.abs(exp).max()) * k, (scale, err)
+    # exact cases: small integers are exact in fp16 and their sums in fp32, whatever the summation order
+    ai = rng.integers(-8, 8, (nb, m, k)).astype(np.float16)
+    bi = rng.integers(-8, 8, (nb, k, n)).astype(np.float16)
+    np.testing.assert_array_equal(run.matmul(ai, bi, abi.F32), np.einsum("bmk,bkn->bmn", ai.astype(np.float32), bi.astype(np.float32)))
+
+
 # ------------------------------------------------------------------------------------------------ DEPTHWISE
 DW_CASES = [
     ("c2_like_small", (2, 14, 14, 144), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -4, 0),
