@@ -163,7 +163,8 @@ int mlel_hip_elementwise_binary(mlel_ctx *ctx, void *stream, int32_t op, const m
     MLEL_REQUIRE(in1->dtype == in2->dtype, MLEL_ERR_INVALID, "elementwise_binary: input types differ");
     MLEL_REQUIRE(in1->rank == out->rank && in2->rank == out->rank, MLEL_ERR_INVALID,
                  "elementwise_binary: ranks differ");
-    const int rc = try_binary_fast(ctx, (hipStream_t)stream, op, out, in1, in2);
+    int rc = try_binary_fast(ctx, (hipStream_t)stream, op, out, in1, in2);
+    if (rc == 0) rc = try_binary_float_fast(ctx, (hipStream_t)stream, op, out, in1, in2);
     if (rc != 0) return rc < 0 ? rc : 0;
     return binary_generic_launch((hipStream_t)stream, op, out, in1, in2, nan_mode);
 }
@@ -177,6 +178,10 @@ int mlel_hip_mul(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel
     MLEL_REQUIRE(in1->dtype == in2->dtype, MLEL_ERR_INVALID, "mul: input types differ");
     MLEL_REQUIRE(in1->rank == out->rank && in2->rank == out->rank, MLEL_ERR_INVALID, "mul: ranks differ");
     MLEL_REQUIRE(shift <= 63, MLEL_ERR_INVALID, "mul: shift %u", shift);
+    {
+        const int rc = try_mul_float_fast(ctx, (hipStream_t)stream, out, in1, in2);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return mul_generic_launch((hipStream_t)stream, out, in1, in2, shift);
 }
 
@@ -187,6 +192,10 @@ int mlel_hip_elementwise_unary(mlel_ctx *ctx, void *stream, int32_t op, const ml
     MLEL_TRY(check_supported(out, "unary out"));
     MLEL_TRY(check_supported(in, "unary in"));
     MLEL_REQUIRE(in->dtype == out->dtype && in->rank == out->rank, MLEL_ERR_INVALID, "unary: type/rank mismatch");
+    {
+        const int rc = try_unary_float_fast(ctx, (hipStream_t)stream, op, out, in);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return unary_generic_launch((hipStream_t)stream, op, out, in);
 }
 
@@ -199,6 +208,10 @@ int mlel_hip_reduce(mlel_ctx *ctx, void *stream, int32_t op, const mlel_tensor *
     MLEL_REQUIRE(in->dtype == out->dtype && in->rank == out->rank, MLEL_ERR_INVALID, "reduce: type/rank mismatch");
     MLEL_REQUIRE((int)axis < in->rank, MLEL_ERR_INVALID, "reduce: axis %u outside rank %d", axis, in->rank);
     if (!dt_is_float(in->dtype)) nan_mode = MLEL_NAN_PROPAGATE;  // reference: compute_graph_op.cpp:1674-1680
+    {
+        const int rc = try_reduce_float_fast(ctx, (hipStream_t)stream, op, out, in, axis, nan_mode);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return reduce_generic_launch((hipStream_t)stream, op, out, in, axis, nan_mode);
 }
 
@@ -247,6 +260,10 @@ int mlel_hip_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mle
     MLEL_TRY(check_supported(out, "cast out"));
     MLEL_TRY(check_supported(in, "cast in"));
     MLEL_REQUIRE(in->rank == out->rank, MLEL_ERR_INVALID, "cast: ranks differ");
+    {
+        const int rc = try_cast_float_fast(ctx, (hipStream_t)stream, out, in);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return cast_generic_launch((hipStream_t)stream, out, in);
 }
 

@@ -208,6 +208,20 @@ __device__ inline void st_f(const TV &t, const int64_t *idx, float v) {
 __device__ inline float rnd_f16(float v) { return __half2float(__float2half_rn(v)); }
 __device__ inline float round_to(int dt, float v) { return dt == MLEL_F16 ? rnd_f16(v) : v; }
 
+// TANH as the reference computes it (elementwise_unary.comp:136-205): saturated beyond |x| > 10, an odd polynomial
+// below 0.2, the library function in between.
+__device__ inline float tanh_clamped(float x) {
+    const float ax = fabsf(x);
+    if (x > 10.0f) return 1.0f;
+    if (x < -10.0f) return -1.0f;
+    if (ax < 0.2f) {
+        const float x2 = x * x;
+        return x * (1.0f - x2 * (1.0f / 3.0f - x2 * (2.0f / 15.0f - 17.0f / 315.0f * x2)));
+    }
+    return tanhf(x);
+}
+
+
 __host__ __device__ inline int64_t narrow_to(int dt, int64_t v) {
     switch (dt) {
     case MLEL_BOOL: return v != 0;

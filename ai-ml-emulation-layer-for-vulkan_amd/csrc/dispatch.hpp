@@ -80,6 +80,16 @@ int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
 int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
                         const mlel_tensor *b, const mlel_matmul_attr *attr);
 
+// ---- floating-point elementwise / reduce specialisations (ops_float.hip) ----
+int try_binary_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in1,
+                          const mlel_tensor *in2);
+int try_mul_float_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in1,
+                       const mlel_tensor *in2);
+int try_unary_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in);
+int try_cast_float_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in);
+int try_reduce_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in,
+                          uint32_t axis, uint32_t nan_mode);
+
 // ---- bandwidth-bound specialisations (ops_fast.hip) ----
 int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                        const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,

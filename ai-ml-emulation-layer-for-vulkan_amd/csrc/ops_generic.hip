@@ -331,17 +331,6 @@ __device__ inline float erf_ref(float x) {
     return s * prod;
 }
 
-__device__ inline float tanh_clamped(float x) {
-    const float ax = fabsf(x);
-    if (x > 10.0f) return 1.0f;
-    if (x < -10.0f) return -1.0f;
-    if (ax < 0.2f) {
-        const float x2 = x * x;
-        return x * (1.0f - x2 * (1.0f / 3.0f - x2 * (2.0f / 15.0f - 17.0f / 315.0f * x2)));
-    }
-    return tanhf(x);
-}
-
 __device__ inline float sin_hybrid(float x) {
     if (fabsf(x) < 1.0e-3f) {
         const float c3 = -1.0f / 6.0f, c5 = 1.0f / 120.0f, c7 = -1.0f / 5040.0f, c9 = 1.0f / 362880.0f,

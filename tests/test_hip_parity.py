@@ -457,6 +457,53 @@ def test_float_unary_and_reduce_tolerance(run, oracle):
                                   oracle.mul(a, b, b.shape, abi.F16).view(np.uint16))
 
 
+def test_float_vectorised_paths_vs_oracle(run, oracle):
+    """Dense fp16/fp32 tensors whose last extent is a multiple of 8 take the 128-bit elementwise kernels and the
+    row-slab reduction: ADD/SUB/MUL/CAST and the sequential fp16 REDUCE_SUM/REDUCE_MAX are bit-exact against the
+    oracle (same fp32-then-round arithmetic, same left-to-right fold); transcendental unaries within 1e-2."""
+    rng = np.random.default_rng(18)
+    bits = lambda t: t.view(np.uint16) if t.dtype == np.float16 else t.view(np.uint32)
+    for dt, odt in ((np.float16, abi.F16), (np.float32, abi.F32)):
+        full = rng.standard_normal((3, 50, 200)).astype(dt)
+        other = rng.standard_normal((3, 50, 200)).astype(dt)
+        per_row = rng.standard_normal((3, 50, 1)).astype(dt)
+        per_col = rng.standard_normal((1, 1, 200)).astype(dt)
+        scalar = rng.standard_normal((1, 1, 1)).astype(dt)
+        for b in (other, per_row, per_col, scalar):
+            for op in ("ADD", "SUB"):
+                np.testing.assert_array_equal(bits(run.binary(op, full, b, full.shape, odt)),
+                                              bits(oracle.elementwise_binary(op, full, b, full.shape, odt)))
+                np.testing.assert_array_equal(bits(run.binary(op, b, full, full.shape, odt)),
+                                              bits(oracle.elementwise_binary(op, b, full, full.shape, odt)))
+            np.testing.assert_array_equal(bits(run.mul(full, b, full.shape, odt)), bits(oracle.mul(full, b, full.shape, odt)))
+        for op in ("EXP", "TANH"):
+            d = np.abs(run.unary(op, full).astype(np.float32) - oracle.elementwise_unary(op, full).astype(np.float32))
+            assert d.max() <= 1e-2, op
+        pos = np.abs(full) + dt(0.25)
+        for op in ("RECIPROCAL", "RSQRT"):
+            d = np.abs(run.unary(op, pos).astype(np.float32) - oracle.elementwise_unary(op, pos).astype(np.float32))
+            assert d.max() <= 1e-2, op
+    f32 = (rng.standard_normal((7, 33, 72)) * 300).astype(np.float32)
+    f32[0, 0, :4] = [1e6, -1e6, 65519.9, 6e-8]
+    np.testing.assert_array_equal(run.cast(f32, abi.F16).view(np.uint16), oracle.cast(f32, abi.F16).view(np.uint16))
+    f16 = rng.standard_normal((5, 40, 64)).astype(np.float16)
+    np.testing.assert_array_equal(run.cast(f16, abi.F32), oracle.cast(f16, abi.F32))
+    # sequential fp16 fold: rows that are not a multiple of 64, columns across several 64-column slabs
+    for shape in ((3, 50, 200), (2, 130, 768), (1, 64, 8), (4, 7, 512)):
+        x = rng.standard_normal(shape).astype(np.float16)
+        for op in ("SUM", "MAX"):
+            np.testing.assert_array_equal(run.reduce(op, x, 2).view(np.uint16), oracle.reduce(op, x, 2).view(np.uint16),
+                                          err_msg=f"{op} {shape}")
+    xn = rng.standard_normal((2, 9, 128)).astype(np.float16)
+    xn[0, 3, 77] = np.nan
+    xn[1, 0, 0] = np.nan
+    for op in ("SUM", "MAX"):
+        for mode in (abi.NAN_PROPAGATE, abi.NAN_IGNORE):
+            got, exp = run.reduce(op, xn, 2, mode), oracle.reduce(op, xn, 2, mode)
+            np.testing.assert_array_equal(np.isnan(got), np.isnan(exp), err_msg=f"{op} {mode}")
+            np.testing.assert_array_equal(got[~np.isnan(exp)].view(np.uint16), exp[~np.isnan(exp)].view(np.uint16))
+
+
 # ------------------------------------------------------------------------------------------------ error paths
 def test_error_conventions(run):
     x = np.zeros((1, 4, 4, 4), np.int8)
