@@ -297,6 +297,10 @@ int mlel_hip_transpose(mlel_ctx *ctx, void *stream, const mlel_tensor *out, cons
                  MLEL_ERR_INVALID, "transpose: bad arguments");
     for (int i = 0; i < out->rank; i++)
         MLEL_REQUIRE((int)perms[i] < out->rank, MLEL_ERR_INVALID, "transpose: perms[%d] = %u", i, perms[i]);
+    {
+        const int rc = try_transpose_fast(ctx, (hipStream_t)stream, out, in, perms);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return move_generic_launch((hipStream_t)stream, kTranspose, out, in, perms, 0, 0);
 }
 

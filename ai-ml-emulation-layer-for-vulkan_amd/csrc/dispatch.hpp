@@ -103,6 +103,8 @@ int try_binary_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out
                     const mlel_tensor *in2);
 int try_avgpool_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                      const mlel_pool2d_attr *a);
+int try_transpose_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                       const uint32_t *perms);
 int rescale_add_rescale_launch(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in1,
                                const FusedEpilogue &s1, const mlel_tensor *in2, const FusedEpilogue &s2,
                                const FusedEpilogue &so);

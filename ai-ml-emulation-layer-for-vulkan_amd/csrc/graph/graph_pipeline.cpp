@@ -611,6 +611,21 @@ void GraphPipeline::fuse() {
         ro.outputs[0]->setProducer(&add);
         ra->fusedAway = rb->fusedAway = ro.fusedAway = true;
     }
+
+    // Pattern 3: RESHAPE between two packed session tensors of the same byte size moves no data (the reference's
+    // reshape.comp:16-27 copies by flat index): the output becomes a second view of the input's storage and the
+    // operator is not executed.  plan() gives both tensors one allocation that lives as long as either is used.
+    for (const auto &opPtr : ops) {
+        OpNode &op = *opPtr;
+        if (op.fusedAway || op.kind != OpKind::Reshape) continue;
+        const auto &in = op.inputs[0];
+        const auto &out = op.outputs[0];
+        if (!isPrivateIntermediate(*in) || !isPrivateIntermediate(*out) || in->getSize() != out->getSize() ||
+            in->getShapeSize() != out->getShapeSize() || dtypeSize(in->getFormat()) != dtypeSize(out->getFormat()))
+            continue;
+        aliasOf[out.get()] = in.get();
+        op.fusedAway = true;
+    }
 }
 
 /*******************************************************************************
@@ -631,9 +646,13 @@ void GraphPipeline::plan() {
     std::map<const TensorDescriptor *, size_t> order;
     for (size_t i = 0; i < tensors.size(); i++) order[tensors[i].get()] = i;
     ranges.clear();
+    const auto root = [&](const TensorDescriptor *t) {
+        for (auto it = aliasOf.find(t); it != aliasOf.end(); it = aliasOf.find(t)) t = it->second;
+        return t;
+    };
     const auto touch = [&](const TensorPtr &t, uint32_t idx) {
         if (!t || order.find(t.get()) == order.end()) return;
-        auto [it, inserted] = ranges.emplace(t.get(), std::array<uint32_t, 2>{idx, idx});
+        auto [it, inserted] = ranges.emplace(root(t.get()), std::array<uint32_t, 2>{idx, idx});
         if (!inserted) {
             it->second[0] = std::min(it->second[0], idx);
             it->second[1] = std::max(it->second[1], idx);
@@ -676,6 +695,11 @@ void GraphPipeline::plan() {
     const auto planResult = details::allocateIntervals(std::move(intervals), unseen, kSessionAlignment);
     offsets.clear();
     for (const auto &[id, off] : planResult.offsets) offsets[tensors[id].get()] = static_cast<size_t>(off);
+    for (const auto &[view, target] : aliasOf) {  // views share the storage of the tensor they alias
+        (void)target;
+        const auto it = offsets.find(root(view));
+        if (it != offsets.end()) offsets[view] = it->second;
+    }
     sessionSize = static_cast<size_t>(planResult.memorySize);
 }
 

@@ -335,6 +335,7 @@ class GraphPipeline {
     std::vector<TensorPtr> inputs, outputs;
     std::map<const TensorDescriptor *, size_t> offsets;
     std::map<const TensorDescriptor *, std::array<uint32_t, 2>> ranges;
+    std::map<const TensorDescriptor *, const TensorDescriptor *> aliasOf;  // elided RESHAPE: output -> input
     size_t sessionSize = 0;
     bool finalized = false;
 

@@ -481,4 +481,143 @@ int try_avgpool_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const
     return 1;
 }
 
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------------------------
+// TRANSPOSE of dense tensors (transpose.comp:19-32: out[o] = in[i] with i[perms[k]] = o[k]).
+//   rows : the last axis stays last: whole rows are moved with 128-bit accesses;
+//   tiles: the last axis moves: 64 x 64 element tiles go through shared memory so that both the reads (along the
+//          input's last axis) and the writes (along the output's last axis) are contiguous.
+// ---------------------------------------------------------------------------------------------------------------
+struct TransposeArgs {
+    const char *in;
+    char *out;
+    int32_t rank;
+    int64_t odims[MLEL_MAX_RANK];     // output extents
+    int64_t istride[MLEL_MAX_RANK];   // byte stride of the input axis that feeds output axis k
+    int64_t ostride[MLEL_MAX_RANK];   // byte strides of the output
+    int64_t vecs;                     // rows kernel: 16-byte pieces in total
+    int32_t segs;                     // rows kernel: 16-byte pieces per row
+    int32_t q;                        // tiles kernel: output axis fed by the input's last axis
+    int64_t tiles_i, tiles_j, batches;
+};
+
+__global__ void __launch_bounds__(kBlock) transpose_rows_kernel(const TransposeArgs a) {
+    const int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (v >= a.vecs) return;
+    int64_t row = v / a.segs;
+    const int64_t seg = v - row * a.segs;
+    int64_t src = seg * 16;
+    for (int k = a.rank - 2; k >= 0; k--) {
+        const int64_t d = a.odims[k];
+        const int64_t o = row % d;
+        row /= d;
+        src += o * a.istride[k];
+    }
+    *reinterpret_cast<uint4 *>(a.out + v * 16) = *reinterpret_cast<const uint4 *>(a.in + src);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) transpose_tiles_kernel(const TransposeArgs a) {
+    __shared__ T tile[64][65];
+    int64_t b = blockIdx.x;
+    const int64_t tj = b % a.tiles_j;
+    b /= a.tiles_j;
+    const int64_t ti = b % a.tiles_i;
+    int64_t batch = b / a.tiles_i;
+    const int last = a.rank - 1;
+    int64_t src = 0, dst = 0;
+    for (int k = last - 1; k >= 0; k--) {  // the remaining output axes enumerate the batch
+        if (k == a.q) continue;
+        const int64_t d = a.odims[k];
+        const int64_t o = batch % d;
+        batch /= d;
+        src += o * a.istride[k];
+        dst += o * a.ostride[k];
+    }
+    const int64_t i0 = ti * 64, j0 = tj * 64;  // i: output axis q = input last axis; j: output last axis
+    const int lx = threadIdx.x & 63, ly = threadIdx.x >> 6;
+    for (int r = ly; r < 64; r += 4) {
+        const int64_t j = j0 + r, i = i0 + lx;
+        if (j < a.odims[last] && i < a.odims[a.q])
+            tile[r][lx] = *reinterpret_cast<const T *>(a.in + src + j * a.istride[last] + i * (int64_t)sizeof(T));
+    }
+    __syncthreads();
+    for (int r = ly; r < 64; r += 4) {
+        const int64_t i = i0 + r, j = j0 + lx;
+        if (i < a.odims[a.q] && j < a.odims[last])
+            *reinterpret_cast<T *>(a.out + dst + i * a.ostride[a.q] + j * (int64_t)sizeof(T)) = tile[lx][r];
+    }
+}
+
+}  // namespace
+
+int try_transpose_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                       const uint32_t *perms) {
+    (void)ctx;
+    const int rank = out->rank;
+    const int esize = dt_size(out->dtype);
+    if (rank < 2 || !is_packed(in) || !is_packed(out)) return 0;
+    uint32_t seen = 0;
+    for (int k = 0; k < rank; k++) {
+        if (perms[k] >= (uint32_t)rank || out->dims[k] != in->dims[perms[k]]) return 0;
+        seen |= 1u << perms[k];
+    }
+    if (seen != (1u << rank) - 1) return 0;
+    if (numel(out) <= 0) return 1;
+    TransposeArgs a{};
+    a.in = static_cast<const char *>(in->ptr);
+    a.out = static_cast<char *>(out->ptr);
+    a.rank = rank;
+    int64_t stride = esize;
+    for (int k = rank - 1; k >= 0; k--) {  // dense strides computed here (a packed tensor may carry any stride on
+        a.ostride[k] = stride;             // an axis of extent 1)
+        stride *= out->dims[k];
+    }
+    int64_t in_dense[MLEL_MAX_RANK];
+    stride = esize;
+    for (int k = rank - 1; k >= 0; k--) {
+        in_dense[k] = stride;
+        stride *= in->dims[k];
+    }
+    for (int k = 0; k < rank; k++) {
+        a.odims[k] = out->dims[k];
+        a.istride[k] = in_dense[perms[k]];
+    }
+    const int last = rank - 1;
+    if (perms[last] == (uint32_t)last) {
+        const int64_t row_bytes = out->dims[last] * esize;
+        if (row_bytes % 16 != 0 || ((uintptr_t)in->ptr % 16) != 0 || ((uintptr_t)out->ptr % 16) != 0) return 0;
+        if (row_bytes / 16 >= (int64_t(1) << 31)) return 0;
+        a.segs = (int32_t)(row_bytes / 16);
+        a.vecs = numel(out) * esize / 16;
+        const int64_t blocks = (a.vecs + kBlock - 1) / kBlock;
+        MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "transpose: too many work items");
+        transpose_rows_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(a);
+        MLEL_TRY(check_launch("transpose rows"));
+        return 1;
+    }
+    if (esize != 1 && esize != 2 && esize != 4) return 0;
+    if (((uintptr_t)in->ptr % esize) != 0 || ((uintptr_t)out->ptr % esize) != 0) return 0;
+    int q = -1;
+    for (int k = 0; k < rank; k++)
+        if (perms[k] == (uint32_t)last) q = k;
+    a.q = q;
+    a.tiles_i = (out->dims[q] + 63) / 64;
+    a.tiles_j = (out->dims[last] + 63) / 64;
+    a.batches = numel(out) / (out->dims[q] * out->dims[last]);
+    const int64_t blocks = a.tiles_i * a.tiles_j * a.batches;
+    MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "transpose: too many tiles");
+    const dim3 grid((unsigned)blocks), block(kBlock);
+    if (esize == 1)
+        transpose_tiles_kernel<uint8_t><<<grid, block, 0, s>>>(a);
+    else if (esize == 2)
+        transpose_tiles_kernel<uint16_t><<<grid, block, 0, s>>>(a);
+    else
+        transpose_tiles_kernel<uint32_t><<<grid, block, 0, s>>>(a);
+    MLEL_TRY(check_launch("transpose tiles"));
+    return 1;
+}
+
 }  // namespace mlel

@@ -195,67 +195,108 @@ namespace {
 // ---------------------------------------------------------------------------------------------------------------
 // REDUCE_SUM / REDUCE_MAX along the last axis of a dense fp16 tensor, with the reference's sequential semantics
 // (reduce.comp:24-70: a left-to-right fold in the storage type, so every partial sum is rounded to fp16).  Each
-// wavefront owns 64 rows: it copies a 64-row x 64-column slab into shared memory with coalesced 128-bit loads and
-// then every lane folds its own row out of shared memory, element by element in order.
+// block owns 64 rows: its four wavefronts copy a slab of 64 rows x up to 1024 columns into shared memory with coalesced
+// 128-bit loads and then the lanes of the first wavefront fold one row each out of shared memory, element by element.
 // ---------------------------------------------------------------------------------------------------------------
-constexpr int kSlabCols = 64;                 // halfs per row and slab
-constexpr int kSlabPitch = kSlabCols * 2 + 8;  // bytes: 8-byte aligned, rows 34 banks apart
+constexpr int kSlabMaxCols = 1024;  // halfs per row and slab: 64 rows x 1024 x 2 B = 128 KB of shared memory at most
 
 struct ReduceArgs {
     const char *in;
     char *out;
     int64_t rows;
-    int32_t cols;  // multiple of 8
+    int32_t cols;       // multiple of 8
+    int32_t slab_cols;  // min(cols, kSlabMaxCols), multiple of 8
     int32_t ignore_nan;
 };
 
 template <bool IS_SUM>
 __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArgs g) {
-    __shared__ __align__(16) char slab[4][64 * kSlabPitch];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    char *mine = slab[wave];
-    const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * 64;
-    const int64_t row = row0 + lane;
+    // A block owns 64 rows.  A fold is sequential along its row, so parallelism comes from rows only and small row
+    // counts (LayerNorm over a few thousand tokens) must still spread over many compute units; all four wavefronts
+    // fetch the slab (many loads in flight), then the first one folds it out of shared memory, one row per lane.
+    extern __shared__ __align__(16) char slab[];
+    const int pitch = g.slab_cols * 2 + 8;  // bytes; 8-byte aligned, consecutive rows two banks apart
+    const int tid = threadIdx.x;
+    const int64_t row0 = (int64_t)blockIdx.x * 64;
+    const int64_t row = row0 + tid;
     float r = IS_SUM ? 0.f : (g.ignore_nan ? NAN : -65504.f);
     bool done = false;
-    for (int c0 = 0; c0 < g.cols; c0 += kSlabCols) {
-        // 64 rows x 8 pieces of 16 bytes; lane handles pieces lane, lane + 64, ...: 8 rows of 128 bytes per load
+    for (int c0 = 0; c0 < g.cols; c0 += g.slab_cols) {
+        const int n = min(g.slab_cols, g.cols - c0);
+        const int segs = n >> 3;       // 16-byte pieces per row
+        const int pieces = 64 * segs;  // consecutive threads take consecutive pieces of a row
+        for (int p0 = 0; p0 < pieces; p0 += kBlock * 8) {
+            uint4 v[8];
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int p = i * 64 + lane;
-            const int rr = p >> 3, seg = p & 7;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (row0 + rr < g.rows && c0 + seg * 8 < g.cols)
-                v = *reinterpret_cast<const uint4 *>(g.in + ((row0 + rr) * g.cols + c0 + seg * 8) * 2);
-            *reinterpret_cast<uint2 *>(mine + rr * kSlabPitch + seg * 16) = make_uint2(v.x, v.y);
-            *reinterpret_cast<uint2 *>(mine + rr * kSlabPitch + seg * 16 + 8) = make_uint2(v.z, v.w);
+            for (int i = 0; i < 8; i++) {
+                const int p = p0 + i * kBlock + tid;
+                const int rr = p / segs, seg = p - rr * segs;
+                v[i] = make_uint4(0, 0, 0, 0);
+                if (p < pieces && row0 + rr < g.rows)
+                    v[i] = *reinterpret_cast<const uint4 *>(g.in + ((row0 + rr) * g.cols + c0 + seg * 8) * 2);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int p = p0 + i * kBlock + tid;
+                const int rr = p / segs, seg = p - rr * segs;
+                if (p < pieces) {
+                    *reinterpret_cast<uint2 *>(slab + rr * pitch + seg * 16) = make_uint2(v[i].x, v[i].y);
+                    *reinterpret_cast<uint2 *>(slab + rr * pitch + seg * 16 + 8) = make_uint2(v[i].z, v[i].w);
+                }
+            }
         }
         __syncthreads();
-        const int n = min(kSlabCols, g.cols - c0);
-        for (int j = 0; j < n; j += 4) {
-            const uint2 raw = *reinterpret_cast<const uint2 *>(mine + lane * kSlabPitch + j * 2);
-            const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
-            const float2 f01 = __half22float2(h[0]), f23 = __half22float2(h[1]);
-            const float e[4] = {f01.x, f01.y, f23.x, f23.y};
+        if (tid < 64) {
+            uint2 next = *reinterpret_cast<const uint2 *>(slab + tid * pitch);
+            for (int j = 0; j < n; j += 4) {
+                const uint2 raw = next;
+                if (j + 4 < n) next = *reinterpret_cast<const uint2 *>(slab + tid * pitch + (j + 4) * 2);
+                const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+                // a NaN among the four halfs: exponent all ones and a non-zero mantissa, tested on the packed pairs
+                const uint32_t nan_bits = (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu)) &
+                                          0x80008000u;
+                if (!__any(done || nan_bits != 0)) {
+                    // no lane of the wavefront is in a special state: the plain fold.  A native fp16 add rounds the
+                    // exact sum once; the generic kernel's fp32 add followed by a conversion gives the same value,
+                    // because the fp32 sum of two halfs is inexact only when the smaller one is far below half an ulp
+                    // of the larger.
+                    if (IS_SUM) {
+                        __half acc = __float2half_rn(r);
+                        acc = __hadd(acc, __low2half(h[0]));
+                        acc = __hadd(acc, __high2half(h[0]));
+                        acc = __hadd(acc, __low2half(h[1]));
+                        acc = __hadd(acc, __high2half(h[1]));
+                        r = __half2float(acc);
+                    } else {
+                        const float2 f01 = __half22float2(h[0]), f23 = __half22float2(h[1]);
+                        const float e[4] = {f01.x, f01.y, f23.x, f23.y};
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const float v = e[t];
-                if (done) continue;
-                if (isnan(v)) {
-                    if (g.ignore_nan) continue;
-                    r = v;
-                    done = true;
+                        for (int t = 0; t < 4; t++) r = isnan(r) ? e[t] : (r < e[t] ? e[t] : r);
+                    }
                     continue;
                 }
-                if (IS_SUM)
-                    r = rnd_f16(r + v);
-                else
-                    r = isnan(r) ? v : (r < v ? v : r);
+                const float2 f01 = __half22float2(h[0]), f23 = __half22float2(h[1]);
+                const float e[4] = {f01.x, f01.y, f23.x, f23.y};
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const float v = e[t];
+                    if (done) continue;
+                    if (isnan(v)) {
+                        if (g.ignore_nan) continue;
+                        r = v;
+                        done = true;
+                        continue;
+                    }
+                    if (IS_SUM)
+                        r = rnd_f16(r + v);
+                    else
+                        r = isnan(r) ? v : (r < v ? v : r);
+                }
             }
         }
         __syncthreads();
     }
-    if (row < g.rows) *reinterpret_cast<__half *>(g.out + row * 2) = __float2half_rn(r);
+    if (tid < 64 && row < g.rows) *reinterpret_cast<__half *>(g.out + row * 2) = __float2half_rn(r);
 }
 
 }  // namespace
@@ -279,12 +320,15 @@ int try_reduce_float_fast(mlel_ctx *, hipStream_t s, int op, const mlel_tensor *
     g.rows = rows;
     g.cols = (int32_t)cols;
     g.ignore_nan = nan_mode == MLEL_NAN_IGNORE ? 1 : 0;
-    const int64_t blocks = (rows + 255) / 256;
+    const int64_t blocks = (rows + 63) / 64;
     MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "reduce: too many rows");
-    if (op == MLEL_RED_SUM)
-        reduce_rows_f16_kernel<true><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(g);
-    else
-        reduce_rows_f16_kernel<false><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(g);
+    g.slab_cols = (int32_t)(cols < kSlabMaxCols ? cols : kSlabMaxCols);
+    const size_t smem = (size_t)64 * (g.slab_cols * 2 + 8);
+    auto kernel = op == MLEL_RED_SUM ? reduce_rows_f16_kernel<true> : reduce_rows_f16_kernel<false>;
+    if (smem > 48 * 1024)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)smem);
+    kernel<<<dim3((unsigned)blocks), dim3(kBlock), smem, s>>>(g);
     MLEL_TRY(check_launch("reduce rows fp16"));
     return 1;
 }

@@ -103,9 +103,13 @@ def test_mobilenetv2_graph_structure_and_plan():
     assert (full.macs["dense"] + full.macs["depthwise"]) // 32 == 300774272
     g = _build_host_only(spec, fuse=True)
     names = g.op_names()
-    assert len(names) == 35 + 17 + 10 + 3  # contractions, residual adds, pool + reshape + fc
+    # contractions, residual adds, pool + fc; the RESHAPE between two session tensors became a view of its input
+    assert len(names) == 35 + 17 + 10 + 2 and "RESHAPE" not in names
     assert names.count("RESCALE+RESCALE+ADD+RESCALE") == 10 and names[-1] == "MATMUL+RESCALE"
     planned = [t for t in g.session_tensors() if t["offset"] is not None]
+    views = [t for t in planned if t["first"] == 0xFFFFFFFF]
+    source = [t for t in planned if t["handle"] == views[0]["handle"] - 1]
+    assert len(views) == 1 and source[0]["offset"] == views[0]["offset"] and source[0]["size"] == views[0]["size"]
     total = sum((t["size"] + 255) // 256 * 256 for t in planned)
     size = gb.C.c_uint64()
     g._check(g.lib.mlel_graph_session_memory_requirements(g.g, gb.C.byref(size), None))

@@ -494,6 +494,9 @@ def test_float_vectorised_paths_vs_oracle(run, oracle):
         for op in ("SUM", "MAX"):
             np.testing.assert_array_equal(run.reduce(op, x, 2).view(np.uint16), oracle.reduce(op, x, 2).view(np.uint16),
                                           err_msg=f"{op} {shape}")
+    wide = rng.standard_normal((2, 3, 2056)).astype(np.float16)  # more than one 1024-column slab per row
+    for op in ("SUM", "MAX"):
+        np.testing.assert_array_equal(run.reduce(op, wide, 2).view(np.uint16), oracle.reduce(op, wide, 2).view(np.uint16))
     xn = rng.standard_normal((2, 9, 128)).astype(np.float16)
     xn[0, 3, 77] = np.nan
     xn[1, 0, 0] = np.nan
@@ -502,6 +505,20 @@ def test_float_vectorised_paths_vs_oracle(run, oracle):
             got, exp = run.reduce(op, xn, 2, mode), oracle.reduce(op, xn, 2, mode)
             np.testing.assert_array_equal(np.isnan(got), np.isnan(exp), err_msg=f"{op} {mode}")
             np.testing.assert_array_equal(got[~np.isnan(exp)].view(np.uint16), exp[~np.isnan(exp)].view(np.uint16))
+
+
+def test_transpose_fast_paths_vs_numpy(run, oracle):
+    """Dense transposes: whole-row moves when the last axis stays, 64x64 shared-memory tiles when it moves."""
+    rng = np.random.default_rng(19)
+    cases = [((2, 5, 12, 64), (0, 2, 1, 3), np.float16), ((2, 7, 3, 40), (0, 2, 3, 1), np.float16),
+             ((3, 70, 130), (0, 2, 1), np.int8), ((65, 67), (1, 0), np.int32), ((4, 33, 9), (2, 0, 1), np.float32),
+             ((2, 3, 4, 5, 16), (3, 1, 0, 2, 4), np.int16), ((6, 128, 64), (0, 2, 1), np.float16),
+             ((2, 16, 4, 8), (0, 2, 1, 3), np.int8), ((1, 1, 200), (2, 1, 0), np.int8)]
+    for shape, perms, dt in cases:
+        x = (rng.standard_normal(shape) * 50).astype(dt)
+        got = run.transpose(x, perms)
+        np.testing.assert_array_equal(got, np.transpose(x, perms), err_msg=f"{shape} {perms}")
+        np.testing.assert_array_equal(got, oracle.transpose(x, perms))
 
 
 # ------------------------------------------------------------------------------------------------ error paths
