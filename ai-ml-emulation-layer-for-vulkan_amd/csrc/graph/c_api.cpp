@@ -29,6 +29,7 @@
 #include "../../../include/mlel_graph.h"
 #include "graph_pipeline.hpp"
 #include "session_planner.hpp"
+#include "spirv_graph_loader.hpp"
 
 using namespace mlel::graph;
 
@@ -326,6 +327,39 @@ int mlel_graph_make_op(mlel_graph *g, const char *tosa_name, const int *inputs, 
         for (int i = 0; i < n_outputs; i++) a.out.push_back(handle(g, outputs[i]));
         it->second(g->pipeline, a);
         return 0;
+    });
+}
+
+int mlel_graph_load_spvasm(mlel_graph *g, const char *text, size_t length, const mlel_graph_spv_binding *bindings,
+                           int n_bindings, const mlel_graph_spv_constant *constants, int n_constants, uint32_t *io,
+                           int io_capacity, int *n_inputs, int *n_outputs) {
+    return guarded([&] {
+        if (!text) throw std::runtime_error("null SPIR-V text");
+        std::vector<SpvBinding> b;
+        for (int i = 0; i < n_bindings; i++)
+            b.push_back({bindings[i].set, bindings[i].binding, bindings[i].array_index, vec64(bindings[i].dims, bindings[i].rank)});
+        std::vector<SpvConstant> c;
+        for (int i = 0; i < n_constants; i++)
+            c.push_back({constants[i].id, constants[i].data, vec64(constants[i].dims, constants[i].rank)});
+        const SpvGraphInfo info = loadSpirvAssembly(g->pipeline, std::string(text, length), b, c);
+        const size_t total = info.inputs.size() + info.outputs.size();
+        if (io && static_cast<size_t>(io_capacity) < 3 * total) throw std::runtime_error("io array too small");
+        size_t k = 0;
+        for (const auto *list : {&info.inputs, &info.outputs})
+            for (const auto &key : *list)
+                for (int j = 0; j < 3 && io; j++) io[k++] = key[static_cast<size_t>(j)];
+        if (n_inputs) *n_inputs = static_cast<int>(info.inputs.size());
+        if (n_outputs) *n_outputs = static_cast<int>(info.outputs.size());
+        return static_cast<int>(info.instructions);
+    });
+}
+
+int mlel_graph_tensor_info(mlel_graph *g, int tensor, int32_t *dtype, int64_t *dims) {
+    return guarded([&] {
+        const TensorPtr t = handle(g, tensor);
+        if (dtype) *dtype = t->getFormat();
+        for (size_t i = 0; i < t->getDimensions().size() && dims; i++) dims[i] = t->getDimensions()[i];
+        return static_cast<int>(t->getRank());
     });
 }
 

@@ -18,6 +18,15 @@ _I64P = C.POINTER(C.c_int64)
 _V = C.c_void_p
 
 
+class SpvBinding(C.Structure):
+    _fields_ = [("set", C.c_uint32), ("binding", C.c_uint32), ("array_index", C.c_uint32), ("rank", C.c_int32),
+                ("dims", C.POINTER(C.c_int64))]
+
+
+class SpvConstant(C.Structure):
+    _fields_ = [("id", C.c_uint32), ("rank", C.c_int32), ("dims", C.POINTER(C.c_int64)), ("data", C.c_void_p)]
+
+
 def load_graph_library():
     global _glib
     if _glib is None:
@@ -40,6 +49,10 @@ def load_graph_library():
         lib.mlel_graph_make_output.argtypes = [_V, C.c_int]
         lib.mlel_graph_make_op.argtypes = [_V, C.c_char_p, C.POINTER(C.c_int), C.c_int, C.POINTER(C.c_int), C.c_int,
                                            _I64P, C.c_int, C.POINTER(C.c_double), C.c_int, C.c_char_p]
+        lib.mlel_graph_load_spvasm.argtypes = [_V, C.c_char_p, C.c_size_t, C.POINTER(SpvBinding), C.c_int,
+                                               C.POINTER(SpvConstant), C.c_int, C.POINTER(C.c_uint32), C.c_int,
+                                               C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        lib.mlel_graph_tensor_info.argtypes = [_V, C.c_int, C.POINTER(C.c_int32), _I64P]
         lib.mlel_graph_finalize.argtypes = [_V, C.c_int]
         lib.mlel_graph_session_memory_requirements.argtypes = [_V, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
         lib.mlel_graph_bind_session_memory.argtypes = [_V, _V]
@@ -153,6 +166,42 @@ class Graph:
         fa = (C.c_double * max(1, len(fattr)))(*[float(v) for v in fattr])
         self._check(self.lib.mlel_graph_make_op(self.g, tosa_name.encode(), ins, len(inputs), outs, len(outputs),
                                                 _i64(iattr), len(iattr), fa, len(fattr), debug_name.encode()))
+
+    # ---- SPIR-V assembly front-end
+    def load_spvasm(self, text, bindings=None, constants=None, names=None):
+        """Decodes a SPIR-V assembly module into this graph.  `bindings`: {(set, binding, element): shape} for
+        interface tensors of unshaped type; `constants`: {graph constant id: ndarray}; `names`: {(set, binding,
+        element): name} for the externals (default "s<set>b<binding>e<element>").  Returns (input names, output
+        names, number of TOSA instructions)."""
+        bindings, constants, names = bindings or {}, constants or {}, names or {}
+        keep = []
+        barr = (SpvBinding * max(1, len(bindings)))()
+        for i, ((s, b, e), shape) in enumerate(bindings.items()):
+            dims = _i64(shape)
+            keep.append(dims)
+            barr[i] = SpvBinding(s, b, e, len(shape), dims)
+        carr = (SpvConstant * max(1, len(constants)))()
+        for i, (cid, array) in enumerate(constants.items()):
+            array = np.ascontiguousarray(array)
+            dims = _i64(array.shape)
+            keep += [dims, array]
+            carr[i] = SpvConstant(cid, array.ndim, dims, array.ctypes.data)
+        io = (C.c_uint32 * 3072)()
+        n_in, n_out = C.c_int(), C.c_int()
+        raw = text.encode()
+        count = self._check(self.lib.mlel_graph_load_spvasm(self.g, raw, len(raw), barr, len(bindings), carr,
+                                                            len(constants), io, 3072, C.byref(n_in), C.byref(n_out)))
+        result = []
+        for k in range(n_in.value + n_out.value):
+            key = (int(io[3 * k]), int(io[3 * k + 1]), int(io[3 * k + 2]))
+            name = names.get(key, "s%db%de%d" % key)
+            h = self._check(self.lib.mlel_graph_get_tensor(self.g, *key))
+            dtype, dims = C.c_int32(), (C.c_int64 * 8)()
+            rank = self._check(self.lib.mlel_graph_tensor_info(self.g, h, C.byref(dtype), dims))
+            self.handles[name] = h
+            self.externals[name] = (key[0], key[1], key[2], int(dtype.value), tuple(int(dims[i]) for i in range(rank)), None)
+            result.append(name)
+        return result[:n_in.value], result[n_in.value:], count
 
     # ---- finalize / memory / run
     def finalize(self, fuse=True):

@@ -48,6 +48,31 @@ int mlel_graph_make_op(mlel_graph *g, const char *tosa_name, const int *inputs, 
                        int n_outputs, const int64_t *iattr, int n_iattr, const double *fattr, int n_fattr,
                        const char *debug_name);
 
+/* Front-end: a data graph written as SPIR-V assembly text (SPV_ARM_graph + SPV_ARM_tensors, "TOSA.001000.1"
+ * extended instructions) is decoded into make<Op> calls on `g` (reference: the layer's SPIR-V pass and
+ * GraphTosa10ExtInst::handleOp, graph/graph_tosa_1_0_ext_inst.cpp:37-1032; constants and tensor shapes that the
+ * reference takes from VkDataGraphPipelineConstantARM / VkTensorDescriptionARM, graph_layer.cpp:343-420, are the
+ * `constants` / `bindings` arguments).  `bindings` give the shape of every interface tensor whose SPIR-V type is
+ * unshaped; `constants` the payload of every OpGraphConstantARM.  On return io[0..3*n_in) holds {set, binding,
+ * array element} of the graph inputs in index order, followed by the same for the outputs.  Returns the number of
+ * TOSA instructions decoded. */
+typedef struct mlel_graph_spv_binding {
+    uint32_t set, binding, array_index;
+    int32_t rank;
+    const int64_t *dims;
+} mlel_graph_spv_binding;
+typedef struct mlel_graph_spv_constant {
+    uint32_t id;
+    int32_t rank;         /* 0 when the SPIR-V type is shaped */
+    const int64_t *dims;
+    const void *data;
+} mlel_graph_spv_constant;
+int mlel_graph_load_spvasm(mlel_graph *g, const char *text, size_t length, const mlel_graph_spv_binding *bindings,
+                           int n_bindings, const mlel_graph_spv_constant *constants, int n_constants, uint32_t *io,
+                           int io_capacity, int *n_inputs, int *n_outputs);
+/* dtype, rank and dimensions of a tensor handle (dims: room for MLEL_MAX_RANK entries); returns the rank. */
+int mlel_graph_tensor_info(mlel_graph *g, int tensor, int32_t *dtype, int64_t *dims);
+
 /* Fusion + session memory planning; then the session requirements
  * (reference: vkGetDataGraphPipelineSessionMemoryRequirementsARM, graph_layer.cpp:1382-1389). */
 int mlel_graph_finalize(mlel_graph *g, int enable_fusion);

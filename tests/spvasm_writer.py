@@ -1,0 +1,300 @@
+"""Test-side generator of SPIR-V assembly text for data graphs (SPV_ARM_graph + SPV_ARM_tensors, "TOSA.001000.1"
+extended instructions), written from the published extension grammar and the operand orders of the TOSA 1.0 instruction
+set.  It produces the modules the front-end tests feed to the loader: either built instruction by instruction
+(`SpvAsm`) or from a neutral graph description (`from_spec`).
+
+Conventions exercised on purpose, because the reference's own test modules use them (tests/shader/*.spvasm): integer
+types are declared unsigned (`OpTypeInt N 0`) although the data is signed, so negative values are written as their
+two's-complement unsigned literal; tensor shapes are `OpConstantComposite` of an `OpTypeArray` of uint; attributes are
+rank-1 tensor constants; zero points are one-element tensor constants.
+"""
+import importlib
+
+import numpy as np
+
+abi = importlib.import_module("ai-ml-emulation-layer-for-vulkan_amd.abi")
+
+_INT_BITS = {abi.I8: 8, abi.U8: 8, abi.I16: 16, abi.U16: 16, abi.I32: 32, abi.U32: 32, abi.I64: 64, abi.U64: 64}
+_FLOAT_BITS = {abi.F16: 16, abi.F32: 32, abi.F64: 64}
+
+
+class SpvAsm:
+    def __init__(self, entry="main"):
+        self.entry = entry
+        self.decorations, self.declarations, self.variables, self.body = [], [], [], []
+        self.cache = {}
+        self.interface_inputs, self.interface_outputs = [], []   # (variable id, tensor type id)
+        self.bindings = {}    # (set, binding, element) -> shape, for unshaped interface tensors
+        self.constants = {}   # graph constant id -> ndarray
+        self.names = {}       # (set, binding, element) -> name
+        self.next_binding = 0
+        self.next_value = 0
+
+    # ---- declarations, cached by content
+    def _declare(self, key, name, text):
+        if key not in self.cache:
+            self.declarations.append(f"{name} = {text}")
+            self.cache[key] = name
+        return self.cache[key]
+
+    def scalar_type(self, dtype):
+        if dtype == abi.BOOL:
+            return self._declare(("type", dtype), "%bool", "OpTypeBool")
+        if dtype in _INT_BITS:
+            bits = _INT_BITS[dtype]
+            return self._declare(("type", bits, "int"), f"%uint{bits}", f"OpTypeInt {bits} 0")
+        if dtype == abi.BF16:
+            return self._declare(("type", dtype), "%bfloat16", "OpTypeFloat 16 BFloat16KHR")
+        bits = _FLOAT_BITS[dtype]
+        return self._declare(("type", bits, "float"), f"%float{bits}", f"OpTypeFloat {bits}")
+
+    def scalar(self, dtype, value):
+        t = self.scalar_type(dtype)
+        if dtype == abi.BOOL:
+            return self._declare(("const", dtype, bool(value)), "%true" if value else "%false",
+                                 f"OpConstant{'True' if value else 'False'} {t}")
+        if dtype in _INT_BITS:
+            bits = _INT_BITS[dtype]
+            literal = int(value) & ((1 << bits) - 1)
+            return self._declare(("const", bits, literal), f"%uint{bits}_{literal}", f"OpConstant {t} {literal}")
+        v = float(value)
+        tag = np.float64(v).view(np.uint64)
+        return self._declare(("const", dtype, int(tag)), f"%{t[1:]}_{int(tag):x}", f"OpConstant {t} {v!r}")
+
+    def u32(self, value):
+        return self.scalar(abi.U32, value)
+
+    def shape(self, dims):
+        n = len(dims)
+        array = self._declare(("array", n), f"%array_uint_{n}", f"OpTypeArray {self.scalar_type(abi.U32)} {self.u32(n)}")
+        members = " ".join(self.u32(d) for d in dims)
+        return self._declare(("shape", tuple(dims)), "%shape_" + "_".join(str(d) for d in dims),
+                             f"OpConstantComposite {array} {members}")
+
+    def tensor_type(self, dtype, dims=None, rank=None):
+        elem = self.scalar_type(dtype)
+        if dims is None:
+            return self._declare(("tensor", dtype, rank), f"%tensor_{elem[1:]}_rank{rank}",
+                                 f"OpTypeTensorARM {elem} {self.u32(rank)}")
+        dims = tuple(int(d) for d in dims)
+        name = f"%tensor_{elem[1:]}_" + "x".join(str(d) for d in dims)
+        return self._declare(("tensor", dtype, dims), name,
+                             f"OpTypeTensorARM {elem} {self.u32(len(dims))} {self.shape(dims)}")
+
+    # ---- constants
+    def _fresh(self, prefix):
+        self.next_value += 1
+        return f"%{prefix}_{self.next_value}"
+
+    def const(self, array, dtype=None, graph_constant=None, replicate=False):
+        """A tensor constant: nested OpConstantComposite (one level per rank), a replicated composite when every
+        element is equal and `replicate` is set, or an OpGraphConstantARM whose data travels beside the module."""
+        array = np.asarray(array)
+        if dtype is None:
+            dtype = abi.dtype_of_numpy(array.dtype)
+        if array.ndim == 0:
+            array = array.reshape(1)
+        t = self.tensor_type(dtype, array.shape)
+        if graph_constant is not None:
+            self.constants[graph_constant] = np.ascontiguousarray(array)
+            name = self._fresh("graph_constant")
+            self.declarations.append(f"{name} = OpGraphConstantARM {t} {graph_constant}")
+            return name
+        if replicate and array.size > 1 and np.all(array == array.flat[0]):
+            if not np.any(array):
+                return self._declare(("null", t), f"%null_{t[1:]}", f"OpConstantNull {t}")
+            key = ("replicate", t, array.flat[0].tobytes())
+            return self._declare(key, self._fresh("splat"),
+                                 f"OpConstantCompositeReplicateEXT {t} {self.scalar(dtype, array.flat[0])}")
+        if array.ndim == 1:
+            members = [self.scalar(dtype, v) for v in array]
+        else:
+            members = [self.const(sub, dtype) for sub in array]
+        key = ("composite", t, array.tobytes())
+        if key in self.cache:
+            return self.cache[key]
+        return self._declare(key, self._fresh("const"), f"OpConstantComposite {t} {' '.join(members)}")
+
+    def attr(self, values, dtype=abi.I32):
+        return self.const(np.asarray(values, dtype=abi.NP_OF[dtype]).reshape(-1), dtype)
+
+    # ---- interface
+    def _variable(self, name, dtype, shape, shaped, set_, binding):
+        if binding is None:
+            binding = self.next_binding
+        self.next_binding = max(self.next_binding, binding + 1)
+        t = self.tensor_type(dtype, shape) if shaped else self.tensor_type(dtype, rank=len(shape))
+        ptr = self._declare(("pointer", t), f"%ptr_{t[1:]}", f"OpTypePointer UniformConstant {t}")
+        var = f"%{name}_var"
+        self.variables.append(f"{var} = OpVariable {ptr} UniformConstant")
+        self.decorations += [f"OpDecorate {var} DescriptorSet {set_}", f"OpDecorate {var} Binding {binding}"]
+        key = (set_, binding, 0)
+        self.names[key] = name
+        if not shaped:
+            self.bindings[key] = tuple(int(d) for d in shape)
+        return var, t
+
+    def input(self, name, dtype, shape, shaped=True, set_=0, binding=None):
+        var, t = self._variable(name, dtype, shape, shaped, set_, binding)
+        index = len(self.interface_inputs)
+        self.interface_inputs.append((var, t))
+        value = f"%{name}"
+        self.body.append(f"{value} = OpGraphInputARM {t} {self.u32(index)}")
+        return value
+
+    def output(self, name, dtype, shape, shaped=True, set_=0, binding=None):
+        """Declares an output; returns its index for set_output()."""
+        var, t = self._variable(name, dtype, shape, shaped, set_, binding)
+        self.interface_outputs.append((var, t))
+        return len(self.interface_outputs) - 1
+
+    def tensor_array(self, name, dtype, shapes, as_input, set_=0, binding=None, used=None):
+        """One variable holding an array of tensors (unshaped element type; per-element shapes in `bindings`).
+        Returns {element: value id} for the `used` elements (inputs) or (output index, element) pairs."""
+        if binding is None:
+            binding = self.next_binding
+        self.next_binding = max(self.next_binding, binding + 1)
+        rank = len(shapes[0])
+        t = self.tensor_type(dtype, rank=rank)
+        n = len(shapes)
+        arr = self._declare(("tensor_array", t, n), f"%array_{t[1:]}_{n}", f"OpTypeArray {t} {self.u32(n)}")
+        ptr = self._declare(("pointer", arr), f"%ptr_{arr[1:]}", f"OpTypePointer UniformConstant {arr}")
+        var = f"%{name}_var"
+        self.variables.append(f"{var} = OpVariable {ptr} UniformConstant")
+        self.decorations += [f"OpDecorate {var} DescriptorSet {set_}", f"OpDecorate {var} Binding {binding}"]
+        for e, shape in enumerate(shapes):
+            self.names[(set_, binding, e)] = f"{name}{e}"
+            self.bindings[(set_, binding, e)] = tuple(int(d) for d in shape)
+        if as_input:
+            index = len(self.interface_inputs)
+            self.interface_inputs.append((var, arr))
+            values = {}
+            for e in (range(n) if used is None else used):
+                values[e] = f"%{name}{e}"
+                self.body.append(f"{values[e]} = OpGraphInputARM {t} {self.u32(index)} {self.u32(e)}")
+            return values
+        self.interface_outputs.append((var, arr))
+        return [(len(self.interface_outputs) - 1, e) for e in range(n)]
+
+    # ---- graph body
+    def op(self, tosa_name, dtype, shape, operands, shaped=True, name=None):
+        t = self.tensor_type(dtype, shape) if shaped else self.tensor_type(dtype, rank=len(shape))
+        value = f"%{name}" if name else self._fresh(tosa_name.lower())
+        self.body.append(f"{value} = OpExtInst {t} %tosa {tosa_name} {' '.join(operands)}")
+        return value
+
+    def set_output(self, value, index, element=None):
+        extra = f" {self.u32(element)}" if element is not None else ""
+        self.body.append(f"OpGraphSetOutputARM {value} {self.u32(index)}{extra}")
+
+    def text(self):
+        interface = self.interface_inputs + self.interface_outputs
+        graph_type = "%graph_type = OpTypeGraphARM {} {}".format(len(self.interface_inputs),
+                                                                 " ".join(t for _, t in interface))
+        lines = ["; generated by tests/spvasm_writer.py",
+                 "OpCapability Shader", "OpCapability VulkanMemoryModel", "OpCapability Int8", "OpCapability Int16",
+                 "OpCapability Int64", "OpCapability Float16", "OpCapability GraphARM", "OpCapability TensorsARM",
+                 'OpExtension "SPV_ARM_graph"', 'OpExtension "SPV_ARM_tensors"',
+                 'OpExtension "SPV_KHR_vulkan_memory_model"', 'OpExtension "SPV_EXT_replicated_composites"',
+                 '%tosa = OpExtInstImport "TOSA.001000.1"', "OpMemoryModel Logical Vulkan"]
+        lines += self.decorations + self.declarations + [graph_type] + self.variables
+        lines.append('OpGraphEntryPointARM %graph "{}" {}'.format(self.entry, " ".join(v for v, _ in interface)))
+        lines.append("%graph = OpGraphARM %graph_type")
+        lines += self.body + ["OpGraphEndARM"]
+        return "\n".join(lines) + "\n"
+
+
+def from_spec(spec, inline_limit=64, shaped_io=True, entry="main"):
+    """Writes a graph description (ai-ml-emulation-layer-for-vulkan_amd.graphs.Spec) as a module.  Constants of up to `inline_limit`
+    elements are inlined as composites, larger ones become graph constants.  Returns the SpvAsm (text(), bindings,
+    constants, names)."""
+    w = SpvAsm(entry)
+    values, dtypes = {}, {}
+    for name, dtype, shape in spec.inputs:
+        values[name] = w.input(name, dtype, shape, shaped=shaped_io)
+        dtypes[name] = dtype
+    out_index = {}
+    for name, dtype, shape in spec.outputs:
+        out_index[name] = w.output(name, dtype, shape, shaped=shaped_io)
+        dtypes[name] = dtype
+    next_constant = [0]
+
+    def operand(name):
+        if name in values:
+            return values[name]
+        array = spec.consts[name]
+        dtypes[name] = abi.dtype_of_numpy(array.dtype)
+        if array.size <= inline_limit:
+            values[name] = w.const(array, replicate=True)
+        else:
+            values[name] = w.const(array, graph_constant=next_constant[0])
+            next_constant[0] += 1
+        return values[name]
+
+    def type_of(name):
+        if name in spec.tensors:
+            return spec.tensors[name]
+        for n, dtype, shape in spec.outputs:
+            if n == name:
+                return dtype, shape
+        raise KeyError(name)
+
+    def dtype_of(name):
+        if name in spec.tensors:
+            return spec.tensors[name][0]
+        if name in spec.consts:
+            return abi.dtype_of_numpy(spec.consts[name].dtype)
+        return dtypes[name]
+
+    for op in spec.ops:
+        kind, ins, ia, fa = op["op"], op["in"], op["iattr"], op["fattr"]
+        out = op["out"][0]
+        out_dtype, out_shape = type_of(out)
+        x = [operand(n) for n in ins]
+        in_dtype = dtype_of(ins[0])
+        zp_dtype = in_dtype if in_dtype in (abi.F16, abi.F32, abi.BF16) else abi.I8
+        if kind in ("CONV2D", "DEPTHWISE_CONV2D"):
+            operands = [w.attr(ia[0:4]), w.attr(ia[4:6]), w.attr(ia[6:8]), w.u32(ia[10]), w.scalar(abi.BOOL, False),
+                        x[0], x[1], x[2], w.attr([ia[8]], zp_dtype), w.attr([ia[9]], zp_dtype)]
+        elif kind == "MATMUL":
+            operands = [x[0], x[1], w.attr([ia[0]], zp_dtype), w.attr([ia[1]], zp_dtype)]
+        elif kind == "RESCALE":
+            operands = [w.scalar(abi.BOOL, ia[2]), w.u32(3 if ia[3] else 1), w.scalar(abi.BOOL, ia[4]),
+                        w.scalar(abi.BOOL, ia[5]), w.scalar(abi.BOOL, ia[6]), x[0], x[1], x[2],
+                        w.attr([ia[0]], in_dtype), w.attr([ia[1]], out_dtype)]
+        elif kind == "CLAMP":
+            lo, hi = (fa[0], fa[1]) if in_dtype in _FLOAT_BITS else (int(fa[0]), int(fa[1]))
+            operands = [w.scalar(in_dtype, lo), w.scalar(in_dtype, hi), w.u32(ia[0]), x[0]]
+        elif kind == "AVG_POOL2D":
+            operands = [w.attr(ia[0:2]), w.attr(ia[2:4]), w.attr(ia[4:8]), w.u32(ia[8]), x[0],
+                        w.attr([ia[9]], zp_dtype), w.attr([ia[10]], zp_dtype)]
+        elif kind == "MAX_POOL2D":
+            operands = [w.attr(ia[0:2]), w.attr(ia[2:4]), w.attr(ia[4:8]), w.u32(ia[8]), x[0]]
+        elif kind in ("MAXIMUM", "MINIMUM"):
+            operands = [w.u32(ia[0]), x[0], x[1]]
+        elif kind == "MUL":
+            operands = [x[0], x[1], w.attr([ia[0] if ia else 0], abi.I8)]
+        elif kind in ("REDUCE_MAX", "REDUCE_MIN"):
+            operands = [w.u32(ia[0]), w.u32(ia[1]), x[0]]
+        elif kind.startswith("REDUCE_"):
+            operands = [w.u32(ia[0]), x[0]]
+        elif kind == "NEGATE":
+            operands = [x[0], w.attr([ia[0]], in_dtype), w.attr([ia[1]], out_dtype)]
+        elif kind == "CONCAT":
+            operands = [w.u32(ia[0])] + x
+        elif kind == "SLICE":
+            operands = [x[0], w.attr(ia), w.attr(out_shape)]
+        elif kind == "TRANSPOSE":
+            operands = [w.attr(ia), x[0]]
+        elif kind == "RESHAPE":
+            operands = [x[0], w.attr(out_shape)]
+        elif kind == "PAD":
+            pad_const = fa[0] if in_dtype in _FLOAT_BITS else ia[0]
+            operands = [x[0], x[1], w.attr([pad_const], in_dtype)]
+        else:  # TABLE, element-wise binary / unary, CAST: tensors only
+            operands = x
+        values[out] = w.op(kind, out_dtype, out_shape, operands, shaped=(out not in out_index or shaped_io),
+                           name=None)
+        if out in out_index:
+            w.set_output(values[out], out_index[out])
+    return w
