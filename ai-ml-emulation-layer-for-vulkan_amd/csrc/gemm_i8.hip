@@ -48,10 +48,24 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
     };
     const Tile tall = BN == 128 ? Tile{0, 128} : (BN == 64 ? Tile{1, 256} : Tile{2, 256});
     const Tile low = BN == 128 ? Tile{3, 64} : (BN == 64 ? Tile{4, 64} : Tile{5, 128});
-    const int64_t tiles_n = (g.N + BN - 1) / BN;
+    int64_t tiles_n = (g.N + BN - 1) / BN;
     const int64_t tall_total = (int64_t)((g.M + tall.bm - 1) / tall.bm) * tiles_n * g.batches;
     const int cus = ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
-    const Tile tile = tall_total >= 2 * (int64_t)cus ? tall : low;
+    Tile tile = tall_total >= 2 * (int64_t)cus ? tall : low;
+    // Direct-to-LDS pipeline (dense 16-byte aligned rows on both sides or a K-major W, K in whole 64-byte steps):
+    // the 256 x 256 tile when that still gives every compute unit a block, else the 128 x 128 tile under the same
+    // condition as the tall tiles above.  Smaller problems keep the short tiles of the register-staged pipeline.
+    const bool dl_ok = xmode == X_PLAIN && (wmode == W_ROWS || wmode == W_KMAJOR) && g.K % BK == 0 && BN == 128;
+    if (dl_ok) {
+        const int64_t total256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * g.batches;
+        const bool big = total256 >= cus, mid = tall_total >= 2 * (int64_t)cus;
+        if (big || mid) {
+            tile = big ? Tile{6, 256} : Tile{0, 128};
+            xmode = X_PLAIN_DL;
+            wmode = wmode == W_ROWS ? W_ROWS_DL : W_KMAJOR_DL;
+        }
+    }
+    if (tile.id == 6) tiles_n = (g.N + 255) / 256;
     g.tiles_m = (g.M + tile.bm - 1) / tile.bm;
     g.tiles_n = (int)tiles_n;
     const int64_t total = (int64_t)g.tiles_m * g.tiles_n * g.batches;
@@ -65,6 +79,7 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
     case 2: launch_gemm_tile2(&g, xmode, wmode, grid, s); break;
     case 3: launch_gemm_tile3(&g, xmode, wmode, grid, s); break;
     case 4: launch_gemm_tile4(&g, xmode, wmode, grid, s); break;
+    case 6: launch_gemm_tile6(&g, xmode, wmode, grid, s); break;
     default: launch_gemm_tile5(&g, xmode, wmode, grid, s); break;
     }
     return check_launch("int8 contraction");

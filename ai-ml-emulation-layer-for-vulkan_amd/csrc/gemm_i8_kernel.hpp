@@ -21,6 +21,9 @@
 #pragma once
 
 #include "common.hpp"
+#include <mutex>
+#include <unordered_set>
+
 #include "dispatch.hpp"
 
 namespace mlel {
@@ -32,6 +35,7 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) v2i lds_v2i;
 
 constexpr int BK = 64;            // bytes of K per step
+constexpr int kGroupM = 8;        // tile rows per band of the tile walk
 constexpr int PITCH = BK + 16;    // LDS row pitch: 80 B keeps 16-lane groups of 128-bit reads on distinct banks
 
 struct GemmArgs {
@@ -221,6 +225,7 @@ enum XMode {
     X_TAP = 1,      // 16-byte pieces, IC % 64 == 0: one K step lies inside one filter tap (uniform tap state)
     X_GENERIC = 2,  // anything else: per-piece tap tracking, 16 / 4 / 1-byte loads
     X_PLAIN4 = 3,   // as X_PLAIN for rows that are only dword aligned (K % 4 == 0): four dword loads per piece
+    X_PLAIN_DL = 4, // as X_PLAIN with K % 16 == 0, fetched straight into LDS (no register staging), deep stage ring
 };
 enum WMode {
     W_ROWS = 0,     // [N][K], 16-byte pieces
@@ -228,7 +233,39 @@ enum WMode {
     W_GENERIC = 2,  // either layout, any alignment
     W_KMAJOR4 = 3,  // as W_KMAJOR for rows that are only dword aligned (N % 4 == 0): four dword loads per piece
     W_ROWS4 = 4,    // as W_ROWS for rows that are only dword aligned (K % 4 == 0)
+    W_ROWS_DL = 5,  // as W_ROWS, fetched straight into LDS (paired with X_PLAIN_DL)
+    W_KMAJOR_DL = 6,  // as W_KMAJOR, fetched straight into LDS (paired with X_PLAIN_DL)
 };
+
+// Direct-to-LDS pipeline (X_PLAIN_DL): `buffer_load_dwordx4 ... lds` writes lane l's 16 bytes at base + 16 l, so a
+// wavefront instruction fills 1 KiB of LDS and which global piece lands in which 16-byte slot is the lane's choice.
+// Tiles are stored unpadded ([rows][64] for row operands, [64][BN] for the K-major operand) with the pieces
+// XOR-swizzled so that the 128-bit / transposing 64-bit operand reads stay free of bank conflicts:
+//   row operand:  piece p (0..3) of row r sits in slot p ^ ((r >> 2) & 3) of the row;
+//   K-major:      the 32-byte unit u of K row k sits in unit u ^ ((k / (256 / BN)) % (BN / 32)).
+// STAGES K steps are resident; one barrier per step.
+template <int BM, int BN>
+constexpr int dl_stages() {
+    return 4;
+}
+// One wavefront-wide 16-byte-per-lane load from a buffer resource straight into LDS at `lds_addr` + 16 * lane.
+// Written as inline assembly on purpose: the compiler orders every LDS read after ALL outstanding loads of this kind
+// (it cannot tell which bytes they write), which would drain the whole stage ring at every step; the loop below does
+// its own counting with s_waitcnt vmcnt(N).  M0 holds the LDS address for this one instruction only; nothing else
+// in these kernels keeps a value in M0.
+__device__ __forceinline__ void load16_to_lds(v4i rsrc, uint32_t lds_addr, uint32_t offset, uint32_t scalar_offset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(offset),
+                 "s"(rsrc), "s"(scalar_offset)
+                 : "memory");
+}
+__device__ __forceinline__ v4i make_rsrc_words(const void *p, uint32_t bytes) {
+    const uint64_t a = reinterpret_cast<uint64_t>(p);
+    return v4i{(int)(uint32_t)a, (int)(uint32_t)(a >> 32), (int)bytes, 0x00020000};
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N) only (expcnt / lgkmcnt untouched)
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int XMODE, int WMODE, bool SUMS, bool Q8>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const GemmArgs g) {
@@ -246,9 +283,13 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     constexpr int N16 = BN / 16;          // 16-byte pieces per K row of the K-major tile
 
     extern __shared__ __align__(16) char smem[];
+    constexpr bool DL = XMODE == X_PLAIN_DL;
+    static_assert(DL == (WMODE == W_ROWS_DL || WMODE == W_KMAJOR_DL), "the direct-to-LDS modes come as a pair");
+    constexpr int DL_S = dl_stages<BM, BN>();
+    constexpr int DL_STAGE = (BM + BN) * BK;  // one stage: X tile [BM][64] then W tile
     char *xs = smem;                     // [2][BM][PITCH]
     char *ws = smem + 2 * BM * PITCH;    // [2][WBUF]
-    ChanParams *cp = reinterpret_cast<ChanParams *>(smem + 2 * BM * PITCH + 2 * WBUF);  // [BN]
+    ChanParams *cp = reinterpret_cast<ChanParams *>(smem + (DL ? DL_S * DL_STAGE : 2 * BM * PITCH + 2 * WBUF));  // [BN]
 
     // ---- XCD-aware tile assignment: consecutive block ids land on different XCDs (8 of them, each with its own
     // L2), so block b is given tile (b % 8) * chunk + b / 8: tiles that share operands stay on one XCD.
@@ -259,8 +300,21 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     // that everything derived from them (base pointers, buffer resources) is scalar as well
     const int batch = __builtin_amdgcn_readfirstlane(lin / tiles_per_batch);
     const int t_in = lin - batch * tiles_per_batch;
-    const int tile_m = __builtin_amdgcn_readfirstlane(t_in / g.tiles_n);
-    const int tile_n = t_in - tile_m * g.tiles_n;
+    // Tiles are walked in bands of GROUP_M tile rows, column by column inside a band: the blocks that run at the
+    // same time on one XCD then share a few row panels of X and a few column panels of W in its L2, instead of one
+    // row panel and every column panel.
+    int tile_m, tile_n;
+    if (g.tiles_m >= 2 * kGroupM) {
+        const int band = __builtin_amdgcn_readfirstlane(t_in / (kGroupM * g.tiles_n));
+        const int first = band * kGroupM;
+        const int rows = min(kGroupM, g.tiles_m - first);
+        const int r = t_in - band * kGroupM * g.tiles_n;
+        tile_n = __builtin_amdgcn_readfirstlane(r / rows);
+        tile_m = first + r - tile_n * rows;
+    } else {
+        tile_m = __builtin_amdgcn_readfirstlane(t_in / g.tiles_n);
+        tile_n = t_in - tile_m * g.tiles_n;
+    }
     const int m_base = tile_m * BM, n_base = tile_n * BN;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -515,6 +569,181 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         }
     };
 
+    if constexpr (DL) {
+        // ---- direct-to-LDS main loop (K % 64 == 0).  The matrix-core instructions and the ordinary vector
+        // instructions of a wavefront share one issue stream, so everything that is not a multiply is kept out of
+        // the loop: the K advance of the fetches rides in the scalar offset of the buffer instruction, the stage
+        // ring is unrolled so that LDS addresses are lane base + immediate, and the zero-point sums of a K half are
+        // taken by one wavefront only (combined through LDS after the loop).
+        constexpr int XI = BM * 4 / NTHREADS, WI = BN * 4 / NTHREADS;  // 16-byte pieces per thread and stage
+        static_assert((BN * 4) % NTHREADS == 0 && BN % 32 == 0 && BN <= 256, "whole W pieces per thread");
+        static_assert(DL_S == 4 && WAVES_M == 2 && WAVES_N >= 2, "ring of four stages, 2 x N wavefronts");
+        constexpr int P16 = BN / 16, UN = BN / 32, RP = 256 / BN;  // K-major: pieces / units per row, rows per 256 B
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        uint32_t xo[XI], wo[WI];
+#pragma unroll
+        for (int i = 0; i < XI; i++) {
+            const int q = i * NTHREADS + tid, r = q >> 2, p = (q & 3) ^ ((r >> 2) & 3);
+            const int m = m_base + r;
+            xo[i] = m < g.M ? (uint32_t)m * (uint32_t)g.x_sx + (uint32_t)(p * 16) : kOobOffset;
+        }
+#pragma unroll
+        for (int i = 0; i < WI; i++) {
+            const int q = i * NTHREADS + tid;
+            if (WMODE == W_ROWS_DL) {
+                const int r = q >> 2, p = (q & 3) ^ ((r >> 2) & 3);
+                const int n = n_base + r;
+                wo[i] = n < g.N ? (uint32_t)n * (uint32_t)g.ldw + (uint32_t)(p * 16) : kOobOffset;
+            } else {
+                const int kr = q / P16, c = q % P16;
+                const int u = (c >> 1) ^ ((kr / RP) % UN);
+                const int n = n_base + u * 32 + (c & 1) * 16;
+                wo[i] = n < g.N ? (uint32_t)kr * (uint32_t)g.ldw + (uint32_t)n : kOobOffset;
+            }
+        }
+        const v4i xres4 = make_rsrc_words(xb, g.x_bytes), wres4 = make_rsrc_words(wb, g.w_bytes);
+        const uint32_t lds0 = (uint32_t) reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char *)smem) +
+                              (uint32_t)(wave_u * 1024);
+        const uint32_t w_kstep = WMODE == W_ROWS_DL ? (uint32_t)BK : (uint32_t)BK * (uint32_t)g.ldw;
+        auto issue = [&](int buf, int step) {  // `step` is wave-uniform: the K advance is a scalar offset
+            const uint32_t xd = lds0 + (uint32_t)(buf * DL_STAGE), wd = xd + BM * BK;
+            const uint32_t xk = (uint32_t)step * BK, wk = (uint32_t)step * w_kstep;
+#pragma unroll
+            for (int i = 0; i < XI; i++) load16_to_lds(xres4, xd + i * NTHREADS * 16, xo[i], xk);
+#pragma unroll
+            for (int i = 0; i < WI; i++) load16_to_lds(wres4, wd + i * NTHREADS * 16, wo[i], wk);
+        };
+        // operand addresses inside a stage: lane base (per K half) + compile-time offset
+        const int h = lane >> 5;
+        const int xswz = ((lane >> 2) & 3);
+        const int kfun = WMODE == W_KMAJOR_DL ? (((lane & 15) >> 1) / RP) % UN : 0;
+        const char *x_base[2], *w_base[2];
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            const int slot = ((kk * 2 + h) ^ xswz) * 16;
+            x_base[kk] = smem + (wave_m * WM + (lane & 31)) * BK + slot;
+            if (WMODE == W_KMAJOR_DL)
+                w_base[kk] = smem + BM * BK + (kk * 32 + h * 16 + ((lane & 15) >> 1)) * BN + ((lane >> 4) & 1) * 16 +
+                             (lane & 1) * 8;
+            else
+                w_base[kk] = smem + BM * BK + (wave_n * WN + (lane & 31)) * BK + slot;
+        }
+        auto read_frags = [&](int buf, int kk, v4i(&xf)[TM], v4i(&wf)[TN]) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                xf[i] = *reinterpret_cast<const v4i *>(x_base[kk] + buf * DL_STAGE + i * 32 * BK);
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                if (WMODE == W_KMAJOR_DL) {
+                    const char *p = w_base[kk] + buf * DL_STAGE + (((wave_n * WN / 32 + j) ^ kfun) * 32);
+                    const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(p));
+                    const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(p + 8 * BN));
+                    wf[j] = v4i{lo.x, lo.y, hi.x, hi.y};
+                } else {
+                    wf[j] = *reinterpret_cast<const v4i *>(w_base[kk] + buf * DL_STAGE + j * 32 * BK);
+                }
+            }
+        };
+        // zero-point sums: K half kk of the X rows is summed by the wavefront column kk, of the W channels by the
+        // wavefront row kk (every row / channel group is owned by exactly one such wavefront)
+        const int wave_n_u = __builtin_amdgcn_readfirstlane(wave_n), wave_m_u = __builtin_amdgcn_readfirstlane(wave_m);
+        const bool xs0 = need_xsum && wave_n_u == 0, xs1 = need_xsum && wave_n_u == 1;
+        const bool ws0 = need_wsum && wave_m_u == 0, ws1 = need_wsum && wave_m_u == 1;
+        auto multiply = [&](const v4i(&xf)[TM], const v4i(&wf)[TN], bool sum_x, bool sum_w) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
+            if (SUMS) {
+                if (sum_x) {  // wave-uniform
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int q = 0; q < 4; q++) xsum[i] = __builtin_amdgcn_sdot4(xf[i][q], 0x01010101, xsum[i], false);
+                }
+                if (sum_w) {
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int q = 0; q < 4; q++) wsum[j] = __builtin_amdgcn_sdot4(wf[j][q], 0x01010101, wsum[j], false);
+                }
+            }
+        };
+        // Stage s lives in buffer s % 4; three stages are requested ahead.  The loop is software-pipelined: while
+        // the first K half of step s is multiplied the second half is being read, and while the second half is
+        // multiplied the first half of step s + 1 is being read.  In between sits the one barrier of the step:
+        // waiting until at most one stage of this thread's requests is outstanding means its part of stage s + 1 has
+        // landed (near the end of K nothing new is requested, so everything is waited for); the barrier extends
+        // that to every thread's part and also says that every wavefront has received its reads of stage s - 1,
+        // whose buffer the next request overwrites.
+        const int nk = g.K / BK;
+        v4i xf0[TM], wf0[TN], xf1[TM], wf1[TN];
+#pragma unroll
+        for (int d = 0; d < DL_S - 1; d++)
+            if (d < nk) issue(d, d);
+        if (nk > 2) wait_vmcnt<2 * (XI + WI)>(); else wait_vmcnt<0>();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        read_frags(0, 0, xf0, wf0);
+        for (int step = 0; step < nk; step += DL_S) {
+#pragma unroll
+            for (int d = 0; d < DL_S; d++) {
+                if (step + d < nk) {  // uniform
+                    read_frags(d, 1, xf1, wf1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    multiply(xf0, wf0, xs0, ws0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const bool more = step + d + DL_S - 1 < nk;
+                    if (more) wait_vmcnt<XI + WI>(); else wait_vmcnt<0>();
+                    asm volatile("" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    if (more) issue((d + DL_S - 1) % DL_S, step + d + DL_S - 1);
+                    read_frags((d + 1) % DL_S, 0, xf0, wf0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    multiply(xf1, wf1, xs1, ws1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        __syncthreads();
+        // ---- combine the split zero-point sums: afterwards every wavefront holds the full sums of its rows (X) and
+        // the wavefronts of row 0 those of their channels (W), as in the other fetch modes
+        if (SUMS) {
+            int32_t *xs_l = reinterpret_cast<int32_t *>(smem);          // [2][BM]
+            int32_t *ws_l = reinterpret_cast<int32_t *>(smem) + 2 * BM;  // [BN]: partial of wavefront row 1
+            if (need_xsum && wave_n < 2) {
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    const int32_t part = xsum[i] + __shfl_xor(xsum[i], 32);
+                    if (lane < 32) xs_l[wave_n * BM + wave_m * WM + i * 32 + lane] = part;
+                }
+            }
+            if (need_wsum && wave_m == 1) {
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const int32_t part = wsum[j] + __shfl_xor(wsum[j], 32);
+                    if (lane < 32) ws_l[wave_n * WN + j * 32 + lane] = part;
+                }
+            }
+            __syncthreads();
+            if (need_xsum) {
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    const int r = wave_m * WM + i * 32 + (lane & 31);
+                    xsum[i] = lane < 32 ? xs_l[r] + xs_l[BM + r] : 0;  // the two lane halves are added up below
+                }
+            }
+            if (need_wsum && wave_m == 0) {
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    if (lane < 32) wsum[j] += ws_l[wave_n * WN + j * 32 + lane];
+            }
+            __syncthreads();
+        }
+    } else {
     // ---- main loop: a ring of DEPTH register sets keeps DEPTH - 1 K steps of global loads in flight while one
     // step is multiplied out of LDS (two LDS buffers).  At the top of sub-iteration s: LDS[s & 1] holds step s and
     // register set (s + j) % DEPTH holds step s + j for j = 1 .. DEPTH - 1; the set of step s is free again.
@@ -540,6 +769,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                 __syncthreads();
             }
         }
+    }
+
     }
 
     if (tid < BN) {
@@ -666,16 +897,20 @@ template <int BM, int BN>
 constexpr size_t smem_bytes() {
     return (size_t)2 * BM * PITCH + (size_t)2 * w_buf_bytes<BN>() + (size_t)BN * sizeof(ChanParams);
 }
+template <int BM, int BN>
+constexpr size_t smem_bytes_dl() {
+    return (size_t)dl_stages<BM, BN>() * (BM + BN) * BK + (size_t)BN * sizeof(ChanParams);
+}
 
 template <typename Kernel>
 void launch_kernel(Kernel kernel, const GemmArgs &g, int threads, size_t sm, dim3 grid, hipStream_t s) {
     if (sm > 48 * 1024) {  // above the default dynamic LDS limit: raise it once per kernel
-        static bool raised = false;
-        if (!raised) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      (int)sm);
-            raised = true;
-        }
+        static std::mutex lock;
+        static std::unordered_set<const void *> raised;
+        const void *key = reinterpret_cast<const void *>(kernel);
+        std::lock_guard<std::mutex> guard(lock);
+        if (raised.insert(key).second)
+            (void)hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm);
     }
     kernel<<<grid, dim3(threads), sm, s>>>(g);
 }
@@ -683,6 +918,14 @@ void launch_kernel(Kernel kernel, const GemmArgs &g, int threads, size_t sm, dim
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool SUMS, bool Q8>
 void launch_tile(const GemmArgs &g, int xmode, int wmode, dim3 grid, hipStream_t s) {
     const size_t sm = smem_bytes<BM, BN>();
+    if constexpr (BM >= 128 && BN >= 128) {  // the direct-to-LDS pipeline exists for the large tiles only
+        if (xmode == X_PLAIN_DL && wmode == W_ROWS_DL)
+            return launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN_DL, W_ROWS_DL, SUMS, Q8>, g,
+                                 WAVES_M * WAVES_N * 64, smem_bytes_dl<BM, BN>(), grid, s);
+        if (xmode == X_PLAIN_DL && wmode == W_KMAJOR_DL)
+            return launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN_DL, W_KMAJOR_DL, SUMS, Q8>, g,
+                                 WAVES_M * WAVES_N * 64, smem_bytes_dl<BM, BN>(), grid, s);
+    }
     if (xmode == X_PLAIN && wmode == W_ROWS)
         launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_ROWS, SUMS, Q8>, g, WAVES_M * WAVES_N * 64, sm, grid, s);
     else if (xmode == X_TAP && wmode == W_ROWS)
@@ -723,6 +966,7 @@ MLEL_DECLARE_GEMM_TILE(2);
 MLEL_DECLARE_GEMM_TILE(3);
 MLEL_DECLARE_GEMM_TILE(4);
 MLEL_DECLARE_GEMM_TILE(5);
+MLEL_DECLARE_GEMM_TILE(6);
 #define MLEL_DEFINE_GEMM_TILE(ID, BM, BN, WAVES_M, WAVES_N)                                          \
     void launch_gemm_tile##ID(const void *args, int xmode, int wmode, dim3 grid, hipStream_t s) {    \
         launch_tile_zp<BM, BN, WAVES_M, WAVES_N>(*static_cast<const GemmArgs *>(args), xmode, wmode, grid, s); \

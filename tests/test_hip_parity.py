@@ -229,6 +229,50 @@ def test_matmul_i8_vs_oracle(run, oracle, case):
     np.testing.assert_array_equal(run.matmul(a, b, abi.I8, za, zb, epilogue=(mult, shift, rattr, None)), exp8)
 
 
+DL_CASES = [
+    # name, batches, M, K, N, a_zp, b_zp: sizes at which the direct-to-LDS tiles are chosen on a 256-CU device
+    ("tile256_kmajor", 1, 4096, 128, 4096, 2, -1),        # 256 tiles of 256 x 256
+    ("tile256_ragged", 1, 4000, 192, 4224, -3, 5),        # partial last tile row and column
+    ("tile256_no_zp", 2, 2048, 64, 4096, 0, 0),           # a single K step, no zero-point sums
+    ("tile128_band_walk", 1, 2944, 192, 2944, 7, 0),      # 529 tiles of 128 x 128, three K steps
+    ("tile128_batched", 16, 640, 320, 1024, 0, -6),       # 5 x 8 tiles per batch, five K steps
+]
+
+
+@pytest.mark.parametrize("case", DL_CASES, ids=[c[0] for c in DL_CASES])
+def test_matmul_i8_direct_to_lds_tiles(run, oracle, case):
+    """Large int8 MATMULs (K a multiple of 64) run on the direct-to-LDS pipeline with 256 x 256 or 128 x 128 tiles
+    and the banded tile walk: int32 result and fused per-tensor RESCALE, bit for bit against the oracle."""
+    name, nb, m, k, n, za, zb = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    a = ri(rng, -128, 127, (nb, m, k), np.int8)
+    b = ri(rng, -128, 127, (nb, k, n), np.int8)
+    exp = oracle.matmul(a, b, abi.I32, za, zb)
+    np.testing.assert_array_equal(run.matmul(a, b, abi.I32, za, zb), exp)
+    mult, shift = np.array([1518500250], np.int32), np.array([37], np.int8)
+    rattr = abi.rescale_attr(0, -4, True, True, False)
+    exp8 = oracle.rescale(exp, mult, shift, abi.I8, rattr)
+    np.testing.assert_array_equal(run.matmul(a, b, abi.I8, za, zb, epilogue=(mult, shift, rattr, None)), exp8)
+    assert len(np.unique(exp8)) > 100
+
+
+def test_conv2d_i8_direct_to_lds_row_weights(run, oracle):
+    """1x1 CONV2D with OHWI weights (row-major W) on the direct-to-LDS pipeline: 4096 positions x 4096 channels,
+    IC = 128, per-channel RESCALE + CLAMP fused, and the int32 accumulator."""
+    rng = np.random.default_rng(4242)
+    x = ri(rng, -128, 127, (4, 32, 32, 128), np.int8)
+    w = ri(rng, -127, 127, (4096, 1, 1, 128), np.int8)
+    bias = ri(rng, -2 ** 15, 2 ** 15, (4096,), np.int32)
+    attr = abi.conv2d_attr(input_zp=-5, weight_zp=3)
+    acc = oracle.conv2d(x, w, bias, (4, 32, 32, 4096), abi.I32, attr)
+    np.testing.assert_array_equal(run.conv2d(x, w, bias, (4, 32, 32, 4096), abi.I32, attr), acc)
+    mult, shift = rescale_params(rng, 4096)
+    rattr = abi.rescale_attr(0, 3, True, True, True)
+    exp = np.clip(oracle.rescale(acc, mult, shift, abi.I8, rattr), -100, 90).astype(np.int8)
+    out = run.conv2d(x, w, bias, (4, 32, 32, 4096), abi.I8, attr, epilogue=(mult, shift, rattr, (-100, 90)))
+    np.testing.assert_array_equal(out, exp)
+
+
 def test_matmul_float_generic(run, oracle):
     rng = np.random.default_rng(8)
     a = rng.standard_normal((2, 9, 33)).astype(np.float32)
