@@ -57,6 +57,20 @@ class Conv2dAttr(C.Structure):
                 ("stride", C.c_int32 * 2), ("dilation", C.c_int32 * 2), ("acc_type", C.c_uint32)]
 
 
+class Conv3dAttr(C.Structure):
+    _fields_ = [("input_zp", C.c_int32), ("weight_zp", C.c_int32), ("pad", C.c_int32 * 6),
+                ("stride", C.c_int32 * 3), ("dilation", C.c_int32 * 3), ("acc_type", C.c_uint32)]
+
+
+class Tconv2dAttr(C.Structure):
+    _fields_ = [("input_zp", C.c_int32), ("weight_zp", C.c_int32), ("out_pad", C.c_int32 * 4),
+                ("stride", C.c_int32 * 2), ("acc_type", C.c_uint32)]
+
+
+class ResizeAttr(C.Structure):
+    _fields_ = [("scale", C.c_int32 * 4), ("offset", C.c_int32 * 2), ("border", C.c_int32 * 2), ("mode", C.c_uint32)]
+
+
 class MatmulAttr(C.Structure):
     _fields_ = [("a_zp", C.c_int32), ("b_zp", C.c_int32)]
 
@@ -88,6 +102,32 @@ def conv2d_attr(pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), input_zp=0, we
     a.pad[:] = [int(v) for v in pad]
     a.stride[:] = [int(v) for v in stride]
     a.dilation[:] = [int(v) for v in dilation]
+    return a
+
+
+def conv3d_attr(pad=(0,) * 6, stride=(1, 1, 1), dilation=(1, 1, 1), input_zp=0, weight_zp=0, acc_type=ACC_I32):
+    a = Conv3dAttr()
+    a.input_zp, a.weight_zp, a.acc_type = input_zp, weight_zp, acc_type
+    a.pad[:] = list(pad)
+    a.stride[:] = list(stride)
+    a.dilation[:] = list(dilation)
+    return a
+
+
+def tconv2d_attr(out_pad=(0, 0, 0, 0), stride=(1, 1), input_zp=0, weight_zp=0, acc_type=ACC_I32):
+    a = Tconv2dAttr()
+    a.input_zp, a.weight_zp, a.acc_type = input_zp, weight_zp, acc_type
+    a.out_pad[:] = list(out_pad)
+    a.stride[:] = list(stride)
+    return a
+
+
+def resize_attr(scale, offset=(0, 0), border=(0, 0), mode=1):
+    a = ResizeAttr()
+    a.scale[:] = list(scale)
+    a.offset[:] = list(offset)
+    a.border[:] = list(border)
+    a.mode = mode
     return a
 
 
@@ -153,6 +193,18 @@ OP_SIGNATURES = {
     "concat": [_T, _T, C.c_uint32, C.c_uint32],
     "slice": [_T, _T, C.POINTER(C.c_uint32)],
     "pad": [_T, _T, _T, C.c_double, C.c_int32],
+    "argmax": [_T, _T, C.c_uint32, C.c_uint32],
+    "arithmetic_right_shift": [_T, _T, _T, C.c_uint32],
+    "conv3d": [_T, _T, _T, _T, C.POINTER(Conv3dAttr)],
+    "transpose_conv2d": [_T, _T, _T, _T, C.POINTER(Tconv2dAttr)],
+    "fft2d": [_T, _T, _T, _T, C.c_int32],
+    "rfft2d": [_T, _T, _T],
+    "gather": [_T, _T, _T],
+    "scatter": [_T, _T, _T, _T],
+    "resize": [_T, _T, C.POINTER(ResizeAttr)],
+    "reverse": [_T, _T, C.c_uint32],
+    "tile": [_T, _T],
+    "select": [_T, _T, _T, _T],
 }
 
 FUSED_SIGNATURES = {

@@ -336,6 +336,155 @@ int mlel_hip_pad(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel
     return pad_generic_launch((hipStream_t)stream, out, in, padding, pad_const, pad_const_int);
 }
 
+// ---- the TOSA operators outside the benchmark graphs (kernels: ops_extra.hip) ----
+
+int mlel_hip_argmax(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis,
+                    uint32_t nan_mode) {
+    MLEL_TRY(require_ctx(ctx, "argmax"));
+    MLEL_TRY(check_supported(out, "argmax out"));
+    MLEL_TRY(check_supported(in, "argmax in"));
+    MLEL_REQUIRE((int)axis < in->rank && out->rank == in->rank - 1 && out->dtype == MLEL_I32, MLEL_ERR_INVALID,
+                 "argmax: the output is int32 with the axis removed");
+    return argmax_launch((hipStream_t)stream, out, in, axis, nan_mode);
+}
+
+int mlel_hip_arithmetic_right_shift(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1,
+                                    const mlel_tensor *in2, uint32_t round) {
+    MLEL_TRY(require_ctx(ctx, "arithmetic_right_shift"));
+    MLEL_TRY(check_supported(out, "arithmetic_right_shift out"));
+    MLEL_TRY(check_supported(in1, "arithmetic_right_shift in1"));
+    MLEL_TRY(check_supported(in2, "arithmetic_right_shift in2"));
+    MLEL_REQUIRE(dt_is_int(out->dtype) && in1->dtype == out->dtype && in2->dtype == out->dtype &&
+                     in1->rank == out->rank && in2->rank == out->rank,
+                 MLEL_ERR_INVALID, "arithmetic_right_shift: one integer type, equal ranks");
+    return arshift_launch((hipStream_t)stream, out, in1, in2, round);
+}
+
+int mlel_hip_conv3d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                    const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv3d_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "conv3d"));
+    MLEL_REQUIRE(attr != nullptr, MLEL_ERR_INVALID, "conv3d: null attribute");
+    MLEL_TRY(check_supported(out, "conv3d out"));
+    MLEL_TRY(check_supported(in, "conv3d in"));
+    MLEL_TRY(check_supported(weights, "conv3d weights"));
+    MLEL_TRY(check_supported(bias, "conv3d bias"));
+    MLEL_REQUIRE(out->rank == 5 && in->rank == 5 && weights->rank == 5 && bias->rank == 1, MLEL_ERR_INVALID,
+                 "conv3d: ranks must be 5,5,5,1");
+    MLEL_REQUIRE(attr->acc_type >= MLEL_ACC_I32 && attr->acc_type <= MLEL_ACC_I64, MLEL_ERR_INVALID,
+                 "Unsupported acc type %u", attr->acc_type);
+    return conv3d_launch((hipStream_t)stream, out, in, weights, bias, attr);
+}
+
+int mlel_hip_transpose_conv2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                              const mlel_tensor *weights, const mlel_tensor *bias, const mlel_tconv2d_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "transpose_conv2d"));
+    MLEL_REQUIRE(attr != nullptr, MLEL_ERR_INVALID, "transpose_conv2d: null attribute");
+    MLEL_TRY(check_supported(out, "transpose_conv2d out"));
+    MLEL_TRY(check_supported(in, "transpose_conv2d in"));
+    MLEL_TRY(check_supported(weights, "transpose_conv2d weights"));
+    MLEL_TRY(check_supported(bias, "transpose_conv2d bias"));
+    MLEL_REQUIRE(out->rank == 4 && in->rank == 4 && weights->rank == 4 && bias->rank == 1, MLEL_ERR_INVALID,
+                 "transpose_conv2d: ranks must be 4,4,4,1");
+    MLEL_REQUIRE(attr->stride[0] > 0 && attr->stride[1] > 0, MLEL_ERR_INVALID, "transpose_conv2d: stride must be positive");
+    MLEL_REQUIRE(attr->acc_type >= MLEL_ACC_I32 && attr->acc_type <= MLEL_ACC_I64, MLEL_ERR_INVALID,
+                 "Unsupported acc type %u", attr->acc_type);
+    return tconv2d_launch((hipStream_t)stream, out, in, weights, bias, attr);
+}
+
+int mlel_hip_fft2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out_real, const mlel_tensor *out_imag,
+                   const mlel_tensor *in_real, const mlel_tensor *in_imag, int32_t inverse) {
+    MLEL_TRY(require_ctx(ctx, "fft2d"));
+    const mlel_tensor *all[4] = {out_real, out_imag, in_real, in_imag};
+    for (const mlel_tensor *t : all) {
+        MLEL_TRY(check_supported(t, "fft2d tensor"));
+        MLEL_REQUIRE(t->rank == 3 && t->dtype == MLEL_F32, MLEL_ERR_INVALID, "fft2d: float32 tensors of rank 3");
+    }
+    return fft2d_launch((hipStream_t)stream, out_real, out_imag, in_real, in_imag, inverse != 0);
+}
+
+int mlel_hip_rfft2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out_real, const mlel_tensor *out_imag,
+                    const mlel_tensor *in) {
+    MLEL_TRY(require_ctx(ctx, "rfft2d"));
+    const mlel_tensor *all[3] = {out_real, out_imag, in};
+    for (const mlel_tensor *t : all) {
+        MLEL_TRY(check_supported(t, "rfft2d tensor"));
+        MLEL_REQUIRE(t->rank == 3 && t->dtype == MLEL_F32, MLEL_ERR_INVALID, "rfft2d: float32 tensors of rank 3");
+    }
+    return rfft2d_launch((hipStream_t)stream, out_real, out_imag, in);
+}
+
+int mlel_hip_gather(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *values,
+                    const mlel_tensor *indices) {
+    MLEL_TRY(require_ctx(ctx, "gather"));
+    MLEL_TRY(check_tensor(out, "gather out"));
+    MLEL_TRY(check_tensor(values, "gather values"));
+    MLEL_TRY(check_supported(indices, "gather indices"));
+    MLEL_REQUIRE(out->rank == 3 && values->rank == 3 && indices->rank == 2 && dt_is_int(indices->dtype) &&
+                     dt_size(out->dtype) == dt_size(values->dtype),
+                 MLEL_ERR_INVALID, "gather: [N,W,C] from [N,K,C] with integer indices [N,W]");
+    return gather_launch((hipStream_t)stream, out, values, indices);
+}
+
+int mlel_hip_scatter(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *values_in,
+                     const mlel_tensor *indices, const mlel_tensor *input) {
+    MLEL_TRY(require_ctx(ctx, "scatter"));
+    MLEL_TRY(check_tensor(out, "scatter out"));
+    MLEL_TRY(check_tensor(values_in, "scatter values_in"));
+    MLEL_TRY(check_supported(indices, "scatter indices"));
+    MLEL_TRY(check_tensor(input, "scatter input"));
+    MLEL_REQUIRE(out->rank == 3 && values_in->rank == 3 && input->rank == 3 && indices->rank == 2 &&
+                     dt_is_int(indices->dtype) && dt_size(out->dtype) == dt_size(values_in->dtype) &&
+                     dt_size(out->dtype) == dt_size(input->dtype),
+                 MLEL_ERR_INVALID, "scatter: [N,K,C] from [N,K,C], integer indices [N,W] and [N,W,C]");
+    return scatter_launch((hipStream_t)stream, out, values_in, indices, input);
+}
+
+int mlel_hip_resize(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                    const mlel_resize_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "resize"));
+    MLEL_REQUIRE(attr != nullptr, MLEL_ERR_INVALID, "resize: null attribute");
+    MLEL_TRY(check_supported(out, "resize out"));
+    MLEL_TRY(check_supported(in, "resize in"));
+    MLEL_REQUIRE(out->rank == 4 && in->rank == 4 && dt_is_float(out->dtype) == dt_is_float(in->dtype), MLEL_ERR_INVALID,
+                 "resize: rank 4, integer to integer or float to float");
+    MLEL_REQUIRE(attr->scale[0] > 0 && attr->scale[2] > 0, MLEL_ERR_INVALID, "resize: scale numerators must be positive");
+    MLEL_REQUIRE(attr->mode == MLEL_RESIZE_NEAREST || attr->mode == MLEL_RESIZE_BILINEAR, MLEL_ERR_INVALID,
+                 "resize: mode %u", attr->mode);
+    return resize_launch((hipStream_t)stream, out, in, attr);
+}
+
+int mlel_hip_reverse(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis) {
+    MLEL_TRY(require_ctx(ctx, "reverse"));
+    MLEL_TRY(check_tensor(out, "reverse out"));
+    MLEL_TRY(check_tensor(in, "reverse in"));
+    MLEL_REQUIRE(in->rank == out->rank && (int)axis < out->rank && dt_size(in->dtype) == dt_size(out->dtype),
+                 MLEL_ERR_INVALID, "reverse: bad arguments");
+    return reverse_launch((hipStream_t)stream, out, in, axis);
+}
+
+int mlel_hip_tile(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in) {
+    MLEL_TRY(require_ctx(ctx, "tile"));
+    MLEL_TRY(check_tensor(out, "tile out"));
+    MLEL_TRY(check_tensor(in, "tile in"));
+    MLEL_REQUIRE(in->rank == out->rank && dt_size(in->dtype) == dt_size(out->dtype), MLEL_ERR_INVALID,
+                 "tile: bad arguments");
+    return tile_launch((hipStream_t)stream, out, in);
+}
+
+int mlel_hip_select(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *condition,
+                    const mlel_tensor *in_true, const mlel_tensor *in_false) {
+    MLEL_TRY(require_ctx(ctx, "select"));
+    MLEL_TRY(check_tensor(out, "select out"));
+    MLEL_TRY(check_supported(condition, "select condition"));
+    MLEL_TRY(check_tensor(in_true, "select in_true"));
+    MLEL_TRY(check_tensor(in_false, "select in_false"));
+    MLEL_REQUIRE(dt_size(condition->dtype) == 1 && condition->rank == out->rank && in_true->rank == out->rank &&
+                     in_false->rank == out->rank && dt_size(in_true->dtype) == dt_size(out->dtype) &&
+                     dt_size(in_false->dtype) == dt_size(out->dtype),
+                 MLEL_ERR_INVALID, "select: one-byte condition, equal ranks and element sizes");
+    return select_launch((hipStream_t)stream, out, condition, in_true, in_false);
+}
+
 // ---- fused entry points ----
 
 int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,

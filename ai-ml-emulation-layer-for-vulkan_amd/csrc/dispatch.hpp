@@ -36,6 +36,25 @@ int move_generic_launch(hipStream_t s, int kind, const mlel_tensor *out, const m
 int pad_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *padding,
                        double pad_const, int32_t pad_const_int);
 
+// ops_extra.hip: the TOSA operators outside the benchmark graphs
+int conv3d_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
+                  const mlel_tensor *bias, const mlel_conv3d_attr *a);
+int tconv2d_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
+                   const mlel_tensor *bias, const mlel_tconv2d_attr *a);
+int argmax_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis, uint32_t nan_mode);
+int arshift_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in1, const mlel_tensor *in2, uint32_t round);
+int gather_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *values, const mlel_tensor *indices);
+int scatter_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *values_in, const mlel_tensor *indices,
+                   const mlel_tensor *input);
+int reverse_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis);
+int tile_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in);
+int select_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *cond, const mlel_tensor *a,
+                  const mlel_tensor *b);
+int resize_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_resize_attr *a);
+int fft2d_launch(hipStream_t s, const mlel_tensor *out_r, const mlel_tensor *out_i, const mlel_tensor *in_r,
+                 const mlel_tensor *in_i, bool inverse);
+int rfft2d_launch(hipStream_t s, const mlel_tensor *out_r, const mlel_tensor *out_i, const mlel_tensor *in);
+
 // ---- int8 MFMA contractions (gemm_i8.hip) ----
 // Optional fused epilogue: when `epi` is non-null the int32 accumulator is requantised (RESCALE [+CLAMP]) and
 // stored as int8/int16/int32 `out`; otherwise the int32 accumulator (plus bias) is stored.

@@ -19,6 +19,18 @@
 //   SLICE                      in: input                    iattr: start[rank]
 //   TRANSPOSE                  in: input                    iattr: perms[rank]
 //   PAD                        in: input, padding           fattr: padConst     iattr: padConstInt
+//   ARGMAX                     in: input                    iattr: axis nanMode
+//   ARITHMETIC_RIGHT_SHIFT     in: input1, input2           iattr: round
+//   CONV3D                     in: input, weights, biases   iattr: pad[6] stride[3] dilation[3] inputZp weightZp accType
+//   TRANSPOSE_CONV2D           in: input, weights, biases   iattr: outPad[4] stride[2] inputZp weightZp accType
+//   GATHER                     in: values, indices
+//   SCATTER                    in: valuesIn, indices, input (the operand order of the TOSA instruction)
+//   REVERSE                    in: input                    iattr: axis
+//   TILE                       in: input
+//   RESIZE                     in: input                    iattr: scale[4] offset[2] border[2] mode
+//   SELECT                     in: condition, onTrue, onFalse
+//   FFT2D                      in: real, imag               out: real, imag       iattr: inverse
+//   RFFT2D                     in: input                    out: real, imag
 //   binary (ADD SUB BITWISE_* LOGICAL_* INTDIV POW EQUAL GREATER GREATER_EQUAL): in: input1, input2
 //   unary (ABS ... TANH), CAST, RESHAPE: in: input
 #include <cstring>
@@ -205,26 +217,34 @@ const std::map<std::string, Maker> &makers() {
         UN("LOGICAL_NOT", makeLogicalNot), UN("RECIPROCAL", makeReciprocal), UN("RSQRT", makeRsqrt),
         UN("SIGMOID", makeSigmoid), UN("SIN", makeSin), UN("TANH", makeTanh), UN("CAST", makeCast),
         UN("RESHAPE", makeReshape),
-        // declared by the reference's surface, no HIP kernel yet: the make call reports MLEL_ERR_UNSUPPORTED
-        {"ARGMAX", [](GraphPipeline &p, const Args &a) { p.makeArgmax(a.I(0), a.O(), 0, 1, a.name); }},
+        {"ARGMAX",
+         [](GraphPipeline &p, const Args &a) {
+             p.makeArgmax(a.I(0), a.O(), static_cast<uint32_t>(a.i(0)), static_cast<uint32_t>(a.i(1)), a.name);
+         }},
         {"ARITHMETIC_RIGHT_SHIFT",
-         [](GraphPipeline &p, const Args &a) { p.makeArithmeticRightShift(a.I(0), a.I(1), a.O(), false, a.name); }},
+         [](GraphPipeline &p, const Args &a) { p.makeArithmeticRightShift(a.I(0), a.I(1), a.O(), a.i(0) != 0, a.name); }},
         {"CONV3D",
          [](GraphPipeline &p, const Args &a) {
-             p.makeConv3D(a.I(0), a.O(), a.I(1), a.I(2), {}, {}, {}, 0, 0, 1, a.name);
+             p.makeConv3D(a.I(0), a.O(), a.I(1), a.I(2), a.iv(0, 6), a.iv(6, 3), a.iv(9, 3), static_cast<int8_t>(a.i(12)),
+                          static_cast<int8_t>(a.i(13)), static_cast<uint32_t>(a.i(14)), a.name);
          }},
-        {"GATHER", [](GraphPipeline &p, const Args &a) { p.makeGather(a.I(0), a.I(1), a.O(), a.name); }},
-        {"REVERSE", [](GraphPipeline &p, const Args &a) { p.makeReverse(a.I(0), a.O(), 0, a.name); }},
-        {"TILE", [](GraphPipeline &p, const Args &a) { p.makeTile(a.I(0), a.O(), a.name); }},
-        {"RESIZE", [](GraphPipeline &p, const Args &a) { p.makeResize(a.I(0), a.O(), {}, {}, {}, 0, a.name); }},
-        {"SELECT", [](GraphPipeline &p, const Args &a) { p.makeSelect(a.I(0), a.I(1), a.I(2), a.O(), a.name); }},
-        {"SCATTER", [](GraphPipeline &p, const Args &a) { p.makeScatter(a.I(0), a.I(1), a.I(2), a.O(), a.name); }},
         {"TRANSPOSE_CONV2D",
          [](GraphPipeline &p, const Args &a) {
-             p.makeTransposeConv2D(a.I(0), a.O(), a.I(1), a.I(2), {}, {}, 0, 0, 1, a.name);
+             p.makeTransposeConv2D(a.I(0), a.O(), a.I(1), a.I(2), a.iv(0, 4), a.iv(4, 2), static_cast<int8_t>(a.i(6)),
+                                   static_cast<int8_t>(a.i(7)), static_cast<uint32_t>(a.i(8)), a.name);
          }},
+        {"GATHER", [](GraphPipeline &p, const Args &a) { p.makeGather(a.I(0), a.I(1), a.O(), a.name); }},
+        {"SCATTER", [](GraphPipeline &p, const Args &a) { p.makeScatter(a.I(2), a.I(0), a.I(1), a.O(), a.name); }},
+        {"REVERSE",
+         [](GraphPipeline &p, const Args &a) { p.makeReverse(a.I(0), a.O(), static_cast<uint32_t>(a.i(0)), a.name); }},
+        {"TILE", [](GraphPipeline &p, const Args &a) { p.makeTile(a.I(0), a.O(), a.name); }},
+        {"RESIZE",
+         [](GraphPipeline &p, const Args &a) {
+             p.makeResize(a.I(0), a.O(), a.iv(0, 4), a.iv(4, 2), a.iv(6, 2), static_cast<uint32_t>(a.i(8)), a.name);
+         }},
+        {"SELECT", [](GraphPipeline &p, const Args &a) { p.makeSelect(a.I(0), a.I(1), a.I(2), a.O(), a.name); }},
         {"FFT2D",
-         [](GraphPipeline &p, const Args &a) { p.makeFft2D(a.I(0), a.I(1), a.O(0), a.O(1), false, a.name); }},
+         [](GraphPipeline &p, const Args &a) { p.makeFft2D(a.I(0), a.I(1), a.O(0), a.O(1), a.i(0) != 0, a.name); }},
         {"RFFT2D", [](GraphPipeline &p, const Args &a) { p.makeRfft2D(a.I(0), a.O(0), a.O(1), a.name); }},
     };
     return m;
@@ -331,7 +351,8 @@ int mlel_graph_make_op(mlel_graph *g, const char *tosa_name, const int *inputs, 
 }
 
 int mlel_graph_load_spvasm(mlel_graph *g, const char *text, size_t length, const mlel_graph_spv_binding *bindings,
-                           int n_bindings, const mlel_graph_spv_constant *constants, int n_constants, uint32_t *io,
+                           int n_bindings, const mlel_graph_spv_constant *constants, int n_constants,
+                           const mlel_graph_spv_specialization *specializations, int n_specializations, uint32_t *io,
                            int io_capacity, int *n_inputs, int *n_outputs) {
     return guarded([&] {
         if (!text) throw std::runtime_error("null SPIR-V text");
@@ -341,7 +362,9 @@ int mlel_graph_load_spvasm(mlel_graph *g, const char *text, size_t length, const
         std::vector<SpvConstant> c;
         for (int i = 0; i < n_constants; i++)
             c.push_back({constants[i].id, constants[i].data, vec64(constants[i].dims, constants[i].rank)});
-        const SpvGraphInfo info = loadSpirvAssembly(g->pipeline, std::string(text, length), b, c);
+        std::vector<SpvSpecialization> sp;
+        for (int i = 0; i < n_specializations; i++) sp.push_back({specializations[i].spec_id, specializations[i].bits});
+        const SpvGraphInfo info = loadSpirvAssembly(g->pipeline, std::string(text, length), b, c, sp);
         const size_t total = info.inputs.size() + info.outputs.size();
         if (io && static_cast<size_t>(io_capacity) < 3 * total) throw std::runtime_error("io array too small");
         size_t k = 0;

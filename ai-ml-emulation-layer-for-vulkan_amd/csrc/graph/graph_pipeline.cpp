@@ -446,51 +446,95 @@ void GraphPipeline::makeTranspose(const TensorPtr &input, const TensorPtr &outpu
     for (uint32_t i = 0; i < input->getRank(); i++) n->vec[i] = perms[i];
 }
 
-// operators of the reference's surface that have no HIP kernel yet: the call fails like an unknown operator does in
-// the reference's decoder (graph_tosa_1_0_ext_inst.cpp:311)
-void GraphPipeline::makeArgmax(const TensorPtr &, const TensorPtr &, uint32_t, uint32_t, const std::string &) {
-    unsupported("ARGMAX");
+void GraphPipeline::makeArgmax(const TensorPtr &input, const TensorPtr &output, const uint32_t axis,
+                               const uint32_t nanMode, const std::string &debugName) {
+    auto n = addOp(OpKind::Argmax, "ARGMAX", debugName, {input}, {output});
+    n->axis = axis;
+    n->nanMode = nanMode;
 }
-void GraphPipeline::makeArithmeticRightShift(const TensorPtr &, const TensorPtr &, const TensorPtr &, bool,
-                                             const std::string &) {
-    unsupported("ARITHMETIC_RIGHT_SHIFT");
+
+void GraphPipeline::makeArithmeticRightShift(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &output,
+                                             const bool round, const std::string &debugName) {
+    addOp(OpKind::ArithmeticRightShift, "ARITHMETIC_RIGHT_SHIFT", debugName, {input1, input2}, {output})->flag = round;
 }
-void GraphPipeline::makeConv3D(const TensorPtr &, const TensorPtr &, const TensorPtr &, const TensorPtr &,
-                               const std::vector<int32_t> &, const std::vector<int32_t> &, const std::vector<int32_t> &,
-                               int8_t, int8_t, uint32_t, const std::string &) {
-    unsupported("CONV3D");
+
+void GraphPipeline::makeConv3D(const TensorPtr &input, const TensorPtr &output, const TensorPtr &weights,
+                               const TensorPtr &biases, const std::vector<int32_t> &pad,
+                               const std::vector<int32_t> &stride, const std::vector<int32_t> &dilation,
+                               const int8_t inputZeroPoint, const int8_t weightZeroPoint, const uint32_t accType,
+                               const std::string &debugName) {
+    if (pad.size() < 6 || stride.size() < 3 || dilation.size() < 3) fail("CONV3D: pad/stride/dilation need 6/3/3 values");
+    auto n = addOp(OpKind::Conv3D, "CONV3D", debugName, {input, weights, biases}, {output});
+    n->conv3d.input_zp = inputZeroPoint;
+    n->conv3d.weight_zp = weightZeroPoint;
+    for (int i = 0; i < 6; i++) n->conv3d.pad[i] = pad[static_cast<size_t>(i)];
+    for (int i = 0; i < 3; i++) {
+        n->conv3d.stride[i] = stride[static_cast<size_t>(i)];
+        n->conv3d.dilation[i] = dilation[static_cast<size_t>(i)];
+    }
+    n->conv3d.acc_type = accType;
 }
-void GraphPipeline::makeFft2D(const TensorPtr &, const TensorPtr &, const TensorPtr &, const TensorPtr &, bool,
-                              const std::string &) {
-    unsupported("FFT2D");
+
+void GraphPipeline::makeTransposeConv2D(const TensorPtr &input, const TensorPtr &output, const TensorPtr &weights,
+                                        const TensorPtr &biases, const std::vector<int32_t> &pad,
+                                        const std::vector<int32_t> &stride, const int8_t inputZeroPoint,
+                                        const int8_t weightZeroPoint, const uint32_t accType,
+                                        const std::string &debugName) {
+    if (pad.size() < 4 || stride.size() < 2) fail("TRANSPOSE_CONV2D: outPad/stride need 4/2 values");
+    auto n = addOp(OpKind::TransposeConv2D, "TRANSPOSE_CONV2D", debugName, {input, weights, biases}, {output});
+    n->tconv.input_zp = inputZeroPoint;
+    n->tconv.weight_zp = weightZeroPoint;
+    for (int i = 0; i < 4; i++) n->tconv.out_pad[i] = pad[static_cast<size_t>(i)];
+    for (int i = 0; i < 2; i++) n->tconv.stride[i] = stride[static_cast<size_t>(i)];
+    n->tconv.acc_type = accType;
 }
-void GraphPipeline::makeGather(const TensorPtr &, const TensorPtr &, const TensorPtr &, const std::string &) {
-    unsupported("GATHER");
+
+void GraphPipeline::makeFft2D(const TensorPtr &inputReal, const TensorPtr &inputImag, const TensorPtr &outputReal,
+                              const TensorPtr &outputImag, const bool inverse, const std::string &debugName) {
+    addOp(OpKind::Fft2D, "FFT2D", debugName, {inputReal, inputImag}, {outputReal, outputImag})->flag = inverse;
 }
-void GraphPipeline::makeResize(const TensorPtr &, const TensorPtr &, const std::vector<int32_t> &,
-                               const std::vector<int32_t> &, const std::vector<int32_t> &, uint32_t,
-                               const std::string &) {
-    unsupported("RESIZE");
+
+void GraphPipeline::makeRfft2D(const TensorPtr &input, const TensorPtr &outputReal, const TensorPtr &outputImag,
+                               const std::string &debugName) {
+    addOp(OpKind::Rfft2D, "RFFT2D", debugName, {input}, {outputReal, outputImag});
 }
-void GraphPipeline::makeReverse(const TensorPtr &, const TensorPtr &, uint32_t, const std::string &) {
-    unsupported("REVERSE");
+
+void GraphPipeline::makeGather(const TensorPtr &values, const TensorPtr &indices, const TensorPtr &output,
+                               const std::string &debugName) {
+    addOp(OpKind::Gather, "GATHER", debugName, {values, indices}, {output});
 }
-void GraphPipeline::makeRfft2D(const TensorPtr &, const TensorPtr &, const TensorPtr &, const std::string &) {
-    unsupported("RFFT2D");
+
+// `input` is the [N, W, C] tensor whose rows are written into `values` [N, K, C] at the rows named by `indices`
+void GraphPipeline::makeScatter(const TensorPtr &input, const TensorPtr &values, const TensorPtr &indices,
+                                const TensorPtr &output, const std::string &debugName) {
+    addOp(OpKind::Scatter, "SCATTER", debugName, {values, indices, input}, {output});
 }
-void GraphPipeline::makeScatter(const TensorPtr &, const TensorPtr &, const TensorPtr &, const TensorPtr &,
-                                const std::string &) {
-    unsupported("SCATTER");
+
+void GraphPipeline::makeResize(const TensorPtr &input, const TensorPtr &output, const std::vector<int32_t> &scale,
+                               const std::vector<int32_t> &offset, const std::vector<int32_t> &border,
+                               const uint32_t mode, const std::string &debugName) {
+    if (scale.size() < 4 || offset.size() < 2 || border.size() < 2) fail("RESIZE: scale/offset/border need 4/2/2 values");
+    auto n = addOp(OpKind::Resize, "RESIZE", debugName, {input}, {output});
+    for (int i = 0; i < 4; i++) n->resize.scale[i] = scale[static_cast<size_t>(i)];
+    for (int i = 0; i < 2; i++) {
+        n->resize.offset[i] = offset[static_cast<size_t>(i)];
+        n->resize.border[i] = border[static_cast<size_t>(i)];
+    }
+    n->resize.mode = mode;
 }
-void GraphPipeline::makeSelect(const TensorPtr &, const TensorPtr &, const TensorPtr &, const TensorPtr &,
-                               const std::string &) {
-    unsupported("SELECT");
+
+void GraphPipeline::makeReverse(const TensorPtr &input, const TensorPtr &output, const uint32_t axis,
+                                const std::string &debugName) {
+    addOp(OpKind::Reverse, "REVERSE", debugName, {input}, {output})->axis = axis;
 }
-void GraphPipeline::makeTile(const TensorPtr &, const TensorPtr &, const std::string &) { unsupported("TILE"); }
-void GraphPipeline::makeTransposeConv2D(const TensorPtr &, const TensorPtr &, const TensorPtr &, const TensorPtr &,
-                                        const std::vector<int32_t> &, const std::vector<int32_t> &, int8_t, int8_t,
-                                        uint32_t, const std::string &) {
-    unsupported("TRANSPOSE_CONV2D");
+
+void GraphPipeline::makeSelect(const TensorPtr &input1, const TensorPtr &input2, const TensorPtr &input3,
+                               const TensorPtr &output, const std::string &debugName) {
+    addOp(OpKind::Select, "SELECT", debugName, {input1, input2, input3}, {output});
+}
+
+void GraphPipeline::makeTile(const TensorPtr &input, const TensorPtr &output, const std::string &debugName) {
+    addOp(OpKind::Tile, "TILE", debugName, {input}, {output});
 }
 
 /*******************************************************************************
@@ -784,6 +828,29 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
     case OpKind::Concat: rc = mlel_hip_concat(ctx, stream, &out, &in[0], op.axis, op.offset); break;
     case OpKind::Slice: rc = mlel_hip_slice(ctx, stream, &out, &in[0], op.vec.data()); break;
     case OpKind::Pad: rc = mlel_hip_pad(ctx, stream, &out, &in[0], &in[1], op.padConst, op.padConstInt); break;
+    case OpKind::Argmax: rc = mlel_hip_argmax(ctx, stream, &out, &in[0], op.axis, op.nanMode); break;
+    case OpKind::ArithmeticRightShift:
+        rc = mlel_hip_arithmetic_right_shift(ctx, stream, &out, &in[0], &in[1], op.flag ? 1u : 0u);
+        break;
+    case OpKind::Conv3D: rc = mlel_hip_conv3d(ctx, stream, &out, &in[0], &in[1], &in[2], &op.conv3d); break;
+    case OpKind::TransposeConv2D:
+        rc = mlel_hip_transpose_conv2d(ctx, stream, &out, &in[0], &in[1], &in[2], &op.tconv);
+        break;
+    case OpKind::Fft2D:
+    case OpKind::Rfft2D: {
+        const mlel_tensor imag = op.outputs[1]->view();
+        if (imag.ptr == nullptr && op.outputs[1]->getShapeSize() != 0)
+            fail(op.tosaName + " (" + op.debugName + "): second output tensor has no memory bound");
+        rc = op.kind == OpKind::Fft2D ? mlel_hip_fft2d(ctx, stream, &out, &imag, &in[0], &in[1], op.flag ? 1 : 0)
+                                      : mlel_hip_rfft2d(ctx, stream, &out, &imag, &in[0]);
+        break;
+    }
+    case OpKind::Gather: rc = mlel_hip_gather(ctx, stream, &out, &in[0], &in[1]); break;
+    case OpKind::Scatter: rc = mlel_hip_scatter(ctx, stream, &out, &in[0], &in[1], &in[2]); break;
+    case OpKind::Resize: rc = mlel_hip_resize(ctx, stream, &out, &in[0], &op.resize); break;
+    case OpKind::Reverse: rc = mlel_hip_reverse(ctx, stream, &out, &in[0], op.axis); break;
+    case OpKind::Tile: rc = mlel_hip_tile(ctx, stream, &out, &in[0]); break;
+    case OpKind::Select: rc = mlel_hip_select(ctx, stream, &out, &in[0], &in[1], &in[2]); break;
     case OpKind::FusedConv2D:
     case OpKind::FusedDepthwiseConv2D:
     case OpKind::FusedMatmul: {

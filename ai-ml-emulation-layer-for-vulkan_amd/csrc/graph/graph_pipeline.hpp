@@ -94,6 +94,7 @@ using TensorPtr = std::shared_ptr<TensorDescriptor>;
 enum class OpKind {
     Conv2D, DepthwiseConv2D, Matmul, Rescale, Clamp, Binary, Mul, Unary, Reduce, AvgPool2D, MaxPool2D, Table, Cast,
     Negate, Reshape, Transpose, Concat, Slice, Pad,
+    Argmax, ArithmeticRightShift, Conv3D, TransposeConv2D, Fft2D, Rfft2D, Gather, Scatter, Resize, Reverse, Tile, Select,
     // produced by the fusion pass only
     FusedConv2D, FusedDepthwiseConv2D, FusedMatmul, FusedRescaleAddRescale,
 };
@@ -118,6 +119,10 @@ class OpNode {
     mlel_rescale_attr rescale{};
     mlel_clamp_attr clamp{};
     mlel_pool2d_attr pool{};
+    mlel_conv3d_attr conv3d{};
+    mlel_tconv2d_attr tconv{};
+    mlel_resize_attr resize{};
+    bool flag = false;  // ARITHMETIC_RIGHT_SHIFT: round; FFT2D: inverse
     int32_t selector = 0;  // mlel_binary_op / mlel_unary_op / mlel_reduce_op
     uint32_t nanMode = MLEL_NAN_PROPAGATE, axis = 0, shift = 0, offset = 0;
     int32_t inputZeroPoint = 0, outputZeroPoint = 0, padConstInt = 0;

@@ -71,7 +71,7 @@ std::vector<Instruction> tokenize(const std::string &text) {
 }
 
 // ---- module objects
-enum class TypeKind { Int, Float, Bool, Array, Tensor, Pointer, Graph, Other };
+enum class TypeKind { Int, Float, Bool, Array, Tensor, Pointer, Graph, Struct, Other };
 
 struct Type {
     TypeKind kind = TypeKind::Other;
@@ -83,7 +83,7 @@ struct Type {
     bool shaped = false;        // Tensor
     std::vector<int64_t> dims;  // Tensor, when shaped
     int numInputs = 0;          // Graph
-    std::vector<std::string> interfaceTypes;  // Graph
+    std::vector<std::string> interfaceTypes;  // Graph; Struct: member types
 };
 
 enum class ConstKind { Scalar, Composite, Null, Replicate, GraphConstant };
@@ -127,8 +127,9 @@ uint16_t floatToHalfBits(const float f) {  // round to nearest even
 
 class Module {
   public:
-    Module(GraphPipeline &p, const std::vector<SpvBinding> &b, const std::vector<SpvConstant> &c)
-        : pipeline(p), bindings(b), constantData(c) {}
+    Module(GraphPipeline &p, const std::vector<SpvBinding> &b, const std::vector<SpvConstant> &c,
+           const std::vector<SpvSpecialization> &sp)
+        : pipeline(p), bindings(b), constantData(c), specializations(sp) {}
 
     SpvGraphInfo build(const std::vector<Instruction> &program);
 
@@ -160,18 +161,34 @@ class Module {
     TensorPtr tensorOperand(const Instruction &at, const std::string &id);
     void registerVariables(const Instruction &at);
     std::vector<int64_t> bindingDims(uint32_t set, uint32_t binding, uint32_t index) const;
-    TensorPtr resultTensor(const Instruction &inst);
+    TensorPtr resultTensor(const Instruction &inst, int member = -1);
+    std::map<std::pair<std::string, int>, std::string> extracts;  // (multi-result id, member) -> OpCompositeExtract id
     void decodeTosa(const Instruction &inst);
 
     GraphPipeline &pipeline;
     const std::vector<SpvBinding> &bindings;
     const std::vector<SpvConstant> &constantData;
+    const std::vector<SpvSpecialization> &specializations;
+    std::map<std::string, uint32_t> specIds;  // decorated ids -> SpecId
+    // a specialization constant keeps its default unless the caller supplies a value for its SpecId
+    // (reference: graph_layer.cpp:71-107 freezes them before the graph is decoded)
+    bool specialized(const std::string &id, uint64_t *bits) const {
+        const auto it = specIds.find(id);
+        if (it == specIds.end()) return false;
+        for (const auto &sp : specializations)
+            if (sp.specId == it->second) {
+                *bits = sp.bits;
+                return true;
+            }
+        return false;
+    }
     std::map<std::string, Type> types;
     std::map<std::string, Constant> consts;
     std::map<std::string, Variable> variables;
     std::vector<std::string> variableOrder;
     std::string tosaImport;
     std::map<std::string, TensorPtr> values;          // graph inputs, instruction results, materialised constants
+    std::map<std::string, std::vector<TensorPtr>> members;  // results of multi-result instructions
     std::map<std::string, std::vector<TensorPtr>> outputTargets;  // value id -> output tensors it is routed to
     bool variablesRegistered = false;
 };
@@ -242,6 +259,8 @@ void Module::declare(const Instruction &inst) {
         if (a[1] == "DescriptorSet" && a.size() >= 3) {
             variables[a[0]].set = static_cast<uint32_t>(std::strtoul(a[2].c_str(), nullptr, 0));
             variables[a[0]].hasSet = true;
+        } else if (a[1] == "SpecId" && a.size() >= 3) {
+            specIds[a[0]] = static_cast<uint32_t>(std::strtoul(a[2].c_str(), nullptr, 0));
         } else if (a[1] == "Binding" && a.size() >= 3) {
             variables[a[0]].binding = static_cast<uint32_t>(std::strtoul(a[2].c_str(), nullptr, 0));
             variables[a[0]].hasBinding = true;
@@ -299,6 +318,11 @@ void Module::declare(const Instruction &inst) {
         t.numInputs = std::atoi(a[0].c_str());
         t.interfaceTypes.assign(a.begin() + 1, a.end());
         types[inst.result] = t;
+    } else if (op == "OpTypeStruct") {
+        Type t;
+        t.kind = TypeKind::Struct;
+        t.interfaceTypes = a;
+        types[inst.result] = t;
     } else if (op.rfind("OpType", 0) == 0) {
         types[inst.result] = Type{};  // struct, vector, ...: only ever named, never inspected
     } else if (op == "OpConstant" || op == "OpSpecConstant") {
@@ -306,6 +330,11 @@ void Module::declare(const Instruction &inst) {
         Constant c;
         c.type = a[0];
         c.bits = parseLiteral(inst, typeOf(inst, a[0]), a[1]);
+        uint64_t replaced = 0;
+        if (op == "OpSpecConstant" && specialized(inst.result, &replaced)) {
+            const Type &t = typeOf(inst, a[0]);
+            c.bits = t.width >= 64 ? replaced : replaced & ((uint64_t(1) << t.width) - 1);
+        }
         consts[inst.result] = c;
     } else if (op == "OpConstantTrue" || op == "OpConstantFalse" || op == "OpSpecConstantTrue" ||
                op == "OpSpecConstantFalse") {
@@ -313,6 +342,8 @@ void Module::declare(const Instruction &inst) {
         Constant c;
         c.type = a[0];
         c.bits = op.find("True") != std::string::npos ? 1 : 0;
+        uint64_t replaced = 0;
+        if (op.rfind("OpSpec", 0) == 0 && specialized(inst.result, &replaced)) c.bits = replaced != 0;
         consts[inst.result] = c;
     } else if (op == "OpConstantNull") {
         need(1);
@@ -516,11 +547,22 @@ TensorPtr Module::tensorOperand(const Instruction &at, const std::string &id) {
     return tensor;
 }
 
-TensorPtr Module::resultTensor(const Instruction &inst) {
-    const auto routed = outputTargets.find(inst.result);
-    if (routed != outputTargets.end()) return routed->second.front();  // the operator writes the graph output itself
-    const Type &t = typeOf(inst, inst.operands[0]);
-    if (t.kind != TypeKind::Tensor) fail(inst, "result is not a tensor (multi-result operators are not supported)");
+// The tensor an instruction result (or member `member` of a multi-result instruction) is written to: the graph
+// output it is routed to, else a new session tensor of the declared type.
+TensorPtr Module::resultTensor(const Instruction &inst, const int member) {
+    std::string valueId = inst.result, typeId = inst.operands[0];
+    if (member >= 0) {
+        const Type &st = typeOf(inst, typeId);
+        if (st.kind != TypeKind::Struct || static_cast<size_t>(member) >= st.interfaceTypes.size())
+            fail(inst, "expected a result structure with at least " + std::to_string(member + 1) + " members");
+        typeId = st.interfaceTypes[static_cast<size_t>(member)];
+        const auto ex = extracts.find({inst.result, member});
+        valueId = ex == extracts.end() ? std::string() : ex->second;
+    }
+    const auto routed = outputTargets.find(valueId);
+    if (!valueId.empty() && routed != outputTargets.end()) return routed->second.front();
+    const Type &t = typeOf(inst, typeId);
+    if (t.kind != TypeKind::Tensor) fail(inst, "result is not a tensor");
     if (!t.shaped) fail(inst, "an intermediate result needs a shaped tensor type");
     return pipeline.makeTensor(dtypeOfScalarType(inst, typeOf(inst, t.element)), t.dims, {});
 }
@@ -543,8 +585,20 @@ void Module::decodeTosa(const Instruction &inst) {
         if (v.empty()) fail(inst, name + ": empty constant");
         return v[0];
     };
-    const TensorPtr out = resultTensor(inst);
     const std::string dbg = inst.result.size() > 1 ? inst.result.substr(1) : name;
+    if (name == "FFT2D" || name == "RFFT2D") {  // two results, picked apart by OpCompositeExtract
+        const TensorPtr real = resultTensor(inst, 0), imag = resultTensor(inst, 1);
+        if (name == "FFT2D") {
+            need(4);  // inverse localBound real imag
+            pipeline.makeFft2D(T(2), T(3), real, imag, S(0) != 0, dbg);
+        } else {
+            need(2);  // localBound input
+            pipeline.makeRfft2D(T(1), real, imag, dbg);
+        }
+        members[inst.result] = {real, imag};
+        return;
+    }
+    const TensorPtr out = resultTensor(inst);
 
     using Unary = void (GraphPipeline::*)(const TensorPtr &, const TensorPtr &, const std::string &);
     using Binary = void (GraphPipeline::*)(const TensorPtr &, const TensorPtr &, const TensorPtr &, const std::string &);
@@ -669,6 +723,12 @@ void Module::decodeTosa(const Instruction &inst) {
     } else if (name == "GATHER") {
         need(2);
         pipeline.makeGather(T(0), T(1), out, dbg);
+    } else if (name == "SCATTER") {
+        need(3);  // valuesIn indices input
+        pipeline.makeScatter(T(2), T(0), T(1), out, dbg);
+    } else if (name == "RESIZE") {
+        need(5);  // mode input scale offset border
+        pipeline.makeResize(T(1), out, to32(V(2)), to32(V(3)), to32(V(4)), static_cast<uint32_t>(S(0)), dbg);
     } else {
         fail(inst, "TOSA operator " + name + " is not decoded by this front-end");
     }
@@ -721,6 +781,10 @@ SpvGraphInfo Module::build(const std::vector<Instruction> &program) {
         return tensor;
     };
 
+    for (const auto *inst : body)
+        if (inst->opcode == "OpCompositeExtract" && inst->operands.size() >= 3)
+            extracts[{inst->operands[1], std::atoi(inst->operands[2].c_str())}] = inst->result;
+
     // pass 2: which values are routed to which outputs (an operator result routed to an output is written in place)
     struct Route {
         const Instruction *inst;
@@ -767,10 +831,17 @@ SpvGraphInfo Module::build(const std::vector<Instruction> &program) {
             if (inst->operands[1] != tosaImport) fail(*inst, "instruction set " + inst->operands[1] + " is not TOSA.001000.1");
             decodeTosa(*inst);
             info.instructions++;
+        } else if (inst->opcode == "OpCompositeExtract") {
+            if (inst->operands.size() < 3) fail(*inst, "expects a type, a composite and an index");
+            const auto m = members.find(inst->operands[1]);
+            const size_t index = static_cast<size_t>(std::atoi(inst->operands[2].c_str()));
+            if (m == members.end() || index >= m->second.size()) fail(*inst, inst->operands[1] + " has no such member");
+            values[inst->result] = m->second[index];
         } else if (inst->opcode == "OpGraphSetOutputARM") {
             continue;
         } else {
-            fail(*inst, "only OpGraphInputARM, OpExtInst and OpGraphSetOutputARM may appear in a graph body");
+            fail(*inst, "only OpGraphInputARM, OpExtInst, OpCompositeExtract and OpGraphSetOutputARM may appear in a "
+                        "graph body");
         }
     }
 
@@ -797,8 +868,9 @@ SpvGraphInfo Module::build(const std::vector<Instruction> &program) {
 }  // namespace
 
 SpvGraphInfo loadSpirvAssembly(GraphPipeline &pipeline, const std::string &text, const std::vector<SpvBinding> &bindings,
-                               const std::vector<SpvConstant> &constants) {
-    Module module(pipeline, bindings, constants);
+                               const std::vector<SpvConstant> &constants,
+                               const std::vector<SpvSpecialization> &specializations) {
+    Module module(pipeline, bindings, constants, specializations);
     return module.build(tokenize(text));
 }
 

@@ -34,6 +34,12 @@ struct SpvConstant {
     std::vector<int64_t> dims;
 };
 
+// value of the specialization constant decorated `SpecId specId` (the bit pattern of its type; booleans 0 / 1)
+struct SpvSpecialization {
+    uint32_t specId;
+    uint64_t bits;
+};
+
 struct SpvGraphInfo {
     std::string entryPoint;
     std::vector<std::array<uint32_t, 3>> inputs;   // {set, binding, arrayIndex} per graph input, in index order
@@ -42,8 +48,9 @@ struct SpvGraphInfo {
 };
 
 // Throws std::runtime_error with the offending line for malformed text, unknown instructions of the graph body,
-// missing shapes or constants; operators the HIP backend has no kernel for throw from GraphPipeline::make<Op>.
+// missing shapes or constants.
 SpvGraphInfo loadSpirvAssembly(GraphPipeline &pipeline, const std::string &text, const std::vector<SpvBinding> &bindings,
-                               const std::vector<SpvConstant> &constants);
+                               const std::vector<SpvConstant> &constants,
+                               const std::vector<SpvSpecialization> &specializations = {});
 
 }  // namespace mlel::graph

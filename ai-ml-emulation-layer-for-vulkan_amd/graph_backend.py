@@ -23,6 +23,10 @@ class SpvBinding(C.Structure):
                 ("dims", C.POINTER(C.c_int64))]
 
 
+class SpvSpecialization(C.Structure):
+    _fields_ = [("spec_id", C.c_uint32), ("bits", C.c_uint64)]
+
+
 class SpvConstant(C.Structure):
     _fields_ = [("id", C.c_uint32), ("rank", C.c_int32), ("dims", C.POINTER(C.c_int64)), ("data", C.c_void_p)]
 
@@ -50,7 +54,8 @@ def load_graph_library():
         lib.mlel_graph_make_op.argtypes = [_V, C.c_char_p, C.POINTER(C.c_int), C.c_int, C.POINTER(C.c_int), C.c_int,
                                            _I64P, C.c_int, C.POINTER(C.c_double), C.c_int, C.c_char_p]
         lib.mlel_graph_load_spvasm.argtypes = [_V, C.c_char_p, C.c_size_t, C.POINTER(SpvBinding), C.c_int,
-                                               C.POINTER(SpvConstant), C.c_int, C.POINTER(C.c_uint32), C.c_int,
+                                               C.POINTER(SpvConstant), C.c_int, C.POINTER(SpvSpecialization), C.c_int,
+                                               C.POINTER(C.c_uint32), C.c_int,
                                                C.POINTER(C.c_int), C.POINTER(C.c_int)]
         lib.mlel_graph_tensor_info.argtypes = [_V, C.c_int, C.POINTER(C.c_int32), _I64P]
         lib.mlel_graph_finalize.argtypes = [_V, C.c_int]
@@ -168,10 +173,11 @@ class Graph:
                                                 _i64(iattr), len(iattr), fa, len(fattr), debug_name.encode()))
 
     # ---- SPIR-V assembly front-end
-    def load_spvasm(self, text, bindings=None, constants=None, names=None):
+    def load_spvasm(self, text, bindings=None, constants=None, names=None, specializations=None):
         """Decodes a SPIR-V assembly module into this graph.  `bindings`: {(set, binding, element): shape} for
         interface tensors of unshaped type; `constants`: {graph constant id: ndarray}; `names`: {(set, binding,
-        element): name} for the externals (default "s<set>b<binding>e<element>").  Returns (input names, output
+        element): name} for the externals (default "s<set>b<binding>e<element>"); `specializations`: {SpecId: value
+        bits}.  Returns (input names, output
         names, number of TOSA instructions)."""
         bindings, constants, names = bindings or {}, constants or {}, names or {}
         keep = []
@@ -186,11 +192,16 @@ class Graph:
             dims = _i64(array.shape)
             keep += [dims, array]
             carr[i] = SpvConstant(cid, array.ndim, dims, array.ctypes.data)
+        specializations = specializations or {}
+        sarr = (SpvSpecialization * max(1, len(specializations)))()
+        for i, (sid, bits) in enumerate(specializations.items()):
+            sarr[i] = SpvSpecialization(int(sid), int(bits) & (2 ** 64 - 1))
         io = (C.c_uint32 * 3072)()
         n_in, n_out = C.c_int(), C.c_int()
         raw = text.encode()
         count = self._check(self.lib.mlel_graph_load_spvasm(self.g, raw, len(raw), barr, len(bindings), carr,
-                                                            len(constants), io, 3072, C.byref(n_in), C.byref(n_out)))
+                                                            len(constants), sarr, len(specializations), io, 3072,
+                                                            C.byref(n_in), C.byref(n_out)))
         result = []
         for k in range(n_in.value + n_out.value):
             key = (int(io[3 * k]), int(io[3 * k + 1]), int(io[3 * k + 2]))

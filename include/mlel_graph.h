@@ -53,7 +53,8 @@ int mlel_graph_make_op(mlel_graph *g, const char *tosa_name, const int *inputs, 
  * GraphTosa10ExtInst::handleOp, graph/graph_tosa_1_0_ext_inst.cpp:37-1032; constants and tensor shapes that the
  * reference takes from VkDataGraphPipelineConstantARM / VkTensorDescriptionARM, graph_layer.cpp:343-420, are the
  * `constants` / `bindings` arguments).  `bindings` give the shape of every interface tensor whose SPIR-V type is
- * unshaped; `constants` the payload of every OpGraphConstantARM.  On return io[0..3*n_in) holds {set, binding,
+ * unshaped; `constants` the payload of every OpGraphConstantARM; `specializations` the values of specialization
+ * constants that differ from their defaults (reference: graph_layer.cpp:71-107).  On return io[0..3*n_in) holds {set, binding,
  * array element} of the graph inputs in index order, followed by the same for the outputs.  Returns the number of
  * TOSA instructions decoded. */
 typedef struct mlel_graph_spv_binding {
@@ -67,8 +68,13 @@ typedef struct mlel_graph_spv_constant {
     const int64_t *dims;
     const void *data;
 } mlel_graph_spv_constant;
+typedef struct mlel_graph_spv_specialization {
+    uint32_t spec_id; /* the SpecId decoration */
+    uint64_t bits;    /* value as the bit pattern of the constant's type; booleans 0 / 1 */
+} mlel_graph_spv_specialization;
 int mlel_graph_load_spvasm(mlel_graph *g, const char *text, size_t length, const mlel_graph_spv_binding *bindings,
-                           int n_bindings, const mlel_graph_spv_constant *constants, int n_constants, uint32_t *io,
+                           int n_bindings, const mlel_graph_spv_constant *constants, int n_constants,
+                           const mlel_graph_spv_specialization *specializations, int n_specializations, uint32_t *io,
                            int io_capacity, int *n_inputs, int *n_outputs);
 /* dtype, rank and dimensions of a tensor handle (dims: room for MLEL_MAX_RANK entries); returns the rank. */
 int mlel_graph_tensor_info(mlel_graph *g, int tensor, int32_t *dtype, int64_t *dims);

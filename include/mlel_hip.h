@@ -125,6 +125,35 @@ typedef struct mlel_pool2d_attr {
     uint32_t nan_mode; /* MAX only */
 } mlel_pool2d_attr;
 
+/* CONV3D (reference: conv3d.comp:29-35 push constants).  pad = {front, back, top, bottom, left, right};
+ * stride = {d, y, x}; dilation = {d, y, x}. */
+typedef struct mlel_conv3d_attr {
+    int32_t input_zp;
+    int32_t weight_zp;
+    int32_t pad[6];
+    int32_t stride[3];
+    int32_t dilation[3];
+    uint32_t acc_type; /* MLEL_ACC_* */
+} mlel_conv3d_attr;
+
+/* TRANSPOSE_CONV2D (reference: transpose_conv2d.comp:25-30).  out_pad = {top, bottom, left, right}; stride = {y, x}. */
+typedef struct mlel_tconv2d_attr {
+    int32_t input_zp;
+    int32_t weight_zp;
+    int32_t out_pad[4];
+    int32_t stride[2];
+    uint32_t acc_type; /* MLEL_ACC_* */
+} mlel_tconv2d_attr;
+
+/* RESIZE (reference: resize.comp:21-44).  scale = {y_n, y_d, x_n, x_d}; offset = {y, x}; border = {y, x}. */
+enum { MLEL_RESIZE_NEAREST = 1, MLEL_RESIZE_BILINEAR = 2 };
+typedef struct mlel_resize_attr {
+    int32_t scale[4];
+    int32_t offset[2];
+    int32_t border[2];
+    uint32_t mode; /* MLEL_RESIZE_* */
+} mlel_resize_attr;
+
 /* Elementwise binary operator selector.  One value per `%operation%` string the reference substitutes into
  * elementwise_binary.comp (reference: graph/compute_graph_op.cpp:2527-2946). */
 typedef enum mlel_binary_op {
@@ -309,6 +338,45 @@ int mlel_hip_slice(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const ml
                    const uint32_t *start);
 int mlel_hip_pad(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
                  const mlel_tensor *padding, double pad_const, int32_t pad_const_int);
+
+/* ---- the remaining TOSA operators: one thread per output element, any strides ---- */
+
+/* ARGMAX: output int32 with the axis removed; first maximum wins.  Replaces class ArgMax, argmax.comp:26-66. */
+int mlel_hip_argmax(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis,
+                    uint32_t nan_mode);
+/* ARITHMETIC_RIGHT_SHIFT with size-1 broadcast.  Replaces class ArithmeticRightShift,
+ * arithmetic_right_shift.comp:22-48. */
+int mlel_hip_arithmetic_right_shift(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1,
+                                    const mlel_tensor *in2, uint32_t round);
+/* CONV3D: NDHWC x ODHWI.  Replaces class Conv3D (reference: graph/compute_graph_op.cpp:1029-1110), conv3d.comp:37-104. */
+int mlel_hip_conv3d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                    const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv3d_attr *attr);
+/* TRANSPOSE_CONV2D: NHWC x OHWI.  Replaces class TransposeConv2D (reference: graph/compute_graph_op.cpp:2211-2290),
+ * transpose_conv2d.comp:31-70. */
+int mlel_hip_transpose_conv2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                              const mlel_tensor *weights, const mlel_tensor *bias, const mlel_tconv2d_attr *attr);
+/* FFT2D / RFFT2D on float32 [N, H, W]: direct evaluation of the transform sums.  Replace classes Fft2D / Rfft2D
+ * (reference: graph/compute_graph_op.cpp:1303-1381, 1931-1990), fft2d.comp:17-52, rfft2d.comp:13-71. */
+int mlel_hip_fft2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out_real, const mlel_tensor *out_imag,
+                   const mlel_tensor *in_real, const mlel_tensor *in_imag, int32_t inverse);
+int mlel_hip_rfft2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out_real, const mlel_tensor *out_imag,
+                    const mlel_tensor *in);
+/* GATHER: out[n,w,c] = values[n, indices[n,w], c].  SCATTER: out = values_in with rows named by indices replaced
+ * by the rows of input.  Replace classes Gather / Scatter, gather.comp:13-25, scatter.comp:14-34. */
+int mlel_hip_gather(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *values,
+                    const mlel_tensor *indices);
+int mlel_hip_scatter(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *values_in,
+                     const mlel_tensor *indices, const mlel_tensor *input);
+/* RESIZE (nearest / bilinear, integer or float).  Replaces class Resize (reference:
+ * graph/compute_graph_op.cpp:1820-1925), resize.comp:57-134. */
+int mlel_hip_resize(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                    const mlel_resize_attr *attr);
+/* REVERSE, TILE, SELECT.  Replace the classes and shaders of the same names (reverse.comp:14-30, tile.comp:12-30,
+ * select.comp:15-41). */
+int mlel_hip_reverse(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis);
+int mlel_hip_tile(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in);
+int mlel_hip_select(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *condition,
+                    const mlel_tensor *in_true, const mlel_tensor *in_false);
 
 /* ---- fused entry points (chosen only by the host-side fusion pass; no counterpart in the reference, which
  * runs one dispatch per TOSA instruction: graph/compute_graph_op.cpp:2500-2509).  Each equals, bit for bit,

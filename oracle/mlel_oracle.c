@@ -1287,3 +1287,456 @@ int mlel_cpu_pad(const mlel_tensor *out, const mlel_tensor *in, const mlel_tenso
     }
     return 0;
 }
+
+/* ============================================================================================================
+ * The remaining TOSA operators
+ * ========================================================================================================== */
+
+/* one multiply-accumulate of a convolution in the accumulator type (as in mlel_cpu_conv2d above) */
+static inline void conv_mac(uint32_t acc_type, int64_t *iacc, double *dacc, const mlel_tensor *in, const int64_t *xi,
+                            const mlel_tensor *w, const int64_t *wi, int32_t zi, int32_t zw) {
+    if (!acc_is_float(acc_type)) {
+        const int64_t v = ld_i(in, xi) - zi;
+        const int64_t ww = ld_i(w, wi) - zw;
+        if (acc_type == MLEL_ACC_I32)
+            *iacc = wadd32((int32_t)*iacc, wmul32((int32_t)v, (int32_t)ww));
+        else
+            *iacc = wadd64(*iacc, wmul64(v, ww));
+    } else {
+        double v = ld_f(in, xi), ww = ld_f(w, wi);
+        if (acc_type == MLEL_ACC_F16) {
+            v = rnd_f16(v);
+            ww = rnd_f16(ww);
+        }
+        const double p = rnd_f32(rnd_f32(v - (double)zi) * rnd_f32(ww - (double)zw));
+        *dacc = acc_type == MLEL_ACC_F16 ? rnd_f16(*dacc + rnd_f16(p)) : rnd_f32(*dacc + p);
+    }
+}
+
+static inline void conv_finish(uint32_t acc_type, int64_t iacc, double dacc, const mlel_tensor *bias, int64_t oc,
+                               const mlel_tensor *out, const int64_t *o) {
+    const int64_t bi[1] = {bias->dims[0] == 1 ? 0 : oc};
+    if (!acc_is_float(acc_type)) {
+        const int64_t b = ld_i(bias, bi);
+        st_i(out, o, acc_type == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)iacc, (int32_t)b) : wadd64(iacc, b));
+    } else {
+        const double b = ld_f(bias, bi);
+        st_f(out, o, acc_type == MLEL_ACC_F16 ? rnd_f16(dacc + rnd_f16(b)) : rnd_f32(dacc + b));
+    }
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * CONV3D (reference: conv3d.comp:37-104): NDHWC input, ODHWI weights; taps outside the input contribute nothing
+ * ---------------------------------------------------------------------------------------------------------- */
+int mlel_cpu_conv3d(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w, const mlel_tensor *bias,
+                    const mlel_conv3d_attr *a) {
+    CHECK(out, "conv3d out");
+    CHECK(in, "conv3d in");
+    CHECK(w, "conv3d weights");
+    CHECK(bias, "conv3d bias");
+    if (out->rank != 5 || in->rank != 5 || w->rank != 5 || bias->rank != 1)
+        return fail(MLEL_ERR_INVALID, "conv3d: ranks must be 5,5,5,1");
+    if (a->acc_type < 1 || a->acc_type > 4) return fail(MLEL_ERR_INVALID, "Unsupported acc type %u", a->acc_type);
+    const int64_t D = in->dims[1], H = in->dims[2], W = in->dims[3], IC = w->dims[4];
+    const int64_t KD = w->dims[1], KH = w->dims[2], KW = w->dims[3];
+    const int64_t total = numel(out);
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK];
+        unflatten(out, flat, o);
+        int64_t iacc = 0;
+        double dacc = 0.0;
+        for (int64_t kd = 0; kd < KD; kd++) {
+            const int64_t d = o[1] * a->stride[0] - a->pad[0] + kd * a->dilation[0];
+            if (d < 0 || d >= D) continue;
+            for (int64_t ky = 0; ky < KH; ky++) {
+                const int64_t y = o[2] * a->stride[1] - a->pad[2] + ky * a->dilation[1];
+                if (y < 0 || y >= H) continue;
+                for (int64_t kx = 0; kx < KW; kx++) {
+                    const int64_t x = o[3] * a->stride[2] - a->pad[4] + kx * a->dilation[2];
+                    if (x < 0 || x >= W) continue;
+                    for (int64_t ic = 0; ic < IC; ic++) {
+                        const int64_t xi[5] = {o[0], d, y, x, ic};
+                        const int64_t wi[5] = {o[4], kd, ky, kx, ic};
+                        conv_mac(a->acc_type, &iacc, &dacc, in, xi, w, wi, a->input_zp, a->weight_zp);
+                    }
+                }
+            }
+        }
+        conv_finish(a->acc_type, iacc, dacc, bias, o[4], out, o);
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * TRANSPOSE_CONV2D (reference: transpose_conv2d.comp:31-70): output position oy receives input row iy through
+ * kernel row ky when oy - out_pad_top - ky == iy * stride_y; the accumulator starts from the bias
+ * ---------------------------------------------------------------------------------------------------------- */
+int mlel_cpu_transpose_conv2d(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
+                              const mlel_tensor *bias, const mlel_tconv2d_attr *a) {
+    CHECK(out, "transpose_conv2d out");
+    CHECK(in, "transpose_conv2d in");
+    CHECK(w, "transpose_conv2d weights");
+    CHECK(bias, "transpose_conv2d bias");
+    if (out->rank != 4 || in->rank != 4 || w->rank != 4 || bias->rank != 1)
+        return fail(MLEL_ERR_INVALID, "transpose_conv2d: ranks must be 4,4,4,1");
+    if (a->acc_type < 1 || a->acc_type > 4) return fail(MLEL_ERR_INVALID, "Unsupported acc type %u", a->acc_type);
+    if (a->stride[0] <= 0 || a->stride[1] <= 0) return fail(MLEL_ERR_INVALID, "transpose_conv2d: stride must be positive");
+    const int64_t H = in->dims[1], W = in->dims[2], IC = in->dims[3], KH = w->dims[1], KW = w->dims[2];
+    const int64_t total = numel(out);
+    const int facc = acc_is_float(a->acc_type);
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK];
+        unflatten(out, flat, o);
+        const int64_t bi[1] = {bias->dims[0] == 1 ? 0 : o[3]};
+        int64_t iacc = facc ? 0 : ld_i(bias, bi);
+        if (!facc && a->acc_type == MLEL_ACC_I32) iacc = (int32_t)iacc;
+        double dacc = facc ? ld_f(bias, bi) : 0.0;
+        if (a->acc_type == MLEL_ACC_F16) dacc = rnd_f16(dacc);
+        for (int64_t ky = 0; ky < KH; ky++) {
+            for (int64_t kx = 0; kx < KW; kx++) {
+                int64_t iy = o[1] - a->out_pad[0] - ky, ix = o[2] - a->out_pad[2] - kx;
+                if (iy % a->stride[0] != 0 || ix % a->stride[1] != 0) continue; /* C remainder, as in GLSL */
+                iy /= a->stride[0];
+                ix /= a->stride[1];
+                if (iy < 0 || ix < 0 || iy >= H || ix >= W) continue;
+                for (int64_t ic = 0; ic < IC; ic++) {
+                    const int64_t xi[4] = {o[0], iy, ix, ic};
+                    const int64_t wi[4] = {o[3], ky, kx, ic};
+                    conv_mac(a->acc_type, &iacc, &dacc, in, xi, w, wi, a->input_zp, a->weight_zp);
+                }
+            }
+        }
+        if (!facc)
+            st_i(out, o, iacc);
+        else
+            st_f(out, o, dacc);
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * ARGMAX (reference: argmax.comp:26-66): int32 output without the axis; the running maximum starts at the lowest
+ * value of the type and only a strictly greater value replaces it, so the first maximum wins
+ * ---------------------------------------------------------------------------------------------------------- */
+int mlel_cpu_argmax(const mlel_tensor *out, const mlel_tensor *in, uint32_t axis, uint32_t nan_mode) {
+    CHECK(out, "argmax out");
+    CHECK(in, "argmax in");
+    if ((int)axis >= in->rank || out->rank != in->rank - 1) return fail(MLEL_ERR_INVALID, "argmax: bad axis or ranks");
+    const int64_t total = numel(out), len = in->dims[axis];
+    const int isf = dt_is_float(in->dtype);
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK], ii[MLEL_MAX_RANK];
+        unflatten(out, flat, o);
+        for (uint32_t i = 0; i < axis; i++) ii[i] = o[i];
+        for (int i = (int)axis; i < out->rank; i++) ii[i + 1] = o[i];
+        int64_t best = 0;
+        if (isf) {
+            /* the shader starts from the lowest FINITE value of the type, so a -inf input never wins */
+            double mx = in->dtype == MLEL_F16 ? -65504.0 : (in->dtype == MLEL_BF16 ? -3.3895313892515355e38 : -3.4028234663852886e38);
+            for (int64_t i = 0; i < len; i++) {
+                ii[axis] = i;
+                const double v = ld_f(in, ii);
+                if (isnan(v)) {
+                    if (nan_mode == MLEL_NAN_IGNORE) continue;
+                    best = i;
+                    break;
+                }
+                if (v > mx) {
+                    mx = v;
+                    best = i;
+                }
+            }
+        } else {
+            int64_t mx = dt_lowest(in->dtype);
+            for (int64_t i = 0; i < len; i++) {
+                ii[axis] = i;
+                const int64_t v = ld_i(in, ii);
+                if (v > mx) {
+                    mx = v;
+                    best = i;
+                }
+            }
+        }
+        st_i(out, o, best);
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * ARITHMETIC_RIGHT_SHIFT (reference: arithmetic_right_shift.comp:22-48)
+ * ---------------------------------------------------------------------------------------------------------- */
+int mlel_cpu_arithmetic_right_shift(const mlel_tensor *out, const mlel_tensor *in1, const mlel_tensor *in2,
+                                    uint32_t round) {
+    CHECK(out, "arithmetic_right_shift out");
+    CHECK(in1, "arithmetic_right_shift in1");
+    CHECK(in2, "arithmetic_right_shift in2");
+    if (!dt_is_int(out->dtype)) return fail(MLEL_ERR_INVALID, "arithmetic_right_shift: integer types only");
+    const int64_t total = numel(out);
+    const int bits = 8 * dt_size(out->dtype);
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK], a[MLEL_MAX_RANK], b[MLEL_MAX_RANK];
+        unflatten(out, flat, o);
+        broadcast_idx(in1, o, a);
+        broadcast_idx(in2, o, b);
+        const int64_t v = ld_i(in1, a), s = ld_i(in2, b);
+        const int sh = (int)(s & (bits - 1)); /* shift counts are taken modulo the width on every target tested */
+        int64_t r = asr64(v, sh);
+        if (round && s > 0 && ((asr64(v, (int)((s - 1) & (bits - 1))) & 1) != 0)) r++;
+        st_i(out, o, narrow_to(out->dtype, r));
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * GATHER / SCATTER (reference: gather.comp:13-25, scatter.comp:14-34)
+ * ---------------------------------------------------------------------------------------------------------- */
+int mlel_cpu_gather(const mlel_tensor *out, const mlel_tensor *values, const mlel_tensor *indices) {
+    CHECK(out, "gather out");
+    CHECK(values, "gather values");
+    CHECK(indices, "gather indices");
+    if (out->rank != 3 || values->rank != 3 || indices->rank != 2) return fail(MLEL_ERR_INVALID, "gather: ranks must be 3,3,2");
+    const int64_t total = numel(out);
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK];
+        unflatten(out, flat, o);
+        const int64_t xi[2] = {o[0], o[1]};
+        const int64_t k = (int64_t)(uint32_t)ld_i(indices, xi);
+        const int64_t vi[3] = {o[0], k, o[2]};
+        copy_elem(out, o, values, vi);
+    }
+    return 0;
+}
+
+int mlel_cpu_scatter(const mlel_tensor *out, const mlel_tensor *values_in, const mlel_tensor *indices,
+                     const mlel_tensor *input) {
+    CHECK(out, "scatter out");
+    CHECK(values_in, "scatter values_in");
+    CHECK(indices, "scatter indices");
+    CHECK(input, "scatter input");
+    if (out->rank != 3 || values_in->rank != 3 || indices->rank != 2 || input->rank != 3)
+        return fail(MLEL_ERR_INVALID, "scatter: ranks must be 3,3,2,3");
+    const int64_t total = numel(out), W = indices->dims[1];
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK];
+        unflatten(out, flat, o);
+        int64_t w_hit = -1;
+        for (int64_t wv = 0; wv < W && w_hit < 0; wv++) {
+            const int64_t xi[2] = {o[0], wv};
+            if ((int64_t)(uint32_t)ld_i(indices, xi) == o[1]) w_hit = wv; /* the first matching row wins */
+        }
+        if (w_hit < 0) {
+            copy_elem(out, o, values_in, o);
+        } else {
+            const int64_t ii[3] = {o[0], w_hit, o[2]};
+            copy_elem(out, o, input, ii);
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * REVERSE / TILE / SELECT (reference: reverse.comp:14-30, tile.comp:12-30, select.comp:15-41)
+ * ---------------------------------------------------------------------------------------------------------- */
+int mlel_cpu_reverse(const mlel_tensor *out, const mlel_tensor *in, uint32_t axis) {
+    CHECK(out, "reverse out");
+    CHECK(in, "reverse in");
+    if (out->rank != in->rank || (int)axis >= out->rank) return fail(MLEL_ERR_INVALID, "reverse: bad rank or axis");
+    const int64_t total = numel(out);
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK], ii[MLEL_MAX_RANK];
+        unflatten(out, flat, ii); /* the shader walks the output grid, reads the input there and writes mirrored */
+        for (int i = 0; i < out->rank; i++) o[i] = ii[i];
+        o[axis] = out->dims[axis] - 1 - ii[axis];
+        copy_elem(out, o, in, ii);
+    }
+    return 0;
+}
+
+int mlel_cpu_tile(const mlel_tensor *out, const mlel_tensor *in) {
+    CHECK(out, "tile out");
+    CHECK(in, "tile in");
+    if (out->rank != in->rank) return fail(MLEL_ERR_INVALID, "tile: ranks differ");
+    const int64_t total = numel(out);
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK], ii[MLEL_MAX_RANK];
+        unflatten(out, flat, o);
+        for (int i = 0; i < out->rank; i++) ii[i] = o[i] % in->dims[i];
+        copy_elem(out, o, in, ii);
+    }
+    return 0;
+}
+
+int mlel_cpu_select(const mlel_tensor *out, const mlel_tensor *condition, const mlel_tensor *in_true,
+                    const mlel_tensor *in_false) {
+    CHECK(out, "select out");
+    CHECK(condition, "select condition");
+    CHECK(in_true, "select in_true");
+    CHECK(in_false, "select in_false");
+    const int64_t total = numel(out);
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK], c[MLEL_MAX_RANK], ii[MLEL_MAX_RANK];
+        unflatten(out, flat, o);
+        broadcast_idx(condition, o, c);
+        const mlel_tensor *src = ld_i(condition, c) != 0 ? in_true : in_false;
+        broadcast_idx(src, o, ii);
+        copy_elem(out, o, src, ii);
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * RESIZE (reference: resize.comp:57-134).  Coordinates are computed in int32 and narrowed to int16 exactly where
+ * the shader narrows them; integer types interpolate with integer weights (unit = scale numerator), floats with
+ * weights in [0, 1].
+ * ---------------------------------------------------------------------------------------------------------- */
+static inline int32_t idiv_floor(int32_t n, int32_t d) {
+    int32_t r = n / d;
+    if ((int64_t)r * d > n) r--;
+    return r;
+}
+
+int mlel_cpu_resize(const mlel_tensor *out, const mlel_tensor *in, const mlel_resize_attr *a) {
+    CHECK(out, "resize out");
+    CHECK(in, "resize in");
+    if (out->rank != 4 || in->rank != 4) return fail(MLEL_ERR_INVALID, "resize: ranks must be 4");
+    if (a->scale[0] <= 0 || a->scale[2] <= 0) return fail(MLEL_ERR_INVALID, "resize: scale numerators must be positive");
+    if (a->mode != MLEL_RESIZE_NEAREST && a->mode != MLEL_RESIZE_BILINEAR) return fail(MLEL_ERR_INVALID, "resize: bad mode");
+    const int64_t total = numel(out);
+    const int isf = dt_is_float(out->dtype);
+    const int32_t yn = a->scale[0], yd = a->scale[1], xn = a->scale[2], xd = a->scale[3];
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK];
+        unflatten(out, flat, o);
+        const int32_t y = (int32_t)((uint32_t)o[1] * (uint32_t)yd + (uint32_t)a->offset[0]);
+        const int16_t iy = (int16_t)idiv_floor(y, yn);
+        const int16_t ry = (int16_t)(y - iy * yn);
+        const int32_t x = (int32_t)((uint32_t)o[2] * (uint32_t)xd + (uint32_t)a->offset[1]);
+        const int16_t ix = (int16_t)idiv_floor(x, xn);
+        const int16_t rx = (int16_t)(x - ix * xn);
+        const int16_t iy0 = (int16_t)(iy > 0 ? iy : 0);
+        const int16_t ix0 = (int16_t)(ix > 0 ? ix : 0);
+        /* min(iy + 1, H - 1) is evaluated in unsigned arithmetic in the shader (the shape is unsigned) */
+        const uint32_t uy1 = (uint32_t)(int32_t)(iy + 1), ux1 = (uint32_t)(int32_t)(ix + 1);
+        const uint32_t hy = (uint32_t)in->dims[1] - 1u, hx = (uint32_t)in->dims[2] - 1u;
+        const int16_t iy1 = (int16_t)(uy1 < hy ? uy1 : hy), ix1 = (int16_t)(ux1 < hx ? ux1 : hx);
+        const int64_t p00[4] = {o[0], iy0, ix0, o[3]}, p01[4] = {o[0], iy0, ix1, o[3]};
+        const int64_t p10[4] = {o[0], iy1, ix0, o[3]}, p11[4] = {o[0], iy1, ix1, o[3]};
+        if (isf) {
+            const int dt = out->dtype;
+            const double dy = round_to(dt, round_to(dt, (double)ry) / round_to(dt, (double)yn));
+            const double dx = round_to(dt, round_to(dt, (double)rx) / round_to(dt, (double)xn));
+            double acc;
+            if (a->mode == MLEL_RESIZE_BILINEAR) {
+                const double wy0 = round_to(dt, 1.0 - dy), wx0 = round_to(dt, 1.0 - dx);
+                acc = round_to(dt, round_to(dt, round_to(dt, ld_f(in, p00)) * wy0) * wx0);
+                acc = round_to(dt, acc + round_to(dt, round_to(dt, round_to(dt, ld_f(in, p01)) * wy0) * dx));
+                acc = round_to(dt, acc + round_to(dt, round_to(dt, round_to(dt, ld_f(in, p10)) * dy) * wx0));
+                acc = round_to(dt, acc + round_to(dt, round_to(dt, round_to(dt, ld_f(in, p11)) * dy) * dx));
+            } else {
+                const int64_t p[4] = {o[0], dy >= 0.5 ? iy1 : iy0, dx >= 0.5 ? ix1 : ix0, o[3]};
+                acc = ld_f(in, p);
+            }
+            st_f(out, o, acc);
+        } else {
+            /* the computation type is that of the output (int32 for int8 data, int64 for int16 data) */
+            const int wide = dt_size(out->dtype) == 8;
+            int64_t acc;
+            if (a->mode == MLEL_RESIZE_BILINEAR) {
+                const int64_t wy1 = ry, wx1 = rx, wy0 = (int16_t)(yn) - ry, wx0 = (int16_t)(xn) - rx;
+                const int64_t v[4] = {ld_i(in, p00), ld_i(in, p01), ld_i(in, p10), ld_i(in, p11)};
+                const int64_t wy[4] = {wy0, wy0, wy1, wy1}, wx[4] = {wx0, wx1, wx0, wx1};
+                acc = 0;
+                for (int t = 0; t < 4; t++) {
+                    if (wide)
+                        acc = wadd64(acc, wmul64(wmul64(v[t], wy[t]), wx[t]));
+                    else
+                        acc = wadd32((int32_t)acc, wmul32(wmul32((int32_t)v[t], (int32_t)wy[t]), (int32_t)wx[t]));
+                }
+            } else {
+                const int64_t p[4] = {o[0], 2 * (int32_t)ry >= yn ? iy1 : iy0, 2 * (int32_t)rx >= xn ? ix1 : ix0, o[3]};
+                acc = ld_i(in, p);
+            }
+            st_i(out, o, narrow_to(out->dtype, acc));
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * FFT2D / RFFT2D (reference: fft2d.comp:17-52, rfft2d.comp:13-71): the transform sums evaluated directly.  The
+ * reference's sine and cosine come from the Vulkan driver; here they are the C library's, so results agree with
+ * the reference to rounding, not bit for bit (parity unpinned beyond the transform's mathematics).
+ * ---------------------------------------------------------------------------------------------------------- */
+int mlel_cpu_fft2d(const mlel_tensor *out_real, const mlel_tensor *out_imag, const mlel_tensor *in_real,
+                   const mlel_tensor *in_imag, int32_t inverse) {
+    CHECK(out_real, "fft2d out_real");
+    CHECK(out_imag, "fft2d out_imag");
+    CHECK(in_real, "fft2d in_real");
+    CHECK(in_imag, "fft2d in_imag");
+    if (out_real->rank != 3 || out_imag->rank != 3 || in_real->rank != 3 || in_imag->rank != 3)
+        return fail(MLEL_ERR_INVALID, "fft2d: ranks must be 3");
+    const int64_t total = numel(out_real), H = out_real->dims[1], W = out_real->dims[2];
+    const float sign = inverse ? -1.0f : 1.0f;
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK];
+        unflatten(out_real, flat, o);
+        double sr = 0.0, si = 0.0;
+        for (int64_t iy = 0; iy < H; iy++) {
+            for (int64_t ix = 0; ix < W; ix++) {
+                const int64_t ii[3] = {o[0], iy, ix};
+                const float re = (float)ld_f(in_real, ii), im = (float)ld_f(in_imag, ii);
+                /* angle in fp32 as in the shader: sign * 2 pi * (float(iy * oy) / H + float(ix) * ox / W) */
+                const float frac = (float)(uint32_t)(iy * o[1]) / (float)H + ((float)ix * (float)o[2]) / (float)W;
+                const float angle = sign * 2.0f * 3.14159265358979323846f * frac;
+                const float c = cosf(angle), s = sinf(angle);
+                sr += (double)(re * c) + (double)(im * s);
+                si += (double)(-(re * s)) + (double)(im * c);
+            }
+        }
+        st_f(out_real, o, (double)(float)sr);
+        st_f(out_imag, o, (double)(float)si);
+    }
+    return 0;
+}
+
+int mlel_cpu_rfft2d(const mlel_tensor *out_real, const mlel_tensor *out_imag, const mlel_tensor *in) {
+    CHECK(out_real, "rfft2d out_real");
+    CHECK(out_imag, "rfft2d out_imag");
+    CHECK(in, "rfft2d in");
+    if (out_real->rank != 3 || out_imag->rank != 3 || in->rank != 3) return fail(MLEL_ERR_INVALID, "rfft2d: ranks must be 3");
+    const int64_t total = numel(out_real), H = in->dims[1], W = in->dims[2];
+#pragma omp parallel for schedule(static)
+    for (int64_t flat = 0; flat < total; flat++) {
+        int64_t o[MLEL_MAX_RANK];
+        unflatten(out_real, flat, o);
+        const int64_t oy = o[1], ox = o[2];
+        /* purely real bins: the imaginary part is left at exactly zero */
+        const int skip_imag = (oy == 0 || oy == H / 2) && (ox == 0 || ox == W / 2);
+        double sr = 0.0, si = 0.0;
+        for (int64_t iy = 0; iy < H; iy++) {
+            for (int64_t ix = 0; ix < W; ix++) {
+                const int64_t ii[3] = {o[0], iy, ix};
+                const double v = ld_f(in, ii);
+                /* the angle numerator is reduced modulo W * H before the division, as in the shader */
+                const double num = fmod((double)(iy * oy * W + ix * ox * H), (double)(W * H));
+                const double angle = 2.0 * 3.14159265358979323846 * num / (double)(W * H);
+                sr += v * cos(angle);
+                if (!skip_imag) si -= v * sin(angle);
+            }
+        }
+        st_f(out_real, o, (double)(float)sr);
+        st_f(out_imag, o, (double)(float)si);
+    }
+    return 0;
+}

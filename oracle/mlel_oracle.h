@@ -69,6 +69,24 @@ int mlel_cpu_concat(const mlel_tensor *out, const mlel_tensor *in, uint32_t axis
 int mlel_cpu_slice(const mlel_tensor *out, const mlel_tensor *in, const uint32_t *start);
 int mlel_cpu_pad(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *padding, double pad_const,
                  int32_t pad_const_int);
+int mlel_cpu_argmax(const mlel_tensor *out, const mlel_tensor *in, uint32_t axis, uint32_t nan_mode);
+int mlel_cpu_arithmetic_right_shift(const mlel_tensor *out, const mlel_tensor *in1, const mlel_tensor *in2,
+                                    uint32_t round);
+int mlel_cpu_conv3d(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w, const mlel_tensor *bias,
+                    const mlel_conv3d_attr *attr);
+int mlel_cpu_transpose_conv2d(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
+                              const mlel_tensor *bias, const mlel_tconv2d_attr *attr);
+int mlel_cpu_fft2d(const mlel_tensor *out_real, const mlel_tensor *out_imag, const mlel_tensor *in_real,
+                   const mlel_tensor *in_imag, int32_t inverse);
+int mlel_cpu_rfft2d(const mlel_tensor *out_real, const mlel_tensor *out_imag, const mlel_tensor *in);
+int mlel_cpu_gather(const mlel_tensor *out, const mlel_tensor *values, const mlel_tensor *indices);
+int mlel_cpu_scatter(const mlel_tensor *out, const mlel_tensor *values_in, const mlel_tensor *indices,
+                     const mlel_tensor *input);
+int mlel_cpu_resize(const mlel_tensor *out, const mlel_tensor *in, const mlel_resize_attr *attr);
+int mlel_cpu_reverse(const mlel_tensor *out, const mlel_tensor *in, uint32_t axis);
+int mlel_cpu_tile(const mlel_tensor *out, const mlel_tensor *in);
+int mlel_cpu_select(const mlel_tensor *out, const mlel_tensor *condition, const mlel_tensor *in_true,
+                    const mlel_tensor *in_false);
 
 /* IEEE binary16 <-> binary32 helpers (round to nearest even), exported for the tests. */
 uint16_t mlel_cpu_f32_to_f16(float f);

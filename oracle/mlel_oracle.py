@@ -182,5 +182,79 @@ def pad(x, padding, out_shape, pad_const=0.0, pad_const_int=0):
     return out
 
 
+def argmax(x, axis, nan_mode=abi.NAN_PROPAGATE):
+    shape = [d for i, d in enumerate(x.shape) if i != axis]
+    out = np.zeros(shape, dtype=np.int32)
+    _call("argmax", _view(out), _view(x), int(axis), int(nan_mode))
+    return out
+
+
+def arithmetic_right_shift(a, b, out_shape, round_=False):
+    out = np.zeros(out_shape, dtype=a.dtype)
+    _call("arithmetic_right_shift", _view(out), _view(a), _view(b), 1 if round_ else 0)
+    return out
+
+
+def conv3d(x, w, bias, out_shape, out_dtype, attr):
+    out = _out(out_shape, out_dtype)
+    _call("conv3d", _view(out, out_dtype), _view(x), _view(w), _view(bias, out_dtype), attr)
+    return out
+
+
+def transpose_conv2d(x, w, bias, out_shape, out_dtype, attr):
+    out = _out(out_shape, out_dtype)
+    _call("transpose_conv2d", _view(out, out_dtype), _view(x), _view(w), _view(bias, out_dtype), attr)
+    return out
+
+
+def fft2d(real, imag, inverse=False):
+    out_r, out_i = np.zeros_like(real), np.zeros_like(imag)
+    _call("fft2d", _view(out_r), _view(out_i), _view(real), _view(imag), 1 if inverse else 0)
+    return out_r, out_i
+
+
+def rfft2d(x):
+    shape = (x.shape[0], x.shape[1], x.shape[2] // 2 + 1)
+    out_r, out_i = np.zeros(shape, np.float32), np.zeros(shape, np.float32)
+    _call("rfft2d", _view(out_r), _view(out_i), _view(x))
+    return out_r, out_i
+
+
+def gather(values, indices):
+    out = np.zeros((values.shape[0], indices.shape[1], values.shape[2]), dtype=values.dtype)
+    _call("gather", _view(out), _view(values), _view(indices))
+    return out
+
+
+def scatter(values_in, indices, input_):
+    out = np.zeros_like(values_in)
+    _call("scatter", _view(out), _view(values_in), _view(indices), _view(input_))
+    return out
+
+
+def resize(x, out_shape, out_dtype, attr):
+    out = _out(out_shape, out_dtype)
+    _call("resize", _view(out, out_dtype), _view(x), attr)
+    return out
+
+
+def reverse(x, axis):
+    out = np.zeros_like(x)
+    _call("reverse", _view(out), _view(x), int(axis))
+    return out
+
+
+def tile(x, out_shape):
+    out = np.zeros(out_shape, dtype=x.dtype)
+    _call("tile", _view(out), _view(x))
+    return out
+
+
+def select(cond, a, b, out_shape):
+    out = np.zeros(out_shape, dtype=a.dtype)
+    _call("select", _view(out), _view(cond, abi.BOOL), _view(a), _view(b))
+    return out
+
+
 def num_threads():
     return lib().mlel_cpu_num_threads()

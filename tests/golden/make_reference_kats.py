@@ -62,6 +62,24 @@ cases["conv2d_acc_int64"] = {
                  "data": [40, -10, 18, -40, 80, -2, 10, -48, 120, 6, 2, -56, 160, 14, -6, -64]},
 }
 
+# tests/vulkan.cpp:1211-1290 + tests/shader/conv3d_large_stride.spvasm: CONV3D i8 -> i32 with a kernel 8192 wide whose only
+# non-zero taps are kx = 8190 and 8191 (weights[oc][kd][kh][8190 + j][ic] = relevant[((oc*2 + kd)*2 + kh)*8 + 4j + ic])
+cases["conv3d_large_stride"] = {
+    "source": "tests/vulkan.cpp:1211-1290, tests/shader/conv3d_large_stride.spvasm",
+    "input": {"dtype": "i8", "shape": [1, 3, 2, 2, 4], "data": [-128] * 48},
+    "weights_shape": [3, 2, 2, 8192, 4],
+    "relevant_weights": [
+        1, -1, 2, -1, 1, 0, -1, 0, 1, 2, 2, -1, 2, 2, 0, 1, 1, -2, -1, -2, 0, 2, -2, 0,
+        1, 1, -2, 1, 0, -2, 2, -1, 1, 0, 0, 2, 2, 0, 0, -1, 0, 0, -1, -1, -1, 0, -1, -2,
+        1, 1, -2, 2, -1, 1, 1, -2, 0, 0, 1, 2, 1, 2, 0, -2, 0, 2, 1, -2, 1, -1, -1, -1,
+        0, -2, 2, -2, 0, -1, 0, -1, 0, 2, 0, -2, 2, 1, 1, 0, -1, 0, 1, -2, -2, 2, 1, 0],
+    "attr": {"pad": [1, 0, 1, 0, 8190, 8192], "stride": [1, 1, 8192], "dilation": [1, 1, 1], "input_zp": 9,
+             "weight_zp": 0, "acc_type": 1},
+    "expected": {"dtype": "i32", "shape": [1, 3, 2, 2, 3], "data": [
+        0, -548, 137, 0, 0, 0, 548, -685, -411, 0, 0, 0, -1233, 274, 685, 0, 0, 0,
+        -822, -411, 274, 0, 0, 0, -1233, 274, 685, 0, 0, 0, -822, -411, 274, 0, 0, 0]},
+}
+
 # tests/vulkan.cpp:1091-1156: all-ones closed form, every output == IC (sizes reduced by the test that uses this)
 cases["conv2d_all_ones"] = {
     "source": "tests/vulkan.cpp:1091-1156 (OC=262144 / H or W = 524281 in the reference)",

@@ -206,3 +206,53 @@ class Runner:
         r = to.download()
         self.done()
         return r
+
+    # ---- the operators outside the benchmark graphs ------------------------------------------------------------
+    def call(self, name, out_specs, inputs, *attrs):
+        """Generic form: uploads `inputs`, allocates one output per (dtype, shape) in `out_specs`, calls
+        mlel_hip_<name>(outputs..., inputs..., attrs...) and returns the downloaded outputs."""
+        outs = [self.new(dt, shape) for dt, shape in out_specs]
+        ins = [self.put(x) for x in inputs]
+        self.dev.op(name, *[t.ref for t in outs], *[t.ref for t in ins], *attrs)
+        result = [t.download() for t in outs]
+        self.done()
+        return result if len(result) > 1 else result[0]
+
+    def argmax(self, x, axis, nan_mode=abi.NAN_PROPAGATE):
+        shape = [d for i, d in enumerate(x.shape) if i != axis]
+        return self.call("argmax", [(abi.I32, shape)], [x], int(axis), int(nan_mode))
+
+    def arithmetic_right_shift(self, a, b, out_shape, round_=False):
+        return self.call("arithmetic_right_shift", [(abi.dtype_of_numpy(a.dtype), out_shape)], [a, b], 1 if round_ else 0)
+
+    def conv3d(self, x, w, b, out_shape, out_dtype, attr):
+        return self.call("conv3d", [(out_dtype, out_shape)], [x, w, b], C.byref(attr))
+
+    def transpose_conv2d(self, x, w, b, out_shape, out_dtype, attr):
+        return self.call("transpose_conv2d", [(out_dtype, out_shape)], [x, w, b], C.byref(attr))
+
+    def fft2d(self, real, imag, inverse=False):
+        return self.call("fft2d", [(abi.F32, real.shape), (abi.F32, real.shape)], [real, imag], 1 if inverse else 0)
+
+    def rfft2d(self, x):
+        shape = (x.shape[0], x.shape[1], x.shape[2] // 2 + 1)
+        return self.call("rfft2d", [(abi.F32, shape), (abi.F32, shape)], [x])
+
+    def gather(self, values, indices):
+        shape = (values.shape[0], indices.shape[1], values.shape[2])
+        return self.call("gather", [(abi.dtype_of_numpy(values.dtype), shape)], [values, indices])
+
+    def scatter(self, values_in, indices, input_):
+        return self.call("scatter", [(abi.dtype_of_numpy(values_in.dtype), values_in.shape)], [values_in, indices, input_])
+
+    def resize(self, x, out_shape, out_dtype, attr):
+        return self.call("resize", [(out_dtype, out_shape)], [x], C.byref(attr))
+
+    def reverse(self, x, axis):
+        return self.call("reverse", [(abi.dtype_of_numpy(x.dtype), x.shape)], [x], int(axis))
+
+    def tile(self, x, out_shape):
+        return self.call("tile", [(abi.dtype_of_numpy(x.dtype), out_shape)], [x])
+
+    def select(self, cond, a, b, out_shape):
+        return self.call("select", [(abi.dtype_of_numpy(a.dtype), out_shape)], [cond, a, b])

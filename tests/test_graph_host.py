@@ -140,7 +140,7 @@ def test_error_conventions_of_the_operator_surface():
         g.op("FROBNICATE", ["x"], ["y"])
     assert e.value.code == abi.ERR_UNSUPPORTED and "Unsupported TOSA operator" in str(e.value)
     with pytest.raises(hb.MlelError) as e:
-        g.op("TILE", ["x"], ["y"])
+        g.op("MIN_SAD", ["x"], ["y"])  # the motion-engine instruction set is not TOSA
     assert e.value.code == abi.ERR_UNSUPPORTED
     g.const("w", __import__("numpy").zeros((4, 1, 1, 4), "int8"))
     g.const("b", __import__("numpy").zeros((4,), "int32"))

@@ -140,3 +140,19 @@ def test_sin_kat(kats, abi, oracle):
     k = kats["sin"]
     out = oracle.elementwise_unary("SIN", np.array([k["input"]], np.float32))
     assert abs(float(out[0]) - k["reference"]) <= k["error_bound"]
+
+
+def conv3d_kat(k):
+    w = np.zeros(k["weights_shape"], np.int8)
+    w[:, :, :, 8190:8192, :] = np.array(k["relevant_weights"], np.int8).reshape(3, 2, 2, 2, 4)
+    a = k["attr"]
+    return arr(k["input"]), w, arr(k["expected"]), (a["pad"], a["stride"], a["dilation"], a["input_zp"], a["weight_zp"],
+                                                   a["acc_type"])
+
+
+def test_kat_conv3d_large_stride(oracle, kats, abi):
+    """tests/vulkan.cpp:1211-1290: CONV3D with a kernel 8192 wide, pad (1,0,1,0,8190,8192), stride (1,1,8192), input
+    zero point 9; a null bias of length 1 is broadcast."""
+    x, w, exp, a = conv3d_kat(kats["conv3d_large_stride"])
+    out = oracle.conv3d(x, w, np.zeros(1, np.int32), exp.shape, abi.I32, abi.conv3d_attr(*a))
+    np.testing.assert_array_equal(out, exp)

@@ -72,6 +72,11 @@ REFERENCE_MODULES = {
                                        2: np.array([3], np.int32), 3: np.array([0], np.int8),
                                        4: np.array([4], np.int32), 5: np.array([0], np.int8)},
                                   [(abi.I8, (5,))] * 2, [(abi.I8, (5,))], ["RESCALE", "RESCALE", "ADD", "RESCALE"]),
+    "fft2d.spvasm": ({}, {}, [(abi.F32, (1, 4, 4096))] * 2, [(abi.F32, (1, 4, 4096))] * 2, ["FFT2D"]),
+    "arshift_specbool.spvasm": ({}, {}, [(abi.I16, (4,))] * 2, [(abi.I16, (4,))], ["ARITHMETIC_RIGHT_SHIFT"]),
+    "conv3d_large_stride.spvasm": ({}, {0: np.zeros((3, 2, 2, 8192, 4), np.int8)}, [(abi.I8, (1, 3, 2, 2, 4))],
+                                   [(abi.I32, (1, 3, 2, 2, 3))], ["CONV3D"]),
+    "conv3d_inline_bf16_constant.spvasm": ({}, {}, [(abi.BF16, (1, 1, 1, 1, 1))], [(abi.BF16, (1, 1, 1, 1, 1))], ["CONV3D"]),
     "nop-outputs.spvasm": ({(0, 0, 0): (1, 8, 8, 3), (0, 1, 0): (1, 2, 2, 2), (0, 2, 0): (1, 8, 8, 3),
                             (0, 3, 0): (1, 8, 8, 3)}, {0: np.zeros((1, 8, 8, 3), np.int8)}, [I8_1883],
                            [(abi.I8, (1, 2, 2, 2)), I8_1883, I8_1883], ["SLICE", "CAST", "CAST"]),
@@ -105,7 +110,6 @@ def test_reference_modules_outside_the_operator_set_are_refused():
     assert "no data supplied for graph constant 1" in error_of("graph-constant-arm.spvasm",
                                                                constants={0: np.array([2], np.int32)})
     assert "no shape for set 0 binding 0 element 1" in error_of("maxpool.spvasm", {(0, 1, 0): (1, 8, 8, 3)})
-    assert "multi-result" in error_of("fft2d.spvasm")
 
 
 # ------------------------------------------------------------------------------------------ writer -> loader, CPU
@@ -466,3 +470,95 @@ def test_config3_mobilenetv2_b32_from_assembly_equals_direct_build(dev):
     assert names == g.op_names() and len(names) == 64
     g.close()
     np.testing.assert_array_equal(got["output"], direct)
+
+
+@pytest.mark.gpu
+def test_kat_conv3d_module(dev, kats):
+    """tests/vulkan.cpp:1211-1290 as a module: weights in an OpGraphConstantARM, null bias of length 1, attribute
+    tensors of six and three values."""
+    from test_oracle_kats import conv3d_kat
+    x, wt, exp, a = conv3d_kat(kats["conv3d_large_stride"])
+    w = sw.SpvAsm("conv3d_large_stride")
+    xin = w.input("input", abi.I8, x.shape)
+    out = w.output("output", abi.I32, exp.shape)
+    operands = [w.attr(a[0]), w.attr(a[1]), w.attr(a[2]), w.u32(a[5]), w.scalar(abi.BOOL, False), xin,
+                w.const(wt, graph_constant=0), w.attr([0]), w.attr([a[3]], abi.I8), w.attr([a[4]], abi.I8)]
+    w.set_output(w.op("CONV3D", abi.I32, exp.shape, operands), out)
+    got, names = run_module(dev, w, {"input": x})
+    assert names == ["CONV3D"]
+    np.testing.assert_array_equal(got["output"], exp)
+
+
+@pytest.mark.gpu
+def test_multi_result_and_specialised_modules(dev, oracle):
+    """FFT2D / RFFT2D (two results picked apart with OpCompositeExtract), ARITHMETIC_RIGHT_SHIFT whose rounding flag is a
+    specialization constant, RESIZE and SCATTER operand decoding."""
+    rng = np.random.default_rng(8)
+    re, im = rng.standard_normal((1, 4, 16)).astype(np.float32), rng.standard_normal((1, 4, 16)).astype(np.float32)
+    w = sw.SpvAsm()
+    a, b = w.input("real", abi.F32, re.shape), w.input("imag", abi.F32, im.shape)
+    o0, o1 = w.output("out_real", abi.F32, re.shape), w.output("out_imag", abi.F32, re.shape)
+    t = w.tensor_type(abi.F32, re.shape)
+    w.declarations.append(f"%pair = OpTypeStruct {t} {t}")
+    w.body.append(f"%fft = OpExtInst %pair %tosa FFT2D {w.scalar(abi.BOOL, False)} {w.scalar(abi.BOOL, False)} {a} {b}")
+    w.body.append(f"%fft_re = OpCompositeExtract {t} %fft 0")
+    w.body.append(f"%fft_im = OpCompositeExtract {t} %fft 1")
+    w.set_output("%fft_re", o0)
+    w.set_output("%fft_im", o1)
+    got, names = run_module(dev, w, {"real": re, "imag": im})
+    er, ei = oracle.fft2d(re, im)
+    assert names == ["FFT2D"]
+    assert np.abs(got["out_real"] - er).max() <= 1e-3 and np.abs(got["out_imag"] - ei).max() <= 1e-3
+
+    # RFFT2D feeding a second operator: the extracted members are ordinary values
+    w = sw.SpvAsm()
+    x = w.input("input", abi.F32, re.shape)
+    out = w.output("output", abi.F32, (1, 4, 9))
+    t = w.tensor_type(abi.F32, (1, 4, 9))
+    w.declarations.append(f"%pair = OpTypeStruct {t} {t}")
+    w.body.append(f"%rfft = OpExtInst %pair %tosa RFFT2D {w.scalar(abi.BOOL, False)} {x}")
+    w.body.append(f"%r_re = OpCompositeExtract {t} %rfft 0")
+    w.body.append(f"%r_im = OpCompositeExtract {t} %rfft 1")
+    w.set_output(w.op("ADD", abi.F32, (1, 4, 9), ["%r_re", "%r_im"]), out)
+    got, names = run_module(dev, w, {"input": re})
+    rr, rimag = oracle.rfft2d(re)
+    assert names == ["RFFT2D", "ADD"] and np.abs(got["output"] - (rr + rimag)).max() <= 1e-3
+
+    # ARITHMETIC_RIGHT_SHIFT: `round` is OpSpecConstantFalse with SpecId 0; specialising it to true changes the result
+    v = np.array([-7, 7, 100, -100, 3, -3, 1, 0], np.int16)
+    s = np.array([1, 1, 3, 3, 2, 2, 1, 5], np.int16)
+    for spec, round_ in (({}, False), ({0: 1}, True)):
+        w = sw.SpvAsm("spec_arshift")
+        i0, i1 = w.input("in0", abi.I16, v.shape), w.input("in1", abi.I16, s.shape)
+        out = w.output("out0", abi.I16, v.shape)
+        w.decorations.append("OpDecorate %roundc SpecId 0")
+        w.declarations.append(f"%roundc = OpSpecConstantFalse {w.scalar_type(abi.BOOL)}")
+        w.set_output(w.op("ARITHMETIC_RIGHT_SHIFT", abi.I16, v.shape, ["%roundc", i0, i1]), out)
+        g = gb.Graph(dev)
+        ins, outs, _ = g.load_spvasm(w.text(), w.bindings, w.constants, w.names, specializations=spec)
+        g.finalize()
+        g.set_input("in0", v)
+        g.set_input("in1", s)
+        g.dispatch()
+        np.testing.assert_array_equal(g.get_output("out0"), oracle.arithmetic_right_shift(v, s, v.shape, round_))
+        g.close()
+
+    # RESIZE (mode input scale offset border) and SCATTER (valuesIn indices input)
+    x8 = rng.integers(-128, 127, (1, 5, 6, 3), endpoint=True).astype(np.int8)
+    w = sw.SpvAsm()
+    xin = w.input("input", abi.I8, x8.shape)
+    out = w.output("output", abi.I32, (1, 9, 11, 3))
+    w.set_output(w.op("RESIZE", abi.I32, (1, 9, 11, 3), [w.u32(2), xin, w.attr([4, 2, 4, 2]), w.attr([0, 0]), w.attr([0, 0])]),
+                 out)
+    got, _ = run_module(dev, w, {"input": x8})
+    np.testing.assert_array_equal(got["output"], oracle.resize(x8, (1, 9, 11, 3), abi.I32,
+                                                             abi.resize_attr((4, 2, 4, 2), (0, 0), (0, 0), 2)))
+    vals = rng.integers(-99, 99, (2, 7, 3)).astype(np.int32)
+    idx = np.array([[1, 3, 5, 0], [6, 2, 4, 1]], np.int32)
+    inp = rng.integers(-99, 99, (2, 4, 3)).astype(np.int32)
+    w = sw.SpvAsm()
+    iv, ii, ix = w.input("values", abi.I32, vals.shape), w.input("indices", abi.I32, idx.shape), w.input("input", abi.I32, inp.shape)
+    out = w.output("output", abi.I32, vals.shape)
+    w.set_output(w.op("SCATTER", abi.I32, vals.shape, [iv, ii, ix]), out)
+    got, _ = run_module(dev, w, {"values": vals, "indices": idx, "input": inp})
+    np.testing.assert_array_equal(got["output"], oracle.scatter(vals, idx, inp))
