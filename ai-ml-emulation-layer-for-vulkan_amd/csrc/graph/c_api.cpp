@@ -386,6 +386,18 @@ int mlel_graph_tensor_info(mlel_graph *g, int tensor, int32_t *dtype, int64_t *d
     });
 }
 
+int mlel_graph_set_memory_planner(mlel_graph *g, int planner) {
+    return guarded([&] {
+        if (planner < 0 || planner > 2) throw std::runtime_error("memory planner: 0 interval, 1 linear, 2 best fit");
+        g->pipeline.setMemoryPlanner(static_cast<GraphPipeline::MemoryPlanner>(planner));
+        return 0;
+    });
+}
+
+int mlel_graph_get_memory_planner(mlel_graph *g) {
+    return guarded([&] { return static_cast<int>(g->pipeline.memoryPlanner()); });
+}
+
 int mlel_graph_finalize(mlel_graph *g, int enable_fusion) {
     return guarded([&] {
         g->pipeline.finalize(enable_fusion != 0);

@@ -1,5 +1,7 @@
 #include "graph_pipeline.hpp"
 
+#include <cstdlib>
+
 #include <algorithm>
 #include <cstring>
 
@@ -100,7 +102,12 @@ mlel_tensor TensorDescriptor::view() const {
 
 // A null context is accepted for building and planning a graph (host-side logic needs no device); constants are
 // then not uploaded and dispatch() refuses to run.
-GraphPipeline::GraphPipeline(mlel_ctx *_ctx) : ctx{_ctx} {}
+GraphPipeline::GraphPipeline(mlel_ctx *_ctx) : ctx{_ctx} {
+    if (const char *env = std::getenv("VMEL_MEMORY_PLANNER")) {
+        if (std::string(env) == "Linear") planner = MemoryPlanner::Linear;
+        if (std::string(env) == "BestFit") planner = MemoryPlanner::BestFit;
+    }
+}
 
 GraphPipeline::~GraphPipeline() {
     if (ctx != nullptr)
@@ -736,7 +743,20 @@ void GraphPipeline::plan() {
         else if (eliminated.find(t) == eliminated.end() || t->isGraphOutput)
             unseen.push_back({i, aligned(t->getSize())});
     }
-    const auto planResult = details::allocateIntervals(std::move(intervals), unseen, kSessionAlignment);
+    details::AllocationPlan planResult;
+    if (planner == MemoryPlanner::Interval) {
+        planResult = details::allocateIntervals(std::move(intervals), unseen, kSessionAlignment);
+    } else if (planner == MemoryPlanner::Linear) {
+        std::vector<details::UnseenAllocation> all;  // creation order, one slot each
+        for (size_t i = 0; i < tensors.size(); i++) {
+            const auto *t = tensors[i].get();
+            if (ranges.find(t) != ranges.end() || eliminated.find(t) == eliminated.end() || t->isGraphOutput)
+                all.push_back({i, aligned(t->getSize())});
+        }
+        planResult = details::allocateLinear(all, kSessionAlignment);
+    } else {
+        planResult = details::allocateBestFit(bestFitTensors(intervals, unseen), kSessionAlignment);
+    }
     offsets.clear();
     for (const auto &[id, off] : planResult.offsets) offsets[tensors[id].get()] = static_cast<size_t>(off);
     for (const auto &[view, target] : aliasOf) {  // views share the storage of the tensor they alias
@@ -745,6 +765,89 @@ void GraphPipeline::plan() {
         if (it != offsets.end()) offsets[view] = it->second;
     }
     sessionSize = static_cast<size_t>(planResult.memorySize);
+}
+
+// Safe-to-reuse sets of the best-fit planner (reference: BestFitMemoryPlanner::liveTensorAnalysis,
+// memory_planner.cpp:139-226): a tensor T may share memory with the outputs of operator P once every operator that
+// reads T is a strict ancestor of P in the operator graph, i.e. T is dead before P can run in ANY topological order.
+// Tensors nobody reads, and tensors no executed operator writes, are never shared.
+std::vector<details::BestFitTensor> GraphPipeline::bestFitTensors(const std::vector<details::LiveInterval> &planned,
+                                                                  const std::vector<details::UnseenAllocation> &unseen) {
+    std::map<const TensorDescriptor *, size_t> index;
+    for (size_t i = 0; i < tensors.size(); i++) index[tensors[i].get()] = i;
+    const auto root = [&](const TensorDescriptor *t) {
+        for (auto it = aliasOf.find(t); it != aliasOf.end(); it = aliasOf.find(t)) t = it->second;
+        return t;
+    };
+    std::vector<const OpNode *> executed;
+    for (const auto &op : ops)
+        if (!op->fusedAway) executed.push_back(op.get());
+    const size_t n = executed.size(), words = (n + 63) / 64;
+    std::map<size_t, size_t> producer;               // tensor index -> operator position
+    std::map<size_t, std::vector<size_t>> consumers;
+    for (size_t p = 0; p < n; p++) {
+        const OpNode &op = *executed[p];
+        const auto reads = [&](const TensorPtr &t) {
+            if (!t) return;
+            const auto it = index.find(root(t.get()));
+            if (it != index.end()) consumers[it->second].push_back(p);
+        };
+        for (const auto &t : op.inputs) reads(t);
+        for (const auto *spec : {&op.epilogue, &op.scaleA, &op.scaleB}) {
+            reads(spec->multiplier);
+            reads(spec->shift);
+        }
+        for (const auto &t : op.outputs) {
+            const auto it = index.find(root(t.get()));
+            if (it != index.end() && producer.find(it->second) == producer.end()) producer[it->second] = p;
+        }
+    }
+    // strict ancestors of every operator (operators are stored in a topological order: creation order)
+    std::vector<std::vector<uint64_t>> ancestors(n, std::vector<uint64_t>(words, 0));
+    for (size_t p = 0; p < n; p++) {
+        const auto inherit = [&](const TensorPtr &t) {
+            if (!t) return;
+            const auto it = index.find(root(t.get()));
+            if (it == index.end()) return;
+            const auto pr = producer.find(it->second);
+            if (pr == producer.end() || pr->second >= p) return;
+            for (size_t w = 0; w < words; w++) ancestors[p][w] |= ancestors[pr->second][w];
+            ancestors[p][pr->second / 64] |= uint64_t(1) << (pr->second % 64);
+        };
+        for (const auto &t : executed[p]->inputs) inherit(t);
+    }
+    std::map<size_t, std::set<size_t>> safe;
+    for (const auto &[t, readers] : consumers) {
+        if (producer.find(t) == producer.end() || tensors[t]->isGraphOutput || tensors[t]->isGraphInput) continue;
+        for (const auto &[u, p] : producer) {
+            if (u == t || tensors[u]->isGraphOutput || tensors[u]->isGraphInput) continue;
+            const bool dead = std::all_of(readers.begin(), readers.end(), [&](size_t r) {
+                return (ancestors[p][r / 64] >> (r % 64)) & 1;
+            });
+            if (dead) {
+                safe[t].insert(u);
+                safe[u].insert(t);
+            }
+        }
+    }
+    std::vector<details::BestFitTensor> out;
+    std::map<size_t, uint64_t> sizes;
+    for (const auto &iv : planned) sizes[iv.id] = iv.size;
+    for (const auto &u : unseen) sizes[u.id] = u.size;
+    for (const auto &[id, size] : sizes) {  // creation order
+        details::BestFitTensor t{id, size, {}};
+        const auto it = safe.find(id);
+        if (it != safe.end())
+            for (const size_t other : it->second)
+                if (sizes.find(other) != sizes.end()) t.safe.push_back(other);
+        out.push_back(std::move(t));
+    }
+    return out;
+}
+
+void GraphPipeline::setMemoryPlanner(const MemoryPlanner p) {
+    if (finalized) fail("the memory planner is chosen before finalize()");
+    planner = p;
 }
 
 std::vector<std::array<uint32_t, 2>> GraphPipeline::liveRanges() const {

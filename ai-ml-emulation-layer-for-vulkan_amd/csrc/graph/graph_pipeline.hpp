@@ -28,6 +28,7 @@
 #include <vector>
 
 #include "../../../include/mlel_hip.h"
+#include "session_planner.hpp"
 
 namespace mlel::graph {
 
@@ -289,6 +290,12 @@ class GraphPipeline {
 
     // ---- HIP side ------------------------------------------------------------------------------------------
     // Runs the fusion pass (unless disabled) and plans session memory.  Called once, after the last make<Op>().
+    // Session-memory planner (reference: GraphPipelineSession::createMemoryPlanner, graph_layer.cpp:282-297).  The
+    // default is read from VMEL_MEMORY_PLANNER ("Linear", "BestFit", anything else: the interval planner) when the
+    // pipeline is created; set before finalize().
+    enum class MemoryPlanner { Interval, Linear, BestFit };
+    void setMemoryPlanner(MemoryPlanner p);
+    MemoryPlanner memoryPlanner() const { return planner; }
     void finalize(bool enableFusion = true);
     bool isFinalized() const { return finalized; }
     // Session memory requirements (reference: vkGetDataGraphPipelineSessionMemoryRequirementsARM,
@@ -325,6 +332,8 @@ class GraphPipeline {
     void *uploadConstant(const TensorDescriptor &t, const void *data);
     void fuse();
     void plan();
+    std::vector<details::BestFitTensor> bestFitTensors(const std::vector<details::LiveInterval> &planned,
+                                                       const std::vector<details::UnseenAllocation> &unseen);
     void run(const OpNode &op, void *stream);
     [[noreturn]] void unsupported(const char *tosaName) const;
 
@@ -342,6 +351,7 @@ class GraphPipeline {
     std::map<const TensorDescriptor *, std::array<uint32_t, 2>> ranges;
     std::map<const TensorDescriptor *, const TensorDescriptor *> aliasOf;  // elided RESHAPE: output -> input
     size_t sessionSize = 0;
+    MemoryPlanner planner = MemoryPlanner::Interval;
     bool finalized = false;
 
     friend class CApi;

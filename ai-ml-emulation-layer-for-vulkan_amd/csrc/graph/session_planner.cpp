@@ -48,4 +48,63 @@ AllocationPlan allocateIntervals(std::vector<LiveInterval> intervals, const std:
     return plan;
 }
 
+AllocationPlan allocateLinear(const std::vector<UnseenAllocation> &tensors, const uint64_t alignment) {
+    const auto alignUp = [alignment](uint64_t v) { return alignment ? (v + alignment - 1) / alignment * alignment : v; };
+    AllocationPlan plan;
+    for (const auto &t : tensors) {
+        const uint64_t where = alignUp(plan.memorySize);
+        plan.offsets[t.id] = where;
+        plan.memorySize = alignUp(where + t.size);
+    }
+    return plan;
+}
+
+AllocationPlan allocateBestFit(const std::vector<BestFitTensor> &tensors, const uint64_t alignment) {
+    const auto alignUp = [alignment](uint64_t v) { return alignment ? (v + alignment - 1) / alignment * alignment : v; };
+    std::map<size_t, const BestFitTensor *> byId;
+    for (const auto &t : tensors) byId[t.id] = &t;
+
+    std::vector<const BestFitTensor *> order;
+    for (const auto &t : tensors) order.push_back(&t);
+    std::stable_sort(order.begin(), order.end(),
+                     [](const BestFitTensor *a, const BestFitTensor *b) { return a->size > b->size; });
+
+    AllocationPlan plan;
+    std::map<size_t, size_t> blockOf;                // tensor id -> block index
+    std::vector<std::vector<size_t>> occupants;      // per block: the tensors placed in it
+    for (const BestFitTensor *t : order) {
+        // alternatives: safe tensors that are large enough, the closest in size first
+        std::vector<const BestFitTensor *> alternatives;
+        for (const size_t other : t->safe) {
+            const auto it = byId.find(other);
+            if (it != byId.end() && it->second->size >= t->size) alternatives.push_back(it->second);
+        }
+        std::stable_sort(alternatives.begin(), alternatives.end(),
+                         [](const BestFitTensor *a, const BestFitTensor *b) { return a->size < b->size; });
+        const std::set<size_t> safe(t->safe.begin(), t->safe.end());
+        const BestFitTensor *host = nullptr;
+        for (const BestFitTensor *alt : alternatives) {
+            const auto placed = blockOf.find(alt->id);
+            if (placed == blockOf.end()) continue;
+            const auto &living = occupants[placed->second];
+            if (std::all_of(living.begin(), living.end(), [&](size_t id) { return safe.count(id) != 0; })) {
+                host = alt;
+                break;
+            }
+        }
+        if (host) {
+            blockOf[t->id] = blockOf[host->id];
+            plan.offsets[t->id] = plan.offsets[host->id];
+            plan.memorySize = std::max(plan.memorySize, plan.offsets[t->id] + t->size);
+        } else {
+            blockOf[t->id] = occupants.size();
+            occupants.emplace_back();
+            plan.offsets[t->id] = plan.memorySize;
+            plan.memorySize = alignUp(std::max(plan.memorySize, plan.memorySize + t->size));
+        }
+        occupants[blockOf[t->id]].push_back(t->id);
+    }
+    return plan;
+}
+
 }  // namespace mlel::graph::details

@@ -40,4 +40,21 @@ struct AllocationPlan {
 AllocationPlan allocateIntervals(std::vector<LiveInterval> intervals, const std::vector<UnseenAllocation> &unseen,
                                  uint64_t alignment);
 
+// The reference's two other planners (graph/memory_planner.cpp), selected there by VMEL_MEMORY_PLANNER.
+//
+// Linear (memory_planner.cpp:52-94): every tensor gets an aligned slot of its own, in the given order.
+AllocationPlan allocateLinear(const std::vector<UnseenAllocation> &tensors, uint64_t alignment);
+
+// BestFit (memory_planner.cpp:100-382): tensors are taken by size, largest first (ties: given order).  A tensor may
+// share the block of an already placed tensor B when B is at least as large and every tensor already living in
+// that block is in the tensor's safe-to-reuse set; among such blocks the one of the smallest B wins (ties: order of
+// `safe`).  Otherwise it goes to the end of the arena, which is then rounded up to the alignment.
+// `safe[i]` lists the ids that may share memory with tensor i (the relation is symmetric).
+struct BestFitTensor {
+    size_t id;
+    uint64_t size;
+    std::vector<size_t> safe;
+};
+AllocationPlan allocateBestFit(const std::vector<BestFitTensor> &tensors, uint64_t alignment);
+
 }  // namespace mlel::graph::details

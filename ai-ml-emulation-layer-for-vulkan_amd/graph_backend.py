@@ -59,6 +59,8 @@ def load_graph_library():
                                                C.POINTER(C.c_int), C.POINTER(C.c_int)]
         lib.mlel_graph_tensor_info.argtypes = [_V, C.c_int, C.POINTER(C.c_int32), _I64P]
         lib.mlel_graph_finalize.argtypes = [_V, C.c_int]
+        lib.mlel_graph_set_memory_planner.argtypes = [_V, C.c_int]
+        lib.mlel_graph_get_memory_planner.argtypes = [_V]
         lib.mlel_graph_session_memory_requirements.argtypes = [_V, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
         lib.mlel_graph_bind_session_memory.argtypes = [_V, _V]
         lib.mlel_graph_bind_external.argtypes = [_V, C.c_uint32, C.c_uint32, C.c_uint32, _V]
@@ -213,6 +215,15 @@ class Graph:
             self.externals[name] = (key[0], key[1], key[2], int(dtype.value), tuple(int(dims[i]) for i in range(rank)), None)
             result.append(name)
         return result[:n_in.value], result[n_in.value:], count
+
+    PLANNERS = {"interval": 0, "linear": 1, "bestfit": 2}
+
+    def set_planner(self, name):
+        self._check(self.lib.mlel_graph_set_memory_planner(self.g, self.PLANNERS[name]))
+
+    def planner(self):
+        code = self._check(self.lib.mlel_graph_get_memory_planner(self.g))
+        return [k for k, v in self.PLANNERS.items() if v == code][0]
 
     # ---- finalize / memory / run
     def finalize(self, fuse=True):

@@ -79,6 +79,13 @@ int mlel_graph_load_spvasm(mlel_graph *g, const char *text, size_t length, const
 /* dtype, rank and dimensions of a tensor handle (dims: room for MLEL_MAX_RANK entries); returns the rank. */
 int mlel_graph_tensor_info(mlel_graph *g, int tensor, int32_t *dtype, int64_t *dims);
 
+/* Session-memory planner, chosen before mlel_graph_finalize: 0 interval (default), 1 linear, 2 best fit.  A new graph
+ * takes its default from the environment variable VMEL_MEMORY_PLANNER = "Linear" | "BestFit", as the reference does
+ * when a session is created (graph_layer.cpp:282-297; planners: graph/memory_planner.cpp:52-382,
+ * graph/interval_memory_planner.cpp). */
+int mlel_graph_set_memory_planner(mlel_graph *g, int planner);
+int mlel_graph_get_memory_planner(mlel_graph *g);
+
 /* Fusion + session memory planning; then the session requirements
  * (reference: vkGetDataGraphPipelineSessionMemoryRequirementsARM, graph_layer.cpp:1382-1389). */
 int mlel_graph_finalize(mlel_graph *g, int enable_fusion);

@@ -154,3 +154,95 @@ def test_error_conventions_of_the_operator_surface():
         g.dispatch()
     assert "no CPU path" in str(e.value)
     g.close()
+
+
+# ---------------------------------------------------------------------------------------- the three memory planners
+def _build_no_device(spec, planner=None):
+    g = gb.Graph(_NoDevice())
+    if planner:
+        g.set_planner(planner)
+    for name, dtype, shape in spec.inputs + spec.outputs:
+        g.external(name, dtype, shape)
+    for name, array in spec.consts.items():
+        g.const(name, array)
+    for name, (dtype, shape) in spec.tensors.items():
+        g.tensor(name, dtype, shape)
+    g.mark_input("input")
+    for op in spec.ops:
+        g.op(op["op"], op["in"], op["out"], op["iattr"], op["fattr"], op["name"])
+    g.mark_output("output")
+    g._check(g.lib.mlel_graph_finalize(g.g, 1))
+    size, align = __import__("ctypes").c_uint64(), __import__("ctypes").c_uint64()
+    g._check(g.lib.mlel_graph_session_memory_requirements(g.g, size, align))
+    return g, size.value, align.value
+
+
+@pytest.mark.parametrize("which", ["mobilenetv2", "transformer", "inverted_residual"])
+def test_memory_planners_give_valid_plans(which):
+    """Interval, Linear and BestFit (VMEL_MEMORY_PLANNER in the reference): tensors whose live ranges overlap never
+    share bytes, every offset is aligned, Linear is the sum of the aligned sizes, the reusing planners need no more
+    than Linear.  The reference has no unit test for Linear / BestFit; the plan's validity is what can be pinned."""
+    spec = {"mobilenetv2": lambda: graphs.mobilenetv2_spec(batch=2, image=64, classes=40),
+            "transformer": lambda: graphs.transformer_block_spec(batch=1, seq=16, d_model=32, heads=2, ffn=64),
+            "inverted_residual": lambda: graphs.inverted_residual_spec(batch=2, hw=14)}[which]()
+    sizes = {}
+    for planner in ("interval", "linear", "bestfit"):
+        g, size, align = _build_no_device(spec, planner)
+        assert g.planner() == planner
+        placed = [t for t in g.session_tensors() if t["offset"] is not None]
+        assert placed and all(t["offset"] % align == 0 for t in placed)
+        assert max(t["offset"] + t["size"] for t in placed) <= size
+        for i, a in enumerate(placed):
+            for b in placed[i + 1:]:
+                same_range = a["first"] == b["first"] and a["last"] == b["last"]
+                if a["handle"] == b["handle"] or (a["offset"] == b["offset"] and a["size"] == b["size"] and same_range):
+                    continue  # a RESHAPE view and the tensor it aliases
+                lives_overlap = a["first"] <= b["last"] and b["first"] <= a["last"]
+                bytes_overlap = a["offset"] < b["offset"] + b["size"] and b["offset"] < a["offset"] + a["size"]
+                assert not (lives_overlap and bytes_overlap), (planner, a, b)
+        sizes[planner] = size
+        if planner == "linear":
+            distinct = {(t["offset"], t["size"]) for t in placed}
+            assert size == sum((s + align - 1) // align * align for _, s in distinct)
+        g.close()
+    assert sizes["interval"] <= sizes["linear"] and sizes["bestfit"] <= sizes["linear"]
+    assert sizes["interval"] < sizes["linear"]  # the graphs do have tensors with disjoint lifetimes
+
+
+def test_memory_planner_from_environment(monkeypatch):
+    spec = graphs.inverted_residual_spec(batch=1, hw=8)
+    for value, expect in (("Linear", "linear"), ("BestFit", "bestfit"), ("Interval", "interval"), ("nonsense", "interval")):
+        monkeypatch.setenv("VMEL_MEMORY_PLANNER", value)
+        g, _, _ = _build_no_device(spec)
+        assert g.planner() == expect
+        g.close()
+    monkeypatch.delenv("VMEL_MEMORY_PLANNER")
+    g, _, _ = _build_no_device(spec)
+    assert g.planner() == "interval"
+    with pytest.raises(hb.MlelError, match="before finalize"):
+        g.set_planner("linear")
+    g.close()
+
+
+def test_best_fit_allocation_rules():
+    """BestFit on a chain a -> b -> c -> d (each read once): c may reuse a, d may reuse a or b; the largest tensor is
+    placed first and a smaller one moves into the smallest block that is large enough."""
+    g = gb.Graph(_NoDevice())
+    g.set_planner("bestfit")
+    g.external("input", abi.I8, (1, 1024))
+    g.external("output", abi.I8, (1, 256))
+    for name, n in (("a", 1024), ("b", 4096), ("c", 512), ("d", 256)):
+        g.tensor(name, abi.I8, (1, n))
+    g.mark_input("input")
+    g.op("ABS", ["input"], ["a"])
+    g.op("TILE", ["a"], ["b"])
+    g.op("SLICE", ["b"], ["c"], [0, 0])
+    g.op("SLICE", ["c"], ["d"], [0, 0])
+    g.op("ABS", ["d"], ["output"])
+    g.mark_output("output")
+    g._check(g.lib.mlel_graph_finalize(g.g, 0))
+    by_size = {t["size"]: t["offset"] for t in g.session_tensors()}
+    assert by_size[4096] == 0 and by_size[1024] == 4096     # placed by size; a and b are alive together
+    assert by_size[512] == by_size[1024]                     # c: only a is dead when c is produced
+    assert by_size[256] == by_size[4096]                     # d: a's block holds c (alive), b's block is free
+    g.close()

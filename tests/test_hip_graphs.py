@@ -126,3 +126,28 @@ def test_config4_transformer_block_full_size(dev):
     assert np.isfinite(out).all()
     assert np.abs(out - ref).max() <= 4e-2, np.abs(out - ref).max()
     assert np.abs(out - ref).mean() <= 2e-3
+
+
+@pytest.mark.parametrize("planner", ["linear", "bestfit"])
+def test_graphs_under_the_other_memory_planners(dev, oracle, planner, monkeypatch):
+    """VMEL_MEMORY_PLANNER = Linear / BestFit (the interval planner is the default everywhere else): same results."""
+    monkeypatch.setenv("VMEL_MEMORY_PLANNER", {"linear": "Linear", "bestfit": "BestFit"}[planner])
+    spec = graphs.mobilenetv2_spec(batch=2, image=64, spread=True, classes=40)
+    x = random_input(spec, 34)
+    exp, _ = run_spec(oracle, spec, {"input": x})
+    g = graphs.build(dev, spec, fuse=True)
+    assert g.planner() == planner
+    g.set_input("input", x)
+    g.dispatch()
+    out = g.get_output("output")
+    g.close()
+    np.testing.assert_array_equal(out, exp["output"])
+    spec = graphs.transformer_block_spec(batch=2, seq=64, d_model=64, heads=4, ffn=128)
+    xf = np.random.default_rng(6).standard_normal(spec.inputs[0][2]).astype(np.float16)
+    exp, _ = run_spec(oracle, spec, {"input": xf})
+    g = graphs.build(dev, spec, fuse=True)
+    g.set_input("input", xf)
+    g.dispatch()
+    out = g.get_output("output")
+    g.close()
+    assert np.max(np.abs(out.astype(np.float32) - exp["output"].astype(np.float32))) <= 1e-2
