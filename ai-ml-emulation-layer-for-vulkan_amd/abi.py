@@ -71,6 +71,15 @@ class ResizeAttr(C.Structure):
     _fields_ = [("scale", C.c_int32 * 4), ("offset", C.c_int32 * 2), ("border", C.c_int32 * 2), ("mode", C.c_uint32)]
 
 
+class ChainStep(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("selector", C.c_int32), ("a", C.c_int32), ("b", C.c_int32), ("dtype", C.c_int32)]
+
+
+class Chain(C.Structure):
+    _fields_ = [("n_inputs", C.c_int32), ("n_steps", C.c_int32), ("inputs", C.POINTER(Tensor) * 8),
+                ("steps", ChainStep * 24)]
+
+
 class MatmulAttr(C.Structure):
     _fields_ = [("a_zp", C.c_int32), ("b_zp", C.c_int32)]
 
@@ -211,6 +220,8 @@ FUSED_SIGNATURES = {
     "conv2d_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
     "matmul_rescale": [_T, _T, _T, C.POINTER(MatmulAttr), C.POINTER(Epilogue)],
     "dwconv_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
+    "matmul_bias_cast": [_T, _T, _T, _T, C.POINTER(MatmulAttr)],
+    "elementwise_chain": [_T, C.POINTER(Chain)],
     "rescale_add_rescale": [_T, _T, C.POINTER(Epilogue), _T, C.POINTER(Epilogue), C.POINTER(Epilogue)],
 }
 

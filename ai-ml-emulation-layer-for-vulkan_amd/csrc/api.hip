@@ -1,5 +1,7 @@
 // extern "C" operator entry points of include/mlel_hip.h: argument validation (the host-side checks that keep
 // every kernel's indexing assumptions true), then dispatch to a specialised gfx950 kernel or the generic path.
+#include <vector>
+
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -528,6 +530,82 @@ int mlel_hip_matmul_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out,
     mlel_tensor acc = packed_like(out, MLEL_I32, scratch.ptr);
     MLEL_TRY(mlel_hip_matmul(ctx, stream, &acc, a, b, attr));
     MLEL_TRY(run_unfused_tail(ctx, (hipStream_t)stream, out, &acc, epi));
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+int mlel_hip_elementwise_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_chain *chain) {
+    MLEL_TRY(require_ctx(ctx, "elementwise_chain"));
+    MLEL_REQUIRE(chain != nullptr, MLEL_ERR_INVALID, "elementwise_chain: null chain");
+    MLEL_REQUIRE(chain->n_inputs >= 1 && chain->n_inputs <= MLEL_CHAIN_MAX_INPUTS && chain->n_steps >= 1 &&
+                     chain->n_steps <= MLEL_CHAIN_MAX_STEPS,
+                 MLEL_ERR_INVALID, "elementwise_chain: %d inputs, %d steps", chain->n_inputs, chain->n_steps);
+    MLEL_TRY(check_supported(out, "elementwise_chain out"));
+    for (int i = 0; i < chain->n_inputs; i++) MLEL_TRY(check_supported(chain->inputs[i], "elementwise_chain input"));
+    const int rc = elementwise_chain_launch((hipStream_t)stream, out, chain);
+    if (rc != MLEL_ERR_UNSUPPORTED) return rc;
+    // the one-pass kernel declined (strides, alignment, too many live values): the operators one after another,
+    // every intermediate in a temporary of its own
+    std::vector<Scratch> temps(static_cast<size_t>(chain->n_steps));
+    std::vector<mlel_tensor> values;
+    for (int i = 0; i < chain->n_inputs; i++) values.push_back(*chain->inputs[i]);
+    for (int i = 0; i < chain->n_steps; i++) {
+        const mlel_chain_step &st = chain->steps[i];
+        const int n = static_cast<int>(values.size());
+        const bool two = st.kind == MLEL_CHAIN_BINARY || st.kind == MLEL_CHAIN_MUL;
+        MLEL_REQUIRE(st.a >= 0 && st.a < n && (!two || (st.b >= 0 && st.b < n)), MLEL_ERR_INVALID,
+                     "elementwise_chain: step %d reads a value that does not exist yet", i);
+        mlel_tensor result;
+        if (i == chain->n_steps - 1) {
+            result = *out;
+        } else {
+            MLEL_HIP_CHECK(hipMalloc(&temps[static_cast<size_t>(i)].ptr, (size_t)numel(out) * 4 + 16));
+            result = packed_like(out, st.dtype, temps[static_cast<size_t>(i)].ptr);
+        }
+        const mlel_tensor *a = &values[static_cast<size_t>(st.a)], *b = two ? &values[static_cast<size_t>(st.b)] : nullptr;
+        switch (st.kind) {
+        case MLEL_CHAIN_BINARY:
+            MLEL_TRY(mlel_hip_elementwise_binary(ctx, stream, st.selector, &result, a, b, MLEL_NAN_PROPAGATE));
+            break;
+        case MLEL_CHAIN_MUL: MLEL_TRY(mlel_hip_mul(ctx, stream, &result, a, b, 0)); break;
+        case MLEL_CHAIN_UNARY: MLEL_TRY(mlel_hip_elementwise_unary(ctx, stream, st.selector, &result, a)); break;
+        case MLEL_CHAIN_CAST: MLEL_TRY(mlel_hip_cast(ctx, stream, &result, a)); break;
+        default: MLEL_REQUIRE(false, MLEL_ERR_INVALID, "elementwise_chain: step kind %d", st.kind);
+        }
+        values.push_back(result);
+    }
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
+                              const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "matmul_bias_cast"));
+    MLEL_REQUIRE(attr != nullptr, MLEL_ERR_INVALID, "matmul_bias_cast: null attributes");
+    MLEL_TRY(check_supported(out, "matmul_bias_cast out"));
+    MLEL_TRY(check_supported(a, "matmul_bias_cast a"));
+    MLEL_TRY(check_supported(b, "matmul_bias_cast b"));
+    if (bias) MLEL_TRY(check_supported(bias, "matmul_bias_cast bias"));
+    MLEL_REQUIRE(out->rank == 3 && a->rank == 3 && b->rank == 3, MLEL_ERR_INVALID, "matmul_bias_cast: rank must be 3");
+    MLEL_REQUIRE(a->dtype == MLEL_F16 && b->dtype == MLEL_F16 && out->dtype == MLEL_F16 &&
+                     (bias == nullptr || (bias->dtype == MLEL_F32 && bias->rank == 3)),
+                 MLEL_ERR_INVALID, "matmul_bias_cast: fp16 operands and output, fp32 bias of rank 3");
+    const int rc = try_matmul_f16_mfma(ctx, (hipStream_t)stream, out, a, b, attr, true, bias);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    // no fused kernel for these strides / alignments: the three operators one after another through temporaries
+    Scratch acc_mem, sum_mem;
+    MLEL_HIP_CHECK(hipMalloc(&acc_mem.ptr, (size_t)numel(out) * 4 + 16));
+    mlel_tensor acc = packed_like(out, MLEL_F32, acc_mem.ptr);
+    MLEL_TRY(mlel_hip_matmul(ctx, stream, &acc, a, b, attr));
+    const mlel_tensor *cast_in = &acc;
+    mlel_tensor sum{};
+    if (bias) {
+        MLEL_HIP_CHECK(hipMalloc(&sum_mem.ptr, (size_t)numel(out) * 4 + 16));
+        sum = packed_like(out, MLEL_F32, sum_mem.ptr);
+        MLEL_TRY(mlel_hip_elementwise_binary(ctx, stream, MLEL_BIN_ADD, &sum, &acc, bias, MLEL_NAN_PROPAGATE));
+        cast_in = &sum;
+    }
+    MLEL_TRY(mlel_hip_cast(ctx, stream, out, cast_in));
     MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
     return 0;
 }

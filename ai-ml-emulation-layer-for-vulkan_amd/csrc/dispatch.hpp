@@ -36,6 +36,8 @@ int move_generic_launch(hipStream_t s, int kind, const mlel_tensor *out, const m
 int pad_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *padding,
                        double pad_const, int32_t pad_const_int);
 
+int elementwise_chain_launch(hipStream_t s, const mlel_tensor *out, const mlel_chain *chain);
+
 // ops_extra.hip: the TOSA operators outside the benchmark graphs
 int conv3d_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
                   const mlel_tensor *bias, const mlel_conv3d_attr *a);
@@ -97,7 +99,8 @@ int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
 
 // ---- fp16 MFMA MATMUL with fp32 result (gemm_f16.hip) ----
 int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
-                        const mlel_tensor *b, const mlel_matmul_attr *attr);
+                        const mlel_tensor *b, const mlel_matmul_attr *attr, bool bias_cast = false,
+                        const mlel_tensor *bias = nullptr);
 
 // ---- floating-point elementwise / reduce specialisations (ops_float.hip) ----
 int try_binary_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in1,

@@ -38,6 +38,9 @@ struct HGemmArgs {
     uint32_t lda, ldb, ldo;             // bytes per row
     uint32_t a_bytes, b_bytes, o_bytes; // per-batch extents (all below 2^31)
     int32_t tiles_m, tiles_n, total_tiles, chunk;
+    // fused epilogue (EPI = 1): out = fp16(acc + bias[n]) with the addition in fp32; bias may be null
+    const float *bias;
+    int32_t bias_len;  // 1 (broadcast) or N
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const void *p, uint32_t bytes) {
@@ -48,7 +51,7 @@ __device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t r, uint32_t off) 
     return make_uint4((uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
 __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -184,37 +187,70 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const int n0 = n_base + wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
-                const uint32_t off = (row_off != kOob && n0 < g.N) ? row_off + (uint32_t)n0 * 4 : kOob;
-                v4i v;
-                v.x = __float_as_int(acc[i][j][4 * q + 0]);
-                v.y = __float_as_int(acc[i][j][4 * q + 1]);
-                v.z = __float_as_int(acc[i][j][4 * q + 2]);
-                v.w = __float_as_int(acc[i][j][4 * q + 3]);
-                __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
+                if (EPI == 0) {
+                    const uint32_t off = (row_off != kOob && n0 < g.N) ? row_off + (uint32_t)n0 * 4 : kOob;
+                    v4i v;
+                    v.x = __float_as_int(acc[i][j][4 * q + 0]);
+                    v.y = __float_as_int(acc[i][j][4 * q + 1]);
+                    v.z = __float_as_int(acc[i][j][4 * q + 2]);
+                    v.w = __float_as_int(acc[i][j][4 * q + 3]);
+                    __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
+                } else {
+                    // ADD in fp32 (one rounding), then CAST to fp16 (round to nearest even): the two operators that
+                    // follow the MATMUL in the unfused graph
+                    const uint32_t off = (row_off != kOob && n0 < g.N) ? row_off + (uint32_t)n0 * 2 : kOob;
+                    float b4[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (g.bias != nullptr && n0 < g.N) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) b4[e] = g.bias[g.bias_len == 1 ? 0 : n0 + e];
+                    }
+                    _Float16 h[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float sum = g.bias != nullptr ? acc[i][j][4 * q + e] + b4[e] : acc[i][j][4 * q + e];
+                        h[e] = (_Float16)sum;
+                    }
+                    typedef int v2i_t __attribute__((ext_vector_type(2)));
+                    v2i_t v;
+                    v.x = (int)((uint32_t)__builtin_bit_cast(unsigned short, h[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[1]) << 16));
+                    v.y = (int)((uint32_t)__builtin_bit_cast(unsigned short, h[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[3]) << 16));
+                    __builtin_amdgcn_raw_buffer_store_b64(v, ores, (int)off, 0, 0);
+                }
             }
         }
     }
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N>
-void launch(const HGemmArgs &g, dim3 grid, hipStream_t s) {
+void launch(const HGemmArgs &g, bool cast_epilogue, dim3 grid, hipStream_t s) {
     constexpr size_t sm = (size_t)2 * BM * XPITCH + (size_t)2 * BKH * (2 * BN + 32);
-    gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N><<<grid, dim3(NT), sm, s>>>(g);
+    if (cast_epilogue)
+        gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 1><<<grid, dim3(NT), sm, s>>>(g);
+    else
+        gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 0><<<grid, dim3(NT), sm, s>>>(g);
 }
 
 bool dense_rows(const mlel_tensor *t) { return t->strides[2] == 2 && t->strides[1] >= t->dims[2] * 2; }
 
 }  // namespace
 
+// `bias_cast` set: the fused form out(fp16) = CAST(MATMUL + bias) with an fp32 bias of length 1 or N (or none)
 int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
-                        const mlel_tensor *b, const mlel_matmul_attr *attr) {
-    if (a->dtype != MLEL_F16 || b->dtype != MLEL_F16 || out->dtype != MLEL_F32) return 0;
+                        const mlel_tensor *b, const mlel_matmul_attr *attr, bool bias_cast, const mlel_tensor *bias) {
+    if (a->dtype != MLEL_F16 || b->dtype != MLEL_F16 || out->dtype != (bias_cast ? MLEL_F16 : MLEL_F32)) return 0;
+    const int osize = bias_cast ? 2 : 4;
+    if (bias_cast && bias != nullptr) {
+        const int64_t n = numel(bias);
+        const bool last_axis = bias->dims[bias->rank - 1] == n && bias->strides[bias->rank - 1] == 4;
+        if (bias->dtype != MLEL_F32 || !last_axis || (n != 1 && n != out->dims[2]) || ((uintptr_t)bias->ptr % 4) != 0)
+            return 0;
+    }
     if (attr->a_zp != 0 || attr->b_zp != 0) return 0;
     const int64_t NB = out->dims[0], M = out->dims[1], N = out->dims[2], K = a->dims[2];
     // what the kernel's indexing assumes: element-contiguous rows, 16-byte aligned rows and bases, K and N in
     // multiples of 8, per-batch extents below 2^31, operands at least as large as the output implies
     if (a->dims[0] < NB || b->dims[0] < NB || a->dims[1] < M || b->dims[1] < K || b->dims[2] < N) return 0;
-    if (!dense_rows(a) || !dense_rows(b) || out->strides[2] != 4) return 0;
+    if (!dense_rows(a) || !dense_rows(b) || out->strides[2] != osize) return 0;
     if (K % 8 != 0 || N % 8 != 0 || K <= 0) return 0;
     auto aligned = [](const mlel_tensor *t) {
         return ((uintptr_t)t->ptr % 16) == 0 && t->strides[0] % 16 == 0 && t->strides[1] % 16 == 0;
@@ -243,6 +279,8 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
     g.a_bytes = (uint32_t)ab;
     g.b_bytes = (uint32_t)bb;
     g.o_bytes = (uint32_t)ob;
+    g.bias = bias_cast && bias != nullptr ? static_cast<const float *>(bias->ptr) : nullptr;
+    g.bias_len = bias_cast && bias != nullptr ? (int)numel(bias) : 0;
     // tile choice: the width with the least padding of N; the tall tile when it still gives every compute unit two
     // blocks, otherwise the short one
     const int BN = ((N + 127) / 128) * 128 <= ((N + 63) / 64) * 64 ? 128 : 64;
@@ -258,13 +296,13 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
     g.chunk = (int)((total + 7) / 8);
     const dim3 grid((unsigned)(g.chunk * 8));
     if (BN == 128 && tall)
-        launch<128, 128, 2, 2>(g, grid, s);
+        launch<128, 128, 2, 2>(g, bias_cast, grid, s);
     else if (BN == 128)
-        launch<64, 128, 1, 4>(g, grid, s);
+        launch<64, 128, 1, 4>(g, bias_cast, grid, s);
     else if (tall)
-        launch<128, 64, 2, 2>(g, grid, s);
+        launch<128, 64, 2, 2>(g, bias_cast, grid, s);
     else
-        launch<64, 64, 2, 2>(g, grid, s);
+        launch<64, 64, 2, 2>(g, bias_cast, grid, s);
     MLEL_TRY(check_launch("matmul fp16"));
     return 1;
 }

@@ -663,6 +663,146 @@ void GraphPipeline::fuse() {
         ra->fusedAway = rb->fusedAway = ro.fusedAway = true;
     }
 
+    // Pattern 4 (fp16 projections): MATMUL (fp16 x fp16 -> fp32)  [-> ADD of an fp32 constant of one or N values]
+    // -> CAST to fp16.  The fused kernel adds in fp32 and rounds once to fp16, exactly like the operators it replaces.
+    for (const auto &opPtr : ops) {
+        OpNode &mm = *opPtr;
+        if (mm.fusedAway || mm.kind != OpKind::Matmul) continue;
+        const auto &acc = mm.outputs[0];
+        if (acc->getFormat() != MLEL_F32 || mm.inputs[0]->getFormat() != MLEL_F16 || mm.inputs[1]->getFormat() != MLEL_F16 ||
+            mm.matmul.a_zp != 0 || mm.matmul.b_zp != 0 || !isPrivateIntermediate(*acc) || acc->getRank() != 3)
+            continue;
+        const int64_t K = mm.inputs[0]->getDimensions()[2], N = acc->getDimensions()[2];
+        if (K % 8 != 0 || N % 8 != 0 || !mm.inputs[0]->isPacked() || !mm.inputs[1]->isPacked()) continue;
+        auto users = consumersOf(ops, acc.get());
+        if (users.size() != 1) continue;
+        OpNode *add = nullptr;
+        TensorPtr bias;
+        TensorPtr value = acc;
+        if (users[0]->kind == OpKind::Binary && users[0]->selector == MLEL_BIN_ADD) {
+            OpNode *cand = users[0];
+            const bool accFirst = cand->inputs[0].get() == acc.get();
+            const TensorPtr other = cand->inputs[accFirst ? 1 : 0];
+            const auto &od = other->getDimensions();
+            const int64_t n = static_cast<int64_t>(other->getShapeSize());
+            const bool vectorOnLastAxis = other->getRank() == 3 && od[2] == n && (n == 1 || n == N);
+            if (other->getKind() != TensorKind::Constant || other->getFormat() != MLEL_F32 || !vectorOnLastAxis ||
+                !other->isPacked() || cand->outputs[0]->getFormat() != MLEL_F32 || !sameShape(*acc, *cand->outputs[0]) ||
+                !isPrivateIntermediate(*cand->outputs[0]))
+                continue;
+            add = cand;
+            bias = other;
+            value = cand->outputs[0];
+            users = consumersOf(ops, value.get());
+            if (users.size() != 1) continue;
+        }
+        OpNode *cast = users[0];
+        if (cast->kind != OpKind::Cast || cast->inputs[0].get() != value.get() ||
+            cast->outputs[0]->getFormat() != MLEL_F16 || !sameShape(*acc, *cast->outputs[0]) ||
+            !cast->outputs[0]->isPacked())
+            continue;
+        mm.kind = OpKind::FusedMatmulBiasCast;
+        if (bias) mm.inputs.push_back(bias);
+        mm.outputs[0] = cast->outputs[0];
+        cast->outputs[0]->setProducer(&mm);
+        cast->fusedAway = true;
+        if (add) add->fusedAway = true;
+    }
+
+    // Pattern 5: regions of floating-point elementwise operators (ADD, SUB, MUL, EXP, RECIPROCAL, RSQRT, TANH, CAST
+    // between fp16 and fp32) collapse into one pass.  A region grows backwards from an operator whose result is needed
+    // elsewhere: a producer is absorbed when it is elementwise too, has the region's shape, and its result is a
+    // private intermediate read only here; everything else the region reads becomes an input and must have the
+    // region's shape or be broadcast along rows and / or the last axis.  The one-pass kernel rounds after every step
+    // like the stand-alone operators, so the result is bit-identical.
+    const auto chainStepOf = [](const OpNode &op, mlel_chain_step *st) {
+        const auto &out = op.outputs[0];
+        const int dt = out->getFormat();
+        if (op.fusedAway || (dt != MLEL_F16 && dt != MLEL_F32) || op.outputs.size() != 1) return false;
+        const auto sameType = [&](size_t n) {
+            for (size_t i = 0; i < n; i++)
+                if (op.inputs[i]->getFormat() != dt) return false;
+            return true;
+        };
+        *st = mlel_chain_step{0, 0, -1, -1, dt};
+        switch (op.kind) {
+        case OpKind::Binary:
+            st->kind = MLEL_CHAIN_BINARY;
+            st->selector = op.selector;
+            return (op.selector == MLEL_BIN_ADD || op.selector == MLEL_BIN_SUB) && sameType(2);
+        case OpKind::Mul: st->kind = MLEL_CHAIN_MUL; return op.shift == 0 && sameType(2);
+        case OpKind::Unary:
+            st->kind = MLEL_CHAIN_UNARY;
+            st->selector = op.selector;
+            return (op.selector == MLEL_UN_EXP || op.selector == MLEL_UN_RECIPROCAL || op.selector == MLEL_UN_RSQRT ||
+                    op.selector == MLEL_UN_TANH) && sameType(1);
+        case OpKind::Cast:
+            st->kind = MLEL_CHAIN_CAST;
+            return op.inputs[0]->getFormat() == MLEL_F16 || op.inputs[0]->getFormat() == MLEL_F32;
+        default: return false;
+        }
+    };
+    for (auto it = ops.rbegin(); it != ops.rend(); ++it) {
+        OpNode &root = **it;
+        mlel_chain_step rootStep{};
+        if (!chainStepOf(root, &rootStep)) continue;
+        const TensorDescriptor &shape = *root.outputs[0];
+        const auto &dims = shape.getDimensions();
+        const bool flat = !dims.empty() && dims.back() % 8 != 0;  // short rows: walked as one long row
+        if (!shape.isPacked() || dims.empty() || (flat && shape.getShapeSize() % 8 != 0)) continue;
+        const auto broadcastable = [&](const TensorDescriptor &t) {
+            const auto &d = t.getDimensions();
+            if (d.size() != dims.size() || !t.isPacked()) return false;
+            if (flat) return t.getShapeSize() == 1 || sameShape(t, shape);
+            bool same = true, ones = true;
+            for (size_t i = 0; i + 1 < d.size(); i++) {
+                same = same && d[i] == dims[i];
+                ones = ones && d[i] == 1;
+            }
+            return (same || ones) && (d.back() == dims.back() || d.back() == 1);
+        };
+        std::vector<TensorPtr> regionInputs;
+        std::vector<mlel_chain_step> steps;   // operands: value >= 0 input index, value < 0 -(step index + 1)
+        std::vector<OpNode *> absorbed;
+        bool ok = true;
+        std::function<int(const TensorPtr &)> valueOf;
+        const auto emit = [&](OpNode &op, mlel_chain_step st) {
+            const bool two = st.kind == MLEL_CHAIN_BINARY || st.kind == MLEL_CHAIN_MUL;
+            st.a = valueOf(op.inputs[0]);
+            st.b = two ? valueOf(op.inputs[1]) : 0;
+            steps.push_back(st);
+            return -static_cast<int>(steps.size());
+        };
+        valueOf = [&](const TensorPtr &t) -> int {
+            OpNode *p = t->getProducer();
+            mlel_chain_step st{};
+            if (p && p != &root && isPrivateIntermediate(*t) && sameShape(*t, shape) && chainStepOf(*p, &st) &&
+                consumersOf(ops, t.get()).size() == 1 && steps.size() + absorbed.size() < MLEL_CHAIN_MAX_STEPS - 1) {
+                absorbed.push_back(p);
+                return emit(*p, st);
+            }
+            for (size_t i = 0; i < regionInputs.size(); i++)
+                if (regionInputs[i].get() == t.get()) return static_cast<int>(i);
+            if (!broadcastable(*t) || regionInputs.size() >= MLEL_CHAIN_MAX_INPUTS) {
+                ok = false;
+                return 0;
+            }
+            regionInputs.push_back(t);
+            return static_cast<int>(regionInputs.size()) - 1;
+        };
+        emit(root, rootStep);
+        if (!ok || steps.size() < 2 || steps.size() > MLEL_CHAIN_MAX_STEPS) continue;
+        const int nIn = static_cast<int>(regionInputs.size());
+        for (auto &st : steps) {
+            if (st.a < 0) st.a = nIn + (-st.a - 1);
+            if (st.b < 0) st.b = nIn + (-st.b - 1);
+        }
+        for (OpNode *p : absorbed) p->fusedAway = true;
+        root.kind = OpKind::FusedElementwise;
+        root.inputs = regionInputs;
+        root.chain = steps;
+    }
+
     // Pattern 3: RESHAPE between two packed session tensors of the same byte size moves no data (the reference's
     // reshape.comp:16-27 copies by flat index): the output becomes a second view of the input's storage and the
     // operator is not executed.  plan() gives both tensors one allocation that lives as long as either is used.
@@ -967,6 +1107,25 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
             rc = mlel_hip_matmul_rescale(ctx, stream, &out, &in[0], &in[1], &op.matmul, &e);
         break;
     }
+    case OpKind::FusedElementwise: {
+        mlel_chain c{};
+        std::vector<mlel_tensor> views;
+        for (const auto &t : op.inputs) {
+            views.push_back(t->view());
+            if (views.back().ptr == nullptr && t->getShapeSize() != 0)
+                fail(op.tosaName + " (" + op.debugName + "): an input of the fused region has no memory bound");
+        }
+        c.n_inputs = static_cast<int32_t>(views.size());
+        for (size_t i = 0; i < views.size(); i++) c.inputs[i] = &views[i];
+        c.n_steps = static_cast<int32_t>(op.chain.size());
+        for (size_t i = 0; i < op.chain.size(); i++) c.steps[i] = op.chain[i];
+        rc = mlel_hip_elementwise_chain(ctx, stream, &out, &c);
+        break;
+    }
+    case OpKind::FusedMatmulBiasCast:
+        rc = mlel_hip_matmul_bias_cast(ctx, stream, &out, &in[0], &in[1], op.inputs.size() > 2 ? &in[2] : nullptr,
+                                       &op.matmul);
+        break;
     case OpKind::FusedRescaleAddRescale: {
         const mlel_tensor ma = op.scaleA.multiplier->view(), sa = op.scaleA.shift->view();
         const mlel_tensor mb = op.scaleB.multiplier->view(), sb = op.scaleB.shift->view();

@@ -97,7 +97,7 @@ enum class OpKind {
     Negate, Reshape, Transpose, Concat, Slice, Pad,
     Argmax, ArithmeticRightShift, Conv3D, TransposeConv2D, Fft2D, Rfft2D, Gather, Scatter, Resize, Reverse, Tile, Select,
     // produced by the fusion pass only
-    FusedConv2D, FusedDepthwiseConv2D, FusedMatmul, FusedRescaleAddRescale,
+    FusedConv2D, FusedDepthwiseConv2D, FusedMatmul, FusedRescaleAddRescale, FusedMatmulBiasCast, FusedElementwise,
 };
 
 struct RescaleSpec {
@@ -124,6 +124,7 @@ class OpNode {
     mlel_tconv2d_attr tconv{};
     mlel_resize_attr resize{};
     bool flag = false;  // ARITHMETIC_RIGHT_SHIFT: round; FFT2D: inverse
+    std::vector<mlel_chain_step> chain;  // FusedElementwise: the program over `inputs` (see mlel_chain)
     int32_t selector = 0;  // mlel_binary_op / mlel_unary_op / mlel_reduce_op
     uint32_t nanMode = MLEL_NAN_PROPAGATE, axis = 0, shift = 0, offset = 0;
     int32_t inputZeroPoint = 0, outputZeroPoint = 0, padConstInt = 0;

@@ -3,6 +3,8 @@
 // bit: operands are widened to fp32, the operator is applied once, and the result is rounded once into the storage
 // type (reference: elementwise_binary.comp:146-173, mul.comp:24-59, elementwise_unary.comp:136-205,
 // cast.comp:22-103, reduce.comp:24-70).  `try_*` returns 0 to decline a case.
+#include <vector>
+
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -22,6 +24,34 @@ struct EwArgs {
     int32_t cols;
     int32_t a_row, a_col, b_row, b_col;  // 1 when the operand varies along rows / columns, 0 when it is broadcast
 };
+
+// Transcendentals.  Results that are stored as fp32 use the accurate library functions; results that are rounded to
+// fp16 use the hardware approximations (v_exp_f32, v_rcp_f32, v_rsq_f32: about one ulp of fp32, three decimal
+// orders below half an ulp of fp16), which matter because these operators are otherwise bound by the vector ALU, not
+// by memory.  The stand-alone kernels and the one-pass chain kernel share these functions, so they agree bit for
+// bit.  (In the reference these functions are the Vulkan driver's and differ from driver to driver.)
+template <bool F16>
+__device__ __forceinline__ float op_exp(float x) {
+    return F16 ? __expf(x) : expf(x);
+}
+template <bool F16>
+__device__ __forceinline__ float op_reciprocal(float x) {
+    return F16 ? __builtin_amdgcn_rcpf(x) : 1.0f / x;
+}
+template <bool F16>
+__device__ __forceinline__ float op_rsqrt(float x) {
+    return F16 ? __builtin_amdgcn_rsqf(x) : 1.0f / sqrtf(x);
+}
+template <bool F16>
+__device__ __forceinline__ float op_tanh(float x) {
+    if (!F16) return tanh_clamped(x);
+    // the reference's three ranges (elementwise_unary.comp:136-155) with tanh(x) = 1 - 2 / (exp(2x) + 1) in between
+    const float ax = fabsf(x);
+    const float x2 = x * x;
+    const float small = x * (1.0f - x2 * (1.0f / 3.0f - x2 * (2.0f / 15.0f - 17.0f / 315.0f * x2)));
+    const float mid = 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * x) + 1.0f);
+    return ax > 10.0f ? copysignf(1.0f, x) : (ax < 0.2f ? small : mid);
+}
 
 template <int SIZE>
 __device__ __forceinline__ void load8(const char *base, int64_t row, int32_t c8, int32_t cols, int varies_row,
@@ -79,14 +109,190 @@ __global__ void __launch_bounds__(kBlock) ew_float_kernel(const EwArgs g) {
         case F_ADD: r[i] = a[i] + b[i]; break;
         case F_SUB: r[i] = a[i] - b[i]; break;
         case F_MUL: r[i] = a[i] * b[i]; break;  // operands already have the output's storage type
-        case F_EXP: r[i] = expf(a[i]); break;
-        case F_RECIPROCAL: r[i] = 1.0f / a[i]; break;
-        case F_RSQRT: r[i] = 1.0f / sqrtf(a[i]); break;
-        case F_TANH: r[i] = tanh_clamped(a[i]); break;
+        case F_EXP: r[i] = op_exp<OUT_SIZE == 2>(a[i]); break;
+        case F_RECIPROCAL: r[i] = op_reciprocal<OUT_SIZE == 2>(a[i]); break;
+        case F_RSQRT: r[i] = op_rsqrt<OUT_SIZE == 2>(a[i]); break;
+        case F_TANH: r[i] = op_tanh<OUT_SIZE == 2>(a[i]); break;
         default: r[i] = a[i]; break;
         }
     }
     store8<OUT_SIZE>(g.out + v * 8 * OUT_SIZE, r);
+}
+
+
+// ---------------------------------------------------------------------------------------------------------------
+// A chain of elementwise operators in one pass.  Eight elements per thread; the values of the chain live in a small
+// per-thread register file in shared memory (the program is data, so registers are addressed at run time): slot r of
+// thread t holds eight floats at [r][half][t], conflict-free for a wavefront.  Each step applies its operator to the
+// fp32 operands and rounds once into the step's storage type, as the stand-alone kernels above do.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kChainRegs = 4;
+
+struct ChainInput {
+    const char *ptr;
+    int32_t size;        // 2 or 4 bytes per element
+    int32_t varies_row;  // as EwArgs
+    int32_t varies_col;
+    int32_t reg;         // register the value is loaded into; single-element inputs: lane of the scalar file
+};
+
+struct ChainStep {
+    int8_t op;          // FOp
+    int8_t f16;         // result rounded to fp16 (else fp32)
+    int8_t a, b;        // operand registers (or scalar-file lanes)
+    int8_t a_sc, b_sc;  // the operand is a single-element input
+    int8_t a_fw, b_fw;  // the operand is the previous step's result, still in vector registers
+    int8_t dst;         // result register, or -1 when only the next step reads the result
+};
+
+struct ChainArgs {
+    char *out;
+    int32_t out_size, out_reg;
+    int64_t vecs;
+    int32_t cols8, cols;
+    int32_t n_inputs, n_steps;
+    ChainInput in[MLEL_CHAIN_MAX_INPUTS];
+    ChainStep step[MLEL_CHAIN_MAX_STEPS];
+};
+
+// HALF: every value of the chain (inputs and results) is fp16, so a register is eight halfs (16 bytes) instead of
+// eight floats: half the shared memory, twice the resident wavefronts, which is what a latency-bound streaming
+// kernel needs.
+template <bool HALF>
+__global__ void __launch_bounds__(kBlock) ew_chain_kernel(const ChainArgs g) {
+    constexpr int kRegs = HALF ? kChainRegs + 2 : kChainRegs;
+    __shared__ uint4 regs[kRegs][HALF ? 1 : 2][kBlock];
+    const int tid = threadIdx.x;
+    const int64_t v = (int64_t)blockIdx.x * kBlock + tid;
+    if (v >= g.vecs) return;  // no barrier below: a thread only touches its own slots
+    const int64_t row = v / g.cols8;
+    const int32_t c8 = (int32_t)(v - row * g.cols8);
+    const auto put = [&](int r, const float (&x)[8]) {
+        if (HALF) {  // the values are fp16 numbers already: the conversion is exact
+            uint4 raw;
+            __half2 *h = reinterpret_cast<__half2 *>(&raw);
+#pragma unroll
+            for (int i = 0; i < 4; i++) h[i] = __halves2half2(__float2half_rn(x[2 * i]), __float2half_rn(x[2 * i + 1]));
+            regs[r][0][tid] = raw;
+        } else {
+            regs[r][0][tid] = make_uint4(__float_as_uint(x[0]), __float_as_uint(x[1]), __float_as_uint(x[2]), __float_as_uint(x[3]));
+            regs[r][HALF ? 0 : 1][tid] =
+                make_uint4(__float_as_uint(x[4]), __float_as_uint(x[5]), __float_as_uint(x[6]), __float_as_uint(x[7]));
+        }
+    };
+    const auto get = [&](int r, float (&x)[8]) {
+        if (HALF) {
+            const uint4 raw = regs[r][0][tid];
+            const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float2 f = __half22float2(h[i]);
+                x[2 * i] = f.x;
+                x[2 * i + 1] = f.y;
+            }
+        } else {
+            const uint4 lo = regs[r][0][tid], hi = regs[r][HALF ? 0 : 1][tid];
+            x[0] = __uint_as_float(lo.x), x[1] = __uint_as_float(lo.y), x[2] = __uint_as_float(lo.z), x[3] = __uint_as_float(lo.w);
+            x[4] = __uint_as_float(hi.x), x[5] = __uint_as_float(hi.y), x[6] = __uint_as_float(hi.z), x[7] = __uint_as_float(hi.w);
+        }
+    };
+    // single-element inputs live in one vector register, lane k holding scalar k (read back with a lane broadcast);
+    // the other inputs are all requested before any is stored, so that their loads overlap
+    int sc_bits = 0;
+    float x[MLEL_CHAIN_MAX_INPUTS][8];
+#pragma unroll
+    for (int k = 0; k < MLEL_CHAIN_MAX_INPUTS; k++) {
+        if (k >= g.n_inputs) continue;  // uniform
+        const ChainInput in = g.in[k];
+        if (!in.varies_row && !in.varies_col) {
+            const float s = in.size == 2 ? __half2float(*reinterpret_cast<const __half *>(in.ptr))
+                                         : *reinterpret_cast<const float *>(in.ptr);
+            sc_bits = (tid & 63) == in.reg ? __float_as_int(s) : sc_bits;
+        } else if (in.size == 2) {
+            load8<2>(in.ptr, row, c8, g.cols, in.varies_row, in.varies_col, x[k]);
+        } else {
+            load8<4>(in.ptr, row, c8, g.cols, in.varies_row, in.varies_col, x[k]);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < MLEL_CHAIN_MAX_INPUTS; k++) {
+        if (k >= g.n_inputs) continue;
+        if (g.in[k].varies_row || g.in[k].varies_col) put(g.in[k].reg, x[k]);
+    }
+    const auto fetch = [&](int r, int is_scalar, float (&y)[8]) {
+        if (is_scalar) {  // uniform
+            const float s = __int_as_float(__builtin_amdgcn_readlane(sc_bits, r));
+#pragma unroll
+            for (int i = 0; i < 8; i++) y[i] = s;
+        } else {
+            get(r, y);
+        }
+    };
+    float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < g.n_steps; s++) {
+        const ChainStep st = g.step[s];
+        float a[8], b[8];
+        if (st.a_fw) {  // uniform
+#pragma unroll
+            for (int i = 0; i < 8; i++) a[i] = r[i];
+        } else {
+            fetch(st.a, st.a_sc, a);
+        }
+        if (st.op == F_ADD || st.op == F_SUB || st.op == F_MUL) {
+            if (st.b_fw) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) b[i] = r[i];
+            } else {
+                fetch(st.b, st.b_sc, b);
+            }
+        }
+        switch (st.op) {  // uniform
+        case F_ADD:
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = a[i] + b[i];
+            break;
+        case F_SUB:
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = a[i] - b[i];
+            break;
+        case F_MUL:
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = a[i] * b[i];
+            break;
+        case F_EXP:
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = st.f16 ? op_exp<true>(a[i]) : op_exp<false>(a[i]);
+            break;
+        case F_RECIPROCAL:
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = st.f16 ? op_reciprocal<true>(a[i]) : op_reciprocal<false>(a[i]);
+            break;
+        case F_RSQRT:
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = st.f16 ? op_rsqrt<true>(a[i]) : op_rsqrt<false>(a[i]);
+            break;
+        case F_TANH:
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = st.f16 ? op_tanh<true>(a[i]) : op_tanh<false>(a[i]);
+            break;
+        default:
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = a[i];
+            break;
+        }
+        if (st.f16) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = rnd_f16(r[i]);
+        }
+        if (s + 1 == g.n_steps) {  // the result goes straight to memory
+            if (g.out_size == 2)
+                store8<2>(g.out + v * 16, r);
+            else
+                store8<4>(g.out + v * 32, r);
+        } else if (st.dst >= 0) {
+            put(st.dst, r);
+        }
+    }
 }
 
 // How `in` relates to the dense output: same extents on every leading dimension (varies along rows) or 1 on all of
@@ -215,7 +421,7 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArg
     // counts (LayerNorm over a few thousand tokens) must still spread over many compute units; all four wavefronts
     // fetch the slab (many loads in flight), then the first one folds it out of shared memory, one row per lane.
     extern __shared__ __align__(16) char slab[];
-    const int pitch = g.slab_cols * 2 + 8;  // bytes; 8-byte aligned, consecutive rows two banks apart
+    const int pitch = g.slab_cols * 2 + 16;  // bytes; 16-byte aligned, consecutive rows four banks apart
     const int tid = threadIdx.x;
     const int64_t row0 = (int64_t)blockIdx.x * 64;
     const int64_t row = row0 + tid;
@@ -240,45 +446,55 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArg
                 const int p = p0 + i * kBlock + tid;
                 const int rr = p / segs, seg = p - rr * segs;
                 if (p < pieces) {
-                    *reinterpret_cast<uint2 *>(slab + rr * pitch + seg * 16) = make_uint2(v[i].x, v[i].y);
-                    *reinterpret_cast<uint2 *>(slab + rr * pitch + seg * 16 + 8) = make_uint2(v[i].z, v[i].w);
+                    *reinterpret_cast<uint4 *>(slab + rr * pitch + seg * 16) = v[i];
                 }
             }
         }
         __syncthreads();
         if (tid < 64) {
-            uint2 next = *reinterpret_cast<const uint2 *>(slab + tid * pitch);
-            for (int j = 0; j < n; j += 4) {
-                const uint2 raw = next;
-                if (j + 4 < n) next = *reinterpret_cast<const uint2 *>(slab + tid * pitch + (j + 4) * 2);
+            const char *mine = slab + tid * pitch;
+            uint4 next = *reinterpret_cast<const uint4 *>(mine);
+            for (int j = 0; j < n; j += 8) {
+                const uint4 raw = next;
+                if (j + 8 < n) next = *reinterpret_cast<const uint4 *>(mine + (j + 8) * 2);
                 const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
-                // a NaN among the four halfs: exponent all ones and a non-zero mantissa, tested on the packed pairs
-                const uint32_t nan_bits = (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu)) &
-                                          0x80008000u;
+                // a NaN among the eight halfs: exponent all ones and a non-zero mantissa, tested on the packed pairs
+                const uint32_t nan_bits =
+                    (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu) |
+                     ((raw.z & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
                 if (!__any(done || nan_bits != 0)) {
                     // no lane of the wavefront is in a special state: the plain fold.  A native fp16 add rounds the
-                    // exact sum once; the generic kernel's fp32 add followed by a conversion gives the same value,
-                    // because the fp32 sum of two halfs is inexact only when the smaller one is far below half an ulp
-                    // of the larger.
+                    // exact sum once; the generic kernel's fp32 add followed by a conversion gives the same value
+                    // (fp32 carries more than twice the fp16 precision plus two bits, so the second rounding cannot
+                    // change the result).
                     if (IS_SUM) {
                         __half acc = __float2half_rn(r);
-                        acc = __hadd(acc, __low2half(h[0]));
-                        acc = __hadd(acc, __high2half(h[0]));
-                        acc = __hadd(acc, __low2half(h[1]));
-                        acc = __hadd(acc, __high2half(h[1]));
+#pragma unroll
+                        for (int t = 0; t < 4; t++) {
+                            acc = __hadd(acc, __low2half(h[t]));
+                            acc = __hadd(acc, __high2half(h[t]));
+                        }
                         r = __half2float(acc);
                     } else {
-                        const float2 f01 = __half22float2(h[0]), f23 = __half22float2(h[1]);
-                        const float e[4] = {f01.x, f01.y, f23.x, f23.y};
-#pragma unroll
-                        for (int t = 0; t < 4; t++) r = isnan(r) ? e[t] : (r < e[t] ? e[t] : r);
+                        // the order of a maximum is free: pairwise on the packed halfs, then against the state
+                        typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+                        const h2_t *p = reinterpret_cast<const h2_t *>(&raw);
+                        const h2_t m = __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]),
+                                                                 __builtin_elementwise_max(p[2], p[3]));
+                        const float e = (float)(m.x > m.y ? m.x : m.y);
+                        r = isnan(r) ? e : (r < e ? e : r);
                     }
                     continue;
                 }
-                const float2 f01 = __half22float2(h[0]), f23 = __half22float2(h[1]);
-                const float e[4] = {f01.x, f01.y, f23.x, f23.y};
+                float e[8];
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
+                    const float2 f = __half22float2(h[t]);
+                    e[2 * t] = f.x;
+                    e[2 * t + 1] = f.y;
+                }
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
                     const float v = e[t];
                     if (done) continue;
                     if (isnan(v)) {
@@ -300,6 +516,120 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArg
 }
 
 }  // namespace
+
+// MLEL_ERR_UNSUPPORTED when the chain does not fit the kernel (types, shapes, alignment, live values): the caller
+// then runs the operators one by one.
+int elementwise_chain_launch(hipStream_t s, const mlel_tensor *out, const mlel_chain *c) {
+    const auto decline = [](const char *why) { return set_error(MLEL_ERR_UNSUPPORTED, "elementwise chain: %s", why); };
+    if (c->n_inputs < 1 || c->n_inputs > MLEL_CHAIN_MAX_INPUTS || c->n_steps < 1 || c->n_steps > MLEL_CHAIN_MAX_STEPS)
+        return set_error(MLEL_ERR_INVALID, "elementwise chain: %d inputs, %d steps", c->n_inputs, c->n_steps);
+    if ((out->dtype != MLEL_F16 && out->dtype != MLEL_F32) || !is_packed(out)) return decline("output type or strides");
+    const int last = out->rank - 1;
+    int64_t cols = out->dims[last];
+    const int64_t total = numel(out);
+    // rows shorter than a vector: the tensors are walked as one long row, which needs every input to have the
+    // output's shape or a single element
+    const bool flat = cols % 8 != 0;
+    if (flat) cols = total;
+    if (cols % 8 != 0 || cols >= (int64_t(1) << 31) || ((uintptr_t)out->ptr % 16) != 0) return decline("row length or alignment");
+    if (total == 0) return 0;
+    ChainArgs g{};
+    g.out = static_cast<char *>(out->ptr);
+    g.out_size = dt_size(out->dtype);
+    g.vecs = total / 8;
+    g.cols = (int32_t)cols;
+    g.cols8 = (int32_t)(cols / 8);
+    g.n_inputs = c->n_inputs;
+    g.n_steps = c->n_steps;
+    const int n_values = c->n_inputs + c->n_steps;
+    // last use of every value, then registers by linear scan
+    std::vector<int> last_use(n_values, -1), reg(n_values, -1);
+    for (int i = 0; i < c->n_steps; i++) {
+        const mlel_chain_step &st = c->steps[i];
+        const bool two = st.kind == MLEL_CHAIN_BINARY || st.kind == MLEL_CHAIN_MUL;
+        if (st.a < 0 || st.a >= c->n_inputs + i || (two && (st.b < 0 || st.b >= c->n_inputs + i)))
+            return set_error(MLEL_ERR_INVALID, "elementwise chain: step %d reads a value that does not exist yet", i);
+        last_use[st.a] = i;
+        if (two) last_use[st.b] = i;
+    }
+    last_use[n_values - 1] = c->n_steps;  // the result
+    bool all_half = out->dtype == MLEL_F16;
+    for (int k = 0; k < c->n_inputs; k++) all_half = all_half && c->inputs[k] != nullptr && c->inputs[k]->dtype == MLEL_F16;
+    for (int i = 0; i < c->n_steps; i++) all_half = all_half && c->steps[i].dtype == MLEL_F16;
+    const int n_regs = all_half ? kChainRegs + 2 : kChainRegs;
+    std::vector<int> free_regs;
+    for (int r = n_regs - 1; r >= 0; r--) free_regs.push_back(r);
+    const auto take = [&](int value) {
+        if (free_regs.empty()) return false;
+        reg[value] = free_regs.back();
+        free_regs.pop_back();
+        return true;
+    };
+    std::vector<bool> is_scalar(n_values, false);
+    int scalars = 0;
+    for (int k = 0; k < c->n_inputs; k++) {
+        const mlel_tensor *t = c->inputs[k];
+        if (t == nullptr || (t->dtype != MLEL_F16 && t->dtype != MLEL_F32)) return decline("input type");
+        int vr = 0, vc = 0;
+        if (!classify(out, t, &vr, &vc)) return decline("input shape, strides or alignment");
+        if (flat) {
+            const bool single = numel(t) == 1, same = numel(t) == total && vr == 1;
+            if (!single && !same) return decline("input shape for short rows");
+            vr = 0;
+            vc = single ? 0 : 1;
+            if (!single && ((uintptr_t)t->ptr % 16) != 0) return decline("input alignment");
+        }
+        if (!vr && !vc) {  // one element: a lane of the scalar file
+            is_scalar[k] = true;
+            reg[k] = scalars++;
+        } else if (last_use[k] >= 0) {
+            if (!take(k)) return decline("too many live values");
+        } else {
+            reg[k] = 0;  // never read: loaded into a register nothing else holds yet
+        }
+        g.in[k] = ChainInput{static_cast<const char *>(t->ptr), dt_size(t->dtype), vr, vc, reg[k]};
+    }
+    for (int i = 0; i < c->n_steps; i++) {
+        const mlel_chain_step &st = c->steps[i];
+        int op;
+        if (st.kind == MLEL_CHAIN_BINARY && st.selector == MLEL_BIN_ADD) op = F_ADD;
+        else if (st.kind == MLEL_CHAIN_BINARY && st.selector == MLEL_BIN_SUB) op = F_SUB;
+        else if (st.kind == MLEL_CHAIN_MUL) op = F_MUL;
+        else if (st.kind == MLEL_CHAIN_UNARY && st.selector == MLEL_UN_EXP) op = F_EXP;
+        else if (st.kind == MLEL_CHAIN_UNARY && st.selector == MLEL_UN_RECIPROCAL) op = F_RECIPROCAL;
+        else if (st.kind == MLEL_CHAIN_UNARY && st.selector == MLEL_UN_RSQRT) op = F_RSQRT;
+        else if (st.kind == MLEL_CHAIN_UNARY && st.selector == MLEL_UN_TANH) op = F_TANH;
+        else if (st.kind == MLEL_CHAIN_CAST) op = F_COPY;
+        else return decline("operator");
+        if (st.dtype != MLEL_F16 && st.dtype != MLEL_F32) return decline("step type");
+        const bool two = op == F_ADD || op == F_SUB || op == F_MUL;
+        const int value = c->n_inputs + i, prev = value - 1;
+        const bool a_fw = i > 0 && st.a == prev, b_fw = two && i > 0 && st.b == prev;
+        // operands die here: their registers may take the result
+        if (!is_scalar[st.a] && last_use[st.a] == i && reg[st.a] >= 0) free_regs.push_back(reg[st.a]);
+        if (two && st.b != st.a && !is_scalar[st.b] && last_use[st.b] == i && reg[st.b] >= 0) free_regs.push_back(reg[st.b]);
+        // a result that only the next step reads stays in vector registers and needs no slot
+        bool needs_slot = i + 1 < c->n_steps && last_use[value] > i + 1;
+        if (i + 1 < c->n_steps && last_use[value] == i + 1) {
+            const mlel_chain_step &nx = c->steps[i + 1];
+            const bool nx_two = nx.kind == MLEL_CHAIN_BINARY || nx.kind == MLEL_CHAIN_MUL;
+            needs_slot = !(nx.a == value || (nx_two && nx.b == value));
+        }
+        if (needs_slot && !take(value)) return decline("too many live values");
+        g.step[i] = ChainStep{(int8_t)op, (int8_t)(st.dtype == MLEL_F16), (int8_t)(a_fw ? 0 : reg[st.a]),
+                              (int8_t)(two && !b_fw ? reg[st.b] : 0), (int8_t)is_scalar[st.a],
+                              (int8_t)(two && is_scalar[st.b]), (int8_t)a_fw, (int8_t)b_fw,
+                              (int8_t)(needs_slot ? reg[value] : -1)};
+    }
+    if (c->steps[c->n_steps - 1].dtype != out->dtype) return decline("the last step must have the output's type");
+    const int64_t blocks = (g.vecs + kBlock - 1) / kBlock;
+    MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "elementwise chain: too many work items");
+    if (all_half)
+        ew_chain_kernel<true><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(g);
+    else
+        ew_chain_kernel<false><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(g);
+    return check_launch("elementwise chain");
+}
 
 int try_reduce_float_fast(mlel_ctx *, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in,
                           uint32_t axis, uint32_t nan_mode) {
@@ -323,7 +653,7 @@ int try_reduce_float_fast(mlel_ctx *, hipStream_t s, int op, const mlel_tensor *
     const int64_t blocks = (rows + 63) / 64;
     MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "reduce: too many rows");
     g.slab_cols = (int32_t)(cols < kSlabMaxCols ? cols : kSlabMaxCols);
-    const size_t smem = (size_t)64 * (g.slab_cols * 2 + 8);
+    const size_t smem = (size_t)64 * (g.slab_cols * 2 + 16);
     auto kernel = op == MLEL_RED_SUM ? reduce_rows_f16_kernel<true> : reduce_rows_f16_kernel<false>;
     if (smem > 48 * 1024)
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,

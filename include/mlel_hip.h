@@ -386,6 +386,10 @@ int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor
                                   const mlel_conv2d_attr *attr, const mlel_epilogue *epi);
 int mlel_hip_matmul_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                             const mlel_tensor *b, const mlel_matmul_attr *attr, const mlel_epilogue *epi);
+/* out(fp16) = CAST( MATMUL(a, b) + bias ): fp16 operands, fp32 accumulation, the fp32 bias [1,1,N] or [1,1,1] (or
+ * NULL) added in fp32, one rounding to fp16 -- bit for bit the unfused MATMUL -> ADD -> CAST (or MATMUL -> CAST). */
+int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
+                              const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr);
 int mlel_hip_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
                                   const mlel_tensor *weights, const mlel_tensor *bias,
                                   const mlel_conv2d_attr *attr, const mlel_epilogue *epi);
@@ -394,6 +398,29 @@ int mlel_hip_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor
 int mlel_hip_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1,
                                  const mlel_epilogue *scale1, const mlel_tensor *in2, const mlel_epilogue *scale2,
                                  const mlel_epilogue *scale_out);
+
+/* A chain of floating-point elementwise operators executed in one pass: ADD, SUB, MUL (shift 0), EXP, RECIPROCAL,
+ * RSQRT, TANH and CAST between fp16 and fp32.  Value v < n_inputs is inputs[v]; step i produces value n_inputs + i
+ * from values a (and b) and rounds it into `dtype` exactly as the stand-alone operator would; the last step's value
+ * is written to `out`.  Every step has the shape of `out`; an input has that shape, or is broadcast along the rows
+ * (all leading extents 1), along the last axis (last extent 1), or both.  Equals the operators run one after
+ * another bit for bit (no counterpart in the reference, which runs one dispatch per operator). */
+#define MLEL_CHAIN_MAX_STEPS 24
+#define MLEL_CHAIN_MAX_INPUTS 8
+enum { MLEL_CHAIN_BINARY = 0, MLEL_CHAIN_MUL = 1, MLEL_CHAIN_UNARY = 2, MLEL_CHAIN_CAST = 3 };
+typedef struct mlel_chain_step {
+    int32_t kind;     /* MLEL_CHAIN_* */
+    int32_t selector; /* mlel_binary_op (ADD, SUB) or mlel_unary_op (EXP, RECIPROCAL, RSQRT, TANH) */
+    int32_t a, b;     /* operand values; b is ignored by unary steps and casts */
+    int32_t dtype;    /* MLEL_F16 or MLEL_F32: the type of the step's result */
+} mlel_chain_step;
+typedef struct mlel_chain {
+    int32_t n_inputs;
+    int32_t n_steps;
+    const mlel_tensor *inputs[MLEL_CHAIN_MAX_INPUTS];
+    mlel_chain_step steps[MLEL_CHAIN_MAX_STEPS];
+} mlel_chain;
+int mlel_hip_elementwise_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_chain *chain);
 
 /* Plain device-to-device copy kernel of `bytes` bytes with 128-bit accesses; the calibration kernel for
  * memory-traffic counters and the measured HBM ceiling. */

@@ -207,6 +207,30 @@ class Runner:
         self.done()
         return r
 
+    def matmul_bias_cast(self, a, b, bias):
+        ta, tb = self.put(a), self.put(b)
+        tbias = self.put(bias) if bias is not None else None
+        to = self.new(abi.F16, (a.shape[0], a.shape[1], b.shape[2]))
+        self.dev.op("matmul_bias_cast", to.ref, ta.ref, tb.ref, tbias.ref if tbias else None, C.byref(abi.MatmulAttr(0, 0)))
+        r = to.download()
+        self.done()
+        return r
+
+    def chain(self, inputs, steps, out_shape, out_dtype):
+        """steps: (kind, selector, a, b, dtype) tuples as in mlel_chain_step."""
+        tin = [self.put(x) for x in inputs]
+        to = self.new(out_dtype, out_shape)
+        c = abi.Chain()
+        c.n_inputs, c.n_steps = len(tin), len(steps)
+        for i, t in enumerate(tin):
+            c.inputs[i] = C.pointer(t.view)
+        for i, st in enumerate(steps):
+            c.steps[i] = abi.ChainStep(*[int(v) for v in st])
+        self.dev.op("elementwise_chain", to.ref, C.byref(c))
+        r = to.download()
+        self.done()
+        return r
+
     # ---- the operators outside the benchmark graphs ------------------------------------------------------------
     def call(self, name, out_specs, inputs, *attrs):
         """Generic form: uploads `inputs`, allocates one output per (dtype, shape) in `out_specs`, calls

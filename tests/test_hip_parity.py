@@ -316,6 +316,70 @@ def test_matmul_f16_mfma_vs_oracle(run, oracle, case):
     np.testing.assert_array_equal(run.matmul(ai, bi, abi.F32), np.einsum("bmk,bkn->bmn", ai.astype(np.float32), bi.astype(np.float32)))
 
 
+@pytest.mark.parametrize("case", HMM_CASES, ids=[c[0] for c in HMM_CASES])
+def test_matmul_bias_cast_equals_the_three_operators(run, oracle, case):
+    """The fused fp16 projection (MATMUL -> ADD fp32 bias -> CAST fp16) is bit-identical to the three operators run one
+    after another on the GPU, and within 1e-2 of the oracle's sequential fp32 accumulation."""
+    name, nb, m, k, n = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()) + 1)
+    a = rng.standard_normal((nb, m, k)).astype(np.float16)
+    b = (0.05 * rng.standard_normal((nb, k, n))).astype(np.float16)
+    for bias in (rng.standard_normal((1, 1, n)).astype(np.float32), np.array([[[0.25]]], np.float32), None):
+        acc = run.matmul(a, b, abi.F32)
+        unfused = run.cast(run.binary("ADD", acc, bias, acc.shape, abi.F32) if bias is not None else acc, abi.F16)
+        fused = run.matmul_bias_cast(a, b, bias)
+        np.testing.assert_array_equal(fused, unfused)
+        exp = oracle.matmul(a, b, abi.F32) + (bias if bias is not None else 0)
+        assert np.abs(fused.astype(np.float32) - exp).max() <= 1e-2
+
+
+def test_elementwise_chain_equals_the_operators_one_by_one(run):
+    """mlel_hip_elementwise_chain against the same operators launched one after another (bit for bit): a GELU-shaped
+    chain over fp16 with scalar constants, a chain with row- and column-broadcast inputs and a cast, short rows, and a
+    chain the one-pass kernel declines (unaligned rows), which takes the operator-by-operator path inside the call."""
+    rng = np.random.default_rng(77)
+    B, U, M, C_ = 0, 2, 1, 3  # step kinds: binary, unary, mul, cast
+    ADD, SUB = abi.BIN["ADD"], abi.BIN["SUB"]
+    f16, f32 = abi.F16, abi.F32
+
+    def scalar(v):
+        return np.array(v, np.float16).reshape(1, 1, 1)
+
+    h = rng.standard_normal((1, 96, 256)).astype(np.float16)
+    consts = [scalar(0.044715), scalar(np.sqrt(2 / np.pi)), scalar(0.5), scalar(1.0)]
+    # values: 0 h, 1..4 constants, then steps
+    steps = [(M, 0, 0, 0, f16), (M, 0, 5, 0, f16), (M, 0, 6, 1, f16), (B, ADD, 0, 7, f16), (M, 0, 8, 2, f16),
+             (U, abi.UN["TANH"], 9, 0, f16), (B, ADD, 10, 4, f16), (M, 0, 0, 3, f16), (M, 0, 12, 11, f16)]
+    got = run.chain([h] + consts, steps, h.shape, f16)
+    t = run.mul(run.mul(run.mul(h, h, h.shape, f16), h, h.shape, f16), consts[0], h.shape, f16)
+    inner = run.mul(run.binary("ADD", h, t, h.shape, f16), consts[1], h.shape, f16)
+    exp = run.mul(run.mul(h, consts[2], h.shape, f16),
+                  run.binary("ADD", run.unary("TANH", inner), consts[3], h.shape, f16), h.shape, f16)
+    np.testing.assert_array_equal(got, exp)
+
+    x32 = rng.standard_normal((4, 24, 64)).astype(np.float32)
+    col = rng.standard_normal((4, 24, 1)).astype(np.float16)
+    row = rng.standard_normal((1, 1, 64)).astype(np.float16)
+    steps = [(C_, 0, 0, 0, f16), (B, SUB, 3, 1, f16), (U, abi.UN["EXP"], 4, 0, f16), (M, 0, 5, 2, f16),
+             (C_, 0, 6, 0, f32)]
+    got = run.chain([x32, col, row], steps, x32.shape, f32)
+    x16 = run.cast(x32, f16)
+    e = run.unary("EXP", run.binary("SUB", x16, col, x32.shape, f16))
+    np.testing.assert_array_equal(got, run.cast(run.mul(e, row, x32.shape, f16), f32))
+
+    v = np.abs(rng.standard_normal((8, 64, 1))).astype(np.float16)
+    steps = [(M, 0, 0, 1, f16), (B, ADD, 3, 2, f16), (U, abi.UN["RSQRT"], 4, 0, f16)]
+    got = run.chain([v, scalar(1 / 64), scalar(1e-3)], steps, v.shape, f16)
+    exp = run.unary("RSQRT", run.binary("ADD", run.mul(v, scalar(1 / 64), v.shape, f16), scalar(1e-3), v.shape, f16))
+    np.testing.assert_array_equal(got, exp)
+
+    odd = rng.standard_normal((3, 5, 12)).astype(np.float16)  # rows of 12: neither a vector multiple nor flat-able
+    steps = [(M, 0, 0, 0, f16), (B, ADD, 2, 1, f16)]
+    rowb = rng.standard_normal((1, 1, 12)).astype(np.float16)
+    got = run.chain([odd, rowb], steps, odd.shape, f16)
+    np.testing.assert_array_equal(got, run.binary("ADD", run.mul(odd, odd, odd.shape, f16), rowb, odd.shape, f16))
+
+
 # ------------------------------------------------------------------------------------------------ DEPTHWISE
 DW_CASES = [
     ("c2_like_small", (2, 14, 14, 144), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -4, 0),
