@@ -218,6 +218,8 @@ OP_SIGNATURES = {
 
 FUSED_SIGNATURES = {
     "conv2d_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
+    "conv2d_rescale_add_rescale": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue), C.POINTER(Epilogue), _T,
+                                   C.POINTER(Epilogue), C.POINTER(Epilogue), C.c_int],
     "matmul_rescale": [_T, _T, _T, C.POINTER(MatmulAttr), C.POINTER(Epilogue)],
     "dwconv_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
     "matmul_bias_cast": [_T, _T, _T, _T, C.POINTER(MatmulAttr)],

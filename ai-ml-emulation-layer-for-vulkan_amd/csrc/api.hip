@@ -512,6 +512,59 @@ int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor
     return 0;
 }
 
+int mlel_hip_conv2d_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                        const mlel_tensor *weights, const mlel_tensor *bias,
+                                        const mlel_conv2d_attr *attr, const mlel_epilogue *epi,
+                                        const mlel_epilogue *scale_conv, const mlel_tensor *residual,
+                                        const mlel_epilogue *scale_residual, const mlel_epilogue *scale_out,
+                                        int residual_first) {
+    MLEL_TRY(require_ctx(ctx, "conv2d_rescale_add_rescale"));
+    MLEL_REQUIRE(out != nullptr && attr != nullptr && epi != nullptr, MLEL_ERR_INVALID,
+                 "conv2d_rescale_add_rescale: null argument");
+    MLEL_TRY(check_tensor(out, "conv2d_rescale_add_rescale out"));
+    MLEL_TRY(check_tensor(residual, "conv2d_rescale_add_rescale residual"));
+    MLEL_REQUIRE(same_shape(out, residual), MLEL_ERR_INVALID, "conv2d_rescale_add_rescale: residual shape differs");
+    MLEL_REQUIRE(scale_conv && scale_residual && scale_out, MLEL_ERR_INVALID,
+                 "conv2d_rescale_add_rescale: null scale");
+    MLEL_REQUIRE(!scale_conv->has_clamp && !scale_residual->has_clamp, MLEL_ERR_INVALID,
+                 "conv2d_rescale_add_rescale: only the output stage of the addition may carry a clamp");
+    // the convolution's own result has the shape and the (8-bit) type of `out`
+    MLEL_REQUIRE(dt_size(out->dtype) == 1 && out->dtype != MLEL_BOOL, MLEL_ERR_INVALID,
+                 "conv2d_rescale_add_rescale: 8-bit output expected");
+    const int conv_dt = out->dtype;
+    mlel_tensor acc_view = packed_like(out, MLEL_I32, out->ptr);  // shape carrier for validation
+    MLEL_TRY(check_conv("conv2d_rescale_add_rescale", &acc_view, in, weights, bias, attr));
+    const int64_t ch = out->dims[3];
+    const bool one_pass = out->dtype == MLEL_I8 && residual->dtype == MLEL_I8 && conv_dt == MLEL_I8 &&
+                          is_packed(out) && is_packed(residual) && !scale_conv->rescale.per_channel &&
+                          !scale_residual->rescale.per_channel && !scale_out->rescale.per_channel;
+    if (one_pass) {
+        mlel_tensor conv_view = packed_like(out, MLEL_I8, out->ptr);
+        ConvResidual cr;
+        cr.res = residual;
+        FusedEpilogue fe;
+        MLEL_TRY(make_epilogue(epi, MLEL_I32, &conv_view, ch, &fe));
+        MLEL_TRY(make_epilogue(scale_residual, residual->dtype, &acc_view, ch, &cr.f_res));
+        MLEL_TRY(make_epilogue(scale_conv, conv_dt, &acc_view, ch, &cr.f_conv));
+        MLEL_TRY(make_epilogue(scale_out, MLEL_I32, out, ch, &cr.f_out));
+        if (cr.f_res.in_dt == MLEL_I8 && cr.f_conv.in_dt == MLEL_I8) {
+            const int rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe, &cr);
+            if (rc != 0) return rc < 0 ? rc : 0;
+        }
+    }
+    // otherwise the two fused halves in sequence through an 8-bit temporary
+    Scratch scratch;
+    MLEL_HIP_CHECK(hipMalloc(&scratch.ptr, (size_t)numel(out) + 16));
+    mlel_tensor conv_out = packed_like(out, conv_dt, scratch.ptr);
+    MLEL_TRY(mlel_hip_conv2d_rescale_clamp(ctx, stream, &conv_out, in, weights, bias, attr, epi));
+    if (residual_first)
+        MLEL_TRY(mlel_hip_rescale_add_rescale(ctx, stream, out, residual, scale_residual, &conv_out, scale_conv, scale_out));
+    else
+        MLEL_TRY(mlel_hip_rescale_add_rescale(ctx, stream, out, &conv_out, scale_conv, residual, scale_residual, scale_out));
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
 int mlel_hip_matmul_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                             const mlel_tensor *b, const mlel_matmul_attr *attr, const mlel_epilogue *epi) {
     MLEL_TRY(require_ctx(ctx, "matmul_rescale"));

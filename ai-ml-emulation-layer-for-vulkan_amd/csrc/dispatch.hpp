@@ -87,9 +87,14 @@ __device__ __forceinline__ int32_t load_mult(const ScaleRef &s, int64_t c) {
                     : reinterpret_cast<const int32_t *>(s.mult)[c];
 }
 
+// residual stage fused behind an int8 convolution: out = rescale_out(rescale_res(res) + rescale_conv(conv result))
+struct ConvResidual {
+    const mlel_tensor *res;
+    FusedEpilogue f_res, f_conv, f_out;
+};
 int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                        const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
-                       const FusedEpilogue *epi);
+                       const FusedEpilogue *epi, const ConvResidual *residual = nullptr);
 // ---- direct (dot4) convolution for very small input channel counts (conv_direct.hip) ----
 int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                          const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,

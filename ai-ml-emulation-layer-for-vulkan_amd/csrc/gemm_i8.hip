@@ -56,7 +56,7 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
     // the 256 x 256 tile when that still gives every compute unit a block, else the 128 x 128 tile under the same
     // condition as the tall tiles above.  Smaller problems keep the short tiles of the register-staged pipeline.
     const bool dl_ok = xmode == X_PLAIN && (wmode == W_ROWS || wmode == W_KMAJOR) && g.K % BK == 0 && BN == 128;
-    if (dl_ok) {
+    if (dl_ok && g.res == nullptr) {
         const int64_t total256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * g.batches;
         const bool big = total256 >= cus, mid = tall_total >= 2 * (int64_t)cus;
         if (big || mid) {
@@ -120,10 +120,13 @@ bool packed_tail(const mlel_tensor *t, int from) {
 
 }  // namespace
 
+// `residual`: the fused residual stage (see GemmArgs::res); the case is declined unless the kernel variant that
+// carries it applies (plain rows, 8-bit epilogue, not the direct-to-LDS tiles)
 int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                        const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
-                       const FusedEpilogue *epi) {
+                       const FusedEpilogue *epi, const ConvResidual *residual) {
     if (in->dtype != MLEL_I8 || w->dtype != MLEL_I8 || bias->dtype != MLEL_I32 || a->acc_type != MLEL_ACC_I32) return 0;
+    if (residual != nullptr && (epi == nullptr || out->dtype != MLEL_I8)) return 0;
     if (epi == nullptr && out->dtype != MLEL_I32) return 0;
     if (epi != nullptr && dt_size(out->dtype) > 4) return 0;
     const int64_t N = out->dims[0], OH = out->dims[1], OW = out->dims[2], OC = out->dims[3];
@@ -186,6 +189,15 @@ int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     g.ldo = OC;
     g.out_batch = 0;
     MLEL_TRY(fill_epilogue(g, out, epi));
+    if (residual != nullptr) {
+        const bool q8 = g.fused && g.out_size == 1 && g.out_vec_ok && g.o_bytes != 0;
+        const bool rows = g.plain && g.xch == 16 && g.wch == 16 && g.x_bytes != 0 && g.w_bytes != 0;
+        if (!q8 || !rows || ((uintptr_t)residual->res->ptr % 4) != 0) return 0;
+        g.res = static_cast<const int8_t *>(residual->res->ptr);
+        g.rs_res = make_ref(residual->f_res);
+        g.rs_conv = make_ref(residual->f_conv);
+        g.rs_out = make_ref(residual->f_out);
+    }
     MLEL_TRY(launch_gemm(ctx, s, g));
     return 1;
 }

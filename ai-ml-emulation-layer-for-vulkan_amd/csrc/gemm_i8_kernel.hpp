@@ -68,6 +68,10 @@ struct GemmArgs {
     const int8_t *shift;
     int32_t mult16;
     RescaleParams rp;
+    // residual stage (Q8 epilogue only): out = rescale_out(rescale_res(res[m][n]) + rescale_conv(y)), y the int8 result
+    // of the fused epilogue above; all three stages per tensor; `res` has the layout of `out`
+    const int8_t *res;
+    ScaleRef rs_res, rs_conv, rs_out;
     // launch geometry
     int32_t tiles_m, tiles_n, total_tiles, chunk;
 };
@@ -267,8 +271,9 @@ __device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N) only (expc
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int XMODE, int WMODE, bool SUMS, bool Q8>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int XMODE, int WMODE, bool SUMS, bool Q8, bool RES = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const GemmArgs g) {
+    static_assert(!RES || Q8, "the residual stage follows the 8-bit epilogue");
     constexpr int NTHREADS = WAVES_M * WAVES_N * 64;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wavefront sub-tile
     constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 MFMA tiles per wavefront
@@ -808,6 +813,14 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         // Fused RESCALE(+CLAMP) to 8-bit outputs, N % 4 == 0, output extent below 2^31: straight-line code.  Rows and
         // channels outside the problem get an offset beyond the buffer bounds, which drops the store.
         const __amdgpu_buffer_rsrc_t ores = make_rsrc(ob, g.o_bytes);
+        const __amdgpu_buffer_rsrc_t rres =
+            make_rsrc(RES ? reinterpret_cast<const char *>(g.res) + (int64_t)batch * g.out_batch : ob, g.o_bytes);
+        ChanScale q_res{}, q_conv{}, q_out{};
+        if (RES) {
+            q_res = make_chan_scale(load_mult(g.rs_res, 0), g.rs_res.shift[0], g.rs_res.p);
+            q_conv = make_chan_scale(load_mult(g.rs_conv, 0), g.rs_conv.shift[0], g.rs_conv.p);
+            q_out = make_chan_scale(load_mult(g.rs_out, 0), g.rs_out.shift[0], g.rs_out.p);
+        }
         uint32_t row_off[TM];
         int32_t xcorr[TM];
 #pragma unroll
@@ -835,6 +848,18 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                         packed |= ((uint32_t)requant_chan(a, c[e].q, g.rp) & 0xffu) << (8 * e);
                     }
                     const uint32_t off = (n0 < g.N && row_off[i] != kOobOffset) ? row_off[i] + (uint32_t)n0 : kOobOffset;
+                    if (RES) {
+                        const uint32_t xw = buf_load4(rres, off);
+                        uint32_t summed = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int32_t x = (int8_t)(xw >> (8 * e)), y = (int8_t)(packed >> (8 * e));
+                            const int32_t r1 = requant_chan(x, q_res, g.rs_res.p), r2 = requant_chan(y, q_conv, g.rs_conv.p);
+                            const int32_t sum = (int32_t)((uint32_t)r1 + (uint32_t)r2);
+                            summed |= ((uint32_t)requant_chan(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
+                        }
+                        packed = summed;
+                    }
                     __builtin_amdgcn_raw_buffer_store_b32(packed, ores, (int)off, 0, 0);
                 }
             }
@@ -925,6 +950,11 @@ void launch_tile(const GemmArgs &g, int xmode, int wmode, dim3 grid, hipStream_t
         if (xmode == X_PLAIN_DL && wmode == W_KMAJOR_DL)
             return launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN_DL, W_KMAJOR_DL, SUMS, Q8>, g,
                                  WAVES_M * WAVES_N * 64, smem_bytes_dl<BM, BN>(), grid, s);
+    }
+    if constexpr (Q8 && BM * BN <= 128 * 128) {  // residual stage: the 1x1 projections (plain rows on both sides)
+        if (g.res != nullptr && xmode == X_PLAIN && wmode == W_ROWS)
+            return launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_ROWS, SUMS, Q8, true>, g,
+                                 WAVES_M * WAVES_N * 64, sm, grid, s);
     }
     if (xmode == X_PLAIN && wmode == W_ROWS)
         launch_kernel(gemm_i8_kernel<BM, BN, WAVES_M, WAVES_N, X_PLAIN, W_ROWS, SUMS, Q8>, g, WAVES_M * WAVES_N * 64, sm, grid, s);

@@ -256,6 +256,8 @@ std::string opLabel(const OpNode &op) {
     case OpKind::FusedDepthwiseConv2D: return std::string("DEPTHWISE_CONV2D+RESCALE") + (op.hasClamp ? "+CLAMP" : "");
     case OpKind::FusedMatmul: return std::string("MATMUL+RESCALE") + (op.hasClamp ? "+CLAMP" : "");
     case OpKind::FusedRescaleAddRescale: return "RESCALE+RESCALE+ADD+RESCALE";
+    case OpKind::FusedConv2DResidual:
+        return std::string("CONV2D+RESCALE") + (op.hasClamp ? "+CLAMP" : "") + "+RESCALE+RESCALE+ADD+RESCALE";
     case OpKind::FusedElementwise: return "ELEMENTWISE x" + std::to_string(op.chain.size());
     case OpKind::FusedMatmulBiasCast: return op.inputs.size() > 2 ? "MATMUL+ADD+CAST" : "MATMUL+CAST";
     default: return op.tosaName;

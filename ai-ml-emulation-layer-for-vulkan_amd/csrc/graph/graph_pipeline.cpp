@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <cstring>
+#include <unordered_map>
 
 #include "session_planner.hpp"
 
@@ -663,6 +664,56 @@ void GraphPipeline::fuse() {
         ra->fusedAway = rb->fusedAway = ro.fusedAway = true;
     }
 
+    // Pattern 3 (residual connection behind a projection): a fused addition one of whose operands is the 8-bit result
+    // of a fused 1x1 convolution read nowhere else moves into that convolution's epilogue, which then reads the
+    // other operand at the position it is about to write.  Legal when the other operand exists before the
+    // convolution runs and all three RESCALE stages of the addition are per tensor; the epilogue applies the same
+    // three stages to the same two 8-bit values, so the result is bit-identical.  Restricted to the layouts the
+    // one-pass kernel takes (dense 1x1, stride 1, unpadded, channel counts in whole 16-byte / 4-byte units), since
+    // the fallback behind the entry point allocates.
+    {
+        std::unordered_map<const OpNode *, size_t> position;
+        for (size_t i = 0; i < ops.size(); i++) position[ops[i].get()] = i;
+        for (const auto &opPtr : ops) {
+            OpNode &add = *opPtr;
+            if (add.fusedAway || add.kind != OpKind::FusedRescaleAddRescale) continue;
+            if (add.outputs[0]->getFormat() != MLEL_I8 || !add.outputs[0]->isPacked()) continue;
+            if (add.scaleA.attr.per_channel || add.scaleB.attr.per_channel || add.epilogue.attr.per_channel ||
+                add.scaleA.attr.input_unsigned || add.scaleB.attr.input_unsigned)
+                continue;
+            for (int side = 0; side < 2; side++) {
+                const TensorPtr &convOut = add.inputs[side], &residual = add.inputs[1 - side];
+                OpNode *conv = convOut->getProducer();
+                if (!conv || conv->fusedAway || conv->kind != OpKind::FusedConv2D || conv->outputs[0].get() != convOut.get())
+                    continue;
+                if (convOut->getFormat() != MLEL_I8 || residual->getFormat() != MLEL_I8 || convOut.get() == residual.get() ||
+                    !isPrivateIntermediate(*convOut) || consumersOf(ops, convOut.get()).size() != 1 || !residual->isPacked())
+                    continue;
+                const OpNode *resProducer = residual->getProducer();
+                if (resProducer != nullptr && position.at(resProducer) >= position.at(conv)) continue;
+                if (residual->getKind() == TensorKind::Session && resProducer == nullptr && !residual->isGraphInput) continue;
+                const auto &x = conv->inputs[0], &w = conv->inputs[1];
+                const auto &wd = w->getDimensions();
+                const mlel_conv2d_attr &a = conv->conv;
+                const bool pointwise = wd[1] == 1 && wd[2] == 1 && a.stride[0] == 1 && a.stride[1] == 1 && a.pad[0] == 0 &&
+                                       a.pad[1] == 0 && a.pad[2] == 0 && a.pad[3] == 0;
+                if (!pointwise || !x->isPacked() || !w->isPacked() || wd[3] % 16 != 0 || wd[0] % 4 != 0 ||
+                    conv->epilogue.attr.output_unsigned)
+                    continue;
+                conv->kind = OpKind::FusedConv2DResidual;
+                conv->scaleA = side == 0 ? add.scaleA : add.scaleB;
+                conv->scaleB = side == 0 ? add.scaleB : add.scaleA;
+                conv->scaleOut = add.epilogue;
+                conv->flag = side == 1;
+                conv->inputs.push_back(residual);
+                conv->outputs[0] = add.outputs[0];
+                add.outputs[0]->setProducer(conv);
+                add.fusedAway = true;
+                break;
+            }
+        }
+    }
+
     // Pattern 4 (fp16 projections): MATMUL (fp16 x fp16 -> fp32)  [-> ADD of an fp32 constant of one or N values]
     // -> CAST to fp16.  The fused kernel adds in fp32 and rounds once to fp16, exactly like the operators it replaces.
     for (const auto &opPtr : ops) {
@@ -856,7 +907,7 @@ void GraphPipeline::plan() {
         if (op->fusedAway) continue;
         for (const auto &t : op->inputs) touch(t, idx);
         for (const auto &t : op->outputs) touch(t, idx);
-        for (const auto *spec : {&op->epilogue, &op->scaleA, &op->scaleB}) {
+        for (const auto *spec : {&op->epilogue, &op->scaleA, &op->scaleB, &op->scaleOut}) {
             touch(spec->multiplier, idx);
             touch(spec->shift, idx);
         }
@@ -933,7 +984,7 @@ std::vector<details::BestFitTensor> GraphPipeline::bestFitTensors(const std::vec
             if (it != index.end()) consumers[it->second].push_back(p);
         };
         for (const auto &t : op.inputs) reads(t);
-        for (const auto *spec : {&op.epilogue, &op.scaleA, &op.scaleB}) {
+        for (const auto *spec : {&op.epilogue, &op.scaleA, &op.scaleB, &op.scaleOut}) {
             reads(spec->multiplier);
             reads(spec->shift);
         }
@@ -1126,6 +1177,20 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
         rc = mlel_hip_matmul_bias_cast(ctx, stream, &out, &in[0], &in[1], op.inputs.size() > 2 ? &in[2] : nullptr,
                                        &op.matmul);
         break;
+    case OpKind::FusedConv2DResidual: {
+        const mlel_tensor mult = op.epilogue.multiplier->view(), shift = op.epilogue.shift->view();
+        const mlel_tensor ma = op.scaleA.multiplier->view(), sa = op.scaleA.shift->view();
+        const mlel_tensor mb = op.scaleB.multiplier->view(), sb = op.scaleB.shift->view();
+        const mlel_tensor mo = op.scaleOut.multiplier->view(), so = op.scaleOut.shift->view();
+        const mlel_clamp_attr none{};
+        const mlel_epilogue e = makeEpilogue(op.epilogue, &mult, &shift, op.hasClamp, op.clamp);
+        const mlel_epilogue ea = makeEpilogue(op.scaleA, &ma, &sa, false, none);
+        const mlel_epilogue eb = makeEpilogue(op.scaleB, &mb, &sb, false, none);
+        const mlel_epilogue eo = makeEpilogue(op.scaleOut, &mo, &so, false, none);
+        rc = mlel_hip_conv2d_rescale_add_rescale(ctx, stream, &out, &in[0], &in[1], &in[2], &op.conv, &e, &ea, &in[3], &eb,
+                                                 &eo, op.flag ? 1 : 0);
+        break;
+    }
     case OpKind::FusedRescaleAddRescale: {
         const mlel_tensor ma = op.scaleA.multiplier->view(), sa = op.scaleA.shift->view();
         const mlel_tensor mb = op.scaleB.multiplier->view(), sb = op.scaleB.shift->view();

@@ -98,6 +98,7 @@ enum class OpKind {
     Argmax, ArithmeticRightShift, Conv3D, TransposeConv2D, Fft2D, Rfft2D, Gather, Scatter, Resize, Reverse, Tile, Select,
     // produced by the fusion pass only
     FusedConv2D, FusedDepthwiseConv2D, FusedMatmul, FusedRescaleAddRescale, FusedMatmulBiasCast, FusedElementwise,
+    FusedConv2DResidual,
 };
 
 struct RescaleSpec {
@@ -135,6 +136,9 @@ class OpNode {
     RescaleSpec epilogue;            // Fused*: RESCALE applied to the accumulator
     bool hasClamp = false;           // Fused*: CLAMP after the RESCALE
     RescaleSpec scaleA, scaleB;      // FusedRescaleAddRescale: the two input stages (epilogue = output stage)
+    // FusedConv2DResidual: epilogue (+ clamp) belongs to the convolution; scaleA rescales its 8-bit result, scaleB the
+    // residual (inputs[3]), scaleOut their sum; `flag` is set when the residual was the addition's first operand
+    RescaleSpec scaleOut;
 };
 
 class GraphPipeline {

@@ -384,6 +384,16 @@ int mlel_hip_select(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const m
 int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
                                   const mlel_tensor *weights, const mlel_tensor *bias,
                                   const mlel_conv2d_attr *attr, const mlel_epilogue *epi);
+/* out = RESCALE_out( RESCALE_conv( CONV2D -> RESCALE -> [CLAMP] (epi) ) + RESCALE_residual(residual) ): the
+ * residual connection behind a projecting convolution, bit for bit mlel_hip_conv2d_rescale_clamp into an 8-bit
+ * temporary of `out`'s type followed by mlel_hip_rescale_add_rescale.  The integer addition wraps, so the operand order
+ * (`residual_first`) only matters to the unfused fallback's argument order. */
+int mlel_hip_conv2d_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                        const mlel_tensor *weights, const mlel_tensor *bias,
+                                        const mlel_conv2d_attr *attr, const mlel_epilogue *epi,
+                                        const mlel_epilogue *scale_conv, const mlel_tensor *residual,
+                                        const mlel_epilogue *scale_residual, const mlel_epilogue *scale_out,
+                                        int residual_first);
 int mlel_hip_matmul_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                             const mlel_tensor *b, const mlel_matmul_attr *attr, const mlel_epilogue *epi);
 /* out(fp16) = CAST( MATMUL(a, b) + bias ): fp16 operands, fp32 accumulation, the fp32 bias [1,1,N] or [1,1,1] (or

@@ -207,6 +207,17 @@ class Runner:
         self.done()
         return r
 
+    def conv2d_rescale_add_rescale(self, x, w, b, attr, epi, e_conv, res, e_res, e_out, residual_first=False,
+                                   res_strides=None):
+        tx, tw, tb, tr = self.put(x), self.put(w), self.put(b), self.put(res, strides=res_strides)
+        to = self.new(abi.I8, res.shape)
+        e0, e1, e2, e3 = self._epi(*epi), self._epi(*e_conv), self._epi(*e_res), self._epi(*e_out)
+        self.dev.op("conv2d_rescale_add_rescale", to.ref, tx.ref, tw.ref, tb.ref, C.byref(attr), C.byref(e0),
+                    C.byref(e1), tr.ref, C.byref(e2), C.byref(e3), int(residual_first))
+        r = to.download()
+        self.done()
+        return r
+
     def matmul_bias_cast(self, a, b, bias):
         ta, tb = self.put(a), self.put(b)
         tbias = self.put(bias) if bias is not None else None

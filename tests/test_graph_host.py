@@ -79,13 +79,14 @@ def _build_host_only(spec, fuse):
 def test_fusion_of_inverted_residual_block():
     spec = graphs.inverted_residual_spec(batch=2, hw=8)
     g = _build_host_only(spec, fuse=True)
-    assert g.op_names() == ["CONV2D+RESCALE+CLAMP", "DEPTHWISE_CONV2D+RESCALE+CLAMP", "CONV2D+RESCALE",
-                            "RESCALE+RESCALE+ADD+RESCALE"]
+    # the residual addition sits in the epilogue of the projection that feeds it
+    assert g.op_names() == ["CONV2D+RESCALE+CLAMP", "DEPTHWISE_CONV2D+RESCALE+CLAMP",
+                            "CONV2D+RESCALE+RESCALE+RESCALE+ADD+RESCALE"]
     u = _build_host_only(spec, fuse=False)
     assert u.op_names() == [o["op"] for o in spec.ops]
     # fused: the int32 accumulators are gone, nothing that is live at the same time overlaps
     live = [t for t in g.session_tensors() if t["offset"] is not None]
-    assert len(live) == 3 and all(t["size"] == 2 * 8 * 8 * c for t, c in zip(live, (144, 144, 24)))
+    assert len(live) == 2 and all(t["size"] == 2 * 8 * 8 * 144 for t in live)
     for a in live:
         for b in live:
             if a is not b and not (a["last"] < b["first"] or b["last"] < a["first"]):
@@ -103,9 +104,10 @@ def test_mobilenetv2_graph_structure_and_plan():
     assert (full.macs["dense"] + full.macs["depthwise"]) // 32 == 300774272
     g = _build_host_only(spec, fuse=True)
     names = g.op_names()
-    # contractions, residual adds, pool + fc; the RESHAPE between two session tensors became a view of its input
-    assert len(names) == 35 + 17 + 10 + 2 and "RESHAPE" not in names
-    assert names.count("RESCALE+RESCALE+ADD+RESCALE") == 10 and names[-1] == "MATMUL+RESCALE"
+    # contractions (10 of the projections carry their block's residual addition), pool + fc; the RESHAPE between
+    # two session tensors became a view of its input
+    assert len(names) == 35 + 17 + 2 and "RESHAPE" not in names
+    assert names.count("CONV2D+RESCALE+RESCALE+RESCALE+ADD+RESCALE") == 10 and names[-1] == "MATMUL+RESCALE"
     planned = [t for t in g.session_tensors() if t["offset"] is not None]
     views = [t for t in planned if t["first"] == 0xFFFFFFFF]
     source = [t for t in planned if t["handle"] == views[0]["handle"] - 1]
@@ -206,7 +208,8 @@ def test_memory_planners_give_valid_plans(which):
             assert size == sum((s + align - 1) // align * align for _, s in distinct)
         g.close()
     assert sizes["interval"] <= sizes["linear"] and sizes["bestfit"] <= sizes["linear"]
-    assert sizes["interval"] < sizes["linear"]  # the graphs do have tensors with disjoint lifetimes
+    if which != "inverted_residual":  # (its two session tensors are live together once the addition is fused away)
+        assert sizes["interval"] < sizes["linear"]  # the graphs do have tensors with disjoint lifetimes
 
 
 def test_memory_planner_from_environment(monkeypatch):

@@ -678,3 +678,40 @@ def test_config1_matmul_rescale_full_size(run, oracle):
     np.testing.assert_array_equal(run.matmul(a, b, abi.I8, 2, -1, epilogue=(mult, shift, rattr, None)), exp)
     # the requantised result uses the whole int8 range (a degenerate all-zero output would prove nothing)
     assert exp.min() < -20 and exp.max() > 20
+
+
+RESIDUAL_CASES = [
+    # name, x shape, OC, kernel, pad: 1x1 projections take the one-pass kernel, the 3x3 case the two-kernel sequence
+    ("project_96_24", (2, 14, 14, 96), 24, (1, 1), (0, 0, 0, 0)),
+    ("project_192_32_ragged", (3, 7, 9, 192), 32, (1, 1), (0, 0, 0, 0)),
+    ("project_960_160", (1, 7, 7, 960), 160, (1, 1), (0, 0, 0, 0)),
+    ("k3_32_16", (1, 8, 8, 32), 16, (3, 3), (1, 1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", RESIDUAL_CASES, ids=[c[0] for c in RESIDUAL_CASES])
+def test_conv2d_rescale_add_rescale_equals_the_operator_sequence(run, oracle, case):
+    name, xs, oc, k, pad = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    x = ri(rng, -128, 127, xs, np.int8)
+    w = ri(rng, -128, 127, (oc,) + k + (xs[3],), np.int8)
+    b = ri(rng, -2 ** 15, 2 ** 15, (oc,), np.int32)
+    attr = abi.conv2d_attr(pad, (1, 1), (1, 1), -4, 0)
+    shape = (xs[0], xs[1], xs[2], oc)
+    res = ri(rng, -128, 127, shape, np.int8)
+    mult, shift = rescale_params(rng, oc)
+    rattr = abi.rescale_attr(0, 3, True, True, True)
+    m1, s1 = np.array([1 << 30], np.int32), np.array([11], np.int8)
+    m2, s2 = np.array([1431655765], np.int32), np.array([12], np.int8)
+    mo, so = np.array([1717986918], np.int32), np.array([50], np.int8)
+    a_conv = abi.rescale_attr(3, 0, True, True, False)
+    a_res = abi.rescale_attr(-7, 0, True, True, False)
+    a_out = abi.rescale_attr(0, -2, True, True, False)
+    conv8 = oracle.clamp(oracle.rescale(oracle.conv2d(x, w, b, shape, abi.I32, attr), mult, shift, abi.I8, rattr), -90, 90)
+    r_conv = oracle.rescale(conv8, m1, s1, abi.I32, a_conv)
+    r_res = oracle.rescale(res, m2, s2, abi.I32, a_res)
+    exp = oracle.rescale(oracle.elementwise_binary("ADD", r_res, r_conv, shape, abi.I32), mo, so, abi.I8, a_out)
+    for first in (False, True):
+        out = run.conv2d_rescale_add_rescale(x, w, b, attr, (mult, shift, rattr, (-90, 90)), (m1, s1, a_conv, None), res,
+                                             (m2, s2, a_res, None), (mo, so, a_out, None), residual_first=first)
+        np.testing.assert_array_equal(out, exp)
