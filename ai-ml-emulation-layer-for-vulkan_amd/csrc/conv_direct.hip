@@ -55,7 +55,7 @@ __host__ __device__ constexpr uint32_t pixel_mask(int p, int d) {
 }
 
 // KD = dwords of gathered input per position; STEM: 3 rows x 3 dwords (IC = ICS), ROWS: IC / 4
-template <int MODE, int ICS, int KD, int OCB, int P>
+template <int MODE, int ICS, int KD, int OCB, int P, bool Q8>
 __global__ void __launch_bounds__(kBlock) conv_direct_i8_kernel(const DirectArgs a) {
     __shared__ __align__(16) uint32_t wl[OCB][KD];
     __shared__ __align__(16) ChanConst cc[OCB];
@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(kBlock) conv_direct_i8_kernel(const DirectArgs
         const int32_t bias = a.bias[a.bias_len == 1 ? 0 : oc0 + oc];
         c.bias_adj = (int32_t)((uint32_t)bias - (uint32_t)a.zx * (uint32_t)wsum +
                                (uint32_t)kreal * (uint32_t)a.zx * (uint32_t)a.zw);
-        if (a.fused) {
+        if (Q8) {
             const int ci = a.scale.p.per_channel ? oc0 + oc : 0;
             c.q = make_chan_scale(load_mult(a.scale, ci), (int32_t)a.scale.shift[ci], a.scale.p);
         }
@@ -186,7 +186,7 @@ __global__ void __launch_bounds__(kBlock) conv_direct_i8_kernel(const DirectArgs
 #pragma unroll
                 for (int j = 0; j < KD; j++) acc = __builtin_amdgcn_sdot4((int)xd[p][j], (int)wv[j], acc, false);
                 const int32_t v = (int32_t)((uint32_t)acc + (uint32_t)c.bias_adj - (uint32_t)xcorr[p]);
-                if (a.out_size == 1) {
+                if (Q8) {
                     packed[p][e / 4] |= ((uint32_t)requant_chan(v, c.q, a.scale.p) & 0xffu) << (8 * (e % 4));
                 } else {
                     packed[p][e % 4] = (uint32_t)v;
@@ -196,7 +196,7 @@ __global__ void __launch_bounds__(kBlock) conv_direct_i8_kernel(const DirectArgs
                 }
             }
         }
-        if (a.out_size == 1) {
+        if (Q8) {
 #pragma unroll
             for (int p = 0; p < P; p++)
                 if (mpos[p] < a.M)
@@ -206,12 +206,38 @@ __global__ void __launch_bounds__(kBlock) conv_direct_i8_kernel(const DirectArgs
     }
 }
 
-template <int MODE, int ICS, int KD>
-void launch_direct(const DirectArgs &g, dim3 grid, hipStream_t s) {
-    if (g.ocb == 32)
-        conv_direct_i8_kernel<MODE, ICS, KD, 32, 1><<<grid, dim3(kBlock), 0, s>>>(g);
+template <int MODE, int ICS, int KD, int P>
+void launch_direct_p(const DirectArgs &g, dim3 grid, hipStream_t s) {
+    // fused 8-bit epilogue or int32 accumulators: a compile-time choice, so that the unrolled channel loop is one
+    // basic block and the requantisation chains of neighbouring channels interleave
+    if (g.ocb == 32 && g.out_size == 1)
+        conv_direct_i8_kernel<MODE, ICS, KD, 32, P, true><<<grid, dim3(kBlock), 0, s>>>(g);
+    else if (g.ocb == 32)
+        conv_direct_i8_kernel<MODE, ICS, KD, 32, P, false><<<grid, dim3(kBlock), 0, s>>>(g);
+    else if (g.out_size == 1)
+        conv_direct_i8_kernel<MODE, ICS, KD, 16, P, true><<<grid, dim3(kBlock), 0, s>>>(g);
     else
-        conv_direct_i8_kernel<MODE, ICS, KD, 16, 1><<<grid, dim3(kBlock), 0, s>>>(g);
+        conv_direct_i8_kernel<MODE, ICS, KD, 16, P, false><<<grid, dim3(kBlock), 0, s>>>(g);
+}
+
+// Positions per thread: every channel's weights and constants are broadcast from shared memory once per thread, so
+// two positions per thread halve that traffic.  It pays for the shortest rows only (16-byte pixels, 32 channels per
+// block, measured); longer rows lose more to the registers the second position holds.
+template <int MODE, int ICS, int KD>
+void launch_direct(DirectArgs &g, int splits, int cus, hipStream_t s) {
+    int p = 1;
+    if (MODE == ROWS && KD == 4 && g.ocb == 32 && g.out_size == 1) {
+        const int64_t blocks = (g.M + (int64_t)kBlock * 2 - 1) / ((int64_t)kBlock * 2);
+        if (blocks * splits >= 2 * (int64_t)cus) p = 2;  // still two blocks per compute unit
+    }
+    g.blocks = (int)((g.M + (int64_t)kBlock * p - 1) / ((int64_t)kBlock * p));
+    g.chunk = (g.blocks + 7) / 8;
+    const dim3 grid((unsigned)(g.chunk * 8), (unsigned)splits);
+    if (p == 2) {
+        if constexpr (MODE == ROWS && KD == 4) launch_direct_p<MODE, ICS, KD, 2>(g, grid, s);
+    } else {
+        launch_direct_p<MODE, ICS, KD, 1>(g, grid, s);
+    }
 }
 
 }  // namespace
@@ -219,7 +245,6 @@ void launch_direct(const DirectArgs &g, dim3 grid, hipStream_t s) {
 int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                          const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
                          const FusedEpilogue *epi) {
-    (void)ctx;
     if (in->dtype != MLEL_I8 || w->dtype != MLEL_I8 || bias->dtype != MLEL_I32 || a->acc_type != MLEL_ACC_I32) return 0;
     if (epi == nullptr && out->dtype != MLEL_I32) return 0;
     if (epi != nullptr && dt_size(out->dtype) != 1) return 0;
@@ -287,23 +312,21 @@ int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, c
     const int splits = (int)(OC / ocb);
     if (splits > 65535) return 0;
     g.ocb = ocb;
-    g.blocks = (int)((M + kBlock - 1) / kBlock);
-    g.chunk = (g.blocks + 7) / 8;
-    const dim3 grid((unsigned)(g.chunk * 8), (unsigned)splits);
+    const int cus = ctx != nullptr ? ctx->props.multiProcessorCount : 256;
     if (mode == STEM) {
         if (IC == 1)
-            launch_direct<STEM, 1, 9>(g, grid, s);
+            launch_direct<STEM, 1, 9>(g, splits, cus, s);
         else if (IC == 3)
-            launch_direct<STEM, 3, 9>(g, grid, s);
+            launch_direct<STEM, 3, 9>(g, splits, cus, s);
         else
-            launch_direct<STEM, 4, 9>(g, grid, s);
+            launch_direct<STEM, 4, 9>(g, splits, cus, s);
     } else {
         if (IC == 16)
-            launch_direct<ROWS, 4, 4>(g, grid, s);
+            launch_direct<ROWS, 4, 4>(g, splits, cus, s);
         else if (IC == 24)
-            launch_direct<ROWS, 4, 6>(g, grid, s);
+            launch_direct<ROWS, 4, 6>(g, splits, cus, s);
         else
-            launch_direct<ROWS, 4, 8>(g, grid, s);
+            launch_direct<ROWS, 4, 8>(g, splits, cus, s);
     }
     MLEL_TRY(check_launch("conv2d direct int8"));
     return 1;

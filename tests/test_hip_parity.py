@@ -143,6 +143,9 @@ CONV_CASES = [
     ("stem_ic4_s3", (1, 14, 15, 4), 48, (3, 3), (2, 1, 0, 2), (3, 2), (1, 1), -7, 1),
     ("pw_32_16_zw", (2, 12, 12, 32), 16, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 6, -6),
     ("pw_32_192", (1, 28, 28, 32), 192, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -100, 0),
+    # enough positions for the direct kernel to take two per thread, ragged last block; a long run of 24-byte pixels
+    ("pw_16_96_two_positions", (2, 223, 225, 16), 96, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 17, 0),
+    ("pw_24_144_many_positions", (1, 251, 243, 24), 144, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -9, 4),
 ]
 
 
