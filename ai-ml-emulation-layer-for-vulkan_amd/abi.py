@@ -46,6 +46,31 @@ def dtype_of_numpy(dt):
     return _OF_NP[np.dtype(dt)]
 
 
+TAGGED = (BF16, F8E4M3, F8E5M2)  # element types carried in an unsigned integer array with a tag
+
+
+class Typed(np.ndarray):
+    """A numpy array that carries the element type of a format numpy has no dtype for: bf16 lives in uint16 words, the
+    fp8 encodings in uint8 bytes.  Views, slices and `zeros_like` keep the tag."""
+
+    def __array_finalize__(self, obj):
+        self.mlel_dtype = getattr(obj, "mlel_dtype", None)
+
+
+def typed(arr, dtype):
+    """Tag `arr` (uint16 words for BF16, uint8 bytes for F8E4M3 / F8E5M2) with its element type."""
+    arr = np.asarray(arr)
+    assert arr.dtype == NP_OF[dtype], (arr.dtype, dtype)
+    v = arr.view(Typed)
+    v.mlel_dtype = dtype
+    return v
+
+
+def dtype_of_array(arr):
+    tag = getattr(arr, "mlel_dtype", None)
+    return tag if tag is not None else dtype_of_numpy(arr.dtype)
+
+
 class Tensor(C.Structure):
     """struct mlel_tensor"""
     _fields_ = [("ptr", C.c_void_p), ("dtype", C.c_int32), ("rank", C.c_int32), ("dims", C.c_int64 * MAX_RANK),
@@ -290,6 +315,12 @@ def bind_oracle(lib):
     lib.mlel_cpu_f32_to_f16.argtypes = [C.c_float]
     lib.mlel_cpu_f16_to_f32.restype = C.c_float
     lib.mlel_cpu_f16_to_f32.argtypes = [C.c_uint16]
+    lib.mlel_cpu_f32_to_bf16.restype = C.c_uint16
+    lib.mlel_cpu_f32_to_bf16.argtypes = [C.c_float, C.c_int]
+    lib.mlel_cpu_f32_to_f8.restype = C.c_uint8
+    lib.mlel_cpu_f32_to_f8.argtypes = [C.c_float, C.c_int]
+    lib.mlel_cpu_f8_to_f32.restype = C.c_float
+    lib.mlel_cpu_f8_to_f32.argtypes = [C.c_uint8, C.c_int]
     return lib
 
 

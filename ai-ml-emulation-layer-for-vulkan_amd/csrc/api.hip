@@ -36,8 +36,12 @@ int check_conv(const char *name, const mlel_tensor *out, const mlel_tensor *in, 
                  "%s: ranks must be 4,4,4,1", name);
     MLEL_REQUIRE(a->acc_type >= 1 && a->acc_type <= 4, MLEL_ERR_INVALID, "Unsupported acc type %u", a->acc_type);
     const bool facc = a->acc_type == MLEL_ACC_F16 || a->acc_type == MLEL_ACC_F32;
-    MLEL_REQUIRE(facc == dt_is_float(in->dtype) && facc == dt_is_float(out->dtype), MLEL_ERR_INVALID,
+    // a floating-point accumulator needs floating-point tensors; an integer accumulator over floating-point storage
+    // truncates the operands toward zero like the shaders' ACC_TYPE(v) conversion (common.comp:636-660)
+    MLEL_REQUIRE(!facc || (dt_is_float(in->dtype) && dt_is_float(out->dtype)), MLEL_ERR_INVALID,
                  "%s: accumulator type %u does not match the tensor types", name, a->acc_type);
+    MLEL_REQUIRE(dt_is_float(in->dtype) == dt_is_float(out->dtype), MLEL_ERR_INVALID,
+                 "%s: input and output must both be integer or both floating point", name);
     MLEL_REQUIRE(bias->dtype == out->dtype, MLEL_ERR_INVALID, "%s: bias must have the output type", name);
     return 0;
 }

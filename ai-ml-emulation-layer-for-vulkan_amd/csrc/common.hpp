@@ -52,7 +52,12 @@ __host__ __device__ inline int dt_size(int dt) {
     }
 }
 __host__ __device__ inline bool dt_is_int(int dt) { return dt >= MLEL_BOOL && dt <= MLEL_U64; }
-__host__ __device__ inline bool dt_is_float(int dt) { return dt == MLEL_F16 || dt == MLEL_F32 || dt == MLEL_F64; }
+__host__ __device__ inline bool dt_is_float(int dt) {
+    return dt == MLEL_F16 || dt == MLEL_F32 || dt == MLEL_F64 || dt == MLEL_BF16 || dt == MLEL_F8E4M3 || dt == MLEL_F8E5M2;
+}
+__host__ __device__ inline bool dt_is_fp8(int dt) { return dt == MLEL_F8E4M3 || dt == MLEL_F8E5M2; }
+// The type arithmetic runs in (getFormatInfo's compType, common/utils.cpp:119-228): fp8 computes in fp16, bf16 in fp32.
+__host__ __device__ inline int dt_comp(int dt) { return dt_is_fp8(dt) ? MLEL_F16 : (dt == MLEL_BF16 ? MLEL_F32 : dt); }
 __host__ __device__ inline int64_t dt_lowest(int dt) {
     switch (dt) {
     case MLEL_I8: return -128;
@@ -169,19 +174,90 @@ __device__ inline void raw_st_i(char *p, int dt, int64_t v) {
     default: break;
     }
 }
+// fp32 -> fp16, nearest even.  The value is made opaque first: the compiler otherwise folds a multiplication that
+// feeds the conversion into v_fma_mix*_f16 with a +0 addend, and (-0) * x + (+0) is +0 where the product is -0.
+__device__ __forceinline__ __half f2h(float v) {
+    asm("" : "+v"(v));
+    return __float2half_rn(v);
+}
+
+// ---- reduced-precision storage formats (graph/shaders/graph_op/common.comp:184-232, 300-418) ----
+// bf16 is the upper half of an fp32; fp8 e5m2 the upper byte of an fp16; fp8 e4m3 has bias 7, no infinities and
+// one NaN code per sign (0x7f).  Every fp8 value is an fp16 value, every bf16 value an fp32 value.
+__device__ inline float decode_bf16(uint16_t x) { return __uint_as_float((uint32_t)x << 16); }
+__device__ inline float decode_f8e5m2(uint8_t x) { return __half2float(__ushort_as_half((unsigned short)((uint32_t)x << 8))); }
+__device__ inline float decode_f8e4m3(uint8_t x) {
+    const uint32_t sign = (x >> 7) & 1u, e = (x >> 3) & 0xfu, m = x & 7u;
+    if (e == 0xfu && m == 7u) return NAN;
+    const float v = e == 0 ? (float)m / 512.0f : ldexpf(1.0f + (float)m / 8.0f, (int)e - 7);
+    return sign ? -v : v;
+}
+// bf16 by truncation (the default store of most operators) and by round-to-nearest-even (ADD-like operators, MUL, CAST)
+__device__ inline uint16_t encode_bf16_trunc(float v) { return (uint16_t)(__float_as_uint(v) >> 16); }
+__device__ inline uint16_t encode_bf16_rne(float v) {
+    uint32_t u = __float_as_uint(v);
+    if ((u & 0x7f800000u) == 0x7f800000u) return (uint16_t)((u >> 16) | ((u & 0x007fffffu) ? 0x0040u : 0u));
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+// fp8 from fp32: e5m2 rounds to fp16 (nearest even) and drops the low byte; beyond +-57344 it saturates to infinity
+__device__ inline uint8_t encode_f8e5m2(float v) {
+    const uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
+    if (isnan(v)) return (uint8_t)(sign | 0x7du);
+    if (isinf(v) || v > 57344.0f || v < -57344.0f) return (uint8_t)(sign | 0x7cu);
+    return (uint8_t)(__half_as_ushort(f2h(v)) >> 8);
+}
+// e4m3 rounds the mantissa to nearest even; NaN, infinities and magnitudes above 448 give the NaN code
+__device__ inline uint8_t encode_f8e4m3(float v) {
+    const uint32_t bits = __float_as_uint(v), sign = (bits >> 24) & 0x80u;
+    const float ax = fabsf(v);
+    if (isnan(v) || isinf(v) || ax > 448.0f) return (uint8_t)(sign | 0x7fu);
+    if (ax == 0.0f) return (uint8_t)sign;
+    if (ax < 0.015625f) {  // below 2^-6: multiples of 2^-9
+        float r = rintf(ax * 512.0f);
+        r = r < 0.f ? 0.f : (r > 8.f ? 8.f : r);
+        const uint32_t m = (uint32_t)r;
+        if (m == 0) return (uint8_t)sign;
+        if (m >= 8) return (uint8_t)(sign | 0x08u);
+        return (uint8_t)(sign | m);
+    }
+    int exponent = (int)((bits >> 23) & 0xffu) - 127;   // floor(log2(ax)) of a normal fp32
+    const uint32_t frac = bits & 0x007fffffu;           // (scaled - 1) * 2^23
+    uint32_t m = (frac + 0x7ffffu + ((frac >> 20) & 1u)) >> 20;  // roundEven((scaled - 1) * 8)
+    if (m == 8u) {
+        m = 0;
+        exponent += 1;
+    }
+    if (exponent > 8) return (uint8_t)(sign | 0x7fu);
+    const uint32_t field = (uint32_t)(exponent + 7);
+    if (field == 0xfu && m == 7u) m = 6u;
+    return (uint8_t)(sign | (field << 3) | m);
+}
+__device__ inline uint8_t encode_f8(int dt, float v) { return dt == MLEL_F8E4M3 ? encode_f8e4m3(v) : encode_f8e5m2(v); }
+
 __device__ inline float raw_ld_f(const char *p, int dt) {
     switch (dt) {
     case MLEL_F16: return __half2float(*(const __half *)p);
     case MLEL_F32: return *(const float *)p;
     case MLEL_F64: return (float)*(const double *)p;
+    case MLEL_BF16: return decode_bf16(*(const uint16_t *)p);
+    case MLEL_F8E4M3: return decode_f8e4m3(*(const uint8_t *)p);
+    case MLEL_F8E5M2: return decode_f8e5m2(*(const uint8_t *)p);
     default: return (float)raw_ld_i(p, dt);
     }
 }
-__device__ inline void raw_st_f(char *p, int dt, float v) {
+// How a computed value becomes storage.  ST_TRUNC is the reference's ENCODE_COMP_TO_STORAGE (bf16 truncates), ST_RNE
+// its ENCODE_COMP_TO_STORAGE_RNE (bf16 rounds to nearest even); both take fp8 through fp16 first (common.comp:618-633).
+// ST_ACC is the convolution family's acc_to_out (common.comp:651-652): bf16 truncates, fp8 encodes the fp32 value.
+enum { ST_TRUNC = 0, ST_RNE = 1, ST_ACC = 2 };
+__device__ inline void raw_st_f(char *p, int dt, float v, int mode = ST_TRUNC) {
     switch (dt) {
-    case MLEL_F16: *(__half *)p = __float2half_rn(v); break;
+    case MLEL_F16: *(__half *)p = f2h(v); break;
     case MLEL_F32: *(float *)p = v; break;
     case MLEL_F64: *(double *)p = (double)v; break;
+    case MLEL_BF16: *(uint16_t *)p = mode == ST_RNE ? encode_bf16_rne(v) : encode_bf16_trunc(v); break;
+    case MLEL_F8E4M3:
+    case MLEL_F8E5M2: *(uint8_t *)p = encode_f8(dt, mode == ST_ACC ? v : __half2float(f2h(v))); break;
     default: break;
     }
 }
@@ -200,13 +276,35 @@ __device__ inline void st_i(const TV &t, const int64_t *idx, int64_t v) {
     if (!elem_off(t, idx, &off)) return;
     raw_st_i(t.ptr + off, t.dtype, v);
 }
-__device__ inline void st_f(const TV &t, const int64_t *idx, float v) {
+__device__ inline void st_f(const TV &t, const int64_t *idx, float v, int mode = ST_TRUNC) {
     int64_t off;
     if (!elem_off(t, idx, &off)) return;
-    raw_st_f(t.ptr + off, t.dtype, v);
+    raw_st_f(t.ptr + off, t.dtype, v, mode);
 }
-__device__ inline float rnd_f16(float v) { return __half2float(__float2half_rn(v)); }
-__device__ inline float round_to(int dt, float v) { return dt == MLEL_F16 ? rnd_f16(v) : v; }
+// Integer accumulators over floating-point storage (the convolution shaders' to_acc / acc_to_out for an integer
+// ACC_TYPE, common.comp:636-660): operands are truncated toward zero, the result is converted back and encoded.
+__device__ inline int64_t ld_acc_i(const TV &t, const int64_t *idx) {
+    return dt_is_float(t.dtype) ? (int64_t)ld_f(t, idx) : ld_i(t, idx);
+}
+__device__ inline void st_acc_i(const TV &t, const int64_t *idx, int64_t v) {
+    if (dt_is_float(t.dtype))
+        st_f(t, idx, (float)v, ST_ACC);
+    else
+        st_i(t, idx, v);
+}
+__device__ inline float rnd_f16(float v) { return __half2float(f2h(v)); }
+// lowest finite value of a floating-point storage type (getFormatInfo's `lowest`, common/utils.cpp:125-131)
+__device__ inline float dt_lowest_f(int dt) {
+    switch (dt) {
+    case MLEL_F16: return -65504.f;
+    case MLEL_BF16: return -3.3895313892515355e+38f;
+    case MLEL_F8E5M2: return -57344.f;
+    case MLEL_F8E4M3: return -448.f;
+    default: return -3.402823466e+38f;
+    }
+}
+// rounding of an intermediate result to the type the arithmetic runs in
+__device__ inline float round_to(int dt, float v) { return dt_comp(dt) == MLEL_F16 ? rnd_f16(v) : v; }
 
 // TANH as the reference computes it (elementwise_unary.comp:136-205): saturated beyond |x| > 10, an odd polynomial
 // below 0.2, the library function in between.

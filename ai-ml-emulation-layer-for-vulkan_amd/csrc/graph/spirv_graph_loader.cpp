@@ -77,6 +77,7 @@ struct Type {
     TypeKind kind = TypeKind::Other;
     int width = 0;              // Int / Float
     bool bfloat = false;        // Float 16 with the BFloat16KHR encoding
+    int fp8 = 0;                // Float 8: 1 = Float8E4M3EXT, 2 = Float8E5M2EXT
     std::string element;        // Array / Tensor / Pointer: element (pointee) type id
     int64_t length = 0;         // Array
     int rank = 0;               // Tensor
@@ -123,6 +124,32 @@ uint16_t floatToHalfBits(const float f) {  // round to nearest even
     const uint32_t rest = mantissa & 0x1fffu;
     if (rest > 0x1000u || (rest == 0x1000u && (half & 1))) half++;
     return static_cast<uint16_t>(sign | half);
+}
+
+// fp8 literals, nearest even like the other widths (values of the formats: graph/shaders/graph_op/common.comp:191-215)
+uint8_t floatToE5M2Bits(const float f) {
+    const uint16_t h = floatToHalfBits(f);
+    if ((h & 0x7c00u) == 0x7c00u) return static_cast<uint8_t>((h >> 8) | ((h & 0x3ffu) ? 0x02u : 0u));  // inf / NaN
+    return static_cast<uint8_t>((h + 0x7fu + ((h >> 8) & 1u)) >> 8);
+}
+uint8_t floatToE4M3Bits(const float f) {
+    const uint8_t sign = std::signbit(f) ? 0x80u : 0u;
+    const float ax = std::fabs(f);
+    if (std::isnan(f) || ax > 464.0f) return sign | 0x7fu;  // no infinities: the NaN code
+    if (ax < 0.015625f) return sign | static_cast<uint8_t>(std::nearbyint(ax * 512.0f));  // multiples of 2^-9 (8 -> 0x08)
+    int e;
+    const float m = std::frexp(ax, &e);  // ax = m * 2^e, m in [0.5, 1)
+    int mant = static_cast<int>(std::nearbyint((m * 2.0f - 1.0f) * 8.0f)), expo = e - 1;
+    if (mant == 8) mant = 0, expo++;
+    const int field = expo + 7;
+    if (field > 15 || (field == 15 && mant == 7)) return sign | 0x7eu;  // rounds to the largest finite value, 448
+    return sign | static_cast<uint8_t>((field << 3) | mant);
+}
+float e4m3BitsToFloat(const uint8_t x) {
+    const int e = (x >> 3) & 0xf, m = x & 7;
+    if (e == 15 && m == 7) return std::nanf("");
+    const float v = e == 0 ? static_cast<float>(m) / 512.0f : std::ldexp(1.0f + static_cast<float>(m) / 8.0f, e - 7);
+    return (x & 0x80u) ? -v : v;
 }
 
 class Module {
@@ -206,6 +233,7 @@ int32_t Module::dtypeOfScalarType(const Instruction &at, const Type &t) const {
         }
         break;
     case TypeKind::Float:
+        if (t.width == 8 && t.fp8 != 0) return t.fp8 == 1 ? MLEL_F8E4M3 : MLEL_F8E5M2;
         if (t.width == 16) return t.bfloat ? MLEL_BF16 : MLEL_F16;
         if (t.width == 32) return MLEL_F32;
         if (t.width == 64) return MLEL_F64;
@@ -236,6 +264,7 @@ uint64_t Module::parseLiteral(const Instruction &at, const Type &t, const std::s
         uint32_t b;
         std::memcpy(&b, &f, 4);
         if (t.width == 32) return b;
+        if (t.width == 8) return t.fp8 == 1 ? floatToE4M3Bits(f) : floatToE5M2Bits(f);
         if (t.bfloat) {  // round to nearest even on the upper 16 bits
             const uint32_t rounded = b + 0x7fffu + ((b >> 16) & 1u);
             return (std::isnan(f) ? (b | 0x400000u) : rounded) >> 16;
@@ -277,7 +306,11 @@ void Module::declare(const Instruction &inst) {
         t.kind = TypeKind::Float;
         t.width = std::atoi(a[0].c_str());
         t.bfloat = a.size() >= 2 && a[1].find("BFloat16") != std::string::npos;
-        if (a.size() >= 2 && !t.bfloat) fail(inst, "floating-point encoding " + a[1] + " is not supported");
+        if (a.size() >= 2 && a[1].find("Float8E4M3") != std::string::npos) t.fp8 = 1;
+        if (a.size() >= 2 && a[1].find("Float8E5M2") != std::string::npos) t.fp8 = 2;
+        if ((a.size() >= 2 && !t.bfloat && t.fp8 == 0) || (t.bfloat && t.width != 16) || ((t.fp8 != 0) != (t.width == 8)))
+            fail(inst, "floating-point type of width " + a[0] + (a.size() >= 2 ? " and encoding " + a[1] : "") +
+                           " is not supported");
         types[inst.result] = t;
     } else if (op == "OpTypeBool") {
         Type t;
@@ -399,9 +432,11 @@ double Module::realFromBits(const Type &t, const uint64_t bits) const {
         return v;
     }
     uint32_t b = static_cast<uint32_t>(bits);
+    if (t.width == 8 && t.fp8 == 1) return e4m3BitsToFloat(static_cast<uint8_t>(bits));
+    if (t.width == 8) b <<= 8;  // e5m2 is the upper byte of a half
     if (t.width == 16 && t.bfloat) {
         b <<= 16;
-    } else if (t.width == 16) {  // half -> float
+    } else if (t.width == 16 || t.width == 8) {  // half -> float
         const uint32_t sign = (b & 0x8000u) << 16, e = (b >> 10) & 0x1f, m = b & 0x3ffu;
         if (e == 0) {
             const float v = std::ldexp(static_cast<float>(m), -24);

@@ -44,7 +44,7 @@ struct Acc {
 __device__ __forceinline__ void conv_mac(uint32_t acc_type, Acc &acc, const TV &in, const int64_t *xi, const TV &w,
                                          const int64_t *wi, int32_t zi, int32_t zw) {
     if (acc_type == MLEL_ACC_I32 || acc_type == MLEL_ACC_I64) {
-        const int64_t v = ld_i(in, xi) - zi, ww = ld_i(w, wi) - zw;
+        const int64_t v = ld_acc_i(in, xi) - zi, ww = ld_acc_i(w, wi) - zw;
         acc.i = acc_type == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)acc.i, wmul32((int32_t)v, (int32_t)ww))
                                          : wadd64(acc.i, wmul64(v, ww));
     } else {
@@ -85,11 +85,11 @@ __global__ void __launch_bounds__(kBlock) conv3d_kernel(TV out, TV in, TV w, TV 
     }
     const int64_t bi[1] = {bias.dims[0] == 1 ? 0 : o[4]};
     if (a.acc == MLEL_ACC_I32 || a.acc == MLEL_ACC_I64) {
-        const int64_t b = ld_i(bias, bi);
-        st_i(out, o, a.acc == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)acc.i, (int32_t)b) : wadd64(acc.i, b));
+        const int64_t b = ld_acc_i(bias, bi);
+        st_acc_i(out, o, a.acc == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)acc.i, (int32_t)b) : wadd64(acc.i, b));
     } else {
         const float b = ld_f(bias, bi);
-        st_f(out, o, a.acc == MLEL_ACC_F16 ? rnd_f16(acc.f + rnd_f16(b)) : acc.f + b);
+        st_f(out, o, a.acc == MLEL_ACC_F16 ? rnd_f16(acc.f + rnd_f16(b)) : acc.f + b, ST_ACC);
     }
 }
 
@@ -109,7 +109,7 @@ __global__ void __launch_bounds__(kBlock) tconv2d_kernel(TV out, TV in, TV w, TV
     const int64_t bi[1] = {bias.dims[0] == 1 ? 0 : o[3]};
     Acc acc{0, 0.f};
     if (integer)
-        acc.i = a.acc == MLEL_ACC_I32 ? (int64_t)(int32_t)ld_i(bias, bi) : ld_i(bias, bi);
+        acc.i = a.acc == MLEL_ACC_I32 ? (int64_t)(int32_t)ld_acc_i(bias, bi) : ld_acc_i(bias, bi);
     else
         acc.f = a.acc == MLEL_ACC_F16 ? rnd_f16(ld_f(bias, bi)) : ld_f(bias, bi);
     for (int64_t ky = 0; ky < w.dims[1]; ky++) {
@@ -127,9 +127,9 @@ __global__ void __launch_bounds__(kBlock) tconv2d_kernel(TV out, TV in, TV w, TV
         }
     }
     if (integer)
-        st_i(out, o, acc.i);
+        st_acc_i(out, o, acc.i);
     else
-        st_f(out, o, acc.f);
+        st_f(out, o, acc.f, ST_ACC);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -145,7 +145,7 @@ __global__ void __launch_bounds__(kBlock) argmax_kernel(TV out, TV in, uint32_t 
     const int64_t len = in.dims[axis];
     int64_t best = 0;
     if (dt_is_float(in.dtype)) {
-        float mx = in.dtype == MLEL_F16 ? -65504.f : -3.402823466e38f;  // lowest finite value of the type
+        float mx = dt_lowest_f(in.dtype);  // lowest finite value of the type
         for (int64_t i = 0; i < len; i++) {
             ii[axis] = i;
             const float v = ld_f(in, ii);

@@ -86,7 +86,7 @@ __device__ __forceinline__ void store8(char *p, const float (&v)[8]) {
         uint4 raw;
         __half2 *h = reinterpret_cast<__half2 *>(&raw);
 #pragma unroll
-        for (int i = 0; i < 4; i++) h[i] = __halves2half2(__float2half_rn(v[2 * i]), __float2half_rn(v[2 * i + 1]));
+        for (int i = 0; i < 4; i++) h[i] = __halves2half2(f2h(v[2 * i]), f2h(v[2 * i + 1]));
         *reinterpret_cast<uint4 *>(p) = raw;
     } else {
         *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
@@ -172,7 +172,7 @@ __global__ void __launch_bounds__(kBlock) ew_chain_kernel(const ChainArgs g) {
             uint4 raw;
             __half2 *h = reinterpret_cast<__half2 *>(&raw);
 #pragma unroll
-            for (int i = 0; i < 4; i++) h[i] = __halves2half2(__float2half_rn(x[2 * i]), __float2half_rn(x[2 * i + 1]));
+            for (int i = 0; i < 4; i++) h[i] = __halves2half2(f2h(x[2 * i]), f2h(x[2 * i + 1]));
             regs[r][0][tid] = raw;
         } else {
             regs[r][0][tid] = make_uint4(__float_as_uint(x[0]), __float_as_uint(x[1]), __float_as_uint(x[2]), __float_as_uint(x[3]));
@@ -468,7 +468,7 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArg
                     // (fp32 carries more than twice the fp16 precision plus two bits, so the second rounding cannot
                     // change the result).
                     if (IS_SUM) {
-                        __half acc = __float2half_rn(r);
+                        __half acc = f2h(r);
 #pragma unroll
                         for (int t = 0; t < 4; t++) {
                             acc = __hadd(acc, __low2half(h[t]));
@@ -512,7 +512,7 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArg
         }
         __syncthreads();
     }
-    if (tid < 64 && row < g.rows) *reinterpret_cast<__half *>(g.out + row * 2) = __float2half_rn(r);
+    if (tid < 64 && row < g.rows) *reinterpret_cast<__half *>(g.out + row * 2) = f2h(r);
 }
 
 }  // namespace

@@ -46,8 +46,8 @@ __global__ void __launch_bounds__(kBlock) conv2d_generic(TV out, TV in, TV w, TV
                 const int64_t xi[4] = {n, yy, xx, ic};
                 const int64_t wi[4] = {oc, ky, kx, ic};
                 if (!facc) {
-                    const int64_t v = ld_i(in, xi) - a.zi;
-                    const int64_t ww = ld_i(w, wi) - a.zw;
+                    const int64_t v = ld_acc_i(in, xi) - a.zi;
+                    const int64_t ww = ld_acc_i(w, wi) - a.zw;
                     if (a.acc == MLEL_ACC_I32)
                         iacc = wadd32((int32_t)iacc, wmul32((int32_t)v, (int32_t)ww));
                     else
@@ -65,11 +65,11 @@ __global__ void __launch_bounds__(kBlock) conv2d_generic(TV out, TV in, TV w, TV
     }
     const int64_t bi[1] = {bias.dims[0] == 1 ? 0 : oc};
     if (!facc) {
-        const int64_t b = ld_i(bias, bi);
-        st_i(out, o, a.acc == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)iacc, (int32_t)b) : wadd64(iacc, b));
+        const int64_t b = ld_acc_i(bias, bi);
+        st_acc_i(out, o, a.acc == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)iacc, (int32_t)b) : wadd64(iacc, b));
     } else {
         const float b = ld_f(bias, bi);
-        st_f(out, o, a.acc == MLEL_ACC_F16 ? rnd_f16(facc_v + rnd_f16(b)) : facc_v + b);
+        st_f(out, o, a.acc == MLEL_ACC_F16 ? rnd_f16(facc_v + rnd_f16(b)) : facc_v + b, ST_ACC);
     }
 }
 
@@ -95,8 +95,8 @@ __global__ void __launch_bounds__(kBlock) dwconv_generic(TV out, TV in, TV w, TV
             const int64_t xi[4] = {n, yy, xx, c};
             const int64_t wi[4] = {ky, kx, c, m};
             if (!facc) {
-                const int64_t v = ld_i(in, xi) - a.zi;
-                const int64_t ww = ld_i(w, wi) - a.zw;
+                const int64_t v = ld_acc_i(in, xi) - a.zi;
+                const int64_t ww = ld_acc_i(w, wi) - a.zw;
                 if (a.acc == MLEL_ACC_I32)
                     iacc = wadd32((int32_t)iacc, wmul32((int32_t)v, (int32_t)ww));
                 else
@@ -109,11 +109,11 @@ __global__ void __launch_bounds__(kBlock) dwconv_generic(TV out, TV in, TV w, TV
     }
     const int64_t bi[1] = {bias.dims[0] == 1 ? 0 : ocm};
     if (!facc) {
-        const int64_t b = ld_i(bias, bi);
-        st_i(out, o, a.acc == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)b, (int32_t)iacc) : wadd64(b, iacc));
+        const int64_t b = ld_acc_i(bias, bi);
+        st_acc_i(out, o, a.acc == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)b, (int32_t)iacc) : wadd64(b, iacc));
     } else {
         const float b = ld_f(bias, bi);
-        st_f(out, o, a.acc == MLEL_ACC_F16 ? rnd_f16(rnd_f16(b) + facc_v) : b + facc_v);
+        st_f(out, o, a.acc == MLEL_ACC_F16 ? rnd_f16(rnd_f16(b) + facc_v) : b + facc_v, ST_ACC);
     }
 }
 
@@ -140,7 +140,7 @@ __global__ void __launch_bounds__(kBlock) matmul_generic(TV out, TV A, TV B, int
                 iacc = wadd64(iacc, wmul64(v1, v2));
         } else {
             const float p = (ld_f(A, ai) - (float)za) * (ld_f(B, bi) - (float)zb);
-            facc = od == MLEL_F16 ? rnd_f16(facc + rnd_f16(p)) : facc + p;
+            facc = dt_comp(od) == MLEL_F16 ? rnd_f16(facc + rnd_f16(p)) : facc + p;
         }
     }
     if (dt_is_int(od))
@@ -249,7 +249,7 @@ __global__ void __launch_bounds__(kBlock) binary_generic(int op, TV out, TV in1,
         if (is_bool)
             st_i(out, o, br);
         else
-            st_f(out, o, r);  // one rounding into the storage type
+            st_f(out, o, r, ST_RNE);  // one rounding into the storage type
     } else {
         const int64_t a = ld_i(in1, i1), b = ld_i(in2, i2);
         int64_t r = 0;
@@ -288,7 +288,7 @@ __global__ void __launch_bounds__(kBlock) mul_generic(TV out, TV in1, TV in2, ui
     broadcast_idx(in1, o, i1);
     broadcast_idx(in2, o, i2);
     if (dt_is_float(in1.dtype)) {
-        st_f(out, o, round_to(out.dtype, ld_f(in1, i1)) * round_to(out.dtype, ld_f(in2, i2)));
+        st_f(out, o, round_to(out.dtype, ld_f(in1, i1)) * round_to(out.dtype, ld_f(in2, i2)), ST_RNE);
     } else {
         int64_t r = wmul64(ld_i(in1, i1), ld_i(in2, i2));
         if (shift > 0) r = wadd64(r, int64_t(1) << (shift - 1)) >> (shift > 63 ? 63 : shift);
@@ -398,7 +398,7 @@ __global__ void __launch_bounds__(kBlock) reduce_generic(int op, TV out, TV in, 
     for (int i = 0; i < MLEL_MAX_RANK; i++) ii[i] = o[i];
     const int dt = in.dtype;
     if (dt_is_float(dt)) {
-        const float lowest = dt == MLEL_F16 ? -65504.f : -3.402823466e+38f;
+        const float lowest = dt_lowest_f(dt);
         float r;
         switch (op) {
         case MLEL_RED_MAX: r = nan_mode == MLEL_NAN_IGNORE ? NAN : lowest; break;
@@ -507,7 +507,7 @@ __global__ void __launch_bounds__(kBlock) maxpool_generic(TV out, TV in, PoolArg
     const int dt = out.dtype;
     const bool isf = dt_is_float(dt);
     int64_t iacc = dt_lowest(dt);
-    float facc = dt == MLEL_F16 ? -65504.f : -3.402823466e+38f;
+    float facc = dt_lowest_f(dt);
     if (isf && a.nan_mode == MLEL_NAN_IGNORE) facc = NAN;
     bool done = false;
     for (int64_t ky = 0; ky < a.kh && !done; ky++) {
@@ -569,8 +569,10 @@ __global__ void __launch_bounds__(kBlock) cast_generic(TV out, TV in, int64_t to
     if (odt == MLEL_BOOL) {
         st_i(out, o, dt_is_float(idt) ? (ld_f(in, o) != 0.f) : (ld_i(in, o) != 0));
     } else if (dt_is_float(odt)) {
+        // to bf16: round to nearest even; to fp8: the fp32 value is encoded directly (cast.comp:36-56)
+        const int mode = odt == MLEL_BF16 ? ST_RNE : ST_ACC;
         if (dt_is_float(idt)) {
-            st_f(out, o, ld_f(in, o));
+            st_f(out, o, ld_f(in, o), mode);
         } else {
             const int64_t v = ld_i(in, o);
             if (odt == MLEL_F16 && idt != MLEL_BOOL && idt != MLEL_I8 && idt != MLEL_U8 && idt != MLEL_I16) {
@@ -578,7 +580,7 @@ __global__ void __launch_bounds__(kBlock) cast_generic(TV out, TV in, int64_t to
                 else if (v < -65504) st_f(out, o, -INFINITY);
                 else st_f(out, o, (float)v);
             } else {
-                st_f(out, o, (float)v);
+                st_f(out, o, (float)v, mode);
             }
         }
     } else {

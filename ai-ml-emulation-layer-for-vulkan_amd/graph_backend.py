@@ -136,7 +136,7 @@ class Graph:
     def const(self, name, array, dtype=None):
         array = np.ascontiguousarray(array)
         if dtype is None:
-            dtype = abi.dtype_of_numpy(array.dtype)
+            dtype = abi.dtype_of_array(array)
         dims = array.shape if array.ndim else (1,)
         h = self._check(self.lib.mlel_graph_make_const_tensor(self.g, self.next_const, int(dtype), len(dims),
                                                               _i64(dims), None, array.ctypes.data))

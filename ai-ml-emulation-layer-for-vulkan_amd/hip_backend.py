@@ -147,9 +147,9 @@ class Device:
         return DeviceTensor(self, dtype, shape, strides, data)
 
     def from_numpy(self, arr, dtype=None, strides=None):
-        arr = np.asarray(arr)
+        arr = np.asanyarray(arr)  # (a tagged bf16 / fp8 array keeps its tag)
         if dtype is None:
-            dtype = abi.dtype_of_numpy(arr.dtype)
+            dtype = abi.dtype_of_array(arr)
         return DeviceTensor(self, dtype, arr.shape, strides, arr)
 
     # ---- operators (asynchronous on self.stream; download() synchronises)

@@ -52,7 +52,22 @@ static int dt_size(int dt) {
     }
 }
 static int dt_is_int(int dt) { return dt >= MLEL_BOOL && dt <= MLEL_U64; }
-static int dt_is_float(int dt) { return dt == MLEL_F16 || dt == MLEL_F32 || dt == MLEL_F64 || dt == MLEL_BF16; }
+static int dt_is_float(int dt) {
+    return dt == MLEL_F16 || dt == MLEL_F32 || dt == MLEL_F64 || dt == MLEL_BF16 || dt == MLEL_F8E4M3 || dt == MLEL_F8E5M2;
+}
+static int dt_is_fp8(int dt) { return dt == MLEL_F8E4M3 || dt == MLEL_F8E5M2; }
+/* the type arithmetic runs in: fp8 -> fp16, bf16 -> fp32 (getFormatInfo compType, common/utils.cpp:125-131) */
+static int dt_comp(int dt) { return dt_is_fp8(dt) ? MLEL_F16 : (dt == MLEL_BF16 ? MLEL_F32 : dt); }
+static double dt_lowest_f(int dt) { /* getFormatInfo `lowest`, common/utils.cpp:119-131 */
+    switch (dt) {
+    case MLEL_F16: return -65504.0;
+    case MLEL_BF16: return -3.3895313892515355e+38;
+    case MLEL_F8E5M2: return -57344.0;
+    case MLEL_F8E4M3: return -448.0;
+    case MLEL_F32: return -(double)3.402823466e+38F;
+    default: return -1.7976931348623157e308;
+    }
+}
 static int64_t dt_lowest(int dt) {
     switch (dt) {
     case MLEL_I8: return -128;
@@ -217,21 +232,99 @@ static inline void raw_st_i(void *p, int dt, int64_t v) {
     default: break;
     }
 }
+/* ---- reduced-precision storage formats, written after graph/shaders/graph_op/common.comp ----
+ * decode: bf16 :185-189, e5m2 :191-195, e4m3 :197-215; encode: bf16 truncation :300-305, bf16 nearest-even :403-418,
+ * e5m2 :312-327, e4m3 :329-371.  The e4m3 encoder keeps the shader's floating-point formulation (floor(log2), exp2,
+ * roundEven) in double precision, where every step is exact for fp32 inputs. */
+static double f8e5m2_to_f64(uint8_t x) { return (double)mlel_cpu_f16_to_f32((uint16_t)((uint32_t)x << 8)); }
+static double f8e4m3_to_f64(uint8_t x) {
+    const unsigned sign = (x >> 7) & 1u, exponent = (x >> 3) & 0xFu, mantissa = x & 7u;
+    if (exponent == 0xFu && mantissa == 7u) return NAN;
+    double value;
+    if (exponent == 0u)
+        value = mantissa == 0u ? 0.0 : (double)mantissa / 512.0;
+    else
+        value = exp2((double)((int)exponent - 7)) * (1.0 + (double)mantissa / 8.0);
+    return sign ? -value : value;
+}
+static uint32_t f32_bits(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+static uint16_t f32_to_bf16_trunc(float x) { return (uint16_t)(f32_bits(x) >> 16); }
+static uint16_t f32_to_bf16_rne(float x) {
+    uint32_t u = f32_bits(x);
+    const uint32_t exp = u & 0x7F800000u, mantissa = u & 0x007FFFFFu;
+    if (exp == 0x7F800000u) return mantissa != 0u ? (uint16_t)((u >> 16) | 0x0040u) : (uint16_t)(u >> 16);
+    const uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7FFFu + lsb;
+    return (uint16_t)(u >> 16);
+}
+static uint8_t f32_to_f8e5m2(float x) {
+    const uint32_t sign = (f32_bits(x) >> 24) & 0x80u;
+    if (isnan(x)) return (uint8_t)(sign | 0x7Du);
+    if (isinf(x) || x > 57344.0f || x < -57344.0f) return (uint8_t)(sign | 0x7Cu);
+    return (uint8_t)(mlel_cpu_f32_to_f16(x) >> 8); /* packHalf2x16 (nearest even), upper byte */
+}
+static double round_even(double v) { return nearbyint(v); } /* default rounding mode: ties to even */
+static double clampd(double v, double lo, double hi) { return v < lo ? lo : (v > hi ? hi : v); }
+static uint8_t f32_to_f8e4m3(float x) {
+    const uint32_t sign = (f32_bits(x) >> 24) & 0x80u;
+    const double ax = fabs((double)x);
+    if (isnan(x) || isinf(x) || ax > 448.0) return (uint8_t)(sign | 0x7Fu);
+    if (ax == 0.0) return (uint8_t)sign;
+    if (ax < exp2(-6.0)) {
+        const unsigned mantissa = (unsigned)clampd(round_even(ax * 512.0), 0.0, 8.0);
+        if (mantissa == 0u) return (uint8_t)sign;
+        if (mantissa >= 8u) return (uint8_t)(sign | 0x08u);
+        return (uint8_t)(sign | mantissa);
+    }
+    int exponent = (int)floor(log2(ax));
+    if (exp2((double)exponent) > ax) exponent--; /* guard the library's log2 at exact powers of two */
+    if (exp2((double)(exponent + 1)) <= ax) exponent++;
+    const double scaled = ax * exp2((double)-exponent);
+    unsigned mantissa = (unsigned)clampd(round_even((scaled - 1.0) * 8.0), 0.0, 8.0);
+    if (mantissa == 8u) {
+        mantissa = 0u;
+        exponent += 1;
+    }
+    if (exponent > 8) return (uint8_t)(sign | 0x7Fu);
+    const unsigned field = (unsigned)(exponent + 7);
+    if (field == 0xFu && mantissa == 0x7u) mantissa = 0x6u;
+    return (uint8_t)(sign | (field << 3) | mantissa);
+}
+uint16_t mlel_cpu_f32_to_bf16(float x, int nearest_even) { return nearest_even ? f32_to_bf16_rne(x) : f32_to_bf16_trunc(x); }
+uint8_t mlel_cpu_f32_to_f8(float x, int dtype) { return dtype == MLEL_F8E4M3 ? f32_to_f8e4m3(x) : f32_to_f8e5m2(x); }
+float mlel_cpu_f8_to_f32(uint8_t x, int dtype) { return (float)(dtype == MLEL_F8E4M3 ? f8e4m3_to_f64(x) : f8e5m2_to_f64(x)); }
+
 static inline double raw_ld_f(const void *p, int dt) {
     switch (dt) {
     case MLEL_F16: return (double)mlel_cpu_f16_to_f32(*(const uint16_t *)p);
     case MLEL_BF16: return (double)bf16_to_f32(*(const uint16_t *)p);
+    case MLEL_F8E4M3: return f8e4m3_to_f64(*(const uint8_t *)p);
+    case MLEL_F8E5M2: return f8e5m2_to_f64(*(const uint8_t *)p);
     case MLEL_F32: return (double)*(const float *)p;
     case MLEL_F64: return *(const double *)p;
     default: return (double)raw_ld_i(p, dt);
     }
 }
-/* store a value that is already representable / to be rounded once into dt */
-static inline void raw_st_f(void *p, int dt, double v) {
+/* How a computed value becomes storage (common.comp:611-633, 651-652).  ST_TRUNC = ENCODE_COMP_TO_STORAGE: bf16
+ * truncates; ST_RNE = ENCODE_COMP_TO_STORAGE_RNE: bf16 rounds to nearest even; both send fp8 through fp16 first.
+ * ST_ACC = the convolution family's acc_to_out and CAST to fp8: bf16 truncates, fp8 encodes the fp32 value itself. */
+enum { ST_TRUNC = 0, ST_RNE = 1, ST_ACC = 2 };
+static inline void raw_st_f_mode(void *p, int dt, double v, int mode) {
     switch (dt) {
     case MLEL_F16: *(uint16_t *)p = f64_to_f16(v); break;
     case MLEL_F32: *(float *)p = (float)v; break;
     case MLEL_F64: *(double *)p = v; break;
+    case MLEL_BF16: *(uint16_t *)p = mode == ST_RNE ? f32_to_bf16_rne((float)v) : f32_to_bf16_trunc((float)v); break;
+    case MLEL_F8E4M3:
+    case MLEL_F8E5M2: {
+        const float f = mode == ST_ACC ? (float)v : mlel_cpu_f16_to_f32(f64_to_f16(v));
+        *(uint8_t *)p = dt == MLEL_F8E4M3 ? f32_to_f8e4m3(f) : f32_to_f8e5m2(f);
+        break;
+    }
     default: break;
     }
 }
@@ -251,10 +344,23 @@ static inline void st_i(const mlel_tensor *t, const int64_t *idx, int64_t v) {
     if (!elem_off(t, idx, &off)) return;
     raw_st_i((char *)t->ptr + off, t->dtype, v);
 }
-static inline void st_f(const mlel_tensor *t, const int64_t *idx, double v) {
+static inline void st_f_mode(const mlel_tensor *t, const int64_t *idx, double v, int mode) {
     int64_t off;
     if (!elem_off(t, idx, &off)) return;
-    raw_st_f((char *)t->ptr + off, t->dtype, v);
+    raw_st_f_mode((char *)t->ptr + off, t->dtype, v, mode);
+}
+static inline void st_f(const mlel_tensor *t, const int64_t *idx, double v) { st_f_mode(t, idx, v, ST_TRUNC); }
+
+/* Integer accumulators over floating-point storage (the convolution shaders' to_acc / acc_to_out with an integer
+ * ACC_TYPE, common.comp:636-660): operands are truncated toward zero, the result is converted back and encoded. */
+static inline int64_t ld_acc_i(const mlel_tensor *t, const int64_t *idx) {
+    return dt_is_float(t->dtype) ? (int64_t)(float)ld_f(t, idx) : ld_i(t, idx);
+}
+static inline void st_acc_i(const mlel_tensor *t, const int64_t *idx, int64_t v) {
+    if (dt_is_float(t->dtype))
+        st_f_mode(t, idx, (double)(float)v, ST_ACC);
+    else
+        st_i(t, idx, v);
 }
 
 /* flat invocation index -> row-major multi-index over `t`'s dims (reference: common.comp:74-128) */
@@ -371,8 +477,8 @@ int mlel_cpu_conv2d(const mlel_tensor *out, const mlel_tensor *in, const mlel_te
                     const int64_t xi[4] = {n, yy, xx, ic};
                     const int64_t wi[4] = {oc, ky, kx, ic};
                     if (!facc) {
-                        const int64_t v = ld_i(in, xi) - a->input_zp;
-                        const int64_t ww = ld_i(w, wi) - a->weight_zp;
+                        const int64_t v = ld_acc_i(in, xi) - a->input_zp;
+                        const int64_t ww = ld_acc_i(w, wi) - a->weight_zp;
                         if (a->acc_type == MLEL_ACC_I32)
                             iacc = wadd32((int32_t)iacc, wmul32((int32_t)v, (int32_t)ww));
                         else
@@ -396,19 +502,19 @@ int mlel_cpu_conv2d(const mlel_tensor *out, const mlel_tensor *in, const mlel_te
         }
         const int64_t bi[1] = {bias->dims[0] == 1 ? 0 : oc};
         if (!facc) {
-            const int64_t b = ld_i(bias, bi);
+            const int64_t b = ld_acc_i(bias, bi);
             if (a->acc_type == MLEL_ACC_I32)
                 iacc = wadd32((int32_t)iacc, (int32_t)b);
             else
                 iacc = wadd64(iacc, b);
-            st_i(out, o, iacc);
+            st_acc_i(out, o, iacc);
         } else {
             double b = ld_f(bias, bi);
             if (a->acc_type == MLEL_ACC_F16)
                 dacc = rnd_f16(dacc + rnd_f16(b));
             else
                 dacc = rnd_f32(dacc + b);
-            st_f(out, o, dacc);
+            st_f_mode(out, o, dacc, ST_ACC);
         }
     }
     return 0;
@@ -447,8 +553,8 @@ int mlel_cpu_depthwise_conv2d(const mlel_tensor *out, const mlel_tensor *in, con
                 const int64_t xi[4] = {n, yy, xx, c};
                 const int64_t wi[4] = {ky, kx, c, m};
                 if (!facc) {
-                    const int64_t v = ld_i(in, xi) - a->input_zp;
-                    const int64_t ww = ld_i(w, wi) - a->weight_zp;
+                    const int64_t v = ld_acc_i(in, xi) - a->input_zp;
+                    const int64_t ww = ld_acc_i(w, wi) - a->weight_zp;
                     if (a->acc_type == MLEL_ACC_I32)
                         iacc = wadd32((int32_t)iacc, wmul32((int32_t)v, (int32_t)ww));
                     else
@@ -466,12 +572,12 @@ int mlel_cpu_depthwise_conv2d(const mlel_tensor *out, const mlel_tensor *in, con
         }
         const int64_t bi[1] = {bias->dims[0] == 1 ? 0 : ocm};
         if (!facc) {
-            const int64_t b = ld_i(bias, bi);
-            st_i(out, o, a->acc_type == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)b, (int32_t)iacc) : wadd64(b, iacc));
+            const int64_t b = ld_acc_i(bias, bi);
+            st_acc_i(out, o, a->acc_type == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)b, (int32_t)iacc) : wadd64(b, iacc));
         } else if (a->acc_type == MLEL_ACC_F16) {
-            st_f(out, o, rnd_f16(rnd_f16(ld_f(bias, bi)) + dacc));
+            st_f_mode(out, o, rnd_f16(rnd_f16(ld_f(bias, bi)) + dacc), ST_ACC);
         } else {
-            st_f(out, o, rnd_f32(ld_f(bias, bi) + dacc));
+            st_f_mode(out, o, rnd_f32(ld_f(bias, bi) + dacc), ST_ACC);
         }
     }
     return 0;
@@ -525,7 +631,7 @@ int mlel_cpu_matmul(const mlel_tensor *out, const mlel_tensor *A, const mlel_ten
                     iacc = wadd32((int32_t)iacc, wmul32((int32_t)v1, (int32_t)v2));
                 else
                     iacc = wadd64(iacc, wmul64(v1, v2));
-            } else if (od == MLEL_F16) {
+            } else if (dt_comp(od) == MLEL_F16) {
                 double v1 = rnd_f16(ld_f(A, ai) - rnd_f16((double)at->a_zp));
                 double v2 = rnd_f16(ld_f(B, bi) - rnd_f16((double)at->b_zp));
                 dacc = rnd_f16(dacc + rnd_f16(v1 * v2));
@@ -627,10 +733,10 @@ int mlel_cpu_clamp(const mlel_tensor *out, const mlel_tensor *in, const mlel_cla
             st_i(out, o, v);
         } else {
             double mn = a->min_val, mx = a->max_val, v = ld_f(in, o);
-            if (dt == MLEL_F16) {
+            if (dt_comp(dt) == MLEL_F16) {
                 mn = rnd_f16(mn);
                 mx = rnd_f16(mx);
-            } else if (dt == MLEL_F32) {
+            } else if (dt_comp(dt) == MLEL_F32) {
                 mn = rnd_f32(mn);
                 mx = rnd_f32(mx);
             }
@@ -653,6 +759,7 @@ static inline void broadcast_idx(const mlel_tensor *t, const int64_t *o, int64_t
 }
 
 static double round_to(int dt, double v) {
+    dt = dt_comp(dt);
     if (dt == MLEL_F16) return rnd_f16(v);
     if (dt == MLEL_F32) return rnd_f32(v);
     return v;
@@ -711,7 +818,7 @@ int mlel_cpu_elementwise_binary(int32_t op, const mlel_tensor *out, const mlel_t
             if (is_bool)
                 st_i(out, o, br);
             else
-                st_f(out, o, r);
+                st_f_mode(out, o, r, ST_RNE);
         } else {
             const int64_t a = ld_i(in1, i1), b = ld_i(in2, i2);
             int64_t r = 0;
@@ -763,7 +870,7 @@ int mlel_cpu_mul(const mlel_tensor *out, const mlel_tensor *in1, const mlel_tens
         broadcast_idx(in1, o, i1);
         broadcast_idx(in2, o, i2);
         if (isf) {
-            st_f(out, o, round_to(out->dtype, round_to(out->dtype, ld_f(in1, i1)) * round_to(out->dtype, ld_f(in2, i2))));
+            st_f_mode(out, o, round_to(out->dtype, round_to(out->dtype, ld_f(in1, i1)) * round_to(out->dtype, ld_f(in2, i2))), ST_RNE);
         } else {
             int64_t r = wmul64(ld_i(in1, i1), ld_i(in2, i2));
             if (shift > 0) r = asr64(wadd64(r, (int64_t)1 << (shift - 1)), (int)shift);
@@ -913,7 +1020,7 @@ int mlel_cpu_reduce(int32_t op, const mlel_tensor *out, const mlel_tensor *in, u
         unflatten(out, flat, o);
         memcpy(ii, o, sizeof(ii));
         if (isf) {
-            double lowest = dt == MLEL_F16 ? -65504.0 : (dt == MLEL_F32 ? -(double)3.402823466e+38F : -1.7976931348623157e308);
+            double lowest = dt_lowest_f(dt);
             double r;
             switch (op) {
             case MLEL_RED_MAX: r = nan_mode == MLEL_NAN_IGNORE ? NAN : lowest; break;
@@ -1043,7 +1150,7 @@ int mlel_cpu_max_pool2d(const mlel_tensor *out, const mlel_tensor *in, const mle
         int64_t o[4];
         unflatten(out, flat, o);
         int64_t iacc = dt_lowest(dt);
-        double dacc = dt == MLEL_F16 ? -65504.0 : -(double)3.402823466e+38F;
+        double dacc = dt_lowest_f(dt);
         if (isf && a->nan_mode == MLEL_NAN_IGNORE) dacc = NAN; /* reference: compute_graph_op.cpp:1490 */
         int done = 0;
         for (int64_t ky = 0; ky < kh && !done; ky++) {
@@ -1122,8 +1229,10 @@ int mlel_cpu_cast(const mlel_tensor *out, const mlel_tensor *in) {
         if (odt == MLEL_BOOL) {
             st_i(out, o, dt_is_float(idt) ? (ld_f(in, o) != 0.0) : (ld_i(in, o) != 0));
         } else if (dt_is_float(odt)) {
+            /* to bf16: nearest even (cast.comp:36-46); to fp8: the fp32 value is encoded directly (:47-56) */
+            const int mode = odt == MLEL_BF16 ? ST_RNE : ST_ACC;
             if (dt_is_float(idt)) {
-                st_f(out, o, ld_f(in, o));
+                st_f_mode(out, o, ld_f(in, o), mode);
             } else {
                 const int64_t v = ld_i(in, o);
                 /* a wide integer going to a narrower float range saturates to +/-Inf */
@@ -1132,7 +1241,7 @@ int mlel_cpu_cast(const mlel_tensor *out, const mlel_tensor *in) {
                     else if (v < -65504) st_f(out, o, -INFINITY);
                     else st_f(out, o, (double)v);
                 } else {
-                    st_f(out, o, (double)v);
+                    st_f_mode(out, o, (double)v, mode);
                 }
             }
         } else {
@@ -1296,8 +1405,8 @@ int mlel_cpu_pad(const mlel_tensor *out, const mlel_tensor *in, const mlel_tenso
 static inline void conv_mac(uint32_t acc_type, int64_t *iacc, double *dacc, const mlel_tensor *in, const int64_t *xi,
                             const mlel_tensor *w, const int64_t *wi, int32_t zi, int32_t zw) {
     if (!acc_is_float(acc_type)) {
-        const int64_t v = ld_i(in, xi) - zi;
-        const int64_t ww = ld_i(w, wi) - zw;
+        const int64_t v = ld_acc_i(in, xi) - zi;
+        const int64_t ww = ld_acc_i(w, wi) - zw;
         if (acc_type == MLEL_ACC_I32)
             *iacc = wadd32((int32_t)*iacc, wmul32((int32_t)v, (int32_t)ww));
         else
@@ -1317,11 +1426,11 @@ static inline void conv_finish(uint32_t acc_type, int64_t iacc, double dacc, con
                                const mlel_tensor *out, const int64_t *o) {
     const int64_t bi[1] = {bias->dims[0] == 1 ? 0 : oc};
     if (!acc_is_float(acc_type)) {
-        const int64_t b = ld_i(bias, bi);
-        st_i(out, o, acc_type == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)iacc, (int32_t)b) : wadd64(iacc, b));
+        const int64_t b = ld_acc_i(bias, bi);
+        st_acc_i(out, o, acc_type == MLEL_ACC_I32 ? (int64_t)wadd32((int32_t)iacc, (int32_t)b) : wadd64(iacc, b));
     } else {
         const double b = ld_f(bias, bi);
-        st_f(out, o, acc_type == MLEL_ACC_F16 ? rnd_f16(dacc + rnd_f16(b)) : rnd_f32(dacc + b));
+        st_f_mode(out, o, acc_type == MLEL_ACC_F16 ? rnd_f16(dacc + rnd_f16(b)) : rnd_f32(dacc + b), ST_ACC);
     }
 }
 
@@ -1390,7 +1499,7 @@ int mlel_cpu_transpose_conv2d(const mlel_tensor *out, const mlel_tensor *in, con
         int64_t o[MLEL_MAX_RANK];
         unflatten(out, flat, o);
         const int64_t bi[1] = {bias->dims[0] == 1 ? 0 : o[3]};
-        int64_t iacc = facc ? 0 : ld_i(bias, bi);
+        int64_t iacc = facc ? 0 : ld_acc_i(bias, bi);
         if (!facc && a->acc_type == MLEL_ACC_I32) iacc = (int32_t)iacc;
         double dacc = facc ? ld_f(bias, bi) : 0.0;
         if (a->acc_type == MLEL_ACC_F16) dacc = rnd_f16(dacc);
@@ -1409,9 +1518,9 @@ int mlel_cpu_transpose_conv2d(const mlel_tensor *out, const mlel_tensor *in, con
             }
         }
         if (!facc)
-            st_i(out, o, iacc);
+            st_acc_i(out, o, iacc);
         else
-            st_f(out, o, dacc);
+            st_f_mode(out, o, dacc, ST_ACC);
     }
     return 0;
 }
@@ -1435,7 +1544,7 @@ int mlel_cpu_argmax(const mlel_tensor *out, const mlel_tensor *in, uint32_t axis
         int64_t best = 0;
         if (isf) {
             /* the shader starts from the lowest FINITE value of the type, so a -inf input never wins */
-            double mx = in->dtype == MLEL_F16 ? -65504.0 : (in->dtype == MLEL_BF16 ? -3.3895313892515355e38 : -3.4028234663852886e38);
+            double mx = dt_lowest_f(in->dtype);
             for (int64_t i = 0; i < len; i++) {
                 ii[axis] = i;
                 const double v = ld_f(in, ii);

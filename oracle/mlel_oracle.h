@@ -91,6 +91,11 @@ int mlel_cpu_select(const mlel_tensor *out, const mlel_tensor *condition, const 
 /* IEEE binary16 <-> binary32 helpers (round to nearest even), exported for the tests. */
 uint16_t mlel_cpu_f32_to_f16(float f);
 float mlel_cpu_f16_to_f32(uint16_t h);
+/* bf16 / fp8 storage codecs as the shaders define them (graph/shaders/graph_op/common.comp:184-232, 300-418);
+ * `dtype` is MLEL_F8E4M3 or MLEL_F8E5M2 */
+uint16_t mlel_cpu_f32_to_bf16(float x, int nearest_even);
+uint8_t mlel_cpu_f32_to_f8(float x, int dtype);
+float mlel_cpu_f8_to_f32(uint8_t x, int dtype);
 
 #ifdef __cplusplus
 }

@@ -38,7 +38,7 @@ class OracleError(RuntimeError):
 def _view(arr, dtype=None):
     """mlel_tensor over a numpy array's own memory (honours its strides)."""
     if dtype is None:
-        dtype = abi.dtype_of_numpy(arr.dtype)
+        dtype = abi.dtype_of_array(arr)
     if arr.ndim == 0:
         arr = arr.reshape(1)
     return abi.make_tensor(arr.ctypes.data, dtype, arr.shape, arr.strides)
@@ -51,7 +51,13 @@ def _call(name, *args):
 
 
 def _out(shape, dtype):
-    return np.zeros(shape, dtype=abi.NP_OF[dtype])
+    out = np.zeros(shape, dtype=abi.NP_OF[dtype])
+    return abi.typed(out, dtype) if dtype in abi.TAGGED else out
+
+
+def _like(x, shape):
+    """zero-filled array of `shape` with the element type of `x` (keeps a bf16 / fp8 tag)"""
+    return _out(shape, abi.dtype_of_array(x))
 
 
 def conv2d(x, w, bias, out_shape, out_dtype, attr, x_dtype=None, w_dtype=None):
@@ -105,19 +111,19 @@ def elementwise_unary(op, x):
 def reduce(op, x, axis, nan_mode=abi.NAN_PROPAGATE):
     shape = list(x.shape)
     shape[axis] = 1
-    out = np.zeros(shape, dtype=x.dtype)
+    out = _like(x, shape)
     _call("reduce", abi.RED[op], _view(out), _view(x), int(axis), int(nan_mode))
     return out
 
 
 def avg_pool2d(x, out_shape, attr):
-    out = np.zeros(out_shape, dtype=x.dtype)
+    out = _like(x, out_shape)
     _call("avg_pool2d", _view(out), _view(x), attr)
     return out
 
 
 def max_pool2d(x, out_shape, attr):
-    out = np.zeros(out_shape, dtype=x.dtype)
+    out = _like(x, out_shape)
     _call("max_pool2d", _view(out), _view(x), attr)
     return out
 
@@ -141,7 +147,7 @@ def negate(x, input_zp=0, output_zp=0):
 
 
 def reshape(x, out_shape):
-    out = np.zeros(out_shape, dtype=x.dtype)
+    out = _like(x, out_shape)
     _call("reshape", _view(out), _view(x))
     return out
 
@@ -151,7 +157,7 @@ def transpose(x, perms):
     # output dim i has the extent of input dim perms[i] (reference: transpose.comp:23-26)
     for i, p in enumerate(perms):
         out_shape[i] = x.shape[p]
-    out = np.zeros(out_shape, dtype=x.dtype)
+    out = _like(x, out_shape)
     arr = (C.c_uint32 * abi.MAX_RANK)(*[int(p) for p in perms])
     _call("transpose", _view(out), _view(x), arr)
     return out
@@ -160,7 +166,7 @@ def transpose(x, perms):
 def concat(inputs, axis):
     shape = list(inputs[0].shape)
     shape[axis] = sum(i.shape[axis] for i in inputs)
-    out = np.zeros(shape, dtype=inputs[0].dtype)
+    out = _like(inputs[0], shape)
     offset = 0
     for i in inputs:
         _call("concat", _view(out), _view(i), int(axis), int(offset))
@@ -169,14 +175,14 @@ def concat(inputs, axis):
 
 
 def slice_(x, start, size):
-    out = np.zeros(size, dtype=x.dtype)
+    out = _like(x, size)
     arr = (C.c_uint32 * abi.MAX_RANK)(*[int(p) for p in start])
     _call("slice", _view(out), _view(x), arr)
     return out
 
 
 def pad(x, padding, out_shape, pad_const=0.0, pad_const_int=0):
-    out = np.zeros(out_shape, dtype=x.dtype)
+    out = _like(x, out_shape)
     padding = np.ascontiguousarray(padding, dtype=np.int32).reshape(-1)
     _call("pad", _view(out), _view(x), _view(padding), float(pad_const), int(pad_const_int))
     return out
@@ -190,7 +196,7 @@ def argmax(x, axis, nan_mode=abi.NAN_PROPAGATE):
 
 
 def arithmetic_right_shift(a, b, out_shape, round_=False):
-    out = np.zeros(out_shape, dtype=a.dtype)
+    out = _like(a, out_shape)
     _call("arithmetic_right_shift", _view(out), _view(a), _view(b), 1 if round_ else 0)
     return out
 
@@ -221,7 +227,7 @@ def rfft2d(x):
 
 
 def gather(values, indices):
-    out = np.zeros((values.shape[0], indices.shape[1], values.shape[2]), dtype=values.dtype)
+    out = _like(values, (values.shape[0], indices.shape[1], values.shape[2]))
     _call("gather", _view(out), _view(values), _view(indices))
     return out
 
@@ -245,13 +251,13 @@ def reverse(x, axis):
 
 
 def tile(x, out_shape):
-    out = np.zeros(out_shape, dtype=x.dtype)
+    out = _like(x, out_shape)
     _call("tile", _view(out), _view(x))
     return out
 
 
 def select(cond, a, b, out_shape):
-    out = np.zeros(out_shape, dtype=a.dtype)
+    out = _like(a, out_shape)
     _call("select", _view(out), _view(cond, abi.BOOL), _view(a), _view(b))
     return out
 

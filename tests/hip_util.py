@@ -23,7 +23,7 @@ class Runner:
         self.live = []
 
     def put(self, arr, dtype=None, strides=None):
-        t = self.dev.from_numpy(np.asarray(arr), dtype, strides)
+        t = self.dev.from_numpy(np.asanyarray(arr), dtype, strides)
         self.live.append(t)
         return t
 
@@ -170,7 +170,7 @@ class Runner:
     def concat(self, inputs, axis):
         shape = list(inputs[0].shape)
         shape[axis] = sum(i.shape[axis] for i in inputs)
-        to = self.new(abi.dtype_of_numpy(inputs[0].dtype), shape)
+        to = self.new(abi.dtype_of_array(inputs[0]), shape)
         off = 0
         for i in inputs:
             ti = self.put(i)
@@ -258,7 +258,7 @@ class Runner:
         return self.call("argmax", [(abi.I32, shape)], [x], int(axis), int(nan_mode))
 
     def arithmetic_right_shift(self, a, b, out_shape, round_=False):
-        return self.call("arithmetic_right_shift", [(abi.dtype_of_numpy(a.dtype), out_shape)], [a, b], 1 if round_ else 0)
+        return self.call("arithmetic_right_shift", [(abi.dtype_of_array(a), out_shape)], [a, b], 1 if round_ else 0)
 
     def conv3d(self, x, w, b, out_shape, out_dtype, attr):
         return self.call("conv3d", [(out_dtype, out_shape)], [x, w, b], C.byref(attr))
@@ -275,19 +275,19 @@ class Runner:
 
     def gather(self, values, indices):
         shape = (values.shape[0], indices.shape[1], values.shape[2])
-        return self.call("gather", [(abi.dtype_of_numpy(values.dtype), shape)], [values, indices])
+        return self.call("gather", [(abi.dtype_of_array(values), shape)], [values, indices])
 
     def scatter(self, values_in, indices, input_):
-        return self.call("scatter", [(abi.dtype_of_numpy(values_in.dtype), values_in.shape)], [values_in, indices, input_])
+        return self.call("scatter", [(abi.dtype_of_array(values_in), values_in.shape)], [values_in, indices, input_])
 
     def resize(self, x, out_shape, out_dtype, attr):
         return self.call("resize", [(out_dtype, out_shape)], [x], C.byref(attr))
 
     def reverse(self, x, axis):
-        return self.call("reverse", [(abi.dtype_of_numpy(x.dtype), x.shape)], [x], int(axis))
+        return self.call("reverse", [(abi.dtype_of_array(x), x.shape)], [x], int(axis))
 
     def tile(self, x, out_shape):
-        return self.call("tile", [(abi.dtype_of_numpy(x.dtype), out_shape)], [x])
+        return self.call("tile", [(abi.dtype_of_array(x), out_shape)], [x])
 
     def select(self, cond, a, b, out_shape):
-        return self.call("select", [(abi.dtype_of_numpy(a.dtype), out_shape)], [cond, a, b])
+        return self.call("select", [(abi.dtype_of_array(a), out_shape)], [cond, a, b])

@@ -45,6 +45,10 @@ class SpvAsm:
             return self._declare(("type", bits, "int"), f"%uint{bits}", f"OpTypeInt {bits} 0")
         if dtype == abi.BF16:
             return self._declare(("type", dtype), "%bfloat16", "OpTypeFloat 16 BFloat16KHR")
+        if dtype == abi.F8E4M3:
+            return self._declare(("type", dtype), "%float8e4m3", "OpTypeFloat 8 Float8E4M3EXT")
+        if dtype == abi.F8E5M2:
+            return self._declare(("type", dtype), "%float8e5m2", "OpTypeFloat 8 Float8E5M2EXT")
         bits = _FLOAT_BITS[dtype]
         return self._declare(("type", bits, "float"), f"%float{bits}", f"OpTypeFloat {bits}")
 

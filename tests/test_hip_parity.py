@@ -718,3 +718,19 @@ def test_conv2d_rescale_add_rescale_equals_the_operator_sequence(run, oracle, ca
         out = run.conv2d_rescale_add_rescale(x, w, b, attr, (mult, shift, rattr, (-90, 90)), (m1, s1, a_conv, None), res,
                                              (m2, s2, a_res, None), (mo, so, a_out, None), residual_first=first)
         np.testing.assert_array_equal(out, exp)
+
+
+def test_fp16_products_keep_the_sign_of_zero(run, oracle):
+    """(-0) * x is -0, also where the product underflows: a multiplication folded into a fused multiply-add with a +0
+    addend would give +0."""
+    a = np.array([[-0.0, 1.0, -6e-8, -1.0, 0.0, 3.0]], np.float16)
+    b = np.array([[1.0, -0.0, 6e-8, 0.0, -2.0, -0.0]], np.float16)
+    got, want = run.mul(a, b, a.shape, abi.F16), oracle.mul(a, b, a.shape, abi.F16)
+    np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
+    assert np.all(np.signbit(got))
+    big_a, big_b = np.tile(a, (64, 16)), np.tile(b, (64, 16))  # the vectorised elementwise kernel
+    np.testing.assert_array_equal(run.mul(big_a, big_b, big_a.shape, abi.F16).view(np.uint16),
+                                  oracle.mul(big_a, big_b, big_a.shape, abi.F16).view(np.uint16))
+    rows = np.array([[-0.0, 1.0, 2.0], [-6e-8, 6e-8, 1.0], [1.0, -1.0, 0.0]], np.float16)
+    np.testing.assert_array_equal(run.reduce("PRODUCT", rows, 1).view(np.uint16),
+                                  oracle.reduce("PRODUCT", rows, 1).view(np.uint16))

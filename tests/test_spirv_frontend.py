@@ -77,6 +77,10 @@ REFERENCE_MODULES = {
     "conv3d_large_stride.spvasm": ({}, {0: np.zeros((3, 2, 2, 8192, 4), np.int8)}, [(abi.I8, (1, 3, 2, 2, 4))],
                                    [(abi.I32, (1, 3, 2, 2, 3))], ["CONV3D"]),
     "conv3d_inline_bf16_constant.spvasm": ({}, {}, [(abi.BF16, (1, 1, 1, 1, 1))], [(abi.BF16, (1, 1, 1, 1, 1))], ["CONV3D"]),
+    "conv3d_inline_fp8e4m3_constant.spvasm": ({}, {}, [(abi.F8E4M3, (1, 1, 1, 1, 1))], [(abi.F8E4M3, (1, 1, 1, 1, 1))],
+                                              ["CONV3D"]),
+    "conv3d_inline_fp8e5m2_constant.spvasm": ({}, {}, [(abi.F8E5M2, (1, 1, 1, 1, 1))], [(abi.F8E5M2, (1, 1, 1, 1, 1))],
+                                              ["CONV3D"]),
     "nop-outputs.spvasm": ({(0, 0, 0): (1, 8, 8, 3), (0, 1, 0): (1, 2, 2, 2), (0, 2, 0): (1, 8, 8, 3),
                             (0, 3, 0): (1, 8, 8, 3)}, {0: np.zeros((1, 8, 8, 3), np.int8)}, [I8_1883],
                            [(abi.I8, (1, 2, 2, 2)), I8_1883, I8_1883], ["SLICE", "CAST", "CAST"]),
@@ -106,7 +110,6 @@ def test_reference_modules_outside_the_operator_set_are_refused():
         return str(e.value)
 
     assert "does not import" in error_of("me_raw_sad_sr0.spvasm")          # motion-engine instruction set
-    assert "Float8E4M3EXT" in error_of("conv3d_inline_fp8e4m3_constant.spvasm")
     assert "no data supplied for graph constant 1" in error_of("graph-constant-arm.spvasm",
                                                                constants={0: np.array([2], np.int32)})
     assert "no shape for set 0 binding 0 element 1" in error_of("maxpool.spvasm", {(0, 1, 0): (1, 8, 8, 3)})
@@ -562,3 +565,34 @@ def test_multi_result_and_specialised_modules(dev, oracle):
     w.set_output(w.op("SCATTER", abi.I32, vals.shape, [iv, ii, ix]), out)
     got, _ = run_module(dev, w, {"values": vals, "indices": idx, "input": inp})
     np.testing.assert_array_equal(got["output"], oracle.scatter(vals, idx, inp))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [abi.BF16, abi.F8E4M3, abi.F8E5M2], ids=["bf16", "f8e4m3", "f8e5m2"])
+def test_inline_constants_of_reduced_precision_types(dev, oracle, dt):
+    """The structure of tests/shader/conv3d_inline_{bf16,fp8e4m3,fp8e5m2}_constant.spvasm (the reference only checks
+    that these pipelines are created and dispatched, tests/vulkan.cpp:1319-1329): a 1x1x1 CONV3D over a tensor of a
+    reduced-precision type whose weights and bias are replicated inline constants, once with the modules' integer
+    accumulator (operands truncated toward zero) and once with the floating-point accumulator of the type."""
+    enc = lambda values: oracle.cast(np.asarray(values, np.float32), dt)
+    shape = (1, 2, 1, 2, 1)
+    x = enc(np.float32([2.0, -3.5, 1.5, 0.75]).reshape(shape))
+    for acc, wv, bv in ((abi.ACC_I32, 1.0, 1.0), (abi.ACC_F32 if dt == abi.BF16 else abi.ACC_F16, 2.5, 0.25)):
+        w = sw.SpvAsm("inline_encoded_constant")
+        xin = w.input("input", dt, shape)
+        out = w.output("output", dt, shape)
+        weights = w.const(np.full((1, 1, 1, 1, 1), wv, np.float32), dt, replicate=True)
+        bias = w.const(np.full((1,), bv, np.float32), dt, replicate=True)
+        operands = [w.attr([0] * 6), w.attr([1] * 3), w.attr([1] * 3), w.u32(acc), w.scalar(abi.BOOL, False), xin,
+                    weights, bias, w.attr([0], abi.I8), w.attr([0], abi.I8)]
+        w.set_output(w.op("CONV3D", dt, shape, operands), out)
+        got, names = run_module(dev, w, {"input": np.asarray(x)})
+        assert names == ["CONV3D"]
+        want = oracle.conv3d(x, enc(np.full((1, 1, 1, 1, 1), wv)), enc(np.full((1,), bv)), shape, dt,
+                             abi.conv3d_attr(acc_type=acc))
+        np.testing.assert_array_equal(got["output"], want)
+        values = oracle.cast(want, abi.F32).ravel()
+        if acc == abi.ACC_I32:
+            np.testing.assert_array_equal(values, [3.0, -2.0, 2.0, 1.0])  # trunc(x) * 1 + 1
+        else:
+            np.testing.assert_array_equal(values, oracle.cast(enc(np.float32([5.25, -8.5, 4.0, 2.125])), abi.F32).ravel())
