@@ -50,11 +50,11 @@ typedef enum mlel_dtype {
     MLEL_I64 = 7,
     MLEL_U64 = 8,
     MLEL_F16 = 9,
-    MLEL_BF16 = 10,
+    MLEL_BF16 = 10,   /* upper half of an fp32; arithmetic in fp32 (graph/shaders/graph_op/common.comp:184-189) */
     MLEL_F32 = 11,
     MLEL_F64 = 12,
-    MLEL_F8E4M3 = 13,
-    MLEL_F8E5M2 = 14,
+    MLEL_F8E4M3 = 13, /* bias 7, no infinities, NaN = 0x7f; arithmetic in fp16 (common.comp:197-215) */
+    MLEL_F8E5M2 = 14, /* upper byte of an fp16; arithmetic in fp16 (common.comp:191-195) */
     MLEL_DTYPE_COUNT = 15
 } mlel_dtype;
 
