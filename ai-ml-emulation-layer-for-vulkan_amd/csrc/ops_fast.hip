@@ -108,11 +108,12 @@ struct DwArgs {
     const int32_t *bias;
     char *out;
     int32_t N, H, W, C, OH, OW;
-    int64_t x_sn, x_sy, x_sx;  // input byte strides (channel stride 1)
+    uint32_t x_sn, x_sy, x_sx;  // input byte strides (channel stride 1); input and output extents are below 2^31
+    uint32_t x_bytes, o_bytes;
     int32_t sy, sx, pad_t, pad_l, zi, zw, bias_len;
     int32_t fused, out_size;
     ScaleRef scale;
-    int64_t items;  // N * row groups * strips * C/4
+    uint32_t items;  // N * row groups * strips * C/4
     int32_t strips, row_groups;
     int32_t blocks, chunk;  // launch geometry: `chunk` consecutive blocks of items per XCD
 };
@@ -128,20 +129,23 @@ __device__ __forceinline__ void transpose_3x4(uint32_t r0, uint32_t r1, uint32_t
     col[3] = __builtin_amdgcn_perm(r2, t1, 0x0c070302u);             // [t1.b2 t1.b3 r2.b3 0]
 }
 
-template <int TX, int TY, int SX, bool ZW>
+// Q8: fused epilogue with 8-bit output (a compile-time choice keeps the unrolled epilogue free of branches).  All
+// index arithmetic is 32-bit (the host checks the extents); loads and stores are buffer instructions with 32-bit
+// offsets, so an address costs one add.
+template <int TX, int TY, int SX, bool ZW, bool Q8>
 __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
     // blocks are dealt round-robin to the XCDs: give XCD k the k-th contiguous run of blocks
     const int bid = (int)(blockIdx.x % 8u) * a.chunk + (int)(blockIdx.x / 8u);
     if (bid >= a.blocks) return;
-    const int64_t item = (int64_t)bid * kBlock + threadIdx.x;
+    const uint32_t item = (uint32_t)bid * kBlock + threadIdx.x;
     if (item >= a.items) return;
-    const int c4n = a.C >> 2;
+    const uint32_t c4n = (uint32_t)a.C >> 2;
     const int c4 = (int)(item % c4n);
-    int64_t rest = item / c4n;
-    const int strip = (int)(rest % a.strips);
-    rest /= a.strips;
-    const int rg = (int)(rest % a.row_groups);
-    const int n = (int)(rest / a.row_groups);
+    uint32_t rest = item / c4n;
+    const int strip = (int)(rest % (uint32_t)a.strips);
+    rest /= (uint32_t)a.strips;
+    const int rg = (int)(rest % (uint32_t)a.row_groups);
+    const int n = (int)(rest / (uint32_t)a.row_groups);
     const int c = c4 * 4;
     const int ox0 = strip * TX, oy0 = rg * TY;
 
@@ -164,7 +168,7 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
         const int32_t bias = a.bias[a.bias_len == 1 ? 0 : c + e];
         bias_adj[e] = (int32_t)((uint32_t)bias - (uint32_t)a.zi * (uint32_t)wsum[e] +
                                 9u * (uint32_t)a.zi * (uint32_t)a.zw);
-        if (a.fused) {
+        if (Q8 || a.fused) {
             const int ci = a.scale.p.per_channel ? c + e : 0;
             q[e] = make_chan_scale(load_mult(a.scale, ci), (int32_t)a.scale.shift[ci], a.scale.p);
         }
@@ -175,7 +179,11 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
     constexpr int sy = SX;  // the host only sends equal strides here
     const int iy0 = oy0 * sy - a.pad_t, ix0 = ox0 * SX - a.pad_l;
     const uint32_t zsplat = (uint32_t)(uint8_t)a.zi * 0x01010101u;
-    const int8_t *xb = a.x + (int64_t)n * a.x_sn + c;
+    const __amdgpu_buffer_rsrc_t xres =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(a.x), 0, (int)a.x_bytes, 0x00020000);
+    // offsets of taps outside the image wrap to values beyond the extent (such loads return 0) or name another
+    // pixel; either way the value is replaced by the zero point below
+    const uint32_t xbase = (uint32_t)n * a.x_sn + (uint32_t)c + (uint32_t)iy0 * a.x_sy + (uint32_t)ix0 * a.x_sx;
     int32_t acc[TY][TX][4], xs[TY][TX][4];
 #pragma unroll
     for (int ty = 0; ty < TY; ty++)
@@ -186,17 +194,18 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
 
     constexpr int NROW_MAX = SX * (TY - 1) + 3;
     uint32_t raw[NROW_MAX][NCOL];
+    bool xin[NCOL];
+#pragma unroll
+    for (int j = 0; j < NCOL; j++) xin[j] = (unsigned)(ix0 + j) < (unsigned)a.W;
 #pragma unroll
     for (int r = 0; r < NROW_MAX; r++) {
-        const int y = iy0 + r;
-        const bool yin = (unsigned)y < (unsigned)a.H;
+        const bool yin = (unsigned)(iy0 + r) < (unsigned)a.H;
+        const uint32_t rowoff = xbase + (uint32_t)r * a.x_sy;
 #pragma unroll
         for (int j = 0; j < NCOL; j++) {
-            const int x = ix0 + j;
-            uint32_t v = zsplat;
-            if (yin && (unsigned)x < (unsigned)a.W)
-                v = *reinterpret_cast<const uint32_t *>(xb + (int64_t)y * a.x_sy + (int64_t)x * a.x_sx);
-            raw[r][j] = v;
+            const uint32_t v =
+                (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(xres, (int)(rowoff + (uint32_t)j * a.x_sx), 0, 0);
+            raw[r][j] = (yin && xin[j]) ? v : zsplat;
         }
     }
 #pragma unroll
@@ -219,11 +228,13 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
     }
 
     // ---- epilogue
+    const __amdgpu_buffer_rsrc_t ores = __builtin_amdgcn_make_buffer_rsrc(a.out, 0, (int)a.o_bytes, 0x00020000);
+    const uint32_t esz = Q8 ? 1u : (uint32_t)a.out_size;
 #pragma unroll
     for (int ty = 0; ty < TY; ty++) {
         const int oy = oy0 + ty;
         if (oy >= a.OH) break;
-        const int64_t orow = ((int64_t)n * a.OH + oy) * a.OW;
+        const uint32_t orow = ((uint32_t)n * (uint32_t)a.OH + (uint32_t)oy) * (uint32_t)a.OW;
 #pragma unroll
         for (int t = 0; t < TX; t++) {
             const int ox = ox0 + t;
@@ -233,19 +244,20 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
             for (int e = 0; e < 4; e++) {
                 int32_t s = (int32_t)((uint32_t)acc[ty][t][e] + (uint32_t)bias_adj[e]);
                 if (ZW) s = (int32_t)((uint32_t)s - (uint32_t)a.zw * (uint32_t)xs[ty][t][e]);
-                if (a.fused) s = requant_chan(s, q[e], a.scale.p);
+                if (Q8 || a.fused) s = requant_chan(s, q[e], a.scale.p);
                 v[e] = s;
             }
-            const int64_t off = (orow + ox) * a.C + c;
-            if (a.out_size == 1) {
-                *reinterpret_cast<uint32_t *>(a.out + off) = ((uint32_t)v[0] & 0xffu) | (((uint32_t)v[1] & 0xffu) << 8) |
-                                                             (((uint32_t)v[2] & 0xffu) << 16) | ((uint32_t)v[3] << 24);
+            const uint32_t off = ((orow + (uint32_t)ox) * (uint32_t)a.C + (uint32_t)c) * esz;
+            if (Q8 || a.out_size == 1) {
+                const uint32_t packed = ((uint32_t)v[0] & 0xffu) | (((uint32_t)v[1] & 0xffu) << 8) |
+                                        (((uint32_t)v[2] & 0xffu) << 16) | ((uint32_t)v[3] << 24);
+                __builtin_amdgcn_raw_buffer_store_b32(packed, ores, (int)off, 0, 0);
             } else if (a.out_size == 2) {
-                *reinterpret_cast<uint2 *>(a.out + off * 2) =
-                    make_uint2((uint32_t)(uint16_t)v[0] | ((uint32_t)(uint16_t)v[1] << 16),
-                               (uint32_t)(uint16_t)v[2] | ((uint32_t)(uint16_t)v[3] << 16));
+                __builtin_amdgcn_raw_buffer_store_b32((uint32_t)(uint16_t)v[0] | ((uint32_t)(uint16_t)v[1] << 16), ores, (int)off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32((uint32_t)(uint16_t)v[2] | ((uint32_t)(uint16_t)v[3] << 16), ores, (int)off + 4, 0, 0);
             } else {
-                *reinterpret_cast<int4 *>(a.out + off * 4) = make_int4(v[0], v[1], v[2], v[3]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) __builtin_amdgcn_raw_buffer_store_b32((uint32_t)v[e], ores, (int)off + 4 * e, 0, 0);
             }
         }
     }
@@ -276,6 +288,10 @@ int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     if (N <= 0 || OH <= 0 || OW <= 0) return 1;
     if (in->dims[1] >= (1 << 30) || in->dims[2] >= (1 << 30) || OH >= (1 << 30) || OW >= (1 << 30)) return 0;
 
+    // 32-bit offsets: both extents and the item count stay below 2^31
+    if (in->strides[0] < 0 || in->strides[1] < 0 || in->strides[2] < 0) return 0;
+    const int64_t x_extent = in->dims[0] * in->strides[0], o_extent = N * OH * OW * C * dt_size(out->dtype);
+    if (x_extent <= 0 || x_extent >= (int64_t(1) << 31) || o_extent >= (int64_t(1) << 31)) return 0;
     constexpr int TX = 4;
     const int TY = OH >= 2 ? 2 : 1;
     DwArgs g{};
@@ -289,9 +305,11 @@ int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     g.C = (int)C;
     g.OH = (int)OH;
     g.OW = (int)OW;
-    g.x_sn = in->strides[0];
-    g.x_sy = in->strides[1];
-    g.x_sx = in->strides[2];
+    g.x_sn = (uint32_t)in->strides[0];
+    g.x_sy = (uint32_t)in->strides[1];
+    g.x_sx = (uint32_t)in->strides[2];
+    g.x_bytes = (uint32_t)x_extent;
+    g.o_bytes = (uint32_t)o_extent;
     g.sy = a->stride[0];
     g.sx = a->stride[1];
     g.pad_t = a->pad[0];
@@ -304,23 +322,38 @@ int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     if (epi) g.scale = make_ref(*epi);
     g.strips = (int)((OW + TX - 1) / TX);
     g.row_groups = (int)((OH + TY - 1) / TY);
-    g.items = N * g.row_groups * g.strips * (C / 4);
-    const int64_t blocks = (g.items + kBlock - 1) / kBlock;
-    MLEL_REQUIRE(blocks < (int64_t(1) << 30), MLEL_ERR_LIMIT, "depthwise_conv2d: too many work items");
+    const int64_t items = N * g.row_groups * g.strips * (C / 4);
+    if (items >= (int64_t(1) << 31) - kBlock) return 0;
+    g.items = (uint32_t)items;
+    const int64_t blocks = (items + kBlock - 1) / kBlock;
     g.blocks = (int)blocks;
     g.chunk = (int)((blocks + 7) / 8);
     const dim3 grid((unsigned)(g.chunk * 8)), block(kBlock);
+    const bool q8 = g.fused && g.out_size == 1;
     const int variant = (TY == 2 ? 4 : 0) + (g.sx == 2 ? 2 : 0) + (g.zw != 0 ? 1 : 0);
+#define MLEL_DW_CASE(ID, TYV, SXV, ZWV)                                                  \
+    case ID:                                                                             \
+        if (q8)                                                                          \
+            dwconv3x3_i8_kernel<TX, TYV, SXV, ZWV, true><<<grid, block, 0, s>>>(g);      \
+        else                                                                             \
+            dwconv3x3_i8_kernel<TX, TYV, SXV, ZWV, false><<<grid, block, 0, s>>>(g);     \
+        break;
     switch (variant) {
-    case 0: dwconv3x3_i8_kernel<TX, 1, 1, false><<<grid, block, 0, s>>>(g); break;
-    case 1: dwconv3x3_i8_kernel<TX, 1, 1, true><<<grid, block, 0, s>>>(g); break;
-    case 2: dwconv3x3_i8_kernel<TX, 1, 2, false><<<grid, block, 0, s>>>(g); break;
-    case 3: dwconv3x3_i8_kernel<TX, 1, 2, true><<<grid, block, 0, s>>>(g); break;
-    case 4: dwconv3x3_i8_kernel<TX, 2, 1, false><<<grid, block, 0, s>>>(g); break;
-    case 5: dwconv3x3_i8_kernel<TX, 2, 1, true><<<grid, block, 0, s>>>(g); break;
-    case 6: dwconv3x3_i8_kernel<TX, 2, 2, false><<<grid, block, 0, s>>>(g); break;
-    default: dwconv3x3_i8_kernel<TX, 2, 2, true><<<grid, block, 0, s>>>(g); break;
+        MLEL_DW_CASE(0, 1, 1, false)
+        MLEL_DW_CASE(1, 1, 1, true)
+        MLEL_DW_CASE(2, 1, 2, false)
+        MLEL_DW_CASE(3, 1, 2, true)
+        MLEL_DW_CASE(4, 2, 1, false)
+        MLEL_DW_CASE(5, 2, 1, true)
+        MLEL_DW_CASE(6, 2, 2, false)
+    default:
+        if (q8)
+            dwconv3x3_i8_kernel<TX, 2, 2, true, true><<<grid, block, 0, s>>>(g);
+        else
+            dwconv3x3_i8_kernel<TX, 2, 2, true, false><<<grid, block, 0, s>>>(g);
+        break;
     }
+#undef MLEL_DW_CASE
     MLEL_TRY(check_launch("depthwise_conv2d 3x3 int8"));
     return 1;
 }
