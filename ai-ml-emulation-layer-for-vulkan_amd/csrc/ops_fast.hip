@@ -190,7 +190,10 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
 #pragma unroll
         for (int t = 0; t < TX; t++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) acc[ty][t][e] = xs[ty][t][e] = 0;
+            for (int e = 0; e < 4; e++) {
+                acc[ty][t][e] = bias_adj[e];  // the dot products accumulate on top of the bias term
+                xs[ty][t][e] = 0;
+            }
 
     constexpr int NROW_MAX = SX * (TY - 1) + 3;
     uint32_t raw[NROW_MAX][NCOL];
@@ -242,7 +245,7 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
             int32_t v[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                int32_t s = (int32_t)((uint32_t)acc[ty][t][e] + (uint32_t)bias_adj[e]);
+                int32_t s = acc[ty][t][e];
                 if (ZW) s = (int32_t)((uint32_t)s - (uint32_t)a.zw * (uint32_t)xs[ty][t][e]);
                 if (Q8 || a.fused) s = requant_chan(s, q[e], a.scale.p);
                 v[e] = s;
