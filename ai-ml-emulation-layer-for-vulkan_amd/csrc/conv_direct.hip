@@ -55,7 +55,7 @@ __host__ __device__ constexpr uint32_t pixel_mask(int p, int d) {
 }
 
 // KD = dwords of gathered input per position; STEM: 3 rows x 3 dwords (IC = ICS), ROWS: IC / 4
-template <int MODE, int ICS, int KD, int OCB, int P, bool Q8>
+template <int MODE, int ICS, int KD, int OCB, int P, bool Q8, bool ZW>
 __global__ void __launch_bounds__(kBlock) conv_direct_i8_kernel(const DirectArgs a) {
     __shared__ __align__(16) uint32_t wl[OCB][KD];
     __shared__ __align__(16) ChanConst cc[OCB];
@@ -157,7 +157,7 @@ __global__ void __launch_bounds__(kBlock) conv_direct_i8_kernel(const DirectArgs
             }
         }
         xcorr[p] = 0;
-        if (a.zw != 0) {
+        if (ZW) {
             int32_t xsum = 0;
 #pragma unroll
             for (int j = 0; j < KD; j++) xsum = __builtin_amdgcn_sdot4((int)xd[p][j], 0x01010101, xsum, false);
@@ -182,10 +182,10 @@ __global__ void __launch_bounds__(kBlock) conv_direct_i8_kernel(const DirectArgs
             const ChanConst c = cc[oc];
 #pragma unroll
             for (int p = 0; p < P; p++) {
-                int32_t acc = 0;
+                // the dot products accumulate on top of the bias term (and the weight zero-point term, if any)
+                int32_t v = ZW ? (int32_t)((uint32_t)c.bias_adj - (uint32_t)xcorr[p]) : c.bias_adj;
 #pragma unroll
-                for (int j = 0; j < KD; j++) acc = __builtin_amdgcn_sdot4((int)xd[p][j], (int)wv[j], acc, false);
-                const int32_t v = (int32_t)((uint32_t)acc + (uint32_t)c.bias_adj - (uint32_t)xcorr[p]);
+                for (int j = 0; j < KD; j++) v = __builtin_amdgcn_sdot4((int)xd[p][j], (int)wv[j], v, false);
                 if (Q8) {
                     packed[p][e / 4] |= ((uint32_t)requant_chan(v, c.q, a.scale.p) & 0xffu) << (8 * (e % 4));
                 } else {
@@ -208,16 +208,22 @@ __global__ void __launch_bounds__(kBlock) conv_direct_i8_kernel(const DirectArgs
 
 template <int MODE, int ICS, int KD, int P>
 void launch_direct_p(const DirectArgs &g, dim3 grid, hipStream_t s) {
-    // fused 8-bit epilogue or int32 accumulators: a compile-time choice, so that the unrolled channel loop is one
-    // basic block and the requantisation chains of neighbouring channels interleave
-    if (g.ocb == 32 && g.out_size == 1)
-        conv_direct_i8_kernel<MODE, ICS, KD, 32, P, true><<<grid, dim3(kBlock), 0, s>>>(g);
-    else if (g.ocb == 32)
-        conv_direct_i8_kernel<MODE, ICS, KD, 32, P, false><<<grid, dim3(kBlock), 0, s>>>(g);
-    else if (g.out_size == 1)
-        conv_direct_i8_kernel<MODE, ICS, KD, 16, P, true><<<grid, dim3(kBlock), 0, s>>>(g);
-    else
-        conv_direct_i8_kernel<MODE, ICS, KD, 16, P, false><<<grid, dim3(kBlock), 0, s>>>(g);
+    // fused 8-bit epilogue or int32 accumulators, weight zero point or none: compile-time choices, so that the unrolled
+    // channel loop is one basic block and the requantisation chains of neighbouring channels interleave
+    const bool q8 = g.out_size == 1, zw = g.zw != 0;
+#define MLEL_DIRECT(OCBV, Q8V, ZWV) conv_direct_i8_kernel<MODE, ICS, KD, OCBV, P, Q8V, ZWV><<<grid, dim3(kBlock), 0, s>>>(g)
+    if (g.ocb == 32) {
+        if (q8 && !zw) MLEL_DIRECT(32, true, false);
+        else if (q8) MLEL_DIRECT(32, true, true);
+        else if (!zw) MLEL_DIRECT(32, false, false);
+        else MLEL_DIRECT(32, false, true);
+    } else {
+        if (q8 && !zw) MLEL_DIRECT(16, true, false);
+        else if (q8) MLEL_DIRECT(16, true, true);
+        else if (!zw) MLEL_DIRECT(16, false, false);
+        else MLEL_DIRECT(16, false, true);
+    }
+#undef MLEL_DIRECT
 }
 
 // Positions per thread: every channel's weights and constants are broadcast from shared memory once per thread, so
