@@ -404,22 +404,23 @@ namespace {
 // block owns 64 rows: its four wavefronts copy a slab of 64 rows x up to 1024 columns into shared memory with coalesced
 // 128-bit loads and then the lanes of the first wavefront fold one row each out of shared memory, element by element.
 // ---------------------------------------------------------------------------------------------------------------
-constexpr int kSlabMaxCols = 1024;  // halfs per row and slab: 64 rows x 1024 x 2 B = 128 KB of shared memory at most
+constexpr int kSlabCols = 256;  // halfs per row and slab: two buffers of 64 rows x 256 x 2 B (+ padding) = 66 KB
 
 struct ReduceArgs {
     const char *in;
     char *out;
     int64_t rows;
     int32_t cols;       // multiple of 8
-    int32_t slab_cols;  // min(cols, kSlabMaxCols), multiple of 8
+    int32_t slab_cols;  // min(cols, kSlabCols), multiple of 8
     int32_t ignore_nan;
 };
 
 template <bool IS_SUM>
 __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArgs g) {
     // A block owns 64 rows.  A fold is sequential along its row, so parallelism comes from rows only and small row
-    // counts (LayerNorm over a few thousand tokens) must still spread over many compute units; all four wavefronts
-    // fetch the slab (many loads in flight), then the first one folds it out of shared memory, one row per lane.
+    // counts (LayerNorm over a few thousand tokens) must still spread over many compute units.  The row is walked in
+    // slabs through two buffers: the first wavefront folds slab k out of shared memory, one row per lane, while the
+    // other three fetch slab k + 1 (the first slab is fetched by all four).
     extern __shared__ __align__(16) char slab[];
     const int pitch = g.slab_cols * 2 + 16;  // bytes; 16-byte aligned, consecutive rows four banks apart
     const int tid = threadIdx.x;
@@ -427,15 +428,15 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArg
     const int64_t row = row0 + tid;
     float r = IS_SUM ? 0.f : (g.ignore_nan ? NAN : -65504.f);
     bool done = false;
-    for (int c0 = 0; c0 < g.cols; c0 += g.slab_cols) {
+    // consecutive threads take consecutive 16-byte pieces of a row; eight loads in flight per thread
+    const auto stage = [&](int c0, char *buf, int first, int nthreads) {
         const int n = min(g.slab_cols, g.cols - c0);
-        const int segs = n >> 3;       // 16-byte pieces per row
-        const int pieces = 64 * segs;  // consecutive threads take consecutive pieces of a row
-        for (int p0 = 0; p0 < pieces; p0 += kBlock * 8) {
+        const int segs = n >> 3, pieces = 64 * segs;
+        for (int p0 = 0; p0 < pieces; p0 += nthreads * 8) {
             uint4 v[8];
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const int p = p0 + i * kBlock + tid;
+                const int p = p0 + i * nthreads + (tid - first);
                 const int rr = p / segs, seg = p - rr * segs;
                 v[i] = make_uint4(0, 0, 0, 0);
                 if (p < pieces && row0 + rr < g.rows)
@@ -443,49 +444,50 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArg
             }
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const int p = p0 + i * kBlock + tid;
+                const int p = p0 + i * nthreads + (tid - first);
                 const int rr = p / segs, seg = p - rr * segs;
-                if (p < pieces) {
-                    *reinterpret_cast<uint4 *>(slab + rr * pitch + seg * 16) = v[i];
-                }
+                if (p < pieces) *reinterpret_cast<uint4 *>(buf + rr * pitch + seg * 16) = v[i];
             }
         }
-        __syncthreads();
-        if (tid < 64) {
-            const char *mine = slab + tid * pitch;
-            uint4 next = *reinterpret_cast<const uint4 *>(mine);
-            for (int j = 0; j < n; j += 8) {
-                const uint4 raw = next;
-                if (j + 8 < n) next = *reinterpret_cast<const uint4 *>(mine + (j + 8) * 2);
+    };
+    const int buf_bytes = 64 * pitch;
+    stage(0, slab, 0, kBlock);
+    __syncthreads();
+    int which = 0;
+    for (int c0 = 0; c0 < g.cols; c0 += g.slab_cols, which ^= 1) {
+        const int n = min(g.slab_cols, g.cols - c0);
+        if (tid >= 64) {
+            if (c0 + g.slab_cols < g.cols) stage(c0 + g.slab_cols, slab + (which ^ 1) * buf_bytes, 64, kBlock - 64);
+        } else {
+            const char *mine = slab + which * buf_bytes + tid * pitch;
+            // a NaN among eight halfs: exponent all ones and a non-zero mantissa, tested on the packed pairs
+            const auto nan_bits = [](const uint4 &raw) {
+                return (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu) |
+                        ((raw.z & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
+            };
+            // No lane of the wavefront in a special state: the plain fold.  A native fp16 add rounds the exact sum
+            // once; the generic kernel's fp32 add followed by a conversion gives the same value (fp32 carries more
+            // than twice the fp16 precision plus two bits, so the second rounding cannot change the result).
+            const auto fold_plain = [&](const uint4 &raw, __half &acc, float &mx) {
                 const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
-                // a NaN among the eight halfs: exponent all ones and a non-zero mantissa, tested on the packed pairs
-                const uint32_t nan_bits =
-                    (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu) |
-                     ((raw.z & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
-                if (!__any(done || nan_bits != 0)) {
-                    // no lane of the wavefront is in a special state: the plain fold.  A native fp16 add rounds the
-                    // exact sum once; the generic kernel's fp32 add followed by a conversion gives the same value
-                    // (fp32 carries more than twice the fp16 precision plus two bits, so the second rounding cannot
-                    // change the result).
-                    if (IS_SUM) {
-                        __half acc = f2h(r);
+                if (IS_SUM) {
 #pragma unroll
-                        for (int t = 0; t < 4; t++) {
-                            acc = __hadd(acc, __low2half(h[t]));
-                            acc = __hadd(acc, __high2half(h[t]));
-                        }
-                        r = __half2float(acc);
-                    } else {
-                        // the order of a maximum is free: pairwise on the packed halfs, then against the state
-                        typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-                        const h2_t *p = reinterpret_cast<const h2_t *>(&raw);
-                        const h2_t m = __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]),
-                                                                 __builtin_elementwise_max(p[2], p[3]));
-                        const float e = (float)(m.x > m.y ? m.x : m.y);
-                        r = isnan(r) ? e : (r < e ? e : r);
+                    for (int t = 0; t < 4; t++) {
+                        acc = __hadd(acc, __low2half(h[t]));
+                        acc = __hadd(acc, __high2half(h[t]));
                     }
-                    continue;
+                } else {
+                    // the order of a maximum is free: pairwise on the packed halfs, then against the state
+                    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+                    const h2_t *p = reinterpret_cast<const h2_t *>(&raw);
+                    const h2_t m = __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]),
+                                                             __builtin_elementwise_max(p[2], p[3]));
+                    const float e = (float)(m.x > m.y ? m.x : m.y);
+                    mx = isnan(mx) ? e : (mx < e ? e : mx);
                 }
+            };
+            const auto fold_careful = [&](const uint4 &raw) {  // NaN-aware, element by element
+                const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
                 float e[8];
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
@@ -508,7 +510,35 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArg
                     else
                         r = isnan(r) ? v : (r < v ? v : r);
                 }
+            };
+            // groups of 32 elements: one test for special values per group keeps the dependent chain of the fold short
+            int j = 0;
+            uint4 nxt[4];
+            if (n >= 32) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) nxt[t] = *reinterpret_cast<const uint4 *>(mine + t * 16);
             }
+            for (; j + 32 <= n; j += 32) {
+                uint4 raw[4];
+#pragma unroll
+                for (int t = 0; t < 4; t++) raw[t] = nxt[t];
+                if (j + 64 <= n) {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) nxt[t] = *reinterpret_cast<const uint4 *>(mine + (j + 32) * 2 + t * 16);
+                }
+                const uint32_t special = nan_bits(raw[0]) | nan_bits(raw[1]) | nan_bits(raw[2]) | nan_bits(raw[3]);
+                if (!__any(done || special != 0)) {
+                    __half acc = f2h(r);
+                    float mx = r;
+#pragma unroll
+                    for (int t = 0; t < 4; t++) fold_plain(raw[t], acc, mx);
+                    r = IS_SUM ? __half2float(acc) : mx;
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) fold_careful(raw[t]);
+                }
+            }
+            for (; j < n; j += 8) fold_careful(*reinterpret_cast<const uint4 *>(mine + j * 2));
         }
         __syncthreads();
     }
@@ -652,8 +682,8 @@ int try_reduce_float_fast(mlel_ctx *, hipStream_t s, int op, const mlel_tensor *
     g.ignore_nan = nan_mode == MLEL_NAN_IGNORE ? 1 : 0;
     const int64_t blocks = (rows + 63) / 64;
     MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "reduce: too many rows");
-    g.slab_cols = (int32_t)(cols < kSlabMaxCols ? cols : kSlabMaxCols);
-    const size_t smem = (size_t)64 * (g.slab_cols * 2 + 16);
+    g.slab_cols = (int32_t)(cols < kSlabCols ? cols : kSlabCols);
+    const size_t smem = (size_t)2 * 64 * (g.slab_cols * 2 + 16);
     auto kernel = op == MLEL_RED_SUM ? reduce_rows_f16_kernel<true> : reduce_rows_f16_kernel<false>;
     if (smem > 48 * 1024)
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
