@@ -33,9 +33,13 @@
 //   RFFT2D                     in: input                    out: real, imag
 //   binary (ADD SUB BITWISE_* LOGICAL_* INTDIV POW EQUAL GREATER GREATER_EQUAL): in: input1, input2
 //   unary (ABS ... TANH), CAST, RESHAPE: in: input
+#include <algorithm>
+#include <cctype>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <map>
+#include <sstream>
 #include <string>
 
 #include "../../../include/mlel_graph.h"
@@ -45,16 +49,34 @@
 
 using namespace mlel::graph;
 
+struct ProfileSample {
+    uint64_t dispatch;  // which mlel_graph_dispatch call of this graph
+    uint32_t index;     // position in the execution list
+    std::string name;
+    double ms;
+};
+
 struct mlel_graph {
     GraphPipeline pipeline;
     mlel_ctx *ctx;
     std::vector<void *> events;  // pairs of profiling events, created on demand
+    bool profiling = false;      // mlel_graph_dispatch records a sample per operator (VMEL_GRAPH_PROFILING)
+    uint64_t dispatches = 0;
+    std::vector<ProfileSample> samples;
     explicit mlel_graph(mlel_ctx *c) : pipeline(c), ctx(c) {}
 };
 
 namespace {
 
 thread_local std::string g_error;
+
+// VMEL_GRAPH_PROFILING: anything but empty, 0, false, off, no (graph/graph_profiler.cpp:29-38)
+bool truthy(const char *value) {
+    if (value == nullptr || value[0] == 0) return false;
+    std::string v(value);
+    for (auto &c : v) c = static_cast<char>(std::tolower(static_cast<unsigned char>(c)));
+    return v != "0" && v != "false" && v != "off" && v != "no";
+}
 
 template <typename F>
 int guarded(F &&f) {
@@ -274,6 +296,7 @@ int mlel_graph_create(mlel_ctx *ctx, mlel_graph **out) {
     return guarded([&] {
         if (out == nullptr) throw std::runtime_error("null out pointer");
         *out = new mlel_graph(ctx);
+        (*out)->profiling = truthy(std::getenv("VMEL_GRAPH_PROFILING"));
         return 0;
     });
 }
@@ -432,31 +455,110 @@ int mlel_graph_bind_external(mlel_graph *g, uint32_t set, uint32_t binding, uint
     });
 }
 
+namespace {
+
+// a pair of events around every operator; milliseconds per operator into `ms` (n entries)
+void dispatchTimed(mlel_graph *g, void *stream, std::vector<float> &ms) {
+    const size_t n = g->pipeline.executionList().size();
+    while (g->events.size() < 2 * n) {
+        void *e = nullptr;
+        if (mlel_hip_event_create(g->ctx, &e) != 0) throw std::runtime_error(mlel_hip_last_error());
+        g->events.push_back(e);
+    }
+    g->pipeline.dispatch(stream, [&](const OpNode &, uint32_t index, bool before) {
+        if (mlel_hip_event_record(g->ctx, g->events[2 * index + (before ? 0 : 1)], stream) != 0)
+            throw std::runtime_error(mlel_hip_last_error());
+    });
+    ms.assign(n, 0.f);
+    for (size_t i = 0; i < n; i++)
+        if (mlel_hip_event_elapsed_ms(g->ctx, g->events[2 * i], g->events[2 * i + 1], &ms[i]) != 0)
+            throw std::runtime_error(mlel_hip_last_error());
+}
+
+}  // namespace
+
 int mlel_graph_dispatch(mlel_graph *g, void *stream) {
     return guarded([&] {
-        g->pipeline.dispatch(stream);
+        if (!g->profiling) {
+            g->pipeline.dispatch(stream);
+            return 0;
+        }
+        // profiling: this dispatch waits for its own events (the reference reads its timestamps back at the fence)
+        std::vector<float> ms;
+        dispatchTimed(g, stream, ms);
+        const auto list = g->pipeline.executionList();
+        for (size_t i = 0; i < list.size(); i++)
+            g->samples.push_back(ProfileSample{g->dispatches, static_cast<uint32_t>(i), opLabel(*list[i]), ms[i]});
+        g->dispatches++;
         return 0;
     });
 }
 
 int mlel_graph_dispatch_profiled(mlel_graph *g, void *stream, float *ms, int capacity) {
     return guarded([&] {
-        const int n = static_cast<int>(g->pipeline.executionList().size());
-        while (static_cast<int>(g->events.size()) < 2 * n) {
-            void *e = nullptr;
-            if (mlel_hip_event_create(g->ctx, &e) != 0) throw std::runtime_error(mlel_hip_last_error());
-            g->events.push_back(e);
-        }
-        g->pipeline.dispatch(stream, [&](const OpNode &, uint32_t index, bool before) {
-            if (mlel_hip_event_record(g->ctx, g->events[2 * index + (before ? 0 : 1)], stream) != 0)
-                throw std::runtime_error(mlel_hip_last_error());
-        });
-        for (int i = 0; i < n && i < capacity; i++)
-            if (mlel_hip_event_elapsed_ms(g->ctx, g->events[2 * static_cast<size_t>(i)],
-                                          g->events[2 * static_cast<size_t>(i) + 1], &ms[i]) != 0)
-                throw std::runtime_error(mlel_hip_last_error());
-        return n;
+        std::vector<float> all;
+        dispatchTimed(g, stream, all);
+        for (size_t i = 0; i < all.size() && static_cast<int>(i) < capacity; i++) ms[i] = all[i];
+        return static_cast<int>(all.size());
     });
+}
+
+int mlel_graph_set_profiling(mlel_graph *g, int enabled) {
+    return guarded([&] {
+        g->profiling = enabled != 0;
+        return 0;
+    });
+}
+
+int mlel_graph_get_profiling(mlel_graph *g) {
+    return guarded([&] { return g->profiling ? 1 : 0; });
+}
+
+int64_t mlel_graph_profiling_json(mlel_graph *g, char *buf, size_t capacity) {
+    int64_t needed = 0;
+    const int rc = guarded([&] {
+        // the report of the reference's profiler (graph/graph_profiler.cpp:563-625): every sample, then count / total /
+        // average / min / max per operator name; times come from event pairs, so there are no cycle counts
+        struct Agg {
+            uint64_t count = 0;
+            double total = 0, mn = 0, mx = 0;
+        };
+        std::map<std::string, Agg> by;
+        std::ostringstream o;
+        o.precision(9);
+        o << "{\n  \"timestamp_period_ns\": null,\n  \"samples\": [";
+        bool first = true;
+        for (const auto &s : g->samples) {
+            o << (first ? "\n" : ",\n") << "    {\"submission\": " << s.dispatch << ", \"graph_dispatch\": " << s.dispatch
+              << ", \"pipeline_index\": " << s.index << ", \"pipeline_kind\": \"tosa\", \"operator_name\": \"" << s.name
+              << "\", \"time_ms\": " << s.ms << "}";
+            first = false;
+            Agg &a = by[s.name];
+            a.mn = a.count == 0 ? s.ms : std::min(a.mn, s.ms);
+            a.mx = a.count == 0 ? s.ms : std::max(a.mx, s.ms);
+            a.count++;
+            a.total += s.ms;
+        }
+        o << (first ? "" : "\n  ") << "],\n  \"by_operator\": [";
+        first = true;
+        for (const auto &[name, a] : by) {
+            o << (first ? "\n" : ",\n") << "    {\"pipeline_kind\": \"tosa\", \"operator_name\": \"" << name
+              << "\", \"dispatch_count\": " << a.count << ", \"total_time_ms\": " << a.total
+              << ", \"average_time_ms\": " << (a.count ? a.total / static_cast<double>(a.count) : 0.0)
+              << ", \"min_time_ms\": " << a.mn << ", \"max_time_ms\": " << a.mx << "}";
+            first = false;
+        }
+        o << (first ? "" : "\n  ") << "]\n}\n";
+        const std::string text = o.str();
+        needed = static_cast<int64_t>(text.size()) + 1;
+        if (buf != nullptr && capacity > 0) {
+            const size_t n = std::min(capacity - 1, text.size());
+            std::memcpy(buf, text.data(), n);
+            buf[n] = 0;
+        }
+        return 0;
+    });
+    return rc != 0 ? rc : needed;
 }
 
 int mlel_graph_op_count(mlel_graph *g) {

@@ -66,6 +66,10 @@ def load_graph_library():
         lib.mlel_graph_bind_external.argtypes = [_V, C.c_uint32, C.c_uint32, C.c_uint32, _V]
         lib.mlel_graph_dispatch.argtypes = [_V, _V]
         lib.mlel_graph_dispatch_profiled.argtypes = [_V, _V, C.POINTER(C.c_float), C.c_int]
+        lib.mlel_graph_set_profiling.argtypes = [_V, C.c_int]
+        lib.mlel_graph_get_profiling.argtypes = [_V]
+        lib.mlel_graph_profiling_json.argtypes = [_V, C.c_char_p, C.c_size_t]
+        lib.mlel_graph_profiling_json.restype = C.c_int64
         lib.mlel_graph_op_count.argtypes = [_V]
         lib.mlel_graph_op_name.argtypes = [_V, C.c_int, C.c_char_p, C.c_size_t]
         lib.mlel_graph_session_tensor_count.argtypes = [_V]
@@ -253,6 +257,21 @@ class Graph:
         ms = (C.c_float * max(1, n))()
         self._check(self.lib.mlel_graph_dispatch_profiled(self.g, self.dev.stream, ms, n))
         return [(self.op_name(i), float(ms[i])) for i in range(n)]
+
+    def set_profiling(self, enabled):
+        """Every dispatch() records per-operator times (a new graph starts from VMEL_GRAPH_PROFILING)."""
+        self._check(self.lib.mlel_graph_set_profiling(self.g, 1 if enabled else 0))
+
+    def profiling(self):
+        return bool(self._check(self.lib.mlel_graph_get_profiling(self.g)))
+
+    def profiling_report(self):
+        """The profiler's report ("samples", "by_operator") as a dict."""
+        import json
+        need = self._check(self.lib.mlel_graph_profiling_json(self.g, None, 0))
+        buf = C.create_string_buffer(int(need))
+        self._check(self.lib.mlel_graph_profiling_json(self.g, buf, need))
+        return json.loads(buf.value.decode())
 
     def op_count(self):
         return self._check(self.lib.mlel_graph_op_count(self.g))

@@ -98,6 +98,14 @@ int mlel_graph_dispatch(mlel_graph *g, void *stream);
 /* Dispatch with a pair of events around every operator; per-operator milliseconds are written to `ms`
  * (reference: the profiler's timestamp pairs, graph/graph_profiler.cpp:157-191).  Returns the operator count. */
 int mlel_graph_dispatch_profiled(mlel_graph *g, void *stream, float *ms, int capacity);
+/* Per-operator profiling of every mlel_graph_dispatch (reference: GraphProfiler, enabled by the environment variable
+ * VMEL_GRAPH_PROFILING, graph/graph_profiler.cpp:107; a new graph takes its default from the same variable).  A
+ * profiled dispatch waits for its own events.  mlel_graph_profiling_json writes the report of
+ * graph/graph_profiler.cpp:563-625 ("samples", "by_operator"; no cycle counts: times come from event pairs) into
+ * `buf` (truncated to `capacity`) and returns the number of bytes the whole text needs, or a negative status. */
+int mlel_graph_set_profiling(mlel_graph *g, int enabled);
+int mlel_graph_get_profiling(mlel_graph *g);
+int64_t mlel_graph_profiling_json(mlel_graph *g, char *buf, size_t capacity);
 
 /* Introspection (tests, profiler). */
 int mlel_graph_op_count(mlel_graph *g);        /* operators executed after fusion */

@@ -249,3 +249,21 @@ def test_best_fit_allocation_rules():
     assert by_size[512] == by_size[1024]                     # c: only a is dead when c is produced
     assert by_size[256] == by_size[4096]                     # d: a's block holds c (alive), b's block is free
     g.close()
+
+
+def test_profiling_switch_from_environment(monkeypatch):
+    """VMEL_GRAPH_PROFILING as the reference reads it (graph/graph_profiler.cpp:29-38, 107): unset, empty, 0, false, off
+    and no (any case) leave profiling off, anything else turns it on; the report of an idle graph is empty."""
+    for value, expect in (("1", True), ("true", True), ("yes", True), ("anything", True), ("0", False), ("FALSE", False),
+                          ("Off", False), ("no", False), ("", False)):
+        monkeypatch.setenv("VMEL_GRAPH_PROFILING", value)
+        g = gb.Graph(_NoDevice())
+        assert g.profiling() is expect, value
+        g.close()
+    monkeypatch.delenv("VMEL_GRAPH_PROFILING")
+    g = gb.Graph(_NoDevice())
+    assert g.profiling() is False
+    g.set_profiling(True)
+    assert g.profiling() is True
+    assert g.profiling_report() == {"timestamp_period_ns": None, "samples": [], "by_operator": []}
+    g.close()

@@ -151,3 +151,32 @@ def test_graphs_under_the_other_memory_planners(dev, oracle, planner, monkeypatc
     out = g.get_output("output")
     g.close()
     assert np.max(np.abs(out.astype(np.float32) - exp["output"].astype(np.float32))) <= 1e-2
+
+
+def test_profiling_report_per_operator(dev, oracle):
+    """Two profiled dispatches: one sample per executed operator and dispatch, aggregates per operator name as in the
+    reference's report (graph/graph_profiler.cpp:563-625), results unchanged by profiling."""
+    spec = graphs.inverted_residual_spec(batch=2, hw=14, spread=True)
+    x = random_input(spec, 21)
+    exp, _ = run_spec(oracle, spec, {"input": x})
+    g = graphs.build(dev, spec, fuse=True)
+    g.set_input("input", x)
+    g.dispatch()
+    assert g.profiling_report()["samples"] == []  # profiling is off by default
+    g.set_profiling(True)
+    g.dispatch()
+    g.dispatch()
+    np.testing.assert_array_equal(g.get_output("output"), exp["output"])
+    report = g.profiling_report()
+    names = g.op_names()
+    assert [(s["graph_dispatch"], s["pipeline_index"], s["operator_name"]) for s in report["samples"]] == \
+        [(d, i, n) for d in (0, 1) for i, n in enumerate(names)]
+    assert all(s["pipeline_kind"] == "tosa" and s["time_ms"] > 0 for s in report["samples"])
+    by = {a["operator_name"]: a for a in report["by_operator"]}
+    assert set(by) == set(names)
+    for name, a in by.items():
+        times = [s["time_ms"] for s in report["samples"] if s["operator_name"] == name]
+        assert a["dispatch_count"] == len(times)
+        assert abs(a["total_time_ms"] - sum(times)) < 1e-6 and abs(a["average_time_ms"] - sum(times) / len(times)) < 1e-6
+        assert abs(a["min_time_ms"] - min(times)) < 1e-6 and abs(a["max_time_ms"] - max(times)) < 1e-6
+    g.close()
