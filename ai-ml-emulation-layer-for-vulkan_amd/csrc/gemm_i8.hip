@@ -39,7 +39,10 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
             best = i;
         }
     }
-    const int BN = bn_opts[best];
+    int BN = bn_opts[best];
+    // a problem of very few rows (a fully connected layer over a small batch): narrower tiles on a tie, so that the
+    // K loop of a handful of blocks is shared by four times as many
+    if (BN == 128 && g.M <= 64 && (int64_t)((g.N + 127) / 128) * g.batches < 32 && (g.N + 31) / 32 * 32 == best_pad) BN = 32;
     // Two tile heights per width: the tall one when there are enough tiles to give every compute unit at least two
     // blocks, otherwise the short one, so that small problems still spread over the machine and several independent
     // blocks per compute unit hide each other's LDS and barrier latency.
