@@ -26,8 +26,6 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4s lds_v4s;
 
 constexpr int NT = 256;
-constexpr int BKH = 32;          // halfs of K per step
-constexpr int XPITCH = 64 + 16;  // bytes per A row in LDS
 constexpr uint32_t kOob = 0x80000000u;
 
 struct HGemmArgs {
@@ -51,11 +49,15 @@ __device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t r, uint32_t off) 
     return make_uint4((uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+// BKH: halfs of K per step (32, or 64 for long contractions: half as many barriers and LDS round trips per K)
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int BKH>
 __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
-    constexpr int XROWS = BM / 64;            // 16-byte pieces of A per thread and step
+    constexpr int XPITCH = BKH * 2 + 16;      // bytes per A row in LDS
+    constexpr int XP16 = BKH / 8;             // 16-byte pieces per A row
+    constexpr int XPASS = NT / XP16;          // A rows covered by one pass of the block
+    constexpr int XROWS = BM / XPASS;         // 16-byte pieces of A per thread and step
     constexpr int WPITCH = 2 * BN + 32;       // bytes per K row of the B tile: 4 rows x 32 B land on distinct banks
     constexpr int WROW16 = BN / 8;            // 16-byte pieces per K row
     constexpr int WCHUNKS = (BKH * WROW16) / NT;
@@ -82,8 +84,8 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
     uint32_t xoff[XROWS], woff[WCHUNKS];
 #pragma unroll
     for (int i = 0; i < XROWS; i++) {
-        const int m = m_base + (tid >> 2) + 64 * i;
-        xoff[i] = m < g.M ? (uint32_t)m * g.lda + (tid & 3) * 16 : kOob;
+        const int m = m_base + tid / XP16 + XPASS * i;
+        xoff[i] = m < g.M ? (uint32_t)m * g.lda + (tid % XP16) * 16 : kOob;
     }
 #pragma unroll
     for (int i = 0; i < WCHUNKS; i++) {
@@ -92,7 +94,7 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
         woff[i] = n < g.N ? (uint32_t)(c / WROW16) * g.ldb + (uint32_t)n * 2 : kOob;
     }
     auto prefetch = [&](int k0, uint4 (&xr)[XROWS], uint4 (&wr)[WCHUNKS]) {
-        const bool kin = k0 + (tid & 3) * 8 < g.K;  // K % 8 == 0: a piece lies wholly inside or outside
+        const bool kin = k0 + (tid % XP16) * 8 < g.K;  // K % 8 == 0: a piece lies wholly inside or outside
 #pragma unroll
         for (int i = 0; i < XROWS; i++) xr[i] = load16(ares, (kin && xoff[i] != kOob) ? xoff[i] + (uint32_t)k0 * 2 : kOob);
 #pragma unroll
@@ -104,7 +106,7 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
     auto stage = [&](int buf, const uint4 (&xr)[XROWS], const uint4 (&wr)[WCHUNKS]) {
 #pragma unroll
         for (int i = 0; i < XROWS; i++)
-            *reinterpret_cast<uint4 *>(xs + buf * XBUF + ((tid >> 2) + 64 * i) * XPITCH + (tid & 3) * 16) = xr[i];
+            *reinterpret_cast<uint4 *>(xs + buf * XBUF + (tid / XP16 + XPASS * i) * XPITCH + (tid % XP16) * 16) = xr[i];
 #pragma unroll
         for (int i = 0; i < WCHUNKS; i++) {
             const int c = tid + NT * i;
@@ -130,7 +132,7 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
         const char *xt = xs + buf * XBUF;
         const char *wt = ws + buf * WBUF;
 #pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
+        for (int kk = 0; kk < BKH / 16; kk++) {
             v8h af[TM], bf[TN];
 #pragma unroll
             for (int i = 0; i < TM; i++)
@@ -157,7 +159,7 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
     };
 
     // ring of DEPTH register sets: DEPTH - 1 steps of global loads in flight while one step is multiplied
-    constexpr int DEPTH = 4;
+    constexpr int DEPTH = BKH == 32 ? 4 : 3;
     const int nk = (g.K + BKH - 1) / BKH;
     uint4 xr[DEPTH][XROWS], wr[DEPTH][WCHUNKS];
 #pragma unroll
@@ -168,9 +170,10 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
             if (step + d < nk) {  // uniform
+                const int cur = (step + d) & 1;  // LDS buffer of this step
                 prefetch((step + d + DEPTH) * BKH, xr[d], wr[d]);
-                compute(d & 1);
-                stage((d + 1) & 1, xr[(d + 1) % DEPTH], wr[(d + 1) % DEPTH]);
+                compute(cur);
+                stage(cur ^ 1, xr[(d + 1) % DEPTH], wr[(d + 1) % DEPTH]);
                 __syncthreads();
             }
         }
@@ -178,6 +181,20 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
 
     // ---- store: lane holds row m = lane % 32 of each sub-tile and, per register quad q, columns 8q + 4 * (lane / 32)
     const __amdgpu_buffer_rsrc_t ores = rsrc(g.out + (int64_t)batch * g.o_batch, g.o_bytes);
+    // the bias of this lane's columns, fetched in one batch before any store (a load after a store would have to
+    // wait for it: the compiler cannot tell that the two do not alias)
+    float bias_r[TN][4][4];
+    if (EPI == 1) {
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int n0 = n_base + wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    bias_r[j][q][e] = (g.bias != nullptr && n0 < g.N) ? g.bias[g.bias_len == 1 ? 0 : n0 + e] : 0.f;
+            }
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
@@ -199,15 +216,10 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
                     // ADD in fp32 (one rounding), then CAST to fp16 (round to nearest even): the two operators that
                     // follow the MATMUL in the unfused graph
                     const uint32_t off = (row_off != kOob && n0 < g.N) ? row_off + (uint32_t)n0 * 2 : kOob;
-                    float b4[4] = {0.f, 0.f, 0.f, 0.f};
-                    if (g.bias != nullptr && n0 < g.N) {
-#pragma unroll
-                        for (int e = 0; e < 4; e++) b4[e] = g.bias[g.bias_len == 1 ? 0 : n0 + e];
-                    }
                     _Float16 h[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const float sum = g.bias != nullptr ? acc[i][j][4 * q + e] + b4[e] : acc[i][j][4 * q + e];
+                        const float sum = g.bias != nullptr ? acc[i][j][4 * q + e] + bias_r[j][q][e] : acc[i][j][4 * q + e];
                         h[e] = (_Float16)sum;
                     }
                     typedef int v2i_t __attribute__((ext_vector_type(2)));
@@ -221,13 +233,31 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
     }
 }
 
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKH>
+void launch_k(const HGemmArgs &g, bool cast_epilogue, dim3 grid, hipStream_t s) {
+    constexpr size_t sm = (size_t)2 * BM * (BKH * 2 + 16) + (size_t)2 * BKH * (2 * BN + 32);
+    // above the default dynamic shared-memory limit the limit is raised once per kernel (thread-safe static)
+    if (cast_epilogue) {
+        auto kernel = gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 1, BKH>;
+        static const bool raised = sm <= 48 * 1024 || hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm) == hipSuccess;
+        (void)raised;
+        kernel<<<grid, dim3(NT), sm, s>>>(g);
+    } else {
+        auto kernel = gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 0, BKH>;
+        static const bool raised = sm <= 48 * 1024 || hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm) == hipSuccess;
+        (void)raised;
+        kernel<<<grid, dim3(NT), sm, s>>>(g);
+    }
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 void launch(const HGemmArgs &g, bool cast_epilogue, dim3 grid, hipStream_t s) {
-    constexpr size_t sm = (size_t)2 * BM * XPITCH + (size_t)2 * BKH * (2 * BN + 32);
-    if (cast_epilogue)
-        gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 1><<<grid, dim3(NT), sm, s>>>(g);
+    if (g.K >= 256)
+        launch_k<BM, BN, WAVES_M, WAVES_N, 64>(g, cast_epilogue, grid, s);
     else
-        gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 0><<<grid, dim3(NT), sm, s>>>(g);
+        launch_k<BM, BN, WAVES_M, WAVES_N, 32>(g, cast_epilogue, grid, s);
 }
 
 bool dense_rows(const mlel_tensor *t) { return t->strides[2] == 2 && t->strides[1] >= t->dims[2] * 2; }
