@@ -635,6 +635,40 @@ int mlel_hip_elementwise_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *o
     return 0;
 }
 
+int mlel_hip_softmax_rows(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in) {
+    MLEL_TRY(require_ctx(ctx, "softmax_rows"));
+    MLEL_TRY(check_supported(out, "softmax_rows out"));
+    MLEL_TRY(check_supported(in, "softmax_rows in"));
+    MLEL_REQUIRE(in->rank >= 1 && same_shape(out, in) && in->dtype == out->dtype && dt_is_float(in->dtype), MLEL_ERR_INVALID,
+                 "softmax_rows: input and output must be floating-point tensors of one shape and type");
+    const int rc = try_softmax_rows_f16(ctx, (hipStream_t)stream, out, in);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    // no one-pass kernel for this type or layout: the six operators one after another through temporaries
+    const int last = in->rank - 1;
+    mlel_tensor row = packed_like(in, in->dtype, nullptr);
+    row.dims[last] = 1;
+    row = packed_like(&row, in->dtype, nullptr);
+    Scratch t_max, t_diff, t_exp, t_sum, t_rcp;
+    const size_t full = (size_t)numel(in) * dt_size(in->dtype) + 16, small = (size_t)numel(&row) * dt_size(in->dtype) + 16;
+    MLEL_HIP_CHECK(hipMalloc(&t_max.ptr, small));
+    MLEL_HIP_CHECK(hipMalloc(&t_diff.ptr, full));
+    MLEL_HIP_CHECK(hipMalloc(&t_exp.ptr, full));
+    MLEL_HIP_CHECK(hipMalloc(&t_sum.ptr, small));
+    MLEL_HIP_CHECK(hipMalloc(&t_rcp.ptr, small));
+    mlel_tensor mx = row, sum = row, rcp = row, diff = packed_like(in, in->dtype, t_diff.ptr), ex = packed_like(in, in->dtype, t_exp.ptr);
+    mx.ptr = t_max.ptr;
+    sum.ptr = t_sum.ptr;
+    rcp.ptr = t_rcp.ptr;
+    MLEL_TRY(mlel_hip_reduce(ctx, stream, MLEL_RED_MAX, &mx, in, (uint32_t)last, MLEL_NAN_PROPAGATE));
+    MLEL_TRY(mlel_hip_elementwise_binary(ctx, stream, MLEL_BIN_SUB, &diff, in, &mx, MLEL_NAN_PROPAGATE));
+    MLEL_TRY(mlel_hip_elementwise_unary(ctx, stream, MLEL_UN_EXP, &ex, &diff));
+    MLEL_TRY(mlel_hip_reduce(ctx, stream, MLEL_RED_SUM, &sum, &ex, (uint32_t)last, MLEL_NAN_PROPAGATE));
+    MLEL_TRY(mlel_hip_elementwise_unary(ctx, stream, MLEL_UN_RECIPROCAL, &rcp, &sum));
+    MLEL_TRY(mlel_hip_mul(ctx, stream, out, &ex, &rcp, 0));
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
 int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                               const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr) {
     MLEL_TRY(require_ctx(ctx, "matmul_bias_cast"));

@@ -116,6 +116,8 @@ int try_unary_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor
 int try_cast_float_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in);
 int try_reduce_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in,
                           uint32_t axis, uint32_t nan_mode);
+// REDUCE_MAX, SUB, EXP, REDUCE_SUM, RECIPROCAL, MUL over the last axis in one pass (fp16)
+int try_softmax_rows_f16(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in);
 
 // ---- bandwidth-bound specialisations (ops_fast.hip) ----
 int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,

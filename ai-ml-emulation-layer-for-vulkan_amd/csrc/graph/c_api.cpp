@@ -277,6 +277,7 @@ std::string opLabel(const OpNode &op) {
     case OpKind::FusedConv2D: return std::string("CONV2D+RESCALE") + (op.hasClamp ? "+CLAMP" : "");
     case OpKind::FusedDepthwiseConv2D: return std::string("DEPTHWISE_CONV2D+RESCALE") + (op.hasClamp ? "+CLAMP" : "");
     case OpKind::FusedMatmul: return std::string("MATMUL+RESCALE") + (op.hasClamp ? "+CLAMP" : "");
+    case OpKind::FusedSoftmax: return "REDUCE_MAX+SUB+EXP+REDUCE_SUM+RECIPROCAL+MUL";
     case OpKind::FusedRescaleAddRescale: return "RESCALE+RESCALE+ADD+RESCALE";
     case OpKind::FusedConv2DResidual:
         return std::string("CONV2D+RESCALE") + (op.hasClamp ? "+CLAMP" : "") + "+RESCALE+RESCALE+ADD+RESCALE";

@@ -760,6 +760,60 @@ void GraphPipeline::fuse() {
         if (add) add->fusedAway = true;
     }
 
+    // Pattern 4b (softmax over the last axis, fp16): REDUCE_MAX -> SUB -> EXP -> REDUCE_SUM -> RECIPROCAL -> MUL with
+    // every intermediate private and read only inside the pattern becomes one pass over the rows
+    // (mlel_hip_softmax_rows), which rounds after every operator like the operators it replaces.
+    for (const auto &opPtr : ops) {
+        OpNode &rmax = *opPtr;
+        if (rmax.fusedAway || rmax.kind != OpKind::Reduce || rmax.selector != MLEL_RED_MAX ||
+            rmax.nanMode != MLEL_NAN_PROPAGATE)
+            continue;
+        const TensorPtr x = rmax.inputs[0], m = rmax.outputs[0];
+        const uint32_t last = static_cast<uint32_t>(x->getRank()) - 1;
+        if (x->getFormat() != MLEL_F16 || x->getRank() < 1 || rmax.axis != last || !x->isPacked() || !isPrivateIntermediate(*m))
+            continue;
+        const auto only = [&](const TensorPtr &t) -> OpNode * {
+            const auto users = consumersOf(ops, t.get());
+            return users.size() == 1 && !users[0]->fusedAway ? users[0] : nullptr;
+        };
+        const auto fullHalf = [&](const TensorPtr &t) {
+            return t->getFormat() == MLEL_F16 && sameShape(*t, *x) && t->isPacked();
+        };
+        OpNode *sub = only(m);
+        if (!sub || sub->kind != OpKind::Binary || sub->selector != MLEL_BIN_SUB || sub->inputs[0].get() != x.get() ||
+            sub->inputs[1].get() != m.get() || !fullHalf(sub->outputs[0]) || !isPrivateIntermediate(*sub->outputs[0]))
+            continue;
+        OpNode *ex = only(sub->outputs[0]);
+        if (!ex || ex->kind != OpKind::Unary || ex->selector != MLEL_UN_EXP || !fullHalf(ex->outputs[0]) ||
+            !isPrivateIntermediate(*ex->outputs[0]))
+            continue;
+        const TensorPtr e = ex->outputs[0];
+        const auto eUsers = consumersOf(ops, e.get());
+        if (eUsers.size() != 2) continue;
+        OpNode *rsum = nullptr, *mul = nullptr;
+        for (OpNode *u : eUsers) {
+            if (u->kind == OpKind::Reduce) rsum = u;
+            if (u->kind == OpKind::Mul) mul = u;
+        }
+        if (!rsum || !mul || rsum->fusedAway || mul->fusedAway || rsum->selector != MLEL_RED_SUM || rsum->axis != last ||
+            rsum->nanMode != MLEL_NAN_PROPAGATE || rsum->inputs[0].get() != e.get() ||
+            rsum->outputs[0]->getFormat() != MLEL_F16 || !isPrivateIntermediate(*rsum->outputs[0]))
+            continue;
+        OpNode *rcp = only(rsum->outputs[0]);
+        if (!rcp || rcp->kind != OpKind::Unary || rcp->selector != MLEL_UN_RECIPROCAL ||
+            rcp->outputs[0]->getFormat() != MLEL_F16 || !isPrivateIntermediate(*rcp->outputs[0]) ||
+            only(rcp->outputs[0]) != mul)
+            continue;
+        const TensorPtr r = rcp->outputs[0];
+        const bool operands = (mul->inputs[0].get() == e.get() && mul->inputs[1].get() == r.get()) ||
+                              (mul->inputs[1].get() == e.get() && mul->inputs[0].get() == r.get());
+        if (!operands || mul->shift != 0 || !fullHalf(mul->outputs[0])) continue;
+        rmax.kind = OpKind::FusedSoftmax;
+        rmax.outputs[0] = mul->outputs[0];
+        mul->outputs[0]->setProducer(&rmax);
+        sub->fusedAway = ex->fusedAway = rsum->fusedAway = rcp->fusedAway = mul->fusedAway = true;
+    }
+
     // Pattern 5: regions of floating-point elementwise operators (ADD, SUB, MUL, EXP, RECIPROCAL, RSQRT, TANH, CAST
     // between fp16 and fp32) collapse into one pass.  A region grows backwards from an operator whose result is needed
     // elsewhere: a producer is absorbed when it is elementwise too, has the region's shape, and its result is a
@@ -1173,6 +1227,7 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
         rc = mlel_hip_elementwise_chain(ctx, stream, &out, &c);
         break;
     }
+    case OpKind::FusedSoftmax: rc = mlel_hip_softmax_rows(ctx, stream, &out, &in[0]); break;
     case OpKind::FusedMatmulBiasCast:
         rc = mlel_hip_matmul_bias_cast(ctx, stream, &out, &in[0], &in[1], op.inputs.size() > 2 ? &in[2] : nullptr,
                                        &op.matmul);

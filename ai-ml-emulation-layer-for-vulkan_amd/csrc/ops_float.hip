@@ -545,6 +545,152 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArg
     if (tid < 64 && row < g.rows) *reinterpret_cast<__half *>(g.out + row * 2) = f2h(r);
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// The softmax operator sequence of a TOSA graph over the last axis of a dense fp16 tensor, in one pass:
+//   m = REDUCE_MAX(x);  d = SUB(x, m);  e = EXP(d);  s = REDUCE_SUM(e);  r = RECIPROCAL(s);  out = MUL(e, r)
+// with every intermediate rounded to fp16 exactly where the stand-alone operators round it (the same device
+// functions, the same order), the maximum taken pairwise (its order is free) and the sum folded left to right in
+// fp16 as reduce.comp:24-70 prescribes.  A block owns 64 rows held in shared memory: all four wavefronts fetch the
+// rows and take the maxima (four threads per row), overwrite the rows with e, then the first wavefront folds one row
+// per lane, and all four scale and store.  Rows that hold a NaN take the element-by-element path of the stand-alone
+// kernels (first NaN wins in both reductions).
+// ---------------------------------------------------------------------------------------------------------------
+struct SoftmaxArgs {
+    const char *in;
+    char *out;
+    int64_t rows;
+    int32_t cols;  // multiple of 8, at most kSoftmaxMaxCols
+};
+constexpr int kSoftmaxMaxCols = 1024;
+
+__global__ void __launch_bounds__(kBlock) softmax_rows_f16_kernel(const SoftmaxArgs g) {
+    extern __shared__ __align__(16) char slab[];
+    const int pitch = g.cols * 2 + 16;
+    __half *row_scale = reinterpret_cast<__half *>(slab + 64 * pitch);  // [64] maximum, later the reciprocal
+    const int tid = threadIdx.x;
+    const int64_t row0 = (int64_t)blockIdx.x * 64;
+    const int segs = g.cols >> 3, pieces = 64 * segs;
+    // ---- fetch: consecutive threads take consecutive 16-byte pieces of a row
+    for (int p0 = 0; p0 < pieces; p0 += kBlock * 8) {
+        uint4 v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int p = p0 + i * kBlock + tid;
+            const int rr = p / segs, seg = p - rr * segs;
+            v[i] = make_uint4(0, 0, 0, 0);
+            if (p < pieces && row0 + rr < g.rows)
+                v[i] = *reinterpret_cast<const uint4 *>(g.in + ((row0 + rr) * g.cols + seg * 8) * 2);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int p = p0 + i * kBlock + tid;
+            const int rr = p / segs, seg = p - rr * segs;
+            if (p < pieces) *reinterpret_cast<uint4 *>(slab + rr * pitch + seg * 16) = v[i];
+        }
+    }
+    __syncthreads();
+    // ---- maximum: four threads per row, pieces interleaved; a NaN anywhere sends the row to the careful path
+    const int r = tid >> 2, part = tid & 3;
+    char *mine = slab + r * pitch;
+    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+    h2_t m2 = {(_Float16)-65504.f, (_Float16)-65504.f};
+    uint32_t special = 0;
+    for (int sg = part; sg < segs; sg += 4) {
+        const uint4 raw = *reinterpret_cast<const uint4 *>(mine + sg * 16);
+        special |= (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu) |
+                    ((raw.z & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
+        const h2_t *p = reinterpret_cast<const h2_t *>(&raw);
+        m2 = __builtin_elementwise_max(m2, __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]),
+                                                                       __builtin_elementwise_max(p[2], p[3])));
+    }
+    float mx = (float)(m2.x > m2.y ? m2.x : m2.y);
+    mx = fmaxf(mx, __shfl_xor(mx, 1));
+    mx = fmaxf(mx, __shfl_xor(mx, 2));
+    special |= (uint32_t)__shfl_xor((int)special, 1);
+    special |= (uint32_t)__shfl_xor((int)special, 2);
+    if (special != 0) {  // REDUCE_MAX as the stand-alone kernel folds a row with a NaN: the first NaN is the result
+        mx = -65504.f;
+        for (int j = 0; j < g.cols; j++) {
+            const float v = __half2float(*reinterpret_cast<const __half *>(mine + j * 2));
+            if (isnan(v)) {
+                mx = v;
+                break;
+            }
+            mx = mx < v ? v : mx;
+        }
+    }
+    // ---- e = EXP(SUB(x, m)), rounded to fp16 after each of the two operators, written over the row
+    for (int sg = part; sg < segs; sg += 4) {
+        uint4 raw = *reinterpret_cast<const uint4 *>(mine + sg * 16);
+        __half2 *h = reinterpret_cast<__half2 *>(&raw);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const float2 f = __half22float2(h[t]);
+            const float d0 = __half2float(f2h(f.x - mx)), d1 = __half2float(f2h(f.y - mx));
+            h[t] = __halves2half2(f2h(op_exp<true>(d0)), f2h(op_exp<true>(d1)));
+        }
+        *reinterpret_cast<uint4 *>(mine + sg * 16) = raw;
+    }
+    __syncthreads();
+    // ---- s = REDUCE_SUM(e) left to right in fp16, r = RECIPROCAL(s): one row per lane of the first wavefront
+    if (tid < 64) {
+        const char *row = slab + tid * pitch;
+        float acc_f = 0.f;
+        bool done = false;
+        for (int j = 0; j < g.cols; j += 8) {
+            const uint4 raw = *reinterpret_cast<const uint4 *>(row + j * 2);
+            const uint32_t nan_bits =
+                (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu) |
+                 ((raw.z & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
+            const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+            if (!__any(done || nan_bits != 0)) {
+                __half acc = f2h(acc_f);
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    acc = __hadd(acc, __low2half(h[t]));
+                    acc = __hadd(acc, __high2half(h[t]));
+                }
+                acc_f = __half2float(acc);
+                continue;
+            }
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const float2 f = __half22float2(h[t]);
+                const float e2[2] = {f.x, f.y};
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    if (done) continue;
+                    if (isnan(e2[u])) {
+                        acc_f = e2[u];
+                        done = true;
+                        continue;
+                    }
+                    acc_f = rnd_f16(acc_f + e2[u]);
+                }
+            }
+        }
+        row_scale[tid] = f2h(op_reciprocal<true>(__half2float(f2h(acc_f))));
+    }
+    __syncthreads();
+    // ---- out = MUL(e, r), rounded once; stored with the fetch's piece order
+    for (int p0 = 0; p0 < pieces; p0 += kBlock) {
+        const int p = p0 + tid;
+        if (p >= pieces) break;
+        const int rr = p / segs, seg = p - rr * segs;
+        if (row0 + rr >= g.rows) continue;
+        const float scale = __half2float(row_scale[rr]);
+        uint4 raw = *reinterpret_cast<const uint4 *>(slab + rr * pitch + seg * 16);
+        __half2 *h = reinterpret_cast<__half2 *>(&raw);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const float2 f = __half22float2(h[t]);
+            h[t] = __halves2half2(f2h(f.x * scale), f2h(f.y * scale));
+        }
+        *reinterpret_cast<uint4 *>(g.out + ((row0 + rr) * g.cols + seg * 8) * 2) = raw;
+    }
+}
+
 }  // namespace
 
 // MLEL_ERR_UNSUPPORTED when the chain does not fit the kernel (types, shapes, alignment, live values): the caller
@@ -690,6 +836,32 @@ int try_reduce_float_fast(mlel_ctx *, hipStream_t s, int op, const mlel_tensor *
                                   (int)smem);
     kernel<<<dim3((unsigned)blocks), dim3(kBlock), smem, s>>>(g);
     MLEL_TRY(check_launch("reduce rows fp16"));
+    return 1;
+}
+
+// Returns 1 when the one-pass kernel ran, 0 when the case is outside what it assumes (the caller then runs the six
+// operators one after another), < 0 on error.
+int try_softmax_rows_f16(mlel_ctx *, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in) {
+    if (in->dtype != MLEL_F16 || out->dtype != MLEL_F16 || in->rank < 1 || !same_shape(out, in)) return 0;
+    if (!is_packed(in) || !is_packed(out) || ((uintptr_t)in->ptr % 16) != 0 || ((uintptr_t)out->ptr % 16) != 0) return 0;
+    const int64_t cols = in->dims[in->rank - 1];
+    if (cols <= 0 || cols % 8 != 0 || cols > kSoftmaxMaxCols) return 0;
+    const int64_t rows = numel(in) / cols;
+    if (rows <= 0) return 1;
+    const int64_t blocks = (rows + 63) / 64;
+    if (blocks >= (int64_t(1) << 31)) return 0;
+    SoftmaxArgs g{};
+    g.in = static_cast<const char *>(in->ptr);
+    g.out = static_cast<char *>(out->ptr);
+    g.rows = rows;
+    g.cols = (int32_t)cols;
+    const size_t smem = (size_t)64 * (cols * 2 + 16) + 64 * 2;
+    static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(softmax_rows_f16_kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   64 * (kSoftmaxMaxCols * 2 + 16) + 128) == hipSuccess;
+    (void)raised;
+    softmax_rows_f16_kernel<<<dim3((unsigned)blocks), dim3(kBlock), smem, s>>>(g);
+    MLEL_TRY(check_launch("softmax rows fp16"));
     return 1;
 }
 

@@ -396,6 +396,11 @@ int mlel_hip_conv2d_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_
                                         int residual_first);
 int mlel_hip_matmul_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                             const mlel_tensor *b, const mlel_matmul_attr *attr, const mlel_epilogue *epi);
+/* The softmax operator sequence over the last axis in one pass:
+ *   m = REDUCE_MAX(in); d = SUB(in, m); e = EXP(d); s = REDUCE_SUM(e); r = RECIPROCAL(s); out = MUL(e, r)
+ * (NaN propagating reductions), every intermediate rounded to the tensors' type as the stand-alone operators round
+ * it: bit for bit the six operators run one after another. */
+int mlel_hip_softmax_rows(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in);
 /* out(fp16) = CAST( MATMUL(a, b) + bias ): fp16 operands, fp32 accumulation, the fp32 bias [1,1,N] or [1,1,1] (or
  * NULL) added in fp32, one rounding to fp16 -- bit for bit the unfused MATMUL -> ADD -> CAST (or MATMUL -> CAST). */
 int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,

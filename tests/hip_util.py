@@ -218,6 +218,14 @@ class Runner:
         self.done()
         return r
 
+    def softmax_rows(self, x):
+        tx = self.put(x)
+        to = self.new(tx.dtype, x.shape)
+        self.dev.op("softmax_rows", to.ref, tx.ref)
+        r = to.download()
+        self.done()
+        return r
+
     def matmul_bias_cast(self, a, b, bias):
         ta, tb = self.put(a), self.put(b)
         tbias = self.put(bias) if bias is not None else None

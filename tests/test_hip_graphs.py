@@ -180,3 +180,20 @@ def test_profiling_report_per_operator(dev, oracle):
         assert abs(a["total_time_ms"] - sum(times)) < 1e-6 and abs(a["average_time_ms"] - sum(times) / len(times)) < 1e-6
         assert abs(a["min_time_ms"] - min(times)) < 1e-6 and abs(a["max_time_ms"] - max(times)) < 1e-6
     g.close()
+
+
+def test_transformer_block_fusions_do_not_change_a_bit(dev):
+    """The fp16 fusions (MATMUL+ADD+CAST epilogue, elementwise regions, the softmax sequence) against the same graph
+    run operator by operator on the GPU: identical bits; the fused list holds the softmax as one operator."""
+    spec = graphs.transformer_block_spec(batch=2, seq=64, d_model=64, heads=4, ffn=128)
+    x = np.random.default_rng(5).standard_normal(spec.inputs[0][2]).astype(np.float16)
+    outs = {}
+    for fuse in (False, True):
+        g = graphs.build(dev, spec, fuse=fuse)
+        g.set_input("input", x)
+        g.dispatch()
+        outs[fuse] = (g.get_output("output"), g.op_names())
+        g.close()
+    np.testing.assert_array_equal(outs[True][0].view(np.uint16), outs[False][0].view(np.uint16))
+    assert outs[True][1].count("REDUCE_MAX+SUB+EXP+REDUCE_SUM+RECIPROCAL+MUL") == 1
+    assert "REDUCE_MAX" not in outs[True][1] and len(outs[True][1]) < len(outs[False][1])

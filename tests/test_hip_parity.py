@@ -734,3 +734,41 @@ def test_fp16_products_keep_the_sign_of_zero(run, oracle):
     rows = np.array([[-0.0, 1.0, 2.0], [-6e-8, 6e-8, 1.0], [1.0, -1.0, 0.0]], np.float16)
     np.testing.assert_array_equal(run.reduce("PRODUCT", rows, 1).view(np.uint16),
                                   oracle.reduce("PRODUCT", rows, 1).view(np.uint16))
+
+
+@pytest.mark.parametrize("shape", [(3, 70, 512), (2, 5, 7, 64), (130, 1024), (4, 8)], ids=str)
+def test_softmax_rows_equals_the_six_operators(run, shape):
+    """REDUCE_MAX, SUB, EXP, REDUCE_SUM, RECIPROCAL, MUL in one pass == the six stand-alone kernels, bit for bit, on
+    ordinary rows and on rows with NaN, infinities, signed zeros and a constant row.  Where the result is NaN only
+    NaN-ness is compared: a product of two NaNs takes the sign of whichever operand the compiler put first, and the
+    reference's shading language leaves the sign and payload of a NaN unspecified."""
+    rng = np.random.default_rng(len(shape) * 1000 + shape[-1])
+    x = (rng.standard_normal(shape) * 3).astype(np.float16)
+    flat = x.reshape(-1, shape[-1])
+    flat[0, 3] = np.nan
+    flat[1, 0] = np.inf
+    flat[2, 1] = -np.inf
+    flat[3, :] = -0.0
+    flat[4 % len(flat), :] = 7.5
+    flat[5 % len(flat), 2:4] = [np.nan, -np.nan]
+    last = len(shape) - 1
+    m = run.reduce("MAX", x, last)
+    e = run.unary("EXP", run.binary("SUB", x, m, x.shape, abi.F16))
+    r = run.unary("RECIPROCAL", run.reduce("SUM", e, last))
+    want = run.mul(e, r, x.shape, abi.F16)
+    got = run.softmax_rows(x)
+    nan = np.isnan(want)
+    np.testing.assert_array_equal(np.isnan(got), nan)
+    np.testing.assert_array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+    ok = ~nan.any(axis=-1)
+    assert np.all(np.abs(got.astype(np.float32)[ok].sum(axis=-1) - 1.0) < 5e-2)  # fp16 sum of up to 1024 rounded terms
+
+
+def test_softmax_rows_falls_back_for_other_layouts(run):
+    """fp32 rows take the operator sequence behind the entry point (no one-pass kernel): same result as the operators"""
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((5, 33)).astype(np.float32)
+    m = run.reduce("MAX", x, 1)
+    e = run.unary("EXP", run.binary("SUB", x, m, x.shape, abi.F32))
+    want = run.mul(e, run.unary("RECIPROCAL", run.reduce("SUM", e, 1)), x.shape, abi.F32)
+    np.testing.assert_array_equal(run.softmax_rows(x).view(np.uint32), want.view(np.uint32))
