@@ -378,30 +378,60 @@ int mlel_graph_make_op(mlel_graph *g, const char *tosa_name, const int *inputs, 
     });
 }
 
+}  // extern "C"
+
+namespace {
+// shared tail of the two SPIR-V entry points: converts the argument arrays, runs `load`, reports the interface
+template <typename Load>
+int load_spirv_module(const mlel_graph_spv_binding *bindings, int n_bindings, const mlel_graph_spv_constant *constants,
+                      int n_constants, const mlel_graph_spv_specialization *specializations, int n_specializations,
+                      uint32_t *io, int io_capacity, int *n_inputs, int *n_outputs, const Load &load) {
+    std::vector<SpvBinding> b;
+    for (int i = 0; i < n_bindings; i++)
+        b.push_back({bindings[i].set, bindings[i].binding, bindings[i].array_index, vec64(bindings[i].dims, bindings[i].rank)});
+    std::vector<SpvConstant> c;
+    for (int i = 0; i < n_constants; i++)
+        c.push_back({constants[i].id, constants[i].data, vec64(constants[i].dims, constants[i].rank)});
+    std::vector<SpvSpecialization> sp;
+    for (int i = 0; i < n_specializations; i++) sp.push_back({specializations[i].spec_id, specializations[i].bits});
+    const SpvGraphInfo info = load(b, c, sp);
+    const size_t total = info.inputs.size() + info.outputs.size();
+    if (io && static_cast<size_t>(io_capacity) < 3 * total) throw std::runtime_error("io array too small");
+    size_t k = 0;
+    for (const auto *list : {&info.inputs, &info.outputs})
+        for (const auto &key : *list)
+            for (int j = 0; j < 3 && io; j++) io[k++] = key[static_cast<size_t>(j)];
+    if (n_inputs) *n_inputs = static_cast<int>(info.inputs.size());
+    if (n_outputs) *n_outputs = static_cast<int>(info.outputs.size());
+    return static_cast<int>(info.instructions);
+}
+}  // namespace
+
+extern "C" {
+
 int mlel_graph_load_spvasm(mlel_graph *g, const char *text, size_t length, const mlel_graph_spv_binding *bindings,
                            int n_bindings, const mlel_graph_spv_constant *constants, int n_constants,
                            const mlel_graph_spv_specialization *specializations, int n_specializations, uint32_t *io,
                            int io_capacity, int *n_inputs, int *n_outputs) {
     return guarded([&] {
         if (!text) throw std::runtime_error("null SPIR-V text");
-        std::vector<SpvBinding> b;
-        for (int i = 0; i < n_bindings; i++)
-            b.push_back({bindings[i].set, bindings[i].binding, bindings[i].array_index, vec64(bindings[i].dims, bindings[i].rank)});
-        std::vector<SpvConstant> c;
-        for (int i = 0; i < n_constants; i++)
-            c.push_back({constants[i].id, constants[i].data, vec64(constants[i].dims, constants[i].rank)});
-        std::vector<SpvSpecialization> sp;
-        for (int i = 0; i < n_specializations; i++) sp.push_back({specializations[i].spec_id, specializations[i].bits});
-        const SpvGraphInfo info = loadSpirvAssembly(g->pipeline, std::string(text, length), b, c, sp);
-        const size_t total = info.inputs.size() + info.outputs.size();
-        if (io && static_cast<size_t>(io_capacity) < 3 * total) throw std::runtime_error("io array too small");
-        size_t k = 0;
-        for (const auto *list : {&info.inputs, &info.outputs})
-            for (const auto &key : *list)
-                for (int j = 0; j < 3 && io; j++) io[k++] = key[static_cast<size_t>(j)];
-        if (n_inputs) *n_inputs = static_cast<int>(info.inputs.size());
-        if (n_outputs) *n_outputs = static_cast<int>(info.outputs.size());
-        return static_cast<int>(info.instructions);
+        return load_spirv_module(bindings, n_bindings, constants, n_constants, specializations, n_specializations, io,
+                                 io_capacity, n_inputs, n_outputs, [&](const auto &b, const auto &c, const auto &sp) {
+                                     return loadSpirvAssembly(g->pipeline, std::string(text, length), b, c, sp);
+                                 });
+    });
+}
+
+int mlel_graph_load_spirv(mlel_graph *g, const uint32_t *words, size_t n_words, const mlel_graph_spv_binding *bindings,
+                          int n_bindings, const mlel_graph_spv_constant *constants, int n_constants,
+                          const mlel_graph_spv_specialization *specializations, int n_specializations, uint32_t *io,
+                          int io_capacity, int *n_inputs, int *n_outputs) {
+    return guarded([&] {
+        if (!words) throw std::runtime_error("null SPIR-V module");
+        return load_spirv_module(bindings, n_bindings, constants, n_constants, specializations, n_specializations, io,
+                                 io_capacity, n_inputs, n_outputs, [&](const auto &b, const auto &c, const auto &sp) {
+                                     return loadSpirvBinary(g->pipeline, words, n_words, b, c, sp);
+                                 });
     });
 }
 

@@ -1,7 +1,8 @@
-// SPIR-V assembly text -> GraphPipeline (see spirv_graph_loader.hpp).
+// SPIR-V assembly text or binary words -> GraphPipeline (see spirv_graph_loader.hpp).
 #include "spirv_graph_loader.hpp"
 
 #include <cmath>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <functional>
@@ -17,11 +18,13 @@ struct Instruction {
     std::string result;                 // "%name" or empty
     std::string opcode;                 // "OpTypeInt", ...
     std::vector<std::string> operands;  // ids keep their '%'; string literals are stored without quotes
-    int line = 0;
+    int line = 0;                       // text: line number; binary: offset of the instruction's first word
+    bool binary = false;
 };
 
 [[noreturn]] void fail(const Instruction &inst, const std::string &what) {
-    throw std::runtime_error("SPIR-V graph, line " + std::to_string(inst.line) + " (" + inst.opcode + "): " + what);
+    throw std::runtime_error(std::string("SPIR-V graph, ") + (inst.binary ? "word " : "line ") + std::to_string(inst.line) +
+                             " (" + inst.opcode + "): " + what);
 }
 
 // ---- lexer: one instruction per line, ';' starts a comment, "..." is one operand
@@ -65,6 +68,207 @@ std::vector<Instruction> tokenize(const std::string &text) {
         }
         inst.opcode = words[first];
         inst.operands.assign(words.begin() + first + 1, words.end());
+        out.push_back(std::move(inst));
+    }
+    return out;
+}
+
+
+// ---- binary modules: the word stream is turned into the same instruction records the lexer above produces (ids as
+// "%<number>", enumerants the loader looks at by name, constants as raw words "!0x..."), so both forms share
+// everything after this point.
+//
+// Operand layouts, one character per operand after the optional result type and result id:
+//   i  one id                       I  ids up to the end of the instruction
+//   l  one literal word             L  literal words up to the end
+//   s  a nul-terminated string      c  the literal of OpConstant: one word, or two for 64-bit types (low word first)
+//   d  Decoration                   f  FPEncoding (optional)          x  TOSA instruction number
+struct OpcodeLayout {
+    uint16_t code;
+    const char *name;
+    bool hasType, hasResult;
+    const char *operands;
+};
+
+// Numbers as published in the SPIR-V specification and the SPV_ARM_tensors / SPV_ARM_graph /
+// SPV_EXT_replicated_composites extension texts.
+const OpcodeLayout kOpcodes[] = {
+    {5, "OpName", false, false, "is"},
+    {10, "OpExtension", false, false, "s"},
+    {11, "OpExtInstImport", false, true, "s"},
+    {12, "OpExtInst", true, true, "ixI"},
+    {14, "OpMemoryModel", false, false, "ll"},
+    {17, "OpCapability", false, false, "l"},
+    {19, "OpTypeVoid", false, true, ""},
+    {20, "OpTypeBool", false, true, ""},
+    {21, "OpTypeInt", false, true, "ll"},
+    {22, "OpTypeFloat", false, true, "lf"},
+    {23, "OpTypeVector", false, true, "il"},
+    {24, "OpTypeMatrix", false, true, "il"},
+    {28, "OpTypeArray", false, true, "ii"},
+    {29, "OpTypeRuntimeArray", false, true, "i"},
+    {30, "OpTypeStruct", false, true, "I"},
+    {32, "OpTypePointer", false, true, "li"},
+    {33, "OpTypeFunction", false, true, "I"},
+    {41, "OpConstantTrue", true, true, ""},
+    {42, "OpConstantFalse", true, true, ""},
+    {43, "OpConstant", true, true, "c"},
+    {44, "OpConstantComposite", true, true, "I"},
+    {46, "OpConstantNull", true, true, ""},
+    {48, "OpSpecConstantTrue", true, true, ""},
+    {49, "OpSpecConstantFalse", true, true, ""},
+    {50, "OpSpecConstant", true, true, "c"},
+    {51, "OpSpecConstantComposite", true, true, "I"},
+    {59, "OpVariable", true, true, "lI"},
+    {71, "OpDecorate", false, false, "idL"},
+    {81, "OpCompositeExtract", true, true, "iL"},
+    {4163, "OpTypeTensorARM", false, true, "I"},
+    {4181, "OpGraphConstantARM", true, true, "l"},
+    {4182, "OpGraphEntryPointARM", false, false, "isI"},
+    {4183, "OpGraphARM", true, true, ""},
+    {4184, "OpGraphInputARM", true, true, "I"},
+    {4185, "OpGraphSetOutputARM", false, false, "I"},
+    {4186, "OpGraphEndARM", false, false, ""},
+    {4190, "OpTypeGraphARM", false, true, "lI"},
+    {4461, "OpConstantCompositeReplicateEXT", true, true, "i"},
+    {4462, "OpSpecConstantCompositeReplicateEXT", true, true, "i"},
+};
+
+// "TOSA.001000.1" instruction numbers: the operators in the order of the TOSA 1.0 specification's chapters
+// (tensor operators, activations, elementwise binary, unary, ternary, comparison, reduction, data layout,
+// scatter / gather, image, type conversion), numbered from 0.  The reference reads them as the TOSA* enumerators
+// of the SPIRV-Headers package (graph/graph_tosa_1_0_ext_inst.cpp:43-110 maps those to the names below); that
+// package is not part of the reference's tree, so these numbers are restated from the published grammar.
+const char *const kTosaNames[] = {
+    "ARGMAX", "AVG_POOL2D", "CONV2D", "CONV3D", "DEPTHWISE_CONV2D", "FFT2D", "MATMUL", "MAX_POOL2D", "RFFT2D",
+    "TRANSPOSE_CONV2D", "CLAMP", "ERF", "SIGMOID", "TANH", "ADD", "ARITHMETIC_RIGHT_SHIFT", "BITWISE_AND",
+    "BITWISE_OR", "BITWISE_XOR", "INTDIV", "LOGICAL_AND", "LOGICAL_LEFT_SHIFT", "LOGICAL_RIGHT_SHIFT", "LOGICAL_OR",
+    "LOGICAL_XOR", "MAXIMUM", "MINIMUM", "MUL", "POW", "SUB", "TABLE", "ABS", "BITWISE_NOT", "CEIL", "CLZ", "COS",
+    "EXP", "FLOOR", "LOG", "LOGICAL_NOT", "NEGATE", "RECIPROCAL", "RSQRT", "SIN", "SELECT", "EQUAL", "GREATER",
+    "GREATER_EQUAL", "REDUCE_ALL", "REDUCE_ANY", "REDUCE_MAX", "REDUCE_MIN", "REDUCE_PRODUCT", "REDUCE_SUM", "CONCAT",
+    "PAD", "RESHAPE", "REVERSE", "SLICE", "TILE", "TRANSPOSE", "GATHER", "SCATTER", "RESIZE", "CAST", "RESCALE"};
+
+constexpr uint32_t kSpirvMagic = 0x07230203u;
+
+std::vector<Instruction> decodeWords(const uint32_t *stream, const size_t count) {
+    if (!stream || count < 5) throw std::runtime_error("SPIR-V graph: a binary module has at least a five-word header");
+    std::vector<uint32_t> words(stream, stream + count);
+    const auto swap = [](const uint32_t w) { return (w >> 24) | ((w >> 8) & 0xff00u) | ((w << 8) & 0xff0000u) | (w << 24); };
+    if (words[0] == swap(kSpirvMagic))  // written on a machine of the other byte order
+        for (auto &w : words) w = swap(w);
+    if (words[0] != kSpirvMagic) throw std::runtime_error("SPIR-V graph: the first word is not the SPIR-V magic number");
+    std::map<uint32_t, const OpcodeLayout *> layouts;
+    for (const auto &l : kOpcodes) layouts[l.code] = &l;
+    std::map<uint32_t, int> scalarWidth;  // result id of OpTypeInt / OpTypeFloat -> width in bits
+    uint32_t tosaSet = 0;
+    const auto hex = [](const uint64_t v) {
+        char buf[24];
+        std::snprintf(buf, sizeof buf, "!0x%llx", static_cast<unsigned long long>(v));
+        return std::string(buf);
+    };
+    std::vector<Instruction> out;
+    size_t at = 5;
+    while (at < words.size()) {
+        const uint32_t length = words[at] >> 16, code = words[at] & 0xffffu;
+        Instruction inst;
+        inst.binary = true;
+        inst.line = static_cast<int>(at);
+        const auto known = layouts.find(code);
+        inst.opcode = known != layouts.end() ? known->second->name : "Op#" + std::to_string(code);
+        if (length == 0) fail(inst, "instruction of zero words");
+        if (at + length > words.size()) fail(inst, "instruction runs past the end of the module");
+        const uint32_t *w = &words[at];
+        size_t k = 1;
+        const auto more = [&] { return k < length; };
+        const auto next = [&] {
+            if (!more()) fail(inst, "too few words");
+            return w[k++];
+        };
+        const auto id = [&] { return "%" + std::to_string(next()); };
+        at += length;
+        if (known == layouts.end()) {  // nothing the loader reads: kept as raw words so that error messages can show it
+            while (more()) inst.operands.push_back(std::to_string(next()));
+            out.push_back(std::move(inst));
+            continue;
+        }
+        const OpcodeLayout &layout = *known->second;
+        uint32_t typeId = 0, resultId = 0;
+        if (layout.hasType) {
+            typeId = next();
+            inst.operands.push_back("%" + std::to_string(typeId));
+        }
+        if (layout.hasResult) {
+            resultId = next();
+            inst.result = "%" + std::to_string(resultId);
+        }
+        uint32_t firstId = 0;
+        for (const char *kind = layout.operands; *kind; kind++) {
+            switch (*kind) {
+            case 'i': {
+                const uint32_t v = next();
+                if (firstId == 0) firstId = v;
+                inst.operands.push_back("%" + std::to_string(v));
+                break;
+            }
+            case 'I':
+                while (more()) inst.operands.push_back(id());
+                break;
+            case 'l': inst.operands.push_back(std::to_string(next())); break;
+            case 'L':
+                while (more()) inst.operands.push_back(std::to_string(next()));
+                break;
+            case 's': {
+                std::string text;
+                bool ended = false;
+                while (!ended) {
+                    const uint32_t v = next();
+                    for (int b = 0; b < 4 && !ended; b++) {
+                        const char c = static_cast<char>((v >> (8 * b)) & 0xffu);
+                        if (c == 0)
+                            ended = true;
+                        else
+                            text.push_back(c);
+                    }
+                }
+                inst.operands.push_back(text);
+                break;
+            }
+            case 'c': {
+                const auto width = scalarWidth.find(typeId);
+                if (width == scalarWidth.end()) fail(inst, "constant of a type that is not a scalar number");
+                uint64_t bits = next();
+                if (width->second > 32) bits |= static_cast<uint64_t>(next()) << 32;
+                inst.operands.push_back(hex(bits));
+                break;
+            }
+            case 'd': {
+                const uint32_t v = next();
+                inst.operands.push_back(v == 1 ? "SpecId" : v == 33 ? "Binding" : v == 34 ? "DescriptorSet" : std::to_string(v));
+                break;
+            }
+            case 'f':
+                if (more()) {
+                    const uint32_t v = next();
+                    inst.operands.push_back(v == 0 ? "BFloat16KHR"
+                                            : v == 4214 ? "Float8E4M3EXT"
+                                            : v == 4215 ? "Float8E5M2EXT"
+                                                        : "FPEncoding#" + std::to_string(v));
+                }
+                break;
+            case 'x': {
+                const uint32_t v = next();
+                if (firstId == tosaSet && tosaSet != 0 && v < sizeof kTosaNames / sizeof kTosaNames[0])
+                    inst.operands.push_back(kTosaNames[v]);
+                else
+                    inst.operands.push_back("instruction#" + std::to_string(v));
+                break;
+            }
+            default: break;
+            }
+        }
+        if (more()) fail(inst, "more words than the instruction takes");
+        if (code == 21 || code == 22) scalarWidth[resultId] = std::atoi(inst.operands[0].c_str());
+        if (code == 11 && inst.operands[0] == "TOSA.001000.1") tosaSet = resultId;
         out.push_back(std::move(inst));
     }
     return out;
@@ -907,6 +1111,13 @@ SpvGraphInfo loadSpirvAssembly(GraphPipeline &pipeline, const std::string &text,
                                const std::vector<SpvSpecialization> &specializations) {
     Module module(pipeline, bindings, constants, specializations);
     return module.build(tokenize(text));
+}
+
+SpvGraphInfo loadSpirvBinary(GraphPipeline &pipeline, const uint32_t *words, const size_t count,
+                             const std::vector<SpvBinding> &bindings, const std::vector<SpvConstant> &constants,
+                             const std::vector<SpvSpecialization> &specializations) {
+    Module module(pipeline, bindings, constants, specializations);
+    return module.build(decodeWords(words, count));
 }
 
 }  // namespace mlel::graph

@@ -1,4 +1,4 @@
-// Front-end for data graphs written as SPIR-V assembly text (SPV_ARM_graph + SPV_ARM_tensors with the
+// Front-end for data graphs as SPIR-V, assembly text or binary words (SPV_ARM_graph + SPV_ARM_tensors with the
 // "TOSA.001000.1" extended instruction set): the module is read, its types, constants and interface variables are
 // resolved, and every instruction of the graph body becomes one GraphPipeline::make<Op> call.
 //
@@ -52,5 +52,12 @@ struct SpvGraphInfo {
 SpvGraphInfo loadSpirvAssembly(GraphPipeline &pipeline, const std::string &text, const std::vector<SpvBinding> &bindings,
                                const std::vector<SpvConstant> &constants,
                                const std::vector<SpvSpecialization> &specializations = {});
+
+// The same for a binary module (the words handed to vkCreateShaderModule, either byte order).  Errors name the
+// offset of the offending instruction's first word.  The opcode, enumerant and TOSA instruction numbers are the
+// published ones; the reference takes them from the SPIRV-Headers package, which is not part of its source tree.
+SpvGraphInfo loadSpirvBinary(GraphPipeline &pipeline, const uint32_t *words, size_t count,
+                             const std::vector<SpvBinding> &bindings, const std::vector<SpvConstant> &constants,
+                             const std::vector<SpvSpecialization> &specializations = {});
 
 }  // namespace mlel::graph

@@ -57,6 +57,10 @@ def load_graph_library():
                                                C.POINTER(SpvConstant), C.c_int, C.POINTER(SpvSpecialization), C.c_int,
                                                C.POINTER(C.c_uint32), C.c_int,
                                                C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        lib.mlel_graph_load_spirv.argtypes = [_V, C.POINTER(C.c_uint32), C.c_size_t, C.POINTER(SpvBinding), C.c_int,
+                                              C.POINTER(SpvConstant), C.c_int, C.POINTER(SpvSpecialization), C.c_int,
+                                              C.POINTER(C.c_uint32), C.c_int,
+                                              C.POINTER(C.c_int), C.POINTER(C.c_int)]
         lib.mlel_graph_tensor_info.argtypes = [_V, C.c_int, C.POINTER(C.c_int32), _I64P]
         lib.mlel_graph_finalize.argtypes = [_V, C.c_int]
         lib.mlel_graph_set_memory_planner.argtypes = [_V, C.c_int]
@@ -179,12 +183,22 @@ class Graph:
                                                 _i64(iattr), len(iattr), fa, len(fattr), debug_name.encode()))
 
     # ---- SPIR-V assembly front-end
+    def load_spirv(self, words, bindings=None, constants=None, names=None, specializations=None):
+        """Decodes a binary SPIR-V module (a sequence of 32-bit words, or bytes) into this graph; arguments and
+        result as load_spvasm."""
+        if isinstance(words, (bytes, bytearray, memoryview)):
+            words = np.frombuffer(bytes(words), dtype=np.uint32)
+        words = np.ascontiguousarray(np.asarray(words, dtype=np.uint32))
+        return self._load_module(words, bindings, constants, names, specializations)
+
     def load_spvasm(self, text, bindings=None, constants=None, names=None, specializations=None):
         """Decodes a SPIR-V assembly module into this graph.  `bindings`: {(set, binding, element): shape} for
         interface tensors of unshaped type; `constants`: {graph constant id: ndarray}; `names`: {(set, binding,
         element): name} for the externals (default "s<set>b<binding>e<element>"); `specializations`: {SpecId: value
-        bits}.  Returns (input names, output
-        names, number of TOSA instructions)."""
+        bits}.  Returns (input names, output names, number of TOSA instructions)."""
+        return self._load_module(text, bindings, constants, names, specializations)
+
+    def _load_module(self, module, bindings=None, constants=None, names=None, specializations=None):
         bindings, constants, names = bindings or {}, constants or {}, names or {}
         keep = []
         barr = (SpvBinding * max(1, len(bindings)))()
@@ -204,10 +218,16 @@ class Graph:
             sarr[i] = SpvSpecialization(int(sid), int(bits) & (2 ** 64 - 1))
         io = (C.c_uint32 * 3072)()
         n_in, n_out = C.c_int(), C.c_int()
-        raw = text.encode()
-        count = self._check(self.lib.mlel_graph_load_spvasm(self.g, raw, len(raw), barr, len(bindings), carr,
-                                                            len(constants), sarr, len(specializations), io, 3072,
-                                                            C.byref(n_in), C.byref(n_out)))
+        if isinstance(module, str):
+            raw = module.encode()
+            count = self._check(self.lib.mlel_graph_load_spvasm(self.g, raw, len(raw), barr, len(bindings), carr,
+                                                                len(constants), sarr, len(specializations), io, 3072,
+                                                                C.byref(n_in), C.byref(n_out)))
+        else:
+            count = self._check(self.lib.mlel_graph_load_spirv(self.g, module.ctypes.data_as(C.POINTER(C.c_uint32)),
+                                                               module.size, barr, len(bindings), carr, len(constants),
+                                                               sarr, len(specializations), io, 3072, C.byref(n_in),
+                                                               C.byref(n_out)))
         result = []
         for k in range(n_in.value + n_out.value):
             key = (int(io[3 * k]), int(io[3 * k + 1]), int(io[3 * k + 2]))

@@ -76,6 +76,13 @@ int mlel_graph_load_spvasm(mlel_graph *g, const char *text, size_t length, const
                            int n_bindings, const mlel_graph_spv_constant *constants, int n_constants,
                            const mlel_graph_spv_specialization *specializations, int n_specializations, uint32_t *io,
                            int io_capacity, int *n_inputs, int *n_outputs);
+/* The same for a binary module: `words` is the word stream a Vulkan application passes to vkCreateShaderModule
+ * (VkShaderModuleCreateInfo::pCode, codeSize / 4 words; either byte order), which the reference hands to
+ * SPIRV-Tools in GraphLayer::vkCreateShaderModule (graph/graph_layer.cpp:2015-2046). */
+int mlel_graph_load_spirv(mlel_graph *g, const uint32_t *words, size_t n_words, const mlel_graph_spv_binding *bindings,
+                          int n_bindings, const mlel_graph_spv_constant *constants, int n_constants,
+                          const mlel_graph_spv_specialization *specializations, int n_specializations, uint32_t *io,
+                          int io_capacity, int *n_inputs, int *n_outputs);
 /* dtype, rank and dimensions of a tensor handle (dims: room for MLEL_MAX_RANK entries); returns the rank. */
 int mlel_graph_tensor_info(mlel_graph *g, int tensor, int32_t *dtype, int64_t *dims);
 
