@@ -599,10 +599,13 @@ int mlel_hip_elementwise_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *o
                  MLEL_ERR_INVALID, "elementwise_chain: %d inputs, %d steps", chain->n_inputs, chain->n_steps);
     MLEL_TRY(check_supported(out, "elementwise_chain out"));
     for (int i = 0; i < chain->n_inputs; i++) MLEL_TRY(check_supported(chain->inputs[i], "elementwise_chain input"));
-    const int rc = elementwise_chain_launch((hipStream_t)stream, out, chain);
+    bool reduces = false;
+    for (int i = 0; i < chain->n_steps; i++) reduces = reduces || chain->steps[i].kind == MLEL_CHAIN_REDUCE;
+    const int rc = reduces ? row_chain_launch((hipStream_t)stream, out, chain)
+                           : elementwise_chain_launch((hipStream_t)stream, out, chain);
     if (rc != MLEL_ERR_UNSUPPORTED) return rc;
     // the one-pass kernel declined (strides, alignment, too many live values): the operators one after another,
-    // every intermediate in a temporary of its own
+    // every intermediate in a temporary of its own with the broadcast shape of its operands
     std::vector<Scratch> temps(static_cast<size_t>(chain->n_steps));
     std::vector<mlel_tensor> values;
     for (int i = 0; i < chain->n_inputs; i++) values.push_back(*chain->inputs[i]);
@@ -612,14 +615,20 @@ int mlel_hip_elementwise_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *o
         const bool two = st.kind == MLEL_CHAIN_BINARY || st.kind == MLEL_CHAIN_MUL;
         MLEL_REQUIRE(st.a >= 0 && st.a < n && (!two || (st.b >= 0 && st.b < n)), MLEL_ERR_INVALID,
                      "elementwise_chain: step %d reads a value that does not exist yet", i);
+        const mlel_tensor *a = &values[static_cast<size_t>(st.a)], *b = two ? &values[static_cast<size_t>(st.b)] : nullptr;
         mlel_tensor result;
         if (i == chain->n_steps - 1) {
             result = *out;
         } else {
-            MLEL_HIP_CHECK(hipMalloc(&temps[static_cast<size_t>(i)].ptr, (size_t)numel(out) * 4 + 16));
-            result = packed_like(out, st.dtype, temps[static_cast<size_t>(i)].ptr);
+            mlel_tensor shape = *a;
+            if (two) {
+                MLEL_REQUIRE(a->rank == b->rank, MLEL_ERR_INVALID, "elementwise_chain: step %d: operand ranks differ", i);
+                for (int d = 0; d < a->rank; d++) shape.dims[d] = std::max(a->dims[d], b->dims[d]);
+            }
+            if (st.kind == MLEL_CHAIN_REDUCE) shape.dims[shape.rank - 1] = 1;
+            MLEL_HIP_CHECK(hipMalloc(&temps[static_cast<size_t>(i)].ptr, (size_t)numel(&shape) * 4 + 16));
+            result = packed_like(&shape, st.dtype, temps[static_cast<size_t>(i)].ptr);
         }
-        const mlel_tensor *a = &values[static_cast<size_t>(st.a)], *b = two ? &values[static_cast<size_t>(st.b)] : nullptr;
         switch (st.kind) {
         case MLEL_CHAIN_BINARY:
             MLEL_TRY(mlel_hip_elementwise_binary(ctx, stream, st.selector, &result, a, b, MLEL_NAN_PROPAGATE));
@@ -627,6 +636,10 @@ int mlel_hip_elementwise_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *o
         case MLEL_CHAIN_MUL: MLEL_TRY(mlel_hip_mul(ctx, stream, &result, a, b, 0)); break;
         case MLEL_CHAIN_UNARY: MLEL_TRY(mlel_hip_elementwise_unary(ctx, stream, st.selector, &result, a)); break;
         case MLEL_CHAIN_CAST: MLEL_TRY(mlel_hip_cast(ctx, stream, &result, a)); break;
+        case MLEL_CHAIN_REDUCE:
+            MLEL_REQUIRE(a->rank >= 1, MLEL_ERR_INVALID, "elementwise_chain: step %d reduces a rank-0 value", i);
+            MLEL_TRY(mlel_hip_reduce(ctx, stream, st.selector, &result, a, (uint32_t)(a->rank - 1), MLEL_NAN_PROPAGATE));
+            break;
         default: MLEL_REQUIRE(false, MLEL_ERR_INVALID, "elementwise_chain: step kind %d", st.kind);
         }
         values.push_back(result);
@@ -641,32 +654,19 @@ int mlel_hip_softmax_rows(mlel_ctx *ctx, void *stream, const mlel_tensor *out, c
     MLEL_TRY(check_supported(in, "softmax_rows in"));
     MLEL_REQUIRE(in->rank >= 1 && same_shape(out, in) && in->dtype == out->dtype && dt_is_float(in->dtype), MLEL_ERR_INVALID,
                  "softmax_rows: input and output must be floating-point tensors of one shape and type");
-    const int rc = try_softmax_rows_f16(ctx, (hipStream_t)stream, out, in);
-    if (rc != 0) return rc < 0 ? rc : 0;
-    // no one-pass kernel for this type or layout: the six operators one after another through temporaries
-    const int last = in->rank - 1;
-    mlel_tensor row = packed_like(in, in->dtype, nullptr);
-    row.dims[last] = 1;
-    row = packed_like(&row, in->dtype, nullptr);
-    Scratch t_max, t_diff, t_exp, t_sum, t_rcp;
-    const size_t full = (size_t)numel(in) * dt_size(in->dtype) + 16, small = (size_t)numel(&row) * dt_size(in->dtype) + 16;
-    MLEL_HIP_CHECK(hipMalloc(&t_max.ptr, small));
-    MLEL_HIP_CHECK(hipMalloc(&t_diff.ptr, full));
-    MLEL_HIP_CHECK(hipMalloc(&t_exp.ptr, full));
-    MLEL_HIP_CHECK(hipMalloc(&t_sum.ptr, small));
-    MLEL_HIP_CHECK(hipMalloc(&t_rcp.ptr, small));
-    mlel_tensor mx = row, sum = row, rcp = row, diff = packed_like(in, in->dtype, t_diff.ptr), ex = packed_like(in, in->dtype, t_exp.ptr);
-    mx.ptr = t_max.ptr;
-    sum.ptr = t_sum.ptr;
-    rcp.ptr = t_rcp.ptr;
-    MLEL_TRY(mlel_hip_reduce(ctx, stream, MLEL_RED_MAX, &mx, in, (uint32_t)last, MLEL_NAN_PROPAGATE));
-    MLEL_TRY(mlel_hip_elementwise_binary(ctx, stream, MLEL_BIN_SUB, &diff, in, &mx, MLEL_NAN_PROPAGATE));
-    MLEL_TRY(mlel_hip_elementwise_unary(ctx, stream, MLEL_UN_EXP, &ex, &diff));
-    MLEL_TRY(mlel_hip_reduce(ctx, stream, MLEL_RED_SUM, &sum, &ex, (uint32_t)last, MLEL_NAN_PROPAGATE));
-    MLEL_TRY(mlel_hip_elementwise_unary(ctx, stream, MLEL_UN_RECIPROCAL, &rcp, &sum));
-    MLEL_TRY(mlel_hip_mul(ctx, stream, out, &ex, &rcp, 0));
-    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
-    return 0;
+    // the six operators as one chain: value 0 is the input, steps produce values 1 .. 6
+    mlel_chain c{};
+    c.n_inputs = 1;
+    c.n_steps = 6;
+    c.inputs[0] = in;
+    const int dt = in->dtype;
+    c.steps[0] = mlel_chain_step{MLEL_CHAIN_REDUCE, MLEL_RED_MAX, 0, 0, dt};
+    c.steps[1] = mlel_chain_step{MLEL_CHAIN_BINARY, MLEL_BIN_SUB, 0, 1, dt};
+    c.steps[2] = mlel_chain_step{MLEL_CHAIN_UNARY, MLEL_UN_EXP, 2, 0, dt};
+    c.steps[3] = mlel_chain_step{MLEL_CHAIN_REDUCE, MLEL_RED_SUM, 3, 0, dt};
+    c.steps[4] = mlel_chain_step{MLEL_CHAIN_UNARY, MLEL_UN_RECIPROCAL, 4, 0, dt};
+    c.steps[5] = mlel_chain_step{MLEL_CHAIN_MUL, 0, 3, 5, dt};
+    return mlel_hip_elementwise_chain(ctx, stream, out, &c);
 }
 
 int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,

@@ -37,6 +37,8 @@ int pad_generic_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor 
                        double pad_const, int32_t pad_const_int);
 
 int elementwise_chain_launch(hipStream_t s, const mlel_tensor *out, const mlel_chain *chain);
+// the same for a chain with reductions over the last axis in it (fp16)
+int row_chain_launch(hipStream_t s, const mlel_tensor *out, const mlel_chain *chain);
 
 // ops_extra.hip: the TOSA operators outside the benchmark graphs
 int conv3d_launch(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
@@ -116,8 +118,6 @@ int try_unary_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor
 int try_cast_float_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in);
 int try_reduce_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in,
                           uint32_t axis, uint32_t nan_mode);
-// REDUCE_MAX, SUB, EXP, REDUCE_SUM, RECIPROCAL, MUL over the last axis in one pass (fp16)
-int try_softmax_rows_f16(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in);
 
 // ---- bandwidth-bound specialisations (ops_fast.hip) ----
 int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,

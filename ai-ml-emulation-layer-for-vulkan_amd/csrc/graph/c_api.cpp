@@ -277,11 +277,14 @@ std::string opLabel(const OpNode &op) {
     case OpKind::FusedConv2D: return std::string("CONV2D+RESCALE") + (op.hasClamp ? "+CLAMP" : "");
     case OpKind::FusedDepthwiseConv2D: return std::string("DEPTHWISE_CONV2D+RESCALE") + (op.hasClamp ? "+CLAMP" : "");
     case OpKind::FusedMatmul: return std::string("MATMUL+RESCALE") + (op.hasClamp ? "+CLAMP" : "");
-    case OpKind::FusedSoftmax: return "REDUCE_MAX+SUB+EXP+REDUCE_SUM+RECIPROCAL+MUL";
     case OpKind::FusedRescaleAddRescale: return "RESCALE+RESCALE+ADD+RESCALE";
     case OpKind::FusedConv2DResidual:
         return std::string("CONV2D+RESCALE") + (op.hasClamp ? "+CLAMP" : "") + "+RESCALE+RESCALE+ADD+RESCALE";
-    case OpKind::FusedElementwise: return "ELEMENTWISE x" + std::to_string(op.chain.size());
+    case OpKind::FusedElementwise: {
+        bool reduces = false;
+        for (const auto &st : op.chain) reduces = reduces || st.kind == MLEL_CHAIN_REDUCE;
+        return (reduces ? "ELEMENTWISE+REDUCE x" : "ELEMENTWISE x") + std::to_string(op.chain.size());
+    }
     case OpKind::FusedMatmulBiasCast: return op.inputs.size() > 2 ? "MATMUL+ADD+CAST" : "MATMUL+CAST";
     default: return op.tosaName;
     }

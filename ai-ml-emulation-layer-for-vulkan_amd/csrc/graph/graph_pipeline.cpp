@@ -760,60 +760,6 @@ void GraphPipeline::fuse() {
         if (add) add->fusedAway = true;
     }
 
-    // Pattern 4b (softmax over the last axis, fp16): REDUCE_MAX -> SUB -> EXP -> REDUCE_SUM -> RECIPROCAL -> MUL with
-    // every intermediate private and read only inside the pattern becomes one pass over the rows
-    // (mlel_hip_softmax_rows), which rounds after every operator like the operators it replaces.
-    for (const auto &opPtr : ops) {
-        OpNode &rmax = *opPtr;
-        if (rmax.fusedAway || rmax.kind != OpKind::Reduce || rmax.selector != MLEL_RED_MAX ||
-            rmax.nanMode != MLEL_NAN_PROPAGATE)
-            continue;
-        const TensorPtr x = rmax.inputs[0], m = rmax.outputs[0];
-        const uint32_t last = static_cast<uint32_t>(x->getRank()) - 1;
-        if (x->getFormat() != MLEL_F16 || x->getRank() < 1 || rmax.axis != last || !x->isPacked() || !isPrivateIntermediate(*m))
-            continue;
-        const auto only = [&](const TensorPtr &t) -> OpNode * {
-            const auto users = consumersOf(ops, t.get());
-            return users.size() == 1 && !users[0]->fusedAway ? users[0] : nullptr;
-        };
-        const auto fullHalf = [&](const TensorPtr &t) {
-            return t->getFormat() == MLEL_F16 && sameShape(*t, *x) && t->isPacked();
-        };
-        OpNode *sub = only(m);
-        if (!sub || sub->kind != OpKind::Binary || sub->selector != MLEL_BIN_SUB || sub->inputs[0].get() != x.get() ||
-            sub->inputs[1].get() != m.get() || !fullHalf(sub->outputs[0]) || !isPrivateIntermediate(*sub->outputs[0]))
-            continue;
-        OpNode *ex = only(sub->outputs[0]);
-        if (!ex || ex->kind != OpKind::Unary || ex->selector != MLEL_UN_EXP || !fullHalf(ex->outputs[0]) ||
-            !isPrivateIntermediate(*ex->outputs[0]))
-            continue;
-        const TensorPtr e = ex->outputs[0];
-        const auto eUsers = consumersOf(ops, e.get());
-        if (eUsers.size() != 2) continue;
-        OpNode *rsum = nullptr, *mul = nullptr;
-        for (OpNode *u : eUsers) {
-            if (u->kind == OpKind::Reduce) rsum = u;
-            if (u->kind == OpKind::Mul) mul = u;
-        }
-        if (!rsum || !mul || rsum->fusedAway || mul->fusedAway || rsum->selector != MLEL_RED_SUM || rsum->axis != last ||
-            rsum->nanMode != MLEL_NAN_PROPAGATE || rsum->inputs[0].get() != e.get() ||
-            rsum->outputs[0]->getFormat() != MLEL_F16 || !isPrivateIntermediate(*rsum->outputs[0]))
-            continue;
-        OpNode *rcp = only(rsum->outputs[0]);
-        if (!rcp || rcp->kind != OpKind::Unary || rcp->selector != MLEL_UN_RECIPROCAL ||
-            rcp->outputs[0]->getFormat() != MLEL_F16 || !isPrivateIntermediate(*rcp->outputs[0]) ||
-            only(rcp->outputs[0]) != mul)
-            continue;
-        const TensorPtr r = rcp->outputs[0];
-        const bool operands = (mul->inputs[0].get() == e.get() && mul->inputs[1].get() == r.get()) ||
-                              (mul->inputs[1].get() == e.get() && mul->inputs[0].get() == r.get());
-        if (!operands || mul->shift != 0 || !fullHalf(mul->outputs[0])) continue;
-        rmax.kind = OpKind::FusedSoftmax;
-        rmax.outputs[0] = mul->outputs[0];
-        mul->outputs[0]->setProducer(&rmax);
-        sub->fusedAway = ex->fusedAway = rsum->fusedAway = rcp->fusedAway = mul->fusedAway = true;
-    }
-
     // Pattern 5: regions of floating-point elementwise operators (ADD, SUB, MUL, EXP, RECIPROCAL, RSQRT, TANH, CAST
     // between fp16 and fp32) collapse into one pass.  A region grows backwards from an operator whose result is needed
     // elsewhere: a producer is absorbed when it is elementwise too, has the region's shape, and its result is a
@@ -847,6 +793,127 @@ void GraphPipeline::fuse() {
         default: return false;
         }
     };
+    // Pattern 4c: regions of fp16 operators that hold reductions over the last axis (REDUCE_SUM / REDUCE_MAX with the
+    // elementwise operators around them: LayerNorm, softmax with its scale) become one pass over the rows.  A region
+    // starts at an operator, takes the later operators that read its values while everything they read is either in
+    // the region or exists before it, and ends at the longest prefix from which exactly one value escapes: the last
+    // one, with the full shape.  All values have the full shape [.., cols], its per-row shape [.., 1], or are inputs
+    // broadcast along rows and / or the last axis.
+    {
+        const auto rowStepOf = [&](const OpNode &op, mlel_chain_step *st) {
+            if (op.fusedAway || op.outputs.size() != 1 || op.outputs[0]->getFormat() != MLEL_F16) return false;
+            if (op.kind == OpKind::Reduce) {
+                const auto &in = op.inputs[0];
+                *st = mlel_chain_step{MLEL_CHAIN_REDUCE, op.selector, -1, -1, MLEL_F16};
+                return (op.selector == MLEL_RED_SUM || op.selector == MLEL_RED_MAX) && op.nanMode == MLEL_NAN_PROPAGATE &&
+                       in->getFormat() == MLEL_F16 && in->getRank() >= 1 && op.axis + 1 == in->getRank();
+            }
+            return op.kind != OpKind::Cast && chainStepOf(op, st);
+        };
+        for (size_t first = 0; first < ops.size(); first++) {
+            mlel_chain_step firstStep{};
+            if (!rowStepOf(*ops[first], &firstStep)) continue;
+            // the full shape: the largest operand or result of the first operator
+            const TensorDescriptor *full = ops[first]->outputs[0].get();
+            for (const auto &in : ops[first]->inputs)
+                if (in->getShapeSize() > full->getShapeSize()) full = in.get();
+            const auto &dims = full->getDimensions();
+            if (dims.empty() || dims.back() % 8 != 0 || dims.back() < 8) continue;
+            enum { kNone, kFull, kRow, kBroadcast };
+            const auto shapeClass = [&](const TensorDescriptor &t) {
+                const auto &d = t.getDimensions();
+                if (d.size() != dims.size() || !t.isPacked() || t.getFormat() != MLEL_F16) return int(kNone);
+                bool same = true, ones = true;
+                for (size_t i = 0; i + 1 < d.size(); i++) {
+                    same = same && d[i] == dims[i];
+                    ones = ones && d[i] == 1;
+                }
+                if (d.back() != dims.back() && d.back() != 1) return int(kNone);
+                if (same) return d.back() == dims.back() ? int(kFull) : int(kRow);
+                return ones ? int(kBroadcast) : int(kNone);
+            };
+            std::vector<OpNode *> region;
+            std::vector<mlel_chain_step> regionSteps;
+            const auto inRegion = [&](const OpNode *p) { return std::find(region.begin(), region.end(), p) != region.end(); };
+            for (size_t i = first; i < ops.size() && region.size() < MLEL_CHAIN_MAX_STEPS; i++) {
+                OpNode &op = *ops[i];
+                mlel_chain_step st{};
+                if (!rowStepOf(op, &st)) continue;
+                const int outClass = shapeClass(*op.outputs[0]);
+                if (outClass != kFull && outClass != kRow) continue;
+                bool connected = region.empty(), readable = true;
+                for (const auto &in : op.inputs) {
+                    OpNode *p = in->getProducer();
+                    if (p && inRegion(p)) {
+                        connected = true;
+                    } else {
+                        // produced before the region starts (or not by the graph at all) and of a usable shape
+                        bool early = p == nullptr;
+                        for (size_t k = 0; k < first && !early; k++) early = ops[k].get() == p;
+                        readable = readable && early && shapeClass(*in) != kNone;
+                    }
+                }
+                if (!connected || !readable) continue;
+                region.push_back(&op);
+                regionSteps.push_back(st);
+            }
+            // the longest prefix with one escaping value, the last, full-shaped, and at least one reduction inside
+            size_t best = 0;
+            for (size_t n = region.size(); n >= 3 && best == 0; n--) {
+                bool ok = shapeClass(*region[n - 1]->outputs[0]) == kFull, reduces = false;
+                for (size_t k = 0; k < n && ok; k++) {
+                    reduces = reduces || region[k]->kind == OpKind::Reduce;
+                    if (k + 1 == n) break;
+                    const auto &t = region[k]->outputs[0];
+                    ok = isPrivateIntermediate(*t);
+                    for (OpNode *user : consumersOf(ops, t.get())) {
+                        bool inside = false;
+                        for (size_t m = 0; m < n; m++) inside = inside || region[m] == user;
+                        ok = ok && inside;
+                    }
+                }
+                if (ok && reduces) best = n;
+            }
+            if (best == 0) continue;
+            // values: region inputs first, then one per step
+            std::vector<TensorPtr> regionInputs;
+            std::vector<mlel_chain_step> steps;
+            bool fits = true;
+            const auto valueOf = [&](const TensorPtr &t) {
+                for (size_t k = 0; k < best; k++)
+                    if (region[k]->outputs[0].get() == t.get() && k < steps.size()) return -static_cast<int>(k) - 1;
+                for (size_t k = 0; k < regionInputs.size(); k++)
+                    if (regionInputs[k].get() == t.get()) return static_cast<int>(k);
+                if (regionInputs.size() >= MLEL_CHAIN_MAX_INPUTS) {
+                    fits = false;
+                    return 0;
+                }
+                regionInputs.push_back(t);
+                return static_cast<int>(regionInputs.size()) - 1;
+            };
+            for (size_t k = 0; k < best; k++) {
+                mlel_chain_step st = regionSteps[k];
+                const bool two = st.kind == MLEL_CHAIN_BINARY || st.kind == MLEL_CHAIN_MUL;
+                st.a = valueOf(region[k]->inputs[0]);
+                st.b = two ? valueOf(region[k]->inputs[1]) : 0;
+                steps.push_back(st);
+            }
+            bool anyFull = false;
+            for (const auto &t : regionInputs) anyFull = anyFull || shapeClass(*t) == kFull;
+            if (!fits || !anyFull) continue;
+            const int nIn = static_cast<int>(regionInputs.size());
+            for (auto &st : steps) {
+                if (st.a < 0) st.a = nIn + (-st.a - 1);
+                if (st.b < 0) st.b = nIn + (-st.b - 1);
+            }
+            OpNode &root = *region[best - 1];
+            for (size_t k = 0; k + 1 < best; k++) region[k]->fusedAway = true;
+            root.kind = OpKind::FusedElementwise;
+            root.inputs = regionInputs;
+            root.chain = steps;
+        }
+    }
+
     for (auto it = ops.rbegin(); it != ops.rend(); ++it) {
         OpNode &root = **it;
         mlel_chain_step rootStep{};
@@ -1227,7 +1294,6 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
         rc = mlel_hip_elementwise_chain(ctx, stream, &out, &c);
         break;
     }
-    case OpKind::FusedSoftmax: rc = mlel_hip_softmax_rows(ctx, stream, &out, &in[0]); break;
     case OpKind::FusedMatmulBiasCast:
         rc = mlel_hip_matmul_bias_cast(ctx, stream, &out, &in[0], &in[1], op.inputs.size() > 2 ? &in[2] : nullptr,
                                        &op.matmul);

@@ -98,7 +98,7 @@ enum class OpKind {
     Argmax, ArithmeticRightShift, Conv3D, TransposeConv2D, Fft2D, Rfft2D, Gather, Scatter, Resize, Reverse, Tile, Select,
     // produced by the fusion pass only
     FusedConv2D, FusedDepthwiseConv2D, FusedMatmul, FusedRescaleAddRescale, FusedMatmulBiasCast, FusedElementwise,
-    FusedConv2DResidual, FusedSoftmax,
+    FusedConv2DResidual,
 };
 
 struct RescaleSpec {

@@ -3,6 +3,7 @@
 // bit: operands are widened to fp32, the operator is applied once, and the result is rounded once into the storage
 // type (reference: elementwise_binary.comp:146-173, mul.comp:24-59, elementwise_unary.comp:136-205,
 // cast.comp:22-103, reduce.comp:24-70).  `try_*` returns 0 to decline a case.
+#include <type_traits>
 #include <vector>
 
 #include "common.hpp"
@@ -547,147 +548,260 @@ __global__ void __launch_bounds__(kBlock) reduce_rows_f16_kernel(const ReduceArg
 
 
 // ---------------------------------------------------------------------------------------------------------------
-// The softmax operator sequence of a TOSA graph over the last axis of a dense fp16 tensor, in one pass:
-//   m = REDUCE_MAX(x);  d = SUB(x, m);  e = EXP(d);  s = REDUCE_SUM(e);  r = RECIPROCAL(s);  out = MUL(e, r)
-// with every intermediate rounded to fp16 exactly where the stand-alone operators round it (the same device
-// functions, the same order), the maximum taken pairwise (its order is free) and the sum folded left to right in
-// fp16 as reduce.comp:24-70 prescribes.  A block owns 64 rows held in shared memory: all four wavefronts fetch the
-// rows and take the maxima (four threads per row), overwrite the rows with e, then the first wavefront folds one row
-// per lane, and all four scale and store.  Rows that hold a NaN take the element-by-element path of the stand-alone
-// kernels (first NaN wins in both reductions).
+// A chain of fp16 operators with reductions over the last axis in it (LayerNorm's moments, softmax with its scale,
+// ...), in one pass.  Values come in four shapes: full [rows, cols], one per row [rows, 1], one per column
+// [1, cols] and single elements.  A block owns R = 4 .. 64 rows; the full values that are alive at the same time
+// sit in shared memory ("row registers", R rows of cols halfs each), the per-row values in a small file of their own.
+// 256 / R threads share a row: elementwise steps walk the row's 16-byte pieces with them (a piece is always handled
+// by the same thread, so consecutive elementwise steps need no barrier), REDUCE_SUM is folded left to right in fp16
+// by the row's first thread (reduce.comp:24-70), REDUCE_MAX is taken pairwise by all of them.  Every step rounds to
+// fp16 where the stand-alone operator rounds, with the same device functions.  A reduction over a row that holds a
+// NaN yields a NaN (the stand-alone kernels return the first one met; payload and sign are not kept here).
 // ---------------------------------------------------------------------------------------------------------------
-struct SoftmaxArgs {
-    const char *in;
+enum { F_RED_SUM = 16, F_RED_MAX = 17 };
+enum RowClass : int8_t { RC_ONE = 0, RC_COL = 1, RC_ROW_IN = 2, RC_ROW = 3, RC_FULL = 4 };
+constexpr int kRowRegs = 4;       // full values alive at once
+constexpr int kRowScalars = 8;    // per-row values alive at once
+constexpr int kRowLdsBudget = 64 * 1024;
+
+struct RowOperand {
+    int8_t cls;  // RowClass
+    int8_t idx;  // RC_FULL: row register; RC_ROW: slot of the per-row file; RC_COL: slot of the column file;
+                 // otherwise the input's index
+};
+struct alignas(8) RowStep {  // eight bytes: one scalar load fetches a step
+    int8_t op;      // FOp or F_RED_*
+    int8_t cls;     // RC_FULL or RC_ROW: shape of the result
+    RowOperand a, b;
+    int8_t dst;     // row register / per-row slot of the result; -1: the result is the output
+    int8_t pad;
+};
+struct RowArgs {
     char *out;
     int64_t rows;
-    int32_t cols;  // multiple of 8, at most kSoftmaxMaxCols
+    const char *in[MLEL_CHAIN_MAX_INPUTS];
+    RowStep step[MLEL_CHAIN_MAX_STEPS];
+    int32_t cols;
+    int32_t log2_r;
+    int32_t n_inputs, n_steps, n_regs;
+    int32_t n_cols;                        // per-column inputs
+    int8_t in_reg[MLEL_CHAIN_MAX_INPUTS];  // row register a full input is fetched into, -1 for the other shapes
+    int8_t in_cls[MLEL_CHAIN_MAX_INPUTS];  // RowClass of the input
+    int8_t in_col[MLEL_CHAIN_MAX_INPUTS];  // per-column inputs: slot of the column file
 };
-constexpr int kSoftmaxMaxCols = 1024;
 
-__global__ void __launch_bounds__(kBlock) softmax_rows_f16_kernel(const SoftmaxArgs g) {
-    extern __shared__ __align__(16) char slab[];
-    const int pitch = g.cols * 2 + 16;
-    __half *row_scale = reinterpret_cast<__half *>(slab + 64 * pitch);  // [64] maximum, later the reciprocal
-    const int tid = threadIdx.x;
-    const int64_t row0 = (int64_t)blockIdx.x * 64;
-    const int segs = g.cols >> 3, pieces = 64 * segs;
-    // ---- fetch: consecutive threads take consecutive 16-byte pieces of a row
-    for (int p0 = 0; p0 < pieces; p0 += kBlock * 8) {
-        uint4 v[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int p = p0 + i * kBlock + tid;
-            const int rr = p / segs, seg = p - rr * segs;
-            v[i] = make_uint4(0, 0, 0, 0);
-            if (p < pieces && row0 + rr < g.rows)
-                v[i] = *reinterpret_cast<const uint4 *>(g.in + ((row0 + rr) * g.cols + seg * 8) * 2);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int p = p0 + i * kBlock + tid;
-            const int rr = p / segs, seg = p - rr * segs;
-            if (p < pieces) *reinterpret_cast<uint4 *>(slab + rr * pitch + seg * 16) = v[i];
-        }
+__device__ __forceinline__ float row_apply(int op, float a, float b) {
+    switch (op) {
+    case F_ADD: return a + b;
+    case F_SUB: return a - b;
+    case F_MUL: return a * b;
+    case F_EXP: return op_exp<true>(a);
+    case F_RECIPROCAL: return op_reciprocal<true>(a);
+    case F_RSQRT: return op_rsqrt<true>(a);
+    case F_TANH: return op_tanh<true>(a);
+    default: return a;
     }
-    __syncthreads();
-    // ---- maximum: four threads per row, pieces interleaved; a NaN anywhere sends the row to the careful path
-    const int r = tid >> 2, part = tid & 3;
-    char *mine = slab + r * pitch;
-    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-    h2_t m2 = {(_Float16)-65504.f, (_Float16)-65504.f};
-    uint32_t special = 0;
-    for (int sg = part; sg < segs; sg += 4) {
-        const uint4 raw = *reinterpret_cast<const uint4 *>(mine + sg * 16);
-        special |= (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu) |
-                    ((raw.z & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
-        const h2_t *p = reinterpret_cast<const h2_t *>(&raw);
-        m2 = __builtin_elementwise_max(m2, __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]),
-                                                                       __builtin_elementwise_max(p[2], p[3])));
-    }
-    float mx = (float)(m2.x > m2.y ? m2.x : m2.y);
-    mx = fmaxf(mx, __shfl_xor(mx, 1));
-    mx = fmaxf(mx, __shfl_xor(mx, 2));
-    special |= (uint32_t)__shfl_xor((int)special, 1);
-    special |= (uint32_t)__shfl_xor((int)special, 2);
-    if (special != 0) {  // REDUCE_MAX as the stand-alone kernel folds a row with a NaN: the first NaN is the result
-        mx = -65504.f;
-        for (int j = 0; j < g.cols; j++) {
-            const float v = __half2float(*reinterpret_cast<const __half *>(mine + j * 2));
-            if (isnan(v)) {
-                mx = v;
-                break;
-            }
-            mx = mx < v ? v : mx;
+}
+
+__global__ void __launch_bounds__(kBlock) row_chain_f16_kernel(const RowArgs g) {
+    extern __shared__ __align__(16) char lds[];
+    const int R = 1 << g.log2_r, tpr_log = 8 - g.log2_r, TPR = 1 << tpr_log;
+    const int pitch = g.cols * 2 + 16, reg_bytes = R * pitch;
+    __half *row_file = reinterpret_cast<__half *>(lds + g.n_regs * reg_bytes);  // [kRowScalars][64]
+    __half *one_file = row_file + kRowScalars * 64;                              // [MLEL_CHAIN_MAX_INPUTS]
+    char *col_file = reinterpret_cast<char *>(one_file + MLEL_CHAIN_MAX_INPUTS); // [n_cols][cols] halfs
+    const int tid = threadIdx.x, rr = tid >> tpr_log, part = tid & (TPR - 1);
+    const int64_t row = (int64_t)blockIdx.x * R + rr;
+    const bool live = row < g.rows;
+    const int segs = g.cols >> 3;
+    char *mine = lds + rr * pitch;  // this thread's row inside row register 0
+
+    // ---- single elements and per-column inputs into their files (read by every thread later: one barrier below),
+    // the full inputs into their row registers, four loads in flight per thread
+    for (int k = 0; k < g.n_inputs; k++) {
+        if (g.in_cls[k] == RC_ONE) {
+            if (tid == k) one_file[k] = *reinterpret_cast<const __half *>(g.in[k]);
+        } else if (g.in_cls[k] == RC_COL) {
+            for (int sg = tid; sg < segs; sg += kBlock)
+                *reinterpret_cast<uint4 *>(col_file + g.in_col[k] * g.cols * 2 + sg * 16) =
+                    *reinterpret_cast<const uint4 *>(g.in[k] + sg * 16);
         }
     }
-    // ---- e = EXP(SUB(x, m)), rounded to fp16 after each of the two operators, written over the row
-    for (int sg = part; sg < segs; sg += 4) {
-        uint4 raw = *reinterpret_cast<const uint4 *>(mine + sg * 16);
-        __half2 *h = reinterpret_cast<__half2 *>(&raw);
+    for (int k = 0; k < g.n_inputs; k++) {
+        if (g.in_reg[k] < 0) continue;  // uniform
+        const char *src = g.in[k] + row * g.cols * 2;
+        char *dst = mine + g.in_reg[k] * reg_bytes;
+        for (int sg0 = part; sg0 < segs; sg0 += 4 * TPR) {
+            uint4 v[4];
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const float2 f = __half22float2(h[t]);
-            const float d0 = __half2float(f2h(f.x - mx)), d1 = __half2float(f2h(f.y - mx));
-            h[t] = __halves2half2(f2h(op_exp<true>(d0)), f2h(op_exp<true>(d1)));
-        }
-        *reinterpret_cast<uint4 *>(mine + sg * 16) = raw;
-    }
-    __syncthreads();
-    // ---- s = REDUCE_SUM(e) left to right in fp16, r = RECIPROCAL(s): one row per lane of the first wavefront
-    if (tid < 64) {
-        const char *row = slab + tid * pitch;
-        float acc_f = 0.f;
-        bool done = false;
-        for (int j = 0; j < g.cols; j += 8) {
-            const uint4 raw = *reinterpret_cast<const uint4 *>(row + j * 2);
-            const uint32_t nan_bits =
-                (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu) |
-                 ((raw.z & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
-            const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
-            if (!__any(done || nan_bits != 0)) {
-                __half acc = f2h(acc_f);
-#pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    acc = __hadd(acc, __low2half(h[t]));
-                    acc = __hadd(acc, __high2half(h[t]));
-                }
-                acc_f = __half2float(acc);
-                continue;
+            for (int i = 0; i < 4; i++) {
+                const int sg = sg0 + i * TPR;
+                v[i] = make_uint4(0, 0, 0, 0);
+                if (live && sg < segs) v[i] = *reinterpret_cast<const uint4 *>(src + sg * 16);
             }
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const float2 f = __half22float2(h[t]);
-                const float e2[2] = {f.x, f.y};
+            for (int i = 0; i < 4; i++) {
+                const int sg = sg0 + i * TPR;
+                if (sg < segs) *reinterpret_cast<uint4 *>(dst + sg * 16) = v[i];
+            }
+        }
+    }
+
+    const auto unpack = [](const uint4 &raw, float (&x)[8]) {
+        const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
 #pragma unroll
-                for (int u = 0; u < 2; u++) {
-                    if (done) continue;
-                    if (isnan(e2[u])) {
-                        acc_f = e2[u];
-                        done = true;
-                        continue;
+        for (int i = 0; i < 4; i++) {
+            const float2 f = __half22float2(h[i]);
+            x[2 * i] = f.x;
+            x[2 * i + 1] = f.y;
+        }
+    };
+    // one element of an operand that does not vary along the row
+    const auto row_value = [&](const RowOperand o) {
+        switch (o.cls) {
+        case RC_ROW: return __half2float(row_file[o.idx * 64 + rr]);
+        case RC_ROW_IN: return live ? __half2float(*reinterpret_cast<const __half *>(g.in[o.idx] + row * 2)) : 0.f;
+        default: return __half2float(one_file[o.idx]);
+        }
+    };
+    // An operand of a full-shaped step is either a row of halfs in shared memory (a row register or a per-column
+    // input) or one value for the whole row.  `OP` is a template argument so that the loop over the pieces holds no
+    // dispatch on the operator.
+    struct Source {
+        const char *base;  // null: `value` for every element
+        float value;
+    };
+    const auto source = [&](const RowOperand o) {
+        if (o.cls == RC_FULL) return Source{mine + o.idx * reg_bytes, 0.f};
+        if (o.cls == RC_COL) return Source{col_file + o.idx * g.cols * 2, 0.f};
+        return Source{nullptr, row_value(o)};
+    };
+    const auto full_step = [&](auto op_tag, const RowStep &st) {
+        constexpr int OP = decltype(op_tag)::value;
+        constexpr bool two = OP == F_ADD || OP == F_SUB || OP == F_MUL;
+        const Source sa = source(st.a), sb = two ? source(st.b) : Source{nullptr, 0.f};
+        char *dst = st.dst >= 0 ? mine + st.dst * reg_bytes : nullptr;
+        char *out_row = g.out + row * g.cols * 2;
+        for (int sg = part; sg < segs; sg += TPR) {
+            float a[8], b[8];
+            if (sa.base) {
+                unpack(*reinterpret_cast<const uint4 *>(sa.base + sg * 16), a);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++) a[i] = sa.value;
+            }
+            if (two && sb.base) {
+                unpack(*reinterpret_cast<const uint4 *>(sb.base + sg * 16), b);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++) b[i] = sb.value;
+            }
+            uint4 raw;
+            __half2 *h = reinterpret_cast<__half2 *>(&raw);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                h[i] = __halves2half2(f2h(row_apply(OP, a[2 * i], b[2 * i])), f2h(row_apply(OP, a[2 * i + 1], b[2 * i + 1])));
+            if (dst)
+                *reinterpret_cast<uint4 *>(dst + sg * 16) = raw;
+            else if (live)
+                *reinterpret_cast<uint4 *>(out_row + sg * 16) = raw;
+        }
+    };
+
+    __syncthreads();  // the files are filled
+    for (int s = 0; s < g.n_steps; s++) {
+        const RowStep st = g.step[s];  // uniform
+        if (st.op == F_RED_SUM || st.op == F_RED_MAX) {
+            __syncthreads();  // the row register is complete
+            const char *src = mine + st.a.idx * reg_bytes;
+            float result = 0.f;
+            if (st.op == F_RED_SUM) {
+                if (part == 0) {
+                    __half acc = f2h(0.f);
+                    const auto add8 = [&](const uint4 &raw) {
+                        const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+#pragma unroll
+                        for (int t = 0; t < 4; t++) {
+                            acc = __hadd(acc, __low2half(h[t]));
+                            acc = __hadd(acc, __high2half(h[t]));
+                        }
+                    };
+                    // the adds form one dependent chain: four pieces are requested while the four before them are
+                    // folded, alternating between two sets of registers
+                    const auto load4 = [&](uint4 (&v)[4], int first) {
+#pragma unroll
+                        for (int t = 0; t < 4; t++) v[t] = *reinterpret_cast<const uint4 *>(src + (first + t) * 16);
+                    };
+                    int sg = 0;
+                    uint4 even[4], odd[4];
+                    if (segs >= 4) load4(even, 0);
+                    for (; sg + 8 <= segs; sg += 8) {
+                        load4(odd, sg + 4);
+#pragma unroll
+                        for (int t = 0; t < 4; t++) add8(even[t]);
+                        if (sg + 12 <= segs) load4(even, sg + 8);
+#pragma unroll
+                        for (int t = 0; t < 4; t++) add8(odd[t]);
                     }
-                    acc_f = rnd_f16(acc_f + e2[u]);
-                }
-            }
-        }
-        row_scale[tid] = f2h(op_reciprocal<true>(__half2float(f2h(acc_f))));
-    }
-    __syncthreads();
-    // ---- out = MUL(e, r), rounded once; stored with the fetch's piece order
-    for (int p0 = 0; p0 < pieces; p0 += kBlock) {
-        const int p = p0 + tid;
-        if (p >= pieces) break;
-        const int rr = p / segs, seg = p - rr * segs;
-        if (row0 + rr >= g.rows) continue;
-        const float scale = __half2float(row_scale[rr]);
-        uint4 raw = *reinterpret_cast<const uint4 *>(slab + rr * pitch + seg * 16);
-        __half2 *h = reinterpret_cast<__half2 *>(&raw);
+                    if (sg + 4 <= segs) {  // `even` holds the pieces sg .. sg + 3
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const float2 f = __half22float2(h[t]);
-            h[t] = __halves2half2(f2h(f.x * scale), f2h(f.y * scale));
+                        for (int t = 0; t < 4; t++) add8(even[t]);
+                        sg += 4;
+                    }
+                    for (; sg < segs; sg++) add8(*reinterpret_cast<const uint4 *>(src + sg * 16));
+                    result = __half2float(acc);
+                }
+            } else {
+                typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+                h2_t m2 = {(_Float16)-65504.f, (_Float16)-65504.f};
+                uint32_t special = 0;
+                for (int sg = part; sg < segs; sg += TPR) {
+                    const uint4 raw = *reinterpret_cast<const uint4 *>(src + sg * 16);
+                    special |= (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu) |
+                                ((raw.z & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
+                    const h2_t *p = reinterpret_cast<const h2_t *>(&raw);
+                    m2 = __builtin_elementwise_max(m2, __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]),
+                                                                                   __builtin_elementwise_max(p[2], p[3])));
+                }
+                float mx = (float)(m2.x > m2.y ? m2.x : m2.y);
+                for (int d = 1; d < TPR; d <<= 1) {  // the row's threads are neighbouring lanes of one wavefront
+                    mx = fmaxf(mx, __shfl_xor(mx, d));
+                    special |= (uint32_t)__shfl_xor((int)special, d);
+                }
+                result = special != 0 ? __builtin_nanf("") : mx;
+            }
+            if (part == 0) {
+                if (st.dst >= 0)
+                    row_file[st.dst * 64 + rr] = f2h(result);
+                else if (live)
+                    *reinterpret_cast<__half *>(g.out + row * 2) = f2h(result);
+            }
+            __syncthreads();
+            continue;
         }
-        *reinterpret_cast<uint4 *>(g.out + ((row0 + rr) * g.cols + seg * 8) * 2) = raw;
+        const bool two = st.op == F_ADD || st.op == F_SUB || st.op == F_MUL;
+        if (st.cls == RC_ROW) {  // one value per row: the row's first thread
+            if (part == 0) {
+                const float a = row_value(st.a), b = two ? row_value(st.b) : 0.f;
+                const __half r = f2h(row_apply(st.op, a, b));
+                if (st.dst >= 0)
+                    row_file[st.dst * 64 + rr] = r;
+                else if (live)
+                    *reinterpret_cast<__half *>(g.out + row * 2) = r;
+            }
+            __syncthreads();
+            continue;
+        }
+        switch (st.op) {  // uniform
+        case F_ADD: full_step(std::integral_constant<int, F_ADD>{}, st); break;
+        case F_SUB: full_step(std::integral_constant<int, F_SUB>{}, st); break;
+        case F_MUL: full_step(std::integral_constant<int, F_MUL>{}, st); break;
+        case F_EXP: full_step(std::integral_constant<int, F_EXP>{}, st); break;
+        case F_RECIPROCAL: full_step(std::integral_constant<int, F_RECIPROCAL>{}, st); break;
+        case F_RSQRT: full_step(std::integral_constant<int, F_RSQRT>{}, st); break;
+        case F_TANH: full_step(std::integral_constant<int, F_TANH>{}, st); break;
+        default: break;
+        }
     }
 }
 
@@ -807,6 +921,172 @@ int elementwise_chain_launch(hipStream_t s, const mlel_tensor *out, const mlel_c
     return check_launch("elementwise chain");
 }
 
+// The chain with reductions.  MLEL_ERR_UNSUPPORTED when it does not fit the kernel (types other than fp16, shapes,
+// alignment, too many values alive at once, rows too long for shared memory).
+int row_chain_launch(hipStream_t s, const mlel_tensor *out, const mlel_chain *c) {
+    const auto decline = [](const char *why) { return set_error(MLEL_ERR_UNSUPPORTED, "row chain: %s", why); };
+    if (c->n_inputs < 1 || c->n_inputs > MLEL_CHAIN_MAX_INPUTS || c->n_steps < 1 || c->n_steps > MLEL_CHAIN_MAX_STEPS)
+        return set_error(MLEL_ERR_INVALID, "row chain: %d inputs, %d steps", c->n_inputs, c->n_steps);
+    if (out->dtype != MLEL_F16 || !is_packed(out) || out->rank < 1) return decline("output type or strides");
+    // the full shape: that of the input with the most elements
+    const mlel_tensor *full = nullptr;
+    for (int k = 0; k < c->n_inputs; k++) {
+        const mlel_tensor *t = c->inputs[k];
+        if (t == nullptr || t->dtype != MLEL_F16 || !is_packed(t) || t->rank != out->rank) return decline("input type, rank or strides");
+        if (full == nullptr || numel(t) > numel(full)) full = t;
+    }
+    const int last = full->rank - 1;
+    const int64_t cols = full->dims[last], total = numel(full);
+    if (total == 0) return 0;
+    if (cols < 8 || cols % 8 != 0) return decline("row length");
+    const int64_t rows = total / cols;
+    const int n_values = c->n_inputs + c->n_steps;
+    std::vector<int8_t> cls(n_values, RC_ONE);
+    const auto class_of = [&](const mlel_tensor *t, int8_t *out_cls) {
+        bool same = true, ones = true;
+        for (int i = 0; i < last; i++) {
+            same = same && t->dims[i] == full->dims[i];
+            ones = ones && t->dims[i] == 1;
+        }
+        const bool wide = t->dims[last] == cols;
+        if (!wide && t->dims[last] != 1) return false;
+        if (same && wide) *out_cls = RC_FULL;
+        else if (ones && wide) *out_cls = RC_COL;
+        else if (ones) *out_cls = RC_ONE;
+        else if (same) *out_cls = RC_ROW_IN;
+        else return false;
+        return true;
+    };
+    RowArgs g{};
+    for (int k = 0; k < c->n_inputs; k++) {
+        const mlel_tensor *t = c->inputs[k];
+        if (!class_of(t, &cls[k])) return decline("input shape");
+        const bool wide = cls[k] == RC_FULL || cls[k] == RC_COL;
+        if (((uintptr_t)t->ptr % (wide ? 16 : 2)) != 0) return decline("input alignment");
+        g.in[k] = static_cast<const char *>(t->ptr);
+        g.in_reg[k] = -1;
+        g.in_cls[k] = cls[k];
+        g.in_col[k] = cls[k] == RC_COL ? (int8_t)g.n_cols++ : (int8_t)-1;
+    }
+    // shapes of the results, last uses
+    std::vector<int> last_use(n_values, -1), op_of(c->n_steps, 0);
+    for (int i = 0; i < c->n_steps; i++) {
+        const mlel_chain_step &st = c->steps[i];
+        if (st.dtype != MLEL_F16) return decline("step type");
+        int op;
+        if (st.kind == MLEL_CHAIN_BINARY && st.selector == MLEL_BIN_ADD) op = F_ADD;
+        else if (st.kind == MLEL_CHAIN_BINARY && st.selector == MLEL_BIN_SUB) op = F_SUB;
+        else if (st.kind == MLEL_CHAIN_MUL) op = F_MUL;
+        else if (st.kind == MLEL_CHAIN_UNARY && st.selector == MLEL_UN_EXP) op = F_EXP;
+        else if (st.kind == MLEL_CHAIN_UNARY && st.selector == MLEL_UN_RECIPROCAL) op = F_RECIPROCAL;
+        else if (st.kind == MLEL_CHAIN_UNARY && st.selector == MLEL_UN_RSQRT) op = F_RSQRT;
+        else if (st.kind == MLEL_CHAIN_UNARY && st.selector == MLEL_UN_TANH) op = F_TANH;
+        else if (st.kind == MLEL_CHAIN_REDUCE && st.selector == MLEL_RED_SUM) op = F_RED_SUM;
+        else if (st.kind == MLEL_CHAIN_REDUCE && st.selector == MLEL_RED_MAX) op = F_RED_MAX;
+        else return decline("operator");
+        op_of[i] = op;
+        const bool two = op == F_ADD || op == F_SUB || op == F_MUL;
+        const int value = c->n_inputs + i;
+        if (st.a < 0 || st.a >= value || (two && (st.b < 0 || st.b >= value)))
+            return set_error(MLEL_ERR_INVALID, "row chain: step %d reads a value that does not exist yet", i);
+        last_use[st.a] = i;
+        if (two) last_use[st.b] = i;
+        const auto along_rows = [](int8_t k) { return k == RC_FULL || k == RC_ROW || k == RC_ROW_IN; };
+        const auto along_cols = [](int8_t k) { return k == RC_FULL || k == RC_COL; };
+        if (op == F_RED_SUM || op == F_RED_MAX) {
+            if (cls[st.a] != RC_FULL) return decline("reduction of a value that is not a full row");
+            cls[value] = RC_ROW;
+        } else {
+            const bool r = along_rows(cls[st.a]) || (two && along_rows(cls[st.b]));
+            const bool w = along_cols(cls[st.a]) || (two && along_cols(cls[st.b]));
+            if (!r) return decline("a step whose result does not vary from row to row");
+            cls[value] = w ? RC_FULL : RC_ROW;
+        }
+    }
+    const int result = n_values - 1;
+    last_use[result] = c->n_steps;
+    {   // the output has the result's shape
+        int8_t out_cls = RC_ONE;
+        if (!class_of(out, &out_cls)) return decline("output shape");
+        const bool want_full = cls[result] == RC_FULL;
+        const bool ok = want_full ? (out_cls == RC_FULL)
+                                  : (out_cls == RC_ROW_IN || (rows == 1 && out_cls == RC_ONE));
+        if (!ok || ((uintptr_t)out->ptr % (want_full ? 16 : 2)) != 0) return decline("output shape or alignment");
+    }
+    // row registers for full values, slots of the per-row file for the others, both by linear scan
+    std::vector<int> slot(n_values, -1), free_regs, free_slots;
+    for (int r = kRowRegs - 1; r >= 0; r--) free_regs.push_back(r);
+    for (int r = kRowScalars - 1; r >= 0; r--) free_slots.push_back(r);
+    int regs_used = 0;
+    const auto take = [&](int value) {
+        std::vector<int> &pool = cls[value] == RC_FULL ? free_regs : free_slots;
+        if (pool.empty()) return false;
+        slot[value] = pool.back();
+        pool.pop_back();
+        if (cls[value] == RC_FULL) regs_used = std::max(regs_used, slot[value] + 1);
+        return true;
+    };
+    const auto release = [&](int value) {
+        if (slot[value] < 0) return;
+        (cls[value] == RC_FULL ? free_regs : free_slots).push_back(slot[value]);
+        slot[value] = -1;
+    };
+    for (int k = 0; k < c->n_inputs; k++) {
+        if (cls[k] != RC_FULL || last_use[k] < 0) continue;
+        if (!take(k)) return decline("too many full values alive at once");
+        g.in_reg[k] = (int8_t)slot[k];
+    }
+    for (int i = 0; i < c->n_steps; i++) {
+        const mlel_chain_step &st = c->steps[i];
+        const int op = op_of[i], value = c->n_inputs + i;
+        const bool two = op == F_ADD || op == F_SUB || op == F_MUL;
+        const auto operand = [&](int v) {
+            const bool held = cls[v] == RC_FULL || cls[v] == RC_ROW;
+            return RowOperand{cls[v], (int8_t)(held ? slot[v] : cls[v] == RC_COL ? g.in_col[v] : v)};
+        };
+        RowStep rs{};
+        rs.op = (int8_t)op;
+        rs.cls = cls[value];
+        rs.a = operand(st.a);
+        rs.b = two ? operand(st.b) : RowOperand{RC_ONE, 0};
+        // operands that die here give their place to the result (a piece is read and written by the same thread)
+        if (last_use[st.a] == i) release(st.a);
+        if (two && st.b != st.a && last_use[st.b] == i) release(st.b);
+        rs.dst = -1;
+        if (value != result) {
+            if (last_use[value] < 0) return decline("a step whose result is never read");
+            if (!take(value)) return decline(cls[value] == RC_FULL ? "too many full values alive at once" : "too many per-row values alive at once");
+            rs.dst = (int8_t)slot[value];
+        }
+        g.step[i] = rs;
+    }
+    if (regs_used == 0) return decline("no full value");
+    const int64_t pitch = cols * 2 + 16;
+    int log2_r = 6;
+    const auto lds_bytes = [&](int lr) {
+        return (int64_t)regs_used * (int64_t(1) << lr) * pitch + kRowScalars * 64 * 2 + MLEL_CHAIN_MAX_INPUTS * 2 +
+               (int64_t)g.n_cols * cols * 2;
+    };
+    while (log2_r > 2 && lds_bytes(log2_r) > kRowLdsBudget) log2_r--;
+    if (lds_bytes(log2_r) > kRowLdsBudget) return decline("rows too long for shared memory");
+    // few rows: smaller blocks, so that the sequential folds spread over the compute units
+    while (log2_r > 2 && (rows + (int64_t(1) << log2_r) - 1) / (int64_t(1) << log2_r) < 512) log2_r--;
+    const int64_t blocks = (rows + (int64_t(1) << log2_r) - 1) >> log2_r;
+    MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "row chain: too many rows");
+    g.out = static_cast<char *>(out->ptr);
+    g.rows = rows;
+    g.cols = (int32_t)cols;
+    g.log2_r = log2_r;
+    g.n_inputs = c->n_inputs;
+    g.n_steps = c->n_steps;
+    g.n_regs = regs_used;
+    static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(row_chain_f16_kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kRowLdsBudget) == hipSuccess;
+    (void)raised;
+    row_chain_f16_kernel<<<dim3((unsigned)blocks), dim3(kBlock), (size_t)lds_bytes(log2_r), s>>>(g);
+    return check_launch("row chain");
+}
+
 int try_reduce_float_fast(mlel_ctx *, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in,
                           uint32_t axis, uint32_t nan_mode) {
     if (in->dtype != MLEL_F16 || out->dtype != MLEL_F16) return 0;
@@ -836,32 +1116,6 @@ int try_reduce_float_fast(mlel_ctx *, hipStream_t s, int op, const mlel_tensor *
                                   (int)smem);
     kernel<<<dim3((unsigned)blocks), dim3(kBlock), smem, s>>>(g);
     MLEL_TRY(check_launch("reduce rows fp16"));
-    return 1;
-}
-
-// Returns 1 when the one-pass kernel ran, 0 when the case is outside what it assumes (the caller then runs the six
-// operators one after another), < 0 on error.
-int try_softmax_rows_f16(mlel_ctx *, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in) {
-    if (in->dtype != MLEL_F16 || out->dtype != MLEL_F16 || in->rank < 1 || !same_shape(out, in)) return 0;
-    if (!is_packed(in) || !is_packed(out) || ((uintptr_t)in->ptr % 16) != 0 || ((uintptr_t)out->ptr % 16) != 0) return 0;
-    const int64_t cols = in->dims[in->rank - 1];
-    if (cols <= 0 || cols % 8 != 0 || cols > kSoftmaxMaxCols) return 0;
-    const int64_t rows = numel(in) / cols;
-    if (rows <= 0) return 1;
-    const int64_t blocks = (rows + 63) / 64;
-    if (blocks >= (int64_t(1) << 31)) return 0;
-    SoftmaxArgs g{};
-    g.in = static_cast<const char *>(in->ptr);
-    g.out = static_cast<char *>(out->ptr);
-    g.rows = rows;
-    g.cols = (int32_t)cols;
-    const size_t smem = (size_t)64 * (cols * 2 + 16) + 64 * 2;
-    static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(softmax_rows_f16_kernel),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   64 * (kSoftmaxMaxCols * 2 + 16) + 128) == hipSuccess;
-    (void)raised;
-    softmax_rows_f16_kernel<<<dim3((unsigned)blocks), dim3(kBlock), smem, s>>>(g);
-    MLEL_TRY(check_launch("softmax rows fp16"));
     return 1;
 }
 

@@ -399,7 +399,7 @@ int mlel_hip_matmul_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out,
 /* The softmax operator sequence over the last axis in one pass:
  *   m = REDUCE_MAX(in); d = SUB(in, m); e = EXP(d); s = REDUCE_SUM(e); r = RECIPROCAL(s); out = MUL(e, r)
  * (NaN propagating reductions), every intermediate rounded to the tensors' type as the stand-alone operators round
- * it: bit for bit the six operators run one after another. */
+ * it: a shorthand for the six-step mlel_chain below (same kernel, same guarantees). */
 int mlel_hip_softmax_rows(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in);
 /* out(fp16) = CAST( MATMUL(a, b) + bias ): fp16 operands, fp32 accumulation, the fp32 bias [1,1,N] or [1,1,1] (or
  * NULL) added in fp32, one rounding to fp16 -- bit for bit the unfused MATMUL -> ADD -> CAST (or MATMUL -> CAST). */
@@ -419,13 +419,20 @@ int mlel_hip_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor 
  * from values a (and b) and rounds it into `dtype` exactly as the stand-alone operator would; the last step's value
  * is written to `out`.  Every step has the shape of `out`; an input has that shape, or is broadcast along the rows
  * (all leading extents 1), along the last axis (last extent 1), or both.  Equals the operators run one after
- * another bit for bit (no counterpart in the reference, which runs one dispatch per operator). */
+ * another bit for bit (no counterpart in the reference, which runs one dispatch per operator).
+ *
+ * A chain may also hold REDUCE_SUM / REDUCE_MAX steps over the last axis (LayerNorm's moments, softmax).  Values then
+ * have the full shape, the full shape with a last extent of 1 (what a reduction yields), or are broadcast inputs as
+ * above; a step's shape is the broadcast of its operands' shapes, a reduction takes a full value, and `out` has the
+ * last step's shape.  Non-NaN results equal the operators run one after another bit for bit; where those yield a NaN
+ * so does the chain, but not necessarily one of the same sign and payload. */
 #define MLEL_CHAIN_MAX_STEPS 24
 #define MLEL_CHAIN_MAX_INPUTS 8
-enum { MLEL_CHAIN_BINARY = 0, MLEL_CHAIN_MUL = 1, MLEL_CHAIN_UNARY = 2, MLEL_CHAIN_CAST = 3 };
+enum { MLEL_CHAIN_BINARY = 0, MLEL_CHAIN_MUL = 1, MLEL_CHAIN_UNARY = 2, MLEL_CHAIN_CAST = 3, MLEL_CHAIN_REDUCE = 4 };
 typedef struct mlel_chain_step {
     int32_t kind;     /* MLEL_CHAIN_* */
-    int32_t selector; /* mlel_binary_op (ADD, SUB) or mlel_unary_op (EXP, RECIPROCAL, RSQRT, TANH) */
+    int32_t selector; /* mlel_binary_op (ADD, SUB), mlel_unary_op (EXP, RECIPROCAL, RSQRT, TANH) or, for
+                         MLEL_CHAIN_REDUCE, mlel_reduce_op (SUM, MAX) over the last axis, NaN propagated */
     int32_t a, b;     /* operand values; b is ignored by unary steps and casts */
     int32_t dtype;    /* MLEL_F16 or MLEL_F32: the type of the step's result */
 } mlel_chain_step;

@@ -383,6 +383,88 @@ def test_elementwise_chain_equals_the_operators_one_by_one(run):
     np.testing.assert_array_equal(got, run.binary("ADD", run.mul(odd, odd, odd.shape, f16), rowb, odd.shape, f16))
 
 
+def _same_bits_or_both_nan(got, want):
+    nan = np.isnan(want)
+    np.testing.assert_array_equal(np.isnan(got), nan)
+    np.testing.assert_array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+
+
+@pytest.mark.parametrize("shape", [(2, 48, 768), (5, 1, 64), (300, 8), (3, 2048), (1, 1, 4096)], ids=str)
+def test_chain_with_reductions_layernorm(run, shape):
+    """LayerNorm as the operators a TOSA graph spells it with (REDUCE_SUM, MUL 1/N, SUB, MUL, REDUCE_SUM, MUL 1/N,
+    ADD eps, RSQRT, MUL, MUL gamma, ADD beta), in one mlel_hip_elementwise_chain call against the eleven stand-alone
+    kernels: the same bits wherever the result is a number (sequential fp16 sums, a rounding after every step)."""
+    rng = np.random.default_rng(shape[-1] + len(shape))
+    B, M, U, R = 0, 1, 2, 4
+    ADD, SUB = abi.BIN["ADD"], abi.BIN["SUB"]
+    f16 = abi.F16
+    n = shape[-1]
+    x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float16)
+    if x.reshape(-1, n).shape[0] > 2:
+        x.reshape(-1, n)[1, 3] = np.nan
+        x.reshape(-1, n)[2, :] = 1.25
+    one = (1,) * len(shape)
+    inv_n, eps = np.full(one, 1.0 / n, np.float16), np.full(one, 1e-3, np.float16)
+    gamma = rng.standard_normal(one[:-1] + (n,)).astype(np.float16)
+    beta = rng.standard_normal(one[:-1] + (n,)).astype(np.float16)
+    # values: 0 x, 1 1/N, 2 eps, 3 gamma, 4 beta; steps start at 5
+    steps = [(R, abi.RED["SUM"], 0, 0, f16), (M, 0, 5, 1, f16), (B, SUB, 0, 6, f16), (M, 0, 7, 7, f16),
+             (R, abi.RED["SUM"], 8, 0, f16), (M, 0, 9, 1, f16), (B, ADD, 10, 2, f16), (U, abi.UN["RSQRT"], 11, 0, f16),
+             (M, 0, 7, 12, f16), (M, 0, 13, 3, f16), (B, ADD, 14, 4, f16)]
+    got = run.chain([x, inv_n, eps, gamma, beta], steps, shape, f16)
+    last = len(shape) - 1
+    rowshape = shape[:-1] + (1,)
+    mean = run.mul(run.reduce("SUM", x, last), inv_n, rowshape, f16)
+    d = run.binary("SUB", x, mean, shape, f16)
+    var = run.mul(run.reduce("SUM", run.mul(d, d, shape, f16), last), inv_n, rowshape, f16)
+    rstd = run.unary("RSQRT", run.binary("ADD", var, eps, rowshape, f16))
+    want = run.binary("ADD", run.mul(run.mul(d, rstd, shape, f16), gamma, shape, f16), beta, shape, f16)
+    _same_bits_or_both_nan(got, want)
+
+
+def test_chain_with_reductions_other_forms(run):
+    """Softmax with its scale in front (seven steps, REDUCE_MAX over rows with infinities and a NaN); a chain that ends
+    in a reduction (one value per row); a per-row input; and chains the one-pass kernel declines (fp32 values, rows
+    that are no multiple of eight), which take the operator-by-operator path inside the call."""
+    rng = np.random.default_rng(4)
+    B, M, U, R = 0, 1, 2, 4
+    ADD, SUB = abi.BIN["ADD"], abi.BIN["SUB"]
+    f16, f32 = abi.F16, abi.F32
+    shape = (3, 40, 256)
+    x = (rng.standard_normal(shape) * 4).astype(np.float16)
+    flat = x.reshape(-1, 256)
+    flat[0, 5] = np.inf
+    flat[1, 7] = -np.inf
+    flat[2, 9] = np.nan
+    flat[3, :] = -0.0
+    k = np.full((1, 1, 1), 0.125, np.float16)
+    steps = [(M, 0, 0, 1, f16), (R, abi.RED["MAX"], 2, 0, f16), (B, SUB, 2, 3, f16), (U, abi.UN["EXP"], 4, 0, f16),
+             (R, abi.RED["SUM"], 5, 0, f16), (U, abi.UN["RECIPROCAL"], 6, 0, f16), (M, 0, 5, 7, f16)]
+    got = run.chain([x, k], steps, shape, f16)
+    s = run.mul(x, k, shape, f16)
+    e = run.unary("EXP", run.binary("SUB", s, run.reduce("MAX", s, 2), shape, f16))
+    want = run.mul(e, run.unary("RECIPROCAL", run.reduce("SUM", e, 2)), shape, f16)
+    _same_bits_or_both_nan(got, want)
+
+    # sum of squares per row, scaled by a per-row input: the result has one value per row
+    w = rng.standard_normal((3, 40, 1)).astype(np.float16)
+    steps = [(M, 0, 0, 0, f16), (R, abi.RED["SUM"], 2, 0, f16), (M, 0, 3, 1, f16)]
+    y = (rng.standard_normal(shape)).astype(np.float16)
+    got = run.chain([y, w], steps, (3, 40, 1), f16)
+    want = run.mul(run.reduce("SUM", run.mul(y, y, shape, f16), 2), w, (3, 40, 1), f16)
+    np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
+
+    # declined by the one-pass kernel: fp32 values; rows of 12
+    y32 = rng.standard_normal((6, 64)).astype(np.float32)
+    steps = [(R, abi.RED["MAX"], 0, 0, f32), (B, SUB, 0, 1, f32)]
+    got = run.chain([y32], steps, y32.shape, f32)
+    np.testing.assert_array_equal(got, run.binary("SUB", y32, run.reduce("MAX", y32, 1), y32.shape, f32))
+    odd = rng.standard_normal((5, 12)).astype(np.float16)
+    steps = [(R, abi.RED["SUM"], 0, 0, f16), (B, SUB, 0, 1, f16)]
+    got = run.chain([odd], steps, odd.shape, f16)
+    np.testing.assert_array_equal(got, run.binary("SUB", odd, run.reduce("SUM", odd, 1), odd.shape, f16))
+
+
 # ------------------------------------------------------------------------------------------------ DEPTHWISE
 DW_CASES = [
     ("c2_like_small", (2, 14, 14, 144), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -4, 0),
