@@ -137,7 +137,7 @@ struct ChainInput {
     int32_t reg;         // register the value is loaded into; single-element inputs: lane of the scalar file
 };
 
-struct ChainStep {
+struct alignas(16) ChainStep {  // sixteen bytes at a sixteen-byte boundary: one scalar load fetches a step
     int8_t op;          // FOp
     int8_t f16;         // result rounded to fp16 (else fp32)
     int8_t a, b;        // operand registers (or scalar-file lanes)
@@ -163,9 +163,24 @@ template <bool HALF>
 __global__ void __launch_bounds__(kBlock) ew_chain_kernel(const ChainArgs g) {
     constexpr int kRegs = HALF ? kChainRegs + 2 : kChainRegs;
     __shared__ uint4 regs[kRegs][HALF ? 1 : 2][kBlock];
+    // The program is indexed at run time; read straight from the kernel arguments that costs a trip to memory per
+    // step and wavefront.  The block copies it into shared memory once and every step is then one broadcast read.
+    __shared__ uint4 program[MLEL_CHAIN_MAX_STEPS];
+    static_assert(sizeof(ChainStep) == sizeof(uint4), "a step is one 16-byte word");
     const int tid = threadIdx.x;
-    const int64_t v = (int64_t)blockIdx.x * kBlock + tid;
-    if (v >= g.vecs) return;  // no barrier below: a thread only touches its own slots
+    const auto step_at = [&](int s) {
+        uint4 w = program[s];
+        w.x = __builtin_amdgcn_readfirstlane(w.x);
+        w.y = __builtin_amdgcn_readfirstlane(w.y);
+        w.z = __builtin_amdgcn_readfirstlane(w.z);
+        ChainStep st;
+        __builtin_memcpy(&st, &w, sizeof st);
+        return st;
+    };
+    // threads past the end repeat the last vector and store nothing: every thread reaches the barrier below
+    const int64_t v_raw = (int64_t)blockIdx.x * kBlock + tid;
+    const bool active = v_raw < g.vecs;
+    const int64_t v = active ? v_raw : g.vecs - 1;
     const int64_t row = v / g.cols8;
     const int32_t c8 = (int32_t)(v - row * g.cols8);
     const auto put = [&](int r, const float (&x)[8]) {
@@ -215,11 +230,14 @@ __global__ void __launch_bounds__(kBlock) ew_chain_kernel(const ChainArgs g) {
             load8<4>(in.ptr, row, c8, g.cols, in.varies_row, in.varies_col, x[k]);
         }
     }
+    // the program is requested after the inputs, so that the two trips to memory overlap
+    if (tid < g.n_steps) program[tid] = reinterpret_cast<const uint4 *>(g.step)[tid];
 #pragma unroll
     for (int k = 0; k < MLEL_CHAIN_MAX_INPUTS; k++) {
         if (k >= g.n_inputs) continue;
         if (g.in[k].varies_row || g.in[k].varies_col) put(g.in[k].reg, x[k]);
     }
+    __syncthreads();  // the program is in place (the registers are private to their thread)
     const auto fetch = [&](int r, int is_scalar, float (&y)[8]) {
         if (is_scalar) {  // uniform
             const float s = __int_as_float(__builtin_amdgcn_readlane(sc_bits, r));
@@ -229,9 +247,77 @@ __global__ void __launch_bounds__(kBlock) ew_chain_kernel(const ChainArgs g) {
             get(r, y);
         }
     };
+    if (HALF) {
+        // Every value is fp16: ADD, SUB and MUL run on packed halfs.  A native fp16 operation rounds the exact result
+        // once; the fp32 operation followed by a conversion (the stand-alone kernels) gives the same value, because
+        // the product of two halfs is exact in fp32 and fp32 carries more than twice the fp16 precision plus two bits,
+        // so that the second rounding of a sum cannot change the result.
+        const auto fetch_h = [&](int r, int is_scalar) {
+            if (!is_scalar) return regs[r][0][tid];
+            const __half s = f2h(__int_as_float(__builtin_amdgcn_readlane(sc_bits, r)));
+            const __half2 s2 = __halves2half2(s, s);
+            const uint32_t w = *reinterpret_cast<const uint32_t *>(&s2);
+            return make_uint4(w, w, w, w);
+        };
+        uint4 rp = make_uint4(0, 0, 0, 0);
+        for (int s = 0; s < g.n_steps; s++) {
+            const ChainStep st = step_at(s);
+            const uint4 a = st.a_fw ? rp : fetch_h(st.a, st.a_sc);
+            const __half2 *ah = reinterpret_cast<const __half2 *>(&a);
+            __half2 *rh = reinterpret_cast<__half2 *>(&rp);
+            if (st.op == F_ADD || st.op == F_SUB || st.op == F_MUL) {
+                const uint4 b = st.b_fw ? rp : fetch_h(st.b, st.b_sc);
+                const __half2 *bh = reinterpret_cast<const __half2 *>(&b);
+                uint4 out4;
+                __half2 *oh = reinterpret_cast<__half2 *>(&out4);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    oh[i] = st.op == F_ADD ? __hadd2(ah[i], bh[i]) : st.op == F_SUB ? __hsub2(ah[i], bh[i]) : __hmul2(ah[i], bh[i]);
+                rp = out4;
+            } else {
+                float x[8], y[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float2 f = __half22float2(ah[i]);
+                    x[2 * i] = f.x;
+                    x[2 * i + 1] = f.y;
+                }
+                switch (st.op) {  // uniform
+                case F_EXP:
+#pragma unroll
+                    for (int i = 0; i < 8; i++) y[i] = op_exp<true>(x[i]);
+                    break;
+                case F_RECIPROCAL:
+#pragma unroll
+                    for (int i = 0; i < 8; i++) y[i] = op_reciprocal<true>(x[i]);
+                    break;
+                case F_RSQRT:
+#pragma unroll
+                    for (int i = 0; i < 8; i++) y[i] = op_rsqrt<true>(x[i]);
+                    break;
+                case F_TANH:
+#pragma unroll
+                    for (int i = 0; i < 8; i++) y[i] = op_tanh<true>(x[i]);
+                    break;
+                default:
+#pragma unroll
+                    for (int i = 0; i < 8; i++) y[i] = x[i];
+                    break;
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) rh[i] = __halves2half2(f2h(y[2 * i]), f2h(y[2 * i + 1]));
+            }
+            if (s + 1 == g.n_steps) {
+                if (active) *reinterpret_cast<uint4 *>(g.out + v * 16) = rp;
+            } else if (st.dst >= 0) {
+                regs[st.dst][0][tid] = rp;
+            }
+        }
+        return;
+    }
     float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < g.n_steps; s++) {
-        const ChainStep st = g.step[s];
+        const ChainStep st = step_at(s);
         float a[8], b[8];
         if (st.a_fw) {  // uniform
 #pragma unroll
@@ -286,10 +372,12 @@ __global__ void __launch_bounds__(kBlock) ew_chain_kernel(const ChainArgs g) {
             for (int i = 0; i < 8; i++) r[i] = rnd_f16(r[i]);
         }
         if (s + 1 == g.n_steps) {  // the result goes straight to memory
-            if (g.out_size == 2)
+            if (!active) {
+            } else if (g.out_size == 2) {
                 store8<2>(g.out + v * 16, r);
-            else
+            } else {
                 store8<4>(g.out + v * 32, r);
+            }
         } else if (st.dst >= 0) {
             put(st.dst, r);
         }
@@ -682,25 +770,33 @@ __global__ void __launch_bounds__(kBlock) row_chain_f16_kernel(const RowArgs g) 
         const Source sa = source(st.a), sb = two ? source(st.b) : Source{nullptr, 0.f};
         char *dst = st.dst >= 0 ? mine + st.dst * reg_bytes : nullptr;
         char *out_row = g.out + row * g.cols * 2;
+        // an operand that is one value for the whole row, as four packed pairs
+        const auto splat = [](float v) {
+            const __half h = f2h(v);
+            const __half2 h2 = __halves2half2(h, h);
+            const uint32_t w = *reinterpret_cast<const uint32_t *>(&h2);
+            return make_uint4(w, w, w, w);
+        };
+        const uint4 a_row = splat(sa.value), b_row = splat(sb.value);
         for (int sg = part; sg < segs; sg += TPR) {
-            float a[8], b[8];
-            if (sa.base) {
-                unpack(*reinterpret_cast<const uint4 *>(sa.base + sg * 16), a);
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; i++) a[i] = sa.value;
-            }
-            if (two && sb.base) {
-                unpack(*reinterpret_cast<const uint4 *>(sb.base + sg * 16), b);
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; i++) b[i] = sb.value;
-            }
+            const uint4 pa = sa.base ? *reinterpret_cast<const uint4 *>(sa.base + sg * 16) : a_row;
             uint4 raw;
             __half2 *h = reinterpret_cast<__half2 *>(&raw);
+            if (two) {
+                // packed fp16 arithmetic: one rounding of the exact result, which is what the fp32 operation followed
+                // by a conversion yields for sums, differences and products of halfs
+                const uint4 pb = sb.base ? *reinterpret_cast<const uint4 *>(sb.base + sg * 16) : b_row;
+                const __half2 *ah = reinterpret_cast<const __half2 *>(&pa), *bh = reinterpret_cast<const __half2 *>(&pb);
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                h[i] = __halves2half2(f2h(row_apply(OP, a[2 * i], b[2 * i])), f2h(row_apply(OP, a[2 * i + 1], b[2 * i + 1])));
+                for (int i = 0; i < 4; i++)
+                    h[i] = OP == F_ADD ? __hadd2(ah[i], bh[i]) : OP == F_SUB ? __hsub2(ah[i], bh[i]) : __hmul2(ah[i], bh[i]);
+            } else {
+                float a[8];
+                unpack(pa, a);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    h[i] = __halves2half2(f2h(row_apply(OP, a[2 * i], 0.f)), f2h(row_apply(OP, a[2 * i + 1], 0.f)));
+            }
             if (dst)
                 *reinterpret_cast<uint4 *>(dst + sg * 16) = raw;
             else if (live)
@@ -708,9 +804,17 @@ __global__ void __launch_bounds__(kBlock) row_chain_f16_kernel(const RowArgs g) 
         }
     };
 
+    // the program as well: indexed at run time, a read from the kernel arguments would be a trip to memory per step
+    __shared__ uint2 program[MLEL_CHAIN_MAX_STEPS];
+    static_assert(sizeof(RowStep) == sizeof(uint2), "a step is one 8-byte word");
+    if (tid < g.n_steps) program[tid] = reinterpret_cast<const uint2 *>(g.step)[tid];
     __syncthreads();  // the files are filled
     for (int s = 0; s < g.n_steps; s++) {
-        const RowStep st = g.step[s];  // uniform
+        uint2 w = program[s];
+        w.x = __builtin_amdgcn_readfirstlane(w.x);
+        w.y = __builtin_amdgcn_readfirstlane(w.y);
+        RowStep st;  // uniform
+        __builtin_memcpy(&st, &w, sizeof st);
         if (st.op == F_RED_SUM || st.op == F_RED_MAX) {
             __syncthreads();  // the row register is complete
             const char *src = mine + st.a.idx * reg_bytes;
