@@ -195,6 +195,48 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
                     bias_r[j][q][e] = (g.bias != nullptr && n0 < g.N) ? g.bias[g.bias_len == 1 ? 0 : n0 + e] : 0.f;
             }
     }
+    if (EPI == 1) {
+        // fp16 result: a lane's four values are only eight bytes of a row, and a store instruction would touch 32 rows.
+        // The tile goes through shared memory instead (the operand buffers are free: the loop ended with a barrier)
+        // and leaves in 16-byte pieces, consecutive lanes along a row, so that every instruction writes whole lines.
+        constexpr int OPITCH = BN * 2 + 16;
+        static_assert(BM * OPITCH <= 2 * XBUF + 2 * WBUF, "the result tile fits in the operand buffers");
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            char *orow = smem + (wave_m * WM + i * 32 + (lane & 31)) * OPITCH;
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    // ADD in fp32 (one rounding), then CAST to fp16 (round to nearest even): the two operators that
+                    // follow the MATMUL in the unfused graph
+                    _Float16 h[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float sum = g.bias != nullptr ? acc[i][j][4 * q + e] + bias_r[j][q][e] : acc[i][j][4 * q + e];
+                        h[e] = (_Float16)sum;
+                    }
+                    uint2 v;
+                    v.x = (uint32_t)__builtin_bit_cast(unsigned short, h[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[1]) << 16);
+                    v.y = (uint32_t)__builtin_bit_cast(unsigned short, h[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[3]) << 16);
+                    *reinterpret_cast<uint2 *>(orow + (wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5)) * 2) = v;
+                }
+            }
+        }
+        __syncthreads();
+        constexpr int PPR = BN / 8;  // 16-byte pieces per row of the tile
+#pragma unroll
+        for (int p0 = 0; p0 < BM * PPR; p0 += NT) {
+            const int p = p0 + tid, r = p / PPR, c = p % PPR;
+            const int m = m_base + r, n = n_base + c * 8;
+            const uint4 piece = *reinterpret_cast<const uint4 *>(smem + r * OPITCH + c * 16);
+            const uint32_t off = (m < g.M && n < g.N) ? (uint32_t)m * g.ldo + (uint32_t)n * 2 : kOob;
+            v4i v;
+            v.x = (int)piece.x, v.y = (int)piece.y, v.z = (int)piece.z, v.w = (int)piece.w;
+            __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
@@ -204,30 +246,13 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const int n0 = n_base + wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
-                if (EPI == 0) {
-                    const uint32_t off = (row_off != kOob && n0 < g.N) ? row_off + (uint32_t)n0 * 4 : kOob;
-                    v4i v;
-                    v.x = __float_as_int(acc[i][j][4 * q + 0]);
-                    v.y = __float_as_int(acc[i][j][4 * q + 1]);
-                    v.z = __float_as_int(acc[i][j][4 * q + 2]);
-                    v.w = __float_as_int(acc[i][j][4 * q + 3]);
-                    __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
-                } else {
-                    // ADD in fp32 (one rounding), then CAST to fp16 (round to nearest even): the two operators that
-                    // follow the MATMUL in the unfused graph
-                    const uint32_t off = (row_off != kOob && n0 < g.N) ? row_off + (uint32_t)n0 * 2 : kOob;
-                    _Float16 h[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const float sum = g.bias != nullptr ? acc[i][j][4 * q + e] + bias_r[j][q][e] : acc[i][j][4 * q + e];
-                        h[e] = (_Float16)sum;
-                    }
-                    typedef int v2i_t __attribute__((ext_vector_type(2)));
-                    v2i_t v;
-                    v.x = (int)((uint32_t)__builtin_bit_cast(unsigned short, h[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[1]) << 16));
-                    v.y = (int)((uint32_t)__builtin_bit_cast(unsigned short, h[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[3]) << 16));
-                    __builtin_amdgcn_raw_buffer_store_b64(v, ores, (int)off, 0, 0);
-                }
+                const uint32_t off = (row_off != kOob && n0 < g.N) ? row_off + (uint32_t)n0 * 4 : kOob;
+                v4i v;
+                v.x = __float_as_int(acc[i][j][4 * q + 0]);
+                v.y = __float_as_int(acc[i][j][4 * q + 1]);
+                v.z = __float_as_int(acc[i][j][4 * q + 2]);
+                v.w = __float_as_int(acc[i][j][4 * q + 3]);
+                __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
             }
         }
     }
