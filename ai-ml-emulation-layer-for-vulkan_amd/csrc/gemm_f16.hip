@@ -337,11 +337,12 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
     g.bias = bias_cast && bias != nullptr ? static_cast<const float *>(bias->ptr) : nullptr;
     g.bias_len = bias_cast && bias != nullptr ? (int)numel(bias) : 0;
     // tile choice: the width with the least padding of N; the tall tile when it still gives every compute unit two
-    // blocks, otherwise the short one
+    // blocks and the contraction is long enough to matter (a K of a few steps is bound by the stores, which the
+    // short tile spreads over more blocks), otherwise the short one
     const int BN = ((N + 127) / 128) * 128 <= ((N + 63) / 64) * 64 ? 128 : 64;
     const int cus = ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
     const int64_t tiles_n = (N + BN - 1) / BN;
-    const bool tall = ((M + 127) / 128) * tiles_n * NB >= 2 * (int64_t)cus;
+    const bool tall = K > 128 && ((M + 127) / 128) * tiles_n * NB >= 2 * (int64_t)cus;
     const int BM = tall ? 128 : 64;
     g.tiles_m = (int)((M + BM - 1) / BM);
     g.tiles_n = (int)tiles_n;
