@@ -587,6 +587,59 @@ __global__ void __launch_bounds__(kBlock) transpose_tiles_kernel(const Transpose
     }
 }
 
+// The same for 2-byte elements when both moving extents are multiples of 8 and everything is 16-byte aligned: the
+// tile enters and leaves in 16-byte pieces (eight elements), the transposition happens in shared memory, where the
+// second phase gathers its eight elements from eight rows.
+__global__ void __launch_bounds__(kBlock) transpose_tiles_u16x8_kernel(const TransposeArgs a) {
+    constexpr int kPitch = 136;  // bytes per tile row: 8-byte aligned, eight rows apart land 16 banks apart
+    __shared__ __align__(16) char tile[64 * kPitch];
+    int64_t b = blockIdx.x;
+    const int64_t tj = b % a.tiles_j;
+    b /= a.tiles_j;
+    const int64_t ti = b % a.tiles_i;
+    int64_t batch = b / a.tiles_i;
+    const int last = a.rank - 1;
+    int64_t src = 0, dst = 0;
+    for (int k = last - 1; k >= 0; k--) {
+        if (k == a.q) continue;
+        const int64_t d = a.odims[k];
+        const int64_t o = batch % d;
+        batch /= d;
+        src += o * a.istride[k];
+        dst += o * a.ostride[k];
+    }
+    const int64_t i0 = ti * 64, j0 = tj * 64;  // i: output axis q = input last axis; j: output last axis
+    const int tid = threadIdx.x;
+    uint4 v[2];
+#pragma unroll
+    for (int k = 0; k < 2; k++) {  // tile row j (an input row), piece c of eight elements along i
+        const int p = tid + kBlock * k, j = p >> 3, c = p & 7;
+        v[k] = make_uint4(0, 0, 0, 0);
+        if (j0 + j < a.odims[last] && i0 + c * 8 < a.odims[a.q])
+            v[k] = *reinterpret_cast<const uint4 *>(a.in + src + (j0 + j) * a.istride[last] + (i0 + c * 8) * 2);
+    }
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const int p = tid + kBlock * k, j = p >> 3, c = p & 7;
+        *reinterpret_cast<uint2 *>(tile + j * kPitch + c * 16) = make_uint2(v[k].x, v[k].y);
+        *reinterpret_cast<uint2 *>(tile + j * kPitch + c * 16 + 8) = make_uint2(v[k].z, v[k].w);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 2; k++) {  // output row i, piece c of eight elements along j
+        const int p = tid + kBlock * k, i = p >> 3, c = p & 7;
+        if (i0 + i >= a.odims[a.q] || j0 + c * 8 >= a.odims[last]) continue;
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t lo = *reinterpret_cast<const uint16_t *>(tile + (c * 8 + 2 * e) * kPitch + i * 2);
+            const uint32_t hi = *reinterpret_cast<const uint16_t *>(tile + (c * 8 + 2 * e + 1) * kPitch + i * 2);
+            w[e] = lo | (hi << 16);
+        }
+        *reinterpret_cast<uint4 *>(a.out + dst + (i0 + i) * a.ostride[a.q] + (j0 + c * 8) * 2) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
 }  // namespace
 
 int try_transpose_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
@@ -646,7 +699,11 @@ int try_transpose_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     const int64_t blocks = a.tiles_i * a.tiles_j * a.batches;
     MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "transpose: too many tiles");
     const dim3 grid((unsigned)blocks), block(kBlock);
-    if (esize == 1)
+    const bool pieces = esize == 2 && out->dims[q] % 8 == 0 && out->dims[last] % 8 == 0 && in->dims[last] % 8 == 0 &&
+                        ((uintptr_t)in->ptr % 16) == 0 && ((uintptr_t)out->ptr % 16) == 0;
+    if (pieces)
+        transpose_tiles_u16x8_kernel<<<grid, block, 0, s>>>(a);
+    else if (esize == 1)
         transpose_tiles_kernel<uint8_t><<<grid, block, 0, s>>>(a);
     else if (esize == 2)
         transpose_tiles_kernel<uint16_t><<<grid, block, 0, s>>>(a);

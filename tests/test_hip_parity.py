@@ -389,7 +389,7 @@ def _same_bits_or_both_nan(got, want):
     np.testing.assert_array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
 
 
-@pytest.mark.parametrize("shape", [(2, 48, 768), (5, 1, 64), (300, 8), (3, 2048), (1, 1, 4096)], ids=str)
+@pytest.mark.parametrize("shape", [(2, 48, 768), (5, 1, 64), (300, 8), (3, 2048), (1, 1, 4096), (16384, 768), (777, 1016)], ids=str)
 def test_chain_with_reductions_layernorm(run, shape):
     """LayerNorm as the operators a TOSA graph spells it with (REDUCE_SUM, MUL 1/N, SUB, MUL, REDUCE_SUM, MUL 1/N,
     ADD eps, RSQRT, MUL, MUL gamma, ADD beta), in one mlel_hip_elementwise_chain call against the eleven stand-alone
@@ -706,7 +706,10 @@ def test_transpose_fast_paths_vs_numpy(run, oracle):
     cases = [((2, 5, 12, 64), (0, 2, 1, 3), np.float16), ((2, 7, 3, 40), (0, 2, 3, 1), np.float16),
              ((3, 70, 130), (0, 2, 1), np.int8), ((65, 67), (1, 0), np.int32), ((4, 33, 9), (2, 0, 1), np.float32),
              ((2, 3, 4, 5, 16), (3, 1, 0, 2, 4), np.int16), ((6, 128, 64), (0, 2, 1), np.float16),
-             ((2, 16, 4, 8), (0, 2, 1, 3), np.int8), ((1, 1, 200), (2, 1, 0), np.int8)]
+             ((2, 16, 4, 8), (0, 2, 1, 3), np.int8), ((1, 1, 200), (2, 1, 0), np.int8),
+             # 2-byte elements, both moving extents in multiples of eight: the 16-byte-piece tile kernel, partial tiles
+             ((2, 72, 3, 40), (0, 2, 3, 1), np.float16), ((3, 136, 200), (0, 2, 1), np.int16), ((8, 8), (1, 0), np.float16),
+             ((2, 512, 12, 64), (0, 2, 3, 1), np.float16)]
     for shape, perms, dt in cases:
         x = (rng.standard_normal(shape) * 50).astype(dt)
         got = run.transpose(x, perms)
