@@ -248,6 +248,7 @@ FUSED_SIGNATURES = {
     "matmul_rescale": [_T, _T, _T, C.POINTER(MatmulAttr), C.POINTER(Epilogue)],
     "dwconv_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
     "matmul_bias_cast": [_T, _T, _T, _T, C.POINTER(MatmulAttr)],
+    "matmul_bias_cast_add": [_T, _T, _T, _T, C.POINTER(MatmulAttr), _T],
     "softmax_rows": [_T, _T],
     "elementwise_chain": [_T, C.POINTER(Chain)],
     "rescale_add_rescale": [_T, _T, C.POINTER(Epilogue), _T, C.POINTER(Epilogue), C.POINTER(Epilogue)],

@@ -701,6 +701,30 @@ int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *ou
     return 0;
 }
 
+int mlel_hip_matmul_bias_cast_add(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
+                                  const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr,
+                                  const mlel_tensor *residual) {
+    MLEL_TRY(require_ctx(ctx, "matmul_bias_cast_add"));
+    MLEL_REQUIRE(attr != nullptr && residual != nullptr, MLEL_ERR_INVALID, "matmul_bias_cast_add: null argument");
+    MLEL_TRY(check_supported(out, "matmul_bias_cast_add out"));
+    MLEL_TRY(check_supported(residual, "matmul_bias_cast_add residual"));
+    MLEL_REQUIRE(out->rank == 3 && residual->dtype == MLEL_F16 && out->dtype == MLEL_F16 && same_shape(out, residual),
+                 MLEL_ERR_INVALID, "matmul_bias_cast_add: the residual is an fp16 tensor of the output's shape");
+    if (a != nullptr && b != nullptr && a->dtype == MLEL_F16 && b->dtype == MLEL_F16 && a->rank == 3 && b->rank == 3 &&
+        (bias == nullptr || (bias->dtype == MLEL_F32 && bias->rank == 3))) {
+        const int rc = try_matmul_f16_mfma(ctx, (hipStream_t)stream, out, a, b, attr, true, bias, residual);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
+    // no fused kernel for these strides / alignments: the projection into a temporary, then the addition
+    Scratch proj_mem;
+    MLEL_HIP_CHECK(hipMalloc(&proj_mem.ptr, (size_t)numel(out) * 2 + 16));
+    const mlel_tensor proj = packed_like(out, MLEL_F16, proj_mem.ptr);
+    MLEL_TRY(mlel_hip_matmul_bias_cast(ctx, stream, &proj, a, b, bias, attr));
+    MLEL_TRY(mlel_hip_elementwise_binary(ctx, stream, MLEL_BIN_ADD, out, &proj, residual, MLEL_NAN_PROPAGATE));
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
 int mlel_hip_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
                                   const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv2d_attr *attr,
                                   const mlel_epilogue *epi) {

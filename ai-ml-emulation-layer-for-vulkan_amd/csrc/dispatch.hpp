@@ -105,9 +105,10 @@ int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
                        const mlel_tensor *b, const mlel_matmul_attr *attr, const FusedEpilogue *epi);
 
 // ---- fp16 MFMA MATMUL with fp32 result (gemm_f16.hip) ----
+// `residual`: an fp16 tensor of the output's shape added to the fused form's fp16 result (a second, fp16 ADD)
 int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
                         const mlel_tensor *b, const mlel_matmul_attr *attr, bool bias_cast = false,
-                        const mlel_tensor *bias = nullptr);
+                        const mlel_tensor *bias = nullptr, const mlel_tensor *residual = nullptr);
 
 // ---- floating-point elementwise / reduce specialisations (ops_float.hip) ----
 int try_binary_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in1,

@@ -39,6 +39,10 @@ struct HGemmArgs {
     // fused epilogue (EPI = 1): out = fp16(acc + bias[n]) with the addition in fp32; bias may be null
     const float *bias;
     int32_t bias_len;  // 1 (broadcast) or N
+    // fp16 tensor of the output's shape added to the rounded result (the ADD of a residual connection), or null
+    const char *res;
+    int64_t r_batch;
+    uint32_t ldr, r_bytes;
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const void *p, uint32_t bytes) {
@@ -224,13 +228,23 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
             }
         }
         __syncthreads();
+        const __amdgpu_buffer_rsrc_t rres = rsrc(g.res != nullptr ? g.res + (int64_t)batch * g.r_batch : g.out, g.res != nullptr ? g.r_bytes : 0);
         constexpr int PPR = BN / 8;  // 16-byte pieces per row of the tile
 #pragma unroll
         for (int p0 = 0; p0 < BM * PPR; p0 += NT) {
             const int p = p0 + tid, r = p / PPR, c = p % PPR;
             const int m = m_base + r, n = n_base + c * 8;
-            const uint4 piece = *reinterpret_cast<const uint4 *>(smem + r * OPITCH + c * 16);
-            const uint32_t off = (m < g.M && n < g.N) ? (uint32_t)m * g.ldo + (uint32_t)n * 2 : kOob;
+            uint4 piece = *reinterpret_cast<const uint4 *>(smem + r * OPITCH + c * 16);
+            const bool inside = m < g.M && n < g.N;
+            const uint32_t off = inside ? (uint32_t)m * g.ldo + (uint32_t)n * 2 : kOob;
+            if (g.res != nullptr) {  // uniform; ADD of two fp16 tensors: one rounding of the exact sum
+                const uint4 other = load16(rres, inside ? (uint32_t)m * g.ldr + (uint32_t)n * 2 : kOob);
+                typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+                h2_t *ph = reinterpret_cast<h2_t *>(&piece);
+                const h2_t *oh = reinterpret_cast<const h2_t *>(&other);
+#pragma unroll
+                for (int e = 0; e < 4; e++) ph[e] = ph[e] + oh[e];
+            }
             v4i v;
             v.x = (int)piece.x, v.y = (int)piece.y, v.z = (int)piece.z, v.w = (int)piece.w;
             __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
@@ -291,7 +305,16 @@ bool dense_rows(const mlel_tensor *t) { return t->strides[2] == 2 && t->strides[
 
 // `bias_cast` set: the fused form out(fp16) = CAST(MATMUL + bias) with an fp32 bias of length 1 or N (or none)
 int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
-                        const mlel_tensor *b, const mlel_matmul_attr *attr, bool bias_cast, const mlel_tensor *bias) {
+                        const mlel_tensor *b, const mlel_matmul_attr *attr, bool bias_cast, const mlel_tensor *bias,
+                        const mlel_tensor *residual) {
+    if (residual != nullptr) {
+        if (!bias_cast || residual->dtype != MLEL_F16 || residual->rank != 3 || !same_shape(residual, out)) return 0;
+        if (residual->strides[2] != 2 || ((uintptr_t)residual->ptr % 16) != 0 || residual->strides[0] % 16 != 0 ||
+            residual->strides[1] % 16 != 0)
+            return 0;
+        const int64_t rb = residual->dims[1] * residual->strides[1];
+        if (rb >= (int64_t(1) << 31) - 64 || residual->strides[1] < residual->dims[2] * 2) return 0;
+    }
     if (a->dtype != MLEL_F16 || b->dtype != MLEL_F16 || out->dtype != (bias_cast ? MLEL_F16 : MLEL_F32)) return 0;
     const int osize = bias_cast ? 2 : 4;
     if (bias_cast && bias != nullptr) {
@@ -336,6 +359,12 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
     g.o_bytes = (uint32_t)ob;
     g.bias = bias_cast && bias != nullptr ? static_cast<const float *>(bias->ptr) : nullptr;
     g.bias_len = bias_cast && bias != nullptr ? (int)numel(bias) : 0;
+    if (residual != nullptr) {
+        g.res = static_cast<const char *>(residual->ptr);
+        g.r_batch = residual->strides[0];
+        g.ldr = (uint32_t)residual->strides[1];
+        g.r_bytes = (uint32_t)(residual->dims[1] * residual->strides[1]);
+    }
     // tile choice: the width with the least padding of N; the tall tile when it still gives every compute unit two
     // blocks and the contraction is long enough to matter (a K of a few steps is bound by the stores, which the
     // short tile spreads over more blocks), otherwise the short one

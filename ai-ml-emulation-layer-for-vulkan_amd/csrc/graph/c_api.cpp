@@ -285,7 +285,8 @@ std::string opLabel(const OpNode &op) {
         for (const auto &st : op.chain) reduces = reduces || st.kind == MLEL_CHAIN_REDUCE;
         return (reduces ? "ELEMENTWISE+REDUCE x" : "ELEMENTWISE x") + std::to_string(op.chain.size());
     }
-    case OpKind::FusedMatmulBiasCast: return op.inputs.size() > 2 ? "MATMUL+ADD+CAST" : "MATMUL+CAST";
+    case OpKind::FusedMatmulBiasCast:
+        return std::string(op.hasBias ? "MATMUL+ADD+CAST" : "MATMUL+CAST") + (op.flag ? "+ADD" : "");
     default: return op.tosaName;
     }
 }

@@ -754,10 +754,45 @@ void GraphPipeline::fuse() {
             continue;
         mm.kind = OpKind::FusedMatmulBiasCast;
         if (bias) mm.inputs.push_back(bias);
+        mm.hasBias = bias != nullptr;
         mm.outputs[0] = cast->outputs[0];
         cast->outputs[0]->setProducer(&mm);
         cast->fusedAway = true;
         if (add) add->fusedAway = true;
+    }
+
+    // Pattern 4d (residual connection behind an fp16 projection): the fp16 result of the pattern above, private and
+    // read only by an fp16 ADD whose other operand has the same shape and exists before the projection runs, takes
+    // that addition into the projection's epilogue (mlel_hip_matmul_bias_cast_add).
+    for (size_t at = 0; at < ops.size(); at++) {
+        OpNode &mm = *ops[at];
+        if (mm.fusedAway || mm.kind != OpKind::FusedMatmulBiasCast || mm.flag) continue;
+        TensorPtr h = mm.outputs[0];
+        if (!isPrivateIntermediate(*h)) continue;
+        auto users = consumersOf(ops, h.get());
+        // a RESHAPE in between only renames the extents of the same packed bytes ([1, rows, N] -> [batch, seq, N])
+        OpNode *reshape = nullptr;
+        if (users.size() == 1 && users[0]->kind == OpKind::Reshape && isPrivateIntermediate(*users[0]->outputs[0]) &&
+            users[0]->outputs[0]->getFormat() == MLEL_F16 && users[0]->outputs[0]->getSize() == h->getSize()) {
+            reshape = users[0];
+            h = reshape->outputs[0];
+            users = consumersOf(ops, h.get());
+        }
+        if (users.size() != 1 || users[0]->kind != OpKind::Binary || users[0]->selector != MLEL_BIN_ADD) continue;
+        OpNode *add = users[0];
+        const TensorPtr other = add->inputs[add->inputs[0].get() == h.get() ? 1 : 0];
+        if (other.get() == h.get() || other->getFormat() != MLEL_F16 || !sameShape(*other, *h) || !other->isPacked() ||
+            add->outputs[0]->getFormat() != MLEL_F16 || !sameShape(*add->outputs[0], *h) || !add->outputs[0]->isPacked())
+            continue;
+        bool early = other->getProducer() == nullptr;
+        for (size_t k = 0; k < at && !early; k++) early = ops[k].get() == other->getProducer();
+        if (!early) continue;
+        mm.inputs.push_back(other);
+        mm.flag = true;
+        mm.outputs[0] = add->outputs[0];
+        add->outputs[0]->setProducer(&mm);
+        add->fusedAway = true;
+        if (reshape) reshape->fusedAway = true;
     }
 
     // Pattern 5: regions of floating-point elementwise operators (ADD, SUB, MUL, EXP, RECIPROCAL, RSQRT, TANH, CAST
@@ -1294,10 +1329,25 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
         rc = mlel_hip_elementwise_chain(ctx, stream, &out, &c);
         break;
     }
-    case OpKind::FusedMatmulBiasCast:
-        rc = mlel_hip_matmul_bias_cast(ctx, stream, &out, &in[0], &in[1], op.inputs.size() > 2 ? &in[2] : nullptr,
-                                       &op.matmul);
+    case OpKind::FusedMatmulBiasCast: {
+        const mlel_tensor *bias = op.hasBias ? &in[2] : nullptr;
+        if (op.flag) {
+            // the addition may have been written with other extents over the same packed bytes: both tensors are
+            // handed over with the product's extents [batches, rows, columns]
+            const auto as_product = [&](mlel_tensor t) {
+                t.rank = 3;
+                t.dims[0] = in[0].dims[0], t.dims[1] = in[0].dims[1], t.dims[2] = in[1].dims[2];
+                t.strides[2] = 2;
+                t.strides[1] = t.dims[2] * 2;
+                t.strides[0] = t.dims[1] * t.strides[1];
+                return t;
+            };
+            const mlel_tensor out3 = as_product(out), res3 = as_product(in[op.inputs.size() - 1]);
+            rc = mlel_hip_matmul_bias_cast_add(ctx, stream, &out3, &in[0], &in[1], bias, &op.matmul, &res3);
+        } else
+            rc = mlel_hip_matmul_bias_cast(ctx, stream, &out, &in[0], &in[1], bias, &op.matmul);
         break;
+    }
     case OpKind::FusedConv2DResidual: {
         const mlel_tensor mult = op.epilogue.multiplier->view(), shift = op.epilogue.shift->view();
         const mlel_tensor ma = op.scaleA.multiplier->view(), sa = op.scaleA.shift->view();

@@ -135,6 +135,8 @@ class OpNode {
     bool fusedAway = false;          // folded into another node; not executed
     RescaleSpec epilogue;            // Fused*: RESCALE applied to the accumulator
     bool hasClamp = false;           // Fused*: CLAMP after the RESCALE
+    bool hasBias = false;            // FusedMatmulBiasCast: inputs[2] is the fp32 bias; `flag`: the last input is an
+                                     // fp16 residual added to the rounded result
     RescaleSpec scaleA, scaleB;      // FusedRescaleAddRescale: the two input stages (epilogue = output stage)
     // FusedConv2DResidual: epilogue (+ clamp) belongs to the convolution; scaleA rescales its 8-bit result, scaleB the
     // residual (inputs[3]), scaleOut their sum; `flag` is set when the residual was the addition's first operand

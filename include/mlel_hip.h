@@ -405,6 +405,12 @@ int mlel_hip_softmax_rows(mlel_ctx *ctx, void *stream, const mlel_tensor *out, c
  * NULL) added in fp32, one rounding to fp16 -- bit for bit the unfused MATMUL -> ADD -> CAST (or MATMUL -> CAST). */
 int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                               const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr);
+/* The same followed by the ADD of a residual connection: out(fp16) = ADD( CAST( MATMUL(a, b) + bias ), residual ),
+ * `residual` an fp16 tensor of the output's shape; the second addition is an fp16 ADD (one rounding of the exact sum
+ * of two halfs), as the stand-alone operator computes it. */
+int mlel_hip_matmul_bias_cast_add(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
+                                  const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr,
+                                  const mlel_tensor *residual);
 int mlel_hip_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
                                   const mlel_tensor *weights, const mlel_tensor *bias,
                                   const mlel_conv2d_attr *attr, const mlel_epilogue *epi);

@@ -235,6 +235,16 @@ class Runner:
         self.done()
         return r
 
+    def matmul_bias_cast_add(self, a, b, bias, residual):
+        ta, tb, tr = self.put(a), self.put(b), self.put(residual)
+        tbias = self.put(bias) if bias is not None else None
+        to = self.new(abi.F16, (a.shape[0], a.shape[1], b.shape[2]))
+        self.dev.op("matmul_bias_cast_add", to.ref, ta.ref, tb.ref, tbias.ref if tbias else None,
+                    C.byref(abi.MatmulAttr(0, 0)), tr.ref)
+        r = to.download()
+        self.done()
+        return r
+
     def chain(self, inputs, steps, out_shape, out_dtype):
         """steps: (kind, selector, a, b, dtype) tuples as in mlel_chain_step."""
         tin = [self.put(x) for x in inputs]

@@ -198,4 +198,5 @@ def test_transformer_block_fusions_do_not_change_a_bit(dev):
     np.testing.assert_array_equal(outs[True][0].view(np.uint16), outs[False][0].view(np.uint16))
     assert outs[True][1].count("ELEMENTWISE+REDUCE x7") == 1      # MUL by 1/sqrt(d), then the six softmax operators
     assert outs[True][1].count("ELEMENTWISE+REDUCE x11") == 2     # the two LayerNorms
+    assert outs[True][1].count("MATMUL+ADD+CAST+ADD") == 2        # both residual connections ride on their projection
     assert not [n for n in outs[True][1] if n.startswith("REDUCE_")] and len(outs[True][1]) < len(outs[False][1])

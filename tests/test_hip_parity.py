@@ -334,6 +334,11 @@ def test_matmul_bias_cast_equals_the_three_operators(run, oracle, case):
         np.testing.assert_array_equal(fused, unfused)
         exp = oracle.matmul(a, b, abi.F32) + (bias if bias is not None else 0)
         assert np.abs(fused.astype(np.float32) - exp).max() <= 1e-2
+        # ... followed by the ADD of a residual connection (an fp16 tensor of the output's shape) in the same launch
+        res = rng.standard_normal((nb, m, n)).astype(np.float16)
+        res[0, 0, :2] = [np.float16(-0.0), np.float16(6e-8)]
+        with_res = run.matmul_bias_cast_add(a, b, bias, res)
+        np.testing.assert_array_equal(with_res.view(np.uint16), run.binary("ADD", unfused, res, res.shape, abi.F16).view(np.uint16))
 
 
 def test_elementwise_chain_equals_the_operators_one_by_one(run):
