@@ -677,12 +677,29 @@ int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *ou
     MLEL_TRY(check_supported(a, "matmul_bias_cast a"));
     MLEL_TRY(check_supported(b, "matmul_bias_cast b"));
     if (bias) MLEL_TRY(check_supported(bias, "matmul_bias_cast bias"));
-    MLEL_REQUIRE(out->rank == 3 && a->rank == 3 && b->rank == 3, MLEL_ERR_INVALID, "matmul_bias_cast: rank must be 3");
+    MLEL_REQUIRE((out->rank == 3 || out->rank == 6) && a->rank == 3 && b->rank == 3, MLEL_ERR_INVALID,
+                 "matmul_bias_cast: operands of rank 3, output of rank 3 or a six-dimensional view");
     MLEL_REQUIRE(a->dtype == MLEL_F16 && b->dtype == MLEL_F16 && out->dtype == MLEL_F16 &&
                      (bias == nullptr || (bias->dtype == MLEL_F32 && bias->rank == 3)),
                  MLEL_ERR_INVALID, "matmul_bias_cast: fp16 operands and output, fp32 bias of rank 3");
     const int rc = try_matmul_f16_mfma(ctx, (hipStream_t)stream, out, a, b, attr, true, bias);
     if (rc != 0) return rc < 0 ? rc : 0;
+    if (out->rank == 6) {
+        // the view without the fused kernel: the product into a dense temporary, then a strided copy
+        Scratch dense_mem;
+        MLEL_HIP_CHECK(hipMalloc(&dense_mem.ptr, (size_t)numel(out) * 2 + 16));
+        mlel_tensor dense3 = *out;
+        dense3.rank = 3;
+        dense3.dims[0] = out->dims[0] * out->dims[1];
+        dense3.dims[1] = out->dims[2] * out->dims[3];
+        dense3.dims[2] = out->dims[4] * out->dims[5];
+        dense3 = packed_like(&dense3, MLEL_F16, dense_mem.ptr);
+        MLEL_TRY(mlel_hip_matmul_bias_cast(ctx, stream, &dense3, a, b, bias, attr));
+        const mlel_tensor dense6 = packed_like(out, MLEL_F16, dense_mem.ptr);
+        MLEL_TRY(mlel_hip_cast(ctx, stream, out, &dense6));
+        MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+        return 0;
+    }
     // no fused kernel for these strides / alignments: the three operators one after another through temporaries
     Scratch acc_mem, sum_mem;
     MLEL_HIP_CHECK(hipMalloc(&acc_mem.ptr, (size_t)numel(out) * 4 + 16));

@@ -43,6 +43,12 @@ struct HGemmArgs {
     const char *res;
     int64_t r_batch;
     uint32_t ldr, r_bytes;
+    // fp16 result written through a six-dimensional view [NB1, NB2, M1, M2, N1, N2] of other strides (a head split
+    // or merge behind the product): batch = nb1 * NB2 + nb2, row = m1 * M2 + m2, column = n1 * N2 + n2 with eight
+    // consecutive n2 contiguous.  view == 0: the plain [batch][row][column] layout above.
+    int32_t view, v_nb2, v_m2, v_n2;
+    int64_t vs_nb1, vs_nb2;
+    uint32_t vs_m1, vs_m2, vs_n1;
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const void *p, uint32_t bytes) {
@@ -184,7 +190,9 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
     }
 
     // ---- store: lane holds row m = lane % 32 of each sub-tile and, per register quad q, columns 8q + 4 * (lane / 32)
-    const __amdgpu_buffer_rsrc_t ores = rsrc(g.out + (int64_t)batch * g.o_batch, g.o_bytes);
+    const int64_t o_base = g.view ? (int64_t)(batch / g.v_nb2) * g.vs_nb1 + (int64_t)(batch % g.v_nb2) * g.vs_nb2
+                                  : (int64_t)batch * g.o_batch;
+    const __amdgpu_buffer_rsrc_t ores = rsrc(g.out + o_base, g.o_bytes);
     // the bias of this lane's columns, fetched in one batch before any store (a load after a store would have to
     // wait for it: the compiler cannot tell that the two do not alias)
     float bias_r[TN][4][4];
@@ -236,7 +244,10 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
             const int m = m_base + r, n = n_base + c * 8;
             uint4 piece = *reinterpret_cast<const uint4 *>(smem + r * OPITCH + c * 16);
             const bool inside = m < g.M && n < g.N;
-            const uint32_t off = inside ? (uint32_t)m * g.ldo + (uint32_t)n * 2 : kOob;
+            uint32_t off = inside ? (uint32_t)m * g.ldo + (uint32_t)n * 2 : kOob;
+            if (g.view && inside)  // uniform
+                off = (uint32_t)(m / g.v_m2) * g.vs_m1 + (uint32_t)(m % g.v_m2) * g.vs_m2 + (uint32_t)(n / g.v_n2) * g.vs_n1 +
+                      (uint32_t)(n % g.v_n2) * 2;
             if (g.res != nullptr) {  // uniform; ADD of two fp16 tensors: one rounding of the exact sum
                 const uint4 other = load16(rres, inside ? (uint32_t)m * g.ldr + (uint32_t)n * 2 : kOob);
                 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
@@ -316,6 +327,29 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
         if (rb >= (int64_t(1) << 31) - 64 || residual->strides[1] < residual->dims[2] * 2) return 0;
     }
     if (a->dtype != MLEL_F16 || b->dtype != MLEL_F16 || out->dtype != (bias_cast ? MLEL_F16 : MLEL_F32)) return 0;
+    // a six-dimensional output is a strided view [NB1, NB2, M1, M2, N1, N2] of the product (fused fp16 form only)
+    mlel_tensor plain_out;
+    const mlel_tensor *view = nullptr;
+    if (out->rank == 6) {
+        if (!bias_cast || residual != nullptr) return 0;
+        view = out;
+        plain_out = *out;
+        plain_out.rank = 3;
+        plain_out.dims[0] = out->dims[0] * out->dims[1];
+        plain_out.dims[1] = out->dims[2] * out->dims[3];
+        plain_out.dims[2] = out->dims[4] * out->dims[5];
+        plain_out.strides[2] = 2;
+        plain_out.strides[1] = plain_out.dims[2] * 2;
+        plain_out.strides[0] = plain_out.dims[1] * plain_out.strides[1];
+        out = &plain_out;  // extents for the checks below; the addresses come from the view
+        if (view->strides[5] != 2 || view->dims[5] % 8 != 0) return 0;
+        int64_t span = view->dims[5] * 2;
+        for (int i = 0; i < 5; i++) {
+            if (view->strides[i] % 16 != 0 || view->strides[i] < 0) return 0;
+            if (i >= 2) span += (view->dims[i] - 1) * view->strides[i];
+        }
+        if (span >= (int64_t(1) << 31) - 64) return 0;
+    }
     const int osize = bias_cast ? 2 : 4;
     if (bias_cast && bias != nullptr) {
         const int64_t n = numel(bias);
@@ -359,6 +393,20 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
     g.o_bytes = (uint32_t)ob;
     g.bias = bias_cast && bias != nullptr ? static_cast<const float *>(bias->ptr) : nullptr;
     g.bias_len = bias_cast && bias != nullptr ? (int)numel(bias) : 0;
+    if (view != nullptr) {
+        g.view = 1;
+        g.v_nb2 = (int32_t)view->dims[1];
+        g.v_m2 = (int32_t)view->dims[3];
+        g.v_n2 = (int32_t)view->dims[5];
+        g.vs_nb1 = view->strides[0];
+        g.vs_nb2 = view->strides[1];
+        g.vs_m1 = (uint32_t)view->strides[2];
+        g.vs_m2 = (uint32_t)view->strides[3];
+        g.vs_n1 = (uint32_t)view->strides[4];
+        int64_t span = view->dims[5] * 2;
+        for (int i = 2; i < 5; i++) span += (view->dims[i] - 1) * view->strides[i];
+        g.o_bytes = (uint32_t)span;
+    }
     if (residual != nullptr) {
         g.res = static_cast<const char *>(residual->ptr);
         g.r_batch = residual->strides[0];

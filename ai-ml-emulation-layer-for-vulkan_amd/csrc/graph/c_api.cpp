@@ -286,7 +286,8 @@ std::string opLabel(const OpNode &op) {
         return (reduces ? "ELEMENTWISE+REDUCE x" : "ELEMENTWISE x") + std::to_string(op.chain.size());
     }
     case OpKind::FusedMatmulBiasCast:
-        return std::string(op.hasBias ? "MATMUL+ADD+CAST" : "MATMUL+CAST") + (op.flag ? "+ADD" : "");
+        return std::string(op.hasBias ? "MATMUL+ADD+CAST" : "MATMUL+CAST") + (op.flag ? "+ADD" : "") +
+               (op.viewDims[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");
     default: return op.tosaName;
     }
 }

@@ -761,12 +761,79 @@ void GraphPipeline::fuse() {
         if (add) add->fusedAway = true;
     }
 
+    // Pattern 4e (head split / merge behind an fp16 product): the fp16 result [NB, M, N], private, read only by a
+    // RESHAPE that splits each of NB, M, N into at most two extents, itself read only by a TRANSPOSE that keeps the
+    // innermost extent innermost.  The product then writes the transposed tensor directly, through a strided view
+    // (mlel_hip_matmul_bias_cast with a six-dimensional output); the two data-movement operators disappear.
+    for (const auto &opPtr : ops) {
+        OpNode &mm = *opPtr;
+        if (mm.fusedAway || mm.kind != OpKind::FusedMatmulBiasCast || mm.flag) continue;
+        const TensorPtr h = mm.outputs[0];
+        if (!isPrivateIntermediate(*h) || h->getRank() != 3) continue;
+        auto users = consumersOf(ops, h.get());
+        if (users.size() != 1 || users[0]->kind != OpKind::Reshape) continue;
+        OpNode *reshape = users[0];
+        const TensorPtr split = reshape->outputs[0];
+        if (!isPrivateIntermediate(*split) || split->getFormat() != MLEL_F16) continue;
+        users = consumersOf(ops, split.get());
+        if (users.size() != 1 || users[0]->kind != OpKind::Transpose) continue;
+        OpNode *transpose = users[0];
+        const TensorPtr moved = transpose->outputs[0];
+        if (moved->getFormat() != MLEL_F16 || !moved->isPacked() || moved->getRank() != split->getRank()) continue;
+        // the split extents, in order, grouped by the product extent they come from (extents of 1 address nothing)
+        const auto &sd = split->getDimensions();
+        const auto &hd = h->getDimensions();
+        std::array<std::vector<size_t>, 3> groups;
+        size_t at = 0;
+        bool ok = true;
+        for (int part = 0; part < 3 && ok; part++) {
+            int64_t product = 1;
+            while (product < hd[static_cast<size_t>(part)] && at < sd.size()) {
+                if (sd[at] != 1) groups[static_cast<size_t>(part)].push_back(at);
+                product *= sd[at++];
+            }
+            ok = product == hd[static_cast<size_t>(part)] && groups[static_cast<size_t>(part)].size() <= 2;
+        }
+        for (; at < sd.size() && ok; at++) ok = sd[at] == 1;
+        if (!ok || groups[2].empty()) continue;
+        // byte strides of the split extents inside the (packed) transposed tensor
+        const size_t rank = sd.size();
+        std::vector<int64_t> movedStride(rank), splitStride(rank);
+        int64_t stride = 2;
+        for (size_t k = rank; k-- > 0;) {
+            movedStride[k] = stride;
+            stride *= moved->getDimensions()[k];
+        }
+        for (size_t k = 0; k < rank; k++) splitStride[transpose->vec[k]] = movedStride[k];
+        std::array<int64_t, 6> vd{}, vs{};
+        for (size_t part = 0; part < 3; part++) {
+            const auto &gr = groups[part];
+            // one extent: (extent, 1); two: (outer, inner); none (the product extent is 1): (1, 1)
+            vd[2 * part] = gr.empty() ? 1 : sd[gr[0]];
+            vs[2 * part] = gr.empty() ? 0 : splitStride[gr[0]];
+            vd[2 * part + 1] = gr.size() == 2 ? sd[gr[1]] : 1;
+            vs[2 * part + 1] = gr.size() == 2 ? splitStride[gr[1]] : 0;
+        }
+        if (groups[2].size() == 1) {  // the columns were not split: they are the inner extent
+            vd[5] = vd[4], vs[5] = vs[4];
+            vd[4] = 1, vs[4] = 0;
+        }
+        bool aligned = vs[5] == 2 && vd[5] % 8 == 0;
+        for (size_t k = 0; k < 5; k++) aligned = aligned && vs[k] % 16 == 0;
+        if (!aligned) continue;
+        mm.viewDims = vd;
+        mm.viewStrides = vs;
+        mm.outputs[0] = moved;
+        moved->setProducer(&mm);
+        reshape->fusedAway = transpose->fusedAway = true;
+    }
+
     // Pattern 4d (residual connection behind an fp16 projection): the fp16 result of the pattern above, private and
     // read only by an fp16 ADD whose other operand has the same shape and exists before the projection runs, takes
     // that addition into the projection's epilogue (mlel_hip_matmul_bias_cast_add).
     for (size_t at = 0; at < ops.size(); at++) {
         OpNode &mm = *ops[at];
-        if (mm.fusedAway || mm.kind != OpKind::FusedMatmulBiasCast || mm.flag) continue;
+        if (mm.fusedAway || mm.kind != OpKind::FusedMatmulBiasCast || mm.flag || mm.viewDims[5] != 0) continue;
         TensorPtr h = mm.outputs[0];
         if (!isPrivateIntermediate(*h)) continue;
         auto users = consumersOf(ops, h.get());
@@ -1344,8 +1411,17 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
             };
             const mlel_tensor out3 = as_product(out), res3 = as_product(in[op.inputs.size() - 1]);
             rc = mlel_hip_matmul_bias_cast_add(ctx, stream, &out3, &in[0], &in[1], bias, &op.matmul, &res3);
-        } else
+        } else if (op.viewDims[5] != 0) {
+            mlel_tensor view = out;  // the transposed tensor's storage, addressed with the product's split extents
+            view.rank = 6;
+            for (size_t k = 0; k < 6; k++) {
+                view.dims[k] = op.viewDims[k];
+                view.strides[k] = op.viewStrides[k];
+            }
+            rc = mlel_hip_matmul_bias_cast(ctx, stream, &view, &in[0], &in[1], bias, &op.matmul);
+        } else {
             rc = mlel_hip_matmul_bias_cast(ctx, stream, &out, &in[0], &in[1], bias, &op.matmul);
+        }
         break;
     }
     case OpKind::FusedConv2DResidual: {

@@ -137,6 +137,9 @@ class OpNode {
     bool hasClamp = false;           // Fused*: CLAMP after the RESCALE
     bool hasBias = false;            // FusedMatmulBiasCast: inputs[2] is the fp32 bias; `flag`: the last input is an
                                      // fp16 residual added to the rounded result
+    // FusedMatmulBiasCast whose result is written through a view [NB1, NB2, M1, M2, N1, N2] of the output tensor's
+    // storage (a RESHAPE -> TRANSPOSE behind the product folded into its stores); extents 0: no view
+    std::array<int64_t, 6> viewDims{}, viewStrides{};
     RescaleSpec scaleA, scaleB;      // FusedRescaleAddRescale: the two input stages (epilogue = output stage)
     // FusedConv2DResidual: epilogue (+ clamp) belongs to the convolution; scaleA rescales its 8-bit result, scaleB the
     // residual (inputs[3]), scaleOut their sum; `flag` is set when the residual was the addition's first operand

@@ -235,6 +235,24 @@ class Runner:
         self.done()
         return r
 
+    def matmul_bias_cast_view(self, a, b, bias, split_shape, perms):
+        """The product written through the view that RESHAPE(split_shape) -> TRANSPOSE(perms) behind it amounts to;
+        split_shape has six extents [NB1, NB2, M1, M2, N1, N2].  Returns the transposed tensor."""
+        ta, tb = self.put(a), self.put(b)
+        tbias = self.put(bias) if bias is not None else None
+        moved_shape = tuple(split_shape[p] for p in perms)
+        to = self.new(abi.F16, moved_shape)
+        moved_strides = abi.packed_strides(moved_shape, 2)
+        strides = [0] * 6
+        for k, p in enumerate(perms):
+            strides[p] = moved_strides[k]
+        view = abi.make_tensor(to.view.ptr, abi.F16, split_shape, strides)
+        self.dev.op("matmul_bias_cast", C.byref(view), ta.ref, tb.ref, tbias.ref if tbias else None,
+                    C.byref(abi.MatmulAttr(0, 0)))
+        r = to.download()
+        self.done()
+        return r
+
     def matmul_bias_cast_add(self, a, b, bias, residual):
         ta, tb, tr = self.put(a), self.put(b), self.put(residual)
         tbias = self.put(bias) if bias is not None else None

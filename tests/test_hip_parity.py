@@ -341,6 +341,26 @@ def test_matmul_bias_cast_equals_the_three_operators(run, oracle, case):
         np.testing.assert_array_equal(with_res.view(np.uint16), run.binary("ADD", unfused, res, res.shape, abi.F16).view(np.uint16))
 
 
+def test_matmul_bias_cast_through_a_view(run):
+    """A six-dimensional output view = the RESHAPE -> TRANSPOSE that splits or merges attention heads behind the
+    product: same bytes as the product followed by numpy's reshape and transpose.  The last case has an inner extent
+    that is no multiple of eight, which the fused kernel declines (dense temporary + strided copy inside the call)."""
+    rng = np.random.default_rng(11)
+    cases = [  # (NB, M, K, N), split [NB1, NB2, M1, M2, N1, N2], perms
+        ((1, 6 * 40, 64, 3 * 16), (1, 1, 6, 40, 3, 16), (0, 1, 2, 4, 3, 5)),   # [B, S, H, d] -> [B, H, S, d]
+        ((2 * 3, 72, 48, 32), (2, 3, 72, 1, 1, 32), (0, 2, 3, 1, 4, 5)),       # [B, H, S, d] -> [B, S, H, d]
+        ((1, 300, 128, 256), (1, 1, 300, 1, 2, 128), (0, 1, 4, 2, 3, 5)),      # columns split, rows not
+        ((1, 4 * 10, 32, 2 * 12), (1, 1, 4, 10, 2, 12), (0, 1, 2, 4, 3, 5)),   # inner extent 12: declined
+    ]
+    for (nb, m, k, n), split, perms in cases:
+        a = rng.standard_normal((nb, m, k)).astype(np.float16)
+        b = (0.1 * rng.standard_normal((nb, k, n))).astype(np.float16)
+        bias = rng.standard_normal((1, 1, n)).astype(np.float32)
+        want = run.matmul_bias_cast(a, b, bias).reshape(split).transpose(perms)
+        got = run.matmul_bias_cast_view(a, b, bias, split, perms)
+        np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16), err_msg=str(split))
+
+
 def test_elementwise_chain_equals_the_operators_one_by_one(run):
     """mlel_hip_elementwise_chain against the same operators launched one after another (bit for bit): a GELU-shaped
     chain over fp16 with scalar constants, a chain with row- and column-broadcast inputs and a cast, short rows, and a
