@@ -56,12 +56,13 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
     const int cus = ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
     Tile tile = tall_total >= 2 * (int64_t)cus ? tall : low;
     // Direct-to-LDS pipeline (dense 16-byte aligned rows on both sides or a K-major W, K in whole 64-byte steps):
-    // the 256 x 256 tile when that still gives every compute unit a block, else the 128 x 128 tile under the same
-    // condition as the tall tiles above.  Smaller problems keep the short tiles of the register-staged pipeline.
+    // the 256 x 256 tile when that still gives every compute unit a block, else the 128 x 128 tile when that does
+    // (one block per compute unit of this pipeline beats two of the register-staged one: 13.3 against 13.9 us on
+    // 8 x 512 x 1024 x 1024).  Smaller problems keep the short tiles of the register-staged pipeline.
     const bool dl_ok = xmode == X_PLAIN && (wmode == W_ROWS || wmode == W_KMAJOR) && g.K % BK == 0 && BN == 128;
     if (dl_ok && g.res == nullptr) {
         const int64_t total256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256) * g.batches;
-        const bool big = total256 >= cus, mid = tall_total >= 2 * (int64_t)cus;
+        const bool big = total256 >= cus, mid = tall_total >= (int64_t)cus;
         if (big || mid) {
             tile = big ? Tile{6, 256} : Tile{0, 128};
             xmode = X_PLAIN_DL;

@@ -28,9 +28,9 @@ INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X published dense int8 peak, TOP/s
 HBM_PEAK_GBS = 8000.0         # MI355X published HBM3E bandwidth, GB/s
 
 # HBM bytes per launch of the config 1 kernel from two rocprofv3 --pmc runs of this script (profiles/):
-# FETCH_SIZE 6216 KiB scaled by 2.0 plus WRITE_SIZE 4096 KiB scaled by 1.0, the factors being what the same
+# FETCH_SIZE 6248 KiB scaled by 2.0 plus WRITE_SIZE 4096 KiB scaled by 1.0, the factors being what the same
 # counters read for the 256 MiB copy kernel below (131083 KiB and 262144 KiB).
-CONFIG1_TRAFFIC_BYTES = int((6216 * 2.0 + 4096 * 1.0) * 1024)
+CONFIG1_TRAFFIC_BYTES = int((6248 * 2.0 + 4096 * 1.0) * 1024)
 
 
 def log(*a):
@@ -191,7 +191,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": c1["kernel_tops"], "peak": INT8_MFMA_PEAK_TOPS / 1.0,
                      "unit": "TFLOP/s", "ops_are": "int8 multiply and add counted as 2 ops", "frac": c1["kernel_tops"] / INT8_MFMA_PEAK_TOPS,
                      "traffic": CONFIG1_TRAFFIC_BYTES,
-                     "kernel": "gemm_i8_kernel<64,128,1,4,X_PLAIN,W_KMAJOR,SUMS,Q8>", "kernel_ms": c1["kernel_ms"],
+                     "kernel": "gemm_i8_kernel<128,128,2,2,X_PLAIN_DL,W_KMAJOR_DL,SUMS,Q8>", "kernel_ms": c1["kernel_ms"],
                      "algorithmic_bytes": c1["algorithmic_bytes"],
                      "hbm_frac_if_bandwidth_bound": c1["algorithmic_bytes"] / (c1["kernel_ms"] * 1e-3) / 1e9 /
                      HBM_PEAK_GBS},
