@@ -25,7 +25,6 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4s lds_v4s;
 
-constexpr int NT = 256;
 constexpr uint32_t kOob = 0x80000000u;
 
 struct HGemmArgs {
@@ -61,7 +60,8 @@ __device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t r, uint32_t off) 
 
 // BKH: halfs of K per step (32, or 64 for long contractions: half as many barriers and LDS round trips per K)
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int BKH>
-__global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
+__global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const HGemmArgs g) {
+    constexpr int NT = 64 * WAVES_M * WAVES_N;  // four or eight wavefronts
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
     constexpr int XPITCH = BKH * 2 + 16;      // bytes per A row in LDS
@@ -71,7 +71,7 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(const HGemmArgs g) {
     constexpr int WPITCH = 2 * BN + 32;       // bytes per K row of the B tile: 4 rows x 32 B land on distinct banks
     constexpr int WROW16 = BN / 8;            // 16-byte pieces per K row
     constexpr int WCHUNKS = (BKH * WROW16) / NT;
-    static_assert(WAVES_M * WAVES_N == 4 && WM % 32 == 0 && WN % 32 == 0 && (BKH * WROW16) % NT == 0, "tile shape");
+    static_assert((WAVES_M * WAVES_N == 4 || WAVES_M * WAVES_N == 8) && BM % XPASS == 0 && WM % 32 == 0 && WN % 32 == 0 && (BKH * WROW16) % NT == 0, "tile shape");
     constexpr int XBUF = BM * XPITCH, WBUF = BKH * WPITCH;
     extern __shared__ __align__(16) char smem[];
     char *xs = smem;             // [2][BM][XPITCH]
@@ -292,13 +292,13 @@ void launch_k(const HGemmArgs &g, bool cast_epilogue, dim3 grid, hipStream_t s) 
         static const bool raised = sm <= 48 * 1024 || hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm) == hipSuccess;
         (void)raised;
-        kernel<<<grid, dim3(NT), sm, s>>>(g);
+        kernel<<<grid, dim3(64 * WAVES_M * WAVES_N), sm, s>>>(g);
     } else {
         auto kernel = gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 0, BKH>;
         static const bool raised = sm <= 48 * 1024 || hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm) == hipSuccess;
         (void)raised;
-        kernel<<<grid, dim3(NT), sm, s>>>(g);
+        kernel<<<grid, dim3(64 * WAVES_M * WAVES_N), sm, s>>>(g);
     }
 }
 
@@ -428,7 +428,12 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
     g.total_tiles = (int)total;
     g.chunk = (int)((total + 7) / 8);
     const dim3 grid((unsigned)(g.chunk * 8));
-    if (BN == 128 && tall)
+    // Eight wavefronts on the 128 x 128 tile when a compute unit gets at most three tiles: with so few blocks
+    // resident nothing else hides the per-step barrier and LDS round trip (4096 x 768 x 3072: 36.4 -> 33.3 us); with
+    // more tiles the four-wavefront blocks overlap each other and the larger wavefront tile wins.
+    if (BN == 128 && tall && g.K >= 256 && total <= 3 * (int64_t)cus)
+        launch_k<128, 128, 2, 4, 64>(g, bias_cast, grid, s);
+    else if (BN == 128 && tall)
         launch<128, 128, 2, 2>(g, bias_cast, grid, s);
     else if (BN == 128)
         launch<64, 128, 1, 4>(g, bias_cast, grid, s);
