@@ -384,6 +384,106 @@ __global__ void __launch_bounds__(kBlock) ew_chain_kernel(const ChainArgs g) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Chains that are known at compile time.  The interpreter above pays for every step with shared-memory round trips
+// and a decode; a chain whose program is a template argument unrolls into straight-line code with every value in
+// vector registers and runs like a stand-alone operator.  A program lists, per step, the operator and the values it
+// reads (value v < n_inputs is input v, value n_inputs + i the result of step i); `full` marks the inputs that have
+// the output's shape, the others are single elements.  The arithmetic is the interpreter's (packed fp16 ADD / SUB /
+// MUL, the shared device functions for the rest, one rounding per step).
+// ---------------------------------------------------------------------------------------------------------------
+struct StaticStep {
+    int op, a, b;
+};
+// x * c1 * (TANH((x + x * x * x * c2) * c3) + c4): the tanh form of GELU as TOSA graphs spell it, in the order in
+// which the region builder emits it
+struct GeluTanhProgram {
+    static constexpr int n_inputs = 5, n_steps = 9;
+    static constexpr bool full[n_inputs] = {true, false, false, false, false};
+    static constexpr StaticStep steps[n_steps] = {{F_MUL, 0, 1}, {F_MUL, 0, 0},  {F_MUL, 6, 0},  {F_MUL, 7, 2}, {F_ADD, 0, 8},
+                                                  {F_MUL, 9, 3}, {F_TANH, 10, 0}, {F_ADD, 11, 4}, {F_MUL, 5, 12}};
+};
+struct StaticArgs {
+    char *out;
+    int64_t vecs;
+    const char *in[MLEL_CHAIN_MAX_INPUTS];
+};
+
+template <int OP>
+__device__ __forceinline__ uint4 static_apply(const uint4 &a, const uint4 &b) {
+    uint4 r;
+    __half2 *rh = reinterpret_cast<__half2 *>(&r);
+    const __half2 *ah = reinterpret_cast<const __half2 *>(&a), *bh = reinterpret_cast<const __half2 *>(&b);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        if (OP == F_ADD) {
+            rh[i] = __hadd2(ah[i], bh[i]);
+        } else if (OP == F_SUB) {
+            rh[i] = __hsub2(ah[i], bh[i]);
+        } else if (OP == F_MUL) {
+            rh[i] = __hmul2(ah[i], bh[i]);
+        } else {
+            const float2 f = __half22float2(ah[i]);
+            const float y0 = OP == F_EXP ? op_exp<true>(f.x) : OP == F_RECIPROCAL ? op_reciprocal<true>(f.x)
+                           : OP == F_RSQRT ? op_rsqrt<true>(f.x) : OP == F_TANH ? op_tanh<true>(f.x) : f.x;
+            const float y1 = OP == F_EXP ? op_exp<true>(f.y) : OP == F_RECIPROCAL ? op_reciprocal<true>(f.y)
+                           : OP == F_RSQRT ? op_rsqrt<true>(f.y) : OP == F_TANH ? op_tanh<true>(f.y) : f.y;
+            rh[i] = __halves2half2(f2h(y0), f2h(y1));
+        }
+    }
+    return r;
+}
+
+template <class P, int S>
+__device__ __forceinline__ void static_run(uint4 (&val)[P::n_inputs + P::n_steps]) {
+    if constexpr (S < P::n_steps) {
+        uint4 r = static_apply<P::steps[S].op>(val[P::steps[S].a], val[P::steps[S].b]);
+        // every step's result is rounded where the stand-alone operator rounds it: the compiler must not see through
+        // it, or it contracts a multiplication and the addition of the next step into one fused operation
+        asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
+        val[P::n_inputs + S] = r;
+        static_run<P, S + 1>(val);
+    }
+}
+
+template <class P>
+__global__ void __launch_bounds__(kBlock) ew_static_half_kernel(const StaticArgs g) {
+    const int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (v >= g.vecs) return;
+    uint4 val[P::n_inputs + P::n_steps];
+#pragma unroll
+    for (int k = 0; k < P::n_inputs; k++) {
+        if (P::full[k]) {
+            val[k] = *reinterpret_cast<const uint4 *>(g.in[k] + v * 16);
+        } else {
+            const uint32_t bits = *reinterpret_cast<const uint16_t *>(g.in[k]);
+            const uint32_t w = bits | (bits << 16);
+            val[k] = make_uint4(w, w, w, w);
+        }
+    }
+    static_run<P, 0>(val);
+    *reinterpret_cast<uint4 *>(g.out + v * 16) = val[P::n_inputs + P::n_steps - 1];
+}
+
+// the chain is P's program over inputs of P's shapes
+template <class P>
+bool matches_static(const mlel_tensor *out, const mlel_chain *c, const int *ops) {
+    if (c->n_inputs != P::n_inputs || c->n_steps != P::n_steps) return false;
+    for (int k = 0; k < P::n_inputs; k++) {
+        const mlel_tensor *t = c->inputs[k];
+        const bool full = same_shape(t, out) && is_packed(t) && ((uintptr_t)t->ptr % 16) == 0;
+        const bool single = numel(t) == 1 && ((uintptr_t)t->ptr % 2) == 0;
+        if (t->dtype != MLEL_F16 || !(P::full[k] ? full : single)) return false;
+    }
+    for (int i = 0; i < P::n_steps; i++) {
+        const bool two = ops[i] == F_ADD || ops[i] == F_SUB || ops[i] == F_MUL;
+        if (ops[i] != P::steps[i].op || c->steps[i].a != P::steps[i].a || (two && c->steps[i].b != P::steps[i].b) ||
+            c->steps[i].dtype != MLEL_F16)
+            return false;
+    }
+    return true;
+}
+
 // How `in` relates to the dense output: same extents on every leading dimension (varies along rows) or 1 on all of
 // them, and the same last extent (varies along columns) or 1.  Returns false when neither pattern applies.
 bool classify(const mlel_tensor *out, const mlel_tensor *in, int *varies_row, int *varies_col) {
@@ -950,6 +1050,28 @@ int elementwise_chain_launch(hipStream_t s, const mlel_tensor *out, const mlel_c
     bool all_half = out->dtype == MLEL_F16;
     for (int k = 0; k < c->n_inputs; k++) all_half = all_half && c->inputs[k] != nullptr && c->inputs[k]->dtype == MLEL_F16;
     for (int i = 0; i < c->n_steps; i++) all_half = all_half && c->steps[i].dtype == MLEL_F16;
+    if (all_half && total % 8 == 0) {  // a program compiled ahead of time?
+        int ops[MLEL_CHAIN_MAX_STEPS];
+        for (int i = 0; i < c->n_steps; i++) {
+            const mlel_chain_step &st = c->steps[i];
+            ops[i] = st.kind == MLEL_CHAIN_MUL ? F_MUL
+                     : st.kind == MLEL_CHAIN_BINARY ? (st.selector == MLEL_BIN_ADD ? F_ADD : st.selector == MLEL_BIN_SUB ? F_SUB : -1)
+                     : st.kind == MLEL_CHAIN_UNARY
+                         ? (st.selector == MLEL_UN_EXP ? F_EXP : st.selector == MLEL_UN_RECIPROCAL ? F_RECIPROCAL
+                            : st.selector == MLEL_UN_RSQRT ? F_RSQRT : st.selector == MLEL_UN_TANH ? F_TANH : -1)
+                         : -1;
+        }
+        if (matches_static<GeluTanhProgram>(out, c, ops)) {
+            StaticArgs sa{};
+            sa.out = static_cast<char *>(out->ptr);
+            sa.vecs = total / 8;
+            for (int k = 0; k < c->n_inputs; k++) sa.in[k] = static_cast<const char *>(c->inputs[k]->ptr);
+            const int64_t static_blocks = (sa.vecs + kBlock - 1) / kBlock;
+            MLEL_REQUIRE(static_blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "elementwise chain: too many work items");
+            ew_static_half_kernel<GeluTanhProgram><<<dim3((unsigned)static_blocks), dim3(kBlock), 0, s>>>(sa);
+            return check_launch("elementwise chain (compiled program)");
+        }
+    }
     const int n_regs = all_half ? kChainRegs + 2 : kChainRegs;
     std::vector<int> free_regs;
     for (int r = n_regs - 1; r >= 0; r--) free_regs.push_back(r);

@@ -385,6 +385,15 @@ def test_elementwise_chain_equals_the_operators_one_by_one(run):
                   run.binary("ADD", run.unary("TANH", inner), consts[3], h.shape, f16), h.shape, f16)
     np.testing.assert_array_equal(got, exp)
 
+    # the same expression in the order the graph's region builder emits it, which has a kernel compiled ahead of time
+    # (values 0 h, 1 half, 2 cubic coefficient, 3 sqrt(2 / pi), 4 one)
+    g_consts = [consts[2], consts[0], consts[1], consts[3]]
+    g_steps = [(M, 0, 0, 1, f16), (M, 0, 0, 0, f16), (M, 0, 6, 0, f16), (M, 0, 7, 2, f16), (B, ADD, 0, 8, f16),
+               (M, 0, 9, 3, f16), (U, abi.UN["TANH"], 10, 0, f16), (B, ADD, 11, 4, f16), (M, 0, 5, 12, f16)]
+    for hh in (h, (8 * rng.standard_normal((3, 5, 24))).astype(np.float16)):
+        np.testing.assert_array_equal(run.chain([hh] + g_consts, g_steps, hh.shape, f16).view(np.uint16),
+                                      run.chain([hh] + consts, steps, hh.shape, f16).view(np.uint16))
+
     x32 = rng.standard_normal((4, 24, 64)).astype(np.float32)
     col = rng.standard_normal((4, 24, 1)).astype(np.float16)
     row = rng.standard_normal((1, 1, 64)).astype(np.float16)
