@@ -1009,6 +1009,240 @@ __global__ void __launch_bounds__(kBlock) row_chain_f16_kernel(const RowArgs g) 
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// Chains with reductions that are known at compile time (LayerNorm and the scaled softmax as TOSA graphs spell them,
+// in the order in which the region builder emits them).  Same shapes of values and same arithmetic as
+// row_chain_f16_kernel, but the program is a template argument: 2^k threads of one wavefront share a row and keep
+// their pieces of every full value in vector registers (at most four 16-byte pieces per thread and value), per-row
+// values live in a register of every thread of the row, REDUCE_MAX is a few shuffles, and only REDUCE_SUM goes
+// through shared memory: the row's threads lay the operand down, the row's first thread folds it left to right in
+// fp16 and hands the sum back with a shuffle.  A row never leaves its wavefront, so there is no block-wide barrier.
+// ---------------------------------------------------------------------------------------------------------------
+enum { SC_FULL, SC_ROW, SC_COL, SC_ONE };
+struct LayerNormProgram {
+    static constexpr int n_inputs = 5, n_steps = 11, n_full = 2, n_row = 2;
+    // values: 0 x, 1 1/N, 2 eps, 3 gamma, 4 beta, then one per step
+    static constexpr int cls[16] = {SC_FULL, SC_ONE, SC_ONE, SC_COL, SC_COL, SC_ROW, SC_ROW, SC_FULL,
+                                    SC_FULL, SC_ROW, SC_ROW, SC_ROW, SC_ROW, SC_FULL, SC_FULL, SC_FULL};
+    // register slot of full and per-row values (a slot is reused once its value is dead); the input index otherwise
+    static constexpr int slot[16] = {0, 1, 2, 3, 4, 0, 0, 0, 1, 1, 1, 1, 1, 1, 1, 1};
+    static constexpr StaticStep steps[n_steps] = {{F_RED_SUM, 0, 0}, {F_MUL, 5, 1},  {F_SUB, 0, 6},    {F_MUL, 7, 7},
+                                                  {F_RED_SUM, 8, 0}, {F_MUL, 9, 1},  {F_ADD, 10, 2},   {F_RSQRT, 11, 0},
+                                                  {F_MUL, 7, 12},    {F_MUL, 13, 3}, {F_ADD, 14, 4}};
+};
+struct ScaledSoftmaxProgram {
+    static constexpr int n_inputs = 2, n_steps = 7, n_full = 1, n_row = 1;
+    // values: 0 x, 1 scale, then one per step
+    static constexpr int cls[9] = {SC_FULL, SC_ONE, SC_FULL, SC_ROW, SC_FULL, SC_FULL, SC_ROW, SC_ROW, SC_FULL};
+    static constexpr int slot[9] = {0, 1, 0, 0, 0, 0, 0, 0, 0};
+    static constexpr StaticStep steps[n_steps] = {{F_MUL, 0, 1},     {F_RED_MAX, 2, 0},    {F_SUB, 2, 3}, {F_EXP, 4, 0},
+                                                  {F_RED_SUM, 5, 0}, {F_RECIPROCAL, 6, 0}, {F_MUL, 5, 7}};
+};
+struct RowStaticArgs {
+    char *out;
+    int64_t rows;
+    int32_t cols, tpr_log;
+    const char *in[MLEL_CHAIN_MAX_INPUTS];
+};
+constexpr int kRowStaticPieces = 4;
+
+template <class P>
+struct RowStaticState {
+    uint4 f[P::n_full][kRowStaticPieces];
+    uint32_t r[P::n_row];              // a per-row value, the half in both halves of the word
+    uint32_t one[P::n_inputs];         // single-element inputs, likewise
+    const RowStaticArgs *g;
+    char *stage;                       // this row's staging area in shared memory
+    int part, tpr, segs;
+    int64_t row;
+    bool live;
+};
+
+__device__ __forceinline__ uint4 splat_word(uint32_t w) { return make_uint4(w, w, w, w); }
+
+template <class P, int V>
+__device__ __forceinline__ uint4 row_static_piece(const RowStaticState<P> &c, int u) {
+    if constexpr (P::cls[V] == SC_FULL) {
+        return c.f[P::slot[V]][u];
+    } else if constexpr (P::cls[V] == SC_ROW) {
+        return splat_word(c.r[P::slot[V]]);
+    } else if constexpr (P::cls[V] == SC_ONE) {
+        return splat_word(c.one[V]);
+    } else {
+        const int sg = c.part + u * c.tpr;
+        return sg < c.segs ? *reinterpret_cast<const uint4 *>(c.g->in[V] + sg * 16) : make_uint4(0, 0, 0, 0);
+    }
+}
+
+template <class P, int S>
+__device__ __forceinline__ void row_static_run(RowStaticState<P> &c) {
+    if constexpr (S < P::n_steps) {
+        constexpr int OP = P::steps[S].op, A = P::steps[S].a, B = P::steps[S].b, V = P::n_inputs + S;
+        constexpr bool last = S + 1 == P::n_steps;
+        if constexpr (OP == F_RED_SUM) {
+            // the operand into the row's staging area, then the row's first thread folds it; the row's threads are
+            // lanes of one wavefront, whose shared-memory operations complete in program order
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+#pragma unroll
+            for (int u = 0; u < kRowStaticPieces; u++) {
+                const int sg = c.part + u * c.tpr;
+                if (sg < c.segs) *reinterpret_cast<uint4 *>(c.stage + sg * 16) = c.f[P::slot[A]][u];
+            }
+            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __half acc = f2h(0.f);
+            if (c.part == 0) {
+                const auto add8 = [&](const uint4 &raw) {
+                    const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        acc = __hadd(acc, __low2half(h[t]));
+                        acc = __hadd(acc, __high2half(h[t]));
+                    }
+                };
+                const auto load4 = [&](uint4 (&v)[4], int first) {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) v[t] = *reinterpret_cast<const uint4 *>(c.stage + (first + t) * 16);
+                };
+                int sg = 0;
+                uint4 even[4], odd[4];
+                if (c.segs >= 4) load4(even, 0);
+                for (; sg + 8 <= c.segs; sg += 8) {
+                    load4(odd, sg + 4);
+#pragma unroll
+                    for (int t = 0; t < 4; t++) add8(even[t]);
+                    if (sg + 12 <= c.segs) load4(even, sg + 8);
+#pragma unroll
+                    for (int t = 0; t < 4; t++) add8(odd[t]);
+                }
+                if (sg + 4 <= c.segs) {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) add8(even[t]);
+                    sg += 4;
+                }
+                for (; sg < c.segs; sg++) add8(*reinterpret_cast<const uint4 *>(c.stage + sg * 16));
+            }
+            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            const uint32_t bits = (uint32_t)__half_as_ushort(acc);
+            const int first_lane = (int)(threadIdx.x & 63u) & ~(c.tpr - 1);
+            const uint32_t sum = (uint32_t)__shfl((int)bits, first_lane);
+            c.r[P::slot[V]] = sum | (sum << 16);
+        } else if constexpr (OP == F_RED_MAX) {
+            typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+            h2_t m2 = {(_Float16)-65504.f, (_Float16)-65504.f};
+            uint32_t special = 0;
+#pragma unroll
+            for (int u = 0; u < kRowStaticPieces; u++) {
+                const int sg = c.part + u * c.tpr;
+                if (sg >= c.segs) continue;
+                const uint4 raw = c.f[P::slot[A]][u];
+                special |= (((raw.x & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.y & 0x7fff7fffu) + 0x03ff03ffu) |
+                            ((raw.z & 0x7fff7fffu) + 0x03ff03ffu) | ((raw.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
+                const h2_t *p = reinterpret_cast<const h2_t *>(&raw);
+                m2 = __builtin_elementwise_max(m2, __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]),
+                                                                               __builtin_elementwise_max(p[2], p[3])));
+            }
+            float mx = (float)(m2.x > m2.y ? m2.x : m2.y);
+            for (int d = 1; d < c.tpr; d <<= 1) {
+                mx = fmaxf(mx, __shfl_xor(mx, d));
+                special |= (uint32_t)__shfl_xor((int)special, d);
+            }
+            const uint32_t bits = (uint32_t)__half_as_ushort(f2h(special != 0 ? __builtin_nanf("") : mx));
+            c.r[P::slot[V]] = bits | (bits << 16);
+        } else if constexpr (P::cls[V] == SC_ROW) {
+            uint4 r = static_apply<OP>(row_static_piece<P, A>(c, 0), row_static_piece<P, B>(c, 0));
+            asm volatile("" : "+v"(r.x));  // rounded here, as the stand-alone operator rounds: no contraction across steps
+            c.r[P::slot[V]] = r.x;
+        } else {
+#pragma unroll
+            for (int u = 0; u < kRowStaticPieces; u++) {
+                uint4 r = static_apply<OP>(row_static_piece<P, A>(c, u), row_static_piece<P, B>(c, u));
+                asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
+                if constexpr (last) {
+                    const int sg = c.part + u * c.tpr;
+                    if (c.live && sg < c.segs)
+                        *reinterpret_cast<uint4 *>(c.g->out + (c.row * c.g->cols + sg * 8) * 2) = r;
+                } else {
+                    c.f[P::slot[V]][u] = r;
+                }
+            }
+        }
+        row_static_run<P, S + 1>(c);
+    }
+}
+
+// the full inputs into registers (four pieces requested at once), the single elements into both halves of a word
+template <class P, int K>
+__device__ __forceinline__ void row_static_load(RowStaticState<P> &c) {
+    if constexpr (K < P::n_inputs) {
+        if constexpr (P::cls[K] == SC_FULL) {
+#pragma unroll
+            for (int u = 0; u < kRowStaticPieces; u++) {
+                const int sg = c.part + u * c.tpr;
+                c.f[P::slot[K]][u] = (c.live && sg < c.segs)
+                                         ? *reinterpret_cast<const uint4 *>(c.g->in[K] + (c.row * c.g->cols + sg * 8) * 2)
+                                         : make_uint4(0, 0, 0, 0);
+            }
+        } else if constexpr (P::cls[K] == SC_ONE) {
+            const uint32_t bits = *reinterpret_cast<const uint16_t *>(c.g->in[K]);
+            c.one[K] = bits | (bits << 16);
+        }
+        row_static_load<P, K + 1>(c);
+    }
+}
+
+template <class P>
+__global__ void __launch_bounds__(kBlock) row_static_f16_kernel(const RowStaticArgs g) {
+    extern __shared__ __align__(16) char lds[];
+    RowStaticState<P> c;
+    c.g = &g;
+    c.tpr = 1 << g.tpr_log;
+    c.part = (int)threadIdx.x & (c.tpr - 1);
+    const int rr = (int)threadIdx.x >> g.tpr_log;
+    c.row = (int64_t)blockIdx.x * (kBlock >> g.tpr_log) + rr;
+    c.live = c.row < g.rows;
+    c.segs = g.cols >> 3;
+    c.stage = lds + rr * (g.cols * 2 + 16);
+    row_static_load<P, 0>(c);
+    row_static_run<P, 0>(c);
+}
+
+// the chain is P's program over inputs of P's shapes (`classes`: the RowClass of every input, `ops`: FOp / F_RED_*)
+template <class P>
+bool matches_row_static(const mlel_chain *c, const int8_t *classes, const int *ops) {
+    if (c->n_inputs != P::n_inputs || c->n_steps != P::n_steps) return false;
+    for (int k = 0; k < P::n_inputs; k++) {
+        const int want = P::cls[k] == SC_FULL ? RC_FULL : P::cls[k] == SC_COL ? RC_COL : RC_ONE;
+        if (classes[k] != want) return false;
+    }
+    for (int i = 0; i < P::n_steps; i++) {
+        const bool two = ops[i] == F_ADD || ops[i] == F_SUB || ops[i] == F_MUL;
+        if (ops[i] != P::steps[i].op || c->steps[i].a != P::steps[i].a || (two && c->steps[i].b != P::steps[i].b)) return false;
+    }
+    return true;
+}
+
+template <class P>
+int launch_row_static(hipStream_t s, const mlel_tensor *out, const mlel_chain *c, int64_t rows, int64_t cols) {
+    RowStaticArgs g{};
+    g.out = static_cast<char *>(out->ptr);
+    g.rows = rows;
+    g.cols = (int32_t)cols;
+    const int64_t segs = cols / 8;
+    int tpr_log = 0;
+    while ((int64_t(kRowStaticPieces) << tpr_log) < segs) tpr_log++;  // at most four pieces per thread
+    g.tpr_log = tpr_log;
+    for (int k = 0; k < c->n_inputs; k++) g.in[k] = static_cast<const char *>(c->inputs[k]->ptr);
+    const int64_t rows_per_block = kBlock >> tpr_log;
+    const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+    MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "row chain: too many rows");
+    const size_t smem = (size_t)rows_per_block * (size_t)(cols * 2 + 16);
+    row_static_f16_kernel<P><<<dim3((unsigned)blocks), dim3(kBlock), smem, s>>>(g);
+    return check_launch("row chain (compiled program)");
+}
+
 }  // namespace
 
 // MLEL_ERR_UNSUPPORTED when the chain does not fit the kernel (types, shapes, alignment, live values): the caller
@@ -1238,6 +1472,13 @@ int row_chain_launch(hipStream_t s, const mlel_tensor *out, const mlel_chain *c)
         const bool ok = want_full ? (out_cls == RC_FULL)
                                   : (out_cls == RC_ROW_IN || (rows == 1 && out_cls == RC_ONE));
         if (!ok || ((uintptr_t)out->ptr % (want_full ? 16 : 2)) != 0) return decline("output shape or alignment");
+    }
+    // a program compiled ahead of time?  (rows of at most 4 x 64 pieces: a row stays inside one wavefront)
+    if (cols <= 8 * kRowStaticPieces * 64 && cls[result] == RC_FULL) {
+        if (matches_row_static<LayerNormProgram>(c, cls.data(), op_of.data()))
+            return launch_row_static<LayerNormProgram>(s, out, c, rows, cols);
+        if (matches_row_static<ScaledSoftmaxProgram>(c, cls.data(), op_of.data()))
+            return launch_row_static<ScaledSoftmaxProgram>(s, out, c, rows, cols);
     }
     // row registers for full values, slots of the per-row file for the others, both by linear scan
     std::vector<int> slot(n_values, -1), free_regs, free_slots;
