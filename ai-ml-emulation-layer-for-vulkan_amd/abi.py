@@ -96,6 +96,10 @@ class ResizeAttr(C.Structure):
     _fields_ = [("scale", C.c_int32 * 4), ("offset", C.c_int32 * 2), ("border", C.c_int32 * 2), ("mode", C.c_uint32)]
 
 
+class MatmulProduct(C.Structure):
+    _fields_ = [("out", C.POINTER(Tensor)), ("b", C.POINTER(Tensor)), ("bias", C.POINTER(Tensor))]
+
+
 class ChainStep(C.Structure):
     _fields_ = [("kind", C.c_int32), ("selector", C.c_int32), ("a", C.c_int32), ("b", C.c_int32), ("dtype", C.c_int32)]
 
@@ -249,6 +253,7 @@ FUSED_SIGNATURES = {
     "dwconv_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
     "matmul_bias_cast": [_T, _T, _T, _T, C.POINTER(MatmulAttr)],
     "matmul_bias_cast_add": [_T, _T, _T, _T, C.POINTER(MatmulAttr), _T],
+    "matmul_bias_cast_group": [C.POINTER(MatmulProduct), C.c_int, _T, C.POINTER(MatmulAttr)],
     "softmax_rows": [_T, _T],
     "elementwise_chain": [_T, C.POINTER(Chain)],
     "rescale_add_rescale": [_T, _T, C.POINTER(Epilogue), _T, C.POINTER(Epilogue), C.POINTER(Epilogue)],

@@ -718,6 +718,28 @@ int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *ou
     return 0;
 }
 
+int mlel_hip_matmul_bias_cast_group(mlel_ctx *ctx, void *stream, const mlel_matmul_product *products, int n_products,
+                                    const mlel_tensor *a, const mlel_matmul_attr *attr) {
+    MLEL_TRY(require_ctx(ctx, "matmul_bias_cast_group"));
+    MLEL_REQUIRE(products != nullptr && n_products >= 1 && n_products <= MLEL_MATMUL_GROUP_MAX && attr != nullptr,
+                 MLEL_ERR_INVALID, "matmul_bias_cast_group: 1 to %d products", MLEL_MATMUL_GROUP_MAX);
+    const mlel_tensor *outs[MLEL_MATMUL_GROUP_MAX], *bs[MLEL_MATMUL_GROUP_MAX], *biases[MLEL_MATMUL_GROUP_MAX];
+    bool fusable = a != nullptr && a->rank == 3 && a->dtype == MLEL_F16;
+    for (int i = 0; i < n_products; i++) {
+        outs[i] = products[i].out, bs[i] = products[i].b, biases[i] = products[i].bias;
+        MLEL_REQUIRE(outs[i] != nullptr && bs[i] != nullptr, MLEL_ERR_INVALID, "matmul_bias_cast_group: null tensor in product %d", i);
+        fusable = fusable && bs[i]->rank == 3 && bs[i]->dtype == MLEL_F16 && outs[i]->dtype == MLEL_F16 &&
+                  (outs[i]->rank == 3 || outs[i]->rank == 6) &&
+                  (biases[i] == nullptr || (biases[i]->dtype == MLEL_F32 && biases[i]->rank == 3));
+    }
+    if (fusable && n_products > 1) {
+        const int rc = try_matmul_f16_group(ctx, (hipStream_t)stream, n_products, outs, a, bs, biases, attr);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
+    for (int i = 0; i < n_products; i++) MLEL_TRY(mlel_hip_matmul_bias_cast(ctx, stream, outs[i], a, bs[i], biases[i], attr));
+    return 0;
+}
+
 int mlel_hip_matmul_bias_cast_add(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                                   const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr,
                                   const mlel_tensor *residual) {

@@ -110,6 +110,10 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
                         const mlel_tensor *b, const mlel_matmul_attr *attr, bool bias_cast = false,
                         const mlel_tensor *bias = nullptr, const mlel_tensor *residual = nullptr);
 
+// two or three fused products (fp16 out = CAST(MATMUL + bias)) of one A in a single launch
+int try_matmul_f16_group(mlel_ctx *ctx, hipStream_t s, int n, const mlel_tensor *const *outs, const mlel_tensor *a,
+                         const mlel_tensor *const *bs, const mlel_tensor *const *biases, const mlel_matmul_attr *attr);
+
 // ---- floating-point elementwise / reduce specialisations (ops_float.hip) ----
 int try_binary_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in1,
                           const mlel_tensor *in2);

@@ -48,6 +48,31 @@ struct HGemmArgs {
     int32_t view, v_nb2, v_m2, v_n2;
     int64_t vs_nb1, vs_nb2;
     uint32_t vs_m1, vs_m2, vs_n1;
+    // Several products of the same A in one launch (the Q, K and V projections): tile columns [k * tiles_n_group,
+    // (k + 1) * tiles_n_group) belong to product k, which has a B, a bias and an output of its own; product 0 uses
+    // the fields above.  All products have the same extents and operand strides.
+    int32_t groups, tiles_n_group;
+    struct Extra {
+        const char *b;
+        const float *bias;
+        char *out;
+        int64_t o_batch;
+        uint32_t ldo, o_bytes;
+        int32_t view, v_nb2, v_m2, v_n2;
+        int64_t vs_nb1, vs_nb2;
+        uint32_t vs_m1, vs_m2, vs_n1;
+    } extra[2];
+};
+// what a block needs of its product: filled from HGemmArgs or from one of its Extra entries
+struct HProduct {
+    const char *b;
+    const float *bias;
+    char *out;
+    int64_t o_batch;
+    uint32_t ldo, o_bytes;
+    int32_t view, v_nb2, v_m2, v_n2;
+    int64_t vs_nb1, vs_nb2;
+    uint32_t vs_m1, vs_m2, vs_n1;
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const void *p, uint32_t bytes) {
@@ -83,13 +108,25 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
     const int per_batch = g.tiles_m * g.tiles_n;
     const int batch = lin / per_batch;
     const int t_in = lin - batch * per_batch;
-    const int tile_m = t_in / g.tiles_n, tile_n = t_in - tile_m * g.tiles_n;
+    const int tile_m = t_in / g.tiles_n;
+    int tile_n = t_in - tile_m * g.tiles_n;
+    HProduct o{g.b, g.bias, g.out, g.o_batch, g.ldo, g.o_bytes, g.view, g.v_nb2, g.v_m2, g.v_n2, g.vs_nb1, g.vs_nb2,
+               g.vs_m1, g.vs_m2, g.vs_n1};
+    if (g.groups > 1) {  // uniform
+        const int product = tile_n / g.tiles_n_group;
+        tile_n -= product * g.tiles_n_group;
+        if (product > 0) {
+            const HGemmArgs::Extra &e = product == 1 ? g.extra[0] : g.extra[1];
+            o = HProduct{e.b, e.bias, e.out, e.o_batch, e.ldo, e.o_bytes, e.view, e.v_nb2, e.v_m2, e.v_n2, e.vs_nb1, e.vs_nb2,
+                         e.vs_m1, e.vs_m2, e.vs_n1};
+        }
+    }
     const int m_base = tile_m * BM, n_base = tile_n * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
 
     const __amdgpu_buffer_rsrc_t ares = rsrc(g.a + (int64_t)batch * g.a_batch, g.a_bytes);
-    const __amdgpu_buffer_rsrc_t bres = rsrc(g.b + (int64_t)batch * g.b_batch, g.b_bytes);
+    const __amdgpu_buffer_rsrc_t bres = rsrc(o.b + (int64_t)batch * g.b_batch, g.b_bytes);
 
     uint32_t xoff[XROWS], woff[WCHUNKS];
 #pragma unroll
@@ -190,9 +227,9 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
     }
 
     // ---- store: lane holds row m = lane % 32 of each sub-tile and, per register quad q, columns 8q + 4 * (lane / 32)
-    const int64_t o_base = g.view ? (int64_t)(batch / g.v_nb2) * g.vs_nb1 + (int64_t)(batch % g.v_nb2) * g.vs_nb2
-                                  : (int64_t)batch * g.o_batch;
-    const __amdgpu_buffer_rsrc_t ores = rsrc(g.out + o_base, g.o_bytes);
+    const int64_t o_base = o.view ? (int64_t)(batch / o.v_nb2) * o.vs_nb1 + (int64_t)(batch % o.v_nb2) * o.vs_nb2
+                                  : (int64_t)batch * o.o_batch;
+    const __amdgpu_buffer_rsrc_t ores = rsrc(o.out + o_base, o.o_bytes);
     // the bias of this lane's columns, fetched in one batch before any store (a load after a store would have to
     // wait for it: the compiler cannot tell that the two do not alias)
     float bias_r[TN][4][4];
@@ -204,7 +241,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
                 const int n0 = n_base + wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    bias_r[j][q][e] = (g.bias != nullptr && n0 < g.N) ? g.bias[g.bias_len == 1 ? 0 : n0 + e] : 0.f;
+                    bias_r[j][q][e] = (o.bias != nullptr && n0 < g.N) ? o.bias[g.bias_len == 1 ? 0 : n0 + e] : 0.f;
             }
     }
     if (EPI == 1) {
@@ -225,7 +262,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
                     _Float16 h[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const float sum = g.bias != nullptr ? acc[i][j][4 * q + e] + bias_r[j][q][e] : acc[i][j][4 * q + e];
+                        const float sum = o.bias != nullptr ? acc[i][j][4 * q + e] + bias_r[j][q][e] : acc[i][j][4 * q + e];
                         h[e] = (_Float16)sum;
                     }
                     uint2 v;
@@ -236,7 +273,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
             }
         }
         __syncthreads();
-        const __amdgpu_buffer_rsrc_t rres = rsrc(g.res != nullptr ? g.res + (int64_t)batch * g.r_batch : g.out, g.res != nullptr ? g.r_bytes : 0);
+        const __amdgpu_buffer_rsrc_t rres = rsrc(g.res != nullptr ? g.res + (int64_t)batch * g.r_batch : o.out, g.res != nullptr ? g.r_bytes : 0);
         constexpr int PPR = BN / 8;  // 16-byte pieces per row of the tile
 #pragma unroll
         for (int p0 = 0; p0 < BM * PPR; p0 += NT) {
@@ -244,10 +281,10 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
             const int m = m_base + r, n = n_base + c * 8;
             uint4 piece = *reinterpret_cast<const uint4 *>(smem + r * OPITCH + c * 16);
             const bool inside = m < g.M && n < g.N;
-            uint32_t off = inside ? (uint32_t)m * g.ldo + (uint32_t)n * 2 : kOob;
-            if (g.view && inside)  // uniform
-                off = (uint32_t)(m / g.v_m2) * g.vs_m1 + (uint32_t)(m % g.v_m2) * g.vs_m2 + (uint32_t)(n / g.v_n2) * g.vs_n1 +
-                      (uint32_t)(n % g.v_n2) * 2;
+            uint32_t off = inside ? (uint32_t)m * o.ldo + (uint32_t)n * 2 : kOob;
+            if (o.view && inside)  // uniform
+                off = (uint32_t)(m / o.v_m2) * o.vs_m1 + (uint32_t)(m % o.v_m2) * o.vs_m2 + (uint32_t)(n / o.v_n2) * o.vs_n1 +
+                      (uint32_t)(n % o.v_n2) * 2;
             if (g.res != nullptr) {  // uniform; ADD of two fp16 tensors: one rounding of the exact sum
                 const uint4 other = load16(rres, inside ? (uint32_t)m * g.ldr + (uint32_t)n * 2 : kOob);
                 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
@@ -265,7 +302,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
-        const uint32_t row_off = m < g.M ? (uint32_t)m * g.ldo : kOob;
+        const uint32_t row_off = m < g.M ? (uint32_t)m * o.ldo : kOob;
 #pragma unroll
         for (int j = 0; j < TN; j++) {
 #pragma unroll
@@ -312,12 +349,10 @@ void launch(const HGemmArgs &g, bool cast_epilogue, dim3 grid, hipStream_t s) {
 
 bool dense_rows(const mlel_tensor *t) { return t->strides[2] == 2 && t->strides[1] >= t->dims[2] * 2; }
 
-}  // namespace
-
-// `bias_cast` set: the fused form out(fp16) = CAST(MATMUL + bias) with an fp32 bias of length 1 or N (or none)
-int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
-                        const mlel_tensor *b, const mlel_matmul_attr *attr, bool bias_cast, const mlel_tensor *bias,
-                        const mlel_tensor *residual) {
+// Checks one product against what the kernel's indexing assumes and describes it.  1: described, 0: not a case for
+// this kernel, 2: nothing to compute.
+int fill_args(const mlel_tensor *out, const mlel_tensor *a, const mlel_tensor *b, const mlel_matmul_attr *attr,
+              bool bias_cast, const mlel_tensor *bias, const mlel_tensor *residual, HGemmArgs *filled) {
     if (residual != nullptr) {
         if (!bias_cast || residual->dtype != MLEL_F16 || residual->rank != 3 || !same_shape(residual, out)) return 0;
         if (residual->strides[2] != 2 || ((uintptr_t)residual->ptr % 16) != 0 || residual->strides[0] % 16 != 0 ||
@@ -372,7 +407,7 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
     const int64_t ab = a->dims[1] * a->strides[1], bb = b->dims[1] * b->strides[1], ob = M * out->strides[1];
     if (ab >= lim || bb >= lim || ob >= lim || a->strides[1] >= lim || b->strides[1] >= lim) return 0;
     if (M >= (1 << 24) || N >= (1 << 24) || K >= (1 << 24)) return 0;
-    if (NB <= 0 || M <= 0 || N <= 0) return 1;
+    if (NB <= 0 || M <= 0 || N <= 0) return 2;
 
     HGemmArgs g{};
     g.a = static_cast<const char *>(a->ptr);
@@ -413,12 +448,21 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
         g.ldr = (uint32_t)residual->strides[1];
         g.r_bytes = (uint32_t)(residual->dims[1] * residual->strides[1]);
     }
+    g.groups = 1;
+    *filled = g;
+    return 1;
+}
+
+// Tile choice and launch of a described product (or group of products).
+int launch_args(mlel_ctx *ctx, hipStream_t s, HGemmArgs &g, bool bias_cast) {
+    const int64_t M = g.M, N = g.N, K = g.K, NB = g.batches;
     // tile choice: the width with the least padding of N; the tall tile when it still gives every compute unit two
     // blocks and the contraction is long enough to matter (a K of a few steps is bound by the stores, which the
     // short tile spreads over more blocks), otherwise the short one
     const int BN = ((N + 127) / 128) * 128 <= ((N + 63) / 64) * 64 ? 128 : 64;
     const int cus = ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
-    const int64_t tiles_n = (N + BN - 1) / BN;
+    g.tiles_n_group = (int)((N + BN - 1) / BN);
+    const int64_t tiles_n = (int64_t)g.tiles_n_group * g.groups;
     const bool tall = K > 128 && ((M + 127) / 128) * tiles_n * NB >= 2 * (int64_t)cus;
     const int BM = tall ? 128 : 64;
     g.tiles_m = (int)((M + BM - 1) / BM);
@@ -443,6 +487,40 @@ int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, co
         launch<64, 64, 2, 2>(g, bias_cast, grid, s);
     MLEL_TRY(check_launch("matmul fp16"));
     return 1;
+}
+
+}  // namespace
+
+// `bias_cast` set: the fused form out(fp16) = CAST(MATMUL + bias) with an fp32 bias of length 1 or N (or none)
+int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
+                        const mlel_tensor *b, const mlel_matmul_attr *attr, bool bias_cast, const mlel_tensor *bias,
+                        const mlel_tensor *residual) {
+    HGemmArgs g{};
+    const int rc = fill_args(out, a, b, attr, bias_cast, bias, residual, &g);
+    if (rc != 1) return rc == 2 ? 1 : 0;
+    return launch_args(ctx, s, g, bias_cast);
+}
+
+// Up to three fused products of one A in a single launch; 0 unless every product is a case for the kernel and they
+// agree in everything but their B, bias and output.
+int try_matmul_f16_group(mlel_ctx *ctx, hipStream_t s, int n, const mlel_tensor *const *outs, const mlel_tensor *a,
+                         const mlel_tensor *const *bs, const mlel_tensor *const *biases, const mlel_matmul_attr *attr) {
+    if (n < 2 || n > 3) return 0;
+    HGemmArgs g[3];
+    for (int i = 0; i < n; i++) {
+        if (fill_args(outs[i], a, bs[i], attr, true, biases[i], nullptr, &g[i]) != 1) return 0;
+        const HGemmArgs &x = g[i], &y = g[0];
+        if (x.M != y.M || x.N != y.N || x.K != y.K || x.batches != y.batches || x.ldb != y.ldb || x.b_bytes != y.b_bytes ||
+            (x.batches > 1 && x.b_batch != y.b_batch) || x.bias_len != y.bias_len || (x.bias == nullptr) != (y.bias == nullptr))
+            return 0;
+    }
+    for (int i = 1; i < n; i++) {
+        const HGemmArgs &x = g[i];
+        g[0].extra[i - 1] = HGemmArgs::Extra{x.b, x.bias, x.out, x.o_batch, x.ldo, x.o_bytes, x.view, x.v_nb2, x.v_m2, x.v_n2,
+                                             x.vs_nb1, x.vs_nb2, x.vs_m1, x.vs_m2, x.vs_n1};
+    }
+    g[0].groups = n;
+    return launch_args(ctx, s, g[0], true);
 }
 
 }  // namespace mlel

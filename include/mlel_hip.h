@@ -408,6 +408,18 @@ int mlel_hip_softmax_rows(mlel_ctx *ctx, void *stream, const mlel_tensor *out, c
  * written: the RESHAPE -> TRANSPOSE that splits or merges attention heads behind a projection costs no pass. */
 int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                               const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr);
+/* Several such products of one `a` (the query, key and value projections of an attention block) in one launch:
+ * products[k].out = CAST( MATMUL(a, products[k].b) + products[k].bias ), every product with the same extents; an
+ * output may be a six-dimensional view as above.  Equals the products computed one after another bit for bit (which
+ * is also what happens when the grouped kernel does not apply). */
+#define MLEL_MATMUL_GROUP_MAX 3
+typedef struct mlel_matmul_product {
+    const mlel_tensor *out;
+    const mlel_tensor *b;
+    const mlel_tensor *bias; /* may be NULL */
+} mlel_matmul_product;
+int mlel_hip_matmul_bias_cast_group(mlel_ctx *ctx, void *stream, const mlel_matmul_product *products, int n_products,
+                                    const mlel_tensor *a, const mlel_matmul_attr *attr);
 /* The same followed by the ADD of a residual connection: out(fp16) = ADD( CAST( MATMUL(a, b) + bias ), residual ),
  * `residual` an fp16 tensor of the output's shape; the second addition is an fp16 ADD (one rounding of the exact sum
  * of two halfs), as the stand-alone operator computes it. */

@@ -253,6 +253,21 @@ class Runner:
         self.done()
         return r
 
+    def matmul_bias_cast_group(self, a, bs, biases):
+        """Several fused products of one `a` in one call; returns the list of results."""
+        ta = self.put(a)
+        tbs = [self.put(b) for b in bs]
+        tbias = [self.put(x) if x is not None else None for x in biases]
+        touts = [self.new(abi.F16, (a.shape[0], a.shape[1], b.shape[2])) for b in bs]
+        products = (abi.MatmulProduct * len(bs))()
+        for i in range(len(bs)):
+            products[i] = abi.MatmulProduct(C.pointer(touts[i].view), C.pointer(tbs[i].view),
+                                            C.pointer(tbias[i].view) if tbias[i] else None)
+        self.dev.op("matmul_bias_cast_group", products, len(bs), ta.ref, C.byref(abi.MatmulAttr(0, 0)))
+        r = [t.download() for t in touts]
+        self.done()
+        return r
+
     def matmul_bias_cast_add(self, a, b, bias, residual):
         ta, tb, tr = self.put(a), self.put(b), self.put(residual)
         tbias = self.put(bias) if bias is not None else None

@@ -341,6 +341,25 @@ def test_matmul_bias_cast_equals_the_three_operators(run, oracle, case):
         np.testing.assert_array_equal(with_res.view(np.uint16), run.binary("ADD", unfused, res, res.shape, abi.F16).view(np.uint16))
 
 
+@pytest.mark.parametrize("shape", [(1, 200, 96, 64), (2, 130, 264, 136), (1, 33, 40, 8), (1, 64, 36, 64)], ids=str)
+def test_matmul_bias_cast_group_equals_the_products_one_by_one(run, shape):
+    """Two and three products of one A in one launch (the query, key and value projections) are the products computed
+    one after another, bit for bit; K = 36 is no multiple of eight, which the grouped kernel declines (one call each
+    inside the entry point)."""
+    nb, m, k, n = shape
+    rng = np.random.default_rng(m * 7 + n)
+    a = rng.standard_normal((nb, m, k)).astype(np.float16)
+    bs = [(0.1 * rng.standard_normal((nb, k, n))).astype(np.float16) for _ in range(3)]
+    biases = [rng.standard_normal((1, 1, n)).astype(np.float32) for _ in range(3)]
+    for count in (2, 3):
+        got = run.matmul_bias_cast_group(a, bs[:count], biases[:count])
+        for i in range(count):
+            np.testing.assert_array_equal(got[i].view(np.uint16), run.matmul_bias_cast(a, bs[i], biases[i]).view(np.uint16))
+    got = run.matmul_bias_cast_group(a, bs[:2], [None, None])
+    for i in range(2):
+        np.testing.assert_array_equal(got[i].view(np.uint16), run.matmul_bias_cast(a, bs[i], None).view(np.uint16))
+
+
 def test_matmul_bias_cast_through_a_view(run):
     """A six-dimensional output view = the RESHAPE -> TRANSPOSE that splits or merges attention heads behind the
     product: same bytes as the product followed by numpy's reshape and transpose.  The last case has an inner extent
