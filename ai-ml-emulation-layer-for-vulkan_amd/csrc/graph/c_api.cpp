@@ -286,8 +286,14 @@ std::string opLabel(const OpNode &op) {
         return (reduces ? "ELEMENTWISE+REDUCE x" : "ELEMENTWISE x") + std::to_string(op.chain.size());
     }
     case OpKind::FusedMatmulBiasCast:
-        return std::string(op.hasBias ? "MATMUL+ADD+CAST" : "MATMUL+CAST") + (op.flag ? "+ADD" : "") +
-               (op.viewDims[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");
+    {
+        std::string name = std::string(op.hasBias ? "MATMUL+ADD+CAST" : "MATMUL+CAST") + (op.flag ? "+ADD" : "") +
+                           (op.viewDims[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");
+        for (const auto &view : op.extraProductViews)
+            name += std::string(" | ") + (op.hasBias ? "MATMUL+ADD+CAST" : "MATMUL+CAST") +
+                    (view.first[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");
+        return name;
+    }
     default: return op.tosaName;
     }
 }

@@ -862,6 +862,41 @@ void GraphPipeline::fuse() {
         if (reshape) reshape->fusedAway = true;
     }
 
+    // Pattern 4f (projections of one tensor): fused fp16 products (pattern 4, possibly with the view of pattern 4e,
+    // without a residual) that read the same A and whose B and bias are not produced by the graph, of equal extents,
+    // become one launch of up to three products (mlel_hip_matmul_bias_cast_group): the query, key and value
+    // projections of an attention block.  The later ones run at the first one's place.
+    for (const auto &opPtr : ops) {
+        OpNode &first = *opPtr;
+        if (first.fusedAway || first.kind != OpKind::FusedMatmulBiasCast || first.flag || !first.extraProductViews.empty()) continue;
+        const auto constantOperands = [](const OpNode &op) {
+            for (size_t i = 1; i < op.inputs.size(); i++)
+                if (op.inputs[i]->getProducer() != nullptr) return false;
+            return true;
+        };
+        if (!constantOperands(first)) continue;
+        bool after = false;
+        for (const auto &otherPtr : ops) {
+            OpNode &other = *otherPtr;
+            if (&other == &first) {
+                after = true;
+                continue;
+            }
+            if (!after || first.outputs.size() >= 3) continue;
+            if (other.fusedAway || other.kind != OpKind::FusedMatmulBiasCast || other.flag || !other.extraProductViews.empty() ||
+                other.outputs.size() != 1 || other.inputs[0].get() != first.inputs[0].get() || other.hasBias != first.hasBias ||
+                !constantOperands(other) || !sameShape(*other.inputs[1], *first.inputs[1]) ||
+                (first.hasBias && !sameShape(*other.inputs[2], *first.inputs[2])) ||
+                other.matmul.a_zp != first.matmul.a_zp || other.matmul.b_zp != first.matmul.b_zp)
+                continue;
+            for (size_t i = 1; i < other.inputs.size(); i++) first.inputs.push_back(other.inputs[i]);
+            first.outputs.push_back(other.outputs[0]);
+            other.outputs[0]->setProducer(&first);
+            first.extraProductViews.emplace_back(other.viewDims, other.viewStrides);
+            other.fusedAway = true;
+        }
+    }
+
     // Pattern 5: regions of floating-point elementwise operators (ADD, SUB, MUL, EXP, RECIPROCAL, RSQRT, TANH, CAST
     // between fp16 and fp32) collapse into one pass.  A region grows backwards from an operator whose result is needed
     // elsewhere: a producer is absorbed when it is elementwise too, has the region's shape, and its result is a
@@ -1309,7 +1344,7 @@ mlel_epilogue makeEpilogue(const RescaleSpec &spec, const mlel_tensor *mult, con
 }  // namespace
 
 void GraphPipeline::run(const OpNode &op, void *stream) {
-    std::array<mlel_tensor, 4> in{};
+    std::array<mlel_tensor, 8> in{};
     for (size_t i = 0; i < op.inputs.size() && i < in.size(); i++) {
         in[i] = op.inputs[i]->view();
         if (in[i].ptr == nullptr && op.inputs[i]->getShapeSize() != 0)
@@ -1397,6 +1432,28 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
         break;
     }
     case OpKind::FusedMatmulBiasCast: {
+        const auto viewed = [](mlel_tensor t, const std::array<int64_t, 6> &dims, const std::array<int64_t, 6> &strides) {
+            t.rank = 6;  // the transposed tensor's storage, addressed with the product's split extents
+            for (size_t k = 0; k < 6; k++) {
+                t.dims[k] = dims[k];
+                t.strides[k] = strides[k];
+            }
+            return t;
+        };
+        if (!op.extraProductViews.empty()) {
+            const size_t perProduct = op.hasBias ? 2 : 1, count = op.outputs.size();
+            std::vector<mlel_tensor> outs(count);
+            std::vector<mlel_matmul_product> products(count);
+            for (size_t k = 0; k < count; k++) {
+                const auto &dims = k == 0 ? op.viewDims : op.extraProductViews[k - 1].first;
+                const auto &strides = k == 0 ? op.viewStrides : op.extraProductViews[k - 1].second;
+                outs[k] = op.outputs[k]->view();
+                if (dims[5] != 0) outs[k] = viewed(outs[k], dims, strides);
+                products[k] = mlel_matmul_product{&outs[k], &in[1 + k * perProduct], op.hasBias ? &in[2 + k * perProduct] : nullptr};
+            }
+            rc = mlel_hip_matmul_bias_cast_group(ctx, stream, products.data(), static_cast<int>(count), &in[0], &op.matmul);
+            break;
+        }
         const mlel_tensor *bias = op.hasBias ? &in[2] : nullptr;
         if (op.flag) {
             // the addition may have been written with other extents over the same packed bytes: both tensors are

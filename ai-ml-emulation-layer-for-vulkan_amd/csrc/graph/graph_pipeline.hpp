@@ -140,6 +140,10 @@ class OpNode {
     // FusedMatmulBiasCast whose result is written through a view [NB1, NB2, M1, M2, N1, N2] of the output tensor's
     // storage (a RESHAPE -> TRANSPOSE behind the product folded into its stores); extents 0: no view
     std::array<int64_t, 6> viewDims{}, viewStrides{};
+    // FusedMatmulBiasCast that computes several products of inputs[0] in one launch: product k > 0 reads the inputs
+    // appended for it (its B, then its bias when hasBias), writes outputs[k], through the view k - 1 of this list
+    // when that view's extents are non-zero
+    std::vector<std::pair<std::array<int64_t, 6>, std::array<int64_t, 6>>> extraProductViews;
     RescaleSpec scaleA, scaleB;      // FusedRescaleAddRescale: the two input stages (epilogue = output stage)
     // FusedConv2DResidual: epilogue (+ clamp) belongs to the convolution; scaleA rescales its 8-bit result, scaleB the
     // residual (inputs[3]), scaleOut their sum; `flag` is set when the residual was the addition's first operand

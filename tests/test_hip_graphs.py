@@ -199,7 +199,8 @@ def test_transformer_block_fusions_do_not_change_a_bit(dev):
     assert outs[True][1].count("ELEMENTWISE+REDUCE x7") == 1      # MUL by 1/sqrt(d), then the six softmax operators
     assert outs[True][1].count("ELEMENTWISE+REDUCE x11") == 2     # the two LayerNorms
     assert outs[True][1].count("MATMUL+ADD+CAST+ADD") == 2        # both residual connections ride on their projection
-    assert outs[True][1].count("MATMUL+ADD+CAST+RESHAPE+TRANSPOSE") == 2   # Q and V leave their projection head-split
+    # the three projections of the normalised input are one launch; Q and V leave it head-split
+    assert outs[True][1].count("MATMUL+ADD+CAST+RESHAPE+TRANSPOSE | MATMUL+ADD+CAST | MATMUL+ADD+CAST+RESHAPE+TRANSPOSE") == 1
     assert outs[True][1].count("MATMUL+CAST+RESHAPE+TRANSPOSE") == 1       # the context leaves the product merged
     assert outs[True][1].count("TRANSPOSE") == 1                           # K^T still moves its innermost extent
     assert not [n for n in outs[True][1] if n.startswith("REDUCE_")] and len(outs[True][1]) < len(outs[False][1])
