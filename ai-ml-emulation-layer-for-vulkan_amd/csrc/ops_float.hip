@@ -1039,6 +1039,13 @@ struct ScaledSoftmaxProgram {
     static constexpr StaticStep steps[n_steps] = {{F_MUL, 0, 1},     {F_RED_MAX, 2, 0},    {F_SUB, 2, 3}, {F_EXP, 4, 0},
                                                   {F_RED_SUM, 5, 0}, {F_RECIPROCAL, 6, 0}, {F_MUL, 5, 7}};
 };
+struct SoftmaxProgram {  // the six operators without a scale in front (mlel_hip_softmax_rows)
+    static constexpr int n_inputs = 1, n_steps = 6, n_full = 1, n_row = 1;
+    static constexpr int cls[7] = {SC_FULL, SC_ROW, SC_FULL, SC_FULL, SC_ROW, SC_ROW, SC_FULL};
+    static constexpr int slot[7] = {0, 0, 0, 0, 0, 0, 0};
+    static constexpr StaticStep steps[n_steps] = {{F_RED_MAX, 0, 0}, {F_SUB, 0, 1},        {F_EXP, 2, 0},
+                                                  {F_RED_SUM, 3, 0}, {F_RECIPROCAL, 4, 0}, {F_MUL, 3, 5}};
+};
 struct RowStaticArgs {
     char *out;
     int64_t rows;
@@ -1479,6 +1486,8 @@ int row_chain_launch(hipStream_t s, const mlel_tensor *out, const mlel_chain *c)
             return launch_row_static<LayerNormProgram>(s, out, c, rows, cols);
         if (matches_row_static<ScaledSoftmaxProgram>(c, cls.data(), op_of.data()))
             return launch_row_static<ScaledSoftmaxProgram>(s, out, c, rows, cols);
+        if (matches_row_static<SoftmaxProgram>(c, cls.data(), op_of.data()))
+            return launch_row_static<SoftmaxProgram>(s, out, c, rows, cols);
     }
     // row registers for full values, slots of the per-row file for the others, both by linear scan
     std::vector<int> slot(n_values, -1), free_regs, free_slots;
