@@ -45,9 +45,11 @@ struct HGemmArgs {
     // fp16 result written through a six-dimensional view [NB1, NB2, M1, M2, N1, N2] of other strides (a head split
     // or merge behind the product): batch = nb1 * NB2 + nb2, row = m1 * M2 + m2, column = n1 * N2 + n2 with eight
     // consecutive n2 contiguous.  view == 0: the plain [batch][row][column] layout above.
+    // view == 2: the same with eight consecutive m2 contiguous instead (the innermost extent of the product ends up
+    // somewhere else: a transposing view) and n2 at a stride of vs_n2 bytes
     int32_t view, v_nb2, v_m2, v_n2;
     int64_t vs_nb1, vs_nb2;
-    uint32_t vs_m1, vs_m2, vs_n1;
+    uint32_t vs_m1, vs_m2, vs_n1, vs_n2;
     // Several products of the same A in one launch (the Q, K and V projections): tile columns [k * tiles_n_group,
     // (k + 1) * tiles_n_group) belong to product k, which has a B, a bias and an output of its own; product 0 uses
     // the fields above.  All products have the same extents and operand strides.
@@ -60,7 +62,7 @@ struct HGemmArgs {
         uint32_t ldo, o_bytes;
         int32_t view, v_nb2, v_m2, v_n2;
         int64_t vs_nb1, vs_nb2;
-        uint32_t vs_m1, vs_m2, vs_n1;
+        uint32_t vs_m1, vs_m2, vs_n1, vs_n2;
     } extra[2];
 };
 // what a block needs of its product: filled from HGemmArgs or from one of its Extra entries
@@ -72,7 +74,7 @@ struct HProduct {
     uint32_t ldo, o_bytes;
     int32_t view, v_nb2, v_m2, v_n2;
     int64_t vs_nb1, vs_nb2;
-    uint32_t vs_m1, vs_m2, vs_n1;
+    uint32_t vs_m1, vs_m2, vs_n1, vs_n2;
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const void *p, uint32_t bytes) {
@@ -111,14 +113,14 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
     const int tile_m = t_in / g.tiles_n;
     int tile_n = t_in - tile_m * g.tiles_n;
     HProduct o{g.b, g.bias, g.out, g.o_batch, g.ldo, g.o_bytes, g.view, g.v_nb2, g.v_m2, g.v_n2, g.vs_nb1, g.vs_nb2,
-               g.vs_m1, g.vs_m2, g.vs_n1};
+               g.vs_m1, g.vs_m2, g.vs_n1, g.vs_n2};
     if (g.groups > 1) {  // uniform
         const int product = tile_n / g.tiles_n_group;
         tile_n -= product * g.tiles_n_group;
         if (product > 0) {
             const HGemmArgs::Extra &e = product == 1 ? g.extra[0] : g.extra[1];
             o = HProduct{e.b, e.bias, e.out, e.o_batch, e.ldo, e.o_bytes, e.view, e.v_nb2, e.v_m2, e.v_n2, e.vs_nb1, e.vs_nb2,
-                         e.vs_m1, e.vs_m2, e.vs_n1};
+                         e.vs_m1, e.vs_m2, e.vs_n1, e.vs_n2};
         }
     }
     const int m_base = tile_m * BM, n_base = tile_n * BN;
@@ -249,7 +251,9 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
         // The tile goes through shared memory instead (the operand buffers are free: the loop ended with a barrier)
         // and leaves in 16-byte pieces, consecutive lanes along a row, so that every instruction writes whole lines.
         constexpr int OPITCH = BN * 2 + 16;
-        static_assert(BM * OPITCH <= 2 * XBUF + 2 * WBUF, "the result tile fits in the operand buffers");
+        constexpr int TPITCH = BM * 2 + 16;  // a column of the tile, for transposing views
+        static_assert(BM * OPITCH <= 2 * XBUF + 2 * WBUF && BN * TPITCH <= 2 * XBUF + 2 * WBUF,
+                      "the result tile fits in the operand buffers");
 #pragma unroll
         for (int i = 0; i < TM; i++) {
             char *orow = smem + (wave_m * WM + i * 32 + (lane & 31)) * OPITCH;
@@ -265,15 +269,40 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
                         const float sum = o.bias != nullptr ? acc[i][j][4 * q + e] + bias_r[j][q][e] : acc[i][j][4 * q + e];
                         h[e] = (_Float16)sum;
                     }
+                    const int col = wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+                    if (o.view == 2) {  // uniform; transposing view: the tile is laid down column by column
+                        const int trow = wave_m * WM + i * 32 + (lane & 31);
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            *reinterpret_cast<_Float16 *>(smem + (col + e) * TPITCH + trow * 2) = h[e];
+                        continue;
+                    }
                     uint2 v;
                     v.x = (uint32_t)__builtin_bit_cast(unsigned short, h[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[1]) << 16);
                     v.y = (uint32_t)__builtin_bit_cast(unsigned short, h[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[3]) << 16);
-                    *reinterpret_cast<uint2 *>(orow + (wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5)) * 2) = v;
+                    *reinterpret_cast<uint2 *>(orow + col * 2) = v;
                 }
             }
         }
         __syncthreads();
         const __amdgpu_buffer_rsrc_t rres = rsrc(g.res != nullptr ? g.res + (int64_t)batch * g.r_batch : o.out, g.res != nullptr ? g.r_bytes : 0);
+        if (o.view == 2) {
+            // transposing view: a piece is eight consecutive rows of one column (tile rows start at multiples of
+            // eight and M2 is one, so a piece never straddles two m1)
+            for (int p = tid; p < BN * (BM / 8); p += NT) {
+                const int c = p / (BM / 8), r8 = p - c * (BM / 8);
+                const int m = m_base + r8 * 8, n = n_base + c;
+                if (m >= g.M || n >= g.N) continue;
+                const uint4 piece = *reinterpret_cast<const uint4 *>(smem + c * TPITCH + r8 * 16);
+                const uint32_t w[4] = {piece.x, piece.y, piece.z, piece.w};
+                const uint32_t off = (uint32_t)(m / o.v_m2) * o.vs_m1 + (uint32_t)(m % o.v_m2) * 2 + (uint32_t)(n / o.v_n2) * o.vs_n1 +
+                                     (uint32_t)(n % o.v_n2) * o.vs_n2;
+                v4i v;
+                v.x = (int)w[0], v.y = (int)w[1], v.z = (int)w[2], v.w = (int)w[3];
+                __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
+            }
+            return;
+        }
         constexpr int PPR = BN / 8;  // 16-byte pieces per row of the tile
 #pragma unroll
         for (int p0 = 0; p0 < BM * PPR; p0 += NT) {
@@ -377,10 +406,12 @@ int fill_args(const mlel_tensor *out, const mlel_tensor *a, const mlel_tensor *b
         plain_out.strides[1] = plain_out.dims[2] * 2;
         plain_out.strides[0] = plain_out.dims[1] * plain_out.strides[1];
         out = &plain_out;  // extents for the checks below; the addresses come from the view
-        if (view->strides[5] != 2 || view->dims[5] % 8 != 0) return 0;
-        int64_t span = view->dims[5] * 2;
-        for (int i = 0; i < 5; i++) {
-            if (view->strides[i] % 16 != 0 || view->strides[i] < 0) return 0;
+        // eight contiguous elements along n2 (strides[5] == 2) or, transposing, along m2 (strides[3] == 2)
+        const int inner = view->strides[5] == 2 ? 5 : 3;
+        if (view->strides[inner] != 2 || view->dims[inner] % 8 != 0) return 0;
+        int64_t span = 16;
+        for (int i = 0; i < 6; i++) {
+            if (i != inner && (view->strides[i] % 16 != 0 || view->strides[i] < 0)) return 0;
             if (i >= 2) span += (view->dims[i] - 1) * view->strides[i];
         }
         if (span >= (int64_t(1) << 31) - 64) return 0;
@@ -438,8 +469,10 @@ int fill_args(const mlel_tensor *out, const mlel_tensor *a, const mlel_tensor *b
         g.vs_m1 = (uint32_t)view->strides[2];
         g.vs_m2 = (uint32_t)view->strides[3];
         g.vs_n1 = (uint32_t)view->strides[4];
-        int64_t span = view->dims[5] * 2;
-        for (int i = 2; i < 5; i++) span += (view->dims[i] - 1) * view->strides[i];
+        g.vs_n2 = (uint32_t)view->strides[5];
+        if (view->strides[5] != 2) g.view = 2;
+        int64_t span = 16;
+        for (int i = 2; i < 6; i++) span += (view->dims[i] - 1) * view->strides[i];
         g.o_bytes = (uint32_t)span;
     }
     if (residual != nullptr) {
@@ -517,7 +550,7 @@ int try_matmul_f16_group(mlel_ctx *ctx, hipStream_t s, int n, const mlel_tensor 
     for (int i = 1; i < n; i++) {
         const HGemmArgs &x = g[i];
         g[0].extra[i - 1] = HGemmArgs::Extra{x.b, x.bias, x.out, x.o_batch, x.ldo, x.o_bytes, x.view, x.v_nb2, x.v_m2, x.v_n2,
-                                             x.vs_nb1, x.vs_nb2, x.vs_m1, x.vs_m2, x.vs_n1};
+                                             x.vs_nb1, x.vs_nb2, x.vs_m1, x.vs_m2, x.vs_n1, x.vs_n2};
     }
     g[0].groups = n;
     return launch_args(ctx, s, g[0], true);

@@ -763,7 +763,8 @@ void GraphPipeline::fuse() {
 
     // Pattern 4e (head split / merge behind an fp16 product): the fp16 result [NB, M, N], private, read only by a
     // RESHAPE that splits each of NB, M, N into at most two extents, itself read only by a TRANSPOSE that keeps the
-    // innermost extent innermost.  The product then writes the transposed tensor directly, through a strided view
+    // innermost extent innermost or makes the inner row extent the innermost one (K transposed for the scores).
+    // The product then writes the transposed tensor directly, through a strided view
     // (mlel_hip_matmul_bias_cast with a six-dimensional output); the two data-movement operators disappear.
     for (const auto &opPtr : ops) {
         OpNode &mm = *opPtr;
@@ -818,8 +819,11 @@ void GraphPipeline::fuse() {
             vd[5] = vd[4], vs[5] = vs[4];
             vd[4] = 1, vs[4] = 0;
         }
-        bool aligned = vs[5] == 2 && vd[5] % 8 == 0;
-        for (size_t k = 0; k < 5; k++) aligned = aligned && vs[k] % 16 == 0;
+        // eight contiguous elements along the innermost column extent or, for a transposing view, along the
+        // innermost row extent
+        const size_t inner = vs[5] == 2 ? 5 : 3;
+        bool aligned = vs[inner] == 2 && vd[inner] % 8 == 0;
+        for (size_t k = 0; k < 6; k++) aligned = aligned && (k == inner || vs[k] % 16 == 0);
         if (!aligned) continue;
         mm.viewDims = vd;
         mm.viewStrides = vs;

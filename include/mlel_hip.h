@@ -404,8 +404,9 @@ int mlel_hip_softmax_rows(mlel_ctx *ctx, void *stream, const mlel_tensor *out, c
 /* out(fp16) = CAST( MATMUL(a, b) + bias ): fp16 operands, fp32 accumulation, the fp32 bias [1,1,N] or [1,1,1] (or
  * NULL) added in fp32, one rounding to fp16 -- bit for bit the unfused MATMUL -> ADD -> CAST (or MATMUL -> CAST).
  * `out` has rank 3, or is a six-dimensional view [NB1, NB2, M1, M2, N1, N2] with byte strides of its own (the last
- * one 2, N2 a multiple of 8) through which element (nb1 * NB2 + nb2, m1 * M2 + m2, n1 * N2 + n2) of the product is
- * written: the RESHAPE -> TRANSPOSE that splits or merges attention heads behind a projection costs no pass. */
+ * one 2, N2 a multiple of 8; or, for a view that transposes, the stride of M2 2 and M2 a multiple of 8) through which
+ * element (nb1 * NB2 + nb2, m1 * M2 + m2, n1 * N2 + n2) of the product is written: the RESHAPE -> TRANSPOSE that splits
+ * or merges attention heads behind a projection costs no pass. */
 int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                               const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr);
 /* Several such products of one `a` (the query, key and value projections of an attention block) in one launch:

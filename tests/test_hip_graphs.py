@@ -200,7 +200,7 @@ def test_transformer_block_fusions_do_not_change_a_bit(dev):
     assert outs[True][1].count("ELEMENTWISE+REDUCE x11") == 2     # the two LayerNorms
     assert outs[True][1].count("MATMUL+ADD+CAST+ADD") == 2        # both residual connections ride on their projection
     # the three projections of the normalised input are one launch; Q and V leave it head-split
-    assert outs[True][1].count("MATMUL+ADD+CAST+RESHAPE+TRANSPOSE | MATMUL+ADD+CAST | MATMUL+ADD+CAST+RESHAPE+TRANSPOSE") == 1
+    assert outs[True][1].count(" | ".join(["MATMUL+ADD+CAST+RESHAPE+TRANSPOSE"] * 3)) == 1
     assert outs[True][1].count("MATMUL+CAST+RESHAPE+TRANSPOSE") == 1       # the context leaves the product merged
-    assert outs[True][1].count("TRANSPOSE") == 1                           # K^T still moves its innermost extent
+    assert outs[True][1].count("TRANSPOSE") == 0                           # K leaves its projection transposed
     assert not [n for n in outs[True][1] if n.startswith("REDUCE_")] and len(outs[True][1]) < len(outs[False][1])

@@ -369,6 +369,8 @@ def test_matmul_bias_cast_through_a_view(run):
         ((1, 6 * 40, 64, 3 * 16), (1, 1, 6, 40, 3, 16), (0, 1, 2, 4, 3, 5)),   # [B, S, H, d] -> [B, H, S, d]
         ((2 * 3, 72, 48, 32), (2, 3, 72, 1, 1, 32), (0, 2, 3, 1, 4, 5)),       # [B, H, S, d] -> [B, S, H, d]
         ((1, 300, 128, 256), (1, 1, 300, 1, 2, 128), (0, 1, 4, 2, 3, 5)),      # columns split, rows not
+        ((1, 6 * 40, 64, 3 * 16), (1, 1, 6, 40, 3, 16), (0, 1, 2, 4, 5, 3)),   # [B, S, H, d] -> [B, H, d, S]: transposing
+        ((1, 2 * 136, 72, 5 * 24), (1, 1, 2, 136, 5, 24), (0, 1, 2, 4, 5, 3)), # the same over partial tiles
         ((1, 4 * 10, 32, 2 * 12), (1, 1, 4, 10, 2, 12), (0, 1, 2, 4, 3, 5)),   # inner extent 12: declined
     ]
     for (nb, m, k, n), split, perms in cases:
