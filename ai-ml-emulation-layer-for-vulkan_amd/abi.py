@@ -256,6 +256,7 @@ FUSED_SIGNATURES = {
     "matmul_bias_cast_group": [C.POINTER(MatmulProduct), C.c_int, _T, C.POINTER(MatmulAttr)],
     "softmax_rows": [_T, _T],
     "elementwise_chain": [_T, C.POINTER(Chain)],
+    "matmul_bias_cast_chain": [_T, _T, _T, _T, C.POINTER(MatmulAttr), C.POINTER(Chain)],
     "rescale_add_rescale": [_T, _T, C.POINTER(Epilogue), _T, C.POINTER(Epilogue), C.POINTER(Epilogue)],
 }
 

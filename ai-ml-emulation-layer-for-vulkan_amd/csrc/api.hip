@@ -718,6 +718,33 @@ int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *ou
     return 0;
 }
 
+int mlel_hip_matmul_bias_cast_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
+                                    const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr,
+                                    const mlel_chain *chain) {
+    MLEL_TRY(require_ctx(ctx, "matmul_bias_cast_chain"));
+    MLEL_REQUIRE(attr != nullptr && chain != nullptr && out != nullptr, MLEL_ERR_INVALID, "matmul_bias_cast_chain: null argument");
+    MLEL_REQUIRE(chain->n_inputs >= 1 && chain->n_inputs <= MLEL_CHAIN_MAX_INPUTS && chain->n_steps >= 1 &&
+                     chain->n_steps <= MLEL_CHAIN_MAX_STEPS,
+                 MLEL_ERR_INVALID, "matmul_bias_cast_chain: %d inputs, %d steps", chain->n_inputs, chain->n_steps);
+    MLEL_TRY(check_supported(out, "matmul_bias_cast_chain out"));
+    if (out->rank == 3 && out->dtype == MLEL_F16 && a != nullptr && b != nullptr && a->rank == 3 && b->rank == 3 &&
+        a->dtype == MLEL_F16 && b->dtype == MLEL_F16 && (bias == nullptr || (bias->dtype == MLEL_F32 && bias->rank == 3)) &&
+        chain_is_gelu_tanh(chain)) {
+        const int rc = try_matmul_f16_mfma(ctx, (hipStream_t)stream, out, a, b, attr, true, bias, nullptr, &chain->inputs[1]);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
+    // the product into a temporary, then the chain over it
+    Scratch product_mem;
+    MLEL_HIP_CHECK(hipMalloc(&product_mem.ptr, (size_t)numel(out) * 2 + 16));
+    const mlel_tensor product = packed_like(out, MLEL_F16, product_mem.ptr);
+    MLEL_TRY(mlel_hip_matmul_bias_cast(ctx, stream, &product, a, b, bias, attr));
+    mlel_chain over = *chain;
+    over.inputs[0] = &product;
+    MLEL_TRY(mlel_hip_elementwise_chain(ctx, stream, out, &over));
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
 int mlel_hip_matmul_bias_cast_group(mlel_ctx *ctx, void *stream, const mlel_matmul_product *products, int n_products,
                                     const mlel_tensor *a, const mlel_matmul_attr *attr) {
     MLEL_TRY(require_ctx(ctx, "matmul_bias_cast_group"));

@@ -108,7 +108,13 @@ int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
 // `residual`: an fp16 tensor of the output's shape added to the fused form's fp16 result (a second, fp16 ADD)
 int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
                         const mlel_tensor *b, const mlel_matmul_attr *attr, bool bias_cast = false,
-                        const mlel_tensor *bias = nullptr, const mlel_tensor *residual = nullptr);
+                        const mlel_tensor *bias = nullptr, const mlel_tensor *residual = nullptr,
+                        const mlel_tensor *const *gelu_inputs = nullptr);
+// `gelu_inputs`: the four single-element fp16 inputs of the tanh form of GELU (see chain_is_gelu_tanh), applied to
+// the fused form's rounded result
+// The chain is the tanh form of GELU over its value 0, as the graph's region builder emits it: inputs 1 .. 4 are
+// single fp16 elements, nine steps (ops_float.hip).
+bool chain_is_gelu_tanh(const mlel_chain *chain);
 
 // two or three fused products (fp16 out = CAST(MATMUL + bias)) of one A in a single launch
 int try_matmul_f16_group(mlel_ctx *ctx, hipStream_t s, int n, const mlel_tensor *const *outs, const mlel_tensor *a,

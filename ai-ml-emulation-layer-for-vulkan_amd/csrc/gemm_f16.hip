@@ -14,6 +14,7 @@
 // All global loads are buffer loads: an offset at or beyond the extent returns 0, which pads M, N and K tails.
 #include "common.hpp"
 #include "dispatch.hpp"
+#include "float_programs.hpp"
 
 namespace mlel {
 namespace {
@@ -53,6 +54,9 @@ struct HGemmArgs {
     // Several products of the same A in one launch (the Q, K and V projections): tile columns [k * tiles_n_group,
     // (k + 1) * tiles_n_group) belong to product k, which has a B, a bias and an output of its own; product 0 uses
     // the fields above.  All products have the same extents and operand strides.
+    // the tanh form of GELU applied to the rounded result (GeluTanhProgram with the result as its value 0): the
+    // program's four single-element fp16 inputs, or null
+    const uint16_t *act[4];
     int32_t groups, tiles_n_group;
     struct Extra {
         const char *b;
@@ -304,6 +308,14 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
             return;
         }
         constexpr int PPR = BN / 8;  // 16-byte pieces per row of the tile
+        uint32_t act_c[4] = {0, 0, 0, 0};
+        if (g.act[0] != nullptr) {  // uniform
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t bits = *g.act[k];
+                act_c[k] = bits | (bits << 16);
+            }
+        }
 #pragma unroll
         for (int p0 = 0; p0 < BM * PPR; p0 += NT) {
             const int p = p0 + tid, r = p / PPR, c = p % PPR;
@@ -314,6 +326,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
             if (o.view && inside)  // uniform
                 off = (uint32_t)(m / o.v_m2) * o.vs_m1 + (uint32_t)(m % o.v_m2) * o.vs_m2 + (uint32_t)(n / o.v_n2) * o.vs_n1 +
                       (uint32_t)(n % o.v_n2) * 2;
+            if (g.act[0] != nullptr) piece = gelu_tanh_piece(piece, act_c);  // uniform
             if (g.res != nullptr) {  // uniform; ADD of two fp16 tensors: one rounding of the exact sum
                 const uint4 other = load16(rres, inside ? (uint32_t)m * g.ldr + (uint32_t)n * 2 : kOob);
                 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
@@ -381,7 +394,13 @@ bool dense_rows(const mlel_tensor *t) { return t->strides[2] == 2 && t->strides[
 // Checks one product against what the kernel's indexing assumes and describes it.  1: described, 0: not a case for
 // this kernel, 2: nothing to compute.
 int fill_args(const mlel_tensor *out, const mlel_tensor *a, const mlel_tensor *b, const mlel_matmul_attr *attr,
-              bool bias_cast, const mlel_tensor *bias, const mlel_tensor *residual, HGemmArgs *filled) {
+              bool bias_cast, const mlel_tensor *bias, const mlel_tensor *residual, HGemmArgs *filled,
+              const mlel_tensor *const *act = nullptr) {
+    if (act != nullptr) {
+        if (!bias_cast || residual != nullptr || out->rank != 3) return 0;
+        for (int k = 0; k < 4; k++)
+            if (act[k] == nullptr || act[k]->dtype != MLEL_F16 || numel(act[k]) != 1 || ((uintptr_t)act[k]->ptr % 2) != 0) return 0;
+    }
     if (residual != nullptr) {
         if (!bias_cast || residual->dtype != MLEL_F16 || residual->rank != 3 || !same_shape(residual, out)) return 0;
         if (residual->strides[2] != 2 || ((uintptr_t)residual->ptr % 16) != 0 || residual->strides[0] % 16 != 0 ||
@@ -481,6 +500,8 @@ int fill_args(const mlel_tensor *out, const mlel_tensor *a, const mlel_tensor *b
         g.ldr = (uint32_t)residual->strides[1];
         g.r_bytes = (uint32_t)(residual->dims[1] * residual->strides[1]);
     }
+    if (act != nullptr)
+        for (int k = 0; k < 4; k++) g.act[k] = static_cast<const uint16_t *>(act[k]->ptr);
     g.groups = 1;
     *filled = g;
     return 1;
@@ -535,9 +556,9 @@ int launch_args(mlel_ctx *ctx, hipStream_t s, HGemmArgs &g, bool bias_cast) {
 // `bias_cast` set: the fused form out(fp16) = CAST(MATMUL + bias) with an fp32 bias of length 1 or N (or none)
 int try_matmul_f16_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *a,
                         const mlel_tensor *b, const mlel_matmul_attr *attr, bool bias_cast, const mlel_tensor *bias,
-                        const mlel_tensor *residual) {
+                        const mlel_tensor *residual, const mlel_tensor *const *gelu_inputs) {
     HGemmArgs g{};
-    const int rc = fill_args(out, a, b, attr, bias_cast, bias, residual, &g);
+    const int rc = fill_args(out, a, b, attr, bias_cast, bias, residual, &g, gelu_inputs);
     if (rc != 1) return rc == 2 ? 1 : 0;
     return launch_args(ctx, s, g, bias_cast);
 }

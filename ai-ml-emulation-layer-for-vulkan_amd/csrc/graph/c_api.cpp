@@ -289,6 +289,7 @@ std::string opLabel(const OpNode &op) {
     {
         std::string name = std::string(op.hasBias ? "MATMUL+ADD+CAST" : "MATMUL+CAST") + (op.flag ? "+ADD" : "") +
                            (op.viewDims[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");
+        if (!op.chain.empty()) name += "+ELEMENTWISE x" + std::to_string(op.chain.size());
         for (const auto &view : op.extraProductViews)
             name += std::string(" | ") + (op.hasBias ? "MATMUL+ADD+CAST" : "MATMUL+CAST") +
                     (view.first[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");

@@ -1116,6 +1116,36 @@ void GraphPipeline::fuse() {
         root.chain = steps;
     }
 
+    // Pattern 6 (activation behind an fp16 product): a fused product (pattern 4; no view, residual or group) whose
+    // private result is read only by a fused elementwise region as its first input, the region's other inputs not
+    // produced by the graph: the region moves into the product's call (mlel_hip_matmul_bias_cast_chain), where the
+    // kernel applies it to the tile on its way out when it knows the chain (the tanh form of GELU).
+    for (const auto &opPtr : ops) {
+        OpNode &mm = *opPtr;
+        if (mm.fusedAway || mm.kind != OpKind::FusedMatmulBiasCast || mm.flag || mm.viewDims[5] != 0 ||
+            !mm.extraProductViews.empty() || !mm.chain.empty())
+            continue;
+        const TensorPtr h = mm.outputs[0];
+        if (!isPrivateIntermediate(*h)) continue;
+        const auto users = consumersOf(ops, h.get());
+        if (users.size() != 1 || users[0]->kind != OpKind::FusedElementwise) continue;
+        OpNode *ew = users[0];
+        if (ew->inputs.empty() || ew->inputs[0].get() != h.get() || !sameShape(*ew->outputs[0], *h) ||
+            ew->outputs[0]->getFormat() != MLEL_F16 || !ew->outputs[0]->isPacked() ||
+            mm.inputs.size() + ew->inputs.size() - 1 > 8)
+            continue;
+        bool ok = true;
+        for (size_t i = 1; i < ew->inputs.size(); i++)
+            ok = ok && ew->inputs[i].get() != h.get() && ew->inputs[i]->getProducer() == nullptr;
+        for (const auto &st : ew->chain) ok = ok && st.kind != MLEL_CHAIN_REDUCE;
+        if (!ok) continue;
+        mm.chain = ew->chain;
+        for (size_t i = 1; i < ew->inputs.size(); i++) mm.inputs.push_back(ew->inputs[i]);
+        mm.outputs[0] = ew->outputs[0];
+        ew->outputs[0]->setProducer(&mm);
+        ew->fusedAway = true;
+    }
+
     // Pattern 3: RESHAPE between two packed session tensors of the same byte size moves no data (the reference's
     // reshape.comp:16-27 copies by flat index): the output becomes a second view of the input's storage and the
     // operator is not executed.  plan() gives both tensors one allocation that lives as long as either is used.
@@ -1459,6 +1489,17 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
             break;
         }
         const mlel_tensor *bias = op.hasBias ? &in[2] : nullptr;
+        if (!op.chain.empty()) {  // the product, then the elementwise region over it
+            mlel_chain c{};
+            const size_t own = op.hasBias ? 3 : 2;  // a, b (, bias); the region's own inputs follow
+            c.n_inputs = static_cast<int32_t>(op.inputs.size() - own + 1);
+            c.n_steps = static_cast<int32_t>(op.chain.size());
+            c.inputs[0] = nullptr;
+            for (size_t i = own; i < op.inputs.size(); i++) c.inputs[i - own + 1] = &in[i];
+            for (size_t i = 0; i < op.chain.size(); i++) c.steps[i] = op.chain[i];
+            rc = mlel_hip_matmul_bias_cast_chain(ctx, stream, &out, &in[0], &in[1], bias, &op.matmul, &c);
+            break;
+        }
         if (op.flag) {
             // the addition may have been written with other extents over the same packed bytes: both tensors are
             // handed over with the product's extents [batches, rows, columns]

@@ -465,6 +465,14 @@ typedef struct mlel_chain {
     mlel_chain_step steps[MLEL_CHAIN_MAX_STEPS];
 } mlel_chain;
 int mlel_hip_elementwise_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_chain *chain);
+/* out(fp16) = chain( CAST( MATMUL(a, b) + bias ) ): the fused product above followed by an elementwise chain whose
+ * value 0 is the product (chain->inputs[0] is ignored and may be NULL; the other inputs are the chain's own).  The
+ * activation of a feed-forward layer costs no pass when the chain is one the product's kernel knows (the tanh form
+ * of GELU); otherwise the product goes through a temporary and the chain runs over it.  Bit for bit the product
+ * followed by mlel_hip_elementwise_chain. */
+int mlel_hip_matmul_bias_cast_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
+                                    const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr,
+                                    const mlel_chain *chain);
 
 /* Plain device-to-device copy kernel of `bytes` bytes with 128-bit accesses; the calibration kernel for
  * memory-traffic counters and the measured HBM ceiling. */

@@ -253,6 +253,25 @@ class Runner:
         self.done()
         return r
 
+    def matmul_bias_cast_chain(self, a, b, bias, inputs, steps):
+        """The fused product followed by an elementwise chain whose value 0 is the product; `inputs`: the chain's
+        other inputs."""
+        ta, tb = self.put(a), self.put(b)
+        tbias = self.put(bias) if bias is not None else None
+        tin = [self.put(x) for x in inputs]
+        to = self.new(abi.F16, (a.shape[0], a.shape[1], b.shape[2]))
+        c = abi.Chain()
+        c.n_inputs, c.n_steps = len(tin) + 1, len(steps)
+        for i, t in enumerate(tin):
+            c.inputs[i + 1] = C.pointer(t.view)
+        for i, st in enumerate(steps):
+            c.steps[i] = abi.ChainStep(*[int(v) for v in st])
+        self.dev.op("matmul_bias_cast_chain", to.ref, ta.ref, tb.ref, tbias.ref if tbias else None,
+                    C.byref(abi.MatmulAttr(0, 0)), C.byref(c))
+        r = to.download()
+        self.done()
+        return r
+
     def matmul_bias_cast_group(self, a, bs, biases):
         """Several fused products of one `a` in one call; returns the list of results."""
         ta = self.put(a)

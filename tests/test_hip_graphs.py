@@ -199,6 +199,7 @@ def test_transformer_block_fusions_do_not_change_a_bit(dev):
     assert outs[True][1].count("ELEMENTWISE+REDUCE x7") == 1      # MUL by 1/sqrt(d), then the six softmax operators
     assert outs[True][1].count("ELEMENTWISE+REDUCE x11") == 2     # the two LayerNorms
     assert outs[True][1].count("MATMUL+ADD+CAST+ADD") == 2        # both residual connections ride on their projection
+    assert outs[True][1].count("MATMUL+ADD+CAST+ELEMENTWISE x9") == 1   # GELU inside the first feed-forward product
     # the three projections of the normalised input are one launch; Q and V leave it head-split
     assert outs[True][1].count(" | ".join(["MATMUL+ADD+CAST+RESHAPE+TRANSPOSE"] * 3)) == 1
     assert outs[True][1].count("MATMUL+CAST+RESHAPE+TRANSPOSE") == 1       # the context leaves the product merged

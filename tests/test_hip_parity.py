@@ -360,6 +360,34 @@ def test_matmul_bias_cast_group_equals_the_products_one_by_one(run, shape):
         np.testing.assert_array_equal(got[i].view(np.uint16), run.matmul_bias_cast(a, bs[i], None).view(np.uint16))
 
 
+def test_matmul_bias_cast_chain_equals_product_then_chain(run):
+    """The activation of a feed-forward layer inside the product's call: the tanh form of GELU (applied by the matrix
+    kernel to the tile on its way out) and a chain the kernel does not know (product into a temporary, then the chain)
+    both equal the product followed by mlel_hip_elementwise_chain, bit for bit."""
+    rng = np.random.default_rng(23)
+    B, M, U = 0, 1, 2
+    ADD = abi.BIN["ADD"]
+    f16 = abi.F16
+
+    def scalar(v):
+        return np.array(v, np.float16).reshape(1, 1, 1)
+
+    gelu_inputs = [scalar(0.5), scalar(0.044715), scalar(np.sqrt(2 / np.pi)), scalar(1.0)]
+    gelu = [(M, 0, 0, 1, f16), (M, 0, 0, 0, f16), (M, 0, 6, 0, f16), (M, 0, 7, 2, f16), (B, ADD, 0, 8, f16),
+            (M, 0, 9, 3, f16), (U, abi.UN["TANH"], 10, 0, f16), (B, ADD, 11, 4, f16), (M, 0, 5, 12, f16)]
+    other_inputs = [scalar(0.25)]
+    other = [(M, 0, 0, 1, f16), (U, abi.UN["EXP"], 2, 0, f16)]
+    for nb, m, k, n in ((1, 200, 96, 256), (2, 70, 40, 72), (1, 64, 36, 64)):
+        a = rng.standard_normal((nb, m, k)).astype(np.float16)
+        b = (0.3 * rng.standard_normal((nb, k, n))).astype(np.float16)
+        bias = rng.standard_normal((1, 1, n)).astype(np.float32)
+        product = run.matmul_bias_cast(a, b, bias)
+        for inputs, steps in ((gelu_inputs, gelu), (other_inputs, other)):
+            want = run.chain([product] + inputs, steps, product.shape, f16)
+            got = run.matmul_bias_cast_chain(a, b, bias, inputs, steps)
+            np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16), err_msg=f"{(nb, m, k, n)} {len(steps)}")
+
+
 def test_matmul_bias_cast_through_a_view(run):
     """A six-dimensional output view = the RESHAPE -> TRANSPOSE that splits or merges attention heads behind the
     product: same bytes as the product followed by numpy's reshape and transpose.  The last case has an inner extent
