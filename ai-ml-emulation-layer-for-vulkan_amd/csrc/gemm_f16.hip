@@ -529,10 +529,11 @@ int launch_args(mlel_ctx *ctx, hipStream_t s, HGemmArgs &g, bool bias_cast) {
     // Eight wavefronts on the 128 x 128 tile when a compute unit gets at most three tiles: with so few blocks
     // resident nothing else hides the per-step barrier and LDS round trip (4096 x 768 x 3072: 36.4 -> 33.3 us); with
     // more tiles the four-wavefront blocks overlap each other and the larger wavefront tile wins.
-    // A long contraction over few tiles (4096 x 3072 x 768: 192 tiles of 128 x 128): the eight-wavefront tile even
-    // when it leaves a quarter of the compute units idle, 43.1 -> 38.4 us against 384 short tiles
+    // A contraction of some length over few tiles (4096 x 3072 x 768 and 4096 x 768 x 768: 192 tiles of 128 x 128):
+    // the eight-wavefront tile even when it leaves a quarter of the compute units idle, 43.1 -> 38.4 us and
+    // 15.5 -> 13.7 us against 384 short tiles
     const int64_t tiles128 = ((M + 127) / 128) * tiles_n * NB;
-    if (BN == 128 && !tall && g.K >= 1024 && tiles128 * 5 >= 3 * (int64_t)cus) {
+    if (BN == 128 && !tall && g.K >= 512 && tiles128 * 5 >= 3 * (int64_t)cus) {
         g.tiles_m = (int)((M + 127) / 128);
         g.total_tiles = (int)tiles128;
         g.chunk = (int)((tiles128 + 7) / 8);
