@@ -288,6 +288,7 @@ RUNTIME_SIGNATURES = {
     "mlel_hip_graph_launch": (C.c_int, [_V, _V, _V]),
     "mlel_hip_graph_destroy": (C.c_int, [_V, _V]),
     "mlel_hip_copy_kernel": (C.c_int, [_V, _V, _V, _V, C.c_size_t]),
+    "mlel_hip_matmul_chain_in_kernel": (C.c_int, [C.POINTER(Chain)]),
 }
 
 

@@ -745,6 +745,13 @@ int mlel_hip_matmul_bias_cast_chain(mlel_ctx *ctx, void *stream, const mlel_tens
     return 0;
 }
 
+int mlel_hip_matmul_chain_in_kernel(const mlel_chain *chain) {
+    return chain != nullptr && chain->n_inputs >= 1 && chain->n_inputs <= MLEL_CHAIN_MAX_INPUTS && chain->n_steps >= 1 &&
+                   chain->n_steps <= MLEL_CHAIN_MAX_STEPS && chain_is_gelu_tanh(chain)
+               ? 1
+               : 0;
+}
+
 int mlel_hip_matmul_bias_cast_group(mlel_ctx *ctx, void *stream, const mlel_matmul_product *products, int n_products,
                                     const mlel_tensor *a, const mlel_matmul_attr *attr) {
     MLEL_TRY(require_ctx(ctx, "matmul_bias_cast_group"));

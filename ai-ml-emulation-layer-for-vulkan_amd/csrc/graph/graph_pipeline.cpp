@@ -1118,8 +1118,9 @@ void GraphPipeline::fuse() {
 
     // Pattern 6 (activation behind an fp16 product): a fused product (pattern 4; no view, residual or group) whose
     // private result is read only by a fused elementwise region as its first input, the region's other inputs not
-    // produced by the graph: the region moves into the product's call (mlel_hip_matmul_bias_cast_chain), where the
-    // kernel applies it to the tile on its way out when it knows the chain (the tanh form of GELU).
+    // produced by the graph, and the chain one that the product's kernel applies to the tile on its way out (the tanh
+    // form of GELU; mlel_hip_matmul_chain_in_kernel): the region moves into the product's call
+    // (mlel_hip_matmul_bias_cast_chain).
     for (const auto &opPtr : ops) {
         OpNode &mm = *opPtr;
         if (mm.fusedAway || mm.kind != OpKind::FusedMatmulBiasCast || mm.flag || mm.viewDims[5] != 0 ||
@@ -1138,7 +1139,19 @@ void GraphPipeline::fuse() {
         for (size_t i = 1; i < ew->inputs.size(); i++)
             ok = ok && ew->inputs[i].get() != h.get() && ew->inputs[i]->getProducer() == nullptr;
         for (const auto &st : ew->chain) ok = ok && st.kind != MLEL_CHAIN_REDUCE;
-        if (!ok) continue;
+        if (!ok || ew->inputs.size() > MLEL_CHAIN_MAX_INPUTS || ew->chain.size() > MLEL_CHAIN_MAX_STEPS) continue;
+        // only a chain the product's kernel applies itself: any other would run as a pass of its own over a temporary
+        // that the call has to allocate, which the stand-alone region does without
+        std::array<mlel_tensor, MLEL_CHAIN_MAX_INPUTS> described{};
+        mlel_chain query{};
+        query.n_inputs = static_cast<int32_t>(ew->inputs.size());
+        query.n_steps = static_cast<int32_t>(ew->chain.size());
+        for (size_t i = 1; i < ew->inputs.size(); i++) {
+            described[i] = ew->inputs[i]->view();
+            query.inputs[i] = &described[i];
+        }
+        for (size_t i = 0; i < ew->chain.size(); i++) query.steps[i] = ew->chain[i];
+        if (mlel_hip_matmul_chain_in_kernel(&query) == 0) continue;
         mm.chain = ew->chain;
         for (size_t i = 1; i < ew->inputs.size(); i++) mm.inputs.push_back(ew->inputs[i]);
         mm.outputs[0] = ew->outputs[0];

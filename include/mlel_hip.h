@@ -473,6 +473,11 @@ int mlel_hip_elementwise_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *o
 int mlel_hip_matmul_bias_cast_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                                     const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr,
                                     const mlel_chain *chain);
+/* 1 when mlel_hip_matmul_bias_cast_chain applies this chain inside the product's kernel, 0 when it would run the
+ * chain as a pass of its own over a temporary (then a caller gains nothing by handing the chain over).  Reads only
+ * the steps and the extents and types of inputs 1 and up; touches no device.  No counterpart in the reference, which
+ * has no fused operators. */
+int mlel_hip_matmul_chain_in_kernel(const mlel_chain *chain);
 
 /* Plain device-to-device copy kernel of `bytes` bytes with 128-bit accesses; the calibration kernel for
  * memory-traffic counters and the measured HBM ceiling. */

@@ -267,3 +267,114 @@ def test_profiling_switch_from_environment(monkeypatch):
     assert g.profiling() is True
     assert g.profiling_report() == {"timestamp_period_ns": None, "samples": [], "by_operator": []}
     g.close()
+
+
+# ------------------------------------------------------------------------------------- fp16 fusion patterns, host only
+def _f16_projection(spec, x, rows, k, n, seed):
+    """MATMUL (fp32 result) + fp32 bias + CAST to fp16, as the transformer block spells a projection."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    w = spec.const("w", (0.02 * rng.standard_normal((1, k, n))).astype(np.float16))
+    b = spec.const("b", (0.02 * rng.standard_normal((1, 1, n))).astype(np.float32))
+    acc = spec.tensor("acc", abi.F32, (1, rows, n))
+    spec.op("MATMUL", [x, w], [acc], [0, 0])
+    summed = spec.tensor("t", abi.F32, (1, rows, n))
+    spec.op("ADD", [acc, b], [summed])
+    out = spec.tensor("t", abi.F16, (1, rows, n))
+    spec.op("CAST", [summed], [out])
+    return out
+
+
+def test_transformer_block_fused_operator_list():
+    """The encoder block after fusion, on the host: nine launches, no stand-alone reduction, transpose or reshape."""
+    spec = graphs.transformer_block_spec(batch=2, seq=64, d_model=64, heads=4, ffn=128)
+    g = _build_host_only(spec, fuse=True)
+    three = " | ".join(["MATMUL+ADD+CAST+RESHAPE+TRANSPOSE"] * 3)
+    assert g.op_names() == ["ELEMENTWISE+REDUCE x11", three, "MATMUL+CAST", "ELEMENTWISE+REDUCE x7",
+                            "MATMUL+CAST+RESHAPE+TRANSPOSE", "MATMUL+ADD+CAST+ADD", "ELEMENTWISE+REDUCE x11",
+                            "MATMUL+ADD+CAST+ELEMENTWISE x9", "MATMUL+ADD+CAST+ADD"]
+    g.close()
+
+
+def test_projection_patterns_leave_observable_or_mismatched_cases_alone():
+    """Residual, grouping and view fusions behind fp16 products apply only when nothing else can observe the product's
+    result and the shapes fit."""
+    import numpy as np
+    rows, d = 64, 32
+
+    def base():
+        spec = graphs.Spec()
+        spec.inputs.append(("input", abi.F16, (1, rows, d)))
+        return spec
+
+    # 1. two projections of one tensor group; a third with other extents does not join; results that are graph
+    #    outputs are still written by the grouped launch
+    spec = base()
+    p1 = _f16_projection(spec, "input", rows, d, d, 1)
+    p2 = _f16_projection(spec, "input", rows, d, d, 2)
+    p3 = _f16_projection(spec, "input", rows, d, 2 * d, 3)
+    spec.op("MUL", [p1, p2], ["out_a"], [0])
+    spec.outputs.append(("out_a", abi.F16, (1, rows, d)))
+    spec.op("CAST", [p3], ["out_b"])
+    spec.outputs.append(("out_b", abi.F32, (1, rows, 2 * d)))
+    g = _build_host_only(spec, fuse=True)
+    assert g.op_names() == ["MATMUL+ADD+CAST | MATMUL+ADD+CAST", "MATMUL+ADD+CAST", "MUL", "CAST"]
+    g.close()
+
+    # 1b. the sum of two projections: the first one's result is the second one's residual, and a product that carries
+    #     a residual joins no group
+    spec = base()
+    p1 = _f16_projection(spec, "input", rows, d, d, 1)
+    p2 = _f16_projection(spec, "input", rows, d, d, 2)
+    spec.op("ADD", [p1, p2], ["out"])
+    spec.outputs.append(("out", abi.F16, (1, rows, d)))
+    g = _build_host_only(spec, fuse=True)
+    assert g.op_names() == ["MATMUL+ADD+CAST", "MATMUL+ADD+CAST+ADD"]
+    g.close()
+
+    # 2. the residual operand is produced after the projection: the ADD stays
+    spec = base()
+    p = _f16_projection(spec, "input", rows, d, d, 4)
+    late = spec.tensor("t", abi.F16, (1, rows, d))
+    spec.op("ABS", ["input"], [late])
+    spec.op("ADD", [p, late], ["out"])
+    spec.outputs.append(("out", abi.F16, (1, rows, d)))
+    g = _build_host_only(spec, fuse=True)
+    assert g.op_names() == ["MATMUL+ADD+CAST", "ABS", "ADD"]
+    g.close()
+
+    # 2b. an elementwise region behind the product moves into its call only when the product's kernel applies it
+    #     itself (the transformer block's GELU above); any other region stays a pass of its own
+    spec = base()
+    p = _f16_projection(spec, "input", rows, d, d, 4)
+    late = spec.tensor("t", abi.F16, (1, rows, d))
+    spec.op("MUL", ["input", "input"], [late], [0])
+    spec.op("ADD", [p, late], ["out"])
+    spec.outputs.append(("out", abi.F16, (1, rows, d)))
+    g = _build_host_only(spec, fuse=True)
+    assert g.op_names() == ["MATMUL+ADD+CAST", "ELEMENTWISE x2"]
+    g.close()
+
+    # 3. the residual exists before the projection: it rides on it; a second reader of the product prevents that
+    for second_reader in (False, True):
+        spec = base()
+        p = _f16_projection(spec, "input", rows, d, d, 5)
+        spec.op("ADD", ["input", p], ["out"])
+        spec.outputs.append(("out", abi.F16, (1, rows, d)))
+        if second_reader:
+            spec.op("CAST", [p], ["tap"])
+            spec.outputs.append(("tap", abi.F32, (1, rows, d)))
+        g = _build_host_only(spec, fuse=True)
+        assert g.op_names() == (["MATMUL+ADD+CAST", "ADD", "CAST"] if second_reader else ["MATMUL+ADD+CAST+ADD"])
+        g.close()
+
+    # 4. a head split whose innermost extent is no multiple of eight keeps its RESHAPE (an alias) and TRANSPOSE
+    spec = base()
+    p = _f16_projection(spec, "input", rows, d, 24, 6)
+    split = spec.tensor("t", abi.F16, (1, rows, 2, 12))
+    spec.op("RESHAPE", [p], [split])
+    spec.op("TRANSPOSE", [split], ["out"], [0, 2, 1, 3])
+    spec.outputs.append(("out", abi.F16, (1, 2, rows, 12)))
+    g = _build_host_only(spec, fuse=True)
+    assert g.op_names() == ["MATMUL+ADD+CAST", "TRANSPOSE"]
+    g.close()

@@ -9,6 +9,7 @@ from hip_util import gpu_available, hb
 from oracle_graph import run_spec
 
 graphs = importlib.import_module("ai-ml-emulation-layer-for-vulkan_amd.graphs")
+abi = importlib.import_module("ai-ml-emulation-layer-for-vulkan_amd.abi")
 
 pytestmark = pytest.mark.gpu
 
@@ -205,3 +206,72 @@ def test_transformer_block_fusions_do_not_change_a_bit(dev):
     assert outs[True][1].count("MATMUL+CAST+RESHAPE+TRANSPOSE") == 1       # the context leaves the product merged
     assert outs[True][1].count("TRANSPOSE") == 0                           # K leaves its projection transposed
     assert not [n for n in outs[True][1] if n.startswith("REDUCE_")] and len(outs[True][1]) < len(outs[False][1])
+
+
+def test_small_projection_graphs_fused_and_unfused_agree(dev):
+    """Graphs around one or two fp16 projections where the residual, grouping, view and in-call region fusions apply or
+    are refused for a reason (a second reader, an operand produced later, an extent the view cannot take): the fused
+    pipeline gives the bits of the operator-by-operator one on every graph output."""
+    from test_graph_host import _f16_projection
+    rows, d = 64, 32
+
+    def base():
+        spec = graphs.Spec()
+        spec.inputs.append(("input", abi.F16, (1, rows, d)))
+        return spec
+
+    def finish(spec, name, dtype, shape):
+        spec.outputs.append((name, dtype, shape))
+        return spec
+
+    cases = {}
+    spec = base()
+    p1, p2 = _f16_projection(spec, "input", rows, d, d, 1), _f16_projection(spec, "input", rows, d, d, 2)
+    p3 = _f16_projection(spec, "input", rows, d, 2 * d, 3)
+    spec.op("MUL", [p1, p2], ["out_a"], [0])
+    spec.op("CAST", [p3], ["out_b"])
+    finish(spec, "out_a", abi.F16, (1, rows, d))
+    cases["group"] = finish(spec, "out_b", abi.F32, (1, rows, 2 * d))
+    spec = base()
+    p1, p2 = _f16_projection(spec, "input", rows, d, d, 1), _f16_projection(spec, "input", rows, d, d, 2)
+    spec.op("ADD", [p1, p2], ["out"])
+    cases["sum_of_projections"] = finish(spec, "out", abi.F16, (1, rows, d))
+    for unary in ("ABS", None):
+        spec = base()
+        p = _f16_projection(spec, "input", rows, d, d, 4)
+        late = spec.tensor("t", abi.F16, (1, rows, d))
+        if unary:
+            spec.op(unary, ["input"], [late])
+        else:
+            spec.op("MUL", ["input", "input"], [late], [0])
+        spec.op("ADD", [p, late], ["out"])
+        cases["late_operand" if unary else "region"] = finish(spec, "out", abi.F16, (1, rows, d))
+    for tapped in (False, True):
+        spec = base()
+        p = _f16_projection(spec, "input", rows, d, d, 5)
+        spec.op("ADD", ["input", p], ["out"])
+        finish(spec, "out", abi.F16, (1, rows, d))
+        if tapped:
+            spec.op("CAST", [p], ["tap"])
+            finish(spec, "tap", abi.F32, (1, rows, d))
+        cases["residual_tapped" if tapped else "residual"] = spec
+    spec = base()
+    p = _f16_projection(spec, "input", rows, d, 24, 6)
+    split = spec.tensor("t", abi.F16, (1, rows, 2, 12))
+    spec.op("RESHAPE", [p], [split])
+    spec.op("TRANSPOSE", [split], ["out"], [0, 2, 1, 3])
+    cases["narrow_heads"] = finish(spec, "out", abi.F16, (1, 2, rows, 12))
+
+    x = np.random.default_rng(9).standard_normal((1, rows, d)).astype(np.float16)
+    for name, spec in cases.items():
+        results = []
+        for fuse in (False, True):
+            g = graphs.build(dev, spec, fuse=fuse)
+            g.set_input("input", x)
+            g.dispatch()
+            results.append({o[0]: g.get_output(o[0]) for o in spec.outputs})
+            g.close()
+        for out in results[0]:
+            a, b = results[0][out], results[1][out]
+            assert a.shape == b.shape and np.array_equal(a.view(np.uint8), b.view(np.uint8)), (name, out)
+            assert np.isfinite(a.astype(np.float32)).all() and np.abs(a.astype(np.float32)).max() > 0, (name, out)
