@@ -29,8 +29,13 @@
  * MAX_POOL2D, RESCALE+ADD, CAST, CONCAT, SLICE, MAXIMUM, RESHAPE) plus brute-force / library cross-checks in
  * tests/ (MATMUL, DEPTHWISE_CONV2D, AVG_POOL2D, TABLE, CLAMP, MUL, SUB, REDUCE, TRANSPOSE, PAD: no reference test
  * exists; they are pinned against numpy int64 restatements of the TOSA formulae and hand-computed cases).
- * Floating-point paths (f16/f32 EXP, RSQRT, TANH, RECIPROCAL, f16-sequential REDUCE/MATMUL rounding) depend on
- * the Vulkan driver's builtins in the reference: PARITY UNPINNED beyond the stated tolerance.
+ * The floating-point unary operators (EXP, LOG, COS, SIGMOID, RECIPROCAL, RSQRT, CEIL, FLOOR, ERF, TANH with its
+ * three branches, SIN), the remaining binary operators (BITWISE_*, LOGICAL_*, shifts, comparisons, MINIMUM, INTDIV,
+ * POW) and REDUCE PRODUCT / MIN / MAX are pinned by tests/test_oracle_pins.py against the C library in double
+ * precision rounded once, Python integers and the shader's polynomial coefficients in exact rationals.
+ * What stays PARITY UNPINNED is what only a run of the reference on its Vulkan driver could fix: the last-ulp
+ * behaviour of the driver's builtins (exp, log, inversesqrt, tanh, sin, cos, pow; this restatement returns the
+ * correctly rounded value) and the payload / sign of NaN results.
  */
 #ifndef MLEL_ORACLE_H
 #define MLEL_ORACLE_H
