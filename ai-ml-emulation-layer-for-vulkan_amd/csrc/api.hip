@@ -71,6 +71,17 @@ struct Scratch {
     }
 };
 
+// Temporary of a fused entry point's operator-by-operator route.  That route allocates, and synchronises the stream
+// before the temporary is freed on return; a stream that is being captured can do neither, so the call is refused there.
+int alloc_fallback(Scratch &t, size_t bytes, void *stream, const char *what) {
+    MLEL_REQUIRE(!stream_is_capturing((hipStream_t)stream), MLEL_ERR_UNSUPPORTED,
+                 "%s: no one-pass kernel takes these operands, and the operator-by-operator route allocates a temporary "
+                 "and synchronises, which is not possible on a stream that is being captured",
+                 what);
+    MLEL_HIP_CHECK(hipMalloc(&t.ptr, bytes));
+    return 0;
+}
+
 int run_unfused_tail(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *acc,
                      const mlel_epilogue *epi) {
     // RESCALE into `out`, then CLAMP in place: exactly the operator sequence the fused kernels replace
@@ -508,7 +519,7 @@ int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor
     if (rc != 0) return rc < 0 ? rc : 0;
     // no specialised kernel for this layout: run the unfused operator sequence through an int32 scratch tensor
     Scratch scratch;
-    MLEL_HIP_CHECK(hipMalloc(&scratch.ptr, (size_t)numel(out) * 4 + 16));
+    MLEL_TRY(alloc_fallback(scratch, (size_t)numel(out) * 4 + 16, stream, __func__));
     mlel_tensor acc = packed_like(out, MLEL_I32, scratch.ptr);
     MLEL_TRY(mlel_hip_conv2d(ctx, stream, &acc, in, weights, bias, attr));
     MLEL_TRY(run_unfused_tail(ctx, (hipStream_t)stream, out, &acc, epi));
@@ -558,7 +569,7 @@ int mlel_hip_conv2d_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_
     }
     // otherwise the two fused halves in sequence through an 8-bit temporary
     Scratch scratch;
-    MLEL_HIP_CHECK(hipMalloc(&scratch.ptr, (size_t)numel(out) + 16));
+    MLEL_TRY(alloc_fallback(scratch, (size_t)numel(out) + 16, stream, __func__));
     mlel_tensor conv_out = packed_like(out, conv_dt, scratch.ptr);
     MLEL_TRY(mlel_hip_conv2d_rescale_clamp(ctx, stream, &conv_out, in, weights, bias, attr, epi));
     if (residual_first)
@@ -583,7 +594,7 @@ int mlel_hip_matmul_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out,
     const int rc = try_matmul_i8_mfma(ctx, (hipStream_t)stream, out, a, b, attr, &fe);
     if (rc != 0) return rc < 0 ? rc : 0;
     Scratch scratch;
-    MLEL_HIP_CHECK(hipMalloc(&scratch.ptr, (size_t)numel(out) * 4 + 16));
+    MLEL_TRY(alloc_fallback(scratch, (size_t)numel(out) * 4 + 16, stream, __func__));
     mlel_tensor acc = packed_like(out, MLEL_I32, scratch.ptr);
     MLEL_TRY(mlel_hip_matmul(ctx, stream, &acc, a, b, attr));
     MLEL_TRY(run_unfused_tail(ctx, (hipStream_t)stream, out, &acc, epi));
@@ -626,7 +637,7 @@ int mlel_hip_elementwise_chain(mlel_ctx *ctx, void *stream, const mlel_tensor *o
                 for (int d = 0; d < a->rank; d++) shape.dims[d] = std::max(a->dims[d], b->dims[d]);
             }
             if (st.kind == MLEL_CHAIN_REDUCE) shape.dims[shape.rank - 1] = 1;
-            MLEL_HIP_CHECK(hipMalloc(&temps[static_cast<size_t>(i)].ptr, (size_t)numel(&shape) * 4 + 16));
+            MLEL_TRY(alloc_fallback(temps[static_cast<size_t>(i)], (size_t)numel(&shape) * 4 + 16, stream, __func__));
             result = packed_like(&shape, st.dtype, temps[static_cast<size_t>(i)].ptr);
         }
         switch (st.kind) {
@@ -687,7 +698,7 @@ int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *ou
     if (out->rank == 6) {
         // the view without the fused kernel: the product into a dense temporary, then a strided copy
         Scratch dense_mem;
-        MLEL_HIP_CHECK(hipMalloc(&dense_mem.ptr, (size_t)numel(out) * 2 + 16));
+        MLEL_TRY(alloc_fallback(dense_mem, (size_t)numel(out) * 2 + 16, stream, __func__));
         mlel_tensor dense3 = *out;
         dense3.rank = 3;
         dense3.dims[0] = out->dims[0] * out->dims[1];
@@ -702,13 +713,13 @@ int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *ou
     }
     // no fused kernel for these strides / alignments: the three operators one after another through temporaries
     Scratch acc_mem, sum_mem;
-    MLEL_HIP_CHECK(hipMalloc(&acc_mem.ptr, (size_t)numel(out) * 4 + 16));
+    MLEL_TRY(alloc_fallback(acc_mem, (size_t)numel(out) * 4 + 16, stream, __func__));
     mlel_tensor acc = packed_like(out, MLEL_F32, acc_mem.ptr);
     MLEL_TRY(mlel_hip_matmul(ctx, stream, &acc, a, b, attr));
     const mlel_tensor *cast_in = &acc;
     mlel_tensor sum{};
     if (bias) {
-        MLEL_HIP_CHECK(hipMalloc(&sum_mem.ptr, (size_t)numel(out) * 4 + 16));
+        MLEL_TRY(alloc_fallback(sum_mem, (size_t)numel(out) * 4 + 16, stream, __func__));
         sum = packed_like(out, MLEL_F32, sum_mem.ptr);
         MLEL_TRY(mlel_hip_elementwise_binary(ctx, stream, MLEL_BIN_ADD, &sum, &acc, bias, MLEL_NAN_PROPAGATE));
         cast_in = &sum;
@@ -727,7 +738,12 @@ int mlel_hip_matmul_bias_cast_chain(mlel_ctx *ctx, void *stream, const mlel_tens
                      chain->n_steps <= MLEL_CHAIN_MAX_STEPS,
                  MLEL_ERR_INVALID, "matmul_bias_cast_chain: %d inputs, %d steps", chain->n_inputs, chain->n_steps);
     MLEL_TRY(check_supported(out, "matmul_bias_cast_chain out"));
-    if (out->rank == 3 && out->dtype == MLEL_F16 && a != nullptr && b != nullptr && a->rank == 3 && b->rank == 3 &&
+    MLEL_TRY(check_supported(a, "matmul_bias_cast_chain a"));
+    MLEL_TRY(check_supported(b, "matmul_bias_cast_chain b"));
+    if (bias) MLEL_TRY(check_supported(bias, "matmul_bias_cast_chain bias"));
+    for (int i = 1; i < chain->n_inputs; i++)  // input 0 is the product itself
+        MLEL_TRY(check_supported(chain->inputs[i], "matmul_bias_cast_chain chain input"));
+    if (out->rank == 3 && out->dtype == MLEL_F16 && a->rank == 3 && b->rank == 3 &&
         a->dtype == MLEL_F16 && b->dtype == MLEL_F16 && (bias == nullptr || (bias->dtype == MLEL_F32 && bias->rank == 3)) &&
         chain_is_gelu_tanh(chain)) {
         const int rc = try_matmul_f16_mfma(ctx, (hipStream_t)stream, out, a, b, attr, true, bias, nullptr, &chain->inputs[1]);
@@ -735,7 +751,7 @@ int mlel_hip_matmul_bias_cast_chain(mlel_ctx *ctx, void *stream, const mlel_tens
     }
     // the product into a temporary, then the chain over it
     Scratch product_mem;
-    MLEL_HIP_CHECK(hipMalloc(&product_mem.ptr, (size_t)numel(out) * 2 + 16));
+    MLEL_TRY(alloc_fallback(product_mem, (size_t)numel(out) * 2 + 16, stream, __func__));
     const mlel_tensor product = packed_like(out, MLEL_F16, product_mem.ptr);
     MLEL_TRY(mlel_hip_matmul_bias_cast(ctx, stream, &product, a, b, bias, attr));
     mlel_chain over = *chain;
@@ -758,10 +774,13 @@ int mlel_hip_matmul_bias_cast_group(mlel_ctx *ctx, void *stream, const mlel_matm
     MLEL_REQUIRE(products != nullptr && n_products >= 1 && n_products <= MLEL_MATMUL_GROUP_MAX && attr != nullptr,
                  MLEL_ERR_INVALID, "matmul_bias_cast_group: 1 to %d products", MLEL_MATMUL_GROUP_MAX);
     const mlel_tensor *outs[MLEL_MATMUL_GROUP_MAX], *bs[MLEL_MATMUL_GROUP_MAX], *biases[MLEL_MATMUL_GROUP_MAX];
-    bool fusable = a != nullptr && a->rank == 3 && a->dtype == MLEL_F16;
+    MLEL_TRY(check_supported(a, "matmul_bias_cast_group a"));
+    bool fusable = a->rank == 3 && a->dtype == MLEL_F16;
     for (int i = 0; i < n_products; i++) {
         outs[i] = products[i].out, bs[i] = products[i].b, biases[i] = products[i].bias;
-        MLEL_REQUIRE(outs[i] != nullptr && bs[i] != nullptr, MLEL_ERR_INVALID, "matmul_bias_cast_group: null tensor in product %d", i);
+        MLEL_TRY(check_supported(outs[i], "matmul_bias_cast_group out"));
+        MLEL_TRY(check_supported(bs[i], "matmul_bias_cast_group b"));
+        if (biases[i]) MLEL_TRY(check_supported(biases[i], "matmul_bias_cast_group bias"));
         fusable = fusable && bs[i]->rank == 3 && bs[i]->dtype == MLEL_F16 && outs[i]->dtype == MLEL_F16 &&
                   (outs[i]->rank == 3 || outs[i]->rank == 6) &&
                   (biases[i] == nullptr || (biases[i]->dtype == MLEL_F32 && biases[i]->rank == 3));
@@ -781,16 +800,19 @@ int mlel_hip_matmul_bias_cast_add(mlel_ctx *ctx, void *stream, const mlel_tensor
     MLEL_REQUIRE(attr != nullptr && residual != nullptr, MLEL_ERR_INVALID, "matmul_bias_cast_add: null argument");
     MLEL_TRY(check_supported(out, "matmul_bias_cast_add out"));
     MLEL_TRY(check_supported(residual, "matmul_bias_cast_add residual"));
+    MLEL_TRY(check_supported(a, "matmul_bias_cast_add a"));
+    MLEL_TRY(check_supported(b, "matmul_bias_cast_add b"));
+    if (bias) MLEL_TRY(check_supported(bias, "matmul_bias_cast_add bias"));
     MLEL_REQUIRE(out->rank == 3 && residual->dtype == MLEL_F16 && out->dtype == MLEL_F16 && same_shape(out, residual),
                  MLEL_ERR_INVALID, "matmul_bias_cast_add: the residual is an fp16 tensor of the output's shape");
-    if (a != nullptr && b != nullptr && a->dtype == MLEL_F16 && b->dtype == MLEL_F16 && a->rank == 3 && b->rank == 3 &&
+    if (a->dtype == MLEL_F16 && b->dtype == MLEL_F16 && a->rank == 3 && b->rank == 3 &&
         (bias == nullptr || (bias->dtype == MLEL_F32 && bias->rank == 3))) {
         const int rc = try_matmul_f16_mfma(ctx, (hipStream_t)stream, out, a, b, attr, true, bias, residual);
         if (rc != 0) return rc < 0 ? rc : 0;
     }
     // no fused kernel for these strides / alignments: the projection into a temporary, then the addition
     Scratch proj_mem;
-    MLEL_HIP_CHECK(hipMalloc(&proj_mem.ptr, (size_t)numel(out) * 2 + 16));
+    MLEL_TRY(alloc_fallback(proj_mem, (size_t)numel(out) * 2 + 16, stream, __func__));
     const mlel_tensor proj = packed_like(out, MLEL_F16, proj_mem.ptr);
     MLEL_TRY(mlel_hip_matmul_bias_cast(ctx, stream, &proj, a, b, bias, attr));
     MLEL_TRY(mlel_hip_elementwise_binary(ctx, stream, MLEL_BIN_ADD, out, &proj, residual, MLEL_NAN_PROPAGATE));
@@ -812,7 +834,7 @@ int mlel_hip_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor
     const int rc = try_dwconv_i8_fast(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe);
     if (rc != 0) return rc < 0 ? rc : 0;
     Scratch scratch;
-    MLEL_HIP_CHECK(hipMalloc(&scratch.ptr, (size_t)numel(out) * 4 + 16));
+    MLEL_TRY(alloc_fallback(scratch, (size_t)numel(out) * 4 + 16, stream, __func__));
     mlel_tensor acc = packed_like(out, MLEL_I32, scratch.ptr);
     MLEL_TRY(mlel_hip_depthwise_conv2d(ctx, stream, &acc, in, weights, bias, attr));
     MLEL_TRY(run_unfused_tail(ctx, (hipStream_t)stream, out, &acc, epi));

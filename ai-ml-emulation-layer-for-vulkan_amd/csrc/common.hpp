@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <mutex>
 
 #include "../../include/mlel_hip.h"
 
@@ -408,7 +409,31 @@ inline dim3 grid_1d(int64_t work_items, int block) { return dim3((unsigned)((wor
 
 }  // namespace mlel
 
+// Device scratch for the contraction kernels' split-K mode: int32 partial tiles and one arrival counter per tile.
+// One workspace per stream that has used the mode (the calls of one stream are ordered, those of different streams
+// are not), created the first time a stream asks for it outside a graph capture and freed with the context.
+struct SplitWorkspace {
+    hipStream_t stream;
+    char *partials;      // kSplitPartialBytes
+    uint32_t *counters;  // kSplitCounters, zero between launches (the last block to arrive resets its counter)
+};
+constexpr size_t kSplitPartialBytes = size_t(16) << 20;
+constexpr int kSplitCounters = 4096;
+constexpr int kMaxSplitWorkspaces = 16;
+
 struct mlel_ctx {
     int device;
     hipDeviceProp_t props;
+    std::mutex ws_lock;
+    SplitWorkspace ws[kMaxSplitWorkspaces];
+    int n_ws = 0;
+    int split_k = 8;  // most blocks per tile in split-K mode; 0 or 1: never split (MLEL_SPLIT_K in the environment)
 };
+
+namespace mlel {
+// The split-K workspace of `stream`, or false when there is none and none can be made now (stream is being
+// captured, table full, allocation failed): the caller then runs without splitting.
+bool split_workspace(mlel_ctx *ctx, hipStream_t stream, SplitWorkspace *out);
+void free_split_workspaces(mlel_ctx *ctx);
+bool stream_is_capturing(hipStream_t s);
+}  // namespace mlel

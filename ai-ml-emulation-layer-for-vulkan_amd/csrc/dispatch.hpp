@@ -94,9 +94,18 @@ struct ConvResidual {
     const mlel_tensor *res;
     FusedEpilogue f_res, f_conv, f_out;
 };
+// `static_scratch`: where a split-K launch keeps its partial tiles and counters instead of the context's per-stream
+// workspace (the counters must be zero); `used_split` reports whether the launch split K
+struct GemmScratch {
+    char *partials;
+    uint32_t *counters;
+    size_t partial_bytes;
+    bool *used_split;
+};
 int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                        const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
-                       const FusedEpilogue *epi, const ConvResidual *residual = nullptr);
+                       const FusedEpilogue *epi, const ConvResidual *residual = nullptr,
+                       const GemmScratch *static_scratch = nullptr);
 // ---- direct (dot4) convolution for very small input channel counts (conv_direct.hip) ----
 int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                          const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,

@@ -2,10 +2,21 @@
 // The kernel itself is in gemm_i8_kernel.hpp; every tile shape is instantiated in its own gemm_i8_tile*.hip.
 #include "gemm_i8_kernel.hpp"
 
+#include <algorithm>
+
 namespace mlel {
 namespace {
 
-int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
+// Where the split-K mode may keep its partial tiles and counters: the context's workspace of the launch stream, or a
+// caller-chosen region (the statically allocated scratch).  `partial_bytes` == 0: never split.
+struct SplitScratch {
+    char *partials = nullptr;
+    uint32_t *counters = nullptr;
+    size_t partial_bytes = 0;
+    bool from_ctx = true;  // look the workspace up in the context when a split is wanted
+};
+
+int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g, const SplitScratch &scratch) {
     // operand fetch modes
     int xmode = X_GENERIC, wmode = W_GENERIC;
     const bool small = g.x_bytes != 0 && g.w_bytes != 0;  // both operand extents fit 31-bit buffer offsets
@@ -75,7 +86,41 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g) {
     const int64_t total = (int64_t)g.tiles_m * g.tiles_n * g.batches;
     MLEL_REQUIRE(total > 0 && total < (int64_t(1) << 30), MLEL_ERR_LIMIT, "contraction: %lld tiles", (long long)total);
     g.total_tiles = (int)total;
-    g.chunk = (int)((total + 7) / 8);
+    // Split K only when the tiles fill less than half of the machine and the K loop is very long.  Measured on
+    // MobileNetV2's 7 x 7 layers (75 - 125 tiles, 9 - 15 K steps): a split removes about 0.3 us per K step from a
+    // block but the exchange of partial tiles through memory (write-through stores, one atomic, loads) costs 4 - 5 us
+    // of latency, so those layers ran 1.5 - 2.5 us SLOWER split; the mode pays from about 24 removed steps on.
+    // At least three K steps per block, at most eight splits.
+    const int steps = (g.K + BK - 1) / BK;
+    g.splits = 1;
+    g.split_steps = steps;
+    g.partials = nullptr;
+    g.counters = nullptr;
+    if (ctx->split_k > 1 && xmode != X_PLAIN_DL && total * 2 <= cus && total <= kSplitCounters && steps >= 32) {
+        int want = (int)std::min<int64_t>(std::min(8, ctx->split_k), (cus + total - 1) / total);
+        int per = std::max(3, (steps + want - 1) / want);
+        const int splits = (steps + per - 1) / per;
+        const size_t need = (size_t)total * splits * tile.bm * BN * sizeof(int32_t);
+        if (splits > 1 && steps - per >= 24) {
+            SplitScratch sc = scratch;
+            if (sc.from_ctx) {
+                SplitWorkspace w;
+                if (split_workspace(ctx, s, &w)) {
+                    sc.partials = w.partials;
+                    sc.counters = w.counters;
+                    sc.partial_bytes = kSplitPartialBytes;
+                }
+            }
+            if (sc.partials != nullptr && need <= sc.partial_bytes) {
+                g.splits = splits;
+                g.split_steps = per;
+                g.partials = reinterpret_cast<int32_t *>(sc.partials);
+                g.counters = sc.counters;
+            }
+        }
+    }
+    const int64_t blocks = total * g.splits;
+    g.chunk = (int)((blocks + 7) / 8);
     const dim3 grid((unsigned)(g.chunk * 8));
     switch (tile.id) {
     case 0: launch_gemm_tile0(&g, xmode, wmode, grid, s); break;
@@ -128,7 +173,7 @@ bool packed_tail(const mlel_tensor *t, int from) {
 // carries it applies (plain rows, 8-bit epilogue, not the direct-to-LDS tiles)
 int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                        const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
-                       const FusedEpilogue *epi, const ConvResidual *residual) {
+                       const FusedEpilogue *epi, const ConvResidual *residual, const GemmScratch *static_scratch) {
     if (in->dtype != MLEL_I8 || w->dtype != MLEL_I8 || bias->dtype != MLEL_I32 || a->acc_type != MLEL_ACC_I32) return 0;
     if (residual != nullptr && (epi == nullptr || out->dtype != MLEL_I8)) return 0;
     if (epi == nullptr && out->dtype != MLEL_I32) return 0;
@@ -202,7 +247,15 @@ int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
         g.rs_conv = make_ref(residual->f_conv);
         g.rs_out = make_ref(residual->f_out);
     }
-    MLEL_TRY(launch_gemm(ctx, s, g));
+    SplitScratch sc;
+    if (static_scratch != nullptr) {  // the caller's region instead of the context's workspace
+        sc.from_ctx = false;
+        sc.partials = static_scratch->partials;
+        sc.counters = static_scratch->counters;
+        sc.partial_bytes = static_scratch->partial_bytes;
+    }
+    MLEL_TRY(launch_gemm(ctx, s, g, sc));
+    if (static_scratch != nullptr && static_scratch->used_split != nullptr) *static_scratch->used_split = g.splits > 1;
     return 1;
 }
 
@@ -253,7 +306,7 @@ int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     g.ldo = N;
     g.out_batch = out->strides[0];
     MLEL_TRY(fill_epilogue(g, out, epi));
-    MLEL_TRY(launch_gemm(ctx, s, g));
+    MLEL_TRY(launch_gemm(ctx, s, g, SplitScratch{}));
     return 1;
 }
 

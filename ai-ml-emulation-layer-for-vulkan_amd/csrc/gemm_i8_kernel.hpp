@@ -74,6 +74,14 @@ struct GemmArgs {
     ScaleRef rs_res, rs_conv, rs_out;
     // launch geometry
     int32_t tiles_m, tiles_n, total_tiles, chunk;
+    // Split K (register-staged pipeline only): `splits` blocks share one output tile, block s multiplies the K steps
+    // [s * split_steps, (s + 1) * split_steps).  Every block writes its int32 partial tile (zero-point terms of its K
+    // range already applied, the bias in split 0) to `partials` and bumps the tile's counter; the block that finds
+    // the counter at splits - 1 adds the other partials to its own (int32 addition wraps, so the order is
+    // immaterial), resets the counter and runs the epilogue.  splits == 1: split_steps = all K steps, no scratch.
+    int32_t splits, split_steps;
+    int32_t *partials;   // [total_tiles][splits][BM * BN], register-major so that every store is coalesced
+    uint32_t *counters;  // [total_tiles], zero before the launch
 };
 
 struct ChanParams {  // per output channel, in LDS: 32 bytes = two 128-bit reads
@@ -298,8 +306,18 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
 
     // ---- XCD-aware tile assignment: consecutive block ids land on different XCDs (8 of them, each with its own
     // L2), so block b is given tile (b % 8) * chunk + b / 8: tiles that share operands stay on one XCD.
-    const int lin = (int)(blockIdx.x % 8) * g.chunk + (int)(blockIdx.x / 8);
-    if (lin >= g.total_tiles) return;
+    const int lin_all = (int)(blockIdx.x % 8) * g.chunk + (int)(blockIdx.x / 8);
+    if (lin_all >= g.total_tiles * g.splits) return;
+    // the splits of one tile are consecutive, so they run on one XCD and exchange their partials through its L2
+    int lin = lin_all, split = 0;
+    if (XMODE != X_PLAIN_DL && g.splits > 1) {
+        lin = __builtin_amdgcn_readfirstlane(lin_all / g.splits);
+        split = lin_all - lin * g.splits;
+    }
+    const int step0 = split * g.split_steps;                                  // first K step of this block
+    const int nk_own = min(g.split_steps, (g.K + BK - 1) / BK - step0);       // and how many it multiplies
+    const int k_begin = step0 * BK;
+    const int k_len = min(g.K, k_begin + nk_own * BK) - k_begin;              // bytes of K in this block's range
     const int tiles_per_batch = g.tiles_m * g.tiles_n;
     // the divisions run on the vector ALU; readfirstlane returns the (wave-uniform) results to scalar registers so
     // that everything derived from them (base pointers, buffer resources) is scalar as well
@@ -335,7 +353,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     const bool chan_live = tid < BN && n_base + tid < g.N;
     if (chan_live) {
         const int gn = n_base + tid;
-        chan_bias = g.bias ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
+        chan_bias = (g.bias && split == 0) ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
         if (g.fused) {
             const int ci = g.rp.per_channel ? gn : 0;
             chan_mult = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
@@ -369,8 +387,14 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         rows[i] = r;
     }
     KState ks{0, 0, 0};                      // X_GENERIC: k position of this thread's piece
-    if (XMODE == X_GENERIC) kstate_advance(ks, x_kc * 16, g.IC, g.KW);
+    if (XMODE == X_GENERIC) kstate_advance(ks, k_begin + x_kc * 16, g.IC, g.KW);
     int tap_ky = 0, tap_kx = 0, tap_ic = 0;  // X_TAP: uniform position of the K step
+    if (XMODE == X_TAP && k_begin > 0) {
+        const int tap = k_begin / g.IC;
+        tap_ic = k_begin - tap * g.IC;
+        tap_ky = tap / g.KW;
+        tap_kx = tap - tap_ky * g.KW;
+    }
     const __amdgpu_buffer_rsrc_t xres = make_rsrc(xb, g.x_bytes), wres = make_rsrc(wb, g.w_bytes);
 
     uint32_t woff[WCHUNKS];  // fast modes: byte offset of the piece at k = 0, or kOobOffset
@@ -757,18 +781,18 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     // loads may remain in flight at each wait instead of draining them all.
     // the generic fetch state is large, and so are the register sets of the widest tiles
     constexpr int DEPTH = (XMODE == X_GENERIC || WMODE == W_GENERIC || XROWS + WCHUNKS > 4) ? 2 : 4;
-    const int nk = (g.K + BK - 1) / BK;
+    const int nk = nk_own;
     uint4 xr[DEPTH][XROWS], wr[DEPTH][WCHUNKS];
     uint32_t xp[DEPTH];
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) prefetch(d * BK, xr[d], wr[d], xp[d]);
+    for (int d = 0; d < DEPTH; d++) prefetch(k_begin + d * BK, xr[d], wr[d], xp[d]);
     stage(0, xr[0], wr[0], xp[0]);
     __syncthreads();
     for (int step = 0; step < nk; step += DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
             if (step + d < nk) {  // uniform
-                prefetch((step + d + DEPTH) * BK, xr[d], wr[d], xp[d]);
+                prefetch(k_begin + (step + d + DEPTH) * BK, xr[d], wr[d], xp[d]);
                 compute(d & 1);
                 stage((d + 1) & 1, xr[(d + 1) % DEPTH], wr[(d + 1) % DEPTH], xp[(d + 1) % DEPTH]);
                 __syncthreads();
@@ -795,7 +819,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             if (lane < 32) {
                 const int n = wave_n * WN + j * 32 + lane;
                 cp[n].bias_adj = (int32_t)((uint32_t)cp[n].bias_adj - (uint32_t)g.zx * (uint32_t)s +
-                                           (uint32_t)g.K * (uint32_t)g.zx * (uint32_t)g.zw);
+                                           (uint32_t)k_len * (uint32_t)g.zx * (uint32_t)g.zw);
             }
         }
     }
@@ -805,6 +829,70 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             xsum[i] = (int32_t)((uint32_t)(xsum[i] + __shfl_xor(xsum[i], 32)) * (uint32_t)g.zw);
     }
     __syncthreads();
+
+    if constexpr (XMODE != X_PLAIN_DL) {
+        if (g.splits > 1) {
+            // ---- split K: this block's partial tile, complete with the bias / zero-point terms of its K range
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                const uint32_t xc = need_xsum ? (uint32_t)xsum[i] : 0u;
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const int nl = wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            acc[i][j][4 * q + e] =
+                                (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)cp[nl + e].bias_adj - xc);
+                    }
+                xsum[i] = 0;
+            }
+            __syncthreads();  // every wavefront has read the per-channel terms: the epilogue must not add them again
+            if (tid < BN) cp[tid].bias_adj = 0;
+            // The exchange uses device-scope atomic stores and loads (relaxed): they are coherent across the GPU's
+            // eight L2 caches by themselves, so no fence is needed -- a device-scope fence would write back and
+            // invalidate the whole L2 (measured: 20 - 50 us per launch).  Order: every thread waits until its own
+            // stores have been acknowledged, the block barrier extends that to the block, then one thread counts the
+            // arrival; the block that arrives last reads the others' tiles after it has seen the count.
+            int32_t *mine = g.partials + ((int64_t)lin * g.splits + split) * (BM * BN) + tid;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        __hip_atomic_store(&mine[((i * TN + j) * 16 + r) * NTHREADS], acc[i][j][r], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            int *last_flag = reinterpret_cast<int *>(smem);  // the operand buffers are free after the main loop
+            __syncthreads();
+            if (tid == 0) {
+                const uint32_t arrived =
+                    __hip_atomic_fetch_add(&g.counters[lin], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const int last = arrived == (uint32_t)(g.splits - 1);
+                if (last)  // ready for the next launch
+                    __hip_atomic_store(&g.counters[lin], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *last_flag = last;
+            }
+            __syncthreads();
+            if (*last_flag == 0) return;
+            for (int o = 0; o < g.splits; o++) {
+                if (o == split) continue;
+                const int32_t *theirs = g.partials + ((int64_t)lin * g.splits + o) * (BM * BN) + tid;
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++)
+                            acc[i][j][r] = (int32_t)((uint32_t)acc[i][j][r] +
+                                                     (uint32_t)__hip_atomic_load(&theirs[((i * TN + j) * 16 + r) * NTHREADS],
+                                                                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            }
+            __syncthreads();  // cp[].bias_adj = 0 is in place for every wavefront
+        }
+    }
 
     // ---- epilogue: lane holds output position m = lane % 32 of each tile row and, per register group q, the four
     // channels n0 .. n0+3 with n0 = 8q + 4 * (lane / 32)

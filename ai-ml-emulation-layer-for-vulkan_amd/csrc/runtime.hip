@@ -2,6 +2,7 @@
 // declared in include/mlel_hip.h.
 #include "common.hpp"
 
+#include <cstdlib>
 #include <cstring>
 
 namespace mlel {
@@ -115,6 +116,50 @@ __global__ void __launch_bounds__(256) copy_kernel(uint4 *__restrict__ dst, cons
     if (blockIdx.x == 0 && threadIdx.x < n_tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
 }
 
+bool stream_is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return st != hipStreamCaptureStatusNone;
+}
+
+bool split_workspace(mlel_ctx *ctx, hipStream_t stream, SplitWorkspace *out) {
+    std::lock_guard<std::mutex> guard(ctx->ws_lock);
+    for (int i = 0; i < ctx->n_ws; i++)
+        if (ctx->ws[i].stream == stream) {
+            *out = ctx->ws[i];
+            return true;
+        }
+    // a new workspace is an allocation: not inside a capture, and not beyond the table
+    if (ctx->n_ws >= kMaxSplitWorkspaces || stream_is_capturing(stream)) return false;
+    SplitWorkspace w{stream, nullptr, nullptr};
+    if (hipMalloc(reinterpret_cast<void **>(&w.partials), kSplitPartialBytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    if (hipMalloc(reinterpret_cast<void **>(&w.counters), sizeof(uint32_t) * kSplitCounters) != hipSuccess ||
+        hipMemset(w.counters, 0, sizeof(uint32_t) * kSplitCounters) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipFree(w.partials);
+        if (w.counters) (void)hipFree(w.counters);
+        return false;
+    }
+    ctx->ws[ctx->n_ws++] = w;
+    *out = w;
+    return true;
+}
+
+void free_split_workspaces(mlel_ctx *ctx) {
+    std::lock_guard<std::mutex> guard(ctx->ws_lock);
+    for (int i = 0; i < ctx->n_ws; i++) {
+        (void)hipFree(ctx->ws[i].partials);
+        (void)hipFree(ctx->ws[i].counters);
+    }
+    ctx->n_ws = 0;
+}
+
 }  // namespace mlel
 
 using namespace mlel;
@@ -150,11 +195,19 @@ int mlel_hip_init(int device, mlel_ctx **out_ctx) {
         delete ctx;
         return set_error(MLEL_ERR_DEVICE, "init: hipGetDeviceProperties: %s", hipGetErrorString(pe));
     }
+    if (const char *env = std::getenv("MLEL_SPLIT_K")) ctx->split_k = std::atoi(env);  // 0: off, n: at most n splits
     *out_ctx = ctx;
     return 0;
 }
 
-void mlel_hip_destroy(mlel_ctx *ctx) { delete ctx; }
+void mlel_hip_destroy(mlel_ctx *ctx) {
+    if (ctx == nullptr) return;
+    if (hipSetDevice(ctx->device) == hipSuccess) {
+        (void)hipDeviceSynchronize();  // no launch may still be using a workspace that is about to be freed
+        free_split_workspaces(ctx);
+    }
+    delete ctx;
+}
 
 int mlel_hip_device_info(mlel_ctx *ctx, int32_t *cu_count, int32_t *clock_khz, int32_t *mem_clock_khz,
                          int32_t *bus_width_bits, char *name, size_t name_len) {

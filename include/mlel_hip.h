@@ -380,7 +380,14 @@ int mlel_hip_select(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const m
 
 /* ---- fused entry points (chosen only by the host-side fusion pass; no counterpart in the reference, which
  * runs one dispatch per TOSA instruction: graph/compute_graph_op.cpp:2500-2509).  Each equals, bit for bit,
- * the unfused sequence <contraction> -> RESCALE -> [CLAMP] with an int32 intermediate. ---- */
+ * the unfused sequence <contraction> -> RESCALE -> [CLAMP] with an int32 intermediate.
+ * When no one-pass kernel takes the operands (strided views, unusual types) these entry points run that operator
+ * sequence themselves: they then hipMalloc temporaries, and synchronise the stream before freeing them on return.
+ * On a stream that is being captured into a graph that route returns MLEL_ERR_UNSUPPORTED instead (nothing is
+ * launched).  The int8 contractions may split K over several blocks when a layer has fewer tiles than the GPU has
+ * compute units; the partial tiles live in a per-stream workspace owned by the context (16 MiB, created the first
+ * time a stream needs it outside a capture; MLEL_SPLIT_K=0 in the environment at mlel_hip_init switches the mode
+ * off).  Integer addition wraps, so a split result is bit-identical. ---- */
 int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
                                   const mlel_tensor *weights, const mlel_tensor *bias,
                                   const mlel_conv2d_attr *attr, const mlel_epilogue *epi);

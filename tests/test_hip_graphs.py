@@ -129,6 +129,97 @@ def test_config4_transformer_block_full_size(dev):
     assert np.abs(out - ref).mean() <= 2e-3
 
 
+def test_config4_full_size_first_batch_element_vs_oracle(dev, oracle):
+    """BASELINE config 4 at full size on the GPU (batch 8, seq 512, d_model 768, 12 heads, FFN 3072) against the oracle
+    at the stated tolerance, max abs error <= 1e-2: no operator of the block mixes batch elements, so the oracle runs
+    the same block (same weights: they do not depend on the batch) on the first element alone."""
+    spec = graphs.transformer_block_spec()
+    x = np.random.default_rng(1004).standard_normal(spec.inputs[0][2]).astype(np.float16)
+    out = run_float_graph(dev, spec, x)
+    one = graphs.transformer_block_spec(batch=1)
+    exp, _ = run_spec(oracle, one, {"input": x[:1]})
+    err = np.abs(out[:1].astype(np.float32) - exp["output"].astype(np.float32)).max()
+    assert np.isfinite(out.astype(np.float32)).all()
+    assert err <= 1e-2, err
+
+
+def capture_and_replay(dev, spec, inputs):
+    """Dispatches `spec` eagerly for every input, then captures one dispatch into a HIP graph and replays it for the
+    same inputs, with uploads, downloads and synchronisations between the replays; returns both result lists."""
+    import ctypes as C
+    lib = dev.lib
+    stream = dev.new_stream()
+    null_stream, dev.stream = dev.stream, stream
+    try:
+        g = graphs.build(dev, spec, fuse=True)
+        eager = []
+        for x in inputs:  # also creates whatever per-stream workspace the kernels want before the capture
+            g.set_input("input", x)
+            g.dispatch()
+            eager.append(g.get_output("output"))
+        dev._check(lib.mlel_hip_capture_begin(dev.ctx, stream))
+        g.dispatch()
+        exe = C.c_void_p()
+        dev._check(lib.mlel_hip_capture_end(dev.ctx, stream, C.byref(exe)))
+        replayed = []
+        for x in inputs + inputs[:1]:
+            g.set_input("input", x)
+            dev._check(lib.mlel_hip_graph_launch(dev.ctx, exe, stream))
+            replayed.append(g.get_output("output"))
+        dev._check(lib.mlel_hip_graph_destroy(dev.ctx, exe))
+        g.close()
+    finally:
+        dev.stream = null_stream
+        dev._check(lib.mlel_hip_stream_destroy(dev.ctx, stream))
+    return eager + eager[:1], replayed
+
+
+def test_captured_graphs_replay_the_eager_bits(dev):
+    """A dispatch of the MobileNetV2-shaped int8 pipeline and of the fp16 encoder block captured into a HIP graph: every
+    replay (several, with other work between them) gives the bits of the eager dispatch on the same input."""
+    spec = graphs.mobilenetv2_spec(batch=4, image=96, spread=True, classes=100)
+    xs = [random_input(spec, 50 + i) for i in range(3)]
+    eager, replayed = capture_and_replay(dev, spec, xs)
+    for a, b in zip(eager, replayed):
+        np.testing.assert_array_equal(a, b)
+    assert not np.array_equal(eager[0], eager[1])
+    spec = graphs.transformer_block_spec(batch=2, seq=128, d_model=256, heads=4, ffn=512)
+    xs = [np.random.default_rng(60 + i).standard_normal(spec.inputs[0][2]).astype(np.float16) for i in range(3)]
+    eager, replayed = capture_and_replay(dev, spec, xs)
+    for a, b in zip(eager, replayed):
+        np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+
+
+def test_fused_entry_point_refuses_its_allocating_route_under_capture(dev):
+    """A fused call that no one-pass kernel takes would allocate and synchronise: on a capturing stream it returns
+    MLEL_ERR_UNSUPPORTED before launching anything, and the capture stays valid."""
+    import ctypes as C
+    from hip_util import Runner
+    run = Runner(dev)
+    lib = dev.lib
+    stream = dev.new_stream()
+    null_stream, dev.stream = dev.stream, stream
+    try:
+        x = run.put(np.zeros((1, 4, 4, 8), np.int8), strides=(4 * 4 * 16, 4 * 16, 16, 2))  # element stride 2
+        w, b = run.put(np.ones((4, 1, 1, 8), np.int8)), run.put(np.zeros(4, np.int32))
+        out = run.new(abi.I8, (1, 4, 4, 4))
+        epi = run._epi(np.full(4, 2 ** 30, np.int32), np.full(4, 30, np.int8), abi.rescale_attr(0, 0, True, True, True), None)
+        attr = abi.conv2d_attr((0, 0, 0, 0), (1, 1), (1, 1), 0, 0)
+        dev._check(lib.mlel_hip_capture_begin(dev.ctx, stream))
+        with pytest.raises(hb.MlelError) as e:
+            dev.op("conv2d_rescale_clamp", out.ref, x.ref, w.ref, b.ref, C.byref(attr), C.byref(epi))
+        exe = C.c_void_p()
+        dev._check(lib.mlel_hip_capture_end(dev.ctx, stream, C.byref(exe)))
+        dev._check(lib.mlel_hip_graph_destroy(dev.ctx, exe))
+        assert e.value.code == abi.ERR_UNSUPPORTED and "being captured" in str(e.value)
+        dev.op("conv2d_rescale_clamp", out.ref, x.ref, w.ref, b.ref, C.byref(attr), C.byref(epi))  # eager: allowed
+        assert out.download().shape == (1, 4, 4, 4)
+    finally:
+        dev.stream = null_stream
+        run.done()
+        dev._check(lib.mlel_hip_stream_destroy(dev.ctx, stream))
+
+
 @pytest.mark.parametrize("planner", ["linear", "bestfit"])
 def test_graphs_under_the_other_memory_planners(dev, oracle, planner, monkeypatch):
     """VMEL_MEMORY_PLANNER = Linear / BestFit (the interval planner is the default everywhere else): same results."""

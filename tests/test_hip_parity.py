@@ -800,6 +800,65 @@ def test_transpose_fast_paths_vs_numpy(run, oracle):
         np.testing.assert_array_equal(got, oracle.transpose(x, perms))
 
 
+# ------------------------------------------------------------------------------------------------ split K
+SPLIT_CONV_CASES = [
+    # name, x shape, OC, kernel, pad, stride, zi, zw: few output tiles and a K of at least 32 steps of 64 bytes, so
+    # that K is split over blocks
+    ("tap_ic256_3x3", (1, 9, 9, 256), 64, (3, 3), (1, 1, 1, 1), (1, 1), -5, 0),         # one tap per K step
+    ("tap_ic320_3x3_s2_zw", (2, 11, 9, 320), 40, (3, 3), (1, 0, 1, 0), (2, 2), 7, -3),
+    ("generic_ic232_3x3", (1, 8, 8, 232), 24, (3, 3), (1, 1, 1, 1), (1, 1), 9, 1),       # byte gathers
+    ("plain_2560_160", (2, 7, 7, 2560), 160, (1, 1), (0, 0, 0, 0), (1, 1), -1, 0),       # 16-byte rows
+    ("plain4_ic2200", (1, 6, 6, 2200), 36, (1, 1), (0, 0, 0, 0), (1, 1), 3, 2),          # dword rows, K tail
+    ("plain_k_tail_2096", (1, 5, 5, 2096), 130, (1, 1), (0, 0, 0, 0), (1, 1), 0, 0),     # last split shorter
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_CONV_CASES, ids=[c[0] for c in SPLIT_CONV_CASES])
+def test_conv2d_i8_split_k_vs_oracle(run, oracle, case):
+    """Contractions with few tiles and a very long K split K over several blocks that exchange int32 partial tiles
+    through the context's workspace: int32 result and fused epilogue, bit for bit, and
+    again on a second launch (the arrival counters are back at zero)."""
+    name, xs, oc, k, pad, stride, zi, zw = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    x = ri(rng, -128, 127, xs, np.int8)
+    w = ri(rng, -128, 127, (oc,) + k + (xs[3],), np.int8)
+    b = ri(rng, -2 ** 15, 2 ** 15, (oc,), np.int32)
+    oh, ow = out_hw(xs[1], xs[2], k, pad, stride, (1, 1))
+    attr = abi.conv2d_attr(pad, stride, (1, 1), zi, zw)
+    shape = (xs[0], oh, ow, oc)
+    exp = oracle.conv2d(x, w, b, shape, abi.I32, attr)
+    mult, shift = rescale_params(rng, oc)
+    rattr = abi.rescale_attr(0, -2, True, True, True)
+    exp8 = oracle.clamp(oracle.rescale(exp, mult, shift, abi.I8, rattr), -100, 110)
+    for _ in range(2):
+        np.testing.assert_array_equal(run.conv2d(x, w, b, shape, abi.I32, attr), exp)
+        np.testing.assert_array_equal(run.conv2d(x, w, b, shape, abi.I8, attr, epilogue=(mult, shift, rattr, (-100, 110))),
+                                      exp8)
+
+
+SPLIT_MM_CASES = [
+    ("kmajor_zp", 1, 64, 4096, 256, 2, -1),
+    ("kmajor4_n100", 2, 40, 2112, 100, -4, 6),
+    ("generic_n29_k2100", 1, 37, 2100, 29, 5, -5),
+    ("fc_like_long_k", 1, 32, 5120, 1000, 3, 0),
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_MM_CASES, ids=[c[0] for c in SPLIT_MM_CASES])
+def test_matmul_i8_split_k_vs_oracle(run, oracle, case):
+    name, nb, m, k, n, za, zb = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    a = ri(rng, -128, 127, (nb, m, k), np.int8)
+    b = ri(rng, -128, 127, (nb, k, n), np.int8)
+    exp = oracle.matmul(a, b, abi.I32, za, zb)
+    mult, shift = np.array([1518500250], np.int32), np.array([39], np.int8)
+    rattr = abi.rescale_attr(0, 1, True, True, False)
+    exp8 = oracle.rescale(exp, mult, shift, abi.I8, rattr)
+    for _ in range(2):
+        np.testing.assert_array_equal(run.matmul(a, b, abi.I32, za, zb), exp)
+        np.testing.assert_array_equal(run.matmul(a, b, abi.I8, za, zb, epilogue=(mult, shift, rattr, None)), exp8)
+
+
 # ------------------------------------------------------------------------------------------------ error paths
 def test_error_conventions(run):
     x = np.zeros((1, 4, 4, 4), np.int8)
@@ -812,6 +871,33 @@ def test_error_conventions(run):
     with pytest.raises(hb.MlelError):
         run.rescale(np.zeros(4, np.int32), np.zeros(1, np.int16), np.zeros(1, np.int8), abi.I8,
                     abi.rescale_attr(scale32=True))
+    run.done()
+
+
+def test_fused_fp16_entry_points_reject_null_data_before_any_launch(run):
+    """A tensor with extents but no data pointer is MLEL_ERR_INVALID in the fused fp16 products, as in every other
+    entry point: the check runs on the host, nothing is launched."""
+    import ctypes as C
+
+    dev = run.dev
+    a = run.put(np.zeros((1, 64, 64), np.float16))
+    b = run.put(np.zeros((1, 64, 64), np.float16))
+    out = run.new(abi.F16, (1, 64, 64))
+    res = run.put(np.zeros((1, 64, 64), np.float16))
+    null16 = abi.make_tensor(None, abi.F16, (1, 64, 64))
+    attr = abi.MatmulAttr(0, 0)
+    for args in ((out.ref, C.byref(null16), b.ref, None, C.byref(attr), res.ref),
+                 (out.ref, a.ref, C.byref(null16), None, C.byref(attr), res.ref)):
+        with pytest.raises(hb.MlelError) as e:
+            dev.op("matmul_bias_cast_add", *args)
+        assert e.value.code == abi.ERR_INVALID and "null data pointer" in str(e.value)
+    prod = (abi.MatmulProduct * 2)()
+    for i in range(2):
+        prod[i].out, prod[i].b, prod[i].bias = C.pointer(out.view), C.pointer(b.view), None
+    prod[1].b = C.pointer(null16)
+    with pytest.raises(hb.MlelError) as e:
+        dev.op("matmul_bias_cast_group", prod, 2, a.ref, C.byref(attr))
+    assert e.value.code == abi.ERR_INVALID and "null data pointer" in str(e.value)
     run.done()
 
 
