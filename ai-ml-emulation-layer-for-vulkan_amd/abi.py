@@ -247,6 +247,7 @@ OP_SIGNATURES = {
 
 FUSED_SIGNATURES = {
     "conv2d_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
+    "conv2d_rescale_clamp_static": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
     "conv2d_rescale_add_rescale": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue), C.POINTER(Epilogue), _T,
                                    C.POINTER(Epilogue), C.POINTER(Epilogue), C.c_int],
     "matmul_rescale": [_T, _T, _T, C.POINTER(MatmulAttr), C.POINTER(Epilogue)],

@@ -527,6 +527,43 @@ int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor
     return 0;
 }
 
+int mlel_hip_conv2d_rescale_clamp_static(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                         const mlel_tensor *weights, const mlel_tensor *bias,
+                                         const mlel_conv2d_attr *attr, const mlel_epilogue *epi) {
+    MLEL_TRY(require_ctx(ctx, "conv2d_rescale_clamp_static"));
+    MLEL_REQUIRE(out != nullptr && attr != nullptr, MLEL_ERR_INVALID, "conv2d_rescale_clamp_static: null argument");
+    MLEL_REQUIRE(ctx->static_scratch != nullptr, MLEL_ERR_DEVICE,
+                 "conv2d_rescale_clamp_static: the static scratch has no address on device %d", ctx->device);
+    MLEL_TRY(check_tensor(out, "conv2d_rescale_clamp_static out"));
+    mlel_tensor acc_view = packed_like(out, MLEL_I32, out->ptr);  // shape carrier for validation
+    MLEL_TRY(check_conv("conv2d_rescale_clamp_static", &acc_view, in, weights, bias, attr));
+    FusedEpilogue fe;
+    MLEL_TRY(make_epilogue(epi, MLEL_I32, out, out->dims[3], &fe));
+    // the fused kernels; a split-K launch keeps its partial tiles and counters in the static array
+    bool used_split = false;
+    const GemmScratch gs{ctx->static_scratch,
+                         reinterpret_cast<uint32_t *>(ctx->static_scratch + kStaticScratchPartialBytes),
+                         kStaticScratchPartialBytes, &used_split};
+    int rc = try_conv2d_i8_direct(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe);
+    if (rc == 0) rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe, nullptr, &gs);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    // no fused kernel for this layout: the operator sequence, its int32 accumulator staged in the static array
+    const size_t need = (size_t)numel(out) * 4;
+    MLEL_REQUIRE(need <= kStaticScratchPartialBytes, MLEL_ERR_LIMIT,
+                 "conv2d_rescale_clamp_static: no one-pass kernel takes these operands and the int32 accumulator of "
+                 "the operator sequence (%zu bytes) exceeds the static scratch (%zu bytes); use "
+                 "mlel_hip_conv2d_rescale_clamp, which allocates",
+                 need, kStaticScratchPartialBytes);
+    mlel_tensor acc = packed_like(out, MLEL_I32, ctx->static_scratch);
+    const GemmScratch no_split{nullptr, nullptr, 0, nullptr};  // the array is taken: the contraction must not split K
+    rc = try_conv2d_i8_direct(ctx, (hipStream_t)stream, &acc, in, weights, bias, attr, nullptr);
+    if (rc == 0) rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, &acc, in, weights, bias, attr, nullptr, nullptr, &no_split);
+    if (rc < 0) return rc;
+    if (rc == 0) MLEL_TRY(conv2d_generic_launch((hipStream_t)stream, &acc, in, weights, bias, attr));
+    MLEL_TRY(run_unfused_tail(ctx, (hipStream_t)stream, out, &acc, epi));
+    return 0;
+}
+
 int mlel_hip_conv2d_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
                                         const mlel_tensor *weights, const mlel_tensor *bias,
                                         const mlel_conv2d_attr *attr, const mlel_epilogue *epi,

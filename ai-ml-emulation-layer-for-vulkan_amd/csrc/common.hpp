@@ -428,6 +428,9 @@ struct mlel_ctx {
     SplitWorkspace ws[kMaxSplitWorkspaces];
     int n_ws = 0;
     int split_k = 8;  // most blocks per tile in split-K mode; 0 or 1: never split (MLEL_SPLIT_K in the environment)
+    // the statically allocated scratch of the entry point that must not allocate: this device's address of the
+    // array (hipGetSymbolAddress at context creation), nullptr if that failed
+    char *static_scratch = nullptr;
 };
 
 namespace mlel {
@@ -435,5 +438,10 @@ namespace mlel {
 // captured, table full, allocation failed): the caller then runs without splitting.
 bool split_workspace(mlel_ctx *ctx, hipStream_t stream, SplitWorkspace *out);
 void free_split_workspaces(mlel_ctx *ctx);
+// static_scratch.hip: the file-scope device array behind mlel_hip_conv2d_rescale_clamp_static
+constexpr size_t kStaticScratchPartialBytes = size_t(8) << 20;
+constexpr size_t kStaticScratchBytes = kStaticScratchPartialBytes + size_t(kSplitCounters) * 4;
+int static_scratch_init(mlel_ctx *ctx);
+int static_scratch_clear_counters(mlel_ctx *ctx, hipStream_t s);
 bool stream_is_capturing(hipStream_t s);
 }  // namespace mlel

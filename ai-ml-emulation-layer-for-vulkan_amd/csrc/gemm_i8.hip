@@ -116,6 +116,9 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g, const SplitScratch &s
                 g.split_steps = per;
                 g.partials = reinterpret_cast<int32_t *>(sc.partials);
                 g.counters = sc.counters;
+                // the context's workspaces start at zero and every launch leaves its counters at zero; the shared
+                // static region is cleared by a small kernel instead of trusting what the last call left there
+                if (!sc.from_ctx) MLEL_TRY(static_scratch_clear_counters(ctx, s));
             }
         }
     }

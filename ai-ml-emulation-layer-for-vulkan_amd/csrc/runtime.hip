@@ -196,6 +196,8 @@ int mlel_hip_init(int device, mlel_ctx **out_ctx) {
         return set_error(MLEL_ERR_DEVICE, "init: hipGetDeviceProperties: %s", hipGetErrorString(pe));
     }
     if (const char *env = std::getenv("MLEL_SPLIT_K")) ctx->split_k = std::atoi(env);  // 0: off, n: at most n splits
+    // this device's address of the static scratch array; a failure only disables the entry point that needs it
+    (void)static_scratch_init(ctx);
     *out_ctx = ctx;
     return 0;
 }

@@ -391,6 +391,17 @@ int mlel_hip_select(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const m
 int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
                                   const mlel_tensor *weights, const mlel_tensor *bias,
                                   const mlel_conv2d_attr *attr, const mlel_epilogue *epi);
+/* mlel_hip_conv2d_rescale_clamp for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and the
+ * same bits in `out`; it calls no hipMalloc / hipFree or allocating library routine.  Whatever scratch its kernels
+ * need -- the partial tiles and arrival counters of a split-K contraction, or the int32 accumulator when no one-pass
+ * kernel takes the operands and the operator sequence runs instead -- lives in one statically allocated device array
+ * of 8 MiB + 16 KiB that each GPU the library runs on holds until the process ends.  A call whose accumulator would
+ * not fit (more than 2 097 152 output elements on the operator-sequence route) returns MLEL_ERR_LIMIT.  All calls on
+ * one GPU share the array: calls that overlap on one GPU (two streams, two threads) race; order them. */
+int mlel_hip_conv2d_rescale_clamp_static(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                         const mlel_tensor *weights, const mlel_tensor *bias,
+                                         const mlel_conv2d_attr *attr, const mlel_epilogue *epi);
 /* out = RESCALE_out( RESCALE_conv( CONV2D -> RESCALE -> [CLAMP] (epi) ) + RESCALE_residual(residual) ): the
  * residual connection behind a projecting convolution, bit for bit mlel_hip_conv2d_rescale_clamp into an 8-bit
  * temporary of `out`'s type followed by mlel_hip_rescale_add_rescale.  The integer addition wraps, so the operand order
