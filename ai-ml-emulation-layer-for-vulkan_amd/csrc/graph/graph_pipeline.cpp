@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <cstring>
+#include <map>
 #include <unordered_map>
 
 #include "session_planner.hpp"
@@ -1077,6 +1078,7 @@ void GraphPipeline::fuse() {
         std::vector<TensorPtr> regionInputs;
         std::vector<mlel_chain_step> steps;   // operands: value >= 0 input index, value < 0 -(step index + 1)
         std::vector<OpNode *> absorbed;
+        std::map<const TensorDescriptor *, int> emitted;  // an absorbed intermediate read twice (MUL(t, t)) is one step
         bool ok = true;
         std::function<int(const TensorPtr &)> valueOf;
         const auto emit = [&](OpNode &op, mlel_chain_step st) {
@@ -1089,10 +1091,14 @@ void GraphPipeline::fuse() {
         valueOf = [&](const TensorPtr &t) -> int {
             OpNode *p = t->getProducer();
             mlel_chain_step st{};
+            const auto seen = emitted.find(t.get());
+            if (seen != emitted.end()) return seen->second;
             if (p && p != &root && isPrivateIntermediate(*t) && sameShape(*t, shape) && chainStepOf(*p, &st) &&
                 consumersOf(ops, t.get()).size() == 1 && steps.size() + absorbed.size() < MLEL_CHAIN_MAX_STEPS - 1) {
                 absorbed.push_back(p);
-                return emit(*p, st);
+                const int value = emit(*p, st);
+                emitted[t.get()] = value;
+                return value;
             }
             for (size_t i = 0; i < regionInputs.size(); i++)
                 if (regionInputs[i].get() == t.get()) return static_cast<int>(i);
@@ -1392,6 +1398,10 @@ mlel_epilogue makeEpilogue(const RescaleSpec &spec, const mlel_tensor *mult, con
 
 void GraphPipeline::run(const OpNode &op, void *stream) {
     std::array<mlel_tensor, 8> in{};
+    // FusedElementwise describes its inputs itself (up to MLEL_CHAIN_MAX_INPUTS); every other kind reads `in`
+    if (op.inputs.size() > in.size() && op.kind != OpKind::FusedElementwise)
+        fail(op.tosaName + " (" + op.debugName + "): " + std::to_string(op.inputs.size()) +
+             " inputs, more than an operator call carries");
     for (size_t i = 0; i < op.inputs.size() && i < in.size(); i++) {
         in[i] = op.inputs[i]->view();
         if (in[i].ptr == nullptr && op.inputs[i]->getShapeSize() != 0)

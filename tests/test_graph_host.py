@@ -378,3 +378,20 @@ def test_projection_patterns_leave_observable_or_mismatched_cases_alone():
     g = _build_host_only(spec, fuse=True)
     assert g.op_names() == ["MATMUL+ADD+CAST", "TRANSPOSE"]
     g.close()
+
+
+def test_elementwise_region_emits_an_absorbed_square_once():
+    """An intermediate that one operator reads twice -- MUL(t, t) over t = EXP(x) -- is absorbed into the region as ONE
+    step: EXP, MUL, ADD make a region of three steps, not four with EXP emitted twice."""
+    spec = graphs.Spec()
+    shape = (1, 16, 64)
+    spec.inputs.append(("input", abi.F16, shape))
+    t = spec.tensor("t", abi.F16, shape)
+    spec.op("EXP", ["input"], [t])
+    sq = spec.tensor("t", abi.F16, shape)
+    spec.op("MUL", [t, t], [sq], [0])
+    spec.op("ADD", [sq, "input"], ["output"])
+    spec.outputs.append(("output", abi.F16, shape))
+    g = _build_host_only(spec, fuse=True)
+    assert g.op_names() == ["ELEMENTWISE x3"]
+    g.close()
