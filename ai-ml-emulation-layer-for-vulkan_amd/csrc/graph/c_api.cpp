@@ -39,6 +39,7 @@
 #include <cstring>
 #include <limits>
 #include <map>
+#include <memory>
 #include <sstream>
 #include <string>
 
@@ -58,12 +59,23 @@ struct ProfileSample {
 
 struct mlel_graph {
     GraphPipeline pipeline;
+    std::unique_ptr<GraphSession> defaultSession;  // behind mlel_graph_bind_* / mlel_graph_dispatch
     mlel_ctx *ctx;
     std::vector<void *> events;  // pairs of profiling events, created on demand
     bool profiling = false;      // mlel_graph_dispatch records a sample per operator (VMEL_GRAPH_PROFILING)
     uint64_t dispatches = 0;
     std::vector<ProfileSample> samples;
     explicit mlel_graph(mlel_ctx *c) : pipeline(c), ctx(c) {}
+    GraphSession &session() {
+        if (!defaultSession) defaultSession = std::make_unique<GraphSession>(pipeline);
+        return *defaultSession;
+    }
+};
+
+struct mlel_graph_session {
+    mlel_graph *graph;
+    GraphSession session;
+    explicit mlel_graph_session(mlel_graph *g) : graph(g), session(g->pipeline) {}
 };
 
 namespace {
@@ -486,14 +498,14 @@ int mlel_graph_session_memory_requirements(mlel_graph *g, uint64_t *size, uint64
 
 int mlel_graph_bind_session_memory(mlel_graph *g, void *device_base) {
     return guarded([&] {
-        g->pipeline.bindSessionMemory(device_base);
+        g->session().bindTransientMemory(device_base);
         return 0;
     });
 }
 
 int mlel_graph_bind_external(mlel_graph *g, uint32_t set, uint32_t binding, uint32_t array_index, void *device_ptr) {
     return guarded([&] {
-        g->pipeline.bindExternal(set, binding, array_index, device_ptr);
+        g->session().bindExternal(set, binding, array_index, device_ptr);
         return 0;
     });
 }
@@ -501,14 +513,14 @@ int mlel_graph_bind_external(mlel_graph *g, uint32_t set, uint32_t binding, uint
 namespace {
 
 // a pair of events around every operator; milliseconds per operator into `ms` (n entries)
-void dispatchTimed(mlel_graph *g, void *stream, std::vector<float> &ms) {
+void dispatchTimed(mlel_graph *g, GraphSession &session, void *stream, std::vector<float> &ms) {
     const size_t n = g->pipeline.executionList().size();
     while (g->events.size() < 2 * n) {
         void *e = nullptr;
         if (mlel_hip_event_create(g->ctx, &e) != 0) throw std::runtime_error(mlel_hip_last_error());
         g->events.push_back(e);
     }
-    g->pipeline.dispatch(stream, [&](const OpNode &, uint32_t index, bool before) {
+    session.dispatch(stream, [&](const OpNode &, uint32_t index, bool before) {
         if (mlel_hip_event_record(g->ctx, g->events[2 * index + (before ? 0 : 1)], stream) != 0)
             throw std::runtime_error(mlel_hip_last_error());
     });
@@ -520,19 +532,103 @@ void dispatchTimed(mlel_graph *g, void *stream, std::vector<float> &ms) {
 
 }  // namespace
 
+namespace {
+
+int dispatchSession(mlel_graph *g, GraphSession &session, void *stream) {
+    if (!g->profiling) {
+        session.dispatch(stream);
+        return 0;
+    }
+    // profiling: this dispatch waits for its own events (the reference reads its timestamps back at the fence)
+    std::vector<float> ms;
+    dispatchTimed(g, session, stream, ms);
+    const auto list = g->pipeline.executionList();
+    for (size_t i = 0; i < list.size(); i++)
+        g->samples.push_back(ProfileSample{g->dispatches, static_cast<uint32_t>(i), opLabel(*list[i]), ms[i]});
+    g->dispatches++;
+    return 0;
+}
+
+}  // namespace
+
 int mlel_graph_dispatch(mlel_graph *g, void *stream) {
+    return guarded([&] { return dispatchSession(g, g->session(), stream); });
+}
+
+// ---- sessions (reference: graph_layer.cpp:1297-1425) ----
+int mlel_graph_session_create(mlel_graph *g, mlel_graph_session **out) {
     return guarded([&] {
-        if (!g->profiling) {
-            g->pipeline.dispatch(stream);
+        if (g == nullptr || out == nullptr) throw std::runtime_error("session_create: null argument");
+        *out = new mlel_graph_session(g);
+        return 0;
+    });
+}
+
+void mlel_graph_session_destroy(mlel_graph_session *s) { delete s; }
+
+int mlel_graph_session_bind_point_requirements(mlel_graph_session *s, uint32_t *count,
+                                               mlel_graph_bind_point_requirement *requirements) {
+    return guarded([&] {
+        if (s == nullptr || count == nullptr) throw std::runtime_error("bind_point_requirements: null argument");
+        const uint32_t required = s->session.needsTransientMemory() ? 1u : 0u;
+        if (requirements == nullptr) {
+            *count = required;
             return 0;
         }
-        // profiling: this dispatch waits for its own events (the reference reads its timestamps back at the fence)
-        std::vector<float> ms;
-        dispatchTimed(g, stream, ms);
-        const auto list = g->pipeline.executionList();
-        for (size_t i = 0; i < list.size(); i++)
-            g->samples.push_back(ProfileSample{g->dispatches, static_cast<uint32_t>(i), opLabel(*list[i]), ms[i]});
-        g->dispatches++;
+        const uint32_t capacity = *count;
+        uint32_t written = 0;
+        if (required) {
+            if (written < capacity)
+                requirements[written] = mlel_graph_bind_point_requirement{MLEL_GRAPH_BIND_POINT_TRANSIENT,
+                                                                          MLEL_GRAPH_BIND_POINT_TYPE_MEMORY, 1};
+            ++written;
+        }
+        *count = written;
+        return capacity < required ? MLEL_GRAPH_INCOMPLETE : 0;
+    });
+}
+
+int mlel_graph_session_get_memory_requirements(mlel_graph_session *s, uint32_t bind_point, uint64_t *size,
+                                               uint64_t *alignment) {
+    return guarded([&] {
+        if (s == nullptr) throw std::runtime_error("session memory requirements: null session");
+        (void)bind_point;  // a graph pipeline answers with its planner's requirements whatever the bind point
+        if (size) *size = s->session.memorySize();
+        if (alignment) *alignment = s->session.memoryAlignment();
+        return 0;
+    });
+}
+
+int mlel_graph_session_bind_memory(mlel_graph_session *s, uint32_t bind_point, void *device_base) {
+    return guarded([&] {
+        if (s == nullptr) throw std::runtime_error("session bind memory: null session");
+        if (bind_point != MLEL_GRAPH_BIND_POINT_TRANSIENT)
+            throw std::runtime_error("Invalid bind point for pipeline type");
+        s->session.bindTransientMemory(device_base);
+        return 0;
+    });
+}
+
+int mlel_graph_session_bind_external(mlel_graph_session *s, uint32_t set, uint32_t binding, uint32_t array_index,
+                                     void *device_ptr) {
+    return guarded([&] {
+        if (s == nullptr) throw std::runtime_error("session bind external: null session");
+        s->session.bindExternal(set, binding, array_index, device_ptr);
+        return 0;
+    });
+}
+
+int mlel_graph_session_dispatch(mlel_graph_session *s, void *stream) {
+    return guarded([&] {
+        if (s == nullptr) throw std::runtime_error("session dispatch: null session");
+        return dispatchSession(s->graph, s->session, stream);
+    });
+}
+
+int mlel_graph_session_dispatch_range(mlel_graph_session *s, void *stream, int first, int count) {
+    return guarded([&] {
+        if (s == nullptr || first < 0 || count < 0) throw std::runtime_error("session dispatch range: bad argument");
+        s->session.dispatch(stream, {}, static_cast<uint32_t>(first), static_cast<uint32_t>(count));
         return 0;
     });
 }
@@ -540,7 +636,7 @@ int mlel_graph_dispatch(mlel_graph *g, void *stream) {
 int mlel_graph_dispatch_profiled(mlel_graph *g, void *stream, float *ms, int capacity) {
     return guarded([&] {
         std::vector<float> all;
-        dispatchTimed(g, stream, all);
+        dispatchTimed(g, g->session(), stream, all);
         for (size_t i = 0; i < all.size() && static_cast<int>(i) < capacity; i++) ms[i] = all[i];
         return static_cast<int>(all.size());
     });

@@ -1374,11 +1374,62 @@ void GraphPipeline::bindSessionMemory(void *deviceBase) {
     if (reinterpret_cast<uintptr_t>(deviceBase) % kSessionAlignment != 0)
         fail("bindSessionMemory: session memory must be aligned to " + std::to_string(kSessionAlignment) + " bytes");
     for (const auto &[t, off] : offsets) const_cast<TensorDescriptor *>(t)->bind(static_cast<char *>(deviceBase) + off);
+    appliedSession = nullptr;  // (a session that calls this records itself afterwards)
 }
 
 void GraphPipeline::bindExternal(const uint32_t set, const uint32_t binding, const uint32_t arrayIndex,
                                  void *devicePtr) {
     getTensor(set, binding, arrayIndex)->bind(devicePtr);
+    appliedSession = nullptr;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// GraphSession
+// ---------------------------------------------------------------------------------------------------------------
+GraphSession::GraphSession(GraphPipeline &p) : pipeline(p) {
+    if (!pipeline.isFinalized()) fail("session: the pipeline's finalize() has not run");
+}
+
+GraphSession::~GraphSession() {
+    if (pipeline.appliedSession == this) pipeline.appliedSession = nullptr;
+}
+
+void GraphSession::bindTransientMemory(void *deviceBase) {
+    if (needsTransientMemory() && deviceBase == nullptr) fail("bindTransientMemory: null session memory");
+    if (reinterpret_cast<uintptr_t>(deviceBase) % GraphPipeline::kSessionAlignment != 0)
+        fail("bindTransientMemory: session memory must be aligned to " +
+             std::to_string(GraphPipeline::kSessionAlignment) + " bytes");
+    base = deviceBase;
+    transientMemoryBound = true;
+    version++;
+}
+
+void GraphSession::bindExternal(const uint32_t set, const uint32_t binding, const uint32_t arrayIndex, void *devicePtr) {
+    externals[pipeline.getTensor(set, binding, arrayIndex).get()] = devicePtr;
+    version++;
+}
+
+void GraphSession::apply() {
+    if (pipeline.appliedSession == this && pipeline.appliedVersion == version) return;
+    if (needsTransientMemory()) pipeline.bindSessionMemory(base);
+    // an external tensor this session has not bound must not keep another session's pointer
+    for (const auto &[set, bindings] : pipeline.tensorMap)
+        for (const auto &[binding, array] : bindings)
+            for (const auto &t : array)
+                if (t) t->bind(nullptr);
+    for (const auto &[t, ptr] : externals) t->bind(ptr);
+    pipeline.appliedSession = this;
+    pipeline.appliedVersion = version;
+}
+
+void GraphSession::dispatch(void *stream, const GraphPipeline::DispatchDecorator &decorator, const uint32_t first,
+                            const uint32_t count) {
+    if (pipeline.ctx == nullptr)
+        fail("dispatch: this GraphPipeline was built without a device context; there is no CPU path");
+    // reference: "session transient memory is not bound" (graph_layer.cpp:1944-1947)
+    if (needsTransientMemory() && !transientMemoryBound) fail("dispatch: session transient memory is not bound");
+    apply();
+    pipeline.dispatch(stream, decorator, first, count);
 }
 
 namespace {
@@ -1578,15 +1629,18 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
     if (rc != 0) fail(op.tosaName + " (" + op.debugName + "): " + mlel_hip_last_error());
 }
 
-void GraphPipeline::dispatch(void *stream, const DispatchDecorator &decorator) {
+void GraphPipeline::dispatch(void *stream, const DispatchDecorator &decorator, const uint32_t first,
+                             const uint32_t count) {
     if (!finalized) fail("dispatch: finalize() has not run");
     if (ctx == nullptr) fail("dispatch: this GraphPipeline was built without a device context; there is no CPU path");
     uint32_t index = 0;
     for (const auto &op : ops) {
         if (op->fusedAway) continue;
-        if (decorator) decorator(*op, index, true);
-        run(*op, stream);
-        if (decorator) decorator(*op, index, false);
+        if (index >= first && index - first < count) {
+            if (decorator) decorator(*op, index, true);
+            run(*op, stream);
+            if (decorator) decorator(*op, index, false);
+        }
         index++;
     }
 }

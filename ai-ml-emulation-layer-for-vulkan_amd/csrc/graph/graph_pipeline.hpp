@@ -324,7 +324,9 @@ class GraphPipeline {
     // Reference: cmdBindAndDispatch (compute_graph_op.cpp:2500-2509).  The decorator, when set, brackets every
     // executed operator (the reference's ComputePipelineDispatchDecorator, used by its profiler).
     using DispatchDecorator = std::function<void(const OpNode &, uint32_t index, bool before)>;
-    void dispatch(void *stream, const DispatchDecorator &decorator = {});
+    // `first` / `count` select a run of the executed operators (positions in executionList()); profiling tools time
+    // single operators with it.
+    void dispatch(void *stream, const DispatchDecorator &decorator = {}, uint32_t first = 0, uint32_t count = UINT32_MAX);
 
     // introspection used by tests and the profiler
     std::vector<const OpNode *> executionList() const;
@@ -369,8 +371,44 @@ class GraphPipeline {
     bool finalized = false;
 
     friend class CApi;
+    friend class GraphSession;
+    const class GraphSession *appliedSession = nullptr;  // whose bindings the tensor descriptors hold right now
+    uint64_t appliedVersion = 0;
   public:
     const std::vector<TensorPtr> &handles() const { return allTensors; }
+};
+
+// One session of a pipeline: its own transient (session) memory and its own external tensor bindings, so that several
+// sessions of one pipeline can be in flight at the same time, each on its own stream.  Reference counterpart:
+// DataGraphPipelineSessionARM (graph/graph_layer.cpp:215-330; entry points :1297-1425).  A session is used from the
+// thread that uses its pipeline (neither is locked, as in the reference); pointers are resolved on the host when a
+// dispatch is issued, so dispatches of different sessions issued one after the other overlap on the GPU.
+class GraphSession {
+  public:
+    explicit GraphSession(GraphPipeline &pipeline);  // the pipeline must be finalized and outlive the session
+    ~GraphSession();
+    GraphSession(const GraphSession &) = delete;
+    GraphSession &operator=(const GraphSession &) = delete;
+
+    // reference: needsTransientRequirements (graph_layer.cpp:239-241): a graph without intermediates needs none
+    bool needsTransientMemory() const { return pipeline.sessionMemorySize() != 0; }
+    size_t memorySize() const { return pipeline.sessionMemorySize(); }
+    size_t memoryAlignment() const { return pipeline.sessionMemoryAlignment(); }
+    // reference: bindTransientMemory (graph_layer.cpp:260-271)
+    void bindTransientMemory(void *deviceBase);
+    // external tensors of this session; may be re-bound between dispatches (update-after-bind)
+    void bindExternal(uint32_t set, uint32_t binding, uint32_t arrayIndex, void *devicePtr);
+    // reference: vkCmdDispatchDataGraphARM with this session (graph_layer.cpp:1844-1980)
+    void dispatch(void *stream, const GraphPipeline::DispatchDecorator &decorator = {}, uint32_t first = 0,
+                  uint32_t count = UINT32_MAX);
+
+  private:
+    void apply();
+    GraphPipeline &pipeline;
+    void *base = nullptr;
+    bool transientMemoryBound = false;
+    std::map<TensorDescriptor *, void *> externals;
+    uint64_t version = 1;  // bumped by every bind: the pipeline re-applies the bindings only when they changed
 };
 
 }  // namespace mlel::graph

@@ -31,6 +31,14 @@ class SpvConstant(C.Structure):
     _fields_ = [("id", C.c_uint32), ("rank", C.c_int32), ("dims", C.POINTER(C.c_int64)), ("data", C.c_void_p)]
 
 
+class BindPointRequirement(C.Structure):
+    _fields_ = [("bind_point", C.c_uint32), ("bind_point_type", C.c_uint32), ("num_objects", C.c_uint32)]
+
+
+INCOMPLETE = 5            # MLEL_GRAPH_INCOMPLETE
+BIND_POINT_TRANSIENT = 0  # MLEL_GRAPH_BIND_POINT_TRANSIENT
+
+
 def load_graph_library():
     global _glib
     if _glib is None:
@@ -69,6 +77,17 @@ def load_graph_library():
         lib.mlel_graph_bind_session_memory.argtypes = [_V, _V]
         lib.mlel_graph_bind_external.argtypes = [_V, C.c_uint32, C.c_uint32, C.c_uint32, _V]
         lib.mlel_graph_dispatch.argtypes = [_V, _V]
+        lib.mlel_graph_session_create.argtypes = [_V, C.POINTER(_V)]
+        lib.mlel_graph_session_destroy.argtypes = [_V]
+        lib.mlel_graph_session_destroy.restype = None
+        lib.mlel_graph_session_bind_point_requirements.argtypes = [_V, C.POINTER(C.c_uint32),
+                                                                  C.POINTER(BindPointRequirement)]
+        lib.mlel_graph_session_get_memory_requirements.argtypes = [_V, C.c_uint32, C.POINTER(C.c_uint64),
+                                                                  C.POINTER(C.c_uint64)]
+        lib.mlel_graph_session_bind_memory.argtypes = [_V, C.c_uint32, _V]
+        lib.mlel_graph_session_bind_external.argtypes = [_V, C.c_uint32, C.c_uint32, C.c_uint32, _V]
+        lib.mlel_graph_session_dispatch.argtypes = [_V, _V]
+        lib.mlel_graph_session_dispatch_range.argtypes = [_V, _V, C.c_int, C.c_int]
         lib.mlel_graph_dispatch_profiled.argtypes = [_V, _V, C.POINTER(C.c_float), C.c_int]
         lib.mlel_graph_set_profiling.argtypes = [_V, C.c_int]
         lib.mlel_graph_get_profiling.argtypes = [_V]
@@ -272,6 +291,11 @@ class Graph:
     def dispatch(self):
         self._check(self.lib.mlel_graph_dispatch(self.g, self.dev.stream))
 
+    def new_session(self, allocate=True):
+        """A further session of this (finalized) pipeline; with `allocate` it gets session memory and external tensors
+        of its own, as the reference's test client gives every dispatch (utilities/pipeline.cpp:297-330)."""
+        return Session(self, allocate)
+
     def dispatch_profiled(self):
         n = self.op_count()
         ms = (C.c_float * max(1, n))()
@@ -314,3 +338,73 @@ class Graph:
             out.append({"handle": h.value, "offset": None if off.value == 2 ** 64 - 1 else off.value,
                         "size": size.value, "first": first.value, "last": last.value})
         return out
+
+
+class Session:
+    """One mlel_graph_session: its own transient memory and external tensors."""
+
+    def __init__(self, graph, allocate=True):
+        self.graph, self.dev, self.lib = graph, graph.dev, graph.lib
+        s = _V()
+        graph._check(self.lib.mlel_graph_session_create(graph.g, C.byref(s)))
+        self.s = s
+        self.session_mem = None
+        self.ext_tensors = {}
+        if allocate:
+            count = C.c_uint32()
+            graph._check(self.lib.mlel_graph_session_bind_point_requirements(self.s, C.byref(count), None))
+            if count.value:
+                size, align = self.memory_requirements()
+                self.session_mem = self.dev.alloc(max(size, 256))
+                self.bind_memory(self.session_mem)
+            for name, (st, b, a, dtype, shape, strides) in graph.externals.items():
+                self.bind(name, self.dev.tensor(dtype, shape, strides))
+
+    def bind_point_requirements(self, capacity=None):
+        """(status, count, entries): capacity None is the counting call of the two-call pattern"""
+        count = C.c_uint32(0 if capacity is None else capacity)
+        arr = None if capacity is None else (BindPointRequirement * max(1, capacity))()
+        rc = self.graph._check(self.lib.mlel_graph_session_bind_point_requirements(self.s, C.byref(count), arr))
+        entries = [] if arr is None else [(arr[i].bind_point, arr[i].bind_point_type, arr[i].num_objects)
+                                          for i in range(min(capacity, count.value))]
+        return rc, count.value, entries
+
+    def memory_requirements(self, bind_point=BIND_POINT_TRANSIENT):
+        size, align = C.c_uint64(), C.c_uint64()
+        self.graph._check(self.lib.mlel_graph_session_get_memory_requirements(self.s, bind_point, C.byref(size),
+                                                                              C.byref(align)))
+        return int(size.value), int(align.value)
+
+    def bind_memory(self, device_base, bind_point=BIND_POINT_TRANSIENT):
+        self.graph._check(self.lib.mlel_graph_session_bind_memory(self.s, bind_point, C.c_void_p(device_base)))
+
+    def bind(self, name, tensor):
+        """binds (or re-binds) the external tensor `name` to a DeviceTensor"""
+        st, b, a = self.graph.externals[name][:3]
+        self.ext_tensors[name] = tensor
+        self.graph._check(self.lib.mlel_graph_session_bind_external(self.s, st, b, a, C.c_void_p(tensor.ptr)))
+
+    def set_input(self, name, array):
+        self.ext_tensors[name].upload(array)
+
+    def get_output(self, name):
+        return self.ext_tensors[name].download()
+
+    def dispatch(self, stream=None):
+        self.graph._check(self.lib.mlel_graph_session_dispatch(self.s, self.dev.stream if stream is None else stream))
+
+    def dispatch_range(self, first, count, stream=None):
+        self.graph._check(self.lib.mlel_graph_session_dispatch_range(
+            self.s, self.dev.stream if stream is None else stream, int(first), int(count)))
+
+    def close(self, free_tensors=True):
+        if self.s:
+            self.lib.mlel_graph_session_destroy(self.s)
+            self.s = None
+        if self.session_mem:
+            self.dev.free(self.session_mem)
+            self.session_mem = None
+        if free_tensors:
+            for t in self.ext_tensors.values():
+                t.free()
+        self.ext_tensors = {}

@@ -24,6 +24,9 @@ class Spec:
         self.outputs = []   # (name, dtype, shape)
         self.ops = []       # dicts: op, in, out, iattr, fattr, name
         self.macs = {"dense": 0, "depthwise": 0}
+        # one entry per launch of the fused int8 graph, in execution order: kind ("conv" | "dw" | "avgpool" | "fc"),
+        # shapes, MACs and the algorithmic bytes of the fused unit (every operand once + the output once)
+        self.layers = []
         self._n = 0
 
     def fresh(self, prefix):
@@ -96,6 +99,9 @@ def _conv_block(spec, q, rng, x, x_zp, cin, cout, k, stride, depthwise, relu6, o
         contraction = k * k * cin
         spec.macs["dense"] += n * oh * ow * cout * k * k * cin
     bias = spec.const("b", rng.integers(-2 ** 15, 2 ** 15, (cout,), endpoint=True).astype(np.int32))
+    spec.layers.append({"kind": "dw" if depthwise else "conv", "in": (n, h, w, cin), "out": (n, oh, ow, cout),
+                        "kernel": k, "stride": stride, "macs": n * oh * ow * cout * contraction,
+                        "bytes": n * h * w * cin + spec.consts[wt].size + 9 * cout + n * oh * ow * cout})
     acc = spec.tensor("acc", abi.I32, (n, oh, ow, cout))
     spec.op("DEPTHWISE_CONV2D" if depthwise else "CONV2D", [x, wt, bias], [acc],
             list(pad) + [stride, stride, 1, 1, x_zp, 0, abi.ACC_I32])
@@ -124,6 +130,9 @@ def _residual(spec, q, rng, x, x_zp, y, y_zp):
     """RESCALE(x -> i32) + RESCALE(y -> i32) -> ADD -> RESCALE(-> i8): the reference's residual-add pattern
     (tests/shader/graph-constant-arm.spvasm)."""
     shape = spec.shape_of(x)
+    if spec.layers:  # the addition runs in the epilogue of the projection before it, which also reads x
+        spec.layers[-1]["bytes"] += int(np.prod(shape))
+        spec.layers[-1]["residual"] = True
     one = lambda v, dt: np.array([v], dt)
     ma = spec.const("m", one(rng.integers(2 ** 30, 2 ** 31 - 1), np.int32))
     mb = spec.const("m", one(rng.integers(2 ** 30, 2 ** 31 - 1), np.int32))
@@ -181,12 +190,16 @@ def mobilenetv2_spec(batch=32, image=224, seed=1003, spread=False, classes=1000)
     n, h, w, c = spec.shape_of(x)
     pooled = spec.tensor("pool", abi.I8, (n, 1, 1, c))
     spec.op("AVG_POOL2D", [x], [pooled], [h, w, 1, 1, 0, 0, 0, 0, abi.ACC_I32, zp, zp])
+    spec.layers.append({"kind": "avgpool", "in": (n, h, w, c), "out": (n, 1, 1, c), "kernel": h, "stride": 1,
+                        "macs": 0, "bytes": n * h * w * c + n * c})
     flat = spec.tensor("flat", abi.I8, (1, n, c))
     spec.op("RESHAPE", [pooled], [flat])
     fc_w = spec.const("fc_w", rng.integers(-127, 127, (1, c, classes), endpoint=True).astype(np.int8))
     logits = spec.tensor("fc_acc", abi.I32, (1, n, classes))
     spec.op("MATMUL", [flat, fc_w], [logits], [zp, 0])
     spec.macs["dense"] += n * c * classes
+    spec.layers.append({"kind": "fc", "in": (1, n, c), "out": (1, n, classes), "kernel": 1, "stride": 1,
+                        "macs": n * c * classes, "bytes": n * c + c * classes + 5 + n * classes})
     mult, shift = q.scale(1, c)
     m, s = spec.const("m", mult), spec.const("s", shift)
     spec.op("RESCALE", [logits, m, s], ["output"], [0, 0, 1, 1, 0, 0, 0])
@@ -317,13 +330,7 @@ def build(dev, spec, fuse=True):
     return g
 
 
-def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32):
-    """Times whole-graph dispatches of BASELINE config 3 (inputs resident in HBM) and returns the extra fields
-    bench.py adds to its JSON line."""
-    spec = mobilenetv2_spec(batch=batch)
-    g = build(dev, spec, fuse=True)
-    rng = np.random.default_rng(1003)
-    g.set_input("input", rng.integers(-128, 127, spec.inputs[0][2], endpoint=True).astype(np.int8))
+def _time_graph(dev, g, steps, warmup):
     for _ in range(warmup):
         g.dispatch()
     dev.sync()
@@ -335,50 +342,119 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32):
     dev.record(ev1)
     dev.sync()
     wall = (time.perf_counter() - t0) / steps
-    gpu_ms = dev.elapsed_ms(ev0, ev1) / steps
+    return wall, dev.elapsed_ms(ev0, ev1) / steps
+
+
+def time_operators(dev, g, reps=50, only=None):
+    """Milliseconds per launch of every executed operator of `g` on its own: the operator is launched `reps` times
+    back to back on the stream (its inputs are whatever the last whole dispatch left in session memory) between two
+    events.  `only`: a list of operator positions."""
+    s = g.new_session(allocate=False)
+    s.bind_memory(g.session_mem)
+    for name, t in g.ext_tensors.items():
+        s.bind(name, t)
+    out = {}
+    ev0, ev1 = dev.event(), dev.event()
+    for i in (range(g.op_count()) if only is None else only):
+        for _ in range(3):
+            s.dispatch_range(i, 1)
+        dev.record(ev0)
+        for _ in range(reps):
+            s.dispatch_range(i, 1)
+        dev.record(ev1)
+        dev.sync()
+        out[i] = dev.elapsed_ms(ev0, ev1) / reps
+    s.close(free_tensors=False)
+    return out
+
+
+def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True):
+    """Times whole-graph dispatches of BASELINE config 3 (inputs resident in HBM) and every launch on its own; returns
+    the extra fields bench.py adds to its JSON line, with the MFMA position of the dense (CONV2D / MATMUL) launches
+    and the HBM position of the bandwidth-bound (DEPTHWISE_CONV2D, AVG_POOL2D) ones."""
+    spec = mobilenetv2_spec(batch=batch)
+    g = build(dev, spec, fuse=True)
+    rng = np.random.default_rng(1003)
+    g.set_input("input", rng.integers(-128, 127, spec.inputs[0][2], endpoint=True).astype(np.int8))
+    wall, gpu_ms = _time_graph(dev, g, steps, warmup)
     per_op = g.dispatch_profiled()
     dev.sync()
     by_kind = {}
     for name, ms in per_op:
         by_kind[name] = by_kind.get(name, 0.0) + ms
     macs = spec.macs["dense"] + spec.macs["depthwise"]
-    res = {"mobilenetv2_b32": {
-        "img_per_s": batch / wall, "ms_per_graph": wall * 1e3, "gpu_ms_per_graph": gpu_ms,
-        "tops": 2.0 * macs / wall / 1e12, "gmac": macs / 1e9, "operators_executed": g.op_count(),
-        "operators_in_graph": len(spec.ops), "session_memory_bytes": g.session_size,
-        "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}}
+    res = {"img_per_s": batch / wall, "ms_per_graph": wall * 1e3, "gpu_ms_per_graph": gpu_ms,
+           "graphs_timed": steps, "tops": 2.0 * macs / wall / 1e12, "gmac": macs / 1e9,
+           "operators_executed": g.op_count(), "operators_in_graph": len(spec.ops),
+           "session_memory_bytes": g.session_size,
+           "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}
+    if per_layer and g.op_count() == len(spec.layers):
+        alone = time_operators(dev, g)
+        layers = []
+        for i, layer in enumerate(spec.layers):
+            ms = alone[i]
+            layers.append({"index": i, "kind": layer["kind"], "in": list(layer["in"]), "out": list(layer["out"]),
+                           "kernel": layer["kernel"], "stride": layer["stride"], "us": round(ms * 1e3, 2),
+                           "tops": round(2.0 * layer["macs"] / (ms * 1e-3) / 1e12, 2),
+                           "gbs": round(layer["bytes"] / (ms * 1e-3) / 1e9, 1)})
+        dense = [(l, spec.layers[l["index"]]) for l in layers if l["kind"] in ("conv", "fc")]
+        band = [(l, spec.layers[l["index"]]) for l in layers if l["kind"] in ("dw", "avgpool")]
+
+        def total(group, key):
+            return float(sum(meta[key] for _, meta in group))
+
+        d_ms = sum(l["us"] for l, _ in dense) * 1e-3
+        b_ms = sum(l["us"] for l, _ in band) * 1e-3
+        top_d = max(dense, key=lambda p: p[0]["us"])
+        top_b = max(band, key=lambda p: p[0]["us"])
+        res["layers"] = layers
+        res["roofline_dense"] = {
+            "bound": "mfma", "unit": "TFLOP/s", "peak": 5000.0, "launches": len(dense),
+            "achieved": 2.0 * total(dense, "macs") / (d_ms * 1e-3) / 1e12,
+            "frac": 2.0 * total(dense, "macs") / (d_ms * 1e-3) / 1e12 / 5000.0,
+            "algorithmic_bytes": total(dense, "bytes"), "us_sum_of_launches": d_ms * 1e3,
+            "hbm_frac_of_the_same_launches": total(dense, "bytes") / (d_ms * 1e-3) / 1e9 / 8000.0,
+            "dominant_launch": dict(top_d[0], frac=top_d[0]["tops"] / 5000.0,
+                                    hbm_frac=top_d[0]["gbs"] / 8000.0)}
+        res["roofline_bandwidth"] = {
+            "bound": "hbm", "unit": "GB/s", "peak": 8000.0, "launches": len(band),
+            "achieved": total(band, "bytes") / (b_ms * 1e-3) / 1e9,
+            "frac": total(band, "bytes") / (b_ms * 1e-3) / 1e9 / 8000.0,
+            "algorithmic_bytes": total(band, "bytes"), "us_sum_of_launches": b_ms * 1e3,
+            "dominant_launch": dict(top_b[0], frac=top_b[0]["gbs"] / 8000.0)}
     g.close()
-    return res
+    return {"mobilenetv2_b32": res}
 
 
-def bench_transformer(dev, steps=5, warmup=2):
-    """Times whole-graph dispatches of BASELINE config 4 (fp16 encoder block, batch 8, seq 512, d_model 768) and
-    returns the extra fields bench.py adds to its JSON line."""
+def bench_transformer(dev, steps=20, warmup=3):
+    """Times whole-graph dispatches of BASELINE config 4 (fp16 encoder block, batch 8, seq 512, d_model 768) and every
+    launch on its own; returns the extra fields bench.py adds to its JSON line, with the fp16 MFMA position of the
+    launches that hold a MATMUL."""
     spec = transformer_block_spec()
     g = build(dev, spec, fuse=True)
     rng = np.random.default_rng(1004)
     g.set_input("input", rng.standard_normal(spec.inputs[0][2]).astype(np.float16))
-    for _ in range(warmup):
-        g.dispatch()
-    dev.sync()
-    ev0, ev1 = dev.event(), dev.event()
-    t0 = time.perf_counter()
-    dev.record(ev0)
-    for _ in range(steps):
-        g.dispatch()
-    dev.record(ev1)
-    dev.sync()
-    wall = (time.perf_counter() - t0) / steps
-    gpu_ms = dev.elapsed_ms(ev0, ev1) / steps
+    wall, gpu_ms = _time_graph(dev, g, steps, warmup)
     per_op = g.dispatch_profiled()
     dev.sync()
     by_kind = {}
     for name, ms in per_op:
         by_kind[name] = by_kind.get(name, 0.0) + ms
+    alone = time_operators(dev, g)
+    names = g.op_names()
+    gemm_ms = sum(ms for i, ms in alone.items() if "MATMUL" in names[i])
+    other_ms = sum(ms for i, ms in alone.items() if "MATMUL" not in names[i])
     res = {"transformer_b8_s512_d768": {
-        "ms_per_graph": wall * 1e3, "gpu_ms_per_graph": gpu_ms, "tflops": spec.flops / wall / 1e12,
+        "ms_per_graph": wall * 1e3, "gpu_ms_per_graph": gpu_ms, "graphs_timed": steps,
+        "tflops": spec.flops / wall / 1e12,
         "gflop": spec.flops / 1e9, "operators_executed": g.op_count(), "operators_in_graph": len(spec.ops),
         "session_memory_bytes": g.session_size,
-        "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}}
+        "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())},
+        "us_by_launch_alone": [{"index": i, "name": names[i], "us": round(ms * 1e3, 2)} for i, ms in alone.items()],
+        "roofline_gemm": {"bound": "mfma", "unit": "TFLOP/s", "peak": 2500.0,
+                          "launches": sum(1 for n in names if "MATMUL" in n),
+                          "achieved": spec.flops / (gemm_ms * 1e-3) / 1e12,
+                          "frac": spec.flops / (gemm_ms * 1e-3) / 1e12 / 2500.0,
+                          "us_sum_of_launches": gemm_ms * 1e3, "us_other_launches": other_ms * 1e3}}}
     g.close()
     return res

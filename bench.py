@@ -7,8 +7,13 @@ multiplier 1518500250 / shift 39, double round), one launch of the MFMA contract
 also reports the MobileNetV2-shaped int8 graph at batch 32 (BASELINE config 3) executed through the host-side
 GraphPipeline, the roofline position of the dominant kernel and a CPU baseline (the oracle on the host cores).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|config1|mobilenetv2|encoder|layer] [--layer N]
+
+`--only` restricts the run to one leg (profiling runs: one kernel family per trace); `--only layer --layer N` launches
+the N-th operator of the fused MobileNetV2 graph 200 times back to back and nothing else, so that counters of a single
+layer can be collected.  The whole-graph legs always time at least 20 graphs.
 """
+import re
 import argparse
 import ctypes as C
 import importlib
@@ -27,10 +32,24 @@ PKG = "ai-ml-emulation-layer-for-vulkan_amd"
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X published dense int8 peak, TOP/s
 HBM_PEAK_GBS = 8000.0         # MI355X published HBM3E bandwidth, GB/s
 
-# HBM bytes per launch of the config 1 kernel from two rocprofv3 --pmc runs of this script (profiles/):
-# FETCH_SIZE 6248 KiB scaled by 2.0 plus WRITE_SIZE 4096 KiB scaled by 1.0, the factors being what the same
-# counters read for the 256 MiB copy kernel below (131083 KiB and 262144 KiB).
-CONFIG1_TRAFFIC_BYTES = int((6248 * 2.0 + 4096 * 1.0) * 1024)
+CONFIG1_KERNEL = "gemm_i8_kernel<128,128,2,2,X_PLAIN_DL,W_KMAJOR_DL,SUMS,Q8>"
+CONFIG1_PROFILE = os.path.join(ROOT, "profiles", "gemm_i8_kernel_config1_matmul_rescale.md")
+
+
+def config1_traffic_bytes():
+    """HBM bytes per launch of the config 1 kernel as the committed counter summary states them (two rocprofv3 --pmc
+    runs, FETCH_SIZE and WRITE_SIZE, each scaled by what it reads for the 256 MiB copy kernel): the line
+    `traffic_bytes_per_launch = N` of the profile of this kernel, or None when the summary is missing or is of another
+    kernel."""
+    try:
+        text = open(CONFIG1_PROFILE).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic_bytes_per_launch\s*=\s*(\d+)", text)
+    k = re.search(r"traffic_kernel\s*=\s*(\S+)", text)
+    if not m or not k or k.group(1).strip("`") != CONFIG1_KERNEL:
+        return None
+    return int(m.group(1))
 
 
 def log(*a):
@@ -128,13 +147,53 @@ def cpu_baseline_config1(abi, inputs, gpu_out):
                       f"{spent:.1f} s of CPU work, OpenMP"}, ok
 
 
+def cpu_baseline_mobilenetv2(abi, budget_s=10.0):
+    """The oracle executing the unfused MobileNetV2-shaped graph (183 operators) on the host cores, batch 4 per pass
+    (one eighth of config 3's batch; every operator is independent across the batch), repeated for about ten seconds."""
+    oracle = importlib.import_module("oracle.mlel_oracle")
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from oracle_graph import run_spec
+    graphs = importlib.import_module(PKG + ".graphs")
+    batch = 4
+    spec = graphs.mobilenetv2_spec(batch=batch)
+    x = np.random.default_rng(1003).integers(-128, 127, spec.inputs[0][2], endpoint=True).astype(np.int8)
+    reps, spent = 0, 0.0
+    while spent < budget_s and reps < 64:
+        t0 = time.perf_counter()
+        run_spec(oracle, spec, {"input": x})
+        spent += time.perf_counter() - t0
+        reps += 1
+    return {"value": batch * reps / spent, "unit": "img/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"{reps} x the unfused graph at batch {batch} (of config 3's 32), {spent:.1f} s of CPU work, OpenMP"}
+
+
+def run_layer(dev, abi, index, reps=200):
+    """One operator of the fused config 3 graph, launched `reps` times back to back (for counter collection)."""
+    graphs = importlib.import_module(PKG + ".graphs")
+    spec = graphs.mobilenetv2_spec(batch=32)
+    g = graphs.build(dev, spec, fuse=True)
+    g.set_input("input", np.random.default_rng(1003).integers(-128, 127, spec.inputs[0][2], endpoint=True).astype(np.int8))
+    g.dispatch()
+    dev.sync()
+    ms = graphs.time_operators(dev, g, reps=reps, only=[index])[index]
+    layer = spec.layers[index]
+    res = {"layer": index, "name": g.op_name(index), "kind": layer["kind"], "in": list(layer["in"]),
+           "out": list(layer["out"]), "us": ms * 1e3, "launches": reps + 3 + 1,
+           "tops": 2.0 * layer["macs"] / (ms * 1e-3) / 1e12, "algorithmic_bytes": layer["bytes"],
+           "gbs": layer["bytes"] / (ms * 1e-3) / 1e9}
+    g.close()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg (profiling runs)")
-    ap.add_argument("--skip-graph", action="store_true", help="omit the MobileNetV2 graph leg")
+    ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline legs (profiling runs)")
+    ap.add_argument("--skip-graph", action="store_true", help="omit the MobileNetV2 and encoder graph legs")
+    ap.add_argument("--only", choices=["all", "config1", "mobilenetv2", "encoder", "layer"], default="all")
+    ap.add_argument("--layer", type=int, default=3, help="with --only layer: position in the fused config 3 graph")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -145,32 +204,54 @@ def main():
     info = dev.info()
     log("device:", info)
 
+    if args.only == "layer":
+        print(json.dumps(run_layer(dev, abi, args.layer)), flush=True)
+        dev.close()
+        return
+
+    want = lambda leg: args.only in ("all", leg)
+    graph_steps = max(20, args.steps // 10)
+
     # one plain 256 MiB device-to-device copy: the kernel of known traffic that calibrates the FETCH_SIZE / WRITE_SIZE
     # counters in profiling runs, and a measured HBM ceiling
     copy_gbs = measure_copy(dev, 256 << 20)
     log(f"copy kernel: {copy_gbs:.0f} GB/s (read + write)")
 
-    c1, inputs = bench_config1(dev, abi, args.steps, args.warmup)
-    log("config 1:", c1)
+    c1, inputs = (None, None)
+    if want("config1"):
+        c1, inputs = bench_config1(dev, abi, args.steps, args.warmup)
+        log("config 1:", c1)
 
     extra = {}
-    if not args.skip_graph:
+    graphs = importlib.import_module(PKG + ".graphs")
+    if want("mobilenetv2") and not args.skip_graph:
         try:
-            graphs = importlib.import_module(PKG + ".graphs")
-            extra = graphs.bench_mobilenetv2(dev, steps=max(5, args.steps // 10), warmup=max(2, args.warmup // 10))
-            log("config 3:", extra)
-            c4 = graphs.bench_transformer(dev)
-            log("config 4:", c4)
-            extra.update(c4)
+            extra.update(graphs.bench_mobilenetv2(dev, steps=graph_steps, warmup=max(3, args.warmup // 10)))
+            log("config 3:", {k: v for k, v in extra["mobilenetv2_b32"].items() if k != "layers"})
         except Exception as e:  # the line below still reports config 1; the failure is visible
             log("config 3 leg failed:", repr(e))
-            extra = {"mobilenetv2_b32": {"error": repr(e)}}
+            extra["mobilenetv2_b32"] = {"error": repr(e)}
+    if want("encoder") and not args.skip_graph:
+        try:
+            extra.update(graphs.bench_transformer(dev, steps=graph_steps, warmup=max(3, args.warmup // 10)))
+            log("config 4:", extra["transformer_b8_s512_d768"])
+        except Exception as e:
+            log("config 4 leg failed:", repr(e))
+            extra["transformer_b8_s512_d768"] = {"error": repr(e)}
 
     cpu = None
     parity_ok = None
-    if not args.skip_cpu:
+    if not args.skip_cpu and c1 is not None:
         cpu, parity_ok = cpu_baseline_config1(abi, inputs, inputs[4])
         log("cpu baseline:", cpu, "gpu==oracle:", parity_ok)
+    if not args.skip_cpu and "mobilenetv2_b32" in extra and "error" not in extra["mobilenetv2_b32"]:
+        extra["mobilenetv2_b32"]["cpu_baseline"] = cpu_baseline_mobilenetv2(abi)
+        log("cpu baseline (config 3):", extra["mobilenetv2_b32"]["cpu_baseline"])
+
+    if c1 is None:  # a single graph leg: its own record, no config 1 fields to report
+        print(json.dumps(dict({"only": args.only, "copy_kernel_gbs": copy_gbs}, **extra)), flush=True)
+        dev.close()
+        return
 
     line = {
         "metric": "int8 TOPS (config 1: MATMUL 8x512x1024x1024 + RESCALE, fused) + MobileNetV2-shape b32 img/s",
@@ -190,8 +271,8 @@ def main():
                    "device": info["name"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "mfma", "achieved": c1["kernel_tops"], "peak": INT8_MFMA_PEAK_TOPS / 1.0,
                      "unit": "TFLOP/s", "ops_are": "int8 multiply and add counted as 2 ops", "frac": c1["kernel_tops"] / INT8_MFMA_PEAK_TOPS,
-                     "traffic": CONFIG1_TRAFFIC_BYTES,
-                     "kernel": "gemm_i8_kernel<128,128,2,2,X_PLAIN_DL,W_KMAJOR_DL,SUMS,Q8>", "kernel_ms": c1["kernel_ms"],
+                     "traffic": config1_traffic_bytes(),
+                     "kernel": CONFIG1_KERNEL, "kernel_ms": c1["kernel_ms"],
                      "algorithmic_bytes": c1["algorithmic_bytes"],
                      "hbm_frac_if_bandwidth_bound": c1["algorithmic_bytes"] / (c1["kernel_ms"] * 1e-3) / 1e9 /
                      HBM_PEAK_GBS},

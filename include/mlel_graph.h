@@ -102,6 +102,40 @@ int mlel_graph_bind_session_memory(mlel_graph *g, void *device_base);
 int mlel_graph_bind_external(mlel_graph *g, uint32_t set, uint32_t binding, uint32_t array_index, void *device_ptr);
 /* Reference: vkCmdDispatchDataGraphARM -> cmdBindAndDispatch (graph_layer.cpp:1844-1980). */
 int mlel_graph_dispatch(mlel_graph *g, void *stream);
+
+/* ---- sessions: one pipeline, several sets of bound memory in flight at once ----
+ * Reference: vkCreateDataGraphPipelineSessionARM (graph/graph_layer.cpp:1297-1330),
+ * vkGetDataGraphPipelineSessionBindPointRequirementsARM (:1332-1380), vkGetDataGraphPipelineSessionMemoryRequirementsARM
+ * (:1382-1389), vkBindDataGraphPipelineSessionMemoryARM (:1391-1420), vkCmdDispatchDataGraphARM (:1844-1980).
+ * A session holds its own transient (session) memory and its own external tensor bindings; the functions above that
+ * take the graph itself (mlel_graph_bind_session_memory, mlel_graph_bind_external, mlel_graph_dispatch) work on a
+ * session the graph creates for itself.  External tensors may be re-bound between dispatches (update-after-bind);
+ * the pointers are resolved when a dispatch is issued, so dispatches of two sessions issued one after the other on
+ * two streams overlap on the GPU.  A session is used from the thread that uses its graph (neither is locked, as in
+ * the reference) and destroyed before its graph. */
+typedef struct mlel_graph_session mlel_graph_session;
+#define MLEL_GRAPH_INCOMPLETE 5 /* positive, like VK_INCOMPLETE: the array was too short, *count entries exist */
+enum { MLEL_GRAPH_BIND_POINT_TRANSIENT = 0 };   /* VK_DATA_GRAPH_PIPELINE_SESSION_BIND_POINT_TRANSIENT_ARM */
+enum { MLEL_GRAPH_BIND_POINT_TYPE_MEMORY = 0 }; /* VK_DATA_GRAPH_PIPELINE_SESSION_BIND_POINT_TYPE_MEMORY_ARM */
+typedef struct mlel_graph_bind_point_requirement {
+    uint32_t bind_point, bind_point_type, num_objects;
+} mlel_graph_bind_point_requirement;
+int mlel_graph_session_create(mlel_graph *g, mlel_graph_session **out); /* after mlel_graph_finalize */
+void mlel_graph_session_destroy(mlel_graph_session *s);
+/* Two-call pattern: requirements == NULL writes the number of bind points to *count (0 for a graph without
+ * intermediate tensors, else 1); otherwise at most *count entries are written, *count becomes the number that exist
+ * and the result is MLEL_GRAPH_INCOMPLETE when the array was shorter than that. */
+int mlel_graph_session_bind_point_requirements(mlel_graph_session *s, uint32_t *count,
+                                               mlel_graph_bind_point_requirement *requirements);
+int mlel_graph_session_get_memory_requirements(mlel_graph_session *s, uint32_t bind_point, uint64_t *size,
+                                               uint64_t *alignment);
+int mlel_graph_session_bind_memory(mlel_graph_session *s, uint32_t bind_point, void *device_base);
+int mlel_graph_session_bind_external(mlel_graph_session *s, uint32_t set, uint32_t binding, uint32_t array_index,
+                                     void *device_ptr);
+int mlel_graph_session_dispatch(mlel_graph_session *s, void *stream);
+/* The operators `first` .. `first + count - 1` of the executed list only (profiling single layers). */
+int mlel_graph_session_dispatch_range(mlel_graph_session *s, void *stream, int first, int count);
+
 /* Dispatch with a pair of events around every operator; per-operator milliseconds are written to `ms`
  * (reference: the profiler's timestamp pairs, graph/graph_profiler.cpp:157-191).  Returns the operator count. */
 int mlel_graph_dispatch_profiled(mlel_graph *g, void *stream, float *ms, int capacity);

@@ -18,6 +18,18 @@ def test_library_exports_every_declared_symbol(abi):
         assert hasattr(lib, name), name
 
 
+def test_graph_library_exports_every_declared_symbol(abi):
+    if not os.path.exists(abi.GRAPH_LIB_PATH):
+        pytest.skip("libmlel_graph.so not built (run __graft_entry__.build())")
+    C.CDLL(abi.HIP_LIB_PATH, mode=C.RTLD_GLOBAL)
+    lib = C.CDLL(abi.GRAPH_LIB_PATH)
+    header = open(os.path.join(abi.REPO_ROOT, "include", "mlel_graph.h")).read()
+    declared = set(re.findall(r"\b(mlel_graph_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 35
+    for name in sorted(declared):
+        assert hasattr(lib, name), name
+
+
 def test_no_gpu_fails_loudly(abi):
     """Without a device every entry point that needs one reports MLEL_ERR_DEVICE; there is no CPU fallback."""
     if not os.path.exists(abi.HIP_LIB_PATH):
