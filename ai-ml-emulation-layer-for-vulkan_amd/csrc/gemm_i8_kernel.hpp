@@ -256,6 +256,8 @@ enum WMode {
 //   row operand:  piece p (0..3) of row r sits in slot p ^ ((r >> 2) & 3) of the row;
 //   K-major:      the 32-byte unit u of K row k sits in unit u ^ ((k / (256 / BN)) % (BN / 32)).
 // STAGES K steps are resident; one barrier per step.
+// Four stages; eight (tried on the 128 x 128 tile, 128 KiB) changed nothing: the fetch path, not the number of
+// requests in flight, bounds the loop.
 template <int BM, int BN>
 constexpr int dl_stages() {
     return 4;
@@ -302,7 +304,6 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     constexpr int DL_STAGE = (BM + BN) * BK;  // one stage: X tile [BM][64] then W tile
     char *xs = smem;                     // [2][BM][PITCH]
     char *ws = smem + 2 * BM * PITCH;    // [2][WBUF]
-    ChanParams *cp = reinterpret_cast<ChanParams *>(smem + (DL ? DL_S * DL_STAGE : 2 * BM * PITCH + 2 * WBUF));  // [BN]
 
     // ---- XCD-aware tile assignment: consecutive block ids land on different XCDs (8 of them, each with its own
     // L2), so block b is given tile (b % 8) * chunk + b / 8: tiles that share operands stay on one XCD.
@@ -346,19 +347,23 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     const int8_t *xb = g.x + (int64_t)batch * g.x_batch;
     const int8_t *wb = g.w + (int64_t)batch * g.w_batch;
 
-    // ---- per-channel epilogue constants: thread n < BN owns channel n.  The loads are issued here, ahead of the
-    // operand prefetch, but only consumed after the main loop, so their latency is never waited for.
-    static_assert(BN <= NTHREADS, "one thread per channel of the tile");
-    int32_t chan_bias = 0, chan_mult = 0, chan_shift = 0;
-    const bool chan_live = tid < BN && n_base + tid < g.N;
-    if (chan_live) {
-        const int gn = n_base + tid;
-        chan_bias = (g.bias && split == 0) ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
-        if (g.fused) {
-            const int ci = g.rp.per_channel ? gn : 0;
-            chan_mult = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
-                                 : reinterpret_cast<const int32_t *>(g.mult)[ci];
-            chan_shift = (int32_t)g.shift[ci];
+    // ---- per-channel epilogue constants.  The accumulators of a wavefront end up with one output channel per lane
+    // (lane % 32 of each 32-channel group j), so every lane loads the bias, multiplier and shift of its own TN
+    // channels.  The loads are issued here, ahead of the operand prefetch, but only consumed after the main loop, so
+    // their latency is never waited for.
+    int32_t chan_bias[TN], chan_mult[TN], chan_shift[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int gn = n_base + wave_n * WN + j * 32 + (lane & 31);
+        chan_bias[j] = chan_mult[j] = chan_shift[j] = 0;
+        if (gn < g.N) {
+            chan_bias[j] = (g.bias && split == 0) ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
+            if (g.fused) {
+                const int ci = g.rp.per_channel ? gn : 0;
+                chan_mult[j] = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
+                                        : reinterpret_cast<const int32_t *>(g.mult)[ci];
+                chan_shift[j] = (int32_t)g.shift[ci];
+            }
         }
     }
 
@@ -584,7 +589,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[i], wf[j], acc[i][j], 0, 0, 0);
             if (SUMS) {  // both sums are kept whenever a zero point is non-zero: 16 dot4 beside 8 MFMAs
 #pragma unroll
                 for (int i = 0; i < TM; i++)
@@ -606,7 +611,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         // taken by one wavefront only (combined through LDS after the loop).
         constexpr int XI = BM * 4 / NTHREADS, WI = BN * 4 / NTHREADS;  // 16-byte pieces per thread and stage
         static_assert((BN * 4) % NTHREADS == 0 && BN % 32 == 0 && BN <= 256, "whole W pieces per thread");
-        static_assert(DL_S == 4 && WAVES_M == 2 && WAVES_N >= 2, "ring of four stages, 2 x N wavefronts");
+        static_assert((DL_S == 4 || DL_S == 8) && WAVES_M == 2 && WAVES_N >= 2, "ring of four or eight stages, 2 x N wavefronts");
         constexpr int P16 = BN / 16, UN = BN / 32, RP = 256 / BN;  // K-major: pieces / units per row, rows per 256 B
         const int wave_u = __builtin_amdgcn_readfirstlane(wave);
         uint32_t xo[XI], wo[WI];
@@ -683,7 +688,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[i], wf[j], acc[i][j], 0, 0, 0);
             if (SUMS) {
                 if (sum_x) {  // wave-uniform
 #pragma unroll
@@ -699,11 +704,24 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                 }
             }
         };
-        // Stage s lives in buffer s % 4; three stages are requested ahead.  The loop is software-pipelined: while
+        // wait until at most `n` stages of this thread's requests are outstanding (n is wave-uniform)
+        auto wait_stages = [&](int n) {
+            switch (n) {
+            case 0: wait_vmcnt<0>(); break;
+            case 1: wait_vmcnt<1 * (XI + WI)>(); break;
+            case 2: wait_vmcnt<2 * (XI + WI)>(); break;
+            case 3: wait_vmcnt<3 * (XI + WI)>(); break;
+            case 4: wait_vmcnt<4 * (XI + WI)>(); break;
+            case 5: wait_vmcnt<5 * (XI + WI)>(); break;
+            default: wait_vmcnt<6 * (XI + WI)>(); break;
+            }
+        };
+        static_assert(6 * (XI + WI) < 64, "the outstanding-request counter has six bits");
+        // Stage s lives in buffer s % DL_S; DL_S - 1 stages are requested ahead.  The loop is software-pipelined: while
         // the first K half of step s is multiplied the second half is being read, and while the second half is
         // multiplied the first half of step s + 1 is being read.  In between sits the one barrier of the step:
-        // waiting until at most one stage of this thread's requests is outstanding means its part of stage s + 1 has
-        // landed (near the end of K nothing new is requested, so everything is waited for); the barrier extends
+        // waiting until at most DL_S - 3 stages of this thread's requests are outstanding means its part of stage
+        // s + 1 has landed (near the end of K fewer stages are outstanding and the count shrinks); the barrier extends
         // that to every thread's part and also says that every wavefront has received its reads of stage s - 1,
         // whose buffer the next request overwrites.
         const int nk = g.K / BK;
@@ -711,7 +729,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
 #pragma unroll
         for (int d = 0; d < DL_S - 1; d++)
             if (d < nk) issue(d, d);
-        if (nk > 2) wait_vmcnt<2 * (XI + WI)>(); else wait_vmcnt<0>();
+        wait_stages(min(nk, DL_S - 1) - 1);  // stage 0 has landed
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -725,7 +743,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                     multiply(xf0, wf0, xs0, ws0);
                     __builtin_amdgcn_sched_barrier(0);
                     const bool more = step + d + DL_S - 1 < nk;
-                    if (more) wait_vmcnt<XI + WI>(); else wait_vmcnt<0>();
+                    // requested so far: stages up to min(nk, step + d + DL_S - 1) - 1; stage step + d + 1 must have
+                    // landed, the later ones may still be in flight
+                    if (more) wait_vmcnt<(DL_S - 3) * (XI + WI)>(); else wait_stages(max(nk - 2 - (step + d), 0));
                     asm volatile("" ::: "memory");
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
@@ -738,11 +758,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             }
         }
         __syncthreads();
-        // ---- combine the split zero-point sums: afterwards every wavefront holds the full sums of its rows (X) and
-        // the wavefronts of row 0 those of their channels (W), as in the other fetch modes
+        // ---- combine the split zero-point sums: afterwards every wavefront holds, per lane half, partial sums whose
+        // total over the two halves is the full sum of its rows (X) and of its channels (W), as in the other fetch modes
         if (SUMS) {
-            int32_t *xs_l = reinterpret_cast<int32_t *>(smem);          // [2][BM]
-            int32_t *ws_l = reinterpret_cast<int32_t *>(smem) + 2 * BM;  // [BN]: partial of wavefront row 1
+            int32_t *xs_l = reinterpret_cast<int32_t *>(smem) + BM;      // [2][BM]: by K half
+            int32_t *ws_l = reinterpret_cast<int32_t *>(smem) + 3 * BM;  // [2][BN]: by K half
             if (need_xsum && wave_n < 2) {
 #pragma unroll
                 for (int i = 0; i < TM; i++) {
@@ -750,11 +770,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                     if (lane < 32) xs_l[wave_n * BM + wave_m * WM + i * 32 + lane] = part;
                 }
             }
-            if (need_wsum && wave_m == 1) {
+            if (need_wsum) {
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
                     const int32_t part = wsum[j] + __shfl_xor(wsum[j], 32);
-                    if (lane < 32) ws_l[wave_n * WN + j * 32 + lane] = part;
+                    if (lane < 32) ws_l[wave_m * BN + wave_n * WN + j * 32 + lane] = part;
                 }
             }
             __syncthreads();
@@ -762,13 +782,15 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
 #pragma unroll
                 for (int i = 0; i < TM; i++) {
                     const int r = wave_m * WM + i * 32 + (lane & 31);
-                    xsum[i] = lane < 32 ? xs_l[r] + xs_l[BM + r] : 0;  // the two lane halves are added up below
+                    xsum[i] = lane < 32 ? xs_l[r] + xs_l[BM + r] : 0;
                 }
             }
-            if (need_wsum && wave_m == 0) {
+            if (need_wsum) {
 #pragma unroll
-                for (int j = 0; j < TN; j++)
-                    if (lane < 32) wsum[j] += ws_l[wave_n * WN + j * 32 + lane];
+                for (int j = 0; j < TN; j++) {
+                    const int c = wave_n * WN + j * 32 + (lane & 31);
+                    wsum[j] = lane < 32 ? ws_l[c] + ws_l[BN + c] : 0;
+                }
             }
             __syncthreads();
         }
@@ -802,54 +824,61 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
 
     }
 
-    if (tid < BN) {
-        ChanParams c{};
-        if (chan_live) {
-            c.bias_adj = chan_bias;
-            if (g.fused) c.q = make_chan_scale(chan_mult, chan_shift, g.rp);
-        }
-        cp[tid] = c;
-    }
-    __syncthreads();
-    // ---- fold the zero-point terms that depend on the channel only into the per-channel bias
-    if (need_wsum && wave_m == 0) {
+    // ---- after the loop a lane holds, per 32 x 32 accumulator tile (i, j) and register 4q + e, the output of
+    // position 32 i + 8 q + 4 (lane / 32) + e and channel 32 j + lane % 32 of the wavefront's sub-tile: one channel per
+    // lane and tile column, so everything that depends on the channel only sits in a few registers.
+    const int half = lane >> 5, cl = lane & 31;
+    int32_t *xs_tab = reinterpret_cast<int32_t *>(smem);  // [BM]: zw * sum_k X[m][k]; the operand buffers are free now
+    int32_t bias_adj[TN];
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int32_t s = wsum[j] + __shfl_xor(wsum[j], 32);
-            if (lane < 32) {
-                const int n = wave_n * WN + j * 32 + lane;
-                cp[n].bias_adj = (int32_t)((uint32_t)cp[n].bias_adj - (uint32_t)g.zx * (uint32_t)s +
-                                           (uint32_t)k_len * (uint32_t)g.zx * (uint32_t)g.zw);
+    for (int j = 0; j < TN; j++) {
+        bias_adj[j] = chan_bias[j];
+        if (need_wsum) {  // -zx * sum_k W[n][k] + K zx zw: the zero-point terms that depend on the channel only
+            const int32_t sw = wsum[j] + __shfl_xor(wsum[j], 32);
+            bias_adj[j] = (int32_t)((uint32_t)bias_adj[j] - (uint32_t)g.zx * (uint32_t)sw +
+                                    (uint32_t)k_len * (uint32_t)g.zx * (uint32_t)g.zw);
+        }
+    }
+    if (need_xsum) {  // the row terms are needed by register index: through a table in shared memory
+        if (wave_n == 0) {
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                const int32_t sx = xsum[i] + __shfl_xor(xsum[i], 32);
+                if (lane < 32) xs_tab[wave_m * WM + i * 32 + lane] = (int32_t)((uint32_t)sx * (uint32_t)g.zw);
             }
         }
+        __syncthreads();
     }
-    if (need_xsum) {
-#pragma unroll
-        for (int i = 0; i < TM; i++)
-            xsum[i] = (int32_t)((uint32_t)(xsum[i] + __shfl_xor(xsum[i], 32)) * (uint32_t)g.zw);
-    }
-    __syncthreads();
+    // zw * sum_k X of the four positions of register group q of tile row i
+    auto row_terms = [&](int i, int q, int32_t (&xc)[4]) {
+        if (need_xsum) {
+            const int4 t = *reinterpret_cast<const int4 *>(xs_tab + wave_m * WM + i * 32 + 8 * q + 4 * half);
+            xc[0] = t.x, xc[1] = t.y, xc[2] = t.z, xc[3] = t.w;
+        } else {
+            xc[0] = xc[1] = xc[2] = xc[3] = 0;
+        }
+    };
+    bool rows_done = false;  // split K: the row and channel terms are already inside the accumulators
 
     if constexpr (XMODE != X_PLAIN_DL) {
         if (g.splits > 1) {
             // ---- split K: this block's partial tile, complete with the bias / zero-point terms of its K range
 #pragma unroll
-            for (int i = 0; i < TM; i++) {
-                const uint32_t xc = need_xsum ? (uint32_t)xsum[i] : 0u;
+            for (int i = 0; i < TM; i++)
 #pragma unroll
-                for (int j = 0; j < TN; j++)
+                for (int q = 0; q < 4; q++) {
+                    int32_t xc[4];
+                    row_terms(i, q, xc);
 #pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        const int nl = wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+                    for (int j = 0; j < TN; j++)
 #pragma unroll
                         for (int e = 0; e < 4; e++)
-                            acc[i][j][4 * q + e] =
-                                (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)cp[nl + e].bias_adj - xc);
-                    }
-                xsum[i] = 0;
-            }
-            __syncthreads();  // every wavefront has read the per-channel terms: the epilogue must not add them again
-            if (tid < BN) cp[tid].bias_adj = 0;
+                            acc[i][j][4 * q + e] = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] -
+                                                             (uint32_t)xc[e]);
+                }
+#pragma unroll
+            for (int j = 0; j < TN; j++) bias_adj[j] = 0;
+            rows_done = true;
             // The exchange uses device-scope atomic stores and loads (relaxed): they are coherent across the GPU's
             // eight L2 caches by themselves, so no fence is needed -- a device-scope fence would write back and
             // invalidate the whole L2 (measured: 20 - 50 us per launch).  Order: every thread waits until its own
@@ -865,7 +894,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                         __hip_atomic_store(&mine[((i * TN + j) * 16 + r) * NTHREADS], acc[i][j][r], __ATOMIC_RELAXED,
                                            __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            int *last_flag = reinterpret_cast<int *>(smem);  // the operand buffers are free after the main loop
+            int *last_flag = reinterpret_cast<int *>(smem) + BM;  // behind the row table
             __syncthreads();
             if (tid == 0) {
                 const uint32_t arrived =
@@ -890,16 +919,55 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                                                      (uint32_t)__hip_atomic_load(&theirs[((i * TN + j) * 16 + r) * NTHREADS],
                                                                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
             }
-            __syncthreads();  // cp[].bias_adj = 0 is in place for every wavefront
         }
     }
 
-    // ---- epilogue: lane holds output position m = lane % 32 of each tile row and, per register group q, the four
-    // channels n0 .. n0+3 with n0 = 8q + 4 * (lane / 32)
     char *ob = g.out + (int64_t)batch * g.out_batch;
     if (Q8) {
-        // Fused RESCALE(+CLAMP) to 8-bit outputs, N % 4 == 0, output extent below 2^31: straight-line code.  Rows and
-        // channels outside the problem get an offset beyond the buffer bounds, which drops the store.
+        // ---- fused RESCALE(+CLAMP) to 8-bit outputs, N % 4 == 0, output extent below 2^31.  The requantisation
+        // constants of a lane's channels are registers.  The four results of a register group are four consecutive
+        // positions of ONE channel; a 4 x 4 byte transpose inside each group of four lanes (two lane exchanges, two
+        // byte permutes) turns them into four consecutive channels of one position, which go to a staging tile in
+        // shared memory as a dword.  The tile then leaves in 16-byte pieces, so that every store instruction writes
+        // whole runs of a row (up to 128 bytes) instead of 8-byte fragments of 32 rows.
+        constexpr int OP = BN + 32;                        // pitch of the staging tile (bytes): rows 8 banks apart
+        char *so = smem + (3 * BM + 2 * BN) * 4;           // behind the tables of the zero-point sums
+        static_assert((3 * BM + 2 * BN) * 4 + BM * OP <= (int)(2 * BM * PITCH + 2 * w_buf_bytes<BN>()),
+                      "the staging tile fits the operand buffers");
+        ChanScale cs[TN];
+#pragma unroll
+        for (int j = 0; j < TN; j++) cs[j] = make_chan_scale(chan_mult[j], chan_shift[j], g.rp);
+        const uint32_t sel_a = (lane & 1) ? 0x03070105u : 0x06020400u;  // exchange with lane ^ 1
+        const uint32_t sel_b = (lane & 2) ? 0x03020706u : 0x05040100u;  // exchange with lane ^ 2
+        char *so_lane = so + (wave_m * WM + 4 * half + (lane & 3)) * OP + wave_n * WN + (cl & ~3);
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int32_t xc[4];
+                if (!rows_done) row_terms(i, q, xc); else xc[0] = xc[1] = xc[2] = xc[3] = 0;
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    int32_t v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] - (uint32_t)xc[e]);
+                        v[e] = requant_chan(a, cs[j], g.rp);
+                    }
+                    // bytes = positions e of this lane's channel
+                    const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
+                    const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
+                    uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                    uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0xb1, 0xf, 0xf, false);  // lane ^ 1
+                    p = __builtin_amdgcn_perm(o, p, sel_a);
+                    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0x4e, 0xf, 0xf, false);           // lane ^ 2
+                    p = __builtin_amdgcn_perm(o, p, sel_b);
+                    // now: position 8q + 4 half + lane % 4 of tile row i, channels 4 (cl / 4) .. + 3 of tile column j
+                    *reinterpret_cast<uint32_t *>(so_lane + (i * 32 + 8 * q) * OP + j * 32) = p;
+                }
+            }
+        }
+        __syncthreads();
         const __amdgpu_buffer_rsrc_t ores = make_rsrc(ob, g.o_bytes);
         const __amdgpu_buffer_rsrc_t rres =
             make_rsrc(RES ? reinterpret_cast<const char *>(g.res) + (int64_t)batch * g.out_batch : ob, g.o_bytes);
@@ -909,97 +977,72 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             q_conv = make_chan_scale(load_mult(g.rs_conv, 0), g.rs_conv.shift[0], g.rs_conv.p);
             q_out = make_chan_scale(load_mult(g.rs_out, 0), g.rs_out.shift[0], g.rs_out.p);
         }
-        uint32_t row_off[TM];
-        int32_t xcorr[TM];
+        constexpr int PPR = BN / 16;  // 16-byte pieces per tile row
+        static_assert((BM * PPR) % NTHREADS == 0, "whole pieces per thread");
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
-            const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
-            row_off[i] = m < g.M ? (uint32_t)m * (uint32_t)g.ldo : kOobOffset;
-            xcorr[i] = need_xsum ? xsum[i] : 0;
-        }
+        for (int t = 0; t < BM * PPR / NTHREADS; t++) {
+            const int piece = t * NTHREADS + tid;
+            const int r = piece / PPR, c16 = (piece % PPR) * 16;
+            const int m = m_base + r, n0 = n_base + c16;
+            uint4 d = *reinterpret_cast<const uint4 *>(so + r * OP + c16);
+            const uint32_t off = (m < g.M && n0 < g.N) ? (uint32_t)m * (uint32_t)g.ldo + (uint32_t)n0 : kOobOffset;
+            const bool whole = n0 + 16 <= g.N;
+            if (RES) {
+                uint32_t w[4] = {d.x, d.y, d.z, d.w};
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int nl = wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
-                const int n0 = n_base + nl;
-                ChanParams c[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) c[e] = cp[nl + e];
-#pragma unroll
-                for (int i = 0; i < TM; i++) {
-                    uint32_t packed = 0;
+                for (int k = 0; k < 4; k++) {
+                    const uint32_t xw = buf_load4(rres, (whole || n0 + 4 * k < g.N) && off != kOobOffset ? off + 4 * k : kOobOffset);
+                    uint32_t summed = 0;
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)c[e].bias_adj -
-                                                    (uint32_t)xcorr[i]);
-                        packed |= ((uint32_t)requant_chan(a, c[e].q, g.rp) & 0xffu) << (8 * e);
+                        const int32_t x = (int8_t)(xw >> (8 * e)), y = (int8_t)(w[k] >> (8 * e));
+                        const int32_t r1 = requant_chan(x, q_res, g.rs_res.p), r2 = requant_chan(y, q_conv, g.rs_conv.p);
+                        const int32_t sum = (int32_t)((uint32_t)r1 + (uint32_t)r2);
+                        summed |= ((uint32_t)requant_chan(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
                     }
-                    const uint32_t off = (n0 < g.N && row_off[i] != kOobOffset) ? row_off[i] + (uint32_t)n0 : kOobOffset;
-                    if (RES) {
-                        const uint32_t xw = buf_load4(rres, off);
-                        uint32_t summed = 0;
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const int32_t x = (int8_t)(xw >> (8 * e)), y = (int8_t)(packed >> (8 * e));
-                            const int32_t r1 = requant_chan(x, q_res, g.rs_res.p), r2 = requant_chan(y, q_conv, g.rs_conv.p);
-                            const int32_t sum = (int32_t)((uint32_t)r1 + (uint32_t)r2);
-                            summed |= ((uint32_t)requant_chan(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
-                        }
-                        packed = summed;
-                    }
-                    __builtin_amdgcn_raw_buffer_store_b32(packed, ores, (int)off, 0, 0);
+                    w[k] = summed;
                 }
+                d = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+            if (whole) {
+                __builtin_amdgcn_raw_buffer_store_b128(v4i{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, 0);
+            } else if (off != kOobOffset) {  // the last channels of a row whose extent is not a multiple of 16
+                const uint32_t w[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+                    if (n0 + 4 * k < g.N) __builtin_amdgcn_raw_buffer_store_b32(w[k], ores, (int)(off + 4 * k), 0, 0);
             }
         }
         return;
     }
+    // ---- every other output form: int32 accumulators, or RESCALE to 16- / 32-bit or unaligned 8-bit outputs; a
+    // store instruction writes 32 consecutive channels of two positions
+    ChanScale cs[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) cs[j] = make_chan_scale(chan_mult[j], chan_shift[j], g.rp);
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-        const int m = m_base + wave_m * WM + i * 32 + (lane & 31);
-        if (m >= g.M) continue;
-        const int32_t xcorr = need_xsum ? xsum[i] : 0;
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
+        for (int q = 0; q < 4; q++) {
+            int32_t xc[4];
+            if (!rows_done) row_terms(i, q, xc); else xc[0] = xc[1] = xc[2] = xc[3] = 0;
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int nl = wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
-                const int n0 = n_base + nl;
-                if (n0 >= g.N) continue;
-                int32_t v[4];
+            for (int e = 0; e < 4; e++) {
+                const int m = m_base + wave_m * WM + i * 32 + 8 * q + 4 * half + e;
+                if (m >= g.M) continue;
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int32_t a =
-                        (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)cp[nl + e].bias_adj - (uint32_t)xcorr);
-                    if (!g.fused)
-                        v[e] = a;
+                for (int j = 0; j < TN; j++) {
+                    const int n = n_base + wave_n * WN + j * 32 + cl;
+                    if (n >= g.N) continue;
+                    const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] - (uint32_t)xc[e]);
+                    const int32_t v = g.fused ? requant_chan(a, cs[j], g.rp) : a;
+                    const int64_t off = (int64_t)m * g.ldo + n;
+                    if (g.out_size == 1)
+                        *reinterpret_cast<int8_t *>(ob + off) = (int8_t)v;
+                    else if (g.out_size == 2)
+                        *reinterpret_cast<int16_t *>(ob + off * 2) = (int16_t)v;
                     else
-                        v[e] = requant_chan(a, cp[nl + e].q, g.rp);
-                }
-                const int64_t off = (int64_t)m * g.ldo + n0;
-                if (g.out_vec_ok && n0 + 3 < g.N) {
-                    if (g.out_size == 1) {
-                        const uint32_t packed = (uint32_t)(uint8_t)v[0] | ((uint32_t)(uint8_t)v[1] << 8) |
-                                                ((uint32_t)(uint8_t)v[2] << 16) | ((uint32_t)(uint8_t)v[3] << 24);
-                        *reinterpret_cast<uint32_t *>(ob + off) = packed;
-                    } else if (g.out_size == 2) {
-                        const uint32_t lo = (uint32_t)(uint16_t)v[0] | ((uint32_t)(uint16_t)v[1] << 16);
-                        const uint32_t hi = (uint32_t)(uint16_t)v[2] | ((uint32_t)(uint16_t)v[3] << 16);
-                        *reinterpret_cast<uint2 *>(ob + off * 2) = make_uint2(lo, hi);
-                    } else {
-                        *reinterpret_cast<int4 *>(ob + off * 4) = make_int4(v[0], v[1], v[2], v[3]);
-                    }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        if (n0 + e >= g.N) break;
-                        if (g.out_size == 1)
-                            *reinterpret_cast<int8_t *>(ob + off + e) = (int8_t)v[e];
-                        else if (g.out_size == 2)
-                            *reinterpret_cast<int16_t *>(ob + (off + e) * 2) = (int16_t)v[e];
-                        else
-                            *reinterpret_cast<int32_t *>(ob + (off + e) * 4) = v[e];
-                    }
+                        *reinterpret_cast<int32_t *>(ob + off * 4) = v;
                 }
             }
         }

@@ -239,6 +239,8 @@ DL_CASES = [
     ("tile256_no_zp", 2, 2048, 64, 4096, 0, 0),           # a single K step, no zero-point sums
     ("tile128_band_walk", 1, 2944, 192, 2944, 7, 0),      # 529 tiles of 128 x 128, three K steps
     ("tile128_batched", 16, 640, 320, 1024, 0, -6),       # 5 x 8 tiles per batch, five K steps
+    ("tile128_ring_once", 8, 512, 576, 1024, -1, 3),      # nine K steps: the eight-stage ring is filled and refilled
+    ("tile128_ring_wraps", 4, 1024, 1600, 1024, 4, -2),   # 25 K steps: the ring wraps three times and drains
 ]
 
 
