@@ -12,6 +12,8 @@
 // Zero points follow the same expansion as the matrix kernel: taps that fall into the padding are filled with the
 // input zero point (they then contribute exactly nothing), and
 //   sum (x - zx)(w - zw) = sum x*w - zw * sum x - zx * sum w + K * zx * zw.
+#include <algorithm>
+
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -246,6 +248,213 @@ void launch_direct(DirectArgs &g, int splits, int cus, hipStream_t s) {
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// ROWS on the matrix cores: 1x1 stride-1 CONV2D + RESCALE (+CLAMP) to 8 bits over a dense image with 8..32-byte
+// pixels and at most 192 output channels (MobileNetV2's expansions 16 -> 96, 24 -> 144, 32 -> 192 and 32 -> 16).
+// The contraction is one or two v_mfma_i32_32x32x16_i8 per 32 positions x 32 channels, so the multiply-adds cost
+// next to nothing; the kernel is built around the two things that do cost: the requantisation arithmetic and the
+// output stream.
+//   * A wavefront owns 32 consecutive positions and ALL output channels; it walks position groups in a grid-stride
+//     loop with the weights (matrix B operand) in registers.  Its output tile is therefore one contiguous run of
+//     32 * OC bytes of the NHWC tensor.
+//   * After the multiply a lane holds one channel per 32-channel column (lane % 32) and 16 positions: the channel's
+//     requantisation constants are read once per column from shared memory (32 bytes per lane) and used 16 times.
+//   * The four results of a register group are four consecutive positions of one channel; a 4 x 4 byte transpose
+//     inside each lane quad turns them into four consecutive channels of one position, which go to the wavefront's
+//     own staging tile in shared memory as a dword.  The tile leaves in 16-byte pieces in memory order: every store
+//     instruction writes one kilobyte of consecutive bytes.  No block-wide barrier after the prologue.
+// ---------------------------------------------------------------------------------------------------------------
+struct RowsMfmaArgs {
+    const int8_t *x, *w;
+    const int32_t *bias;
+    char *out;
+    int32_t M, IC, OC, zx, bias_len;
+    int32_t groups;  // ceil(M / 32)
+    int32_t op;      // pitch of a staging row (bytes): OC + padding, chosen so that four consecutive rows start in
+                     // different bank octets
+    uint32_t x_bytes, o_bytes;
+    ScaleRef scale;
+};
+
+typedef int v16i32 __attribute__((ext_vector_type(16)));
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+
+template <int NJ, int KC>
+__global__ void __launch_bounds__(kBlock) conv_rows_mfma_i8_kernel(const RowsMfmaArgs a) {
+    extern __shared__ __align__(16) char smem[];
+    ChanConst *cc = reinterpret_cast<ChanConst *>(smem);  // [NJ * 32], channels at or beyond OC hold zeros
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cl = lane & 31, half = lane >> 5;
+
+    const __amdgpu_buffer_rsrc_t xres =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(a.x), 0, (int)a.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ores = __builtin_amdgcn_make_buffer_rsrc(a.out, 0, (int)a.o_bytes, 0x00020000);
+    const uint32_t kOob = 0x80000000u;
+    auto fetch = [&](int g, long (&xf)[KC]) {  // matrix A operand: lane = position lane % 32 of the group
+        const int m = g * 32 + cl;
+#pragma unroll
+        for (int c = 0; c < KC; c++) {
+            const int k0 = c * 16 + half * 8;
+            const uint32_t off = (g < a.groups && m < a.M && k0 < a.IC) ? (uint32_t)m * (uint32_t)a.IC + (uint32_t)k0 : kOob;
+            const auto v = __builtin_amdgcn_raw_buffer_load_b64(xres, (int)off, 0, 0);
+            xf[c] = (long)(((uint64_t)v[1] << 32) | (uint64_t)v[0]);
+        }
+    };
+    // the first group's pixels and the weights are requested before the constants are worked out, so that the
+    // prologue waits for memory once
+    const int nwaves = (int)gridDim.x * (kBlock / 64);
+    int g = (int)blockIdx.x * (kBlock / 64) + wave;
+    long xf[KC], xn[KC];
+    fetch(g, xf);
+    // ---- the weights as matrix B operand: lane = channel lane % 32 of column j, 8 bytes of K from 16 c + 8 (lane / 32)
+    long wf[NJ][KC];
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+        for (int c = 0; c < KC; c++) {
+            const int oc = j * 32 + cl, k0 = c * 16 + half * 8;
+            wf[j][c] = (oc < a.OC && k0 < a.IC) ? *reinterpret_cast<const long *>(a.w + (int64_t)oc * a.IC + k0) : 0;
+        }
+    // ---- per-channel constants (the input zero point folded into the bias term)
+    for (int oc = tid; oc < NJ * 32; oc += kBlock) {
+        ChanConst c{};
+        if (oc < a.OC) {
+            int32_t wsum = 0;
+            const uint32_t *wp = reinterpret_cast<const uint32_t *>(a.w + (int64_t)oc * a.IC);
+            for (int j = 0; j < a.IC / 4; j++) wsum = __builtin_amdgcn_sdot4((int)wp[j], 0x01010101, wsum, false);
+            const int32_t bias = a.bias[a.bias_len == 1 ? 0 : oc];
+            c.bias_adj = (int32_t)((uint32_t)bias - (uint32_t)a.zx * (uint32_t)wsum);
+            const int ci = a.scale.p.per_channel ? oc : 0;
+            c.q = make_chan_scale(load_mult(a.scale, ci), (int32_t)a.scale.shift[ci], a.scale.p);
+        }
+        cc[oc] = c;
+    }
+    __syncthreads();
+
+    int32_t bias_adj[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; j++) bias_adj[j] = cc[j * 32 + cl].bias_adj;
+    char *so = smem + NJ * 32 * sizeof(ChanConst) + wave * 32 * a.op;  // this wavefront's staging tile [32][op]
+    // the tile's 16-byte pieces in memory order: piece p = row p / (OC / 16), 16-byte column p % (OC / 16)
+    const int ppr = a.OC >> 4, npieces = 32 * ppr;
+    uint32_t piece_lds[NJ], piece_row[NJ];
+#pragma unroll
+    for (int t = 0; t < NJ; t++) {
+        const int p = t * 64 + lane;
+        const int r = p / ppr;
+        piece_row[t] = p < npieces ? (uint32_t)r : 0xffffu;  // beyond the tile: never below a row count
+        piece_lds[t] = p < npieces ? (uint32_t)(r * a.op + (p - r * ppr) * 16) : 0u;
+    }
+    const uint32_t sel_a = (lane & 1) ? 0x03070105u : 0x06020400u;  // exchange with lane ^ 1
+    const uint32_t sel_b = (lane & 2) ? 0x03020706u : 0x05040100u;  // exchange with lane ^ 2
+    char *so_lane = so + (4 * half + (lane & 3)) * a.op + (cl & ~3);
+    for (; g < a.groups; g += nwaves) {
+        fetch(g + nwaves, xn);  // the next group's pixels travel while this one is requantised
+        // the accumulators start from the channel's bias term (every register of a lane is the same channel)
+        v16i32 accs[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) accs[j][r] = bias_adj[j];
+#pragma unroll
+            for (int kc = 0; kc < KC; kc++)
+                accs[j] = __builtin_amdgcn_mfma_i32_32x32x16_i8(xf[kc], wf[j][kc], accs[j], 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const ChanConst c = cc[j * 32 + cl];
+            const bool col_live = j * 32 + (cl & ~3) < a.OC;  // OC is a multiple of 16: whole dwords are in or out
+            const v16i32 acc = accs[j];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int32_t v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    v[e] = requant_chan(acc[4 * q + e], c.q, a.scale.p);
+                }
+                const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
+                const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
+                uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // bytes = positions e of this lane's channel
+                uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0xb1, 0xf, 0xf, false);
+                p = __builtin_amdgcn_perm(o, p, sel_a);
+                o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0x4e, 0xf, 0xf, false);
+                p = __builtin_amdgcn_perm(o, p, sel_b);
+                // now: position 8 q + 4 (lane / 32) + lane % 4, channels 32 j + 4 (lane % 32 / 4) .. + 3
+                if (col_live) *reinterpret_cast<uint32_t *>(so_lane + 8 * q * a.op + j * 32) = p;
+            }
+        }
+        // the wavefront's own writes and reads of its tile execute in order; the compiler must keep that order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const uint32_t rows = (uint32_t)min(32, a.M - g * 32);
+        const uint32_t obase = (uint32_t)g * 32u * (uint32_t)a.OC;
+#pragma unroll
+        for (int t = 0; t < NJ; t++) {
+            const uint4 d = *reinterpret_cast<const uint4 *>(so + piece_lds[t]);
+            const uint32_t off = piece_row[t] < rows ? obase + (uint32_t)(t * 64 + lane) * 16u : kOob;
+            __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int c = 0; c < KC; c++) xf[c] = xn[c];
+    }
+}
+
+template <int NJ>
+void launch_rows_mfma(const RowsMfmaArgs &g, int kc, dim3 grid, size_t sm, hipStream_t s) {
+    if (kc == 1)
+        conv_rows_mfma_i8_kernel<NJ, 1><<<grid, dim3(kBlock), sm, s>>>(g);
+    else
+        conv_rows_mfma_i8_kernel<NJ, 2><<<grid, dim3(kBlock), sm, s>>>(g);
+}
+
+// returns 1 when the case was taken
+int try_rows_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
+                  const mlel_tensor *bias, const mlel_conv2d_attr *a, const FusedEpilogue *epi, int64_t M, int64_t IC,
+                  int64_t OC, int64_t xbytes) {
+    if (epi == nullptr || a->weight_zp != 0) return 0;
+    if (IC % 8 != 0 || IC > 32 || OC % 16 != 0 || OC > 192) return 0;
+    if (((uintptr_t)in->ptr % 8) != 0 || ((uintptr_t)w->ptr % 8) != 0) return 0;
+    if (M * OC >= (int64_t(1) << 31) || M * IC >= (int64_t(1) << 31)) return 0;
+    RowsMfmaArgs g{};
+    g.x = static_cast<const int8_t *>(in->ptr);
+    g.w = static_cast<const int8_t *>(w->ptr);
+    g.bias = static_cast<const int32_t *>(bias->ptr);
+    g.out = static_cast<char *>(out->ptr);
+    g.M = (int)M;
+    g.IC = (int)IC;
+    g.OC = (int)OC;
+    g.zx = a->input_zp;
+    g.bias_len = (int)bias->dims[0];
+    g.groups = (int)((M + 31) / 32);
+    int op = (int)OC;
+    while (op % 128 != 32 && op % 128 != 96) op += 16;
+    g.op = op;
+    g.x_bytes = (uint32_t)xbytes;
+    g.o_bytes = (uint32_t)(M * OC);
+    g.scale = make_ref(*epi);
+    const int nj = (int)((OC + 31) / 32), kc = IC > 16 ? 2 : 1;
+    const size_t sm = (size_t)nj * 32 * sizeof(ChanConst) + (size_t)(kBlock / 64) * 32 * op;
+    const int cus = ctx != nullptr && ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
+    // three blocks (twelve wavefronts) per compute unit (measured: two to four are equal within 3 %), fewer when the
+    // problem has fewer position groups
+    const int64_t want = std::min<int64_t>((int64_t)cus * 3, (g.groups + kBlock / 64 - 1) / (kBlock / 64));
+    const dim3 grid((unsigned)std::max<int64_t>(want, 1));
+    switch (nj) {
+    case 1: launch_rows_mfma<1>(g, kc, grid, sm, s); break;
+    case 2: launch_rows_mfma<2>(g, kc, grid, sm, s); break;
+    case 3: launch_rows_mfma<3>(g, kc, grid, sm, s); break;
+    case 4: launch_rows_mfma<4>(g, kc, grid, sm, s); break;
+    case 5: launch_rows_mfma<5>(g, kc, grid, sm, s); break;
+    default: launch_rows_mfma<6>(g, kc, grid, sm, s); break;
+    }
+    return 1;
+}
+
 }  // namespace
 
 int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
@@ -281,8 +490,15 @@ int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, c
                in->strides[0] == H * in->strides[1] && ((uintptr_t)in->ptr % 4) == 0 && ((uintptr_t)w->ptr % 4) == 0) {
         mode = ROWS;
     }
+    if (M <= 0 && mode >= 0) return 1;
+    const bool rows_shape = KH == 1 && KW == 1 && a->stride[0] == 1 && a->stride[1] == 1 && a->pad[0] == 0 &&
+                            a->pad[2] == 0 && OH == H && OW == W && in->strides[1] == W * in->strides[2] &&
+                            in->strides[0] == H * in->strides[1];
+    if (rows_shape && M > 0 && try_rows_mfma(ctx, s, out, in, w, bias, a, epi, M, IC, OC, xbytes)) {
+        MLEL_TRY(check_launch("conv2d rows int8"));
+        return 1;
+    }
     if (mode < 0) return 0;
-    if (M <= 0) return 1;
 
     DirectArgs g{};
     g.x = static_cast<const int8_t *>(in->ptr);

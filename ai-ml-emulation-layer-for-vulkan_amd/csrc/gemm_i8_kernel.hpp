@@ -934,12 +934,40 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         char *so = smem + (3 * BM + 2 * BN) * 4;           // behind the tables of the zero-point sums
         static_assert((3 * BM + 2 * BN) * 4 + BM * OP <= (int)(2 * BM * PITCH + 2 * w_buf_bytes<BN>()),
                       "the staging tile fits the operand buffers");
+        // Narrow tiles (fewer than 128 channels) store the dwords directly instead: runs of 32 bytes per row, without
+        // the barrier and the trip through shared memory, which is what their few outputs per thread can afford.
+        constexpr bool STAGED = BN >= 128;
+        const __amdgpu_buffer_rsrc_t ores = make_rsrc(ob, g.o_bytes);
+        const __amdgpu_buffer_rsrc_t rres =
+            make_rsrc(RES ? reinterpret_cast<const char *>(g.res) + (int64_t)batch * g.out_batch : ob, g.o_bytes);
+        ChanScale q_res{}, q_conv{}, q_out{};
+        if (RES) {
+            q_res = make_chan_scale(load_mult(g.rs_res, 0), g.rs_res.shift[0], g.rs_res.p);
+            q_conv = make_chan_scale(load_mult(g.rs_conv, 0), g.rs_conv.shift[0], g.rs_conv.p);
+            q_out = make_chan_scale(load_mult(g.rs_out, 0), g.rs_out.shift[0], g.rs_out.p);
+        }
         ChanScale cs[TN];
 #pragma unroll
         for (int j = 0; j < TN; j++) cs[j] = make_chan_scale(chan_mult[j], chan_shift[j], g.rp);
         const uint32_t sel_a = (lane & 1) ? 0x03070105u : 0x06020400u;  // exchange with lane ^ 1
         const uint32_t sel_b = (lane & 2) ? 0x03020706u : 0x05040100u;  // exchange with lane ^ 2
         char *so_lane = so + (wave_m * WM + 4 * half + (lane & 3)) * OP + wave_n * WN + (cl & ~3);
+        // direct stores: where this lane's dwords go, and the residual operand's dwords, requested before the arithmetic
+        uint32_t d_off[STAGED ? 1 : TM * 4 * TN], d_res[(STAGED || !RES) ? 1 : TM * 4 * TN];
+        if constexpr (!STAGED) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const int m = m_base + wave_m * WM + i * 32 + 8 * q + 4 * half + (lane & 3);
+                        const int n0 = n_base + wave_n * WN + j * 32 + (cl & ~3);
+                        const int k = (i * 4 + q) * TN + j;
+                        d_off[k] = (m < g.M && n0 < g.N) ? (uint32_t)m * (uint32_t)g.ldo + (uint32_t)n0 : kOobOffset;
+                        if constexpr (RES) d_res[k] = buf_load4(rres, d_off[k]);
+                    }
+        }
 #pragma unroll
         for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -963,20 +991,29 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                     o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0x4e, 0xf, 0xf, false);           // lane ^ 2
                     p = __builtin_amdgcn_perm(o, p, sel_b);
                     // now: position 8q + 4 half + lane % 4 of tile row i, channels 4 (cl / 4) .. + 3 of tile column j
-                    *reinterpret_cast<uint32_t *>(so_lane + (i * 32 + 8 * q) * OP + j * 32) = p;
+                    if constexpr (STAGED) {
+                        *reinterpret_cast<uint32_t *>(so_lane + (i * 32 + 8 * q) * OP + j * 32) = p;
+                    } else {
+                        const uint32_t off = d_off[(i * 4 + q) * TN + j];
+                        if constexpr (RES) {
+                            const uint32_t xw = d_res[(i * 4 + q) * TN + j];
+                            uint32_t summed = 0;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                const int32_t x = (int8_t)(xw >> (8 * e)), y = (int8_t)(p >> (8 * e));
+                                const int32_t r1 = requant_chan(x, q_res, g.rs_res.p), r2 = requant_chan(y, q_conv, g.rs_conv.p);
+                                const int32_t sum = (int32_t)((uint32_t)r1 + (uint32_t)r2);
+                                summed |= ((uint32_t)requant_chan(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
+                            }
+                            p = summed;
+                        }
+                        __builtin_amdgcn_raw_buffer_store_b32(p, ores, (int)off, 0, 0);
+                    }
                 }
             }
         }
+        if constexpr (!STAGED) return;
         __syncthreads();
-        const __amdgpu_buffer_rsrc_t ores = make_rsrc(ob, g.o_bytes);
-        const __amdgpu_buffer_rsrc_t rres =
-            make_rsrc(RES ? reinterpret_cast<const char *>(g.res) + (int64_t)batch * g.out_batch : ob, g.o_bytes);
-        ChanScale q_res{}, q_conv{}, q_out{};
-        if (RES) {
-            q_res = make_chan_scale(load_mult(g.rs_res, 0), g.rs_res.shift[0], g.rs_res.p);
-            q_conv = make_chan_scale(load_mult(g.rs_conv, 0), g.rs_conv.shift[0], g.rs_conv.p);
-            q_out = make_chan_scale(load_mult(g.rs_out, 0), g.rs_out.shift[0], g.rs_out.p);
-        }
         constexpr int PPR = BN / 16;  // 16-byte pieces per tile row
         static_assert((BM * PPR) % NTHREADS == 0, "whole pieces per thread");
 #pragma unroll

@@ -146,6 +146,12 @@ CONV_CASES = [
     # enough positions for the direct kernel to take two per thread, ragged last block; a long run of 24-byte pixels
     ("pw_16_96_two_positions", (2, 223, 225, 16), 96, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 17, 0),
     ("pw_24_144_many_positions", (1, 251, 243, 24), 144, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -9, 4),
+    # short contractions on the matrix cores: half-used channel columns, 8-byte pixels, fewer positions than a group
+    ("pw_8_16_tiny", (1, 5, 5, 8), 16, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 33, 0),
+    ("pw_16_48", (2, 9, 11, 16), 48, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -77, 0),
+    ("pw_32_80", (3, 13, 7, 32), 80, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 127, 0),
+    ("pw_24_176", (1, 31, 33, 24), 176, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -128, 0),
+    ("pw_32_16_many", (4, 56, 57, 32), 16, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 5, 0),
 ]
 
 
