@@ -98,10 +98,13 @@ namespace {
 // taps; a v_dot4_i32_i8 against the matching weight column then adds three taps at once, and a column is shared by
 // up to three neighbouring outputs.  Padded taps are filled with the input zero point, so the expansion
 //   sum (x - zi)(w - zw) = sum x*w - zw * sum x - zi * sum w + 9 * zi * zw
-// gives exactly the reference's result (padded taps contribute nothing).  Every thread prepares the weight columns
-// and requantisation constants of its own four channels in registers (dword loads that hit in cache), so there is
-// no shared-memory stage and no barrier.  Consecutive blocks are dealt to the XCDs in contiguous runs, so rows
-// shared by vertically adjacent items are fetched into one L2 only.
+// gives exactly the reference's result (padded taps contribute nothing).  A block covers CB channel quads x SPB
+// spatial items of one image; its first 4 CB threads work out one channel each (three weight columns, the bias with
+// the zero-point terms folded in, the requantisation constants) into shared memory, and after one barrier every
+// thread reads the 48 bytes of each of its four channels.  (Every thread preparing its own four channels cost
+// 8 of 25 vector instructions per output, three runtime divisions for its position among them.)  Consecutive
+// blocks are dealt to the XCDs in contiguous runs, so rows shared by vertically adjacent items are fetched into
+// one L2 only.
 // ---------------------------------------------------------------------------------------------------------------
 struct DwArgs {
     const int8_t *x, *w;
@@ -113,10 +116,21 @@ struct DwArgs {
     int32_t sy, sx, pad_t, pad_l, zi, zw, bias_len;
     int32_t fused, out_size;
     ScaleRef scale;
-    uint32_t items;  // N * row groups * strips * C/4
     int32_t strips, row_groups;
-    int32_t blocks, chunk;  // launch geometry: `chunk` consecutive blocks of items per XCD
+    // block = cb_size channel quads x spb spatial items (row group, strip) of one image; blocks are ordered
+    // [image][spatial block][channel block]
+    int32_t cb_size, cb_count, spb, sb_count;
+    uint32_t cb_magic, strips_magic;  // floor(2^32 / d) + 1: x / d == umulhi(x, magic) for x < 2^16, 1 < d < 2^16
+    int32_t blocks, chunk;  // launch geometry: `chunk` consecutive blocks per XCD
 };
+
+struct DwChan {  // per channel, in shared memory: 48 bytes
+    ChanScale q;
+    int32_t bias_adj;
+    uint32_t wcol[3];  // column kx: bytes = the taps (0, kx), (1, kx), (2, kx), 0
+    uint32_t pad[2];
+};
+static_assert(sizeof(DwChan) == 48, "DwChan layout");
 
 // 3 rows x 4 channels (bytes) -> 4 channels x (3 taps, 0)
 __device__ __forceinline__ void transpose_3x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t (&col)[4]) {
@@ -134,44 +148,61 @@ __device__ __forceinline__ void transpose_3x4(uint32_t r0, uint32_t r1, uint32_t
 // offsets, so an address costs one add.
 template <int TX, int TY, int SX, bool ZW, bool Q8>
 __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
+    __shared__ __align__(16) DwChan chan[kBlock];
     // blocks are dealt round-robin to the XCDs: give XCD k the k-th contiguous run of blocks
     const int bid = (int)(blockIdx.x % 8u) * a.chunk + (int)(blockIdx.x / 8u);
     if (bid >= a.blocks) return;
-    const uint32_t item = (uint32_t)bid * kBlock + threadIdx.x;
-    if (item >= a.items) return;
-    const uint32_t c4n = (uint32_t)a.C >> 2;
-    const int c4 = (int)(item % c4n);
-    uint32_t rest = item / c4n;
-    const int strip = (int)(rest % (uint32_t)a.strips);
-    rest /= (uint32_t)a.strips;
-    const int rg = (int)(rest % (uint32_t)a.row_groups);
-    const int n = (int)(rest / (uint32_t)a.row_groups);
+    // block -> (image, spatial block, channel block): uniform, on the scalar unit
+    const int cb = bid % a.cb_count;
+    const int rest_b = bid / a.cb_count;
+    const int sb = rest_b % a.sb_count;
+    const int n = rest_b / a.sb_count;
+    const int tid = threadIdx.x;
+
+    // ---- one channel per thread: weight columns, bias with the zero-point terms folded in, scales
+    if (tid < 4 * a.cb_size) {
+        const int ch = cb * a.cb_size * 4 + tid;
+        DwChan d{};
+        if (ch < a.C) {
+            int32_t wsum = 0;
+#pragma unroll
+            for (int kx = 0; kx < 3; kx++) {
+                const uint32_t w0 = (uint8_t)a.w[(0 * 3 + kx) * a.C + ch], w1 = (uint8_t)a.w[(1 * 3 + kx) * a.C + ch],
+                               w2 = (uint8_t)a.w[(2 * 3 + kx) * a.C + ch];
+                d.wcol[kx] = w0 | (w1 << 8) | (w2 << 16);
+                wsum = __builtin_amdgcn_sdot4((int)d.wcol[kx], 0x00010101, wsum, false);
+            }
+            const int32_t bias = a.bias[a.bias_len == 1 ? 0 : ch];
+            d.bias_adj = (int32_t)((uint32_t)bias - (uint32_t)a.zi * (uint32_t)wsum + 9u * (uint32_t)a.zi * (uint32_t)a.zw);
+            if (Q8 || a.fused) {
+                const int ci = a.scale.p.per_channel ? ch : 0;
+                d.q = make_chan_scale(load_mult(a.scale, ci), (int32_t)a.scale.shift[ci], a.scale.p);
+            }
+        }
+        chan[(tid & 3) * 64 + (tid >> 2)] = d;  // [channel of the quad][quad]: a lane's reads are 48 bytes apart
+    }
+    __syncthreads();
+
+    // ---- thread -> (channel quad, spatial item) of the block
+    const uint32_t sl = a.cb_size == 1 ? (uint32_t)tid : __umulhi((uint32_t)tid, a.cb_magic);  // tid / cb_size
+    const int cl = tid - (int)sl * a.cb_size;
+    const int c4 = cb * a.cb_size + cl;
+    const uint32_t sp = (uint32_t)sb * (uint32_t)a.spb + sl;  // spatial item of the image: row group * strips + strip
+    if ((int)sl >= a.spb || c4 * 4 >= a.C || sp >= (uint32_t)(a.row_groups * a.strips)) return;
+    const int rg = a.strips == 1 ? (int)sp : (int)__umulhi(sp, a.strips_magic);
+    const int strip = (int)sp - rg * a.strips;
     const int c = c4 * 4;
     const int ox0 = strip * TX, oy0 = rg * TY;
 
-    // ---- this thread's constants: weight columns, bias with the zero-point terms folded in, scales
     uint32_t wc[3][4];
-    int32_t wsum[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (int kx = 0; kx < 3; kx++) {
-        const uint32_t w0 = *reinterpret_cast<const uint32_t *>(a.w + (0 * 3 + kx) * a.C + c);
-        const uint32_t w1 = *reinterpret_cast<const uint32_t *>(a.w + (1 * 3 + kx) * a.C + c);
-        const uint32_t w2 = *reinterpret_cast<const uint32_t *>(a.w + (2 * 3 + kx) * a.C + c);
-        transpose_3x4(w0, w1, w2, wc[kx]);
-#pragma unroll
-        for (int e = 0; e < 4; e++) wsum[e] = __builtin_amdgcn_sdot4((int)wc[kx][e], 0x00010101, wsum[e], false);
-    }
     int32_t bias_adj[4];
     ChanScale q[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) {
-        const int32_t bias = a.bias[a.bias_len == 1 ? 0 : c + e];
-        bias_adj[e] = (int32_t)((uint32_t)bias - (uint32_t)a.zi * (uint32_t)wsum[e] +
-                                9u * (uint32_t)a.zi * (uint32_t)a.zw);
-        if (Q8 || a.fused) {
-            const int ci = a.scale.p.per_channel ? c + e : 0;
-            q[e] = make_chan_scale(load_mult(a.scale, ci), (int32_t)a.scale.shift[ci], a.scale.p);
-        }
+        const DwChan d = chan[e * 64 + cl];
+        wc[0][e] = d.wcol[0], wc[1][e] = d.wcol[1], wc[2][e] = d.wcol[2];
+        bias_adj[e] = d.bias_adj;
+        q[e] = d.q;
     }
 
     // ---- input columns ix0 .. ix0 + NCOL - 1 of rows iy0 .. iy0 + NROW - 1
@@ -325,10 +356,19 @@ int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     if (epi) g.scale = make_ref(*epi);
     g.strips = (int)((OW + TX - 1) / TX);
     g.row_groups = (int)((OH + TY - 1) / TY);
-    const int64_t items = N * g.row_groups * g.strips * (C / 4);
-    if (items >= (int64_t(1) << 31) - kBlock) return 0;
-    g.items = (uint32_t)items;
-    const int64_t blocks = (items + kBlock - 1) / kBlock;
+    // channel quads per block: all of them up to 64, else the even split into the fewest chunks of at most 64
+    const int c4n = (int)(C / 4);
+    const int chunks = (c4n + 63) / 64;
+    g.cb_size = (c4n + chunks - 1) / chunks;
+    g.cb_count = (c4n + g.cb_size - 1) / g.cb_size;
+    g.spb = kBlock / g.cb_size;
+    const int64_t spatial = (int64_t)g.row_groups * g.strips;
+    if (spatial >= (1 << 16)) return 0;  // the magic-number divisions hold below 2^16
+    g.sb_count = (int)((spatial + g.spb - 1) / g.spb);
+    g.cb_magic = (uint32_t)((uint64_t(1) << 32) / (uint64_t)g.cb_size + 1);
+    g.strips_magic = (uint32_t)((uint64_t(1) << 32) / (uint64_t)g.strips + 1);
+    const int64_t blocks = N * g.sb_count * g.cb_count;
+    if (blocks >= (int64_t(1) << 31) - 8) return 0;
     g.blocks = (int)blocks;
     g.chunk = (int)((blocks + 7) / 8);
     const dim3 grid((unsigned)(g.chunk * 8)), block(kBlock);

@@ -569,6 +569,9 @@ DW_CASES = [
     ("stride2_odd", (2, 15, 13, 20), 1, (3, 3), (1, 1, 1, 1), (2, 2), (1, 1), 2, -1),
     ("stride_2x1", (1, 9, 9, 8), 1, (3, 3), (1, 1, 1, 1), (2, 1), (1, 1), 1, 0),
     ("c2052", (1, 4, 5, 2052), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -3, 0),
+    ("one_strip_many_rows", (2, 9, 4, 384), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), 5, 0),
+    ("one_quad", (1, 10, 9, 4), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -6, 2),
+    ("many_spatial_blocks", (2, 32, 32, 32), 1, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), 7, 0),
 ]
 
 
