@@ -255,6 +255,8 @@ int mlel_hip_max_pool2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, con
     MLEL_TRY(check_supported(in, "max_pool2d in"));
     MLEL_REQUIRE(out->rank == 4 && in->rank == 4 && in->dtype == out->dtype, MLEL_ERR_INVALID,
                  "max_pool2d: rank 4 tensors of one type");
+    const int rc = try_maxpool_fast(ctx, (hipStream_t)stream, out, in, attr);
+    if (rc != 0) return rc < 0 ? rc : 0;
     return pool_generic_launch((hipStream_t)stream, false, out, in, attr);
 }
 
@@ -269,6 +271,8 @@ int mlel_hip_table(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const ml
                  "table: the table is a rank-1 tensor of the input type");
     MLEL_REQUIRE(out->dtype == (in->dtype == MLEL_I8 ? MLEL_I8 : MLEL_I32) && out->rank == in->rank, MLEL_ERR_INVALID,
                  "table: i8 -> i8 or i16 -> i32");
+    const int rc = try_table_fast(ctx, (hipStream_t)stream, out, in, table);
+    if (rc != 0) return rc < 0 ? rc : 0;
     return table_generic_launch((hipStream_t)stream, out, in, table);
 }
 

@@ -152,6 +152,11 @@ int try_binary_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out
                     const mlel_tensor *in2);
 int try_avgpool_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                      const mlel_pool2d_attr *a);
+// ops_vec.hip: packed integer tensors, 128 bits per thread
+int try_maxpool_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                     const mlel_pool2d_attr *a);
+int try_table_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                   const mlel_tensor *table);
 int try_transpose_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
                        const uint32_t *perms);
 int rescale_add_rescale_launch(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in1,

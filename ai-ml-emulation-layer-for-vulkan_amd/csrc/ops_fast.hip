@@ -401,16 +401,6 @@ int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     return 1;
 }
 
-int try_rescale_fast(mlel_ctx *, hipStream_t, const mlel_tensor *, const mlel_tensor *, const mlel_tensor *,
-                     const mlel_tensor *, const mlel_rescale_attr *, const RescaleParams &) {
-    return 0;
-}
-int try_clamp_fast(mlel_ctx *, hipStream_t, const mlel_tensor *, const mlel_tensor *, const mlel_clamp_attr *) {
-    return 0;
-}
-int try_binary_fast(mlel_ctx *, hipStream_t, int, const mlel_tensor *, const mlel_tensor *, const mlel_tensor *) {
-    return 0;
-}
 namespace {
 
 // ---------------------------------------------------------------------------------------------------------------

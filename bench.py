@@ -7,11 +7,12 @@ multiplier 1518500250 / shift 39, double round), one launch of the MFMA contract
 also reports the MobileNetV2-shaped int8 graph at batch 32 (BASELINE config 3) executed through the host-side
 GraphPipeline, the roofline position of the dominant kernel and a CPU baseline (the oracle on the host cores).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|config1|mobilenetv2|encoder|layer] [--layer N]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|config1|mobilenetv2|encoder|layer|standalone] [--layer N]
 
 `--only` restricts the run to one leg (profiling runs: one kernel family per trace); `--only layer --layer N` launches
 the N-th operator of the fused MobileNetV2 graph 200 times back to back and nothing else, so that counters of a single
-layer can be collected.  The whole-graph legs always time at least 20 graphs.
+layer can be collected; `--only standalone` times the bandwidth-bound operators of the unfused config 2 graph (RESCALE,
+CLAMP, ADD, TABLE, MAX_POOL2D) as stand-alone launches.  The whole-graph legs always time at least 20 graphs.
 """
 import re
 import argparse
@@ -185,6 +186,54 @@ def run_layer(dev, abi, index, reps=200):
     return res
 
 
+def bench_standalone(dev, abi, reps=100):
+    """The bandwidth-bound operators of the UNFUSED config 2 graph as stand-alone launches on its tensor sizes
+    (16 x 56 x 56 x 144 int32 accumulators / int8 activations): microseconds per launch and algorithmic GB/s (input +
+    output bytes once) of the packed 128-bit kernels, `reps` back-to-back launches each between two events."""
+    rng = np.random.default_rng(1005)
+    shape = (16, 56, 56, 144)
+    n = int(np.prod(shape))
+    acc = rng.integers(-2 ** 22, 2 ** 22, shape).astype(np.int32)
+    acc2 = rng.integers(-2 ** 22, 2 ** 22, shape).astype(np.int32)
+    x8 = rng.integers(-128, 127, shape, endpoint=True).astype(np.int8)
+    mult = rng.integers(2 ** 30, 2 ** 31 - 1, (144,), endpoint=True).astype(np.int32)
+    shift = rng.integers(30, 38, (144,), endpoint=True).astype(np.int8)
+    tab = rng.integers(-128, 127, (256,), endpoint=True).astype(np.int8)
+    t_acc, t_acc2, t_x8 = dev.from_numpy(acc), dev.from_numpy(acc2), dev.from_numpy(x8)
+    t_m, t_s, t_tab = dev.from_numpy(mult), dev.from_numpy(shift), dev.from_numpy(tab)
+    o8, o32 = dev.tensor(abi.I8, shape), dev.tensor(abi.I32, shape)
+    o_pool = dev.tensor(abi.I8, (16, 28, 28, 144))
+    r_down = abi.rescale_attr(0, 3, True, True, True)
+    r_up = abi.rescale_attr(-5, 0, True, True, True)
+    clamp = abi.ClampAttr(0.0, 96.0, int(abi.NAN_PROPAGATE))
+    pool = abi.pool2d_attr((3, 3), (2, 2), (0, 1, 0, 1))
+    cases = [
+        ("RESCALE int32->int8 per channel", 5 * n,
+         lambda: dev.op("rescale", o8.ref, t_acc.ref, t_m.ref, t_s.ref, C.byref(r_down))),
+        ("RESCALE int8->int32 per channel", 5 * n,
+         lambda: dev.op("rescale", o32.ref, t_x8.ref, t_m.ref, t_s.ref, C.byref(r_up))),
+        ("CLAMP int8", 2 * n, lambda: dev.op("clamp", o8.ref, t_x8.ref, C.byref(clamp))),
+        ("ADD int32", 12 * n, lambda: dev.op("elementwise_binary", abi.BIN["ADD"], o32.ref, t_acc.ref, t_acc2.ref,
+                                             int(abi.NAN_PROPAGATE))),
+        ("TABLE int8", 2 * n, lambda: dev.op("table", o8.ref, t_x8.ref, t_tab.ref)),
+        ("MAX_POOL2D int8 3x3 stride 2", n + n // 4, lambda: dev.op("max_pool2d", o_pool.ref, t_x8.ref, C.byref(pool))),
+    ]
+    out = []
+    ev0, ev1 = dev.event(), dev.event()
+    for name, nbytes, fn in cases:
+        for _ in range(5):
+            fn()
+        dev.record(ev0)
+        for _ in range(reps):
+            fn()
+        dev.record(ev1)
+        dev.sync()
+        us = dev.elapsed_ms(ev0, ev1) / reps * 1e3
+        out.append({"operator": name, "shape": list(shape), "us": round(us, 2), "algorithmic_bytes": nbytes,
+                    "gbs": round(nbytes / (us * 1e-6) / 1e9, 1), "hbm_frac": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -192,7 +241,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline legs (profiling runs)")
     ap.add_argument("--skip-graph", action="store_true", help="omit the MobileNetV2 and encoder graph legs")
-    ap.add_argument("--only", choices=["all", "config1", "mobilenetv2", "encoder", "layer"], default="all")
+    ap.add_argument("--only", choices=["all", "config1", "mobilenetv2", "encoder", "layer", "standalone"], default="all")
     ap.add_argument("--layer", type=int, default=3, help="with --only layer: position in the fused config 3 graph")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -206,6 +255,11 @@ def main():
 
     if args.only == "layer":
         print(json.dumps(run_layer(dev, abi, args.layer)), flush=True)
+        dev.close()
+        return
+
+    if args.only == "standalone":
+        print(json.dumps({"only": "standalone", "operators": bench_standalone(dev, abi)}), flush=True)
         dev.close()
         return
 

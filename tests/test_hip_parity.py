@@ -669,6 +669,65 @@ def test_clamp_binary_mul_table_vs_oracle(run, oracle):
     np.testing.assert_array_equal(run.table(x16, t16, abi.I32), oracle.table(x16, t16, abi.I32))
 
 
+def test_packed_integer_operators_vs_oracle(run, oracle):
+    """The 128-bit kernels behind stand-alone RESCALE, CLAMP, TABLE, MAX_POOL2D and same-shape int32 elementwise
+    operators: packed tensors large enough for several blocks, element counts with a tail behind the last 16 bytes,
+    every input / output width, extreme values, bit for bit against the oracle."""
+    rng = np.random.default_rng(1313)
+    # RESCALE: int32 accumulators -> int8 / int16 / int32 per channel (24 channels: not a multiple of 16), extremes
+    acc = ri(rng, -2 ** 27, 2 ** 27, (2, 29, 31, 24), np.int32)
+    acc[0, 0, 0, :6] = [2 ** 31 - 1, -2 ** 31, 0, -1, 1, 2 ** 30]
+    mult, shift = rescale_params(rng, 24)
+    shift[:5] = [2, 31, 32, 48, 62]
+    for dr in (False, True):
+        for zi, zo in ((0, 3), (-77, -128)):
+            attr = abi.rescale_attr(zi, zo, True, dr, True)
+            for odt in (abi.I8, abi.I16, abi.I32):
+                np.testing.assert_array_equal(run.rescale(acc, mult, shift, odt, attr),
+                                              oracle.rescale(acc, mult, shift, odt, attr), err_msg=f"{dr} {zi} {odt}")
+    # int8 / int16 inputs, signed and unsigned, per tensor, into int32 and int8 (the operands of the residual ADD)
+    x8 = ri(rng, -128, 127, (3, 17, 13, 20), np.int8)
+    x16 = ri(rng, -32768, 32767, (3, 17, 13, 20), np.int16)
+    m1, s1 = np.array([1 << 30], np.int32), np.array([11], np.int8)
+    for x in (x8, x16):
+        for unsigned in (False, True):
+            attr = abi.rescale_attr(5, 0, True, True, False, input_unsigned=unsigned)
+            np.testing.assert_array_equal(run.rescale(x, m1, s1, abi.I32, attr), oracle.rescale(x, m1, s1, abi.I32, attr))
+    attru = abi.rescale_attr(128, 128, True, False, False, input_unsigned=True, output_unsigned=True)
+    m2, s2 = np.array([1234567890], np.int32), np.array([30], np.int8)
+    np.testing.assert_array_equal(run.rescale(x8, m2, s2, abi.I8, attru), oracle.rescale(x8, m2, s2, abi.I8, attru))
+    m16, s16 = ri(rng, 1, 32767, (20,), np.int16), ri(rng, 8, 20, (20,), np.int8)
+    attr16 = abi.rescale_attr(0, -1, False, False, True)
+    np.testing.assert_array_equal(run.rescale(x16, m16, s16, abi.I8, attr16), oracle.rescale(x16, m16, s16, abi.I8, attr16))
+    # CLAMP: every signed width, odd element counts (a tail behind the last 16 bytes)
+    for dt, lo, hi in ((np.int8, -128, 127), (np.int16, -32768, 32767), (np.int32, -2 ** 31, 2 ** 31 - 1)):
+        x = ri(rng, lo, hi, (7, 1009), dt)
+        for mn, mx in ((-3, 100), (lo, hi), (5, 5)):
+            np.testing.assert_array_equal(run.clamp(x, mn, mx), oracle.clamp(x, mn, mx), err_msg=f"{dt} {mn} {mx}")
+    # int32 elementwise, same shape, with a tail
+    a = ri(rng, -2 ** 31, 2 ** 31 - 1, (5, 1001), np.int32)
+    b = ri(rng, -2 ** 31, 2 ** 31 - 1, (5, 1001), np.int32)
+    for op in ("ADD", "SUB", "MAXIMUM", "MINIMUM", "BITWISE_AND", "BITWISE_OR", "BITWISE_XOR"):
+        np.testing.assert_array_equal(run.binary(op, a, b, a.shape, abi.I32),
+                                      oracle.elementwise_binary(op, a, b, a.shape, abi.I32), err_msg=op)
+    # TABLE
+    t8 = ri(rng, -128, 127, (256,), np.int8)
+    xt = ri(rng, -128, 127, (3, 4099), np.int8)
+    xt[0, :256] = np.arange(-128, 128)
+    np.testing.assert_array_equal(run.table(xt, t8, abi.I8), oracle.table(xt, t8, abi.I8))
+    t16 = ri(rng, -32768, 32767, (513,), np.int16)
+    xt16 = ri(rng, -32768, 32767, (4101,), np.int16)
+    xt16[:4] = [-32768, 32767, 0, -1]
+    np.testing.assert_array_equal(run.table(xt16, t16, abi.I32), oracle.table(xt16, t16, abi.I32))
+    # MAX_POOL2D int8: stride 2 with padding, a window larger than the image, all-lowest input
+    xp = ri(rng, -128, 127, (2, 19, 23, 36), np.int8)
+    xp[1, :3] = -128
+    ap = abi.pool2d_attr((3, 3), (2, 2), (1, 1, 1, 1))
+    np.testing.assert_array_equal(run.pool("max_pool2d", xp, (2, 10, 12, 36), ap), oracle.max_pool2d(xp, (2, 10, 12, 36), ap))
+    ap2 = abi.pool2d_attr((2, 5), (1, 3), (0, 1, 2, 1))
+    np.testing.assert_array_equal(run.pool("max_pool2d", xp, (2, 19, 8, 36), ap2), oracle.max_pool2d(xp, (2, 19, 8, 36), ap2))
+
+
 def test_pool_reduce_cast_negate_vs_oracle(run, oracle):
     rng = np.random.default_rng(14)
     x = ri(rng, -128, 127, (2, 7, 7, 40), np.int8)
