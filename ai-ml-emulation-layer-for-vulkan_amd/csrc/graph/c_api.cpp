@@ -44,6 +44,7 @@
 #include <string>
 
 #include "../../../include/mlel_graph.h"
+#include "graph_log.hpp"
 #include "graph_pipeline.hpp"
 #include "session_planner.hpp"
 #include "spirv_graph_loader.hpp"
@@ -96,9 +97,11 @@ int guarded(F &&f) {
         return f();
     } catch (const std::out_of_range &e) {
         g_error = std::string("not found: ") + e.what();
+        MLEL_GRAPH_LOG(Error, g_error);
         return MLEL_ERR_INVALID;
     } catch (const std::exception &e) {
         g_error = e.what();
+        MLEL_GRAPH_LOG(Error, g_error);
         const bool unsupported = g_error.find("has no kernel") != std::string::npos;
         return unsupported ? MLEL_ERR_UNSUPPORTED : MLEL_ERR_INVALID;
     }
@@ -640,6 +643,12 @@ int mlel_graph_dispatch_profiled(mlel_graph *g, void *stream, float *ms, int cap
         for (size_t i = 0; i < all.size() && static_cast<int>(i) < capacity; i++) ms[i] = all[i];
         return static_cast<int>(all.size());
     });
+}
+
+int mlel_graph_log_level(void) { return (int)mlel::graphlog::level(); }
+int mlel_graph_log_reload(void) {
+    mlel::graphlog::reload();
+    return (int)mlel::graphlog::level();
 }
 
 int mlel_graph_set_profiling(mlel_graph *g, int enabled) {

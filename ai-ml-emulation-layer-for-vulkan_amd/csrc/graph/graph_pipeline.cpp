@@ -1,5 +1,7 @@
 #include "graph_pipeline.hpp"
 
+#include "graph_log.hpp"
+
 #include <cstdlib>
 
 #include <algorithm>
@@ -119,6 +121,8 @@ GraphPipeline::~GraphPipeline() {
 TensorPtr GraphPipeline::registerTensor(TensorPtr t) {
     t->id = static_cast<int>(allTensors.size());
     allTensors.push_back(t);
+    MLEL_GRAPH_LOG(Debug, "Create tensor. tensor=" << t->id << " dtype=" << t->getFormat() << " rank=" << t->getRank()
+                                                   << " bytes=" << t->getSize());
     return t;
 }
 
@@ -1246,6 +1250,10 @@ void GraphPipeline::plan() {
             unseen.push_back({i, aligned(t->getSize())});
     }
     details::AllocationPlan planResult;
+    // the reference reports its choice at this severity when a session is created (graph_layer.cpp:286-295)
+    MLEL_GRAPH_LOG(Info, (planner == MemoryPlanner::Interval ? "Using interval memory planner"
+                          : planner == MemoryPlanner::Linear ? "Using linear memory planner"
+                                                             : "Using best-fit memory planner"));
     if (planner == MemoryPlanner::Interval) {
         planResult = details::allocateIntervals(std::move(intervals), unseen, kSessionAlignment);
     } else if (planner == MemoryPlanner::Linear) {
@@ -1363,9 +1371,14 @@ std::vector<std::array<uint32_t, 2>> GraphPipeline::liveRanges() const {
 
 void GraphPipeline::finalize(const bool enableFusion) {
     if (finalized) return;
+    const size_t recorded = ops.size();
     if (enableFusion) fuse();
     plan();
     finalized = true;
+    size_t launches = 0;
+    for (const auto &op : ops) launches += op->fusedAway ? 0 : 1;
+    MLEL_GRAPH_LOG(Info, "Graph pipeline created: " << recorded << " operators recorded, " << launches
+                                                    << " launches per dispatch, session memory " << sessionSize << " bytes");
 }
 
 void GraphPipeline::bindSessionMemory(void *deviceBase) {

@@ -1,6 +1,8 @@
 // SPIR-V assembly text or binary words -> GraphPipeline (see spirv_graph_loader.hpp).
 #include "spirv_graph_loader.hpp"
 
+#include "graph_log.hpp"
+
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -825,6 +827,12 @@ void Module::decodeTosa(const Instruction &inst) {
         return v[0];
     };
     const std::string dbg = inst.result.size() > 1 ? inst.result.substr(1) : name;
+    // one line per decoded instruction, as the reference's handlers print (graph_tosa_1_0_ext_inst.cpp:453-457)
+    MLEL_GRAPH_LOG(Info, "OpExtInst result=" << inst.result << ',' << dbg << ", " << name << [&] {
+        std::string list;
+        for (size_t i = 0; i < a.size(); i++) list += (i ? ", " : " ") + a[i];
+        return list;
+    }());
     if (name == "FFT2D" || name == "RFFT2D") {  // two results, picked apart by OpCompositeExtract
         const TensorPtr real = resultTensor(inst, 0), imag = resultTensor(inst, 1);
         if (name == "FFT2D") {

@@ -148,6 +148,16 @@ int mlel_graph_set_profiling(mlel_graph *g, int enabled);
 int mlel_graph_get_profiling(mlel_graph *g);
 int64_t mlel_graph_profiling_json(mlel_graph *g, char *buf, size_t capacity);
 
+/* The graph layer's log (reference: graphLog, graph/graph_log.cpp:19, common/log.cpp:29-87).  The environment variable
+ * VMEL_GRAPH_SEVERITY = Error | Warning | Info | Debug (case-insensitive, default Error) is read when the first message
+ * is considered; lines go to standard output as "<date> <time>,<ms> [Graph][<severity>] <text>".  Info: one line per
+ * decoded TOSA instruction (graph_tosa_1_0_ext_inst.cpp:453-457), the memory planner in use (graph_layer.cpp:286-295),
+ * a summary per created pipeline; Error: every failure a mlel_graph_* call reports; Debug: tensor creation
+ * (graph/tensor.cpp:90).  mlel_graph_log_level returns 0 .. 3 for Error .. Debug; mlel_graph_log_reload reads the
+ * variable again and returns the new level. */
+int mlel_graph_log_level(void);
+int mlel_graph_log_reload(void);
+
 /* Introspection (tests, profiler). */
 int mlel_graph_op_count(mlel_graph *g);        /* operators executed after fusion */
 int mlel_graph_op_name(mlel_graph *g, int index, char *buf, size_t len); /* "CONV2D+RESCALE+CLAMP", ... */

@@ -395,3 +395,66 @@ def test_elementwise_region_emits_an_absorbed_square_once():
     g = _build_host_only(spec, fuse=True)
     assert g.op_names() == ["ELEMENTWISE x3"]
     g.close()
+
+
+def test_graph_log_severity_from_environment(tmp_path):
+    """VMEL_GRAPH_SEVERITY as the reference reads it (common/log.cpp:29-71, graph/graph_log.cpp:19): unset or unknown
+    words mean Error, names compare without case; at Info the loader prints one line per decoded instruction
+    (graph_tosa_1_0_ext_inst.cpp:453-457), the planner in use (graph_layer.cpp:286-295) and a line per pipeline; failures
+    are Error lines.  Lines have the reference's shape: timestamp, logger name, severity."""
+    import os
+    import re
+    import subprocess
+    import sys
+
+    script = tmp_path / "log_probe.py"
+    script.write_text('''
+import importlib, os, sys
+sys.path.insert(0, os.environ["MLEL_REPO"])
+sys.path.insert(0, os.path.join(os.environ["MLEL_REPO"], "tests"))
+gb = importlib.import_module("ai-ml-emulation-layer-for-vulkan_amd.graph_backend")
+graphs = importlib.import_module("ai-ml-emulation-layer-for-vulkan_amd.graphs")
+import spvasm_writer
+lib = gb.load_graph_library()
+print("LEVEL", lib.mlel_graph_log_level(), flush=True)
+class NoDevice:
+    ctx = None
+    stream = None
+spec = graphs.inverted_residual_spec(batch=1, hw=8)
+w = spvasm_writer.from_spec(spec)
+g = gb.Graph(NoDevice())
+g.load_spvasm(w.text(), w.bindings, w.constants, w.names)
+g._check(g.lib.mlel_graph_finalize(g.g, 1))
+try:
+    gb.Graph(NoDevice()).load_spvasm("OpCapability Nonsense\\n%1 = OpBogus", [], [], [])
+except Exception as e:
+    print("RAISED", flush=True)
+''')
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+    def run(value):
+        env = dict(os.environ, MLEL_REPO=repo)
+        env.pop("VMEL_GRAPH_SEVERITY", None)
+        if value is not None:
+            env["VMEL_GRAPH_SEVERITY"] = value
+        out = subprocess.run([sys.executable, str(script)], env=env, capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        return out.stdout.splitlines()
+
+    line = re.compile(r"^\d{4}-\d\d-\d\d \d\d:\d\d:\d\d,\d{3} \[Graph\]\[(Error|Warning|Info|Debug)\] .+")
+    for value, level in ((None, 0), ("nonsense", 0), ("warning", 1), ("INFO", 2), ("Debug", 3)):
+        lines = run(value)
+        assert lines[0] == f"LEVEL {level}", (value, lines[:2])
+        logged = [l for l in lines if "[Graph][" in l]
+        assert all(line.match(l) for l in logged), logged[:3]
+        kinds = {line.match(l).group(1) for l in logged}
+        assert "RAISED" in lines
+        assert "Error" in kinds  # the refused module is reported at every level
+        if level < 2:
+            assert kinds == {"Error"}
+        else:
+            ops = [l for l in logged if "OpExtInst result=%" in l]
+            assert len(ops) == 12 and any("CONV2D" in l for l in ops) and any("RESCALE" in l for l in ops), ops[:3]
+            assert sum("Using interval memory planner" in l for l in logged) == 1
+            assert sum("Graph pipeline created: 12 operators recorded, 3 launches" in l for l in logged) == 1
+            assert ("Debug" in kinds) == (level == 3)
