@@ -258,6 +258,7 @@ FUSED_SIGNATURES = {
     "softmax_rows": [_T, _T],
     "elementwise_chain": [_T, C.POINTER(Chain)],
     "matmul_bias_cast_chain": [_T, _T, _T, _T, C.POINTER(MatmulAttr), C.POINTER(Chain)],
+    "attention_f16": [_T, _T, _T, _T, C.POINTER(Chain)],
     "rescale_add_rescale": [_T, _T, C.POINTER(Epilogue), _T, C.POINTER(Epilogue), C.POINTER(Epilogue)],
 }
 
@@ -290,6 +291,7 @@ RUNTIME_SIGNATURES = {
     "mlel_hip_graph_destroy": (C.c_int, [_V, _V]),
     "mlel_hip_copy_kernel": (C.c_int, [_V, _V, _V, _V, C.c_size_t]),
     "mlel_hip_matmul_chain_in_kernel": (C.c_int, [C.POINTER(Chain)]),
+    "mlel_hip_attention_f16_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Chain)]),
 }
 
 

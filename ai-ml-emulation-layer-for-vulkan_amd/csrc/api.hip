@@ -802,6 +802,37 @@ int mlel_hip_matmul_bias_cast_chain(mlel_ctx *ctx, void *stream, const mlel_tens
     return 0;
 }
 
+int mlel_hip_attention_f16(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *q,
+                           const mlel_tensor *kt, const mlel_tensor *v, const mlel_chain *softmax) {
+    MLEL_TRY(require_ctx(ctx, "attention_f16"));
+    MLEL_REQUIRE(softmax != nullptr, MLEL_ERR_INVALID, "attention_f16: null chain");
+    MLEL_REQUIRE(softmax->n_inputs >= 1 && softmax->n_inputs <= MLEL_CHAIN_MAX_INPUTS && softmax->n_steps >= 1 &&
+                     softmax->n_steps <= MLEL_CHAIN_MAX_STEPS,
+                 MLEL_ERR_INVALID, "attention_f16: %d inputs, %d steps", softmax->n_inputs, softmax->n_steps);
+    MLEL_TRY(check_supported(out, "attention_f16 out"));
+    MLEL_TRY(check_supported(q, "attention_f16 q"));
+    MLEL_TRY(check_supported(kt, "attention_f16 kt"));
+    MLEL_TRY(check_supported(v, "attention_f16 v"));
+    for (int i = 1; i < softmax->n_inputs; i++)  // input 0 is the first product
+        MLEL_TRY(check_supported(softmax->inputs[i], "attention_f16 chain input"));
+    const int rc = try_attention_f16(ctx, (hipStream_t)stream, out, q, kt, v, softmax);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    return set_error(MLEL_ERR_UNSUPPORTED,
+                     "attention_f16: fp16 heads of 64, M a multiple of 64, 64 <= S <= 512 in multiples of 64, dense "
+                     "16-byte aligned rows and the softmax chain only; run the three operators instead");
+}
+
+int mlel_hip_attention_f16_in_kernel(const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt,
+                                     const mlel_tensor *v, const mlel_chain *softmax) {
+    if (out == nullptr || q == nullptr || kt == nullptr || v == nullptr || softmax == nullptr) return 0;
+    if (softmax->n_inputs < 1 || softmax->n_inputs > MLEL_CHAIN_MAX_INPUTS || softmax->n_steps < 1 ||
+        softmax->n_steps > MLEL_CHAIN_MAX_STEPS)
+        return 0;
+    for (int i = 1; i < softmax->n_inputs; i++)
+        if (softmax->inputs[i] == nullptr) return 0;
+    return attention_f16_supported(out, q, kt, v, softmax) ? 1 : 0;
+}
+
 int mlel_hip_matmul_chain_in_kernel(const mlel_chain *chain) {
     return chain != nullptr && chain->n_inputs >= 1 && chain->n_inputs <= MLEL_CHAIN_MAX_INPUTS && chain->n_steps >= 1 &&
                    chain->n_steps <= MLEL_CHAIN_MAX_STEPS && chain_is_gelu_tanh(chain)

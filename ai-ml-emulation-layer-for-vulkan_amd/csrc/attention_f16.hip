@@ -1,0 +1,435 @@
+// Scores, softmax and the product with V of an fp16 attention head in one launch:
+//     S = CAST_f16( MATMUL(Q, K^T) )                      [NB, M, S]   (fp32 accumulate)
+//     P = softmax chain over the last axis of S           ([MUL by a scale,] REDUCE_MAX, SUB, EXP, REDUCE_SUM,
+//                                                           RECIPROCAL, MUL: every step rounded to fp16)
+//     O = CAST_f16( MATMUL(P, V) )                        [NB, M, 64]  (fp32 accumulate), optionally stored through the
+//                                                          six-dimensional view of a head merge
+// with every rounding of the three launches it replaces (the fp16 product of gemm_f16.hip, the compiled row program
+// of ops_float.hip, the product again), so the result is theirs bit for bit wherever it is a number.  S and P never
+// leave the chip: a block owns 64 query rows of one head and keeps their whole score rows in shared memory
+// (64 x (2 S + 16) bytes), K^T and V stream through one 10 KiB chunk buffer 64 keys at a time.
+//
+// Same arithmetic as the separate kernels, on purpose:
+//   * both products use v_mfma_f32_32x32x16_f16 with the K-major operand as the instruction's first operand and walk
+//     k in ascending order into one accumulator per output, which is the summation order of gemm_f16_kernel;
+//   * the elementwise steps are the shared static_apply<> functions on 16-byte pieces; REDUCE_MAX is exact;
+//     REDUCE_SUM is the reference's left-to-right fp16 fold (reduce.comp:24-70), here one lane per row: a single
+//     wavefront folds the block's 64 rows at once while the other three fetch the first chunk of V.
+#include "common.hpp"
+#include "dispatch.hpp"
+#include "float_programs.hpp"
+
+namespace mlel {
+namespace {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4s lds_v4s;
+
+constexpr uint32_t kOob = 0x80000000u;
+constexpr int kBlock = 256;
+constexpr int kRows = 64;       // query rows per block
+constexpr int kHead = 64;       // head size: K of the first product, N of the second
+constexpr int kChunk = 64;      // keys per chunk of K^T / V
+constexpr int kChunkPitch = 2 * kChunk + 32;  // bytes per K row of a chunk: 4 rows x 32 B land on distinct banks
+constexpr int kMaxKeys = 512;   // 16 pieces of 16 bytes per thread
+
+struct AttnArgs {
+    const char *q, *kt, *v;
+    char *out;
+    const uint16_t *scale;  // the chain's single-element fp16 input (SCALED), else unused
+    int32_t M, S, batches, strips;
+    int64_t q_batch, kt_batch, v_batch, o_batch;  // bytes
+    uint32_t ldq, ldkt, ldv, ldo;                 // bytes per row
+    uint32_t q_bytes, kt_bytes, v_bytes, o_bytes; // per-batch extents (all below 2^31)
+    // result written through a six-dimensional view [NB1, NB2, M1, M2, N1, N2] (see gemm_f16.hip); view == 0: plain
+    int32_t view, v_nb2, v_m2, v_n2;
+    int64_t vs_nb1, vs_nb2;
+    uint32_t vs_m1, vs_m2, vs_n1;
+    int32_t total, chunk;
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+    const v4i v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+    return make_uint4((uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w);
+}
+__device__ __forceinline__ v8h as_v8h(const uint4 &u) {
+    union {
+        uint4 u;
+        v8h h;
+    } c;
+    c.u = u;
+    return c.h;
+}
+
+template <bool SCALED>
+__global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g) {
+    extern __shared__ __align__(16) char smem[];
+    const int SP = g.S * 2 + 16;   // pitch of a score row (bytes): consecutive rows start four banks apart
+    char *st = smem;               // [64][SP]: S, then EXP(..), then P
+    char *cb = smem + kRows * SP;  // [64][kChunkPitch]: a chunk of K^T or V; the row sums; the staged result
+
+    const int lin = __builtin_amdgcn_readfirstlane((int)(blockIdx.x % 8u) * g.chunk + (int)(blockIdx.x / 8u));
+    if (lin >= g.total) return;
+    const int batch = lin / g.strips;
+    const int m0 = (lin - batch * g.strips) * kRows;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;  // the wavefront's 32 x 32 tile of a 64 x 64 product
+
+    const __amdgpu_buffer_rsrc_t qres = rsrc(g.q + (int64_t)batch * g.q_batch, g.q_bytes);
+    const __amdgpu_buffer_rsrc_t kres = rsrc(g.kt + (int64_t)batch * g.kt_batch, g.kt_bytes);
+    const __amdgpu_buffer_rsrc_t vres = rsrc(g.v + (int64_t)batch * g.v_batch, g.v_bytes);
+
+    // operand addresses inside a tile, as in gemm_f16_kernel: row operand: row = lane % 32, k group = lane / 32 (8 halfs);
+    // K-major operand: 16-lane group q = lane / 16 covers columns 16 (q & 1) .., k group q / 2; lane s = lane % 16
+    // points at row s / 4, columns 4 (s % 4) of the 4 x 16 block
+    const int a_row = lane & 31, a_kg = lane >> 5;
+    const int s16 = lane & 15, q16 = lane >> 4;
+    const int b_row = 8 * (q16 >> 1) + (s16 >> 2), b_col = 16 * (q16 & 1) + 4 * (s16 & 3);
+    const char *b_base = cb + b_row * kChunkPitch + (wn * 32 + b_col) * 2;
+    auto b_frag = [&](int kk) {
+        const char *p = b_base + kk * 16 * kChunkPitch;
+        const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)p);
+        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)(p + 4 * kChunkPitch));
+        union {
+            v4s s[2];
+            v8h h;
+        } u;
+        u.s[0] = lo;
+        u.s[1] = hi;
+        return u.h;
+    };
+    // a chunk is 64 rows of 128 bytes: two 16-byte pieces per thread
+    const int c_row = tid >> 2, c_piece = (tid & 3) * 2;
+    auto chunk_store = [&](const uint4 (&r)[2]) {
+        *reinterpret_cast<uint4 *>(cb + c_row * kChunkPitch + c_piece * 16) = r[0];
+        *reinterpret_cast<uint4 *>(cb + c_row * kChunkPitch + c_piece * 16 + 16) = r[1];
+    };
+
+    // ---- phase 1: S = fp16(Q K^T), 64 keys at a time.  The query rows of this wavefront are matrix operands in registers.
+    v8h qf[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++)
+        qf[kk] = as_v8h(load16(qres, (uint32_t)(m0 + wm * 32 + a_row) * g.ldq + (uint32_t)(kk * 16 + a_kg * 8) * 2));
+    const int nchunks = g.S / kChunk;
+    uint4 cr[2];
+    auto fetch_kt = [&](int c) {  // rows = k (the head dimension), columns = the chunk's keys
+        const uint32_t off = (uint32_t)c_row * g.ldkt + (uint32_t)(c * kChunk + c_piece * 8) * 2;
+        cr[0] = load16(kres, c < nchunks ? off : kOob);
+        cr[1] = load16(kres, c < nchunks ? off + 16 : kOob);
+    };
+    auto fetch_v = [&](int c) {  // rows = the chunk's keys, columns = the head dimension
+        const uint32_t off = (uint32_t)(c * kChunk + c_row) * g.ldv + (uint32_t)(c_piece * 8) * 2;
+        cr[0] = load16(vres, c < nchunks ? off : kOob);
+        cr[1] = load16(vres, c < nchunks ? off + 16 : kOob);
+    };
+    fetch_kt(0);
+    for (int c = 0; c < nchunks; c++) {
+        __syncthreads();  // every wavefront has read the previous chunk
+        chunk_store(cr);
+        __syncthreads();
+        fetch_kt(c + 1);
+        v16f acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag(kk), qf[kk], acc, 0, 0, 0);
+        // lane holds row lane % 32 of the tile and, per register quad q, columns 8 q + 4 (lane / 32) .. + 3
+        char *srow = st + (wm * 32 + (lane & 31)) * SP + (c * kChunk + wn * 32 + 4 * (lane >> 5)) * 2;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            _Float16 h[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) h[e] = (_Float16)acc[4 * q + e];  // CAST: round to nearest even
+            uint2 w;
+            w.x = (uint32_t)__builtin_bit_cast(unsigned short, h[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[1]) << 16);
+            w.y = (uint32_t)__builtin_bit_cast(unsigned short, h[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[3]) << 16);
+            *reinterpret_cast<uint2 *>(srow + q * 16) = w;
+        }
+    }
+    __syncthreads();
+
+    // ---- phase 2: the softmax chain.  Four threads share a row (pieces quarter, quarter + 4, ...); the chain's full
+    // values stay in registers.
+    const int row = tid >> 2, quarter = tid & 3;
+    const int ppt = g.S >> 5;  // pieces per thread: S / 8 / 4, at most 16
+    char *myrow = st + row * SP;
+    uint4 val[kMaxKeys / 32];
+    uint32_t scale_w = 0;
+    if (SCALED) {
+        const uint32_t bits = *g.scale;
+        scale_w = bits | (bits << 16);
+    }
+    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+    h2_t m2 = {(_Float16)-65504.f, (_Float16)-65504.f};
+    uint32_t special = 0;
+#pragma unroll
+    for (int u = 0; u < kMaxKeys / 32; u++) {
+        if (u < ppt) {
+            uint4 x = *reinterpret_cast<const uint4 *>(myrow + (quarter + 4 * u) * 16);
+            if (SCALED) {
+                x = static_apply<F_MUL>(x, make_uint4(scale_w, scale_w, scale_w, scale_w));
+                asm volatile("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));
+            }
+            val[u] = x;
+            // REDUCE_MAX: exact; a NaN or an infinity anywhere in the row makes the maximum a NaN (as the row program)
+            special |= (((x.x & 0x7fff7fffu) + 0x03ff03ffu) | ((x.y & 0x7fff7fffu) + 0x03ff03ffu) |
+                        ((x.z & 0x7fff7fffu) + 0x03ff03ffu) | ((x.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
+            const h2_t *p = reinterpret_cast<const h2_t *>(&x);
+            m2 = __builtin_elementwise_max(m2, __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]),
+                                                                           __builtin_elementwise_max(p[2], p[3])));
+        }
+    }
+    float mx = (float)(m2.x > m2.y ? m2.x : m2.y);
+#pragma unroll
+    for (int d = 1; d < 4; d <<= 1) {
+        mx = fmaxf(mx, __shfl_xor(mx, d));
+        special |= (uint32_t)__shfl_xor((int)special, d);
+    }
+    const uint32_t mbits = (uint32_t)__half_as_ushort(f2h(special != 0 ? __builtin_nanf("") : mx));
+    const uint4 mrow = make_uint4(mbits | (mbits << 16), mbits | (mbits << 16), mbits | (mbits << 16), mbits | (mbits << 16));
+#pragma unroll
+    for (int u = 0; u < kMaxKeys / 32; u++) {
+        if (u < ppt) {
+            uint4 d = static_apply<F_SUB>(val[u], mrow);
+            asm volatile("" : "+v"(d.x), "+v"(d.y), "+v"(d.z), "+v"(d.w));
+            uint4 e = static_apply<F_EXP>(d, d);
+            asm volatile("" : "+v"(e.x), "+v"(e.y), "+v"(e.z), "+v"(e.w));
+            val[u] = e;
+            *reinterpret_cast<uint4 *>(myrow + (quarter + 4 * u) * 16) = e;  // for the fold
+        }
+    }
+    __syncthreads();
+    // REDUCE_SUM: left to right in fp16, one lane per row; meanwhile the other wavefronts request the first chunk of V
+    uint16_t *sums = reinterpret_cast<uint16_t *>(cb);  // [64]
+    if (wave == 0) {
+        const char *r = st + lane * SP;
+        __half acc = f2h(0.f);
+        const int segs = g.S >> 3;
+        uint4 cur = *reinterpret_cast<const uint4 *>(r);
+        for (int sg = 0; sg < segs; sg++) {
+            const uint4 nxt = *reinterpret_cast<const uint4 *>(r + (sg + 1 < segs ? sg + 1 : sg) * 16);
+            const __half2 *h = reinterpret_cast<const __half2 *>(&cur);
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                acc = __hadd(acc, __low2half(h[t]));
+                acc = __hadd(acc, __high2half(h[t]));
+            }
+            cur = nxt;
+        }
+        sums[lane] = __half_as_ushort(acc);
+    }
+    fetch_v(0);
+    __syncthreads();
+    {
+        const uint32_t sbits = sums[row];
+        const uint32_t sw = sbits | (sbits << 16);
+        uint4 rc = static_apply<F_RECIPROCAL>(make_uint4(sw, sw, sw, sw), make_uint4(sw, sw, sw, sw));
+        asm volatile("" : "+v"(rc.x));
+        const uint4 rrow = make_uint4(rc.x, rc.x, rc.x, rc.x);
+#pragma unroll
+        for (int u = 0; u < kMaxKeys / 32; u++) {
+            if (u < ppt) {
+                uint4 p = static_apply<F_MUL>(val[u], rrow);
+                asm volatile("" : "+v"(p.x), "+v"(p.y), "+v"(p.z), "+v"(p.w));
+                *reinterpret_cast<uint4 *>(myrow + (quarter + 4 * u) * 16) = p;
+            }
+        }
+    }
+
+    // ---- phase 3: O = fp16(P V), 64 keys at a time
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    const char *p_base = st + (wm * 32 + a_row) * SP + a_kg * 16;
+    for (int c = 0; c < nchunks; c++) {
+        __syncthreads();  // the previous chunk (or the row sums) has been read; P is complete
+        chunk_store(cr);
+        __syncthreads();
+        fetch_v(c + 1);
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            const v8h pf = *reinterpret_cast<const v8h *>(p_base + (c * kChunk + kk * 16) * 2);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag(kk), pf, acc, 0, 0, 0);
+        }
+    }
+    __syncthreads();
+    // the 64 x 64 result through shared memory, so that it leaves in 16-byte pieces (whole 128-byte rows)
+    constexpr int OP = kHead * 2 + 16;
+    {
+        char *orow = cb + (wm * 32 + (lane & 31)) * OP + (wn * 32 + 4 * (lane >> 5)) * 2;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            _Float16 h[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) h[e] = (_Float16)acc[4 * q + e];
+            uint2 w;
+            w.x = (uint32_t)__builtin_bit_cast(unsigned short, h[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[1]) << 16);
+            w.y = (uint32_t)__builtin_bit_cast(unsigned short, h[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[3]) << 16);
+            *reinterpret_cast<uint2 *>(orow + q * 16) = w;
+        }
+    }
+    __syncthreads();
+    const int64_t o_base = g.view ? (int64_t)(batch / g.v_nb2) * g.vs_nb1 + (int64_t)(batch % g.v_nb2) * g.vs_nb2
+                                  : (int64_t)batch * g.o_batch;
+    const __amdgpu_buffer_rsrc_t ores = rsrc(g.out + o_base, g.o_bytes);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int p = i * kBlock + tid, r = p >> 3, c8 = p & 7;
+        const int m = m0 + r, n = c8 * 8;
+        const uint4 piece = *reinterpret_cast<const uint4 *>(cb + r * OP + c8 * 16);
+        uint32_t off = (uint32_t)m * g.ldo + (uint32_t)n * 2;
+        if (g.view)  // uniform
+            off = (uint32_t)(m / g.v_m2) * g.vs_m1 + (uint32_t)(m % g.v_m2) * g.vs_m2 + (uint32_t)(n / g.v_n2) * g.vs_n1 +
+                  (uint32_t)(n % g.v_n2) * 2;
+        v4i v;
+        v.x = (int)piece.x, v.y = (int)piece.y, v.z = (int)piece.z, v.w = (int)piece.w;
+        __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
+    }
+}
+
+bool dense_rows(const mlel_tensor *t) { return t->strides[2] == 2 && t->strides[1] >= t->dims[2] * 2; }
+bool aligned16(const mlel_tensor *t, bool with_ptr) {
+    return (!with_ptr || ((uintptr_t)t->ptr % 16) == 0) && t->strides[0] % 16 == 0 && t->strides[1] % 16 == 0;
+}
+
+// 0: the softmax chain without a scale, 1: with a scale in front, -1: another chain
+int softmax_form(const mlel_chain *c) {
+    if (c == nullptr) return -1;
+    struct Want {
+        int kind, selector, a, b;
+    };
+    static const Want plain[6] = {{MLEL_CHAIN_REDUCE, MLEL_RED_MAX, 0, 0},       {MLEL_CHAIN_BINARY, MLEL_BIN_SUB, 0, 1},
+                                  {MLEL_CHAIN_UNARY, MLEL_UN_EXP, 2, 0},         {MLEL_CHAIN_REDUCE, MLEL_RED_SUM, 3, 0},
+                                  {MLEL_CHAIN_UNARY, MLEL_UN_RECIPROCAL, 4, 0}, {MLEL_CHAIN_MUL, 0, 3, 5}};
+    const int scaled = c->n_inputs == 2 && c->n_steps == 7 ? 1 : (c->n_inputs == 1 && c->n_steps == 6 ? 0 : -1);
+    if (scaled < 0) return -1;
+    if (scaled) {
+        const mlel_chain_step &s = c->steps[0];
+        if (s.kind != MLEL_CHAIN_MUL || s.a != 0 || s.b != 1 || s.dtype != MLEL_F16) return -1;
+        const mlel_tensor *k = c->inputs[1];
+        if (k == nullptr || k->dtype != MLEL_F16 || numel(k) != 1) return -1;
+    }
+    // with a scale every value index moves up by two: one more input, one more step
+    for (int i = 0; i < 6; i++) {
+        const mlel_chain_step &s = c->steps[i + scaled];
+        const Want &w = plain[i];
+        const auto shifted = [&](int v) { return scaled ? v + 2 : v; };
+        const bool two = w.kind == MLEL_CHAIN_BINARY || w.kind == MLEL_CHAIN_MUL;
+        if (s.kind != w.kind || s.dtype != MLEL_F16 || s.a != shifted(w.a) || (two && s.b != shifted(w.b))) return -1;
+        if (w.kind != MLEL_CHAIN_MUL && s.selector != w.selector) return -1;
+    }
+    return scaled;
+}
+
+// 1 when the three operators are a case for the kernel; `with_pointers`: also check the base addresses
+int describe(const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt, const mlel_tensor *v,
+             const mlel_chain *chain, bool with_pointers, AttnArgs *filled) {
+    const int form = softmax_form(chain);
+    if (form < 0) return 0;
+    if (q->dtype != MLEL_F16 || kt->dtype != MLEL_F16 || v->dtype != MLEL_F16 || out->dtype != MLEL_F16) return 0;
+    if (q->rank != 3 || kt->rank != 3 || v->rank != 3 || (out->rank != 3 && out->rank != 6)) return 0;
+    const int64_t NB = q->dims[0], M = q->dims[1], S = kt->dims[2];
+    if (q->dims[2] != kHead || kt->dims[0] != NB || kt->dims[1] != kHead || v->dims[0] != NB || v->dims[1] != S ||
+        v->dims[2] != kHead)
+        return 0;
+    if (NB <= 0 || M <= 0 || M % kRows != 0 || S < kChunk || S > kMaxKeys || S % kChunk != 0) return 0;
+    if (!dense_rows(q) || !dense_rows(kt) || !dense_rows(v)) return 0;
+    if (!aligned16(q, with_pointers) || !aligned16(kt, with_pointers) || !aligned16(v, with_pointers)) return 0;
+    const int64_t lim = (int64_t(1) << 31) - 64;
+    const int64_t qb = M * q->strides[1], kb = kHead * kt->strides[1], vb = S * v->strides[1];
+    if (qb >= lim || kb >= lim || vb >= lim || NB * (M / kRows) >= (int64_t(1) << 30)) return 0;
+    AttnArgs g{};
+    if (out->rank == 3) {
+        if (out->dims[0] != NB || out->dims[1] != M || out->dims[2] != kHead || out->strides[2] != 2) return 0;
+        if (!aligned16(out, with_pointers) || M * out->strides[1] >= lim || out->strides[1] < kHead * 2) return 0;
+        g.o_batch = out->strides[0];
+        g.ldo = (uint32_t)out->strides[1];
+        g.o_bytes = (uint32_t)(M * out->strides[1]);
+    } else {
+        // [NB1, NB2, M1, M2, N1, N2] with eight consecutive n2 contiguous
+        if (out->dims[0] * out->dims[1] != NB || out->dims[2] * out->dims[3] != M || out->dims[4] * out->dims[5] != kHead) return 0;
+        if (out->strides[5] != 2 || out->dims[5] % 8 != 0) return 0;
+        if (with_pointers && ((uintptr_t)out->ptr % 16) != 0) return 0;
+        int64_t span = 16;
+        for (int i = 0; i < 6; i++) {
+            if (i != 5 && (out->strides[i] % 16 != 0 || out->strides[i] < 0)) return 0;
+            if (i >= 2) span += (out->dims[i] - 1) * out->strides[i];
+        }
+        if (span >= lim) return 0;
+        g.view = 1;
+        g.v_nb2 = (int32_t)out->dims[1];
+        g.v_m2 = (int32_t)out->dims[3];
+        g.v_n2 = (int32_t)out->dims[5];
+        g.vs_nb1 = out->strides[0];
+        g.vs_nb2 = out->strides[1];
+        g.vs_m1 = (uint32_t)out->strides[2];
+        g.vs_m2 = (uint32_t)out->strides[3];
+        g.vs_n1 = (uint32_t)out->strides[4];
+        g.o_bytes = (uint32_t)span;
+    }
+    g.q = static_cast<const char *>(q->ptr);
+    g.kt = static_cast<const char *>(kt->ptr);
+    g.v = static_cast<const char *>(v->ptr);
+    g.out = static_cast<char *>(out->ptr);
+    g.scale = form == 1 ? static_cast<const uint16_t *>(chain->inputs[1]->ptr) : nullptr;
+    if (with_pointers && form == 1 && (g.scale == nullptr || ((uintptr_t)g.scale % 2) != 0)) return 0;
+    g.M = (int32_t)M;
+    g.S = (int32_t)S;
+    g.batches = (int32_t)NB;
+    g.strips = (int32_t)(M / kRows);
+    g.q_batch = q->strides[0];
+    g.kt_batch = kt->strides[0];
+    g.v_batch = v->strides[0];
+    g.ldq = (uint32_t)q->strides[1];
+    g.ldkt = (uint32_t)kt->strides[1];
+    g.ldv = (uint32_t)v->strides[1];
+    g.q_bytes = (uint32_t)qb;
+    g.kt_bytes = (uint32_t)kb;
+    g.v_bytes = (uint32_t)vb;
+    g.total = (int32_t)(NB * (M / kRows));
+    g.chunk = (g.total + 7) / 8;
+    if (filled != nullptr) *filled = g;
+    return form == 1 ? 2 : 1;
+}
+
+}  // namespace
+
+bool attention_f16_supported(const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt, const mlel_tensor *v,
+                             const mlel_chain *chain) {
+    return describe(out, q, kt, v, chain, false, nullptr) != 0;
+}
+
+int try_attention_f16(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt,
+                      const mlel_tensor *v, const mlel_chain *chain) {
+    (void)ctx;
+    AttnArgs g{};
+    const int form = describe(out, q, kt, v, chain, true, &g);
+    if (form == 0) return 0;
+    const size_t sm = (size_t)kRows * (g.S * 2 + 16) + (size_t)kChunk * kChunkPitch;
+    const dim3 grid((unsigned)(g.chunk * 8));
+    if (form == 2) {
+        auto kernel = attention_f16_kernel<true>;
+        static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                       kRows * (kMaxKeys * 2 + 16) + kChunk * kChunkPitch) == hipSuccess;
+        (void)raised;
+        kernel<<<grid, dim3(kBlock), sm, s>>>(g);
+    } else {
+        auto kernel = attention_f16_kernel<false>;
+        static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                       kRows * (kMaxKeys * 2 + 16) + kChunk * kChunkPitch) == hipSuccess;
+        (void)raised;
+        kernel<<<grid, dim3(kBlock), sm, s>>>(g);
+    }
+    MLEL_TRY(check_launch("attention fp16"));
+    return 1;
+}
+
+}  // namespace mlel

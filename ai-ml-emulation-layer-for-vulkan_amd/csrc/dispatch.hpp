@@ -129,6 +129,12 @@ bool chain_is_gelu_tanh(const mlel_chain *chain);
 int try_matmul_f16_group(mlel_ctx *ctx, hipStream_t s, int n, const mlel_tensor *const *outs, const mlel_tensor *a,
                          const mlel_tensor *const *bs, const mlel_tensor *const *biases, const mlel_matmul_attr *attr);
 
+// ---- scores, softmax and the product with V of fp16 attention heads in one launch (attention_f16.hip) ----
+bool attention_f16_supported(const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt, const mlel_tensor *v,
+                             const mlel_chain *chain);
+int try_attention_f16(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt,
+                      const mlel_tensor *v, const mlel_chain *chain);
+
 // ---- floating-point elementwise / reduce specialisations (ops_float.hip) ----
 int try_binary_float_fast(mlel_ctx *ctx, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in1,
                           const mlel_tensor *in2);

@@ -310,6 +310,9 @@ std::string opLabel(const OpNode &op) {
                     (view.first[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");
         return name;
     }
+    case OpKind::FusedAttention:
+        return std::string("MATMUL+CAST+ELEMENTWISE+REDUCE x") + std::to_string(op.chain.size()) + "+MATMUL+CAST" +
+               (op.viewDims[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");
     default: return op.tosaName;
     }
 }

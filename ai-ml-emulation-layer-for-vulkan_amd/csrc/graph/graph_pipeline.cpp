@@ -1169,6 +1169,61 @@ void GraphPipeline::fuse() {
         ew->fusedAway = true;
     }
 
+    // Pattern 7 (attention): a fused fp16 product (no bias, view, residual, group or chain) whose private result is
+    // read only by a fused region as its value 0, the region being the softmax chain over the last axis
+    // (mlel_hip_attention_f16_in_kernel decides), and the region's private result read only as the first operand of
+    // another such product (which may carry the view of a head merge): the three become one launch that keeps the
+    // scores on the chip (mlel_hip_attention_f16), bit for bit the three launches.
+    for (const auto &opPtr : ops) {
+        OpNode &sm = *opPtr;
+        if (sm.fusedAway || sm.kind != OpKind::FusedElementwise || sm.inputs.empty() || sm.inputs.size() > 4) continue;
+        const TensorPtr scores = sm.inputs[0];
+        OpNode *first = scores->getProducer();
+        const auto plainProduct = [](const OpNode *mm) {
+            return mm != nullptr && !mm->fusedAway && mm->kind == OpKind::FusedMatmulBiasCast && !mm->hasBias && !mm->flag &&
+                   mm->extraProductViews.empty() && mm->chain.empty();
+        };
+        if (!plainProduct(first) || first->viewDims[5] != 0 || !isPrivateIntermediate(*scores)) continue;
+        const auto scoreUsers = consumersOf(ops, scores.get());
+        if (scoreUsers.size() != 1 || scoreUsers[0] != &sm) continue;
+        const TensorPtr prob = sm.outputs[0];
+        if (!isPrivateIntermediate(*prob) || !sameShape(*prob, *scores)) continue;
+        const auto probUsers = consumersOf(ops, prob.get());
+        if (probUsers.size() != 1 || !plainProduct(probUsers[0])) continue;
+        OpNode *second = probUsers[0];
+        if (second->inputs[0].get() != prob.get() || second->inputs[1].get() == prob.get()) continue;
+        bool ok = true;
+        for (size_t i = 1; i < sm.inputs.size(); i++)
+            ok = ok && sm.inputs[i].get() != scores.get() && sm.inputs[i]->getProducer() == nullptr;
+        if (!ok || sm.chain.size() > MLEL_CHAIN_MAX_STEPS) continue;
+        std::array<mlel_tensor, MLEL_CHAIN_MAX_INPUTS> described{};
+        mlel_chain query{};
+        query.n_inputs = static_cast<int32_t>(sm.inputs.size());
+        query.n_steps = static_cast<int32_t>(sm.chain.size());
+        for (size_t i = 1; i < sm.inputs.size(); i++) {
+            described[i] = sm.inputs[i]->view();
+            query.inputs[i] = &described[i];
+        }
+        for (size_t i = 0; i < sm.chain.size(); i++) query.steps[i] = sm.chain[i];
+        const mlel_tensor q = first->inputs[0]->view(), kt = first->inputs[1]->view(), v = second->inputs[1]->view();
+        mlel_tensor out = second->outputs[0]->view();
+        if (second->viewDims[5] != 0) {
+            out.rank = 6;
+            for (size_t k = 0; k < 6; k++) {
+                out.dims[k] = second->viewDims[k];
+                out.strides[k] = second->viewStrides[k];
+            }
+        }
+        if (mlel_hip_attention_f16_in_kernel(&out, &q, &kt, &v, &query) == 0) continue;
+        const TensorPtr qT = first->inputs[0], ktT = first->inputs[1], vT = second->inputs[1];
+        second->kind = OpKind::FusedAttention;
+        second->inputs = {qT, ktT, vT};
+        for (size_t i = 1; i < sm.inputs.size(); i++) second->inputs.push_back(sm.inputs[i]);
+        second->chain = sm.chain;
+        first->fusedAway = true;
+        sm.fusedAway = true;
+    }
+
     // Pattern 3: RESHAPE between two packed session tensors of the same byte size moves no data (the reference's
     // reshape.comp:16-27 copies by flat index): the output becomes a second view of the input's storage and the
     // operator is not executed.  plan() gives both tensors one allocation that lives as long as either is used.
@@ -1611,6 +1666,24 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
         } else {
             rc = mlel_hip_matmul_bias_cast(ctx, stream, &out, &in[0], &in[1], bias, &op.matmul);
         }
+        break;
+    }
+    case OpKind::FusedAttention: {
+        mlel_chain c{};
+        c.n_inputs = static_cast<int32_t>(op.inputs.size() - 3 + 1);  // q, kt, v, then the chain's inputs from 1 on
+        c.n_steps = static_cast<int32_t>(op.chain.size());
+        c.inputs[0] = nullptr;
+        for (size_t i = 3; i < op.inputs.size(); i++) c.inputs[i - 3 + 1] = &in[i];
+        for (size_t i = 0; i < op.chain.size(); i++) c.steps[i] = op.chain[i];
+        mlel_tensor view = out;
+        if (op.viewDims[5] != 0) {
+            view.rank = 6;
+            for (size_t k = 0; k < 6; k++) {
+                view.dims[k] = op.viewDims[k];
+                view.strides[k] = op.viewStrides[k];
+            }
+        }
+        rc = mlel_hip_attention_f16(ctx, stream, &view, &in[0], &in[1], &in[2], &c);
         break;
     }
     case OpKind::FusedConv2DResidual: {

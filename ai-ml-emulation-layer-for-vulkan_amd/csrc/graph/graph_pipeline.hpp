@@ -98,7 +98,7 @@ enum class OpKind {
     Argmax, ArithmeticRightShift, Conv3D, TransposeConv2D, Fft2D, Rfft2D, Gather, Scatter, Resize, Reverse, Tile, Select,
     // produced by the fusion pass only
     FusedConv2D, FusedDepthwiseConv2D, FusedMatmul, FusedRescaleAddRescale, FusedMatmulBiasCast, FusedElementwise,
-    FusedConv2DResidual,
+    FusedConv2DResidual, FusedAttention,
 };
 
 struct RescaleSpec {
@@ -144,6 +144,8 @@ class OpNode {
     // appended for it (its B, then its bias when hasBias), writes outputs[k], through the view k - 1 of this list
     // when that view's extents are non-zero
     std::vector<std::pair<std::array<int64_t, 6>, std::array<int64_t, 6>>> extraProductViews;
+    // FusedAttention: inputs = {q, kt, v, the softmax chain's inputs from 1 on}; `chain` is the softmax region between
+    // the two products (its value 0 is the first product); viewDims / viewStrides as for FusedMatmulBiasCast
     RescaleSpec scaleA, scaleB;      // FusedRescaleAddRescale: the two input stages (epilogue = output stage)
     // FusedConv2DResidual: epilogue (+ clamp) belongs to the convolution; scaleA rescales its 8-bit result, scaleB the
     // residual (inputs[3]), scaleOut their sum; `flag` is set when the residual was the addition's first operand

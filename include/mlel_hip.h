@@ -497,6 +497,22 @@ int mlel_hip_matmul_bias_cast_chain(mlel_ctx *ctx, void *stream, const mlel_tens
  * has no fused operators. */
 int mlel_hip_matmul_chain_in_kernel(const mlel_chain *chain);
 
+/* out(fp16) = CAST( MATMUL( softmax( CAST( MATMUL(q, kt) ) ), v ) ) for fp16 attention heads of 64: q [NB, M, 64],
+ * kt [NB, 64, S], v [NB, S, 64], out [NB, M, 64] or a rank-6 view of it as in mlel_hip_matmul_bias_cast.  `softmax` is
+ * the chain between the two products as a TOSA graph spells it (REDUCE_MAX, SUB, EXP, REDUCE_SUM, RECIPROCAL, MUL over
+ * the last axis, optionally a MUL by a single-element scale in front; its input 0 is the first product and may be
+ * NULL).  One launch that keeps the scores on the chip; bit for bit mlel_hip_matmul_bias_cast, mlel_hip_elementwise_chain
+ * and mlel_hip_matmul_bias_cast one after another wherever the result is a number (rows that meet a NaN or an infinity
+ * are NaN in both).  M a multiple of 64, S a multiple of 64 up to 512, dense 16-byte aligned rows; anything else is
+ * MLEL_ERR_UNSUPPORTED (nothing is allocated and nothing falls back).  Replaces three of the reference's dispatches
+ * (matmul.comp, the elementwise / reduce shaders of the softmax, matmul.comp); it has no single counterpart there. */
+int mlel_hip_attention_f16(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *q,
+                           const mlel_tensor *kt, const mlel_tensor *v, const mlel_chain *softmax);
+/* 1 when mlel_hip_attention_f16 takes these operands, judged by types, extents, strides and the chain's steps only
+ * (data pointers are not looked at; no device is touched), else 0. */
+int mlel_hip_attention_f16_in_kernel(const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt,
+                                     const mlel_tensor *v, const mlel_chain *softmax);
+
 /* Plain device-to-device copy kernel of `bytes` bytes with 128-bit accesses; the calibration kernel for
  * memory-traffic counters and the measured HBM ceiling. */
 int mlel_hip_copy_kernel(mlel_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes);

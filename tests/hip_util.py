@@ -297,6 +297,34 @@ class Runner:
         self.done()
         return r
 
+    def attention(self, q, kt, v, chain_inputs, steps, split_shape=None, perms=None):
+        """mlel_hip_attention_f16: `chain_inputs` are the softmax chain's inputs from 1 on (the scale, if any);
+        with split_shape / perms the result goes through the view of a RESHAPE -> TRANSPOSE behind it."""
+        tq, tk, tv = self.put(q), self.put(kt), self.put(v)
+        tin = [self.put(x) for x in chain_inputs]
+        c = abi.Chain()
+        c.n_inputs, c.n_steps = len(tin) + 1, len(steps)
+        for i, t in enumerate(tin):
+            c.inputs[i + 1] = C.pointer(t.view)
+        for i, st in enumerate(steps):
+            c.steps[i] = abi.ChainStep(*[int(x) for x in st])
+        shape = (q.shape[0], q.shape[1], v.shape[2])
+        if split_shape is None:
+            to = self.new(abi.F16, shape)
+            self.dev.op("attention_f16", to.ref, tq.ref, tk.ref, tv.ref, C.byref(c))
+        else:
+            moved_shape = tuple(split_shape[p] for p in perms)
+            to = self.new(abi.F16, moved_shape)
+            moved_strides = abi.packed_strides(moved_shape, 2)
+            strides = [0] * 6
+            for k, p in enumerate(perms):
+                strides[p] = moved_strides[k]
+            view = abi.make_tensor(to.view.ptr, abi.F16, split_shape, strides)
+            self.dev.op("attention_f16", C.byref(view), tq.ref, tk.ref, tv.ref, C.byref(c))
+        r = to.download()
+        self.done()
+        return r
+
     def chain(self, inputs, steps, out_shape, out_dtype):
         """steps: (kind, selector, a, b, dtype) tuples as in mlel_chain_step."""
         tin = [self.put(x) for x in inputs]

@@ -296,6 +296,28 @@ def test_transformer_block_fused_operator_list():
     g.close()
 
 
+def test_attention_fusion_on_heads_of_64():
+    """Scores, softmax and the product with V become one launch when the heads are 64 wide and the key count is a
+    multiple of 64 up to 512 (config 4: seven launches); other head sizes or key counts keep the three launches."""
+    three = " | ".join(["MATMUL+ADD+CAST+RESHAPE+TRANSPOSE"] * 3)
+    attention = "MATMUL+CAST+ELEMENTWISE+REDUCE x7+MATMUL+CAST+RESHAPE+TRANSPOSE"
+    fused = ["ELEMENTWISE+REDUCE x11", three, attention, "MATMUL+ADD+CAST+ADD", "ELEMENTWISE+REDUCE x11",
+             "MATMUL+ADD+CAST+ELEMENTWISE x9", "MATMUL+ADD+CAST+ADD"]
+    g = _build_host_only(graphs.transformer_block_spec(), fuse=True)
+    assert g.op_names() == fused
+    g.close()
+    g = _build_host_only(graphs.transformer_block_spec(batch=1, seq=128, d_model=128, heads=2, ffn=256), fuse=True)
+    assert attention in g.op_names() and "ELEMENTWISE+REDUCE x7" not in g.op_names()
+    g.close()
+    for kwargs in (dict(batch=1, seq=576, d_model=128, heads=2, ffn=256),   # 576 keys
+                   dict(batch=1, seq=96, d_model=128, heads=2, ffn=256),    # 96 keys and query rows
+                   dict(batch=1, seq=128, d_model=128, heads=4, ffn=256)):  # heads of 32
+        g = _build_host_only(graphs.transformer_block_spec(**kwargs), fuse=True)
+        names = g.op_names()
+        assert attention not in names and "ELEMENTWISE+REDUCE x7" in names, kwargs
+        g.close()
+
+
 def test_projection_patterns_leave_observable_or_mismatched_cases_alone():
     """Residual, grouping and view fusions behind fp16 products apply only when nothing else can observe the product's
     result and the shapes fit."""

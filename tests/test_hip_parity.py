@@ -418,6 +418,62 @@ def test_matmul_bias_cast_through_a_view(run):
         np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16), err_msg=str(split))
 
 
+ATTENTION_CASES = [  # heads, queries, keys, scaled, head-merge view
+    (3, 64, 64, True, False),
+    (2, 128, 512, True, False),
+    (5, 192, 320, False, False),
+    (2 * 3, 64, 128, True, True),
+]
+
+
+@pytest.mark.parametrize("case", ATTENTION_CASES, ids=[f"h{c[0]}_m{c[1]}_s{c[2]}_{'scaled' if c[3] else 'plain'}{'_view' if c[4] else ''}"
+                                                       for c in ATTENTION_CASES])
+def test_attention_equals_the_three_launches(run, case):
+    """mlel_hip_attention_f16 against the launches it replaces: the fp16 product QK^T, the softmax chain over its rows,
+    the fp16 product with V (optionally written through a head-merge view) -- the same bits."""
+    nb, m, s, scaled, view = case
+    rng = np.random.default_rng(zlib.crc32(repr(case).encode()))
+    q = rng.standard_normal((nb, m, 64)).astype(np.float16)
+    kt = rng.standard_normal((nb, 64, s)).astype(np.float16)
+    v = rng.standard_normal((nb, s, 64)).astype(np.float16)
+    Bk, Mk, Uk, Rk = 0, 1, 2, 4  # step kinds: binary, mul, unary, reduce
+    f16 = abi.F16
+    o = 2 if scaled else 0  # with a scale every value index moves up by two
+    steps = [(Rk, abi.RED["MAX"], o, 0, f16), (Bk, abi.BIN["SUB"], o, o + 1, f16), (Uk, abi.UN["EXP"], o + 2, 0, f16),
+             (Rk, abi.RED["SUM"], o + 3, 0, f16), (Uk, abi.UN["RECIPROCAL"], o + 4, 0, f16), (Mk, 0, o + 3, o + 5, f16)]
+    extra = []
+    if scaled:
+        steps = [(Mk, 0, 0, 1, f16)] + steps
+        extra = [np.array(0.125, np.float16).reshape(1, 1, 1)]
+    scores = run.matmul_bias_cast(q, kt, None)
+    prob = run.chain([scores] + extra, steps, scores.shape, f16)
+    assert np.isfinite(prob.astype(np.float32)).all() and len(np.unique(prob)) > 100
+    want = run.matmul_bias_cast(prob, v, None)
+    if view:
+        split, perms = (2, 3, m, 1, 1, 64), (0, 2, 3, 1, 4, 5)  # [B, H, S, d] -> [B, S, H, d]
+        want = want.reshape(split).transpose(perms)
+        got = run.attention(q, kt, v, extra, steps, split, perms)
+    else:
+        got = run.attention(q, kt, v, extra, steps)
+    np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_attention_declines_what_the_kernel_was_not_written_for(run):
+    """Other head sizes, row counts or chains are MLEL_ERR_UNSUPPORTED: nothing is allocated, nothing falls back."""
+    rng = np.random.default_rng(5)
+    f16 = abi.F16
+    steps = [(4, abi.RED["MAX"], 0, 0, f16), (0, abi.BIN["SUB"], 0, 1, f16), (2, abi.UN["EXP"], 2, 0, f16),
+             (4, abi.RED["SUM"], 3, 0, f16), (2, abi.UN["RECIPROCAL"], 4, 0, f16), (1, 0, 3, 5, f16)]
+    mk = lambda *shape: rng.standard_normal(shape).astype(np.float16)
+    for q, kt, v, st in ((mk(1, 64, 32), mk(1, 32, 64), mk(1, 64, 32), steps),      # heads of 32
+                         (mk(1, 40, 64), mk(1, 64, 64), mk(1, 64, 64), steps),      # 40 query rows
+                         (mk(1, 64, 64), mk(1, 64, 576), mk(1, 576, 64), steps),    # 576 keys
+                         (mk(1, 64, 64), mk(1, 64, 64), mk(1, 64, 64), steps[:5] + [(1, 0, 3, 3, f16)])):  # another chain
+        with pytest.raises(hb.MlelError) as err:
+            run.attention(q, kt, v, [], st)
+        assert err.value.code == abi.ERR_UNSUPPORTED
+
+
 def test_elementwise_chain_equals_the_operators_one_by_one(run):
     """mlel_hip_elementwise_chain against the same operators launched one after another (bit for bit): a GELU-shaped
     chain over fp16 with scalar constants, a chain with row- and column-broadcast inputs and a cast, short rows, and a
