@@ -167,6 +167,14 @@ class Runner:
         self.done()
         return r
 
+    def concat_at(self, base, part, axis, offset):
+        """One CONCAT part written into an output that starts as `base`, at `offset` along `axis`."""
+        to, ti = self.put(base), self.put(part)
+        self.dev.op("concat", to.ref, ti.ref, int(axis), int(offset))
+        r = to.download()
+        self.done()
+        return r
+
     def concat(self, inputs, axis):
         shape = list(inputs[0].shape)
         shape[axis] = sum(i.shape[axis] for i in inputs)

@@ -1,6 +1,7 @@
 """GPU parity: every operator of the C ABI against the CPU oracle on the same seeded inputs (bit-exact for
 integers, stated tolerance for floats), the reference's known-answer vectors run on the GPU, and the
 BASELINE configs 0 and 1 at full size."""
+import os
 import zlib
 
 import numpy as np
@@ -833,6 +834,65 @@ def test_data_movement_vs_oracle(run, oracle):
     h = rng.standard_normal((8, 16, 4, 6)).astype(np.float16)
     np.testing.assert_array_equal(run.transpose(h, (0, 2, 1, 3)).view(np.uint16),
                                   h.transpose(0, 2, 1, 3).view(np.uint16))
+
+
+def test_out_of_bounds_reads_are_zero_and_writes_are_dropped(run, oracle):
+    """The reference's tensor accessors (tensor/shaders/tensor.glsl:26-86, graph_op/common.comp:64-182): an element read
+    outside a tensor's extents is 0, an element written outside is dropped.  Operands whose extents disagree with the
+    output reach that rule: an addend shorter than the output along two axes, a MATMUL whose B has fewer K rows than A
+    has columns, and a CONCAT part that sticks out of the output."""
+    rng = np.random.default_rng(99)
+    a = ri(rng, -1000, 1000, (2, 5, 12), np.int32)
+    b = ri(rng, -1000, 1000, (2, 3, 7), np.int32)
+    exp = a.copy()
+    exp[:, :3, :7] += b
+    np.testing.assert_array_equal(oracle.elementwise_binary("ADD", a, b, a.shape, abi.I32), exp)
+    np.testing.assert_array_equal(run.binary("ADD", a, b, a.shape, abi.I32), exp)
+    x = ri(rng, -128, 127, (1, 8, 16), np.int8)
+    w = ri(rng, -128, 127, (1, 12, 8), np.int8)   # K rows 12 .. 15 do not exist: they read as 0, not as the zero point
+    got = run.matmul(x, w, abi.I32, 3, -2)
+    ref = np.einsum("bmk,bkn->bmn", x.astype(np.int64)[:, :, :12] - 3, w.astype(np.int64) + 2) + \
+        ((x.astype(np.int64)[:, :, 12:] - 3).sum(axis=2, keepdims=True) * (0 + 2))
+    np.testing.assert_array_equal(oracle.matmul(x, w, abi.I32, 3, -2), ref.astype(np.int32))
+    np.testing.assert_array_equal(got, ref.astype(np.int32))
+    # CONCAT writes its part at an offset along the axis: what lands beyond the output's extent is dropped
+    part = ri(rng, -128, 127, (2, 4), np.int8)
+    out = run.concat_at(np.zeros((2, 5), np.int8), part, axis=1, offset=3)
+    want = np.zeros((2, 5), np.int8)
+    want[:, 3:] = part[:, :2]
+    np.testing.assert_array_equal(out, want)
+
+
+def test_external_memory_import_by_file_descriptor(run):
+    """mlel_hip_arena_import_fd (what vkBindDataGraphPipelineSessionMemoryARM would call with the fd of an exported
+    VkDeviceMemory, graph_layer.cpp:1391-1420): a device allocation exported as a dma-buf fd through HIP stands in for
+    the Vulkan export; the imported mapping shows the same bytes, operators run on it, and the import is released."""
+    import ctypes as C
+    dev = run.dev
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemGetHandleForAddressRange.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_ulonglong]
+    n = 1 << 20
+    src = dev.alloc(n)
+    data = np.random.default_rng(3).integers(-128, 127, n, endpoint=True).astype(np.int8)
+    dev._check(dev.lib.mlel_hip_memcpy_h2d(dev.ctx, C.c_void_p(src), data.ctypes.data_as(C.c_void_p), n, None))
+    fd = C.c_int(-1)
+    if hip.hipMemGetHandleForAddressRange(C.byref(fd), C.c_void_p(src), n, 1, 0) != 0:  # hipMemRangeHandleTypeDmaBufFd
+        dev.free(src)
+        pytest.skip("this driver does not export device memory as a dma-buf fd")
+    mapped, handle = C.c_void_p(), C.c_void_p()
+    dev._check(dev.lib.mlel_hip_arena_import_fd(dev.ctx, fd.value, n, C.byref(mapped), C.byref(handle)))
+    back = np.zeros(n, np.int8)
+    dev._check(dev.lib.mlel_hip_memcpy_d2h(dev.ctx, back.ctypes.data_as(C.c_void_p), mapped, n, None))
+    np.testing.assert_array_equal(back, data)
+    # an operator reading the imported mapping and writing an ordinary allocation
+    tin = abi.make_tensor(mapped.value, abi.I8, (n,), (1,))
+    tout = dev.tensor(abi.I8, (n,))
+    dev.op("clamp", tout.ref, C.byref(tin), C.byref(abi.ClampAttr(-5.0, 9.0, int(abi.NAN_PROPAGATE))))
+    np.testing.assert_array_equal(tout.download(), np.clip(data, -5, 9))
+    dev._check(dev.lib.mlel_hip_arena_release_import(dev.ctx, handle))
+    os.close(fd.value)
+    dev.free(src)
+    tout.free()
 
 
 def test_float_unary_and_reduce_tolerance(run, oracle):
