@@ -252,6 +252,8 @@ FUSED_SIGNATURES = {
                                    C.POINTER(Epilogue), C.POINTER(Epilogue), C.c_int],
     "matmul_rescale": [_T, _T, _T, C.POINTER(MatmulAttr), C.POINTER(Epilogue)],
     "dwconv_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
+    "conv2d_dwconv_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue), _T, _T,
+                                    C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
     "matmul_bias_cast": [_T, _T, _T, _T, C.POINTER(MatmulAttr)],
     "matmul_bias_cast_add": [_T, _T, _T, _T, C.POINTER(MatmulAttr), _T],
     "matmul_bias_cast_group": [C.POINTER(MatmulProduct), C.c_int, _T, C.POINTER(MatmulAttr)],
@@ -292,6 +294,8 @@ RUNTIME_SIGNATURES = {
     "mlel_hip_copy_kernel": (C.c_int, [_V, _V, _V, _V, C.c_size_t]),
     "mlel_hip_matmul_chain_in_kernel": (C.c_int, [C.POINTER(Chain)]),
     "mlel_hip_attention_f16_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Chain)]),
+    "mlel_hip_conv2d_dwconv_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Conv2dAttr), _T, _T,
+                                                   C.POINTER(Conv2dAttr)]),
 }
 
 

@@ -914,6 +914,62 @@ int mlel_hip_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor
     return 0;
 }
 
+namespace {
+// the intermediate tensor [N, H, W, C] of the fused pair, as the first operator would have written it (no memory)
+int conv_dw_prepare(const char *name, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w1,
+                    const mlel_tensor *b1, const mlel_conv2d_attr *a1, const mlel_epilogue *e1, const mlel_tensor *w2,
+                    const mlel_tensor *b2, const mlel_conv2d_attr *a2, const mlel_epilogue *e2, FusedEpilogue *f1,
+                    FusedEpilogue *f2) {
+    MLEL_REQUIRE(out != nullptr && in != nullptr && w1 != nullptr && b1 != nullptr && a1 != nullptr && e1 != nullptr &&
+                     w2 != nullptr && b2 != nullptr && a2 != nullptr && e2 != nullptr,
+                 MLEL_ERR_INVALID, "%s: null argument", name);
+    MLEL_TRY(check_tensor(out, name));
+    MLEL_TRY(check_tensor(in, name));
+    MLEL_TRY(check_tensor(w1, name));
+    MLEL_REQUIRE(in->rank == 4 && w1->rank == 4 && out->rank == 4, MLEL_ERR_INVALID, "%s: rank-4 tensors expected", name);
+    mlel_tensor mid{};
+    mid.dtype = MLEL_I8;
+    mid.rank = 4;
+    mid.dims[0] = in->dims[0], mid.dims[1] = in->dims[1], mid.dims[2] = in->dims[2], mid.dims[3] = w1->dims[0];
+    mid.strides[3] = 1;
+    for (int i = 2; i >= 0; i--) mid.strides[i] = mid.strides[i + 1] * mid.dims[i + 1];
+    mid.ptr = out->ptr;  // shape carrier for validation only
+    mlel_tensor acc1 = packed_like(&mid, MLEL_I32, out->ptr);
+    MLEL_TRY(check_conv(name, &acc1, in, w1, b1, a1));
+    mlel_tensor acc2 = packed_like(out, MLEL_I32, out->ptr);
+    MLEL_TRY(check_conv(name, &acc2, &mid, w2, b2, a2));
+    MLEL_TRY(make_epilogue(e1, MLEL_I32, &mid, mid.dims[3], f1));
+    MLEL_TRY(make_epilogue(e2, MLEL_I32, out, out->dims[3], f2));
+    return 0;
+}
+}  // namespace
+
+int mlel_hip_conv2d_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                         const mlel_tensor *w1, const mlel_tensor *b1, const mlel_conv2d_attr *a1,
+                                         const mlel_epilogue *e1, const mlel_tensor *w2, const mlel_tensor *b2,
+                                         const mlel_conv2d_attr *a2, const mlel_epilogue *e2) {
+    MLEL_TRY(require_ctx(ctx, "conv2d_dwconv_rescale_clamp"));
+    FusedEpilogue f1, f2;
+    MLEL_TRY(conv_dw_prepare("conv2d_dwconv_rescale_clamp", out, in, w1, b1, a1, e1, w2, b2, a2, e2, &f1, &f2));
+    const int rc = try_conv2d_dwconv_i8(ctx, (hipStream_t)stream, out, in, w1, b1, a1, &f1, w2, b2, a2, &f2, true);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    return set_error(MLEL_ERR_UNSUPPORTED,
+                     "conv2d_dwconv_rescale_clamp: int8, 1x1 unit-stride convolution of 32..160 input channels (a "
+                     "multiple of 32) to a multiple of 32 channels, 3x3 depthwise of stride 1 or 2, images of at most "
+                     "32 x 32 positions, zero weight zero points, dense 16-byte aligned operands only; run the two "
+                     "operators instead");
+}
+
+int mlel_hip_conv2d_dwconv_in_kernel(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w1,
+                                     const mlel_tensor *b1, const mlel_conv2d_attr *a1, const mlel_tensor *w2,
+                                     const mlel_tensor *b2, const mlel_conv2d_attr *a2) {
+    if (out == nullptr || in == nullptr || w1 == nullptr || b1 == nullptr || a1 == nullptr || w2 == nullptr ||
+        b2 == nullptr || a2 == nullptr)
+        return 0;
+    const FusedEpilogue unused{};  // the requantisation constants do not decide whether the kernel takes the case
+    return try_conv2d_dwconv_i8(nullptr, nullptr, out, in, w1, b1, a1, &unused, w2, b2, a2, &unused, false) == 1 ? 1 : 0;
+}
+
 int mlel_hip_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1,
                                  const mlel_epilogue *scale1, const mlel_tensor *in2, const mlel_epilogue *scale2,
                                  const mlel_epilogue *scale_out) {

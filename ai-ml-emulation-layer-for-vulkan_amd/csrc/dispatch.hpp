@@ -129,6 +129,13 @@ bool chain_is_gelu_tanh(const mlel_chain *chain);
 int try_matmul_f16_group(mlel_ctx *ctx, hipStream_t s, int n, const mlel_tensor *const *outs, const mlel_tensor *a,
                          const mlel_tensor *const *bs, const mlel_tensor *const *biases, const mlel_matmul_attr *attr);
 
+// ---- 1x1 CONV2D + RESCALE (+CLAMP) and 3x3 DEPTHWISE_CONV2D + RESCALE (+CLAMP) in one launch (conv_dw_i8.hip) ----
+// 1 when taken (with `launch` false: when the extents, types and strides are covered; pointers are not looked at)
+int try_conv2d_dwconv_i8(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
+                         const mlel_tensor *w1, const mlel_tensor *b1, const mlel_conv2d_attr *a1,
+                         const FusedEpilogue *e1, const mlel_tensor *w2, const mlel_tensor *b2,
+                         const mlel_conv2d_attr *a2, const FusedEpilogue *e2, bool launch);
+
 // ---- scores, softmax and the product with V of fp16 attention heads in one launch (attention_f16.hip) ----
 bool attention_f16_supported(const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt, const mlel_tensor *v,
                              const mlel_chain *chain);

@@ -310,6 +310,9 @@ std::string opLabel(const OpNode &op) {
                     (view.first[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");
         return name;
     }
+    case OpKind::FusedConv2DDepthwise:
+        return std::string("CONV2D+RESCALE") + (op.hasClampFirst ? "+CLAMP" : "") + "+DEPTHWISE_CONV2D+RESCALE" +
+               (op.hasClamp ? "+CLAMP" : "");
     case OpKind::FusedAttention:
         return std::string("MATMUL+CAST+ELEMENTWISE+REDUCE x") + std::to_string(op.chain.size()) + "+MATMUL+CAST" +
                (op.viewDims[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");

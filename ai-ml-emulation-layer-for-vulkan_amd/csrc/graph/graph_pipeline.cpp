@@ -1224,6 +1224,31 @@ void GraphPipeline::fuse() {
         sm.fusedAway = true;
     }
 
+    // Pattern 8 (expansion + depthwise): a fused 1x1 CONV2D (+RESCALE, +CLAMP) whose private int8 result is read only
+    // by a fused 3x3 DEPTHWISE_CONV2D (+RESCALE, +CLAMP) as its image, on shapes the one-launch kernel takes
+    // (mlel_hip_conv2d_dwconv_in_kernel decides: small images, channel counts in multiples of 32).  The expanded
+    // tensor then lives in shared memory only; byte for byte the two launches.
+    for (const auto &opPtr : ops) {
+        OpNode &dw = *opPtr;
+        if (dw.fusedAway || dw.kind != OpKind::FusedDepthwiseConv2D) continue;
+        const TensorPtr mid = dw.inputs[0];
+        OpNode *conv = mid->getProducer();
+        if (!conv || conv->fusedAway || conv->kind != OpKind::FusedConv2D || conv->outputs[0].get() != mid.get() ||
+            !isPrivateIntermediate(*mid) || consumersOf(ops, mid.get()).size() != 1)
+            continue;
+        const mlel_tensor out = dw.outputs[0]->view(), x = conv->inputs[0]->view(), w1 = conv->inputs[1]->view(),
+                          b1 = conv->inputs[2]->view(), w2 = dw.inputs[1]->view(), b2 = dw.inputs[2]->view();
+        if (mlel_hip_conv2d_dwconv_in_kernel(&out, &x, &w1, &b1, &conv->conv, &w2, &b2, &dw.conv) == 0) continue;
+        const TensorPtr w2T = dw.inputs[1], b2T = dw.inputs[2];
+        dw.kind = OpKind::FusedConv2DDepthwise;
+        dw.inputs = {conv->inputs[0], conv->inputs[1], conv->inputs[2], w2T, b2T};
+        dw.convFirst = conv->conv;
+        dw.scaleA = conv->epilogue;
+        dw.hasClampFirst = conv->hasClamp;
+        dw.clampFirst = conv->clamp;
+        conv->fusedAway = true;
+    }
+
     // Pattern 3: RESHAPE between two packed session tensors of the same byte size moves no data (the reference's
     // reshape.comp:16-27 copies by flat index): the output becomes a second view of the input's storage and the
     // operator is not executed.  plan() gives both tensors one allocation that lives as long as either is used.
@@ -1684,6 +1709,15 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
             }
         }
         rc = mlel_hip_attention_f16(ctx, stream, &view, &in[0], &in[1], &in[2], &c);
+        break;
+    }
+    case OpKind::FusedConv2DDepthwise: {
+        const mlel_tensor m1 = op.scaleA.multiplier->view(), s1 = op.scaleA.shift->view();
+        const mlel_tensor m2 = op.epilogue.multiplier->view(), s2 = op.epilogue.shift->view();
+        const mlel_epilogue e1 = makeEpilogue(op.scaleA, &m1, &s1, op.hasClampFirst, op.clampFirst);
+        const mlel_epilogue e2 = makeEpilogue(op.epilogue, &m2, &s2, op.hasClamp, op.clamp);
+        rc = mlel_hip_conv2d_dwconv_rescale_clamp(ctx, stream, &out, &in[0], &in[1], &in[2], &op.convFirst, &e1, &in[3],
+                                                  &in[4], &op.conv, &e2);
         break;
     }
     case OpKind::FusedConv2DResidual: {

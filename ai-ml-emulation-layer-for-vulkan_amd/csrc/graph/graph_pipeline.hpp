@@ -98,7 +98,7 @@ enum class OpKind {
     Argmax, ArithmeticRightShift, Conv3D, TransposeConv2D, Fft2D, Rfft2D, Gather, Scatter, Resize, Reverse, Tile, Select,
     // produced by the fusion pass only
     FusedConv2D, FusedDepthwiseConv2D, FusedMatmul, FusedRescaleAddRescale, FusedMatmulBiasCast, FusedElementwise,
-    FusedConv2DResidual, FusedAttention,
+    FusedConv2DResidual, FusedAttention, FusedConv2DDepthwise,
 };
 
 struct RescaleSpec {
@@ -150,6 +150,12 @@ class OpNode {
     // FusedConv2DResidual: epilogue (+ clamp) belongs to the convolution; scaleA rescales its 8-bit result, scaleB the
     // residual (inputs[3]), scaleOut their sum; `flag` is set when the residual was the addition's first operand
     RescaleSpec scaleOut;
+    // FusedConv2DDepthwise: inputs = {x, the 1x1 convolution's weights and bias, the depthwise weights and bias};
+    // conv / epilogue / hasClamp / clamp belong to the depthwise stage, convFirst / scaleA / hasClampFirst /
+    // clampFirst to the 1x1 convolution in front of it
+    mlel_conv2d_attr convFirst{};
+    mlel_clamp_attr clampFirst{};
+    bool hasClampFirst = false;
 };
 
 class GraphPipeline {

@@ -513,6 +513,25 @@ int mlel_hip_attention_f16(mlel_ctx *ctx, void *stream, const mlel_tensor *out, 
 int mlel_hip_attention_f16_in_kernel(const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt,
                                      const mlel_tensor *v, const mlel_chain *softmax);
 
+/* out(int8) = CLAMP?(RESCALE(DEPTHWISE_CONV2D( CLAMP?(RESCALE(CONV2D(in, w1, b1))), w2, b2 ))): the expansion (1x1,
+ * unit stride, no padding) and the 3x3 depthwise stage (stride 1 or 2) of an inverted-residual block in one launch.  A
+ * thread block keeps 32 expanded channels of a whole image in shared memory, so the expanded tensor never reaches
+ * memory.  Byte for byte mlel_hip_conv2d_rescale_clamp followed by mlel_hip_dwconv_rescale_clamp.  in [N, H, W, IC]
+ * with IC a multiple of 32 up to 160 and H, W <= 32; w1 [C, 1, 1, IC] with C a multiple of 32; w2 [3, 3, C, 1];
+ * out [N, OH, OW, C]; zero weight zero points; dense operands, `in` and `w1` 16-byte aligned.  Anything else is
+ * MLEL_ERR_UNSUPPORTED (nothing is allocated and nothing falls back).  Replaces two pairs of the reference's
+ * dispatches (conv2d.comp + rescale.comp, depthwise_conv2d.comp + rescale.comp, each with clamp.comp when present);
+ * it has no single counterpart there. */
+int mlel_hip_conv2d_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                         const mlel_tensor *w1, const mlel_tensor *b1, const mlel_conv2d_attr *a1,
+                                         const mlel_epilogue *e1, const mlel_tensor *w2, const mlel_tensor *b2,
+                                         const mlel_conv2d_attr *a2, const mlel_epilogue *e2);
+/* 1 when mlel_hip_conv2d_dwconv_rescale_clamp takes these operands, judged by types, extents, strides and attributes
+ * only (data pointers are not looked at; no device is touched), else 0. */
+int mlel_hip_conv2d_dwconv_in_kernel(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w1,
+                                     const mlel_tensor *b1, const mlel_conv2d_attr *a1, const mlel_tensor *w2,
+                                     const mlel_tensor *b2, const mlel_conv2d_attr *a2);
+
 /* Plain device-to-device copy kernel of `bytes` bytes with 128-bit accesses; the calibration kernel for
  * memory-traffic counters and the measured HBM ceiling. */
 int mlel_hip_copy_kernel(mlel_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes);

@@ -226,6 +226,22 @@ class Runner:
         self.done()
         return r
 
+    def conv2d_dwconv(self, x, w1, b1, attr1, epi1, w2, b2, attr2, epi2, out_shape, expect=0):
+        tx, tw1, tb1, tw2, tb2 = self.put(x), self.put(w1), self.put(b1), self.put(w2), self.put(b2)
+        to = self.new(abi.I8, out_shape)
+        e1, e2 = self._epi(*epi1), self._epi(*epi2)
+        args = (tx.ref, tw1.ref, tb1.ref, C.byref(attr1), C.byref(e1), tw2.ref, tb2.ref, C.byref(attr2), C.byref(e2))
+        covered = self.dev.lib.mlel_hip_conv2d_dwconv_in_kernel(to.ref, tx.ref, tw1.ref, tb1.ref, C.byref(attr1),
+                                                                tw2.ref, tb2.ref, C.byref(attr2))
+        if expect != 0:
+            rc = self.dev.lib.mlel_hip_conv2d_dwconv_rescale_clamp(self.dev.ctx, self.dev.stream, to.ref, *args)
+            self.done()
+            return covered, rc
+        self.dev.op("conv2d_dwconv_rescale_clamp", to.ref, *args)
+        r = to.download()
+        self.done()
+        return covered, r
+
     def softmax_rows(self, x):
         tx = self.put(x)
         to = self.new(tx.dtype, x.shape)

@@ -80,7 +80,7 @@ def test_config3_mobilenetv2_b32_full_size(dev, oracle):
     spec = graphs.mobilenetv2_spec(batch=32, spread=True)
     x = random_input(spec, 1003)
     out, names = run_graph(dev, spec, x, True)
-    assert len(names) == 54
+    assert len(names) == 41
     exp, _ = run_spec(oracle, spec, {"input": x})
     np.testing.assert_array_equal(out, exp["output"])
     one = graphs.mobilenetv2_spec(batch=1, spread=True)

@@ -652,6 +652,73 @@ def test_depthwise_vs_oracle(run, oracle, case):
     np.testing.assert_array_equal(out8, exp8)
 
 
+# ------------------------------------------------------------------------------- 1x1 CONV2D + 3x3 DEPTHWISE, one launch
+#   name, input [N, H, W, IC], expanded channels, depthwise padding, stride, conv input zp, depthwise input zp
+CONV_DW_CASES = [
+    ("b14_64_to_64", (2, 14, 14, 64), 64, (1, 1, 1, 1), 1, -3, 5),
+    ("b7_160_to_64", (3, 7, 7, 160), 64, (1, 1, 1, 1), 1, 7, -128),
+    ("b28_32_to_32", (1, 28, 28, 32), 32, (1, 1, 1, 1), 1, -128, -9),
+    ("stride2_even", (2, 16, 16, 32), 96, (0, 1, 0, 1), 2, 4, 2),
+    ("stride2_odd", (1, 15, 13, 96), 32, (1, 1, 1, 1), 2, 0, -1),
+    ("ragged_9x10", (2, 9, 10, 128), 32, (1, 1, 1, 1), 1, -20, 11),
+    ("no_padding", (1, 12, 6, 32), 32, (0, 0, 0, 0), 1, 1, 3),
+    ("pad_2_one_side", (1, 5, 7, 64), 32, (2, 0, 0, 2), 1, -1, -4),
+    ("one_position", (4, 1, 1, 32), 32, (1, 1, 1, 1), 1, 9, 9),
+    ("widest_32x32", (1, 32, 32, 32), 32, (1, 1, 1, 1), 1, 2, -2),
+]
+
+
+@pytest.mark.parametrize("case", CONV_DW_CASES, ids=[c[0] for c in CONV_DW_CASES])
+def test_conv2d_dwconv_one_launch_vs_oracle(run, oracle, case):
+    name, xs, c, pad, stride, zx, zi = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    n, h, w_, ic = xs
+    x = ri(rng, -128, 127, xs, np.int8)
+    w1 = ri(rng, -128, 127, (c, 1, 1, ic), np.int8)
+    b1 = ri(rng, -2 ** 12, 2 ** 12, (c,), np.int32)
+    w2 = ri(rng, -128, 127, (3, 3, c, 1), np.int8)
+    b2 = ri(rng, -2 ** 10, 2 ** 10, (c,), np.int32)
+    m1, s1 = ri(rng, 2 ** 30, 2 ** 31 - 1, (c,), np.int32), ri(rng, 40, 43, (c,), np.int8)
+    m2, s2 = ri(rng, 2 ** 30, 2 ** 31 - 1, (c,), np.int32), ri(rng, 36, 39, (c,), np.int8)
+    a1 = abi.conv2d_attr((0, 0, 0, 0), (1, 1), (1, 1), zx, 0)
+    a2 = abi.conv2d_attr(pad, (stride, stride), (1, 1), zi, 0)
+    r1 = abi.rescale_attr(0, zi, True, True, True)
+    r2 = abi.rescale_attr(0, -11, True, True, True)
+    clamp1, clamp2 = (-100, 127), None
+    oh, ow = out_hw(h, w_, (3, 3), pad, (stride, stride), (1, 1))
+    mid_shape, out_shape = (n, h, w_, c), (n, oh, ow, c)
+    mid = oracle.clamp(oracle.rescale(oracle.conv2d(x, w1, b1, mid_shape, abi.I32, a1), m1, s1, abi.I8, r1), *clamp1)
+    assert len(np.unique(mid)) > 50, "the intermediate values must not all sit on the clamp"
+    exp = oracle.rescale(oracle.depthwise_conv2d(mid, w2, b2, out_shape, abi.I32, a2), m2, s2, abi.I8, r2)
+    covered, got = run.conv2d_dwconv(x, w1, b1, a1, (m1, s1, r1, clamp1), w2, b2, a2, (m2, s2, r2, clamp2), out_shape)
+    assert covered == 1
+    np.testing.assert_array_equal(got, exp)
+
+
+def test_conv2d_dwconv_declines_what_the_kernel_was_not_written_for(run):
+    rng = np.random.default_rng(5)
+
+    def attempt(xs, c, zw1=0, zw2=0, stride=1, kernel=(3, 3)):
+        n, h, w_, ic = xs
+        x = ri(rng, -128, 127, xs, np.int8)
+        w1 = ri(rng, -128, 127, (c, 1, 1, ic), np.int8)
+        w2 = ri(rng, -128, 127, kernel + (c, 1), np.int8)
+        b = ri(rng, -100, 100, (c,), np.int32)
+        m, s = rescale_params(rng, c)
+        a1 = abi.conv2d_attr((0, 0, 0, 0), (1, 1), (1, 1), 0, zw1)
+        pad = (kernel[0] // 2,) * 4
+        a2 = abi.conv2d_attr(pad, (stride, stride), (1, 1), 0, zw2)
+        r = abi.rescale_attr(0, 0, True, True, True)
+        oh, ow = out_hw(h, w_, kernel, pad, (stride, stride), (1, 1))
+        return run.conv2d_dwconv(x, w1, b, a1, (m, s, r, None), w2, b, a2, (m, s, r, None), (n, oh, ow, c), expect=-1)
+
+    assert attempt((1, 8, 8, 32), 32) == (1, abi.OK)
+    for kwargs in (dict(xs=(1, 8, 8, 48), c=32), dict(xs=(1, 8, 8, 192), c=32), dict(xs=(1, 8, 8, 32), c=48),
+                   dict(xs=(1, 40, 8, 32), c=32), dict(xs=(1, 8, 8, 32), c=32, zw1=1),
+                   dict(xs=(1, 8, 8, 32), c=32, zw2=-1), dict(xs=(1, 8, 8, 32), c=32, kernel=(5, 5))):
+        assert attempt(**kwargs) == (0, abi.ERR_UNSUPPORTED), kwargs
+
+
 # ------------------------------------------------------------------------------------------------ RESCALE & co
 @pytest.mark.parametrize("double_round", [False, True])
 @pytest.mark.parametrize("per_channel", [False, True])
