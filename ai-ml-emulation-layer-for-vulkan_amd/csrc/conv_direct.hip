@@ -440,9 +440,13 @@ int try_rows_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const ml
     const int nj = (int)((OC + 31) / 32), kc = IC > 16 ? 2 : 1;
     const size_t sm = (size_t)nj * 32 * sizeof(ChanConst) + (size_t)(kBlock / 64) * 32 * op;
     const int cus = ctx != nullptr && ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
-    // three blocks (twelve wavefronts) per compute unit (measured: two to four are equal within 3 %), fewer when the
-    // problem has fewer position groups
-    const int64_t want = std::min<int64_t>((int64_t)cus * 3, (g.groups + kBlock / 64 - 1) / (kBlock / 64));
+    // Sixteen position groups per block (four per wavefront) amortise the prologue (weights, channel constants);
+    // between two and three blocks per compute unit, never more blocks than a group per wavefront needs.  Measured:
+    // 16 -> 96 channels on 112 x 112 images is flat from two to four blocks per compute unit, 24 -> 144 on 56 x 56
+    // (a quarter of the groups) loses 15 % at three.
+    const int64_t per_wave = (g.groups + kBlock / 64 - 1) / (kBlock / 64);
+    const int64_t want =
+        std::min<int64_t>(per_wave, std::min<int64_t>((int64_t)cus * 3, std::max<int64_t>((int64_t)cus * 2, (g.groups + 15) / 16)));
     const dim3 grid((unsigned)std::max<int64_t>(want, 1));
     switch (nj) {
     case 1: launch_rows_mfma<1>(g, kc, grid, sm, s); break;
