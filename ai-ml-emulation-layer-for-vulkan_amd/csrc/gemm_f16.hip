@@ -12,6 +12,8 @@
 //           lane L of a 16-lane group the four k values of column L out of a 4(k) x 16(n) block whose rows are
 //           addressed by the group's lanes (lane s points at row s / 4, columns 4 * (s % 4) ..).
 // All global loads are buffer loads: an offset at or beyond the extent returns 0, which pads M, N and K tails.
+#include <algorithm>
+
 #include "common.hpp"
 #include "dispatch.hpp"
 #include "float_programs.hpp"
@@ -256,8 +258,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
         // and leaves in 16-byte pieces, consecutive lanes along a row, so that every instruction writes whole lines.
         constexpr int OPITCH = BN * 2 + 16;
         constexpr int TPITCH = BM * 2 + 16;  // a column of the tile, for transposing views
-        static_assert(BM * OPITCH <= 2 * XBUF + 2 * WBUF && BN * TPITCH <= 2 * XBUF + 2 * WBUF,
-                      "the result tile fits in the operand buffers");
+        // the launch sizes shared memory for the larger of the operand buffers and the result tile
 #pragma unroll
         for (int i = 0; i < TM; i++) {
             char *orow = smem + (wave_m * WM + i * 32 + (lane & 31)) * OPITCH;
@@ -364,7 +365,10 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BKH>
 void launch_k(const HGemmArgs &g, bool cast_epilogue, dim3 grid, hipStream_t s) {
-    constexpr size_t sm = (size_t)2 * BM * (BKH * 2 + 16) + (size_t)2 * BKH * (2 * BN + 32);
+    constexpr size_t operands = (size_t)2 * BM * (BKH * 2 + 16) + (size_t)2 * BKH * (2 * BN + 32);
+    constexpr size_t result = std::max((size_t)BM * (BN * 2 + 16), (size_t)BN * (BM * 2 + 16));
+    constexpr size_t sm = std::max(operands, result);
+    static_assert(sm <= 160 * 1024, "shared memory of a compute unit");
     // above the default dynamic shared-memory limit the limit is raised once per kernel (thread-safe static)
     if (cast_epilogue) {
         auto kernel = gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 1, BKH>;
@@ -533,7 +537,20 @@ int launch_args(mlel_ctx *ctx, hipStream_t s, HGemmArgs &g, bool bias_cast) {
     // the eight-wavefront tile even when it leaves a quarter of the compute units idle, 43.1 -> 38.4 us and
     // 15.5 -> 13.7 us against 384 short tiles
     const int64_t tiles128 = ((M + 127) / 128) * tiles_n * NB;
-    if (BN == 128 && !tall && g.K >= 512 && tiles128 * 5 >= 3 * (int64_t)cus) {
+    // The 256 x 256 tile of eight wavefronts (128 x 64 each: a third fewer operand reads from shared memory per
+    // multiply) when it still occupies three quarters of the compute units: 4096 x 768 x 3072 in 192 tiles,
+    // 37.7 -> 34.7 us.  With fewer tiles the idle compute units cost more than the reads (144 tiles: no gain;
+    // 48 tiles: twice the time), and so does an activation in the epilogue, whose arithmetic then runs on three
+    // quarters of the machine (the same product with the tanh GELU: 40.9 -> 44.1 us).
+    const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256) * NB;
+    if (BN == 128 && g.groups == 1 && g.act[0] == nullptr && g.K >= 256 && tiles256 * 4 >= 3 * (int64_t)cus && tiles256 <= 2 * (int64_t)cus) {
+        g.tiles_m = (int)((M + 255) / 256);
+        g.tiles_n_group = (int)((N + 255) / 256);
+        g.tiles_n = g.tiles_n_group;
+        g.total_tiles = (int)tiles256;
+        g.chunk = (int)((tiles256 + 7) / 8);
+        launch_k<256, 256, 2, 4, 32>(g, bias_cast, dim3((unsigned)(g.chunk * 8)), s);
+    } else if (BN == 128 && !tall && g.K >= 512 && tiles128 * 5 >= 3 * (int64_t)cus) {
         g.tiles_m = (int)((M + 127) / 128);
         g.total_tiles = (int)tiles128;
         g.chunk = (int)((tiles128 + 7) / 8);
