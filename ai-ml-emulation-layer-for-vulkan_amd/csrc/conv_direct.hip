@@ -189,7 +189,7 @@ __global__ void __launch_bounds__(kBlock) conv_direct_i8_kernel(const DirectArgs
 #pragma unroll
                 for (int j = 0; j < KD; j++) v = __builtin_amdgcn_sdot4((int)xd[p][j], (int)wv[j], v, false);
                 if (Q8) {
-                    packed[p][e / 4] |= ((uint32_t)requant_chan(v, c.q, a.scale.p) & 0xffu) << (8 * (e % 4));
+                    packed[p][e / 4] |= ((uint32_t)requant_acc(v, c.q, a.scale.p) & 0xffu) << (8 * (e % 4));
                 } else {
                     packed[p][e % 4] = (uint32_t)v;
                     if (e % 4 == 3 && mpos[p] < a.M)
@@ -371,14 +371,14 @@ __global__ void __launch_bounds__(kBlock) conv_rows_mfma_i8_kernel(const RowsMfm
                 int32_t v[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    v[e] = requant_chan(acc[4 * q + e], c.q, a.scale.p);
+                    v[e] = requant_acc(acc[4 * q + e], c.q, a.scale.p);
                 }
                 const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
                 const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
                 uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // bytes = positions e of this lane's channel
-                uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0xb1, 0xf, 0xf, false);
+                uint32_t o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0xb1, 0xf, 0xf, true);
                 p = __builtin_amdgcn_perm(o, p, sel_a);
-                o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0x4e, 0xf, 0xf, false);
+                o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0x4e, 0xf, 0xf, true);
                 p = __builtin_amdgcn_perm(o, p, sel_b);
                 // now: position 8 q + 4 (lane / 32) + lane % 4, channels 32 j + 4 (lane % 32 / 4) .. + 3
                 if (col_live) *reinterpret_cast<uint32_t *>(so_lane + 8 * q * a.op + j * 32) = p;
@@ -467,6 +467,9 @@ int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, c
     if (in->dtype != MLEL_I8 || w->dtype != MLEL_I8 || bias->dtype != MLEL_I32 || a->acc_type != MLEL_ACC_I32) return 0;
     if (epi == nullptr && out->dtype != MLEL_I32) return 0;
     if (epi != nullptr && dt_size(out->dtype) != 1) return 0;
+    // the kernels' requantisation assumes the int32 accumulator's RESCALE has input_zp == 0 (requant_acc); an
+    // operator that names another runs as the general operator sequence
+    if (epi != nullptr && epi->p.in_zp != 0) return 0;
     const int64_t N = out->dims[0], OH = out->dims[1], OW = out->dims[2], OC = out->dims[3];
     const int64_t H = in->dims[1], W = in->dims[2], IC = in->dims[3];
     const int64_t KH = w->dims[1], KW = w->dims[2];

@@ -181,13 +181,13 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
         for (int q = 0; q < 4; q++) {
             int32_t v[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = requant_chan(acc[4 * q + e], q1, a.s1.p);
+            for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[4 * q + e], q1, a.s1.p);
             const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
             const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
             uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // bytes = positions e of this lane's channel
-            uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0xb1, 0xf, 0xf, false);
+            uint32_t o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0xb1, 0xf, 0xf, true);
             p = __builtin_amdgcn_perm(o, p, sel_a);
-            o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0x4e, 0xf, 0xf, false);
+            o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0x4e, 0xf, 0xf, true);
             p = __builtin_amdgcn_perm(o, p, sel_b);
             // now: position 32 g + 8 q + 4 (lane / 32) + lane % 4 of the band's rows, channels 4 (lane % 32 / 4) .. + 3
             const int pos = g * 32 + 8 * q + 4 * half + (lane & 3);
@@ -263,7 +263,7 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
                 if (ox >= a.OW) break;
                 int32_t v[4];
 #pragma unroll
-                for (int e = 0; e < 4; e++) v[e] = requant_chan(acc[ty][t][e], q2[e], a.s2.p);
+                for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[ty][t][e], q2[e], a.s2.p);
                 const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
                 const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
                 const uint32_t off = (orow + (uint32_t)ox) * (uint32_t)a.C + c;
@@ -371,6 +371,8 @@ int try_conv2d_dwconv_i8(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, c
     const size_t sm = kSliceCh * sizeof(DwConst) + tile_bytes;
     if (sm > 64 * 1024) return 0;
     if (!launch) return 1;
+    // requant_acc: both RESCALEs read int32 accumulators, whose input_zp TOSA fixes at 0
+    if (e1->p.in_zp != 0 || e2->p.in_zp != 0) return 0;
     if (((uintptr_t)in->ptr % 16) != 0 || ((uintptr_t)w1->ptr % 16) != 0 || ((uintptr_t)out->ptr % 4) != 0) return 0;
     if (((uintptr_t)b1->ptr % 4) != 0 || ((uintptr_t)b2->ptr % 4) != 0) return 0;
 

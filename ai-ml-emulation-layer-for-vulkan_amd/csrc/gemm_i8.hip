@@ -179,6 +179,9 @@ int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
                        const FusedEpilogue *epi, const ConvResidual *residual, const GemmScratch *static_scratch) {
     if (in->dtype != MLEL_I8 || w->dtype != MLEL_I8 || bias->dtype != MLEL_I32 || a->acc_type != MLEL_ACC_I32) return 0;
     if (residual != nullptr && (epi == nullptr || out->dtype != MLEL_I8)) return 0;
+    // the kernels' requantisation assumes the int32 accumulator's RESCALE has input_zp == 0 (requant_acc); an
+    // operator that names another runs as the general operator sequence
+    if (epi != nullptr && epi->p.in_zp != 0) return 0;
     if (epi == nullptr && out->dtype != MLEL_I32) return 0;
     if (epi != nullptr && dt_size(out->dtype) > 4) return 0;
     const int64_t N = out->dims[0], OH = out->dims[1], OW = out->dims[2], OC = out->dims[3];
@@ -265,6 +268,9 @@ int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
 int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *A,
                        const mlel_tensor *B, const mlel_matmul_attr *attr, const FusedEpilogue *epi) {
     if (A->dtype != MLEL_I8 || B->dtype != MLEL_I8) return 0;
+    // the kernels' requantisation assumes the int32 accumulator's RESCALE has input_zp == 0 (requant_acc); an
+    // operator that names another runs as the general operator sequence
+    if (epi != nullptr && epi->p.in_zp != 0) return 0;
     if (epi == nullptr && out->dtype != MLEL_I32) return 0;
     if (epi != nullptr && dt_size(out->dtype) > 4) return 0;
     const int64_t NB = out->dims[0], M = out->dims[1], N = out->dims[2], K = A->dims[2];

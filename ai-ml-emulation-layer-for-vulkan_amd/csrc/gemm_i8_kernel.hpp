@@ -980,15 +980,15 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] - (uint32_t)xc[e]);
-                        v[e] = requant_chan(a, cs[j], g.rp);
+                        v[e] = requant_acc(a, cs[j], g.rp);
                     }
                     // bytes = positions e of this lane's channel
                     const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
                     const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
                     uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-                    uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0xb1, 0xf, 0xf, false);  // lane ^ 1
+                    uint32_t o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0xb1, 0xf, 0xf, true);  // lane ^ 1
                     p = __builtin_amdgcn_perm(o, p, sel_a);
-                    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)p, 0x4e, 0xf, 0xf, false);           // lane ^ 2
+                    o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0x4e, 0xf, 0xf, true);           // lane ^ 2
                     p = __builtin_amdgcn_perm(o, p, sel_b);
                     // now: position 8q + 4 half + lane % 4 of tile row i, channels 4 (cl / 4) .. + 3 of tile column j
                     if constexpr (STAGED) {
@@ -1072,7 +1072,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                     const int n = n_base + wave_n * WN + j * 32 + cl;
                     if (n >= g.N) continue;
                     const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] - (uint32_t)xc[e]);
-                    const int32_t v = g.fused ? requant_chan(a, cs[j], g.rp) : a;
+                    const int32_t v = g.fused ? requant_acc(a, cs[j], g.rp) : a;
                     const int64_t off = (int64_t)m * g.ldo + n;
                     if (g.out_size == 1)
                         *reinterpret_cast<int8_t *>(ob + off) = (int8_t)v;

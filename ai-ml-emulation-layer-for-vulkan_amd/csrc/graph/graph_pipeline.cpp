@@ -1236,6 +1236,9 @@ void GraphPipeline::fuse() {
         if (!conv || conv->fusedAway || conv->kind != OpKind::FusedConv2D || conv->outputs[0].get() != mid.get() ||
             !isPrivateIntermediate(*mid) || consumersOf(ops, mid.get()).size() != 1)
             continue;
+        // the one-launch kernel requantises int32 accumulators, whose RESCALE has input_zp 0 in TOSA; it has no
+        // general route of its own for a graph that names another
+        if (conv->epilogue.attr.input_zp != 0 || dw.epilogue.attr.input_zp != 0) continue;
         const mlel_tensor out = dw.outputs[0]->view(), x = conv->inputs[0]->view(), w1 = conv->inputs[1]->view(),
                           b1 = conv->inputs[2]->view(), w2 = dw.inputs[1]->view(), b2 = dw.inputs[2]->view();
         if (mlel_hip_conv2d_dwconv_in_kernel(&out, &x, &w1, &b1, &conv->conv, &w2, &b2, &dw.conv) == 0) continue;

@@ -278,7 +278,7 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
             for (int e = 0; e < 4; e++) {
                 int32_t s = acc[ty][t][e];
                 if (ZW) s = (int32_t)((uint32_t)s - (uint32_t)a.zw * (uint32_t)xs[ty][t][e]);
-                if (Q8 || a.fused) s = requant_chan(s, q[e], a.scale.p);
+                if (Q8 || a.fused) s = requant_acc(s, q[e], a.scale.p);
                 v[e] = s;
             }
             const uint32_t off = ((orow + (uint32_t)ox) * (uint32_t)a.C + (uint32_t)c) * esz;
@@ -306,6 +306,9 @@ int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     if (in->dtype != MLEL_I8 || w->dtype != MLEL_I8 || bias->dtype != MLEL_I32 || a->acc_type != MLEL_ACC_I32) return 0;
     if (epi == nullptr && out->dtype != MLEL_I32) return 0;
     if (epi != nullptr && (dt_size(out->dtype) > 4 || out->dtype == MLEL_BOOL)) return 0;
+    // the kernels' requantisation assumes the int32 accumulator's RESCALE has input_zp == 0 (requant_acc); an
+    // operator that names another runs as the general operator sequence
+    if (epi != nullptr && epi->p.in_zp != 0) return 0;
     const int64_t N = out->dims[0], OH = out->dims[1], OW = out->dims[2], C = out->dims[3];
     // the kernel's indexing assumes: 3x3 taps, multiplier 1, unit dilation, stride 1 or 2, channels in quads, dense
     // weights [3][3][C][1], packed output, channel-contiguous 4-byte aligned input

@@ -719,6 +719,37 @@ def test_conv2d_dwconv_declines_what_the_kernel_was_not_written_for(run):
         assert attempt(**kwargs) == (0, abi.ERR_UNSUPPORTED), kwargs
 
 
+def test_fused_epilogue_with_nonzero_input_zero_point_vs_oracle(run, oracle):
+    """TOSA fixes the input zero point of a RESCALE of int32 values at 0 and the fused kernels rely on it; an
+    operator that names another must still give the reference's result (it runs as the operator sequence)."""
+    rng = np.random.default_rng(77)
+    x = ri(rng, -128, 127, (1, 9, 9, 32), np.int8)
+    w = ri(rng, -128, 127, (32, 1, 1, 32), np.int8)
+    b = ri(rng, -2 ** 10, 2 ** 10, (32,), np.int32)
+    mult, shift = ri(rng, 2 ** 30, 2 ** 31 - 1, (32,), np.int32), ri(rng, 38, 41, (32,), np.int8)
+    attr = abi.conv2d_attr((0, 0, 0, 0), (1, 1), (1, 1), 3, 0)
+    for zp in (0, 1500, -1500):
+        rattr = abi.rescale_attr(zp, -4, True, True, True)
+        acc = oracle.conv2d(x, w, b, (1, 9, 9, 32), abi.I32, attr)
+        exp = oracle.rescale(acc, mult, shift, abi.I8, rattr)
+        got = run.conv2d(x, w, b, (1, 9, 9, 32), abi.I8, attr, epilogue=(mult, shift, rattr, None))
+        np.testing.assert_array_equal(got, exp)
+        wd = ri(rng, -128, 127, (3, 3, 32, 1), np.int8)
+        dattr = abi.conv2d_attr((1, 1, 1, 1), (1, 1), (1, 1), -2, 0)
+        dacc = oracle.depthwise_conv2d(x, wd, b, (1, 9, 9, 32), abi.I32, dattr)
+        mult2, shift2 = mult, (shift - 3).astype(np.int8)
+        dexp = oracle.rescale(dacc, mult2, shift2, abi.I8, rattr)
+        dgot = run.conv2d(x, wd, b, (1, 9, 9, 32), abi.I8, dattr, depthwise=True, epilogue=(mult2, shift2, rattr, None))
+        np.testing.assert_array_equal(dgot, dexp)
+        assert len(np.unique(got)) > 20 and len(np.unique(dgot)) > 20
+        a = ri(rng, -128, 127, (2, 40, 64), np.int8)
+        bm = ri(rng, -128, 127, (2, 64, 32), np.int8)
+        macc = oracle.matmul(a, bm, abi.I32, 1, -1)
+        mexp = oracle.rescale(macc, mult, shift, abi.I8, rattr)
+        mgot = run.matmul(a, bm, abi.I8, 1, -1, epilogue=(mult, shift, rattr, None))
+        np.testing.assert_array_equal(mgot, mexp)
+
+
 # ------------------------------------------------------------------------------------------------ RESCALE & co
 @pytest.mark.parametrize("double_round", [False, True])
 @pytest.mark.parametrize("per_channel", [False, True])
