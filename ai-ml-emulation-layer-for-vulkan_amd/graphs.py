@@ -368,6 +368,33 @@ def time_operators(dev, g, reps=50, only=None):
     return out
 
 
+def launch_layers(g, spec):
+    """The layers of `spec` (one per CONV2D / DEPTHWISE_CONV2D / AVG_POOL2D / MATMUL of the graph) grouped by the
+    launches of the fused graph `g`: a launch whose name holds both CONV2D and DEPTHWISE_CONV2D covers the 1x1
+    convolution and the depthwise layer behind it, whose intermediate tensor never reaches memory (its bytes leave
+    the launch's algorithmic bytes).  None when the names do not account for every layer."""
+    out, at = [], 0
+    for i in range(g.op_count()):
+        name = g.op_name(i)
+        if at >= len(spec.layers):
+            return None
+        if name.startswith("CONV2D") and "DEPTHWISE_CONV2D" in name:
+            if at + 1 >= len(spec.layers):
+                return None
+            conv, dw = spec.layers[at], spec.layers[at + 1]
+            if conv["kind"] != "conv" or dw["kind"] != "dw":
+                return None
+            mid = int(np.prod(conv["out"]))
+            out.append({"kind": "conv+dw", "in": conv["in"], "out": dw["out"], "kernel": dw["kernel"],
+                        "stride": dw["stride"], "macs": conv["macs"] + dw["macs"],
+                        "bytes": conv["bytes"] + dw["bytes"] - 2 * mid, "layers": [at, at + 1]})
+            at += 2
+        else:
+            out.append(dict(spec.layers[at], layers=[at]))
+            at += 1
+    return out if at == len(spec.layers) else None
+
+
 def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True):
     """Times whole-graph dispatches of BASELINE config 3 (inputs resident in HBM) and every launch on its own; returns
     the extra fields bench.py adds to its JSON line, with the MFMA position of the dense (CONV2D / MATMUL) launches
@@ -388,17 +415,20 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True):
            "operators_executed": g.op_count(), "operators_in_graph": len(spec.ops),
            "session_memory_bytes": g.session_size,
            "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}
-    if per_layer and g.op_count() == len(spec.layers):
+    launches = launch_layers(g, spec) if per_layer else None
+    if launches is not None:
         alone = time_operators(dev, g)
         layers = []
-        for i, layer in enumerate(spec.layers):
+        for i, layer in enumerate(launches):
             ms = alone[i]
             layers.append({"index": i, "kind": layer["kind"], "in": list(layer["in"]), "out": list(layer["out"]),
                            "kernel": layer["kernel"], "stride": layer["stride"], "us": round(ms * 1e3, 2),
                            "tops": round(2.0 * layer["macs"] / (ms * 1e-3) / 1e12, 2),
                            "gbs": round(layer["bytes"] / (ms * 1e-3) / 1e9, 1)})
-        dense = [(l, spec.layers[l["index"]]) for l in layers if l["kind"] in ("conv", "fc")]
-        band = [(l, spec.layers[l["index"]]) for l in layers if l["kind"] in ("dw", "avgpool")]
+        # a launch that holds a CONV2D or MATMUL (also the expansion + depthwise pairs) is priced against the matrix
+        # cores, a stand-alone DEPTHWISE_CONV2D or AVG_POOL2D against HBM
+        dense = [(l, launches[l["index"]]) for l in layers if l["kind"] in ("conv", "fc", "conv+dw")]
+        band = [(l, launches[l["index"]]) for l in layers if l["kind"] in ("dw", "avgpool")]
 
         def total(group, key):
             return float(sum(meta[key] for _, meta in group))

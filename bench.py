@@ -169,7 +169,8 @@ def cpu_baseline_mobilenetv2(abi, budget_s=10.0):
 
 
 def run_layer(dev, abi, index, reps=200):
-    """One operator of the fused config 3 graph, launched `reps` times back to back (for counter collection)."""
+    """One launch of the fused config 3 graph (position `index` among its launches), `reps` times back to back (for
+    counter collection)."""
     graphs = importlib.import_module(PKG + ".graphs")
     spec = graphs.mobilenetv2_spec(batch=32)
     g = graphs.build(dev, spec, fuse=True)
@@ -177,7 +178,10 @@ def run_layer(dev, abi, index, reps=200):
     g.dispatch()
     dev.sync()
     ms = graphs.time_operators(dev, g, reps=reps, only=[index])[index]
-    layer = spec.layers[index]
+    launches = graphs.launch_layers(g, spec)
+    if launches is None:
+        raise SystemExit("bench.py: the fused graph's launches do not line up with the layers of its specification")
+    layer = launches[index]
     res = {"layer": index, "name": g.op_name(index), "kind": layer["kind"], "in": list(layer["in"]),
            "out": list(layer["out"]), "us": ms * 1e3, "launches": reps + 3 + 1,
            "tops": 2.0 * layer["macs"] / (ms * 1e-3) / 1e12, "algorithmic_bytes": layer["bytes"],
