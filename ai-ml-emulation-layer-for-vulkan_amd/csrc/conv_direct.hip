@@ -459,6 +459,225 @@ int try_rows_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const ml
     return 1;
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// STEM on the matrix cores: 3x3 CONV2D over 3-byte pixels (an RGB image stem, K = 27) + RESCALE (+CLAMP) to 8 bits
+// with 16 or 32 output channels.  The structure of conv_rows_mfma_i8_kernel (a wavefront owns 32 consecutive output
+// positions and all channels, weights in registers, per-wavefront staging tile), with one v_mfma_i32_32x32x32_i8 per
+// group and an operand fetch that gathers the patch: k = 9 ky + 3 kx + c, so a patch row is 9 consecutive bytes of
+// the image.  Lane (position, half) supplies k = 16 half .. 16 half + 15: it loads the two patch rows it needs
+// (half 0: rows 0 and 1, half 1: rows 1 and 2) as three dwords each around the unaligned 9 bytes, shifts them into
+// place (v_alignbyte_b32), replaces the bytes of pixels outside the image by the input zero point (such taps then
+// contribute nothing) and takes 16 bytes of the stream [row a, row b, zeros] from byte 0 or 7.  The weights of
+// k = 27 .. 31 are zero.
+// ---------------------------------------------------------------------------------------------------------------
+struct StemMfmaArgs {
+    const int8_t *x, *w;
+    const int32_t *bias;
+    char *out;
+    int32_t M, OC, H, W, OW, OHW, zx, bias_len;
+    int32_t sy, sx, pad_t, pad_l;
+    uint32_t ow_magic;  // floor(2^32 / OW) + 1: x / OW == umulhi(x, magic) while x * OW < 2^32 (the host checks)
+    int32_t groups, op;
+    uint32_t x_bytes, o_bytes;
+    ScaleRef scale;
+};
+
+__global__ void __launch_bounds__(kBlock) conv_stem_mfma_i8_kernel(const StemMfmaArgs a) {
+    extern __shared__ __align__(16) char smem[];
+    ChanConst *cc = reinterpret_cast<ChanConst *>(smem);  // [32], channels at or beyond OC hold zeros
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cl = lane & 31, half = lane >> 5;
+    const __amdgpu_buffer_rsrc_t xres =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(a.x), 0, (int)a.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ores = __builtin_amdgcn_make_buffer_rsrc(a.out, 0, (int)a.o_bytes, 0x00020000);
+    const uint32_t kOob = 0x80000000u;
+    const uint32_t zsplat = (uint32_t)(uint8_t)a.zx * 0x01010101u;
+
+    // the six dwords around the lane's two patch rows, and what is needed to put them in place afterwards
+    struct Patch {
+        uint32_t d[2][3];
+        uint32_t shift;       // byte offset of the patch row inside its first dword
+        uint32_t m0, m1, m2;  // which bytes of a row are inside the image (by pixel), per dword of the shifted row
+        bool row_in[2];
+    };
+    auto fetch = [&](int g, Patch &p) {
+        const int m = g * 32 + cl;
+        const bool live = g < a.groups && m < a.M;
+        // image and position inside it: the group's first position is divided on the scalar side (g is uniform),
+        // a lane is at most one image further (an image has at least 32 positions)
+        const uint32_t m0 = (uint32_t)__builtin_amdgcn_readfirstlane(g) * 32u;
+        uint32_t n = m0 / (uint32_t)a.OHW;
+        uint32_t rem = m0 - n * (uint32_t)a.OHW + (uint32_t)cl;
+        if (rem >= (uint32_t)a.OHW) rem -= (uint32_t)a.OHW, n++;
+        const uint32_t oy = __umulhi(rem, a.ow_magic), ox = rem - oy * (uint32_t)a.OW;
+        const int iy0 = (int)oy * a.sy - a.pad_t + half, ix0 = (int)ox * a.sx - a.pad_l;
+        const bool px0 = (unsigned)ix0 < (unsigned)a.W, px1 = (unsigned)(ix0 + 1) < (unsigned)a.W,
+                   px2 = (unsigned)(ix0 + 2) < (unsigned)a.W;
+        p.m0 = (px0 ? 0x00ffffffu : 0u) | (px1 ? 0xff000000u : 0u);
+        p.m1 = (px1 ? 0x0000ffffu : 0u) | (px2 ? 0xffff0000u : 0u);
+        p.m2 = px2 ? 0x000000ffu : 0u;
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const int iy = iy0 + r;
+            p.row_in[r] = live && (unsigned)iy < (unsigned)a.H;
+            // byte address of pixel (iy, ix0); a negative ix0 names bytes before the row, which the masks discard
+            const int32_t addr = (int32_t)((n * (uint32_t)a.H + (uint32_t)iy) * (uint32_t)a.W) * 3 + ix0 * 3;
+            const int32_t base = addr & ~3;
+            if (r == 0) p.shift = (uint32_t)addr & 3u;
+#pragma unroll
+            for (int k = 0; k < 3; k++) {
+                const int32_t off = base + 4 * k;
+                p.d[r][k] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(xres, (p.row_in[r] && off >= 0) ? off : (int)kOob, 0, 0);
+            }
+        }
+    };
+    // rows of a lane start at the same column, and consecutive rows are W * 3 bytes apart: the shift of row 1 is
+    // (shift of row 0 + 3 W) & 3, worked out in place below
+    auto operand = [&](const Patch &p) -> v4i32 {
+        uint32_t q[2][3];
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const uint32_t sh = (p.shift + (uint32_t)(r * 3 * a.W)) & 3u;
+            const uint32_t q0 = __builtin_amdgcn_alignbyte(p.d[r][1], p.d[r][0], sh);
+            const uint32_t q1 = __builtin_amdgcn_alignbyte(p.d[r][2], p.d[r][1], sh);
+            const uint32_t q2 = __builtin_amdgcn_alignbyte(0u, p.d[r][2], sh);
+            const uint32_t m0 = p.row_in[r] ? p.m0 : 0u, m1 = p.row_in[r] ? p.m1 : 0u, m2 = p.row_in[r] ? p.m2 : 0u;
+            q[r][0] = (q0 & m0) | (zsplat & ~m0);
+            q[r][1] = (q1 & m1) | (zsplat & ~m1);
+            q[r][2] = (q2 & m2) | (zsplat & ~m2);  // byte 0 = byte 8 of the row
+        }
+        // the stream [a0 .. a8, b0 .. b8, 0 ...] as dwords
+        const uint32_t s0 = q[0][0], s1 = q[0][1];
+        const uint32_t s2 = __builtin_amdgcn_perm(q[1][0], q[0][2], 0x06050400u);      // a8 b0 b1 b2
+        const uint32_t s3 = __builtin_amdgcn_alignbyte(q[1][1], q[1][0], 3u);           // b3 b4 b5 b6
+        const uint32_t s4 = __builtin_amdgcn_perm(q[1][2], q[1][1], 0x0c0c0403u);      // b7 b8 0 0
+        // half 0 takes bytes 0 .. 15, half 1 bytes 7 .. 22
+        v4i32 f;
+        if (half == 0) {
+            f = v4i32{(int)s0, (int)s1, (int)s2, (int)s3};
+        } else {
+            f = v4i32{(int)__builtin_amdgcn_alignbyte(s2, s1, 3u), (int)__builtin_amdgcn_alignbyte(s3, s2, 3u),
+                      (int)__builtin_amdgcn_alignbyte(s4, s3, 3u), (int)__builtin_amdgcn_alignbyte(0u, s4, 3u)};
+        }
+        return f;
+    };
+
+    const int nwaves = (int)gridDim.x * (kBlock / 64);
+    int g = (int)blockIdx.x * (kBlock / 64) + wave;
+    Patch cur, nxt;
+    fetch(g, cur);
+    // ---- the weights as matrix B operand: lane = channel lane % 32, bytes k = 16 half .. 16 half + 15 (k < 27)
+    v4i32 wf;
+    {
+        uint32_t wd[4] = {0, 0, 0, 0};
+        if (cl < a.OC) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                const int kk = 16 * half + k;
+                if (kk < 27) wd[k >> 2] |= (uint32_t)(uint8_t)a.w[cl * 27 + kk] << (8 * (k & 3));
+            }
+        }
+        wf = v4i32{(int)wd[0], (int)wd[1], (int)wd[2], (int)wd[3]};
+    }
+    // ---- per-channel constants (the input zero point folded into the bias term)
+    if (tid < 32) {
+        ChanConst c{};
+        if (tid < a.OC) {
+            int32_t wsum = 0;
+            for (int k = 0; k < 27; k++) wsum += (int32_t)a.w[tid * 27 + k];
+            const int32_t bias = a.bias[a.bias_len == 1 ? 0 : tid];
+            c.bias_adj = (int32_t)((uint32_t)bias - (uint32_t)a.zx * (uint32_t)wsum);
+            const int ci = a.scale.p.per_channel ? tid : 0;
+            c.q = make_chan_scale(load_mult(a.scale, ci), (int32_t)a.scale.shift[ci], a.scale.p);
+        }
+        cc[tid] = c;
+    }
+    __syncthreads();
+    const ChanConst c = cc[cl];
+    char *so = smem + 32 * sizeof(ChanConst) + wave * 32 * a.op;  // this wavefront's staging tile [32][op]
+    const int ppr = a.OC >> 4, npieces = 32 * ppr;                 // 16-byte pieces per row / per tile (at most 64)
+    const int prow = lane / ppr;
+    const uint32_t piece_row = lane < npieces ? (uint32_t)prow : 0xffffu;
+    const uint32_t piece_lds = lane < npieces ? (uint32_t)(prow * a.op + (lane - prow * ppr) * 16) : 0u;
+    const uint32_t sel_a = (lane & 1) ? 0x03070105u : 0x06020400u;  // exchange with lane ^ 1
+    const uint32_t sel_b = (lane & 2) ? 0x03020706u : 0x05040100u;  // exchange with lane ^ 2
+    char *so_lane = so + (4 * half + (lane & 3)) * a.op + (cl & ~3);
+    const bool col_live = (cl & ~3) < a.OC;
+    for (; g < a.groups; g += nwaves) {
+        fetch(g + nwaves, nxt);
+        const v4i32 xf = operand(cur);
+        v16i32 acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = c.bias_adj;
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf, wf, acc, 0, 0, 0);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            int32_t v[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[4 * q + e], c.q, a.scale.p);
+            const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
+            const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
+            uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // bytes = positions e of this lane's channel
+            uint32_t o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0xb1, 0xf, 0xf, true);
+            p = __builtin_amdgcn_perm(o, p, sel_a);
+            o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0x4e, 0xf, 0xf, true);
+            p = __builtin_amdgcn_perm(o, p, sel_b);
+            // now: position 8 q + 4 (lane / 32) + lane % 4, channels 4 (lane % 32 / 4) .. + 3
+            if (col_live) *reinterpret_cast<uint32_t *>(so_lane + 8 * q * a.op) = p;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const uint32_t rows = (uint32_t)min(32, a.M - g * 32);
+        const uint4 d = *reinterpret_cast<const uint4 *>(so + piece_lds);
+        const uint32_t off = piece_row < rows ? (uint32_t)g * 32u * (uint32_t)a.OC + (uint32_t)lane * 16u : kOob;
+        __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, 0);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        cur = nxt;
+    }
+}
+
+// returns 1 when the case was taken
+int try_stem_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
+                  const mlel_tensor *bias, const mlel_conv2d_attr *a, const FusedEpilogue *epi, int64_t M, int64_t xbytes) {
+    const int64_t OH = out->dims[1], OW = out->dims[2], OC = out->dims[3], H = in->dims[1], W = in->dims[2];
+    if (epi == nullptr || a->weight_zp != 0 || in->dims[3] != 3 || w->dims[1] != 3 || w->dims[2] != 3) return 0;
+    if ((OC != 16 && OC != 32) || ((uintptr_t)in->ptr % 4) != 0) return 0;
+    // dense image: rows of W * 3 bytes, images of H rows
+    if (in->strides[2] != 3 || in->strides[1] != W * 3 || in->strides[0] != H * W * 3) return 0;
+    if (a->stride[0] < 1 || a->stride[0] > 4 || a->stride[1] < 1 || a->stride[1] > 4) return 0;
+    if (a->pad[0] < 0 || a->pad[0] > 4 || a->pad[2] < 0 || a->pad[2] > 4) return 0;
+    // the quotient by the magic number is exact while dividend * divisor < 2^32; an image holds at least one group
+    if (OH * OW * OW >= (int64_t(1) << 32) || OH * OW < 32 || OW < 2) return 0;
+    if (xbytes >= (int64_t(1) << 31) - 16 || M * OC >= (int64_t(1) << 31)) return 0;
+    StemMfmaArgs g{};
+    g.x = static_cast<const int8_t *>(in->ptr);
+    g.w = static_cast<const int8_t *>(w->ptr);
+    g.bias = static_cast<const int32_t *>(bias->ptr);
+    g.out = static_cast<char *>(out->ptr);
+    g.M = (int)M, g.OC = (int)OC, g.H = (int)H, g.W = (int)W, g.OW = (int)OW, g.OHW = (int)(OH * OW);
+    g.zx = a->input_zp;
+    g.bias_len = (int)bias->dims[0];
+    g.sy = a->stride[0], g.sx = a->stride[1], g.pad_t = a->pad[0], g.pad_l = a->pad[2];
+    g.ow_magic = (uint32_t)((uint64_t(1) << 32) / (uint64_t)g.OW + 1);
+    g.groups = (int)((M + 31) / 32);
+    int op = (int)OC;
+    while (op % 128 != 32 && op % 128 != 96) op += 16;  // as in the rows kernel
+    g.op = op;
+    g.x_bytes = (uint32_t)((xbytes + 3) & ~int64_t(3));
+    g.o_bytes = (uint32_t)(M * OC);
+    g.scale = make_ref(*epi);
+    const size_t sm = 32 * sizeof(ChanConst) + (size_t)(kBlock / 64) * 32 * g.op;
+    const int cus = ctx != nullptr && ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
+    const int64_t per_wave = (g.groups + kBlock / 64 - 1) / (kBlock / 64);
+    const int64_t want =
+        std::min<int64_t>(per_wave, std::min<int64_t>((int64_t)cus * 3, std::max<int64_t>((int64_t)cus * 2, (g.groups + 15) / 16)));
+    conv_stem_mfma_i8_kernel<<<dim3((unsigned)std::max<int64_t>(want, 1)), dim3(kBlock), sm, s>>>(g);
+    return 1;
+}
+
 }  // namespace
 
 int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in,
@@ -506,6 +725,10 @@ int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, c
         return 1;
     }
     if (mode < 0) return 0;
+    if (mode == STEM && IC == 3 && M > 0 && try_stem_mfma(ctx, s, out, in, w, bias, a, epi, M, xbytes)) {
+        MLEL_TRY(check_launch("conv2d stem int8"));
+        return 1;
+    }
 
     DirectArgs g{};
     g.x = static_cast<const int8_t *>(in->ptr);

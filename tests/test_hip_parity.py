@@ -141,6 +141,10 @@ CONV_CASES = [
     ("stem_ic3_s1_pad1_zw", (2, 11, 13, 3), 16, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -128, 5),
     ("stem_ic3_s2_big", (3, 33, 31, 3), 32, (3, 3), (1, 0, 1, 0), (2, 2), (1, 1), 127, 0),
     ("stem_ic1", (2, 9, 10, 1), 16, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), 3, -3),
+    ("stem_ic3_s1_pad1_16ch", (2, 12, 14, 3), 16, (3, 3), (1, 1, 1, 1), (1, 1), (1, 1), -9, 0),
+    ("stem_ic3_s3_pad2", (1, 20, 23, 3), 32, (3, 3), (2, 1, 2, 0), (3, 3), (1, 1), 5, 0),
+    ("stem_ic3_tall_s1x2", (3, 70, 9, 3), 32, (3, 3), (1, 1, 1, 1), (1, 2), (1, 1), -128, 0),
+    ("stem_ic3_images_of_40", (5, 10, 12, 3), 32, (3, 3), (0, 0, 1, 1), (2, 1), (1, 1), 1, 0),
     ("stem_ic4_s3", (1, 14, 15, 4), 48, (3, 3), (2, 1, 0, 2), (3, 2), (1, 1), -7, 1),
     ("pw_32_16_zw", (2, 12, 12, 32), 16, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 6, -6),
     ("pw_32_192", (1, 28, 28, 32), 192, (1, 1), (0, 0, 0, 0), (1, 1), (1, 1), -100, 0),
