@@ -754,6 +754,21 @@ def test_fused_epilogue_with_nonzero_input_zero_point_vs_oracle(run, oracle):
         np.testing.assert_array_equal(mgot, mexp)
 
 
+def test_fp16_product_on_the_256_tile_equals_its_halves(run):
+    """4096 x 768 x 3072 runs on the 256 x 256 tile of eight wavefronts; each half of its columns alone runs on the
+    128 x 128 tile.  The order of the additions along K is the same in both, so the bits are."""
+    rng = np.random.default_rng(31)
+    a = (rng.standard_normal((1, 4096, 768)) * 0.5).astype(np.float16)
+    b = (rng.standard_normal((1, 768, 3072)) * 0.05).astype(np.float16)
+    bias = rng.standard_normal((1, 1, 3072)).astype(np.float32)
+    whole = run.matmul_bias_cast(a, b, bias)
+    left = run.matmul_bias_cast(a, np.ascontiguousarray(b[:, :, :1536]), np.ascontiguousarray(bias[:, :, :1536]))
+    right = run.matmul_bias_cast(a, np.ascontiguousarray(b[:, :, 1536:]), np.ascontiguousarray(bias[:, :, 1536:]))
+    np.testing.assert_array_equal(whole.view(np.uint16), np.concatenate([left, right], axis=2).view(np.uint16))
+    ref = (a[0, :64].astype(np.float64) @ b[0].astype(np.float64) + bias[0, 0]).astype(np.float32)
+    assert np.max(np.abs(whole[0, :64].astype(np.float32) - ref)) <= 1e-2
+
+
 # ------------------------------------------------------------------------------------------------ RESCALE & co
 @pytest.mark.parametrize("double_round", [False, True])
 @pytest.mark.parametrize("per_channel", [False, True])
