@@ -699,6 +699,68 @@ def test_conv2d_dwconv_one_launch_vs_oracle(run, oracle, case):
     np.testing.assert_array_equal(got, exp)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_conv2d_dwconv_one_launch_random_shapes(run, oracle, seed):
+    """Extents, strides, paddings and zero points drawn at random inside what the kernel takes (bands, partial
+    strips, odd widths, one to five 32-byte pieces per pixel)."""
+    rng = np.random.default_rng(9000 + seed)
+    stride = int(rng.integers(1, 3))
+    h, w_ = int(rng.integers(3, 33)), int(rng.integers(3, 33))
+    ic, c = 32 * int(rng.integers(1, 6)), 32 * int(rng.integers(1, 4))
+    n = int(rng.integers(1, 4))
+    pad = tuple(int(v) for v in rng.integers(0, 3, size=4))
+    zx, zi = int(rng.integers(-128, 128)), int(rng.integers(-128, 128))
+    oh, ow = out_hw(h, w_, (3, 3), pad, (stride, stride), (1, 1))
+    if oh < 1 or ow < 1:
+        pytest.skip("no output position")
+    x = ri(rng, -128, 127, (n, h, w_, ic), np.int8)
+    w1 = ri(rng, -128, 127, (c, 1, 1, ic), np.int8)
+    b1 = ri(rng, -2 ** 12, 2 ** 12, (c,), np.int32)
+    w2 = ri(rng, -128, 127, (3, 3, c, 1), np.int8)
+    b2 = ri(rng, -2 ** 10, 2 ** 10, (c,), np.int32)
+    per_channel = bool(rng.integers(0, 2))
+    k = c if per_channel else 1
+    m1, s1 = ri(rng, 2 ** 30, 2 ** 31 - 1, (k,), np.int32), ri(rng, 40, 44, (k,), np.int8)
+    m2, s2 = ri(rng, 2 ** 30, 2 ** 31 - 1, (k,), np.int32), ri(rng, 36, 39, (k,), np.int8)
+    a1 = abi.conv2d_attr((0, 0, 0, 0), (1, 1), (1, 1), zx, 0)
+    a2 = abi.conv2d_attr(pad, (stride, stride), (1, 1), zi, 0)
+    double_round = bool(rng.integers(0, 2))
+    r1 = abi.rescale_attr(0, zi, True, double_round, per_channel)
+    r2 = abi.rescale_attr(0, int(rng.integers(-20, 20)), True, double_round, per_channel)
+    clamp1 = (-90, 110) if rng.integers(0, 2) else None
+    mid_shape, out_shape = (n, h, w_, c), (n, oh, ow, c)
+    mid = oracle.rescale(oracle.conv2d(x, w1, b1, mid_shape, abi.I32, a1), m1, s1, abi.I8, r1)
+    if clamp1:
+        mid = oracle.clamp(mid, *clamp1)
+    exp = oracle.rescale(oracle.depthwise_conv2d(mid, w2, b2, out_shape, abi.I32, a2), m2, s2, abi.I8, r2)
+    covered, got = run.conv2d_dwconv(x, w1, b1, a1, (m1, s1, r1, clamp1), w2, b2, a2, (m2, s2, r2, None), out_shape)
+    assert covered == 1
+    np.testing.assert_array_equal(got, exp)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_rgb_stem_random_shapes(run, oracle, seed):
+    """The 3x3 convolution over 3-byte pixels on the matrix cores: extents, strides and paddings drawn at random."""
+    rng = np.random.default_rng(9100 + seed)
+    n, h, w_ = int(rng.integers(1, 4)), int(rng.integers(8, 40)), int(rng.integers(8, 40))
+    oc = 16 * int(rng.integers(1, 3))
+    stride = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+    pad = tuple(int(v) for v in rng.integers(0, 3, size=4))
+    zx = int(rng.integers(-128, 128))
+    oh, ow = out_hw(h, w_, (3, 3), pad, stride, (1, 1))
+    x = ri(rng, -128, 127, (n, h, w_, 3), np.int8)
+    w = ri(rng, -128, 127, (oc, 3, 3, 3), np.int8)
+    b = ri(rng, -2 ** 12, 2 ** 12, (oc,), np.int32)
+    mult, shift = ri(rng, 2 ** 30, 2 ** 31 - 1, (oc,), np.int32), ri(rng, 38, 42, (oc,), np.int8)
+    attr = abi.conv2d_attr(pad, stride, (1, 1), zx, 0)
+    rattr = abi.rescale_attr(0, int(rng.integers(-20, 20)), True, bool(rng.integers(0, 2)), True)
+    shape = (n, oh, ow, oc)
+    exp = oracle.clamp(oracle.rescale(oracle.conv2d(x, w, b, shape, abi.I32, attr), mult, shift, abi.I8, rattr), -100, 120)
+    got = run.conv2d(x, w, b, shape, abi.I8, attr, epilogue=(mult, shift, rattr, (-100, 120)))
+    np.testing.assert_array_equal(got, exp)
+    assert len(np.unique(got)) > 20
+
+
 def test_conv2d_dwconv_declines_what_the_kernel_was_not_written_for(run):
     rng = np.random.default_rng(5)
 
