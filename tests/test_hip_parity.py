@@ -252,6 +252,11 @@ DL_CASES = [
     ("tile128_batched", 16, 640, 320, 1024, 0, -6),       # 5 x 8 tiles per batch, five K steps
     ("tile128_ring_once", 8, 512, 576, 1024, -1, 3),      # nine K steps: the eight-stage ring is filled and refilled
     ("tile128_ring_wraps", 4, 1024, 1600, 1024, 4, -2),   # 25 K steps: the ring wraps three times and drains
+    # exactly one 128 x 128 tile per compute unit of a 256-CU device (config 1's geometry), even numbers of K steps
+    ("tile128_one_per_cu_4_steps", 8, 512, 256, 1024, -2, 5),
+    ("tile128_one_per_cu_no_zp", 8, 512, 384, 1024, 0, 0),
+    ("tile128_one_per_cu_18_steps", 4, 1024, 1152, 1024, -7, -1),
+    ("tile128_one_per_cu_ragged", 1, 2000, 512, 2032, 1, 2),      # partial last tile row and column
 ]
 
 
