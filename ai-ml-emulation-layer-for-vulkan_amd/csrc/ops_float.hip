@@ -412,6 +412,121 @@ bool classify(const mlel_tensor *out, const mlel_tensor *in, int *varies_row, in
     return ((uintptr_t)in->ptr % align) == 0;
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same for the reduced-precision storage types (bf16, fp8 e4m3 / e5m2; reference codecs common.comp:184-611):
+// ADD, SUB, MUL and CAST, eight elements per thread with one 64-, 128- or 2 x 128-bit access per operand.  Every
+// element goes through the codec functions of the generic kernels (decode to fp32, one operation, raw_st_f's
+// rounding rule for the operator), so the results are theirs to the bit.
+// ---------------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float lowp_decode(int dt, uint32_t bits) {
+    switch (dt) {
+    case MLEL_F16: return __half2float(__ushort_as_half((unsigned short)bits));
+    case MLEL_BF16: return decode_bf16((uint16_t)bits);
+    case MLEL_F8E4M3: return decode_f8e4m3((uint8_t)bits);
+    case MLEL_F8E5M2: return decode_f8e5m2((uint8_t)bits);
+    default: return __uint_as_float(bits);
+    }
+}
+__device__ __forceinline__ uint32_t lowp_encode(int dt, float v, int mode) {
+    switch (dt) {
+    case MLEL_F16: return (uint32_t)__half_as_ushort(f2h(v));
+    case MLEL_BF16: return mode == ST_RNE ? encode_bf16_rne(v) : encode_bf16_trunc(v);
+    case MLEL_F8E4M3:
+    case MLEL_F8E5M2: return encode_f8(dt, mode == ST_ACC ? v : __half2float(f2h(v)));
+    default: return __float_as_uint(v);
+    }
+}
+// eight consecutive elements of `size` bytes each as dwords (size 1: two, 2: four, 4: eight)
+template <int SIZE>
+__device__ __forceinline__ void lowp_load8(const char *base, int dt, int64_t row, int32_t c8, int32_t cols, int varies_row,
+                                           int varies_col, float (&v)[8]) {
+    const int64_t r = varies_row ? row : 0;
+    if (!varies_col) {
+        const char *p = base + r * SIZE;
+        const uint32_t bits = SIZE == 1 ? *reinterpret_cast<const uint8_t *>(p)
+                                        : (SIZE == 2 ? *reinterpret_cast<const uint16_t *>(p) : *reinterpret_cast<const uint32_t *>(p));
+        const float s = lowp_decode(dt, bits);
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = s;
+        return;
+    }
+    const char *p = base + (r * cols + (int64_t)c8 * 8) * SIZE;
+    uint32_t w[2 * SIZE];
+    if (SIZE == 1) {
+        const uint2 raw = *reinterpret_cast<const uint2 *>(p);
+        w[0] = raw.x, w[1] = raw.y;
+    } else {
+#pragma unroll
+        for (int k = 0; k < SIZE / 2; k++) {
+            const uint4 raw = *reinterpret_cast<const uint4 *>(p + 16 * k);
+            w[4 * k] = raw.x, w[4 * k + 1] = raw.y, w[4 * k + 2] = raw.z, w[4 * k + 3] = raw.w;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t bits = SIZE == 1 ? (w[i >> 2] >> (8 * (i & 3))) & 0xffu
+                                        : (SIZE == 2 ? (w[i >> 1] >> (16 * (i & 1))) & 0xffffu : w[i]);
+        v[i] = lowp_decode(dt, bits);
+    }
+}
+template <int SIZE>
+__device__ __forceinline__ void lowp_store8(char *p, int dt, int mode, const float (&v)[8]) {
+    uint32_t w[2 * SIZE];
+#pragma unroll
+    for (int k = 0; k < 2 * SIZE; k++) w[k] = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t bits = lowp_encode(dt, v[i], mode);
+        if (SIZE == 1) w[i >> 2] |= (bits & 0xffu) << (8 * (i & 3));
+        else if (SIZE == 2) w[i >> 1] |= (bits & 0xffffu) << (16 * (i & 1));
+        else w[i] = bits;
+    }
+    if (SIZE == 1) {
+        *reinterpret_cast<uint2 *>(p) = make_uint2(w[0], w[1]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < SIZE / 2; k++) *reinterpret_cast<uint4 *>(p + 16 * k) = make_uint4(w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3]);
+    }
+}
+
+template <int OP, int IN_SIZE, int OUT_SIZE>
+__global__ void __launch_bounds__(kBlock) ew_lowp_kernel(const EwArgs g, int in_dt, int out_dt, int mode) {
+    const int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (v >= g.vecs) return;
+    const int64_t row = v / g.cols8;
+    const int32_t c8 = (int32_t)(v - row * g.cols8);
+    float a[8], b[8], r[8];
+    lowp_load8<IN_SIZE>(g.a, in_dt, row, c8, g.cols, g.a_row, g.a_col, a);
+    if (OP != F_COPY) lowp_load8<IN_SIZE>(g.b, in_dt, row, c8, g.cols, g.b_row, g.b_col, b);
+#pragma unroll
+    for (int i = 0; i < 8; i++) r[i] = OP == F_ADD ? a[i] + b[i] : (OP == F_SUB ? a[i] - b[i] : (OP == F_MUL ? a[i] * b[i] : a[i]));
+    lowp_store8<OUT_SIZE>(g.out + v * 8 * OUT_SIZE, out_dt, mode, r);
+}
+
+bool lowp_dt(int dt) { return dt == MLEL_BF16 || dt == MLEL_F8E4M3 || dt == MLEL_F8E5M2; }
+
+template <int OP>
+int launch_lowp(hipStream_t s, const EwArgs &g, int in_dt, int out_dt, int mode) {
+    const int64_t blocks = (g.vecs + kBlock - 1) / kBlock;
+    MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "elementwise: too many work items");
+    const dim3 grid((unsigned)blocks), block(kBlock);
+    const int is = dt_size(in_dt), os = dt_size(out_dt);
+#define MLEL_LOWP_CASE(IS, OS) \
+    if (is == IS && os == OS) ew_lowp_kernel<OP, IS, OS><<<grid, block, 0, s>>>(g, in_dt, out_dt, mode)
+    MLEL_LOWP_CASE(1, 1);
+    else MLEL_LOWP_CASE(2, 2);
+    else MLEL_LOWP_CASE(1, 2);
+    else MLEL_LOWP_CASE(1, 4);
+    else MLEL_LOWP_CASE(2, 1);
+    else MLEL_LOWP_CASE(2, 4);
+    else MLEL_LOWP_CASE(4, 1);
+    else MLEL_LOWP_CASE(4, 2);
+    else return 0;
+#undef MLEL_LOWP_CASE
+    MLEL_TRY(check_launch("elementwise reduced precision"));
+    return 1;
+}
+
 template <int OP>
 int launch_ew(hipStream_t s, const EwArgs &g, int in_size, int out_size) {
     const int64_t blocks = (g.vecs + kBlock - 1) / kBlock;
@@ -454,7 +569,14 @@ bool describe(const mlel_tensor *out, const mlel_tensor *a, const mlel_tensor *b
 
 int try_binary_float_fast(mlel_ctx *, hipStream_t s, int op, const mlel_tensor *out, const mlel_tensor *in1,
                           const mlel_tensor *in2) {
-    if (!float_dt(out->dtype) || in1->dtype != out->dtype || in2->dtype != out->dtype) return 0;
+    if (in1->dtype != out->dtype || in2->dtype != out->dtype) return 0;
+    if (lowp_dt(out->dtype)) {  // ADD and SUB round to nearest even into the storage type (binary_generic)
+        EwArgs l{};
+        if ((op != MLEL_BIN_ADD && op != MLEL_BIN_SUB) || !describe(out, in1, in2, &l)) return 0;
+        return op == MLEL_BIN_ADD ? launch_lowp<F_ADD>(s, l, out->dtype, out->dtype, ST_RNE)
+                                  : launch_lowp<F_SUB>(s, l, out->dtype, out->dtype, ST_RNE);
+    }
+    if (!float_dt(out->dtype)) return 0;
     EwArgs g{};
     if (!describe(out, in1, in2, &g)) return 0;
     const int sz = dt_size(out->dtype);
@@ -467,7 +589,13 @@ int try_binary_float_fast(mlel_ctx *, hipStream_t s, int op, const mlel_tensor *
 
 int try_mul_float_fast(mlel_ctx *, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in1,
                        const mlel_tensor *in2) {
-    if (!float_dt(out->dtype) || in1->dtype != out->dtype || in2->dtype != out->dtype) return 0;
+    if (in1->dtype != out->dtype || in2->dtype != out->dtype) return 0;
+    if (lowp_dt(out->dtype)) {  // operands of the output's type are their own rounding (mul_generic)
+        EwArgs l{};
+        if (!describe(out, in1, in2, &l)) return 0;
+        return launch_lowp<F_MUL>(s, l, out->dtype, out->dtype, ST_RNE);
+    }
+    if (!float_dt(out->dtype)) return 0;
     EwArgs g{};
     if (!describe(out, in1, in2, &g)) return 0;
     const int sz = dt_size(out->dtype);
@@ -489,7 +617,14 @@ int try_unary_float_fast(mlel_ctx *, hipStream_t s, int op, const mlel_tensor *o
 }
 
 int try_cast_float_fast(mlel_ctx *, hipStream_t s, const mlel_tensor *out, const mlel_tensor *in) {
-    if (!float_dt(out->dtype) || !float_dt(in->dtype) || in->dtype == out->dtype || !same_shape(out, in)) return 0;
+    if (in->dtype == out->dtype || !same_shape(out, in)) return 0;
+    if ((lowp_dt(out->dtype) && (lowp_dt(in->dtype) || float_dt(in->dtype))) || (lowp_dt(in->dtype) && float_dt(out->dtype))) {
+        // to bf16: round to nearest even; to fp8: the fp32 value is encoded directly (cast_generic)
+        EwArgs l{};
+        if (!describe(out, in, nullptr, &l)) return 0;
+        return launch_lowp<F_COPY>(s, l, in->dtype, out->dtype, out->dtype == MLEL_BF16 ? ST_RNE : ST_ACC);
+    }
+    if (!float_dt(out->dtype) || !float_dt(in->dtype)) return 0;
     EwArgs g{};
     if (!describe(out, in, nullptr, &g)) return 0;
     return launch_ew<F_COPY>(s, g, dt_size(in->dtype), dt_size(out->dtype));

@@ -207,6 +207,11 @@ def bench_standalone(dev, abi, reps=100):
     t_m, t_s, t_tab = dev.from_numpy(mult), dev.from_numpy(shift), dev.from_numpy(tab)
     o8, o32 = dev.tensor(abi.I8, shape), dev.tensor(abi.I32, shape)
     o_pool = dev.tensor(abi.I8, (16, 28, 28, 144))
+    # reduced-precision storage: bf16 values as the upper halves of fp32 numbers, fp32 values inside e4m3's range
+    f32 = (rng.standard_normal(shape) * 20).astype(np.float32)
+    bf = (f32.view(np.uint32) >> 16).astype(np.uint16)
+    t_bf1, t_bf2, t_f32 = dev.from_numpy(bf, abi.BF16), dev.from_numpy(bf[::-1].copy(), abi.BF16), dev.from_numpy(f32)
+    o_bf, o_f8 = dev.tensor(abi.BF16, shape), dev.tensor(abi.F8E4M3, shape)
     r_down = abi.rescale_attr(0, 3, True, True, True)
     r_up = abi.rescale_attr(-5, 0, True, True, True)
     clamp = abi.ClampAttr(0.0, 96.0, int(abi.NAN_PROPAGATE))
@@ -221,6 +226,9 @@ def bench_standalone(dev, abi, reps=100):
                                              int(abi.NAN_PROPAGATE))),
         ("TABLE int8", 2 * n, lambda: dev.op("table", o8.ref, t_x8.ref, t_tab.ref)),
         ("MAX_POOL2D int8 3x3 stride 2", n + n // 4, lambda: dev.op("max_pool2d", o_pool.ref, t_x8.ref, C.byref(pool))),
+        ("ADD bf16", 6 * n, lambda: dev.op("elementwise_binary", abi.BIN["ADD"], o_bf.ref, t_bf1.ref, t_bf2.ref,
+                                           int(abi.NAN_PROPAGATE))),
+        ("CAST fp32->fp8 e4m3", 5 * n, lambda: dev.op("cast", o_f8.ref, t_f32.ref)),
     ]
     out = []
     ev0, ev1 = dev.event(), dev.event()

@@ -275,6 +275,31 @@ def test_hip_elementwise_cast_reduce_in_low_precision_formats(run, oracle, dt):
 @pytest.mark.gpu
 @pytestmark_gpu
 @pytest.mark.parametrize("dt", LOWP, ids=[NAMES[d] for d in LOWP])
+def test_hip_packed_elementwise_and_cast_in_low_precision_formats(run, oracle, dt):
+    """Dense tensors whose rows are a multiple of eight elements take the kernels with 64- / 128-bit accesses:
+    ADD, SUB, MUL (same shape, a row broadcast, a column broadcast, a single element) and CAST in both directions."""
+    rng = np.random.default_rng(50 + dt)
+    shape = (5, 7, 48)
+    a = random_codes(rng, dt, shape)
+    for b in (random_codes(rng, dt, shape), random_codes(rng, dt, (1, 1, 48)), random_codes(rng, dt, (5, 7, 1)),
+              random_codes(rng, dt, (1, 1, 1))):
+        for op in ("ADD", "SUB"):
+            np.testing.assert_array_equal(run.binary(op, a, b, shape, dt), oracle.elementwise_binary(op, a, b, shape, dt),
+                                          err_msg=f"{op} {b.shape}")
+        np.testing.assert_array_equal(run.mul(a, b, shape, dt), oracle.mul(a, b, shape, dt), err_msg=f"MUL {b.shape}")
+    for out_dt in (abi.F32, abi.F16, BF16, E4M3, E5M2):
+        if out_dt != dt:
+            np.testing.assert_array_equal(run.cast(a, out_dt), oracle.cast(a, out_dt), err_msg=f"cast to {out_dt}")
+    x = np.concatenate([sample_floats(rng, 4088, -20, 18), np.float32([0, -0.0, np.inf, -np.inf, 448, 449, 57344, 6e4])])
+    with np.errstate(over="ignore"):
+        halves = x.astype(np.float16)
+    for src in (x.reshape(8, 512), halves.reshape(64, 64)):
+        np.testing.assert_array_equal(run.cast(src, dt), oracle.cast(src, dt), err_msg=str(src.dtype))
+
+
+@pytest.mark.gpu
+@pytestmark_gpu
+@pytest.mark.parametrize("dt", LOWP, ids=[NAMES[d] for d in LOWP])
 def test_hip_contractions_pools_and_movement_in_low_precision_formats(run, oracle, dt):
     rng = np.random.default_rng(40 + dt)
     acc = abi.ACC_F32 if dt == BF16 else abi.ACC_F16
