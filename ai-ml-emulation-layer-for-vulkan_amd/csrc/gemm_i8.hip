@@ -253,6 +253,20 @@ int try_conv2d_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
         g.rs_conv = make_ref(residual->f_conv);
         g.rs_out = make_ref(residual->f_out);
     }
+    {
+        // Few tiles of a 1x1 convolution (the projections of an inverted-residual network below 56 x 56): one
+        // 32 x 32 tile per wavefront with both operands straight from memory, no LDS and no barrier (gemm_i8_cols.hip).
+        // Its operand traffic is 64 K bytes per tile, all of it from L2, so it is bounded: 64 MiB.  Measured on
+        // MobileNetV2 b32: 7.1 -> 4.6 us (96 -> 24 at 56 x 56), 5.3 -> 3.7 (144 -> 32 at 28 x 28), 9.0 -> 6.2
+        // (960 -> 160 at 7 x 7 with the residual addition), 17 launches, 19 us in all.
+        const bool q8 = g.fused && g.out_size == 1 && g.out_vec_ok && g.o_bytes != 0;
+        const bool rows = g.plain && g.xch == 16 && g.wch == 16 && g.x_bytes != 0 && g.w_bytes != 0;
+        const int64_t tiles = ((M + 31) / 32) * ((OC + 31) / 32);
+        if (q8 && rows && tiles <= 8192 && tiles * K <= (int64_t(1) << 20) && launch_conv_cols_mfma(&g, s)) {
+            MLEL_TRY(check_launch("conv2d 1x1 int8, one tile per wavefront"));
+            return 1;
+        }
+    }
     SplitScratch sc;
     if (static_scratch != nullptr) {  // the caller's region instead of the context's workspace
         sc.from_ctx = false;

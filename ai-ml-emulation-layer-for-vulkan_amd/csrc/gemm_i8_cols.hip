@@ -1,0 +1,182 @@
+// int8 1x1 CONV2D + RESCALE (+CLAMP) (+ residual ADD) for contractions whose operands can stay out of shared memory:
+// every wavefront owns one 32 x 32 output tile (32 consecutive positions x 32 consecutive channels) and streams its
+// 32 pixel rows and its 32 weight rows straight from memory into the operands of v_mfma_i32_32x32x32_i8 (lane =
+// row lane % 32, 16 bytes of K from 32 c + 16 (lane / 32)), four K chunks per round with the next round's loads in
+// flight.  No LDS, no barrier, no tile shared between wavefronts: the layers this serves (the projections of an
+// inverted-residual network below 56 x 56: a few thousand tiles of K = 144 .. 960) are chains of latencies in the
+// staged kernel (fetch, LDS round trip and barrier per 64 bytes of K), not throughput.  Arithmetic as
+// gemm_i8_kernel with a zero weight zero point: sum x w - zx * sum w + bias, requantised (reference:
+// conv2d.comp:40-116, rescale.comp:28-63, clamp.comp:18-31), then the residual stage of that kernel.
+#include "gemm_i8_kernel.hpp"
+
+namespace mlel {
+namespace {
+
+constexpr int kColsBlock = 256;
+constexpr int KR = 4;  // 32-byte K chunks per round
+
+// KS == 1: a wavefront per tile.  KS == 4 (few tiles): the four wavefronts of a block share a tile, each takes a
+// quarter of the K chunks, the partial tiles are added through shared memory (int32 addition wraps: the order is
+// immaterial) and the first wavefront requantises.
+template <bool RES, int KS>
+__global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const GemmArgs g, int groups_n, int total_waves) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wid = KS == 1 ? (int)blockIdx.x * (kColsBlock / 64) + wave : (int)blockIdx.x;
+    if (KS == 1 && wid >= total_waves) return;  // whole wavefronts leave; this form has no barrier
+    const int mg = wid / groups_n, ng = wid - mg * groups_n;
+    const int cl = lane & 31, half = lane >> 5;
+    const int m = mg * 32 + cl, n = ng * 32 + cl;
+    const __amdgpu_buffer_rsrc_t xres = make_rsrc(g.x, g.x_bytes), wres = make_rsrc(g.w, g.w_bytes);
+    const uint32_t xoff = m < g.M ? (uint32_t)m * (uint32_t)g.x_sx + (uint32_t)half * 16u : kOobOffset;
+    const uint32_t woff = n < g.N ? (uint32_t)n * (uint32_t)g.ldw + (uint32_t)half * 16u : kOobOffset;
+    auto fetch = [&](int round, v4i (&xf)[KR], v4i (&wf)[KR]) {
+#pragma unroll
+        for (int c = 0; c < KR; c++) {
+            const int k = (round * KR + c) * 32;
+            const bool in = k + half * 16 < g.K;  // K % 16 == 0: a piece lies wholly inside or outside the row
+            const uint4 xv = buf_load16(xres, (in && xoff != kOobOffset) ? xoff + (uint32_t)k : kOobOffset);
+            const uint4 wv = buf_load16(wres, (in && woff != kOobOffset) ? woff + (uint32_t)k : kOobOffset);
+            xf[c] = v4i{(int)xv.x, (int)xv.y, (int)xv.z, (int)xv.w};
+            wf[c] = v4i{(int)wv.x, (int)wv.y, (int)wv.z, (int)wv.w};
+        }
+    };
+    // rounds of this wavefront: all of them, or its quarter [first, first + rounds)
+    const int all_rounds = (g.K + KR * 32 - 1) / (KR * 32);
+    const int per = KS == 1 ? all_rounds : (all_rounds + KS - 1) / KS;
+    const int first = KS == 1 ? 0 : wave * per;
+    const int rounds = max(0, min(per, all_rounds - first));
+    v4i xa[KR], wa[KR], xb[KR], wb[KR];
+    fetch(first, xa, wa);
+
+    // ---- where this lane's results go: position 8 q + 4 half + lane % 4 of the tile, channels 4 (cl / 4) .. + 3
+    char *ob = g.out;
+    const __amdgpu_buffer_rsrc_t ores = make_rsrc(ob, g.o_bytes);
+    const __amdgpu_buffer_rsrc_t rres = make_rsrc(RES ? reinterpret_cast<const char *>(g.res) : ob, g.o_bytes);
+    uint32_t d_off[4], d_res[RES ? 4 : 1];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int pm = mg * 32 + 8 * q + 4 * half + (lane & 3), pn = ng * 32 + (cl & ~3);
+        d_off[q] = (pm < g.M && pn < g.N) ? (uint32_t)pm * (uint32_t)g.ldo + (uint32_t)pn : kOobOffset;
+        if constexpr (RES) d_res[q] = buf_load4(rres, d_off[q]);
+    }
+    // ---- this lane's channel: bias, requantisation constants
+    int32_t bias = 0, mult = 0, shift = 0;
+    if (n < g.N) {
+        bias = g.bias ? g.bias[g.bias_len == 1 ? 0 : n] : 0;
+        const int ci = g.rp.per_channel ? n : 0;
+        mult = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci] : reinterpret_cast<const int32_t *>(g.mult)[ci];
+        shift = (int32_t)g.shift[ci];
+    }
+
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0;
+    int32_t wsum = 0;
+    const bool need_wsum = g.zx != 0;
+    auto multiply = [&](const v4i (&xf)[KR], const v4i (&wf)[KR]) {
+#pragma unroll
+        for (int c = 0; c < KR; c++) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[c], wf[c], acc, 0, 0, 0);
+        if (need_wsum) {  // uniform
+#pragma unroll
+            for (int c = 0; c < KR; c++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) wsum = __builtin_amdgcn_sdot4(wf[c][e], 0x01010101, wsum, false);
+        }
+    };
+    for (int r = 0; r < rounds; r += 2) {
+        if (r + 1 < rounds) fetch(first + r + 1, xb, wb);
+        multiply(xa, wa);
+        if (r + 1 < rounds) {
+            if (r + 2 < rounds) fetch(first + r + 2, xa, wa);
+            multiply(xb, wb);
+        }
+    }
+    if constexpr (KS > 1) {
+        __shared__ int32_t part[KS - 1][17][64];  // [wavefront][register, then the weight sum][lane]
+        if (wave > 0) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) part[wave - 1][r][lane] = acc[r];
+            part[wave - 1][16][lane] = wsum;
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int o = 0; o < KS - 1; o++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r] = (int32_t)((uint32_t)acc[r] + (uint32_t)part[o][r][lane]);
+            wsum = (int32_t)((uint32_t)wsum + (uint32_t)part[o][16][lane]);
+        }
+    }
+
+    // ---- epilogue: the channel's constants are registers; a 4 x 4 byte transpose inside lane quads turns four
+    // positions of one channel into four channels of one position, stored as a dword
+    const int32_t sw = wsum + __shfl_xor(wsum, 32);
+    const int32_t bias_adj = (int32_t)((uint32_t)bias - (uint32_t)g.zx * (uint32_t)sw);
+    const ChanScale cs = make_chan_scale(mult, shift, g.rp);
+    ChanScale q_res{}, q_conv{}, q_out{};
+    if constexpr (RES) {
+        q_res = make_chan_scale(load_mult(g.rs_res, 0), g.rs_res.shift[0], g.rs_res.p);
+        q_conv = make_chan_scale(load_mult(g.rs_conv, 0), g.rs_conv.shift[0], g.rs_conv.p);
+        q_out = make_chan_scale(load_mult(g.rs_out, 0), g.rs_out.shift[0], g.rs_out.p);
+    }
+    const uint32_t sel_a = (lane & 1) ? 0x03070105u : 0x06020400u;  // exchange with lane ^ 1
+    const uint32_t sel_b = (lane & 2) ? 0x03020706u : 0x05040100u;  // exchange with lane ^ 2
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        int32_t v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = requant_acc((int32_t)((uint32_t)acc[4 * q + e] + (uint32_t)bias_adj), cs, g.rp);
+        const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
+        const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
+        uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        uint32_t o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0xb1, 0xf, 0xf, true);
+        p = __builtin_amdgcn_perm(o, p, sel_a);
+        o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0x4e, 0xf, 0xf, true);
+        p = __builtin_amdgcn_perm(o, p, sel_b);
+        if constexpr (RES) {
+            const uint32_t xw = d_res[q];
+            uint32_t summed = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int32_t x = (int8_t)(xw >> (8 * e)), y = (int8_t)(p >> (8 * e));
+                const int32_t r1 = requant_chan(x, q_res, g.rs_res.p), r2 = requant_chan(y, q_conv, g.rs_conv.p);
+                const int32_t sum = (int32_t)((uint32_t)r1 + (uint32_t)r2);
+                summed |= ((uint32_t)requant_chan(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
+            }
+            p = summed;
+        }
+        __builtin_amdgcn_raw_buffer_store_b32(p, ores, (int)d_off[q], 0, 0);
+    }
+}
+
+}  // namespace
+
+// What the kernel's indexing assumes is checked by the caller (plain rows on both sides in 16-byte pieces, 8-bit
+// fused epilogue with dword stores, 31-bit extents) and here (zero weight zero point, K in 16-byte pieces).
+// Returns 1 when launched.
+int launch_conv_cols_mfma(const void *args, hipStream_t s) {
+    const GemmArgs &g = *static_cast<const GemmArgs *>(args);
+    if (g.zw != 0 || g.K % 16 != 0 || g.batches != 1 || !g.plain) return 0;
+    const int64_t groups_m = (g.M + 31) / 32, groups_n = (g.N + 31) / 32;
+    const int64_t waves = groups_m * groups_n;
+    if (waves >= (int64_t(1) << 30)) return 0;
+    // At most 700 tiles of at least eight K chunks: the four wavefronts of a block share a tile (384 -> 64 at
+    // 14 x 14 with the residual: 7.2 -> 6.3 us, 960 -> 160 at 7 x 7: 8.3 -> 6.2 us; 1960 tiles of 320 -> 1280 lose)
+    if (waves <= 700 && g.K >= 2 * KR * 32) {
+        const dim3 grid((unsigned)waves);
+        if (g.res != nullptr)
+            conv_cols_mfma_i8_kernel<true, 4><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
+        else
+            conv_cols_mfma_i8_kernel<false, 4><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
+        return 1;
+    }
+    const dim3 grid((unsigned)((waves + kColsBlock / 64 - 1) / (kColsBlock / 64)));
+    if (g.res != nullptr)
+        conv_cols_mfma_i8_kernel<true, 1><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
+    else
+        conv_cols_mfma_i8_kernel<false, 1><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
+    return 1;
+}
+
+}  // namespace mlel

@@ -1307,11 +1307,48 @@ def test_config1_matmul_rescale_full_size(run, oracle):
     assert exp.min() < -20 and exp.max() > 20
 
 
+POINTWISE_CASES = [
+    # name, x shape, OC, input zp, per channel: 1x1 convolutions of few 32 x 32 tiles (one tile per wavefront, or
+    # four wavefronts per tile when the contraction is long and the tiles are very few)
+    ("p_96_24_56x56", (1, 56, 56, 96), 24, -3, True),
+    ("p_144_32_28x28", (2, 28, 28, 144), 32, 7, True),
+    ("p_192_64_14x14", (3, 14, 14, 192), 64, 0, False),
+    ("p_384_96_14x14", (2, 14, 14, 384), 96, -128, True),
+    ("p_960_320_7x7", (2, 7, 7, 960), 320, 5, True),
+    ("p_320_1280_7x7", (1, 7, 7, 320), 1280, -9, False),
+    ("p_208_44_ragged", (1, 5, 13, 208), 44, 11, True),
+    ("p_1040_36_one_position", (3, 1, 1, 1040), 36, -1, True),
+]
+
+
+@pytest.mark.parametrize("case", POINTWISE_CASES, ids=[c[0] for c in POINTWISE_CASES])
+def test_pointwise_conv_of_few_tiles_vs_oracle(run, oracle, case):
+    name, xs, oc, zx, per_channel = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    x = ri(rng, -128, 127, xs, np.int8)
+    w = ri(rng, -128, 127, (oc, 1, 1, xs[3]), np.int8)
+    b = ri(rng, -2 ** 15, 2 ** 15, (oc,), np.int32)
+    attr = abi.conv2d_attr((0, 0, 0, 0), (1, 1), (1, 1), zx, 0)
+    shape = xs[:3] + (oc,)
+    n = oc if per_channel else 1
+    mult, shift = ri(rng, 2 ** 30, 2 ** 31 - 1, (n,), np.int32), ri(rng, 39, 43, (n,), np.int8)
+    rattr = abi.rescale_attr(0, -6, True, True, per_channel)
+    acc = oracle.conv2d(x, w, b, shape, abi.I32, attr)
+    exp = oracle.clamp(oracle.rescale(acc, mult, shift, abi.I8, rattr), -100, 110)
+    got = run.conv2d(x, w, b, shape, abi.I8, attr, epilogue=(mult, shift, rattr, (-100, 110)))
+    np.testing.assert_array_equal(got, exp)
+    assert len(np.unique(exp)) > 50
+
+
 RESIDUAL_CASES = [
     # name, x shape, OC, kernel, pad: 1x1 projections take the one-pass kernel, the 3x3 case the two-kernel sequence
     ("project_96_24", (2, 14, 14, 96), 24, (1, 1), (0, 0, 0, 0)),
     ("project_192_32_ragged", (3, 7, 9, 192), 32, (1, 1), (0, 0, 0, 0)),
     ("project_960_160", (1, 7, 7, 960), 160, (1, 1), (0, 0, 0, 0)),
+    ("project_384_64_b4", (4, 14, 14, 384), 64, (1, 1), (0, 0, 0, 0)),
+    ("project_576_96", (2, 14, 14, 576), 96, (1, 1), (0, 0, 0, 0)),
+    ("project_144_24_many_tiles", (2, 56, 56, 144), 24, (1, 1), (0, 0, 0, 0)),
+    ("project_208_44_ragged", (1, 9, 11, 208), 44, (1, 1), (0, 0, 0, 0)),
     ("k3_32_16", (1, 8, 8, 32), 16, (3, 3), (1, 1, 1, 1)),
 ]
 
