@@ -22,8 +22,12 @@ template <bool RES, int KS>
 __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const GemmArgs g, int groups_n, int total_waves) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wid = KS == 1 ? (int)blockIdx.x * (kColsBlock / 64) + wave : (int)blockIdx.x;
-    if (KS == 1 && wid >= total_waves) return;  // whole wavefronts leave; this form has no barrier
+    // blocks are dealt round-robin to the XCDs: XCD k gets the k-th contiguous run of blocks, so the tiles of a
+    // pixel row group (which read the same 32 pixel rows) fetch them into one L2
+    const int chunk = (int)gridDim.x >> 3;  // the grid is a multiple of eight blocks
+    const int bid = (int)(blockIdx.x % 8u) * chunk + (int)(blockIdx.x / 8u);
+    const int wid = KS == 1 ? bid * (kColsBlock / 64) + wave : bid;
+    if (wid >= total_waves) return;  // whole wavefronts (KS == 1) or whole blocks (KS == 4) leave: no barrier is missed
     const int mg = wid / groups_n, ng = wid - mg * groups_n;
     const int cl = lane & 31, half = lane >> 5;
     const int m = mg * 32 + cl, n = ng * 32 + cl;
@@ -69,6 +73,26 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
         shift = (int32_t)g.shift[ci];
     }
 
+    // The residual stage rescales two 8-bit values per output with per-tensor constants: both are functions of a
+    // byte, so the wavefront tabulates them (256 dwords each, four entries per lane, in its own piece of shared
+    // memory: no block barrier) and an output costs two lookups instead of two requantisations.
+    ChanScale q_out{};
+    __shared__ int32_t res_tab[RES ? kColsBlock / 64 : 1][2][256];
+    int32_t(*tab)[256] = res_tab[RES ? (KS == 1 ? wave : 0) : 0];
+    if (RES && (KS == 1 || wave == 0)) {  // while the first operands travel
+        const ChanScale q_res = make_chan_scale(load_mult(g.rs_res, 0), g.rs_res.shift[0], g.rs_res.p);
+        const ChanScale q_conv = make_chan_scale(load_mult(g.rs_conv, 0), g.rs_conv.shift[0], g.rs_conv.p);
+        q_out = make_chan_scale(load_mult(g.rs_out, 0), g.rs_out.shift[0], g.rs_out.p);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int b = t * 64 + lane;  // the byte as stored; its value is (int8_t)b
+            tab[0][b] = requant_chan((int32_t)(int8_t)b, q_res, g.rs_res.p);
+            tab[1][b] = requant_chan((int32_t)(int8_t)b, q_conv, g.rs_conv.p);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0;
@@ -114,12 +138,6 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
     const int32_t sw = wsum + __shfl_xor(wsum, 32);
     const int32_t bias_adj = (int32_t)((uint32_t)bias - (uint32_t)g.zx * (uint32_t)sw);
     const ChanScale cs = make_chan_scale(mult, shift, g.rp);
-    ChanScale q_res{}, q_conv{}, q_out{};
-    if constexpr (RES) {
-        q_res = make_chan_scale(load_mult(g.rs_res, 0), g.rs_res.shift[0], g.rs_res.p);
-        q_conv = make_chan_scale(load_mult(g.rs_conv, 0), g.rs_conv.shift[0], g.rs_conv.p);
-        q_out = make_chan_scale(load_mult(g.rs_out, 0), g.rs_out.shift[0], g.rs_out.p);
-    }
     const uint32_t sel_a = (lane & 1) ? 0x03070105u : 0x06020400u;  // exchange with lane ^ 1
     const uint32_t sel_b = (lane & 2) ? 0x03020706u : 0x05040100u;  // exchange with lane ^ 2
 #pragma unroll
@@ -139,8 +157,7 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
             uint32_t summed = 0;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const int32_t x = (int8_t)(xw >> (8 * e)), y = (int8_t)(p >> (8 * e));
-                const int32_t r1 = requant_chan(x, q_res, g.rs_res.p), r2 = requant_chan(y, q_conv, g.rs_conv.p);
+                const int32_t r1 = tab[0][(xw >> (8 * e)) & 0xffu], r2 = tab[1][(p >> (8 * e)) & 0xffu];
                 const int32_t sum = (int32_t)((uint32_t)r1 + (uint32_t)r2);
                 summed |= ((uint32_t)requant_chan(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
             }
@@ -164,14 +181,14 @@ int launch_conv_cols_mfma(const void *args, hipStream_t s) {
     // At most 700 tiles of at least eight K chunks: the four wavefronts of a block share a tile (384 -> 64 at
     // 14 x 14 with the residual: 7.2 -> 6.3 us, 960 -> 160 at 7 x 7: 8.3 -> 6.2 us; 1960 tiles of 320 -> 1280 lose)
     if (waves <= 700 && g.K >= 2 * KR * 32) {
-        const dim3 grid((unsigned)waves);
+        const dim3 grid((unsigned)((waves + 7) / 8 * 8));
         if (g.res != nullptr)
             conv_cols_mfma_i8_kernel<true, 4><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
         else
             conv_cols_mfma_i8_kernel<false, 4><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
         return 1;
     }
-    const dim3 grid((unsigned)((waves + kColsBlock / 64 - 1) / (kColsBlock / 64)));
+    const dim3 grid((unsigned)(((waves + kColsBlock / 64 - 1) / (kColsBlock / 64) + 7) / 8 * 8));
     if (g.res != nullptr)
         conv_cols_mfma_i8_kernel<true, 1><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
     else
