@@ -34,6 +34,7 @@ struct HGemmArgs {
     const char *a, *b;
     char *out;
     int32_t M, N, K, batches;
+    int32_t b_rows;                     // B is laid down row-wise, [N][K]: ldb is then the pitch of a row of K
     int64_t a_batch, b_batch, o_batch;  // bytes
     uint32_t lda, ldb, ldo;             // bytes per row
     uint32_t a_bytes, b_bytes, o_bytes; // per-batch extents (all below 2^31)
@@ -91,8 +92,31 @@ __device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t r, uint32_t off) 
     return make_uint4((uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w);
 }
 
+// One wavefront-wide 16-byte-per-lane load from a buffer resource straight into LDS at `lds_addr` + 16 * lane.
+// Inline assembly on purpose: the compiler orders every LDS read after ALL outstanding loads of this kind (it cannot
+// tell which bytes they write), which would drain the stage ring at every step; the loop does its own counting with
+// s_waitcnt vmcnt(N).  M0 holds the LDS address for this one instruction only.
+__device__ __forceinline__ void load16_to_lds(v4i res, uint32_t lds_addr, uint32_t offset, uint32_t scalar_offset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(offset),
+                 "s"(res), "s"(scalar_offset)
+                 : "memory");
+}
+__device__ __forceinline__ v4i rsrc_words(const void *p, uint32_t bytes) {
+    const uint64_t a = reinterpret_cast<uint64_t>(p);
+    return v4i{(int)(uint32_t)a, (int)(uint32_t)(a >> 32), (int)bytes, 0x00020000};
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N) only (expcnt / lgkmcnt untouched)
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
 // BKH: halfs of K per step (32, or 64 for long contractions: half as many barriers and LDS round trips per K)
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int BKH>
+// BROWS: B is given row-wise, [N][K] (a weight matrix laid down transposed once, ahead of time): both operands are
+// then rows of K, and the main loop is the direct-to-LDS pipeline of the int8 kernel (gemm_i8_kernel.hpp): 64 bytes of
+// K per step, `buffer_load ... lds` into a ring of four unpadded stages whose 16-byte pieces are XOR-swizzled (piece p
+// of row r in slot p ^ ((r >> 2) & 3)), 128-bit operand reads without bank conflicts and without the transposing
+// reads of the K-major tile, one barrier per step, reads of the next half step issued before the multiplies of this one.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int BKH, bool BROWS = false>
 __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const HGemmArgs g) {
     constexpr int NT = 64 * WAVES_M * WAVES_N;  // four or eight wavefronts
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -136,6 +160,114 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
     const __amdgpu_buffer_rsrc_t ares = rsrc(g.a + (int64_t)batch * g.a_batch, g.a_bytes);
     const __amdgpu_buffer_rsrc_t bres = rsrc(o.b + (int64_t)batch * g.b_batch, g.b_bytes);
 
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    if constexpr (BROWS) {
+        // ---- direct-to-LDS main loop (K % 32 == 0: whole 64-byte steps)
+        constexpr int BK = 64, DL_S = 4, DL_STAGE = (BM + BN) * BK;
+        constexpr int XI = BM * 4 / NT, WI = BN * 4 / NT;  // 16-byte pieces per thread and stage
+        static_assert((BM * 4) % NT == 0 && (BN * 4) % NT == 0 && 6 * (XI + WI) < 64, "whole pieces per thread");
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        uint32_t xo[XI], wo[WI];
+#pragma unroll
+        for (int i = 0; i < XI; i++) {
+            const int q = i * NT + tid, r = q >> 2, p = (q & 3) ^ ((r >> 2) & 3);
+            const int m = m_base + r;
+            xo[i] = m < g.M ? (uint32_t)m * g.lda + (uint32_t)(p * 16) : kOob;
+        }
+#pragma unroll
+        for (int i = 0; i < WI; i++) {
+            const int q = i * NT + tid, r = q >> 2, p = (q & 3) ^ ((r >> 2) & 3);
+            const int n = n_base + r;
+            wo[i] = n < g.N ? (uint32_t)n * g.ldb + (uint32_t)(p * 16) : kOob;
+        }
+        const v4i xres4 = rsrc_words(g.a + (int64_t)batch * g.a_batch, g.a_bytes);
+        const v4i wres4 = rsrc_words(o.b + (int64_t)batch * g.b_batch, g.b_bytes);
+        const uint32_t lds0 = (uint32_t) reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char *)smem) +
+                              (uint32_t)(wave_u * 1024);
+        auto issue = [&](int buf, int step) {  // `step` is wave-uniform: the K advance is a scalar offset
+            const uint32_t xd = lds0 + (uint32_t)(buf * DL_STAGE), wd = xd + BM * BK;
+            const uint32_t kb = (uint32_t)step * BK;
+#pragma unroll
+            for (int i = 0; i < XI; i++) load16_to_lds(xres4, xd + i * NT * 16, xo[i], kb);
+#pragma unroll
+            for (int i = 0; i < WI; i++) load16_to_lds(wres4, wd + i * NT * 16, wo[i], kb);
+        };
+        // operand addresses inside a stage: row lane % 32 of a 32-row group, the lane half's eight halfs of K half kk
+        const int h = lane >> 5, swz = (lane >> 2) & 3;
+        const char *x_base[2], *w_base[2];
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            const int slot = ((kk * 2 + h) ^ swz) * 16;
+            x_base[kk] = smem + (wave_m * WM + (lane & 31)) * BK + slot;
+            w_base[kk] = smem + BM * BK + (wave_n * WN + (lane & 31)) * BK + slot;
+        }
+        auto read_frags = [&](int buf, int kk, v8h(&xf)[TM], v8h(&wf)[TN]) {
+#pragma unroll
+            for (int i = 0; i < TM; i++) xf[i] = *reinterpret_cast<const v8h *>(x_base[kk] + buf * DL_STAGE + i * 32 * BK);
+#pragma unroll
+            for (int j = 0; j < TN; j++) wf[j] = *reinterpret_cast<const v8h *>(w_base[kk] + buf * DL_STAGE + j * 32 * BK);
+        };
+        auto multiply = [&](const v8h(&xf)[TM], const v8h(&wf)[TN]) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[i][j], 0, 0, 0);
+        };
+        // wait until at most `n` stages of this thread's requests are outstanding (n is wave-uniform)
+        auto wait_stages = [&](int n) {
+            switch (n) {
+            case 0: wait_vmcnt<0>(); break;
+            case 1: wait_vmcnt<1 * (XI + WI)>(); break;
+            case 2: wait_vmcnt<2 * (XI + WI)>(); break;
+            default: wait_vmcnt<3 * (XI + WI)>(); break;
+            }
+        };
+        // Stage s lives in buffer s % DL_S; DL_S - 1 stages are requested ahead.  While the first K half of step s is
+        // multiplied the second half is being read, and while the second half is multiplied the first half of step
+        // s + 1 is being read.  In between sits the one barrier of the step: waiting until at most DL_S - 3 stages
+        // of this thread's requests are outstanding means its part of stage s + 1 has landed; the barrier extends
+        // that to every thread's part and also says that every wavefront has received its reads of stage s - 1,
+        // whose buffer the next request overwrites.
+        const int nk = g.K / 32;
+        v8h xf0[TM], wf0[TN], xf1[TM], wf1[TN];
+#pragma unroll
+        for (int d = 0; d < DL_S - 1; d++)
+            if (d < nk) issue(d, d);
+        wait_stages(min(nk, DL_S - 1) - 1);  // stage 0 has landed
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        read_frags(0, 0, xf0, wf0);
+        for (int step = 0; step < nk; step += DL_S) {
+#pragma unroll
+            for (int d = 0; d < DL_S; d++) {
+                if (step + d < nk) {  // uniform
+                    read_frags(d, 1, xf1, wf1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    multiply(xf0, wf0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const bool more = step + d + DL_S - 1 < nk;
+                    if (more) wait_vmcnt<(DL_S - 3) * (XI + WI)>(); else wait_stages(max(nk - 2 - (step + d), 0));
+                    asm volatile("" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    if (more) issue((d + DL_S - 1) % DL_S, step + d + DL_S - 1);
+                    read_frags((d + 1) % DL_S, 0, xf0, wf0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    multiply(xf1, wf1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        __syncthreads();
+    } else {
     uint32_t xoff[XROWS], woff[WCHUNKS];
 #pragma unroll
     for (int i = 0; i < XROWS; i++) {
@@ -168,14 +300,6 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
             *reinterpret_cast<uint4 *>(ws + buf * WBUF + (c / WROW16) * WPITCH + (c % WROW16) * 16) = wr[i];
         }
     };
-
-    v16f acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     // operand addresses inside a tile: A row = lane % 32, k group = lane / 32 (8 halfs each);
     // B: 16-lane group q = lane / 16 covers columns 16 * (q & 1) .., k group q / 2; lane s = lane % 16 points at
@@ -232,6 +356,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
                 __syncthreads();
             }
         }
+    }
     }
 
     // ---- store: lane holds row m = lane % 32 of each sub-tile and, per register quad q, columns 8q + 4 * (lane / 32)
@@ -363,21 +488,22 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BKH>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKH, bool BROWS = false>
 void launch_k(const HGemmArgs &g, bool cast_epilogue, dim3 grid, hipStream_t s) {
-    constexpr size_t operands = (size_t)2 * BM * (BKH * 2 + 16) + (size_t)2 * BKH * (2 * BN + 32);
+    constexpr size_t operands = BROWS ? (size_t)4 * (BM + BN) * 64
+                                      : (size_t)2 * BM * (BKH * 2 + 16) + (size_t)2 * BKH * (2 * BN + 32);
     constexpr size_t result = std::max((size_t)BM * (BN * 2 + 16), (size_t)BN * (BM * 2 + 16));
     constexpr size_t sm = std::max(operands, result);
     static_assert(sm <= 160 * 1024, "shared memory of a compute unit");
     // above the default dynamic shared-memory limit the limit is raised once per kernel (thread-safe static)
     if (cast_epilogue) {
-        auto kernel = gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 1, BKH>;
+        auto kernel = gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 1, BKH, BROWS>;
         static const bool raised = sm <= 48 * 1024 || hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm) == hipSuccess;
         (void)raised;
         kernel<<<grid, dim3(64 * WAVES_M * WAVES_N), sm, s>>>(g);
     } else {
-        auto kernel = gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 0, BKH>;
+        auto kernel = gemm_f16_kernel<BM, BN, WAVES_M, WAVES_N, 0, BKH, BROWS>;
         static const bool raised = sm <= 48 * 1024 || hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm) == hipSuccess;
         (void)raised;
@@ -451,15 +577,21 @@ int fill_args(const mlel_tensor *out, const mlel_tensor *a, const mlel_tensor *b
     // what the kernel's indexing assumes: element-contiguous rows, 16-byte aligned rows and bases, K and N in
     // multiples of 8, per-batch extents below 2^31, operands at least as large as the output implies
     if (a->dims[0] < NB || b->dims[0] < NB || a->dims[1] < M || b->dims[1] < K || b->dims[2] < N) return 0;
-    if (!dense_rows(a) || !dense_rows(b) || out->strides[2] != osize) return 0;
-    if (K % 8 != 0 || N % 8 != 0 || K <= 0) return 0;
+    // B row-wise: element (k, n) at n * pitch + 2 k, i.e. a [K][N] view of a matrix stored as [N][K] (K > 1, so the
+    // two layouts cannot be confused); the direct-to-LDS loop then wants whole 64-byte steps of K
+    const bool b_rows = K > 1 && b->strides[1] == 2 && b->strides[2] >= b->dims[1] * 2;
+    if (!dense_rows(a) || !(b_rows || dense_rows(b)) || out->strides[2] != osize) return 0;
+    if (K % 8 != 0 || N % 8 != 0 || K <= 0 || (b_rows && K % 32 != 0)) return 0;
     auto aligned = [](const mlel_tensor *t) {
         return ((uintptr_t)t->ptr % 16) == 0 && t->strides[0] % 16 == 0 && t->strides[1] % 16 == 0;
     };
-    if (!aligned(a) || !aligned(b) || !aligned(out)) return 0;
+    if (!aligned(a) || !aligned(out) || (b_rows ? ((uintptr_t)b->ptr % 16) != 0 || b->strides[0] % 16 != 0 || b->strides[2] % 16 != 0
+                                                : !aligned(b)))
+        return 0;
     const int64_t lim = (int64_t(1) << 31) - 64;
-    const int64_t ab = a->dims[1] * a->strides[1], bb = b->dims[1] * b->strides[1], ob = M * out->strides[1];
-    if (ab >= lim || bb >= lim || ob >= lim || a->strides[1] >= lim || b->strides[1] >= lim) return 0;
+    const int64_t b_pitch = b_rows ? b->strides[2] : b->strides[1];
+    const int64_t ab = a->dims[1] * a->strides[1], bb = (b_rows ? b->dims[2] : b->dims[1]) * b_pitch, ob = M * out->strides[1];
+    if (ab >= lim || bb >= lim || ob >= lim || a->strides[1] >= lim || b_pitch >= lim) return 0;
     if (M >= (1 << 24) || N >= (1 << 24) || K >= (1 << 24)) return 0;
     if (NB <= 0 || M <= 0 || N <= 0) return 2;
 
@@ -475,7 +607,8 @@ int fill_args(const mlel_tensor *out, const mlel_tensor *a, const mlel_tensor *b
     g.b_batch = b->strides[0];
     g.o_batch = out->strides[0];
     g.lda = (uint32_t)a->strides[1];
-    g.ldb = (uint32_t)b->strides[1];
+    g.ldb = (uint32_t)b_pitch;
+    g.b_rows = b_rows ? 1 : 0;
     g.ldo = (uint32_t)out->strides[1];
     g.a_bytes = (uint32_t)ab;
     g.b_bytes = (uint32_t)bb;
@@ -543,6 +676,30 @@ int launch_args(mlel_ctx *ctx, hipStream_t s, HGemmArgs &g, bool bias_cast) {
     // 48 tiles: twice the time), and so does an activation in the epilogue, whose arithmetic then runs on three
     // quarters of the machine (the same product with the tanh GELU: 40.9 -> 44.1 us).
     const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256) * NB;
+    if (g.b_rows) {
+        // row-wise B: the direct-to-LDS loop; the 256 x 256 tile under the same condition as below, else 128 x 128 of
+        // eight wavefronts, whatever the extents (rows beyond M or N are fetched as zeros)
+        const int64_t tn128 = (N + 127) / 128;
+        if (g.groups == 1 && g.act[0] == nullptr && g.K >= 256 && tiles256 * 4 >= 3 * (int64_t)cus && tiles256 <= 2 * (int64_t)cus) {
+            g.tiles_m = (int)((M + 255) / 256);
+            g.tiles_n_group = (int)((N + 255) / 256);
+            g.tiles_n = g.tiles_n_group;
+            g.total_tiles = (int)tiles256;
+            g.chunk = (int)((tiles256 + 7) / 8);
+            launch_k<256, 256, 2, 4, 32, true>(g, bias_cast, dim3((unsigned)(g.chunk * 8)), s);
+        } else {
+            g.tiles_m = (int)((M + 127) / 128);
+            g.tiles_n_group = (int)tn128;
+            g.tiles_n = (int)(tn128 * g.groups);
+            const int64_t t = (int64_t)g.tiles_m * g.tiles_n * NB;
+            MLEL_REQUIRE(t < (int64_t(1) << 30), MLEL_ERR_LIMIT, "matmul: %lld tiles", (long long)t);
+            g.total_tiles = (int)t;
+            g.chunk = (int)((t + 7) / 8);
+            launch_k<128, 128, 2, 4, 32, true>(g, bias_cast, dim3((unsigned)(g.chunk * 8)), s);
+        }
+        MLEL_TRY(check_launch("matmul fp16, row-wise B"));
+        return 1;
+    }
     if (BN == 128 && g.groups == 1 && g.act[0] == nullptr && g.K >= 256 && tiles256 * 4 >= 3 * (int64_t)cus && tiles256 <= 2 * (int64_t)cus) {
         g.tiles_m = (int)((M + 255) / 256);
         g.tiles_n_group = (int)((N + 255) / 256);
@@ -590,7 +747,7 @@ int try_matmul_f16_group(mlel_ctx *ctx, hipStream_t s, int n, const mlel_tensor 
     for (int i = 0; i < n; i++) {
         if (fill_args(outs[i], a, bs[i], attr, true, biases[i], nullptr, &g[i]) != 1) return 0;
         const HGemmArgs &x = g[i], &y = g[0];
-        if (x.M != y.M || x.N != y.N || x.K != y.K || x.batches != y.batches || x.ldb != y.ldb || x.b_bytes != y.b_bytes ||
+        if (x.M != y.M || x.N != y.N || x.K != y.K || x.batches != y.batches || x.ldb != y.ldb || x.b_rows != y.b_rows || x.b_bytes != y.b_bytes ||
             (x.batches > 1 && x.b_batch != y.b_batch) || x.bias_len != y.bias_len || (x.bias == nullptr) != (y.bias == nullptr))
             return 0;
     }

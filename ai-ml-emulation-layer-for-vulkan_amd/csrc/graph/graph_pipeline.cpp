@@ -1452,10 +1452,62 @@ std::vector<std::array<uint32_t, 2>> GraphPipeline::liveRanges() const {
     return r;
 }
 
+// Constant weight matrices of the fused fp16 products are laid down row-wise once, [N][K] instead of the operator's
+// [K][N] (one transposing launch per matrix while the pipeline is created), and handed to the kernel as the same [K][N]
+// tensor with the two strides exchanged: both operands of the product are then rows of K, which the matrix kernel
+// fetches straight into shared memory (gemm_f16.hip).  The values and the operator are unchanged.  Pipeline creation is
+// also where the reference spends its one-time work (shader specialisation, compute_graph_op.cpp:526-590).
+void GraphPipeline::prepackConstants() {
+    if (ctx == nullptr) return;
+    std::map<const TensorDescriptor *, TensorPtr> rowWise;
+    bool launched = false;
+    for (const auto &opPtr : ops) {
+        OpNode &op = *opPtr;
+        if (op.fusedAway || op.kind != OpKind::FusedMatmulBiasCast) continue;
+        const size_t perProduct = op.hasBias ? 2 : 1;
+        const size_t products = op.extraProductViews.empty() ? 1 : op.outputs.size();
+        for (size_t k = 0; k < products; k++) {
+            const size_t idx = 1 + k * perProduct;
+            if (idx >= op.inputs.size()) break;
+            const TensorPtr b = op.inputs[idx];
+            const auto &d = b->getDimensions();
+            // what the row-wise form of the kernel takes: one fp16 matrix, K in whole 64-byte steps, N in 16-byte pieces
+            if (b->getKind() != TensorKind::Constant || b->devicePointer() == nullptr || b->getFormat() != MLEL_F16 ||
+                d.size() != 3 || d[0] != 1 || !b->isPacked() || d[1] % 32 != 0 || d[2] % 8 != 0 || d[1] <= 0 || d[2] <= 0)
+                continue;
+            auto found = rowWise.find(b.get());
+            if (found == rowWise.end()) {
+                const int64_t K = d[1], N = d[2];
+                auto t = std::make_shared<TensorDescriptor>(MLEL_F16, std::vector<int64_t>{1, K, N},
+                                                            std::vector<int64_t>{K * N * 2, 2, K * 2}, TensorKind::Constant);
+                void *dptr = nullptr;
+                check(mlel_hip_arena_alloc(ctx, static_cast<size_t>(K * N * 2), &dptr), "allocating a row-wise weight matrix");
+                constantsDeviceMemory.push_back(dptr);
+                const mlel_tensor src = b->view();
+                mlel_tensor dst{};
+                dst.ptr = dptr;
+                dst.dtype = MLEL_F16;
+                dst.rank = 3;
+                dst.dims[0] = 1, dst.dims[1] = N, dst.dims[2] = K;
+                dst.strides[0] = K * N * 2, dst.strides[1] = K * 2, dst.strides[2] = 2;
+                const uint32_t perms[3] = {0, 2, 1};
+                check(mlel_hip_transpose(ctx, nullptr, &dst, &src, perms), "laying a weight matrix down row-wise");
+                launched = true;
+                t->bind(dptr);
+                found = rowWise.emplace(b.get(), registerTensor(std::move(t))).first;
+            }
+            op.inputs[idx] = found->second;
+            MLEL_GRAPH_LOG(Debug, "Weight matrix row-wise. op=" << op.debugName << " input=" << idx << " tensor=" << found->second->id);
+        }
+    }
+    if (launched) check(mlel_hip_sync(ctx, nullptr), "laying weight matrices down row-wise");
+}
+
 void GraphPipeline::finalize(const bool enableFusion) {
     if (finalized) return;
     const size_t recorded = ops.size();
     if (enableFusion) fuse();
+    if (enableFusion) prepackConstants();
     plan();
     finalized = true;
     size_t launches = 0;

@@ -355,6 +355,7 @@ class GraphPipeline {
     TensorPtr registerTensor(TensorPtr t);
     void *uploadConstant(const TensorDescriptor &t, const void *data);
     void fuse();
+    void prepackConstants();
     void plan();
     std::vector<details::BestFitTensor> bestFitTensors(const std::vector<details::LiveInterval> &planned,
                                                        const std::vector<details::UnseenAllocation> &unseen);

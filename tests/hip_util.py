@@ -250,11 +250,20 @@ class Runner:
         self.done()
         return r
 
-    def matmul_bias_cast(self, a, b, bias):
-        ta, tb = self.put(a), self.put(b)
+    def _b_operand(self, b, b_rows):
+        """B [NB, K, N] as the operators define it, or (b_rows) the same tensor described over a matrix stored
+        row-wise, [NB, N, K]: element (k, n) at n * 2K + 2k bytes.  Returns what a call takes as its B argument."""
+        if not b_rows:
+            return self.put(b).view
+        nb, k, n = b.shape
+        stored = self.put(np.ascontiguousarray(np.transpose(b, (0, 2, 1))))
+        return abi.make_tensor(stored.view.ptr, abi.F16, b.shape, [n * k * 2, 2, k * 2])
+
+    def matmul_bias_cast(self, a, b, bias, b_rows=False):
+        ta, tb = self.put(a), self._b_operand(b, b_rows)
         tbias = self.put(bias) if bias is not None else None
         to = self.new(abi.F16, (a.shape[0], a.shape[1], b.shape[2]))
-        self.dev.op("matmul_bias_cast", to.ref, ta.ref, tb.ref, tbias.ref if tbias else None, C.byref(abi.MatmulAttr(0, 0)))
+        self.dev.op("matmul_bias_cast", to.ref, ta.ref, C.byref(tb), tbias.ref if tbias else None, C.byref(abi.MatmulAttr(0, 0)))
         r = to.download()
         self.done()
         return r
@@ -277,10 +286,10 @@ class Runner:
         self.done()
         return r
 
-    def matmul_bias_cast_chain(self, a, b, bias, inputs, steps):
+    def matmul_bias_cast_chain(self, a, b, bias, inputs, steps, b_rows=False):
         """The fused product followed by an elementwise chain whose value 0 is the product; `inputs`: the chain's
         other inputs."""
-        ta, tb = self.put(a), self.put(b)
+        ta, tb = self.put(a), self._b_operand(b, b_rows)
         tbias = self.put(bias) if bias is not None else None
         tin = [self.put(x) for x in inputs]
         to = self.new(abi.F16, (a.shape[0], a.shape[1], b.shape[2]))
@@ -290,32 +299,32 @@ class Runner:
             c.inputs[i + 1] = C.pointer(t.view)
         for i, st in enumerate(steps):
             c.steps[i] = abi.ChainStep(*[int(v) for v in st])
-        self.dev.op("matmul_bias_cast_chain", to.ref, ta.ref, tb.ref, tbias.ref if tbias else None,
+        self.dev.op("matmul_bias_cast_chain", to.ref, ta.ref, C.byref(tb), tbias.ref if tbias else None,
                     C.byref(abi.MatmulAttr(0, 0)), C.byref(c))
         r = to.download()
         self.done()
         return r
 
-    def matmul_bias_cast_group(self, a, bs, biases):
+    def matmul_bias_cast_group(self, a, bs, biases, b_rows=False):
         """Several fused products of one `a` in one call; returns the list of results."""
         ta = self.put(a)
-        tbs = [self.put(b) for b in bs]
+        tbs = [self._b_operand(b, b_rows) for b in bs]
         tbias = [self.put(x) if x is not None else None for x in biases]
         touts = [self.new(abi.F16, (a.shape[0], a.shape[1], b.shape[2])) for b in bs]
         products = (abi.MatmulProduct * len(bs))()
         for i in range(len(bs)):
-            products[i] = abi.MatmulProduct(C.pointer(touts[i].view), C.pointer(tbs[i].view),
+            products[i] = abi.MatmulProduct(C.pointer(touts[i].view), C.pointer(tbs[i]),
                                             C.pointer(tbias[i].view) if tbias[i] else None)
         self.dev.op("matmul_bias_cast_group", products, len(bs), ta.ref, C.byref(abi.MatmulAttr(0, 0)))
         r = [t.download() for t in touts]
         self.done()
         return r
 
-    def matmul_bias_cast_add(self, a, b, bias, residual):
-        ta, tb, tr = self.put(a), self.put(b), self.put(residual)
+    def matmul_bias_cast_add(self, a, b, bias, residual, b_rows=False):
+        ta, tb, tr = self.put(a), self._b_operand(b, b_rows), self.put(residual)
         tbias = self.put(bias) if bias is not None else None
         to = self.new(abi.F16, (a.shape[0], a.shape[1], b.shape[2]))
-        self.dev.op("matmul_bias_cast_add", to.ref, ta.ref, tb.ref, tbias.ref if tbias else None,
+        self.dev.op("matmul_bias_cast_add", to.ref, ta.ref, C.byref(tb), tbias.ref if tbias else None,
                     C.byref(abi.MatmulAttr(0, 0)), tr.ref)
         r = to.download()
         self.done()

@@ -406,6 +406,45 @@ def test_matmul_bias_cast_chain_equals_product_then_chain(run):
             np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16), err_msg=f"{(nb, m, k, n)} {len(steps)}")
 
 
+BROWS_SHAPES = [(1, 256, 768, 768), (2, 130, 96, 136), (1, 33, 32, 8), (1, 512, 3072, 768), (1, 300, 64, 392), (3, 64, 160, 128),
+                (1, 1024, 768, 1024)]
+
+
+@pytest.mark.parametrize("shape", BROWS_SHAPES, ids=str)
+def test_fp16_products_with_row_wise_b_equal_the_k_major_form(run, shape):
+    """B handed over as a [K][N] view of a matrix stored row-wise ([N][K], what a graph does once with a constant
+    weight matrix) takes the direct-to-LDS loop; the result is the K-major kernel's bit for bit (same matrix
+    instruction, same order of K), for the plain fused form, with a residual, with the GELU chain, for grouped products
+    and through a head-splitting view; rows beyond M and N are padding."""
+    nb, m, k, n = shape
+    rng = np.random.default_rng(m * 13 + n)
+    a = rng.standard_normal((nb, m, k)).astype(np.float16)
+    bs = [(0.1 * rng.standard_normal((nb, k, n))).astype(np.float16) for _ in range(3)]
+    biases = [rng.standard_normal((1, 1, n)).astype(np.float32) for _ in range(3)]
+    b, bias = bs[0], biases[0]
+    want = run.matmul_bias_cast(a, b, bias)
+    assert len(np.unique(want)) > 100
+    np.testing.assert_array_equal(run.matmul_bias_cast(a, b, bias, b_rows=True).view(np.uint16), want.view(np.uint16))
+    np.testing.assert_array_equal(run.matmul_bias_cast(a, b, None, b_rows=True).view(np.uint16),
+                                  run.matmul_bias_cast(a, b, None).view(np.uint16))
+    res = rng.standard_normal((nb, m, n)).astype(np.float16)
+    np.testing.assert_array_equal(run.matmul_bias_cast_add(a, b, bias, res, b_rows=True).view(np.uint16),
+                                  run.matmul_bias_cast_add(a, b, bias, res).view(np.uint16))
+    got = run.matmul_bias_cast_group(a, bs, biases, b_rows=True)
+    for i in range(3):
+        np.testing.assert_array_equal(got[i].view(np.uint16), run.matmul_bias_cast(a, bs[i], biases[i]).view(np.uint16))
+
+    def scalar(v):
+        return np.array(v, np.float16).reshape(1, 1, 1)
+
+    B, M, U, ADD, f16 = 0, 1, 2, abi.BIN["ADD"], abi.F16
+    gelu_inputs = [scalar(0.5), scalar(0.044715), scalar(np.sqrt(2 / np.pi)), scalar(1.0)]
+    gelu = [(M, 0, 0, 1, f16), (M, 0, 0, 0, f16), (M, 0, 6, 0, f16), (M, 0, 7, 2, f16), (B, ADD, 0, 8, f16),
+            (M, 0, 9, 3, f16), (U, abi.UN["TANH"], 10, 0, f16), (B, ADD, 11, 4, f16), (M, 0, 5, 12, f16)]
+    np.testing.assert_array_equal(run.matmul_bias_cast_chain(a, b, bias, gelu_inputs, gelu, b_rows=True).view(np.uint16),
+                                  run.matmul_bias_cast_chain(a, b, bias, gelu_inputs, gelu).view(np.uint16))
+
+
 def test_matmul_bias_cast_through_a_view(run):
     """A six-dimensional output view = the RESHAPE -> TRANSPOSE that splits or merges attention heads behind the
     product: same bytes as the product followed by numpy's reshape and transpose.  The last case has an inner extent
