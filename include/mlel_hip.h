@@ -424,7 +424,11 @@ int mlel_hip_softmax_rows(mlel_ctx *ctx, void *stream, const mlel_tensor *out, c
  * `out` has rank 3, or is a six-dimensional view [NB1, NB2, M1, M2, N1, N2] with byte strides of its own (the last
  * one 2, N2 a multiple of 8; or, for a view that transposes, the stride of M2 2 and M2 a multiple of 8) through which
  * element (nb1 * NB2 + nb2, m1 * M2 + m2, n1 * N2 + n2) of the product is written: the RESHAPE -> TRANSPOSE that splits
- * or merges attention heads behind a projection costs no pass. */
+ * or merges attention heads behind a projection costs no pass.
+ * `b` is the operator's [NB, K, N] tensor; its byte strides may describe a matrix that is stored row-wise ([N][K]:
+ * strides[1] == 2, strides[2] the pitch of a row of K) -- with K a multiple of 32 such a B takes the faster
+ * direct-to-LDS loop, with the same bits.  A caller whose B is a constant lays it down that way once (the graph layer
+ * does at pipeline creation); the same holds for the _add, _group and _chain forms below. */
 int mlel_hip_matmul_bias_cast(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *a,
                               const mlel_tensor *b, const mlel_tensor *bias, const mlel_matmul_attr *attr);
 /* Several such products of one `a` (the query, key and value projections of an attention block) in one launch:
