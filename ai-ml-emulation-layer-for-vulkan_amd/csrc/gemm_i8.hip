@@ -289,7 +289,10 @@ int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     if (epi != nullptr && dt_size(out->dtype) > 4) return 0;
     const int64_t NB = out->dims[0], M = out->dims[1], N = out->dims[2], K = A->dims[2];
     if (A->dims[0] < NB || B->dims[0] < NB || A->dims[1] < M || B->dims[1] != K || B->dims[2] < N) return 0;
-    if (A->strides[2] != 1 || B->strides[2] != 1 || !is_packed(out)) return 0;
+    // B row-wise: element (k, n) at n * pitch + k, i.e. the operator's [K][N] tensor described over a matrix stored as
+    // [N][K] (what a graph does once with a constant weight matrix): the weights are then rows of K as a convolution's
+    const bool b_rows = K > 1 && N > 1 && B->strides[1] == 1 && B->strides[2] >= K;
+    if (A->strides[2] != 1 || (B->strides[2] != 1 && !b_rows) || !is_packed(out)) return 0;
     if (M <= 0 || N <= 0 || NB <= 0) return 1;
     if (K <= 0) return 0;
     if (M >= (int64_t(1) << 30) || N >= (int64_t(1) << 30) || K >= (int64_t(1) << 30) || NB >= (1 << 20)) return 0;
@@ -313,15 +316,16 @@ int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     g.plain = 1;
     g.xch = align_of(A->ptr, K, A->strides[0], A->strides[1]);
     {
-        const int64_t xb = (M - 1) * A->strides[1] + K, wbytes = (K - 1) * B->strides[1] + N;
+        const int64_t xb = (M - 1) * A->strides[1] + K;
+        const int64_t wbytes = b_rows ? (N - 1) * B->strides[2] + K : (K - 1) * B->strides[1] + N;
         g.x_bytes = xb < (int64_t(1) << 31) ? (uint32_t)xb : 0;
         g.w_bytes = wbytes < (int64_t(1) << 31) ? (uint32_t)wbytes : 0;
     }
     g.w = static_cast<const int8_t *>(B->ptr);
     g.w_batch = B->strides[0];
-    g.ldw = B->strides[1];
-    g.w_kmajor = 1;
-    g.wch = align_of(B->ptr, N, B->strides[0], B->strides[1]);
+    g.ldw = b_rows ? B->strides[2] : B->strides[1];
+    g.w_kmajor = b_rows ? 0 : 1;
+    g.wch = b_rows ? align_of(B->ptr, K, B->strides[0], B->strides[2]) : align_of(B->ptr, N, B->strides[0], B->strides[1]);
     g.zx = attr->a_zp;
     g.zw = attr->b_zp;
     g.bias = nullptr;
@@ -329,6 +333,15 @@ int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     g.ldo = N;
     g.out_batch = out->strides[0];
     MLEL_TRY(fill_epilogue(g, out, epi));
+    if (b_rows) {  // few tiles (a fully connected layer over a batch of rows): one tile per wavefront, as for 1x1 convolutions
+        const bool q8 = g.fused && g.out_size == 1 && g.out_vec_ok && g.o_bytes != 0;
+        const bool rows = g.xch == 16 && g.wch == 16 && g.x_bytes != 0 && g.w_bytes != 0;
+        const int64_t tiles = ((M + 31) / 32) * ((N + 31) / 32);
+        if (q8 && rows && tiles <= 8192 && tiles * K <= (int64_t(1) << 20) && launch_conv_cols_mfma(&g, s)) {
+            MLEL_TRY(check_launch("matmul int8, one tile per wavefront"));
+            return 1;
+        }
+    }
     MLEL_TRY(launch_gemm(ctx, s, g, SplitScratch{}));
     return 1;
 }

@@ -1452,10 +1452,10 @@ std::vector<std::array<uint32_t, 2>> GraphPipeline::liveRanges() const {
     return r;
 }
 
-// Constant weight matrices of the fused fp16 products are laid down row-wise once, [N][K] instead of the operator's
-// [K][N] (one transposing launch per matrix while the pipeline is created), and handed to the kernel as the same [K][N]
-// tensor with the two strides exchanged: both operands of the product are then rows of K, which the matrix kernel
-// fetches straight into shared memory (gemm_f16.hip).  The values and the operator are unchanged.  Pipeline creation is
+// Constant weight matrices of the fused products (fp16 MATMUL + bias + CAST, int8 MATMUL + RESCALE) are laid down
+// row-wise once, [N][K] instead of the operator's [K][N] (one transposing launch per matrix while the pipeline is created), and handed to the kernel as the same [K][N]
+// tensor with the two strides exchanged: both operands of the product are then rows of K, which the fp16 kernel
+// fetches straight into shared memory (gemm_f16.hip) and the int8 kernels read like a convolution's weights.  The values and the operator are unchanged.  Pipeline creation is
 // also where the reference spends its one-time work (shader specialisation, compute_graph_op.cpp:526-590).
 void GraphPipeline::prepackConstants() {
     if (ctx == nullptr) return;
@@ -1463,33 +1463,38 @@ void GraphPipeline::prepackConstants() {
     bool launched = false;
     for (const auto &opPtr : ops) {
         OpNode &op = *opPtr;
-        if (op.fusedAway || op.kind != OpKind::FusedMatmulBiasCast) continue;
+        if (op.fusedAway || (op.kind != OpKind::FusedMatmulBiasCast && op.kind != OpKind::FusedMatmul)) continue;
+        const bool int8 = op.kind == OpKind::FusedMatmul;  // MATMUL + RESCALE: a fully connected layer
         const size_t perProduct = op.hasBias ? 2 : 1;
-        const size_t products = op.extraProductViews.empty() ? 1 : op.outputs.size();
+        const size_t products = int8 || op.extraProductViews.empty() ? 1 : op.outputs.size();
         for (size_t k = 0; k < products; k++) {
             const size_t idx = 1 + k * perProduct;
             if (idx >= op.inputs.size()) break;
             const TensorPtr b = op.inputs[idx];
             const auto &d = b->getDimensions();
             // what the row-wise form of the kernel takes: one fp16 matrix, K in whole 64-byte steps, N in 16-byte pieces
-            if (b->getKind() != TensorKind::Constant || b->devicePointer() == nullptr || b->getFormat() != MLEL_F16 ||
-                d.size() != 3 || d[0] != 1 || !b->isPacked() || d[1] % 32 != 0 || d[2] % 8 != 0 || d[1] <= 0 || d[2] <= 0)
+            // (fp16) or, for int8, K in 16-byte pieces and N in dwords
+            const int32_t want = int8 ? MLEL_I8 : MLEL_F16;
+            const int64_t es = int8 ? 1 : 2;
+            if (b->getKind() != TensorKind::Constant || b->devicePointer() == nullptr || b->getFormat() != want ||
+                d.size() != 3 || d[0] != 1 || !b->isPacked() || d[1] <= 1 || d[2] <= 1)
                 continue;
+            if (int8 ? (d[1] % 16 != 0 || d[2] % 4 != 0) : (d[1] % 32 != 0 || d[2] % 8 != 0)) continue;
             auto found = rowWise.find(b.get());
             if (found == rowWise.end()) {
                 const int64_t K = d[1], N = d[2];
-                auto t = std::make_shared<TensorDescriptor>(MLEL_F16, std::vector<int64_t>{1, K, N},
-                                                            std::vector<int64_t>{K * N * 2, 2, K * 2}, TensorKind::Constant);
+                auto t = std::make_shared<TensorDescriptor>(want, std::vector<int64_t>{1, K, N},
+                                                            std::vector<int64_t>{K * N * es, es, K * es}, TensorKind::Constant);
                 void *dptr = nullptr;
-                check(mlel_hip_arena_alloc(ctx, static_cast<size_t>(K * N * 2), &dptr), "allocating a row-wise weight matrix");
+                check(mlel_hip_arena_alloc(ctx, static_cast<size_t>(K * N * es), &dptr), "allocating a row-wise weight matrix");
                 constantsDeviceMemory.push_back(dptr);
                 const mlel_tensor src = b->view();
                 mlel_tensor dst{};
                 dst.ptr = dptr;
-                dst.dtype = MLEL_F16;
+                dst.dtype = want;
                 dst.rank = 3;
                 dst.dims[0] = 1, dst.dims[1] = N, dst.dims[2] = K;
-                dst.strides[0] = K * N * 2, dst.strides[1] = K * 2, dst.strides[2] = 2;
+                dst.strides[0] = K * N * es, dst.strides[1] = K * es, dst.strides[2] = es;
                 const uint32_t perms[3] = {0, 2, 1};
                 check(mlel_hip_transpose(ctx, nullptr, &dst, &src, perms), "laying a weight matrix down row-wise");
                 launched = true;

@@ -55,15 +55,23 @@ class Runner:
     def _epi(self, mult, shift, rattr, clamp):
         return self.dev.epilogue(self.put(mult), self.put(shift), rattr, clamp)
 
-    def matmul(self, a, b, out_dtype, a_zp=0, b_zp=0, epilogue=None):
-        ta, tb = self.put(a), self.put(b)
+    def matmul(self, a, b, out_dtype, a_zp=0, b_zp=0, epilogue=None, b_rows=False):
+        """b_rows: B described as the operator's [NB, K, N] tensor over a matrix stored row-wise, [NB, N, K]."""
+        ta = self.put(a)
+        if b_rows:
+            nb, k, n = b.shape
+            es = b.dtype.itemsize
+            stored = self.put(np.ascontiguousarray(np.transpose(b, (0, 2, 1))))
+            tb = abi.make_tensor(stored.view.ptr, stored.view.dtype, b.shape, [n * k * es, es, k * es])
+        else:
+            tb = self.put(b).view
         to = self.new(out_dtype, (a.shape[0], a.shape[1], b.shape[2]))
         attr = abi.MatmulAttr(int(a_zp), int(b_zp))
         if epilogue is None:
-            self.dev.op("matmul", to.ref, ta.ref, tb.ref, C.byref(attr))
+            self.dev.op("matmul", to.ref, ta.ref, C.byref(tb), C.byref(attr))
         else:
             e = self._epi(*epilogue)
-            self.dev.op("matmul_rescale", to.ref, ta.ref, tb.ref, C.byref(attr), C.byref(e))
+            self.dev.op("matmul_rescale", to.ref, ta.ref, C.byref(tb), C.byref(attr), C.byref(e))
         r = to.download()
         self.done()
         return r

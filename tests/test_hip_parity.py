@@ -241,6 +241,9 @@ def test_matmul_i8_vs_oracle(run, oracle, case):
     rattr = abi.rescale_attr(0, 0, True, True, False)
     exp8 = oracle.rescale(exp, mult, shift, abi.I8, rattr)
     np.testing.assert_array_equal(run.matmul(a, b, abi.I8, za, zb, epilogue=(mult, shift, rattr, None)), exp8)
+    # B handed over as a view of a matrix stored row-wise (what a graph does once with a constant weight matrix)
+    np.testing.assert_array_equal(run.matmul(a, b, abi.I32, za, zb, b_rows=True), exp)
+    np.testing.assert_array_equal(run.matmul(a, b, abi.I8, za, zb, epilogue=(mult, shift, rattr, None), b_rows=True), exp8)
 
 
 DL_CASES = [
