@@ -345,6 +345,35 @@ def _time_graph(dev, g, steps, warmup):
     return wall, dev.elapsed_ms(ev0, ev1) / steps
 
 
+def _time_sessions(dev, g, input_name, output_name, steps, batch, count):
+    """Throughput with `count` batches in flight: that many sessions of the one pipeline (session memory and external
+    tensors of their own, the same input data) dispatched in turn on a stream each, as a serving loop that keeps the
+    next batches queued behind the current one.  A dependent launch costs about 5 us whatever the batch, and the other
+    streams' launches fill the gaps.  Every graph is a whole batch; every output is checked against the
+    single-session result.  (With four sessions the host's launch rate, about 4 us per launch, is the limit.)"""
+    want = g.get_output(output_name)
+    x = g.ext_tensors[input_name].download()
+    sessions = [g.new_session() for _ in range(count)]
+    streams = [dev.new_stream() for _ in range(count)]
+    for s in sessions:
+        s.set_input(input_name, x)
+    sync_all = lambda: dev._check(dev.lib.mlel_hip_sync(dev.ctx, None))
+    for k in range(2 * count):
+        sessions[k % count].dispatch(streams[k % count])
+    sync_all()
+    same = all(np.array_equal(s.get_output(output_name), want) for s in sessions)
+    n = count * max(steps, 10)
+    t0 = time.perf_counter()
+    for k in range(n):
+        sessions[k % count].dispatch(streams[k % count])
+    sync_all()
+    wall = (time.perf_counter() - t0) / n
+    for s in sessions:
+        s.close()
+    return {"img_per_s": batch / wall, "ms_per_graph": wall * 1e3, "graphs_timed": n, "streams": count,
+            "outputs_equal_single_session": bool(same)}
+
+
 def time_operators(dev, g, reps=50, only=None):
     """Milliseconds per launch of every executed operator of `g` on its own: the operator is launched `reps` times
     back to back on the stream (its inputs are whatever the last whole dispatch left in session memory) between two
@@ -415,6 +444,7 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True):
            "operators_executed": g.op_count(), "operators_in_graph": len(spec.ops),
            "session_memory_bytes": g.session_size,
            "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}
+    res["sessions_in_flight"] = [_time_sessions(dev, g, "input", "output", steps, batch, c) for c in (2, 4)]
     launches = launch_layers(g, spec) if per_layer else None
     if launches is not None:
         alone = time_operators(dev, g)
@@ -470,6 +500,10 @@ def bench_transformer(dev, steps=20, warmup=3):
     by_kind = {}
     for name, ms in per_op:
         by_kind[name] = by_kind.get(name, 0.0) + ms
+    in_flight = [_time_sessions(dev, g, "input", "output", steps, spec.inputs[0][2][0], c) for c in (2, 4)]
+    for r in in_flight:  # a "graph" is one encoder block over the whole batch
+        r["tflops"] = spec.flops / (r["ms_per_graph"] * 1e-3) / 1e12
+        r["blocks_per_s"] = r.pop("img_per_s") / spec.inputs[0][2][0]
     alone = time_operators(dev, g)
     names = g.op_names()
     gemm_ms = sum(ms for i, ms in alone.items() if "MATMUL" in names[i])
@@ -478,7 +512,7 @@ def bench_transformer(dev, steps=20, warmup=3):
         "ms_per_graph": wall * 1e3, "gpu_ms_per_graph": gpu_ms, "graphs_timed": steps,
         "tflops": spec.flops / wall / 1e12,
         "gflop": spec.flops / 1e9, "operators_executed": g.op_count(), "operators_in_graph": len(spec.ops),
-        "session_memory_bytes": g.session_size,
+        "session_memory_bytes": g.session_size, "sessions_in_flight": in_flight,
         "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())},
         "us_by_launch_alone": [{"index": i, "name": names[i], "us": round(ms * 1e3, 2)} for i, ms in alone.items()],
         "roofline_gemm": {"bound": "mfma", "unit": "TFLOP/s", "peak": 2500.0,
