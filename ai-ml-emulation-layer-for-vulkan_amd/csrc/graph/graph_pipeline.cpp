@@ -1505,7 +1505,19 @@ void GraphPipeline::prepackConstants() {
             MLEL_GRAPH_LOG(Debug, "Weight matrix row-wise. op=" << op.debugName << " input=" << idx << " tensor=" << found->second->id);
         }
     }
-    if (launched) check(mlel_hip_sync(ctx, nullptr), "laying weight matrices down row-wise");
+    if (!launched) return;
+    check(mlel_hip_sync(ctx, nullptr), "laying weight matrices down row-wise");
+    // the K-major copy of a matrix that no operator reads any more is given back (a weight then costs its size once)
+    for (const auto &[kMajor, unused] : rowWise) {
+        (void)unused;
+        if (!consumersOf(ops, kMajor).empty()) continue;
+        void *old = kMajor->devicePointer();
+        const auto held = std::find(constantsDeviceMemory.begin(), constantsDeviceMemory.end(), old);
+        if (held == constantsDeviceMemory.end()) continue;
+        constantsDeviceMemory.erase(held);
+        (void)mlel_hip_arena_free(ctx, old);
+        const_cast<TensorDescriptor *>(kMajor)->bind(nullptr);
+    }
 }
 
 void GraphPipeline::finalize(const bool enableFusion) {
