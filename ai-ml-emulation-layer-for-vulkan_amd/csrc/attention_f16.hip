@@ -278,15 +278,22 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
     const int64_t o_base = g.view ? (int64_t)(batch / g.v_nb2) * g.vs_nb1 + (int64_t)(batch % g.v_nb2) * g.vs_nb2
                                   : (int64_t)batch * g.o_batch;
     const __amdgpu_buffer_rsrc_t ores = rsrc(g.out + o_base, g.o_bytes);
+    // the view's two divisions per piece as multiplications (the divisors are the same for every piece; exact while
+    // index * divisor < 2^32, else the plain division)
+    const uint32_t dm = (uint32_t)(g.view ? g.v_m2 : 1), dn = (uint32_t)(g.view ? g.v_n2 : 1);
+    const bool fast_m = dm > 1 && (uint64_t)(uint32_t)g.M * dm < (uint64_t(1) << 32), fast_n = dn > 1 && (uint64_t)kHead * dn < (uint64_t(1) << 32);
+    const uint32_t magic_m = fast_m ? 0xffffffffu / dm + 1u : 0u, magic_n = fast_n ? 0xffffffffu / dn + 1u : 0u;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         const int p = i * kBlock + tid, r = p >> 3, c8 = p & 7;
         const int m = m0 + r, n = c8 * 8;
         const uint4 piece = *reinterpret_cast<const uint4 *>(cb + r * OP + c8 * 16);
         uint32_t off = (uint32_t)m * g.ldo + (uint32_t)n * 2;
-        if (g.view)  // uniform
-            off = (uint32_t)(m / g.v_m2) * g.vs_m1 + (uint32_t)(m % g.v_m2) * g.vs_m2 + (uint32_t)(n / g.v_n2) * g.vs_n1 +
-                  (uint32_t)(n % g.v_n2) * 2;
+        if (g.view) {  // uniform
+            const uint32_t m1 = fast_m ? __umulhi((uint32_t)m, magic_m) : (dm == 1 ? (uint32_t)m : (uint32_t)m / dm);
+            const uint32_t n1 = fast_n ? __umulhi((uint32_t)n, magic_n) : (dn == 1 ? (uint32_t)n : (uint32_t)n / dn);
+            off = m1 * g.vs_m1 + ((uint32_t)m - m1 * dm) * g.vs_m2 + n1 * g.vs_n1 + ((uint32_t)n - n1 * dn) * 2;
+        }
         v4i v;
         v.x = (int)piece.x, v.y = (int)piece.y, v.z = (int)piece.z, v.w = (int)piece.w;
         __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);

@@ -110,6 +110,20 @@ __device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N) only (expc
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
+// Division of the row and column indices of a view by its inner extents, once per 16-byte piece: the extents are the
+// same for every piece, so the quotient is one multiplication by floor((2^32 - 1) / d) + 1 (exact while x * d < 2^32,
+// which `usable` says for the tile's largest index; otherwise, and for d == 1, the plain division).
+struct ViewDiv {
+    uint32_t d, magic;
+    bool usable;
+    __device__ __forceinline__ ViewDiv(int32_t divisor, int32_t largest) {
+        d = (uint32_t)divisor;
+        usable = d > 1 && (uint64_t)(uint32_t)largest * d < (uint64_t(1) << 32);
+        magic = usable ? 0xffffffffu / d + 1u : 0u;
+    }
+    __device__ __forceinline__ uint32_t quotient(uint32_t x) const { return usable ? __umulhi(x, magic) : (d == 1 ? x : x / d); }
+};
+
 // BKH: halfs of K per step (32, or 64 for long contractions: half as many barriers and LDS round trips per K)
 // BROWS: B is given row-wise, [N][K] (a weight matrix laid down transposed once, ahead of time): both operands are
 // then rows of K, and the main loop is the direct-to-LDS pipeline of the int8 kernel (gemm_i8_kernel.hpp): 64 bytes of
@@ -416,6 +430,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
         }
         __syncthreads();
         const __amdgpu_buffer_rsrc_t rres = rsrc(g.res != nullptr ? g.res + (int64_t)batch * g.r_batch : o.out, g.res != nullptr ? g.r_bytes : 0);
+        const ViewDiv by_m2(o.view ? o.v_m2 : 1, g.M), by_n2(o.view ? o.v_n2 : 1, g.N);
         if (o.view == 2) {
             // transposing view: a piece is eight consecutive rows of one column (tile rows start at multiples of
             // eight and M2 is one, so a piece never straddles two m1)
@@ -425,8 +440,9 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
                 if (m >= g.M || n >= g.N) continue;
                 const uint4 piece = *reinterpret_cast<const uint4 *>(smem + c * TPITCH + r8 * 16);
                 const uint32_t w[4] = {piece.x, piece.y, piece.z, piece.w};
-                const uint32_t off = (uint32_t)(m / o.v_m2) * o.vs_m1 + (uint32_t)(m % o.v_m2) * 2 + (uint32_t)(n / o.v_n2) * o.vs_n1 +
-                                     (uint32_t)(n % o.v_n2) * o.vs_n2;
+                const uint32_t m1 = by_m2.quotient((uint32_t)m), n1 = by_n2.quotient((uint32_t)n);
+                const uint32_t off = m1 * o.vs_m1 + ((uint32_t)m - m1 * (uint32_t)o.v_m2) * 2 + n1 * o.vs_n1 +
+                                     ((uint32_t)n - n1 * (uint32_t)o.v_n2) * o.vs_n2;
                 v4i v;
                 v.x = (int)w[0], v.y = (int)w[1], v.z = (int)w[2], v.w = (int)w[3];
                 __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
@@ -449,9 +465,11 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
             uint4 piece = *reinterpret_cast<const uint4 *>(smem + r * OPITCH + c * 16);
             const bool inside = m < g.M && n < g.N;
             uint32_t off = inside ? (uint32_t)m * o.ldo + (uint32_t)n * 2 : kOob;
-            if (o.view && inside)  // uniform
-                off = (uint32_t)(m / o.v_m2) * o.vs_m1 + (uint32_t)(m % o.v_m2) * o.vs_m2 + (uint32_t)(n / o.v_n2) * o.vs_n1 +
-                      (uint32_t)(n % o.v_n2) * 2;
+            if (o.view && inside) {  // uniform
+                const uint32_t m1 = by_m2.quotient((uint32_t)m), n1 = by_n2.quotient((uint32_t)n);
+                off = m1 * o.vs_m1 + ((uint32_t)m - m1 * (uint32_t)o.v_m2) * o.vs_m2 + n1 * o.vs_n1 +
+                      ((uint32_t)n - n1 * (uint32_t)o.v_n2) * 2;
+            }
             if (g.act[0] != nullptr) piece = gelu_tanh_piece(piece, act_c);  // uniform
             if (g.res != nullptr) {  // uniform; ADD of two fp16 tensors: one rounding of the exact sum
                 const uint4 other = load16(rres, inside ? (uint32_t)m * g.ldr + (uint32_t)n * 2 : kOob);
