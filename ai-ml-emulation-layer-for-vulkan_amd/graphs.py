@@ -424,7 +424,7 @@ def launch_layers(g, spec):
     return out if at == len(spec.layers) else None
 
 
-def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True):
+def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True, in_flight=(2, 4)):
     """Times whole-graph dispatches of BASELINE config 3 (inputs resident in HBM) and every launch on its own; returns
     the extra fields bench.py adds to its JSON line, with the MFMA position of the dense (CONV2D / MATMUL) launches
     and the HBM position of the bandwidth-bound (DEPTHWISE_CONV2D, AVG_POOL2D) ones."""
@@ -444,7 +444,7 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True):
            "operators_executed": g.op_count(), "operators_in_graph": len(spec.ops),
            "session_memory_bytes": g.session_size,
            "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}
-    res["sessions_in_flight"] = [_time_sessions(dev, g, "input", "output", steps, batch, c) for c in (2, 4)]
+    res["sessions_in_flight"] = [_time_sessions(dev, g, "input", "output", steps, batch, c) for c in in_flight]
     launches = launch_layers(g, spec) if per_layer else None
     if launches is not None:
         alone = time_operators(dev, g)
@@ -486,7 +486,7 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True):
     return {"mobilenetv2_b32": res}
 
 
-def bench_transformer(dev, steps=20, warmup=3):
+def bench_transformer(dev, steps=20, warmup=3, in_flight=(2, 4)):
     """Times whole-graph dispatches of BASELINE config 4 (fp16 encoder block, batch 8, seq 512, d_model 768) and every
     launch on its own; returns the extra fields bench.py adds to its JSON line, with the fp16 MFMA position of the
     launches that hold a MATMUL."""
@@ -500,7 +500,7 @@ def bench_transformer(dev, steps=20, warmup=3):
     by_kind = {}
     for name, ms in per_op:
         by_kind[name] = by_kind.get(name, 0.0) + ms
-    in_flight = [_time_sessions(dev, g, "input", "output", steps, spec.inputs[0][2][0], c) for c in (2, 4)]
+    in_flight = [_time_sessions(dev, g, "input", "output", steps, spec.inputs[0][2][0], c) for c in in_flight]
     for r in in_flight:  # a "graph" is one encoder block over the whole batch
         r["tflops"] = spec.flops / (r["ms_per_graph"] * 1e-3) / 1e12
         r["blocks_per_s"] = r.pop("img_per_s") / spec.inputs[0][2][0]

@@ -64,7 +64,7 @@ def config1_inputs():
     return a, b, np.array([1518500250], np.int32), np.array([39], np.int8)
 
 
-def bench_config1(dev, abi, steps, warmup):
+def bench_config1(dev, abi, steps, warmup, in_flight_counts=(2, 4)):
     a, b, mult, shift = config1_inputs()
     ta, tb, tm, ts = dev.from_numpy(a), dev.from_numpy(b), dev.from_numpy(mult), dev.from_numpy(shift)
     to = dev.tensor(abi.I8, (8, 512, 1024))
@@ -102,7 +102,7 @@ def bench_config1(dev, abi, steps, warmup):
     # delivers when its fixed latency (launch, first fetch, last store) is hidden behind another launch's loop.
     # Reported beside the one-stream figures, which stay the step time and the roofline of the JSON line.
     in_flight = []
-    for count in (2, 4):
+    for count in in_flight_counts:
         streams = [dev.new_stream() for _ in range(count)]
         outs = [dev.tensor(abi.I8, (8, 512, 1024)) for _ in range(count)]
         n = count * max(steps // count, 10)
@@ -274,6 +274,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline legs (profiling runs)")
+    ap.add_argument("--one-stream", action="store_true",
+                    help="omit the legs with several launches / sessions in flight (profiling runs: one kernel at a time)")
     ap.add_argument("--skip-graph", action="store_true", help="omit the MobileNetV2 and encoder graph legs")
     ap.add_argument("--only", choices=["all", "config1", "mobilenetv2", "encoder", "layer", "standalone"], default="all")
     ap.add_argument("--layer", type=int, default=3, help="with --only layer: position in the fused config 3 graph")
@@ -307,21 +309,23 @@ def main():
 
     c1, inputs = (None, None)
     if want("config1"):
-        c1, inputs = bench_config1(dev, abi, args.steps, args.warmup)
+        c1, inputs = bench_config1(dev, abi, args.steps, args.warmup, () if args.one_stream else (2, 4))
         log("config 1:", c1)
 
     extra = {}
     graphs = importlib.import_module(PKG + ".graphs")
     if want("mobilenetv2") and not args.skip_graph:
         try:
-            extra.update(graphs.bench_mobilenetv2(dev, steps=graph_steps, warmup=max(3, args.warmup // 10)))
+            extra.update(graphs.bench_mobilenetv2(dev, steps=graph_steps, warmup=max(3, args.warmup // 10),
+                                                  in_flight=() if args.one_stream else (2, 4)))
             log("config 3:", {k: v for k, v in extra["mobilenetv2_b32"].items() if k != "layers"})
         except Exception as e:  # the line below still reports config 1; the failure is visible
             log("config 3 leg failed:", repr(e))
             extra["mobilenetv2_b32"] = {"error": repr(e)}
     if want("encoder") and not args.skip_graph:
         try:
-            extra.update(graphs.bench_transformer(dev, steps=graph_steps, warmup=max(3, args.warmup // 10)))
+            extra.update(graphs.bench_transformer(dev, steps=graph_steps, warmup=max(3, args.warmup // 10),
+                                                  in_flight=() if args.one_stream else (2, 4)))
             log("config 4:", extra["transformer_b8_s512_d768"])
         except Exception as e:
             log("config 4 leg failed:", repr(e))
