@@ -370,6 +370,8 @@ def _time_sessions(dev, g, input_name, output_name, steps, batch, count):
     wall = (time.perf_counter() - t0) / n
     for s in sessions:
         s.close()
+    for st in streams:
+        dev.free_stream(st)
     return {"img_per_s": batch / wall, "ms_per_graph": wall * 1e3, "graphs_timed": n, "streams": count,
             "outputs_equal_single_session": bool(same)}
 

@@ -184,3 +184,6 @@ class Device:
         s = C.c_void_p()
         self._check(self.lib.mlel_hip_stream_create(self.ctx, C.byref(s)))
         return s
+
+    def free_stream(self, stream):
+        self._check(self.lib.mlel_hip_stream_destroy(self.ctx, stream))

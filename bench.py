@@ -119,6 +119,8 @@ def bench_config1(dev, abi, steps, warmup, in_flight_counts=(2, 4)):
                           "frac_of_int8_peak": ops / per / 1e12 / 5000.0, "outputs_equal": bool(same)})
         for t in outs:
             t.free()
+        for st in streams:
+            dev.free_stream(st)
     res["launches_in_flight"] = in_flight
     dev.stream = None
     # the same step when the caller hands over host buffers: upload A and B, launch, download the result
