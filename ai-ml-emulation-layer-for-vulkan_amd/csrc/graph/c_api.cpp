@@ -634,6 +634,15 @@ int mlel_graph_session_dispatch(mlel_graph_session *s, void *stream) {
     });
 }
 
+int mlel_graph_session_dispatch_replayed(mlel_graph_session *s, void *stream) {
+    return guarded([&] {
+        if (s == nullptr) throw std::runtime_error("session dispatch: null session");
+        if (s->graph->profiling) return dispatchSession(s->graph, s->session, stream);  // per-operator events: eagerly
+        s->session.dispatchReplayed(stream);
+        return 0;
+    });
+}
+
 int mlel_graph_session_dispatch_range(mlel_graph_session *s, void *stream, int first, int count) {
     return guarded([&] {
         if (s == nullptr || first < 0 || count < 0) throw std::runtime_error("session dispatch range: bad argument");

@@ -1556,7 +1556,13 @@ GraphSession::GraphSession(GraphPipeline &p) : pipeline(p) {
 }
 
 GraphSession::~GraphSession() {
+    dropRecording();
     if (pipeline.appliedSession == this) pipeline.appliedSession = nullptr;
+}
+
+void GraphSession::dropRecording() {
+    if (recording != nullptr && pipeline.ctx != nullptr) (void)mlel_hip_graph_destroy(pipeline.ctx, recording);
+    recording = nullptr;
 }
 
 void GraphSession::bindTransientMemory(void *deviceBase) {
@@ -1595,6 +1601,32 @@ void GraphSession::dispatch(void *stream, const GraphPipeline::DispatchDecorator
     if (needsTransientMemory() && !transientMemoryBound) fail("dispatch: session transient memory is not bound");
     apply();
     pipeline.dispatch(stream, decorator, first, count);
+}
+
+void GraphSession::dispatchReplayed(void *stream) {
+    if (pipeline.ctx == nullptr)
+        fail("dispatch: this GraphPipeline was built without a device context; there is no CPU path");
+    if (needsTransientMemory() && !transientMemoryBound) fail("dispatch: session transient memory is not bound");
+    if (recording == nullptr || recordingVersion != version || recordingStream != stream) {
+        // the recording holds the addresses of this session's tensors as they are bound now
+        dropRecording();
+        apply();
+        check(mlel_hip_capture_begin(pipeline.ctx, stream), "recording a dispatch");
+        void *exec = nullptr;
+        try {
+            pipeline.dispatch(stream, {}, 0, UINT32_MAX);
+        } catch (...) {
+            // the stream must leave capture mode whatever happened; what was recorded is thrown away
+            if (mlel_hip_capture_end(pipeline.ctx, stream, &exec) == 0 && exec != nullptr)
+                (void)mlel_hip_graph_destroy(pipeline.ctx, exec);
+            throw;
+        }
+        check(mlel_hip_capture_end(pipeline.ctx, stream, &exec), "recording a dispatch");
+        recording = exec;
+        recordingVersion = version;
+        recordingStream = stream;
+    }
+    check(mlel_hip_graph_launch(pipeline.ctx, recording, stream), "replaying a recorded dispatch");
 }
 
 namespace {

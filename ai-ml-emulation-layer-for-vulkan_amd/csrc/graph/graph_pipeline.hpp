@@ -410,9 +410,18 @@ class GraphSession {
     // reference: vkCmdDispatchDataGraphARM with this session (graph_layer.cpp:1844-1980)
     void dispatch(void *stream, const GraphPipeline::DispatchDecorator &decorator = {}, uint32_t first = 0,
                   uint32_t count = UINT32_MAX);
+    // The same launches, recorded into a HIP graph the first time (and again after a bind or on another stream) and
+    // replayed with one submission afterwards: the host side of a dispatch shrinks from one launch call per operator
+    // to one.  Reference counterpart: a command buffer with vkCmdDispatchDataGraphARM recorded once and submitted
+    // many times (graph_layer.cpp:1844-1980).
+    void dispatchReplayed(void *stream);
 
   private:
     void apply();
+    void dropRecording();
+    void *recording = nullptr;       // the instantiated HIP graph of this session's dispatch
+    void *recordingStream = nullptr;
+    uint64_t recordingVersion = 0;
     GraphPipeline &pipeline;
     void *base = nullptr;
     bool transientMemoryBound = false;

@@ -87,6 +87,7 @@ def load_graph_library():
         lib.mlel_graph_session_bind_memory.argtypes = [_V, C.c_uint32, _V]
         lib.mlel_graph_session_bind_external.argtypes = [_V, C.c_uint32, C.c_uint32, C.c_uint32, _V]
         lib.mlel_graph_session_dispatch.argtypes = [_V, _V]
+        lib.mlel_graph_session_dispatch_replayed.argtypes = [_V, _V]
         lib.mlel_graph_session_dispatch_range.argtypes = [_V, _V, C.c_int, C.c_int]
         lib.mlel_graph_dispatch_profiled.argtypes = [_V, _V, C.POINTER(C.c_float), C.c_int]
         lib.mlel_graph_set_profiling.argtypes = [_V, C.c_int]
@@ -392,6 +393,10 @@ class Session:
 
     def dispatch(self, stream=None):
         self.graph._check(self.lib.mlel_graph_session_dispatch(self.s, self.dev.stream if stream is None else stream))
+
+    def dispatch_replayed(self, stream=None):
+        """dispatch() through a HIP graph recorded on first use (one submission per dispatch afterwards)"""
+        self.graph._check(self.lib.mlel_graph_session_dispatch_replayed(self.s, self.dev.stream if stream is None else stream))
 
     def dispatch_range(self, first, count, stream=None):
         self.graph._check(self.lib.mlel_graph_session_dispatch_range(

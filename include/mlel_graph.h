@@ -133,6 +133,13 @@ int mlel_graph_session_bind_memory(mlel_graph_session *s, uint32_t bind_point, v
 int mlel_graph_session_bind_external(mlel_graph_session *s, uint32_t set, uint32_t binding, uint32_t array_index,
                                      void *device_ptr);
 int mlel_graph_session_dispatch(mlel_graph_session *s, void *stream);
+/* The same dispatch with its launches recorded into a HIP graph the first time (and again after a bind on this session,
+ * or on another stream) and replayed with one submission afterwards: the host's share of a dispatch drops from one
+ * launch call per operator (about 4 us each) to one, which is what bounds several sessions in flight.  Same results.
+ * The recording holds the addresses bound at that moment; `stream` must not be capturing already.  Reference
+ * counterpart: a command buffer with vkCmdDispatchDataGraphARM recorded once and submitted many times
+ * (graph/graph_layer.cpp:1844-1980).  With profiling enabled the dispatch runs eagerly (per-operator events). */
+int mlel_graph_session_dispatch_replayed(mlel_graph_session *s, void *stream);
 /* The operators `first` .. `first + count - 1` of the executed list only (profiling single layers). */
 int mlel_graph_session_dispatch_range(mlel_graph_session *s, void *stream, int first, int count);
 

@@ -151,3 +151,68 @@ def test_multi_sessions_on_two_streams_and_one_at_a_time(dev, kats):
         p.close()
     for st in streams:
         dev._check(dev.lib.mlel_hip_stream_destroy(dev.ctx, st))
+
+
+@pytest.mark.gpu
+def test_replayed_dispatch_equals_the_eager_one(dev, kats):
+    """mlel_graph_session_dispatch_replayed: the launches of a dispatch recorded once and submitted many times (the
+    command buffer of tests/vulkan.cpp:918-996, re-submitted).  Same bytes as the eager dispatch; a bind after the
+    recording is honoured (the recording is made again); two sessions replay on two streams at once; a MobileNetV2-shaped
+    graph of 41 launches replays to the bits of its eager dispatch."""
+    g, x, exp = maxpool_graph(dev, kats, 2)
+    streams = [dev.new_stream(), dev.new_stream()]
+    s = g.new_session()
+    s.set_input("input", x)
+    for _ in range(3):
+        s.dispatch_replayed(streams[0])
+    dev._check(dev.lib.mlel_hip_sync(dev.ctx, streams[0]))
+    np.testing.assert_array_equal(s.get_output("output"), exp)
+    # new contents of the same input tensor: the recording reads the tensor, not a copy of its bytes
+    s.set_input("input", np.zeros_like(x))
+    s.dispatch_replayed(streams[0])
+    dev._check(dev.lib.mlel_hip_sync(dev.ctx, streams[0]))
+    assert not s.get_output("output").any()
+    # another output tensor bound after the recording: it is written, the first one keeps its bytes
+    first = s.ext_tensors["output"]
+    second = dev.tensor(abi.I8, exp.shape)
+    s.bind("output", second)
+    s.ext_tensors["keep"] = first
+    s.set_input("input", x)
+    s.dispatch_replayed(streams[0])
+    dev._check(dev.lib.mlel_hip_sync(dev.ctx, streams[0]))
+    np.testing.assert_array_equal(second.download(), exp)
+    assert not first.download().any()
+    # the same session on another stream, and a second session beside it
+    t = g.new_session()
+    t.set_input("input", x)
+    for _ in range(3):
+        s.dispatch_replayed(streams[1])
+        t.dispatch_replayed(streams[0])
+    for st in streams:
+        dev._check(dev.lib.mlel_hip_sync(dev.ctx, st))
+    np.testing.assert_array_equal(second.download(), exp)
+    np.testing.assert_array_equal(t.get_output("output"), exp)
+    s.close()
+    t.close()
+    g.close()
+
+    graphs = importlib.import_module("ai-ml-emulation-layer-for-vulkan_amd.graphs")
+    spec = graphs.mobilenetv2_spec(batch=2, image=64, spread=True)
+    net = graphs.build(dev, spec, fuse=True)
+    rng = np.random.default_rng(3)
+    image = rng.integers(-128, 127, spec.inputs[0][2], endpoint=True).astype(np.int8)
+    net.set_input("input", image)
+    net.dispatch()
+    dev.sync()
+    want = net.get_output("output")
+    assert len(np.unique(want)) > 3
+    r = net.new_session()
+    r.set_input("input", image)
+    for _ in range(3):
+        r.dispatch_replayed(streams[0])
+    dev._check(dev.lib.mlel_hip_sync(dev.ctx, streams[0]))
+    np.testing.assert_array_equal(r.get_output("output"), want)
+    r.close()
+    net.close()
+    for st in streams:
+        dev._check(dev.lib.mlel_hip_stream_destroy(dev.ctx, st))
