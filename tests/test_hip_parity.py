@@ -1382,6 +1382,45 @@ def test_pointwise_conv_of_few_tiles_vs_oracle(run, oracle, case):
     assert len(np.unique(exp)) > 50
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_pointwise_conv_random_shapes_with_and_without_residual(run, oracle, seed):
+    """1x1 convolutions whose extents, channel counts (16-byte pieces of K, dwords of output channels), zero points and
+    scale forms are drawn at random over the range the one-tile-per-wavefront kernel serves: whole and partial tiles
+    in both directions, one or four wavefronts per tile, grids that do not fill their last group of eight blocks;
+    with the residual addition behind it on every second draw."""
+    rng = np.random.default_rng(9500 + seed)
+    n, h, w_ = int(rng.integers(1, 4)), int(rng.integers(1, 30)), int(rng.integers(1, 30))
+    ic, oc = 16 * int(rng.integers(1, 61)), 4 * int(rng.integers(1, 81))
+    zx = int(rng.integers(-128, 128))
+    per_channel = bool(rng.integers(0, 2))
+    x = ri(rng, -128, 127, (n, h, w_, ic), np.int8)
+    w = ri(rng, -128, 127, (oc, 1, 1, ic), np.int8)
+    b = ri(rng, -2 ** 15, 2 ** 15, (oc,), np.int32)
+    attr = abi.conv2d_attr((0, 0, 0, 0), (1, 1), (1, 1), zx, 0)
+    shape = (n, h, w_, oc)
+    k = oc if per_channel else 1
+    mult, shift = ri(rng, 2 ** 30, 2 ** 31 - 1, (k,), np.int32), ri(rng, 38, 44, (k,), np.int8)
+    rattr = abi.rescale_attr(0, int(rng.integers(-20, 20)), True, bool(rng.integers(0, 2)), per_channel)
+    conv8 = oracle.clamp(oracle.rescale(oracle.conv2d(x, w, b, shape, abi.I32, attr), mult, shift, abi.I8, rattr), -100, 110)
+    if seed % 2 == 0:
+        got = run.conv2d(x, w, b, shape, abi.I8, attr, epilogue=(mult, shift, rattr, (-100, 110)))
+        np.testing.assert_array_equal(got, conv8)
+        return
+    res = ri(rng, -128, 127, shape, np.int8)
+    m1, s1 = np.array([int(rng.integers(2 ** 29, 2 ** 31 - 1))], np.int32), np.array([int(rng.integers(8, 14))], np.int8)
+    m2, s2 = np.array([int(rng.integers(2 ** 29, 2 ** 31 - 1))], np.int32), np.array([int(rng.integers(8, 14))], np.int8)
+    mo, so = np.array([int(rng.integers(2 ** 30, 2 ** 31 - 1))], np.int32), np.array([int(rng.integers(48, 52))], np.int8)
+    a_conv = abi.rescale_attr(int(rattr.output_zp), 0, True, True, False)
+    a_res = abi.rescale_attr(int(rng.integers(-20, 20)), 0, True, True, False)
+    a_out = abi.rescale_attr(0, int(rng.integers(-20, 20)), True, True, False)
+    r_conv = oracle.rescale(conv8, m1, s1, abi.I32, a_conv)
+    r_res = oracle.rescale(res, m2, s2, abi.I32, a_res)
+    exp = oracle.rescale(oracle.elementwise_binary("ADD", r_res, r_conv, shape, abi.I32), mo, so, abi.I8, a_out)
+    got = run.conv2d_rescale_add_rescale(x, w, b, attr, (mult, shift, rattr, (-100, 110)), (m1, s1, a_conv, None), res,
+                                         (m2, s2, a_res, None), (mo, so, a_out, None), residual_first=bool(rng.integers(0, 2)))
+    np.testing.assert_array_equal(got, exp)
+
+
 RESIDUAL_CASES = [
     # name, x shape, OC, kernel, pad: 1x1 projections take the one-pass kernel, the 3x3 case the two-kernel sequence
     ("project_96_24", (2, 14, 14, 96), 24, (1, 1), (0, 0, 0, 0)),
