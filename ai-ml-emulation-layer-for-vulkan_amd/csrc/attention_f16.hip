@@ -6,15 +6,18 @@
 //                                                          six-dimensional view of a head merge
 // with every rounding of the three launches it replaces (the fp16 product of gemm_f16.hip, the compiled row program
 // of ops_float.hip, the product again), so the result is theirs bit for bit wherever it is a number.  S and P never
-// leave the chip: a block owns 64 query rows of one head and keeps their whole score rows in shared memory
-// (64 x (2 S + 16) bytes), K^T and V stream through one 10 KiB chunk buffer 64 keys at a time.
+// leave the chip: a block owns 64 query rows of one head; four threads share a row and keep its values in registers
+// from the scores to P, shared memory holds 256 keys of the 64 rows at a time (where the products leave and fetch
+// their operands and where the fold reads: 33 KiB, so that three blocks fit a compute unit and the 768 blocks of
+// 96 heads x 512 queries run in one round), K^T and V stream through one 10 KiB chunk buffer 64 keys at a time.
 //
 // Same arithmetic as the separate kernels, on purpose:
 //   * both products use v_mfma_f32_32x32x16_f16 with the K-major operand as the instruction's first operand and walk
 //     k in ascending order into one accumulator per output, which is the summation order of gemm_f16_kernel;
 //   * the elementwise steps are the shared static_apply<> functions on 16-byte pieces; REDUCE_MAX is exact;
 //     REDUCE_SUM is the reference's left-to-right fp16 fold (reduce.comp:24-70), here one lane per row: a single
-//     wavefront folds the block's 64 rows at once while the other three fetch the first chunk of V.
+//     wavefront folds the block's 64 rows at once (32 values per row in flight from shared memory while 32 are
+//     added) while the first chunk of V is on its way.
 #include "common.hpp"
 #include "dispatch.hpp"
 #include "float_programs.hpp"
@@ -35,6 +38,10 @@ constexpr int kHead = 64;       // head size: K of the first product, N of the s
 constexpr int kChunk = 64;      // keys per chunk of K^T / V
 constexpr int kChunkPitch = 2 * kChunk + 32;  // bytes per K row of a chunk: 4 rows x 32 B land on distinct banks
 constexpr int kMaxKeys = 512;   // 16 pieces of 16 bytes per thread
+constexpr int kPassKeys = 256;  // keys of a row that sit in shared memory at a time
+constexpr int kPasses = kMaxKeys / kPassKeys;
+constexpr int kPassChunks = kPassKeys / kChunk;
+constexpr int kPassPieces = kPassKeys / 32;  // 16-byte pieces per thread and pass
 
 struct AttnArgs {
     const char *q, *kt, *v;
@@ -70,8 +77,8 @@ __device__ __forceinline__ v8h as_v8h(const uint4 &u) {
 template <bool SCALED>
 __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g) {
     extern __shared__ __align__(16) char smem[];
-    const int SP = g.S * 2 + 16;   // pitch of a score row (bytes): consecutive rows start four banks apart
-    char *st = smem;               // [64][SP]: S, then EXP(..), then P
+    const int SP = min(g.S, kPassKeys) * 2 + 16;  // pitch of a score row (bytes): consecutive rows start four banks apart
+    char *st = smem;               // [64][SP]: one pass of S, later of EXP(..), later of P
     char *cb = smem + kRows * SP;  // [64][kChunkPitch]: a chunk of K^T or V; the row sums; the staged result
 
     const int lin = __builtin_amdgcn_readfirstlane((int)(blockIdx.x % 8u) * g.chunk + (int)(blockIdx.x / 8u));
@@ -110,12 +117,6 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
         *reinterpret_cast<uint4 *>(cb + c_row * kChunkPitch + c_piece * 16) = r[0];
         *reinterpret_cast<uint4 *>(cb + c_row * kChunkPitch + c_piece * 16 + 16) = r[1];
     };
-
-    // ---- phase 1: S = fp16(Q K^T), 64 keys at a time.  The query rows of this wavefront are matrix operands in registers.
-    v8h qf[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; kk++)
-        qf[kk] = as_v8h(load16(qres, (uint32_t)(m0 + wm * 32 + a_row) * g.ldq + (uint32_t)(kk * 16 + a_kg * 8) * 2));
     const int nchunks = g.S / kChunk;
     uint4 cr[2];
     auto fetch_kt = [&](int c) {  // rows = k (the head dimension), columns = the chunk's keys
@@ -128,34 +129,9 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
         cr[0] = load16(vres, c < nchunks ? off : kOob);
         cr[1] = load16(vres, c < nchunks ? off + 16 : kOob);
     };
-    fetch_kt(0);
-    for (int c = 0; c < nchunks; c++) {
-        __syncthreads();  // every wavefront has read the previous chunk
-        chunk_store(cr);
-        __syncthreads();
-        fetch_kt(c + 1);
-        v16f acc;
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[r] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag(kk), qf[kk], acc, 0, 0, 0);
-        // lane holds row lane % 32 of the tile and, per register quad q, columns 8 q + 4 (lane / 32) .. + 3
-        char *srow = st + (wm * 32 + (lane & 31)) * SP + (c * kChunk + wn * 32 + 4 * (lane >> 5)) * 2;
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            _Float16 h[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) h[e] = (_Float16)acc[4 * q + e];  // CAST: round to nearest even
-            uint2 w;
-            w.x = (uint32_t)__builtin_bit_cast(unsigned short, h[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[1]) << 16);
-            w.y = (uint32_t)__builtin_bit_cast(unsigned short, h[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[3]) << 16);
-            *reinterpret_cast<uint2 *>(srow + q * 16) = w;
-        }
-    }
-    __syncthreads();
-
-    // ---- phase 2: the softmax chain.  Four threads share a row (pieces quarter, quarter + 4, ...); the chain's full
-    // values stay in registers.
+    // The softmax chain: four threads share a row (pieces quarter, quarter + 4, ...) and keep the row's values in
+    // registers from the scores to P.  Shared memory holds one pass (256 keys) of a row at a time: it is where the
+    // products leave and fetch their operands and where the fold reads, and a thread always meets its own pieces there.
     const int row = tid >> 2, quarter = tid & 3;
     const int ppt = g.S >> 5;  // pieces per thread: S / 8 / 4, at most 16
     char *myrow = st + row * SP;
@@ -168,23 +144,64 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
     typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
     h2_t m2 = {(_Float16)-65504.f, (_Float16)-65504.f};
     uint32_t special = 0;
+
+    // ---- phase 1: S = fp16(Q K^T), 64 keys at a time.  The query rows of this wavefront are matrix operands in registers.
+    v8h qf[4];
 #pragma unroll
-    for (int u = 0; u < kMaxKeys / 32; u++) {
-        if (u < ppt) {
-            uint4 x = *reinterpret_cast<const uint4 *>(myrow + (quarter + 4 * u) * 16);
-            if (SCALED) {
-                x = static_apply<F_MUL>(x, make_uint4(scale_w, scale_w, scale_w, scale_w));
-                asm volatile("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));
+    for (int kk = 0; kk < 4; kk++)
+        qf[kk] = as_v8h(load16(qres, (uint32_t)(m0 + wm * 32 + a_row) * g.ldq + (uint32_t)(kk * 16 + a_kg * 8) * 2));
+    fetch_kt(0);
+#pragma unroll
+    for (int h = 0; h < kPasses; h++) {
+        if (h * kPassChunks < nchunks) {  // uniform
+            const int c_end = min(nchunks, (h + 1) * kPassChunks);
+            for (int c = h * kPassChunks; c < c_end; c++) {
+                __syncthreads();  // every wavefront has read the previous chunk (and the previous pass its scores)
+                chunk_store(cr);
+                __syncthreads();
+                fetch_kt(c + 1);
+                v16f acc;
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[r] = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag(kk), qf[kk], acc, 0, 0, 0);
+                // lane holds row lane % 32 of the tile and, per register quad q, columns 8 q + 4 (lane / 32) .. + 3
+                char *srow = st + (wm * 32 + (lane & 31)) * SP + ((c - h * kPassChunks) * kChunk + wn * 32 + 4 * (lane >> 5)) * 2;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    _Float16 hh[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) hh[e] = (_Float16)acc[4 * q + e];  // CAST: round to nearest even
+                    uint2 w;
+                    w.x = (uint32_t)__builtin_bit_cast(unsigned short, hh[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, hh[1]) << 16);
+                    w.y = (uint32_t)__builtin_bit_cast(unsigned short, hh[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, hh[3]) << 16);
+                    *reinterpret_cast<uint2 *>(srow + q * 16) = w;
+                }
             }
-            val[u] = x;
-            // REDUCE_MAX: exact; a NaN or an infinity anywhere in the row makes the maximum a NaN (as the row program)
-            special |= (((x.x & 0x7fff7fffu) + 0x03ff03ffu) | ((x.y & 0x7fff7fffu) + 0x03ff03ffu) |
-                        ((x.z & 0x7fff7fffu) + 0x03ff03ffu) | ((x.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
-            const h2_t *p = reinterpret_cast<const h2_t *>(&x);
-            m2 = __builtin_elementwise_max(m2, __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]),
-                                                                           __builtin_elementwise_max(p[2], p[3])));
+            __syncthreads();
+            // this pass's scores into registers, through the scale; the maximum as they pass
+#pragma unroll
+            for (int uu = 0; uu < kPassPieces; uu++) {
+                const int u = h * kPassPieces + uu;
+                if (u < ppt) {
+                    uint4 x = *reinterpret_cast<const uint4 *>(myrow + (quarter + 4 * uu) * 16);
+                    if (SCALED) {
+                        x = static_apply<F_MUL>(x, make_uint4(scale_w, scale_w, scale_w, scale_w));
+                        asm volatile("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));
+                    }
+                    val[u] = x;
+                    // REDUCE_MAX: exact; a NaN or an infinity anywhere in the row makes the maximum a NaN (as the row program)
+                    special |= (((x.x & 0x7fff7fffu) + 0x03ff03ffu) | ((x.y & 0x7fff7fffu) + 0x03ff03ffu) |
+                                ((x.z & 0x7fff7fffu) + 0x03ff03ffu) | ((x.w & 0x7fff7fffu) + 0x03ff03ffu)) & 0x80008000u;
+                    const h2_t *p = reinterpret_cast<const h2_t *>(&x);
+                    m2 = __builtin_elementwise_max(m2, __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]),
+                                                                                   __builtin_elementwise_max(p[2], p[3])));
+                }
+            }
         }
     }
+
+    // ---- phase 2: the rest of the softmax chain
     float mx = (float)(m2.x > m2.y ? m2.x : m2.y);
 #pragma unroll
     for (int d = 1; d < 4; d <<= 1) {
@@ -201,61 +218,99 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
             uint4 e = static_apply<F_EXP>(d, d);
             asm volatile("" : "+v"(e.x), "+v"(e.y), "+v"(e.z), "+v"(e.w));
             val[u] = e;
-            *reinterpret_cast<uint4 *>(myrow + (quarter + 4 * u) * 16) = e;  // for the fold
         }
     }
-    __syncthreads();
-    // REDUCE_SUM: left to right in fp16, one lane per row; meanwhile the other wavefronts request the first chunk of V
+    // REDUCE_SUM: left to right in fp16, one lane per row, a pass of the rows at a time; the first chunk of V is on its
+    // way meanwhile
     uint16_t *sums = reinterpret_cast<uint16_t *>(cb);  // [64]
-    if (wave == 0) {
-        const char *r = st + lane * SP;
-        __half acc = f2h(0.f);
-        const int segs = g.S >> 3;
-        uint4 cur = *reinterpret_cast<const uint4 *>(r);
-        for (int sg = 0; sg < segs; sg++) {
-            const uint4 nxt = *reinterpret_cast<const uint4 *>(r + (sg + 1 < segs ? sg + 1 : sg) * 16);
-            const __half2 *h = reinterpret_cast<const __half2 *>(&cur);
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                acc = __hadd(acc, __low2half(h[t]));
-                acc = __hadd(acc, __high2half(h[t]));
-            }
-            cur = nxt;
-        }
-        sums[lane] = __half_as_ushort(acc);
-    }
     fetch_v(0);
+    __half facc = f2h(0.f);
+#pragma unroll
+    for (int h = 0; h < kPasses; h++) {
+        if (h * kPassChunks < nchunks) {  // uniform
+            if (h > 0) __syncthreads();  // the previous pass has been folded
+#pragma unroll
+            for (int uu = 0; uu < kPassPieces; uu++) {
+                const int u = h * kPassPieces + uu;
+                if (u < ppt) *reinterpret_cast<uint4 *>(myrow + (quarter + 4 * uu) * 16) = val[u];
+            }
+            __syncthreads();
+            if (wave == 0) {
+                const char *r = st + lane * SP;
+                // 64 bytes (32 values) at a time through two register sets: one is folded while the other is on its
+                // way (a pass is a multiple of 64 keys, so it has an even number of sets)
+                const int sets = (min(g.S - h * kPassKeys, kPassKeys)) >> 5;
+                uint4 a[4], b[4];
+                auto fetch = [&](uint4 (&x)[4], int set) {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) x[t] = *reinterpret_cast<const uint4 *>(r + set * 64 + t * 16);
+                };
+                auto fold = [&](const uint4 (&x)[4]) {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const __half2 *hp = reinterpret_cast<const __half2 *>(&x[t]);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            facc = __hadd(facc, __low2half(hp[e]));
+                            facc = __hadd(facc, __high2half(hp[e]));
+                        }
+                    }
+                };
+                fetch(a, 0);
+                for (int set = 0; set < sets; set += 2) {
+                    fetch(b, set + 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    fold(a);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (set + 2 < sets) fetch(a, set + 2);  // uniform
+                    __builtin_amdgcn_sched_barrier(0);
+                    fold(b);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    }
+    if (wave == 0) sums[lane] = __half_as_ushort(facc);
     __syncthreads();
+    uint4 rrow;
     {
         const uint32_t sbits = sums[row];
         const uint32_t sw = sbits | (sbits << 16);
         uint4 rc = static_apply<F_RECIPROCAL>(make_uint4(sw, sw, sw, sw), make_uint4(sw, sw, sw, sw));
         asm volatile("" : "+v"(rc.x));
-        const uint4 rrow = make_uint4(rc.x, rc.x, rc.x, rc.x);
-#pragma unroll
-        for (int u = 0; u < kMaxKeys / 32; u++) {
-            if (u < ppt) {
-                uint4 p = static_apply<F_MUL>(val[u], rrow);
-                asm volatile("" : "+v"(p.x), "+v"(p.y), "+v"(p.z), "+v"(p.w));
-                *reinterpret_cast<uint4 *>(myrow + (quarter + 4 * u) * 16) = p;
-            }
-        }
+        rrow = make_uint4(rc.x, rc.x, rc.x, rc.x);
     }
 
-    // ---- phase 3: O = fp16(P V), 64 keys at a time
+    // ---- phase 3: O = fp16(P V), 64 keys at a time, P a pass at a time
     v16f acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
     const char *p_base = st + (wm * 32 + a_row) * SP + a_kg * 16;
-    for (int c = 0; c < nchunks; c++) {
-        __syncthreads();  // the previous chunk (or the row sums) has been read; P is complete
-        chunk_store(cr);
-        __syncthreads();
-        fetch_v(c + 1);
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
-            const v8h pf = *reinterpret_cast<const v8h *>(p_base + (c * kChunk + kk * 16) * 2);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag(kk), pf, acc, 0, 0, 0);
+    for (int h = 0; h < kPasses; h++) {
+        if (h * kPassChunks < nchunks) {  // uniform
+            if (h > 0) __syncthreads();  // the previous pass of P has been multiplied
+#pragma unroll
+            for (int uu = 0; uu < kPassPieces; uu++) {
+                const int u = h * kPassPieces + uu;
+                if (u < ppt) {
+                    uint4 p = static_apply<F_MUL>(val[u], rrow);
+                    asm volatile("" : "+v"(p.x), "+v"(p.y), "+v"(p.z), "+v"(p.w));
+                    *reinterpret_cast<uint4 *>(myrow + (quarter + 4 * uu) * 16) = p;
+                }
+            }
+            const int c_end = min(nchunks, (h + 1) * kPassChunks);
+            for (int c = h * kPassChunks; c < c_end; c++) {
+                __syncthreads();  // the previous chunk (or the row sums) has been read; this pass of P is complete
+                chunk_store(cr);
+                __syncthreads();
+                fetch_v(c + 1);
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {
+                    const v8h pf = *reinterpret_cast<const v8h *>(p_base + ((c - h * kPassChunks) * kChunk + kk * 16) * 2);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(b_frag(kk), pf, acc, 0, 0, 0);
+                }
+            }
         }
     }
     __syncthreads();
@@ -418,20 +473,20 @@ int try_attention_f16(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, cons
     AttnArgs g{};
     const int form = describe(out, q, kt, v, chain, true, &g);
     if (form == 0) return 0;
-    const size_t sm = (size_t)kRows * (g.S * 2 + 16) + (size_t)kChunk * kChunkPitch;
+    const size_t sm = (size_t)kRows * (std::min(g.S, kPassKeys) * 2 + 16) + (size_t)kChunk * kChunkPitch;
     const dim3 grid((unsigned)(g.chunk * 8));
     if (form == 2) {
         auto kernel = attention_f16_kernel<true>;
         static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                       kRows * (kMaxKeys * 2 + 16) + kChunk * kChunkPitch) == hipSuccess;
+                                                       kRows * (kPassKeys * 2 + 16) + kChunk * kChunkPitch) == hipSuccess;
         (void)raised;
         kernel<<<grid, dim3(kBlock), sm, s>>>(g);
     } else {
         auto kernel = attention_f16_kernel<false>;
         static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                       kRows * (kMaxKeys * 2 + 16) + kChunk * kChunkPitch) == hipSuccess;
+                                                       kRows * (kPassKeys * 2 + 16) + kChunk * kChunkPitch) == hipSuccess;
         (void)raised;
         kernel<<<grid, dim3(kBlock), sm, s>>>(g);
     }

@@ -475,6 +475,8 @@ ATTENTION_CASES = [  # heads, queries, keys, scaled, head-merge view
     (2, 128, 512, True, False),
     (5, 192, 320, False, False),
     (2 * 3, 64, 128, True, True),
+    (4, 64, 256, True, False),   # the keys of exactly one pass through shared memory
+    (2 * 3, 128, 448, False, True),  # a full pass and three chunks of a second one
 ]
 
 
