@@ -55,7 +55,7 @@ struct AttnArgs {
     int32_t view, v_nb2, v_m2, v_n2;
     int64_t vs_nb1, vs_nb2;
     uint32_t vs_m1, vs_m2, vs_n1;
-    int32_t total, chunk;
+    int32_t total, chunk, fold_span;
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const void *p, uint32_t bytes) {
@@ -169,12 +169,9 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
                 char *srow = st + (wm * 32 + (lane & 31)) * SP + ((c - h * kPassChunks) * kChunk + wn * 32 + 4 * (lane >> 5)) * 2;
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    _Float16 hh[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) hh[e] = (_Float16)acc[4 * q + e];  // CAST: round to nearest even
-                    uint2 w;
-                    w.x = (uint32_t)__builtin_bit_cast(unsigned short, hh[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, hh[1]) << 16);
-                    w.y = (uint32_t)__builtin_bit_cast(unsigned short, hh[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, hh[3]) << 16);
+                    uint2 w;  // CAST: round to nearest even
+                    w.x = __builtin_bit_cast(uint32_t, pack_f16(acc[4 * q + 0], acc[4 * q + 1]));
+                    w.y = __builtin_bit_cast(uint32_t, pack_f16(acc[4 * q + 2], acc[4 * q + 3]));
                     *reinterpret_cast<uint2 *>(srow + q * 16) = w;
                 }
             }
@@ -223,6 +220,10 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
     // REDUCE_SUM: left to right in fp16, one lane per row, a pass of the rows at a time; the first chunk of V is on its
     // way meanwhile
     uint16_t *sums = reinterpret_cast<uint16_t *>(cb);  // [64]
+    // The blocks that share a compute unit run in step and fold at the same time; three chains on one SIMD would take
+    // turns (a wavefront instruction holds the SIMD for four clocks), so the folding wavefront rotates with the round
+    // of blocks (blocks are dealt to a unit one round at a time: g.fold_span = blocks per round and XCD).
+    const int fold_wave = (int)((uint32_t)(blockIdx.x / 8u) / (uint32_t)g.fold_span) & 3;
     fetch_v(0);
     __half facc = f2h(0.f);
 #pragma unroll
@@ -235,7 +236,7 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
                 if (u < ppt) *reinterpret_cast<uint4 *>(myrow + (quarter + 4 * uu) * 16) = val[u];
             }
             __syncthreads();
-            if (wave == 0) {
+            if (wave == fold_wave) {
                 const char *r = st + lane * SP;
                 // 64 bytes (32 values) at a time through two register sets: one is folded while the other is on its
                 // way (a pass is a multiple of 64 keys, so it has an even number of sets)
@@ -270,7 +271,7 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
             }
         }
     }
-    if (wave == 0) sums[lane] = __half_as_ushort(facc);
+    if (wave == fold_wave) sums[lane] = __half_as_ushort(facc);
     __syncthreads();
     uint4 rrow;
     {
@@ -320,12 +321,9 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
         char *orow = cb + (wm * 32 + (lane & 31)) * OP + (wn * 32 + 4 * (lane >> 5)) * 2;
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            _Float16 h[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) h[e] = (_Float16)acc[4 * q + e];
             uint2 w;
-            w.x = (uint32_t)__builtin_bit_cast(unsigned short, h[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[1]) << 16);
-            w.y = (uint32_t)__builtin_bit_cast(unsigned short, h[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, h[3]) << 16);
+            w.x = __builtin_bit_cast(uint32_t, pack_f16(acc[4 * q + 0], acc[4 * q + 1]));
+            w.y = __builtin_bit_cast(uint32_t, pack_f16(acc[4 * q + 2], acc[4 * q + 3]));
             *reinterpret_cast<uint2 *>(orow + q * 16) = w;
         }
     }
@@ -469,12 +467,12 @@ bool attention_f16_supported(const mlel_tensor *out, const mlel_tensor *q, const
 
 int try_attention_f16(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt,
                       const mlel_tensor *v, const mlel_chain *chain) {
-    (void)ctx;
     AttnArgs g{};
     const int form = describe(out, q, kt, v, chain, true, &g);
     if (form == 0) return 0;
     const size_t sm = (size_t)kRows * (std::min(g.S, kPassKeys) * 2 + 16) + (size_t)kChunk * kChunkPitch;
     const dim3 grid((unsigned)(g.chunk * 8));
+    g.fold_span = std::max(1, (ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256) / 8);
     if (form == 2) {
         auto kernel = attention_f16_kernel<true>;
         static const bool raised = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),

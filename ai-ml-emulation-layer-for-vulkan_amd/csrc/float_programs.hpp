@@ -17,7 +17,10 @@ enum FOp { F_ADD, F_SUB, F_MUL, F_EXP, F_RECIPROCAL, F_RSQRT, F_TANH, F_COPY };
 // bit.  (In the reference these functions are the Vulkan driver's and differ from driver to driver.)
 template <bool F16>
 __device__ __forceinline__ float op_exp(float x) {
-    return F16 ? __expf(x) : expf(x);
+    // v_exp_f32 of x * log2(e); written as a fused multiply-add with zero so that an argument that has just been
+    // widened from fp16 takes one v_fma_mix_f32 instead of a conversion and a multiplication (same bits: the
+    // product is rounded once either way)
+    return F16 ? __builtin_amdgcn_exp2f(__builtin_fmaf(x, 1.44269504088896340736f, 0.0f)) : expf(x);
 }
 template <bool F16>
 __device__ __forceinline__ float op_reciprocal(float x) {
@@ -63,6 +66,16 @@ struct StaticArgs {
     const char *in[MLEL_CHAIN_MAX_INPUTS];
 };
 
+// two fp32 results rounded to fp16 (nearest even) with one v_cvt_pk_f16_f32
+__device__ __forceinline__ __half2 pack_f16(float a, float b) {
+    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+    typedef float f2_t __attribute__((ext_vector_type(2)));
+    asm("" : "+v"(a), "+v"(b));  // the values as computed: nothing is folded into the rounding
+    const f2_t v = {a, b};
+    const h2_t h = __builtin_convertvector(v, h2_t);
+    return __builtin_bit_cast(__half2, h);
+}
+
 template <int OP>
 __device__ __forceinline__ uint4 static_apply(const uint4 &a, const uint4 &b) {
     uint4 r;
@@ -82,7 +95,7 @@ __device__ __forceinline__ uint4 static_apply(const uint4 &a, const uint4 &b) {
                            : OP == F_RSQRT ? op_rsqrt<true>(f.x) : OP == F_TANH ? op_tanh<true>(f.x) : f.x;
             const float y1 = OP == F_EXP ? op_exp<true>(f.y) : OP == F_RECIPROCAL ? op_reciprocal<true>(f.y)
                            : OP == F_RSQRT ? op_rsqrt<true>(f.y) : OP == F_TANH ? op_tanh<true>(f.y) : f.y;
-            rh[i] = __halves2half2(f2h(y0), f2h(y1));
+            rh[i] = pack_f16(y0, y1);
         }
     }
     return r;
