@@ -34,11 +34,13 @@ template <bool F16>
 __device__ __forceinline__ float op_tanh(float x) {
     if (!F16) return tanh_clamped(x);
     // the reference's three ranges (elementwise_unary.comp:136-155) with tanh(x) = 1 - 2 / (exp(2x) + 1) in between
-    const float ax = fabsf(x);
+    // exp(2x) as one v_exp_f32 of x * 2 log2(e) (doubling commutes with the rounding of the product).  Beyond
+    // |x| = 10 the middle formula already gives exactly +-1 (and NaN for NaN), so the third range needs no test.
     const float x2 = x * x;
     const float small = x * (1.0f - x2 * (1.0f / 3.0f - x2 * (2.0f / 15.0f - 17.0f / 315.0f * x2)));
-    const float mid = 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * x) + 1.0f);
-    return ax > 10.0f ? copysignf(1.0f, x) : (ax < 0.2f ? small : mid);
+    const float e2x = __builtin_amdgcn_exp2f(__builtin_fmaf(x, 2.0f * 1.44269504088896340736f, 0.0f));
+    const float mid = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e2x + 1.0f);
+    return fabsf(x) < 0.2f ? small : mid;
 }
 
 // ---------------------------------------------------------------------------------------------------------------
