@@ -186,7 +186,8 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
         // ---- direct-to-LDS main loop (K % 32 == 0: whole 64-byte steps)
         constexpr int BK = 64, DL_S = 4, DL_STAGE = (BM + BN) * BK;
         constexpr int XI = BM * 4 / NT, WI = BN * 4 / NT;  // 16-byte pieces per thread and stage
-        static_assert((BM * 4) % NT == 0 && (BN * 4) % NT == 0 && 6 * (XI + WI) < 64, "whole pieces per thread");
+        // (request counts above 15 need the upper bits of the vmcnt field, a path no instance has exercised)
+        static_assert((BM * 4) % NT == 0 && (BN * 4) % NT == 0 && (DL_S - 1) * (XI + WI) < 16, "whole pieces per thread");
         const int wave_u = __builtin_amdgcn_readfirstlane(wave);
         uint32_t xo[XI], wo[WI];
 #pragma unroll
