@@ -512,6 +512,33 @@ def test_attention_equals_the_three_launches(run, case):
     np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
 
 
+def test_attention_with_special_values_equals_the_three_launches(run):
+    """Rows whose scores overflow to +-infinity or hold a NaN: a row with a NaN or +infinity comes out all NaN from both
+    paths, a row with -infinity scores (a masked key) stays finite and keeps the launches' bits; 320 keys, so the rows
+    cross the boundary between two passes through shared memory."""
+    nb, m, s = 2, 64, 320
+    rng = np.random.default_rng(77)
+    q = rng.standard_normal((nb, m, 64)).astype(np.float16)
+    kt = rng.standard_normal((nb, 64, s)).astype(np.float16)
+    v = rng.standard_normal((nb, s, 64)).astype(np.float16)
+    q[0, 3, :] = 200.0
+    q[0, 5, :] = -200.0
+    kt[0, :, 300] = 200.0       # row 3: +inf at key 300, row 5: -inf there
+    q[1, 7, 10] = np.nan        # row 7 of the second head: NaN scores everywhere
+    kt[1, :, 17] = -65504.0     # a key that is very negative for positive queries
+    Bk, Mk, Uk, Rk = 0, 1, 2, 4
+    f16 = abi.F16
+    steps = [(Rk, abi.RED["MAX"], 0, 0, f16), (Bk, abi.BIN["SUB"], 0, 1, f16), (Uk, abi.UN["EXP"], 2, 0, f16),
+             (Rk, abi.RED["SUM"], 3, 0, f16), (Uk, abi.UN["RECIPROCAL"], 4, 0, f16), (Mk, 0, 3, 5, f16)]
+    scores = run.matmul_bias_cast(q, kt, None)
+    assert np.isposinf(scores[0, 3, 300]) and np.isneginf(scores[0, 5, 300]) and np.isnan(scores[1, 7]).all()
+    prob = run.chain([scores], steps, scores.shape, f16)
+    want = run.matmul_bias_cast(prob, v, None)
+    got = run.attention(q, kt, v, [], steps)
+    assert np.isnan(want[0, 3]).all() and np.isnan(want[1, 7]).all() and np.isfinite(want[0, 5].astype(np.float32)).all()
+    _same_bits_or_both_nan(got, want)
+
+
 def test_attention_declines_what_the_kernel_was_not_written_for(run):
     """Other head sizes, row counts or chains are MLEL_ERR_UNSUPPORTED: nothing is allocated, nothing falls back."""
     rng = np.random.default_rng(5)
