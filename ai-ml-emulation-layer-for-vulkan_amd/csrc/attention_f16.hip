@@ -135,6 +135,11 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
     const int row = tid >> 2, quarter = tid & 3;
     const int ppt = g.S >> 5;  // pieces per thread: S / 8 / 4, at most 16
     char *myrow = st + row * SP;
+    // Which of a row's 16-byte pieces its four threads take in a pass: piece 2 quarter + uu % 2 + 8 (uu / 2), i.e. the
+    // four threads of a row are 32 bytes apart and rows 33 pieces: a 128-bit access of the wavefront then runs at
+    // full rate (measured: quarter + 4 uu, the threads 16 bytes apart, takes 1.6 times as long).  A pass has an even
+    // number of pieces per thread, so this is a bijection onto the row's pieces.
+    auto piece_off = [&](int, int uu) { return (2 * quarter + (uu & 1) + 8 * (uu >> 1)) * 16; };
     uint4 val[kMaxKeys / 32];
     uint32_t scale_w = 0;
     if (SCALED) {
@@ -181,7 +186,7 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
             for (int uu = 0; uu < kPassPieces; uu++) {
                 const int u = h * kPassPieces + uu;
                 if (u < ppt) {
-                    uint4 x = *reinterpret_cast<const uint4 *>(myrow + (quarter + 4 * uu) * 16);
+                    uint4 x = *reinterpret_cast<const uint4 *>(myrow + piece_off(h, uu));
                     if (SCALED) {
                         x = static_apply<F_MUL>(x, make_uint4(scale_w, scale_w, scale_w, scale_w));
                         asm volatile("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));
@@ -233,7 +238,7 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
 #pragma unroll
             for (int uu = 0; uu < kPassPieces; uu++) {
                 const int u = h * kPassPieces + uu;
-                if (u < ppt) *reinterpret_cast<uint4 *>(myrow + (quarter + 4 * uu) * 16) = val[u];
+                if (u < ppt) *reinterpret_cast<uint4 *>(myrow + piece_off(h, uu)) = val[u];
             }
             __syncthreads();
             if (wave == fold_wave) {
@@ -297,7 +302,7 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
                 if (u < ppt) {
                     uint4 p = static_apply<F_MUL>(val[u], rrow);
                     asm volatile("" : "+v"(p.x), "+v"(p.y), "+v"(p.z), "+v"(p.w));
-                    *reinterpret_cast<uint4 *>(myrow + (quarter + 4 * uu) * 16) = p;
+                    *reinterpret_cast<uint4 *>(myrow + piece_off(h, uu)) = p;
                 }
             }
             const int c_end = min(nchunks, (h + 1) * kPassChunks);
