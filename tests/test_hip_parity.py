@@ -539,6 +539,44 @@ def test_attention_with_special_values_equals_the_three_launches(run):
     _same_bits_or_both_nan(got, want)
 
 
+def test_random_sweep_of_attention_and_row_wise_products(run):
+    """Random extents: the attention kernel against the three launches it replaces (1 - 4 heads, 64 - 256 queries, 64 -
+    512 keys, with and without the scale, queries of different spread), and fp16 products with a row-wise B against the
+    K-major form (M 1 - 599, K 32 - 1248, N 8 - 472, with and without bias): the same bits."""
+    rng0 = np.random.default_rng(4242)
+    Bk, Mk, Uk, Rk = 0, 1, 2, 4
+    f16 = abi.F16
+    for i in range(60):
+        nb, m, s = int(rng0.integers(1, 5)), 64 * int(rng0.integers(1, 5)), 64 * int(rng0.integers(1, 9))
+        scaled, spread = bool(rng0.integers(0, 2)), float(rng0.uniform(0.3, 3))
+        rng = np.random.default_rng(i)
+        q = (rng.standard_normal((nb, m, 64)) * spread).astype(np.float16)
+        kt = rng.standard_normal((nb, 64, s)).astype(np.float16)
+        v = rng.standard_normal((nb, s, 64)).astype(np.float16)
+        o = 2 if scaled else 0
+        steps = [(Rk, abi.RED["MAX"], o, 0, f16), (Bk, abi.BIN["SUB"], o, o + 1, f16), (Uk, abi.UN["EXP"], o + 2, 0, f16),
+                 (Rk, abi.RED["SUM"], o + 3, 0, f16), (Uk, abi.UN["RECIPROCAL"], o + 4, 0, f16), (Mk, 0, o + 3, o + 5, f16)]
+        extra = []
+        if scaled:
+            steps = [(Mk, 0, 0, 1, f16)] + steps
+            extra = [np.array(0.125, np.float16).reshape(1, 1, 1)]
+        scores = run.matmul_bias_cast(q, kt, None)
+        prob = run.chain([scores] + extra, steps, scores.shape, f16)
+        want = run.matmul_bias_cast(prob, v, None)
+        got = run.attention(q, kt, v, extra, steps)
+        _same_bits_or_both_nan(got, want)
+    for i in range(60):
+        rng = np.random.default_rng(1000 + i)
+        nb, m = int(rng.integers(1, 3)), int(rng.integers(1, 600))
+        k, n = 32 * int(rng.integers(1, 40)), 8 * int(rng.integers(1, 60))
+        a = rng.standard_normal((nb, m, k)).astype(np.float16)
+        b = (0.1 * rng.standard_normal((nb, k, n))).astype(np.float16)
+        bias = rng.standard_normal((1, 1, n)).astype(np.float32) if i % 2 else None
+        want = run.matmul_bias_cast(a, b, bias)
+        got = run.matmul_bias_cast(a, b, bias, b_rows=True)
+        np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16), err_msg=str((nb, m, k, n)))
+
+
 def test_attention_declines_what_the_kernel_was_not_written_for(run):
     """Other head sizes, row counts or chains are MLEL_ERR_UNSUPPORTED: nothing is allocated, nothing falls back."""
     rng = np.random.default_rng(5)
@@ -1448,6 +1486,75 @@ def test_pointwise_conv_random_shapes_with_and_without_residual(run, oracle, see
     got = run.conv2d_rescale_add_rescale(x, w, b, attr, (mult, shift, rattr, (-100, 110)), (m1, s1, a_conv, None), res,
                                          (m2, s2, a_res, None), (mo, so, a_out, None), residual_first=bool(rng.integers(0, 2)))
     np.testing.assert_array_equal(got, exp)
+
+
+def test_random_sweep_of_fused_contractions(run, oracle):
+    """A few hundred random draws each of the fused CONV2D (any kernel up to 3x3, stride, padding, dilation, channel
+    counts that are and are not multiples of four), DEPTHWISE_CONV2D (kernels up to 5x5, channel multiplier 1 or 2) and
+    int8 MATMUL + RESCALE (K-major and row-wise B) against the oracle, bit for bit: whichever kernel the dispatcher
+    picks for a draw has to agree."""
+    ran = [0, 0, 0]
+    for i in range(400):
+        rng = np.random.default_rng(20000 + i)
+        n, h, w_ = int(rng.integers(1, 4)), int(rng.integers(3, 40)), int(rng.integers(3, 40))
+        kh, kw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        sy, sx = int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        dy, dx = (int(rng.integers(1, 3)), int(rng.integers(1, 3))) if i % 5 == 0 else (1, 1)
+        ic = int(rng.choice([3, 4, 8, 16, 24, 32, 48, 64, 96, 100, 144]))
+        oc = int(rng.choice([1, 4, 8, 16, 24, 32, 40, 64, 96, 130]))
+        pt, pb, pl, pr = [int(v) for v in rng.integers(0, 2, 4)]
+        eh, ew = (kh - 1) * dy + 1, (kw - 1) * dx + 1
+        if h + pt + pb < eh or w_ + pl + pr < ew or (h + pt + pb - eh) % sy or (w_ + pl + pr - ew) % sx:
+            continue
+        shape = (n, (h + pt + pb - eh) // sy + 1, (w_ + pl + pr - ew) // sx + 1, oc)
+        x = ri(rng, -128, 127, (n, h, w_, ic), np.int8)
+        w = ri(rng, -127, 127, (oc, kh, kw, ic), np.int8)
+        b = ri(rng, -2 ** 15, 2 ** 15, (oc,), np.int32)
+        attr = abi.conv2d_attr((pt, pb, pl, pr), (sy, sx), (dy, dx), int(rng.integers(-128, 128)), 0)
+        per_channel = bool(rng.integers(0, 2))
+        k = oc if per_channel else 1
+        mult, shift = ri(rng, 2 ** 30, 2 ** 31 - 1, (k,), np.int32), ri(rng, 36, 46, (k,), np.int8)
+        rattr = abi.rescale_attr(0, int(rng.integers(-20, 20)), True, bool(rng.integers(0, 2)), per_channel)
+        exp = oracle.clamp(oracle.rescale(oracle.conv2d(x, w, b, shape, abi.I32, attr), mult, shift, abi.I8, rattr), -110, 100)
+        got = run.conv2d(x, w, b, shape, abi.I8, attr, epilogue=(mult, shift, rattr, (-110, 100)))
+        np.testing.assert_array_equal(got, exp, err_msg=f"conv draw {i}")
+        ran[0] += 1
+    for i in range(400):
+        rng = np.random.default_rng(30000 + i)
+        n, h, w_ = int(rng.integers(1, 4)), int(rng.integers(3, 40)), int(rng.integers(3, 40))
+        kh, kw = (3, 3) if i % 3 else (int(rng.integers(1, 6)), int(rng.integers(1, 6)))
+        st = int(rng.integers(1, 3))
+        c, mch = int(rng.choice([4, 8, 16, 32, 48, 96, 144, 20, 36])), 1 if i % 7 else 2
+        pt, pb, pl, pr = [int(v) for v in rng.integers(0, 2, 4)]
+        if h + pt + pb < kh or w_ + pl + pr < kw or (h + pt + pb - kh) % st or (w_ + pl + pr - kw) % st:
+            continue
+        oc = c * mch
+        shape = (n, (h + pt + pb - kh) // st + 1, (w_ + pl + pr - kw) // st + 1, oc)
+        x = ri(rng, -128, 127, (n, h, w_, c), np.int8)
+        w = ri(rng, -127, 127, (kh, kw, c, mch), np.int8)
+        b = ri(rng, -2 ** 15, 2 ** 15, (oc,), np.int32)
+        attr = abi.conv2d_attr((pt, pb, pl, pr), (st, st), (1, 1), int(rng.integers(-128, 128)), 0)
+        mult, shift = ri(rng, 2 ** 30, 2 ** 31 - 1, (oc,), np.int32), ri(rng, 32, 40, (oc,), np.int8)
+        rattr = abi.rescale_attr(0, int(rng.integers(-20, 20)), True, True, True)
+        exp = oracle.clamp(oracle.rescale(oracle.depthwise_conv2d(x, w, b, shape, abi.I32, attr), mult, shift, abi.I8, rattr), -128, 127)
+        got = run.conv2d(x, w, b, shape, abi.I8, attr, depthwise=True, epilogue=(mult, shift, rattr, (-128, 127)))
+        np.testing.assert_array_equal(got, exp, err_msg=f"depthwise draw {i}")
+        ran[1] += 1
+    for i in range(200):
+        rng = np.random.default_rng(40000 + i)
+        nb, m = int(rng.integers(1, 4)), int(rng.integers(1, 300))
+        k, n = int(rng.choice([16, 32, 48, 64, 100, 256, 500, 1024])), int(rng.choice([1, 4, 16, 20, 64, 128, 200, 512]))
+        a, b = ri(rng, -128, 127, (nb, m, k), np.int8), ri(rng, -128, 127, (nb, k, n), np.int8)
+        za, zb = int(rng.integers(-128, 128)), (int(rng.integers(-128, 128)) if i % 2 else 0)
+        mult = np.array([int(rng.integers(2 ** 30, 2 ** 31 - 1))], np.int32)
+        shift = np.array([int(rng.integers(36, 46))], np.int8)
+        rattr = abi.rescale_attr(0, int(rng.integers(-20, 20)), True, True, False)
+        exp = oracle.rescale(oracle.matmul(a, b, abi.I32, za, zb), mult, shift, abi.I8, rattr)
+        for rows in (False, True):
+            got = run.matmul(a, b, abi.I8, za, zb, epilogue=(mult, shift, rattr, None), b_rows=rows)
+            np.testing.assert_array_equal(got, exp, err_msg=f"matmul draw {i} b_rows={rows}")
+        ran[2] += 1
+    assert ran[0] > 150 and ran[1] > 150 and ran[2] == 200, ran
 
 
 RESIDUAL_CASES = [
