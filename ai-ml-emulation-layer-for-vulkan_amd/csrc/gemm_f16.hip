@@ -429,8 +429,21 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
                 }
             }
         }
-        __syncthreads();
         const __amdgpu_buffer_rsrc_t rres = rsrc(g.res != nullptr ? g.res + (int64_t)batch * g.r_batch : o.out, g.res != nullptr ? g.r_bytes : 0);
+        // the residual's pieces of this thread, requested before the barrier and before any store (a load behind a
+        // store waits for it, and one fetch per piece in the store loop would expose its latency four times over)
+        constexpr int PIECES = BM * (BN / 8) / NT;
+        constexpr bool RES_AHEAD = PIECES <= 4;
+        uint4 res_r[RES_AHEAD ? PIECES : 1];
+        if (RES_AHEAD && g.res != nullptr && o.view != 2) {  // uniform
+#pragma unroll
+            for (int i = 0; i < (RES_AHEAD ? PIECES : 1); i++) {
+                const int p = i * NT + tid, r = p / (BN / 8), c = p % (BN / 8);
+                const int m = m_base + r, n = n_base + c * 8;
+                res_r[i] = load16(rres, (m < g.M && n < g.N) ? (uint32_t)m * g.ldr + (uint32_t)n * 2 : kOob);
+            }
+        }
+        __syncthreads();
         const ViewDiv by_m2(o.view ? o.v_m2 : 1, g.M), by_n2(o.view ? o.v_n2 : 1, g.N);
         if (o.view == 2) {
             // transposing view: a piece is eight consecutive rows of one column (tile rows start at multiples of
@@ -473,7 +486,8 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
             }
             if (g.act[0] != nullptr) piece = gelu_tanh_piece(piece, act_c);  // uniform
             if (g.res != nullptr) {  // uniform; ADD of two fp16 tensors: one rounding of the exact sum
-                const uint4 other = load16(rres, inside ? (uint32_t)m * g.ldr + (uint32_t)n * 2 : kOob);
+                const uint4 other = RES_AHEAD ? res_r[RES_AHEAD ? p0 / NT : 0]
+                                              : load16(rres, inside ? (uint32_t)m * g.ldr + (uint32_t)n * 2 : kOob);
                 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
                 h2_t *ph = reinterpret_cast<h2_t *>(&piece);
                 const h2_t *oh = reinterpret_cast<const h2_t *>(&other);
