@@ -706,14 +706,16 @@ int launch_args(mlel_ctx *ctx, hipStream_t s, HGemmArgs &g, bool bias_cast) {
     // The 256 x 256 tile of eight wavefronts (128 x 64 each: a third fewer operand reads from shared memory per
     // multiply) when it still occupies three quarters of the compute units: 4096 x 768 x 3072 in 192 tiles,
     // 37.7 -> 34.7 us.  With fewer tiles the idle compute units cost more than the reads (144 tiles: no gain;
-    // 48 tiles: twice the time), and so does an activation in the epilogue, whose arithmetic then runs on three
-    // quarters of the machine (the same product with the tanh GELU: 40.9 -> 44.1 us).
+    // 48 tiles: twice the time).  With the K-major loop an activation in the epilogue loses too, its arithmetic
+    // running on three quarters of the machine (the same product with the tanh GELU: 40.9 -> 44.1 us); with the
+    // direct-to-LDS loop it gains a little (38.4 -> 37.3 us inside the encoder block), so that path takes the large
+    // tile with or without one.
     const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256) * NB;
     if (g.b_rows) {
         // row-wise B: the direct-to-LDS loop; the 256 x 256 tile under the same condition as below, else 128 x 128 of
         // eight wavefronts, whatever the extents (rows beyond M or N are fetched as zeros)
         const int64_t tn128 = (N + 127) / 128;
-        if (g.groups == 1 && g.act[0] == nullptr && g.K >= 256 && tiles256 * 4 >= 3 * (int64_t)cus && tiles256 <= 2 * (int64_t)cus) {
+        if (g.groups == 1 && g.K >= 256 && tiles256 * 4 >= 3 * (int64_t)cus && tiles256 <= 2 * (int64_t)cus) {
             g.tiles_m = (int)((M + 255) / 256);
             g.tiles_n_group = (int)((N + 255) / 256);
             g.tiles_n = g.tiles_n_group;

@@ -410,7 +410,7 @@ def test_matmul_bias_cast_chain_equals_product_then_chain(run):
 
 
 BROWS_SHAPES = [(1, 256, 768, 768), (2, 130, 96, 136), (1, 33, 32, 8), (1, 512, 3072, 768), (1, 300, 64, 392), (3, 64, 160, 128),
-                (1, 1024, 768, 1024), (1, 200, 2080, 136)]
+                (1, 1024, 768, 1024), (1, 200, 2080, 136), (1, 4096, 256, 3072)]  # the last one: 192 tiles of 256 x 256
 
 
 @pytest.mark.parametrize("shape", BROWS_SHAPES, ids=str)
