@@ -272,6 +272,8 @@ RUNTIME_SIGNATURES = {
     "mlel_hip_destroy": (None, [_V]),
     "mlel_hip_device_info": (C.c_int, [_V, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32),
                                        C.POINTER(C.c_int32), C.c_char_p, C.c_size_t]),
+    "mlel_hip_static_scratch_last_use": (C.c_int, [_V]),
+    "mlel_hip_split_workspaces": (C.c_int, [_V]),
     "mlel_hip_arena_alloc": (C.c_int, [_V, C.c_size_t, C.POINTER(_V)]),
     "mlel_hip_arena_free": (C.c_int, [_V, _V]),
     "mlel_hip_arena_import_fd": (C.c_int, [_V, C.c_int, C.c_size_t, C.POINTER(_V), C.POINTER(_V)]),
@@ -292,6 +294,7 @@ RUNTIME_SIGNATURES = {
     "mlel_hip_graph_launch": (C.c_int, [_V, _V, _V]),
     "mlel_hip_graph_destroy": (C.c_int, [_V, _V]),
     "mlel_hip_copy_kernel": (C.c_int, [_V, _V, _V, _V, C.c_size_t]),
+    "mlel_hip_copy_kernel_variant": (C.c_int, [_V, _V, _V, _V, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int]),
     "mlel_hip_matmul_chain_in_kernel": (C.c_int, [C.POINTER(Chain)]),
     "mlel_hip_attention_f16_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Chain)]),
     "mlel_hip_conv2d_dwconv_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Conv2dAttr), _T, _T,
@@ -320,27 +323,6 @@ def bind_hip(lib):
     return lib
 
 
-def bind_oracle(lib):
-    for name, args in OP_SIGNATURES.items():
-        fn = getattr(lib, "mlel_cpu_" + name)
-        fn.restype = C.c_int
-        fn.argtypes = args
-    lib.mlel_cpu_last_error.restype = C.c_char_p
-    lib.mlel_cpu_num_threads.restype = C.c_int
-    lib.mlel_cpu_f32_to_f16.restype = C.c_uint16
-    lib.mlel_cpu_f32_to_f16.argtypes = [C.c_float]
-    lib.mlel_cpu_f16_to_f32.restype = C.c_float
-    lib.mlel_cpu_f16_to_f32.argtypes = [C.c_uint16]
-    lib.mlel_cpu_f32_to_bf16.restype = C.c_uint16
-    lib.mlel_cpu_f32_to_bf16.argtypes = [C.c_float, C.c_int]
-    lib.mlel_cpu_f32_to_f8.restype = C.c_uint8
-    lib.mlel_cpu_f32_to_f8.argtypes = [C.c_float, C.c_int]
-    lib.mlel_cpu_f8_to_f32.restype = C.c_float
-    lib.mlel_cpu_f8_to_f32.argtypes = [C.c_uint8, C.c_int]
-    return lib
-
-
 REPO_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HIP_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libmlel_hip.so")
 GRAPH_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libmlel_graph.so")
-ORACLE_LIB_PATH = os.path.join(REPO_ROOT, "oracle", "libmlel_oracle.so")

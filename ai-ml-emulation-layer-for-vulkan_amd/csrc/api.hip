@@ -550,6 +550,7 @@ int mlel_hip_conv2d_rescale_clamp_static(mlel_ctx *ctx, void *stream, const mlel
                          kStaticScratchPartialBytes, &used_split};
     int rc = try_conv2d_i8_direct(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe);
     if (rc == 0) rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe, nullptr, &gs);
+    ctx->static_last_use = used_split ? 1 : 0;
     if (rc != 0) return rc < 0 ? rc : 0;
     // no fused kernel for this layout: the operator sequence, its int32 accumulator staged in the static array
     const size_t need = (size_t)numel(out) * 4;
@@ -559,6 +560,7 @@ int mlel_hip_conv2d_rescale_clamp_static(mlel_ctx *ctx, void *stream, const mlel
                  "mlel_hip_conv2d_rescale_clamp, which allocates",
                  need, kStaticScratchPartialBytes);
     mlel_tensor acc = packed_like(out, MLEL_I32, ctx->static_scratch);
+    ctx->static_last_use = 2;
     const GemmScratch no_split{nullptr, nullptr, 0, nullptr};  // the array is taken: the contraction must not split K
     rc = try_conv2d_i8_direct(ctx, (hipStream_t)stream, &acc, in, weights, bias, attr, nullptr);
     if (rc == 0) rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, &acc, in, weights, bias, attr, nullptr, nullptr, &no_split);
@@ -566,6 +568,11 @@ int mlel_hip_conv2d_rescale_clamp_static(mlel_ctx *ctx, void *stream, const mlel
     if (rc == 0) MLEL_TRY(conv2d_generic_launch((hipStream_t)stream, &acc, in, weights, bias, attr));
     MLEL_TRY(run_unfused_tail(ctx, (hipStream_t)stream, out, &acc, epi));
     return 0;
+}
+
+int mlel_hip_static_scratch_last_use(mlel_ctx *ctx) {
+    if (ctx == nullptr) return set_error(MLEL_ERR_INVALID, "static_scratch_last_use: null ctx");
+    return ctx->static_last_use;
 }
 
 int mlel_hip_conv2d_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
@@ -603,7 +610,8 @@ int mlel_hip_conv2d_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_
         MLEL_TRY(make_epilogue(scale_residual, residual->dtype, &acc_view, ch, &cr.f_res));
         MLEL_TRY(make_epilogue(scale_conv, conv_dt, &acc_view, ch, &cr.f_conv));
         MLEL_TRY(make_epilogue(scale_out, MLEL_I32, out, ch, &cr.f_out));
-        if (cr.f_res.in_dt == MLEL_I8 && cr.f_conv.in_dt == MLEL_I8) {
+        // the kernels requantise the sum as an accumulator, which assumes the output stage's input_zp is 0
+        if (cr.f_res.in_dt == MLEL_I8 && cr.f_conv.in_dt == MLEL_I8 && cr.f_out.p.in_zp == 0) {
             const int rc = try_conv2d_i8_mfma(ctx, (hipStream_t)stream, out, in, weights, bias, attr, &fe, &cr);
             if (rc != 0) return rc < 0 ? rc : 0;
         }

@@ -446,6 +446,7 @@ struct mlel_ctx {
     // the statically allocated scratch of the entry point that must not allocate: this device's address of the
     // array (hipGetSymbolAddress at context creation), nullptr if that failed
     char *static_scratch = nullptr;
+    int static_last_use = 0;  // what the last call of that entry point kept there: 0 nothing, 1 split-K tiles, 2 accumulator
 };
 
 namespace mlel {

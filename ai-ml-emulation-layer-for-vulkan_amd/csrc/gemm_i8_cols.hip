@@ -15,6 +15,26 @@ namespace {
 constexpr int kColsBlock = 256;
 constexpr int KR = 4;  // 32-byte K chunks per round
 
+// table[byte e of w]: the byte is scaled to a dword offset by one SDWA shift
+template <int E>
+__device__ __forceinline__ uint32_t byte_times_4(uint32_t w) {
+    uint32_t r;
+    const uint32_t two = 2;
+    if constexpr (E == 0)
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(r) : "v"(two), "v"(w));
+    else if constexpr (E == 1)
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(r) : "v"(two), "v"(w));
+    else if constexpr (E == 2)
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2" : "=v"(r) : "v"(two), "v"(w));
+    else
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3" : "=v"(r) : "v"(two), "v"(w));
+    return r;
+}
+__device__ __forceinline__ int32_t lds_entry(const int32_t *table, uint32_t w, int e) {
+    const uint32_t off = e == 0 ? byte_times_4<0>(w) : e == 1 ? byte_times_4<1>(w) : e == 2 ? byte_times_4<2>(w) : byte_times_4<3>(w);
+    return *reinterpret_cast<const int32_t *>(reinterpret_cast<const char *>(table) + off);
+}
+
 // KS == 1: a wavefront per tile.  KS == 4 (few tiles): the four wavefronts of a block share a tile, each takes a
 // quarter of the K chunks, the partial tiles are added through shared memory (int32 addition wraps: the order is
 // immaterial) and the first wavefront requantises.
@@ -27,7 +47,9 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
     const int chunk = (int)gridDim.x >> 3;  // the grid is a multiple of eight blocks
     const int bid = (int)(blockIdx.x % 8u) * chunk + (int)(blockIdx.x / 8u);
     const int wid = KS == 1 ? bid * (kColsBlock / 64) + wave : bid;
-    if (wid >= total_waves) return;  // whole wavefronts (KS == 1) or whole blocks (KS == 4) leave: no barrier is missed
+    // whole wavefronts (KS == 1) or whole blocks (KS == 4) have nothing to do; with the residual stage a wavefront
+    // stays for the block's table and its barrier and leaves behind it
+    if (!(RES && KS == 1) && wid >= total_waves) return;
     const int mg = wid / groups_n, ng = wid - mg * groups_n;
     const int cl = lane & 31, half = lane >> 5;
     const int m = mg * 32 + cl, n = ng * 32 + cl;
@@ -74,25 +96,20 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
     }
 
     // The residual stage rescales two 8-bit values per output with per-tensor constants: both are functions of a
-    // byte, so the wavefront tabulates them (256 dwords each, four entries per lane, in its own piece of shared
-    // memory: no block barrier) and an output costs two lookups instead of two requantisations.
+    // byte, so the block tabulates them once (256 dwords each, one entry of either table per thread, while the first
+    // operands travel) and an output costs two lookups instead of two requantisations.
     ChanScale q_out{};
-    __shared__ int32_t res_tab[RES ? kColsBlock / 64 : 1][2][256];
-    int32_t(*tab)[256] = res_tab[RES ? (KS == 1 ? wave : 0) : 0];
-    if (RES && (KS == 1 || wave == 0)) {  // while the first operands travel
+    __shared__ int32_t res_tab[RES ? 2 : 1][256];
+    if constexpr (RES) {
         const ChanScale q_res = make_chan_scale(load_mult(g.rs_res, 0), g.rs_res.shift[0], g.rs_res.p);
         const ChanScale q_conv = make_chan_scale(load_mult(g.rs_conv, 0), g.rs_conv.shift[0], g.rs_conv.p);
         q_out = make_chan_scale(load_mult(g.rs_out, 0), g.rs_out.shift[0], g.rs_out.p);
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const int b = t * 64 + lane;  // the byte as stored; its value is (int8_t)b
-            tab[0][b] = requant_chan((int32_t)(int8_t)b, q_res, g.rs_res.p);
-            tab[1][b] = requant_chan((int32_t)(int8_t)b, q_conv, g.rs_conv.p);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // entry `tid`: the byte as stored; its value is (int8_t)tid
+        res_tab[0][tid] = requant_chan((int32_t)(int8_t)tid, q_res, g.rs_res.p);
+        res_tab[1][tid] = requant_chan((int32_t)(int8_t)tid, q_conv, g.rs_conv.p);
+        __syncthreads();
     }
+    if (RES && KS == 1 && wid >= total_waves) return;
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0;
@@ -153,15 +170,17 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
         o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0x4e, 0xf, 0xf, true);
         p = __builtin_amdgcn_perm(o, p, sel_b);
         if constexpr (RES) {
+            // the sum is an int32 accumulator rescaled with input_zp 0 (checked by the host): requant_acc
             const uint32_t xw = d_res[q];
-            uint32_t summed = 0;
+            int32_t o4[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const int32_t r1 = tab[0][(xw >> (8 * e)) & 0xffu], r2 = tab[1][(p >> (8 * e)) & 0xffu];
-                const int32_t sum = (int32_t)((uint32_t)r1 + (uint32_t)r2);
-                summed |= ((uint32_t)requant_chan(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
+                const int32_t r1 = lds_entry(res_tab[0], xw, e), r2 = lds_entry(res_tab[1], p, e);
+                o4[e] = requant_acc((int32_t)((uint32_t)r1 + (uint32_t)r2), q_out, g.rs_out.p);
             }
-            p = summed;
+            const uint32_t l2 = __builtin_amdgcn_perm((uint32_t)o4[1], (uint32_t)o4[0], 0x0c0c0400u);
+            const uint32_t h2 = __builtin_amdgcn_perm((uint32_t)o4[3], (uint32_t)o4[2], 0x0c0c0400u);
+            p = __builtin_amdgcn_perm(h2, l2, 0x05040100u);
         }
         __builtin_amdgcn_raw_buffer_store_b32(p, ores, (int)d_off[q], 0, 0);
     }

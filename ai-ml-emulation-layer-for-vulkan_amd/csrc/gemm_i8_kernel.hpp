@@ -1003,7 +1003,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                                 const int32_t x = (int8_t)(xw >> (8 * e)), y = (int8_t)(p >> (8 * e));
                                 const int32_t r1 = requant_chan(x, q_res, g.rs_res.p), r2 = requant_chan(y, q_conv, g.rs_conv.p);
                                 const int32_t sum = (int32_t)((uint32_t)r1 + (uint32_t)r2);
-                                summed |= ((uint32_t)requant_chan(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
+                                summed |= ((uint32_t)requant_acc(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
                             }
                             p = summed;
                         }
@@ -1035,7 +1035,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                         const int32_t x = (int8_t)(xw >> (8 * e)), y = (int8_t)(w[k] >> (8 * e));
                         const int32_t r1 = requant_chan(x, q_res, g.rs_res.p), r2 = requant_chan(y, q_conv, g.rs_conv.p);
                         const int32_t sum = (int32_t)((uint32_t)r1 + (uint32_t)r2);
-                        summed |= ((uint32_t)requant_chan(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
+                        summed |= ((uint32_t)requant_acc(sum, q_out, g.rs_out.p) & 0xffu) << (8 * e);
                     }
                     w[k] = summed;
                 }

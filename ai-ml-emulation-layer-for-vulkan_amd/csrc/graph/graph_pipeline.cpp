@@ -1607,21 +1607,37 @@ void GraphSession::dispatchReplayed(void *stream) {
     if (pipeline.ctx == nullptr)
         fail("dispatch: this GraphPipeline was built without a device context; there is no CPU path");
     if (needsTransientMemory() && !transientMemoryBound) fail("dispatch: session transient memory is not bound");
+    if (eagerVersion == version && eagerStream == stream) {
+        // this session's dispatch could not be recorded with these bindings (below): it is issued launch by launch
+        apply();
+        pipeline.dispatch(stream, {}, 0, UINT32_MAX);
+        return;
+    }
     if (recording == nullptr || recordingVersion != version || recordingStream != stream) {
         // the recording holds the addresses of this session's tensors as they are bound now
         dropRecording();
         apply();
         check(mlel_hip_capture_begin(pipeline.ctx, stream), "recording a dispatch");
         void *exec = nullptr;
+        bool recorded = true;
         try {
             pipeline.dispatch(stream, {}, 0, UINT32_MAX);
         } catch (...) {
-            // the stream must leave capture mode whatever happened; what was recorded is thrown away
-            if (mlel_hip_capture_end(pipeline.ctx, stream, &exec) == 0 && exec != nullptr)
-                (void)mlel_hip_graph_destroy(pipeline.ctx, exec);
-            throw;
+            recorded = false;
         }
-        check(mlel_hip_capture_end(pipeline.ctx, stream, &exec), "recording a dispatch");
+        // the stream must leave capture mode whatever happened
+        const int endStatus = mlel_hip_capture_end(pipeline.ctx, stream, &exec);
+        if (!recorded) {
+            // An operator that needs a temporary (an operator-by-operator route of a fused call) refuses to run under
+            // capture.  What was recorded is thrown away and the dispatch is issued eagerly, now and until the
+            // bindings change; a failure that is not about the capture shows again there, with its own message.
+            if (endStatus == 0 && exec != nullptr) (void)mlel_hip_graph_destroy(pipeline.ctx, exec);
+            eagerVersion = version;
+            eagerStream = stream;
+            pipeline.dispatch(stream, {}, 0, UINT32_MAX);
+            return;
+        }
+        check(endStatus, "recording a dispatch");
         recording = exec;
         recordingVersion = version;
         recordingStream = stream;

@@ -422,6 +422,8 @@ class GraphSession {
     void *recording = nullptr;       // the instantiated HIP graph of this session's dispatch
     void *recordingStream = nullptr;
     uint64_t recordingVersion = 0;
+    uint64_t eagerVersion = UINT64_MAX;  // bindings under which recording failed: replayed dispatches run eagerly
+    void *eagerStream = nullptr;
     GraphPipeline &pipeline;
     void *base = nullptr;
     bool transientMemoryBound = false;

@@ -110,8 +110,10 @@ __device__ __forceinline__ uint32_t clamp_word(uint32_t x, int32_t lo, int32_t h
     }
 }
 
+// `out` may be `in` (CLAMP in place behind an unfused RESCALE): a thread reads its 16 bytes before it writes them, and
+// the pointers carry no no-alias promise.  The same holds for the int32 elementwise and the 8-bit TABLE kernels below.
 template <int SZ>
-__global__ void __launch_bounds__(kBlock) clamp_vec_kernel(char *__restrict__ out, const char *__restrict__ in, int32_t lo,
+__global__ void __launch_bounds__(kBlock) clamp_vec_kernel(char *out, const char *in, int32_t lo,
                                                            int32_t hi, int64_t n_vec, int64_t total) {
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (i < n_vec) {
@@ -151,8 +153,8 @@ __device__ __forceinline__ int32_t bin_i32(int32_t a, int32_t b) {
 }
 
 template <int OP>
-__global__ void __launch_bounds__(kBlock) binary_i32x4_kernel(int32_t *__restrict__ out, const int32_t *__restrict__ a,
-                                                              const int32_t *__restrict__ b, int64_t n_vec, int64_t total) {
+__global__ void __launch_bounds__(kBlock) binary_i32x4_kernel(int32_t *out, const int32_t *a, const int32_t *b, int64_t n_vec,
+                                                              int64_t total) {
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (i < n_vec) {
         const int4 x = reinterpret_cast<const int4 *>(a)[i], y = reinterpret_cast<const int4 *>(b)[i];
@@ -168,8 +170,8 @@ __global__ void __launch_bounds__(kBlock) binary_i32x4_kernel(int32_t *__restric
 // entries in shared memory, out = (table[i] << 7) + (table[i + 1] - table[i]) * (in & 127) with i = (in + 32768) >> 7,
 // 8 elements per thread (16 bytes in, 32 bytes out).
 // ---------------------------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(kBlock) table_i8x16_kernel(uint8_t *__restrict__ out, const uint8_t *__restrict__ in,
-                                                             const uint8_t *__restrict__ table, int64_t n_vec, int64_t total) {
+__global__ void __launch_bounds__(kBlock) table_i8x16_kernel(uint8_t *out, const uint8_t *in, const uint8_t *__restrict__ table,
+                                                             int64_t n_vec, int64_t total) {
     __shared__ uint8_t tab[256];
     tab[threadIdx.x] = table[threadIdx.x];  // kBlock == 256
     __syncthreads();
@@ -219,42 +221,106 @@ __global__ void __launch_bounds__(kBlock) table_i16x8_kernel(int32_t *__restrict
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// MAX_POOL2D, int8 NHWC.  Work item = 4 consecutive channels of one output position (lanes run over the channel
-// quads: a wavefront reads consecutive dwords of each input pixel); taps outside the image are skipped and the
-// accumulator starts from the lowest value of the type, as the shader does.
+// MAX_POOL2D, int8 NHWC (reference: maxpool2d.comp:23-72).  Work item = 4 * V consecutive channels of one output
+// position (lanes run over the channel groups: a wavefront reads consecutive pieces of each input pixel, V dwords per
+// lane and tap).  A block covers 256 items of one output row (n, oy), so the row is decoded on the scalar unit and a
+// thread needs one magic-number division; blocks are dealt to the XCDs in contiguous runs of rows, so the input rows
+// that vertically adjacent output rows share are fetched into one L2.  Taps outside the image are replaced by -128,
+// the value the shader's accumulator starts from.  The maximum runs on packed 16-bit halves: x ^ 0x80 turns the
+// signed order of a byte into the unsigned one, the even and the odd bytes of a dword are two v_pk_max_u16 operands
+// (the odd ones in place, as value << 8), and the result is flipped back.
 // ---------------------------------------------------------------------------------------------------------------
 struct MaxPoolArgs {
     const int8_t *x;
     int8_t *out;
     int32_t H, W, C, OH, OW;
-    int64_t x_sn, x_sy, x_sx;
+    uint32_t x_sn, x_sy, x_sx, x_bytes, o_bytes;
     int32_t kh, kw, sy, sx, pad_t, pad_l;
-    int64_t items;  // N * OH * OW * C / 4
+    int32_t groups;       // channel groups per pixel: C / (4 V)
+    int32_t row_items;    // OW * groups, below 2^16
+    int32_t row_blocks;   // ceil(row_items / 256)
+    uint32_t groups_magic;  // floor(2^32 / groups) + 1
+    int32_t blocks, chunk;  // launch geometry: `chunk` consecutive blocks per XCD
 };
 
-__global__ void __launch_bounds__(kBlock) maxpool_i8x4_kernel(const MaxPoolArgs a) {
-    const int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (item >= a.items) return;
-    const int c4n = a.C >> 2;
-    const int c = (int)(item % c4n) * 4;
-    int64_t rest = item / c4n;
-    const int ox = (int)(rest % a.OW);
-    rest /= a.OW;
-    const int oy = (int)(rest % a.OH);
-    const int n = (int)(rest / a.OH);
-    const int y0 = max(0, oy * a.sy - a.pad_t), y1 = min(a.H, oy * a.sy - a.pad_t + a.kh);
-    const int x0 = max(0, ox * a.sx - a.pad_l), x1 = min(a.W, ox * a.sx - a.pad_l + a.kw);
-    int32_t m[4] = {-128, -128, -128, -128};
-    const int8_t *xb = a.x + (int64_t)n * a.x_sn + c;
-    for (int y = y0; y < y1; y++)
-        for (int x = x0; x < x1; x++) {
-            const uint32_t v = *reinterpret_cast<const uint32_t *>(xb + (int64_t)y * a.x_sy + (int64_t)x * a.x_sx);
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_pk_max_u16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
+// K > 0: a K x K window, unrolled, so that all its loads are in flight together; K == 0: any window, tap by tap
+template <int V, int K>
+__global__ void __launch_bounds__(kBlock) maxpool_i8_kernel(const MaxPoolArgs a) {
+    const int bid = (int)(blockIdx.x % 8u) * a.chunk + (int)(blockIdx.x / 8u);
+    if (bid >= a.blocks) return;
+    const int row = bid / a.row_blocks, part = bid - row * a.row_blocks;  // uniform: scalar unit
+    const int n = row / a.OH, oy = row - n * a.OH;
+    const uint32_t item = (uint32_t)part * kBlock + threadIdx.x;
+    if (item >= (uint32_t)a.row_items) return;
+    const uint32_t ox = a.groups == 1 ? item : __umulhi(item, a.groups_magic);
+    const uint32_t cg = item - ox * (uint32_t)a.groups;
+    const int iy0 = oy * a.sy - a.pad_t, ix0 = (int)ox * a.sx - a.pad_l;
+    const __amdgpu_buffer_rsrc_t xres =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(a.x), 0, (int)a.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ores = __builtin_amdgcn_make_buffer_rsrc(a.out, 0, (int)a.o_bytes, 0x00020000);
+    const uint32_t base = (uint32_t)n * a.x_sn + (uint32_t)iy0 * a.x_sy + (uint32_t)ix0 * a.x_sx + cg * (4u * V);
+    uint32_t even[V], odd[V];  // running maxima in the flipped (unsigned) order: 0 is the lowest value, -128
 #pragma unroll
-            for (int e = 0; e < 4; e++) m[e] = max(m[e], (int32_t)(int8_t)(v >> (8 * e)));
+    for (int v = 0; v < V; v++) even[v] = odd[v] = 0u;
+    auto load = [&](uint32_t off, uint32_t (&w)[V]) {
+        if constexpr (V == 4) {
+            const auto q = __builtin_amdgcn_raw_buffer_load_b128(xres, (int)off, 0, 0);
+            w[0] = q[0], w[1] = q[1], w[2] = q[2], w[3] = q[3];
+        } else {
+            w[0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(xres, (int)off, 0, 0);
         }
-    const uint32_t lo = __builtin_amdgcn_perm((uint32_t)m[1], (uint32_t)m[0], 0x0c0c0400u);
-    const uint32_t hi = __builtin_amdgcn_perm((uint32_t)m[3], (uint32_t)m[2], 0x0c0c0400u);
-    reinterpret_cast<uint32_t *>(a.out)[item] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+    };
+    auto fold = [&](bool in, const uint32_t (&w)[V]) {
+#pragma unroll
+        for (int v = 0; v < V; v++) {
+            const uint32_t f = in ? (w[v] ^ 0x80808080u) : 0u;
+            even[v] = pk_max_u16(even[v], f & 0x00ff00ffu);
+            odd[v] = pk_max_u16(odd[v], f & 0xff00ff00u);
+        }
+    };
+    // The offset of a tap outside the image wraps to another pixel or beyond the extent (such a load returns 0);
+    // either way its value is replaced by the lowest one.
+    if constexpr (K > 0) {
+        uint32_t w[K][K][V];
+#pragma unroll
+        for (int ky = 0; ky < K; ky++)
+#pragma unroll
+            for (int kx = 0; kx < K; kx++) load(base + (uint32_t)ky * a.x_sy + (uint32_t)kx * a.x_sx, w[ky][kx]);
+#pragma unroll
+        for (int ky = 0; ky < K; ky++) {
+            const bool yin = (unsigned)(iy0 + ky) < (unsigned)a.H;
+#pragma unroll
+            for (int kx = 0; kx < K; kx++) fold(yin && (unsigned)(ix0 + kx) < (unsigned)a.W, w[ky][kx]);
+        }
+    } else {
+        for (int ky = 0; ky < a.kh; ky++) {
+            if ((unsigned)(iy0 + ky) >= (unsigned)a.H) continue;  // uniform
+            const uint32_t rowoff = base + (uint32_t)ky * a.x_sy;
+            for (int kx = 0; kx < a.kw; kx++) {
+                uint32_t w[V];
+                load(rowoff + (uint32_t)kx * a.x_sx, w);
+                fold((unsigned)(ix0 + kx) < (unsigned)a.W, w);
+            }
+        }
+    }
+    uint32_t r[V];
+#pragma unroll
+    for (int v = 0; v < V; v++) r[v] = (even[v] | odd[v]) ^ 0x80808080u;
+    const uint32_t ooff = (((uint32_t)row * (uint32_t)a.OW + ox) * (uint32_t)a.groups + cg) * (4u * V);
+    if constexpr (V == 4) {
+        typedef int v4i32 __attribute__((ext_vector_type(4)));
+        __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)r[0], (int)r[1], (int)r[2], (int)r[3]}, ores, (int)ooff, 0, 0);
+    } else {
+        __builtin_amdgcn_raw_buffer_store_b32(r[0], ores, (int)ooff, 0, 0);
+    }
 }
 
 }  // namespace
@@ -393,9 +459,15 @@ int try_maxpool_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const
     if (a->kernel[0] > (1 << 16) || a->kernel[1] > (1 << 16) || a->stride[0] > (1 << 16) || a->stride[1] > (1 << 16)) return 0;
     if (a->pad[0] < 0 || a->pad[2] < 0 || a->pad[0] > (1 << 16) || a->pad[2] > (1 << 16)) return 0;
     if (in->dims[1] >= (1 << 30) || in->dims[2] >= (1 << 30) || OH >= (1 << 14) || OW >= (1 << 14) || C >= (1 << 24)) return 0;
-    const int64_t items = N * OH * OW * (C / 4);
-    if (items == 0) return 1;
-    if (items >= (int64_t(1) << 40)) return 0;
+    if (N * OH * OW * C == 0) return 1;
+    // 32-bit buffer offsets on both sides; taps outside the image are sent to an offset beyond either extent
+    if (in->strides[0] < 0 || in->strides[1] < 0 || in->strides[2] < 0) return 0;
+    const int64_t x_extent = in->dims[0] * in->strides[0], o_extent = N * OH * OW * C;
+    if (x_extent <= 0 || x_extent >= (int64_t(1) << 31) || o_extent >= (int64_t(1) << 31)) return 0;
+    // 16 channels per thread when pixels and rows are 16-byte aligned on both sides, else 4
+    const bool wide = C % 16 == 0 && ((uintptr_t)in->ptr % 16) == 0 && ((uintptr_t)out->ptr % 16) == 0 &&
+                      in->strides[0] % 16 == 0 && in->strides[1] % 16 == 0 && in->strides[2] % 16 == 0;
+    const int v = wide ? 4 : 1;
     MaxPoolArgs g{};
     g.x = static_cast<const int8_t *>(in->ptr);
     g.out = static_cast<int8_t *>(out->ptr);
@@ -404,20 +476,43 @@ int try_maxpool_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const
     g.C = (int)C;
     g.OH = (int)OH;
     g.OW = (int)OW;
-    g.x_sn = in->strides[0];
-    g.x_sy = in->strides[1];
-    g.x_sx = in->strides[2];
+    g.x_sn = (uint32_t)in->strides[0];
+    g.x_sy = (uint32_t)in->strides[1];
+    g.x_sx = (uint32_t)in->strides[2];
+    g.x_bytes = (uint32_t)x_extent;
+    g.o_bytes = (uint32_t)o_extent;
     g.kh = a->kernel[0];
     g.kw = a->kernel[1];
     g.sy = a->stride[0];
     g.sx = a->stride[1];
     g.pad_t = a->pad[0];
     g.pad_l = a->pad[2];
-    g.items = items;
-    const int64_t blocks = (items + kBlock - 1) / kBlock;
-    if (blocks >= (int64_t(1) << 31)) return 0;
-    maxpool_i8x4_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(g);
-    MLEL_TRY(check_launch("max_pool2d (int8 quads)"));
+    g.groups = (int)(C / (4 * v));
+    const int64_t row_items = OW * g.groups;
+    if (row_items >= (1 << 16)) return 0;  // the magic-number division holds below 2^16
+    g.row_items = (int)row_items;
+    g.row_blocks = (int)((row_items + kBlock - 1) / kBlock);
+    g.groups_magic = (uint32_t)((uint64_t(1) << 32) / (uint64_t)g.groups + 1);
+    const int64_t blocks = N * OH * g.row_blocks;
+    if (blocks >= (int64_t(1) << 31) - 8) return 0;
+    g.blocks = (int)blocks;
+    g.chunk = (int)((blocks + 7) / 8);
+    const dim3 grid((unsigned)(g.chunk * 8));
+    const int k = (g.kh == g.kw && (g.kh == 2 || g.kh == 3)) ? g.kh : 0;
+#define MLEL_MAXPOOL(VV)                                                              \
+    if (k == 3)                                                                       \
+        maxpool_i8_kernel<VV, 3><<<grid, dim3(kBlock), 0, s>>>(g);                    \
+    else if (k == 2)                                                                  \
+        maxpool_i8_kernel<VV, 2><<<grid, dim3(kBlock), 0, s>>>(g);                    \
+    else                                                                              \
+        maxpool_i8_kernel<VV, 0><<<grid, dim3(kBlock), 0, s>>>(g);
+    if (wide) {
+        MLEL_MAXPOOL(4)
+    } else {
+        MLEL_MAXPOOL(1)
+    }
+#undef MLEL_MAXPOOL
+    MLEL_TRY(check_launch("max_pool2d (int8)"));
     return 1;
 }
 

@@ -330,19 +330,24 @@ def build(dev, spec, fuse=True):
     return g
 
 
-def _time_graph(dev, g, steps, warmup):
+def _time_graph(dev, g, steps, warmup, rounds=5):
+    """(wall seconds, event milliseconds) per graph: the median over `rounds` rounds of `steps` dispatches each, every
+    round between two events and two host time stamps."""
     for _ in range(warmup):
         g.dispatch()
     dev.sync()
     ev0, ev1 = dev.event(), dev.event()
-    t0 = time.perf_counter()
-    dev.record(ev0)
-    for _ in range(steps):
-        g.dispatch()
-    dev.record(ev1)
-    dev.sync()
-    wall = (time.perf_counter() - t0) / steps
-    return wall, dev.elapsed_ms(ev0, ev1) / steps
+    walls, gpus = [], []
+    for _ in range(rounds):
+        t0 = time.perf_counter()
+        dev.record(ev0)
+        for _ in range(steps):
+            g.dispatch()
+        dev.record(ev1)
+        dev.sync()
+        walls.append((time.perf_counter() - t0) / steps)
+        gpus.append(dev.elapsed_ms(ev0, ev1) / steps)
+    return float(np.median(walls)), float(np.median(gpus))
 
 
 _STREAMS = {}
@@ -452,7 +457,8 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True, in_flig
     g = build(dev, spec, fuse=True)
     rng = np.random.default_rng(1003)
     g.set_input("input", rng.integers(-128, 127, spec.inputs[0][2], endpoint=True).astype(np.int8))
-    wall, gpu_ms = _time_graph(dev, g, steps, warmup)
+    rounds = max(5, -(-50 // steps))
+    wall, gpu_ms = _time_graph(dev, g, steps, warmup, rounds)
     per_op = g.dispatch_profiled()
     dev.sync()
     by_kind = {}
@@ -460,7 +466,7 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True, in_flig
         by_kind[name] = by_kind.get(name, 0.0) + ms
     macs = spec.macs["dense"] + spec.macs["depthwise"]
     res = {"img_per_s": batch / wall, "ms_per_graph": wall * 1e3, "gpu_ms_per_graph": gpu_ms,
-           "graphs_timed": steps, "tops": 2.0 * macs / wall / 1e12, "gmac": macs / 1e9,
+           "graphs_timed": steps * rounds, "timing": f"median of {rounds} rounds of {steps} dispatches", "tops": 2.0 * macs / wall / 1e12, "gmac": macs / 1e9,
            "operators_executed": g.op_count(), "operators_in_graph": len(spec.ops),
            "session_memory_bytes": g.session_size,
            "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}
@@ -508,6 +514,35 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True, in_flig
     return {"mobilenetv2_b32": res}
 
 
+def bench_inverted_residual(dev, steps=20, warmup=3):
+    """BASELINE config 2 (one int8 inverted-residual block with its residual addition, 16 x 56 x 56 x 24) through the
+    GraphPipeline: microseconds per graph, TOP/s, every launch of the fused graph on its own, and the position of the
+    block against both rooflines (its launches are few and short: neither is close)."""
+    spec = inverted_residual_spec()
+    g = build(dev, spec, fuse=True)
+    rng = np.random.default_rng(1002)
+    g.set_input("input", rng.integers(-128, 127, spec.inputs[0][2], endpoint=True).astype(np.int8))
+    rounds = max(5, -(-50 // steps))
+    wall, gpu_ms = _time_graph(dev, g, steps, warmup, rounds)
+    macs = spec.macs["dense"] + spec.macs["depthwise"]
+    names = g.op_names()
+    alone = time_operators(dev, g)
+    launches = launch_layers(g, spec)
+    # algorithmic bytes of the fused block: the input twice (expansion and residual), weights and constants, the two
+    # intermediate activations written and read once each, the output once
+    nbytes = sum(l["bytes"] for l in launches) + int(np.prod(spec.inputs[0][2])) if launches else None
+    res = {"us_per_graph": wall * 1e6, "gpu_us_per_graph": gpu_ms * 1e3, "graphs_timed": steps * rounds,
+           "timing": f"median of {rounds} rounds of {steps} dispatches", "img_per_s": spec.inputs[0][2][0] / wall,
+           "tops": 2.0 * macs / wall / 1e12, "gmac": macs / 1e9, "operators_in_graph": len(spec.ops),
+           "operators_executed": g.op_count(),
+           "us_by_launch_alone": [{"index": i, "name": names[i], "us": round(ms * 1e3, 2)} for i, ms in alone.items()],
+           "roofline": {"mfma_frac": 2.0 * macs / (gpu_ms * 1e-3) / 1e12 / 5000.0, "mfma_peak_tops": 5000.0,
+                        "algorithmic_bytes": nbytes, "hbm_peak_gbs": 8000.0,
+                        "hbm_frac": None if nbytes is None else nbytes / (gpu_ms * 1e-3) / 1e9 / 8000.0}}
+    g.close()
+    return {"config2_inverted_residual_b16": res}
+
+
 def bench_transformer(dev, steps=20, warmup=3, in_flight=(2, 3, 4)):
     """Times whole-graph dispatches of BASELINE config 4 (fp16 encoder block, batch 8, seq 512, d_model 768) and every
     launch on its own; returns the extra fields bench.py adds to its JSON line, with the fp16 MFMA position of the
@@ -516,7 +551,8 @@ def bench_transformer(dev, steps=20, warmup=3, in_flight=(2, 3, 4)):
     g = build(dev, spec, fuse=True)
     rng = np.random.default_rng(1004)
     g.set_input("input", rng.standard_normal(spec.inputs[0][2]).astype(np.float16))
-    wall, gpu_ms = _time_graph(dev, g, steps, warmup)
+    rounds = max(5, -(-50 // steps))
+    wall, gpu_ms = _time_graph(dev, g, steps, warmup, rounds)
     per_op = g.dispatch_profiled()
     dev.sync()
     by_kind = {}
@@ -534,8 +570,8 @@ def bench_transformer(dev, steps=20, warmup=3, in_flight=(2, 3, 4)):
     gemm_ms = sum(ms for i, ms in alone.items() if "MATMUL" in names[i])
     other_ms = sum(ms for i, ms in alone.items() if "MATMUL" not in names[i])
     res = {"transformer_b8_s512_d768": {
-        "ms_per_graph": wall * 1e3, "gpu_ms_per_graph": gpu_ms, "graphs_timed": steps,
-        "tflops": spec.flops / wall / 1e12,
+        "ms_per_graph": wall * 1e3, "gpu_ms_per_graph": gpu_ms, "graphs_timed": steps * rounds,
+        "timing": f"median of {rounds} rounds of {steps} dispatches", "tflops": spec.flops / wall / 1e12,
         "gflop": spec.flops / 1e9, "operators_executed": g.op_count(), "operators_in_graph": len(spec.ops),
         "session_memory_bytes": g.session_size, "sessions_in_flight": in_flight,
         "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())},

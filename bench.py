@@ -7,12 +7,16 @@ multiplier 1518500250 / shift 39, double round), one launch of the MFMA contract
 also reports the MobileNetV2-shaped int8 graph at batch 32 (BASELINE config 3) executed through the host-side
 GraphPipeline, the roofline position of the dominant kernel and a CPU baseline (the oracle on the host cores).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only all|config1|mobilenetv2|encoder|layer|standalone] [--layer N]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only LEG] [--layer N]
 
-`--only` restricts the run to one leg (profiling runs: one kernel family per trace); `--only layer --layer N` launches
-the N-th operator of the fused MobileNetV2 graph 200 times back to back and nothing else, so that counters of a single
-layer can be collected; `--only standalone` times the bandwidth-bound operators of the unfused config 2 graph (RESCALE,
-CLAMP, ADD, TABLE, MAX_POOL2D) as stand-alone launches.  The whole-graph legs always time at least 20 graphs.
+`--only` restricts the run to one leg (profiling runs: one kernel family per trace): `config0` (fused CONV2D + RESCALE,
+1x56x56x64), `config1`, `config2` (the inverted-residual block), `mobilenetv2` (config 3), `encoder` (config 4),
+`gemm_large` (the config 1 operator at 4096^3 and 8192^3), `layer --layer N` (the N-th launch of the fused MobileNetV2
+graph 200 times back to back and nothing else, so that counters of a single layer can be collected), `standalone`
+(the bandwidth-bound operators as stand-alone launches on config 2's and on config 3's largest tensors), `copy` (the
+plain copy kernel over grid and size: the measured HBM ceiling), `extra` (data-movement operators outside the
+benchmark graphs).  `ms_per_step` is the median over at least 10 rounds of `--steps` launches; the whole-graph legs
+report the median over rounds that hold at least 50 graphs.
 """
 import re
 import argparse
@@ -32,6 +36,46 @@ PKG = "ai-ml-emulation-layer-for-vulkan_amd"
 
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X published dense int8 peak, TOP/s
 HBM_PEAK_GBS = 8000.0         # MI355X published HBM3E bandwidth, GB/s
+
+
+def device_peaks(info):
+    """The published peaks next to what the device's own properties give: matrix cores = compute units x 4 SIMDs x
+    1024 int8 multiply-adds per clock x 2 ops x the reported shader clock; HBM = reported memory clock x 4 transfers
+    per clock (HBM3E at 8 Gbit/s per pin reports 2000 MHz) x bus width.  The roofline fractions of this file use the
+    published figures."""
+    cus, clk = info["compute_units"], info["clock_khz"] * 1e3
+    return {"int8_mfma_published_tops": INT8_MFMA_PEAK_TOPS,
+            "int8_mfma_from_device_tops": cus * 4 * 1024 * 2 * clk / 1e12,
+            "fp16_mfma_from_device_tflops": cus * 4 * 512 * 2 * clk / 1e12,
+            "hbm_published_gbs": HBM_PEAK_GBS,
+            "hbm_from_device_properties_gbs": info["mem_clock_khz"] * 1e3 * 4 * info["bus_width_bits"] / 8 / 1e9,
+            "compute_units": cus, "clock_mhz": info["clock_khz"] / 1e3, "mem_clock_mhz": info["mem_clock_khz"] / 1e3,
+            "bus_width_bits": info["bus_width_bits"]}
+
+
+def reference_layer_probe():
+    """Looks for what a run of the reference layer itself would need on this host -- a Vulkan loader, the lavapipe
+    ICD manifest and the layer's manifest (VK_LAYER_ML_Graph_Emulation) -- without installing or loading anything.
+    With all three the CPU baseline could be the reference on lavapipe; without them it is the oracle (kind "port")."""
+    import ctypes.util
+    import glob
+    loader = ctypes.util.find_library("vulkan")
+    roots = ["/usr/share/vulkan", "/usr/local/share/vulkan", "/etc/vulkan", os.path.expanduser("~/.local/share/vulkan")]
+    layer_dirs = [os.path.join(r, d) for r in roots for d in ("explicit_layer.d", "implicit_layer.d")]
+    for var in ("VK_LAYER_PATH", "VK_ADD_LAYER_PATH"):
+        layer_dirs += [d for d in os.environ.get(var, "").split(os.pathsep) if d]
+    layer = None
+    for d in layer_dirs:
+        for f in sorted(glob.glob(os.path.join(d, "*.json"))):
+            try:
+                if "VK_LAYER_ML_Graph_Emulation" in open(f, errors="replace").read():
+                    layer = f
+            except OSError:
+                pass
+    icds = [f for r in roots for f in glob.glob(os.path.join(r, "icd.d", "lvp_icd*.json"))]
+    icds += [f for f in os.environ.get("VK_ICD_FILENAMES", "").split(os.pathsep) if "lvp" in f and os.path.exists(f)]
+    return {"vulkan_loader": loader, "lavapipe_icd": icds[0] if icds else None, "layer_manifest": layer,
+            "reference_layer_found": bool(loader and icds and layer)}
 
 CONFIG1_KERNEL = "gemm_i8_kernel<128,128,2,2,X_PLAIN_DL,W_KMAJOR_DL,SUMS,Q8>"
 CONFIG1_PROFILE = os.path.join(ROOT, "profiles", "gemm_i8_kernel_config1_matmul_rescale.md")
@@ -64,7 +108,7 @@ def config1_inputs():
     return a, b, np.array([1518500250], np.int32), np.array([39], np.int8)
 
 
-def bench_config1(dev, abi, steps, warmup, in_flight_counts=(2, 4)):
+def bench_config1(dev, abi, steps, warmup, in_flight_counts=(2, 4), rounds=10):
     a, b, mult, shift = config1_inputs()
     ta, tb, tm, ts = dev.from_numpy(a), dev.from_numpy(b), dev.from_numpy(mult), dev.from_numpy(shift)
     to = dev.tensor(abi.I8, (8, 512, 1024))
@@ -80,20 +124,25 @@ def bench_config1(dev, abi, steps, warmup, in_flight_counts=(2, 4)):
         step()
     dev.sync()
     ev0, ev1 = dev.event(), dev.event()
-    t0 = time.perf_counter()
-    dev.record(ev0)
-    for _ in range(steps):
-        step()
-    dev.record(ev1)
-    dev.sync()
-    wall = time.perf_counter() - t0
-    kernel_ms = dev.elapsed_ms(ev0, ev1) / steps  # back-to-back launches of the one kernel on its own stream
+    walls, kernels = [], []
+    for _ in range(rounds):  # every round: `steps` launches between two events and two host time stamps
+        t0 = time.perf_counter()
+        dev.record(ev0)
+        for _ in range(steps):
+            step()
+        dev.record(ev1)
+        dev.sync()
+        walls.append((time.perf_counter() - t0) / steps)
+        kernels.append(dev.elapsed_ms(ev0, ev1) / steps)  # back-to-back launches of the one kernel on its own stream
+    wall, kernel_ms = float(np.median(walls)), float(np.median(kernels))
     ops = 2.0 * 8 * 512 * 1024 * 1024
     res = {
-        "ms_per_step": wall * 1e3 / steps,
-        "tops": ops / (wall / steps) / 1e12,
+        "ms_per_step": wall * 1e3,
+        "tops": ops / wall / 1e12,
         "kernel_ms": kernel_ms,
         "kernel_tops": ops / (kernel_ms * 1e-3) / 1e12,
+        "rounds": rounds,
+        "ms_per_step_min_max": [min(walls) * 1e3, max(walls) * 1e3],
         "algorithmic_bytes": 8 * (512 * 1024 + 1024 * 1024 + 512 * 1024) + 5,
         "ops": ops,
     }
@@ -130,6 +179,120 @@ def bench_config1(dev, abi, steps, warmup, in_flight_counts=(2, 4)):
         to.download()
     res["host_buffers_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / 3
     return res, (a, b, mult, shift, out)
+
+
+def _median_us(dev, fn, reps, rounds=5, warm=3):
+    """Microseconds per call of `fn`: `reps` back-to-back calls between two events on the launch stream, the median of
+    `rounds` such measurements."""
+    for _ in range(warm):
+        fn()
+    ev0, ev1 = dev.event(), dev.event()
+    got = []
+    for _ in range(rounds):
+        dev.record(ev0)
+        for _ in range(reps):
+            fn()
+        dev.record(ev1)
+        dev.sync()
+        got.append(dev.elapsed_ms(ev0, ev1) / reps * 1e3)
+    return float(np.median(got))
+
+
+def bench_config0(dev, abi, steps, warmup, check=True):
+    """BASELINE config 0: CONV2D 3x3 (1x56x56x64 -> 64 channels, stride 1, pad 1, input_zp -5) + per-channel RESCALE
+    (double round, output_zp 3) to int8, one fused launch."""
+    rng = np.random.default_rng(1000)
+    x = rng.integers(-128, 127, (1, 56, 56, 64), endpoint=True).astype(np.int8)
+    w = rng.integers(-127, 127, (64, 3, 3, 64), endpoint=True).astype(np.int8)
+    b = rng.integers(-2 ** 15, 2 ** 15, (64,), endpoint=True).astype(np.int32)
+    mult = rng.integers(2 ** 30, 2 ** 31 - 1, (64,), endpoint=True).astype(np.int32)
+    shift = rng.integers(30, 38, (64,), endpoint=True).astype(np.int8)
+    attr = abi.conv2d_attr((1, 1, 1, 1), (1, 1), (1, 1), -5, 0)
+    rattr = abi.rescale_attr(0, 3, True, True, True)
+    tx, tw, tb, tm, ts = (dev.from_numpy(v) for v in (x, w, b, mult, shift))
+    to = dev.tensor(abi.I8, (1, 56, 56, 64))
+    epi = dev.epilogue(tm, ts, rattr)
+    fn = lambda: dev.op("conv2d_rescale_clamp", to.ref, tx.ref, tw.ref, tb.ref, C.byref(attr), C.byref(epi))
+    us = _median_us(dev, fn, max(steps, 20), rounds=10, warm=max(warmup, 3))
+    ops = 2.0 * 56 * 56 * 64 * 9 * 64
+    nbytes = x.size + w.size + 9 * 64 + x.size
+    res = {"us_per_launch": us, "launches_timed": 10 * max(steps, 20), "tops": ops / (us * 1e-6) / 1e12, "ops": ops,
+           "algorithmic_bytes": nbytes,
+           "roofline": {"mfma_frac": ops / (us * 1e-6) / 1e12 / INT8_MFMA_PEAK_TOPS,
+                        "hbm_frac": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                        "note": "0.23 GOP and 0.44 MB: a launch of this size is bound by its own latency"}}
+    if check:
+        oracle = importlib.import_module("oracle.mlel_oracle")
+        exp = oracle.rescale(oracle.conv2d(x, w, b, (1, 56, 56, 64), abi.I32, attr), mult, shift, abi.I8, rattr)
+        res["bit_exact_vs_oracle"] = bool(np.array_equal(to.download(), exp))
+    for t in (tx, tw, tb, tm, ts, to):
+        t.free()
+    return res
+
+
+def bench_gemm_large(dev, abi, sizes=(4096, 8192), check=True):
+    """The config 1 operator (int8 MATMUL, a_zp 2, b_zp -1, + per-tensor RESCALE to int8, one fused launch) on square
+    problems large enough to fill the machine for many tile rounds: what the contraction kernel reaches when launch
+    latency, prologue and epilogue are a small share."""
+    out = []
+    for n in sizes:
+        rng = np.random.default_rng(n)
+        a = rng.integers(-128, 127, (1, n, n), endpoint=True).astype(np.int8)
+        b = rng.integers(-128, 127, (1, n, n), endpoint=True).astype(np.int8)
+        ta, tb = dev.from_numpy(a), dev.from_numpy(b)
+        tm, ts = dev.from_numpy(np.array([1518500250], np.int32)), dev.from_numpy(np.array([39], np.int8))
+        to = dev.tensor(abi.I8, (1, n, n))
+        attr = abi.MatmulAttr(2, -1)
+        rattr = abi.rescale_attr(0, 0, True, True, False)
+        epi = dev.epilogue(tm, ts, rattr)
+        fn = lambda: dev.op("matmul_rescale", to.ref, ta.ref, tb.ref, C.byref(attr), C.byref(epi))
+        us = _median_us(dev, fn, 10, rounds=5, warm=2)
+        ops = 2.0 * n * n * n
+        rec = {"shape": [n, n, n], "us_per_launch": us, "launches_timed": 50, "tops": ops / (us * 1e-6) / 1e12,
+               "frac_of_int8_peak": ops / (us * 1e-6) / 1e12 / INT8_MFMA_PEAK_TOPS, "algorithmic_bytes": 3 * n * n + 5}
+        if check:  # a band of rows against the oracle
+            oracle = importlib.import_module("oracle.mlel_oracle")
+            rows = slice(n - 24, n - 8)
+            exp = oracle.rescale(oracle.matmul(a[:, rows], b, abi.I32, 2, -1), np.array([1518500250], np.int32),
+                                 np.array([39], np.int8), abi.I8, rattr)
+            rec["rows_checked_vs_oracle"] = 16
+            rec["bit_exact_vs_oracle"] = bool(np.array_equal(to.download()[:, rows], exp))
+        out.append(rec)
+        for t in (ta, tb, tm, ts, to):
+            t.free()
+    return out
+
+
+def bench_copy_sweep(dev, info):
+    """The plain copy kernel over grid size, 16-byte pieces in flight per thread and temporal / non-temporal accesses,
+    on 1 GiB (beyond the 256 MiB last-level cache) and on 64 MiB (inside it), plus a read-only and a write-only pass:
+    what the memory system of this part delivers to the simplest streaming kernel, i.e. the ceiling every
+    bandwidth-bound kernel here is to be read against."""
+    cus = info["compute_units"]
+    rows = []
+    for nbytes in (1 << 30, 64 << 20):
+        src, dst = dev.alloc(nbytes), dev.alloc(nbytes)
+        for mode, name, moved in ((0, "copy", 2.0), (1, "read", 1.0), (2, "write", 1.0)):
+            for nt in (0, 1):
+                for u in (1, 2, 4, 8):
+                    for blocks in (0, cus * 4, cus * 8, cus * 16, cus * 32):
+                        if mode != 0 and (blocks not in (0, cus * 8) or u not in (1, 4)):
+                            continue
+                        fn = lambda: dev._check(dev.lib.mlel_hip_copy_kernel_variant(
+                            dev.ctx, dev.stream, C.c_void_p(dst), C.c_void_p(src), nbytes, blocks, u, nt, mode))
+                        us = _median_us(dev, fn, 5, rounds=3, warm=1)
+                        rows.append({"bytes": nbytes, "mode": name, "non_temporal": nt, "pieces_in_flight": u,
+                                     "blocks": blocks, "us": round(us, 1),
+                                     "gbs": round(moved * nbytes / (us * 1e-6) / 1e9, 1)})
+        dev.free(src)
+        dev.free(dst)
+    best = {}
+    for r in rows:
+        key = f"{r['mode']}_{r['bytes'] >> 20}MiB"
+        if key not in best or r["gbs"] > best[key]["gbs"]:
+            best[key] = r
+    return {"rows": rows, "best": best,
+            "hbm_ceiling_gbs": best["copy_1024MiB"]["gbs"], "hbm_ceiling_frac_of_published": best["copy_1024MiB"]["gbs"] / HBM_PEAK_GBS}
 
 
 def measure_copy(dev, nbytes, reps=5):
@@ -212,28 +375,32 @@ def run_layer(dev, abi, index, reps=200):
     return res
 
 
-def bench_standalone(dev, abi, reps=100):
-    """The bandwidth-bound operators of the UNFUSED config 2 graph as stand-alone launches on its tensor sizes
-    (16 x 56 x 56 x 144 int32 accumulators / int8 activations): microseconds per launch and algorithmic GB/s (input +
+def bench_standalone(dev, abi, shape=(16, 56, 56, 144), reps=100):
+    """The bandwidth-bound operators of an UNFUSED int8 graph as stand-alone launches: on config 2's tensor sizes
+    (16 x 56 x 56 x 144 int32 accumulators / int8 activations, 7 - 36 MB per tensor, where the launch floor is a third
+    of the time) and on config 3's largest tensor (32 x 112 x 112 x 96: 38.5 MB as int8, 154 MB as int32, beyond what
+    the last-level cache holds for a three-tensor operator).  Microseconds per launch and algorithmic GB/s (input +
     output bytes once) of the packed 128-bit kernels, `reps` back-to-back launches each between two events."""
     rng = np.random.default_rng(1005)
-    shape = (16, 56, 56, 144)
     n = int(np.prod(shape))
+    ch = shape[3]
     acc = rng.integers(-2 ** 22, 2 ** 22, shape).astype(np.int32)
     acc2 = rng.integers(-2 ** 22, 2 ** 22, shape).astype(np.int32)
     x8 = rng.integers(-128, 127, shape, endpoint=True).astype(np.int8)
-    mult = rng.integers(2 ** 30, 2 ** 31 - 1, (144,), endpoint=True).astype(np.int32)
-    shift = rng.integers(30, 38, (144,), endpoint=True).astype(np.int8)
+    mult = rng.integers(2 ** 30, 2 ** 31 - 1, (ch,), endpoint=True).astype(np.int32)
+    shift = rng.integers(30, 38, (ch,), endpoint=True).astype(np.int8)
     tab = rng.integers(-128, 127, (256,), endpoint=True).astype(np.int8)
     t_acc, t_acc2, t_x8 = dev.from_numpy(acc), dev.from_numpy(acc2), dev.from_numpy(x8)
     t_m, t_s, t_tab = dev.from_numpy(mult), dev.from_numpy(shift), dev.from_numpy(tab)
     o8, o32 = dev.tensor(abi.I8, shape), dev.tensor(abi.I32, shape)
-    o_pool = dev.tensor(abi.I8, (16, 28, 28, 144))
+    o_pool = dev.tensor(abi.I8, (shape[0], shape[1] // 2, shape[2] // 2, ch))
+    held = [t_acc, t_acc2, t_x8, t_m, t_s, t_tab, o8, o32, o_pool]
     # reduced-precision storage: bf16 values as the upper halves of fp32 numbers, fp32 values inside e4m3's range
     f32 = (rng.standard_normal(shape) * 20).astype(np.float32)
     bf = (f32.view(np.uint32) >> 16).astype(np.uint16)
     t_bf1, t_bf2, t_f32 = dev.from_numpy(bf, abi.BF16), dev.from_numpy(bf[::-1].copy(), abi.BF16), dev.from_numpy(f32)
     o_bf, o_f8 = dev.tensor(abi.BF16, shape), dev.tensor(abi.F8E4M3, shape)
+    held += [t_bf1, t_bf2, t_f32, o_bf, o_f8]
     r_down = abi.rescale_attr(0, 3, True, True, True)
     r_up = abi.rescale_attr(-5, 0, True, True, True)
     clamp = abi.ClampAttr(0.0, 96.0, int(abi.NAN_PROPAGATE))
@@ -265,7 +432,15 @@ def bench_standalone(dev, abi, reps=100):
         us = dev.elapsed_ms(ev0, ev1) / reps * 1e3
         out.append({"operator": name, "shape": list(shape), "us": round(us, 2), "algorithmic_bytes": nbytes,
                     "gbs": round(nbytes / (us * 1e-6) / 1e9, 1), "hbm_frac": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+    for t in held:
+        t.free()
     return out
+
+
+def bench_extra(dev, abi):
+    """Data-movement operators outside the benchmark graphs (TILE, REVERSE, PAD, SLICE, CONCAT, GATHER) on dense int8
+    tensors of config 3's 56x56 stage: microseconds and algorithmic GB/s (input + output bytes once)."""
+    raise SystemExit("bench.py --only extra: not built yet")
 
 
 def main():
@@ -277,7 +452,8 @@ def main():
     ap.add_argument("--one-stream", action="store_true",
                     help="omit the legs with several launches / sessions in flight (profiling runs: one kernel at a time)")
     ap.add_argument("--skip-graph", action="store_true", help="omit the MobileNetV2 and encoder graph legs")
-    ap.add_argument("--only", choices=["all", "config1", "mobilenetv2", "encoder", "layer", "standalone"], default="all")
+    ap.add_argument("--only", choices=["all", "config0", "config1", "config2", "mobilenetv2", "encoder", "gemm_large",
+                                       "layer", "standalone", "copy", "extra"], default="all")
     ap.add_argument("--layer", type=int, default=3, help="with --only layer: position in the fused config 3 graph")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -295,7 +471,18 @@ def main():
         return
 
     if args.only == "standalone":
-        print(json.dumps({"only": "standalone", "operators": bench_standalone(dev, abi)}), flush=True)
+        print(json.dumps({"only": "standalone", "operators": bench_standalone(dev, abi) +
+                          bench_standalone(dev, abi, (32, 112, 112, 96), reps=30)}), flush=True)
+        dev.close()
+        return
+
+    if args.only == "copy":
+        print(json.dumps(dict({"only": "copy"}, **bench_copy_sweep(dev, info))), flush=True)
+        dev.close()
+        return
+
+    if args.only == "extra":
+        print(json.dumps({"only": "extra", "operators": bench_extra(dev, abi)}), flush=True)
         dev.close()
         return
 
@@ -314,6 +501,15 @@ def main():
 
     extra = {}
     graphs = importlib.import_module(PKG + ".graphs")
+    if want("config0"):
+        extra["config0_conv2d_rescale_1x56x56x64"] = bench_config0(dev, abi, args.steps, args.warmup, not args.skip_cpu)
+        log("config 0:", extra["config0_conv2d_rescale_1x56x56x64"])
+    if want("config2") and not args.skip_graph:
+        extra.update(graphs.bench_inverted_residual(dev, steps=graph_steps, warmup=max(3, args.warmup // 10)))
+        log("config 2:", extra["config2_inverted_residual_b16"])
+    if want("gemm_large"):
+        extra["gemm_large"] = bench_gemm_large(dev, abi, check=not args.skip_cpu)
+        log("large products:", extra["gemm_large"])
     if want("mobilenetv2") and not args.skip_graph:
         try:
             extra.update(graphs.bench_mobilenetv2(dev, steps=graph_steps, warmup=max(3, args.warmup // 10),
@@ -335,13 +531,15 @@ def main():
     parity_ok = None
     if not args.skip_cpu and c1 is not None:
         cpu, parity_ok = cpu_baseline_config1(abi, inputs, inputs[4])
+        cpu.update(reference_layer_probe())
         log("cpu baseline:", cpu, "gpu==oracle:", parity_ok)
     if not args.skip_cpu and "mobilenetv2_b32" in extra and "error" not in extra["mobilenetv2_b32"]:
         extra["mobilenetv2_b32"]["cpu_baseline"] = cpu_baseline_mobilenetv2(abi)
         log("cpu baseline (config 3):", extra["mobilenetv2_b32"]["cpu_baseline"])
 
     if c1 is None:  # a single graph leg: its own record, no config 1 fields to report
-        print(json.dumps(dict({"only": args.only, "copy_kernel_gbs": copy_gbs}, **extra)), flush=True)
+        print(json.dumps(dict({"only": args.only, "copy_kernel_gbs": copy_gbs, "peaks": device_peaks(info)}, **extra)),
+              flush=True)
         dev.close()
         return
 
@@ -363,12 +561,16 @@ def main():
                    "device": info["name"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "mfma", "achieved": c1["kernel_tops"], "peak": INT8_MFMA_PEAK_TOPS / 1.0,
                      "unit": "TFLOP/s", "ops_are": "int8 multiply and add counted as 2 ops", "frac": c1["kernel_tops"] / INT8_MFMA_PEAK_TOPS,
+                     "frac_of_peak_from_device_properties": c1["kernel_tops"] / device_peaks(info)["int8_mfma_from_device_tops"],
                      "traffic": config1_traffic_bytes(),
                      "kernel": CONFIG1_KERNEL, "kernel_ms": c1["kernel_ms"],
                      "algorithmic_bytes": c1["algorithmic_bytes"],
                      "hbm_frac_if_bandwidth_bound": c1["algorithmic_bytes"] / (c1["kernel_ms"] * 1e-3) / 1e9 /
                      HBM_PEAK_GBS},
         "cpu_baseline": cpu,
+        "peaks": device_peaks(info),
+        "timing": f"ms_per_step: median of {c1['rounds']} rounds of {args.steps} launches "
+                  f"(min {c1['ms_per_step_min_max'][0]:.5f}, max {c1['ms_per_step_min_max'][1]:.5f} ms)",
         "bit_exact_vs_oracle": parity_ok,
         "copy_kernel_gbs": copy_gbs,
         "host_buffers_ms_per_step": c1["host_buffers_ms_per_step"],

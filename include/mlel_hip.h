@@ -245,10 +245,15 @@ int mlel_hip_arena_release_import(mlel_ctx *ctx, void *handle);
 int mlel_hip_memcpy_h2d(mlel_ctx *ctx, void *dst, const void *src, size_t bytes, void *stream);
 int mlel_hip_memcpy_d2h(mlel_ctx *ctx, void *dst, const void *src, size_t bytes, void *stream);
 int mlel_hip_memcpy_d2d(mlel_ctx *ctx, void *dst, const void *src, size_t bytes, void *stream);
+/* Asynchronous byte fill on `stream`.  On a stream that is being captured into a graph the fill is recorded as a
+ * kernel, not as a memset node. */
 int mlel_hip_memset(mlel_ctx *ctx, void *dst, int value, size_t bytes, void *stream);
 
 int mlel_hip_stream_create(mlel_ctx *ctx, void **out_stream);
+/* Waits for the stream, frees the split-K workspace the context kept for it (if it ever split), destroys it. */
 int mlel_hip_stream_destroy(mlel_ctx *ctx, void *stream);
+/* Number of per-stream split-K workspaces (16 MiB + 16 KiB each, at most 16) the context holds right now. */
+int mlel_hip_split_workspaces(mlel_ctx *ctx);
 int mlel_hip_sync(mlel_ctx *ctx, void *stream); /* NULL = whole device */
 
 /* Per-operator timing.  Replaces the reference's timestamp queries around each dispatch
@@ -402,6 +407,11 @@ int mlel_hip_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor
 int mlel_hip_conv2d_rescale_clamp_static(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
                                          const mlel_tensor *weights, const mlel_tensor *bias,
                                          const mlel_conv2d_attr *attr, const mlel_epilogue *epi);
+/* What the last mlel_hip_conv2d_rescale_clamp_static call on this context kept in the static array: 0 nothing (a
+ * one-pass kernel without scratch), 1 the partial tiles and counters of a split-K contraction, 2 the int32
+ * accumulator of the operator sequence.  No counterpart in the reference; for tests and for callers that want to
+ * know which route a shape takes. */
+int mlel_hip_static_scratch_last_use(mlel_ctx *ctx);
 /* out = RESCALE_out( RESCALE_conv( CONV2D -> RESCALE -> [CLAMP] (epi) ) + RESCALE_residual(residual) ): the
  * residual connection behind a projecting convolution, bit for bit mlel_hip_conv2d_rescale_clamp into an 8-bit
  * temporary of `out`'s type followed by mlel_hip_rescale_add_rescale.  The integer addition wraps, so the operand order
@@ -539,6 +549,12 @@ int mlel_hip_conv2d_dwconv_in_kernel(const mlel_tensor *out, const mlel_tensor *
 /* Plain device-to-device copy kernel of `bytes` bytes with 128-bit accesses; the calibration kernel for
  * memory-traffic counters and the measured HBM ceiling. */
 int mlel_hip_copy_kernel(mlel_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes);
+/* The same kernel with its launch geometry as arguments, for measuring what this part's memory system delivers:
+ * `blocks` of 256 threads (<= 0: as many as give every thread one pass), 1 / 2 / 4 / 8 16-byte pieces in flight per
+ * thread, temporal or non-temporal accesses; mode 0 copies, 1 only reads `src`, 2 only writes `dst`.  `bytes` in whole
+ * 16-byte pieces.  No counterpart in the reference; a measurement aid. */
+int mlel_hip_copy_kernel_variant(mlel_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes, int blocks,
+                                 int pieces_in_flight, int non_temporal, int mode);
 
 #ifdef __cplusplus
 }

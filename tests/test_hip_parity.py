@@ -1076,6 +1076,14 @@ def test_packed_integer_operators_vs_oracle(run, oracle):
     np.testing.assert_array_equal(run.pool("max_pool2d", xp, (2, 10, 12, 36), ap), oracle.max_pool2d(xp, (2, 10, 12, 36), ap))
     ap2 = abi.pool2d_attr((2, 5), (1, 3), (0, 1, 2, 1))
     np.testing.assert_array_equal(run.pool("max_pool2d", xp, (2, 19, 8, 36), ap2), oracle.max_pool2d(xp, (2, 19, 8, 36), ap2))
+    # 16 channels per thread (pixels of whole 16-byte pieces): the same windows, the extreme values in every byte lane
+    xw = ri(rng, -128, 127, (3, 19, 23, 48), np.int8)
+    xw[0, :2, :, :16] = -128
+    xw[1, 5, 7] = np.tile(np.array([127, -128, -1, 0], np.int8), 12)
+    np.testing.assert_array_equal(run.pool("max_pool2d", xw, (3, 10, 12, 48), ap), oracle.max_pool2d(xw, (3, 10, 12, 48), ap))
+    np.testing.assert_array_equal(run.pool("max_pool2d", xw, (3, 19, 8, 48), ap2), oracle.max_pool2d(xw, (3, 19, 8, 48), ap2))
+    ap3 = abi.pool2d_attr((30, 30), (7, 9), (4, 4, 4, 4))  # the window holds the whole image
+    np.testing.assert_array_equal(run.pool("max_pool2d", xw, (3, 1, 1, 48), ap3), oracle.max_pool2d(xw, (3, 1, 1, 48), ap3))
 
 
 def test_pool_reduce_cast_negate_vs_oracle(run, oracle):
@@ -1336,6 +1344,69 @@ def test_matmul_i8_split_k_vs_oracle(run, oracle, case):
     for _ in range(2):
         np.testing.assert_array_equal(run.matmul(a, b, abi.I32, za, zb), exp)
         np.testing.assert_array_equal(run.matmul(a, b, abi.I8, za, zb, epilogue=(mult, shift, rattr, None)), exp8)
+
+
+def test_copy_kernels_move_exactly_the_requested_bytes(run):
+    """mlel_hip_copy_kernel (ragged length: whole pieces by the one-pass kernel, the tail bytewise) and every mode of
+    mlel_hip_copy_kernel_variant leave the destination equal to the source over the requested bytes and untouched
+    behind them; the read-only mode writes nothing."""
+    import ctypes as C
+    dev, lib = run.dev, run.dev.lib
+    rng = np.random.default_rng(8)
+    n = 3 * 4096 * 16 + 7
+    src = ri(rng, 0, 255, (n + 64,), np.uint8)
+    ts = run.put(src)
+    td = run.put(np.full(n + 64, 0xEE, np.uint8))
+    dev._check(lib.mlel_hip_copy_kernel(dev.ctx, dev.stream, C.c_void_p(td.ptr), C.c_void_p(ts.ptr), n))
+    got = td.download()
+    np.testing.assert_array_equal(got[:n], src[:n])
+    assert (got[n:] == 0xEE).all()
+    whole = (n // 16) * 16
+    for blocks in (0, 7, 64):
+        for pieces in (1, 2, 4, 8):
+            for nt in (0, 1):
+                td.upload(np.full(n + 64, 0xEE, np.uint8))
+                dev._check(lib.mlel_hip_copy_kernel_variant(dev.ctx, dev.stream, C.c_void_p(td.ptr), C.c_void_p(ts.ptr),
+                                                            whole, blocks, pieces, nt, 0))
+                got = td.download()
+                np.testing.assert_array_equal(got[:whole], src[:whole], err_msg=str((blocks, pieces, nt)))
+                assert (got[whole:] == 0xEE).all()
+    td.upload(np.full(n + 64, 0xEE, np.uint8))
+    dev._check(lib.mlel_hip_copy_kernel_variant(dev.ctx, dev.stream, C.c_void_p(td.ptr), C.c_void_p(ts.ptr), whole, 0, 4, 1, 1))
+    assert (td.download() == 0xEE).all()
+    dev._check(lib.mlel_hip_copy_kernel_variant(dev.ctx, dev.stream, C.c_void_p(td.ptr), C.c_void_p(ts.ptr), whole, 0, 4, 0, 2))
+    got = td.download()
+    assert (got[:whole].view(np.uint32).reshape(-1, 4) == np.array([1, 2, 3, 4], np.uint32)).all() and (got[whole:] == 0xEE).all()
+    run.done()
+    with pytest.raises(hb.MlelError):
+        dev._check(lib.mlel_hip_copy_kernel_variant(dev.ctx, dev.stream, C.c_void_p(ts.ptr), C.c_void_p(ts.ptr), 24, 0, 1, 0, 0))
+
+
+def test_split_k_workspaces_are_released_with_their_streams(run, oracle):
+    """More streams than the context has workspace slots, one after the other: each splits K (its workspace appears),
+    matches the oracle, and gives the workspace back when it is destroyed -- the twentieth stream still splits."""
+    dev, lib = run.dev, run.dev.lib
+    name, xs, oc, k, pad, stride, zi, zw = SPLIT_CONV_CASES[3]
+    rng = np.random.default_rng(5)
+    x = ri(rng, -128, 127, xs, np.int8)
+    w = ri(rng, -128, 127, (oc,) + k + (xs[3],), np.int8)
+    b = ri(rng, -2 ** 15, 2 ** 15, (oc,), np.int32)
+    attr = abi.conv2d_attr(pad, stride, (1, 1), zi, zw)
+    shape = (xs[0], xs[1], xs[2], oc)
+    exp = oracle.conv2d(x, w, b, shape, abi.I32, attr)
+    base = lib.mlel_hip_split_workspaces(dev.ctx)
+    keep = dev.stream
+    try:
+        for i in range(20):
+            dev.stream = dev.new_stream()
+            got = run.conv2d(x, w, b, shape, abi.I32, attr)
+            assert lib.mlel_hip_split_workspaces(dev.ctx) == base + 1, i
+            stream, dev.stream = dev.stream, keep
+            dev.free_stream(stream)
+            assert lib.mlel_hip_split_workspaces(dev.ctx) == base, i
+            np.testing.assert_array_equal(got, exp, err_msg=f"stream {i}")
+    finally:
+        dev.stream = keep
 
 
 # ------------------------------------------------------------------------------------------------ error paths
