@@ -288,6 +288,7 @@ RUNTIME_SIGNATURES = {
     "mlel_hip_event_create": (C.c_int, [_V, C.POINTER(_V)]),
     "mlel_hip_event_destroy": (C.c_int, [_V, _V]),
     "mlel_hip_event_record": (C.c_int, [_V, _V, _V]),
+    "mlel_hip_stream_wait_event": (C.c_int, [_V, _V, _V]),
     "mlel_hip_event_elapsed_ms": (C.c_int, [_V, _V, _V, C.POINTER(C.c_float)]),
     "mlel_hip_capture_begin": (C.c_int, [_V, _V]),
     "mlel_hip_capture_end": (C.c_int, [_V, _V, C.POINTER(_V)]),

@@ -489,6 +489,20 @@ int mlel_graph_get_memory_planner(mlel_graph *g) {
     return guarded([&] { return static_cast<int>(g->pipeline.memoryPlanner()); });
 }
 
+int mlel_graph_set_batch_split(mlel_graph *g, int enabled) {
+    return guarded([&] {
+        g->pipeline.setBatchSplit(enabled != 0);
+        return 0;
+    });
+}
+
+int mlel_graph_get_batch_split(mlel_graph *g) {
+    return guarded([&] {
+        return g->pipeline.isFinalized() ? static_cast<int>(g->pipeline.batchSplitLaunches())
+                                         : (g->pipeline.batchSplitRequested() ? 1 : 0);
+    });
+}
+
 int mlel_graph_finalize(mlel_graph *g, int enable_fusion) {
     return guarded([&] {
         g->pipeline.finalize(enable_fusion != 0);

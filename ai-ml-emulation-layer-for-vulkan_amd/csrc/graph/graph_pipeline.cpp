@@ -1332,6 +1332,38 @@ void GraphPipeline::plan() {
         else if (eliminated.find(t) == eliminated.end() || t->isGraphOutput)
             unseen.push_back({i, aligned(t->getSize())});
     }
+    // Batch split: session tensors that only the split run touches are stored as two halves, each planned at half
+    // its size in a region of its own (see setBatchSplit); a tensor with a view (an elided RESHAPE) stays whole.
+    splitInterior.clear();
+    std::vector<details::LiveInterval> halfIntervals;
+    if (splitPrefix > 0 && planner == MemoryPlanner::Interval) {
+        std::set<const TensorDescriptor *> viewed;
+        for (const auto &[view, target] : aliasOf) {
+            viewed.insert(view);
+            viewed.insert(target);
+        }
+        std::vector<details::LiveInterval> whole;
+        for (const auto &iv : intervals) {
+            const auto *t = tensors[iv.id].get();
+            const bool interior = iv.first >= splitFirst + 1 && iv.last <= splitPrefix && !t->isGraphInput && !t->isGraphOutput &&
+                                  viewed.find(t) == viewed.end() && t->getRank() == 4 &&
+                                  t->getDimensions()[0] == splitBatch && t->isPacked();
+            if (interior) {
+                splitInterior.insert(t);
+                halfIntervals.push_back({iv.id, iv.first, iv.last, aligned(t->getSize() / 2), iv.order});
+            } else {
+                // a whole tensor the split run touches is written or read by two chains that are out of step: it
+                // shares no byte with any other such tensor, which the planner sees as a range over the whole run
+                auto w = iv;
+                if (w.first <= splitPrefix && w.last >= splitFirst + 1) {
+                    w.first = std::min<uint32_t>(w.first, splitFirst + 1);
+                    w.last = std::max<uint32_t>(w.last, splitPrefix);
+                }
+                whole.push_back(w);
+            }
+        }
+        intervals = std::move(whole);
+    }
     details::AllocationPlan planResult;
     // the reference reports its choice at this severity when a session is created (graph_layer.cpp:286-295)
     MLEL_GRAPH_LOG(Info, (planner == MemoryPlanner::Interval ? "Using interval memory planner"
@@ -1352,12 +1384,21 @@ void GraphPipeline::plan() {
     }
     offsets.clear();
     for (const auto &[id, off] : planResult.offsets) offsets[tensors[id].get()] = static_cast<size_t>(off);
+    splitFullRegion = static_cast<size_t>(planResult.memorySize);
+    splitHalfRegion = 0;
+    if (!halfIntervals.empty()) {
+        const auto halfPlan = details::allocateIntervals(std::move(halfIntervals), {}, kSessionAlignment);
+        splitHalfRegion = aligned(static_cast<size_t>(halfPlan.memorySize));
+        splitFullRegion = aligned(splitFullRegion);
+        for (const auto &[id, off] : halfPlan.offsets)
+            offsets[tensors[id].get()] = splitFullRegion + static_cast<size_t>(off);  // the first half's place
+    }
     for (const auto &[view, target] : aliasOf) {  // views share the storage of the tensor they alias
         (void)target;
         const auto it = offsets.find(root(view));
         if (it != offsets.end()) offsets[view] = it->second;
     }
-    sessionSize = static_cast<size_t>(planResult.memorySize);
+    sessionSize = splitHalfRegion != 0 ? splitFullRegion + 2 * splitHalfRegion : static_cast<size_t>(planResult.memorySize);
 }
 
 // Safe-to-reuse sets of the best-fit planner (reference: BestFitMemoryPlanner::liveTensorAnalysis,
@@ -1525,12 +1566,141 @@ void GraphPipeline::finalize(const bool enableFusion) {
     const size_t recorded = ops.size();
     if (enableFusion) fuse();
     if (enableFusion) prepackConstants();
+    if (splitRequested) analyzeBatchSplit();
     plan();
+    if (splitPrefix > 0) validateSplitPlan();
     finalized = true;
     size_t launches = 0;
     for (const auto &op : ops) launches += op->fusedAway ? 0 : 1;
     MLEL_GRAPH_LOG(Info, "Graph pipeline created: " << recorded << " operators recorded, " << launches
                                                     << " launches per dispatch, session memory " << sessionSize << " bytes");
+    if (splitRequested)
+        MLEL_GRAPH_LOG(Info, "Batch split: launches " << splitFirst << " to " << splitPrefix
+                                                      << " (exclusive) issued per half batch of " << splitBatch / 2
+                                                      << " on two streams");
+}
+
+void GraphPipeline::setBatchSplit(const bool enabled) {
+    if (finalized) fail("setBatchSplit: the pipeline is already finalized");
+    splitRequested = enabled;
+}
+
+namespace {
+
+// The operands of `op` that carry the batch in their outermost extent (positions in op.inputs), for the operator kinds
+// that treat the images of a batch independently; false for every other kind.
+bool batchOperands(const OpNode &op, std::vector<size_t> &ins) {
+    ins.clear();
+    switch (op.kind) {
+    case OpKind::Conv2D:
+    case OpKind::DepthwiseConv2D:
+    case OpKind::FusedConv2D:
+    case OpKind::FusedDepthwiseConv2D:
+    case OpKind::FusedConv2DDepthwise:
+    case OpKind::AvgPool2D:
+    case OpKind::MaxPool2D:
+    case OpKind::Rescale:
+    case OpKind::Clamp:
+    case OpKind::Table:
+        ins = {0};
+        return true;
+    case OpKind::FusedConv2DResidual:
+        ins = {0, 3};
+        return true;
+    case OpKind::FusedRescaleAddRescale:
+        ins = {0, 1};
+        return true;
+    default:
+        return false;
+    }
+}
+
+}  // namespace
+
+void GraphPipeline::analyzeBatchSplit() {
+    splitFirst = 0;
+    splitPrefix = 0;
+    splitBatch = 0;
+    if (planner == MemoryPlanner::BestFit || inputs.empty()) return;
+    const auto &first = inputs.front();
+    if (first->getRank() != 4) return;
+    const int64_t n = first->getDimensions()[0];
+    if (n < 2 || n % 2 != 0) return;
+    const auto carriesBatch = [&](const TensorPtr &t) {
+        return t && t->getKind() != TensorKind::Constant && t->getRank() == 4 && t->getDimensions()[0] == n &&
+               t->isPacked();
+    };
+    uint32_t count = 0;
+    std::vector<size_t> act;
+    for (const auto &op : ops) {
+        if (op->fusedAway) continue;
+        if (!batchOperands(*op, act) || op->outputs.size() != 1 || !carriesBatch(op->outputs[0])) break;
+        bool ok = true;
+        for (size_t i = 0; i < op->inputs.size() && ok; i++) {
+            const bool isAct = std::find(act.begin(), act.end(), i) != act.end();
+            // everything but the activations is a constant of the pipeline (weights, bias, scales, tables)
+            ok = isAct ? carriesBatch(op->inputs[i]) : (op->inputs[i] && op->inputs[i]->getKind() == TensorKind::Constant);
+        }
+        for (const auto *spec : {&op->epilogue, &op->scaleA, &op->scaleB, &op->scaleOut})
+            for (const auto &t : {spec->multiplier, spec->shift}) ok = ok && (!t || t->getKind() == TensorKind::Constant);
+        if (!ok) break;
+        count++;
+    }
+    if (count < 2) return;
+    // Where the two chains start: at the first launch.  Measured on the MobileNetV2-shaped graph at batch 32 (replayed
+    // dispatch, 0.340 ms unsplit): 0.319 ms from launch 0, 0.314 from 4, 0.324 from 8, 0.329 from 12, 0.337 from 16,
+    // 0.351 from 26 -- the large early launches lose nothing beside their other half and the short late ones gain
+    // little, so the whole run is split.  MLEL_GRAPH_SPLIT_FROM in the environment names another position.
+    uint32_t from = 0;
+    if (const char *env = std::getenv("MLEL_GRAPH_SPLIT_FROM")) from = static_cast<uint32_t>(std::max(0, std::atoi(env)));
+    if (from + 2 > count) return;
+    splitFirst = from;
+    splitPrefix = count;
+    splitBatch = n;
+}
+
+// What the split dispatch relies on, checked on the host when the pipeline is finalized: inside either region no
+// two tensors whose live ranges overlap share a byte (a region is used by one chain of launches), the half regions
+// hold the halves they were planned for, and the three regions do not overlap.
+void GraphPipeline::validateSplitPlan() const {
+    struct Slot {
+        const TensorDescriptor *t;
+        size_t off, size;
+        std::array<uint32_t, 2> range;
+    };
+    std::vector<Slot> whole, halves;
+    for (const auto &[t, off] : offsets) {
+        if (aliasOf.find(t) != aliasOf.end()) continue;  // a view of another tensor's storage
+        const auto r = ranges.find(t);
+        if (r == ranges.end()) continue;
+        if (splitInterior.count(t))
+            halves.push_back({t, off - splitFullRegion, t->getSize() / 2, r->second});
+        else
+            whole.push_back({t, off, t->getSize(), r->second});
+    }
+    const auto disjoint = [&](const std::vector<Slot> &v, size_t region, const char *what, bool wholeRegion) {
+        for (size_t i = 0; i < v.size(); i++) {
+            if (v[i].off + v[i].size > region) fail(std::string("batch split: a tensor leaves the ") + what + " region");
+            for (size_t j = i + 1; j < v.size(); j++) {
+                const bool bytes = v[i].off < v[j].off + v[j].size && v[j].off < v[i].off + v[i].size;
+                // inside the split run two chains are out of step: every tensor it touches counts as live throughout
+                const auto inRun = [&](const Slot &x) { return x.range[0] <= splitPrefix && x.range[1] >= splitFirst + 1; };
+                const bool bothInRun = wholeRegion && inRun(v[i]) && inRun(v[j]);
+                const bool time = bothInRun || (v[i].range[0] <= v[j].range[1] && v[j].range[0] <= v[i].range[1]);
+                if (bytes && time) fail(std::string("batch split: two live tensors share bytes in the ") + what + " region");
+            }
+        }
+    };
+    disjoint(whole, splitHalfRegion != 0 ? splitFullRegion : sessionSize, "whole-tensor", true);
+    disjoint(halves, splitHalfRegion, "half-batch", false);
+    for (const auto &s : halves) {
+        if (s.range[0] < splitFirst + 1 || s.range[1] > splitPrefix)
+            fail("batch split: a half-stored tensor is used outside the split run");
+        if (s.t->getDimensions().empty() || s.t->getDimensions()[0] != splitBatch || !s.t->isPacked())
+            fail("batch split: a half-stored tensor does not carry the batch");
+    }
+    if (splitHalfRegion != 0 && sessionSize != splitFullRegion + 2 * splitHalfRegion)
+        fail("batch split: session memory size does not match its regions");
 }
 
 void GraphPipeline::bindSessionMemory(void *deviceBase) {
@@ -1557,7 +1727,25 @@ GraphSession::GraphSession(GraphPipeline &p) : pipeline(p) {
 
 GraphSession::~GraphSession() {
     dropRecording();
+    if (pipeline.ctx != nullptr) {
+        if (splitLane.stream) {
+            (void)mlel_hip_sync(pipeline.ctx, splitLane.stream);
+            (void)mlel_hip_stream_destroy(pipeline.ctx, splitLane.stream);
+        }
+        if (splitLane.fork) (void)mlel_hip_event_destroy(pipeline.ctx, splitLane.fork);
+        if (splitLane.join) (void)mlel_hip_event_destroy(pipeline.ctx, splitLane.join);
+    }
     if (pipeline.appliedSession == this) pipeline.appliedSession = nullptr;
+}
+
+const GraphPipeline::SplitLane *GraphSession::lane() {
+    if (pipeline.batchSplitLaunches() == 0) return nullptr;
+    if (splitLane.stream == nullptr) {
+        check(mlel_hip_stream_create(pipeline.ctx, &splitLane.stream), "creating the second stream of a split dispatch");
+        check(mlel_hip_event_create(pipeline.ctx, &splitLane.fork), "creating the fork event");
+        check(mlel_hip_event_create(pipeline.ctx, &splitLane.join), "creating the join event");
+    }
+    return &splitLane;
 }
 
 void GraphSession::dropRecording() {
@@ -1600,7 +1788,7 @@ void GraphSession::dispatch(void *stream, const GraphPipeline::DispatchDecorator
     // reference: "session transient memory is not bound" (graph_layer.cpp:1944-1947)
     if (needsTransientMemory() && !transientMemoryBound) fail("dispatch: session transient memory is not bound");
     apply();
-    pipeline.dispatch(stream, decorator, first, count);
+    pipeline.dispatch(stream, decorator, first, count, lane());
 }
 
 void GraphSession::dispatchReplayed(void *stream) {
@@ -1610,7 +1798,7 @@ void GraphSession::dispatchReplayed(void *stream) {
     if (eagerVersion == version && eagerStream == stream) {
         // this session's dispatch could not be recorded with these bindings (below): it is issued launch by launch
         apply();
-        pipeline.dispatch(stream, {}, 0, UINT32_MAX);
+        pipeline.dispatch(stream, {}, 0, UINT32_MAX, lane());
         return;
     }
     if (recording == nullptr || recordingVersion != version || recordingStream != stream) {
@@ -1621,7 +1809,7 @@ void GraphSession::dispatchReplayed(void *stream) {
         void *exec = nullptr;
         bool recorded = true;
         try {
-            pipeline.dispatch(stream, {}, 0, UINT32_MAX);
+            pipeline.dispatch(stream, {}, 0, UINT32_MAX, lane());
         } catch (...) {
             recorded = false;
         }
@@ -1634,7 +1822,7 @@ void GraphSession::dispatchReplayed(void *stream) {
             if (endStatus == 0 && exec != nullptr) (void)mlel_hip_graph_destroy(pipeline.ctx, exec);
             eagerVersion = version;
             eagerStream = stream;
-            pipeline.dispatch(stream, {}, 0, UINT32_MAX);
+            pipeline.dispatch(stream, {}, 0, UINT32_MAX, lane());
             return;
         }
         check(endStatus, "recording a dispatch");
@@ -1660,7 +1848,7 @@ mlel_epilogue makeEpilogue(const RescaleSpec &spec, const mlel_tensor *mult, con
 
 }  // namespace
 
-void GraphPipeline::run(const OpNode &op, void *stream) {
+void GraphPipeline::run(const OpNode &op, void *stream, const int half) {
     std::array<mlel_tensor, 8> in{};
     // FusedElementwise describes its inputs itself (up to MLEL_CHAIN_MAX_INPUTS); every other kind reads `in`
     if (op.inputs.size() > in.size() && op.kind != OpKind::FusedElementwise)
@@ -1674,6 +1862,19 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
     mlel_tensor out = op.outputs[0]->view();
     if (out.ptr == nullptr && op.outputs[0]->getShapeSize() != 0)
         fail(op.tosaName + " (" + op.debugName + "): output tensor has no memory bound");
+    if (half >= 0) {
+        // one half of the batch: half the outermost extent; the second half of a tensor stored as two halves lies one
+        // region further, that of a whole tensor half its size further
+        const auto halved = [&](mlel_tensor &v, const TensorDescriptor *t) {
+            v.dims[0] = splitBatch / 2;
+            const size_t step = splitInterior.count(t) ? splitHalfRegion : static_cast<size_t>(v.dims[0] * v.strides[0]);
+            v.ptr = static_cast<char *>(v.ptr) + static_cast<size_t>(half) * step;
+        };
+        std::vector<size_t> act;
+        if (!batchOperands(op, act)) fail(op.tosaName + " (" + op.debugName + "): not an operator of the split run");
+        for (const size_t i : act) halved(in[i], op.inputs[i].get());
+        halved(out, op.outputs[0].get());
+    }
     int rc = 0;
     switch (op.kind) {
     case OpKind::Conv2D: rc = mlel_hip_conv2d(ctx, stream, &out, &in[0], &in[1], &in[2], &op.conv); break;
@@ -1870,19 +2071,56 @@ void GraphPipeline::run(const OpNode &op, void *stream) {
 }
 
 void GraphPipeline::dispatch(void *stream, const DispatchDecorator &decorator, const uint32_t first,
-                             const uint32_t count) {
+                             const uint32_t count, const SplitLane *lane) {
     if (!finalized) fail("dispatch: finalize() has not run");
     if (ctx == nullptr) fail("dispatch: this GraphPipeline was built without a device context; there is no CPU path");
+    // two streams only for a whole, undecorated dispatch; otherwise the two halves of a split launch follow each
+    // other on `stream`
+    const bool fork = splitPrefix > 0 && lane != nullptr && lane->stream != nullptr && !decorator && first == 0 &&
+                      count == UINT32_MAX;
+    const auto check = [&](int rc, const char *what) {
+        if (rc != 0) fail(std::string("dispatch: ") + what + ": " + mlel_hip_last_error());
+    };
+    bool forked = false, joined = !fork;
+    const auto forkNow = [&] {
+        if (!fork || forked) return;
+        check(mlel_hip_event_record(ctx, lane->fork, stream), "recording the fork");
+        check(mlel_hip_stream_wait_event(ctx, lane->stream, lane->fork), "starting the second half");
+        forked = true;
+    };
+    const auto join = [&] {
+        if (joined || !forked) return;
+        check(mlel_hip_event_record(ctx, lane->join, lane->stream), "recording the join");
+        check(mlel_hip_stream_wait_event(ctx, stream, lane->join), "waiting for the second half");
+        joined = true;
+    };
     uint32_t index = 0;
-    for (const auto &op : ops) {
-        if (op->fusedAway) continue;
-        if (index >= first && index - first < count) {
-            if (decorator) decorator(*op, index, true);
-            run(*op, stream);
-            if (decorator) decorator(*op, index, false);
+    try {
+        for (const auto &op : ops) {
+            if (op->fusedAway) continue;
+            if (index >= first && index - first < count) {
+                if (decorator) decorator(*op, index, true);
+                if (index >= splitFirst && index < splitPrefix) {
+                    forkNow();
+                    run(*op, stream, 0);
+                    run(*op, fork ? lane->stream : stream, 1);
+                } else {
+                    join();
+                    run(*op, stream);
+                }
+                if (decorator) decorator(*op, index, false);
+            }
+            index++;
         }
-        index++;
+    } catch (...) {
+        // the second stream must come back to `stream` whatever happened (a capture cannot end with it forked)
+        if (forked && !joined) {
+            (void)mlel_hip_event_record(ctx, lane->join, lane->stream);
+            (void)mlel_hip_stream_wait_event(ctx, stream, lane->join);
+        }
+        throw;
     }
+    join();
 }
 
 }  // namespace mlel::graph

@@ -320,6 +320,23 @@ class GraphPipeline {
     MemoryPlanner memoryPlanner() const { return planner; }
     void finalize(bool enableFusion = true);
     bool isFinalized() const { return finalized; }
+    // Batch split (opt-in, set before finalize()).  The reference records a graph as one chain of dispatches
+    // (cmdBindAndDispatch, compute_graph_op.cpp:2379-2521); on a GPU of 256 compute units a chain of short dependent
+    // launches leaves most of the machine idle.  With the split the leading run of operators that treat the images of
+    // a batch independently (convolutions, depthwise convolutions, pooling, RESCALE / CLAMP / TABLE, the residual
+    // additions; activations [N, ...] with N even) is issued as two launches each, over the first and the second half
+    // of the batch, on two streams that fork at the start of the dispatch and join behind the run; the operators
+    // after it run on whole tensors as before.  Every launch computes the bytes it computes unsplit.  Session
+    // tensors that only the run touches live in two regions, one per half, planned like a graph of half the batch, so
+    // the two streams never share a byte while they are out of step; everything else keeps one contiguous
+    // allocation.  Interval and linear planners only (the best-fit planner's sharing rules assume one chain).
+    void setBatchSplit(bool enabled);
+    bool batchSplitRequested() const { return splitRequested; }
+    uint32_t batchSplitLaunches() const { return splitPrefix - splitFirst; }  // executed operators issued per half (0: not split)
+    uint32_t batchSplitFirst() const { return splitFirst; }
+    struct SplitLane {  // the second stream of a split dispatch and its fork / join events (owned by the session)
+        void *stream = nullptr, *fork = nullptr, *join = nullptr;
+    };
     // Session memory requirements (reference: vkGetDataGraphPipelineSessionMemoryRequirementsARM,
     // graph_layer.cpp:1382-1389): size and alignment of the one allocation all intermediates live in.
     size_t sessionMemorySize() const { return sessionSize; }
@@ -334,7 +351,10 @@ class GraphPipeline {
     using DispatchDecorator = std::function<void(const OpNode &, uint32_t index, bool before)>;
     // `first` / `count` select a run of the executed operators (positions in executionList()); profiling tools time
     // single operators with it.
-    void dispatch(void *stream, const DispatchDecorator &decorator = {}, uint32_t first = 0, uint32_t count = UINT32_MAX);
+    // `lane`: with a batch split, the half-batch launches of the second half go to the lane's stream (a whole
+    // dispatch without decorator only; otherwise, and without a lane, both halves are issued to `stream` in turn).
+    void dispatch(void *stream, const DispatchDecorator &decorator = {}, uint32_t first = 0, uint32_t count = UINT32_MAX,
+                  const SplitLane *lane = nullptr);
 
     // introspection used by tests and the profiler
     std::vector<const OpNode *> executionList() const;
@@ -359,7 +379,9 @@ class GraphPipeline {
     void plan();
     std::vector<details::BestFitTensor> bestFitTensors(const std::vector<details::LiveInterval> &planned,
                                                        const std::vector<details::UnseenAllocation> &unseen);
-    void run(const OpNode &op, void *stream);
+    void run(const OpNode &op, void *stream, int half = -1);  // half 0 / 1: that half of the batch (split run only)
+    void analyzeBatchSplit();
+    void validateSplitPlan() const;
     [[noreturn]] void unsupported(const char *tosaName) const;
 
     mlel_ctx *ctx;
@@ -376,6 +398,13 @@ class GraphPipeline {
     std::map<const TensorDescriptor *, std::array<uint32_t, 2>> ranges;
     std::map<const TensorDescriptor *, const TensorDescriptor *> aliasOf;  // elided RESHAPE: output -> input
     size_t sessionSize = 0;
+    bool splitRequested = false;
+    uint32_t splitFirst = 0;      // executed operators [splitFirst, splitPrefix) are issued as two half-batch launches
+    uint32_t splitPrefix = 0;
+    int64_t splitBatch = 0;       // N of the activations of that run
+    size_t splitFullRegion = 0;   // session memory: [whole tensors | first halves | second halves]
+    size_t splitHalfRegion = 0;
+    std::set<const TensorDescriptor *> splitInterior;  // session tensors stored as two halves, one per region
     MemoryPlanner planner = MemoryPlanner::Interval;
     bool finalized = false;
 
@@ -422,6 +451,8 @@ class GraphSession {
     void *recording = nullptr;       // the instantiated HIP graph of this session's dispatch
     void *recordingStream = nullptr;
     uint64_t recordingVersion = 0;
+    const GraphPipeline::SplitLane *lane();  // created on first use when the pipeline splits the batch
+    GraphPipeline::SplitLane splitLane;
     uint64_t eagerVersion = UINT64_MAX;  // bindings under which recording failed: replayed dispatches run eagerly
     void *eagerStream = nullptr;
     GraphPipeline &pipeline;

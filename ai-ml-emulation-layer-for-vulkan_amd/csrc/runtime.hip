@@ -447,6 +447,12 @@ int mlel_hip_event_record(mlel_ctx *ctx, void *event, void *stream) {
     return 0;
 }
 
+int mlel_hip_stream_wait_event(mlel_ctx *ctx, void *stream, void *event) {
+    MLEL_REQUIRE(ctx != nullptr && event != nullptr, MLEL_ERR_INVALID, "stream_wait_event: null argument");
+    MLEL_HIP_CHECK(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0));
+    return 0;
+}
+
 int mlel_hip_event_elapsed_ms(mlel_ctx *ctx, void *start, void *stop, float *ms) {
     MLEL_REQUIRE(ctx != nullptr && start && stop && ms, MLEL_ERR_INVALID, "event_elapsed_ms: null argument");
     MLEL_HIP_CHECK(hipEventSynchronize((hipEvent_t)stop));

@@ -71,6 +71,8 @@ def load_graph_library():
                                               C.POINTER(C.c_int), C.POINTER(C.c_int)]
         lib.mlel_graph_tensor_info.argtypes = [_V, C.c_int, C.POINTER(C.c_int32), _I64P]
         lib.mlel_graph_finalize.argtypes = [_V, C.c_int]
+        lib.mlel_graph_set_batch_split.argtypes = [_V, C.c_int]
+        lib.mlel_graph_get_batch_split.argtypes = [_V]
         lib.mlel_graph_set_memory_planner.argtypes = [_V, C.c_int]
         lib.mlel_graph_get_memory_planner.argtypes = [_V]
         lib.mlel_graph_session_memory_requirements.argtypes = [_V, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
@@ -268,6 +270,13 @@ class Graph:
     def planner(self):
         code = self._check(self.lib.mlel_graph_get_memory_planner(self.g))
         return [k for k, v in self.PLANNERS.items() if v == code][0]
+
+    def set_batch_split(self, enabled=True):
+        """Before finalize(): the leading batch-separable operators are issued per half batch on two streams."""
+        self._check(self.lib.mlel_graph_set_batch_split(self.g, 1 if enabled else 0))
+
+    def batch_split_launches(self):
+        return self._check(self.lib.mlel_graph_get_batch_split(self.g))
 
     # ---- finalize / memory / run
     def finalize(self, fuse=True):

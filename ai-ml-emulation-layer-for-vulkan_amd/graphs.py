@@ -310,10 +310,12 @@ def _retarget_output(spec, produced, name):
     spec.outputs.append((name, dtype, shape))
 
 
-def build(dev, spec, fuse=True):
+def build(dev, spec, fuse=True, split=False):
     """Creates the GraphPipeline for `spec` on `dev`: constants are uploaded, inputs/outputs become external
-    tensors, everything else lives in planned session memory."""
+    tensors, everything else lives in planned session memory.  `split`: the batch split over two streams."""
     g = Graph(dev)
+    if split:
+        g.set_batch_split(True)
     for name, dtype, shape in spec.inputs + spec.outputs:
         g.external(name, dtype, shape)
     for name, array in spec.consts.items():
@@ -399,6 +401,49 @@ def _time_sessions(dev, g, input_name, output_name, steps, batch, count, replaye
             "outputs_equal_single_session": bool(same)}
 
 
+def _time_replayed(dev, g, input_name, output_name, want, steps, rounds=5):
+    """Milliseconds per graph of one session's replayed dispatch (mlel_graph_session_dispatch_replayed: the launches
+    recorded into a HIP graph once, one submission per dispatch), one batch in flight: the median over `rounds`
+    rounds of `steps` dispatches on one stream; and whether the output equals `want`."""
+    stream = in_flight_streams(dev, 1)[0]
+    s = g.new_session()
+    s.set_input(input_name, g.ext_tensors[input_name].download())
+    for _ in range(3):
+        s.dispatch_replayed(stream)
+    dev._check(dev.lib.mlel_hip_sync(dev.ctx, stream))
+    same = bool(np.array_equal(s.get_output(output_name), want))
+    walls = []
+    for _ in range(rounds):
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            s.dispatch_replayed(stream)
+        dev._check(dev.lib.mlel_hip_sync(dev.ctx, stream))
+        walls.append((time.perf_counter() - t0) / steps)
+    s.close()
+    return float(np.median(walls)) * 1e3, same
+
+
+def bench_batch_split(dev, spec, g, input_name, output_name, steps, warmup):
+    """One batch in flight, four ways: the pipeline `g` dispatched eagerly (timed by the caller) and replayed, and the
+    same graph with the batch split over two streams (mlel_graph_set_batch_split) dispatched eagerly and replayed.
+    Every output is compared with the eager unsplit one."""
+    want = g.get_output(output_name)
+    x = g.ext_tensors[input_name].download()
+    rounds = max(5, -(-50 // steps))
+    replayed_ms, same_r = _time_replayed(dev, g, input_name, output_name, want, steps, rounds)
+    sp = build(dev, spec, fuse=True, split=True)
+    sp.set_input(input_name, x)
+    wall, _ = _time_graph(dev, sp, steps, warmup, rounds)
+    same_e = bool(np.array_equal(sp.get_output(output_name), want))
+    split_replayed_ms, same_s = _time_replayed(dev, sp, input_name, output_name, want, steps, rounds)
+    res = {"launches_split": sp.batch_split_launches(), "session_memory_bytes": sp.session_size,
+           "ms_per_graph": {"one_stream_eager": None, "one_stream_replayed": replayed_ms,
+                            "split_eager": wall * 1e3, "split_replayed": split_replayed_ms},
+           "outputs_equal_unsplit_eager": bool(same_r and same_e and same_s)}
+    sp.close()
+    return res
+
+
 def time_operators(dev, g, reps=50, only=None):
     """Milliseconds per launch of every executed operator of `g` on its own: the operator is launched `reps` times
     back to back on the stream (its inputs are whatever the last whole dispatch left in session memory) between two
@@ -470,6 +515,13 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True, in_flig
            "operators_executed": g.op_count(), "operators_in_graph": len(spec.ops),
            "session_memory_bytes": g.session_size,
            "ms_by_operator": {k: round(v, 4) for k, v in sorted(by_kind.items())}}
+    # one batch in flight, the other ways to issue it: replayed, and with the batch split over two streams
+    split = bench_batch_split(dev, spec, g, "input", "output", steps, warmup)
+    split["ms_per_graph"]["one_stream_eager"] = wall * 1e3
+    best = min(split["ms_per_graph"], key=lambda k: split["ms_per_graph"][k])
+    split["best"] = best
+    split["img_per_s_best"] = batch / (split["ms_per_graph"][best] * 1e-3)
+    res["one_batch_dispatch_modes"] = split
     res["sessions_in_flight"] = [_time_sessions(dev, g, "input", "output", steps, batch, c) for c in in_flight]
     if in_flight:
         res["sessions_in_flight"].append(_time_sessions(dev, g, "input", "output", steps, batch, max(in_flight), replayed=True))

@@ -93,6 +93,16 @@ int mlel_graph_tensor_info(mlel_graph *g, int tensor, int32_t *dtype, int64_t *d
 int mlel_graph_set_memory_planner(mlel_graph *g, int planner);
 int mlel_graph_get_memory_planner(mlel_graph *g);
 
+/* Batch split, opt-in, before mlel_graph_finalize.  The reference records a graph as one chain of dispatches
+ * (cmdBindAndDispatch, graph/compute_graph_op.cpp:2379-2521); with the split, the leading run of operators that
+ * treat the images of a batch independently is issued as two launches each -- the first and the second half of the
+ * batch -- on two streams that fork where the dispatch starts and join behind the run, so that one chain's launch
+ * latencies are covered by the other's work.  Same bytes in every output as the unsplit dispatch.  The session needs
+ * the memory mlel_graph_session_memory_requirements reports after finalize (the tensors inside the run are stored as
+ * two halves).  Interval and linear planners; a graph the split cannot serve is left unsplit.
+ * mlel_graph_get_batch_split: after finalize, the number of launches that are issued per half (0: not split). */
+int mlel_graph_set_batch_split(mlel_graph *g, int enabled);
+int mlel_graph_get_batch_split(mlel_graph *g);
 /* Fusion + session memory planning; then the session requirements
  * (reference: vkGetDataGraphPipelineSessionMemoryRequirementsARM, graph_layer.cpp:1382-1389). */
 int mlel_graph_finalize(mlel_graph *g, int enable_fusion);

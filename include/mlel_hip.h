@@ -261,6 +261,10 @@ int mlel_hip_sync(mlel_ctx *ctx, void *stream); /* NULL = whole device */
 int mlel_hip_event_create(mlel_ctx *ctx, void **out_event);
 int mlel_hip_event_destroy(mlel_ctx *ctx, void *event);
 int mlel_hip_event_record(mlel_ctx *ctx, void *event, void *stream);
+/* Work issued to `stream` after this call starts when the work recorded in `event` (its latest record) is done:
+ * the fork and the join of a dispatch that runs on two streams.  Legal on a stream that is being captured (the
+ * other stream joins the capture).  Reference counterpart: a pipeline barrier between two queues' submissions. */
+int mlel_hip_stream_wait_event(mlel_ctx *ctx, void *stream, void *event);
 int mlel_hip_event_elapsed_ms(mlel_ctx *ctx, void *start, void *stop, float *ms); /* synchronises on stop */
 
 /* HIP-graph capture of a sequence of launches on `stream`, used to replay a whole TOSA graph with one

@@ -214,6 +214,75 @@ def test_memory_planners_give_valid_plans(which):
         assert sizes["interval"] < sizes["linear"]  # the graphs do have tensors with disjoint lifetimes
 
 
+def _build_split(spec, planner="interval"):
+    g = gb.Graph(_NoDevice())
+    g.set_planner(planner)
+    g.set_batch_split(True)
+    for name, dtype, shape in spec.inputs + spec.outputs:
+        g.external(name, dtype, shape)
+    for name, array in spec.consts.items():
+        g.const(name, array)
+    for name, (dtype, shape) in spec.tensors.items():
+        g.tensor(name, dtype, shape)
+    for name, _, _ in spec.inputs:
+        g.mark_input(name)
+    for op in spec.ops:
+        g.op(op["op"], op["in"], op["out"], op["iattr"], op["fattr"], op["name"])
+    for name, _, _ in spec.outputs:
+        g.mark_output(name)
+    g._check(g.lib.mlel_graph_finalize(g.g, 1))
+    size = gb.C.c_uint64()
+    g._check(g.lib.mlel_graph_session_memory_requirements(g.g, gb.C.byref(size), None))
+    return g, size.value
+
+
+def test_batch_split_plan():
+    """The plan of a pipeline whose leading launches are issued per half batch on two streams: session tensors that
+    only the split run touches are stored as two halves behind the whole tensors -- [whole | first halves | second
+    halves] -- and inside the half region no two tensors whose live ranges overlap share a byte at half their size;
+    whole tensors the run touches (here the pooled tensor the fully connected layer reads behind the join) share
+    nothing with each other.  The library checks the same on its side at finalize and refuses a plan that fails."""
+    spec = graphs.mobilenetv2_spec(batch=4, image=64, classes=40)
+    plain = _build_host_only(spec, fuse=True)
+    g, size = _build_split(spec)
+    assert g.op_names() == plain.op_names()
+    launches = g.batch_split_launches()
+    assert launches == len(g.op_names()) - 1  # everything but the fully connected layer
+    placed = [t for t in g.session_tensors() if t["offset"] is not None and t["first"] != 0xFFFFFFFF]
+    halves = [t for t in placed if t["first"] >= 1 and t["last"] <= launches]
+    whole = [t for t in placed if t not in halves]
+    assert halves and whole
+    whole_end = max(t["offset"] + t["size"] for t in whole)
+    half_start = min(t["offset"] for t in halves)
+    assert half_start >= whole_end and half_start % 256 == 0
+    region = (size - half_start) // 2
+    assert half_start + 2 * region == size
+    for i, a in enumerate(halves):
+        assert a["offset"] - half_start + a["size"] // 2 <= region
+        for b in halves[i + 1:]:
+            lives_overlap = a["first"] <= b["last"] and b["first"] <= a["last"]
+            bytes_overlap = a["offset"] < b["offset"] + b["size"] // 2 and b["offset"] < a["offset"] + a["size"] // 2
+            assert not (lives_overlap and bytes_overlap), (a, b)
+    g.close()
+    plain.close()
+    # an odd batch, or the best-fit planner: left unsplit, the plan is the unsplit one
+    odd, _ = _build_split(graphs.mobilenetv2_spec(batch=3, image=64, classes=40))
+    assert odd.batch_split_launches() == 0
+    odd.close()
+    bf, bf_size = _build_split(spec, "bestfit")
+    ref, ref_size, _ = _build_no_device(spec, "bestfit")
+    assert bf.batch_split_launches() == 0 and bf_size == ref_size
+    bf.close()
+    ref.close()
+    lin, _ = _build_split(spec, "linear")  # no reuse at all: every tensor stays whole
+    assert lin.batch_split_launches() == launches
+    lin.close()
+    # the fp16 encoder block starts with a LayerNorm region: nothing to split
+    enc, _ = _build_split(graphs.transformer_block_spec(batch=2, seq=16, d_model=32, heads=2, ffn=64))
+    assert enc.batch_split_launches() == 0
+    enc.close()
+
+
 def test_memory_planner_from_environment(monkeypatch):
     spec = graphs.inverted_residual_spec(batch=1, hw=8)
     for value, expect in (("Linear", "linear"), ("BestFit", "bestfit"), ("Interval", "interval"), ("nonsense", "interval")):

@@ -438,3 +438,49 @@ def test_replayed_dispatch_of_a_graph_that_cannot_be_recorded_runs_eagerly(dev, 
     s.close()
     g.close()
     dev._check(dev.lib.mlel_hip_stream_destroy(dev.ctx, stream))
+
+
+def test_batch_split_dispatch_gives_the_unsplit_bytes(dev):
+    """mlel_graph_set_batch_split: the leading batch-separable launches issued per half batch on two streams.  A
+    MobileNetV2-shaped graph (40 of its 41 launches split; the fully connected layer behind the join runs whole) and
+    the inverted-residual block (every launch split): the same bytes as the unsplit pipeline from an eager dispatch,
+    from the replayed one (the fork and join recorded into the HIP graph; several replays over changing inputs), from a
+    profiled dispatch (both halves on one stream) and from two sessions in flight at once."""
+    cases = [(graphs.mobilenetv2_spec(batch=8, image=96, spread=True, classes=100), 40),
+             (graphs.inverted_residual_spec(batch=6, hw=14, spread=True), 3)]
+    for spec, launches in cases:
+        xs = [random_input(spec, 70 + i) for i in range(3)]
+        plain = graphs.build(dev, spec, fuse=True)
+        want = []
+        for x in xs:
+            plain.set_input("input", x)
+            plain.dispatch()
+            want.append(plain.get_output("output"))
+        plain.close()
+        assert not np.array_equal(want[0], want[1])
+        g = graphs.build(dev, spec, fuse=True, split=True)
+        assert g.batch_split_launches() == launches
+        for x, w in zip(xs, want):  # eager, forked
+            g.set_input("input", x)
+            g.dispatch()
+            np.testing.assert_array_equal(g.get_output("output"), w)
+        g.set_input("input", xs[0])
+        g.dispatch_profiled()  # decorated: the halves follow each other on one stream
+        dev.sync()
+        np.testing.assert_array_equal(g.get_output("output"), want[0])
+        streams = [dev.new_stream(), dev.new_stream()]
+        a, b = g.new_session(), g.new_session()
+        for rep in range(4):  # replayed, two sessions in flight on two streams, inputs changing between replays
+            a.set_input("input", xs[rep % 3])
+            b.set_input("input", xs[(rep + 1) % 3])
+            a.dispatch_replayed(streams[0])
+            b.dispatch_replayed(streams[1])
+            for st in streams:
+                dev._check(dev.lib.mlel_hip_sync(dev.ctx, st))
+            np.testing.assert_array_equal(a.get_output("output"), want[rep % 3], err_msg=f"replay {rep}")
+            np.testing.assert_array_equal(b.get_output("output"), want[(rep + 1) % 3], err_msg=f"replay {rep}")
+        a.close()
+        b.close()
+        g.close()
+        for st in streams:
+            dev.free_stream(st)
