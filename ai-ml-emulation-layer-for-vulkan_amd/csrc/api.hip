@@ -332,6 +332,10 @@ int mlel_hip_concat(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const m
     MLEL_TRY(check_tensor(in, "concat in"));
     MLEL_REQUIRE(in->rank == out->rank && (int)axis < in->rank && dt_size(in->dtype) == dt_size(out->dtype),
                  MLEL_ERR_INVALID, "concat: bad arguments");
+    {
+        const int rc = try_concat_fast((hipStream_t)stream, out, in, axis, offset);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return move_generic_launch((hipStream_t)stream, kConcat, out, in, nullptr, axis, offset);
 }
 
@@ -342,6 +346,10 @@ int mlel_hip_slice(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const ml
     MLEL_TRY(check_tensor(in, "slice in"));
     MLEL_REQUIRE(start != nullptr && in->rank == out->rank && dt_size(in->dtype) == dt_size(out->dtype),
                  MLEL_ERR_INVALID, "slice: bad arguments");
+    {
+        const int rc = try_slice_fast((hipStream_t)stream, out, in, start);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return move_generic_launch((hipStream_t)stream, kSlice, out, in, start, 0, 0);
 }
 
@@ -354,6 +362,10 @@ int mlel_hip_pad(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel
     MLEL_REQUIRE(in->rank == out->rank && in->dtype == out->dtype, MLEL_ERR_INVALID, "pad: type/rank mismatch");
     MLEL_REQUIRE(padding->rank == 1 && padding->dtype == MLEL_I32 && padding->dims[0] >= 2 * in->rank,
                  MLEL_ERR_INVALID, "pad: padding must be int32[2*rank]");
+    {
+        const int rc = try_pad_fast((hipStream_t)stream, out, in, padding, pad_const, pad_const_int);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return pad_generic_launch((hipStream_t)stream, out, in, padding, pad_const, pad_const_int);
 }
 
@@ -443,6 +455,10 @@ int mlel_hip_gather(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const m
     MLEL_REQUIRE(out->rank == 3 && values->rank == 3 && indices->rank == 2 && dt_is_int(indices->dtype) &&
                      dt_size(out->dtype) == dt_size(values->dtype),
                  MLEL_ERR_INVALID, "gather: [N,W,C] from [N,K,C] with integer indices [N,W]");
+    {
+        const int rc = try_gather_fast((hipStream_t)stream, out, values, indices);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return gather_launch((hipStream_t)stream, out, values, indices);
 }
 
@@ -480,6 +496,10 @@ int mlel_hip_reverse(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const 
     MLEL_TRY(check_tensor(in, "reverse in"));
     MLEL_REQUIRE(in->rank == out->rank && (int)axis < out->rank && dt_size(in->dtype) == dt_size(out->dtype),
                  MLEL_ERR_INVALID, "reverse: bad arguments");
+    {
+        const int rc = try_reverse_fast((hipStream_t)stream, out, in, axis);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return reverse_launch((hipStream_t)stream, out, in, axis);
 }
 
@@ -489,6 +509,10 @@ int mlel_hip_tile(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mle
     MLEL_TRY(check_tensor(in, "tile in"));
     MLEL_REQUIRE(in->rank == out->rank && dt_size(in->dtype) == dt_size(out->dtype), MLEL_ERR_INVALID,
                  "tile: bad arguments");
+    {
+        const int rc = try_tile_fast((hipStream_t)stream, out, in);
+        if (rc != 0) return rc < 0 ? rc : 0;
+    }
     return tile_launch((hipStream_t)stream, out, in);
 }
 

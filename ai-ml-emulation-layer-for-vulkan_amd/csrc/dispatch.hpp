@@ -176,4 +176,13 @@ int rescale_add_rescale_launch(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *
                                const FusedEpilogue &s1, const mlel_tensor *in2, const FusedEpilogue &s2,
                                const FusedEpilogue &so);
 
+// ---- data movement in whole pieces on packed tensors (ops_move.hip); each returns 1 when launched, 0 to decline ----
+int try_slice_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const uint32_t *start);
+int try_concat_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis, uint32_t offset);
+int try_pad_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *padding,
+                 double pad_const, int32_t pad_const_int);
+int try_tile_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in);
+int try_reverse_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis);
+int try_gather_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *values, const mlel_tensor *indices);
+
 }  // namespace mlel

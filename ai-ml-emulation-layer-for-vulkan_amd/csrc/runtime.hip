@@ -171,6 +171,43 @@ void launch_copy_variant(int mode, unsigned blocks, hipStream_t s, uint4 *dst, c
         hipLaunchKernelGGL((copy_variant_kernel<U, NT, 0>), dim3(blocks), dim3(256), 0, s, dst, src, n_vec);
 }
 
+// The matrix cores on their own: every wavefront keeps eight independent 32 x 32 int8 accumulator tiles going from
+// operands that sit in registers (loaded once from `operands`: zeros, or random bytes -- the rate this part sustains
+// depends on how many bits toggle), `iters` rounds of eight v_mfma_i32_32x32x32_i8, then one store per lane so that
+// nothing is optimised away.  What a contraction kernel could reach if operand delivery cost nothing.
+typedef int v4i_probe __attribute__((ext_vector_type(4)));
+typedef int v16i_probe __attribute__((ext_vector_type(16)));
+__global__ void __launch_bounds__(256) mfma_rate_kernel(const v4i_probe *__restrict__ operands, int32_t *__restrict__ out,
+                                                        int iters) {
+    const int tid = threadIdx.x + blockIdx.x * 256;
+    v4i_probe a[2], b[4];
+#pragma unroll
+    for (int i = 0; i < 2; i++) a[i] = operands[(tid * 6 + i) & 4095];
+#pragma unroll
+    for (int j = 0; j < 4; j++) b[j] = operands[(tid * 6 + 2 + j) & 4095];
+    v16i_probe acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    int32_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) sum += acc[i][j][r];
+    out[tid] = sum;
+}
+
 // Byte fill for streams under capture, where a memset node must not be recorded: 16-byte stores over the aligned
 // middle, single bytes at the two ragged ends.
 __global__ void __launch_bounds__(256) fill_kernel(unsigned char *__restrict__ dst, size_t head, size_t n_vec,
@@ -511,6 +548,16 @@ int mlel_hip_copy_kernel(mlel_ctx *ctx, void *stream, void *dst, const void *src
         hipLaunchKernelGGL(copy_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (uint4 *)dst, (const uint4 *)src,
                            (size_t)0, (char *)dst + n_vec * 16, (const char *)src + n_vec * 16, n_tail);
     return check_launch("copy_kernel");
+}
+
+int mlel_hip_mfma_rate_probe(mlel_ctx *ctx, void *stream, const void *operands, void *out, int blocks, int iters) {
+    MLEL_REQUIRE(ctx != nullptr && operands != nullptr && out != nullptr, MLEL_ERR_INVALID, "mfma_rate_probe: null argument");
+    MLEL_REQUIRE(blocks > 0 && blocks <= (1 << 20) && iters > 0, MLEL_ERR_INVALID, "mfma_rate_probe: blocks and iters must be positive");
+    MLEL_REQUIRE(((uintptr_t)operands % 16) == 0 && ((uintptr_t)out % 4) == 0, MLEL_ERR_INVALID,
+                 "mfma_rate_probe: operands must be 16-byte aligned");
+    hipLaunchKernelGGL(mfma_rate_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const v4i_probe *)operands, (int32_t *)out, iters);
+    return check_launch("mfma_rate_probe");
 }
 
 int mlel_hip_copy_kernel_variant(mlel_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes, int blocks,

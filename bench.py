@@ -295,6 +295,28 @@ def bench_copy_sweep(dev, info):
             "hbm_ceiling_gbs": best["copy_1024MiB"]["gbs"], "hbm_ceiling_frac_of_published": best["copy_1024MiB"]["gbs"] / HBM_PEAK_GBS}
 
 
+def bench_mfma_rate(dev, info):
+    """The int8 matrix cores with operands in registers (no memory, no LDS in the loop), two resident blocks per compute
+    unit: TOP/s with all-zero operands and with random bytes.  The sustained rate of this part depends on the operand
+    data; the random-data figure is what a contraction over real tensors can at most approach."""
+    cus = info["compute_units"]
+    blocks, iters = cus * 2, 4000
+    out = dev.alloc(blocks * 256 * 4)
+    res = {}
+    for name, data in (("zeros", np.zeros(65536, np.uint8)),
+                       ("random", np.random.default_rng(7).integers(0, 255, 65536, endpoint=True).astype(np.uint8))):
+        t = dev.from_numpy(data)
+        fn = lambda: dev._check(dev.lib.mlel_hip_mfma_rate_probe(dev.ctx, dev.stream, C.c_void_p(t.ptr), C.c_void_p(out),
+                                                                 blocks, iters))
+        us = _median_us(dev, fn, 3, rounds=5, warm=2)
+        ops = 2.0 * 32 * 32 * 32 * 8 * iters * blocks * 4
+        res[name] = {"us": round(us, 1), "tops": round(ops / (us * 1e-6) / 1e12, 1),
+                     "frac_of_published_peak": round(ops / (us * 1e-6) / 1e12 / INT8_MFMA_PEAK_TOPS, 4)}
+        t.free()
+    dev.free(out)
+    return res
+
+
 def measure_copy(dev, nbytes, reps=5):
     src, dst = dev.alloc(nbytes), dev.alloc(nbytes)
     best = 0.0
@@ -437,10 +459,56 @@ def bench_standalone(dev, abi, shape=(16, 56, 56, 144), reps=100):
     return out
 
 
-def bench_extra(dev, abi):
-    """Data-movement operators outside the benchmark graphs (TILE, REVERSE, PAD, SLICE, CONCAT, GATHER) on dense int8
-    tensors of config 3's 56x56 stage: microseconds and algorithmic GB/s (input + output bytes once)."""
-    raise SystemExit("bench.py --only extra: not built yet")
+def bench_extra(dev, abi, reps=50):
+    """Data-movement operators outside the benchmark graphs (SLICE, CONCAT, PAD, TILE, REVERSE, GATHER) on dense int8
+    tensors of config 3's 56 x 56 stage (32 x 56 x 56 x 144, 14.5 MB): microseconds and algorithmic GB/s (bytes read
+    once + bytes written once)."""
+    rng = np.random.default_rng(1006)
+    n, h, w, c = 32, 56, 56, 144
+    x = rng.integers(-128, 127, (n, h, w, c), endpoint=True).astype(np.int8)
+    tx = dev.from_numpy(x)
+    held = [tx]
+
+    def new(shape, dtype=abi.I8):
+        t = dev.tensor(dtype, shape)
+        held.append(t)
+        return t
+
+    u32 = lambda v: (C.c_uint32 * abi.MAX_RANK)(*[int(p) for p in v])
+    o_slice = new((n, h - 2, w - 2, c))
+    start = u32((0, 1, 1, 0))
+    half = dev.from_numpy(x[..., : c // 2].copy())
+    held.append(half)
+    o_cat = new((n, h, w, c))
+    o_pad = new((n, h + 2, w + 2, c))
+    t_pad = dev.from_numpy(np.array([0, 0, 1, 1, 1, 1, 0, 0], np.int32))
+    held.append(t_pad)
+    small = dev.from_numpy(x[: n // 2].copy())
+    held.append(small)
+    o_tile = new((n, h, w, c))
+    o_rev = new((n, h, w, c))
+    vals = dev.from_numpy(x.reshape(n, h * w, c))
+    idx = dev.from_numpy(np.stack([rng.permutation(h * w) for _ in range(n)]).astype(np.int32))
+    held += [vals, idx]
+    o_gather = new((n, h * w, c))
+    size = x.size
+    cases = [
+        ("SLICE crop of one pixel all round", o_slice.nbytes * 2, lambda: dev.op("slice", o_slice.ref, tx.ref, start)),
+        ("CONCAT of two halves along the channels", size * 2,
+         lambda: (dev.op("concat", o_cat.ref, half.ref, 3, 0), dev.op("concat", o_cat.ref, half.ref, 3, c // 2))),
+        ("PAD of one pixel all round", size + o_pad.nbytes, lambda: dev.op("pad", o_pad.ref, tx.ref, t_pad.ref, 0.0, 0)),
+        ("TILE of the batch, twice", size // 2 + size, lambda: dev.op("tile", o_tile.ref, small.ref)),
+        ("REVERSE along the width", size * 2, lambda: dev.op("reverse", o_rev.ref, tx.ref, 2)),
+        ("GATHER of every pixel row, permuted", size * 2 + idx.nbytes, lambda: dev.op("gather", o_gather.ref, vals.ref, idx.ref)),
+    ]
+    out = []
+    for name, nbytes, fn in cases:
+        us = _median_us(dev, fn, reps, rounds=5, warm=3)
+        out.append({"operator": name, "shape": [n, h, w, c], "us": round(us, 2), "algorithmic_bytes": int(nbytes),
+                    "gbs": round(nbytes / (us * 1e-6) / 1e9, 1), "hbm_frac": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+    for t in held:
+        t.free()
+    return out
 
 
 def main():
@@ -477,7 +545,8 @@ def main():
         return
 
     if args.only == "copy":
-        print(json.dumps(dict({"only": "copy"}, **bench_copy_sweep(dev, info))), flush=True)
+        print(json.dumps(dict({"only": "copy", "mfma_rate": bench_mfma_rate(dev, info)}, **bench_copy_sweep(dev, info))),
+              flush=True)
         dev.close()
         return
 

@@ -559,6 +559,12 @@ int mlel_hip_copy_kernel(mlel_ctx *ctx, void *stream, void *dst, const void *src
  * 16-byte pieces.  No counterpart in the reference; a measurement aid. */
 int mlel_hip_copy_kernel_variant(mlel_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes, int blocks,
                                  int pieces_in_flight, int non_temporal, int mode);
+/* The matrix cores without operand delivery: `blocks` blocks of four wavefronts, each wavefront `iters` rounds of
+ * eight independent v_mfma_i32_32x32x32_i8 on operands held in registers, which it reads once from `operands`
+ * (64 KiB: zeros or random bytes -- the sustained rate depends on the data); `out` receives blocks x 256 int32.
+ * 2 x 32 x 32 x 32 x 8 x iters operations per wavefront.  No counterpart in the reference; a measurement aid: the
+ * rate a contraction kernel on this part is to be read against beside the published peak. */
+int mlel_hip_mfma_rate_probe(mlel_ctx *ctx, void *stream, const void *operands, void *out, int blocks, int iters);
 
 #ifdef __cplusplus
 }

@@ -201,6 +201,77 @@ def test_data_movement_ops_vs_oracle(run, oracle):
 
 
 @pytest.mark.gpu
+def test_data_movement_in_pieces_vs_oracle(run, oracle):
+    """SLICE, CONCAT, PAD, TILE, REVERSE and GATHER on packed tensors go through the kernel that moves whole pieces:
+    shapes whose runs are multiples of 16, 8, 4, 2 and 1 bytes, operators acting on the innermost dimension, padding
+    constants of every kind of type, indices outside the source, ranks from 1 to 6 (six non-trivial outer dimensions
+    fall back to the element-wise kernel), and -- for SLICE and CONCAT -- ranges that leave a tensor (the
+    out-of-bounds rules, also element-wise).  Bit for bit the oracle's (= the shaders') results."""
+    rng = np.random.default_rng(21)
+
+    def values(shape, dt):
+        if np.issubdtype(dt, np.floating):
+            return (rng.standard_normal(shape) * 40).astype(dt)
+        info = np.iinfo(dt)
+        return rng.integers(max(info.min, -2 ** 31), min(info.max, 2 ** 31 - 1), shape, endpoint=True).astype(dt)
+
+    for dt, c in ((np.int8, 144), (np.int8, 24), (np.int8, 6), (np.int8, 5), (np.int16, 24), (np.int32, 5),
+                  (np.float16, 7), (np.float32, 64), (np.int64, 3)):
+        x = values((3, 10, 12, c), dt)
+        # SLICE: spatial crop (runs of whole pixels), crop of the channels (unaligned start), nothing cropped
+        for start, size in (((0, 2, 3, 0), (3, 7, 8, c)), ((1, 0, 0, 1), (2, 10, 12, c - 1)), ((0, 0, 0, 0), x.shape),
+                            ((2, 9, 11, c - 1), (1, 1, 1, 1))):
+            np.testing.assert_array_equal(run.slice_(x, start, size), oracle.slice_(x, start, size), err_msg=str((dt, c, start)))
+        # a range that leaves the input: zeros, by the out-of-bounds rule
+        np.testing.assert_array_equal(run.slice_(x, (1, 5, 0, 0), (3, 7, 12, c)), oracle.slice_(x, (1, 5, 0, 0), (3, 7, 12, c)))
+        # CONCAT along every axis
+        for axis in range(4):
+            parts = [values(tuple(d if i != axis else k for i, d in enumerate(x.shape)), dt) for k in (3, 1, 5)]
+            np.testing.assert_array_equal(run.concat(parts, axis), oracle.concat(parts, axis), err_msg=str((dt, c, axis)))
+        # PAD: spatial, channels, everything, nothing
+        const = dict(pad_const=-7.5, pad_const_int=-123456)
+        for pads in (((0, 0), (1, 2), (3, 0), (0, 0)), ((0, 0), (0, 0), (0, 0), (2, 1)), ((1, 1), (1, 1), (1, 1), (1, 1)),
+                     ((0, 0), (0, 0), (0, 0), (0, 0))):
+            shape = tuple(d + a + b for d, (a, b) in zip(x.shape, pads))
+            np.testing.assert_array_equal(run.pad(x, pads, shape, **const), oracle.pad(x, pads, shape, **const),
+                                          err_msg=str((dt, c, pads)))
+        # TILE: outer dimensions, the innermost one, a broadcast from extent 1
+        small = values((2, 1, 4, c), dt)
+        for shape in ((4, 3, 4, c), (2, 1, 12, 2 * c), (2, 5, 4, c)):
+            np.testing.assert_array_equal(run.tile(small, shape), oracle.tile(small, shape), err_msg=str((dt, c, shape)))
+        for axis in range(4):
+            np.testing.assert_array_equal(run.reverse(x, axis), oracle.reverse(x, axis), err_msg=str((dt, c, axis)))
+        # GATHER: some rows outside the source read as zeros; one batch, and several
+        for n in (1, 3):
+            v = values((n, 29, c), dt)
+            idx = rng.integers(0, 28, (n, 17), endpoint=True).astype(np.int32)
+            idx[0, 3], idx[-1, 5] = 29, -1
+            np.testing.assert_array_equal(run.gather(v, idx), oracle.gather(v, idx), err_msg=str((dt, c, n)))
+    # ranks 1, 2 and 6; six outer dimensions that all change stay with the element-wise kernel
+    v1 = values((77,), np.int8)
+    np.testing.assert_array_equal(run.slice_(v1, (5,), (60,)), oracle.slice_(v1, (5,), (60,)))
+    np.testing.assert_array_equal(run.reverse(v1, 0), oracle.reverse(v1, 0))
+    v2 = values((9, 32), np.int16)
+    np.testing.assert_array_equal(run.tile(v2, (27, 32)), oracle.tile(v2, (27, 32)))
+    np.testing.assert_array_equal(run.pad(v2, ((2, 1), (0, 0)), (12, 32)), oracle.pad(v2, ((2, 1), (0, 0)), (12, 32)))
+    v6 = values((2, 3, 2, 3, 4, 16), np.int8)
+    np.testing.assert_array_equal(run.slice_(v6, (1, 1, 0, 1, 2, 0), (1, 2, 2, 2, 2, 16)),
+                                  oracle.slice_(v6, (1, 1, 0, 1, 2, 0), (1, 2, 2, 2, 2, 16)))
+    np.testing.assert_array_equal(run.tile(v6, (4, 6, 4, 6, 8, 32)), oracle.tile(v6, (4, 6, 4, 6, 8, 32)))
+    for axis in range(6):
+        np.testing.assert_array_equal(run.reverse(v6, axis), oracle.reverse(v6, axis))
+    # CONCAT into an output with other data around the part, and a part that does not fit (its overhang is dropped)
+    base = values((2, 6, 8, 16), np.int8)
+    part = values((2, 3, 8, 16), np.int8)
+    want = base.copy()
+    want[:, 2:5] = part
+    np.testing.assert_array_equal(run.concat_at(base, part, 1, 2), want)
+    want = base.copy()
+    want[:, 4:6] = part[:, :2]
+    np.testing.assert_array_equal(run.concat_at(base, part, 1, 4), want)
+
+
+@pytest.mark.gpu
 def test_argmax_and_arithmetic_right_shift_vs_oracle(run, oracle):
     rng = np.random.default_rng(11)
     for dt in (np.int8, np.int16, np.int32):
