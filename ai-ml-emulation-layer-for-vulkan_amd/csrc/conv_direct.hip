@@ -37,11 +37,13 @@ struct DirectArgs {
     int32_t ocb;            // output channels per block (grid.y blocks cover OC)
 };
 
-struct ChanConst {  // per output channel, in shared memory: 32 bytes
+struct ChanConst {  // per output channel, in shared memory.  48 bytes: lane l reads entry l with 128-bit accesses, and
+                    // entries 32 bytes apart put two lanes of every group of sixteen on the same banks
     ChanScale q;
     int32_t bias_adj;
-    int32_t pad;
+    int32_t pad[5];
 };
+static_assert(sizeof(ChanConst) == 48, "ChanConst layout");
 
 enum { STEM = 0, ROWS = 1 };
 
@@ -336,16 +338,22 @@ __global__ void __launch_bounds__(kBlock) conv_rows_mfma_i8_kernel(const RowsMfm
 #pragma unroll
     for (int j = 0; j < NJ; j++) bias_adj[j] = cc[j * 32 + cl].bias_adj;
     char *so = smem + NJ * 32 * sizeof(ChanConst) + wave * 32 * a.op;  // this wavefront's staging tile [32][op]
-    // the tile's 16-byte pieces in memory order: piece p = row p / (OC / 16), 16-byte column p % (OC / 16)
-    const int ppr = a.OC >> 4, npieces = 32 * ppr;
-    uint32_t piece_lds[NJ], piece_row[NJ];
+    // The tile leaves in 16-byte pieces.  Lanes walk the staging tile itself, padding included: slot s = 64 t + lane
+    // is bytes 16 s .. 16 s + 15 of the tile, so a 128-bit read of the wavefront covers one kilobyte of consecutive
+    // shared memory (no bank is asked twice); a slot that falls into a row's padding moves nothing.  Slot s is row
+    // s / (op / 16), 16-byte column s % (op / 16).
+    constexpr int NP = NJ + 1;  // op <= OC + 48 and OC > 32 (NJ - 1): at most NJ + 1 rounds of 64 slots
+    const int spr = a.op >> 4, ppr = a.OC >> 4, nslots = 32 * spr;
+    uint32_t piece_row[NP], piece_out[NP];
 #pragma unroll
-    for (int t = 0; t < NJ; t++) {
-        const int p = t * 64 + lane;
-        const int r = p / ppr;
-        piece_row[t] = p < npieces ? (uint32_t)r : 0xffffu;  // beyond the tile: never below a row count
-        piece_lds[t] = p < npieces ? (uint32_t)(r * a.op + (p - r * ppr) * 16) : 0u;
+    for (int t = 0; t < NP; t++) {
+        const int sl = t * 64 + lane;
+        const int r = sl / spr, c = sl - r * spr;
+        const bool live = sl < nslots && c < ppr;
+        piece_row[t] = live ? (uint32_t)r : 0xffffu;  // a dead slot: never below a row count
+        piece_out[t] = (uint32_t)(r * a.OC + c * 16);
     }
+    const int rounds = (nslots + 63) >> 6;
     const uint32_t sel_a = (lane & 1) ? 0x03070105u : 0x06020400u;  // exchange with lane ^ 1
     const uint32_t sel_b = (lane & 2) ? 0x03020706u : 0x05040100u;  // exchange with lane ^ 2
     char *so_lane = so + (4 * half + (lane & 3)) * a.op + (cl & ~3);
@@ -391,10 +399,12 @@ __global__ void __launch_bounds__(kBlock) conv_rows_mfma_i8_kernel(const RowsMfm
         const uint32_t rows = (uint32_t)min(32, a.M - g * 32);
         const uint32_t obase = (uint32_t)g * 32u * (uint32_t)a.OC;
 #pragma unroll
-        for (int t = 0; t < NJ; t++) {
-            const uint4 d = *reinterpret_cast<const uint4 *>(so + piece_lds[t]);
-            const uint32_t off = piece_row[t] < rows ? obase + (uint32_t)(t * 64 + lane) * 16u : kOob;
-            __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, 0);
+        for (int t = 0; t < NP; t++) {
+            if (t < rounds) {  // uniform
+                const uint4 d = *reinterpret_cast<const uint4 *>(so + (t * 64 + lane) * 16);
+                const uint32_t off = piece_row[t] < rows ? obase + piece_out[t] : kOob;
+                __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, 0);
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -438,7 +448,8 @@ int try_rows_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const ml
     g.o_bytes = (uint32_t)(M * OC);
     g.scale = make_ref(*epi);
     const int nj = (int)((OC + 31) / 32), kc = IC > 16 ? 2 : 1;
-    const size_t sm = (size_t)nj * 32 * sizeof(ChanConst) + (size_t)(kBlock / 64) * 32 * op;
+    // (the last round of slots may read up to 512 bytes past the last wavefront's tile: they are part of the allocation)
+    const size_t sm = (size_t)nj * 32 * sizeof(ChanConst) + (size_t)(kBlock / 64) * 32 * op + 512;
     const int cus = ctx != nullptr && ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
     // Sixteen position groups per block (four per wavefront) amortise the prologue (weights, channel constants);
     // between two and three blocks per compute unit, never more blocks than a group per wavefront needs.  Measured:
