@@ -254,6 +254,8 @@ FUSED_SIGNATURES = {
     "dwconv_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
     "conv2d_dwconv_rescale_clamp": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue), _T, _T,
                                     C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
+    "conv2d_conv2d_rescale_clamp": [_T, _T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue), _T, _T,
+                                    C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
     "matmul_bias_cast": [_T, _T, _T, _T, C.POINTER(MatmulAttr)],
     "matmul_bias_cast_add": [_T, _T, _T, _T, C.POINTER(MatmulAttr), _T],
     "matmul_bias_cast_group": [C.POINTER(MatmulProduct), C.c_int, _T, C.POINTER(MatmulAttr)],
@@ -300,6 +302,8 @@ RUNTIME_SIGNATURES = {
     "mlel_hip_matmul_chain_in_kernel": (C.c_int, [C.POINTER(Chain)]),
     "mlel_hip_attention_f16_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Chain)]),
     "mlel_hip_conv2d_dwconv_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Conv2dAttr), _T, _T,
+                                                   C.POINTER(Conv2dAttr)]),
+    "mlel_hip_conv2d_conv2d_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Conv2dAttr), _T, _T,
                                                    C.POINTER(Conv2dAttr)]),
 }
 

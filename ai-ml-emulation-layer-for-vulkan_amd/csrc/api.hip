@@ -1002,6 +1002,54 @@ int mlel_hip_conv2d_dwconv_in_kernel(const mlel_tensor *out, const mlel_tensor *
     return try_conv2d_dwconv_i8(nullptr, nullptr, out, in, w1, b1, a1, &unused, w2, b2, a2, &unused, false) == 1 ? 1 : 0;
 }
 
+int mlel_hip_conv2d_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *mid,
+                                         const mlel_tensor *in, const mlel_tensor *w1, const mlel_tensor *b1,
+                                         const mlel_conv2d_attr *a1, const mlel_epilogue *e1, const mlel_tensor *w2,
+                                         const mlel_tensor *b2, const mlel_conv2d_attr *a2, const mlel_epilogue *e2) {
+    MLEL_TRY(require_ctx(ctx, "conv2d_conv2d_rescale_clamp"));
+    FusedEpilogue f1, f2;
+    MLEL_TRY(conv_dw_prepare("conv2d_conv2d_rescale_clamp", out, in, w1, b1, a1, e1, w2, b2, a2, e2, &f1, &f2));
+    if (mid != nullptr) {
+        MLEL_TRY(check_tensor(mid, "conv2d_conv2d_rescale_clamp mid"));
+        MLEL_REQUIRE(mid->rank == 4 && mid->dims[0] == in->dims[0] && mid->dims[1] == in->dims[1] &&
+                         mid->dims[2] == in->dims[2] && mid->dims[3] == w1->dims[0] && dt_size(mid->dtype) == 1,
+                     MLEL_ERR_INVALID, "conv2d_conv2d_rescale_clamp: the intermediate tensor is 8-bit [N, H, W, OC1]");
+    }
+    const int mid_dt = mid != nullptr ? mid->dtype : MLEL_I8;
+    const int rc = try_conv2d_pair_rows(ctx, (hipStream_t)stream, out, mid, in, w1, b1, a1, &f1, mid_dt, w2, b2, a2, &f2, false);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    // no one-pass kernel for these operands: the two fused operators one after the other, through the caller's
+    // intermediate tensor or a temporary
+    if (mid != nullptr) {
+        MLEL_TRY(mlel_hip_conv2d_rescale_clamp(ctx, stream, mid, in, w1, b1, a1, e1));
+        return mlel_hip_conv2d_rescale_clamp(ctx, stream, out, mid, w2, b2, a2, e2);
+    }
+    Scratch scratch;
+    const size_t bytes = (size_t)(in->dims[0] * in->dims[1] * in->dims[2] * w1->dims[0]);
+    MLEL_TRY(alloc_fallback(scratch, bytes + 16, stream, __func__));
+    mlel_tensor tmp{};
+    tmp.dtype = MLEL_I8;
+    tmp.rank = 4;
+    tmp.dims[0] = in->dims[0], tmp.dims[1] = in->dims[1], tmp.dims[2] = in->dims[2], tmp.dims[3] = w1->dims[0];
+    tmp.strides[3] = 1;
+    for (int i = 2; i >= 0; i--) tmp.strides[i] = tmp.strides[i + 1] * tmp.dims[i + 1];
+    tmp.ptr = scratch.ptr;
+    MLEL_TRY(mlel_hip_conv2d_rescale_clamp(ctx, stream, &tmp, in, w1, b1, a1, e1));
+    MLEL_TRY(mlel_hip_conv2d_rescale_clamp(ctx, stream, out, &tmp, w2, b2, a2, e2));
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+int mlel_hip_conv2d_conv2d_in_kernel(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w1,
+                                     const mlel_tensor *b1, const mlel_conv2d_attr *a1, const mlel_tensor *w2,
+                                     const mlel_tensor *b2, const mlel_conv2d_attr *a2) {
+    if (out == nullptr || in == nullptr || w1 == nullptr || b1 == nullptr || a1 == nullptr || w2 == nullptr ||
+        b2 == nullptr || a2 == nullptr)
+        return 0;
+    const FusedEpilogue unused{};  // the requantisation constants do not decide whether the kernel takes the case
+    return try_conv2d_pair_rows(nullptr, nullptr, out, nullptr, in, w1, b1, a1, &unused, MLEL_I8, w2, b2, a2, &unused, true) == 1 ? 1 : 0;
+}
+
 int mlel_hip_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1,
                                  const mlel_epilogue *scale1, const mlel_tensor *in2, const mlel_epilogue *scale2,
                                  const mlel_epilogue *scale_out) {

@@ -471,6 +471,227 @@ int try_rows_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const ml
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// Two 1x1 CONV2D + RESCALE (+CLAMP) in a row in one launch: a projection to at most 32 channels followed by the
+// expansion that reads it (MobileNetV2: 32 -> 16 -> 96 at 112 x 112, 96 -> 24 -> 144 at 56 x 56).  Both operators
+// treat positions independently, so the wavefront that owns 32 positions runs the first product (K = IC0 in steps of
+// 16 on v_mfma_i32_32x32x16_i8, rows straight from memory, weights in registers), requantises its 32 x OC0 bytes into
+// a tile of its own in shared memory -- the bytes the first operator would have stored -- and reads them back as the
+// row operand of conv_rows_mfma_i8_kernel's loop.  When another operator reads the intermediate tensor as well (a
+// residual connection further on) the tile is also written to memory, as consecutive bytes; otherwise it never
+// leaves the chip.  Reference arithmetic: conv2d.comp:40-116, rescale.comp:28-63, clamp.comp:18-31, twice.
+// ---------------------------------------------------------------------------------------------------------------
+struct Rows2Args {
+    RowsMfmaArgs r;          // the second operator; r.x is unused, r.IC = OC0
+    const int8_t *x0, *w0;   // the first operator's input [M][IC0] and weights [OC0][IC0]
+    const int32_t *bias0;
+    char *mid;               // where the intermediate tensor [M][OC0] is stored as well, or nullptr
+    int32_t IC0, zx0, bias0_len;
+    uint32_t x0_bytes, mid_bytes;
+    ScaleRef scale0;
+};
+
+template <int NJ, int KC, int KC0>
+__global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NJ <= 3 ? 3 : 2, NJ <= 3 ? 3 : 2)))
+conv_rows2_mfma_i8_kernel(const Rows2Args b) {
+    const RowsMfmaArgs &a = b.r;
+    extern __shared__ __align__(16) char smem[];
+    ChanConst *cc = reinterpret_cast<ChanConst *>(smem);  // [NJ * 32] second operator, then [32] first operator
+    ChanConst *cc0 = cc + NJ * 32;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cl = lane & 31, half = lane >> 5;
+    const int OC0 = a.IC;
+
+    const __amdgpu_buffer_rsrc_t xres =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(b.x0), 0, (int)b.x0_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ores = __builtin_amdgcn_make_buffer_rsrc(a.out, 0, (int)a.o_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t mres =
+        __builtin_amdgcn_make_buffer_rsrc(b.mid != nullptr ? b.mid : a.out, 0, (int)(b.mid != nullptr ? b.mid_bytes : 0u), 0x00020000);
+    const uint32_t kOob = 0x80000000u;
+    auto fetch = [&](int g, long (&xf)[KC0]) {  // first product's row operand: lane = position lane % 32 of the group
+        const int m = g * 32 + cl;
+#pragma unroll
+        for (int c = 0; c < KC0; c++) {
+            const int k0 = c * 16 + half * 8;
+            const uint32_t off = (g < a.groups && m < a.M && k0 < b.IC0) ? (uint32_t)m * (uint32_t)b.IC0 + (uint32_t)k0 : kOob;
+            const auto v = __builtin_amdgcn_raw_buffer_load_b64(xres, (int)off, 0, 0);
+            xf[c] = (long)(((uint64_t)v[1] << 32) | (uint64_t)v[0]);
+        }
+    };
+    const int nwaves = (int)gridDim.x * (kBlock / 64);
+    int g = (int)blockIdx.x * (kBlock / 64) + wave;
+    long xf0[KC0], xn0[KC0];
+    fetch(g, xf0);
+    // ---- both weight sets as matrix B operands: lane = channel lane % 32 (of column j), 8 bytes of K per lane half
+    long wf0[KC0];
+#pragma unroll
+    for (int c = 0; c < KC0; c++) {
+        const int k0 = c * 16 + half * 8;
+        wf0[c] = (cl < OC0 && k0 < b.IC0) ? *reinterpret_cast<const long *>(b.w0 + (int64_t)cl * b.IC0 + k0) : 0;
+    }
+    long wf[NJ][KC];
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+        for (int c = 0; c < KC; c++) {
+            const int oc = j * 32 + cl, k0 = c * 16 + half * 8;
+            wf[j][c] = (oc < a.OC && k0 < OC0) ? *reinterpret_cast<const long *>(a.w + (int64_t)oc * OC0 + k0) : 0;
+        }
+    // ---- per-channel constants of both operators (each input zero point folded into its bias term)
+    for (int oc = tid; oc < NJ * 32 + 32; oc += kBlock) {
+        ChanConst c{};
+        const bool first = oc >= NJ * 32;
+        const int ch = first ? oc - NJ * 32 : oc;
+        const int chans = first ? OC0 : a.OC, kk = first ? b.IC0 : OC0;
+        if (ch < chans) {
+            int32_t wsum = 0;
+            const uint32_t *wp = reinterpret_cast<const uint32_t *>((first ? b.w0 : a.w) + (int64_t)ch * kk);
+            for (int j = 0; j < kk / 4; j++) wsum = __builtin_amdgcn_sdot4((int)wp[j], 0x01010101, wsum, false);
+            const int32_t bias = first ? b.bias0[b.bias0_len == 1 ? 0 : ch] : a.bias[a.bias_len == 1 ? 0 : ch];
+            c.bias_adj = (int32_t)((uint32_t)bias - (uint32_t)(first ? b.zx0 : a.zx) * (uint32_t)wsum);
+            const ScaleRef &sc = first ? b.scale0 : a.scale;
+            const int ci = sc.p.per_channel ? ch : 0;
+            c.q = make_chan_scale(load_mult(sc, ci), (int32_t)sc.shift[ci], sc.p);
+        }
+        cc[oc] = c;
+    }
+    __syncthreads();
+
+    int32_t bias_adj[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; j++) bias_adj[j] = cc[j * 32 + cl].bias_adj;
+    const ChanConst c0 = cc0[cl];  // the first operator's constants of this lane's channel stay in registers
+    // this wavefront's tiles: the intermediate [32][OC0] (+ 16 bytes that the last row's second K piece may read),
+    // then the staging tile [32][op] of the result
+    const int mid_tile = 32 * OC0 + 16;
+    char *mt = smem + (NJ * 32 + 32) * sizeof(ChanConst) + wave * (mid_tile + 32 * a.op);
+    char *so = mt + mid_tile;
+    constexpr int NP = NJ + 1;
+    const int spr = a.op >> 4, ppr = a.OC >> 4, nslots = 32 * spr;
+    uint32_t piece_row[NP], piece_out[NP];
+#pragma unroll
+    for (int t = 0; t < NP; t++) {
+        const int sl = t * 64 + lane;
+        const int r = sl / spr, c = sl - r * spr;
+        const bool live = sl < nslots && c < ppr;
+        piece_row[t] = live ? (uint32_t)r : 0xffffu;
+        piece_out[t] = (uint32_t)(r * a.OC + c * 16);
+    }
+    const int rounds = (nslots + 63) >> 6;
+    const uint32_t sel_a = (lane & 1) ? 0x03070105u : 0x06020400u;  // exchange with lane ^ 1
+    const uint32_t sel_b = (lane & 2) ? 0x03020706u : 0x05040100u;  // exchange with lane ^ 2
+    char *so_lane = so + (4 * half + (lane & 3)) * a.op + (cl & ~3);
+    char *mt_lane = mt + (4 * half + (lane & 3)) * OC0 + (cl & ~3);
+    const bool mid_col_live = (cl & ~3) < OC0;  // OC0 is a multiple of 8: whole dwords are in or out
+    const int mid_pieces = 2 * OC0;             // 16-byte pieces of the intermediate tile: 32 * OC0 / 16
+    auto pack4 = [&](const int32_t (&v)[4]) {
+        const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
+        const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
+        uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // bytes = positions e of this lane's channel
+        uint32_t o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0xb1, 0xf, 0xf, true);
+        p = __builtin_amdgcn_perm(o, p, sel_a);
+        o = (uint32_t)__builtin_amdgcn_mov_dpp((int)p, 0x4e, 0xf, 0xf, true);
+        return __builtin_amdgcn_perm(o, p, sel_b);  // position 8 q + 4 (lane / 32) + lane % 4, four channels
+    };
+    auto wave_sync = [] {
+        // the wavefront's own writes and reads of its tiles execute in order; the compiler must keep that order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    for (; g < a.groups; g += nwaves) {
+        fetch(g + nwaves, xn0);  // the next group's pixels travel while this one is worked on
+        const uint32_t rows = (uint32_t)min(32, a.M - g * 32);
+        // ---- first operator: 32 positions x OC0 channels into the intermediate tile
+        {
+            v16i32 acc0;
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc0[r] = c0.bias_adj;
+#pragma unroll
+            for (int kc = 0; kc < KC0; kc++) acc0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(xf0[kc], wf0[kc], acc0, 0, 0, 0);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int32_t v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = requant_acc(acc0[4 * q + e], c0.q, b.scale0.p);
+                const uint32_t p = pack4(v);
+                if (mid_col_live) *reinterpret_cast<uint32_t *>(mt_lane + 8 * q * OC0) = p;
+            }
+        }
+        wave_sync();
+        if (b.mid != nullptr && lane < mid_pieces) {  // the intermediate tensor's 32 rows are consecutive in memory
+            const uint4 d = *reinterpret_cast<const uint4 *>(mt + lane * 16);
+            const uint32_t off = (uint32_t)(lane * 16) < rows * (uint32_t)OC0 ? (uint32_t)g * 32u * (uint32_t)OC0 + (uint32_t)lane * 16u : kOob;
+            __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, mres, (int)off, 0, 0);
+        }
+        long xf[KC];
+#pragma unroll
+        for (int c = 0; c < KC; c++) xf[c] = *reinterpret_cast<const long *>(mt + cl * OC0 + c * 16 + half * 8);
+        // ---- second operator, as conv_rows_mfma_i8_kernel, one 32-channel column after the other: only two
+        // accumulator tiles are alive at a time (the next column's product runs while this one is requantised), which
+        // keeps the register count low enough for several wavefronts per SIMD
+        auto column = [&](int j) {
+            v16i32 acc;
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r] = bias_adj[j];
+#pragma unroll
+            for (int kc = 0; kc < KC; kc++) acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(xf[kc], wf[j][kc], acc, 0, 0, 0);
+            return acc;
+        };
+        v16i32 acc = column(0);
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            v16i32 next = acc;
+            if (j + 1 < NJ) next = column(j + 1);
+            const ChanConst c = cc[j * 32 + cl];
+            const bool col_live = j * 32 + (cl & ~3) < a.OC;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int32_t v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[4 * q + e], c.q, a.scale.p);
+                const uint32_t p = pack4(v);
+                if (col_live) *reinterpret_cast<uint32_t *>(so_lane + 8 * q * a.op + j * 32) = p;
+            }
+            acc = next;
+            __builtin_amdgcn_sched_barrier(0);  // (the scheduler would otherwise start every column's product first)
+        }
+        wave_sync();
+        const uint32_t obase = (uint32_t)g * 32u * (uint32_t)a.OC;
+#pragma unroll
+        for (int t = 0; t < NP; t++) {
+            if (t < rounds) {  // uniform
+                const uint4 d = *reinterpret_cast<const uint4 *>(so + (t * 64 + lane) * 16);
+                const uint32_t off = piece_row[t] < rows ? obase + piece_out[t] : kOob;
+                __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, 0);
+            }
+        }
+        wave_sync();
+#pragma unroll
+        for (int c = 0; c < KC0; c++) xf0[c] = xn0[c];
+    }
+}
+
+// The shapes the two-operator kernel exists for (each is its own kernel): second operator's 32-channel columns,
+// 16-byte K pieces of the second and of the first operator.
+template <int NJ, int KC, int KC0>
+void launch_rows2(const Rows2Args &g, dim3 grid, size_t sm, hipStream_t s) {
+    auto kernel = conv_rows2_mfma_i8_kernel<NJ, KC, KC0>;
+    if (sm > 48 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm);
+    kernel<<<grid, dim3(kBlock), sm, s>>>(g);
+}
+
+bool rows2_shape(int64_t IC0, int64_t OC0, int64_t OC, int *nj, int *kc, int *kc0) {
+    if (IC0 % 16 != 0 || OC0 % 8 != 0 || OC0 > 32 || OC0 <= 0 || OC % 16 != 0 || OC > 192 || OC <= 0) return false;
+    *nj = (int)((OC + 31) / 32);
+    *kc = OC0 > 16 ? 2 : 1;
+    *kc0 = (int)(IC0 / 16);
+    // the instantiated combinations: 32 -> 16 -> 96, 96 -> 24 -> 144 (MobileNetV2) and their neighbours
+    const bool known = (*nj == 3 && *kc == 1 && *kc0 == 2) || (*nj == 5 && *kc == 2 && *kc0 == 6) ||
+                       (*nj == 6 && *kc == 2 && *kc0 == 2) || (*nj == 6 && *kc == 2 && *kc0 == 6);
+    return known;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // STEM on the matrix cores: 3x3 CONV2D over 3-byte pixels (an RGB image stem, K = 27) + RESCALE (+CLAMP) to 8 bits
 // with 16 or 32 output channels.  The structure of conv_rows_mfma_i8_kernel (a wavefront owns 32 consecutive output
 // positions and all channels, weights in registers, per-wavefront staging tile), with one v_mfma_i32_32x32x32_i8 per
@@ -792,6 +1013,91 @@ int try_conv2d_i8_direct(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, c
             launch_direct<ROWS, 4, 8>(g, splits, cus, s);
     }
     MLEL_TRY(check_launch("conv2d direct int8"));
+    return 1;
+}
+
+// Two 1x1 CONV2D + RESCALE (+CLAMP) in a row (conv_rows2_mfma_i8_kernel).  `mid`: the intermediate tensor when something
+// else reads it too, else nullptr.  Returns 1 when launched, 0 to decline; `probe`: judge only, launch nothing.
+int try_conv2d_pair_rows(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *mid,
+                         const mlel_tensor *in, const mlel_tensor *w1, const mlel_tensor *b1, const mlel_conv2d_attr *a1,
+                         const FusedEpilogue *e1, int mid_dtype, const mlel_tensor *w2, const mlel_tensor *b2,
+                         const mlel_conv2d_attr *a2, const FusedEpilogue *e2, bool probe) {
+    if (in->dtype != MLEL_I8 || w1->dtype != MLEL_I8 || w2->dtype != MLEL_I8 || b1->dtype != MLEL_I32 ||
+        b2->dtype != MLEL_I32 || out->dtype != MLEL_I8 || mid_dtype != MLEL_I8)
+        return 0;
+    if (a1->acc_type != MLEL_ACC_I32 || a2->acc_type != MLEL_ACC_I32 || a1->weight_zp != 0 || a2->weight_zp != 0) return 0;
+    if (e1 == nullptr || e2 == nullptr || e1->p.in_zp != 0 || e2->p.in_zp != 0) return 0;
+    if (in->rank != 4 || out->rank != 4 || w1->rank != 4 || w2->rank != 4) return 0;
+    const int64_t N = out->dims[0], H = out->dims[1], W = out->dims[2], OC = out->dims[3];
+    const int64_t IC0 = in->dims[3], OC0 = w1->dims[0];
+    for (const mlel_conv2d_attr *a : {a1, a2})
+        if (a->stride[0] != 1 || a->stride[1] != 1 || a->dilation[0] != 1 || a->dilation[1] != 1 || a->pad[0] != 0 ||
+            a->pad[1] != 0 || a->pad[2] != 0 || a->pad[3] != 0)
+            return 0;
+    if (w1->dims[1] != 1 || w1->dims[2] != 1 || w1->dims[3] != IC0 || w2->dims[0] != OC || w2->dims[1] != 1 ||
+        w2->dims[2] != 1 || w2->dims[3] != OC0)
+        return 0;
+    if (in->dims[0] != N || in->dims[1] != H || in->dims[2] != W) return 0;
+    if (!is_packed(in) || !is_packed(out) || !is_packed(w1) || !is_packed(w2)) return 0;
+    if (mid != nullptr && (!is_packed(mid) || mid->dtype != MLEL_I8 || mid->rank != 4 || mid->dims[0] != N ||
+                           mid->dims[1] != H || mid->dims[2] != W || mid->dims[3] != OC0))
+        return 0;
+    for (const mlel_tensor *bt : {b1, b2})
+        if (bt->rank != 1 || bt->strides[0] != 4 || ((uintptr_t)bt->ptr % 4) != 0) return 0;
+    if (!(b1->dims[0] == 1 || b1->dims[0] >= OC0) || !(b2->dims[0] == 1 || b2->dims[0] >= OC)) return 0;
+    int nj = 0, kc = 0, kc0 = 0;
+    if (!rows2_shape(IC0, OC0, OC, &nj, &kc, &kc0)) return 0;
+    const int64_t M = N * H * W;
+    if (M <= 0) return probe ? 1 : 1;
+    if (M * OC >= (int64_t(1) << 31) || M * IC0 >= (int64_t(1) << 31)) return 0;
+    // the intermediate tensor leaves in 16-byte pieces: its extent must be whole pieces (a probe does not know whether
+    // it will be stored, so it asks for this as well)
+    if ((M * OC0) % 16 != 0) return 0;
+    if (probe) return 1;  // (alignment is a property of the bound memory: checked at launch, the caller then falls back)
+    if (((uintptr_t)in->ptr % 8) != 0 || ((uintptr_t)w1->ptr % 8) != 0 || ((uintptr_t)w2->ptr % 8) != 0 ||
+        ((uintptr_t)out->ptr % 16) != 0 || (mid != nullptr && ((uintptr_t)mid->ptr % 16) != 0))
+        return 0;
+    Rows2Args g{};
+    g.r.w = static_cast<const int8_t *>(w2->ptr);
+    g.r.bias = static_cast<const int32_t *>(b2->ptr);
+    g.r.out = static_cast<char *>(out->ptr);
+    g.r.M = (int)M;
+    g.r.IC = (int)OC0;
+    g.r.OC = (int)OC;
+    g.r.zx = a2->input_zp;
+    g.r.bias_len = (int)b2->dims[0];
+    g.r.groups = (int)((M + 31) / 32);
+    int op = (int)OC;
+    while (op % 128 != 32 && op % 128 != 96) op += 16;
+    g.r.op = op;
+    g.r.o_bytes = (uint32_t)(M * OC);
+    g.r.scale = make_ref(*e2);
+    g.x0 = static_cast<const int8_t *>(in->ptr);
+    g.w0 = static_cast<const int8_t *>(w1->ptr);
+    g.bias0 = static_cast<const int32_t *>(b1->ptr);
+    g.mid = mid != nullptr ? static_cast<char *>(mid->ptr) : nullptr;
+    g.IC0 = (int)IC0;
+    g.zx0 = a1->input_zp;
+    g.bias0_len = (int)b1->dims[0];
+    g.x0_bytes = (uint32_t)(M * IC0);
+    g.mid_bytes = (uint32_t)(M * OC0);
+    g.scale0 = make_ref(*e1);
+    const size_t sm = (size_t)(nj * 32 + 32) * sizeof(ChanConst) +
+                      (size_t)(kBlock / 64) * (32 * (size_t)OC0 + 16 + 32 * (size_t)op) + 512;
+    const int cus = ctx != nullptr && ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;
+    const int64_t per_wave = (g.r.groups + kBlock / 64 - 1) / (kBlock / 64);
+    const int64_t want = std::min<int64_t>(
+        per_wave, std::min<int64_t>((int64_t)cus * 3, std::max<int64_t>((int64_t)cus * 2, (g.r.groups + 15) / 16)));
+    const dim3 grid((unsigned)std::max<int64_t>(want, 1));
+    if (nj == 3 && kc == 1 && kc0 == 2)
+        launch_rows2<3, 1, 2>(g, grid, sm, s);
+    else if (nj == 5 && kc == 2 && kc0 == 6)
+        launch_rows2<5, 2, 6>(g, grid, sm, s);
+    else if (nj == 6 && kc == 2 && kc0 == 2)
+        launch_rows2<6, 2, 2>(g, grid, sm, s);
+    else
+        launch_rows2<6, 2, 6>(g, grid, sm, s);
+    MLEL_TRY(check_launch("conv2d pair rows int8"));
     return 1;
 }
 

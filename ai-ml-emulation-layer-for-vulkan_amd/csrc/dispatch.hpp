@@ -176,6 +176,11 @@ int rescale_add_rescale_launch(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *
                                const FusedEpilogue &s1, const mlel_tensor *in2, const FusedEpilogue &s2,
                                const FusedEpilogue &so);
 
+// ---- two 1x1 CONV2D + RESCALE (+CLAMP) in a row, one launch (conv_direct.hip); `probe`: judge only ----
+int try_conv2d_pair_rows(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, const mlel_tensor *mid,
+                         const mlel_tensor *in, const mlel_tensor *w1, const mlel_tensor *b1, const mlel_conv2d_attr *a1,
+                         const FusedEpilogue *e1, int mid_dtype, const mlel_tensor *w2, const mlel_tensor *b2,
+                         const mlel_conv2d_attr *a2, const FusedEpilogue *e2, bool probe);
 // ---- data movement in whole pieces on packed tensors (ops_move.hip); each returns 1 when launched, 0 to decline ----
 int try_slice_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const uint32_t *start);
 int try_concat_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis, uint32_t offset);

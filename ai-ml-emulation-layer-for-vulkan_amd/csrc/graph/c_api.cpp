@@ -313,6 +313,10 @@ std::string opLabel(const OpNode &op) {
     case OpKind::FusedConv2DDepthwise:
         return std::string("CONV2D+RESCALE") + (op.hasClampFirst ? "+CLAMP" : "") + "+DEPTHWISE_CONV2D+RESCALE" +
                (op.hasClamp ? "+CLAMP" : "");
+    case OpKind::FusedConv2DConv2D:
+        // "+KEEP": the first convolution's result is stored as well (a later operator reads it)
+        return std::string("CONV2D+RESCALE") + (op.hasClampFirst ? "+CLAMP" : "") + (op.outputs.size() > 1 ? "+KEEP" : "") +
+               "+CONV2D+RESCALE" + (op.hasClamp ? "+CLAMP" : "");
     case OpKind::FusedAttention:
         return std::string("MATMUL+CAST+ELEMENTWISE+REDUCE x") + std::to_string(op.chain.size()) + "+MATMUL+CAST" +
                (op.viewDims[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");

@@ -1252,6 +1252,50 @@ void GraphPipeline::fuse() {
         conv->fusedAway = true;
     }
 
+    // Pattern 9 (projection + expansion): a fused 1x1 CONV2D whose int8 result is the image of another fused 1x1
+    // CONV2D, on shapes the one-launch kernel takes (mlel_hip_conv2d_conv2d_in_kernel decides).  Positions are
+    // independent in both operators, so a wavefront hands its 32 positions from one product to the next through
+    // shared memory.  When the second convolution is the only reader the intermediate tensor disappears; when later
+    // operators read it too (a residual connection) it is still written, by the same launch.  Byte for byte the two
+    // launches.
+    for (size_t bi = 0; bi < ops.size(); bi++) {
+        OpNode &second = *ops[bi];
+        if (second.fusedAway || second.kind != OpKind::FusedConv2D) continue;
+        const TensorPtr mid = second.inputs[0];
+        OpNode *first = mid->getProducer();
+        if (!first || first->fusedAway || first->kind != OpKind::FusedConv2D || first->outputs[0].get() != mid.get() ||
+            !isPrivateIntermediate(*mid))
+            continue;
+        if (first->epilogue.attr.input_zp != 0 || second.epilogue.attr.input_zp != 0) continue;
+        // every other reader of the intermediate tensor runs after the second convolution
+        bool later = true, others = false;
+        for (size_t k = 0; k < ops.size(); k++) {
+            if (ops[k]->fusedAway || ops[k].get() == &second) continue;
+            bool reads = false;
+            for (const auto &t : ops[k]->inputs) reads = reads || t.get() == mid.get();
+            if (reads) {
+                others = true;
+                later = later && k > bi;
+            }
+        }
+        if (!later) continue;
+        const mlel_tensor out = second.outputs[0]->view(), x = first->inputs[0]->view(), w1 = first->inputs[1]->view(),
+                          b1 = first->inputs[2]->view(), w2 = second.inputs[1]->view(), b2 = second.inputs[2]->view();
+        if (mlel_hip_conv2d_conv2d_in_kernel(&out, &x, &w1, &b1, &first->conv, &w2, &b2, &second.conv) == 0) continue;
+        const TensorPtr w2T = second.inputs[1], b2T = second.inputs[2];
+        second.kind = OpKind::FusedConv2DConv2D;
+        second.inputs = {first->inputs[0], first->inputs[1], first->inputs[2], w2T, b2T};
+        second.convFirst = first->conv;
+        second.scaleA = first->epilogue;
+        second.hasClampFirst = first->hasClamp;
+        second.clampFirst = first->clamp;
+        if (others) {
+            second.outputs.push_back(mid);
+            mid->setProducer(&second);
+        }
+        first->fusedAway = true;
+    }
+
     // Pattern 3: RESHAPE between two packed session tensors of the same byte size moves no data (the reference's
     // reshape.comp:16-27 copies by flat index): the output becomes a second view of the input's storage and the
     // operator is not executed.  plan() gives both tensors one allocation that lives as long as either is used.
@@ -1597,6 +1641,7 @@ bool batchOperands(const OpNode &op, std::vector<size_t> &ins) {
     case OpKind::FusedConv2D:
     case OpKind::FusedDepthwiseConv2D:
     case OpKind::FusedConv2DDepthwise:
+    case OpKind::FusedConv2DConv2D:
     case OpKind::AvgPool2D:
     case OpKind::MaxPool2D:
     case OpKind::Rescale:
@@ -1634,7 +1679,11 @@ void GraphPipeline::analyzeBatchSplit() {
     std::vector<size_t> act;
     for (const auto &op : ops) {
         if (op->fusedAway) continue;
-        if (!batchOperands(*op, act) || op->outputs.size() != 1 || !carriesBatch(op->outputs[0])) break;
+        if (!batchOperands(*op, act) || !carriesBatch(op->outputs[0])) break;
+        // a second output only where the launch writes one (the stored intermediate of a convolution pair)
+        if (op->outputs.size() != 1 &&
+            !(op->kind == OpKind::FusedConv2DConv2D && op->outputs.size() == 2 && carriesBatch(op->outputs[1])))
+            break;
         bool ok = true;
         for (size_t i = 0; i < op->inputs.size() && ok; i++) {
             const bool isAct = std::find(act.begin(), act.end(), i) != act.end();
@@ -1862,14 +1911,14 @@ void GraphPipeline::run(const OpNode &op, void *stream, const int half) {
     mlel_tensor out = op.outputs[0]->view();
     if (out.ptr == nullptr && op.outputs[0]->getShapeSize() != 0)
         fail(op.tosaName + " (" + op.debugName + "): output tensor has no memory bound");
+    // one half of the batch: half the outermost extent; the second half of a tensor stored as two halves lies one
+    // region further, that of a whole tensor half its size further
+    const auto halved = [&](mlel_tensor &v, const TensorDescriptor *t) {
+        v.dims[0] = splitBatch / 2;
+        const size_t step = splitInterior.count(t) ? splitHalfRegion : static_cast<size_t>(v.dims[0] * v.strides[0]);
+        v.ptr = static_cast<char *>(v.ptr) + static_cast<size_t>(half) * step;
+    };
     if (half >= 0) {
-        // one half of the batch: half the outermost extent; the second half of a tensor stored as two halves lies one
-        // region further, that of a whole tensor half its size further
-        const auto halved = [&](mlel_tensor &v, const TensorDescriptor *t) {
-            v.dims[0] = splitBatch / 2;
-            const size_t step = splitInterior.count(t) ? splitHalfRegion : static_cast<size_t>(v.dims[0] * v.strides[0]);
-            v.ptr = static_cast<char *>(v.ptr) + static_cast<size_t>(half) * step;
-        };
         std::vector<size_t> act;
         if (!batchOperands(op, act)) fail(op.tosaName + " (" + op.debugName + "): not an operator of the split run");
         for (const size_t i : act) halved(in[i], op.inputs[i].get());
@@ -2039,6 +2088,23 @@ void GraphPipeline::run(const OpNode &op, void *stream, const int half) {
         const mlel_epilogue e2 = makeEpilogue(op.epilogue, &m2, &s2, op.hasClamp, op.clamp);
         rc = mlel_hip_conv2d_dwconv_rescale_clamp(ctx, stream, &out, &in[0], &in[1], &in[2], &op.convFirst, &e1, &in[3],
                                                   &in[4], &op.conv, &e2);
+        break;
+    }
+    case OpKind::FusedConv2DConv2D: {
+        const mlel_tensor m1 = op.scaleA.multiplier->view(), s1 = op.scaleA.shift->view();
+        const mlel_tensor m2 = op.epilogue.multiplier->view(), s2 = op.epilogue.shift->view();
+        const mlel_epilogue e1 = makeEpilogue(op.scaleA, &m1, &s1, op.hasClampFirst, op.clampFirst);
+        const mlel_epilogue e2 = makeEpilogue(op.epilogue, &m2, &s2, op.hasClamp, op.clamp);
+        mlel_tensor mid{};
+        const bool keep = op.outputs.size() > 1;
+        if (keep) {
+            mid = op.outputs[1]->view();
+            if (mid.ptr == nullptr && op.outputs[1]->getShapeSize() != 0)
+                fail(op.tosaName + " (" + op.debugName + "): the intermediate tensor has no memory bound");
+            if (half >= 0) halved(mid, op.outputs[1].get());
+        }
+        rc = mlel_hip_conv2d_conv2d_rescale_clamp(ctx, stream, &out, keep ? &mid : nullptr, &in[0], &in[1], &in[2],
+                                                  &op.convFirst, &e1, &in[3], &in[4], &op.conv, &e2);
         break;
     }
     case OpKind::FusedConv2DResidual: {

@@ -98,7 +98,7 @@ enum class OpKind {
     Argmax, ArithmeticRightShift, Conv3D, TransposeConv2D, Fft2D, Rfft2D, Gather, Scatter, Resize, Reverse, Tile, Select,
     // produced by the fusion pass only
     FusedConv2D, FusedDepthwiseConv2D, FusedMatmul, FusedRescaleAddRescale, FusedMatmulBiasCast, FusedElementwise,
-    FusedConv2DResidual, FusedAttention, FusedConv2DDepthwise,
+    FusedConv2DResidual, FusedAttention, FusedConv2DDepthwise, FusedConv2DConv2D,
 };
 
 struct RescaleSpec {
@@ -153,6 +153,9 @@ class OpNode {
     // FusedConv2DDepthwise: inputs = {x, the 1x1 convolution's weights and bias, the depthwise weights and bias};
     // conv / epilogue / hasClamp / clamp belong to the depthwise stage, convFirst / scaleA / hasClampFirst /
     // clampFirst to the 1x1 convolution in front of it
+    // FusedConv2DConv2D: two 1x1 convolutions in a row; inputs = {x, the first convolution's weights and bias, the
+    // second's}; conv / epilogue / hasClamp / clamp belong to the second, convFirst / scaleA / hasClampFirst / clampFirst
+    // to the first; outputs[1], when present, is the first convolution's result, which a later operator reads too
     mlel_conv2d_attr convFirst{};
     mlel_clamp_attr clampFirst{};
     bool hasClampFirst = false;

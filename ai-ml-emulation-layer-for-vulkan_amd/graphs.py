@@ -488,6 +488,20 @@ def launch_layers(g, spec):
                         "stride": dw["stride"], "macs": conv["macs"] + dw["macs"],
                         "bytes": conv["bytes"] + dw["bytes"] - 2 * mid, "layers": [at, at + 1]})
             at += 2
+        elif name.startswith("CONV2D") and name.count("CONV2D") == 2:
+            # a projection and the expansion behind it: the intermediate tensor is neither written nor read, or, with
+            # "+KEEP", written once for a later reader
+            if at + 1 >= len(spec.layers):
+                return None
+            c1, c2 = spec.layers[at], spec.layers[at + 1]
+            if c1["kind"] != "conv" or c2["kind"] != "conv":
+                return None
+            mid = int(np.prod(c1["out"]))
+            kept = "+KEEP" in name
+            out.append({"kind": "conv+conv", "in": c1["in"], "out": c2["out"], "kernel": 1, "stride": 1,
+                        "macs": c1["macs"] + c2["macs"], "bytes": c1["bytes"] + c2["bytes"] - (mid if kept else 2 * mid),
+                        "layers": [at, at + 1]})
+            at += 2
         else:
             out.append(dict(spec.layers[at], layers=[at]))
             at += 1
@@ -537,7 +551,7 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True, in_flig
                            "gbs": round(layer["bytes"] / (ms * 1e-3) / 1e9, 1)})
         # a launch that holds a CONV2D or MATMUL (also the expansion + depthwise pairs) is priced against the matrix
         # cores, a stand-alone DEPTHWISE_CONV2D or AVG_POOL2D against HBM
-        dense = [(l, launches[l["index"]]) for l in layers if l["kind"] in ("conv", "fc", "conv+dw")]
+        dense = [(l, launches[l["index"]]) for l in layers if l["kind"] in ("conv", "fc", "conv+dw", "conv+conv")]
         band = [(l, launches[l["index"]]) for l in layers if l["kind"] in ("dw", "avgpool")]
 
         def total(group, key):

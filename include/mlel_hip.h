@@ -544,6 +544,25 @@ int mlel_hip_conv2d_dwconv_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel
                                          const mlel_tensor *w1, const mlel_tensor *b1, const mlel_conv2d_attr *a1,
                                          const mlel_epilogue *e1, const mlel_tensor *w2, const mlel_tensor *b2,
                                          const mlel_conv2d_attr *a2, const mlel_epilogue *e2);
+/* out(int8) = CLAMP?(RESCALE(CONV2D( CLAMP?(RESCALE(CONV2D(in, w1, b1))), w2, b2 ))): two 1x1 convolutions in a row
+ * (unit stride, no padding), the projection of one inverted-residual block and the expansion of the next, in one
+ * launch: a wavefront requantises 32 positions of the first operator into shared memory and reads them back as the
+ * second product's row operand.  `mid` (may be NULL): the intermediate tensor [N, H, W, OC1] when another operator
+ * reads it too -- it is then stored as well; with NULL it never reaches memory.  Byte for byte
+ * mlel_hip_conv2d_rescale_clamp twice.  One pass for int8, IC a multiple of 16, OC1 a multiple of 8 up to 32, OC2 a
+ * multiple of 16 up to 192, zero weight zero points, dense operands (the shapes of
+ * mlel_hip_conv2d_conv2d_in_kernel); anything else runs the two fused operators one after the other, through `mid`
+ * or, with NULL, through a temporary (which allocates and synchronises: MLEL_ERR_UNSUPPORTED on a capturing stream).
+ * Replaces two pairs of the reference's dispatches (conv2d.comp + rescale.comp [+ clamp.comp], twice). */
+int mlel_hip_conv2d_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *mid,
+                                         const mlel_tensor *in, const mlel_tensor *w1, const mlel_tensor *b1,
+                                         const mlel_conv2d_attr *a1, const mlel_epilogue *e1, const mlel_tensor *w2,
+                                         const mlel_tensor *b2, const mlel_conv2d_attr *a2, const mlel_epilogue *e2);
+/* 1 when mlel_hip_conv2d_conv2d_rescale_clamp runs these operands in one pass, judged by types, extents, strides and
+ * attributes only (data pointers are not looked at; no device is touched), else 0. */
+int mlel_hip_conv2d_conv2d_in_kernel(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w1,
+                                     const mlel_tensor *b1, const mlel_conv2d_attr *a1, const mlel_tensor *w2,
+                                     const mlel_tensor *b2, const mlel_conv2d_attr *a2);
 /* 1 when mlel_hip_conv2d_dwconv_rescale_clamp takes these operands, judged by types, extents, strides and attributes
  * only (data pointers are not looked at; no device is touched), else 0. */
 int mlel_hip_conv2d_dwconv_in_kernel(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w1,

@@ -250,6 +250,21 @@ class Runner:
         self.done()
         return covered, r
 
+    def conv2d_conv2d(self, x, w1, b1, attr1, epi1, w2, b2, attr2, epi2, out_shape, keep_mid=False):
+        """(covered by the one-pass kernel?, output, intermediate tensor or None)"""
+        tx, tw1, tb1, tw2, tb2 = self.put(x), self.put(w1), self.put(b1), self.put(w2), self.put(b2)
+        to = self.new(abi.I8, out_shape)
+        tm = self.new(abi.I8, tuple(x.shape[:3]) + (w1.shape[0],)) if keep_mid else None
+        e1, e2 = self._epi(*epi1), self._epi(*epi2)
+        covered = self.dev.lib.mlel_hip_conv2d_conv2d_in_kernel(to.ref, tx.ref, tw1.ref, tb1.ref, C.byref(attr1),
+                                                                tw2.ref, tb2.ref, C.byref(attr2))
+        self.dev.op("conv2d_conv2d_rescale_clamp", to.ref, tm.ref if keep_mid else None, tx.ref, tw1.ref, tb1.ref,
+                    C.byref(attr1), C.byref(e1), tw2.ref, tb2.ref, C.byref(attr2), C.byref(e2))
+        r = to.download()
+        m = tm.download() if keep_mid else None
+        self.done()
+        return covered, r, m
+
     def softmax_rows(self, x):
         tx = self.put(x)
         to = self.new(tx.dtype, x.shape)

@@ -1346,6 +1346,50 @@ def test_matmul_i8_split_k_vs_oracle(run, oracle, case):
         np.testing.assert_array_equal(run.matmul(a, b, abi.I8, za, zb, epilogue=(mult, shift, rattr, None)), exp8)
 
 
+PAIR_CASES = [
+    # name, (N, H, W), IC, OC1, OC2, one pass expected
+    ("mnv2_32_16_96", (2, 12, 16), 32, 16, 96, True),
+    ("mnv2_96_24_144", (1, 10, 16), 96, 24, 144, True),
+    ("wide_32_32_192", (3, 4, 8), 32, 32, 192, True),
+    ("wide_96_32_192", (1, 6, 16), 96, 32, 192, True),
+    ("ragged_rows_32_16_96", (1, 5, 7), 32, 16, 96, True),       # 35 positions: a partial last group
+    ("ragged_rows_96_24_144", (1, 5, 6), 96, 24, 144, True),
+    ("odd_extent_96_24_144", (1, 5, 7), 96, 24, 144, True),       # 35 x 24 bytes: not whole 16-byte pieces, two launches
+    ("not_instantiated_64_16_96", (1, 4, 8), 64, 16, 96, False),  # runs as the two fused operators
+    ("odd_channels_32_12_96", (1, 4, 8), 32, 12, 96, False),
+]
+
+
+@pytest.mark.parametrize("case", PAIR_CASES, ids=[c[0] for c in PAIR_CASES])
+def test_conv2d_conv2d_pair_vs_oracle(run, oracle, case):
+    """mlel_hip_conv2d_conv2d_rescale_clamp: a 1x1 projection and the 1x1 expansion behind it in one launch, with and
+    without the intermediate tensor stored, against the oracle running CONV2D, RESCALE, CLAMP twice; shapes outside
+    the one-pass kernel give the same bytes through the two fused operators."""
+    name, nhw, ic, oc1, oc2, one_pass = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    n, h, w = nhw
+    x = ri(rng, -128, 127, (n, h, w, ic), np.int8)
+    w1 = ri(rng, -127, 127, (oc1, 1, 1, ic), np.int8)
+    b1 = ri(rng, -2 ** 15, 2 ** 15, (oc1,), np.int32)
+    w2 = ri(rng, -127, 127, (oc2, 1, 1, oc1), np.int8)
+    b2 = ri(rng, -2 ** 15, 2 ** 15, (oc2,), np.int32)
+    m1, s1 = rescale_params(rng, oc1)
+    m2, s2 = rescale_params(rng, oc2)
+    a1 = abi.conv2d_attr((0, 0, 0, 0), (1, 1), (1, 1), -5, 0)
+    a2 = abi.conv2d_attr((0, 0, 0, 0), (1, 1), (1, 1), 7, 0)
+    r1, r2 = abi.rescale_attr(0, 7, True, True, True), abi.rescale_attr(0, -128, True, True, True)
+    mid = oracle.rescale(oracle.conv2d(x, w1, b1, (n, h, w, oc1), abi.I32, a1), m1, s1, abi.I8, r1)
+    exp = oracle.clamp(oracle.rescale(oracle.conv2d(mid, w2, b2, (n, h, w, oc2), abi.I32, a2), m2, s2, abi.I8, r2), -128, 60)
+    for keep in (False, True):
+        covered, got, got_mid = run.conv2d_conv2d(x, w1, b1, a1, (m1, s1, r1, None), w2, b2, a2, (m2, s2, r2, (-128, 60)),
+                                                  (n, h, w, oc2), keep_mid=keep)
+        ragged = (n * h * w * oc1) % 16 != 0
+        assert bool(covered) == (one_pass and not ragged), name
+        np.testing.assert_array_equal(got, exp, err_msg=f"{name}, intermediate stored: {keep}")
+        if keep:
+            np.testing.assert_array_equal(got_mid, mid, err_msg=name)
+
+
 def test_copy_kernels_move_exactly_the_requested_bytes(run):
     """mlel_hip_copy_kernel (ragged length: whole pieces by the one-pass kernel, the tail bytewise) and every mode of
     mlel_hip_copy_kernel_variant leave the destination equal to the source over the requested bytes and untouched
