@@ -469,8 +469,13 @@ def bench_extra(dev, abi, reps=50):
     tx = dev.from_numpy(x)
     held = [tx]
 
-    def new(shape, dtype=abi.I8):
-        t = dev.tensor(dtype, shape)
+    def new(shape, dtype=abi.I8, loose=False):
+        # loose: 64 bytes between the batch elements, which sends the operator to the one-thread-per-element kernel
+        strides = None
+        if loose:
+            strides = list(abi.packed_strides(shape, abi.DTYPE_SIZE[dtype]))
+            strides[0] += 64
+        t = dev.tensor(dtype, shape, strides)
         held.append(t)
         return t
 
@@ -492,20 +497,28 @@ def bench_extra(dev, abi, reps=50):
     held += [vals, idx]
     o_gather = new((n, h * w, c))
     size = x.size
+    l_slice, l_cat, l_pad = new(o_slice.shape, loose=True), new(o_cat.shape, loose=True), new(o_pad.shape, loose=True)
+    l_tile, l_rev, l_gather = new(o_tile.shape, loose=True), new(o_rev.shape, loose=True), new(o_gather.shape, loose=True)
     cases = [
-        ("SLICE crop of one pixel all round", o_slice.nbytes * 2, lambda: dev.op("slice", o_slice.ref, tx.ref, start)),
+        ("SLICE crop of one pixel all round", o_slice.nbytes * 2,
+         lambda o=o_slice: dev.op("slice", o.ref, tx.ref, start), l_slice),
         ("CONCAT of two halves along the channels", size * 2,
-         lambda: (dev.op("concat", o_cat.ref, half.ref, 3, 0), dev.op("concat", o_cat.ref, half.ref, 3, c // 2))),
-        ("PAD of one pixel all round", size + o_pad.nbytes, lambda: dev.op("pad", o_pad.ref, tx.ref, t_pad.ref, 0.0, 0)),
-        ("TILE of the batch, twice", size // 2 + size, lambda: dev.op("tile", o_tile.ref, small.ref)),
-        ("REVERSE along the width", size * 2, lambda: dev.op("reverse", o_rev.ref, tx.ref, 2)),
-        ("GATHER of every pixel row, permuted", size * 2 + idx.nbytes, lambda: dev.op("gather", o_gather.ref, vals.ref, idx.ref)),
+         lambda o=o_cat: (dev.op("concat", o.ref, half.ref, 3, 0), dev.op("concat", o.ref, half.ref, 3, c // 2)), l_cat),
+        ("PAD of one pixel all round", size + o_pad.nbytes,
+         lambda o=o_pad: dev.op("pad", o.ref, tx.ref, t_pad.ref, 0.0, 0), l_pad),
+        ("TILE of the batch, twice", size // 2 + size, lambda o=o_tile: dev.op("tile", o.ref, small.ref), l_tile),
+        ("REVERSE along the width", size * 2, lambda o=o_rev: dev.op("reverse", o.ref, tx.ref, 2), l_rev),
+        ("GATHER of every pixel row, permuted", size * 2 + idx.nbytes,
+         lambda o=o_gather: dev.op("gather", o.ref, vals.ref, idx.ref), l_gather),
     ]
     out = []
-    for name, nbytes, fn in cases:
+    for name, nbytes, fn, loose in cases:
         us = _median_us(dev, fn, reps, rounds=5, warm=3)
+        # the same operator into an output whose batch elements lie 64 bytes apart: the element-wise kernel takes it
+        us_elem = _median_us(dev, lambda: fn(loose), max(reps // 5, 3), rounds=3, warm=1)
         out.append({"operator": name, "shape": [n, h, w, c], "us": round(us, 2), "algorithmic_bytes": int(nbytes),
-                    "gbs": round(nbytes / (us * 1e-6) / 1e9, 1), "hbm_frac": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+                    "gbs": round(nbytes / (us * 1e-6) / 1e9, 1), "hbm_frac": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                    "us_one_thread_per_element": round(us_elem, 2)})
     for t in held:
         t.free()
     return out
@@ -523,6 +536,7 @@ def main():
     ap.add_argument("--only", choices=["all", "config0", "config1", "config2", "mobilenetv2", "encoder", "gemm_large",
                                        "layer", "standalone", "copy", "extra"], default="all")
     ap.add_argument("--layer", type=int, default=3, help="with --only layer: position in the fused config 3 graph")
+    ap.add_argument("--gemm-size", type=int, default=0, help="with --only gemm_large: this one size instead of 4096 and 8192")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -577,7 +591,8 @@ def main():
         extra.update(graphs.bench_inverted_residual(dev, steps=graph_steps, warmup=max(3, args.warmup // 10)))
         log("config 2:", extra["config2_inverted_residual_b16"])
     if want("gemm_large"):
-        extra["gemm_large"] = bench_gemm_large(dev, abi, check=not args.skip_cpu)
+        extra["gemm_large"] = bench_gemm_large(dev, abi, sizes=(args.gemm_size,) if args.gemm_size > 0 else (4096, 8192),
+                                               check=not args.skip_cpu)
         log("large products:", extra["gemm_large"])
     if want("mobilenetv2") and not args.skip_graph:
         try:
