@@ -354,7 +354,7 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
         }
         v4i v;
         v.x = (int)piece.x, v.y = (int)piece.y, v.z = (int)piece.z, v.w = (int)piece.w;
-        __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, kOutAux);
     }
 }
 

@@ -14,6 +14,24 @@
 
 namespace mlel {
 
+// Cache policy of the stores that write an operator's result: sc0 | sc1 (write-through).  A result is read next by
+// another launch, usually under another XCD's L2, so keeping it dirty in this one only moves its write-back to the
+// end of the kernel, where nothing overlaps it.
+#ifndef MLEL_OUT_AUX
+#define MLEL_OUT_AUX 17
+#endif
+constexpr int kOutAux = MLEL_OUT_AUX;
+// The same policy for a 16-byte result store through a plain pointer.
+__device__ __forceinline__ void store16_result(void *p, uint4 v) {
+    typedef unsigned int u32x4_st __attribute__((ext_vector_type(4)));
+    const u32x4_st d = {v.x, v.y, v.z, v.w};
+    if (kOutAux == 17)
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(d) : "memory");
+    else
+        *reinterpret_cast<uint4 *>(p) = v;
+}
+
+
 // ---------------------------------------------------------------------------------------------------------------
 // errors
 // ---------------------------------------------------------------------------------------------------------------

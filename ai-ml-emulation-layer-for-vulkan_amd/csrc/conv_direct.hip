@@ -403,7 +403,7 @@ __global__ void __launch_bounds__(kBlock) conv_rows_mfma_i8_kernel(const RowsMfm
             if (t < rounds) {  // uniform
                 const uint4 d = *reinterpret_cast<const uint4 *>(so + (t * 64 + lane) * 16);
                 const uint32_t off = piece_row[t] < rows ? obase + piece_out[t] : kOob;
-                __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, kOutAux);
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -621,7 +621,7 @@ conv_rows2_mfma_i8_kernel(const Rows2Args b) {
         if (b.mid != nullptr && lane < mid_pieces) {  // the intermediate tensor's 32 rows are consecutive in memory
             const uint4 d = *reinterpret_cast<const uint4 *>(mt + lane * 16);
             const uint32_t off = (uint32_t)(lane * 16) < rows * (uint32_t)OC0 ? (uint32_t)g * 32u * (uint32_t)OC0 + (uint32_t)lane * 16u : kOob;
-            __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, mres, (int)off, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, mres, (int)off, 0, kOutAux);
         }
         long xf[KC];
 #pragma unroll
@@ -662,7 +662,7 @@ conv_rows2_mfma_i8_kernel(const Rows2Args b) {
             if (t < rounds) {  // uniform
                 const uint4 d = *reinterpret_cast<const uint4 *>(so + (t * 64 + lane) * 16);
                 const uint32_t off = piece_row[t] < rows ? obase + piece_out[t] : kOob;
-                __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, kOutAux);
             }
         }
         wave_sync();
@@ -863,7 +863,7 @@ __global__ void __launch_bounds__(kBlock) conv_stem_mfma_i8_kernel(const StemMfm
         const uint32_t rows = (uint32_t)min(32, a.M - g * 32);
         const uint4 d = *reinterpret_cast<const uint4 *>(so + piece_lds);
         const uint32_t off = piece_row < rows ? (uint32_t)g * 32u * (uint32_t)a.OC + (uint32_t)lane * 16u : kOob;
-        __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, kOutAux);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");

@@ -267,7 +267,7 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
                 const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
                 const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
                 const uint32_t off = (orow + (uint32_t)ox) * (uint32_t)a.C + c;
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_amdgcn_perm(hi, lo, 0x05040100u), ores, (int)off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_amdgcn_perm(hi, lo, 0x05040100u), ores, (int)off, 0, kOutAux);
             }
         }
     }

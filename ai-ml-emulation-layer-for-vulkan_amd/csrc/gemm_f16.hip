@@ -459,7 +459,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
                                      ((uint32_t)n - n1 * (uint32_t)o.v_n2) * o.vs_n2;
                 v4i v;
                 v.x = (int)w[0], v.y = (int)w[1], v.z = (int)w[2], v.w = (int)w[3];
-                __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, kOutAux);
             }
             return;
         }
@@ -496,7 +496,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
             }
             v4i v;
             v.x = (int)piece.x, v.y = (int)piece.y, v.z = (int)piece.z, v.w = (int)piece.w;
-            __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, kOutAux);
         }
         return;
     }
@@ -515,7 +515,7 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
                 v.y = __float_as_int(acc[i][j][4 * q + 1]);
                 v.z = __float_as_int(acc[i][j][4 * q + 2]);
                 v.w = __float_as_int(acc[i][j][4 * q + 3]);
-                __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(v, ores, (int)off, 0, kOutAux);
             }
         }
     }

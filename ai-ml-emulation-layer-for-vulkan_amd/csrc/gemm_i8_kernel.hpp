@@ -1042,7 +1042,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                 d = make_uint4(w[0], w[1], w[2], w[3]);
             }
             if (whole) {
-                __builtin_amdgcn_raw_buffer_store_b128(v4i{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(v4i{(int)d.x, (int)d.y, (int)d.z, (int)d.w}, ores, (int)off, 0, kOutAux);
             } else if (off != kOobOffset) {  // the last channels of a row whose extent is not a multiple of 16
                 const uint32_t w[4] = {d.x, d.y, d.z, d.w};
 #pragma unroll

@@ -57,7 +57,7 @@ __global__ void __launch_bounds__(kBlock) rescale_add_rescale_i8x16_kernel(uint4
         }
         ov[d] = packed;
     }
-    out[i] = make_uint4(ov[0], ov[1], ov[2], ov[3]);
+    store16_result(out + i, make_uint4(ov[0], ov[1], ov[2], ov[3]));
 }
 
 }  // namespace
@@ -285,7 +285,7 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
             if (Q8 || a.out_size == 1) {
                 const uint32_t packed = ((uint32_t)v[0] & 0xffu) | (((uint32_t)v[1] & 0xffu) << 8) |
                                         (((uint32_t)v[2] & 0xffu) << 16) | ((uint32_t)v[3] << 24);
-                __builtin_amdgcn_raw_buffer_store_b32(packed, ores, (int)off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(packed, ores, (int)off, 0, kOutAux);
             } else if (a.out_size == 2) {
                 __builtin_amdgcn_raw_buffer_store_b32((uint32_t)(uint16_t)v[0] | ((uint32_t)(uint16_t)v[1] << 16), ores, (int)off, 0, 0);
                 __builtin_amdgcn_raw_buffer_store_b32((uint32_t)(uint16_t)v[2] | ((uint32_t)(uint16_t)v[3] << 16), ores, (int)off + 4, 0, 0);

@@ -372,7 +372,7 @@ __global__ void __launch_bounds__(kBlock) ew_static_half_kernel(const StaticArgs
         }
     }
     static_run<P, 0>(val);
-    *reinterpret_cast<uint4 *>(g.out + v * 16) = val[P::n_inputs + P::n_steps - 1];
+    store16_result(g.out + v * 16, val[P::n_inputs + P::n_steps - 1]);
 }
 
 // the chain is P's program over inputs of P's shapes
@@ -1215,7 +1215,7 @@ __device__ __forceinline__ void row_static_run(RowStaticState<P> &c) {
                 if constexpr (last) {
                     const int sg = c.part + u * c.tpr;
                     if (c.live && sg < c.segs)
-                        *reinterpret_cast<uint4 *>(c.g->out + (c.row * c.g->cols + sg * 8) * 2) = r;
+                        store16_result(c.g->out + (c.row * c.g->cols + sg * 8) * 2, r);
                 } else {
                     c.f[P::slot[V]][u] = r;
                 }

@@ -317,7 +317,7 @@ __global__ void __launch_bounds__(kBlock) maxpool_i8_kernel(const MaxPoolArgs a)
     const uint32_t ooff = (((uint32_t)row * (uint32_t)a.OW + ox) * (uint32_t)a.groups + cg) * (4u * V);
     if constexpr (V == 4) {
         typedef int v4i32 __attribute__((ext_vector_type(4)));
-        __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)r[0], (int)r[1], (int)r[2], (int)r[3]}, ores, (int)ooff, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(v4i32{(int)r[0], (int)r[1], (int)r[2], (int)r[3]}, ores, (int)ooff, 0, kOutAux);
     } else {
         __builtin_amdgcn_raw_buffer_store_b32(r[0], ores, (int)ooff, 0, 0);
     }
