@@ -37,7 +37,7 @@ __device__ __forceinline__ int32_t lds_entry(const int32_t *table, uint32_t w, i
 
 // KS == 1: a wavefront per tile.  KS == 4 (few tiles): the four wavefronts of a block share a tile, each takes a
 // quarter of the K chunks, the partial tiles are added through shared memory (int32 addition wraps: the order is
-// immaterial) and the first wavefront requantises.
+// immaterial) and each wavefront requantises and stores a quarter of the tile (eight of its 32 positions).
 template <bool RES, int KS>
 __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const GemmArgs g, int groups_n, int total_waves) {
     const int tid = threadIdx.x, lane = tid & 63;
@@ -79,12 +79,15 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
     char *ob = g.out;
     const __amdgpu_buffer_rsrc_t ores = make_rsrc(ob, g.o_bytes);
     const __amdgpu_buffer_rsrc_t rres = make_rsrc(RES ? reinterpret_cast<const char *>(g.res) : ob, g.o_bytes);
-    uint32_t d_off[4], d_res[RES ? 4 : 1];
+    // KS == 4: the four wavefronts share the epilogue as well, wavefront w takes register group q = w
+    constexpr int NQ = KS == 1 ? 4 : 1;
+    uint32_t d_off[NQ], d_res[RES ? NQ : 1];
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
+    for (int i = 0; i < NQ; i++) {
+        const int q = KS == 1 ? i : wave;
         const int pm = mg * 32 + 8 * q + 4 * half + (lane & 3), pn = ng * 32 + (cl & ~3);
-        d_off[q] = (pm < g.M && pn < g.N) ? (uint32_t)pm * (uint32_t)g.ldo + (uint32_t)pn : kOobOffset;
-        if constexpr (RES) d_res[q] = buf_load4(rres, d_off[q]);
+        d_off[i] = (pm < g.M && pn < g.N) ? (uint32_t)pm * (uint32_t)g.ldo + (uint32_t)pn : kOobOffset;
+        if constexpr (RES) d_res[i] = buf_load4(rres, d_off[i]);
     }
     // ---- this lane's channel: bias, requantisation constants
     int32_t bias = 0, mult = 0, shift = 0;
@@ -133,21 +136,29 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
             multiply(xb, wb);
         }
     }
+    int32_t own[4 * NQ];  // the accumulators this wavefront requantises
     if constexpr (KS > 1) {
-        __shared__ int32_t part[KS - 1][17][64];  // [wavefront][register, then the weight sum][lane]
-        if (wave > 0) {
+        // every wavefront leaves its partial tile in shared memory and picks up, summed over the four, the register
+        // group it requantises (int32 addition wraps: the order is immaterial) and the weight sum
+        __shared__ int32_t part[KS][17][64];  // [wavefront][register, then the weight sum][lane]
 #pragma unroll
-            for (int r = 0; r < 16; r++) part[wave - 1][r][lane] = acc[r];
-            part[wave - 1][16][lane] = wsum;
-        }
+        for (int r = 0; r < 16; r++) part[wave][r][lane] = acc[r];
+        part[wave][16][lane] = wsum;
         __syncthreads();
-        if (wave > 0) return;
 #pragma unroll
-        for (int o = 0; o < KS - 1; o++) {
+        for (int e = 0; e < 4; e++) {
+            uint32_t t = 0;
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[r] = (int32_t)((uint32_t)acc[r] + (uint32_t)part[o][r][lane]);
-            wsum = (int32_t)((uint32_t)wsum + (uint32_t)part[o][16][lane]);
+            for (int o = 0; o < KS; o++) t += (uint32_t)part[o][4 * wave + e][lane];
+            own[e] = (int32_t)t;
         }
+        uint32_t t = 0;
+#pragma unroll
+        for (int o = 0; o < KS; o++) t += (uint32_t)part[o][16][lane];
+        wsum = (int32_t)t;
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) own[r] = acc[r];
     }
 
     // ---- epilogue: the channel's constants are registers; a 4 x 4 byte transpose inside lane quads turns four
@@ -158,10 +169,10 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
     const uint32_t sel_a = (lane & 1) ? 0x03070105u : 0x06020400u;  // exchange with lane ^ 1
     const uint32_t sel_b = (lane & 2) ? 0x03020706u : 0x05040100u;  // exchange with lane ^ 2
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
+    for (int q = 0; q < NQ; q++) {
         int32_t v[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) v[e] = requant_acc((int32_t)((uint32_t)acc[4 * q + e] + (uint32_t)bias_adj), cs, g.rp);
+        for (int e = 0; e < 4; e++) v[e] = requant_acc((int32_t)((uint32_t)own[4 * q + e] + (uint32_t)bias_adj), cs, g.rp);
         const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
         const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
         uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
