@@ -143,6 +143,27 @@ __device__ __forceinline__ void transpose_3x4(uint32_t r0, uint32_t r1, uint32_t
     col[3] = __builtin_amdgcn_perm(r2, t1, 0x0c070302u);             // [t1.b2 t1.b3 r2.b3 0]
 }
 
+// 4 rows x 4 channels (bytes) -> 4 channels x 4 vertical taps: output row 0 multiplies the column by the weights
+// (w0, w1, w2, 0), output row 1 by (0, w0, w1, w2), so one transpose serves both rows of a work item
+__device__ __forceinline__ void transpose_4x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, uint32_t (&col)[4]) {
+    const uint32_t t0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);  // [r0.b0 r1.b0 r0.b1 r1.b1]
+    const uint32_t t1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);  // [r0.b2 r1.b2 r0.b3 r1.b3]
+    const uint32_t u0 = __builtin_amdgcn_perm(r3, r2, 0x05010400u);  // [r2.b0 r3.b0 r2.b1 r3.b1]
+    const uint32_t u1 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+    col[0] = __builtin_amdgcn_perm(u0, t0, 0x05040100u);             // [t0.b0 t0.b1 u0.b0 u0.b1]
+    col[1] = __builtin_amdgcn_perm(u0, t0, 0x07060302u);
+    col[2] = __builtin_amdgcn_perm(u1, t1, 0x05040100u);
+    col[3] = __builtin_amdgcn_perm(u1, t1, 0x07060302u);
+}
+
+// d = dot4(a, b) + c with c in a register of its own: the first tap of an output starts from the bias term without
+// a copy of it into the accumulator (the two-operand form the compiler prefers accumulates in place)
+__device__ __forceinline__ int32_t dot4_from(uint32_t a, uint32_t b, int32_t c) {
+    int32_t d;
+    asm("v_dot4_i32_i8 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+
 // Q8: fused epilogue with 8-bit output (a compile-time choice keeps the unrolled epilogue free of branches).  All
 // index arithmetic is 32-bit (the host checks the extents); loads and stores are buffer instructions with 32-bit
 // offsets, so an address costs one add.
@@ -215,16 +236,13 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
     // offsets of taps outside the image wrap to values beyond the extent (such loads return 0) or name another
     // pixel; either way the value is replaced by the zero point below
     const uint32_t xbase = (uint32_t)n * a.x_sn + (uint32_t)c + (uint32_t)iy0 * a.x_sy + (uint32_t)ix0 * a.x_sx;
-    int32_t acc[TY][TX][4], xs[TY][TX][4];
+    int32_t acc[TY][TX][4], xs[TY][TX][4];  // tap kx == 0 of an output starts its accumulator from the bias term
 #pragma unroll
     for (int ty = 0; ty < TY; ty++)
 #pragma unroll
         for (int t = 0; t < TX; t++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                acc[ty][t][e] = bias_adj[e];  // the dot products accumulate on top of the bias term
-                xs[ty][t][e] = 0;
-            }
+            for (int e = 0; e < 4; e++) xs[ty][t][e] = 0;
 
     constexpr int NROW_MAX = SX * (TY - 1) + 3;
     uint32_t raw[NROW_MAX][NCOL];
@@ -242,20 +260,56 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
             raw[r][j] = (yin && xin[j]) ? v : zsplat;
         }
     }
+    if constexpr (TY == 2 && SX == 1) {
+        // both output rows from one 4 x 4 transpose per column: row 1 uses the weights one byte up
+        uint32_t wc1[3][4];
 #pragma unroll
-    for (int ty = 0; ty < TY; ty++) {
+        for (int kx = 0; kx < 3; kx++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) wc1[kx][e] = wc[kx][e] << 8;
 #pragma unroll
         for (int j = 0; j < NCOL; j++) {
             uint32_t col[4];
-            transpose_3x4(raw[ty * SX][j], raw[ty * SX + 1][j], raw[ty * SX + 2][j], col);
+            transpose_4x4(raw[0][j], raw[1][j], raw[2][j], raw[3][j], col);
 #pragma unroll
             for (int t = 0; t < TX; t++) {
-                const int kx = j - t * SX;  // this column is tap kx of output t (compile-time after unrolling)
+                const int kx = j - t;
                 if (kx < 0 || kx > 2) continue;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    acc[ty][t][e] = __builtin_amdgcn_sdot4((int)col[e], (int)wc[kx][e], acc[ty][t][e], false);
-                    if (ZW) xs[ty][t][e] = __builtin_amdgcn_sdot4((int)col[e], 0x00010101, xs[ty][t][e], false);
+                    if (kx == 0) {
+                        acc[0][t][e] = dot4_from(col[e], wc[0][e], bias_adj[e]);
+                        acc[1][t][e] = dot4_from(col[e], wc1[0][e], bias_adj[e]);
+                    } else {
+                        acc[0][t][e] = __builtin_amdgcn_sdot4((int)col[e], (int)wc[kx][e], acc[0][t][e], false);
+                        acc[1][t][e] = __builtin_amdgcn_sdot4((int)col[e], (int)wc1[kx][e], acc[1][t][e], false);
+                    }
+                    if (ZW) {
+                        xs[0][t][e] = __builtin_amdgcn_sdot4((int)col[e], 0x00010101, xs[0][t][e], false);
+                        xs[1][t][e] = __builtin_amdgcn_sdot4((int)col[e], 0x01010100, xs[1][t][e], false);
+                    }
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int ty = 0; ty < TY; ty++) {
+#pragma unroll
+            for (int j = 0; j < NCOL; j++) {
+                uint32_t col[4];
+                transpose_3x4(raw[ty * SX][j], raw[ty * SX + 1][j], raw[ty * SX + 2][j], col);
+#pragma unroll
+                for (int t = 0; t < TX; t++) {
+                    const int kx = j - t * SX;  // this column is tap kx of output t (compile-time after unrolling)
+                    if (kx < 0 || kx > 2) continue;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (kx == 0)
+                            acc[ty][t][e] = dot4_from(col[e], wc[0][e], bias_adj[e]);
+                        else
+                            acc[ty][t][e] = __builtin_amdgcn_sdot4((int)col[e], (int)wc[kx][e], acc[ty][t][e], false);
+                        if (ZW) xs[ty][t][e] = __builtin_amdgcn_sdot4((int)col[e], 0x00010101, xs[ty][t][e], false);
+                    }
                 }
             }
         }
@@ -283,8 +337,10 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
             }
             const uint32_t off = ((orow + (uint32_t)ox) * (uint32_t)a.C + (uint32_t)c) * esz;
             if (Q8 || a.out_size == 1) {
-                const uint32_t packed = ((uint32_t)v[0] & 0xffu) | (((uint32_t)v[1] & 0xffu) << 8) |
-                                        (((uint32_t)v[2] & 0xffu) << 16) | ((uint32_t)v[3] << 24);
+                // the low bytes of the four results, by three byte permutes
+                const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
+                const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
+                const uint32_t packed = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
                 __builtin_amdgcn_raw_buffer_store_b32(packed, ores, (int)off, 0, kOutAux);
             } else if (a.out_size == 2) {
                 __builtin_amdgcn_raw_buffer_store_b32((uint32_t)(uint16_t)v[0] | ((uint32_t)(uint16_t)v[1] << 16), ores, (int)off, 0, 0);
