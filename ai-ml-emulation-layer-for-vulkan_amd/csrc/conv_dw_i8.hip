@@ -215,6 +215,11 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
         q2[e] = d.q;
     }
     constexpr int NCOL = SX * (TX - 1) + 3, NROW = SX * (TY - 1) + 3;
+    uint32_t wc1[3][4];  // the weight columns one byte up (second output row of a 4 x 4 transpose)
+#pragma unroll
+    for (int kx = 0; kx < 3; kx++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) wc1[kx][e] = wc[kx][e] << 8;
     const uint32_t c = (uint32_t)(c0 + cq * 4);
     for (int item = tid; item < a.items; item += kBlock) {
         const uint32_t sp = (uint32_t)item >> 3;
@@ -229,26 +234,48 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
 #pragma unroll
             for (int j = 0; j < NCOL; j++) raw[r][j] = *reinterpret_cast<const uint32_t *>(rp + j * YP);
         }
-        int32_t acc[TY][TX][4];
-#pragma unroll
-        for (int ty = 0; ty < TY; ty++)
-#pragma unroll
-            for (int t = 0; t < TX; t++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) acc[ty][t][e] = bias_adj[e];
-#pragma unroll
-        for (int ty = 0; ty < TY; ty++) {
+        int32_t acc[TY][TX][4];  // tap kx == 0 of an output starts its accumulator from the bias term
+        if constexpr (TY == 2 && SX == 1) {
+            // both output rows from one 4 x 4 transpose per column: row 1 uses the weights one byte up
 #pragma unroll
             for (int j = 0; j < NCOL; j++) {
                 uint32_t col[4];
-                rows_to_taps(raw[ty * SX][j], raw[ty * SX + 1][j], raw[ty * SX + 2][j], col);
+                transpose_4x4(raw[0][j], raw[1][j], raw[2][j], raw[3][j], col);
 #pragma unroll
                 for (int t = 0; t < TX; t++) {
-                    const int kx = j - t * SX;
+                    const int kx = j - t;
                     if (kx < 0 || kx > 2) continue;
 #pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        acc[ty][t][e] = __builtin_amdgcn_sdot4((int)col[e], (int)wc[kx][e], acc[ty][t][e], false);
+                    for (int e = 0; e < 4; e++) {
+                        if (kx == 0) {
+                            acc[0][t][e] = dot4_from(col[e], wc[0][e], bias_adj[e]);
+                            acc[1][t][e] = dot4_from(col[e], wc1[0][e], bias_adj[e]);
+                        } else {
+                            acc[0][t][e] = __builtin_amdgcn_sdot4((int)col[e], (int)wc[kx][e], acc[0][t][e], false);
+                            acc[1][t][e] = __builtin_amdgcn_sdot4((int)col[e], (int)wc1[kx][e], acc[1][t][e], false);
+                        }
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int ty = 0; ty < TY; ty++) {
+#pragma unroll
+                for (int j = 0; j < NCOL; j++) {
+                    uint32_t col[4];
+                    rows_to_taps(raw[ty * SX][j], raw[ty * SX + 1][j], raw[ty * SX + 2][j], col);
+#pragma unroll
+                    for (int t = 0; t < TX; t++) {
+                        const int kx = j - t * SX;
+                        if (kx < 0 || kx > 2) continue;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            if (kx == 0)
+                                acc[ty][t][e] = dot4_from(col[e], wc[0][e], bias_adj[e]);
+                            else
+                                acc[ty][t][e] = __builtin_amdgcn_sdot4((int)col[e], (int)wc[kx][e], acc[ty][t][e], false);
+                        }
+                    }
                 }
             }
         }

@@ -143,27 +143,6 @@ __device__ __forceinline__ void transpose_3x4(uint32_t r0, uint32_t r1, uint32_t
     col[3] = __builtin_amdgcn_perm(r2, t1, 0x0c070302u);             // [t1.b2 t1.b3 r2.b3 0]
 }
 
-// 4 rows x 4 channels (bytes) -> 4 channels x 4 vertical taps: output row 0 multiplies the column by the weights
-// (w0, w1, w2, 0), output row 1 by (0, w0, w1, w2), so one transpose serves both rows of a work item
-__device__ __forceinline__ void transpose_4x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, uint32_t (&col)[4]) {
-    const uint32_t t0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);  // [r0.b0 r1.b0 r0.b1 r1.b1]
-    const uint32_t t1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);  // [r0.b2 r1.b2 r0.b3 r1.b3]
-    const uint32_t u0 = __builtin_amdgcn_perm(r3, r2, 0x05010400u);  // [r2.b0 r3.b0 r2.b1 r3.b1]
-    const uint32_t u1 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
-    col[0] = __builtin_amdgcn_perm(u0, t0, 0x05040100u);             // [t0.b0 t0.b1 u0.b0 u0.b1]
-    col[1] = __builtin_amdgcn_perm(u0, t0, 0x07060302u);
-    col[2] = __builtin_amdgcn_perm(u1, t1, 0x05040100u);
-    col[3] = __builtin_amdgcn_perm(u1, t1, 0x07060302u);
-}
-
-// d = dot4(a, b) + c with c in a register of its own: the first tap of an output starts from the bias term without
-// a copy of it into the accumulator (the two-operand form the compiler prefers accumulates in place)
-__device__ __forceinline__ int32_t dot4_from(uint32_t a, uint32_t b, int32_t c) {
-    int32_t d;
-    asm("v_dot4_i32_i8 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
-    return d;
-}
-
 // Q8: fused epilogue with 8-bit output (a compile-time choice keeps the unrolled epilogue free of branches).  All
 // index arithmetic is 32-bit (the host checks the extents); loads and stores are buffer instructions with 32-bit
 // offsets, so an address costs one add.
