@@ -102,6 +102,59 @@ mlel_tensor packed_like(const mlel_tensor *t, int dtype, void *ptr) {
     return r;
 }
 
+// CONV3D over int8 operands with an int32 result as ONE CONV2D on the matrix cores: the depth taps become channels
+// (launch_conv3d_regroup), which costs KD copies of the input in a temporary.  A kernel one slice deep without depth
+// padding needs no copy at all: its operands are CONV2D's already.  Returns 1 when done, 0 to decline.
+int try_conv3d_as_conv2d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w,
+                         const mlel_tensor *bias, const mlel_conv3d_attr *a) {
+    if (in->dtype != MLEL_I8 || w->dtype != MLEL_I8 || out->dtype != MLEL_I32 || bias->dtype != MLEL_I32 ||
+        a->acc_type != MLEL_ACC_I32)
+        return 0;
+    if (!is_packed(in) || !is_packed(w) || !is_packed(out)) return 0;
+    const int64_t N = out->dims[0], OD = out->dims[1], OH = out->dims[2], OW = out->dims[3], OC = out->dims[4];
+    const int64_t D = in->dims[1], H = in->dims[2], W = in->dims[3], IC = in->dims[4];
+    const int64_t KD = w->dims[1], KH = w->dims[2], KW = w->dims[3];
+    if (in->dims[0] != N || w->dims[0] != OC || w->dims[4] != IC || N <= 0 || OD <= 0 || OH <= 0 || OW <= 0 || OC <= 0 ||
+        IC <= 0 || KD <= 0 || KH <= 0 || KW <= 0 || D <= 0)
+        return 0;
+    if (a->stride[0] <= 0 || a->dilation[0] <= 0 || a->pad[0] < 0 || a->pad[1] < 0) return 0;
+    mlel_conv2d_attr a2{};
+    a2.input_zp = a->input_zp, a2.weight_zp = a->weight_zp, a2.acc_type = a->acc_type;
+    for (int i = 0; i < 4; i++) a2.pad[i] = a->pad[2 + i];
+    a2.stride[0] = a->stride[1], a2.stride[1] = a->stride[2];
+    a2.dilation[0] = a->dilation[1], a2.dilation[1] = a->dilation[2];
+    mlel_tensor o2{};
+    o2.dtype = MLEL_I32, o2.rank = 4, o2.ptr = out->ptr;
+    o2.dims[0] = N * OD, o2.dims[1] = OH, o2.dims[2] = OW, o2.dims[3] = OC;
+    mlel_tensor x2 = o2, w2 = o2;
+    x2.dtype = w2.dtype = MLEL_I8;
+    x2.dims[1] = H, x2.dims[2] = W, x2.dims[3] = KD * IC;
+    w2.dims[0] = OC, w2.dims[1] = KH, w2.dims[2] = KW, w2.dims[3] = KD * IC;
+    const auto pack = [](mlel_tensor &t) {
+        int64_t st = dt_size(t.dtype);
+        for (int i = t.rank - 1; i >= 0; i--) t.strides[i] = st, st *= t.dims[i];
+        return st;
+    };
+    pack(o2);
+    const int64_t x_bytes = pack(x2), w_bytes = pack(w2);
+    if (KD == 1 && a->pad[0] == 0 && a->pad[1] == 0 && a->stride[0] == 1 && OD == D) {
+        x2.ptr = in->ptr, w2.ptr = w->ptr;  // [N * D][H][W][IC] and [OC][KH][KW][IC] as they lie
+        MLEL_TRY(mlel_hip_conv2d(ctx, stream, &o2, &x2, &w2, bias, &a2));
+        return 1;
+    }
+    // the copies pay from a few million multiply-adds on; they go to the stream's staging memory (no allocation and no
+    // wait once it is large enough; when it is not and cannot grow -- a capturing stream -- the generic kernel runs)
+    const int64_t macs = N * OD * OH * OW * OC * KD * KH * KW * IC;
+    if (macs < (int64_t(1) << 22) || x_bytes >= (int64_t(1) << 31) || w_bytes >= (int64_t(1) << 31)) return 0;
+    const size_t x_room = ((size_t)x_bytes + 255) & ~size_t(255);
+    char *stage = stage_workspace(ctx, (hipStream_t)stream, x_room + (size_t)w_bytes + 256);
+    if (stage == nullptr) return 0;
+    x2.ptr = stage, w2.ptr = stage + x_room;
+    MLEL_TRY(launch_conv3d_regroup((hipStream_t)stream, x2.ptr, w2.ptr, in, w, OD, a));
+    MLEL_TRY(mlel_hip_conv2d(ctx, stream, &o2, &x2, &w2, bias, &a2));
+    return 1;
+}
+
 }  // namespace
 
 extern "C" {
@@ -405,6 +458,10 @@ int mlel_hip_conv3d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const m
                  "conv3d: ranks must be 5,5,5,1");
     MLEL_REQUIRE(attr->acc_type >= MLEL_ACC_I32 && attr->acc_type <= MLEL_ACC_I64, MLEL_ERR_INVALID,
                  "Unsupported acc type %u", attr->acc_type);
+    {
+        const int r = try_conv3d_as_conv2d(ctx, stream, out, in, weights, bias, attr);
+        if (r != 0) return r < 0 ? r : 0;
+    }
     return conv3d_launch((hipStream_t)stream, out, in, weights, bias, attr);
 }
 

@@ -475,12 +475,24 @@ constexpr size_t kSplitPartialBytes = size_t(16) << 20;
 constexpr int kSplitCounters = 4096;
 constexpr int kMaxSplitWorkspaces = 16;
 
+// Device staging memory of the operators that rearrange an operand before the kernel proper (CONV3D as CONV2D): one
+// grow-only buffer per stream that has used such an operator (the calls of one stream are ordered, so the next call may
+// overwrite it), freed with the stream or the context.
+struct StageWorkspace {
+    hipStream_t stream;
+    char *ptr;
+    size_t bytes;
+};
+constexpr size_t kMaxStageBytes = size_t(2) << 30;
+
 struct mlel_ctx {
     int device;
     hipDeviceProp_t props;
     std::mutex ws_lock;
     SplitWorkspace ws[kMaxSplitWorkspaces];
     int n_ws = 0;
+    StageWorkspace stage[kMaxSplitWorkspaces];
+    int n_stage = 0;
     int split_k = 8;  // most blocks per tile in split-K mode; 0 or 1: never split (MLEL_SPLIT_K in the environment)
     // the statically allocated scratch of the entry point that must not allocate: this device's address of the
     // array (hipGetSymbolAddress at context creation), nullptr if that failed
@@ -493,6 +505,9 @@ namespace mlel {
 // captured, table full, allocation failed): the caller then runs without splitting.
 bool split_workspace(mlel_ctx *ctx, hipStream_t stream, SplitWorkspace *out);
 void free_split_workspaces(mlel_ctx *ctx);
+// `bytes` of staging memory for `stream`, or nullptr when it cannot be had now: growing it allocates (and waits for the
+// stream, whose earlier calls may still read the old buffer), which a capturing stream cannot do.
+char *stage_workspace(mlel_ctx *ctx, hipStream_t stream, size_t bytes);
 // static_scratch.hip: the file-scope device array behind mlel_hip_conv2d_rescale_clamp_static
 constexpr size_t kStaticScratchPartialBytes = size_t(8) << 20;
 constexpr size_t kStaticScratchBytes = kStaticScratchPartialBytes + size_t(kSplitCounters) * 4;

@@ -189,5 +189,8 @@ int try_pad_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, c
 int try_tile_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in);
 int try_reverse_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis);
 int try_gather_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *values, const mlel_tensor *indices);
+// CONV3D as CONV2D (ops_move.hip): the depth taps side by side along the channels of x2, the weights regrouped to match
+int launch_conv3d_regroup(hipStream_t s, void *x2, void *w2, const mlel_tensor *in, const mlel_tensor *w, int64_t OD,
+                          const mlel_conv3d_attr *a);
 
 }  // namespace mlel

@@ -299,4 +299,118 @@ int try_gather_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *va
                        static_cast<const int32_t *>(indices->ptr));
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// CONV3D as CONV2D: the KD depth taps of an output slice are laid side by side along the channels,
+//   x2[n * OD + od][h][w][kd * IC + c] = in[n][od * sd + kd * dd - pad_front][h][w][c]   (the input zero point where
+//   that depth lies outside the tensor: such taps then contribute nothing, as in conv3d.comp:37-104),
+//   w2[oc][ky][kx][kd * IC + c] = w[oc][kd][ky][kx][c],
+// after which out[n * OD + od] = CONV2D(x2, w2) with the height / width attributes.  One thread moves one piece of
+// 16, 4 or 1 bytes of a pixel.
+// ---------------------------------------------------------------------------------------------------------------
+namespace {
+
+struct DepthGatherArgs {
+    const char *in;
+    char *x2;
+    int64_t pieces;            // N * OD * HW * KD * (IC / piece)
+    int32_t D, OD, KD, sd, dd, pad_d, piece, ppp;  // ppp: pieces per pixel (IC / piece)
+    int64_t HW, in_sn, in_sd;  // positions per slice; byte strides of the dense input: image, depth slice
+    uint32_t zsplat;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) conv3d_depth_gather_kernel(const DepthGatherArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= a.pieces) return;
+    const int64_t c = i % a.ppp;
+    int64_t r = i / a.ppp;
+    const int64_t kd = r % a.KD;
+    r /= a.KD;
+    const int64_t hw = r % a.HW;
+    r /= a.HW;
+    const int64_t od = r % a.OD, n = r / a.OD;
+    const int64_t d = od * a.sd + kd * a.dd - a.pad_d;
+    T v;
+    if (d >= 0 && d < a.D) {
+        v = *reinterpret_cast<const T *>(a.in + n * a.in_sn + d * a.in_sd + (hw * a.ppp + c) * a.piece);
+    } else {
+        if constexpr (sizeof(T) == 16) v = make_uint4(a.zsplat, a.zsplat, a.zsplat, a.zsplat);
+        else v = (T)a.zsplat;
+    }
+    *reinterpret_cast<T *>(a.x2 + i * a.piece) = v;
+}
+
+struct WeightRegroupArgs {
+    const char *w;
+    char *w2;
+    int64_t pieces;  // OC * KHW * KD * (IC / piece)
+    int32_t KD, KHW, piece, ppp;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) conv3d_weight_regroup_kernel(const WeightRegroupArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= a.pieces) return;
+    const int64_t c = i % a.ppp;
+    int64_t r = i / a.ppp;
+    const int64_t kd = r % a.KD;
+    r /= a.KD;
+    const int64_t khw = r % a.KHW, oc = r / a.KHW;
+    *reinterpret_cast<T *>(a.w2 + i * a.piece) =
+        *reinterpret_cast<const T *>(a.w + (((oc * a.KD + kd) * a.KHW + khw) * a.ppp + c) * a.piece);
+}
+
+int piece_of(int64_t ic, const void *p0, const void *p1) {
+    const uintptr_t bits = (uintptr_t)ic | (uintptr_t)p0 | (uintptr_t)p1;
+    return (bits % 16) == 0 ? 16 : (bits % 4) == 0 ? 4 : 1;
+}
+
+}  // namespace
+
+// x2 / w2: dense device buffers of N*OD*H*W*KD*IC resp. OC*KH*KW*KD*IC bytes (int8 operands)
+int launch_conv3d_regroup(hipStream_t s, void *x2, void *w2, const mlel_tensor *in, const mlel_tensor *w, int64_t OD,
+                          const mlel_conv3d_attr *a) {
+    const int64_t N = in->dims[0], D = in->dims[1], H = in->dims[2], W = in->dims[3], IC = in->dims[4];
+    const int64_t OC = w->dims[0], KD = w->dims[1], KHW = w->dims[2] * w->dims[3];
+    {
+        const int piece = piece_of(IC, in->ptr, x2);
+        DepthGatherArgs g{};
+        g.in = static_cast<const char *>(in->ptr);
+        g.x2 = static_cast<char *>(x2);
+        g.piece = piece;
+        g.ppp = (int32_t)(IC / piece);
+        g.pieces = N * OD * H * W * KD * g.ppp;
+        g.D = (int32_t)D, g.OD = (int32_t)OD, g.KD = (int32_t)KD;
+        g.sd = a->stride[0], g.dd = a->dilation[0], g.pad_d = a->pad[0];
+        g.HW = H * W;
+        g.in_sn = in->strides[0], g.in_sd = in->strides[1];
+        g.zsplat = (uint32_t)(uint8_t)a->input_zp * 0x01010101u;
+        if (g.pieces > 0) {
+            const dim3 grid = grid_1d(g.pieces, kBlock);
+            if (piece == 16) hipLaunchKernelGGL(conv3d_depth_gather_kernel<uint4>, grid, dim3(kBlock), 0, s, g);
+            else if (piece == 4) hipLaunchKernelGGL(conv3d_depth_gather_kernel<uint32_t>, grid, dim3(kBlock), 0, s, g);
+            else hipLaunchKernelGGL(conv3d_depth_gather_kernel<uint8_t>, grid, dim3(kBlock), 0, s, g);
+            MLEL_TRY(check_launch("conv3d depth gather"));
+        }
+    }
+    {
+        const int piece = piece_of(IC, w->ptr, w2);
+        WeightRegroupArgs g{};
+        g.w = static_cast<const char *>(w->ptr);
+        g.w2 = static_cast<char *>(w2);
+        g.piece = piece;
+        g.ppp = (int32_t)(IC / piece);
+        g.KD = (int32_t)KD, g.KHW = (int32_t)KHW;
+        g.pieces = OC * KHW * KD * g.ppp;
+        if (g.pieces > 0) {
+            const dim3 grid = grid_1d(g.pieces, kBlock);
+            if (piece == 16) hipLaunchKernelGGL(conv3d_weight_regroup_kernel<uint4>, grid, dim3(kBlock), 0, s, g);
+            else if (piece == 4) hipLaunchKernelGGL(conv3d_weight_regroup_kernel<uint32_t>, grid, dim3(kBlock), 0, s, g);
+            else hipLaunchKernelGGL(conv3d_weight_regroup_kernel<uint8_t>, grid, dim3(kBlock), 0, s, g);
+            MLEL_TRY(check_launch("conv3d weight regroup"));
+        }
+    }
+    return 0;
+}
+
 }  // namespace mlel

@@ -277,6 +277,44 @@ void free_split_workspaces(mlel_ctx *ctx) {
         (void)hipFree(ctx->ws[i].counters);
     }
     ctx->n_ws = 0;
+    for (int i = 0; i < ctx->n_stage; i++) (void)hipFree(ctx->stage[i].ptr);
+    ctx->n_stage = 0;
+}
+
+char *stage_workspace(mlel_ctx *ctx, hipStream_t stream, size_t bytes) {
+    if (bytes == 0 || bytes > kMaxStageBytes) return nullptr;
+    std::lock_guard<std::mutex> guard(ctx->ws_lock);
+    int slot = -1;
+    for (int i = 0; i < ctx->n_stage; i++)
+        if (ctx->stage[i].stream == stream) slot = i;
+    if (slot >= 0 && ctx->stage[slot].bytes >= bytes) return ctx->stage[slot].ptr;
+    if (stream_is_capturing(stream) || (slot < 0 && ctx->n_stage >= kMaxSplitWorkspaces)) return nullptr;
+    if (slot >= 0) {  // grow: earlier calls of the stream may still be reading the old buffer
+        if (hipStreamSynchronize(stream) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        (void)hipFree(ctx->stage[slot].ptr);
+        ctx->stage[slot] = ctx->stage[--ctx->n_stage];
+    }
+    char *p = nullptr;
+    const size_t rounded = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    if (hipMalloc(reinterpret_cast<void **>(&p), rounded) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    ctx->stage[ctx->n_stage++] = StageWorkspace{stream, p, rounded};
+    return p;
+}
+
+void release_stage_workspace(mlel_ctx *ctx, hipStream_t stream) {
+    std::lock_guard<std::mutex> guard(ctx->ws_lock);
+    for (int i = 0; i < ctx->n_stage; i++)
+        if (ctx->stage[i].stream == stream) {
+            (void)hipFree(ctx->stage[i].ptr);
+            ctx->stage[i] = ctx->stage[--ctx->n_stage];
+            return;
+        }
 }
 
 }  // namespace mlel
@@ -444,6 +482,7 @@ int mlel_hip_stream_destroy(mlel_ctx *ctx, void *stream) {
         // the stream's split-K workspace (if it ever split) is freed with it; nothing may still be using it
         MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
         release_split_workspace(ctx, (hipStream_t)stream);
+        release_stage_workspace(ctx, (hipStream_t)stream);
         MLEL_HIP_CHECK(hipStreamDestroy((hipStream_t)stream));
     }
     return 0;

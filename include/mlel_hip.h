@@ -357,7 +357,13 @@ int mlel_hip_argmax(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const m
  * arithmetic_right_shift.comp:22-48. */
 int mlel_hip_arithmetic_right_shift(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1,
                                     const mlel_tensor *in2, uint32_t round);
-/* CONV3D: NDHWC x ODHWI.  Replaces class Conv3D (reference: graph/compute_graph_op.cpp:1029-1110), conv3d.comp:37-104. */
+/* CONV3D: NDHWC x ODHWI.  Replaces class Conv3D (reference: graph/compute_graph_op.cpp:1029-1110), conv3d.comp:37-104.
+ * Dense int8 operands with an int32 result and at least four million multiply-adds run as ONE CONV2D on the matrix
+ * cores: the KD depth taps of an output slice are laid side by side along the channels of a copy of the input in the
+ * stream's staging memory (KD times the input; grown on demand outside a capture, released by
+ * mlel_hip_stream_destroy / mlel_hip_destroy), the weights regrouped to match.  A kernel one slice deep without depth
+ * padding or stride needs no copy.  Everything else, and a capturing stream whose staging memory is too small, takes
+ * the one-thread-per-output kernel.  The bits are the same. */
 int mlel_hip_conv3d(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
                     const mlel_tensor *weights, const mlel_tensor *bias, const mlel_conv3d_attr *attr);
 /* TRANSPOSE_CONV2D: NHWC x OHWI.  Replaces class TransposeConv2D (reference: graph/compute_graph_op.cpp:2211-2290),

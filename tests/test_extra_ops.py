@@ -7,6 +7,8 @@ ARITHMETIC_RIGHT_SHIFT are only created).  FFT2D / RFFT2D depend on the driver's
 are compared with numpy's FFT to a tolerance: parity unpinned beyond the mathematics of the transform.
 GPU part: every operator through the C ABI against the oracle on the same seeded inputs, bit for bit for integers.
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -369,6 +371,73 @@ def test_fft_vs_oracle_and_numpy(run, oracle):
     er, ei = oracle.rfft2d(re)
     assert np.abs(gr - er).max() <= 1e-4 and np.abs(gi - ei).max() <= 1e-4
     assert gi[0, 0, 0] == 0 and gi[0, 8, 16] == 0
+
+
+@pytest.mark.gpu
+def test_conv3d_through_conv2d_vs_oracle(run, oracle):
+    """int8 CONV3D with an int32 result and a few million multiply-adds runs as one CONV2D on the matrix cores (the depth
+    taps laid side by side along the channels of a temporary; a kernel one slice deep needs no temporary): 16-, 4- and
+    1-byte pieces, depth padding / stride / dilation, both zero points, bias of one value."""
+    rng = np.random.default_rng(77)
+    cases = [  # x shape, w shape, pad (front, back, top, bottom, left, right), stride, dilation, zi, zw, bias length
+        ((2, 6, 12, 12, 16), (32, 3, 3, 3, 16), (1, 1, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1), -7, 4, 32),
+        ((2, 7, 20, 20, 5), (40, 2, 3, 3, 5), (0, 1, 1, 0, 2, 1), (2, 1, 2), (2, 1, 1), 3, 0, 40),
+        ((1, 9, 16, 16, 4), (48, 3, 3, 3, 4), (3, 3, 0, 0, 1, 1), (1, 1, 1), (2, 2, 1), 0, -5, 1),
+        ((3, 5, 14, 14, 32), (16, 2, 1, 1, 32), (0, 0, 0, 0, 0, 0), (1, 1, 1), (1, 1, 1), -128, 0, 16),
+        ((2, 4, 9, 9, 8), (16, 1, 3, 3, 8), (0, 0, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1), 5, 2, 16),   # one slice deep
+        ((1, 3, 6, 6, 8), (8, 3, 3, 3, 8), (1, 1, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1), 1, 1, 8),     # small: generic kernel
+    ]
+    for xs, ws, pad, stride, dil, zi, zw, bl in cases:
+        x = ri(rng, -128, 127, xs, np.int8)
+        w = ri(rng, -128, 127, ws, np.int8)
+        b = ri(rng, -2 ** 20, 2 ** 20, (bl,), np.int32)
+        od = (xs[1] + pad[0] + pad[1] - (ws[1] - 1) * dil[0] - 1) // stride[0] + 1
+        oh = (xs[2] + pad[2] + pad[3] - (ws[2] - 1) * dil[1] - 1) // stride[1] + 1
+        ow = (xs[3] + pad[4] + pad[5] - (ws[3] - 1) * dil[2] - 1) // stride[2] + 1
+        shape = (xs[0], od, oh, ow, ws[0])
+        attr = abi.conv3d_attr(pad, stride, dil, zi, zw)
+        np.testing.assert_array_equal(run.conv3d(x, w, b, shape, abi.I32, attr), oracle.conv3d(x, w, b, shape, abi.I32, attr),
+                                      err_msg=str((xs, ws, pad, stride, dil)))
+
+
+@pytest.mark.gpu
+def test_conv3d_on_a_capturing_stream(run, oracle):
+    """CONV3D recorded into a HIP graph on a fresh stream (no staging memory yet and none can be allocated: the
+    one-thread-per-output kernel is recorded) and again after an eager call has given the stream its staging memory
+    (the CONV2D route is recorded); every replay over new inputs gives the oracle's bits."""
+    dev, lib = run.dev, run.dev.lib
+    rng = np.random.default_rng(79)
+    xs, ws = (1, 5, 12, 12, 16), (32, 3, 3, 3, 16)
+    w = ri(rng, -128, 127, ws, np.int8)
+    b = ri(rng, -2 ** 20, 2 ** 20, (32,), np.int32)
+    attr = abi.conv3d_attr((1, 1, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1), -4, 3)
+    shape = (1, 5, 12, 12, 32)
+    stream = dev.new_stream()
+    null_stream, dev.stream = dev.stream, stream
+    try:
+        tx, tw, tb = run.put(np.zeros(xs, np.int8)), run.put(w), run.put(b)
+        to = run.new(abi.I32, shape)
+        for phase in ("no staging memory", "staging memory from an eager call"):
+            if phase.startswith("staging"):
+                dev.op("conv3d", to.ref, tx.ref, tw.ref, tb.ref, C.byref(attr))
+                dev.sync()
+            dev._check(lib.mlel_hip_capture_begin(dev.ctx, stream))
+            try:
+                dev.op("conv3d", to.ref, tx.ref, tw.ref, tb.ref, C.byref(attr))
+            finally:
+                exe = C.c_void_p()
+                dev._check(lib.mlel_hip_capture_end(dev.ctx, stream, C.byref(exe)))
+            for rep in range(2):
+                x = ri(rng, -128, 127, xs, np.int8)
+                tx.upload(x)
+                dev._check(lib.mlel_hip_graph_launch(dev.ctx, exe, stream))
+                np.testing.assert_array_equal(to.download(), oracle.conv3d(x, w, b, shape, abi.I32, attr),
+                                              err_msg=f"{phase}, replay {rep}")
+            dev._check(lib.mlel_hip_graph_destroy(dev.ctx, exe))
+    finally:
+        dev.stream = null_stream
+        run.done()
+        dev._check(lib.mlel_hip_stream_destroy(dev.ctx, stream))
 
 
 @pytest.mark.gpu
