@@ -256,6 +256,8 @@ FUSED_SIGNATURES = {
                                     C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
     "conv2d_conv2d_rescale_clamp": [_T, _T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue), _T, _T,
                                     C.POINTER(Conv2dAttr), C.POINTER(Epilogue)],
+    "conv2d_rescale_clamp_avgpool": [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.POINTER(Epilogue), C.c_int32,
+                                     C.POINTER(Pool2dAttr)],
     "matmul_bias_cast": [_T, _T, _T, _T, C.POINTER(MatmulAttr)],
     "matmul_bias_cast_add": [_T, _T, _T, _T, C.POINTER(MatmulAttr), _T],
     "matmul_bias_cast_group": [C.POINTER(MatmulProduct), C.c_int, _T, C.POINTER(MatmulAttr)],
@@ -305,6 +307,8 @@ RUNTIME_SIGNATURES = {
                                                    C.POINTER(Conv2dAttr)]),
     "mlel_hip_conv2d_conv2d_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Conv2dAttr), _T, _T,
                                                    C.POINTER(Conv2dAttr)]),
+    "mlel_hip_conv2d_avgpool_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Conv2dAttr), C.c_int32,
+                                                    C.POINTER(Pool2dAttr)]),
 }
 
 

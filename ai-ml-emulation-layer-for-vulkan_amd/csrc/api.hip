@@ -1107,6 +1107,65 @@ int mlel_hip_conv2d_conv2d_in_kernel(const mlel_tensor *out, const mlel_tensor *
     return try_conv2d_pair_rows(nullptr, nullptr, out, nullptr, in, w1, b1, a1, &unused, MLEL_I8, w2, b2, a2, &unused, true) == 1 ? 1 : 0;
 }
 
+namespace {
+// the convolution's result as a dense tensor of `dtype` at `ptr`: [N, OH, OW, OC] from the operands and attributes
+bool conv_result_like(mlel_tensor *t, const mlel_tensor *in, const mlel_tensor *w, const mlel_conv2d_attr *a, int dtype,
+                      void *ptr) {
+    if (in == nullptr || w == nullptr || a == nullptr || in->rank != 4 || w->rank != 4) return false;
+    if (a->stride[0] <= 0 || a->stride[1] <= 0 || a->dilation[0] <= 0 || a->dilation[1] <= 0) return false;
+    const int64_t eh = (w->dims[1] - 1) * a->dilation[0] + 1, ew = (w->dims[2] - 1) * a->dilation[1] + 1;
+    const int64_t ih = in->dims[1] + a->pad[0] + a->pad[1], iw = in->dims[2] + a->pad[2] + a->pad[3];
+    if (ih < eh || iw < ew) return false;
+    *t = mlel_tensor{};
+    t->dtype = dtype, t->rank = 4, t->ptr = ptr;
+    t->dims[0] = in->dims[0], t->dims[1] = (ih - eh) / a->stride[0] + 1, t->dims[2] = (iw - ew) / a->stride[1] + 1;
+    t->dims[3] = w->dims[0];
+    int64_t st = dt_size(dtype);
+    for (int i = 3; i >= 0; i--) t->strides[i] = st, st *= t->dims[i];
+    return true;
+}
+}  // namespace
+
+int mlel_hip_conv2d_rescale_clamp_avgpool(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                          const mlel_tensor *weights, const mlel_tensor *bias,
+                                          const mlel_conv2d_attr *attr, const mlel_epilogue *epi, int32_t conv_dtype,
+                                          const mlel_pool2d_attr *pool) {
+    MLEL_TRY(require_ctx(ctx, "conv2d_rescale_clamp_avgpool"));
+    MLEL_REQUIRE(out != nullptr && attr != nullptr && pool != nullptr && epi != nullptr, MLEL_ERR_INVALID,
+                 "conv2d_rescale_clamp_avgpool: null argument");
+    MLEL_TRY(check_tensor(out, "conv2d_rescale_clamp_avgpool out"));
+    mlel_tensor mid;
+    // (the pooled tensor's pointer stands in where validation wants one: the convolution's result has no memory here)
+    MLEL_REQUIRE(conv_result_like(&mid, in, weights, attr, conv_dtype, out->ptr), MLEL_ERR_INVALID,
+                 "conv2d_rescale_clamp_avgpool: operands do not describe a convolution");
+    MLEL_REQUIRE(dt_is_int(conv_dtype) && dt_size(conv_dtype) <= 4 && conv_dtype == out->dtype, MLEL_ERR_INVALID,
+                 "conv2d_rescale_clamp_avgpool: the convolution's result and the pooled tensor have one integer type");
+    mlel_tensor acc_view = packed_like(&mid, MLEL_I32, out->ptr);  // shape carrier for validation
+    MLEL_TRY(check_conv("conv2d_rescale_clamp_avgpool", &acc_view, in, weights, bias, attr));
+    FusedEpilogue fe;
+    MLEL_TRY(make_epilogue(epi, MLEL_I32, &mid, mid.dims[3], &fe));
+    const int rc = try_conv2d_avgpool_cols((hipStream_t)stream, out, &mid, in, weights, bias, attr, &fe, pool, false);
+    if (rc != 0) return rc < 0 ? rc : 0;
+    // no one-pass kernel for these operands: the fused convolution into a temporary, then the pooling
+    Scratch scratch;
+    MLEL_TRY(alloc_fallback(scratch, (size_t)numel(&mid) * dt_size(conv_dtype) + 16, stream, __func__));
+    mid.ptr = scratch.ptr;
+    MLEL_TRY(mlel_hip_conv2d_rescale_clamp(ctx, stream, &mid, in, weights, bias, attr, epi));
+    MLEL_TRY(mlel_hip_avg_pool2d(ctx, stream, out, &mid, pool));
+    MLEL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+int mlel_hip_conv2d_avgpool_in_kernel(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *weights,
+                                      const mlel_tensor *bias, const mlel_conv2d_attr *attr, int32_t conv_dtype,
+                                      const mlel_pool2d_attr *pool) {
+    if (out == nullptr || in == nullptr || weights == nullptr || bias == nullptr || attr == nullptr || pool == nullptr) return 0;
+    mlel_tensor mid;
+    if (!conv_result_like(&mid, in, weights, attr, conv_dtype, nullptr)) return 0;
+    const FusedEpilogue unused{};  // the requantisation constants do not decide whether the kernel takes the case
+    return try_conv2d_avgpool_cols(nullptr, out, &mid, in, weights, bias, attr, &unused, pool, true) == 1 ? 1 : 0;
+}
+
 int mlel_hip_rescale_add_rescale(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in1,
                                  const mlel_epilogue *scale1, const mlel_tensor *in2, const mlel_epilogue *scale2,
                                  const mlel_epilogue *scale_out) {

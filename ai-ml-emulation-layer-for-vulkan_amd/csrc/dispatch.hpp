@@ -181,6 +181,11 @@ int try_conv2d_pair_rows(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, c
                          const mlel_tensor *in, const mlel_tensor *w1, const mlel_tensor *b1, const mlel_conv2d_attr *a1,
                          const FusedEpilogue *e1, int mid_dtype, const mlel_tensor *w2, const mlel_tensor *b2,
                          const mlel_conv2d_attr *a2, const FusedEpilogue *e2, bool probe);
+// 1x1 CONV2D + RESCALE (+CLAMP) + global AVG_POOL2D in one launch (gemm_i8.hip / gemm_i8_cols.hip); `conv_out` is a
+// shape and type carrier
+int try_conv2d_avgpool_cols(hipStream_t s, const mlel_tensor *pool_out, const mlel_tensor *conv_out, const mlel_tensor *in,
+                            const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
+                            const FusedEpilogue *epi, const mlel_pool2d_attr *pool, bool probe);
 // ---- data movement in whole pieces on packed tensors (ops_move.hip); each returns 1 when launched, 0 to decline ----
 int try_slice_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, const uint32_t *start);
 int try_concat_fast(hipStream_t s, const mlel_tensor *out, const mlel_tensor *in, uint32_t axis, uint32_t offset);

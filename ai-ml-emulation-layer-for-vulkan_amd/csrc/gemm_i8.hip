@@ -346,4 +346,55 @@ int try_matmul_i8_mfma(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     return 1;
 }
 
+// 1x1 CONV2D + RESCALE (+CLAMP) to int8 whose only reader is a global AVG_POOL2D, in one launch
+// (conv_cols_pool_i8_kernel).  `conv_out` carries the convolution's result shape and type, its memory is not touched.
+// Returns 1 when launched (or, with `probe`, when the shapes are the kernel's), 0 to decline.
+int try_conv2d_avgpool_cols(hipStream_t s, const mlel_tensor *pool_out, const mlel_tensor *conv_out, const mlel_tensor *in,
+                            const mlel_tensor *w, const mlel_tensor *bias, const mlel_conv2d_attr *a,
+                            const FusedEpilogue *epi, const mlel_pool2d_attr *pool, bool probe) {
+    if (in->dtype != MLEL_I8 || w->dtype != MLEL_I8 || bias->dtype != MLEL_I32 || a->acc_type != MLEL_ACC_I32) return 0;
+    if (conv_out->dtype != MLEL_I8 || pool_out->dtype != MLEL_I8 || epi == nullptr) return 0;
+    if (!probe && epi->p.in_zp != 0) return 0;
+    if (conv_out->rank != 4 || pool_out->rank != 4 || in->rank != 4 || w->rank != 4) return 0;
+    const int64_t N = conv_out->dims[0], H = conv_out->dims[1], W = conv_out->dims[2], OC = conv_out->dims[3];
+    const int64_t IC = in->dims[3];
+    if (in->dims[0] != N || in->dims[1] != H || in->dims[2] != W || w->dims[0] != OC || w->dims[1] != 1 || w->dims[2] != 1 ||
+        w->dims[3] != IC)
+        return 0;
+    if (a->stride[0] != 1 || a->stride[1] != 1 || a->pad[0] != 0 || a->pad[1] != 0 || a->pad[2] != 0 || a->pad[3] != 0 ||
+        a->weight_zp != 0)
+        return 0;
+    if (!(bias->dims[0] == 1 || bias->dims[0] >= OC) || bias->strides[0] != 4) return 0;
+    if (!is_packed(in) || !is_packed(w) || !is_packed(pool_out)) return 0;
+    // the pooling takes every position of an image into one value per channel
+    if (pool->kernel[0] != H || pool->kernel[1] != W || pool->pad[0] != 0 || pool->pad[1] != 0 || pool->pad[2] != 0 ||
+        pool->pad[3] != 0 || pool->acc_type != MLEL_ACC_I32)
+        return 0;
+    if (pool_out->dims[0] != N || pool_out->dims[1] != 1 || pool_out->dims[2] != 1 || pool_out->dims[3] != OC) return 0;
+    const int64_t P = H * W, M = N * P;
+    if (P <= 0 || P > 64 || N <= 0 || OC <= 0 || IC <= 0 || IC % 16 != 0 || M >= (int64_t(1) << 24)) return 0;
+    if (M * IC >= (int64_t(1) << 31) || OC * IC >= (int64_t(1) << 31)) return 0;
+    GemmArgs g{};
+    g.M = (int)M, g.N = (int)OC, g.K = (int)IC, g.batches = 1;
+    g.plain = 1;
+    g.x_sx = IC;
+    g.x_bytes = (uint32_t)(M * IC);
+    g.ldw = IC;
+    g.w_bytes = (uint32_t)(OC * IC);
+    g.zx = a->input_zp, g.zw = 0;
+    g.bias_len = (int)bias->dims[0];
+    if (probe) return launch_conv_cols_pool(&g, nullptr, (int)N, (int)P, 0, 0, true, s);
+    if (((uintptr_t)in->ptr % 16) != 0 || ((uintptr_t)w->ptr % 16) != 0 || ((uintptr_t)bias->ptr % 4) != 0) return 0;
+    g.x = static_cast<const int8_t *>(in->ptr);
+    g.w = static_cast<const int8_t *>(w->ptr);
+    g.bias = static_cast<const int32_t *>(bias->ptr);
+    g.ldo = OC;
+    MLEL_TRY(fill_epilogue(g, conv_out, epi));
+    if (!launch_conv_cols_pool(&g, static_cast<int8_t *>(pool_out->ptr), (int)N, (int)P, pool->input_zp, pool->output_zp,
+                               false, s))
+        return 0;
+    MLEL_TRY(check_launch("conv2d 1x1 int8 + global avg_pool2d"));
+    return 1;
+}
+
 }  // namespace mlel

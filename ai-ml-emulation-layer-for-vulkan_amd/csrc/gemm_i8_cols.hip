@@ -197,7 +197,126 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// 1x1 CONV2D + RESCALE (+CLAMP) to int8 followed by a global AVG_POOL2D (the head of a classification network: the
+// last expansion of MobileNetV2 and the pooling over its 7 x 7 positions): the convolution's result never leaves the
+// registers.  A block owns one image and two groups of 32 channels; a wavefront owns one group and the positions
+// 0 .. 31 or 32 .. 63 of the image (at most 64 positions, those beyond the image multiply zeros and are not summed).
+// Loop and requantisation as conv_cols_mfma_i8_kernel; then every lane adds up the int8 results of its positions, the
+// two lane halves and the two wavefronts of a group are combined (a shuffle, then shared memory), and the pooling
+// arithmetic of avgpool2d.comp:27-75 is applied to the sum: minus count * input_zp, divided by the count with
+// rounding half away from zero, plus output_zp, clamped to int8.
+// ---------------------------------------------------------------------------------------------------------------
+struct ColsPoolArgs {
+    int8_t *out;       // [images][channels]
+    int32_t positions; // per image (H * W <= 64)
+    int32_t images, pairs, total_blocks;
+    int32_t zi, zo;
+};
+
+__global__ void __launch_bounds__(kColsBlock) conv_cols_pool_i8_kernel(const GemmArgs g, const ColsPoolArgs pa) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int chunk = (int)gridDim.x >> 3;
+    const int bid = (int)(blockIdx.x % 8u) * chunk + (int)(blockIdx.x / 8u);
+    if (bid >= pa.total_blocks) return;
+    const int image = bid / pa.pairs, pair = bid - image * pa.pairs;
+    const int t = wave & 1, ng = pair * 2 + (wave >> 1);
+    const int cl = lane & 31, half = lane >> 5;
+    const int pos = 32 * t + cl;  // this lane's pixel row of the image
+    const int n = ng * 32 + cl;   // and its channel
+    const __amdgpu_buffer_rsrc_t xres = make_rsrc(g.x, g.x_bytes), wres = make_rsrc(g.w, g.w_bytes);
+    const uint32_t xoff = pos < pa.positions
+                              ? (uint32_t)(image * pa.positions + pos) * (uint32_t)g.x_sx + (uint32_t)half * 16u
+                              : kOobOffset;
+    const uint32_t woff = n < g.N ? (uint32_t)n * (uint32_t)g.ldw + (uint32_t)half * 16u : kOobOffset;
+    auto fetch = [&](int round, v4i (&xf)[KR], v4i (&wf)[KR]) {
+#pragma unroll
+        for (int c = 0; c < KR; c++) {
+            const int k = (round * KR + c) * 32;
+            const bool in = k + half * 16 < g.K;
+            const uint4 xv = buf_load16(xres, (in && xoff != kOobOffset) ? xoff + (uint32_t)k : kOobOffset);
+            const uint4 wv = buf_load16(wres, (in && woff != kOobOffset) ? woff + (uint32_t)k : kOobOffset);
+            xf[c] = v4i{(int)xv.x, (int)xv.y, (int)xv.z, (int)xv.w};
+            wf[c] = v4i{(int)wv.x, (int)wv.y, (int)wv.z, (int)wv.w};
+        }
+    };
+    const int rounds = (g.K + KR * 32 - 1) / (KR * 32);
+    v4i xa[KR], wa[KR], xb[KR], wb[KR];
+    fetch(0, xa, wa);
+    int32_t bias = 0, mult = 0, shift = 0;
+    if (n < g.N) {
+        bias = g.bias ? g.bias[g.bias_len == 1 ? 0 : n] : 0;
+        const int ci = g.rp.per_channel ? n : 0;
+        mult = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci] : reinterpret_cast<const int32_t *>(g.mult)[ci];
+        shift = (int32_t)g.shift[ci];
+    }
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0;
+    int32_t wsum = 0;
+    const bool need_wsum = g.zx != 0;
+    auto multiply = [&](const v4i (&xf)[KR], const v4i (&wf)[KR]) {
+#pragma unroll
+        for (int c = 0; c < KR; c++) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[c], wf[c], acc, 0, 0, 0);
+        if (need_wsum) {  // uniform
+#pragma unroll
+            for (int c = 0; c < KR; c++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) wsum = __builtin_amdgcn_sdot4(wf[c][e], 0x01010101, wsum, false);
+        }
+    };
+    for (int r = 0; r < rounds; r += 2) {
+        if (r + 1 < rounds) fetch(r + 1, xb, wb);
+        multiply(xa, wa);
+        if (r + 1 < rounds) {
+            if (r + 2 < rounds) fetch(r + 2, xa, wa);
+            multiply(xb, wb);
+        }
+    }
+    // register 4 q + e of a lane: position 32 t + 8 q + 4 half + e of the image, channel n
+    const int32_t sw = wsum + __shfl_xor(wsum, 32);
+    const int32_t bias_adj = (int32_t)((uint32_t)bias - (uint32_t)g.zx * (uint32_t)sw);
+    const ChanScale cs = make_chan_scale(mult, shift, g.rp);
+    int32_t sum = 0;
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int32_t v = requant_acc((int32_t)((uint32_t)acc[4 * q + e] + (uint32_t)bias_adj), cs, g.rp);
+            sum += (32 * t + 8 * q + 4 * half + e < pa.positions) ? v : 0;
+        }
+    sum += __shfl_xor(sum, 32);
+    __shared__ int32_t part[2][32];  // [group of the block][channel]: the sum over positions 32 .. 63
+    if (t == 1 && half == 0) part[wave >> 1][cl] = sum;
+    __syncthreads();
+    if (t == 1 || half != 0 || n >= g.N) return;
+    const int32_t count = pa.positions;
+    const int32_t total = (int32_t)((uint32_t)sum + (uint32_t)part[wave >> 1][cl] - (uint32_t)pa.zi * (uint32_t)count);
+    int32_t r = (total + (total < 0 ? -(count >> 1) : (count >> 1))) / count;
+    r = (int32_t)((uint32_t)r + (uint32_t)pa.zo);
+    r = r < -128 ? -128 : (r > 127 ? 127 : r);
+    pa.out[(int64_t)image * g.N + n] = (int8_t)r;
+}
+
 }  // namespace
+
+// The pooled form: `g` describes the plain 1x1 convolution over images * positions rows (its output pointer is not
+// used), `pool_out` is [images][g.N] int8.  Returns 1 when launched (or when `probe` and it would be).
+int launch_conv_cols_pool(const void *args, int8_t *pool_out, int images, int positions, int zi, int zo, bool probe,
+                          hipStream_t s) {
+    const GemmArgs &g = *static_cast<const GemmArgs *>(args);
+    if (g.zw != 0 || g.K % 16 != 0 || g.batches != 1 || !g.plain || positions <= 0 || positions > 64 || images <= 0) return 0;
+    if ((int64_t)images * positions != g.M) return 0;
+    const int64_t groups_n = (g.N + 31) / 32, pairs = (groups_n + 1) / 2;
+    const int64_t blocks = (int64_t)images * pairs;
+    if (blocks >= (int64_t(1) << 24)) return 0;
+    if (probe) return 1;
+    ColsPoolArgs pa{pool_out, positions, images, (int)pairs, (int)blocks, zi, zo};
+    const dim3 grid((unsigned)((blocks + 7) / 8 * 8));
+    conv_cols_pool_i8_kernel<<<grid, dim3(kColsBlock), 0, s>>>(g, pa);
+    return 1;
+}
 
 // What the kernel's indexing assumes is checked by the caller (plain rows on both sides in 16-byte pieces, 8-bit
 // fused epilogue with dword stores, 31-bit extents) and here (zero weight zero point, K in 16-byte pieces).

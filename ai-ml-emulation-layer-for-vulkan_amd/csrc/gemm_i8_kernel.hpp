@@ -1167,6 +1167,8 @@ MLEL_DECLARE_GEMM_TILE(5);
 MLEL_DECLARE_GEMM_TILE(6);
 // the LDS-free form for 1x1 convolutions of few tiles (gemm_i8_cols.hip); 1 when launched
 int launch_conv_cols_mfma(const void *args, hipStream_t s);
+int launch_conv_cols_pool(const void *args, int8_t *pool_out, int images, int positions, int zi, int zo, bool probe,
+                          hipStream_t s);
 #define MLEL_DEFINE_GEMM_TILE(ID, BM, BN, WAVES_M, WAVES_N)                                          \
     void launch_gemm_tile##ID(const void *args, int xmode, int wmode, dim3 grid, hipStream_t s) {    \
         launch_tile_zp<BM, BN, WAVES_M, WAVES_N>(*static_cast<const GemmArgs *>(args), xmode, wmode, grid, s); \

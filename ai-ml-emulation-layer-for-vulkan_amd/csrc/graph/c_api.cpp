@@ -317,6 +317,8 @@ std::string opLabel(const OpNode &op) {
         // "+KEEP": the first convolution's result is stored as well (a later operator reads it)
         return std::string("CONV2D+RESCALE") + (op.hasClampFirst ? "+CLAMP" : "") + (op.outputs.size() > 1 ? "+KEEP" : "") +
                "+CONV2D+RESCALE" + (op.hasClamp ? "+CLAMP" : "");
+    case OpKind::FusedConv2DAvgPool:
+        return std::string("CONV2D+RESCALE") + (op.hasClamp ? "+CLAMP" : "") + "+AVG_POOL2D";
     case OpKind::FusedAttention:
         return std::string("MATMUL+CAST+ELEMENTWISE+REDUCE x") + std::to_string(op.chain.size()) + "+MATMUL+CAST" +
                (op.viewDims[5] != 0 ? "+RESHAPE+TRANSPOSE" : "");

@@ -1296,6 +1296,32 @@ void GraphPipeline::fuse() {
         first->fusedAway = true;
     }
 
+    // Pattern 10 (head of a classifier): a fused 1x1 CONV2D whose private int8 result is read only by an AVG_POOL2D
+    // over all positions of an image, on shapes the one-launch kernel takes (mlel_hip_conv2d_avgpool_in_kernel
+    // decides).  The convolution's result then stays in registers; byte for byte the two launches.
+    for (const auto &opPtr : ops) {
+        OpNode &pool = *opPtr;
+        if (pool.fusedAway || pool.kind != OpKind::AvgPool2D) continue;
+        const TensorPtr mid = pool.inputs[0];
+        OpNode *conv = mid->getProducer();
+        if (!conv || conv->fusedAway || conv->kind != OpKind::FusedConv2D || conv->outputs[0].get() != mid.get() ||
+            !isPrivateIntermediate(*mid) || consumersOf(ops, mid.get()).size() != 1)
+            continue;
+        if (conv->epilogue.attr.input_zp != 0) continue;
+        const mlel_tensor out = pool.outputs[0]->view(), x = conv->inputs[0]->view(), w = conv->inputs[1]->view(),
+                          b = conv->inputs[2]->view();
+        const int32_t midType = mid->view().dtype;
+        if (mlel_hip_conv2d_avgpool_in_kernel(&out, &x, &w, &b, &conv->conv, midType, &pool.pool) == 0) continue;
+        pool.kind = OpKind::FusedConv2DAvgPool;
+        pool.inputs = {conv->inputs[0], conv->inputs[1], conv->inputs[2]};
+        pool.conv = conv->conv;
+        pool.epilogue = conv->epilogue;
+        pool.hasClamp = conv->hasClamp;
+        pool.clamp = conv->clamp;
+        pool.selector = midType;
+        conv->fusedAway = true;
+    }
+
     // Pattern 3: RESHAPE between two packed session tensors of the same byte size moves no data (the reference's
     // reshape.comp:16-27 copies by flat index): the output becomes a second view of the input's storage and the
     // operator is not executed.  plan() gives both tensors one allocation that lives as long as either is used.
@@ -1642,6 +1668,7 @@ bool batchOperands(const OpNode &op, std::vector<size_t> &ins) {
     case OpKind::FusedDepthwiseConv2D:
     case OpKind::FusedConv2DDepthwise:
     case OpKind::FusedConv2DConv2D:
+    case OpKind::FusedConv2DAvgPool:
     case OpKind::AvgPool2D:
     case OpKind::MaxPool2D:
     case OpKind::Rescale:
@@ -2088,6 +2115,13 @@ void GraphPipeline::run(const OpNode &op, void *stream, const int half) {
         const mlel_epilogue e2 = makeEpilogue(op.epilogue, &m2, &s2, op.hasClamp, op.clamp);
         rc = mlel_hip_conv2d_dwconv_rescale_clamp(ctx, stream, &out, &in[0], &in[1], &in[2], &op.convFirst, &e1, &in[3],
                                                   &in[4], &op.conv, &e2);
+        break;
+    }
+    case OpKind::FusedConv2DAvgPool: {
+        const mlel_tensor mult = op.epilogue.multiplier->view(), shift = op.epilogue.shift->view();
+        const mlel_epilogue e = makeEpilogue(op.epilogue, &mult, &shift, op.hasClamp, op.clamp);
+        rc = mlel_hip_conv2d_rescale_clamp_avgpool(ctx, stream, &out, &in[0], &in[1], &in[2], &op.conv, &e, op.selector,
+                                                   &op.pool);
         break;
     }
     case OpKind::FusedConv2DConv2D: {

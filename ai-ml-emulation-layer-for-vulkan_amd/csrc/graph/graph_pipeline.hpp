@@ -98,7 +98,7 @@ enum class OpKind {
     Argmax, ArithmeticRightShift, Conv3D, TransposeConv2D, Fft2D, Rfft2D, Gather, Scatter, Resize, Reverse, Tile, Select,
     // produced by the fusion pass only
     FusedConv2D, FusedDepthwiseConv2D, FusedMatmul, FusedRescaleAddRescale, FusedMatmulBiasCast, FusedElementwise,
-    FusedConv2DResidual, FusedAttention, FusedConv2DDepthwise, FusedConv2DConv2D,
+    FusedConv2DResidual, FusedAttention, FusedConv2DDepthwise, FusedConv2DConv2D, FusedConv2DAvgPool,
 };
 
 struct RescaleSpec {
@@ -156,6 +156,9 @@ class OpNode {
     // FusedConv2DConv2D: two 1x1 convolutions in a row; inputs = {x, the first convolution's weights and bias, the
     // second's}; conv / epilogue / hasClamp / clamp belong to the second, convFirst / scaleA / hasClampFirst / clampFirst
     // to the first; outputs[1], when present, is the first convolution's result, which a later operator reads too
+    // FusedConv2DAvgPool: a 1x1 convolution (+RESCALE, +CLAMP) and the AVG_POOL2D over all positions behind it; inputs =
+    // {x, weights, bias}; conv / epilogue / hasClamp / clamp belong to the convolution, pool to the pooling, selector
+    // is the type the convolution's result had
     mlel_conv2d_attr convFirst{};
     mlel_clamp_attr clampFirst{};
     bool hasClampFirst = false;

@@ -502,6 +502,18 @@ def launch_layers(g, spec):
                         "macs": c1["macs"] + c2["macs"], "bytes": c1["bytes"] + c2["bytes"] - (mid if kept else 2 * mid),
                         "layers": [at, at + 1]})
             at += 2
+        elif name.startswith("CONV2D") and name.endswith("AVG_POOL2D"):
+            # the head: the convolution's result is pooled in registers and never reaches memory
+            if at + 1 >= len(spec.layers):
+                return None
+            conv, pool = spec.layers[at], spec.layers[at + 1]
+            if conv["kind"] != "conv" or pool["kind"] != "avgpool":
+                return None
+            mid = int(np.prod(conv["out"]))
+            out.append({"kind": "conv+avgpool", "in": conv["in"], "out": pool["out"], "kernel": 1, "stride": 1,
+                        "macs": conv["macs"] + pool["macs"], "bytes": conv["bytes"] + pool["bytes"] - 2 * mid,
+                        "layers": [at, at + 1]})
+            at += 2
         else:
             out.append(dict(spec.layers[at], layers=[at]))
             at += 1
@@ -559,7 +571,7 @@ def bench_mobilenetv2(dev, steps=20, warmup=3, batch=32, per_layer=True, in_flig
                            "gbs": round(layer["bytes"] / (ms * 1e-3) / 1e9, 1)})
         # a launch that holds a CONV2D or MATMUL (also the expansion + depthwise pairs) is priced against the matrix
         # cores, a stand-alone DEPTHWISE_CONV2D or AVG_POOL2D against HBM
-        dense = [(l, launches[l["index"]]) for l in layers if l["kind"] in ("conv", "fc", "conv+dw", "conv+conv")]
+        dense = [(l, launches[l["index"]]) for l in layers if l["kind"] in ("conv", "fc", "conv+dw", "conv+conv", "conv+avgpool")]
         band = [(l, launches[l["index"]]) for l in layers if l["kind"] in ("dw", "avgpool")]
 
         def total(group, key):

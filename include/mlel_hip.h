@@ -569,6 +569,23 @@ int mlel_hip_conv2d_conv2d_rescale_clamp(mlel_ctx *ctx, void *stream, const mlel
 int mlel_hip_conv2d_conv2d_in_kernel(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w1,
                                      const mlel_tensor *b1, const mlel_conv2d_attr *a1, const mlel_tensor *w2,
                                      const mlel_tensor *b2, const mlel_conv2d_attr *a2);
+
+/* 1x1 CONV2D + RESCALE (+CLAMP) whose int8 result is read only by an AVG_POOL2D over all positions of an image (the
+ * head of a classification network), as one launch: the convolution's result stays in registers.  `out` is the pooled
+ * tensor [N, 1, 1, OC]; `conv_dtype` is the type the convolution's result would have had.  Composition of
+ * conv2d.comp:40-116, rescale.comp:28-63, clamp.comp:18-31 and avgpool2d.comp:27-75: the bytes are those of
+ * mlel_hip_conv2d_rescale_clamp followed by mlel_hip_avg_pool2d, which is also what runs (through a temporary: the call
+ * then allocates and waits, and is refused on a capturing stream) when the one-launch kernel declines the operands:
+ * int8, zero weight zero point, RESCALE input zero point 0, at most 64 positions per image, input channels in 16-byte
+ * units, no padding, dense operands.  mlel_hip_conv2d_avgpool_in_kernel answers that beforehand without touching the
+ * device (1: one launch). */
+int mlel_hip_conv2d_rescale_clamp_avgpool(mlel_ctx *ctx, void *stream, const mlel_tensor *out, const mlel_tensor *in,
+                                          const mlel_tensor *weights, const mlel_tensor *bias,
+                                          const mlel_conv2d_attr *attr, const mlel_epilogue *epi, int32_t conv_dtype,
+                                          const mlel_pool2d_attr *pool);
+int mlel_hip_conv2d_avgpool_in_kernel(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *weights,
+                                      const mlel_tensor *bias, const mlel_conv2d_attr *attr, int32_t conv_dtype,
+                                      const mlel_pool2d_attr *pool);
 /* 1 when mlel_hip_conv2d_dwconv_rescale_clamp takes these operands, judged by types, extents, strides and attributes
  * only (data pointers are not looked at; no device is touched), else 0. */
 int mlel_hip_conv2d_dwconv_in_kernel(const mlel_tensor *out, const mlel_tensor *in, const mlel_tensor *w1,

@@ -265,6 +265,19 @@ class Runner:
         self.done()
         return covered, r, m
 
+    def conv2d_avgpool(self, x, w, b, attr, epi, pool):
+        """(covered by the one-launch kernel?, pooled output [N, 1, 1, OC])"""
+        tx, tw, tb = self.put(x), self.put(w), self.put(b)
+        to = self.new(abi.I8, (x.shape[0], 1, 1, w.shape[0]))
+        e = self._epi(*epi)
+        covered = self.dev.lib.mlel_hip_conv2d_avgpool_in_kernel(to.ref, tx.ref, tw.ref, tb.ref, C.byref(attr), abi.I8,
+                                                                 C.byref(pool))
+        self.dev.op("conv2d_rescale_clamp_avgpool", to.ref, tx.ref, tw.ref, tb.ref, C.byref(attr), C.byref(e), abi.I8,
+                    C.byref(pool))
+        r = to.download()
+        self.done()
+        return covered, r
+
     def softmax_rows(self, x):
         tx = self.put(x)
         to = self.new(tx.dtype, x.shape)

@@ -107,8 +107,10 @@ def test_mobilenetv2_graph_structure_and_plan():
     # contractions (10 of the projections carry their block's residual addition; from 28 x 28 positions down the 13
     # expansions run in one launch with the depthwise stage behind them; in front of that stage two projections share
     # a launch with the expansion that reads them, the second one still storing its result for the residual
-    # connection of the next block), pool + fc; the RESHAPE between two session tensors became a view of its input
-    assert len(names) == 35 + 17 + 2 - 13 - 2 and "RESHAPE" not in names
+    # connection of the next block; the last expansion pools its result in the same launch), fc; the RESHAPE between two
+    # session tensors became a view of its input
+    assert len(names) == 35 + 17 + 2 - 13 - 2 - 1 and "RESHAPE" not in names
+    assert names[-2] == "CONV2D+RESCALE+CLAMP+AVG_POOL2D"
     assert names.count("CONV2D+RESCALE+CLAMP+DEPTHWISE_CONV2D+RESCALE+CLAMP") == 13
     assert names[2] == "CONV2D+RESCALE+CONV2D+RESCALE+CLAMP" and names[4] == "CONV2D+RESCALE+KEEP+CONV2D+RESCALE+CLAMP"
     assert names.count("CONV2D+RESCALE+RESCALE+RESCALE+ADD+RESCALE") == 10 and names[-1] == "MATMUL+RESCALE"

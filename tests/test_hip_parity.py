@@ -1390,6 +1390,40 @@ def test_conv2d_conv2d_pair_vs_oracle(run, oracle, case):
             np.testing.assert_array_equal(got_mid, mid, err_msg=name)
 
 
+POOL_CASES = [
+    # name, (N, H, W), IC, OC, conv input zp, pool zps (in, out), one launch expected
+    ("mnv2_head_320_1280", (3, 7, 7), 320, 1280, -3, (-128, -128), True),
+    ("whole_64_positions", (2, 8, 8), 64, 96, 0, (5, -7), True),
+    ("one_group_of_channels", (1, 5, 6), 48, 24, 9, (0, 0), True),        # 30 positions, 24 channels: ragged both ways
+    ("odd_group_count", (2, 3, 3), 32, 72, -128, (-4, 3), True),          # three groups of 32 channels: an idle wavefront pair
+    ("single_position", (4, 1, 1), 16, 40, 1, (2, 2), True),
+    ("too_many_positions", (1, 9, 9), 32, 32, 0, (0, 0), False),          # 81 positions: convolution, then pooling
+    ("odd_channels_in", (1, 4, 4), 24, 32, 0, (0, 0), False),             # 24 bytes of K: not whole 16-byte pieces
+]
+
+
+@pytest.mark.parametrize("case", POOL_CASES, ids=[c[0] for c in POOL_CASES])
+def test_conv2d_avgpool_vs_oracle(run, oracle, case):
+    """mlel_hip_conv2d_rescale_clamp_avgpool: a 1x1 CONV2D + RESCALE + CLAMP and the AVG_POOL2D over all positions of an
+    image in one launch, against the oracle running the four operators; shapes outside the kernel give the same bytes
+    through the fused convolution and the pooling operator."""
+    name, nhw, ic, oc, zi, (pzi, pzo), one_launch = case
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    n, h, w_ = nhw
+    x = ri(rng, -128, 127, (n, h, w_, ic), np.int8)
+    w = ri(rng, -127, 127, (oc, 1, 1, ic), np.int8)
+    b = ri(rng, -2 ** 15, 2 ** 15, (oc,), np.int32)
+    m, s = rescale_params(rng, oc)
+    a = abi.conv2d_attr((0, 0, 0, 0), (1, 1), (1, 1), zi, 0)
+    r = abi.rescale_attr(0, pzi, True, True, True)
+    pool = abi.pool2d_attr((h, w_), (1, 1), (0, 0, 0, 0), pzi, pzo)
+    mid = oracle.clamp(oracle.rescale(oracle.conv2d(x, w, b, (n, h, w_, oc), abi.I32, a), m, s, abi.I8, r), -100, 127)
+    exp = oracle.avg_pool2d(mid, (n, 1, 1, oc), pool)
+    covered, got = run.conv2d_avgpool(x, w, b, a, (m, s, r, (-100, 127)), pool)
+    assert bool(covered) == one_launch, name
+    np.testing.assert_array_equal(got, exp, err_msg=name)
+
+
 def test_copy_kernels_move_exactly_the_requested_bytes(run):
     """mlel_hip_copy_kernel (ragged length: whole pieces by the one-pass kernel, the tail bytewise) and every mode of
     mlel_hip_copy_kernel_variant leave the destination equal to the source over the requested bytes and untouched

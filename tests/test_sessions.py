@@ -158,7 +158,7 @@ def test_replayed_dispatch_equals_the_eager_one(dev, kats):
     """mlel_graph_session_dispatch_replayed: the launches of a dispatch recorded once and submitted many times (the
     command buffer of tests/vulkan.cpp:918-996, re-submitted).  Same bytes as the eager dispatch; a bind after the
     recording is honoured (the recording is made again); two sessions replay on two streams at once; a MobileNetV2-shaped
-    graph of 39 launches replays to the bits of its eager dispatch."""
+    graph of 38 launches replays to the bits of its eager dispatch."""
     g, x, exp = maxpool_graph(dev, kats, 2)
     streams = [dev.new_stream(), dev.new_stream()]
     s = g.new_session()

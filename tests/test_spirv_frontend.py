@@ -470,7 +470,7 @@ def test_config3_mobilenetv2_b32_from_assembly_equals_direct_build(dev):
     g.set_input("input", x)
     g.dispatch()
     direct = g.get_output("output")
-    assert names == g.op_names() and len(names) == 39
+    assert names == g.op_names() and len(names) == 38
     g.close()
     np.testing.assert_array_equal(got["output"], direct)
 
