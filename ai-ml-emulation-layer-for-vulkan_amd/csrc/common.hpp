@@ -454,6 +454,26 @@ __device__ __forceinline__ int32_t dot4_from(uint32_t a, uint32_t b, int32_t c) 
     return d;
 }
 
+// The clamp's upper bound in a vector register that the compiler may not re-create from the scalar one: v_med3 takes
+// one scalar operand only, and left alone the compiler moves both bounds into registers again for every few values
+// (3 - 4 % of the vector instructions of the requantisation-bound kernels).  The staged matrix kernel keeps the
+// three-argument form: its 128 x 128 direct-to-LDS variant measured 1 % slower with this one.
+__device__ __forceinline__ int32_t pin_vgpr(int32_t s) {
+    int32_t v;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(v) : "s"(s));
+    return v;
+}
+__device__ __forceinline__ int32_t requant_acc(int32_t acc, const ChanScale &c, const RescaleParams &p, int32_t hi_v) {
+    const int32_t fix = (int32_t)((uint64_t)c.round_neg - (uint64_t)c.round_pos);
+    const int64_t r = (int64_t)(int32_t)((uint32_t)acc >> 31) * (int64_t)fix + c.round_pos;
+    const uint64_t t = (uint64_t)((int64_t)acc * (int64_t)c.mult) + (uint64_t)r;
+    int32_t v = (int32_t)((int64_t)t >> c.shift);
+    v = (int32_t)((uint32_t)v + (uint32_t)p.out_zp);
+    int32_t clamped;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(clamped) : "v"(v), "s"(p.out_lo), "v"(hi_v));
+    return clamped;
+}
+
 int make_rescale_params(const mlel_rescale_attr *attr, int in_dtype, int out_dtype, const mlel_clamp_attr *clamp,
                         RescaleParams *out);
 int check_scale_tensors(const mlel_tensor *mult, const mlel_tensor *shift, const mlel_rescale_attr *attr,

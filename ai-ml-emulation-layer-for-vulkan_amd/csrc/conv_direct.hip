@@ -284,6 +284,7 @@ typedef int v4i32 __attribute__((ext_vector_type(4)));
 
 template <int NJ, int KC>
 __global__ void __launch_bounds__(kBlock) conv_rows_mfma_i8_kernel(const RowsMfmaArgs a) {
+    const int32_t hi_v = pin_vgpr(a.scale.p.out_hi);
     extern __shared__ __align__(16) char smem[];
     ChanConst *cc = reinterpret_cast<ChanConst *>(smem);  // [NJ * 32], channels at or beyond OC hold zeros
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -379,7 +380,7 @@ __global__ void __launch_bounds__(kBlock) conv_rows_mfma_i8_kernel(const RowsMfm
                 int32_t v[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    v[e] = requant_acc(acc[4 * q + e], c.q, a.scale.p);
+                    v[e] = requant_acc(acc[4 * q + e], c.q, a.scale.p, hi_v);
                 }
                 const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
                 const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
@@ -494,6 +495,7 @@ template <int NJ, int KC, int KC0>
 __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(NJ <= 3 ? 3 : 2, NJ <= 3 ? 3 : 2)))
 conv_rows2_mfma_i8_kernel(const Rows2Args b) {
     const RowsMfmaArgs &a = b.r;
+    const int32_t hi_v = pin_vgpr(a.scale.p.out_hi), hi0_v = pin_vgpr(b.scale0.p.out_hi);
     extern __shared__ __align__(16) char smem[];
     ChanConst *cc = reinterpret_cast<ChanConst *>(smem);  // [NJ * 32] second operator, then [32] first operator
     ChanConst *cc0 = cc + NJ * 32;
@@ -612,7 +614,7 @@ conv_rows2_mfma_i8_kernel(const Rows2Args b) {
             for (int q = 0; q < 4; q++) {
                 int32_t v[4];
 #pragma unroll
-                for (int e = 0; e < 4; e++) v[e] = requant_acc(acc0[4 * q + e], c0.q, b.scale0.p);
+                for (int e = 0; e < 4; e++) v[e] = requant_acc(acc0[4 * q + e], c0.q, b.scale0.p, hi0_v);
                 const uint32_t p = pack4(v);
                 if (mid_col_live) *reinterpret_cast<uint32_t *>(mt_lane + 8 * q * OC0) = p;
             }
@@ -648,7 +650,7 @@ conv_rows2_mfma_i8_kernel(const Rows2Args b) {
             for (int q = 0; q < 4; q++) {
                 int32_t v[4];
 #pragma unroll
-                for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[4 * q + e], c.q, a.scale.p);
+                for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[4 * q + e], c.q, a.scale.p, hi_v);
                 const uint32_t p = pack4(v);
                 if (col_live) *reinterpret_cast<uint32_t *>(so_lane + 8 * q * a.op + j * 32) = p;
             }
@@ -715,6 +717,7 @@ struct StemMfmaArgs {
 };
 
 __global__ void __launch_bounds__(kBlock) conv_stem_mfma_i8_kernel(const StemMfmaArgs a) {
+    const int32_t hi_v = pin_vgpr(a.scale.p.out_hi);
     extern __shared__ __align__(16) char smem[];
     ChanConst *cc = reinterpret_cast<ChanConst *>(smem);  // [32], channels at or beyond OC hold zeros
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -846,7 +849,7 @@ __global__ void __launch_bounds__(kBlock) conv_stem_mfma_i8_kernel(const StemMfm
         for (int q = 0; q < 4; q++) {
             int32_t v[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[4 * q + e], c.q, a.scale.p);
+            for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[4 * q + e], c.q, a.scale.p, hi_v);
             const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
             const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
             uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // bytes = positions e of this lane's channel

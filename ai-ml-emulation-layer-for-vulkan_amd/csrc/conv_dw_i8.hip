@@ -100,6 +100,7 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
     const int p_lo = y_lo * a.W, p_count = (y_hi - y_lo) * a.W;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cl = lane & 31, half = lane >> 5;
+    const int32_t hi1_v = pin_vgpr(a.s1.p.out_hi), hi2_v = pin_vgpr(a.s2.p.out_hi);
 
     // ---- requests first: the slice's weights (matrix B operand: lane = channel lane % 32, 16 bytes of K from
     // 32 kc + 16 (lane / 32)) and the wavefront's first position group
@@ -181,7 +182,7 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
         for (int q = 0; q < 4; q++) {
             int32_t v[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[4 * q + e], q1, a.s1.p);
+            for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[4 * q + e], q1, a.s1.p, hi1_v);
             const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
             const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
             uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // bytes = positions e of this lane's channel
@@ -290,7 +291,7 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
                 if (ox >= a.OW) break;
                 int32_t v[4];
 #pragma unroll
-                for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[ty][t][e], q2[e], a.s2.p);
+                for (int e = 0; e < 4; e++) v[e] = requant_acc(acc[ty][t][e], q2[e], a.s2.p, hi2_v);
                 const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
                 const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
                 const uint32_t off = (orow + (uint32_t)ox) * (uint32_t)a.C + c;

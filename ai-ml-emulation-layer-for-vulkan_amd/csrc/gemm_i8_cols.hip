@@ -166,13 +166,15 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
     const int32_t sw = wsum + __shfl_xor(wsum, 32);
     const int32_t bias_adj = (int32_t)((uint32_t)bias - (uint32_t)g.zx * (uint32_t)sw);
     const ChanScale cs = make_chan_scale(mult, shift, g.rp);
+    const int32_t hi_v = pin_vgpr(g.rp.out_hi), hi_out_v = RES ? pin_vgpr(g.rs_out.p.out_hi) : 0;
+    (void)hi_out_v;
     const uint32_t sel_a = (lane & 1) ? 0x03070105u : 0x06020400u;  // exchange with lane ^ 1
     const uint32_t sel_b = (lane & 2) ? 0x03020706u : 0x05040100u;  // exchange with lane ^ 2
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
         int32_t v[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) v[e] = requant_acc((int32_t)((uint32_t)own[4 * q + e] + (uint32_t)bias_adj), cs, g.rp);
+        for (int e = 0; e < 4; e++) v[e] = requant_acc((int32_t)((uint32_t)own[4 * q + e] + (uint32_t)bias_adj), cs, g.rp, hi_v);
         const uint32_t lo = __builtin_amdgcn_perm((uint32_t)v[1], (uint32_t)v[0], 0x0c0c0400u);
         const uint32_t hi = __builtin_amdgcn_perm((uint32_t)v[3], (uint32_t)v[2], 0x0c0c0400u);
         uint32_t p = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
@@ -187,7 +189,7 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int32_t r1 = lds_entry(res_tab[0], xw, e), r2 = lds_entry(res_tab[1], p, e);
-                o4[e] = requant_acc((int32_t)((uint32_t)r1 + (uint32_t)r2), q_out, g.rs_out.p);
+                o4[e] = requant_acc((int32_t)((uint32_t)r1 + (uint32_t)r2), q_out, g.rs_out.p, hi_out_v);
             }
             const uint32_t l2 = __builtin_amdgcn_perm((uint32_t)o4[1], (uint32_t)o4[0], 0x0c0c0400u);
             const uint32_t h2 = __builtin_amdgcn_perm((uint32_t)o4[3], (uint32_t)o4[2], 0x0c0c0400u);
@@ -278,12 +280,13 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_pool_i8_kernel(const Gem
     const int32_t sw = wsum + __shfl_xor(wsum, 32);
     const int32_t bias_adj = (int32_t)((uint32_t)bias - (uint32_t)g.zx * (uint32_t)sw);
     const ChanScale cs = make_chan_scale(mult, shift, g.rp);
+    const int32_t hi_v = pin_vgpr(g.rp.out_hi);
     int32_t sum = 0;
 #pragma unroll
     for (int q = 0; q < 4; q++)
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const int32_t v = requant_acc((int32_t)((uint32_t)acc[4 * q + e] + (uint32_t)bias_adj), cs, g.rp);
+            const int32_t v = requant_acc((int32_t)((uint32_t)acc[4 * q + e] + (uint32_t)bias_adj), cs, g.rp, hi_v);
             sum += (32 * t + 8 * q + 4 * half + e < pa.positions) ? v : 0;
         }
     sum += __shfl_xor(sum, 32);

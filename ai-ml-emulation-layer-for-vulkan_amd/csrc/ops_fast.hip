@@ -295,6 +295,7 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
     }
 
     // ---- epilogue
+    const int32_t hi_v = pin_vgpr(a.scale.p.out_hi);
     const __amdgpu_buffer_rsrc_t ores = __builtin_amdgcn_make_buffer_rsrc(a.out, 0, (int)a.o_bytes, 0x00020000);
     const uint32_t esz = Q8 ? 1u : (uint32_t)a.out_size;
 #pragma unroll
@@ -311,7 +312,7 @@ __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
             for (int e = 0; e < 4; e++) {
                 int32_t s = acc[ty][t][e];
                 if (ZW) s = (int32_t)((uint32_t)s - (uint32_t)a.zw * (uint32_t)xs[ty][t][e]);
-                if (Q8 || a.fused) s = requant_acc(s, q[e], a.scale.p);
+                if (Q8 || a.fused) s = requant_acc(s, q[e], a.scale.p, hi_v);
                 v[e] = s;
             }
             const uint32_t off = ((orow + (uint32_t)ox) * (uint32_t)a.C + (uint32_t)c) * esz;
