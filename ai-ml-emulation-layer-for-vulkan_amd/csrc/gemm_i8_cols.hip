@@ -57,12 +57,15 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const Gem
     const uint32_t xoff = m < g.M ? (uint32_t)m * (uint32_t)g.x_sx + (uint32_t)half * 16u : kOobOffset;
     const uint32_t woff = n < g.N ? (uint32_t)n * (uint32_t)g.ldw + (uint32_t)half * 16u : kOobOffset;
     auto fetch = [&](int round, v4i (&xf)[KR], v4i (&wf)[KR]) {
+        // a round wholly inside K needs no test: the offset of a row outside the tensor stays beyond the buffer's
+        // extent when k is added to it (kOobOffset + k < 2^32), and such loads return zeros
+        const bool whole = (round + 1) * KR * 32 <= g.K;  // uniform
 #pragma unroll
         for (int c = 0; c < KR; c++) {
             const int k = (round * KR + c) * 32;
-            const bool in = k + half * 16 < g.K;  // K % 16 == 0: a piece lies wholly inside or outside the row
-            const uint4 xv = buf_load16(xres, (in && xoff != kOobOffset) ? xoff + (uint32_t)k : kOobOffset);
-            const uint4 wv = buf_load16(wres, (in && woff != kOobOffset) ? woff + (uint32_t)k : kOobOffset);
+            const bool in = whole || k + half * 16 < g.K;  // K % 16 == 0: a piece lies wholly inside or outside the row
+            const uint4 xv = buf_load16(xres, in ? xoff + (uint32_t)k : kOobOffset);
+            const uint4 wv = buf_load16(wres, in ? woff + (uint32_t)k : kOobOffset);
             xf[c] = v4i{(int)xv.x, (int)xv.y, (int)xv.z, (int)xv.w};
             wf[c] = v4i{(int)wv.x, (int)wv.y, (int)wv.z, (int)wv.w};
         }
@@ -236,9 +239,9 @@ __global__ void __launch_bounds__(kColsBlock) conv_cols_pool_i8_kernel(const Gem
 #pragma unroll
         for (int c = 0; c < KR; c++) {
             const int k = (round * KR + c) * 32;
-            const bool in = k + half * 16 < g.K;
-            const uint4 xv = buf_load16(xres, (in && xoff != kOobOffset) ? xoff + (uint32_t)k : kOobOffset);
-            const uint4 wv = buf_load16(wres, (in && woff != kOobOffset) ? woff + (uint32_t)k : kOobOffset);
+            const bool in = k + half * 16 < g.K;  // (a row outside the tensor: kOobOffset + k stays beyond the extent)
+            const uint4 xv = buf_load16(xres, in ? xoff + (uint32_t)k : kOobOffset);
+            const uint4 wv = buf_load16(wres, in ? woff + (uint32_t)k : kOobOffset);
             xf[c] = v4i{(int)xv.x, (int)xv.y, (int)xv.z, (int)xv.w};
             wf[c] = v4i{(int)wv.x, (int)wv.y, (int)wv.z, (int)wv.w};
         }
