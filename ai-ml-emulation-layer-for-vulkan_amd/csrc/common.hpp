@@ -403,6 +403,16 @@ __host__ __device__ inline ChanScale make_chan_scale(int32_t mult, int32_t shift
     const uint64_t round = base - (uint64_t)(int64_t)p.in_zp * (uint64_t)(int64_t)mult;
     c.round_pos = (int64_t)(round + nudge);
     c.round_neg = (int64_t)(round - nudge);
+#if defined(__HIP_DEVICE_COMPILE__)
+    {
+        // In a kernel the compiler sees how the two constants were made and would multiply their exact 64-bit
+        // difference by the sign bit with two unsigned 64-bit multiply-adds per value (requant_acc); as an opaque
+        // pair of registers the difference is truncated to 32 bits there and the product is one v_mad_i64_i32.
+        int32_t lo = (int32_t)(uint32_t)(uint64_t)c.round_neg, hi = (int32_t)((uint64_t)c.round_neg >> 32);
+        asm volatile("" : "+v"(lo), "+v"(hi));
+        c.round_neg = (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo);
+    }
+#endif
     return c;
 }
 

@@ -165,12 +165,6 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
         bias_adj1 = (int32_t)((uint32_t)bias - (uint32_t)a.zx * (uint32_t)wsum);
         const int ci = a.s1.p.per_channel ? ch : 0;
         q1 = make_chan_scale(load_mult(a.s1, ci), (int32_t)a.s1.shift[ci], a.s1.p);
-        // The compiler sees how the two rounding constants were made and would multiply their exact 64-bit difference
-        // by the sign bit with two unsigned 64-bit multiply-adds per value; as an opaque pair of registers the
-        // difference is truncated to 32 bits (requant_acc) and the product is one v_mad_i64_i32.
-        int32_t lo = (int32_t)(uint32_t)(uint64_t)q1.round_neg, hi = (int32_t)((uint64_t)q1.round_neg >> 32);
-        asm volatile("" : "+v"(lo), "+v"(hi));
-        q1.round_neg = (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo);
     }
     __syncthreads();  // the fill is complete before any position is written
 
