@@ -15,7 +15,8 @@ GraphPipeline, the roofline position of the dominant kernel and a CPU baseline (
 graph 200 times back to back and nothing else, so that counters of a single layer can be collected), `standalone`
 (the bandwidth-bound operators as stand-alone launches on config 2's and on config 3's largest tensors), `copy` (the
 plain copy kernel over grid and size: the measured HBM ceiling), `extra` (data-movement operators outside the
-benchmark graphs).  `ms_per_step` is the median over at least 10 rounds of `--steps` launches; the whole-graph legs
+benchmark graphs), `vendor` (the GPU vendor's matrix library through torch on the products timed here, as a calibration
+of the box; nothing of the product runs in that leg).  `ms_per_step` is the median over at least 10 rounds of `--steps` launches; the whole-graph legs
 report the median over rounds that hold at least 50 graphs.
 """
 import re
@@ -544,6 +545,56 @@ def bench_extra(dev, abi, reps=50):
     return out
 
 
+def bench_vendor_library():
+    """The GPU vendor's matrix library (through torch._int_mm / torch.matmul) on the shapes this file times, on the same
+    box: a calibration of what the hardware gives a tuned library, not part of the product (which links no BLAS).  The
+    int8 product there is plain: int32 result, no zero points, no RESCALE."""
+    import torch
+
+    def med_us(fn, n, rounds=5):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t = []
+        for _ in range(rounds):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for _ in range(n):
+                fn()
+            e.record()
+            torch.cuda.synchronize()
+            t.append(s.elapsed_time(e) / n * 1e3)
+        return sorted(t)[len(t) // 2]
+
+    rows = []
+    dev = "cuda:0"
+    for m, k, n, reps in ((4096, 1024, 1024, 200), (4096, 4096, 4096, 10), (8192, 8192, 8192, 5)):
+        a = torch.randint(-128, 128, (m, k), dtype=torch.int8, device=dev)
+        b = torch.randint(-128, 128, (k, n), dtype=torch.int8, device=dev)
+        for layout, bb in (("B [K][N]", b), ("B [N][K]", b.t().contiguous().t())):
+            try:
+                us = med_us(lambda: torch._int_mm(a, bb), reps)
+                rows.append({"product": f"int8 {m}x{k}x{n}", "layout": layout, "us": round(us, 2),
+                             "tops": round(2.0 * m * k * n / us / 1e6, 1)})
+            except Exception as e:
+                rows.append({"product": f"int8 {m}x{k}x{n}", "layout": layout, "error": repr(e)[:160]})
+            log("vendor:", rows[-1])
+    for m, k, n in ((4096, 768, 768), (4096, 768, 2304), (4096, 768, 3072), (4096, 3072, 768), (8192, 8192, 8192)):
+        a = torch.randn(m, k, dtype=torch.float16, device=dev)
+        b = torch.randn(k, n, dtype=torch.float16, device=dev)
+        for layout, bb in (("B [K][N]", b), ("B [N][K]", b.t().contiguous().t())):
+            us = med_us(lambda: torch.matmul(a, bb), 20 if m < 8192 else 5)
+            rows.append({"product": f"fp16 {m}x{k}x{n}", "layout": layout, "us": round(us, 2),
+                         "tflops": round(2.0 * m * k * n / us / 1e6, 1)})
+            log("vendor:", rows[-1])
+    q = torch.randn(96, 512, 64, dtype=torch.float16, device=dev)
+    kt = torch.randn(96, 64, 512, dtype=torch.float16, device=dev)
+    rows.append({"product": "fp16 scores only, 96 heads x (512x64 . 64x512)", "layout": "batched",
+                 "us": round(med_us(lambda: torch.bmm(q, kt), 20), 2)})
+    log("vendor:", rows[-1])
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -554,12 +605,17 @@ def main():
                     help="omit the legs with several launches / sessions in flight (profiling runs: one kernel at a time)")
     ap.add_argument("--skip-graph", action="store_true", help="omit the MobileNetV2 and encoder graph legs")
     ap.add_argument("--only", choices=["all", "config0", "config1", "config2", "mobilenetv2", "encoder", "gemm_large",
-                                       "layer", "standalone", "copy", "extra"], default="all")
+                                       "layer", "standalone", "copy", "extra", "vendor"], default="all")
     ap.add_argument("--layer", type=int, default=3, help="with --only layer: position in the fused config 3 graph")
     ap.add_argument("--gemm-size", type=int, default=0, help="with --only gemm_large: this one size instead of 4096 and 8192")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    if args.only == "vendor":
+        print(json.dumps({"only": "vendor", "library": "torch._int_mm / torch.matmul / torch.bmm",
+                          "products": bench_vendor_library()}), flush=True)
+        return
 
     abi = importlib.import_module(PKG + ".abi")
     hb = importlib.import_module(PKG + ".hip_backend")
