@@ -25,8 +25,11 @@ constexpr int kOutAux = MLEL_OUT_AUX;
 __device__ __forceinline__ void store16_result(void *p, uint4 v) {
     typedef unsigned int u32x4_st __attribute__((ext_vector_type(4)));
     const u32x4_st d = {v.x, v.y, v.z, v.w};
+    // The two wait states behind the store belong to it: a store of more than eight bytes reads its data registers
+    // after it has issued, and a vector instruction that overwrites them within two wait states changes what is
+    // stored.  The compiler keeps that distance for the stores it emits itself; it cannot see into this one.
     if (kOutAux == 17)
-        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(d) : "memory");
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(d) : "memory");
     else
         *reinterpret_cast<uint4 *>(p) = v;
 }
