@@ -268,7 +268,7 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
                     __builtin_amdgcn_sched_barrier(0);
                     fold(a);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (set + 2 < sets) fetch(a, set + 2);  // uniform
+                    fetch(a, min(set + 2, sets - 1));  // unconditional (the last one is not used): the sets keep their registers
                     __builtin_amdgcn_sched_barrier(0);
                     fold(b);
                     __builtin_amdgcn_sched_barrier(0);

@@ -1097,11 +1097,12 @@ struct RowStaticArgs {
     int32_t cols, tpr_log;
     const char *in[MLEL_CHAIN_MAX_INPUTS];
 };
-constexpr int kRowStaticPieces = 4;
+constexpr int kRowStaticPieces = 4;      // pieces per thread and value when a row is spread as widely as it goes
+constexpr int kRowStaticMaxPieces = 12;  // the most a thread holds when rows are packed more densely into wavefronts
 
-template <class P>
+template <class P, int NP>
 struct RowStaticState {
-    uint4 f[P::n_full][kRowStaticPieces];
+    uint4 f[P::n_full][NP];
     uint32_t r[P::n_row];              // a per-row value, the half in both halves of the word
     uint32_t one[P::n_inputs];         // single-element inputs, likewise
     const RowStaticArgs *g;
@@ -1113,8 +1114,8 @@ struct RowStaticState {
 
 __device__ __forceinline__ uint4 splat_word(uint32_t w) { return make_uint4(w, w, w, w); }
 
-template <class P, int V>
-__device__ __forceinline__ uint4 row_static_piece(const RowStaticState<P> &c, int u) {
+template <class P, int NP, int V>
+__device__ __forceinline__ uint4 row_static_piece(const RowStaticState<P, NP> &c, int u) {
     if constexpr (P::cls[V] == SC_FULL) {
         return c.f[P::slot[V]][u];
     } else if constexpr (P::cls[V] == SC_ROW) {
@@ -1127,8 +1128,8 @@ __device__ __forceinline__ uint4 row_static_piece(const RowStaticState<P> &c, in
     }
 }
 
-template <class P, int S>
-__device__ __forceinline__ void row_static_run(RowStaticState<P> &c) {
+template <class P, int NP, int S>
+__device__ __forceinline__ void row_static_run(RowStaticState<P, NP> &c) {
     if constexpr (S < P::n_steps) {
         constexpr int OP = P::steps[S].op, A = P::steps[S].a, B = P::steps[S].b, V = P::n_inputs + S;
         constexpr bool last = S + 1 == P::n_steps;
@@ -1137,13 +1138,16 @@ __device__ __forceinline__ void row_static_run(RowStaticState<P> &c) {
             // lanes of one wavefront, whose shared-memory operations complete in program order
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
 #pragma unroll
-            for (int u = 0; u < kRowStaticPieces; u++) {
+            for (int u = 0; u < NP; u++) {
                 const int sg = c.part + u * c.tpr;
                 if (sg < c.segs) *reinterpret_cast<uint4 *>(c.stage + sg * 16) = c.f[P::slot[A]][u];
             }
             __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __half acc = f2h(0.f);
+            // lgkmcnt(0): no scalar load of a kernel argument is left in flight.  With one pending the compiler cannot
+            // count shared-memory reads (scalar loads return out of order) and waits for all of them at every use.
+            __builtin_amdgcn_s_waitcnt(0xc07f);
             if (c.part == 0) {
                 const auto add8 = [&](const uint4 &raw) {
                     const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
@@ -1157,23 +1161,34 @@ __device__ __forceinline__ void row_static_run(RowStaticState<P> &c) {
 #pragma unroll
                     for (int t = 0; t < 4; t++) v[t] = *reinterpret_cast<const uint4 *>(c.stage + (first + t) * 16);
                 };
-                int sg = 0;
-                uint4 even[4], odd[4];
-                if (c.segs >= 4) load4(even, 0);
-                for (; sg + 8 <= c.segs; sg += 8) {
-                    load4(odd, sg + 4);
+                // batches of four pieces, two register sets: while one is added the other is on its way.  Every load is
+                // issued unconditionally (the last one of an even count reads the last batch again and is not used),
+                // so the sets keep their registers and the waits count exactly the loads of the other set.
+                const int n4 = c.segs >> 2;
+                int done = 0;
+                if (n4 >= 2) {
+                    uint4 even[4], odd[4];
+                    int i = 0;
+                    load4(even, 0);
+                    for (; i + 2 <= n4; i += 2) {
+                        load4(odd, (i + 1) * 4);
+                        __builtin_amdgcn_sched_barrier(0);  // the loads first: they travel while the other set is added
 #pragma unroll
-                    for (int t = 0; t < 4; t++) add8(even[t]);
-                    if (sg + 12 <= c.segs) load4(even, sg + 8);
+                        for (int t = 0; t < 4; t++) add8(even[t]);
+                        __builtin_amdgcn_sched_barrier(0);
+                        load4(even, min(i + 2, n4 - 1) * 4);
+                        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int t = 0; t < 4; t++) add8(odd[t]);
+                        for (int t = 0; t < 4; t++) add8(odd[t]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    if (i < n4) {
+#pragma unroll
+                        for (int t = 0; t < 4; t++) add8(even[t]);
+                    }
+                    done = n4 * 4;
                 }
-                if (sg + 4 <= c.segs) {
-#pragma unroll
-                    for (int t = 0; t < 4; t++) add8(even[t]);
-                    sg += 4;
-                }
-                for (; sg < c.segs; sg++) add8(*reinterpret_cast<const uint4 *>(c.stage + sg * 16));
+                for (int sg = done; sg < c.segs; sg++) add8(*reinterpret_cast<const uint4 *>(c.stage + sg * 16));
             }
             __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
             __builtin_amdgcn_wave_barrier();
@@ -1186,7 +1201,7 @@ __device__ __forceinline__ void row_static_run(RowStaticState<P> &c) {
             h2_t m2 = {(_Float16)-65504.f, (_Float16)-65504.f};
             uint32_t special = 0;
 #pragma unroll
-            for (int u = 0; u < kRowStaticPieces; u++) {
+            for (int u = 0; u < NP; u++) {
                 const int sg = c.part + u * c.tpr;
                 if (sg >= c.segs) continue;
                 const uint4 raw = c.f[P::slot[A]][u];
@@ -1204,13 +1219,13 @@ __device__ __forceinline__ void row_static_run(RowStaticState<P> &c) {
             const uint32_t bits = (uint32_t)__half_as_ushort(f2h(special != 0 ? __builtin_nanf("") : mx));
             c.r[P::slot[V]] = bits | (bits << 16);
         } else if constexpr (P::cls[V] == SC_ROW) {
-            uint4 r = static_apply<OP>(row_static_piece<P, A>(c, 0), row_static_piece<P, B>(c, 0));
+            uint4 r = static_apply<OP>(row_static_piece<P, NP, A>(c, 0), row_static_piece<P, NP, B>(c, 0));
             asm volatile("" : "+v"(r.x));  // rounded here, as the stand-alone operator rounds: no contraction across steps
             c.r[P::slot[V]] = r.x;
         } else {
 #pragma unroll
-            for (int u = 0; u < kRowStaticPieces; u++) {
-                uint4 r = static_apply<OP>(row_static_piece<P, A>(c, u), row_static_piece<P, B>(c, u));
+            for (int u = 0; u < NP; u++) {
+                uint4 r = static_apply<OP>(row_static_piece<P, NP, A>(c, u), row_static_piece<P, NP, B>(c, u));
                 asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
                 if constexpr (last) {
                     const int sg = c.part + u * c.tpr;
@@ -1221,17 +1236,17 @@ __device__ __forceinline__ void row_static_run(RowStaticState<P> &c) {
                 }
             }
         }
-        row_static_run<P, S + 1>(c);
+        row_static_run<P, NP, S + 1>(c);
     }
 }
 
 // the full inputs into registers (four pieces requested at once), the single elements into both halves of a word
-template <class P, int K>
-__device__ __forceinline__ void row_static_load(RowStaticState<P> &c) {
+template <class P, int NP, int K>
+__device__ __forceinline__ void row_static_load(RowStaticState<P, NP> &c) {
     if constexpr (K < P::n_inputs) {
         if constexpr (P::cls[K] == SC_FULL) {
 #pragma unroll
-            for (int u = 0; u < kRowStaticPieces; u++) {
+            for (int u = 0; u < NP; u++) {
                 const int sg = c.part + u * c.tpr;
                 c.f[P::slot[K]][u] = (c.live && sg < c.segs)
                                          ? *reinterpret_cast<const uint4 *>(c.g->in[K] + (c.row * c.g->cols + sg * 8) * 2)
@@ -1241,14 +1256,14 @@ __device__ __forceinline__ void row_static_load(RowStaticState<P> &c) {
             const uint32_t bits = *reinterpret_cast<const uint16_t *>(c.g->in[K]);
             c.one[K] = bits | (bits << 16);
         }
-        row_static_load<P, K + 1>(c);
+        row_static_load<P, NP, K + 1>(c);
     }
 }
 
-template <class P>
+template <class P, int NP>
 __global__ void __launch_bounds__(kBlock) row_static_f16_kernel(const RowStaticArgs g) {
     extern __shared__ __align__(16) char lds[];
-    RowStaticState<P> c;
+    RowStaticState<P, NP> c;
     c.g = &g;
     c.tpr = 1 << g.tpr_log;
     c.part = (int)threadIdx.x & (c.tpr - 1);
@@ -1257,8 +1272,8 @@ __global__ void __launch_bounds__(kBlock) row_static_f16_kernel(const RowStaticA
     c.live = c.row < g.rows;
     c.segs = g.cols >> 3;
     c.stage = lds + rr * (g.cols * 2 + 16);
-    row_static_load<P, 0>(c);
-    row_static_run<P, 0>(c);
+    row_static_load<P, NP, 0>(c);
+    row_static_run<P, NP, 0>(c);
 }
 
 // the chain is P's program over inputs of P's shapes (`classes`: the RowClass of every input, `ops`: FOp / F_RED_*)
@@ -1276,6 +1291,16 @@ bool matches_row_static(const mlel_chain *c, const int8_t *classes, const int *o
     return true;
 }
 
+template <class P, int NP>
+int launch_row_static_pieces(hipStream_t s, const RowStaticArgs &g, int64_t rows, int64_t cols) {
+    const int64_t rows_per_block = kBlock >> g.tpr_log;
+    const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+    MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "row chain: too many rows");
+    const size_t smem = (size_t)rows_per_block * (size_t)(cols * 2 + 16);
+    row_static_f16_kernel<P, NP><<<dim3((unsigned)blocks), dim3(kBlock), smem, s>>>(g);
+    return check_launch("row chain (compiled program)");
+}
+
 template <class P>
 int launch_row_static(hipStream_t s, const mlel_tensor *out, const mlel_chain *c, int64_t rows, int64_t cols) {
     RowStaticArgs g{};
@@ -1284,15 +1309,21 @@ int launch_row_static(hipStream_t s, const mlel_tensor *out, const mlel_chain *c
     g.cols = (int32_t)cols;
     const int64_t segs = cols / 8;
     int tpr_log = 0;
-    while ((int64_t(kRowStaticPieces) << tpr_log) < segs) tpr_log++;  // at most four pieces per thread
+    while ((int64_t(kRowStaticPieces) << tpr_log) < segs) tpr_log++;  // as wide as a row goes: four pieces per thread
+    // The left-to-right fold of a REDUCE_SUM is issued once per wavefront whatever the number of rows in it.  One
+    // wavefront alone issues a vector instruction every 6.5 clocks (measured: dependent or not), a SIMD takes one
+    // every 4: two wavefronts fold side by side on a SIMD at full speed each, a third slows all three.  Rows are
+    // therefore packed more densely (fewer threads per row, more pieces per thread) until there are at most two
+    // wavefronts per SIMD of the device (256 compute units of four) or a thread is full.
+    const auto pieces = [&](int log) { return (segs + (int64_t(1) << log) - 1) >> log; };
+    const auto wavefronts = [&](int log) { return (rows + (64 >> log) - 1) / (64 >> log); };
+    while (tpr_log > 0 && wavefronts(tpr_log) > 2048 && pieces(tpr_log - 1) <= kRowStaticMaxPieces) tpr_log--;
     g.tpr_log = tpr_log;
     for (int k = 0; k < c->n_inputs; k++) g.in[k] = static_cast<const char *>(c->inputs[k]->ptr);
-    const int64_t rows_per_block = kBlock >> tpr_log;
-    const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-    MLEL_REQUIRE(blocks < (int64_t(1) << 31), MLEL_ERR_LIMIT, "row chain: too many rows");
-    const size_t smem = (size_t)rows_per_block * (size_t)(cols * 2 + 16);
-    row_static_f16_kernel<P><<<dim3((unsigned)blocks), dim3(kBlock), smem, s>>>(g);
-    return check_launch("row chain (compiled program)");
+    const int64_t np = pieces(tpr_log);
+    if (np <= 4) return launch_row_static_pieces<P, 4>(s, g, rows, cols);
+    if (np <= 8) return launch_row_static_pieces<P, 8>(s, g, rows, cols);
+    return launch_row_static_pieces<P, kRowStaticMaxPieces>(s, g, rows, cols);
 }
 
 }  // namespace

@@ -655,7 +655,8 @@ def _same_bits_or_both_nan(got, want):
     np.testing.assert_array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
 
 
-@pytest.mark.parametrize("shape", [(2, 48, 768), (5, 1, 64), (300, 8), (3, 2048), (1, 1, 4096), (16384, 768), (777, 1016)], ids=str)
+@pytest.mark.parametrize("shape", [(2, 48, 768), (5, 1, 64), (300, 8), (3, 2048), (1, 1, 4096), (16384, 768), (777, 1016),
+                                   (8192, 768), (2100, 1000)], ids=str)
 def test_chain_with_reductions_layernorm(run, shape):
     """LayerNorm as the operators a TOSA graph spells it with (REDUCE_SUM, MUL 1/N, SUB, MUL, REDUCE_SUM, MUL 1/N,
     ADD eps, RSQRT, MUL, MUL gamma, ADD beta), in one mlel_hip_elementwise_chain call against the eleven stand-alone
@@ -1763,7 +1764,8 @@ def test_fp16_products_keep_the_sign_of_zero(run, oracle):
                                   oracle.reduce("PRODUCT", rows, 1).view(np.uint16))
 
 
-@pytest.mark.parametrize("shape", [(3, 70, 512), (2, 5, 7, 64), (130, 1024), (4, 8)], ids=str)
+@pytest.mark.parametrize("shape", [(3, 70, 512), (2, 5, 7, 64), (130, 1024), (4, 8), (12000, 512), (9000, 776),
+                                   (20000, 768)], ids=str)
 def test_softmax_rows_equals_the_six_operators(run, shape):
     """REDUCE_MAX, SUB, EXP, REDUCE_SUM, RECIPROCAL, MUL in one pass == the six stand-alone kernels, bit for bit, on
     ordinary rows and on rows with NaN, infinities, signed zeros and a constant row.  Where the result is NaN only
