@@ -182,11 +182,16 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
             }
             __syncthreads();
             // this pass's scores into registers, through the scale; the maximum as they pass
+            // (all of a pass's pieces are requested before the first is used, also those beyond a short row, which are
+            // inside the pass buffer and not used: one shared-memory round trip per pass instead of one per piece)
+            uint4 raw[kPassPieces];
+#pragma unroll
+            for (int uu = 0; uu < kPassPieces; uu++) raw[uu] = *reinterpret_cast<const uint4 *>(myrow + piece_off(h, uu));
 #pragma unroll
             for (int uu = 0; uu < kPassPieces; uu++) {
                 const int u = h * kPassPieces + uu;
                 if (u < ppt) {
-                    uint4 x = *reinterpret_cast<const uint4 *>(myrow + piece_off(h, uu));
+                    uint4 x = raw[uu];
                     if (SCALED) {
                         x = static_apply<F_MUL>(x, make_uint4(scale_w, scale_w, scale_w, scale_w));
                         asm volatile("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));

@@ -662,120 +662,205 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             else
                 w_base[kk] = smem + BM * BK + (wave_n * WN + (lane & 31)) * BK + slot;
         }
-        auto read_frags = [&](int buf, int kk, v4i(&xf)[TM], v4i(&wf)[TN]) {
+        // ---- the loop.  A wavefront issues in order and is alone on its SIMD here, so whatever is not a matrix
+        // instruction delays the next one unless it is issued while the matrix core works on the last (35 clocks
+        // per instruction on random operands).  Measured on one wavefront per SIMD: shared-memory reads, loads into
+        // shared memory and ordinary vector instructions (v_add, v_xor, v_sad_u8) issue in that shadow for free;
+        // v_dot4 does not (a dot product and a matrix instruction take turns), and four loads issued back to back
+        // hold the wavefront for 3 x 64 clocks (the address path takes a wavefront's kilobyte in 64).  A K half is
+        // therefore one straight line: a matrix instruction, then a share of the next half's operand reads, of the
+        // requests and of the zero-point sums, then the next matrix instruction.  (Steps of 0.40 us became 0.22 us
+        // on 8 x 512 x 1024 x 1024; the requests alone, with the same barrier and waits, take 0.165 us per step.)
+        //
+        // Zero-point sums on the matrix cores, one small instruction per operand fragment: the 16 bytes a lane holds
+        // for v_mfma_i32_32x32x32_i8 (row lane % 32, K bytes 16 (lane / 32) ...) are, read as an operand of
+        // v_mfma_i32_16x16x64_i8 (row lane % 16, K block lane / 16), row r of the fragment in K blocks 0 and 2 of row
+        // r % 16 when r < 16 and in blocks 1 and 3 when r >= 16.  Against a constant operand that is all ones in
+        // blocks 0 and 2 for its first eight columns and in blocks 1 and 3 for the other eight, the 16 x 16 result holds
+        // sum_k of row r (< 16) in columns 0 - 7 and of row r + 16 in columns 8 - 15: four accumulator registers and
+        // 16 clocks of the matrix core per fragment, where v_dot4 takes four instructions that take turns with the
+        // matrix instructions and v_xor + v_sad_u8 eight that crowd the issue stream (measured per K step of a
+        // 128 x 128 tile: about 35 clocks against 217 and 142).  Which wavefront sums what in which
+        // K half (wave-uniform, fixed for the kernel): with 2 x 2 wavefronts the two that share a row panel take one
+        // K half each and so do the two that share a channel panel, arranged so that every wavefront has exactly one
+        // of the two duties in every half; otherwise the first two wavefront columns take the row panels' halves
+        // and the wavefront rows the channel panels' halves.
+        const int sel_w = (((lane & 15) < 8) != (((lane >> 4) & 1) != 0)) ? 0x01010101 : 0;
+        const v4i selv = v4i{sel_w, sel_w, sel_w, sel_w};
+        v4i sx4[TM], sw4[TN];
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-                xf[i] = *reinterpret_cast<const v4i *>(x_base[kk] + buf * DL_STAGE + i * 32 * BK);
+        for (int i = 0; i < TM; i++) sx4[i] = v4i{0, 0, 0, 0};
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-                if (WMODE == W_KMAJOR_DL) {
-                    const char *p = w_base[kk] + buf * DL_STAGE + (((wave_n * WN / 32 + j) ^ kfun) * 32);
-                    const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(p));
-                    const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(p + 8 * BN));
-                    wf[j] = v4i{lo.x, lo.y, hi.x, hi.y};
-                } else {
-                    wf[j] = *reinterpret_cast<const v4i *>(w_base[kk] + buf * DL_STAGE + j * 32 * BK);
-                }
-            }
-        };
-        // zero-point sums: K half kk of the X rows is summed by the wavefront column kk, of the W channels by the
-        // wavefront row kk (every row / channel group is owned by exactly one such wavefront)
+        for (int j = 0; j < TN; j++) sw4[j] = v4i{0, 0, 0, 0};
         const int wave_n_u = __builtin_amdgcn_readfirstlane(wave_n), wave_m_u = __builtin_amdgcn_readfirstlane(wave_m);
-        const bool xs0 = need_xsum && wave_n_u == 0, xs1 = need_xsum && wave_n_u == 1;
-        const bool ws0 = need_wsum && wave_m_u == 0, ws1 = need_wsum && wave_m_u == 1;
-        auto multiply = [&](const v4i(&xf)[TM], const v4i(&wf)[TN], bool sum_x, bool sum_w) {
+        constexpr bool BALANCED = WAVES_M == 2 && WAVES_N == 2;
+        bool dx[2], dw[2];
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[i], wf[j], acc[i][j], 0, 0, 0);
-            if (SUMS) {
-                if (sum_x) {  // wave-uniform
-#pragma unroll
-                    for (int i = 0; i < TM; i++)
-#pragma unroll
-                        for (int q = 0; q < 4; q++) xsum[i] = __builtin_amdgcn_sdot4(xf[i][q], 0x01010101, xsum[i], false);
-                }
-                if (sum_w) {
-#pragma unroll
-                    for (int j = 0; j < TN; j++)
-#pragma unroll
-                        for (int q = 0; q < 4; q++) wsum[j] = __builtin_amdgcn_sdot4(wf[j][q], 0x01010101, wsum[j], false);
-                }
-            }
-        };
-        // wait until at most `n` stages of this thread's requests are outstanding (n is wave-uniform)
-        auto wait_stages = [&](int n) {
-            switch (n) {
-            case 0: wait_vmcnt<0>(); break;
-            case 1: wait_vmcnt<1 * (XI + WI)>(); break;
-            case 2: wait_vmcnt<2 * (XI + WI)>(); break;
-            case 3: wait_vmcnt<3 * (XI + WI)>(); break;
-            case 4: wait_vmcnt<4 * (XI + WI)>(); break;
-            case 5: wait_vmcnt<5 * (XI + WI)>(); break;
-            default: wait_vmcnt<6 * (XI + WI)>(); break;
-            }
-        };
-        static_assert(6 * (XI + WI) < 64, "the outstanding-request counter has six bits");
-        // Stage s lives in buffer s % DL_S; DL_S - 1 stages are requested ahead.  The loop is software-pipelined: while
-        // the first K half of step s is multiplied the second half is being read, and while the second half is
-        // multiplied the first half of step s + 1 is being read.  In between sits the one barrier of the step:
-        // waiting until at most DL_S - 3 stages of this thread's requests are outstanding means its part of stage
-        // s + 1 has landed (near the end of K fewer stages are outstanding and the count shrinks); the barrier extends
-        // that to every thread's part and also says that every wavefront has received its reads of stage s - 1,
-        // whose buffer the next request overwrites.
+        for (int hh = 0; hh < 2; hh++) {
+            dx[hh] = need_xsum && (BALANCED ? wave_n_u == (wave_m_u ^ hh) : wave_n_u == hh);
+            dw[hh] = need_wsum && (BALANCED ? wave_n_u != (wave_m_u ^ hh) : wave_m_u == hh);
+        }
+        constexpr bool KM = WMODE == W_KMAJOR_DL;
+        const v4i null4 = v4i{xres4[0], xres4[1], 0, xres4[3]};  // no bytes: a request through it fetches nothing
         const int nk = g.K / BK;
+        // one K half: multiplies (xc, wc), reads K half `rkk` of stage `rbuf` into (xn, wn), and -- after the step's
+        // barrier -- requests stage `ibuf` (K step `istep`, nothing beyond the last step)
+        auto half = [&](auto dx_t, auto dw_t, auto issue_t, const v4i(&xc)[TM], const v4i(&wc)[TN], v4i(&xn)[TM],
+                        v4i(&wn)[TN], int rbuf, int rkk, int ibuf, int istep) {
+            // LP: which part of a stage's requests rides in this half (0 none, 1 the first half of them, 2 the second)
+            constexpr bool DX = decltype(dx_t)::value, DW = decltype(dw_t)::value;
+            constexpr int LP = decltype(issue_t)::value;
+            constexpr bool ISSUE = LP != 0;
+            constexpr int NM = TM * TN;
+            constexpr int NR = TM + TN * (KM ? 2 : 1), RPER = (NR + NM / 2 - 1) / (NM / 2);  // reads early in the half
+            constexpr int NS = (DX ? TM : 0) + (DW ? TN : 0), SPER = (NS + NM - 1) / NM;
+            constexpr int NLA = XI + WI, L0 = LP == 2 ? NLA / 2 : 0, L1 = LP == 1 ? NLA / 2 : (LP == 2 ? NLA : 0);
+            constexpr int NL = L1 - L0, LPER = (NL + NM - 1) / NM;
+            const bool live = ISSUE && istep < nk;
+            const v4i xr = live ? xres4 : null4, wr = live ? wres4 : null4;
+            const uint32_t xd = lds0 + (uint32_t)(ibuf * DL_STAGE), wd = xd + BM * BK;
+            const uint32_t xk = (uint32_t)istep * BK, wk = (uint32_t)istep * w_kstep;
+#pragma unroll
+            for (int t = 0; t < NM; t++) {
+                const int i = t / TN, j = t % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xc[i], wc[j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < RPER; u++) {
+                    const int r = t * RPER + u;
+                    if (r < TM) {
+                        xn[r] = *reinterpret_cast<const v4i *>(x_base[rkk] + rbuf * DL_STAGE + r * 32 * BK);
+                    } else if (r < NR) {
+                        const int e = r - TM;
+                        if (KM) {
+                            const int jj = e >> 1;
+                            const char *pw = w_base[rkk] + rbuf * DL_STAGE + (((wave_n * WN / 32 + jj) ^ kfun) * 32);
+                            const v2i part = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(pw + (e & 1) * 8 * BN));
+                            if (e & 1) {
+                                wn[jj][2] = part.x;
+                                wn[jj][3] = part.y;
+                            } else {
+                                wn[jj][0] = part.x;
+                                wn[jj][1] = part.y;
+                            }
+                        } else {
+                            wn[e] = *reinterpret_cast<const v4i *>(w_base[rkk] + rbuf * DL_STAGE + e * 32 * BK);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < LPER; u++) {
+                    const int l = L0 + t * LPER + u;
+                    if (l < L1) {
+                        if (l < XI) load16_to_lds(xr, xd + l * NTHREADS * 16, xo[l], xk);
+                        else load16_to_lds(wr, wd + (l - XI) * NTHREADS * 16, wo[l - XI], wk);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < SPER; u++) {
+                    const int f = t * SPER + u;  // fragment of the duty: row tiles first
+                    if (f < NS) {
+                        if (DX && f < TM) {
+                            sx4[f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xc[f], selv, sx4[f], 0, 0, 0);
+                        } else {
+                            const int jj = f - (DX ? TM : 0);
+                            sw4[jj] = __builtin_amdgcn_mfma_i32_16x16x64_i8(selv, wc[jj], sw4[jj], 0, 0, 0);
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        using T_ = std::true_type;
+        using F_ = std::false_type;
+        // Stage s lives in buffer s % DL_S; DL_S - 1 stages are requested ahead, every step requests one more (beyond
+        // the last step through the empty resource, so that the number of requests in flight is the same at every
+        // step and the waits below count exactly).  While the first K half of step s is multiplied the second half
+        // is read, and while the second half is multiplied the first half of step s + 1 is read.  In between sits
+        // the one barrier of the step: at most DL_S - 3 stages of this thread's requests outstanding means its part
+        // of stage s + 1 has landed; the barrier extends that to every thread's part and also says that every
+        // wavefront has received its reads of stage s - 1, whose buffer the step's request overwrites.
         v4i xf0[TM], wf0[TN], xf1[TM], wf1[TN];
 #pragma unroll
-        for (int d = 0; d < DL_S - 1; d++)
-            if (d < nk) issue(d, d);
-        wait_stages(min(nk, DL_S - 1) - 1);  // stage 0 has landed
+        for (int d = 0; d < DL_S - 1; d++) {
+            const v4i xr = d < nk ? xres4 : null4, wr = d < nk ? wres4 : null4;
+            const uint32_t xd = lds0 + (uint32_t)(d * DL_STAGE), wd = xd + BM * BK;
+#pragma unroll
+            for (int l = 0; l < XI + WI; l++) {
+                if (d == DL_S - 2 && l >= (XI + WI) / 2) continue;  // its second part rides in the first half of step 0
+                if (l < XI) load16_to_lds(xr, xd + l * NTHREADS * 16, xo[l], (uint32_t)d * BK);
+                else load16_to_lds(wr, wd + (l - XI) * NTHREADS * 16, wo[l - XI], (uint32_t)d * w_kstep);
+            }
+        }
+        wait_vmcnt<(DL_S - 2) * (XI + WI) - (XI + WI) / 2>();  // stage 0 has landed
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        read_frags(0, 0, xf0, wf0);
-        for (int step = 0; step < nk; step += DL_S) {
 #pragma unroll
-            for (int d = 0; d < DL_S; d++) {
-                if (step + d < nk) {  // uniform
-                    read_frags(d, 1, xf1, wf1);
-                    __builtin_amdgcn_sched_barrier(0);
-                    multiply(xf0, wf0, xs0, ws0);
-                    __builtin_amdgcn_sched_barrier(0);
-                    const bool more = step + d + DL_S - 1 < nk;
-                    // requested so far: stages up to min(nk, step + d + DL_S - 1) - 1; stage step + d + 1 must have
-                    // landed, the later ones may still be in flight
-                    if (more) wait_vmcnt<(DL_S - 3) * (XI + WI)>(); else wait_stages(max(nk - 2 - (step + d), 0));
-                    asm volatile("" ::: "memory");
-                    __builtin_amdgcn_s_barrier();
-                    asm volatile("" ::: "memory");
-                    if (more) issue((d + DL_S - 1) % DL_S, step + d + DL_S - 1);
-                    read_frags((d + 1) % DL_S, 0, xf0, wf0);
-                    __builtin_amdgcn_sched_barrier(0);
-                    multiply(xf1, wf1, xs1, ws1);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+        for (int i = 0; i < TM; i++) xf0[i] = *reinterpret_cast<const v4i *>(x_base[0] + i * 32 * BK);
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            if (KM) {
+                const char *pw = w_base[0] + (((wave_n * WN / 32 + j) ^ kfun) * 32);
+                const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(pw));
+                const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(pw + 8 * BN));
+                wf0[j] = v4i{lo.x, lo.y, hi.x, hi.y};
+            } else {
+                wf0[j] = *reinterpret_cast<const v4i *>(w_base[0] + j * 32 * BK);
             }
         }
+        // The loop exists once per combination of duties (a template argument each) and the wavefront picks its copy
+        // in front of it: chosen inside the loop, the variants of a half would meet again behind it, and the register
+        // allocator then has them leave the accumulators in different registers and copies all 64 at every joint.
+        auto loop = [&](auto dx0_t, auto dw0_t, auto dx1_t, auto dw1_t) {
+            for (int step = 0; step < nk; step += DL_S) {
+#pragma unroll
+                for (int d = 0; d < DL_S; d++) {
+                    if (step + d < nk) {  // uniform
+                        half(dx0_t, dw0_t, std::integral_constant<int, 2>{}, xf0, wf0, xf1, wf1, d, 1,
+                             (d + DL_S - 2) % DL_S, step + d + DL_S - 2);
+                        wait_vmcnt<(DL_S - 3) * (XI + WI)>();
+                        asm volatile("" ::: "memory");
+                        __builtin_amdgcn_s_barrier();
+                        asm volatile("" ::: "memory");
+                        half(dx1_t, dw1_t, std::integral_constant<int, 1>{}, xf1, wf1, xf0, wf0, (d + 1) % DL_S, 0,
+                             (d + DL_S - 1) % DL_S, step + d + DL_S - 1);
+                    }
+                }
+            }
+        };
+        // a wavefront never has the same duty in both halves, and with balanced duties never both in one half
+        const int duties = !SUMS ? 0 : (int)dx[0] | ((int)dw[0] << 1) | ((int)dx[1] << 2) | ((int)dw[1] << 3);
+#define MLEL_DUTY_CASE(C)                                                                                          \
+    case C:                                                                                                        \
+        if constexpr (SUMS && !((C & 5) == 5) && !((C & 10) == 10) && !(BALANCED && ((C & 3) == 3 || (C & 12) == 12)))   \
+            loop(std::bool_constant<(C & 1) != 0>{}, std::bool_constant<(C & 2) != 0>{},                           \
+                 std::bool_constant<(C & 4) != 0>{}, std::bool_constant<(C & 8) != 0>{});                          \
+        break;
+        switch (duties) {
+            MLEL_DUTY_CASE(1) MLEL_DUTY_CASE(2) MLEL_DUTY_CASE(3) MLEL_DUTY_CASE(4) MLEL_DUTY_CASE(6) MLEL_DUTY_CASE(8)
+            MLEL_DUTY_CASE(9) MLEL_DUTY_CASE(12)
+        default: loop(F_{}, F_{}, F_{}, F_{}); break;
+        }
+#undef MLEL_DUTY_CASE
+        wait_vmcnt<0>();  // the requests beyond the last step write (zeros) into the ring, which the epilogue reuses
         __syncthreads();
         // ---- combine the split zero-point sums: afterwards every wavefront holds, per lane half, partial sums whose
         // total over the two halves is the full sum of its rows (X) and of its channels (W), as in the other fetch modes
         if (SUMS) {
             int32_t *xs_l = reinterpret_cast<int32_t *>(smem) + BM;      // [2][BM]: by K half
             int32_t *ws_l = reinterpret_cast<int32_t *>(smem) + 3 * BM;  // [2][BN]: by K half
-            if (need_xsum && wave_n < 2) {
+            // a fragment's row sums sit in lanes 16 g (rows 4 g .. 4 g + 3) and 16 g + 8 (rows 16 + 4 g ...), its channel
+            // sums in register 0 of lanes 0 - 15 (channels 0 - 15) and 32 - 47 (channels 16 - 31)
+            if (need_xsum && wave_n < 2 && (lane & 7) == 0) {
 #pragma unroll
-                for (int i = 0; i < TM; i++) {
-                    const int32_t part = xsum[i] + __shfl_xor(xsum[i], 32);
-                    if (lane < 32) xs_l[wave_n * BM + wave_m * WM + i * 32 + lane] = part;
-                }
+                for (int i = 0; i < TM; i++)
+                    *reinterpret_cast<v4i *>(&xs_l[wave_n * BM + wave_m * WM + i * 32 + ((lane >> 3) & 1) * 16 + (lane >> 4) * 4]) = sx4[i];
             }
-            if (need_wsum) {
+            if (need_wsum && (lane & 16) == 0) {
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const int32_t part = wsum[j] + __shfl_xor(wsum[j], 32);
-                    if (lane < 32) ws_l[wave_m * BN + wave_n * WN + j * 32 + lane] = part;
-                }
+                for (int j = 0; j < TN; j++)
+                    ws_l[wave_m * BN + wave_n * WN + j * 32 + (lane & 15) + ((lane >> 5) << 4)] = sw4[j][0];
             }
             __syncthreads();
             if (need_xsum) {
