@@ -124,6 +124,10 @@ int launch_gemm(mlel_ctx *ctx, hipStream_t s, GemmArgs &g, const SplitScratch &s
     }
     const int64_t blocks = total * g.splits;
     g.chunk = (int)((blocks + 7) / 8);
+    g.div_tiles_per_batch = make_div_magic((uint32_t)(g.tiles_m * g.tiles_n));
+    g.div_tiles_n = make_div_magic((uint32_t)g.tiles_n);
+    g.div_band = make_div_magic((uint32_t)(kGroupM * g.tiles_n));
+    g.div_last_rows = make_div_magic((uint32_t)(g.tiles_m % kGroupM == 0 ? kGroupM : g.tiles_m % kGroupM));
     const dim3 grid((unsigned)(g.chunk * 8));
     switch (tile.id) {
     case 0: launch_gemm_tile0(&g, xmode, wmode, grid, s); break;

@@ -38,6 +38,25 @@ constexpr int BK = 64;            // bytes of K per step
 constexpr int kGroupM = 8;        // tile rows per band of the tile walk
 constexpr int PITCH = BK + 16;    // LDS row pitch: 80 B keeps 16-lane groups of 128-bit reads on distinct banks
 
+// floor(n / d) for 0 <= n < 2^31 as (n * m) >> (31 + s) with s = ceil(log2 d), m = ceil(2^(31 + s) / d)
+// (2^(31+s) <= m d <= 2^(31+s) + 2^s, the condition of Granlund and Montgomery's theorem 4.2 for 31-bit n)
+struct DivMagic {
+    uint32_t m, s;
+};
+inline DivMagic make_div_magic(uint32_t d) {
+    DivMagic r{1u << 31, 0};
+    if (d <= 1) return r;
+    uint32_t s = 0;
+    while ((uint64_t(1) << s) < d) s++;
+    const uint64_t p = uint64_t(1) << (31 + s);
+    r.m = (uint32_t)((p + d - 1) / d);
+    r.s = s;
+    return r;
+}
+__device__ __forceinline__ int div_magic(int n, const DivMagic &d) {
+    return (int)(((uint64_t)(uint32_t)n * d.m) >> (31 + d.s));
+}
+
 struct GemmArgs {
     // problem
     int32_t M, N, K, batches;
@@ -74,6 +93,10 @@ struct GemmArgs {
     ScaleRef rs_res, rs_conv, rs_out;
     // launch geometry
     int32_t tiles_m, tiles_n, total_tiles, chunk;
+    // Divisions of the tile index by numbers that are fixed for the launch (tiles per batch, tiles per row, tiles per
+    // band of kGroupM rows, rows of the last band), as a multiplication and a shift: a division costs a wavefront
+    // some thirty dependent scalar instructions, and the first operand request waits for three of them.
+    DivMagic div_tiles_per_batch, div_tiles_n, div_band, div_last_rows;
     // Split K (register-staged pipeline only): `splits` blocks share one output tile, block s multiplies the K steps
     // [s * split_steps, (s + 1) * split_steps).  Every block writes its int32 partial tile (zero-point terms of its K
     // range already applied, the bias in split 0) to `partials` and bumps the tile's counter; the block that finds
@@ -320,23 +343,21 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     const int k_begin = step0 * BK;
     const int k_len = min(g.K, k_begin + nk_own * BK) - k_begin;              // bytes of K in this block's range
     const int tiles_per_batch = g.tiles_m * g.tiles_n;
-    // the divisions run on the vector ALU; readfirstlane returns the (wave-uniform) results to scalar registers so
-    // that everything derived from them (base pointers, buffer resources) is scalar as well
-    const int batch = __builtin_amdgcn_readfirstlane(lin / tiles_per_batch);
+    const int batch = div_magic(lin, g.div_tiles_per_batch);
     const int t_in = lin - batch * tiles_per_batch;
     // Tiles are walked in bands of GROUP_M tile rows, column by column inside a band: the blocks that run at the
     // same time on one XCD then share a few row panels of X and a few column panels of W in its L2, instead of one
     // row panel and every column panel.
     int tile_m, tile_n;
     if (g.tiles_m >= 2 * kGroupM) {
-        const int band = __builtin_amdgcn_readfirstlane(t_in / (kGroupM * g.tiles_n));
+        const int band = div_magic(t_in, g.div_band);
         const int first = band * kGroupM;
         const int rows = min(kGroupM, g.tiles_m - first);
         const int r = t_in - band * kGroupM * g.tiles_n;
-        tile_n = __builtin_amdgcn_readfirstlane(r / rows);
+        tile_n = rows == kGroupM ? r / kGroupM : div_magic(r, g.div_last_rows);
         tile_m = first + r - tile_n * rows;
     } else {
-        tile_m = __builtin_amdgcn_readfirstlane(t_in / g.tiles_n);
+        tile_m = div_magic(t_in, g.div_tiles_n);
         tile_n = t_in - tile_m * g.tiles_n;
     }
     const int m_base = tile_m * BM, n_base = tile_n * BN;
@@ -352,20 +373,24 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     // channels.  The loads are issued here, ahead of the operand prefetch, but only consumed after the main loop, so
     // their latency is never waited for.
     int32_t chan_bias[TN], chan_mult[TN], chan_shift[TN];
+    auto load_chan_constants = [&]() {
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const int gn = n_base + wave_n * WN + j * 32 + (lane & 31);
-        chan_bias[j] = chan_mult[j] = chan_shift[j] = 0;
-        if (gn < g.N) {
-            chan_bias[j] = (g.bias && split == 0) ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
-            if (g.fused) {
-                const int ci = g.rp.per_channel ? gn : 0;
-                chan_mult[j] = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
-                                        : reinterpret_cast<const int32_t *>(g.mult)[ci];
-                chan_shift[j] = (int32_t)g.shift[ci];
+        for (int j = 0; j < TN; j++) {
+            const int gn = n_base + wave_n * WN + j * 32 + (lane & 31);
+            chan_bias[j] = chan_mult[j] = chan_shift[j] = 0;
+            if (gn < g.N) {
+                chan_bias[j] = (g.bias && split == 0) ? g.bias[g.bias_len == 1 ? 0 : gn] : 0;
+                if (g.fused) {
+                    const int ci = g.rp.per_channel ? gn : 0;
+                    chan_mult[j] = g.mult16 ? (int32_t) reinterpret_cast<const int16_t *>(g.mult)[ci]
+                                            : reinterpret_cast<const int32_t *>(g.mult)[ci];
+                    chan_shift[j] = (int32_t)g.shift[ci];
+                }
             }
         }
-    }
+    };
+    // (the direct-to-LDS form requests its first operand stages before anything else and these constants behind them)
+    if constexpr (XMODE != X_PLAIN_DL) load_chan_constants();
 
     // ---- loader state
     const int x_kc = tid & 3;  // which 16-byte piece of the 64-byte K step this thread stages
@@ -792,6 +817,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                 else load16_to_lds(wr, wd + (l - XI) * NTHREADS * 16, wo[l - XI], (uint32_t)d * w_kstep);
             }
         }
+        // the epilogue's per-channel constants: requested behind the first stages, used behind the loop.  They are
+        // younger than the first stages and older than every later request, so the counted waits below and in the
+        // loop hold with them in flight (how many there are depends on the operator: the waits count none of them,
+        // which only makes the first ones wait for a few requests more).
+        load_chan_constants();
         wait_vmcnt<(DL_S - 2) * (XI + WI) - (XI + WI) / 2>();  // stage 0 has landed
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
@@ -854,8 +884,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             // sums in register 0 of lanes 0 - 15 (channels 0 - 15) and 32 - 47 (channels 16 - 31)
             if (need_xsum && wave_n < 2 && (lane & 7) == 0) {
 #pragma unroll
-                for (int i = 0; i < TM; i++)
-                    *reinterpret_cast<v4i *>(&xs_l[wave_n * BM + wave_m * WM + i * 32 + ((lane >> 3) & 1) * 16 + (lane >> 4) * 4]) = sx4[i];
+                for (int i = 0; i < TM; i++)  // times the weight zero point: what the epilogue subtracts per row
+                    *reinterpret_cast<v4i *>(&xs_l[wave_n * BM + wave_m * WM + i * 32 + ((lane >> 3) & 1) * 16 + (lane >> 4) * 4]) =
+                        sx4[i] * g.zw;
             }
             if (need_wsum && (lane & 16) == 0) {
 #pragma unroll
@@ -863,13 +894,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                     ws_l[wave_m * BN + wave_n * WN + j * 32 + (lane & 15) + ((lane >> 5) << 4)] = sw4[j][0];
             }
             __syncthreads();
-            if (need_xsum) {
-#pragma unroll
-                for (int i = 0; i < TM; i++) {
-                    const int r = wave_m * WM + i * 32 + (lane & 31);
-                    xsum[i] = lane < 32 ? xs_l[r] + xs_l[BM + r] : 0;
-                }
-            }
+            // the channel sums into the registers of the lower lane half (the epilogue adds the halves, as in the
+            // other fetch modes); the row terms stay in the two tables, which the epilogue reads as it goes
             if (need_wsum) {
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
@@ -877,7 +903,6 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                     wsum[j] = lane < 32 ? ws_l[c] + ws_l[BN + c] : 0;
                 }
             }
-            __syncthreads();
         }
     } else {
     // ---- main loop: a ring of DEPTH register sets keeps DEPTH - 1 K steps of global loads in flight while one
@@ -924,7 +949,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                                     (uint32_t)k_len * (uint32_t)g.zx * (uint32_t)g.zw);
         }
     }
-    if (need_xsum) {  // the row terms are needed by register index: through a table in shared memory
+    if (need_xsum && !DL) {  // the row terms are needed by register index: through a table in shared memory
         if (wave_n == 0) {
 #pragma unroll
             for (int i = 0; i < TM; i++) {
@@ -936,7 +961,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     }
     // zw * sum_k X of the four positions of register group q of tile row i
     auto row_terms = [&](int i, int q, int32_t (&xc)[4]) {
-        if (need_xsum) {
+        if (need_xsum && DL) {  // the two K halves' tables of the direct-to-LDS loop, behind the row table's place
+            const int32_t *p0 = xs_tab + BM + wave_m * WM + i * 32 + 8 * q + 4 * half;
+            const int4 t = *reinterpret_cast<const int4 *>(p0), u = *reinterpret_cast<const int4 *>(p0 + BM);
+            xc[0] = t.x + u.x, xc[1] = t.y + u.y, xc[2] = t.z + u.z, xc[3] = t.w + u.w;
+        } else if (need_xsum) {
             const int4 t = *reinterpret_cast<const int4 *>(xs_tab + wave_m * WM + i * 32 + 8 * q + 4 * half);
             xc[0] = t.x, xc[1] = t.y, xc[2] = t.z, xc[3] = t.w;
         } else {
