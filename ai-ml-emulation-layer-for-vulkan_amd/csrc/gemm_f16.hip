@@ -206,14 +206,6 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
         const v4i wres4 = rsrc_words(o.b + (int64_t)batch * g.b_batch, g.b_bytes);
         const uint32_t lds0 = (uint32_t) reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char *)smem) +
                               (uint32_t)(wave_u * 1024);
-        auto issue = [&](int buf, int step) {  // `step` is wave-uniform: the K advance is a scalar offset
-            const uint32_t xd = lds0 + (uint32_t)(buf * DL_STAGE), wd = xd + BM * BK;
-            const uint32_t kb = (uint32_t)step * BK;
-#pragma unroll
-            for (int i = 0; i < XI; i++) load16_to_lds(xres4, xd + i * NT * 16, xo[i], kb);
-#pragma unroll
-            for (int i = 0; i < WI; i++) load16_to_lds(wres4, wd + i * NT * 16, wo[i], kb);
-        };
         // operand addresses inside a stage: row lane % 32 of a 32-row group, the lane half's eight halfs of K half kk
         const int h = lane >> 5, swz = (lane >> 2) & 3;
         const char *x_base[2], *w_base[2];
@@ -223,64 +215,86 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
             x_base[kk] = smem + (wave_m * WM + (lane & 31)) * BK + slot;
             w_base[kk] = smem + BM * BK + (wave_n * WN + (lane & 31)) * BK + slot;
         }
-        auto read_frags = [&](int buf, int kk, v8h(&xf)[TM], v8h(&wf)[TN]) {
+        // The loop, as in the int8 kernel's direct-to-LDS form: a wavefront issues in order, so a K half is one
+        // straight line -- a matrix instruction, then a share of the next half's operand reads and of the requests,
+        // which issue while the matrix core works, then the next matrix instruction.  Stage s lives in buffer
+        // s % DL_S; a stage's requests ride in the second K half of a step, behind the step's barrier, which frees the
+        // buffer (spread over both halves of a step they arrive a step later, which the long contractions whose
+        // operands come from memory rather than from the L2 pay for: 4096 x 3072 x 768 ran 5 % slower).  Beyond the last step they go through an
+        // empty resource and fetch nothing, so every step has the same requests in flight and the waits count exactly:
+        // at most DL_S - 3 stages outstanding at the barrier of step s means this thread's part of stage s + 1 has
+        // landed; the barrier extends that to every thread's part and says that every wavefront has received its
+        // reads of stage s - 1, whose buffer the step's requests overwrite.
+        const int nk = g.K / 32;
+        const v4i null4 = v4i{xres4[0], xres4[1], 0, xres4[3]};
+        constexpr int NLA = XI + WI;
+        auto half = [&](auto lp_t, const v8h(&xc)[TM], const v8h(&wc)[TN], v8h(&xn)[TM], v8h(&wn)[TN], int rbuf, int rkk,
+                        int ibuf, int istep) {
+            constexpr int LP = decltype(lp_t)::value;  // 1: the stage's requests ride in this half, 0: none
+            constexpr int NM = TM * TN, NR = TM + TN;
+            constexpr int L0 = 0, L1 = LP == 1 ? NLA : 0, NL = L1 - L0, LPER = (NL + NM - 1) / NM;
+            const bool live = istep < nk;
+            const v4i xr = live ? xres4 : null4, wr = live ? wres4 : null4;
+            const uint32_t xd = lds0 + (uint32_t)(ibuf * DL_STAGE), wd = xd + BM * BK;
+            const uint32_t kb = (uint32_t)istep * BK;
+            // (two wavefronts share a SIMD here and fill each other's gaps: the reads go first, so that their data
+            // is there when the next half starts; only the requests are dealt out behind the matrix instructions)
 #pragma unroll
-            for (int i = 0; i < TM; i++) xf[i] = *reinterpret_cast<const v8h *>(x_base[kk] + buf * DL_STAGE + i * 32 * BK);
+            for (int r = 0; r < NR; r++) {
+                if (r < TM) xn[r] = *reinterpret_cast<const v8h *>(x_base[rkk] + rbuf * DL_STAGE + r * 32 * BK);
+                else wn[r - TM] = *reinterpret_cast<const v8h *>(w_base[rkk] + rbuf * DL_STAGE + (r - TM) * 32 * BK);
+            }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int j = 0; j < TN; j++) wf[j] = *reinterpret_cast<const v8h *>(w_base[kk] + buf * DL_STAGE + j * 32 * BK);
-        };
-        auto multiply = [&](const v8h(&xf)[TM], const v8h(&wf)[TN]) {
+            for (int t = 0; t < NM; t++) {
+                const int i = t / TN, j = t % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wc[j], xc[i], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[i][j], 0, 0, 0);
-        };
-        // wait until at most `n` stages of this thread's requests are outstanding (n is wave-uniform)
-        auto wait_stages = [&](int n) {
-            switch (n) {
-            case 0: wait_vmcnt<0>(); break;
-            case 1: wait_vmcnt<1 * (XI + WI)>(); break;
-            case 2: wait_vmcnt<2 * (XI + WI)>(); break;
-            default: wait_vmcnt<3 * (XI + WI)>(); break;
+                for (int u = 0; u < LPER; u++) {
+                    const int l = L0 + t * LPER + u;
+                    if (l < L1) {
+                        if (l < XI) load16_to_lds(xr, xd + l * NT * 16, xo[l], kb);
+                        else load16_to_lds(wr, wd + (l - XI) * NT * 16, wo[l - XI], kb);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         };
-        // Stage s lives in buffer s % DL_S; DL_S - 1 stages are requested ahead.  While the first K half of step s is
-        // multiplied the second half is being read, and while the second half is multiplied the first half of step
-        // s + 1 is being read.  In between sits the one barrier of the step: waiting until at most DL_S - 3 stages
-        // of this thread's requests are outstanding means its part of stage s + 1 has landed; the barrier extends
-        // that to every thread's part and also says that every wavefront has received its reads of stage s - 1,
-        // whose buffer the next request overwrites.
-        const int nk = g.K / 32;
         v8h xf0[TM], wf0[TN], xf1[TM], wf1[TN];
 #pragma unroll
-        for (int d = 0; d < DL_S - 1; d++)
-            if (d < nk) issue(d, d);
-        wait_stages(min(nk, DL_S - 1) - 1);  // stage 0 has landed
+        for (int d = 0; d < DL_S - 1; d++) {
+            const v4i xr = d < nk ? xres4 : null4, wr = d < nk ? wres4 : null4;
+            const uint32_t xd = lds0 + (uint32_t)(d * DL_STAGE), wd = xd + BM * BK;
+#pragma unroll
+            for (int l = 0; l < NLA; l++) {
+                if (l < XI) load16_to_lds(xr, xd + l * NT * 16, xo[l], (uint32_t)d * BK);
+                else load16_to_lds(wr, wd + (l - XI) * NT * 16, wo[l - XI], (uint32_t)d * BK);
+            }
+        }
+        wait_vmcnt<(DL_S - 2) * NLA>();  // stage 0 has landed: what was requested behind it may be in flight
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        read_frags(0, 0, xf0, wf0);
+#pragma unroll
+        for (int i = 0; i < TM; i++) xf0[i] = *reinterpret_cast<const v8h *>(x_base[0] + i * 32 * BK);
+#pragma unroll
+        for (int j = 0; j < TN; j++) wf0[j] = *reinterpret_cast<const v8h *>(w_base[0] + j * 32 * BK);
         for (int step = 0; step < nk; step += DL_S) {
 #pragma unroll
             for (int d = 0; d < DL_S; d++) {
                 if (step + d < nk) {  // uniform
-                    read_frags(d, 1, xf1, wf1);
-                    __builtin_amdgcn_sched_barrier(0);
-                    multiply(xf0, wf0);
-                    __builtin_amdgcn_sched_barrier(0);
-                    const bool more = step + d + DL_S - 1 < nk;
-                    if (more) wait_vmcnt<(DL_S - 3) * (XI + WI)>(); else wait_stages(max(nk - 2 - (step + d), 0));
+                    half(std::integral_constant<int, 0>{}, xf0, wf0, xf1, wf1, d, 1, 0, 0);
+                    wait_vmcnt<(DL_S - 3) * NLA>();
                     asm volatile("" ::: "memory");
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
-                    if (more) issue((d + DL_S - 1) % DL_S, step + d + DL_S - 1);
-                    read_frags((d + 1) % DL_S, 0, xf0, wf0);
-                    __builtin_amdgcn_sched_barrier(0);
-                    multiply(xf1, wf1);
-                    __builtin_amdgcn_sched_barrier(0);
+                    half(std::integral_constant<int, 1>{}, xf1, wf1, xf0, wf0, (d + 1) % DL_S, 0, (d + DL_S - 1) % DL_S,
+                         step + d + DL_S - 1);
                 }
             }
         }
+        wait_vmcnt<0>();  // the requests beyond the last step write (zeros) into the ring, which the epilogue reuses
         __syncthreads();
     } else {
     uint32_t xoff[XROWS], woff[WCHUNKS];

@@ -732,14 +732,14 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         // barrier -- requests stage `ibuf` (K step `istep`, nothing beyond the last step)
         auto half = [&](auto dx_t, auto dw_t, auto issue_t, const v4i(&xc)[TM], const v4i(&wc)[TN], v4i(&xn)[TM],
                         v4i(&wn)[TN], int rbuf, int rkk, int ibuf, int istep) {
-            // LP: which part of a stage's requests rides in this half (0 none, 1 the first half of them, 2 the second)
+            // LP: 1 when the stage's requests ride in this half (the one behind the step's barrier), 0 otherwise
             constexpr bool DX = decltype(dx_t)::value, DW = decltype(dw_t)::value;
             constexpr int LP = decltype(issue_t)::value;
             constexpr bool ISSUE = LP != 0;
             constexpr int NM = TM * TN;
             constexpr int NR = TM + TN * (KM ? 2 : 1), RPER = (NR + NM / 2 - 1) / (NM / 2);  // reads early in the half
             constexpr int NS = (DX ? TM : 0) + (DW ? TN : 0), SPER = (NS + NM - 1) / NM;
-            constexpr int NLA = XI + WI, L0 = LP == 2 ? NLA / 2 : 0, L1 = LP == 1 ? NLA / 2 : (LP == 2 ? NLA : 0);
+            constexpr int NLA = XI + WI, L0 = 0, L1 = LP == 1 ? NLA : 0;
             constexpr int NL = L1 - L0, LPER = (NL + NM - 1) / NM;
             const bool live = ISSUE && istep < nk;
             const v4i xr = live ? xres4 : null4, wr = live ? wres4 : null4;
@@ -812,7 +812,6 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             const uint32_t xd = lds0 + (uint32_t)(d * DL_STAGE), wd = xd + BM * BK;
 #pragma unroll
             for (int l = 0; l < XI + WI; l++) {
-                if (d == DL_S - 2 && l >= (XI + WI) / 2) continue;  // its second part rides in the first half of step 0
                 if (l < XI) load16_to_lds(xr, xd + l * NTHREADS * 16, xo[l], (uint32_t)d * BK);
                 else load16_to_lds(wr, wd + (l - XI) * NTHREADS * 16, wo[l - XI], (uint32_t)d * w_kstep);
             }
@@ -822,7 +821,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         // loop hold with them in flight (how many there are depends on the operator: the waits count none of them,
         // which only makes the first ones wait for a few requests more).
         load_chan_constants();
-        wait_vmcnt<(DL_S - 2) * (XI + WI) - (XI + WI) / 2>();  // stage 0 has landed
+        wait_vmcnt<(DL_S - 2) * (XI + WI)>();  // stage 0 has landed: what was requested behind it may be in flight
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -847,8 +846,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
 #pragma unroll
                 for (int d = 0; d < DL_S; d++) {
                     if (step + d < nk) {  // uniform
-                        half(dx0_t, dw0_t, std::integral_constant<int, 2>{}, xf0, wf0, xf1, wf1, d, 1,
-                             (d + DL_S - 2) % DL_S, step + d + DL_S - 2);
+                        half(dx0_t, dw0_t, std::integral_constant<int, 0>{}, xf0, wf0, xf1, wf1, d, 1, 0, 0);
                         wait_vmcnt<(DL_S - 3) * (XI + WI)>();
                         asm volatile("" ::: "memory");
                         __builtin_amdgcn_s_barrier();
