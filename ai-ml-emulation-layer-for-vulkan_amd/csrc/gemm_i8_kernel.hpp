@@ -882,9 +882,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             // sums in register 0 of lanes 0 - 15 (channels 0 - 15) and 32 - 47 (channels 16 - 31)
             if (need_xsum && wave_n < 2 && (lane & 7) == 0) {
 #pragma unroll
-                for (int i = 0; i < TM; i++)  // times the weight zero point: what the epilogue subtracts per row
+                for (int i = 0; i < TM; i++)  // times minus the weight zero point: what the epilogue adds per row
                     *reinterpret_cast<v4i *>(&xs_l[wave_n * BM + wave_m * WM + i * 32 + ((lane >> 3) & 1) * 16 + (lane >> 4) * 4]) =
-                        sx4[i] * g.zw;
+                        sx4[i] * -g.zw;
             }
             if (need_wsum && (lane & 16) == 0) {
 #pragma unroll
@@ -936,7 +936,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     // position 32 i + 8 q + 4 (lane / 32) + e and channel 32 j + lane % 32 of the wavefront's sub-tile: one channel per
     // lane and tile column, so everything that depends on the channel only sits in a few registers.
     const int half = lane >> 5, cl = lane & 31;
-    int32_t *xs_tab = reinterpret_cast<int32_t *>(smem);  // [BM]: zw * sum_k X[m][k]; the operand buffers are free now
+    int32_t *xs_tab = reinterpret_cast<int32_t *>(smem);  // [BM]: -zw * sum_k X[m][k]; the operand buffers are free now
     int32_t bias_adj[TN];
 #pragma unroll
     for (int j = 0; j < TN; j++) {
@@ -952,12 +952,13 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
 #pragma unroll
             for (int i = 0; i < TM; i++) {
                 const int32_t sx = xsum[i] + __shfl_xor(xsum[i], 32);
-                if (lane < 32) xs_tab[wave_m * WM + i * 32 + lane] = (int32_t)((uint32_t)sx * (uint32_t)g.zw);
+                if (lane < 32) xs_tab[wave_m * WM + i * 32 + lane] = (int32_t)(0u - (uint32_t)sx * (uint32_t)g.zw);
             }
         }
         __syncthreads();
     }
-    // zw * sum_k X of the four positions of register group q of tile row i
+    // minus zw * sum_k X of the four positions of register group q of tile row i (minus, so that accumulator + channel
+    // term + row term is one three-operand addition)
     auto row_terms = [&](int i, int q, int32_t (&xc)[4]) {
         if (need_xsum && DL) {  // the two K halves' tables of the direct-to-LDS loop, behind the row table's place
             const int32_t *p0 = xs_tab + BM + wave_m * WM + i * 32 + 8 * q + 4 * half;
@@ -985,7 +986,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                     for (int j = 0; j < TN; j++)
 #pragma unroll
                         for (int e = 0; e < 4; e++)
-                            acc[i][j][4 * q + e] = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] -
+                            acc[i][j][4 * q + e] = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] +
                                                              (uint32_t)xc[e]);
                 }
 #pragma unroll
@@ -1091,7 +1092,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                     int32_t v[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] - (uint32_t)xc[e]);
+                        const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] + (uint32_t)xc[e]);
                         v[e] = requant_acc(a, cs[j], g.rp);
                     }
                     // bytes = positions e of this lane's channel
@@ -1183,7 +1184,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                 for (int j = 0; j < TN; j++) {
                     const int n = n_base + wave_n * WN + j * 32 + cl;
                     if (n >= g.N) continue;
-                    const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] - (uint32_t)xc[e]);
+                    const int32_t a = (int32_t)((uint32_t)acc[i][j][4 * q + e] + (uint32_t)bias_adj[j] + (uint32_t)xc[e]);
                     const int32_t v = g.fused ? requant_acc(a, cs[j], g.rp) : a;
                     const int64_t off = (int64_t)m * g.ldo + n;
                     if (g.out_size == 1)
