@@ -51,6 +51,7 @@ struct ConvDwArgs {
     uint32_t strips_magic, w_magic;      // floor(2^32 / d) + 1 for d = strips, W: x / d == umulhi(x, magic) for
                                          // x < 2^16 and 1 < d < 2^16
     int32_t blocks, chunk;               // `chunk` consecutive blocks per XCD
+    DivMagic div_slices, div_bands;      // block index / slices, / bands as a multiplication and a shift
 };
 
 struct DwConst {  // per channel of the slice, in shared memory: 48 bytes
@@ -87,10 +88,16 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
     DwConst *dwc = reinterpret_cast<DwConst *>(smem);  // [4][8]: [channel of the quad][quad]
     char *tile = smem + kSliceCh * sizeof(DwConst);
 
+    // Every argument that the first requests depend on is asked for here, in one batch: left alone the compiler loads
+    // arguments where they are first used, behind the early exit and behind each other's results, and a wavefront
+    // waits for four trips to memory in a row before it has computed its first address.
+    asm volatile("" ::"s"(a.chunk), "s"(a.blocks), "s"(a.slices), "s"(a.bands), "s"(a.band_out), "s"(a.OH), "s"(a.pad_t),
+                 "s"(a.th), "s"(a.H), "s"(a.W), "s"(a.x), "s"(a.x_bytes), "s"(a.P), "s"(a.IC), "s"(a.w1), "s"(a.div_slices.m),
+                 "s"(a.div_slices.s), "s"(a.div_bands.m), "s"(a.div_bands.s));
     const int bid = (int)(blockIdx.x % 8u) * a.chunk + (int)(blockIdx.x / 8u);
     if (bid >= a.blocks) return;
-    const int slice = bid % a.slices, rest_b = bid / a.slices;
-    const int band = rest_b % a.bands, n = rest_b / a.bands;
+    const int rest_b = div_magic(bid, a.div_slices), slice = bid - rest_b * a.slices;
+    const int n = div_magic(rest_b, a.div_bands), band = rest_b - n * a.bands;
     const int c0 = slice * kSliceCh;
     // the band's output rows [ob0, ob1) read the input rows y_base .. y_base + th - 1 (tile row r = input row
     // y_base + r); the rows of the image among them are [y_lo, y_hi)
@@ -430,6 +437,8 @@ int try_conv2d_dwconv_i8(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, c
     if (blocks >= (int64_t(1) << 31) - 8) return 0;
     g.blocks = (int)blocks;
     g.chunk = (int)((blocks + 7) / 8);
+    g.div_slices = make_div_magic((uint32_t)g.slices);
+    g.div_bands = make_div_magic((uint32_t)g.bands);
     const dim3 grid((unsigned)(g.chunk * 8));
     if (nt == 512)
         launch_conv_dw_k<512>(g, (int)(IC / 32), sx, ty, grid, sm, s);

@@ -38,25 +38,6 @@ constexpr int BK = 64;            // bytes of K per step
 constexpr int kGroupM = 8;        // tile rows per band of the tile walk
 constexpr int PITCH = BK + 16;    // LDS row pitch: 80 B keeps 16-lane groups of 128-bit reads on distinct banks
 
-// floor(n / d) for 0 <= n < 2^31 as (n * m) >> (31 + s) with s = ceil(log2 d), m = ceil(2^(31 + s) / d)
-// (2^(31+s) <= m d <= 2^(31+s) + 2^s, the condition of Granlund and Montgomery's theorem 4.2 for 31-bit n)
-struct DivMagic {
-    uint32_t m, s;
-};
-inline DivMagic make_div_magic(uint32_t d) {
-    DivMagic r{1u << 31, 0};
-    if (d <= 1) return r;
-    uint32_t s = 0;
-    while ((uint64_t(1) << s) < d) s++;
-    const uint64_t p = uint64_t(1) << (31 + s);
-    r.m = (uint32_t)((p + d - 1) / d);
-    r.s = s;
-    return r;
-}
-__device__ __forceinline__ int div_magic(int n, const DivMagic &d) {
-    return (int)(((uint64_t)(uint32_t)n * d.m) >> (31 + d.s));
-}
-
 struct GemmArgs {
     // problem
     int32_t M, N, K, batches;
