@@ -311,6 +311,14 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
 
     // ---- XCD-aware tile assignment: consecutive block ids land on different XCDs (8 of them, each with its own
     // L2), so block b is given tile (b % 8) * chunk + b / 8: tiles that share operands stay on one XCD.
+    // Every argument that the tile assignment and the first operand requests depend on is asked for here, in one
+    // batch: left alone the compiler loads arguments where they are first used, behind the early exit and behind each
+    // other's results, and a wavefront waits for several trips to memory in a row before its first address.
+    asm volatile("" ::"s"(g.chunk), "s"(g.total_tiles), "s"(g.splits), "s"(g.tiles_m), "s"(g.tiles_n),
+                 "s"(g.div_tiles_per_batch.m), "s"(g.div_tiles_per_batch.s), "s"(g.div_tiles_n.m), "s"(g.div_tiles_n.s),
+                 "s"(g.div_band.m), "s"(g.div_band.s), "s"(g.div_last_rows.m), "s"(g.div_last_rows.s), "s"(g.x), "s"(g.w),
+                 "s"(g.x_batch), "s"(g.w_batch), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.x_sx), "s"(g.ldw), "s"(g.x_bytes),
+                 "s"(g.w_bytes));
     const int lin_all = (int)(blockIdx.x % 8) * g.chunk + (int)(blockIdx.x / 8);
     if (lin_all >= g.total_tiles * g.splits) return;
     // the splits of one tile are consecutive, so they run on one XCD and exchange their partials through its L2
