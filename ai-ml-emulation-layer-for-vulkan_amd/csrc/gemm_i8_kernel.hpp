@@ -719,8 +719,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         const int nk = g.K / BK;
         // one K half: multiplies (xc, wc), reads K half `rkk` of stage `rbuf` into (xn, wn), and -- after the step's
         // barrier -- requests stage `ibuf` (K step `istep`, nothing beyond the last step)
-        auto half = [&](auto dx_t, auto dw_t, auto issue_t, const v4i(&xc)[TM], const v4i(&wc)[TN], v4i(&xn)[TM],
-                        v4i(&wn)[TN], int rbuf, int rkk, int ibuf, int istep) {
+        auto half = [&](auto dx_t, auto dw_t, auto issue_t, auto steady_t, const v4i(&xc)[TM], const v4i(&wc)[TN],
+                        v4i(&xn)[TM], v4i(&wn)[TN], int rbuf, int rkk, int ibuf, int istep) {
             // LP: 1 when the stage's requests ride in this half (the one behind the step's barrier), 0 otherwise
             constexpr bool DX = decltype(dx_t)::value, DW = decltype(dw_t)::value;
             constexpr int LP = decltype(issue_t)::value;
@@ -730,7 +730,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
             constexpr int NS = (DX ? TM : 0) + (DW ? TN : 0), SPER = (NS + NM - 1) / NM;
             constexpr int NLA = XI + WI, L0 = 0, L1 = LP == 1 ? NLA : 0;
             constexpr int NL = L1 - L0, LPER = (NL + NM - 1) / NM;
-            const bool live = ISSUE && istep < nk;
+            // (steady: the caller knows that the requested step exists, and the choice of the resource falls away)
+            const bool live = ISSUE && (decltype(steady_t)::value || istep < nk);
             const v4i xr = live ? xres4 : null4, wr = live ? wres4 : null4;
             const uint32_t xd = lds0 + (uint32_t)(ibuf * DL_STAGE), wd = xd + BM * BK;
             const uint32_t xk = (uint32_t)istep * BK, wk = (uint32_t)istep * w_kstep;
@@ -831,16 +832,30 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         // in front of it: chosen inside the loop, the variants of a half would meet again behind it, and the register
         // allocator then has them leave the accumulators in different registers and copies all 64 at every joint.
         auto loop = [&](auto dx0_t, auto dw0_t, auto dx1_t, auto dw1_t) {
-            for (int step = 0; step < nk; step += DL_S) {
+            // groups of DL_S steps that all still have a step to request run without the tests of the general form
+            int step = 0;
+            for (; step + 2 * DL_S - 1 <= nk; step += DL_S) {
+#pragma unroll
+                for (int d = 0; d < DL_S; d++) {
+                    half(dx0_t, dw0_t, std::integral_constant<int, 0>{}, T_{}, xf0, wf0, xf1, wf1, d, 1, 0, 0);
+                    wait_vmcnt<(DL_S - 3) * (XI + WI)>();
+                    asm volatile("" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    half(dx1_t, dw1_t, std::integral_constant<int, 1>{}, T_{}, xf1, wf1, xf0, wf0, (d + 1) % DL_S, 0,
+                         (d + DL_S - 1) % DL_S, step + d + DL_S - 1);
+                }
+            }
+            for (; step < nk; step += DL_S) {
 #pragma unroll
                 for (int d = 0; d < DL_S; d++) {
                     if (step + d < nk) {  // uniform
-                        half(dx0_t, dw0_t, std::integral_constant<int, 0>{}, xf0, wf0, xf1, wf1, d, 1, 0, 0);
+                        half(dx0_t, dw0_t, std::integral_constant<int, 0>{}, F_{}, xf0, wf0, xf1, wf1, d, 1, 0, 0);
                         wait_vmcnt<(DL_S - 3) * (XI + WI)>();
                         asm volatile("" ::: "memory");
                         __builtin_amdgcn_s_barrier();
                         asm volatile("" ::: "memory");
-                        half(dx1_t, dw1_t, std::integral_constant<int, 1>{}, xf1, wf1, xf0, wf0, (d + 1) % DL_S, 0,
+                        half(dx1_t, dw1_t, std::integral_constant<int, 1>{}, F_{}, xf1, wf1, xf0, wf0, (d + 1) % DL_S, 0,
                              (d + DL_S - 1) % DL_S, step + d + DL_S - 1);
                     }
                 }
