@@ -300,6 +300,7 @@ RUNTIME_SIGNATURES = {
     "mlel_hip_graph_destroy": (C.c_int, [_V, _V]),
     "mlel_hip_copy_kernel": (C.c_int, [_V, _V, _V, _V, C.c_size_t]),
     "mlel_hip_mfma_rate_probe": (C.c_int, [_V, _V, _V, _V, C.c_int, C.c_int]),
+    "mlel_hip_issue_probe": (C.c_int, [_V, _V, _V, _V, C.c_int, C.c_int]),
     "mlel_hip_copy_kernel_variant": (C.c_int, [_V, _V, _V, _V, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int]),
     "mlel_hip_matmul_chain_in_kernel": (C.c_int, [C.POINTER(Chain)]),
     "mlel_hip_attention_f16_in_kernel": (C.c_int, [_T, _T, _T, _T, C.POINTER(Chain)]),

@@ -618,11 +618,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     };
 
     if constexpr (DL) {
-        // ---- direct-to-LDS main loop (K % 64 == 0).  The matrix-core instructions and the ordinary vector
-        // instructions of a wavefront share one issue stream, so everything that is not a multiply is kept out of
-        // the loop: the K advance of the fetches rides in the scalar offset of the buffer instruction, the stage
-        // ring is unrolled so that LDS addresses are lane base + immediate, and the zero-point sums of a K half are
-        // taken by one wavefront only (combined through LDS after the loop).
+        // ---- direct-to-LDS main loop (K % 64 == 0).  The matrix-core instructions and everything else a wavefront
+        // does share one issue stream, so what need not be in the loop is kept out of it: the K advance of the
+        // requests rides in the scalar offset of the buffer instruction, the stage ring is unrolled so that LDS
+        // addresses are lane base + immediate, and the zero-point sums of a K half are taken by one wavefront only
+        // (combined through LDS after the loop).
         constexpr int XI = BM * 4 / NTHREADS, WI = BN * 4 / NTHREADS;  // 16-byte pieces per thread and stage
         static_assert((BN * 4) % NTHREADS == 0 && BN % 32 == 0 && BN <= 256, "whole W pieces per thread");
         static_assert((DL_S == 4 || DL_S == 8) && WAVES_M == 2 && WAVES_N >= 2, "ring of four or eight stages, 2 x N wavefronts");
@@ -653,14 +653,6 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         const uint32_t lds0 = (uint32_t) reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char *)smem) +
                               (uint32_t)(wave_u * 1024);
         const uint32_t w_kstep = WMODE == W_ROWS_DL ? (uint32_t)BK : (uint32_t)BK * (uint32_t)g.ldw;
-        auto issue = [&](int buf, int step) {  // `step` is wave-uniform: the K advance is a scalar offset
-            const uint32_t xd = lds0 + (uint32_t)(buf * DL_STAGE), wd = xd + BM * BK;
-            const uint32_t xk = (uint32_t)step * BK, wk = (uint32_t)step * w_kstep;
-#pragma unroll
-            for (int i = 0; i < XI; i++) load16_to_lds(xres4, xd + i * NTHREADS * 16, xo[i], xk);
-#pragma unroll
-            for (int i = 0; i < WI; i++) load16_to_lds(wres4, wd + i * NTHREADS * 16, wo[i], wk);
-        };
         // operand addresses inside a stage: lane base (per K half) + compile-time offset
         const int h = lane >> 5;
         const int xswz = ((lane >> 2) & 3);

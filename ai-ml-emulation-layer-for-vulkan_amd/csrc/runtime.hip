@@ -208,6 +208,120 @@ __global__ void __launch_bounds__(256) mfma_rate_kernel(const v4i_probe *__restr
     out[tid] = sum;
 }
 
+// What a wavefront that is alone on its SIMD can issue while its matrix instructions run: one round of `MODE` per
+// iteration, written as inline assembly so that the order is the order below; the first wavefront of block 0 reports
+// the clocks it took (s_memtime) per iteration.  The modes are the pieces of a contraction loop: four
+// v_mfma_i32_32x32x32_i8; sixteen v_dot4 / v_add_u32 / v_sad_u8 (zero-point sums); six 128-bit reads of shared memory;
+// four 16-byte-per-lane loads into shared memory; four v_mfma_i32_16x16x64_i8 -- each alone, behind the four matrix
+// instructions, and dealt out between them.
+#define MLEL_PROBE_MF(a, x, w) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(a) : "v"(x), "v"(w))
+#define MLEL_PROBE_MS(a, x, w) asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(a) : "v"(x), "v"(w))
+#define MLEL_PROBE_DOT(s, x) asm volatile("v_dot4c_i32_i8 %0, %1, %2" : "+v"(s) : "v"(ones), "v"(x))
+#define MLEL_PROBE_ADD(s, x) asm volatile("v_add_u32 %0, %0, %1" : "+v"(s) : "v"(x))
+#define MLEL_PROBE_SAD(s, x) asm volatile("v_sad_u8 %0, %1, 0, %0" : "+v"(s) : "v"(x))
+#define MLEL_PROBE_READ(d, p, off) asm volatile("ds_read_b128 %0, %1 offset:" #off : "=v"(d) : "v"(p))
+#define MLEL_PROBE_LOAD(off)                                                                                      \
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_wave + off), "v"(goff), \
+                 "s"(rs)                                                                                          \
+                 : "memory")
+template <int MODE>
+__global__ void __launch_bounds__(256) issue_probe_kernel(const int32_t *__restrict__ operands, uint32_t *__restrict__ out,
+                                                          int iters) {
+    __shared__ __align__(16) char lds[32768];
+    v16i_probe a0, a1, a2, a3;
+#pragma unroll
+    for (int r = 0; r < 16; r++) a0[r] = a1[r] = a2[r] = a3[r] = 0;
+    const int t = threadIdx.x;
+    v4i_probe x0, x1, w0, w1, m0 = {0, 0, 0, 0}, m1 = {0, 0, 0, 0}, m2 = {0, 0, 0, 0}, m3 = {0, 0, 0, 0};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        x0[e] = operands[(t * 16 + e) & 16383];
+        x1[e] = operands[(t * 16 + 4 + e) & 16383];
+        w0[e] = operands[(t * 16 + 8 + e) & 16383];
+        w1[e] = operands[(t * 16 + 12 + e) & 16383];
+    }
+    int s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+    const int ones = 0x01010101;
+    const uint32_t p = (uint32_t)(t * 16);
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(
+        (uint32_t) reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char *)lds) + (uint32_t)(t >> 6) * 4096u);
+    const uint32_t goff = (uint32_t)(t & 63) * 16u + (uint32_t)(blockIdx.x & 15) * 4096u;
+    const uint64_t ga = reinterpret_cast<uint64_t>(operands);
+    const v4i_probe rs = {(int)(uint32_t)ga, (int)(uint32_t)(ga >> 32), 65536, 0x00020000};
+    v4i_probe d0 = x0, d1 = x0, d2 = x0, d3 = x0, d4 = x0, d5 = x0;
+    for (int i = t; i < 8192; i += 256) reinterpret_cast<int *>(lds)[i] = i;
+    __syncthreads();
+    const uint64_t t0 = __builtin_readcyclecounter();
+    for (int it = 0; it < iters; it++) {
+        if (MODE == 0) { MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_MF(a3, x1, w1); }
+        if (MODE == 1 || MODE == 2) {
+            if (MODE == 2) { MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_MF(a3, x1, w1); }
+#pragma unroll
+            for (int e = 0; e < 4; e++) { MLEL_PROBE_DOT(s0, x0[e]); MLEL_PROBE_DOT(s1, x1[e]); MLEL_PROBE_DOT(s2, w0[e]); MLEL_PROBE_DOT(s3, w1[e]); }
+        }
+        if (MODE == 3) {
+            MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_DOT(s0, x0[0]); MLEL_PROBE_DOT(s1, x1[0]); MLEL_PROBE_DOT(s2, w0[0]); MLEL_PROBE_DOT(s3, w1[0]);
+            MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_DOT(s0, x0[1]); MLEL_PROBE_DOT(s1, x1[1]); MLEL_PROBE_DOT(s2, w0[1]); MLEL_PROBE_DOT(s3, w1[1]);
+            MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_DOT(s0, x0[2]); MLEL_PROBE_DOT(s1, x1[2]); MLEL_PROBE_DOT(s2, w0[2]); MLEL_PROBE_DOT(s3, w1[2]);
+            MLEL_PROBE_MF(a3, x1, w1); MLEL_PROBE_DOT(s0, x0[3]); MLEL_PROBE_DOT(s1, x1[3]); MLEL_PROBE_DOT(s2, w0[3]); MLEL_PROBE_DOT(s3, w1[3]);
+        }
+        if (MODE == 4 || MODE == 5) {
+            if (MODE == 5) { MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_MF(a3, x1, w1); }
+#pragma unroll
+            for (int e = 0; e < 4; e++) { MLEL_PROBE_ADD(s0, x0[e]); MLEL_PROBE_ADD(s1, x1[e]); MLEL_PROBE_ADD(s2, w0[e]); MLEL_PROBE_ADD(s3, w1[e]); }
+        }
+        if (MODE == 6) {
+            MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_ADD(s0, x0[0]); MLEL_PROBE_ADD(s1, x1[0]); MLEL_PROBE_ADD(s2, w0[0]); MLEL_PROBE_ADD(s3, w1[0]);
+            MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_ADD(s0, x0[1]); MLEL_PROBE_ADD(s1, x1[1]); MLEL_PROBE_ADD(s2, w0[1]); MLEL_PROBE_ADD(s3, w1[1]);
+            MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_ADD(s0, x0[2]); MLEL_PROBE_ADD(s1, x1[2]); MLEL_PROBE_ADD(s2, w0[2]); MLEL_PROBE_ADD(s3, w1[2]);
+            MLEL_PROBE_MF(a3, x1, w1); MLEL_PROBE_ADD(s0, x0[3]); MLEL_PROBE_ADD(s1, x1[3]); MLEL_PROBE_ADD(s2, w0[3]); MLEL_PROBE_ADD(s3, w1[3]);
+        }
+        if (MODE == 7) {
+            MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_SAD(s0, x0[0]); MLEL_PROBE_SAD(s1, x1[0]); MLEL_PROBE_SAD(s2, w0[0]); MLEL_PROBE_SAD(s3, w1[0]);
+            MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_SAD(s0, x0[1]); MLEL_PROBE_SAD(s1, x1[1]); MLEL_PROBE_SAD(s2, w0[1]); MLEL_PROBE_SAD(s3, w1[1]);
+            MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_SAD(s0, x0[2]); MLEL_PROBE_SAD(s1, x1[2]); MLEL_PROBE_SAD(s2, w0[2]); MLEL_PROBE_SAD(s3, w1[2]);
+            MLEL_PROBE_MF(a3, x1, w1); MLEL_PROBE_SAD(s0, x0[3]); MLEL_PROBE_SAD(s1, x1[3]); MLEL_PROBE_SAD(s2, w0[3]); MLEL_PROBE_SAD(s3, w1[3]);
+        }
+        if (MODE == 8 || MODE == 9) {
+            if (MODE == 9) { MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_MF(a3, x1, w1); }
+            MLEL_PROBE_READ(d0, p, 0); MLEL_PROBE_READ(d1, p, 4096); MLEL_PROBE_READ(d2, p, 8192);
+            MLEL_PROBE_READ(d3, p, 12288); MLEL_PROBE_READ(d4, p, 16384); MLEL_PROBE_READ(d5, p, 20480);
+            asm volatile("s_waitcnt lgkmcnt(0)");
+        }
+        if (MODE == 10) {
+            MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_READ(d0, p, 0); MLEL_PROBE_READ(d1, p, 4096);
+            MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_READ(d2, p, 8192); MLEL_PROBE_READ(d3, p, 12288);
+            MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_READ(d4, p, 16384); MLEL_PROBE_READ(d5, p, 20480);
+            MLEL_PROBE_MF(a3, x1, w1);
+            asm volatile("s_waitcnt lgkmcnt(0)");
+        }
+        if (MODE == 11 || MODE == 12) {
+            if (MODE == 12) { MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_MF(a3, x1, w1); }
+            MLEL_PROBE_LOAD(0); MLEL_PROBE_LOAD(1024); MLEL_PROBE_LOAD(2048); MLEL_PROBE_LOAD(3072);
+            asm volatile("s_waitcnt vmcnt(4)");
+        }
+        if (MODE == 13) {
+            MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_LOAD(0); MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_LOAD(1024);
+            MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_LOAD(2048); MLEL_PROBE_MF(a3, x1, w1); MLEL_PROBE_LOAD(3072);
+            asm volatile("s_waitcnt vmcnt(4)");
+        }
+        if (MODE == 14) {
+            MLEL_PROBE_MF(a0, x0, w0); MLEL_PROBE_MS(m0, x0, w0); MLEL_PROBE_MF(a1, x0, w1); MLEL_PROBE_MS(m1, x1, w0);
+            MLEL_PROBE_MF(a2, x1, w0); MLEL_PROBE_MS(m2, w0, x0); MLEL_PROBE_MF(a3, x1, w1); MLEL_PROBE_MS(m3, w1, x0);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)");
+    const uint64_t t1 = __builtin_readcyclecounter();
+    int sum = s0 + s1 + s2 + s3 + d0[0] + d1[1] + d2[2] + d3[3] + d4[0] + d5[1] + m0[0] + m1[1] + m2[2] + m3[3];
+#pragma unroll
+    for (int r = 0; r < 16; r++) sum += a0[r] + a1[r] + a2[r] + a3[r];
+    out[2 + blockIdx.x * 256 + t] = (uint32_t)sum;
+    if (t == 0 && blockIdx.x == 0) {
+        out[0] = (uint32_t)(t1 - t0);
+        out[1] = (uint32_t)((t1 - t0) >> 32);
+    }
+}
+
 // Byte fill for streams under capture, where a memset node must not be recorded: 16-byte stores over the aligned
 // middle, single bytes at the two ragged ends.
 __global__ void __launch_bounds__(256) fill_kernel(unsigned char *__restrict__ dst, size_t head, size_t n_vec,
@@ -597,6 +711,25 @@ int mlel_hip_mfma_rate_probe(mlel_ctx *ctx, void *stream, const void *operands, 
     hipLaunchKernelGGL(mfma_rate_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                        (const v4i_probe *)operands, (int32_t *)out, iters);
     return check_launch("mfma_rate_probe");
+}
+
+int mlel_hip_issue_probe(mlel_ctx *ctx, void *stream, const void *operands, void *out, int mode, int iters) {
+    MLEL_REQUIRE(ctx != nullptr && operands != nullptr && out != nullptr, MLEL_ERR_INVALID, "issue_probe: null argument");
+    MLEL_REQUIRE(iters > 0 && mode >= 0 && mode <= 14, MLEL_ERR_INVALID, "issue_probe: mode 0 .. 14, iters positive");
+    MLEL_REQUIRE(((uintptr_t)operands % 16) == 0 && ((uintptr_t)out % 4) == 0, MLEL_ERR_INVALID,
+                 "issue_probe: operands must be 16-byte aligned");
+    const int blocks = ctx->props.multiProcessorCount > 0 ? ctx->props.multiProcessorCount : 256;  // one wavefront per SIMD
+    const int32_t *ops = (const int32_t *)operands;
+    uint32_t *o = (uint32_t *)out;
+    hipStream_t st = (hipStream_t)stream;
+#define MLEL_ISSUE_CASE(M) case M: hipLaunchKernelGGL(issue_probe_kernel<M>, dim3((unsigned)blocks), dim3(256), 0, st, ops, o, iters); break;
+    switch (mode) {
+        MLEL_ISSUE_CASE(0) MLEL_ISSUE_CASE(1) MLEL_ISSUE_CASE(2) MLEL_ISSUE_CASE(3) MLEL_ISSUE_CASE(4) MLEL_ISSUE_CASE(5)
+        MLEL_ISSUE_CASE(6) MLEL_ISSUE_CASE(7) MLEL_ISSUE_CASE(8) MLEL_ISSUE_CASE(9) MLEL_ISSUE_CASE(10) MLEL_ISSUE_CASE(11)
+        MLEL_ISSUE_CASE(12) MLEL_ISSUE_CASE(13) MLEL_ISSUE_CASE(14)
+    }
+#undef MLEL_ISSUE_CASE
+    return check_launch("issue_probe");
 }
 
 int mlel_hip_copy_kernel_variant(mlel_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes, int blocks,

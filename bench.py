@@ -16,7 +16,8 @@ graph 200 times back to back and nothing else, so that counters of a single laye
 (the bandwidth-bound operators as stand-alone launches on config 2's and on config 3's largest tensors), `copy` (the
 plain copy kernel over grid and size: the measured HBM ceiling), `extra` (data-movement operators outside the
 benchmark graphs), `vendor` (the GPU vendor's matrix library through torch on the products timed here, as a calibration
-of the box; nothing of the product runs in that leg).  `ms_per_step` is the median over at least 10 rounds of `--steps` launches; the whole-graph legs
+of the box; nothing of the product runs in that leg), `issue` (what a lone wavefront issues while its matrix
+instructions run: the instruction mixes of a contraction loop alone, behind and between the matrix instructions).  `ms_per_step` is the median over at least 10 rounds of `--steps` launches; the whole-graph legs
 report the median over rounds that hold at least 50 graphs.
 """
 import re
@@ -318,6 +319,40 @@ def bench_mfma_rate(dev, info):
     return res
 
 
+ISSUE_MODES = [
+    (0, "4 x v_mfma_i32_32x32x32_i8"),
+    (1, "16 x v_dot4"), (2, "4 matrix instructions, then 16 x v_dot4"), (3, "matrix instruction + 4 x v_dot4, four times"),
+    (4, "16 x v_add_u32"), (5, "4 matrix instructions, then 16 x v_add_u32"), (6, "matrix instruction + 4 x v_add_u32, four times"),
+    (7, "matrix instruction + 4 x v_sad_u8, four times"),
+    (8, "6 x ds_read_b128 + wait"), (9, "4 matrix instructions, then 6 x ds_read_b128 + wait"),
+    (10, "matrix instruction + 2 reads, three times, matrix instruction, wait"),
+    (11, "4 x buffer_load_dwordx4 ... lds"), (12, "4 matrix instructions, then 4 loads to LDS"),
+    (13, "matrix instruction + load to LDS, four times"),
+    (14, "matrix instruction + v_mfma_i32_16x16x64_i8, four times"),
+]
+
+
+def bench_issue_probe(dev, info, iters=512):
+    """What a wavefront alone on its SIMD issues in the shadow of its matrix instructions (mlel_hip_issue_probe): clocks
+    per round of every instruction mix, one block of four wavefronts per compute unit, random operand bytes."""
+    data = np.random.default_rng(11).integers(0, 255, 65536, endpoint=True).astype(np.uint8)
+    t = dev.from_numpy(data)
+    n_out = 2 + 256 * info["compute_units"]
+    out = dev.tensor(importlib.import_module(PKG + ".abi").I32, (n_out,))
+    rows = []
+    for mode, name in ISSUE_MODES:
+        for _ in range(2):  # the second launch is the one that counts (code and operands are then resident)
+            dev._check(dev.lib.mlel_hip_issue_probe(dev.ctx, dev.stream, C.c_void_p(t.ptr), C.c_void_p(out.ptr), mode, iters))
+        dev.sync()
+        w = out.download().view(np.uint32)
+        clocks = int(w[0]) | (int(w[1]) << 32)
+        rows.append({"mode": mode, "instructions": name, "clocks_per_round": round(clocks / iters, 1)})
+        log("issue probe:", rows[-1])
+    t.free()
+    out.free()
+    return rows
+
+
 def measure_copy(dev, nbytes, reps=5):
     src, dst = dev.alloc(nbytes), dev.alloc(nbytes)
     best = 0.0
@@ -605,7 +640,7 @@ def main():
                     help="omit the legs with several launches / sessions in flight (profiling runs: one kernel at a time)")
     ap.add_argument("--skip-graph", action="store_true", help="omit the MobileNetV2 and encoder graph legs")
     ap.add_argument("--only", choices=["all", "config0", "config1", "config2", "mobilenetv2", "encoder", "gemm_large",
-                                       "layer", "standalone", "copy", "extra", "vendor"], default="all")
+                                       "layer", "standalone", "copy", "extra", "vendor", "issue"], default="all")
     ap.add_argument("--layer", type=int, default=3, help="with --only layer: position in the fused config 3 graph")
     ap.add_argument("--gemm-size", type=int, default=0, help="with --only gemm_large: this one size instead of 4096 and 8192")
     args = ap.parse_args()
@@ -637,6 +672,11 @@ def main():
     if args.only == "copy":
         print(json.dumps(dict({"only": "copy", "mfma_rate": bench_mfma_rate(dev, info)}, **bench_copy_sweep(dev, info))),
               flush=True)
+        dev.close()
+        return
+
+    if args.only == "issue":
+        print(json.dumps({"only": "issue", "rounds": bench_issue_probe(dev, info)}), flush=True)
         dev.close()
         return
 

@@ -607,6 +607,14 @@ int mlel_hip_copy_kernel_variant(mlel_ctx *ctx, void *stream, void *dst, const v
  * 2 x 32 x 32 x 32 x 8 x iters operations per wavefront.  No counterpart in the reference; a measurement aid: the
  * rate a contraction kernel on this part is to be read against beside the published peak. */
 int mlel_hip_mfma_rate_probe(mlel_ctx *ctx, void *stream, const void *operands, void *out, int blocks, int iters);
+/* What a wavefront that is alone on its SIMD issues while its matrix instructions run: one block of four wavefronts
+ * per compute unit, `iters` rounds of the instruction mix `mode` each (0 four v_mfma_i32_32x32x32_i8; 1 sixteen
+ * v_dot4, 2 behind the four matrix instructions, 3 dealt out between them; 4 / 5 / 6 the same with v_add_u32, 7 with
+ * v_sad_u8 dealt out; 8 / 9 / 10 six 128-bit shared-memory reads; 11 / 12 / 13 four loads into shared memory; 14 four
+ * v_mfma_i32_16x16x64_i8 dealt out).  `operands`: 64 KiB; `out`: (2 + 256 x compute units) dwords, of which the first two
+ * receive the clocks the first wavefront took for all rounds.  No counterpart in the reference; a measurement aid:
+ * the order of the instructions in the contraction kernels' loops follows from these figures. */
+int mlel_hip_issue_probe(mlel_ctx *ctx, void *stream, const void *operands, void *out, int mode, int iters);
 
 #ifdef __cplusplus
 }
