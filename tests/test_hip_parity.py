@@ -1461,6 +1461,35 @@ def test_copy_kernels_move_exactly_the_requested_bytes(run):
         dev._check(lib.mlel_hip_copy_kernel_variant(dev.ctx, dev.stream, C.c_void_p(ts.ptr), C.c_void_p(ts.ptr), 24, 0, 1, 0, 0))
 
 
+def test_issue_probe_runs_every_mix_and_rejects_bad_arguments(run):
+    """mlel_hip_issue_probe: every instruction mix finishes and reports a clock count that grows with the rounds; the
+    matrix instructions alone are never slower than the same four with other instructions behind them; a mode outside
+    the list, no rounds and a misaligned operand pointer are refused before any launch."""
+    import ctypes as C
+    dev, lib = run.dev, run.dev.lib
+    ops = run.put(ri(np.random.default_rng(3), 0, 255, (65536,), np.uint8))
+    cus = int(dev.info()["compute_units"])
+    out = run.put(np.zeros(2 + 256 * cus, np.int32))
+
+    def clocks(mode, iters):
+        dev._check(lib.mlel_hip_issue_probe(dev.ctx, dev.stream, C.c_void_p(ops.ptr), C.c_void_p(out.ptr), mode, iters))
+        w = out.download().view(np.uint32)
+        return int(w[0]) | (int(w[1]) << 32)
+
+    alone = None
+    for mode in range(15):
+        clocks(mode, 64)
+        short, long_ = clocks(mode, 64), clocks(mode, 256)
+        assert 0 < short < long_ < 256 * 4000, (mode, short, long_)
+        if mode == 0:
+            alone = long_
+    assert alone * 0.9 <= clocks(2, 256)
+    for mode, iters, ptr in ((15, 8, ops.ptr), (-1, 8, ops.ptr), (0, 0, ops.ptr), (0, 8, ops.ptr + 4)):
+        with pytest.raises(hb.MlelError):
+            dev._check(lib.mlel_hip_issue_probe(dev.ctx, dev.stream, C.c_void_p(ptr), C.c_void_p(out.ptr), mode, iters))
+    run.done()
+
+
 def test_split_k_workspaces_are_released_with_their_streams(run, oracle):
     """More streams than the context has workspace slots, one after the other: each splits K (its workspace appears),
     matches the oracle, and gives the workspace back when it is destroyed -- the twentieth stream still splits."""
