@@ -319,6 +319,12 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                  "s"(g.div_band.m), "s"(g.div_band.s), "s"(g.div_last_rows.m), "s"(g.div_last_rows.s), "s"(g.x), "s"(g.w),
                  "s"(g.x_batch), "s"(g.w_batch), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.x_sx), "s"(g.ldw), "s"(g.x_bytes),
                  "s"(g.w_bytes));
+    // The epilogue's arguments ride along: the compiler asks for them up here in any case, but behind the early exit
+    // and in registers that the tile assignment is still writing, so the assignment waited for them to arrive first.
+    asm volatile("" ::"s"(g.out), "s"(g.out_batch), "s"(g.ldo), "s"(g.o_bytes), "s"(g.fused), "s"(g.mult), "s"(g.shift),
+                 "s"(g.mult16), "s"(g.rp.in_zp), "s"(g.rp.out_zp), "s"(g.rp.out_lo), "s"(g.rp.out_hi),
+                 "s"(g.rp.double_round), "s"(g.rp.per_channel), "s"(g.rp.clamp_out), "s"(g.zx), "s"(g.zw), "s"(g.bias),
+                 "s"(g.bias_len));
     const int lin_all = (int)(blockIdx.x % 8) * g.chunk + (int)(blockIdx.x / 8);
     if (lin_all >= g.total_tiles * g.splits) return;
     // the splits of one tile are consecutive, so they run on one XCD and exchange their partials through its L2
