@@ -56,6 +56,7 @@ struct AttnArgs {
     int64_t vs_nb1, vs_nb2;
     uint32_t vs_m1, vs_m2, vs_n1;
     int32_t total, chunk, fold_span;
+    DivMagic div_strips;  // block index / strips as a multiplication and a shift
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const void *p, uint32_t bytes) {
@@ -81,9 +82,16 @@ __global__ void __launch_bounds__(kBlock) attention_f16_kernel(const AttnArgs g)
     char *st = smem;               // [64][SP]: one pass of S, later of EXP(..), later of P
     char *cb = smem + kRows * SP;  // [64][kChunkPitch]: a chunk of K^T or V; the row sums; the staged result
 
+    // every argument in one batch: left alone the compiler loads all but the exit test's behind the exit, a second
+    // trip to memory in a row before the first address
+    asm volatile("" ::"s"(g.chunk), "s"(g.total), "s"(g.fold_span), "s"(g.div_strips.m), "s"(g.div_strips.s), "s"(g.q),
+                 "s"(g.kt), "s"(g.v), "s"(g.out), "s"(g.scale), "s"(g.M), "s"(g.S), "s"(g.batches), "s"(g.strips),
+                 "s"(g.q_batch), "s"(g.kt_batch), "s"(g.v_batch), "s"(g.o_batch), "s"(g.ldq), "s"(g.ldkt), "s"(g.ldv),
+                 "s"(g.ldo), "s"(g.q_bytes), "s"(g.kt_bytes), "s"(g.v_bytes), "s"(g.o_bytes), "s"(g.view), "s"(g.v_nb2),
+                 "s"(g.v_m2), "s"(g.v_n2), "s"(g.vs_nb1), "s"(g.vs_nb2), "s"(g.vs_m1), "s"(g.vs_m2), "s"(g.vs_n1));
     const int lin = __builtin_amdgcn_readfirstlane((int)(blockIdx.x % 8u) * g.chunk + (int)(blockIdx.x / 8u));
     if (lin >= g.total) return;
-    const int batch = lin / g.strips;
+    const int batch = div_magic(lin, g.div_strips);
     const int m0 = (lin - batch * g.strips) * kRows;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;  // the wavefront's 32 x 32 tile of a 64 x 64 product
@@ -453,6 +461,7 @@ int describe(const mlel_tensor *out, const mlel_tensor *q, const mlel_tensor *kt
     g.S = (int32_t)S;
     g.batches = (int32_t)NB;
     g.strips = (int32_t)(M / kRows);
+    g.div_strips = make_div_magic((uint32_t)g.strips);
     g.q_batch = q->strides[0];
     g.kt_batch = kt->strides[0];
     g.v_batch = v->strides[0];

@@ -94,6 +94,15 @@ __global__ void __launch_bounds__(NT) conv1x1_dw3x3_i8_kernel(const ConvDwArgs a
     asm volatile("" ::"s"(a.chunk), "s"(a.blocks), "s"(a.slices), "s"(a.bands), "s"(a.band_out), "s"(a.OH), "s"(a.pad_t),
                  "s"(a.th), "s"(a.H), "s"(a.W), "s"(a.x), "s"(a.x_bytes), "s"(a.P), "s"(a.IC), "s"(a.w1), "s"(a.div_slices.m),
                  "s"(a.div_slices.s), "s"(a.div_bands.m), "s"(a.div_bands.s));
+    // the rest of what the kernel reads before its first request, and every dword of the wide loads that bring it (a
+    // register that nobody waits for is given away at once, and whoever gets it waits for the load to land first)
+    asm volatile("" ::"s"(a.o_bytes), "s"(a.tw), "s"(a.strips), "s"(a.row_groups), "s"(a.items), "s"(a.strips_magic),
+                 "s"(a.w_magic), "s"(a.zx), "s"(a.zi), "s"(a.b1_len), "s"(a.b2_len), "s"(a.pad_l), "s"(a.C), "s"(a.OW),
+                 "s"(a.N), "s"(a.w2), "s"(a.b1), "s"(a.b2), "s"(a.out), "s"(a.s1.mult), "s"(a.s1.shift), "s"(a.s1.mult16),
+                 "s"(a.s1.p.in_zp), "s"(a.s1.p.out_zp), "s"(a.s1.p.out_lo), "s"(a.s1.p.out_hi), "s"(a.s1.p.double_round),
+                 "s"(a.s1.p.per_channel), "s"(a.s1.p.clamp_out), "s"(a.s2.mult), "s"(a.s2.shift), "s"(a.s2.mult16),
+                 "s"(a.s2.p.in_zp), "s"(a.s2.p.out_zp), "s"(a.s2.p.out_lo), "s"(a.s2.p.out_hi), "s"(a.s2.p.double_round),
+                 "s"(a.s2.p.per_channel), "s"(a.s2.p.clamp_out));
     const int bid = (int)(blockIdx.x % 8u) * a.chunk + (int)(blockIdx.x / 8u);
     if (bid >= a.blocks) return;
     const int rest_b = div_magic(bid, a.div_slices), slice = bid - rest_b * a.slices;

@@ -39,6 +39,9 @@ struct HGemmArgs {
     uint32_t lda, ldb, ldo;             // bytes per row
     uint32_t a_bytes, b_bytes, o_bytes; // per-batch extents (all below 2^31)
     int32_t tiles_m, tiles_n, total_tiles, chunk;
+    // the tile index divided by tiles per batch, tiles per row and tiles per product as a multiplication and a shift
+    // (set by launch_k from the fields above and tiles_n_group)
+    DivMagic div_per_batch, div_tiles_n, div_group;
     // fused epilogue (EPI = 1): out = fp16(acc + bias[n]) with the addition in fp32; bias may be null
     const float *bias;
     int32_t bias_len;  // 1 (broadcast) or N
@@ -148,24 +151,38 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
     char *xs = smem;             // [2][BM][XPITCH]
     char *ws = smem + 2 * XBUF;  // [2][BKH][WPITCH]
 
+    // Every argument that the tile assignment and the first operand requests depend on is asked for here, in one
+    // batch (every dword of the wide loads that bring them named: a register nobody waits for is given away at once,
+    // and whoever gets it waits for the load first).  Left alone the compiler loads arguments where they are first
+    // used, behind the early exit, behind three divisions and behind each other: five to nine trips to memory in a
+    // row before a wavefront's first address.
+    asm volatile("" ::"s"(g.chunk), "s"(g.total_tiles), "s"(g.tiles_m), "s"(g.tiles_n), "s"(g.div_per_batch.m),
+                 "s"(g.div_per_batch.s), "s"(g.div_tiles_n.m), "s"(g.div_tiles_n.s), "s"(g.div_group.m), "s"(g.div_group.s),
+                 "s"(g.groups), "s"(g.tiles_n_group), "s"(g.a), "s"(g.b), "s"(g.extra[0].b), "s"(g.extra[1].b), "s"(g.out),
+                 "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.batches), "s"(g.b_rows), "s"(g.a_batch), "s"(g.b_batch), "s"(g.o_batch),
+                 "s"(g.lda), "s"(g.ldb), "s"(g.ldo), "s"(g.a_bytes), "s"(g.b_bytes), "s"(g.o_bytes),
+                 // the pointers of the epilogue, which the compiler follows up here already (the activation's scalars)
+                 "s"(g.bias), "s"(g.bias_len), "s"(g.res), "s"(g.act[0]), "s"(g.act[1]), "s"(g.act[2]), "s"(g.act[3]));
     // consecutive tiles (sharing operand panels) go to the same XCD; blocks are dealt to XCDs round-robin
     const int lin = __builtin_amdgcn_readfirstlane((int)(blockIdx.x % 8u) * g.chunk + (int)(blockIdx.x / 8u));
     if (lin >= g.total_tiles) return;
     const int per_batch = g.tiles_m * g.tiles_n;
-    const int batch = lin / per_batch;
+    const int batch = div_magic(lin, g.div_per_batch);
     const int t_in = lin - batch * per_batch;
-    const int tile_m = t_in / g.tiles_n;
+    const int tile_m = div_magic(t_in, g.div_tiles_n);
     int tile_n = t_in - tile_m * g.tiles_n;
     HProduct o{g.b, g.bias, g.out, g.o_batch, g.ldo, g.o_bytes, g.view, g.v_nb2, g.v_m2, g.v_n2, g.vs_nb1, g.vs_nb2,
                g.vs_m1, g.vs_m2, g.vs_n1, g.vs_n2};
     if (g.groups > 1) {  // uniform
-        const int product = tile_n / g.tiles_n_group;
+        const int product = div_magic(tile_n, g.div_group);
         tile_n -= product * g.tiles_n_group;
         if (product > 0) {
             const HGemmArgs::Extra &e = product == 1 ? g.extra[0] : g.extra[1];
             o = HProduct{e.b, e.bias, e.out, e.o_batch, e.ldo, e.o_bytes, e.view, e.v_nb2, e.v_m2, e.v_n2, e.vs_nb1, e.vs_nb2,
                          e.vs_m1, e.vs_m2, e.vs_n1, e.vs_n2};
         }
+        // the operand pointer is on the way to the first request: picked from registers that are already there
+        o.b = product == 0 ? g.b : (product == 1 ? g.extra[0].b : g.extra[1].b);
     }
     const int m_base = tile_m * BM, n_base = tile_n * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -536,7 +553,11 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BKH, bool BROWS = false>
-void launch_k(const HGemmArgs &g, bool cast_epilogue, dim3 grid, hipStream_t s) {
+void launch_k(const HGemmArgs &args, bool cast_epilogue, dim3 grid, hipStream_t s) {
+    HGemmArgs g = args;
+    g.div_per_batch = make_div_magic((uint32_t)(g.tiles_m * g.tiles_n));
+    g.div_tiles_n = make_div_magic((uint32_t)g.tiles_n);
+    g.div_group = make_div_magic((uint32_t)(g.tiles_n_group > 0 ? g.tiles_n_group : 1));
     constexpr size_t operands = BROWS ? (size_t)4 * (BM + BN) * 64
                                       : (size_t)2 * BM * (BKH * 2 + 16) + (size_t)2 * BKH * (2 * BN + 32);
     constexpr size_t result = std::max((size_t)BM * (BN * 2 + 16), (size_t)BN * (BM * 2 + 16));

@@ -39,18 +39,26 @@ __device__ __forceinline__ int32_t lds_entry(const int32_t *table, uint32_t w, i
 // quarter of the K chunks, the partial tiles are added through shared memory (int32 addition wraps: the order is
 // immaterial) and each wavefront requantises and stores a quarter of the tile (eight of its 32 positions).
 template <bool RES, int KS>
-__global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const GemmArgs g, int groups_n, int total_waves) {
+__global__ void __launch_bounds__(kColsBlock) conv_cols_mfma_i8_kernel(const GemmArgs g, int groups_n, int total_waves,
+                                                                         const DivMagic div_groups_n, int chunk) {
+    // every argument that the tile assignment, the first operand requests and the epilogue depend on, asked for in one
+    // batch: left alone the compiler loads most of them behind the early exit, a second trip to memory in a row
+    asm volatile("" ::"s"(total_waves), "s"(groups_n), "s"(div_groups_n.m), "s"(div_groups_n.s), "s"(chunk), "s"(g.x), "s"(g.w),
+                 "s"(g.x_bytes), "s"(g.w_bytes), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.batches), "s"(g.x_sx), "s"(g.ldw), "s"(g.ldo),
+                 "s"(g.o_bytes), "s"(g.out), "s"(g.bias), "s"(g.bias_len), "s"(g.zx), "s"(g.mult), "s"(g.shift),
+                 "s"(g.mult16), "s"(g.rp.out_zp), "s"(g.rp.out_lo), "s"(g.rp.out_hi), "s"(g.rp.double_round),
+                 "s"(g.rp.per_channel));
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // blocks are dealt round-robin to the XCDs: XCD k gets the k-th contiguous run of blocks, so the tiles of a
     // pixel row group (which read the same 32 pixel rows) fetch them into one L2
-    const int chunk = (int)gridDim.x >> 3;  // the grid is a multiple of eight blocks
+    // (`chunk`: an eighth of the grid, which is a multiple of eight blocks)
     const int bid = (int)(blockIdx.x % 8u) * chunk + (int)(blockIdx.x / 8u);
     const int wid = KS == 1 ? bid * (kColsBlock / 64) + wave : bid;
     // whole wavefronts (KS == 1) or whole blocks (KS == 4) have nothing to do; with the residual stage a wavefront
     // stays for the block's table and its barrier and leaves behind it
     if (!(RES && KS == 1) && wid >= total_waves) return;
-    const int mg = wid / groups_n, ng = wid - mg * groups_n;
+    const int mg = div_magic(wid, div_groups_n), ng = wid - mg * groups_n;
     const int cl = lane & 31, half = lane >> 5;
     const int m = mg * 32 + cl, n = ng * 32 + cl;
     const __amdgpu_buffer_rsrc_t xres = make_rsrc(g.x, g.x_bytes), wres = make_rsrc(g.w, g.w_bytes);
@@ -217,15 +225,21 @@ struct ColsPoolArgs {
     int32_t positions; // per image (H * W <= 64)
     int32_t images, pairs, total_blocks;
     int32_t zi, zo;
+    DivMagic div_pairs;  // block index / pairs
+    int32_t chunk;       // an eighth of the grid
 };
 
 __global__ void __launch_bounds__(kColsBlock) conv_cols_pool_i8_kernel(const GemmArgs g, const ColsPoolArgs pa) {
+    asm volatile("" ::"s"(pa.total_blocks), "s"(pa.pairs), "s"(pa.div_pairs.m), "s"(pa.div_pairs.s), "s"(pa.chunk), "s"(pa.positions),
+                 "s"(pa.out), "s"(pa.zi), "s"(pa.zo), "s"(g.x), "s"(g.w), "s"(g.x_bytes), "s"(g.w_bytes), "s"(g.M), "s"(g.N), "s"(g.K),
+                 "s"(g.batches), "s"(g.x_sx), "s"(g.ldw), "s"(g.bias), "s"(g.bias_len), "s"(g.zx), "s"(g.mult), "s"(g.shift), "s"(g.mult16),
+                 "s"(g.rp.out_zp), "s"(g.rp.out_lo), "s"(g.rp.out_hi), "s"(g.rp.double_round), "s"(g.rp.per_channel),
+                 "s"(g.rp.clamp_out));  // (every dword of a wide load named: a register nobody waits for is given away at once)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int chunk = (int)gridDim.x >> 3;
-    const int bid = (int)(blockIdx.x % 8u) * chunk + (int)(blockIdx.x / 8u);
+    const int bid = (int)(blockIdx.x % 8u) * pa.chunk + (int)(blockIdx.x / 8u);
     if (bid >= pa.total_blocks) return;
-    const int image = bid / pa.pairs, pair = bid - image * pa.pairs;
+    const int image = div_magic(bid, pa.div_pairs), pair = bid - image * pa.pairs;
     const int t = wave & 1, ng = pair * 2 + (wave >> 1);
     const int cl = lane & 31, half = lane >> 5;
     const int pos = 32 * t + cl;  // this lane's pixel row of the image
@@ -318,8 +332,8 @@ int launch_conv_cols_pool(const void *args, int8_t *pool_out, int images, int po
     const int64_t blocks = (int64_t)images * pairs;
     if (blocks >= (int64_t(1) << 24)) return 0;
     if (probe) return 1;
-    ColsPoolArgs pa{pool_out, positions, images, (int)pairs, (int)blocks, zi, zo};
     const dim3 grid((unsigned)((blocks + 7) / 8 * 8));
+    ColsPoolArgs pa{pool_out, positions, images, (int)pairs, (int)blocks, zi, zo, make_div_magic((uint32_t)pairs), (int)(grid.x / 8)};
     conv_cols_pool_i8_kernel<<<grid, dim3(kColsBlock), 0, s>>>(g, pa);
     return 1;
 }
@@ -333,21 +347,22 @@ int launch_conv_cols_mfma(const void *args, hipStream_t s) {
     const int64_t groups_m = (g.M + 31) / 32, groups_n = (g.N + 31) / 32;
     const int64_t waves = groups_m * groups_n;
     if (waves >= (int64_t(1) << 30)) return 0;
+    const DivMagic div_n = make_div_magic((uint32_t)groups_n);
     // At most 700 tiles of at least eight K chunks: the four wavefronts of a block share a tile (384 -> 64 at
     // 14 x 14 with the residual: 7.2 -> 6.3 us, 960 -> 160 at 7 x 7: 8.3 -> 6.2 us; 1960 tiles of 320 -> 1280 lose)
     if (waves <= 700 && g.K >= 2 * KR * 32) {
         const dim3 grid((unsigned)((waves + 7) / 8 * 8));
         if (g.res != nullptr)
-            conv_cols_mfma_i8_kernel<true, 4><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
+            conv_cols_mfma_i8_kernel<true, 4><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves, div_n, (int)(grid.x / 8));
         else
-            conv_cols_mfma_i8_kernel<false, 4><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
+            conv_cols_mfma_i8_kernel<false, 4><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves, div_n, (int)(grid.x / 8));
         return 1;
     }
     const dim3 grid((unsigned)(((waves + kColsBlock / 64 - 1) / (kColsBlock / 64) + 7) / 8 * 8));
     if (g.res != nullptr)
-        conv_cols_mfma_i8_kernel<true, 1><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
+        conv_cols_mfma_i8_kernel<true, 1><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves, div_n, (int)(grid.x / 8));
     else
-        conv_cols_mfma_i8_kernel<false, 1><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves);
+        conv_cols_mfma_i8_kernel<false, 1><<<grid, dim3(kColsBlock), 0, s>>>(g, (int)groups_n, (int)waves, div_n, (int)(grid.x / 8));
     return 1;
 }
 

@@ -122,6 +122,7 @@ struct DwArgs {
     int32_t cb_size, cb_count, spb, sb_count;
     uint32_t cb_magic, strips_magic;  // floor(2^32 / d) + 1: x / d == umulhi(x, magic) for x < 2^16, 1 < d < 2^16
     int32_t blocks, chunk;  // launch geometry: `chunk` consecutive blocks per XCD
+    DivMagic div_cb, div_sb;  // block index / cb_count, / sb_count as a multiplication and a shift
 };
 
 struct DwChan {  // per channel, in shared memory: 48 bytes
@@ -149,14 +150,25 @@ __device__ __forceinline__ void transpose_3x4(uint32_t r0, uint32_t r1, uint32_t
 template <int TX, int TY, int SX, bool ZW, bool Q8>
 __global__ void __launch_bounds__(kBlock) dwconv3x3_i8_kernel(const DwArgs a) {
     __shared__ __align__(16) DwChan chan[kBlock];
+    // Every argument asked for in one batch (left alone the compiler loads them in three trips to memory in a row:
+    // behind the early exit, and again where a register of a wide load that nobody was waiting for had been given
+    // away), every dword of the wide loads named for that reason.
+    asm volatile("" ::"s"(a.chunk), "s"(a.blocks), "s"(a.div_cb.m), "s"(a.div_cb.s), "s"(a.div_sb.m), "s"(a.div_sb.s),
+                 "s"(a.cb_size), "s"(a.cb_count), "s"(a.spb), "s"(a.sb_count), "s"(a.cb_magic), "s"(a.strips_magic),
+                 "s"(a.strips), "s"(a.row_groups), "s"(a.x), "s"(a.w), "s"(a.bias), "s"(a.out), "s"(a.N), "s"(a.H), "s"(a.W),
+                 "s"(a.C), "s"(a.OH), "s"(a.OW), "s"(a.x_sn), "s"(a.x_sy), "s"(a.x_sx), "s"(a.x_bytes), "s"(a.o_bytes),
+                 "s"(a.sy), "s"(a.sx), "s"(a.pad_t), "s"(a.pad_l), "s"(a.zi), "s"(a.zw), "s"(a.bias_len), "s"(a.fused),
+                 "s"(a.out_size), "s"(a.scale.mult), "s"(a.scale.shift), "s"(a.scale.mult16), "s"(a.scale.p.in_zp),
+                 "s"(a.scale.p.out_zp), "s"(a.scale.p.out_lo), "s"(a.scale.p.out_hi), "s"(a.scale.p.double_round),
+                 "s"(a.scale.p.per_channel), "s"(a.scale.p.clamp_out));
     // blocks are dealt round-robin to the XCDs: give XCD k the k-th contiguous run of blocks
     const int bid = (int)(blockIdx.x % 8u) * a.chunk + (int)(blockIdx.x / 8u);
     if (bid >= a.blocks) return;
     // block -> (image, spatial block, channel block): uniform, on the scalar unit
-    const int cb = bid % a.cb_count;
-    const int rest_b = bid / a.cb_count;
-    const int sb = rest_b % a.sb_count;
-    const int n = rest_b / a.sb_count;
+    const int rest_b = div_magic(bid, a.div_cb);
+    const int cb = bid - rest_b * a.cb_count;
+    const int n = div_magic(rest_b, a.div_sb);
+    const int sb = rest_b - n * a.sb_count;
     const int tid = threadIdx.x;
 
     // ---- one channel per thread: weight columns, bias with the zero-point terms folded in, scales
@@ -410,6 +422,8 @@ int try_dwconv_i8_fast(mlel_ctx *ctx, hipStream_t s, const mlel_tensor *out, con
     if (blocks >= (int64_t(1) << 31) - 8) return 0;
     g.blocks = (int)blocks;
     g.chunk = (int)((blocks + 7) / 8);
+    g.div_cb = make_div_magic((uint32_t)g.cb_count);
+    g.div_sb = make_div_magic((uint32_t)g.sb_count);
     const dim3 grid((unsigned)(g.chunk * 8)), block(kBlock);
     const bool q8 = g.fused && g.out_size == 1;
     const int variant = (TY == 2 ? 4 : 0) + (g.sx == 2 ? 2 : 0) + (g.zw != 0 ? 1 : 0);
