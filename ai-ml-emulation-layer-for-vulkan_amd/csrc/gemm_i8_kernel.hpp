@@ -894,14 +894,18 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                     ws_l[wave_m * BN + wave_n * WN + j * 32 + (lane & 15) + ((lane >> 5) << 4)] = sw4[j][0];
             }
             __syncthreads();
-            // the channel sums into the registers of the lower lane half (the epilogue adds the halves, as in the
-            // other fetch modes); the row terms stay in the two tables, which the epilogue reads as it goes
+            // every lane takes the whole sum of its channel from the two tables (the other fetch modes leave partial
+            // sums in the two lane halves, which the epilogue adds); the row terms stay in their tables, which the
+            // epilogue reads
             if (need_wsum) {
+                int32_t lo[TN], hi[TN];
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
                     const int c = wave_n * WN + j * 32 + (lane & 31);
-                    wsum[j] = lane < 32 ? ws_l[c] + ws_l[BN + c] : 0;
+                    lo[j] = ws_l[c], hi[j] = ws_l[BN + c];
                 }
+#pragma unroll
+                for (int j = 0; j < TN; j++) wsum[j] = lo[j] + hi[j];
             }
         }
     } else {
@@ -944,7 +948,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
     for (int j = 0; j < TN; j++) {
         bias_adj[j] = chan_bias[j];
         if (need_wsum) {  // -zx * sum_k W[n][k] + K zx zw: the zero-point terms that depend on the channel only
-            const int32_t sw = wsum[j] + __shfl_xor(wsum[j], 32);
+            const int32_t sw = DL ? wsum[j] : wsum[j] + __shfl_xor(wsum[j], 32);
             bias_adj[j] = (int32_t)((uint32_t)bias_adj[j] - (uint32_t)g.zx * (uint32_t)sw +
                                     (uint32_t)k_len * (uint32_t)g.zx * (uint32_t)g.zw);
         }
@@ -1083,12 +1087,45 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
                         if constexpr (RES) d_res[k] = buf_load4(rres, d_off[k]);
                     }
         }
+        // The row terms of every register group are read from their tables up front where the registers allow it: a
+        // wavefront alone on its SIMD issues in order, and a read in front of each group's arithmetic made it wait for
+        // a trip to shared memory (and for the staging write in front of it) once per group.
+        constexpr bool ROWS_AHEAD = TM * 16 <= 32;
+        int32_t xca[ROWS_AHEAD ? TM : 1][4][4];
+        if constexpr (ROWS_AHEAD) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) xca[i][q][0] = xca[i][q][1] = xca[i][q][2] = xca[i][q][3] = 0;
+            if (need_xsum && !rows_done) {  // uniform: one test around all reads, so that they are issued together
+                int4 t[TM][4], u[TM][4];
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const int32_t *p0 = xs_tab + (DL ? BM : 0) + wave_m * WM + i * 32 + 8 * q + 4 * half;
+                        t[i][q] = *reinterpret_cast<const int4 *>(p0);
+                        u[i][q] = DL ? *reinterpret_cast<const int4 *>(p0 + BM) : int4{0, 0, 0, 0};
+                    }
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        xca[i][q][0] = t[i][q].x + u[i][q].x, xca[i][q][1] = t[i][q].y + u[i][q].y;
+                        xca[i][q][2] = t[i][q].z + u[i][q].z, xca[i][q][3] = t[i][q].w + u[i][q].w;
+                    }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < TM; i++) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 int32_t xc[4];
-                if (!rows_done) row_terms(i, q, xc); else xc[0] = xc[1] = xc[2] = xc[3] = 0;
+                if constexpr (ROWS_AHEAD) {
+                    xc[0] = xca[i][q][0], xc[1] = xca[i][q][1], xc[2] = xca[i][q][2], xc[3] = xca[i][q][3];
+                } else {
+                    if (!rows_done) row_terms(i, q, xc); else xc[0] = xc[1] = xc[2] = xc[3] = 0;
+                }
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
                     int32_t v[4];
@@ -1131,6 +1168,26 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_i8_kernel(const Ge
         __syncthreads();
         constexpr int PPR = BN / 16;  // 16-byte pieces per tile row
         static_assert((BM * PPR) % NTHREADS == 0, "whole pieces per thread");
+        if (!RES && (g.N & 15) == 0) {
+            // every piece inside the tensor is whole (uniform): all of a thread's pieces are read first and leave
+            // without a test (a piece outside the tensor has an offset beyond the buffer's extent and is dropped)
+            constexpr int NP = BM * PPR / NTHREADS;
+            uint4 d[NP];
+            uint32_t off[NP];
+#pragma unroll
+            for (int t = 0; t < NP; t++) {
+                const int piece = t * NTHREADS + tid;
+                const int r = piece / PPR, c16 = (piece % PPR) * 16;
+                const int m = m_base + r, n0 = n_base + c16;
+                d[t] = *reinterpret_cast<const uint4 *>(so + r * OP + c16);
+                off[t] = (m < g.M && n0 < g.N) ? (uint32_t)m * (uint32_t)g.ldo + (uint32_t)n0 : kOobOffset;
+            }
+#pragma unroll
+            for (int t = 0; t < NP; t++)
+                __builtin_amdgcn_raw_buffer_store_b128(v4i{(int)d[t].x, (int)d[t].y, (int)d[t].z, (int)d[t].w}, ores, (int)off[t], 0,
+                                                       kOutAux);
+            return;
+        }
 #pragma unroll
         for (int t = 0; t < BM * PPR / NTHREADS; t++) {
             const int piece = t * NTHREADS + tid;
