@@ -199,6 +199,26 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
+    // the bias of this lane's columns (fused form): lane holds, per register quad q, columns 8q + 4 * (lane / 32) ...
+    // (where to fetch it: behind the first stages of the direct-to-LDS loop when that costs 16 registers; the wide tile's
+    // 32 cost its GELU epilogue more than the trip to memory they hide, 35.5 -> 36.0 us)
+    constexpr bool BIAS_AHEAD = BROWS && TN == 1;
+    float bias_r[TN][4][4];
+    auto fetch_bias = [&]() {
+        // through a buffer resource of the bias's extent: a column beyond N (or no bias at all) reads as zero without a test
+        const __amdgpu_buffer_rsrc_t bias_res =
+            rsrc(o.bias, o.bias != nullptr ? (g.bias_len == 1 ? 4u : (uint32_t)g.N * 4u) : 0u);
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int n0 = n_base + wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    bias_r[j][q][e] = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(bias_res, g.bias_len == 1 ? 0 : (n0 + e) * 4, 0, 0));
+            }
+    };
     if constexpr (BROWS) {
         // ---- direct-to-LDS main loop (K % 32 == 0: whole 64-byte steps)
         constexpr int BK = 64, DL_S = 4, DL_STAGE = (BM + BN) * BK;
@@ -289,6 +309,11 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
                 else load16_to_lds(wr, wd + (l - XI) * NT * 16, wo[l - XI], (uint32_t)d * BK);
             }
         }
+        // The bias is asked for behind the first stages and used behind the loop (asked for there, its trip to memory
+        // was waited out by every wavefront in front of the first store).  These loads are younger than the first
+        // stages and older than every later request, so the counted waits hold with them in flight: the first ones
+        // only wait for a few requests more.
+        if (EPI == 1 && BIAS_AHEAD) fetch_bias();
         wait_vmcnt<(DL_S - 2) * NLA>();  // stage 0 has landed: what was requested behind it may be in flight
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
@@ -409,20 +434,9 @@ __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N) gemm_f16_kernel(const 
     const int64_t o_base = o.view ? (int64_t)(batch / o.v_nb2) * o.vs_nb1 + (int64_t)(batch % o.v_nb2) * o.vs_nb2
                                   : (int64_t)batch * o.o_batch;
     const __amdgpu_buffer_rsrc_t ores = rsrc(o.out + o_base, o.o_bytes);
-    // the bias of this lane's columns, fetched in one batch before any store (a load after a store would have to
-    // wait for it: the compiler cannot tell that the two do not alias)
-    float bias_r[TN][4][4];
-    if (EPI == 1) {
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int n0 = n_base + wave_n * WN + j * 32 + 8 * q + 4 * (lane >> 5);
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    bias_r[j][q][e] = (o.bias != nullptr && n0 < g.N) ? o.bias[g.bias_len == 1 ? 0 : n0 + e] : 0.f;
-            }
-    }
+    // otherwise fetched here, in one batch before any store (a load after a store would have to wait for it: the
+    // compiler cannot tell that the two do not alias)
+    if (EPI == 1 && !BIAS_AHEAD) fetch_bias();
     if (EPI == 1) {
         // fp16 result: a lane's four values are only eight bytes of a row, and a store instruction would touch 32 rows.
         // The tile goes through shared memory instead (the operand buffers are free: the loop ended with a barrier)
