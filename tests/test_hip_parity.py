@@ -297,6 +297,25 @@ def test_conv2d_i8_direct_to_lds_row_weights(run, oracle):
     np.testing.assert_array_equal(out, exp)
 
 
+def test_conv2d_i8_direct_to_lds_ragged_channels(run, oracle):
+    """The 128 x 128 tile of the direct-to-LDS pipeline where the channel extent is not a multiple of 16 and the positions
+    are not a multiple of 128: the staged 8-bit tile leaves through the general stores (whole pieces, then the dwords of
+    the last channels of a row), nothing is written beyond a row's end, and the int32 accumulator agrees as well."""
+    rng = np.random.default_rng(777)
+    oc = 2036  # 15 whole tiles of channels and one of 116: 7 whole pieces and a dword
+    x = ri(rng, -128, 127, (4, 32, 31, 128), np.int8)
+    w = ri(rng, -127, 127, (oc, 1, 1, 128), np.int8)
+    bias = ri(rng, -2 ** 15, 2 ** 15, (oc,), np.int32)
+    attr = abi.conv2d_attr(input_zp=7, weight_zp=-2)
+    acc = oracle.conv2d(x, w, bias, (4, 32, 31, oc), abi.I32, attr)
+    np.testing.assert_array_equal(run.conv2d(x, w, bias, (4, 32, 31, oc), abi.I32, attr), acc)
+    mult, shift = rescale_params(rng, oc)
+    rattr = abi.rescale_attr(0, -3, True, True, True)
+    exp = np.clip(oracle.rescale(acc, mult, shift, abi.I8, rattr), -128, 100).astype(np.int8)
+    out = run.conv2d(x, w, bias, (4, 32, 31, oc), abi.I8, attr, epilogue=(mult, shift, rattr, (-128, 100)))
+    np.testing.assert_array_equal(out, exp)
+
+
 def test_matmul_float_generic(run, oracle):
     rng = np.random.default_rng(8)
     a = rng.standard_normal((2, 9, 33)).astype(np.float32)
